@@ -1,0 +1,112 @@
+"""ctypes binding of libam_hip.so — the same C ABI (include/am_hip.h) a Nim `{.importc.}` layer
+binds. There is no fallback: if the library is missing or a call fails, an exception is raised."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libam_hip.so")
+
+AM_OK, AM_E_ARG, AM_E_SHAPE, AM_E_DTYPE, AM_E_ALLOC, AM_E_HIP, AM_E_NODEVICE = 0, -1, -2, -3, -4, -5, -6
+AM_MAXRANK = 6
+
+OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
+          relu_bwd=8, max=9, min=10)
+UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
+EPI = dict(none=0, bias=1, relu=2, bias_relu=3)
+
+SFX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64",
+       np.dtype(np.int32): "i32", np.dtype(np.int64): "i64"}
+CTYPE = {"f32": ctypes.c_float, "f64": ctypes.c_double, "i32": ctypes.c_int32, "i64": ctypes.c_int64}
+
+
+class HipError(RuntimeError):
+    """A HIP runtime call failed, no device is usable, or the library is missing."""
+
+
+class HipAllocError(HipError, MemoryError):
+    pass
+
+
+# Every symbol include/am_hip.h declares, with its ctypes signature.
+def _signatures():
+    ci, i64, vp, sz = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t
+    pp = ctypes.POINTER(ctypes.c_void_p)
+    sig = {
+        "am_hip_last_error": (ctypes.c_char_p, []),
+        "am_hip_version": (ctypes.c_char_p, []),
+        "am_hip_init": (ci, [ci]),
+        "am_hip_device_count": (ci, [ctypes.POINTER(ci)]),
+        "am_hip_device_info": (ci, [ctypes.c_char_p, sz, ctypes.POINTER(ci), ctypes.POINTER(ci),
+                                    ctypes.POINTER(sz), ctypes.POINTER(ci)]),
+        "am_hip_malloc": (ci, [sz, pp]),
+        "am_hip_free": (ci, [vp]),
+        "am_hip_memcpy_h2d": (ci, [vp, vp, sz]),
+        "am_hip_memcpy_d2h": (ci, [vp, vp, sz]),
+        "am_hip_memcpy_d2d": (ci, [vp, vp, sz]),
+        "am_hip_memset": (ci, [vp, ci, sz]),
+        "am_hip_sync": (ci, []),
+        "am_hip_stream": (vp, []),
+        "am_hip_event_create": (ci, [pp]),
+        "am_hip_event_record": (ci, [vp]),
+        "am_hip_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),
+        "am_hip_event_destroy": (ci, [vp]),
+    }
+    for sfx, ct in CTYPE.items():
+        gemm = [i64, i64, i64, ct, vp, i64, i64, vp, i64, i64, ct, vp, i64, i64]
+        sig[f"am_hip_gemm_{sfx}"] = (ci, gemm)
+        if sfx in ("f32", "f64"):
+            sig[f"am_hip_gemm_ex_{sfx}"] = (ci, gemm + [ci, vp, i64, i64])
+        sig[f"am_hip_ew_binary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp, vp, vp])
+        sig[f"am_hip_ew_scalar_{sfx}"] = (ci, [ci, ci, ci, vp, vp, vp, vp, vp, ct])
+        sig[f"am_hip_ew_unary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp])
+    return sig
+
+
+SIGNATURES = _signatures()
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the built library (no build is attempted here) and binds every exported symbol."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HipError(f"{LIB_PATH} is missing: build it with `python -m arraymancer_amd.build` "
+                       f"(there is no CPU fallback)")
+    L = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(L, name)          # AttributeError here = the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def last_error() -> str:
+    return (load().am_hip_last_error() or b"").decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    """Maps a status code to the exception the reference raises in the same situation:
+    shape problems are ValueError (src/arraymancer/tensor/private/p_checks_cuda.nim:15-19),
+    everything the device reports is HipError."""
+    if rc == AM_OK:
+        return
+    msg = last_error()
+    if rc in (AM_E_ARG, AM_E_SHAPE):
+        raise ValueError(msg)
+    if rc == AM_E_DTYPE:
+        raise TypeError(msg)
+    if rc == AM_E_ALLOC:
+        raise HipAllocError(msg)
+    raise HipError(f"[{rc}] {msg}")
+
+
+def i64_array(values):
+    values = [int(v) for v in values]
+    return (ctypes.c_int64 * max(1, len(values)))(*values)

@@ -1,0 +1,39 @@
+// Shared host-side helpers of libam_hip.so: status codes, thread-local error text, the
+// library stream, and the shape/stride container that kernels take by value.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/am_hip.h"
+
+namespace am {
+
+// Records `msg` (printf style) as the calling thread's last error and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// Lazily initialises the device context (device 0 unless am_hip_init chose another).
+int ensure_init();
+hipStream_t stream();
+int num_cus();
+
+#define AM_HIP_TRY(expr)                                                                    \
+  do {                                                                                      \
+    hipError_t _e = (expr);                                                                 \
+    if (_e != hipSuccess)                                                                   \
+      return ::am::fail(AM_E_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e),    \
+                        __FILE__, __LINE__);                                                \
+  } while (0)
+
+#define AM_TRY(expr)                 \
+  do {                               \
+    int _rc = (expr);                \
+    if (_rc != AM_OK) return _rc;    \
+  } while (0)
+
+// Checks the launch that was just enqueued.
+static inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(AM_E_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+  return AM_OK;
+}
+
+}  // namespace am

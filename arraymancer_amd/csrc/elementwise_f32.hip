@@ -1,0 +1,4 @@
+// Element-wise / broadcast / map entry points for float tensors.
+#include "elementwise_impl.h"
+
+AM_EW_DEFINE_ENTRY_POINTS(float, f32)

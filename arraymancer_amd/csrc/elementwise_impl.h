@@ -1,0 +1,458 @@
+// Element-wise / broadcast / map kernels for gfx950 and their host-side dispatch, generic over
+// the element type. Each elementwise_<dtype>.hip includes this header and instantiates the
+// C-ABI entry points for one type.
+//
+// Two kernel families:
+//   ew_rows     the HBM-streaming path. After dimension collapsing the operands are seen as
+//               `rows` x `L` with a unit (or zero) innermost stride; every lane moves 16-byte
+//               vectors (dwordx4) with non-temporal loads/stores, several in flight per lane.
+//               Broadcast operands are either a vector re-read per row (row vector, stays in
+//               L2) or one scalar per row (column vector, read through the scalar path).
+//   ew_generic  any strides (transposed, negative, non-unit inner): C-order index -> offsets by
+//               per-dimension div/mod on the collapsed shape.
+// The reference walks every operand in C order through its own strides
+// (src/arraymancer/tensor/private/p_accessors.nim:181-208, 378-413); both kernels compute the
+// same element correspondence in closed form instead of carrying coordinates.
+#pragma once
+#include <type_traits>
+#include "common.h"
+
+namespace am {
+namespace ew {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;  // 16-byte vectors in flight per lane per operand
+
+template <typename T> struct Traits;
+template <> struct Traits<float> {
+  typedef float U; typedef float V __attribute__((ext_vector_type(4)));
+  static constexpr int kVec = 4; static constexpr bool kFloat = true;
+};
+template <> struct Traits<double> {
+  typedef double U; typedef double V __attribute__((ext_vector_type(2)));
+  static constexpr int kVec = 2; static constexpr bool kFloat = true;
+};
+template <> struct Traits<int32_t> {
+  typedef uint32_t U; typedef int32_t V __attribute__((ext_vector_type(4)));
+  static constexpr int kVec = 4; static constexpr bool kFloat = false;
+};
+template <> struct Traits<int64_t> {
+  typedef uint64_t U; typedef int64_t V __attribute__((ext_vector_type(2)));
+  static constexpr int kVec = 2; static constexpr bool kFloat = false;
+};
+
+__device__ __forceinline__ float dev_exp(float x) { return expf(x); }
+__device__ __forceinline__ double dev_exp(double x) { return exp(x); }
+__device__ __forceinline__ float dev_tanh(float x) { return tanhf(x); }
+__device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
+
+// ---- binary op bodies. Integer arithmetic is carried out in the unsigned twin so that it wraps.
+template <typename T, int OP> struct BinOp {
+  typedef typename Traits<T>::U U;
+  static __device__ __forceinline__ T apply(T x, T y) {
+    if constexpr (OP == AM_OP_ADD) return (T)((U)x + (U)y);
+    else if constexpr (OP == AM_OP_SUB) return (T)((U)x - (U)y);
+    else if constexpr (OP == AM_OP_MUL) return (T)((U)x * (U)y);
+    else if constexpr (OP == AM_OP_DIV) {
+      if constexpr (Traits<T>::kFloat) return x / y;
+      else {
+        if (y == 0) return 0;
+        if (y == (T)-1) return (T)((U)0 - (U)x);
+        return x / y;
+      }
+    } else if constexpr (OP == AM_OP_MOD) {
+      if (y == 0 || y == (T)-1) return 0;
+      return x % y;
+    } else if constexpr (OP == AM_OP_ADD_RELU) {
+      T t = (T)((U)x + (U)y);
+      return ((T)0 >= t) ? (T)0 : t;
+    } else if constexpr (OP == AM_OP_ADD_SIGMOID) {
+      T t = x + y;
+      return (T)1 / ((T)1 + dev_exp(-t));
+    } else if constexpr (OP == AM_OP_ADD_TANH) {
+      return dev_tanh(x + y);
+    } else if constexpr (OP == AM_OP_RELU_BWD) {
+      return (x <= (T)0) ? (T)0 : y;
+    } else if constexpr (OP == AM_OP_MAX) {
+      return (y <= x) ? x : y;
+    } else {  // AM_OP_MIN
+      return (x <= y) ? x : y;
+    }
+  }
+};
+
+// Unary ops ride the same kernels with the second operand ignored.
+constexpr int kUnaryBase = 100;
+template <typename T, int UOP> struct UnOp {
+  typedef typename Traits<T>::U U;
+  static __device__ __forceinline__ T apply(T x, T) {
+    if constexpr (UOP == AM_UOP_COPY) return x;
+    else if constexpr (UOP == AM_UOP_NEG) {
+      if constexpr (Traits<T>::kFloat) return -x; else return (T)((U)0 - (U)x);
+    } else if constexpr (UOP == AM_UOP_RELU) return ((T)0 >= x) ? (T)0 : x;
+    else if constexpr (UOP == AM_UOP_SIGMOID) return (T)1 / ((T)1 + dev_exp(-x));
+    else if constexpr (UOP == AM_UOP_TANH) return dev_tanh(x);
+    else if constexpr (UOP == AM_UOP_EXP) return dev_exp(x);
+    else {  // ABS
+      if constexpr (Traits<T>::kFloat) return __builtin_fabs(x);
+      else return (x < 0) ? (T)((U)0 - (U)x) : x;
+    }
+  }
+};
+
+template <typename T, int CODE> struct OpSel {
+  typedef typename std::conditional<(CODE >= kUnaryBase), UnOp<T, CODE - kUnaryBase>, BinOp<T, CODE>>::type type;
+};
+
+// ---- layouts passed to kernels by value
+constexpr int kMaxOuter = AM_MAXRANK - 1;
+
+enum Kind : int { kVecOperand = 0, kRowScalar = 1, kConst = 2 };
+
+template <typename T> struct RowsArgs {
+  T* dst; const T* a; const T* b;
+  T scalar;               // the kConst operand
+  int a_stream, b_stream; // 1: operand is read once (non-temporal loads); 0: re-read per row, keep cached
+  int64_t L;              // inner extent (elements)
+  uint32_t tiles_per_row; // ceil(L / tile)
+  uint32_t total_tiles;   // rows * tiles_per_row
+  int outer_rank;         // 0..5 collapsed outer dims (row-major over them = row index)
+  int64_t oshape[kMaxOuter];
+  int64_t od[kMaxOuter], oa[kMaxOuter], ob[kMaxOuter];  // outer strides per operand (elements)
+};
+
+template <typename T> struct GenericArgs {
+  T* dst; const T* a; const T* b;
+  T scalar;
+  int64_t n;
+  int rank;
+  int64_t shape[AM_MAXRANK];
+  int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK];
+};
+
+template <typename T, int CODE, int AK, int BK, bool SWAP>
+__global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
+  typedef typename Traits<T>::V V;
+  typedef typename OpSel<T, CODE>::type Op;
+  constexpr int VEC = Traits<T>::kVec;
+  constexpr int64_t TILE = (int64_t)kThreads * VEC * kUnroll;
+
+  for (uint32_t tile = blockIdx.x; tile < p.total_tiles; tile += gridDim.x) {
+    const uint32_t row = tile / p.tiles_per_row;
+    const uint32_t ct = tile - row * p.tiles_per_row;
+    int64_t offd = 0, offa = 0, offb = 0;
+    {
+      uint32_t rem = row;
+      for (int d = p.outer_rank - 1; d >= 0; --d) {
+        const uint32_t ext = (uint32_t)p.oshape[d];
+        const uint32_t q = rem / ext;
+        const int64_t c = (int64_t)(rem - q * ext);
+        rem = q;
+        offd += c * p.od[d];
+        offa += c * p.oa[d];
+        if constexpr (BK != kConst) offb += c * p.ob[d];
+      }
+    }
+    T* __restrict__ drow = p.dst + offd;
+    const T* __restrict__ arow = p.a + offa;
+    const T* __restrict__ brow = (BK != kConst) ? p.b + offb : nullptr;
+    T asc = (T)0, bsc = p.scalar;
+    if constexpr (AK == kRowScalar) asc = arow[0];
+    if constexpr (BK == kRowScalar) bsc = brow[0];
+
+    const int64_t col0 = (int64_t)ct * TILE + (int64_t)threadIdx.x * VEC;
+    V av[kUnroll], bv[kUnroll];
+    bool full[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t col = col0 + (int64_t)u * kThreads * VEC;
+      full[u] = (col + VEC <= p.L);
+      if (full[u]) {
+        if constexpr (AK == kVecOperand)
+          av[u] = p.a_stream ? __builtin_nontemporal_load((const V*)(arow + col)) : *(const V*)(arow + col);
+        if constexpr (BK == kVecOperand)
+          bv[u] = p.b_stream ? __builtin_nontemporal_load((const V*)(brow + col)) : *(const V*)(brow + col);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t col = col0 + (int64_t)u * kThreads * VEC;
+      if (full[u]) {
+        V r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const T x = (AK == kVecOperand) ? av[u][e] : asc;
+          const T y = (BK == kVecOperand) ? bv[u][e] : bsc;
+          r[e] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+        }
+        __builtin_nontemporal_store(r, (V*)(drow + col));
+      } else {
+        for (int64_t c = col; c < p.L; ++c) {   // ragged end of the row (< VEC elements)
+          const T x = (AK == kVecOperand) ? arow[c] : asc;
+          const T y = (BK == kVecOperand) ? brow[c] : bsc;
+          drow[c] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int CODE, bool BCONST, bool SWAP, typename IDX>
+__global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T> p) {
+  typedef typename OpSel<T, CODE>::type Op;
+  const IDX n = (IDX)p.n;
+  const IDX step = (IDX)gridDim.x * kThreads;
+  for (IDX i = (IDX)blockIdx.x * kThreads + threadIdx.x; i < n; i += step) {
+    IDX rem = i;
+    int64_t offd = 0, offa = 0, offb = 0;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      const IDX ext = (IDX)p.shape[d];
+      const IDX q = rem / ext;
+      const int64_t c = (int64_t)(rem - q * ext);
+      rem = q;
+      offd += c * p.sd[d];
+      offa += c * p.sa[d];
+      if constexpr (!BCONST) offb += c * p.sb[d];
+    }
+    const T x = p.a[offa];
+    const T y = BCONST ? p.scalar : p.b[offb];
+    p.dst[offd] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------
+struct Collapsed {
+  int rank;
+  int64_t shape[AM_MAXRANK];
+  int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK];
+  int64_t n;
+};
+
+// Drops extent-1 dims and merges neighbours that every operand walks as one run
+// (stride[i] == shape[i+1] * stride[i+1] for dst, a and b alike).
+static inline int collapse(int rank, const int64_t* shape, const int64_t* sd, const int64_t* sa,
+                           const int64_t* sb, Collapsed* out) {
+  out->rank = 0;
+  out->n = 1;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] < 0) return fail(AM_E_ARG, "negative extent %lld in dimension %d", (long long)shape[i], i);
+    out->n *= shape[i];
+  }
+  if (out->n == 0) return AM_OK;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] == 1) continue;
+    const int64_t d = sd[i], a = sa[i], b = sb ? sb[i] : 0;
+    if (d == 0) return fail(AM_E_SHAPE, "destination has stride 0 on dimension %d of extent %lld", i, (long long)shape[i]);
+    const int r = out->rank;
+    if (r > 0 && out->sd[r - 1] == shape[i] * d && out->sa[r - 1] == shape[i] * a &&
+        out->sb[r - 1] == shape[i] * b) {
+      out->shape[r - 1] *= shape[i];
+      out->sd[r - 1] = d; out->sa[r - 1] = a; out->sb[r - 1] = b;
+    } else {
+      out->shape[r] = shape[i];
+      out->sd[r] = d; out->sa[r] = a; out->sb[r] = b;
+      out->rank = r + 1;
+    }
+  }
+  if (out->rank == 0) {  // a single element
+    out->rank = 1; out->shape[0] = 1; out->sd[0] = 1; out->sa[0] = 1; out->sb[0] = 1;
+  }
+  return AM_OK;
+}
+
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <typename T, int CODE, bool BCONST, bool SWAP>
+static int launch_generic(const Collapsed& c, T* dst, const T* a, const T* b, T scalar) {
+  GenericArgs<T> g;
+  g.dst = dst; g.a = a; g.b = b; g.scalar = scalar; g.n = c.n; g.rank = c.rank;
+  for (int i = 0; i < AM_MAXRANK; ++i) {
+    g.shape[i] = i < c.rank ? c.shape[i] : 1;
+    g.sd[i] = i < c.rank ? c.sd[i] : 0;
+    g.sa[i] = i < c.rank ? c.sa[i] : 0;
+    g.sb[i] = i < c.rank ? c.sb[i] : 0;
+  }
+  int64_t blocks = (c.n + kThreads - 1) / kThreads;
+  const int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  if (c.n < ((int64_t)1 << 31)) {
+    hipLaunchKernelGGL((ew_generic<T, CODE, BCONST, SWAP, uint32_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+  } else {
+    hipLaunchKernelGGL((ew_generic<T, CODE, BCONST, SWAP, uint64_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+  }
+  return check_launch("ew_generic");
+}
+
+// Runs dst = op(a, b) (BCONST: b is `scalar`). Chooses the streaming kernel when every
+// operand's innermost collapsed stride is 1 (or 0 for a/b) and rows start 16-byte aligned.
+template <typename T, int CODE, bool BCONST, bool SWAP>
+static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a,
+               const int64_t* sa, const T* b, const int64_t* sb, T scalar) {
+  constexpr int VEC = Traits<T>::kVec;
+  Collapsed c;
+  AM_TRY(collapse(rank, shape, sd, sa, BCONST ? nullptr : sb, &c));
+  if (c.n == 0) return AM_OK;
+  AM_TRY(ensure_init());
+
+  const int in = c.rank - 1;
+  const int64_t L = c.shape[in];
+  const int64_t id = c.sd[in], ia = c.sa[in], ib = BCONST ? 0 : c.sb[in];
+  bool ok = (id == 1) && (ia == 0 || ia == 1) && (ib == 0 || ib == 1) && !(ia == 0 && ib == 0 && !BCONST);
+  if (BCONST && ia == 0) ok = false;
+  if (ok) {
+    ok = aligned16(dst) && (ia == 0 || aligned16(a)) && (BCONST || ib == 0 || aligned16(b));
+    for (int d = 0; d < in && ok; ++d) {
+      if (c.sd[d] % VEC != 0) ok = false;
+      if (ia == 1 && c.sa[d] % VEC != 0) ok = false;
+      if (!BCONST && ib == 1 && c.sb[d] % VEC != 0) ok = false;
+    }
+  }
+  int64_t rows = 1;
+  for (int d = 0; d < in; ++d) rows *= c.shape[d];
+  const int64_t tile = (int64_t)kThreads * VEC * kUnroll;
+  const int64_t tiles_per_row = (L + tile - 1) / tile;
+  // Short rows would leave most lanes of a tile idle: those shapes go to the generic kernel.
+  if (ok && rows > 1 && L < tile / 4) ok = false;
+  if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31) || rows >= ((int64_t)1 << 31))) ok = false;
+  if (!ok) return launch_generic<T, CODE, BCONST, SWAP>(c, dst, a, b, scalar);
+
+  RowsArgs<T> r;
+  r.dst = dst; r.a = a; r.b = b; r.scalar = scalar; r.L = L;
+  r.tiles_per_row = (uint32_t)tiles_per_row;
+  r.total_tiles = (uint32_t)(tiles_per_row * rows);
+  r.outer_rank = in;
+  // An operand whose outer strides are all zero is one row re-read `rows` times: keep it cached.
+  r.a_stream = 0; r.b_stream = 0;
+  for (int d = 0; d < in; ++d) {
+    if (c.sa[d] != 0) r.a_stream = 1;
+    if (c.sb[d] != 0) r.b_stream = 1;
+  }
+  if (in == 0) { r.a_stream = 1; r.b_stream = 1; }
+  for (int d = 0; d < kMaxOuter; ++d) {
+    r.oshape[d] = d < in ? c.shape[d] : 1;
+    r.od[d] = d < in ? c.sd[d] : 0;
+    r.oa[d] = d < in ? c.sa[d] : 0;
+    r.ob[d] = d < in ? c.sb[d] : 0;
+  }
+  int64_t blocks = r.total_tiles;
+  const int64_t cap = (int64_t)num_cus() * 32;
+  if (blocks > cap) blocks = cap;
+  const dim3 grid((unsigned)blocks), block(kThreads);
+  if constexpr (BCONST) {
+    hipLaunchKernelGGL((ew_rows<T, CODE, kVecOperand, kConst, SWAP>), grid, block, 0, stream(), r);
+  } else {
+    if (ia == 1 && ib == 1) hipLaunchKernelGGL((ew_rows<T, CODE, kVecOperand, kVecOperand, false>), grid, block, 0, stream(), r);
+    else if (ia == 1) hipLaunchKernelGGL((ew_rows<T, CODE, kVecOperand, kRowScalar, false>), grid, block, 0, stream(), r);
+    else hipLaunchKernelGGL((ew_rows<T, CODE, kRowScalar, kVecOperand, false>), grid, block, 0, stream(), r);
+  }
+  return check_launch("ew_rows");
+}
+
+static inline int check_common(const char* fn, int rank, const int64_t* shape, const void* dst,
+                               const int64_t* sd, const void* a, const int64_t* sa) {
+  if (rank < 0 || rank > AM_MAXRANK) return fail(AM_E_ARG, "%s: rank %d outside 0..%d", fn, rank, AM_MAXRANK);
+  if (rank > 0 && (!shape || !sd || !sa)) return fail(AM_E_ARG, "%s: null shape/stride array", fn);
+  if (!dst || !a) {
+    // empty tensors may carry null pointers
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= shape[i];
+    if (n != 0) return fail(AM_E_ARG, "%s: null data pointer", fn);
+  }
+  return AM_OK;
+}
+
+template <typename T>
+static int binary(const char* fn, int op, int rank, const int64_t* shape, T* dst, const int64_t* sd,
+                  const T* a, const int64_t* sa, const T* b, const int64_t* sb) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  if (rank > 0 && !sb) return fail(AM_E_ARG, "%s: null stride array", fn);
+  {
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= shape[i];
+    if (n != 0 && !b) return fail(AM_E_ARG, "%s: null data pointer", fn);
+  }
+  constexpr bool F = Traits<T>::kFloat;
+  switch (op) {
+#define AM_CASE(code) case code: return run<T, code, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0)
+    AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
+    AM_CASE(AM_OP_ADD_RELU); AM_CASE(AM_OP_RELU_BWD); AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN);
+#undef AM_CASE
+    case AM_OP_MOD:
+      if constexpr (!F) return run<T, AM_OP_MOD, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
+      else return fail(AM_E_DTYPE, "%s: mod is defined for integer tensors only", fn);
+    case AM_OP_ADD_SIGMOID:
+      if constexpr (F) return run<T, AM_OP_ADD_SIGMOID, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
+      else return fail(AM_E_DTYPE, "%s: add_sigmoid is defined for float tensors only", fn);
+    case AM_OP_ADD_TANH:
+      if constexpr (F) return run<T, AM_OP_ADD_TANH, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
+      else return fail(AM_E_DTYPE, "%s: add_tanh is defined for float tensors only", fn);
+    default:
+      return fail(AM_E_ARG, "%s: unknown op %d", fn, op);
+  }
+}
+
+template <typename T, int CODE>
+static int scalar_lr(bool left, int rank, const int64_t* shape, T* dst, const int64_t* sd,
+                     const T* a, const int64_t* sa, T s) {
+  if (left) return run<T, CODE, true, true>(rank, shape, dst, sd, a, sa, nullptr, nullptr, s);
+  return run<T, CODE, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, s);
+}
+
+template <typename T>
+static int scalar(const char* fn, int op, int left, int rank, const int64_t* shape, T* dst,
+                  const int64_t* sd, const T* a, const int64_t* sa, T s) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  constexpr bool F = Traits<T>::kFloat;
+  switch (op) {
+#define AM_CASE(code) case code: return scalar_lr<T, code>(left != 0, rank, shape, dst, sd, a, sa, s)
+    AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
+    AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN);
+#undef AM_CASE
+    case AM_OP_MOD:
+      if constexpr (!F) return scalar_lr<T, AM_OP_MOD>(left != 0, rank, shape, dst, sd, a, sa, s);
+      else return fail(AM_E_DTYPE, "%s: mod is defined for integer tensors only", fn);
+    default:
+      return fail(AM_E_ARG, "%s: op %d has no tensor-scalar form", fn, op);
+  }
+}
+
+template <typename T>
+static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst, const int64_t* sd,
+                 const T* a, const int64_t* sa) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  constexpr bool F = Traits<T>::kFloat;
+  switch (op) {
+#define AM_CASE(code) case code: return run<T, kUnaryBase + code, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0)
+    AM_CASE(AM_UOP_COPY); AM_CASE(AM_UOP_NEG); AM_CASE(AM_UOP_RELU); AM_CASE(AM_UOP_ABS);
+#undef AM_CASE
+    case AM_UOP_SIGMOID:
+      if constexpr (F) return run<T, kUnaryBase + AM_UOP_SIGMOID, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
+      else return fail(AM_E_DTYPE, "%s: sigmoid is defined for float tensors only", fn);
+    case AM_UOP_TANH:
+      if constexpr (F) return run<T, kUnaryBase + AM_UOP_TANH, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
+      else return fail(AM_E_DTYPE, "%s: tanh is defined for float tensors only", fn);
+    case AM_UOP_EXP:
+      if constexpr (F) return run<T, kUnaryBase + AM_UOP_EXP, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
+      else return fail(AM_E_DTYPE, "%s: exp is defined for float tensors only", fn);
+    default:
+      return fail(AM_E_ARG, "%s: unknown unary op %d", fn, op);
+  }
+}
+
+}  // namespace ew
+}  // namespace am
+
+#define AM_EW_DEFINE_ENTRY_POINTS(T, SFX)                                                              \
+  extern "C" int am_hip_ew_binary_##SFX(int op, int rank, const int64_t* shape, T* dst,                \
+                                        const int64_t* ds, const T* a, const int64_t* as_,             \
+                                        const T* b, const int64_t* bs) {                               \
+    return ::am::ew::binary<T>("am_hip_ew_binary_" #SFX, op, rank, shape, dst, ds, a, as_, b, bs);     \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_scalar_##SFX(int op, int left, int rank, const int64_t* shape, T* dst,      \
+                                        const int64_t* ds, const T* a, const int64_t* as_, T s) {      \
+    return ::am::ew::scalar<T>("am_hip_ew_scalar_" #SFX, op, left, rank, shape, dst, ds, a, as_, s);   \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_unary_##SFX(int op, int rank, const int64_t* shape, T* dst,                 \
+                                       const int64_t* ds, const T* a, const int64_t* as_) {            \
+    return ::am::ew::unary<T>("am_hip_ew_unary_" #SFX, op, rank, shape, dst, ds, a, as_);              \
+  }

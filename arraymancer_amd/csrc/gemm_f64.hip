@@ -1,0 +1,37 @@
+// float64 GEMM entry points (MFMA path): am_hip_gemm_f64, am_hip_gemm_ex_f64.
+#include "gemm_mfma_impl.h"
+
+using namespace am;
+using namespace am::gemm;
+
+static int run_f64(Args<double>& g) {
+  const int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
+  const int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
+  // Candidate workgroup tiles, largest first, with the relative MFMA efficiency of each.
+  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.7}, {32, 32, 0.4}};
+  switch (choose_tile(cand, 3, g.M, g.N, "AM_HIP_GEMM_TILE_F64")) {
+    case 0: return launch_kinds<double, 128, 128, 16, 2, 2>(g, ak, bk);
+    case 1: return launch_kinds<double, 64, 64, 16, 2, 2>(g, ak, bk);
+    default: return launch_kinds<double, 32, 32, 16, 2, 2>(g, ak, bk);
+  }
+}
+
+extern "C" int am_hip_gemm_ex_f64(int64_t M, int64_t N, int64_t K, double alpha, const double* A, int64_t rsA,
+                                  int64_t csA, const double* B, int64_t rsB, int64_t csB, double beta, double* C,
+                                  int64_t rsC, int64_t csC, int epilogue, const double* bias,
+                                  int64_t bias_rs, int64_t bias_cs) {
+  Args<double> g;
+  const int rc = prepare<double>("am_hip_gemm_f64", M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC,
+                            epilogue, bias, bias_rs, bias_cs, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  return run_f64(g);
+}
+
+extern "C" int am_hip_gemm_f64(int64_t M, int64_t N, int64_t K, double alpha, const double* A, int64_t rsA,
+                               int64_t csA, const double* B, int64_t rsB, int64_t csB, double beta, double* C,
+                               int64_t rsC, int64_t csC) {
+  return am_hip_gemm_ex_f64(M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC, AM_EPI_NONE,
+                            nullptr, 0, 0);
+}

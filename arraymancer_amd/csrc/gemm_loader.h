@@ -1,0 +1,148 @@
+// Global -> register -> LDS movers for one operand slab of a GEMM workgroup tile, shared by the
+// MFMA (f32/f64) and VALU (i32/i64) kernels. An operand is X(mn, k) = X[mn * ld_mn + k * ld_k];
+// a slab is BMN rows/cols by BK k values. Out-of-range elements are zero-filled.
+//
+// LDS layouts:
+//   k-group  [k / VK][mn][VK]   (16-byte slot per (k-group, mn)); only for kKContig with KG = true
+//   k-row    [k][mn]            everything else
+// VK = 16 bytes / sizeof(T).
+#pragma once
+#include "gemm_common.h"
+
+namespace am {
+namespace gemm {
+
+template <typename T> struct VecTraits;
+template <> struct VecTraits<float> { static constexpr int VK = 4; typedef float vec_t __attribute__((ext_vector_type(4))); };
+template <> struct VecTraits<double> { static constexpr int VK = 2; typedef double vec_t __attribute__((ext_vector_type(2))); };
+template <> struct VecTraits<int32_t> { static constexpr int VK = 4; typedef int32_t vec_t __attribute__((ext_vector_type(4))); };
+template <> struct VecTraits<int64_t> { static constexpr int VK = 2; typedef int64_t vec_t __attribute__((ext_vector_type(2))); };
+
+// LDS geometry of one operand slab (BMN rows/cols x BK k values).
+template <typename T, int KIND, int BMN, int BK, bool KG = true> struct Slab {
+  static constexpr int VK = VecTraits<T>::VK;
+  static constexpr int LDKG = BMN + 4;   // k-group layout: 16-byte slots per k-group plane
+  static constexpr int LDMN = BMN + 8;   // k-row layout: elements per k row
+  static constexpr int ELEMS = (KIND == kKContig && KG) ? (BK / VK) * LDKG * VK : BK * LDMN;
+};
+
+// Moves one operand slab global -> registers (fetch) -> LDS (commit).
+template <typename T, int KIND, int BMN, int BK, int NT, bool KG = true> struct Loader;
+
+template <typename T, int BMN, int BK, int NT, bool KG> struct Loader<T, kKContig, BMN, BK, NT, KG> {
+  typedef typename VecTraits<T>::vec_t vec_t;
+  static constexpr int VK = VecTraits<T>::VK;
+  static constexpr int QN = BK / VK;               // vectors per row
+  static constexpr int NV = BMN * QN / NT;         // vectors per thread
+  static_assert(BMN * QN % NT == 0 && NV >= 1, "slab must divide evenly over the workgroup");
+  const T* ptr[NV];
+  bool rowok[NV];
+  int64_t K;
+  vec_t reg[NV];
+  __device__ __forceinline__ Loader(const T* X, int64_t ld_mn, int64_t, int64_t mn0, int64_t MN, int64_t K_, int) : K(K_) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = threadIdx.x + i * NT;
+      const int q = v % QN, mn = v / QN;
+      rowok[i] = (mn0 + mn) < MN;
+      ptr[i] = X + (mn0 + mn) * ld_mn + q * VK;
+    }
+  }
+  __device__ __forceinline__ void fetch(int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int q = (threadIdx.x + i * NT) % QN;
+      vec_t z = {};
+      reg[i] = (rowok[i] && (k0 + q * VK) < K) ? *(const vec_t*)(ptr[i] + k0) : z;
+    }
+  }
+  __device__ __forceinline__ void commit(T* lds) const {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = threadIdx.x + i * NT;
+      const int q = v % QN, mn = v / QN;
+      if constexpr (KG) {
+        constexpr int LD = Slab<T, kKContig, BMN, BK, true>::LDKG;
+        *(vec_t*)(lds + (q * LD + mn) * VK) = reg[i];
+      } else {  // k-row layout wanted: scatter the VK k values of this row
+        constexpr int LD = Slab<T, kKContig, BMN, BK, false>::LDMN;
+#pragma unroll
+        for (int s = 0; s < VK; ++s) lds[(q * VK + s) * LD + mn] = reg[i][s];
+      }
+    }
+  }
+};
+
+template <typename T, int BMN, int BK, int NT, bool KG> struct Loader<T, kMNContig, BMN, BK, NT, KG> {
+  typedef typename VecTraits<T>::vec_t vec_t;
+  static constexpr int VK = VecTraits<T>::VK;
+  static constexpr int CN = BMN / VK;              // vectors per k row
+  static constexpr int NV = CN * BK / NT;
+  static_assert(CN * BK % NT == 0 && NV >= 1, "slab must divide evenly over the workgroup");
+  const T* ptr[NV];
+  bool colok[NV];
+  int64_t K, ld_k;
+  vec_t reg[NV];
+  __device__ __forceinline__ Loader(const T* X, int64_t, int64_t ld_k_, int64_t mn0, int64_t MN, int64_t K_, int) : K(K_), ld_k(ld_k_) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = threadIdx.x + i * NT;
+      const int c = v % CN, k = v / CN;
+      colok[i] = (mn0 + c * VK) < MN;
+      ptr[i] = X + (mn0 + c * VK) + k * ld_k;
+    }
+  }
+  __device__ __forceinline__ void fetch(int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int k = (threadIdx.x + i * NT) / CN;
+      vec_t z = {};
+      reg[i] = (colok[i] && (k0 + k) < K) ? *(const vec_t*)(ptr[i] + k0 * ld_k) : z;
+    }
+  }
+  __device__ __forceinline__ void commit(T* lds) const {
+    constexpr int LD = Slab<T, kMNContig, BMN, BK>::LDMN;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = threadIdx.x + i * NT;
+      const int c = v % CN, k = v / CN;
+      *(vec_t*)(lds + k * LD + c * VK) = reg[i];
+    }
+  }
+};
+
+template <typename T, int BMN, int BK, int NT, bool KG> struct Loader<T, kGeneric, BMN, BK, NT, KG> {
+  static constexpr int NE = BMN * BK / NT;         // elements per thread
+  static_assert(BMN * BK % NT == 0 && NE >= 1, "slab must divide evenly over the workgroup");
+  const T* X;
+  int64_t ld_mn, ld_k, mn0, MN, K;
+  int kfast;
+  T reg[NE];
+  __device__ __forceinline__ Loader(const T* X_, int64_t ld_mn_, int64_t ld_k_, int64_t mn0_, int64_t MN_, int64_t K_, int kfast_)
+      : X(X_), ld_mn(ld_mn_), ld_k(ld_k_), mn0(mn0_), MN(MN_), K(K_), kfast(kfast_) {}
+  __device__ __forceinline__ void coords(int i, int& mn, int& k) const {
+    const int e = threadIdx.x + i * NT;
+    if (kfast) { k = e % BK; mn = e / BK; } else { mn = e % BMN; k = e / BMN; }
+  }
+  __device__ __forceinline__ void fetch(int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+      int mn, k;
+      coords(i, mn, k);
+      const bool ok = (mn0 + mn) < MN && (k0 + k) < K;
+      reg[i] = ok ? X[(mn0 + mn) * ld_mn + (k0 + k) * ld_k] : (T)0;
+    }
+  }
+  __device__ __forceinline__ void commit(T* lds) const {
+    constexpr int LD = Slab<T, kGeneric, BMN, BK>::LDMN;
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+      int mn, k;
+      coords(i, mn, k);
+      lds[k * LD + mn] = reg[i];
+    }
+  }
+};
+
+}  // namespace gemm
+}  // namespace am

@@ -1,0 +1,211 @@
+// MFMA GEMM for gfx950 (CDNA4), float32 (v_mfma_f32_32x32x2_f32) and float64
+// (v_mfma_f64_16x16x4_f64). C[MxN] <- alpha * A * B + beta * C with arbitrary element strides
+// on every operand and an optional fused bias / ReLU epilogue.
+//
+// Replaces the reference's CPU blocked GEMM (src/arraymancer/laser/primitives/
+// matrix_multiplication/gemm.nim:117-184: pack B panel, pack A block, micro-kernel) with a
+// GPU decomposition built for 64-wide wavefronts:
+//   * one workgroup per BM x BN tile of C, WAVES_M x WAVES_N wavefronts, each owning a
+//     (BM/WAVES_M) x (BN/WAVES_N) sub-tile as TM x TN MFMA accumulators held in registers
+//     for the whole K loop;
+//   * K is walked in BK-wide slabs, double-buffered in LDS: while the matrix cores work on slab
+//     t, the global loads of slab t+1 are in flight into registers and are written to the other
+//     LDS buffer afterwards (one barrier per slab);
+//   * "packing" (gemm_packing.nim:24-99) becomes the choice of LDS layout per operand, so that
+//     both the global->LDS copy and the LDS->register fragment reads are 16-byte accesses when
+//     the operand has a unit stride in either direction, with no transpose through registers:
+//       - unit stride along k  -> "k-group" layout [k/VK][mn][VK]; a lane reads the VK
+//         consecutive k values of its row with one ds_read_b128;
+//       - unit stride along mn -> "k-row" layout [k][mn]; a lane reads its VK k values with VK
+//         ds_read_b32/b64 (conflict-free: consecutive lanes, consecutive addresses);
+//       - anything else (zero / negative / non-unit strides) -> scalar gathers into the k-row
+//         layout. No host-side copy is ever made (the reference copies non-contiguous float
+//         operands first: src/arraymancer/tensor/private/p_operator_blas_l2l3.nim:151-152).
+//     The MFMA k index is a free permutation as long as A and B agree, which is what lets a
+//     lane own VK consecutive k values: MFMA step s of a KSTEP = VK * (64/TILE) wide k-step
+//     multiplies k = VK*kl + s for lane group kl on both operands.
+//   * out-of-range rows/columns/k are zero-filled on load (the reference zero-pads its packed
+//     panels the same way, gemm_packing.nim:54-55, 98-99) and masked on store.
+#pragma once
+#include "gemm_loader.h"
+
+namespace am {
+namespace gemm {
+
+template <typename T> struct Mfma;
+
+template <> struct Mfma<float> {
+  static constexpr int TILE = 32;  // output tile edge
+  static constexpr int KL = 2;     // lane groups along k (64 / TILE)
+  static constexpr int VK = 4;     // k values per lane per k-step (16 bytes)
+  static constexpr int NACC = 16;  // accumulator registers per lane per tile
+  typedef float acc_t __attribute__((ext_vector_type(16)));
+  typedef float vec_t __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+  // Row of the 32x32 tile held in accumulator register r of `lane` (column = lane % 32).
+  static __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+};
+
+template <> struct Mfma<double> {
+  static constexpr int TILE = 16;
+  static constexpr int KL = 4;
+  static constexpr int VK = 2;
+  static constexpr int NACC = 4;
+  typedef double acc_t __attribute__((ext_vector_type(4)));
+  typedef double vec_t __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+
+// Reads the VK k values that `lane` feeds to the MFMA steps of k-step `ks` for row/col `mn`.
+template <typename T, int KIND, int BMN, int BK>
+__device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, T (&out)[Mfma<T>::VK]) {
+  typedef typename Mfma<T>::vec_t vec_t;
+  constexpr int VK = Mfma<T>::VK, KL = Mfma<T>::KL;
+  if constexpr (KIND == kKContig) {
+    constexpr int LD = Slab<T, KIND, BMN, BK>::LDKG;
+    const vec_t v = *(const vec_t*)(lds + ((ks * KL + kl) * LD + mn) * VK);
+#pragma unroll
+    for (int s = 0; s < VK; ++s) out[s] = v[s];
+  } else {
+    constexpr int LD = Slab<T, KIND, BMN, BK>::LDMN;
+#pragma unroll
+    for (int s = 0; s < VK; ++s) out[s] = lds[((ks * KL + kl) * VK + s) * LD + mn];
+  }
+}
+
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int AK, int BKIND>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p) {
+  typedef Mfma<T> MF;
+  typedef typename MF::acc_t acc_t;
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int TILE = MF::TILE, VK = MF::VK, KL = MF::KL, KSTEP = VK * KL;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / TILE, TN = WN / TILE;
+  static_assert(BK % KSTEP == 0 && WM % TILE == 0 && WN % TILE == 0, "tile shape");
+  constexpr int A_ELEMS = Slab<T, AK, BM, BK>::ELEMS, B_ELEMS = Slab<T, BKIND, BN, BK>::ELEMS;
+
+  __shared__ __attribute__((aligned(16))) T sA[2][A_ELEMS];
+  __shared__ __attribute__((aligned(16))) T sB[2][B_ELEMS];
+
+  // Workgroup -> tile. Hardware deals consecutive workgroup ids round-robin to the 8 XCDs; give
+  // each XCD a contiguous band of tile rows so that its private L2 sees the same A/B panels.
+  int bid = blockIdx.x;
+  const int nb = p.tiles_m * p.tiles_n;
+  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+  const int tile_m = bid / p.tiles_n, tile_n = bid - tile_m * p.tiles_n;
+  const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+  const int lrow = lane % TILE, kl = lane / TILE;
+
+  Loader<T, AK, BM, BK, NT> la(p.A, p.a_mn, p.a_k, m0, p.M, p.K, p.a_kfast);
+  Loader<T, BKIND, BN, BK, NT> lb(p.B, p.b_mn, p.b_k, n0, p.N, p.K, p.b_kfast);
+
+  acc_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < MF::NACC; ++r) acc[i][j][r] = (T)0;
+
+  const int64_t ktiles = (p.K + BK - 1) / BK;
+  la.fetch(0);
+  lb.fetch(0);
+  la.commit(sA[0]);
+  lb.commit(sB[0]);
+  __syncthreads();
+
+  for (int64_t kt = 0; kt < ktiles; ++kt) {
+    const int cur = (int)(kt & 1);
+    const bool more = (kt + 1) < ktiles;
+    if (more) {
+      la.fetch((kt + 1) * BK);
+      lb.fetch((kt + 1) * BK);
+    }
+    const T* a_lds = sA[cur];
+    const T* b_lds = sB[cur];
+#pragma unroll
+    for (int ks = 0; ks < BK / KSTEP; ++ks) {
+      T af[TM][VK], bf[TN][VK];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) read_frag<T, AK, BM, BK>(a_lds, wave_m * WM + i * TILE + lrow, ks, kl, af[i]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) read_frag<T, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[j]);
+#pragma unroll
+      for (int s = 0; s < VK; ++s)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[i][s], bf[j][s], acc[i][j]);
+    }
+    if (more) {
+      la.commit(sA[cur ^ 1]);
+      lb.commit(sB[cur ^ 1]);
+    }
+    __syncthreads();
+  }
+
+  // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
+  // C += alpha * AB, each rounded on its own; then the optional fused bias / ReLU.
+  const T alpha = p.alpha, beta = p.beta;
+  const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
+#pragma unroll
+      for (int r = 0; r < MF::NACC; ++r) {
+        const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
+        if (row < p.M && col < p.N) {
+          T* cp = p.C + row * p.c_m + col * p.c_n;
+          T ab = acc[i][j][r];
+          if (alpha != (T)1) ab = alpha * ab;
+          T v = ab;
+          if (beta != (T)0) {
+            T c = *cp;
+            if (beta != (T)1) c = c * beta;
+            v = c + ab;
+          }
+          if (has_bias) v = v + p.bias[row * p.bias_m + col * p.bias_n];
+          if (relu) v = ((T)0 >= v) ? (T)0 : v;
+          *cp = v;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+static int launch_kinds(Args<T>& g, int ak, int bk) {
+  g.tiles_m = (int)((g.M + BM - 1) / BM);
+  g.tiles_n = (int)((g.N + BN - 1) / BN);
+  const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
+  if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
+  const dim3 grid((unsigned)nb), block(WAVES_M * WAVES_N * 64);
+#define AM_LAUNCH(AKIND, BKIND_)                                                                   \
+  hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, AKIND, BKIND_>), grid, block, 0, \
+                     stream(), g)
+  switch (ak * 3 + bk) {
+    case 0: AM_LAUNCH(kKContig, kKContig); break;
+    case 1: AM_LAUNCH(kKContig, kMNContig); break;
+    case 2: AM_LAUNCH(kKContig, kGeneric); break;
+    case 3: AM_LAUNCH(kMNContig, kKContig); break;
+    case 4: AM_LAUNCH(kMNContig, kMNContig); break;
+    case 5: AM_LAUNCH(kMNContig, kGeneric); break;
+    case 6: AM_LAUNCH(kGeneric, kKContig); break;
+    case 7: AM_LAUNCH(kGeneric, kMNContig); break;
+    default: AM_LAUNCH(kGeneric, kGeneric); break;
+  }
+#undef AM_LAUNCH
+  return check_launch("gemm_mfma");
+}
+
+}  // namespace gemm
+}  // namespace am

@@ -1,0 +1,187 @@
+// Device context, stream, memory and timing entry points of the C ABI.
+#include <mutex>
+#include <stdarg.h>
+#include <string.h>
+#include "common.h"
+
+namespace am {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static std::mutex g_mu;
+static bool g_ready = false;
+static int g_device = -1;
+static hipStream_t g_stream = nullptr;
+static hipDeviceProp_t g_prop;
+
+static int init_locked(int device) {
+  if (g_ready) {
+    if (device == g_device) return AM_OK;
+    return fail(AM_E_ARG, "am_hip_init(%d): library already initialised on device %d", device, g_device);
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0)
+    return fail(AM_E_NODEVICE, "no HIP device available (%s)", e == hipSuccess ? "count = 0" : hipGetErrorString(e));
+  if (device < 0 || device >= count) return fail(AM_E_ARG, "device %d out of range [0, %d)", device, count);
+  AM_HIP_TRY(hipSetDevice(device));
+  AM_HIP_TRY(hipGetDeviceProperties(&g_prop, device));
+  if (strncmp(g_prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(AM_E_NODEVICE, "device %d is %s; this library carries gfx950 code only", device, g_prop.gcnArchName);
+  AM_HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  g_device = device;
+  g_ready = true;
+  return AM_OK;
+}
+
+int ensure_init() {
+  if (g_ready) return AM_OK;
+  std::lock_guard<std::mutex> lk(g_mu);
+  return init_locked(0);
+}
+
+hipStream_t stream() { return g_stream; }
+int num_cus() { return g_ready ? g_prop.multiProcessorCount : 256; }
+
+}  // namespace am
+
+using namespace am;
+
+extern "C" {
+
+const char* am_hip_last_error(void) { return g_err; }
+const char* am_hip_version(void) { return "arraymancer-hip 0.1 (gfx950)"; }
+
+int am_hip_init(int device) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  return init_locked(device);
+}
+
+int am_hip_device_count(int* count) {
+  if (!count) return fail(AM_E_ARG, "am_hip_device_count: null pointer");
+  int c = 0;
+  hipError_t e = hipGetDeviceCount(&c);
+  *count = (e == hipSuccess) ? c : 0;
+  return AM_OK;
+}
+
+int am_hip_device_info(char* name, size_t name_cap, int* compute_units, int* clock_khz,
+                       size_t* hbm_bytes, int* lds_bytes_per_cu) {
+  AM_TRY(ensure_init());
+  if (name && name_cap > 0) {
+    snprintf(name, name_cap, "%s (%s)", g_prop.name, g_prop.gcnArchName);
+  }
+  if (compute_units) *compute_units = g_prop.multiProcessorCount;
+  if (clock_khz) *clock_khz = g_prop.clockRate;
+  if (hbm_bytes) *hbm_bytes = g_prop.totalGlobalMem;
+  if (lds_bytes_per_cu) *lds_bytes_per_cu = (int)g_prop.maxSharedMemoryPerMultiProcessor;
+  return AM_OK;
+}
+
+int am_hip_malloc(size_t bytes, void** out) {
+  if (!out) return fail(AM_E_ARG, "am_hip_malloc: null out pointer");
+  *out = nullptr;
+  if (bytes == 0) return AM_OK;
+  AM_TRY(ensure_init());
+  hipError_t e = hipMalloc(out, bytes);
+  if (e != hipSuccess) {
+    *out = nullptr;
+    (void)hipGetLastError();
+    return fail(AM_E_ALLOC, "hipMalloc(%zu bytes) failed: %s", bytes, hipGetErrorString(e));
+  }
+  return AM_OK;
+}
+
+int am_hip_free(void* dptr) {
+  if (!dptr) return AM_OK;
+  AM_TRY(ensure_init());
+  // Work that still reads or writes the buffer is on the library stream: drain it first.
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  AM_HIP_TRY(hipFree(dptr));
+  return AM_OK;
+}
+
+int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return AM_OK;
+  if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_h2d: null pointer");
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  return AM_OK;
+}
+
+int am_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return AM_OK;
+  if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_d2h: null pointer");
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  return AM_OK;
+}
+
+int am_hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return AM_OK;
+  if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_d2d: null pointer");
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+  return AM_OK;
+}
+
+int am_hip_memset(void* dst, int byte_value, size_t bytes) {
+  if (bytes == 0) return AM_OK;
+  if (!dst) return fail(AM_E_ARG, "am_hip_memset: null pointer");
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipMemsetAsync(dst, byte_value, bytes, g_stream));
+  return AM_OK;
+}
+
+int am_hip_sync(void) {
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  return AM_OK;
+}
+
+void* am_hip_stream(void) {
+  if (ensure_init() != AM_OK) return nullptr;
+  return (void*)g_stream;
+}
+
+int am_hip_event_create(void** ev) {
+  if (!ev) return fail(AM_E_ARG, "am_hip_event_create: null pointer");
+  AM_TRY(ensure_init());
+  hipEvent_t e;
+  AM_HIP_TRY(hipEventCreate(&e));
+  *ev = (void*)e;
+  return AM_OK;
+}
+
+int am_hip_event_record(void* ev) {
+  if (!ev) return fail(AM_E_ARG, "am_hip_event_record: null event");
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipEventRecord((hipEvent_t)ev, g_stream));
+  return AM_OK;
+}
+
+int am_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!start || !stop || !ms) return fail(AM_E_ARG, "am_hip_event_elapsed_ms: null pointer");
+  AM_TRY(ensure_init());
+  AM_HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+  AM_HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return AM_OK;
+}
+
+int am_hip_event_destroy(void* ev) {
+  if (!ev) return AM_OK;
+  AM_HIP_TRY(hipEventDestroy((hipEvent_t)ev));
+  return AM_OK;
+}
+
+}  // extern "C"

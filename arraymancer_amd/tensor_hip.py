@@ -1,0 +1,469 @@
+"""`HipTensor`: the host-side mirror of the reference's GPU tensor backends for the GEMM +
+broadcast/map hot path, on top of the C ABI of libam_hip.so.
+
+It occupies the slot of `CudaTensor` (src/arraymancer/tensor/data_structure.nim:29-67): a shape /
+strides / offset view over reference-counted device storage, with the same operator set
+(src/arraymancer/tensor/operators_blas_l2l3_cuda.nim, operators_blas_l1_cuda.nim,
+operators_broadcasted_cuda.nim, shapeshifting_cuda.nim, init_cuda.nim), extended to the four
+element types of the CPU path (float32, float64, int32, int64) and to arbitrary strides.
+
+Reference operator          here
+  t.cuda / t.cpu            toHip(ndarray) / t.toCpu()
+  a * b (matrices)          a * b          (also a @ b);   gemm(alpha, A, B, beta, C)
+  a + b, a - b, +=, -=      same
+  t * s, s * t, t / s       same (scalar s)
+  a +. b  a -. b  a *. b  a /. b  a mod b      bc_add / bc_sub / bc_mul / bc_div / bc_mod  (OPERATORS["+."] ...)
+  a +.= b ... (rhs broadcast only)              a.bc_iadd(b) / bc_isub / bc_imul / bc_idiv
+  map2_inline(a, b, <expr>)                     map2(op_name, a, b) for the enumerated bodies
+  t.transpose, t[slices], t.broadcast(shape)    same, metadata only
+Python has no `+.` token, hence the names; the argument order and error behaviour follow the
+reference (ValueError for shape mismatches, IndexError for matrix dimension mismatches).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence
+
+import numpy as np
+
+from . import _lib
+from . import metadata as md
+from ._lib import CTYPE, EPI, OP, SFX, UOP, check, i64_array
+from .metadata import Layout, Step
+
+
+class HipStorage:
+    """Owns one device allocation; freed when the last view goes away
+    (the reference frees in the ref-tracker's destructor, data_structure.nim:60-67)."""
+
+    __slots__ = ("ptr", "nelems", "itemsize", "__weakref__")
+
+    def __init__(self, nelems: int, itemsize: int):
+        L = _lib.load()
+        out = ctypes.c_void_p()
+        check(L.am_hip_malloc(ctypes.c_size_t(nelems * itemsize), ctypes.byref(out)))
+        self.ptr = out.value or 0
+        self.nelems = nelems
+        self.itemsize = itemsize
+
+    def __del__(self):
+        ptr, self.ptr = getattr(self, "ptr", 0), 0
+        if ptr:
+            try:
+                _lib.load().am_hip_free(ctypes.c_void_p(ptr))
+            except Exception:  # interpreter shutdown
+                pass
+
+
+def _dtype_sfx(dtype) -> str:
+    try:
+        return SFX[np.dtype(dtype)]
+    except KeyError:
+        raise TypeError(f"HipTensor supports float32, float64, int32 and int64, not {dtype}")
+
+
+class HipTensor:
+    __slots__ = ("layout", "storage", "dtype")
+
+    def __init__(self, layout: Layout, storage: HipStorage, dtype):
+        self.layout = layout
+        self.storage = storage
+        self.dtype = np.dtype(dtype)
+
+    # ------------------------------------------------------------------ metadata
+    @property
+    def shape(self):
+        return self.layout.shape
+
+    @property
+    def strides(self):
+        return self.layout.strides
+
+    @property
+    def offset(self):
+        return self.layout.offset
+
+    @property
+    def rank(self):
+        return self.layout.rank
+
+    @property
+    def size(self):
+        return self.layout.size
+
+    @property
+    def sfx(self) -> str:
+        return SFX[self.dtype]
+
+    def data_ptr(self) -> int:
+        """Device address of element [0, 0, ...] (get_offset_ptr, data_structure.nim:206-211)."""
+        return self.storage.ptr + self.layout.offset * self.dtype.itemsize
+
+    def is_C_contiguous(self):
+        return md.is_C_contiguous(self.layout)
+
+    def is_F_contiguous(self):
+        return md.is_F_contiguous(self.layout)
+
+    def isContiguous(self):
+        return self.is_C_contiguous() or self.is_F_contiguous()
+
+    def __repr__(self):
+        return f"HipTensor[{self.dtype}](shape={list(self.shape)}, strides={list(self.strides)}, offset={self.offset})"
+
+    # ------------------------------------------------------------------ views (no data movement)
+    def transpose(self) -> "HipTensor":
+        return HipTensor(md.transpose(self.layout), self.storage, self.dtype)
+
+    @property
+    def T(self):
+        return self.transpose()
+
+    def __getitem__(self, key) -> "HipTensor":
+        return HipTensor(md.py_index(self.layout, key), self.storage, self.dtype)
+
+    def slice_(self, *steps: Step) -> "HipTensor":
+        """Slicing in the reference's notation: Step(first, last, step) with inclusive ends."""
+        return HipTensor(md.slicer(self.layout, steps), self.storage, self.dtype)
+
+    def broadcast(self, shape: Sequence[int]) -> "HipTensor":
+        return HipTensor(md.broadcast(self.layout, shape), self.storage, self.dtype)
+
+    bc = broadcast
+
+    def reshape(self, *shape) -> "HipTensor":
+        if len(shape) == 1 and not isinstance(shape[0], int):
+            shape = tuple(shape[0])
+        n = 1
+        for s in shape:
+            n *= s
+        if n != self.size:
+            raise ValueError(f"The total number of elements in the old ({self.size}) and the new ({n}) "
+                             f"reshaped tensor must be the same")
+        src = self if self.is_C_contiguous() else self.clone()
+        lay = md.contiguous(shape)
+        return HipTensor(Layout(lay.shape, lay.strides, src.layout.offset), src.storage, self.dtype)
+
+    # ------------------------------------------------------------------ transfers and copies
+    def toCpu(self) -> np.ndarray:
+        """Blocking copy back. Like the reference's `cpu` (init_cuda.nim:43-59) the whole storage
+        is copied and shape / strides / offset are kept, so the result is the same view of the
+        same bytes (a NumPy strided view here)."""
+        host = np.empty(self.storage.nelems, dtype=self.dtype)
+        if self.storage.nelems:
+            check(_lib.load().am_hip_memcpy_d2h(host.ctypes.data, ctypes.c_void_p(self.storage.ptr),
+                                                ctypes.c_size_t(host.nbytes)))
+        if self.size == 0:
+            return np.empty(self.shape, dtype=self.dtype)
+        it = self.dtype.itemsize
+        lo, hi = md.extent_in_storage(self.layout)
+        assert 0 <= lo and hi < self.storage.nelems
+        return np.lib.stride_tricks.as_strided(host[self.layout.offset:], shape=self.shape,
+                                               strides=tuple(s * it for s in self.strides))
+
+    def clone(self) -> "HipTensor":
+        """Fresh C-contiguous copy (device-side strided gather)."""
+        out = empty(self.shape, self.dtype)
+        _unary_into("copy", out, self)
+        return out
+
+    def asContiguous(self) -> "HipTensor":
+        return self if self.is_C_contiguous() else self.clone()
+
+    # ------------------------------------------------------------------ operators
+    def __mul__(self, other):
+        if isinstance(other, HipTensor):
+            return matmul(self, other)
+        return scalar_op("mul", self, other)
+
+    def __rmul__(self, other):
+        return scalar_op("mul", self, other, scalar_on_left=True)
+
+    __matmul__ = lambda self, other: matmul(self, other)
+
+    def __truediv__(self, other):
+        if isinstance(other, HipTensor):
+            raise TypeError("tensor / tensor is spelled bc_div (`/.`)")
+        return scalar_op("div", self, other)
+
+    def __add__(self, other):
+        _check_elementwise(self, other)
+        return map2("add", self, other)
+
+    def __sub__(self, other):
+        _check_elementwise(self, other)
+        return map2("sub", self, other)
+
+    def __iadd__(self, other):
+        _check_elementwise(self, other)
+        _binary_into("add", self, self, other)
+        return self
+
+    def __isub__(self, other):
+        _check_elementwise(self, other)
+        _binary_into("sub", self, self, other)
+        return self
+
+    def __imul__(self, scalar):
+        _scalar_into("mul", self, self, scalar, False)
+        return self
+
+    def __itruediv__(self, scalar):
+        _scalar_into("div", self, self, scalar, False)
+        return self
+
+    def __neg__(self):
+        return unary("neg", self)
+
+    # in-place broadcast forms: only the right-hand side may be broadcast
+    # (src/arraymancer/tensor/operators_broadcasted.nim:65-102)
+    def bc_iadd(self, other):
+        return _bc_inplace("add", self, other)
+
+    def bc_isub(self, other):
+        return _bc_inplace("sub", self, other)
+
+    def bc_imul(self, other):
+        return _bc_inplace("mul", self, other)
+
+    def bc_idiv(self, other):
+        return _bc_inplace("div", self, other)
+
+
+# ---------------------------------------------------------------------- construction
+def empty(shape: Sequence[int], dtype) -> HipTensor:
+    """newTensorUninit on the device: row-major, uninitialised."""
+    dtype = np.dtype(dtype)
+    _dtype_sfx(dtype)
+    lay = md.contiguous(shape)
+    return HipTensor(lay, HipStorage(lay.size, dtype.itemsize), dtype)
+
+
+def zeros(shape: Sequence[int], dtype) -> HipTensor:
+    t = empty(shape, dtype)
+    if t.size:
+        check(_lib.load().am_hip_memset(ctypes.c_void_p(t.storage.ptr), 0,
+                                        ctypes.c_size_t(t.size * t.dtype.itemsize)))
+    return t
+
+
+def toHip(arr) -> HipTensor:
+    """Host -> device. Row-major on the device, like CPU tensors (the CUDA backend's forced
+    column-major copy, init_cuda.nim:31, is not kept). A non-contiguous ndarray is packed on
+    the host first; strided device views are made with transpose / slicing on the HipTensor."""
+    arr = np.asarray(arr)
+    _dtype_sfx(arr.dtype)
+    host = np.ascontiguousarray(arr)
+    t = empty(host.shape, host.dtype)
+    if host.size:
+        check(_lib.load().am_hip_memcpy_h2d(ctypes.c_void_p(t.storage.ptr), host.ctypes.data,
+                                            ctypes.c_size_t(host.nbytes)))
+    return t
+
+
+def sync() -> None:
+    check(_lib.load().am_hip_sync())
+
+
+# ---------------------------------------------------------------------- checks
+def _same_dtype(*ts):
+    d = ts[0].dtype
+    for t in ts[1:]:
+        if t.dtype != d:
+            raise TypeError(f"element types differ: {d} and {t.dtype}")
+    return d
+
+
+def _check_elementwise(a: HipTensor, b: HipTensor):
+    """check_elementwise (src/arraymancer/tensor/private/p_checks.nim:59-62)."""
+    if not isinstance(b, HipTensor):
+        raise TypeError("operand must be a HipTensor")
+    if a.shape != b.shape:
+        raise ValueError(f"Both Tensors should have the same shape. Left-hand side has shape "
+                         f"{list(a.shape)} while right-hand side has shape {list(b.shape)}")
+
+
+# ---------------------------------------------------------------------- GEMM
+def gemm(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none", bias: HipTensor | None = None):
+    """C <- alpha * A * B + beta * C in place (C may be any non-overlapping strided view).
+    src/arraymancer/tensor/operators_blas_l2l3.nim:58-81. Optional fused epilogue
+    ("bias", "relu", "bias_relu") with `bias` broadcastable to C's shape (float types)."""
+    dtype = _same_dtype(A, B, C)
+    if A.rank != 2 or B.rank != 2 or C.rank != 2:
+        raise ValueError("gemm: A, B and C must be matrices")
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2:   # check_matmat raises IndexDefect, src/arraymancer/tensor/private/p_checks.nim:159-167
+        raise IndexError(f"Number of columns in the first matrix: {K}, must be the same as the number "
+                         f"of rows in the second matrix: {K2}")
+    if C.shape != (M, N):
+        raise IndexError(f"gemm: C has shape {list(C.shape)}, expected {[M, N]}")
+    L = _lib.load()
+    sfx = C.sfx
+    ct = CTYPE[sfx]
+    args = [M, N, K, ct(alpha), ctypes.c_void_p(A.data_ptr()), A.strides[0], A.strides[1],
+            ctypes.c_void_p(B.data_ptr()), B.strides[0], B.strides[1], ct(beta),
+            ctypes.c_void_p(C.data_ptr()), C.strides[0], C.strides[1]]
+    epi = EPI[epilogue] if isinstance(epilogue, str) else int(epilogue)
+    if epi != 0:
+        if sfx not in ("f32", "f64"):
+            raise TypeError("fused epilogues are defined for float tensors")
+        bptr, brs, bcs = None, 0, 0
+        if epi & 1:
+            if bias is None:
+                raise ValueError("bias epilogue needs a bias tensor")
+            _same_dtype(C, bias)
+            bb = bias.broadcast((M, N))
+            bptr, brs, bcs = ctypes.c_void_p(bb.data_ptr()), bb.strides[0], bb.strides[1]
+        check(getattr(L, f"am_hip_gemm_ex_{sfx}")(*args, epi, bptr, brs, bcs))
+    else:
+        check(getattr(L, f"am_hip_gemm_{sfx}")(*args))
+    return C
+
+
+def matmul(a: HipTensor, b: HipTensor) -> HipTensor:
+    """`*` (src/arraymancer/tensor/operators_blas_l2l3.nim:88-100): matrix-matrix, or
+    matrix-vector (run as an N = 1 product); anything else is a ValueError."""
+    _same_dtype(a, b)
+    if a.rank == 2 and b.rank == 2:
+        if a.shape[1] != b.shape[0]:
+            raise IndexError(f"Number of columns in the first matrix: {a.shape[1]}, must be the same as the "
+                             f"number of rows in the second matrix: {b.shape[0]}")
+        out = empty((a.shape[0], b.shape[1]), a.dtype)
+        return gemm(1, a, b, 0, out)
+    if a.rank == 2 and b.rank == 1:
+        if a.shape[1] != b.shape[0]:
+            raise IndexError(f"Number of columns in the matrix: {a.shape[1]}, must be the same as the "
+                             f"number of rows in the vector: {b.shape[0]}")
+        out = empty((a.shape[0],), a.dtype)
+        bcol = HipTensor(Layout((b.shape[0], 1), (b.strides[0], 1), b.offset), b.storage, b.dtype)
+        ocol = HipTensor(Layout((a.shape[0], 1), (1, 1), 0), out.storage, out.dtype)
+        gemm(1, a, bcol, 0, ocol)
+        return out
+    raise ValueError("Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a "
+                     "Matrix and second is a Matrix or Vector")
+
+
+def linear(x: HipTensor, weight: HipTensor, bias: HipTensor | None = None, relu: bool = False) -> HipTensor:
+    """out = x * weight.transpose (+ bias) (then ReLU) in ONE kernel — the three passes of
+    src/arraymancer/nn_primitives/nnp_linear.nim:20-29 + nnp_activation.nim:35-36 fused into the
+    GEMM epilogue. weight is [out_features, in_features], bias [1, out_features]."""
+    out = empty((x.shape[0], weight.shape[0]), x.dtype)
+    epi = ("bias_relu" if relu else "bias") if bias is not None else ("relu" if relu else "none")
+    return gemm(1, x, weight.transpose(), 0, out, epilogue=epi, bias=bias)
+
+
+# ---------------------------------------------------------------------- element-wise
+def _binary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor):
+    sfx = dst.sfx
+    code = OP[op] if isinstance(op, str) else int(op)
+    check(getattr(_lib.load(), f"am_hip_ew_binary_{sfx}")(
+        code, dst.rank, i64_array(dst.shape),
+        ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
+        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides),
+        ctypes.c_void_p(b.data_ptr()), i64_array(b.strides)))
+
+
+def _scalar_into(op, dst: HipTensor, a: HipTensor, scalar, left: bool):
+    sfx = dst.sfx
+    code = OP[op] if isinstance(op, str) else int(op)
+    check(getattr(_lib.load(), f"am_hip_ew_scalar_{sfx}")(
+        code, int(bool(left)), dst.rank, i64_array(dst.shape),
+        ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
+        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides), CTYPE[sfx](scalar)))
+
+
+def _unary_into(op, dst: HipTensor, a: HipTensor):
+    sfx = dst.sfx
+    code = UOP[op] if isinstance(op, str) else int(op)
+    check(getattr(_lib.load(), f"am_hip_ew_unary_{sfx}")(
+        code, dst.rank, i64_array(dst.shape),
+        ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
+        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides)))
+
+
+def map2(op, a: HipTensor, b: HipTensor) -> HipTensor:
+    """map2_inline with one of the enumerated bodies: fresh C-contiguous result; operands must
+    already have equal shapes (src/arraymancer/tensor/higher_order_applymap.nim:92-120)."""
+    _same_dtype(a, b)
+    _check_elementwise(a, b)
+    out = empty(a.shape, a.dtype)
+    _binary_into(op, out, a, b)
+    return out
+
+
+def apply2(op, dest: HipTensor, src: HipTensor) -> HipTensor:
+    """apply2_inline: dest[i] = op(dest[i], src[i]) through dest's own strides (:40-47)."""
+    _same_dtype(dest, src)
+    _check_elementwise(dest, src)
+    _binary_into(op, dest, dest, src)
+    return dest
+
+
+def _bc(op, a: HipTensor, b: HipTensor) -> HipTensor:
+    _same_dtype(a, b)
+    la, lb = md.broadcast2(a.layout, b.layout)
+    return map2(op, HipTensor(la, a.storage, a.dtype), HipTensor(lb, b.storage, b.dtype))
+
+
+def bc_add(a, b): return _bc_or_scalar("add", a, b)
+def bc_sub(a, b): return _bc_or_scalar("sub", a, b)
+def bc_mul(a, b): return _bc_or_scalar("mul", a, b)
+def bc_div(a, b): return _bc_or_scalar("div", a, b)
+def bc_mod(a, b): return _bc_or_scalar("mod", a, b)
+
+
+def _bc_or_scalar(op, a, b):
+    """`+.` and friends: tensor-tensor with implicit broadcasting, tensor-scalar, scalar-tensor
+    (src/arraymancer/tensor/operators_broadcasted.nim:28-60, 107-161)."""
+    ta, tb = isinstance(a, HipTensor), isinstance(b, HipTensor)
+    if ta and tb:
+        return _bc(op, a, b)
+    if ta:
+        return scalar_op(op, a, b)
+    if tb:
+        return scalar_op(op, b, a, scalar_on_left=True)
+    raise TypeError("at least one operand must be a HipTensor")
+
+
+def _bc_inplace(op, a: HipTensor, b):
+    if not isinstance(b, HipTensor):
+        _scalar_into(op, a, a, b, False)
+        return a
+    _same_dtype(a, b)
+    bb = b.broadcast(a.shape)
+    _binary_into(op, a, a, bb)
+    return a
+
+
+def scalar_op(op, t: HipTensor, scalar, scalar_on_left: bool = False) -> HipTensor:
+    out = empty(t.shape, t.dtype)
+    if t.size:
+        _scalar_into(op, out, t, scalar, scalar_on_left)
+    return out
+
+
+def unary(op, t: HipTensor) -> HipTensor:
+    out = empty(t.shape, t.dtype)
+    if t.size:
+        _unary_into(op, out, t)
+    return out
+
+
+def relu(t: HipTensor) -> HipTensor:
+    """src/arraymancer/nn_primitives/nnp_activation.nim:35-36."""
+    return unary("relu", t)
+
+
+def sigmoid(t: HipTensor) -> HipTensor:
+    return unary("sigmoid", t)
+
+
+def bias_relu(x: HipTensor, b: HipTensor) -> HipTensor:
+    """map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass."""
+    return _bc("add_relu", x, b)
+
+
+OPERATORS = {"+.": bc_add, "-.": bc_sub, "*.": bc_mul, "/.": bc_div, "mod": bc_mod,
+             "+.=": HipTensor.bc_iadd, "-.=": HipTensor.bc_isub, "*.=": HipTensor.bc_imul,
+             "/.=": HipTensor.bc_idiv}

@@ -1,0 +1,228 @@
+/*
+ * am_hip.h — C ABI of libam_hip.so, the MI355X (gfx950) backend for Arraymancer's
+ * GEMM + broadcast/map hot path.
+ *
+ * Everything here is plain C: device pointers are `void*`/`T*` obtained from
+ * am_hip_malloc, sizes and strides are int64_t counted in ELEMENTS (as in the
+ * reference's Tensor metadata, src/arraymancer/laser/tensor/datatypes.nim:19-48),
+ * and every entry point returns an int status (0 = AM_OK, negative = error; the text of
+ * the last error of the calling thread is available from am_hip_last_error()).
+ *
+ * All work is enqueued on one library-owned HIP stream; results are visible to the host
+ * after am_hip_sync() or any am_hip_memcpy_d2h(). The library keeps no caller pointer
+ * after a call returns. One host thread at a time may call into the library (the
+ * reference's GPU backends have the same contract:
+ * src/arraymancer/tensor/backend/cuda_global_state.nim:21-39).
+ *
+ * "Reference" citations below are paths under the Arraymancer source tree.
+ */
+#ifndef AM_HIP_H
+#define AM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------------------------------------------------------------- status codes */
+#define AM_OK          0
+#define AM_E_ARG      (-1)  /* null pointer, negative size, rank outside 0..6, unknown op      */
+#define AM_E_SHAPE    (-2)  /* shapes/strides that the operation cannot accept                  */
+#define AM_E_DTYPE    (-3)  /* op not defined for this element type (e.g. tanh on int32)        */
+#define AM_E_ALLOC    (-4)  /* device allocation failed                                         */
+#define AM_E_HIP      (-5)  /* a HIP runtime call failed; see am_hip_last_error()               */
+#define AM_E_NODEVICE (-6)  /* no usable gfx950 device                                          */
+
+#define AM_MAXRANK 6        /* LASER_MAXRANK, src/arraymancer/laser/dynamic_stack_arrays.nim:6  */
+
+/* ---------------------------------------------------------------- runtime
+ * Replaces the CUDA backend's global state + memory glue:
+ *   src/arraymancer/tensor/backend/cuda_global_state.nim:21-39 (stream/handle creation)
+ *   src/arraymancer/tensor/backend/cuda.nim:23-57            (cudaMalloc / deallocCuda)
+ *   src/arraymancer/tensor/init_cuda.nim:23-59               (H2D async copy, D2H blocking copy)
+ */
+const char* am_hip_last_error(void);
+const char* am_hip_version(void);
+
+/* Select and initialise `device` (>= 0). Idempotent; called lazily with device 0 by every
+ * other entry point if the caller never calls it. */
+int am_hip_init(int device);
+int am_hip_device_count(int* count);
+/* name: caller buffer of name_cap bytes (NUL terminated on return); any out pointer may be NULL. */
+int am_hip_device_info(char* name, size_t name_cap, int* compute_units, int* clock_khz,
+                       size_t* hbm_bytes, int* lds_bytes_per_cu);
+
+int am_hip_malloc(size_t bytes, void** out);   /* bytes == 0 -> *out = NULL, AM_OK */
+int am_hip_free(void* dptr);                   /* NULL is a no-op */
+int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes);  /* host buffer reusable on return */
+int am_hip_memcpy_d2h(void* dst, const void* src, size_t bytes);  /* blocking, ordered after prior work */
+int am_hip_memcpy_d2d(void* dst, const void* src, size_t bytes);  /* stream ordered */
+int am_hip_memset(void* dst, int byte_value, size_t bytes);       /* stream ordered */
+int am_hip_sync(void);
+/* The library's hipStream_t as an opaque pointer (for callers that enqueue their own work). */
+void* am_hip_stream(void);
+
+/* Timing on the library stream (HIP events). */
+int am_hip_event_create(void** ev);
+int am_hip_event_record(void* ev);
+int am_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* synchronises on `stop` */
+int am_hip_event_destroy(void* ev);
+
+/* ---------------------------------------------------------------- GEMM
+ * C[M x N] <- alpha * A[M x K] * B[K x N] + beta * C, element X[r,c] = X[r*rsX + c*csX].
+ *
+ * Replaces laser `gemm_strided`
+ *   src/arraymancer/laser/primitives/matrix_multiplication/gemm.nim:192-201 (signature)
+ *   gemm.nim:117-184 (loop nest), gemm_ukernel_generic.nim:53-125 (epilogues)
+ * and what reaches it through the Tensor API:
+ *   src/arraymancer/tensor/operators_blas_l2l3.nim:58-100 (`*`, gemm)
+ *   src/arraymancer/tensor/private/p_operator_blas_l2l3.nim:110-215.
+ *
+ * Semantics kept from the reference:
+ *   - pointers already include the tensor offset; strides are in elements and may be
+ *     zero or negative for A and B (views, broadcast, reversed slices). No host copy is made.
+ *   - beta == 0 overwrites C (old NaN/Inf in C never propagate); beta is applied once.
+ *   - alpha == 0 is not special-cased (NaN/Inf in A or B propagate).
+ *   - K == 0 (or M == 0 or N == 0) leaves C untouched, beta is NOT applied.
+ *   - integer types wrap modulo 2^32 / 2^64.
+ * C must not overlap itself (no zero stride on a dimension of extent > 1) nor A or B.
+ */
+int am_hip_gemm_f32(int64_t M, int64_t N, int64_t K, float alpha,
+                    const float* A, int64_t rsA, int64_t csA,
+                    const float* B, int64_t rsB, int64_t csB,
+                    float beta, float* C, int64_t rsC, int64_t csC);
+int am_hip_gemm_f64(int64_t M, int64_t N, int64_t K, double alpha,
+                    const double* A, int64_t rsA, int64_t csA,
+                    const double* B, int64_t rsB, int64_t csB,
+                    double beta, double* C, int64_t rsC, int64_t csC);
+int am_hip_gemm_i32(int64_t M, int64_t N, int64_t K, int32_t alpha,
+                    const int32_t* A, int64_t rsA, int64_t csA,
+                    const int32_t* B, int64_t rsB, int64_t csB,
+                    int32_t beta, int32_t* C, int64_t rsC, int64_t csC);
+int am_hip_gemm_i64(int64_t M, int64_t N, int64_t K, int64_t alpha,
+                    const int64_t* A, int64_t rsA, int64_t csA,
+                    const int64_t* B, int64_t rsB, int64_t csB,
+                    int64_t beta, int64_t* C, int64_t rsC, int64_t csC);
+
+/* GEMM with a fused element-wise epilogue:
+ *   C <- act( alpha*A*B + beta*C + bias ),  bias[r,c] = bias[r*bias_rs + c*bias_cs]
+ * (bias_rs = 0, bias_cs = 1 is the [1,N] row vector of `linear`).
+ * Fuses the three passes of the reference's dense layer
+ *   src/arraymancer/nn_primitives/nnp_linear.nim:20-29 (gemm, then `+.=` bias)
+ *   src/arraymancer/nn_primitives/nnp_activation.nim:35-36 (relu = max(0, x))
+ * at the spot the reference marks for it (gemm_ukernel_generic.nim:50-51,78-79; gemm.nim:204).
+ */
+#define AM_EPI_NONE      0
+#define AM_EPI_BIAS      1   /* + bias                      */
+#define AM_EPI_RELU      2   /* (0 >= x) ? 0 : x            */
+#define AM_EPI_BIAS_RELU 3   /* relu(x + bias)              */
+int am_hip_gemm_ex_f32(int64_t M, int64_t N, int64_t K, float alpha,
+                       const float* A, int64_t rsA, int64_t csA,
+                       const float* B, int64_t rsB, int64_t csB,
+                       float beta, float* C, int64_t rsC, int64_t csC,
+                       int epilogue, const float* bias, int64_t bias_rs, int64_t bias_cs);
+int am_hip_gemm_ex_f64(int64_t M, int64_t N, int64_t K, double alpha,
+                       const double* A, int64_t rsA, int64_t csA,
+                       const double* B, int64_t rsB, int64_t csB,
+                       double beta, double* C, int64_t rsC, int64_t csC,
+                       int epilogue, const double* bias, int64_t bias_rs, int64_t bias_cs);
+
+/* ---------------------------------------------------------------- element-wise / broadcast / map
+ * dst[i] = op(a[i], b[i]) over a common `shape` of `rank` dims (0 <= rank <= 6); each operand
+ * is traversed in C order through its own strides (elements; 0 = broadcast, negative allowed
+ * for inputs). `shape` and the stride arrays are HOST arrays of `rank` entries, passed to the
+ * kernel by value (the CUDA backend cudaMallocs them on every call:
+ * src/arraymancer/tensor/backend/cuda.nim:102-132).
+ *
+ * One entry point covers both reference families:
+ *   map2_inline  (src/arraymancer/tensor/higher_order_applymap.nim:92-120): dst = fresh
+ *                contiguous tensor; behind `+` `-` (operators_blas_l1.nim:44-51) and
+ *                `+.` `-.` `*.` `/.` `mod` (operators_broadcasted.nim:28-60) after
+ *                broadcast2 (private/p_shapeshifting.nim:96-134);
+ *   apply2_inline (higher_order_applymap.nim:40-47): dst == a with a's own strides; behind
+ *                `+=` `-=` (operators_blas_l1.nim:53-61) and `+.=` `-.=` `*.=` `/.=`
+ *                (operators_broadcasted.nim:65-102).
+ * GPU precedent: cuda_apply3 / cuda_apply2
+ *   (src/arraymancer/tensor/private/incl_higher_order_cuda.nim:31-119).
+ * dst may alias a or b exactly (same pointer, same strides); any other overlap is undefined.
+ * dst must not have a zero stride on a dimension of extent > 1.
+ */
+#define AM_OP_ADD         0
+#define AM_OP_SUB         1
+#define AM_OP_MUL         2
+#define AM_OP_DIV         3   /* floats: IEEE /; integers: truncating `div`; x div 0 -> 0 on device */
+#define AM_OP_MOD         4   /* integers only: C `%` (sign of dividend), x mod 0 -> 0 on device     */
+#define AM_OP_ADD_RELU    5   /* t = a + b; (0 >= t) ? 0 : t        (fused bias + ReLU)              */
+#define AM_OP_ADD_SIGMOID 6   /* floats: 1 / (1 + exp(-(a + b)))    (GRU gates, nnp_gru.nim:78)      */
+#define AM_OP_ADD_TANH    7   /* floats: tanh(a + b)                                                */
+#define AM_OP_RELU_BWD    8   /* (a <= 0) ? 0 : b                   (nnp_activation.nim:61-74)       */
+#define AM_OP_MAX         9
+#define AM_OP_MIN        10
+#define AM_OP_BINARY_COUNT 11
+
+int am_hip_ew_binary_f32(int op, int rank, const int64_t* shape,
+                         float* dst, const int64_t* dst_strides,
+                         const float* a, const int64_t* a_strides,
+                         const float* b, const int64_t* b_strides);
+int am_hip_ew_binary_f64(int op, int rank, const int64_t* shape,
+                         double* dst, const int64_t* dst_strides,
+                         const double* a, const int64_t* a_strides,
+                         const double* b, const int64_t* b_strides);
+int am_hip_ew_binary_i32(int op, int rank, const int64_t* shape,
+                         int32_t* dst, const int64_t* dst_strides,
+                         const int32_t* a, const int64_t* a_strides,
+                         const int32_t* b, const int64_t* b_strides);
+int am_hip_ew_binary_i64(int op, int rank, const int64_t* shape,
+                         int64_t* dst, const int64_t* dst_strides,
+                         const int64_t* a, const int64_t* a_strides,
+                         const int64_t* b, const int64_t* b_strides);
+
+/* dst[i] = scalar_on_left ? op(scalar, a[i]) : op(a[i], scalar); ops AM_OP_ADD..AM_OP_MOD,
+ * AM_OP_MAX, AM_OP_MIN. Replaces the tensor-scalar forms
+ *   src/arraymancer/tensor/operators_broadcasted.nim:107-194, operators_blas_l1.nim:66-136
+ * (GPU precedent: cuda_apply_rscal / _lscal / _scal, incl_higher_order_cuda.nim:121-229).
+ * dst may alias a exactly (the in-place `+.=`, `*=` ... forms). */
+int am_hip_ew_scalar_f32(int op, int scalar_on_left, int rank, const int64_t* shape,
+                         float* dst, const int64_t* dst_strides,
+                         const float* a, const int64_t* a_strides, float scalar);
+int am_hip_ew_scalar_f64(int op, int scalar_on_left, int rank, const int64_t* shape,
+                         double* dst, const int64_t* dst_strides,
+                         const double* a, const int64_t* a_strides, double scalar);
+int am_hip_ew_scalar_i32(int op, int scalar_on_left, int rank, const int64_t* shape,
+                         int32_t* dst, const int64_t* dst_strides,
+                         const int32_t* a, const int64_t* a_strides, int32_t scalar);
+int am_hip_ew_scalar_i64(int op, int scalar_on_left, int rank, const int64_t* shape,
+                         int64_t* dst, const int64_t* dst_strides,
+                         const int64_t* a, const int64_t* a_strides, int64_t scalar);
+
+/* dst[i] = op(a[i]). AM_UOP_COPY is the strided gather behind `clone` / `asContiguous`
+ * (src/arraymancer/tensor/shapeshifting.nim:38-57; CUDA: shapeshifting_cuda.nim:34-66).
+ * map_inline / apply_inline: src/arraymancer/tensor/higher_order_applymap.nim:27-32,69-90;
+ * relu: nn_primitives/nnp_activation.nim:35-36; sigmoid: nn_primitives/private/p_activation.nim:17-18. */
+#define AM_UOP_COPY    0
+#define AM_UOP_NEG     1
+#define AM_UOP_RELU    2   /* (0 >= x) ? 0 : x */
+#define AM_UOP_SIGMOID 3   /* floats only      */
+#define AM_UOP_TANH    4   /* floats only      */
+#define AM_UOP_EXP     5   /* floats only      */
+#define AM_UOP_ABS     6
+#define AM_UOP_COUNT   7
+int am_hip_ew_unary_f32(int op, int rank, const int64_t* shape,
+                        float* dst, const int64_t* dst_strides,
+                        const float* a, const int64_t* a_strides);
+int am_hip_ew_unary_f64(int op, int rank, const int64_t* shape,
+                        double* dst, const int64_t* dst_strides,
+                        const double* a, const int64_t* a_strides);
+int am_hip_ew_unary_i32(int op, int rank, const int64_t* shape,
+                        int32_t* dst, const int64_t* dst_strides,
+                        const int32_t* a, const int64_t* a_strides);
+int am_hip_ew_unary_i64(int op, int rank, const int64_t* shape,
+                        int64_t* dst, const int64_t* dst_strides,
+                        const int64_t* a, const int64_t* a_strides);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AM_HIP_H */

@@ -1,0 +1,313 @@
+"""TEST INFRASTRUCTURE — ctypes front end of the CPU oracle (oracle/libam_oracle.so) plus
+closed-form NumPy checks that pin it.
+
+Only tests, ``__graft_entry__.smoke()`` and the CPU-baseline leg of ``bench.py`` may import this
+module. Nothing under ``arraymancer_amd/`` does: the product path runs on the HIP library only.
+
+The C library restates the reference's algorithms (see the headers of laser_gemm.c and
+strided_map.c for the file:line map). The functions named ``closed_*`` below do NOT restate the
+reference: they compute what the mathematics fixes (modular integer products, higher-precision
+float products, NumPy broadcasting) and are what the restatement is checked against.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from fractions import Fraction
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libam_oracle.so")
+
+_SFX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64",
+        np.dtype(np.int32): "i32", np.dtype(np.int64): "i64"}
+_CT = {"f32": ctypes.c_float, "f64": ctypes.c_double, "i32": ctypes.c_int32, "i64": ctypes.c_int64}
+
+# op codes of include/am_hip.h
+OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
+          relu_bwd=8, max=9, min=10)
+UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with its Makefile (gcc). Returns the library path."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "-B" if force else "-s", "libam_oracle.so"],
+                       check=True, capture_output=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_LIB_PATH)
+        i64, p, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+        for sfx, ct in _CT.items():
+            f = getattr(L, f"am_oracle_gemm_strided_{sfx}")
+            f.restype = ci
+            f.argtypes = [i64, i64, i64, ct, p, i64, i64, p, i64, i64, ct, p, i64, i64]
+            f = getattr(L, f"am_oracle_map2_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, p, p, p, p, p, p]
+            f = getattr(L, f"am_oracle_scalar_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, ci, p, p, p, p, p, ct]
+            f = getattr(L, f"am_oracle_unary_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, p, p, p, p]
+        L.am_oracle_num_threads.restype = ci
+        L.am_oracle_set_num_threads.argtypes = [ci]
+        _lib = L
+    return _lib
+
+
+def num_threads() -> int:
+    return lib().am_oracle_num_threads()
+
+
+def set_num_threads(n: int) -> None:
+    lib().am_oracle_set_num_threads(int(n))
+
+
+def _sfx(arr: np.ndarray) -> str:
+    try:
+        return _SFX[arr.dtype]
+    except KeyError:
+        raise TypeError(f"oracle supports float32/float64/int32/int64, not {arr.dtype}")
+
+
+def _estrides(arr: np.ndarray):
+    it = arr.dtype.itemsize
+    assert all(s % it == 0 for s in arr.strides)
+    return [s // it for s in arr.strides]
+
+
+def _i64arr(vals):
+    return (ctypes.c_int64 * max(1, len(vals)))(*vals)
+
+
+# ----------------------------------------------------------------------------- restatement
+def gemm_strided(alpha, A: np.ndarray, B: np.ndarray, beta, C: np.ndarray) -> np.ndarray:
+    """C <- alpha*A*B + beta*C in place through laser's blocked algorithm. A, B, C are rank-2
+    NumPy arrays or views (any strides, incl. negative and zero for A/B); C is written through
+    its own strides. Returns C."""
+    assert A.ndim == B.ndim == C.ndim == 2 and A.dtype == B.dtype == C.dtype
+    M, K = A.shape
+    K2, N = B.shape
+    assert K == K2 and C.shape == (M, N)
+    sfx = _sfx(A)
+    ct = _CT[sfx]
+    (rsa, csa), (rsb, csb), (rsc, csc) = _estrides(A), _estrides(B), _estrides(C)
+    rc = getattr(lib(), f"am_oracle_gemm_strided_{sfx}")(
+        M, N, K, ct(alpha), A.ctypes.data, rsa, csa, B.ctypes.data, rsb, csb,
+        ct(beta), C.ctypes.data, rsc, csc)
+    if rc != 0:
+        raise MemoryError("oracle gemm_strided: packing buffers")
+    return C
+
+
+def matmul(A: np.ndarray, B: np.ndarray) -> np.ndarray:
+    """`*` of the Tensor API: fresh row-major C, gemm(1, A, B, 0, C)
+    (src/arraymancer/tensor/operators_blas_l2l3.nim:88-100)."""
+    C = np.empty((A.shape[0], B.shape[1]), dtype=A.dtype)
+    C.fill(np.nan if C.dtype.kind == "f" else -77)   # beta == 0 must overwrite whatever is there
+    return gemm_strided(1, A, B, 0, C)
+
+
+def broadcast2(a: np.ndarray, b: np.ndarray):
+    """broadcast2Impl (src/arraymancer/tensor/private/p_shapeshifting.nim:96-134): equal ranks,
+    size-1 axes get stride 0; anything else raises ValueError."""
+    if a.ndim != b.ndim:
+        raise ValueError("broadcast2: ranks differ")
+    shape = []
+    for sa, sb in zip(a.shape, b.shape):
+        if sa == sb or sb == 1:
+            shape.append(sa)
+        elif sa == 1:
+            shape.append(sb)
+        else:
+            raise ValueError(f"Broadcasting error: non-singleton dimensions must be the same in both tensors. "
+                             f"Tensors' shapes were: {a.shape} and {b.shape}")
+    return _bc(a, shape), _bc(b, shape)
+
+
+def _bc(t: np.ndarray, shape):
+    strides = [0 if (ts == 1 and s != 1) else st for ts, s, st in zip(t.shape, shape, t.strides)]
+    return np.lib.stride_tricks.as_strided(t, shape=tuple(shape), strides=tuple(strides), writeable=False)
+
+
+def broadcast(t: np.ndarray, shape):
+    """broadcastImpl (p_shapeshifting.nim:76-94)."""
+    if t.ndim != len(shape):
+        raise ValueError("broadcast: ranks differ")
+    for ts, s in zip(t.shape, shape):
+        if ts != 1 and ts != s:
+            raise ValueError(f"The broadcasted size of the tensor {list(shape)}, must match existing size "
+                             f"{list(t.shape)} for non-singleton dimension")
+    return _bc(t, shape)
+
+
+def map2(op, a: np.ndarray, b: np.ndarray, out: np.ndarray | None = None) -> np.ndarray:
+    """out[i] = op(a[i], b[i]) over equal shapes, each operand walked in C order through its own
+    strides. out=None allocates the fresh contiguous result of map2_inline; out=a is apply2_inline."""
+    op = OP[op] if isinstance(op, str) else op
+    assert a.shape == b.shape and a.dtype == b.dtype
+    if out is None:
+        out = np.empty(a.shape, dtype=a.dtype)
+    assert out.shape == a.shape and out.dtype == a.dtype
+    sfx = _sfx(a)
+    rc = getattr(lib(), f"am_oracle_map2_{sfx}")(
+        op, a.ndim, _i64arr(a.shape), out.ctypes.data, _i64arr(_estrides(out)),
+        a.ctypes.data, _i64arr(_estrides(a)), b.ctypes.data, _i64arr(_estrides(b)))
+    if rc != 0:
+        raise ValueError(f"oracle map2: op {op} not defined for {a.dtype} (rc={rc})")
+    return out
+
+
+def scalar_op(op, a: np.ndarray, scalar, scalar_on_left=False, out: np.ndarray | None = None) -> np.ndarray:
+    op = OP[op] if isinstance(op, str) else op
+    if out is None:
+        out = np.empty(a.shape, dtype=a.dtype)
+    sfx = _sfx(a)
+    rc = getattr(lib(), f"am_oracle_scalar_{sfx}")(
+        op, int(bool(scalar_on_left)), a.ndim, _i64arr(a.shape), out.ctypes.data,
+        _i64arr(_estrides(out)), a.ctypes.data, _i64arr(_estrides(a)), _CT[sfx](scalar))
+    if rc != 0:
+        raise ValueError(f"oracle scalar_op: op {op} not defined for {a.dtype} (rc={rc})")
+    return out
+
+
+def unary(op, a: np.ndarray, out: np.ndarray | None = None) -> np.ndarray:
+    op = UOP[op] if isinstance(op, str) else op
+    if out is None:
+        out = np.empty(a.shape, dtype=a.dtype)
+    sfx = _sfx(a)
+    rc = getattr(lib(), f"am_oracle_unary_{sfx}")(
+        op, a.ndim, _i64arr(a.shape), out.ctypes.data, _i64arr(_estrides(out)),
+        a.ctypes.data, _i64arr(_estrides(a)))
+    if rc != 0:
+        raise ValueError(f"oracle unary: op {op} not defined for {a.dtype} (rc={rc})")
+    return out
+
+
+# ----------------------------------------------------------------------------- closed forms
+def closed_gemm_int(alpha, A, B, beta, C):
+    """Exact integer result of alpha*A*B + beta*C reduced modulo 2^w (w = bit width of the dtype).
+    Ring arithmetic is order independent, so this fixes every bit of the result. Uses Python
+    integers (object arrays): keep the sizes small, or use closed_gemm_int_fast."""
+    w = A.dtype.itemsize * 8
+    Ao, Bo, Co = A.astype(object), B.astype(object), C.astype(object)
+    R = int(alpha) * Ao.dot(Bo) + int(beta) * Co if A.shape[1] > 0 else Co
+    return _wrap_obj(R, w).astype(A.dtype)
+
+
+def _wrap_obj(R, w):
+    mod, half = 1 << w, 1 << (w - 1)
+    f = np.vectorize(lambda v: ((int(v) + half) % mod) - half, otypes=[object])
+    return f(R) if R.size else R
+
+
+def closed_gemm_int_fast(alpha, A, B, beta, C):
+    """Same value as closed_gemm_int through NumPy uint64 arithmetic (wraps modulo 2^64, and
+    2^32 divides 2^64, so reducing afterwards is exact for int32 too)."""
+    w = A.dtype.itemsize * 8
+    Au, Bu, Cu = (x.astype(np.int64).view(np.uint64) for x in (A, B, C))
+    with np.errstate(over="ignore"):
+        R = np.uint64(int(alpha) % (1 << 64)) * (Au @ Bu) + np.uint64(int(beta) % (1 << 64)) * Cu
+    if w == 32:
+        return (R & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32)
+    return R.view(np.int64)
+
+
+def closed_gemm_float(alpha, A, B, beta, C, dtype=np.longdouble):
+    """alpha*A*B + beta*C evaluated in a wider type (float64 for float32 inputs is enough;
+    long double for float64 inputs). beta == 0 ignores C, as the reference does."""
+    Aw, Bw = A.astype(dtype), B.astype(dtype)
+    R = dtype(alpha) * (Aw @ Bw)
+    if beta != 0:
+        R = R + dtype(beta) * C.astype(dtype)
+    return R
+
+
+def closed_gemm_exact(alpha, A, B, beta, C):
+    """Exact rational result (tiny inputs only)."""
+    fr = np.vectorize(lambda v: Fraction(float(v)) if not isinstance(v, (int, np.integer)) else Fraction(int(v)),
+                      otypes=[object])
+    R = Fraction(alpha) * fr(A).dot(fr(B))
+    if beta != 0:
+        R = R + Fraction(beta) * fr(C)
+    return R
+
+
+def rel_frobenius(got, want) -> float:
+    want = np.asarray(want, dtype=np.longdouble)
+    got = np.asarray(got, dtype=np.longdouble)
+    den = np.sqrt((want * want).sum())
+    num = np.sqrt(((got - want) ** 2).sum())
+    return float(num / den) if den != 0 else float(num)
+
+
+def closed_map2(op, a, b):
+    """NumPy statement of the binary ops (single IEEE operation or integer ring operation per
+    element, so bit-exact)."""
+    name = op if isinstance(op, str) else {v: k for k, v in OP.items()}[op]
+    with np.errstate(all="ignore"):
+        if name == "add":
+            return a + b
+        if name == "sub":
+            return a - b
+        if name == "mul":
+            return a * b
+        if name == "div":
+            if a.dtype.kind == "f":
+                return a / b
+            return _trunc_div(a, b)
+        if name == "mod":
+            return _trunc_mod(a, b)
+        if name == "add_relu":
+            t = a + b
+            return np.where(0 >= t, np.zeros_like(t), t)
+        if name == "add_sigmoid":
+            t = a + b
+            return (1 / (1 + np.exp(-t))).astype(a.dtype)
+        if name == "add_tanh":
+            return np.tanh(a + b).astype(a.dtype)
+        if name == "relu_bwd":
+            return np.where(a <= 0, np.zeros_like(b), b)
+        if name == "max":
+            return np.where(b <= a, a, b)
+        if name == "min":
+            return np.where(a <= b, a, b)
+    raise KeyError(name)
+
+
+def _trunc_div(a, b):
+    """C / Nim `div`: truncation toward zero; x div 0 -> 0; min div -1 wraps to min."""
+    info = np.iinfo(a.dtype)
+    a, b = np.broadcast_arrays(a, b)
+    out = np.zeros(a.shape, dtype=a.dtype)
+    nz = b != 0
+    safe_b = np.where(nz, b, 1)
+    ovf = nz & (a == info.min) & (b == -1)
+    safe_a = np.where(ovf, 0, a)
+    q = np.abs(safe_a.astype(object)) // np.abs(safe_b.astype(object))
+    sign = np.where((safe_a < 0) ^ (safe_b < 0), -1, 1).astype(object)
+    out[...] = np.where(nz, (q * sign), 0).astype(a.dtype)
+    out[ovf] = info.min
+    return out
+
+
+def _trunc_mod(a, b):
+    a, b = np.broadcast_arrays(a, b)
+    q = _trunc_div(a, b).astype(object)
+    r = a.astype(object) - q * b.astype(object)
+    r = np.where(b == 0, 0, r)
+    info = np.iinfo(a.dtype)
+    r = np.where((a == info.min) & (b == -1), 0, r)
+    return r.astype(a.dtype)
