@@ -58,7 +58,8 @@ template <> struct Mfma<double> {
   static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
+  // v_mfma_f64_16x16x4: register r of lane group g = lane / 16 holds row 4 * r + g (column = lane % 16).
+  static __device__ __forceinline__ int acc_row(int r, int lane) { return 4 * r + (lane >> 4); }
 };
 
 // Reads the VK k values that `lane` feeds to the MFMA steps of k-step `ks` for row/col `mn`.

@@ -10,6 +10,14 @@ for p in (ROOT, os.path.join(ROOT, "oracle")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
+import zlib
+
+
+def seed_of(*parts) -> int:
+    """Deterministic 32-bit seed from a test's parameters (str hashes vary per process)."""
+    return zlib.crc32(repr(parts).encode())
+
+
 DTYPES = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "i64": np.int64}
 
 
@@ -67,29 +75,31 @@ def hip_apply_ops(t, ops):
     return t
 
 
+PARENT_SHAPE = {
+    "C": lambda m, n: (m, n), "F": lambda m, n: (n, m), "rowstep2": lambda m, n: (2 * m, n),
+    "colstep2": lambda m, n: (m, 2 * n), "neg_rows": lambda m, n: (m, n), "neg_cols": lambda m, n: (m, n),
+    "inner_block": lambda m, n: (m + 3, n + 5), "bcast_rows": lambda m, n: (1, n),
+}
+
+
+def view_of(parent: np.ndarray, kind: str, shape):
+    """The [m, n] view of geometry `kind` over `parent` (which has PARENT_SHAPE[kind](m, n))."""
+    m, n = shape
+    return {
+        "C": lambda p: p, "F": lambda p: p.T, "rowstep2": lambda p: p[::2], "colstep2": lambda p: p[:, ::2],
+        "neg_rows": lambda p: p[::-1], "neg_cols": lambda p: p[:, ::-1],
+        "inner_block": lambda p: p[2:2 + m, 1:1 + n], "bcast_rows": lambda p: np.broadcast_to(p, (m, n)),
+    }[kind](parent)
+
+
 def strided_view(rng, shape, dtype, kind):
     """A NumPy array of `shape` whose memory layout is `kind`; returns (view, parent)."""
-    m, n = shape
-    def fill(s):
-        if np.dtype(dtype).kind == "f":
-            return rng.uniform(-1, 1, size=s).astype(dtype)
-        return rng.integers(-100, 101, size=s).astype(dtype)
-    if kind == "C":
-        p = fill((m, n)); return p, p
-    if kind == "F":
-        p = fill((n, m)); return p.T, p
-    if kind == "rowstep2":
-        p = fill((2 * m, n)); return p[::2], p
-    if kind == "colstep2":
-        p = fill((m, 2 * n)); return p[:, ::2], p
-    if kind == "neg_rows":
-        p = fill((m, n)); return p[::-1], p
-    if kind == "neg_cols":
-        p = fill((m, n)); return p[:, ::-1], p
-    if kind == "inner_block":
-        p = fill((m + 3, n + 5)); return p[2:2 + m, 1:1 + n], p
-    if kind == "bcast_rows":
-        p = fill((1, n)); return np.broadcast_to(p, (m, n)), p
-    raise KeyError(kind)
+    ps = PARENT_SHAPE[kind](*shape)
+    if np.dtype(dtype).kind == "f":
+        parent = rng.uniform(-1, 1, size=ps).astype(dtype)
+    else:
+        parent = rng.integers(-100, 101, size=ps).astype(dtype)
+    return view_of(parent, kind, shape), parent
+
 
 VIEW_KINDS = ["C", "F", "rowstep2", "colstep2", "neg_rows", "neg_cols", "inner_block", "bcast_rows"]

@@ -1,0 +1,266 @@
+"""Element-wise / broadcast / map parity on the GPU (through the C ABI): bit-exact against the CPU
+oracle and NumPy for every single-operation body; transcendental bodies within a stated tolerance."""
+import numpy as np
+import pytest
+
+from conftest import DTYPES, seed_of
+
+pytestmark = pytest.mark.gpu
+ALL = ["f32", "f64", "i32", "i64"]
+INT, FLT = ["i32", "i64"], ["f32", "f64"]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def _kinds(kind):
+    return {"int": INT, "float": FLT, "any": ALL, "float64_only": ["f64"]}[kind]
+
+
+def fill(rng, shape, dt, lo=-50, hi=50):
+    if np.dtype(dt).kind == "f":
+        return rng.uniform(-4, 4, size=shape).astype(dt)
+    return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
+
+
+# ------------------------------------------------------------------ reference vectors
+def test_reference_elementwise_vectors(hip, vectors):
+    for case in vectors["elementwise"]:
+        for sfx in _kinds(case["kind"]):
+            dt = DTYPES[sfx]
+            say("ew vector", case["name"], sfx)
+            a, b = hip.toHip(np.array(case["a"], dtype=dt)), hip.toHip(np.array(case["b"], dtype=dt))
+            op = {"add": "+.", "sub": "-.", "mul": "*.", "div": "/.", "mod": "mod"}[case["op"]]
+            got = hip.OPERATORS[op](a, b).toCpu()
+            assert np.array_equal(got, np.array(case["expect"], dtype=dt)), (case["name"], sfx)
+
+
+def test_reference_explicit_broadcast(hip, vectors):
+    for case in vectors["explicit_broadcast"]:
+        t = hip.toHip(np.array(case["t"], dtype=np.int64))
+        assert np.array_equal(t.bc(case["shape"]).clone().toCpu(), np.array(case["expect"]))
+        assert np.array_equal(t.bc(case["shape"]).toCpu(), np.array(case["expect"]))
+
+
+def test_reference_inplace_broadcast(hip, vectors):
+    for case in vectors["inplace_broadcast"]:
+        for sfx in _kinds(case["kind"]):
+            dt = DTYPES[sfx]
+            say("ew inplace", case["source"], sfx)
+            a, b = hip.toHip(np.array(case["a"], dtype=dt)), hip.toHip(np.array(case["b"], dtype=dt))
+            op = {"add": "+.=", "sub": "-.=", "mul": "*.=", "div": "/.="}[case["op"]]
+            hip.OPERATORS[op](a, b)
+            assert np.array_equal(a.toCpu(), np.array(case["expect"], dtype=dt))
+
+
+def test_reference_scalar_chains(hip, vectors):
+    for case in vectors["scalar_chains"]:
+        for sfx in _kinds(case["kind"]):
+            dt = DTYPES[sfx]
+            say("ew scalar", case["source"], sfx)
+            t = hip.toHip(np.array(case["a"], dtype=dt))
+            for op, s, side in case["steps"]:
+                f = hip.OPERATORS[{"add": "+.", "sub": "-.", "mul": "*.", "div": "/.", "mod": "mod"}[op]]
+                t = f(s, t) if side == "left" else f(t, s)
+            assert np.array_equal(t.toCpu(), np.array(case["expect"], dtype=dt)), (case["source"], sfx)
+
+
+def test_reference_sigmoid_chain(hip, vectors):
+    c = vectors["sigmoid_chain"]
+    t = hip.toHip(np.array(c["t"], dtype=np.float32))
+    e = hip.unary("exp", hip.bc_sub(0.0, t))
+    got = hip.bc_div(1.0, hip.bc_add(1.0, e))
+    assert np.array_equal(got.toCpu(), np.array(c["expect"], dtype=np.float32))
+    assert np.array_equal(hip.sigmoid(t).toCpu(), np.array(c["expect"], dtype=np.float32))
+
+
+def test_reference_sliced_add_sub(hip, vectors):
+    c = vectors["sliced_add_sub"]
+    a = hip.toHip(np.array(c["a"], dtype=np.float64))
+    a_t = a.transpose()
+    for case in c["cases"]:
+        (r0, r1, _), (c0, c1, _) = case["slice"]
+        x, y = a[r0:r1 + 1, c0:c1 + 1], a_t[r0:r1 + 1, c0:c1 + 1]
+        got = (x + y) if case["op"] == "add" else (x - y)
+        assert np.array_equal(got.toCpu(), np.array(case["expect"], dtype=np.float64))
+
+
+def test_reference_inplace_on_transposed(hip, vectors):
+    c = vectors["inplace_on_transposed"]
+    t = np.array(c["vandermonde"], dtype=np.float32)
+    z = hip.toHip(t).clone().transpose()
+    z += z
+    assert np.array_equal(z.toCpu(), np.array(c["after_z_plus_z"], dtype=np.float32))
+    z += hip.toHip(t)
+    assert np.array_equal(z.toCpu(), np.array(c["after_plus_t2"], dtype=np.float32))
+    with pytest.raises(ValueError):
+        z += hip.toHip(t)[0:2, 0:2]
+
+
+def test_reference_map2_bool(hip, vectors):
+    c = vectors["map2_bool"]
+    a, b = hip.toHip(np.array(c["a"], dtype=np.int64)), hip.toHip(np.array(c["b"], dtype=np.int64))
+    m = hip.map2("mod", a, b).toCpu()
+    assert np.array_equal(m == 0, np.array(c["expect"]))
+
+
+# ------------------------------------------------------------------ oracle / NumPy parity
+SHAPES = [(1,), (3,), (1000,), (4099,), (7, 13), (64, 4096), (33, 4100), (5, 6, 7), (2, 3, 4, 5, 6, 2), (300, 1), (1, 300)]
+BIN_OPS = ["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min"]
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("shape", SHAPES)
+def test_same_shape_ops_bit_exact(hip, oracle, sfx, shape):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, shape))
+    a, b = fill(rng, shape, dt), fill(rng, shape, dt)
+    if sfx in INT:
+        a.ravel()[:2] = [np.iinfo(dt).max, np.iinfo(dt).min][: min(2, a.size)]   # force wraparound cases
+    da, db = hip.toHip(a), hip.toHip(b)
+    for op in BIN_OPS + (["mod"] if sfx in INT else []):
+        say("same-shape", sfx, shape, op)
+        got = hip.map2(op, da, db).toCpu()
+        want = oracle.map2(op, a, b)
+        assert np.array_equal(got, want, equal_nan=True), op
+        assert np.array_equal(got, oracle.closed_map2(op, a, b), equal_nan=True), op
+
+
+BC_CASES = [((64, 4096), (1, 4096)), ((64, 4096), (64, 1)), ((1, 4096), (64, 4096)), ((64, 1), (64, 4096)),
+            ((4, 1), (1, 3)), ((5, 1, 7), (1, 6, 1)), ((2, 3, 2048), (2, 1, 2048)), ((3, 1, 4096), (1, 5, 1)),
+            ((1, 1), (9, 1031))]
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("shapes", BC_CASES)
+def test_broadcast_ops_bit_exact(hip, oracle, sfx, shapes):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, shapes))
+    a, b = fill(rng, shapes[0], dt), fill(rng, shapes[1], dt)
+    b[b == 0] = 3
+    da, db = hip.toHip(a), hip.toHip(b)
+    for name, npf in [("+.", np.add), ("-.", np.subtract), ("*.", np.multiply)]:
+        say("broadcast", sfx, shapes, name)
+        got = hip.OPERATORS[name](da, db).toCpu()
+        with np.errstate(over="ignore"):
+            assert np.array_equal(got, npf(a, b)), name
+    say("broadcast", sfx, shapes, "/.")
+    ba, bb = oracle.broadcast2(a, b)
+    assert np.array_equal(hip.bc_div(da, db).toCpu(), oracle.map2("div", ba, bb))
+    assert np.array_equal(hip.bias_relu(da, db).toCpu(), oracle.map2("add_relu", ba, bb))
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_strided_operands_and_destinations(hip, oracle, sfx):
+    """Transposed, stepped, reversed and column-sliced operands, out of place and in place."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "strided"))
+    P, Q = fill(rng, (96, 80), dt), fill(rng, (80, 96), dt)
+    dP, dQ = hip.toHip(P), hip.toHip(Q)
+    cases = [
+        ("transposed b", dP, P, dQ.transpose(), Q.T),
+        ("both stepped", dP[::2, ::2], P[::2, ::2], dQ.transpose()[::2, ::2], Q.T[::2, ::2]),
+        ("reversed", dP[::-1, ::-1], P[::-1, ::-1], dQ.transpose(), Q.T),
+        ("column block (GRU gate slices)", dP[:, 16:48], P[:, 16:48], dP[:, 48:80], P[:, 48:80]),
+    ]
+    for name, da, a, db, b in cases:
+        say("strided", sfx, name)
+        assert np.array_equal(hip.map2("add", da, db).toCpu(), oracle.map2("add", a, b)), name
+        assert np.array_equal(hip.map2("mul", da, db).toCpu(), oracle.map2("mul", a, b)), name
+    # in place through a strided destination: parent[:, 16:48] +.= row vector
+    say("strided inplace", sfx)
+    v = fill(rng, (1, 32), dt)
+    dP[:, 16:48].bc_iadd(hip.toHip(v))
+    P2 = P.copy(); P2[:, 16:48] += v
+    assert np.array_equal(dP.toCpu(), P2)
+    # in place on a transposed destination
+    dQt = dQ.transpose()
+    dQt += dP
+    assert np.array_equal(dQ.toCpu(), (Q.T + P2).T)
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_scalar_and_unary(hip, oracle, sfx):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "scalar"))
+    a = fill(rng, (37, 1028), dt)
+    a[a == 0] = 5
+    da = hip.toHip(a)
+    for op in ["add", "sub", "mul", "div", "max", "min"] + (["mod"] if sfx in INT else []):
+        for left in (False, True):
+            say("scalar", sfx, op, left)
+            got = hip.scalar_op(op, da, 3, scalar_on_left=left).toCpu()
+            assert np.array_equal(got, oracle.scalar_op(op, a, 3, scalar_on_left=left)), (op, left)
+    for op in ["copy", "neg", "relu", "abs"]:
+        say("unary", sfx, op)
+        assert np.array_equal(hip.unary(op, da).toCpu(), oracle.unary(op, a)), op
+        assert np.array_equal(hip.unary(op, da.transpose()).toCpu(), oracle.unary(op, a.T)), op
+    assert np.array_equal((da * 2).toCpu(), a * dt(2))
+    assert np.array_equal((2 * da).toCpu(), a * dt(2))
+    assert np.array_equal((-da).toCpu(), -a)
+    assert np.array_equal(da.transpose().clone().toCpu(), a.T)
+    assert np.array_equal(da.reshape(1028, 37).toCpu(), a.reshape(1028, 37))
+    assert np.array_equal(da.transpose().reshape(37, 1028).toCpu(), a.T.reshape(37, 1028))
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_transcendental_bodies(hip, oracle, sfx):
+    """exp / tanh / sigmoid come from the device math library: not bit-comparable with libm.
+    Tolerance: 4 ulp-scale relative error (float32 4e-7 * 4, float64 1e-15 * 8)."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "trans"))
+    a, b = fill(rng, (64, 1024), dt), fill(rng, (1, 1024), dt)
+    rtol = 2e-6 if sfx == "f32" else 1e-14
+    da, db = hip.toHip(a), hip.toHip(b)
+    ba, bb = oracle.broadcast2(a, b)
+    for op in ("add_sigmoid", "add_tanh"):
+        say("transcendental", sfx, op)
+        la, lb = da, db.broadcast(a.shape)
+        np.testing.assert_allclose(hip.map2(op, la, lb).toCpu(), oracle.map2(op, ba, bb), rtol=rtol, atol=rtol)
+    for op in ("sigmoid", "tanh", "exp"):
+        np.testing.assert_allclose(hip.unary(op, da).toCpu(), oracle.unary(op, a), rtol=rtol, atol=rtol)
+
+
+def test_relu_special_values(hip):
+    x = np.array([-1.0, -0.0, 0.0, 2.5, np.nan, -np.inf, np.inf] * 3, dtype=np.float32)
+    r = hip.relu(hip.toHip(x)).toCpu()
+    assert r[:4].tolist() == [0.0, 0.0, 0.0, 2.5] and not np.signbit(r[1])
+    assert np.isnan(r[4]) and r[5] == 0 and r[6] == np.inf
+
+
+def test_int_division_conventions(hip):
+    a = hip.toHip(np.array([7, -7, 7, -7, 0, 5, -2**31], dtype=np.int32))
+    b = hip.toHip(np.array([2, 2, -2, -2, 3, 0, -1], dtype=np.int32))
+    assert hip.bc_div(a, b).toCpu().tolist() == [3, -3, -3, 3, 0, 0, -2**31]
+    assert hip.bc_mod(a, b).toCpu().tolist() == [1, -1, 1, -1, 0, 0, 0]
+
+
+def test_errors(hip):
+    a = hip.toHip(np.zeros((4, 2), np.float32))
+    with pytest.raises(ValueError):
+        hip.bc_add(a, hip.toHip(np.zeros((1, 3), np.float32)))
+    with pytest.raises(TypeError):
+        hip.bc_mod(a, a)
+    with pytest.raises(TypeError):
+        hip.map2("add_tanh", hip.toHip(np.zeros(3, np.int32)), hip.toHip(np.zeros(3, np.int32)))
+    with pytest.raises(ValueError):   # zero-stride destination
+        hip.apply2("add", hip.toHip(np.zeros((1, 2), np.float32)).broadcast((4, 2)), a)
+    empty = hip.empty((0, 5), np.float32)
+    assert (empty + empty).shape == (0, 5)
+
+
+# ------------------------------------------------------------------ BASELINE config 4, full size
+def test_config4_8192_bit_exact(hip):
+    X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
+    b = np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32)
+    s = np.random.default_rng(4003).uniform(-1, 1, (8192, 1)).astype(np.float32)
+    dX, db, ds = hip.toHip(X), hip.toHip(b), hip.toHip(s)
+    say("config4 +.")
+    dY = hip.bc_add(dX, db)
+    Y = X + b
+    assert np.array_equal(dY.toCpu(), Y)
+    say("config4 *.")
+    assert np.array_equal(hip.bc_mul(dY, ds).toCpu(), Y * s)
+    say("config4 bias+relu")
+    assert np.array_equal(hip.bias_relu(dX, db).toCpu(), np.where(0 >= Y, np.float32(0), Y))

@@ -1,0 +1,334 @@
+"""GEMM parity on the GPU: the HIP kernels (through the C ABI) against the CPU oracle, the
+reference's known-answer vectors, and size-independent properties at the full BASELINE sizes.
+
+Bars: integers bit-exact; float32 <= 1e-4, float64 <= 1e-12 relative Frobenius error."""
+import numpy as np
+import pytest
+
+from conftest import seed_of, DTYPES, VIEW_KINDS, hip_apply_ops, np_apply_ops
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f32": 1e-4, "f64": 1e-12}
+ALL = ["f32", "f64", "i32", "i64"]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def _mat(vectors, name, dt):
+    return np.array(vectors["matrices"][name], dtype=dt)
+
+
+def fill(rng, shape, dt, lo=-100, hi=100):
+    if np.dtype(dt).kind == "f":
+        return rng.uniform(-1, 1, size=shape).astype(dt)
+    return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
+
+
+def assert_parity(oracle, sfx, got, want, what=""):
+    if sfx in ("i32", "i64"):
+        assert np.array_equal(got, want), what
+    else:
+        err = oracle.rel_frobenius(got, want)
+        assert err <= TOL[sfx], f"{what}: rel Frobenius {err:.3e}"
+
+
+# ------------------------------------------------------------------ reference vectors
+@pytest.mark.parametrize("sfx", ALL)
+def test_reference_vectors(hip, vectors, sfx):
+    dt = DTYPES[sfx]
+    for case in vectors["gemm"]:
+        say("gemm vector", case["name"], sfx)
+        a, b = hip.toHip(_mat(vectors, case["a"], dt)), hip.toHip(_mat(vectors, case["b"], dt))
+        assert np.array_equal((a * b).toCpu(), _mat(vectors, case["expect"], dt)), case["name"]
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_reference_view_vectors(hip, vectors, sfx):
+    dt = DTYPES[sfx]
+    for case in vectors["gemm_views"]:
+        say("gemm view vector", case["name"], sfx)
+        a = hip_apply_ops(hip.toHip(_mat(vectors, case["a"], dt)), case["a_ops"])
+        b = hip_apply_ops(hip.toHip(_mat(vectors, case["b"], dt)), case["b_ops"])
+        want = np.array(case["expect_literal"], dtype=dt) if "expect_literal" in case else _mat(vectors, case["expect"], dt)
+        assert np.array_equal((a * b).toCpu(), want), case["name"]
+
+
+def test_reference_colmajor_reversed_slice(hip, vectors):
+    c = vectors["gemm_colmajor_reversed_slice"]
+    a = hip.toHip(np.array(c["a"], dtype=np.float64))
+    # column-major parent made on the device: upload the transpose, view it transposed
+    eig = hip.toHip(np.array(c["eigvecs_logical"], dtype=np.float64).T.copy()).transpose()
+    assert eig.is_F_contiguous()
+    b = hip_apply_ops(eig, c["b_ops"])
+    assert b.strides == (1, -2)
+    val = (a * b).toCpu()
+    assert np.abs(val - np.array(c["expect"])).mean() < c["mean_abs_tol"]
+
+
+def test_reference_fusion_vector(hip, vectors):
+    c = vectors["gemm_fusion"]
+    A, x, b = (hip.toHip(np.array(c[k], dtype=np.float64)) for k in ("A", "x", "b"))
+    for _ in range(5):
+        out = b.clone()
+        hip.gemm(1.0, A, x, 1.0, out)
+        assert out.toCpu()[0, 0] == 12.0 and b.toCpu()[0, 0] == 0.0
+
+
+# ------------------------------------------------------------------ oracle parity, edge shapes
+EDGE_SHAPES = [(1, 1, 1), (1, 7, 3), (5, 1, 9), (33, 31, 2), (64, 64, 16), (65, 63, 17), (127, 129, 15),
+               (128, 128, 128), (255, 257, 33), (256, 256, 64), (300, 200, 100), (97, 513, 65)]
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("shape", EDGE_SHAPES)
+def test_edge_shapes_vs_oracle(hip, oracle, sfx, shape):
+    dt = DTYPES[sfx]
+    M, N, K = shape
+    rng = np.random.default_rng(seed_of(sfx, shape))
+    info = None if np.dtype(dt).kind == "f" else np.iinfo(dt)
+    lo, hi = (-100, 100) if info is None else (info.min, info.max)   # integers: full range, wraps
+    A, B, C = fill(rng, (M, K), dt, lo, hi), fill(rng, (K, N), dt, lo, hi), fill(rng, (M, N), dt, lo, hi)
+    for alpha, beta in [(1, 0), (1, 1), (3, -2)]:
+        say("edge", sfx, shape, alpha, beta)
+        want = oracle.gemm_strided(alpha, A, B, beta, C.copy())
+        dC = hip.toHip(C)
+        hip.gemm(alpha, hip.toHip(A), hip.toHip(B), beta, dC)
+        assert_parity(oracle, sfx, dC.toCpu(), want, f"{shape} a={alpha} b={beta}")
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("tile", ["0", "1", "2"])
+def test_every_tile_shape(hip, oracle, sfx, tile, monkeypatch):
+    """Forces each workgroup tile candidate on a ragged problem."""
+    if sfx in ("i32", "i64") and tile == "2":
+        pytest.skip("integer path has two tile candidates")
+    monkeypatch.setenv(f"AM_HIP_GEMM_TILE_{sfx.upper()}", tile)
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(int(tile) + 17)
+    M, N, K = 261, 389, 77
+    A, B, C = fill(rng, (M, K), dt), fill(rng, (K, N), dt), fill(rng, (M, N), dt)
+    say("tile", sfx, tile)
+    want = oracle.gemm_strided(2, A, B, 1, C.copy())
+    dC = hip.toHip(C)
+    hip.gemm(2, hip.toHip(A), hip.toHip(B), 1, dC)
+    assert_parity(oracle, sfx, dC.toCpu(), want, f"tile {tile}")
+
+
+# ------------------------------------------------------------------ strided / transposed views
+def device_view(hip, parent_np, kind, shape):
+    """The same geometry as conftest.strided_view, built with view ops on the device tensor."""
+    m, n = shape
+    t = hip.toHip(parent_np)
+    if kind == "C":
+        return t
+    if kind == "F":
+        return t.transpose()
+    if kind == "rowstep2":
+        return t[::2]
+    if kind == "colstep2":
+        return t[:, ::2]
+    if kind == "neg_rows":
+        return t[::-1]
+    if kind == "neg_cols":
+        return t[:, ::-1]
+    if kind == "inner_block":
+        return t[2:2 + m, 1:1 + n]
+    if kind == "bcast_rows":
+        return t.broadcast((m, n))
+    raise KeyError(kind)
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("ka", VIEW_KINDS)
+@pytest.mark.parametrize("kb", VIEW_KINDS)
+def test_views_without_host_copy(hip, oracle, sfx, ka, kb):
+    from conftest import strided_view
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, ka, kb))
+    M, N, K = 72, 52, 40      # multiples of 4: the vector loaders are eligible where strides allow
+    A, pa = strided_view(rng, (M, K), dt, ka)
+    B, pb = strided_view(rng, (K, N), dt, kb)
+    say("views", sfx, ka, kb)
+    dA, dB = device_view(hip, pa, ka, (M, K)), device_view(hip, pb, kb, (K, N))
+    assert dA.shape == A.shape and dB.shape == B.shape
+    got = (dA * dB).toCpu()
+    want = oracle.matmul(A, B)
+    assert_parity(oracle, sfx, got, want, f"{ka} x {kb}")
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("kc", ["F", "rowstep2", "colstep2", "neg_rows", "inner_block"])
+def test_strided_destination(hip, oracle, sfx, kc):
+    from conftest import strided_view, view_of
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, kc))
+    M, N, K = 37, 45, 29
+    A, B = fill(rng, (M, K), dt), fill(rng, (K, N), dt)
+    Cv, parent = strided_view(rng, (M, N), dt, kc)
+    say("dest", sfx, kc)
+    before = parent.copy()
+    dC = device_view(hip, parent, kc, (M, N))               # uploads `parent`, views it on the device
+    hip.gemm(2, hip.toHip(A), hip.toHip(B), 3, dC)
+    oracle.gemm_strided(2, A, B, 3, Cv)                      # writes through the NumPy view into `parent`
+    after = hip.HipTensor(hip.Layout(parent.shape, tuple(s // parent.itemsize for s in parent.strides), 0),
+                          dC.storage, dC.dtype).toCpu()
+    assert_parity(oracle, sfx, view_of(after, kc, (M, N)), Cv, kc)
+    inside = np.zeros(parent.shape, dtype=bool)
+    view_of(inside, kc, (M, N))[...] = True
+    assert np.array_equal(after[~inside], before[~inside])   # nothing outside the view was written
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_float_semantics(hip, sfx):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(9)
+    A, B = fill(rng, (70, 30), dt), fill(rng, (30, 90), dt)
+    say("beta0 NaN", sfx)
+    dC = hip.toHip(np.full((70, 90), np.nan, dtype=dt))
+    hip.gemm(1, hip.toHip(A), hip.toHip(B), 0, dC)
+    assert np.isfinite(dC.toCpu()).all()                      # beta == 0 never reads C
+    say("alpha0 NaN", sfx)
+    A2 = A.copy(); A2[3, 4] = np.nan
+    dC = hip.toHip(np.zeros((70, 90), dtype=dt))
+    hip.gemm(0, hip.toHip(A2), hip.toHip(B), 1, dC)
+    assert np.isnan(dC.toCpu()[3]).all()                      # alpha == 0 is not special-cased
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_empty_extents_leave_c_untouched(hip, sfx):
+    dt = DTYPES[sfx]
+    C = np.arange(20, dtype=dt).reshape(4, 5)
+    dC = hip.toHip(C)
+    hip.gemm(1, hip.empty((4, 0), dt), hip.empty((0, 5), dt), 0, dC)
+    assert np.array_equal(dC.toCpu(), C)
+    assert (hip.empty((0, 3), dt) * hip.empty((3, 4), dt)).shape == (0, 4)
+
+
+def test_int_wrap_known_answers(hip):
+    A = hip.toHip(np.array([[2**31 - 1, 1]], dtype=np.int32))
+    B = hip.toHip(np.array([[2], [3]], dtype=np.int32))
+    assert (A * B).toCpu()[0, 0] == 1
+    A = hip.toHip(np.array([[2**62, -1]], dtype=np.int64))
+    B = hip.toHip(np.array([[4], [5]], dtype=np.int64))
+    assert (A * B).toCpu()[0, 0] == -5
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_fused_epilogue(hip, oracle, sfx):
+    """linear + bias + ReLU in the GEMM epilogue == the reference's three passes
+    (nnp_linear.nim:28-29 then relu)."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(21)
+    x, W, b = fill(rng, (64, 100), dt), fill(rng, (50, 100), dt), fill(rng, (1, 50), dt)
+    say("epilogue", sfx)
+    out = oracle.matmul(x, W.T)
+    oracle.map2("add", out, oracle.broadcast(b, out.shape), out=out)
+    want_lin = out.copy()
+    want_relu = oracle.unary("relu", out)
+    dx, dW, db = hip.toHip(x), hip.toHip(W), hip.toHip(b)
+    assert_parity(oracle, sfx, hip.linear(dx, dW, db).toCpu(), want_lin, "bias")
+    got = hip.linear(dx, dW, db, relu=True).toCpu()
+    assert_parity(oracle, sfx, got, want_relu, "bias+relu")
+    assert (got >= 0).all() and (got == 0).any()
+    # column-vector bias [M, 1]
+    bcol = fill(rng, (64, 1), dt)
+    o = hip.empty((64, 50), dt)
+    hip.gemm(1, dx, dW.transpose(), 0, o, epilogue="bias", bias=hip.toHip(bcol))
+    assert_parity(oracle, sfx, o.toCpu(), oracle.matmul(x, W.T) + bcol, "col bias")
+
+
+# ------------------------------------------------------------------ BASELINE configs
+def test_config1_f32_1024(hip, oracle):
+    rng_a, rng_b = np.random.default_rng(1001), np.random.default_rng(1002)
+    A = rng_a.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    B = rng_b.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    say("config1 f32 1024^3")
+    got = (hip.toHip(A) * hip.toHip(B)).toCpu()
+    assert oracle.rel_frobenius(got, oracle.matmul(A, B)) <= 1e-4
+    assert oracle.rel_frobenius(got, A.astype(np.float64) @ B.astype(np.float64)) <= 1e-4
+
+
+def test_config2_i32_1500_bit_exact(hip, oracle):
+    A = np.random.default_rng(2001).integers(-100, 100, (1500, 1500), endpoint=True).astype(np.int32)
+    B = np.random.default_rng(2002).integers(-100, 100, (1500, 1500), endpoint=True).astype(np.int32)
+    say("config2 i32 1500^3")
+    got = (hip.toHip(A) * hip.toHip(B)).toCpu()
+    assert np.array_equal(got, oracle.matmul(A, B))
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+def test_config2_4096_ring_checksum(hip, oracle, sfx):
+    """Full size, checked through a property that holds exactly in Z / 2^w:
+    (A B) v == A (B v) for any v, plus a bit-exact block against the oracle."""
+    dt = DTYPES[sfx]
+    n = 4096
+    A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(dt)
+    B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(dt)
+    say("config2 4096^3", sfx)
+    C = (hip.toHip(A) * hip.toHip(B)).toCpu()
+    v = np.random.default_rng(5).integers(-2**31, 2**31 - 1, (n, 1)).astype(np.int64).view(np.uint64)
+    U = lambda x: x.astype(np.int64).view(np.uint64)
+    with np.errstate(over="ignore"):
+        lhs = U(C) @ v
+        rhs = U(A) @ (U(B) @ v)
+    mask = np.uint64(0xFFFFFFFF) if sfx == "i32" else np.uint64(0xFFFFFFFFFFFFFFFF)
+    assert np.array_equal(lhs & mask, rhs & mask)
+    rows = slice(1000, 1192)
+    assert np.array_equal(C[rows], oracle.matmul(A[rows], B))
+
+
+def test_config3_f64_views(hip, oracle):
+    """gemm(1.5, A, B, 0.5, C): A a transposed view, B every other column of a 1024 x 6144 parent."""
+    pa = np.random.default_rng(3001).standard_normal((1024, 2048))
+    pb = np.random.default_rng(3002).standard_normal((1024, 6144))
+    C = np.random.default_rng(3003).standard_normal((2048, 3072))
+    dA = hip.toHip(pa).transpose()
+    dB = hip.toHip(pb)[:, ::2]
+    assert dA.strides == (1, 2048) and dB.strides == (6144, 2)
+    dC = hip.toHip(C)
+    say("config3 f64 2048x3072x1024 views")
+    hip.gemm(1.5, dA, dB, 0.5, dC)
+    got = dC.toCpu()
+    want = oracle.gemm_strided(1.5, pa.T, pb[:, ::2], 0.5, C.copy())
+    assert oracle.rel_frobenius(got, want) <= 1e-12
+    rows = np.arange(0, 2048, 64)
+    wide = 1.5 * (pa.T[rows].astype(np.longdouble) @ pb[:, ::2].astype(np.longdouble)) + 0.5 * C[rows].astype(np.longdouble)
+    assert oracle.rel_frobenius(got[rows], wide) <= 1e-12
+
+
+def test_config5_inference_chain(hip, oracle):
+    rng = np.random.default_rng(5001)
+    g = lambda *s: rng.normal(0, 0.1, s).astype(np.float32)
+    k1, x1 = g(20, 25), g(25, 36864)
+    k2, x2 = g(50, 500), g(500, 4096)
+    x3, w3, b3 = g(64, 800), g(500, 800), g(1, 500)
+    w4 = g(10, 500)
+    say("config5 chain")
+    f64 = lambda a: a.astype(np.float64)
+    o1 = (hip.toHip(k1) * hip.toHip(x1)).toCpu()
+    assert oracle.rel_frobenius(o1, f64(k1) @ f64(x1)) <= 1e-4
+    o2 = (hip.toHip(k2) * hip.toHip(x2)).toCpu()
+    assert oracle.rel_frobenius(o2, f64(k2) @ f64(x2)) <= 1e-4
+    h = hip.linear(hip.toHip(x3), hip.toHip(w3), hip.toHip(b3), relu=True)
+    want_h = np.maximum(f64(x3) @ f64(w3).T + f64(b3), 0)
+    assert oracle.rel_frobenius(h.toCpu(), want_h) <= 1e-4
+    o4 = (h * hip.toHip(w4).transpose()).toCpu()
+    assert oracle.rel_frobenius(o4, want_h @ f64(w4).T) <= 1e-4
+
+
+def test_fp32_4096_properties(hip, oracle):
+    """Full headline size: linearity in alpha and agreement of a row block with float64."""
+    n = 4096
+    A = np.random.default_rng(1001).uniform(-1, 1, (n, n)).astype(np.float32)
+    B = np.random.default_rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
+    dA, dB = hip.toHip(A), hip.toHip(B)
+    say("f32 4096^3")
+    C1 = (dA * dB).toCpu()
+    rows = slice(2048, 2048 + 128)
+    assert oracle.rel_frobenius(C1[rows], A[rows].astype(np.float64) @ B.astype(np.float64)) <= 1e-4
+    dC = hip.empty((n, n), np.float32)
+    hip.gemm(2.0, dA, dB, 0.0, dC)
+    assert np.array_equal(dC.toCpu(), 2.0 * C1)       # scaling by 2 is exact in binary floating point

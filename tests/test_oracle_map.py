@@ -1,0 +1,189 @@
+"""Pins the CPU oracle's strided map / apply restatement (oracle/strided_map.c) — CPU only.
+
+Anchors: the reference's literal vectors (test_broadcasting.nim, test_operators_blas*.nim,
+test_higherorder.nim) and NumPy's own broadcasting / strided views (each element is one IEEE or
+ring operation, so the comparison is bit-exact)."""
+import numpy as np
+import pytest
+from hypothesis import given, settings, strategies as st
+
+from conftest import DTYPES
+
+INT = ["i32", "i64"]
+FLT = ["f32", "f64"]
+
+
+def _kinds(kind):
+    return {"int": INT, "float": FLT, "any": INT + FLT, "float64_only": ["f64"]}[kind]
+
+
+def test_reference_elementwise_vectors(vectors, oracle):
+    for case in vectors["elementwise"]:
+        for sfx in _kinds(case["kind"]):
+            dt = DTYPES[sfx]
+            a, b = np.array(case["a"], dtype=dt), np.array(case["b"], dtype=dt)
+            ba, bb = oracle.broadcast2(a, b)
+            got = oracle.map2(case["op"], ba, bb)
+            assert np.array_equal(got, np.array(case["expect"], dtype=dt)), (case["name"], sfx)
+
+
+def test_reference_explicit_broadcast(vectors, oracle):
+    for case in vectors["explicit_broadcast"]:
+        t = np.array(case["t"], dtype=np.int64)
+        got = oracle.unary("copy", oracle.broadcast(t, case["shape"]))
+        assert np.array_equal(got, np.array(case["expect"]))
+
+
+def test_reference_inplace_broadcast(vectors, oracle):
+    for case in vectors["inplace_broadcast"]:
+        for sfx in _kinds(case["kind"]):
+            dt = DTYPES[sfx]
+            a, b = np.array(case["a"], dtype=dt), np.array(case["b"], dtype=dt)
+            oracle.map2(case["op"], a, oracle.broadcast(b, a.shape), out=a)   # apply2: dst is a
+            assert np.array_equal(a, np.array(case["expect"], dtype=dt)), (case["source"], sfx)
+
+
+def test_reference_scalar_chains(vectors, oracle):
+    for case in vectors["scalar_chains"]:
+        for sfx in _kinds(case["kind"]):
+            dt = DTYPES[sfx]
+            t = np.array(case["a"], dtype=dt)
+            for op, s, side in case["steps"]:
+                t = oracle.scalar_op(op, t, s, scalar_on_left=(side == "left"))
+            assert np.array_equal(t, np.array(case["expect"], dtype=dt)), (case["source"], sfx)
+
+
+def test_reference_sigmoid_chain(vectors, oracle):
+    c = vectors["sigmoid_chain"]
+    t = np.array(c["t"], dtype=np.float32)
+    # 1 /. (1 +. exp(0 -. t))
+    e = oracle.unary("exp", oracle.scalar_op("sub", t, 0.0, scalar_on_left=True))
+    got = oracle.scalar_op("div", oracle.scalar_op("add", e, 1.0, scalar_on_left=True), 1.0, scalar_on_left=True)
+    assert np.array_equal(got, np.array(c["expect"], dtype=np.float32))
+    assert np.array_equal(oracle.unary("sigmoid", t), np.array(c["expect"], dtype=np.float32))
+
+
+def test_reference_sliced_add_sub(vectors, oracle):
+    c = vectors["sliced_add_sub"]
+    a = np.array(c["a"], dtype=np.float64)
+    for case in c["cases"]:
+        (r0, r1, _), (c0, c1, _) = case["slice"]
+        got = oracle.map2(case["op"], a[r0:r1 + 1, c0:c1 + 1], a.T[r0:r1 + 1, c0:c1 + 1])
+        assert np.array_equal(got, np.array(case["expect"], dtype=np.float64))
+
+
+def test_reference_inplace_on_transposed(vectors, oracle):
+    c = vectors["inplace_on_transposed"]
+    t = np.array(c["vandermonde"], dtype=np.float32)
+    z = t.copy().T                   # a transposed (column-major) view of its own buffer
+    assert not z.flags["C_CONTIGUOUS"]
+    oracle.map2("add", z, z, out=z)
+    assert np.array_equal(z, np.array(c["after_z_plus_z"], dtype=np.float32))
+    oracle.map2("add", z, t, out=z)
+    assert np.array_equal(z, np.array(c["after_plus_t2"], dtype=np.float32))
+
+
+def test_reference_map2_bool(vectors, oracle):
+    c = vectors["map2_bool"]
+    a, b = np.array(c["a"], dtype=np.int64), np.array(c["b"], dtype=np.int64)
+    m = oracle.map2("mod", a, b)
+    assert np.array_equal(m, np.array(c["expect_mod"]))
+    assert np.array_equal(m == 0, np.array(c["expect"]))
+
+
+def test_int_division_truncates_toward_zero(oracle):
+    a = np.array([7, -7, 7, -7, 0, 5, -2**31], dtype=np.int32)
+    b = np.array([2, 2, -2, -2, 3, 0, -1], dtype=np.int32)
+    assert oracle.map2("div", a, b).tolist() == [3, -3, -3, 3, 0, 0, -2**31]
+    assert oracle.map2("mod", a, b).tolist() == [1, -1, 1, -1, 0, 0, 0]
+    assert np.array_equal(oracle.closed_map2("div", a, b), oracle.map2("div", a, b))
+    assert np.array_equal(oracle.closed_map2("mod", a, b), oracle.map2("mod", a, b))
+
+
+def test_relu_forms(oracle):
+    x = np.array([-1.0, -0.0, 0.0, 2.5, np.nan, -np.inf, np.inf], dtype=np.float32)
+    r = oracle.unary("relu", x)
+    assert r[:4].tolist() == [0.0, 0.0, 0.0, 2.5] and not np.signbit(r[1])
+    assert np.isnan(r[4]) and r[5] == 0 and r[6] == np.inf
+    b = np.zeros_like(x)
+    assert np.array_equal(oracle.map2("add_relu", x, b), r, equal_nan=True)
+
+
+# ---- random shapes and strides against NumPy (hypothesis) ---------------------------------
+@st.composite
+def strided_pair(draw):
+    rank = draw(st.integers(1, 6))
+    shape = tuple(draw(st.integers(1, 5)) for _ in range(rank))
+    views = []
+    for _ in range(2):
+        # parent twice as large in every axis; random start / step sign / broadcast per axis
+        key, bcast = [], []
+        for n in shape:
+            mode = draw(st.sampled_from(["full", "step2", "rev", "bcast"]))
+            bcast.append(mode == "bcast")
+            key.append({"full": slice(0, n), "step2": slice(0, 2 * n, 2), "rev": slice(n - 1, None, -1),
+                        "bcast": slice(0, 1)}[mode])
+        perm = draw(st.permutations(range(rank)))
+        views.append((tuple(key), tuple(bcast), tuple(perm)))
+    return shape, views
+
+
+def _make(rng, shape, dt, spec):
+    key, bcast, perm = spec
+    pshape = tuple(2 * n for n in shape)
+    # build the parent in a permuted memory order so that inner strides are not always unit
+    parent = np.empty([pshape[p] for p in perm], dtype=dt)
+    if np.dtype(dt).kind == "f":
+        parent[...] = rng.uniform(-4, 4, parent.shape)
+    else:
+        parent[...] = rng.integers(-50, 50, parent.shape)
+    parent = parent.transpose(np.argsort(perm))
+    v = parent[key]
+    tgt = tuple(shape)
+    strides = tuple(0 if b else s for b, s in zip(bcast, v.strides))
+    return np.lib.stride_tricks.as_strided(v, shape=tgt, strides=strides, writeable=False)
+
+
+@settings(max_examples=120, deadline=None)
+@given(strided_pair(), st.sampled_from(["f32", "f64", "i32", "i64"]),
+       st.sampled_from(["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min"]), st.integers(0, 2**31))
+def test_random_strides_match_numpy(oracle, spec, sfx, op, seed):
+    shape, views = spec
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed)
+    a, b = _make(rng, shape, dt, views[0]), _make(rng, shape, dt, views[1])
+    got = oracle.map2(op, a, b)
+    want = oracle.closed_map2(op, a, b)
+    assert got.dtype == want.dtype and np.array_equal(got, want, equal_nan=True)
+
+
+def test_block_split_large(oracle):
+    """n >= 1000 takes the multi-block path of omp_parallel_blocks; result must not depend on it."""
+    rng = np.random.default_rng(1)
+    a = rng.uniform(-1, 1, (257, 129)).astype(np.float32)
+    b = rng.uniform(-1, 1, (1, 129)).astype(np.float32)
+    s = rng.uniform(-1, 1, (257, 1)).astype(np.float32)
+    ba, bb = oracle.broadcast2(a, b)
+    y = oracle.map2("add", ba, bb)
+    assert np.array_equal(y, a + b)
+    by, bs = oracle.broadcast2(y, s)
+    assert np.array_equal(oracle.map2("mul", by, bs), y * s)
+    assert np.array_equal(oracle.map2("add_relu", ba, bb), np.maximum(a + b, 0))
+
+
+def test_transcendental_bodies_close_to_numpy(oracle):
+    rng = np.random.default_rng(2)
+    for dt, tol in ((np.float32, 2e-6), (np.float64, 1e-14)):
+        a = rng.uniform(-3, 3, (33, 17)).astype(dt)
+        b = rng.uniform(-3, 3, (33, 17)).astype(dt)
+        np.testing.assert_allclose(oracle.map2("add_sigmoid", a, b), 1 / (1 + np.exp(-(a + b).astype(np.float64))), rtol=tol)
+        np.testing.assert_allclose(oracle.map2("add_tanh", a, b), np.tanh((a + b).astype(np.float64)), rtol=tol, atol=tol)
+
+
+def test_broadcast_errors(oracle):
+    with pytest.raises(ValueError):
+        oracle.broadcast2(np.zeros((3, 2)), np.zeros((2, 2)))
+    with pytest.raises(ValueError):
+        oracle.broadcast(np.zeros((3, 2)), (3, 3))
+    with pytest.raises(ValueError):
+        oracle.map2("mod", np.zeros(3, np.float32), np.zeros(3, np.float32))

@@ -1,0 +1,118 @@
+"""The HipTensor operator surface exercised the way the reference exercises its CUDA backend
+(tests/tensor/test_operators_blas_cuda.nim, test_broadcasting_cuda.nim, test_init_cuda.nim,
+test_shapeshifting_cuda.nim): small literals round-tripped toHip ... toCpu."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_round_trip_and_clone_of_reversed_slice(hip):
+    # test_init_cuda.nim:20-33: clone of a reversed slice
+    a = np.arange(1, 26, dtype=np.float64).reshape(5, 5)
+    d = hip.toHip(a)
+    assert np.array_equal(d.toCpu(), a)
+    r = d[::-1, ::-1]
+    assert np.array_equal(r.toCpu(), a[::-1, ::-1])
+    c = r.clone()
+    assert c.is_C_contiguous() and np.array_equal(c.toCpu(), a[::-1, ::-1])
+
+
+def test_gemm_gemv_literals(hip):
+    # test_operators_blas_cuda.nim:19-113
+    a = hip.toHip(np.array([[1.0, 2, 3], [4, 5, 6]]))
+    b = hip.toHip(np.array([[7.0, 8], [9, 10], [11, 12]]))
+    assert np.array_equal((a * b).toCpu(), [[58, 64], [139, 154]])
+    d = hip.toHip(np.array([[1.0, -1, 2], [0, -3, 1]]))
+    e = hip.toHip(np.array([2.0, 1, 0]))
+    assert np.array_equal((d * e).toCpu(), [1.0, -3.0])
+    c = hip.toHip(np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32))
+    with pytest.raises(IndexError):
+        c * c
+    with pytest.raises(ValueError):
+        e * a
+
+
+def test_inplace_and_out_of_place_add_sub(hip):
+    # test_operators_blas_cuda.nim:121-227
+    u = hip.toHip(np.array([1.0, 3, -5]))
+    v = hip.toHip(np.array([4.0, -2, -1]))
+    u += v
+    assert np.array_equal(u.toCpu(), [5.0, 1, -6])
+    u -= v
+    assert np.array_equal(u.toCpu(), [1.0, 3, -5])
+    assert np.array_equal((u + v).toCpu(), [5.0, 1, -6])
+    assert np.array_equal((u - v).toCpu(), [-3.0, 5, -4])
+    a = hip.toHip(np.array([7.0, 4, 3, 1, 8, 6, 8, 1, 6, 2]).reshape(5, 2))
+    b = hip.toHip(np.array([6.0, 6, 2, 0, 4, 3, 2, 0, 0, 3]).reshape(5, 2))
+    assert np.array_equal((a + b).toCpu().ravel(), [13.0, 10, 5, 1, 12, 9, 10, 1, 6, 5])
+    a -= b
+    assert np.array_equal(a.toCpu().ravel(), [1.0, -2, 1, 1, 4, 3, 6, 1, 6, -1])
+    with pytest.raises(ValueError):
+        a += b[0:2, 0:2]
+    with pytest.raises(ValueError):
+        a + b[0:2, 0:2]
+
+
+def test_scalar_mul_div(hip):
+    # test_operators_blas_cuda.nim:229-240
+    u = hip.toHip(np.array([2.0, 6, -10]))
+    assert np.array_equal((u / 2).toCpu(), [1.0, 3, -5])
+    a = hip.toHip(np.array([1, 3, -5], dtype=np.float32))
+    assert np.array_equal((2 * a).toCpu(), [2, 6, -10])
+    assert np.array_equal((a * 2).toCpu(), [2, 6, -10])
+    a *= 2
+    assert np.array_equal(a.toCpu(), [2, 6, -10])
+    a /= 2
+    assert np.array_equal(a.toCpu(), [1, 3, -5])
+
+
+def test_broadcast_literals(hip):
+    # test_broadcasting_cuda.nim:18-189
+    a = hip.toHip(np.array([0.0, 10, 20, 30]).reshape(4, 1))
+    b = hip.toHip(np.array([0.0, 1, 2]).reshape(1, 3))
+    assert np.array_equal(hip.bc_add(a, b).toCpu(), [[0, 1, 2], [10, 11, 12], [20, 21, 22], [30, 31, 32]])
+    assert np.array_equal(hip.bc_sub(a, b).toCpu(), [[0, -1, -2], [10, 9, 8], [20, 19, 18], [30, 29, 28]])
+    assert np.array_equal(hip.bc_mul(a, b).toCpu(), [[0, 0, 0], [0, 10, 20], [0, 20, 40], [0, 30, 60]])
+    c = hip.toHip(np.array([100.0, 10, 20, 30]).reshape(4, 1))
+    d = hip.toHip(np.array([2.0, 5, 10]).reshape(1, 3))
+    assert np.array_equal(hip.bc_div(c, d).toCpu(), [[50, 20, 10], [5, 2, 1], [10, 4, 2], [15, 6, 3]])
+    e = a.broadcast((4, 3)).clone()
+    e.bc_iadd(b)
+    assert np.array_equal(e.toCpu(), [[0, 1, 2], [10, 11, 12], [20, 21, 22], [30, 31, 32]])
+    assert np.array_equal(hip.bc_add(hip.bc_add(100.0, a), 200.0).toCpu().ravel(), [300, 310, 320, 330])
+    assert np.array_equal(hip.bc_sub(hip.bc_sub(100.0, a), 200.0).toCpu().ravel(), [-100, -110, -120, -130])
+
+
+def test_views_share_storage(hip):
+    # test_shapeshifting_cuda.nim:57-78 / test_accessors_slicer_cuda.nim:58-104
+    a = hip.toHip(np.arange(24, dtype=np.int32).reshape(4, 6))
+    t = a.transpose()
+    assert t.storage is a.storage
+    a[1:3, 2:5].bc_iadd(1000)
+    want = np.arange(24, dtype=np.int32).reshape(4, 6)
+    want[1:3, 2:5] += 1000
+    assert np.array_equal(a.toCpu(), want) and np.array_equal(t.toCpu(), want.T)
+    assert np.array_equal(a[::2, ::-3].toCpu(), want[::2, ::-3])
+
+
+def test_conv_as_im2col_gemm(hip, vectors):
+    """tests/nn_primitives/test_nnp_convolution.nim:21-134: im2col on the host (the reference's
+    per-image loop, fallback/conv.nim:99-103), GEMM + bias on the device."""
+    for case in vectors["conv_im2col"]:
+        for dt in (np.float32, np.int32):
+            x = np.array(case["input"], dtype=dt)[0]
+            k = np.array(case["kernel"], dtype=dt)
+            (ph, pw), (sh, sw) = case["padding"], case["stride"]
+            C, H, W = x.shape
+            Co, _, kh, kw = k.shape
+            Ho, Wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+            xp = np.zeros((C, H + 2 * ph, W + 2 * pw), dtype=dt)
+            xp[:, ph:ph + H, pw:pw + W] = x
+            col = np.empty((C * kh * kw, Ho * Wo), dtype=dt)
+            for c in range(C * kh * kw):
+                wo, ho, co = c % kw, (c // kw) % kh, c // (kw * kh)
+                col[c] = xp[co, ho:ho + sh * Ho:sh, wo:wo + sw * Wo:sw].reshape(-1)
+            out = hip.toHip(k.reshape(Co, -1)) * hip.toHip(col)
+            out.bc_iadd(hip.toHip(np.array(case["bias"], dtype=dt).reshape(Co, 1)))
+            assert np.array_equal(out.toCpu().reshape(1, Co, Ho, Wo), np.array(case["target"], dtype=dt)), case["name"]
