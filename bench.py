@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM + broadcast hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu]
+
+Prints ONE JSON line. The headline workload is the float32 GEMM C = A*B at M = N = K = 4096
+(row-major, A and B iid uniform[-1, 1) from fixed seeds, resident in HBM before the timed
+region). A step is one launch of the GEMM. `value` is TFLOP/s over the K timed steps, wall clock
+bracketed by stream synchronisation; `roofline` prices the same kernel against the MFMA fp32
+peak using HIP events recorded on the library's stream; `cpu_baseline` times the CPU restatement
+of the reference's laser gemm_strided (oracle/, OpenMP, all host cores) on the same workload.
+`others` carries the remaining configurations of the path (int32 4096^3, the float64 strided
+config, the 8192^2 broadcast ops), each with its own bound.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix peak: 256 CU x 256 FLOP/clk x 2.4 GHz
+MFMA_F64_PEAK_TFLOPS = 78.6
+HBM_PEAK_GBS = 8000.0
+# Measured separately with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), see profiles/; None = not measured.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def device_info(L):
+    name = ctypes.create_string_buffer(128)
+    cus, khz, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    hbm = ctypes.c_size_t()
+    L.am_hip_device_info(name, 128, ctypes.byref(cus), ctypes.byref(khz), ctypes.byref(hbm), ctypes.byref(lds))
+    return dict(name=name.value.decode(), compute_units=cus.value, clock_mhz=khz.value / 1000.0,
+                hbm_gib=round(hbm.value / 2**30, 1))
+
+
+class Timer:
+    """HIP events on the library stream + host wall clock around a synchronised region."""
+
+    def __init__(self, am, L):
+        self.am, self.L = am, L
+        self.e0, self.e1 = ctypes.c_void_p(), ctypes.c_void_p()
+        L.am_hip_event_create(ctypes.byref(self.e0))
+        L.am_hip_event_create(ctypes.byref(self.e1))
+
+    def run(self, fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        self.am.sync()
+        t0 = time.perf_counter()
+        self.L.am_hip_event_record(self.e0)
+        for _ in range(steps):
+            fn()
+        self.L.am_hip_event_record(self.e1)
+        self.am.sync()
+        wall = time.perf_counter() - t0
+        ms = ctypes.c_float()
+        self.L.am_hip_event_elapsed_ms(self.e0, self.e1, ctypes.byref(ms))
+        return wall, ms.value / 1e3     # seconds: wall clock for all steps, event time for all steps
+
+
+def load_traffic(key):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+
+
+def bench_gemm_f32(am, timer, steps, warmup, n=4096):
+    A = np.random.default_rng(1001).uniform(-1, 1, (n, n)).astype(np.float32)
+    B = np.random.default_rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
+    dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.float32)
+    wall, ev = timer.run(lambda: am.gemm(1.0, dA, dB, 0.0, dC), steps, warmup)
+    flops = 2.0 * n ** 3
+    return dict(wall=wall, ev=ev, flops=flops, host=(A, B))
+
+
+def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
+    """Times the oracle's blocked gemm_strided (the port of the reference's CPU algorithm) on the
+    full 4096^3 workload: one untimed run, then as many timed runs as fit the budget (>= 1)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import am_oracle
+    n = A.shape[0]
+    C = np.empty((n, n), dtype=np.float32)
+    am_oracle.gemm_strided(1.0, A, B, 0.0, C)
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while not times or (time.perf_counter() < t_end and len(times) < 20):
+        t0 = time.perf_counter()
+        am_oracle.gemm_strided(1.0, A, B, 0.0, C)
+        times.append(time.perf_counter() - t0)
+    best = min(times)
+    return dict(value=round(2.0 * n ** 3 / best / 1e12, 4), unit="TFLOP/s", cores=am_oracle.num_threads(),
+                kind="port",
+                sample=f"full workload (f32 GEMM {n}^3), best of {len(times)} runs after 1 warm-up, "
+                       f"oracle/laser_gemm.c (laser blocking, 6x16 AVX2+FMA register tile, OpenMP)")
+
+
+def other_workloads(am, timer, steps, warmup):
+    out = []
+    # --- int32 GEMM 4096^3, entries in [-100, 100], wraparound accumulate (VALU bound)
+    n = 4096
+    A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
+    B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
+    dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
+    k = max(3, steps // 4)
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+    out.append(dict(workload="i32 GEMM 4096^3 (wraparound, VALU)", unit="Top/s", dtype="i32",
+                    value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4)))
+    del dA, dB, dC
+    # --- float64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C), M=2048 N=3072 K=1024
+    pa = np.random.default_rng(3001).standard_normal((1024, 2048))
+    pb = np.random.default_rng(3002).standard_normal((1024, 6144))
+    C = np.random.default_rng(3003).standard_normal((2048, 3072))
+    dA, dB, dC = am.toHip(pa).transpose(), am.toHip(pb)[:, ::2], am.toHip(C)
+    wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, warmup)
+    fl = 2.0 * 2048 * 3072 * 1024
+    out.append(dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", unit="TFLOP/s",
+                    dtype="f64", value=round(fl * steps / wall / 1e12, 3), ms_per_step=round(ev / steps * 1e3, 4),
+                    roofline=dict(bound="mfma", achieved=round(fl / (ev / steps) / 1e12, 3), peak=MFMA_F64_PEAK_TFLOPS,
+                                  unit="TFLOP/s", frac=round(fl / (ev / steps) / 1e12 / MFMA_F64_PEAK_TFLOPS, 4))))
+    del dA, dB, dC
+    # --- broadcast ops on X[8192, 8192] f32 (HBM bound): 536 903 680 algorithmic bytes per op
+    X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
+    b = np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32)
+    s = np.random.default_rng(4003).uniform(-1, 1, (8192, 1)).astype(np.float32)
+    dX, db, ds = am.toHip(X), am.toHip(b), am.toHip(s)
+    dY = am.empty((8192, 8192), np.float32)
+    from arraymancer_amd import tensor_hip as th
+    bb = db.broadcast((8192, 8192))
+    sb = ds.broadcast((8192, 8192))
+    nbytes = 2 * 8192 * 8192 * 4 + 8192 * 4
+    for name, fn in [("X +. b[1,8192]", lambda: th._binary_into("add", dY, dX, bb)),
+                     ("Y *. s[8192,1]", lambda: th._binary_into("mul", dY, dX, sb)),
+                     ("map2(X, b, max(0, x+y)) (fused bias+ReLU)", lambda: th._binary_into("add_relu", dY, dX, bb))]:
+        wall, ev = timer.run(fn, steps, warmup)
+        gbs = nbytes / (ev / steps) / 1e9
+        out.append(dict(workload=f"f32 8192x8192 {name}", unit="GB/s", dtype="f32",
+                        value=round(nbytes * steps / wall / 1e9, 1), ms_per_step=round(ev / steps * 1e3, 4),
+                        roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                                      frac=round(gbs / HBM_PEAK_GBS, 4))))
+    return out
+
+
+def run_only(am, timer, which, steps, warmup):
+    """One workload, nothing else on the stream: what the rocprofv3 summaries under profiles/ time."""
+    from arraymancer_amd import tensor_hip as th
+    if which == "gemm_f32":
+        r = bench_gemm_f32(am, timer, steps, warmup)
+        return dict(only=which, ms_per_launch=round(r["ev"] / steps * 1e3, 4), launches=steps + warmup)
+    if which == "gemm_i32":
+        n = 4096
+        A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
+        B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
+        dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
+        fn = lambda: am.gemm(1, dA, dB, 0, dC)
+    elif which == "gemm_f64":
+        pa = np.random.default_rng(3001).standard_normal((1024, 2048))
+        pb = np.random.default_rng(3002).standard_normal((1024, 6144))
+        dA, dB = am.toHip(pa).transpose(), am.toHip(pb)[:, ::2]
+        dC = am.toHip(np.random.default_rng(3003).standard_normal((2048, 3072)))
+        fn = lambda: am.gemm(1.5, dA, dB, 0.5, dC)
+    else:
+        X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
+        dX, dY = am.toHip(X), am.empty((8192, 8192), np.float32)
+        if which == "copy":      # plain copy of known size: 268 435 456 B read + 268 435 456 B written
+            fn = lambda: th._unary_into("copy", dY, dX)
+        else:
+            b = am.toHip(np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32))
+            bb = b.broadcast((8192, 8192))
+            fn = lambda: th._binary_into("add", dY, dX, bb)
+    wall, ev = timer.run(fn, steps, warmup)
+    return dict(only=which, ms_per_launch=round(ev / steps * 1e3, 4), launches=steps + warmup)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy"],
+                    help="profiling aid: run just this workload's launches and print a short JSON line")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one MI355X; --gpus above 1 is not supported "
+              "(no collective or multi-GPU code is part of this path)", file=sys.stderr)
+        sys.exit(2)
+
+    import arraymancer_amd as am
+    L = am.load_library()
+    am.sync()
+    info = device_info(L)
+    timer = Timer(am, L)
+
+    if args.only:
+        print(json.dumps(run_only(am, timer, args.only, args.steps, args.warmup)))
+        return
+
+    r = bench_gemm_f32(am, timer, args.steps, args.warmup)
+    tflops = r["flops"] * args.steps / r["wall"] / 1e12
+    kern_tflops = r["flops"] / (r["ev"] / args.steps) / 1e12
+    line = {
+        "metric": "GEMM TFLOP/s (%MFMA peak) fp32/int32 4096^3; broadcast op HBM GB/s (%peak)",
+        "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["wall"] / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "f32 GEMM C=A*B, M=N=K=4096, row-major contiguous, uniform[-1,1) seeds 1001/1002 "
+                               "(the 4096^3 size the metric is quoted on)"},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": MFMA_F32_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(kern_tflops / MFMA_F32_PEAK_TFLOPS, 4),
+                     "traffic": load_traffic("gemm_f32_4096")},
+        "device": info,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_gemm_f32(*r["host"])
+    if not args.no_others:
+        line["others"] = other_workloads(am, timer, args.steps, args.warmup)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
