@@ -1,0 +1,121 @@
+## Raw `{.importc.}` binding of libam_hip.so (the C ABI of include/am_hip.h).
+##
+## This file is what a maintainer adds to Arraymancer (e.g. as
+## src/arraymancer/tensor/backend/hip.nim) to reach the MI355X kernels; it takes the place of
+## nimcuda + src/arraymancer/tensor/backend/{cuda,cublas,cuda_global_state}.nim.
+##
+## NOT COMPILED in the environment this repository is built in (no Nim toolchain there): every
+## signature below is mechanically the one in include/am_hip.h, whose symbols and ctypes twins are
+## checked by tests/test_abi.py.
+
+const libAmHip* {.strdefine.} = "libam_hip.so"
+
+{.push cdecl, dynlib: libAmHip.}
+
+# ---- status codes
+const
+  AM_OK* = 0.cint
+  AM_E_ARG* = -1.cint
+  AM_E_SHAPE* = -2.cint
+  AM_E_DTYPE* = -3.cint
+  AM_E_ALLOC* = -4.cint
+  AM_E_HIP* = -5.cint
+  AM_E_NODEVICE* = -6.cint
+
+# ---- runtime
+proc am_hip_last_error*(): cstring {.importc.}
+proc am_hip_version*(): cstring {.importc.}
+proc am_hip_init*(device: cint): cint {.importc.}
+proc am_hip_device_count*(count: ptr cint): cint {.importc.}
+proc am_hip_device_info*(name: cstring, name_cap: csize_t, compute_units, clock_khz: ptr cint,
+                         hbm_bytes: ptr csize_t, lds_bytes_per_cu: ptr cint): cint {.importc.}
+proc am_hip_malloc*(bytes: csize_t, dptr: ptr pointer): cint {.importc.}
+proc am_hip_free*(dptr: pointer): cint {.importc.}
+proc am_hip_memcpy_h2d*(dst, src: pointer, bytes: csize_t): cint {.importc.}
+proc am_hip_memcpy_d2h*(dst, src: pointer, bytes: csize_t): cint {.importc.}
+proc am_hip_memcpy_d2d*(dst, src: pointer, bytes: csize_t): cint {.importc.}
+proc am_hip_memset*(dst: pointer, byte_value: cint, bytes: csize_t): cint {.importc.}
+proc am_hip_sync*(): cint {.importc.}
+proc am_hip_stream*(): pointer {.importc.}
+proc am_hip_event_create*(ev: ptr pointer): cint {.importc.}
+proc am_hip_event_record*(ev: pointer): cint {.importc.}
+proc am_hip_event_elapsed_ms*(start, stop: pointer, ms: ptr cfloat): cint {.importc.}
+proc am_hip_event_destroy*(ev: pointer): cint {.importc.}
+
+# ---- GEMM (strides in elements; pointers already offset)
+proc am_hip_gemm_f32*(M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64,
+                      B: ptr cfloat, rsB, csB: int64, beta: cfloat,
+                      C: ptr cfloat, rsC, csC: int64): cint {.importc.}
+proc am_hip_gemm_f64*(M, N, K: int64, alpha: cdouble, A: ptr cdouble, rsA, csA: int64,
+                      B: ptr cdouble, rsB, csB: int64, beta: cdouble,
+                      C: ptr cdouble, rsC, csC: int64): cint {.importc.}
+proc am_hip_gemm_i32*(M, N, K: int64, alpha: int32, A: ptr int32, rsA, csA: int64,
+                      B: ptr int32, rsB, csB: int64, beta: int32,
+                      C: ptr int32, rsC, csC: int64): cint {.importc.}
+proc am_hip_gemm_i64*(M, N, K: int64, alpha: int64, A: ptr int64, rsA, csA: int64,
+                      B: ptr int64, rsB, csB: int64, beta: int64,
+                      C: ptr int64, rsC, csC: int64): cint {.importc.}
+
+const
+  AM_EPI_NONE* = 0.cint
+  AM_EPI_BIAS* = 1.cint
+  AM_EPI_RELU* = 2.cint
+  AM_EPI_BIAS_RELU* = 3.cint
+
+proc am_hip_gemm_ex_f32*(M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64,
+                         B: ptr cfloat, rsB, csB: int64, beta: cfloat,
+                         C: ptr cfloat, rsC, csC: int64,
+                         epilogue: cint, bias: ptr cfloat, bias_rs, bias_cs: int64): cint {.importc.}
+proc am_hip_gemm_ex_f64*(M, N, K: int64, alpha: cdouble, A: ptr cdouble, rsA, csA: int64,
+                         B: ptr cdouble, rsB, csB: int64, beta: cdouble,
+                         C: ptr cdouble, rsC, csC: int64,
+                         epilogue: cint, bias: ptr cdouble, bias_rs, bias_cs: int64): cint {.importc.}
+
+# ---- element-wise / broadcast / map
+type
+  AmBinaryOp* {.size: sizeof(cint).} = enum
+    opAdd = 0, opSub = 1, opMul = 2, opDiv = 3, opMod = 4, opAddRelu = 5, opAddSigmoid = 6,
+    opAddTanh = 7, opReluBwd = 8, opMax = 9, opMin = 10
+  AmUnaryOp* {.size: sizeof(cint).} = enum
+    uopCopy = 0, uopNeg = 1, uopRelu = 2, uopSigmoid = 3, uopTanh = 4, uopExp = 5, uopAbs = 6
+
+proc am_hip_ew_binary_f32*(op: cint, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
+                           a: ptr cfloat, a_strides: ptr int64, b: ptr cfloat, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_binary_f64*(op: cint, rank: cint, shape: ptr int64, dst: ptr cdouble, dst_strides: ptr int64,
+                           a: ptr cdouble, a_strides: ptr int64, b: ptr cdouble, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_binary_i32*(op: cint, rank: cint, shape: ptr int64, dst: ptr int32, dst_strides: ptr int64,
+                           a: ptr int32, a_strides: ptr int64, b: ptr int32, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_binary_i64*(op: cint, rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                           a: ptr int64, a_strides: ptr int64, b: ptr int64, b_strides: ptr int64): cint {.importc.}
+
+proc am_hip_ew_scalar_f32*(op, scalar_on_left, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
+                           a: ptr cfloat, a_strides: ptr int64, scalar: cfloat): cint {.importc.}
+proc am_hip_ew_scalar_f64*(op, scalar_on_left, rank: cint, shape: ptr int64, dst: ptr cdouble, dst_strides: ptr int64,
+                           a: ptr cdouble, a_strides: ptr int64, scalar: cdouble): cint {.importc.}
+proc am_hip_ew_scalar_i32*(op, scalar_on_left, rank: cint, shape: ptr int64, dst: ptr int32, dst_strides: ptr int64,
+                           a: ptr int32, a_strides: ptr int64, scalar: int32): cint {.importc.}
+proc am_hip_ew_scalar_i64*(op, scalar_on_left, rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                           a: ptr int64, a_strides: ptr int64, scalar: int64): cint {.importc.}
+
+proc am_hip_ew_unary_f32*(op, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
+                          a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_unary_f64*(op, rank: cint, shape: ptr int64, dst: ptr cdouble, dst_strides: ptr int64,
+                          a: ptr cdouble, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_unary_i32*(op, rank: cint, shape: ptr int64, dst: ptr int32, dst_strides: ptr int64,
+                          a: ptr int32, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_unary_i64*(op, rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                          a: ptr int64, a_strides: ptr int64): cint {.importc.}
+
+{.pop.}
+
+# ---- status -> exception, the role of nimcuda's `check` (src/arraymancer/tensor/backend/cuda.nim:27)
+type HipError* = object of CatchableError
+
+proc check*(rc: cint) {.inline.} =
+  if rc == AM_OK: return
+  let msg = $am_hip_last_error()
+  case rc
+  of AM_E_ARG, AM_E_SHAPE: raise newException(ValueError, msg)
+  of AM_E_DTYPE: raise newException(ValueError, msg)
+  of AM_E_ALLOC: raise newException(OutOfMemDefect, msg)
+  else: raise newException(HipError, msg)

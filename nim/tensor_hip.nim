@@ -1,0 +1,317 @@
+## `HipTensor`: storage backend for AMD Instinct MI355X (gfx950), enabled with `-d:hip`.
+##
+## Occupies the slot of `CudaTensor` (src/arraymancer/tensor/data_structure.nim:29-67 and the
+## `*_cuda.nim` operator files), for T in {float32, float64, int32, int64}, row-major by default,
+## arbitrary strides everywhere. All device work goes through hip_abi.nim; there is no inline
+## device code and no C++ backend requirement (`nim c` is enough).
+##
+## Hook-up inside Arraymancer (see INTEGRATION.md):
+##   tensor.nim:77-79      add  `when defined(hip): import ./tensor/tensor_hip; export tensor_hip`
+##
+## NOT COMPILED in the environment this repository is built in (no Nim toolchain there). The
+## Python twin arraymancer_amd/tensor_hip.py issues exactly the same ABI calls and is what the
+## parity tests drive.
+
+import ./hip_abi
+import arraymancer/laser/dynamic_stack_arrays      # Metadata
+import arraymancer/laser/tensor/datatypes          # Tensor[T], KnownSupportsCopyMem
+import arraymancer/tensor/data_structure            # shape_to_strides, is_C_contiguous, get_offset_ptr
+import arraymancer/tensor/init_cpu                  # newTensorUninit
+import arraymancer/tensor/shapeshifting             # asContiguous (host side, upload only)
+
+type
+  HipScalar* = float32 | float64 | int32 | int64
+
+  HipRefTrackerObj*[T: HipScalar] = object
+    value*: ptr UncheckedArray[T]
+  HipRefTracker*[T] = ref HipRefTrackerObj[T]
+
+  HipStorage*[T: HipScalar] = object
+    Flen*: int
+    Fdata*: ptr UncheckedArray[T]
+    Fref_tracking*: HipRefTracker[T]
+
+  HipTensor*[T: HipScalar] = object
+    ## Same fields as Tensor / CudaTensor: views share `storage`; shape, strides, offset in elements.
+    shape*: Metadata
+    strides*: Metadata
+    offset*: int
+    storage*: HipStorage[T]
+
+proc `=destroy`*[T](p: HipRefTrackerObj[T]) =
+  if not p.value.isNil:
+    discard am_hip_free(p.value)
+
+# ---------------------------------------------------------------- allocation / metadata
+proc newHipStorage[T: HipScalar](length: int): HipStorage[T] =
+  result.Flen = length
+  new result.Fref_tracking
+  var p: pointer
+  check am_hip_malloc(csize_t(length * sizeof(T)), p.addr)
+  result.Fdata = cast[ptr UncheckedArray[T]](p)
+  result.Fref_tracking.value = result.Fdata
+
+proc size*(t: HipTensor): int {.inline.} = t.shape.product
+proc rank*(t: HipTensor): int {.inline.} = t.shape.len
+
+proc newHipTensor*[T: HipScalar](shape: varargs[int] | Metadata): HipTensor[T] =
+  ## Row-major, uninitialised.
+  result.shape.copyFrom(shape)
+  shape_to_strides(result.shape, rowMajor, result.strides)
+  result.offset = 0
+  result.storage = newHipStorage[T](result.shape.product)
+
+proc get_offset_ptr*[T](t: HipTensor[T]): ptr T {.inline.} =
+  t.storage.Fdata[t.offset].unsafeAddr
+
+proc is_C_contiguous*(t: HipTensor): bool =
+  var cur = 1
+  for i in countdown(t.rank - 1, 0):
+    if t.shape[i] != 1 and t.strides[i] != cur: return false
+    cur *= t.shape[i]
+  true
+
+template i64s(m: Metadata): array[LASER_MAXRANK, int64] =
+  var r: array[LASER_MAXRANK, int64]
+  for i in 0 ..< m.len: r[i] = int64(m[i])
+  r
+
+# ---------------------------------------------------------------- transfers
+proc toHip*[T: HipScalar](t: Tensor[T]): HipTensor[T] =
+  ## Host -> device (the `cuda` proc, init_cuda.nim:23-41). Row-major on the device.
+  let contig = t.asContiguous(rowMajor, force = true)
+  result = newHipTensor[T](t.shape)
+  if result.size > 0:
+    check am_hip_memcpy_h2d(result.storage.Fdata, contig.get_offset_ptr, csize_t(result.size * sizeof(T)))
+
+proc toCpu*[T: HipScalar](t: HipTensor[T]): Tensor[T] =
+  ## Device -> host, blocking (the `cpu` proc, init_cuda.nim:43-59): the whole storage is copied
+  ## and shape / strides / offset are kept.
+  result = newTensorUninit[T](t.storage.Flen)
+  if t.storage.Flen > 0:
+    check am_hip_memcpy_d2h(result.get_offset_ptr, t.storage.Fdata, csize_t(t.storage.Flen * sizeof(T)))
+  result.shape = t.shape
+  result.strides = t.strides
+  result.offset = t.offset
+
+# ---------------------------------------------------------------- views (metadata only)
+proc transpose*(t: HipTensor): HipTensor =
+  t.shape.reversed(result.shape)
+  t.strides.reversed(result.strides)
+  result.offset = t.offset
+  result.storage = t.storage
+
+proc slice*[T](t: HipTensor[T], axis, first, last: int, step = 1): HipTensor[T] =
+  ## `t[.., first..last|step, ..]` on one axis (inclusive ends), the arithmetic of slicerImpl
+  ## (private/p_accessors_macros_read.nim:39-58).
+  result = t
+  result.offset += first * t.strides[axis]
+  result.strides[axis] *= step
+  result.shape[axis] = abs((last - first) div step) + 1
+
+proc broadcast*[T](t: HipTensor[T], shape: varargs[int]): HipTensor[T] =
+  ## broadcastImpl, private/p_shapeshifting.nim:76-94
+  result = t
+  doAssert t.rank == shape.len
+  for i in 0 ..< t.rank:
+    if t.shape[i] == 1:
+      if shape[i] != 1:
+        result.shape[i] = shape[i]
+        result.strides[i] = 0
+    elif t.shape[i] != shape[i]:
+      raise newException(ValueError, "The broadcasted size of the tensor must match existing size for non-singleton dimension")
+
+proc broadcast2*[T](a, b: HipTensor[T]): tuple[a, b: HipTensor[T]] =
+  ## broadcast2Impl, private/p_shapeshifting.nim:96-134
+  if a.rank != b.rank:
+    raise newException(ValueError, "Broadcasting error: ranks differ")
+  result.a = a
+  result.b = b
+  for i in 0 ..< a.rank:
+    if a.shape[i] == b.shape[i]: continue
+    if a.shape[i] == 1:
+      result.a.shape[i] = b.shape[i]; result.a.strides[i] = 0
+    elif b.shape[i] == 1:
+      result.b.shape[i] = a.shape[i]; result.b.strides[i] = 0
+    else:
+      raise newException(ValueError, "Broadcasting error: non-singleton dimensions must be the same in both tensors. Tensors' shapes were: " &
+        $a.shape & " and " & $b.shape)
+
+# ---------------------------------------------------------------- element-wise plumbing
+template ewBinary(T: typedesc, op: AmBinaryOp, dst, a, b: untyped) =
+  var sh = i64s(dst.shape)
+  var sd = i64s(dst.strides)
+  var sa = i64s(a.strides)
+  var sb = i64s(b.strides)
+  when T is float32:
+    check am_hip_ew_binary_f32(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+  elif T is float64:
+    check am_hip_ew_binary_f64(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+  elif T is int32:
+    check am_hip_ew_binary_i32(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+  else:
+    check am_hip_ew_binary_i64(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+
+template ewScalar(T: typedesc, op: AmBinaryOp, left: bool, dst, a: untyped, s: untyped) =
+  var sh = i64s(dst.shape)
+  var sd = i64s(dst.strides)
+  var sa = i64s(a.strides)
+  when T is float32:
+    check am_hip_ew_scalar_f32(cint(op), cint(left), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+  elif T is float64:
+    check am_hip_ew_scalar_f64(cint(op), cint(left), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+  elif T is int32:
+    check am_hip_ew_scalar_i32(cint(op), cint(left), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+  else:
+    check am_hip_ew_scalar_i64(cint(op), cint(left), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+
+template ewUnary(T: typedesc, op: AmUnaryOp, dst, a: untyped) =
+  var sh = i64s(dst.shape)
+  var sd = i64s(dst.strides)
+  var sa = i64s(a.strides)
+  when T is float32:
+    check am_hip_ew_unary_f32(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr)
+  elif T is float64:
+    check am_hip_ew_unary_f64(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr)
+  elif T is int32:
+    check am_hip_ew_unary_i32(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr)
+  else:
+    check am_hip_ew_unary_i64(cint(op), cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr)
+
+proc check_elementwise(a, b: HipTensor) =
+  if a.shape != b.shape:
+    raise newException(ValueError, "Both Tensors should have the same shape. Left-hand side has shape " &
+      $a.shape & " while right-hand side has shape " & $b.shape)
+
+proc map2*[T](a: HipTensor[T], op: AmBinaryOp, b: HipTensor[T]): HipTensor[T] =
+  ## map2_inline with an enumerated body (a C ABI cannot carry a Nim expression).
+  check_elementwise(a, b)
+  result = newHipTensor[T](a.shape)
+  if result.size > 0: ewBinary(T, op, result, a, b)
+
+proc apply2*[T](dest: var HipTensor[T], op: AmBinaryOp, src: HipTensor[T]) =
+  check_elementwise(dest, src)
+  if dest.size > 0: ewBinary(T, op, dest, dest, src)
+
+proc clone*[T](t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewUnary(T, uopCopy, result, t)
+
+# ---------------------------------------------------------------- BLAS L1-like operators
+proc `+`*[T](a, b: HipTensor[T]): HipTensor[T] = map2(a, opAdd, b)
+proc `-`*[T](a, b: HipTensor[T]): HipTensor[T] = map2(a, opSub, b)
+proc `+=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opAdd, b)
+proc `-=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opSub, b)
+
+proc `*`*[T](s: T, t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opMul, true, result, t, s)
+proc `*`*[T](t: HipTensor[T], s: T): HipTensor[T] = s * t
+proc `/`*[T](t: HipTensor[T], s: T): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opDiv, false, result, t, s)
+proc `*=`*[T](t: var HipTensor[T], s: T) =
+  if t.size > 0: ewScalar(T, opMul, false, t, t, s)
+proc `/=`*[T](t: var HipTensor[T], s: T) =
+  if t.size > 0: ewScalar(T, opDiv, false, t, t, s)
+
+# ---------------------------------------------------------------- broadcasting operators
+proc `+.`*[T](a, b: HipTensor[T]): HipTensor[T] =
+  let (ta, tb) = broadcast2(a, b)
+  ta + tb
+proc `-.`*[T](a, b: HipTensor[T]): HipTensor[T] =
+  let (ta, tb) = broadcast2(a, b)
+  ta - tb
+proc `*.`*[T](a, b: HipTensor[T]): HipTensor[T] =
+  let (ta, tb) = broadcast2(a, b)
+  map2(ta, opMul, tb)
+proc `/.`*[T](a, b: HipTensor[T]): HipTensor[T] =
+  let (ta, tb) = broadcast2(a, b)
+  map2(ta, opDiv, tb)       # integers: truncating `div`
+proc `mod`*[T: int32 | int64](a, b: HipTensor[T]): HipTensor[T] =
+  let (ta, tb) = broadcast2(a, b)
+  map2(ta, opMod, tb)
+
+proc `+.=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opAdd, b.broadcast(a.shape.toSeq))
+proc `-.=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opSub, b.broadcast(a.shape.toSeq))
+proc `*.=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opMul, b.broadcast(a.shape.toSeq))
+proc `/.=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opDiv, b.broadcast(a.shape.toSeq))
+
+proc `+.`*[T](t: HipTensor[T], s: T): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opAdd, false, result, t, s)
+proc `+.`*[T](s: T, t: HipTensor[T]): HipTensor[T] = t +. s
+proc `-.`*[T](t: HipTensor[T], s: T): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opSub, false, result, t, s)
+proc `-.`*[T](s: T, t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opSub, true, result, t, s)
+proc `*.`*[T](t: HipTensor[T], s: T): HipTensor[T] = s * t
+proc `*.`*[T](s: T, t: HipTensor[T]): HipTensor[T] = s * t
+proc `/.`*[T](t: HipTensor[T], s: T): HipTensor[T] = t / s
+proc `/.`*[T](s: T, t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opDiv, true, result, t, s)
+
+proc relu*[T: float32 | float64](t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewUnary(T, uopRelu, result, t)
+
+proc biasRelu*[T: float32 | float64](x, b: HipTensor[T]): HipTensor[T] =
+  ## map2_inline(x, b.broadcast(x.shape), max(0.T, x + y)) in one pass.
+  map2(x, opAddRelu, b.broadcast(x.shape.toSeq))
+
+# ---------------------------------------------------------------- GEMM
+proc gemm*[T: HipScalar](alpha: T, A, B: HipTensor[T], beta: T, C: var HipTensor[T]) =
+  ## C <- alpha A B + beta C (operators_blas_l2l3.nim:58-81). Any strides; no host copy.
+  if A.rank != 2 or B.rank != 2 or C.rank != 2:
+    raise newException(ValueError, "gemm: A, B and C must be matrices")
+  when compileOption("boundChecks"):
+    if A.shape[1] != B.shape[0]:
+      raise newException(IndexDefect, "Number of columns in the first matrix: " & $A.shape[1] &
+        ", must be the same as the number of rows in the second matrix: " & $B.shape[0])
+  let (M, N, K) = (int64 A.shape[0], int64 B.shape[1], int64 A.shape[1])
+  template call(f: untyped) =
+    check f(M, N, K, alpha, A.get_offset_ptr, int64 A.strides[0], int64 A.strides[1],
+            B.get_offset_ptr, int64 B.strides[0], int64 B.strides[1], beta,
+            C.get_offset_ptr, int64 C.strides[0], int64 C.strides[1])
+  when T is float32: call am_hip_gemm_f32
+  elif T is float64: call am_hip_gemm_f64
+  elif T is int32: call am_hip_gemm_i32
+  else: call am_hip_gemm_i64
+
+proc `*`*[T: HipScalar](a, b: HipTensor[T]): HipTensor[T] =
+  ## Matrix-matrix product (operators_blas_l2l3.nim:88-100). Matrix-vector runs as an N = 1 product.
+  if a.rank == 2 and b.rank == 2:
+    result = newHipTensor[T]([a.shape[0], b.shape[1]])
+    gemm(T(1), a, b, T(0), result)
+  elif a.rank == 2 and b.rank == 1:
+    result = newHipTensor[T]([a.shape[0]])
+    var bcol = b
+    bcol.shape.add 1; bcol.strides.add 1
+    var ocol = result
+    ocol.shape.add 1; ocol.strides.add 1
+    gemm(T(1), a, bcol, T(0), ocol)
+  else:
+    raise newException(ValueError, "Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a Matrix and second is a Matrix or Vector")
+
+proc linear*[T: float32 | float64](x, weight, bias: HipTensor[T], relu = false): HipTensor[T] =
+  ## out = x * weight.transpose +. bias (then relu): nnp_linear.nim:20-29 + nnp_activation.nim:35-36
+  ## as ONE kernel (fused GEMM epilogue).
+  result = newHipTensor[T]([x.shape[0], weight.shape[0]])
+  let wt = weight.transpose
+  let bb = bias.broadcast(result.shape.toSeq)
+  let epi = if relu: AM_EPI_BIAS_RELU else: AM_EPI_BIAS
+  when T is float32:
+    check am_hip_gemm_ex_f32(int64 x.shape[0], int64 wt.shape[1], int64 x.shape[1], 1'f32,
+      x.get_offset_ptr, int64 x.strides[0], int64 x.strides[1],
+      wt.get_offset_ptr, int64 wt.strides[0], int64 wt.strides[1], 0'f32,
+      result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
+      epi, bb.get_offset_ptr, int64 bb.strides[0], int64 bb.strides[1])
+  else:
+    check am_hip_gemm_ex_f64(int64 x.shape[0], int64 wt.shape[1], int64 x.shape[1], 1'f64,
+      x.get_offset_ptr, int64 x.strides[0], int64 x.strides[1],
+      wt.get_offset_ptr, int64 wt.strides[0], int64 wt.strides[1], 0'f64,
+      result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
+      epi, bb.get_offset_ptr, int64 bb.strides[0], int64 bb.strides[1])
