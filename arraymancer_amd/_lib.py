@@ -8,7 +8,8 @@ import os
 import numpy as np
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG_DIR, "libam_hip.so")
+# AM_HIP_LIBRARY overrides the location of the built library (same role as -d:libAmHip=... in Nim).
+LIB_PATH = os.environ.get("AM_HIP_LIBRARY") or os.path.join(PKG_DIR, "libam_hip.so")
 
 AM_OK, AM_E_ARG, AM_E_SHAPE, AM_E_DTYPE, AM_E_ALLOC, AM_E_HIP, AM_E_NODEVICE = 0, -1, -2, -3, -4, -5, -6
 AM_MAXRANK = 6
@@ -54,6 +55,7 @@ def _signatures():
         "am_hip_event_record": (ci, [vp]),
         "am_hip_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),
         "am_hip_event_destroy": (ci, [vp]),
+        "am_hip_diag_peak": (ci, [ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
     }
     for sfx, ct in CTYPE.items():
         gemm = [i64, i64, i64, ct, vp, i64, i64, vp, i64, i64, ct, vp, i64, i64]

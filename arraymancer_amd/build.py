@@ -18,7 +18,7 @@ OBJ_DIR = os.path.join(CSRC, "_obj")
 LIB_PATH = os.path.join(PKG_DIR, "libam_hip.so")
 
 SOURCES = [
-    "runtime.hip",
+    "runtime.hip", "diag.hip",
     "elementwise_f32.hip", "elementwise_f64.hip", "elementwise_i32.hip", "elementwise_i64.hip",
     "gemm_f32.hip", "gemm_f64.hip", "gemm_i32.hip", "gemm_i64.hip",
 ]
@@ -31,7 +31,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
-]
+] + os.environ.get("AM_HIP_EXTRA_FLAGS", "").split()
 
 
 def _hipcc() -> str:

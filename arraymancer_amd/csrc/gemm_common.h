@@ -97,12 +97,32 @@ static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int6
   int best = 0;
   double best_cost = 0;
   for (int i = 0; i < ncand; ++i) {
+    if (cand[i].eff <= 0) continue;   // experimental shape: only when forced
     const int64_t tiles = ((M + cand[i].bm - 1) / cand[i].bm) * ((N + cand[i].bn - 1) / cand[i].bn);
     const int64_t rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * cand[i].bm * cand[i].bn / cand[i].eff;
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
   }
   return best;
+}
+
+// Workgroup id -> (tile_m, tile_n).
+//  1. Hardware deals consecutive workgroup ids round-robin to the 8 XCDs (each with its own L2):
+//     id -> (id mod 8) * (n / 8) + id div 8 hands every XCD one contiguous run of tile numbers.
+//  2. Tile numbers walk the grid in groups of kGroupM tile rows, column by column inside a group,
+//     so the tiles an XCD works on at any moment form a roughly square patch: fewer distinct A and
+//     B panels per XCD, hence fewer fetches into its L2.
+constexpr int kGroupM = 8;
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+  const int nb = tiles_m * tiles_n;
+  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+  const int in_group = kGroupM * tiles_n;
+  const int group = bid / in_group;
+  const int first_m = group * kGroupM;
+  const int rows = (tiles_m - first_m < kGroupM) ? tiles_m - first_m : kGroupM;
+  const int r = bid - group * in_group;
+  tile_m = first_m + r % rows;
+  tile_n = r / rows;
 }
 
 }  // namespace gemm

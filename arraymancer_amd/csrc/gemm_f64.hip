@@ -8,11 +8,13 @@ static int run_f64(Args<double>& g) {
   const int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   const int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
   // Candidate workgroup tiles, largest first, with the relative MFMA efficiency of each.
-  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.7}, {32, 32, 0.4}};
-  switch (choose_tile(cand, 3, g.M, g.N, "AM_HIP_GEMM_TILE_F64")) {
+  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.98}, {32, 32, 0.8}, {256, 128, 0.96}, {128, 64, 0.97}};
+  switch (choose_tile(cand, 5, g.M, g.N, "AM_HIP_GEMM_TILE_F64")) {
     case 0: return launch_kinds<double, 128, 128, 16, 2, 2>(g, ak, bk);
     case 1: return launch_kinds<double, 64, 64, 16, 2, 2>(g, ak, bk);
-    default: return launch_kinds<double, 32, 32, 16, 2, 2>(g, ak, bk);
+    case 2: return launch_kinds<double, 32, 32, 16, 2, 2>(g, ak, bk);
+    case 3: return launch_kinds<double, 256, 128, 16, 4, 2>(g, ak, bk);
+    default: return launch_kinds<double, 128, 64, 16, 2, 2>(g, ak, bk);
   }
 }
 

@@ -15,7 +15,7 @@ extern "C" int am_hip_gemm_i32(int64_t M, int64_t N, int64_t K, int32_t alpha, c
   AM_TRY(ensure_init());
   const int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   const int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
-  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.6}};
+  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 1.0}};
   switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_GEMM_TILE_I32")) {
     case 0: return launch_valu<int32_t, 8, 8, 16>(g, ak, bk);
     default: return launch_valu<int32_t, 4, 4, 16>(g, ak, bk);

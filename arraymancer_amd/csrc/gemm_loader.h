@@ -21,7 +21,12 @@ template <> struct VecTraits<int64_t> { static constexpr int VK = 2; typedef int
 // LDS geometry of one operand slab (BMN rows/cols x BK k values).
 template <typename T, int KIND, int BMN, int BK, bool KG = true> struct Slab {
   static constexpr int VK = VecTraits<T>::VK;
-  static constexpr int LDKG = BMN + 4;   // k-group layout: 16-byte slots per k-group plane
+  // Padding of the k-group planes. A 16-byte LDS access is served 8 lanes at a time (8 x 16 B =
+  // all 32 banks); the 8 lanes of a global->LDS write step through the BK/VK k-groups of a row
+  // first, so consecutive planes must start 8/(BK/VK) slots apart modulo 8 to spread them over
+  // the banks (measured on f64: +7 % over a padding that is a multiple of 4).
+  static constexpr int QN_ = BK / VK;
+  static constexpr int LDKG = BMN + (QN_ >= 8 ? 1 : 8 / QN_);   // 16-byte slots per k-group plane
   static constexpr int LDMN = BMN + 8;   // k-row layout: elements per k row
   static constexpr int ELEMS = (KIND == kKContig && KG) ? (BK / VK) * LDKG * VK : BK * LDMN;
 };

@@ -92,12 +92,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
   __shared__ __attribute__((aligned(16))) T sA[2][A_ELEMS];
   __shared__ __attribute__((aligned(16))) T sB[2][B_ELEMS];
 
-  // Workgroup -> tile. Hardware deals consecutive workgroup ids round-robin to the 8 XCDs; give
-  // each XCD a contiguous band of tile rows so that its private L2 sees the same A/B panels.
-  int bid = blockIdx.x;
-  const int nb = p.tiles_m * p.tiles_n;
-  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
-  const int tile_m = bid / p.tiles_n, tile_n = bid - tile_m * p.tiles_n;
+  int tile_m, tile_n;
+  tile_of_block((int)blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -138,16 +134,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
       for (int i = 0; i < TM; ++i) read_frag<T, AK, BM, BK>(a_lds, wave_m * WM + i * TILE + lrow, ks, kl, af[i]);
 #pragma unroll
       for (int j = 0; j < TN; ++j) read_frag<T, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[j]);
+      // The other LDS buffer has been free since the barrier that ended the previous slab, so the
+      // next slab is written into it in the middle of this slab's MFMA stream (before the last
+      // k-step) instead of after it: the wait for the global loads and the LDS writes then overlap
+      // with matrix-core work still queued, and only the barrier is left at the end of the slab.
+      if (ks == BK / KSTEP - 1 && more) {
+        la.commit(sA[cur ^ 1]);
+        lb.commit(sB[cur ^ 1]);
+      }
 #pragma unroll
       for (int s = 0; s < VK; ++s)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[i][s], bf[j][s], acc[i][j]);
-    }
-    if (more) {
-      la.commit(sA[cur ^ 1]);
-      lb.commit(sB[cur ^ 1]);
     }
     __syncthreads();
   }

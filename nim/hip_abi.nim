@@ -42,6 +42,8 @@ proc am_hip_event_record*(ev: pointer): cint {.importc.}
 proc am_hip_event_elapsed_ms*(start, stop: pointer, ms: ptr cfloat): cint {.importc.}
 proc am_hip_event_destroy*(ev: pointer): cint {.importc.}
 
+proc am_hip_diag_peak*(kind, iters, waves_per_simd: cint, ops_per_second: ptr cdouble): cint {.importc.}
+
 # ---- GEMM (strides in elements; pointers already offset)
 proc am_hip_gemm_f32*(M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64,
                       B: ptr cfloat, rsB, csB: int64, beta: cfloat,
