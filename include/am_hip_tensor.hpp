@@ -1,0 +1,349 @@
+// am_hip_tensor.hpp — header-only C++ host layer over the C ABI of am_hip.h.
+//
+// The reference is written in Nim (a compiled language whose toolchain is not available where this
+// repository is built), so the compiled host-side mirror of its GPU tensor backend is given in
+// C++: `am::HipTensor<T>` has the fields and operator set of `CudaTensor`
+// (src/arraymancer/tensor/data_structure.nim:29-67; operators_blas_l2l3_cuda.nim,
+// operators_blas_l1_cuda.nim, operators_broadcasted_cuda.nim, shapeshifting_cuda.nim,
+// init_cuda.nim) for float, double, int32_t and int64_t, row-major by default, any strides.
+// Every operation is exactly one call into libam_hip.so; nothing is computed on the host.
+//
+//   reference                         here
+//   t.cuda / t.cpu                    am::toHip(ptr, shape) / t.toCpu()
+//   a * b, gemm(alpha, A, B, beta, C) a * b, am::gemm(alpha, A, B, beta, C)
+//   a + b, a - b, a += b, a -= b      same
+//   s * t, t * s, t / s               same
+//   a +. b, a -. b, a *. b, a /. b    am::bc_add / bc_sub / bc_mul / bc_div   (also tensor-scalar)
+//   a +.= b ...                       a.bc_iadd(b) / bc_isub / bc_imul / bc_idiv
+//   t.transpose, t[a..b|s, ...]       t.transpose(), t.slice(axis, first, last, step)
+//   t.broadcast(shape)                t.broadcast(shape)
+// Errors: std::invalid_argument where the reference raises ValueError, std::out_of_range where it
+// raises IndexDefect, am::HipError for device failures.
+#pragma once
+#include <cstdint>
+#include <cstdlib>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "am_hip.h"
+
+namespace am {
+
+struct HipError : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+inline void check(int rc) {
+  if (rc == AM_OK) return;
+  const std::string msg = am_hip_last_error();
+  if (rc == AM_E_ARG || rc == AM_E_SHAPE || rc == AM_E_DTYPE) throw std::invalid_argument(msg);
+  if (rc == AM_E_ALLOC) throw std::bad_alloc();
+  throw HipError(msg);
+}
+
+using Shape = std::vector<int64_t>;
+
+namespace detail {
+// One overload set per element type keeps the templates below free of dispatch code.
+#define AM_HPP_BIND(T, SFX)                                                                              \
+  inline int gemm_(int64_t M, int64_t N, int64_t K, T al, const T* A, int64_t ra, int64_t ca, const T* B, \
+                   int64_t rb, int64_t cb, T be, T* C, int64_t rc, int64_t cc) {                         \
+    return am_hip_gemm_##SFX(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc);                           \
+  }                                                                                                      \
+  inline int binary_(int op, int rank, const int64_t* sh, T* d, const int64_t* sd, const T* a,           \
+                     const int64_t* sa, const T* b, const int64_t* sb) {                                 \
+    return am_hip_ew_binary_##SFX(op, rank, sh, d, sd, a, sa, b, sb);                                     \
+  }                                                                                                      \
+  inline int scalar_(int op, int left, int rank, const int64_t* sh, T* d, const int64_t* sd, const T* a, \
+                     const int64_t* sa, T s) {                                                           \
+    return am_hip_ew_scalar_##SFX(op, left, rank, sh, d, sd, a, sa, s);                                   \
+  }                                                                                                      \
+  inline int unary_(int op, int rank, const int64_t* sh, T* d, const int64_t* sd, const T* a,            \
+                    const int64_t* sa) {                                                                 \
+    return am_hip_ew_unary_##SFX(op, rank, sh, d, sd, a, sa);                                             \
+  }
+AM_HPP_BIND(float, f32)
+AM_HPP_BIND(double, f64)
+AM_HPP_BIND(int32_t, i32)
+AM_HPP_BIND(int64_t, i64)
+#undef AM_HPP_BIND
+inline int gemm_ex_(int64_t M, int64_t N, int64_t K, float al, const float* A, int64_t ra, int64_t ca,
+                    const float* B, int64_t rb, int64_t cb, float be, float* C, int64_t rc, int64_t cc, int epi,
+                    const float* bias, int64_t brs, int64_t bcs) {
+  return am_hip_gemm_ex_f32(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc, epi, bias, brs, bcs);
+}
+inline int gemm_ex_(int64_t M, int64_t N, int64_t K, double al, const double* A, int64_t ra, int64_t ca,
+                    const double* B, int64_t rb, int64_t cb, double be, double* C, int64_t rc, int64_t cc, int epi,
+                    const double* bias, int64_t brs, int64_t bcs) {
+  return am_hip_gemm_ex_f64(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc, epi, bias, brs, bcs);
+}
+
+inline std::string str(const Shape& s) {
+  std::string r = "[";
+  for (size_t i = 0; i < s.size(); ++i) r += (i ? ", " : "") + std::to_string(s[i]);
+  return r + "]";
+}
+}  // namespace detail
+
+// Device allocation shared by every view of it; freed with the last view
+// (the role of CudaTensorRefTracker, data_structure.nim:29-67).
+template <typename T>
+struct HipStorage {
+  T* data = nullptr;
+  int64_t len = 0;
+  explicit HipStorage(int64_t n) : len(n) {
+    void* p = nullptr;
+    check(am_hip_malloc((size_t)n * sizeof(T), &p));
+    data = static_cast<T*>(p);
+  }
+  ~HipStorage() { am_hip_free(data); }
+  HipStorage(const HipStorage&) = delete;
+  HipStorage& operator=(const HipStorage&) = delete;
+};
+
+template <typename T>
+class HipTensor {
+  static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value ||
+                    std::is_same<T, int32_t>::value || std::is_same<T, int64_t>::value,
+                "HipTensor supports float, double, int32_t and int64_t");
+
+ public:
+  Shape shape, strides;     // elements
+  int64_t offset = 0;
+  std::shared_ptr<HipStorage<T>> storage;
+
+  HipTensor() = default;
+  // newTensorUninit: row-major, uninitialised.
+  explicit HipTensor(const Shape& shp) : shape(shp), strides(shp.size()) {
+    if (shp.size() > AM_MAXRANK) throw std::invalid_argument("rank exceeds " + std::to_string(AM_MAXRANK));
+    int64_t acc = 1;
+    for (int i = (int)shp.size() - 1; i >= 0; --i) { strides[i] = acc; acc *= shp[i]; }
+    storage = std::make_shared<HipStorage<T>>(acc);
+  }
+
+  int rank() const { return (int)shape.size(); }
+  int64_t size() const { int64_t n = 1; for (auto s : shape) n *= s; return n; }
+  T* ptr() const { return storage->data + offset; }   // get_offset_ptr
+
+  bool is_C_contiguous() const {
+    int64_t cur = 1;
+    for (int i = rank() - 1; i >= 0; --i) {
+      if (shape[i] != 1 && strides[i] != cur) return false;
+      cur *= shape[i];
+    }
+    return true;
+  }
+
+  // ---- views: metadata only, storage shared -------------------------------------------------
+  HipTensor transpose() const {   // shapeshifting.nim:27-36
+    HipTensor r = *this;
+    r.shape.assign(shape.rbegin(), shape.rend());
+    r.strides.assign(strides.rbegin(), strides.rend());
+    return r;
+  }
+  // t[.., first..last|step, ..] on one axis, inclusive ends (p_accessors_macros_read.nim:39-58).
+  HipTensor slice(int axis, int64_t first, int64_t last, int64_t step = 1) const {
+    if (axis < 0 || axis >= rank()) throw std::out_of_range("slice: axis out of range");
+    if (first < 0 || first >= shape[axis] || last < 0 || last >= shape[axis] || step == 0 ||
+        (first < last && step < 0) || (first > last && step > 0))
+      throw std::out_of_range("slice " + std::to_string(first) + ".." + std::to_string(last) + "|" +
+                              std::to_string(step) + " invalid for extent " + std::to_string(shape[axis]));
+    HipTensor r = *this;
+    r.offset += first * strides[axis];
+    r.strides[axis] *= step;
+    r.shape[axis] = std::llabs(last - first) / std::llabs(step) + 1;
+    return r;
+  }
+  HipTensor broadcast(const Shape& shp) const {   // p_shapeshifting.nim:76-94
+    if ((int)shp.size() != rank()) throw std::invalid_argument("broadcast: ranks differ");
+    HipTensor r = *this;
+    for (int i = 0; i < rank(); ++i) {
+      if (shape[i] == 1) {
+        if (shp[i] != 1) { r.shape[i] = shp[i]; r.strides[i] = 0; }
+      } else if (shape[i] != shp[i]) {
+        throw std::invalid_argument("The broadcasted size of the tensor " + detail::str(shp) +
+                                    ", must match existing size " + detail::str(shape) +
+                                    " for non-singleton dimension");
+      }
+    }
+    return r;
+  }
+
+  // ---- transfers ----------------------------------------------------------------------------
+  // Blocking copy of the logical contents in C order (a device-side gather first if strided).
+  std::vector<T> toCpu() const {
+    const HipTensor c = is_C_contiguous() ? *this : clone();
+    std::vector<T> host((size_t)size());
+    if (!host.empty()) check(am_hip_memcpy_d2h(host.data(), c.ptr(), host.size() * sizeof(T)));
+    return host;
+  }
+  HipTensor clone() const {
+    HipTensor r(shape);
+    if (size() > 0) check(detail::unary_(AM_UOP_COPY, rank(), shape.data(), r.ptr(), r.strides.data(), ptr(), strides.data()));
+    return r;
+  }
+
+  // ---- in-place forms -------------------------------------------------------------------------
+  HipTensor& operator+=(const HipTensor& b) { return apply2(AM_OP_ADD, b); }
+  HipTensor& operator-=(const HipTensor& b) { return apply2(AM_OP_SUB, b); }
+  HipTensor& operator*=(T s) { return apply_scalar(AM_OP_MUL, s); }
+  HipTensor& operator/=(T s) { return apply_scalar(AM_OP_DIV, s); }
+  // only the right-hand side may be broadcast (operators_broadcasted.nim:65-102)
+  HipTensor& bc_iadd(const HipTensor& b) { return apply2(AM_OP_ADD, b.broadcast(shape)); }
+  HipTensor& bc_isub(const HipTensor& b) { return apply2(AM_OP_SUB, b.broadcast(shape)); }
+  HipTensor& bc_imul(const HipTensor& b) { return apply2(AM_OP_MUL, b.broadcast(shape)); }
+  HipTensor& bc_idiv(const HipTensor& b) { return apply2(AM_OP_DIV, b.broadcast(shape)); }
+
+  // apply2_inline (higher_order_applymap.nim:40-47) with an enumerated body.
+  HipTensor& apply2(int op, const HipTensor& src) {
+    if (shape != src.shape)
+      throw std::invalid_argument("Both Tensors should have the same shape. Left-hand side has shape " +
+                                  detail::str(shape) + " while right-hand side has shape " + detail::str(src.shape));
+    if (size() > 0)
+      check(detail::binary_(op, rank(), shape.data(), ptr(), strides.data(), ptr(), strides.data(), src.ptr(), src.strides.data()));
+    return *this;
+  }
+  HipTensor& apply_scalar(int op, T s) {
+    if (size() > 0) check(detail::scalar_(op, 0, rank(), shape.data(), ptr(), strides.data(), ptr(), strides.data(), s));
+    return *this;
+  }
+};
+
+// ---- construction -----------------------------------------------------------------------------
+template <typename T>
+HipTensor<T> toHip(const T* host, const Shape& shape) {   // init_cuda.nim:23-41, row-major here
+  HipTensor<T> t(shape);
+  if (t.size() > 0) check(am_hip_memcpy_h2d(t.ptr(), host, (size_t)t.size() * sizeof(T)));
+  return t;
+}
+template <typename T>
+HipTensor<T> toHip(const std::vector<T>& host, const Shape& shape) {
+  HipTensor<T> probe;   // shape check without allocating
+  int64_t n = 1;
+  for (auto s : shape) n *= s;
+  if ((int64_t)host.size() != n) throw std::invalid_argument("toHip: " + std::to_string(host.size()) + " values for shape " + detail::str(shape));
+  return toHip(host.data(), shape);
+}
+
+// ---- map2 / operators ---------------------------------------------------------------------------
+template <typename T>
+HipTensor<T> map2(int op, const HipTensor<T>& a, const HipTensor<T>& b) {   // map2_inline, :92-120
+  if (a.shape != b.shape)
+    throw std::invalid_argument("Both Tensors should have the same shape. Left-hand side has shape " +
+                                detail::str(a.shape) + " while right-hand side has shape " + detail::str(b.shape));
+  HipTensor<T> r(a.shape);
+  if (r.size() > 0)
+    check(detail::binary_(op, r.rank(), r.shape.data(), r.ptr(), r.strides.data(), a.ptr(), a.strides.data(), b.ptr(), b.strides.data()));
+  return r;
+}
+template <typename T>
+HipTensor<T> scalar_op(int op, const HipTensor<T>& t, T s, bool scalar_on_left = false) {
+  HipTensor<T> r(t.shape);
+  if (r.size() > 0)
+    check(detail::scalar_(op, scalar_on_left ? 1 : 0, r.rank(), r.shape.data(), r.ptr(), r.strides.data(), t.ptr(), t.strides.data(), s));
+  return r;
+}
+template <typename T>
+HipTensor<T> unary(int op, const HipTensor<T>& t) {
+  HipTensor<T> r(t.shape);
+  if (r.size() > 0) check(detail::unary_(op, r.rank(), r.shape.data(), r.ptr(), r.strides.data(), t.ptr(), t.strides.data()));
+  return r;
+}
+
+template <typename T> HipTensor<T> operator+(const HipTensor<T>& a, const HipTensor<T>& b) { return map2(AM_OP_ADD, a, b); }
+template <typename T> HipTensor<T> operator-(const HipTensor<T>& a, const HipTensor<T>& b) { return map2(AM_OP_SUB, a, b); }
+template <typename T> HipTensor<T> operator*(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_MUL, t, s); }
+template <typename T> HipTensor<T> operator*(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_MUL, t, s, true); }
+template <typename T> HipTensor<T> operator/(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_DIV, t, s); }
+template <typename T> HipTensor<T> relu(const HipTensor<T>& t) { return unary(AM_UOP_RELU, t); }
+
+// broadcast2Impl, p_shapeshifting.nim:96-134
+template <typename T>
+std::pair<HipTensor<T>, HipTensor<T>> broadcast2(const HipTensor<T>& a, const HipTensor<T>& b) {
+  if (a.rank() != b.rank()) throw std::invalid_argument("Broadcasting error: ranks differ");
+  HipTensor<T> ra = a, rb = b;
+  for (int i = 0; i < a.rank(); ++i) {
+    if (a.shape[i] == b.shape[i]) continue;
+    if (a.shape[i] == 1) { ra.shape[i] = b.shape[i]; ra.strides[i] = 0; }
+    else if (b.shape[i] == 1) { rb.shape[i] = a.shape[i]; rb.strides[i] = 0; }
+    else
+      throw std::invalid_argument("Broadcasting error: non-singleton dimensions must be the same in both tensors. "
+                                  "Tensors' shapes were: " + detail::str(a.shape) + " and " + detail::str(b.shape));
+  }
+  return {ra, rb};
+}
+template <typename T> HipTensor<T> bc(int op, const HipTensor<T>& a, const HipTensor<T>& b) {
+  auto p = broadcast2(a, b);
+  return map2(op, p.first, p.second);
+}
+template <typename T> HipTensor<T> bc_add(const HipTensor<T>& a, const HipTensor<T>& b) { return bc(AM_OP_ADD, a, b); }   // +.
+template <typename T> HipTensor<T> bc_sub(const HipTensor<T>& a, const HipTensor<T>& b) { return bc(AM_OP_SUB, a, b); }   // -.
+template <typename T> HipTensor<T> bc_mul(const HipTensor<T>& a, const HipTensor<T>& b) { return bc(AM_OP_MUL, a, b); }   // *.
+template <typename T> HipTensor<T> bc_div(const HipTensor<T>& a, const HipTensor<T>& b) { return bc(AM_OP_DIV, a, b); }   // /.
+template <typename T> HipTensor<T> bc_mod(const HipTensor<T>& a, const HipTensor<T>& b) { return bc(AM_OP_MOD, a, b); }   // mod
+template <typename T> HipTensor<T> bc_add(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_ADD, t, s); }
+template <typename T> HipTensor<T> bc_add(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_ADD, t, s, true); }
+template <typename T> HipTensor<T> bc_sub(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_SUB, t, s); }
+template <typename T> HipTensor<T> bc_sub(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_SUB, t, s, true); }
+template <typename T> HipTensor<T> bc_mul(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_MUL, t, s); }
+template <typename T> HipTensor<T> bc_mul(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_MUL, t, s, true); }
+template <typename T> HipTensor<T> bc_div(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_DIV, t, s); }
+template <typename T> HipTensor<T> bc_div(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_DIV, t, s, true); }
+// map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass
+template <typename T> HipTensor<T> bias_relu(const HipTensor<T>& x, const HipTensor<T>& b) { return map2(AM_OP_ADD_RELU, x, b.broadcast(x.shape)); }
+
+// ---- GEMM -----------------------------------------------------------------------------------------
+// C <- alpha A B + beta C (operators_blas_l2l3.nim:58-81); any strides on A, B and C.
+template <typename T>
+void gemm(T alpha, const HipTensor<T>& A, const HipTensor<T>& B, T beta, HipTensor<T>& C) {
+  if (A.rank() != 2 || B.rank() != 2 || C.rank() != 2) throw std::invalid_argument("gemm: A, B and C must be matrices");
+  if (A.shape[1] != B.shape[0])   // check_matmat -> IndexDefect (p_checks.nim:159-167)
+    throw std::out_of_range("Number of columns in the first matrix: " + std::to_string(A.shape[1]) +
+                            ", must be the same as the number of rows in the second matrix: " + std::to_string(B.shape[0]));
+  if (C.shape[0] != A.shape[0] || C.shape[1] != B.shape[1]) throw std::out_of_range("gemm: C has the wrong shape " + detail::str(C.shape));
+  check(detail::gemm_(A.shape[0], B.shape[1], A.shape[1], alpha, A.ptr(), A.strides[0], A.strides[1], B.ptr(),
+                      B.strides[0], B.strides[1], beta, C.ptr(), C.strides[0], C.strides[1]));
+}
+
+// `*` (operators_blas_l2l3.nim:88-100): matrix-matrix, or matrix-vector (run as an N = 1 product).
+template <typename T>
+HipTensor<T> operator*(const HipTensor<T>& a, const HipTensor<T>& b) {
+  if (a.rank() == 2 && b.rank() == 2) {
+    if (a.shape[1] != b.shape[0])
+      throw std::out_of_range("Number of columns in the first matrix: " + std::to_string(a.shape[1]) +
+                              ", must be the same as the number of rows in the second matrix: " + std::to_string(b.shape[0]));
+    HipTensor<T> r(Shape{a.shape[0], b.shape[1]});
+    gemm(T(1), a, b, T(0), r);
+    return r;
+  }
+  if (a.rank() == 2 && b.rank() == 1) {
+    HipTensor<T> r(Shape{a.shape[0]});
+    HipTensor<T> bcol = b, ocol = r;
+    bcol.shape.push_back(1); bcol.strides.push_back(1);
+    ocol.shape.push_back(1); ocol.strides.push_back(1);
+    gemm(T(1), a, bcol, T(0), ocol);
+    return r;
+  }
+  throw std::invalid_argument("Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a Matrix "
+                              "and second is a Matrix or Vector");
+}
+
+// out = x * weight^T +. bias (then ReLU) as ONE kernel: nnp_linear.nim:20-29 + nnp_activation.nim:35-36.
+template <typename T>
+HipTensor<T> linear(const HipTensor<T>& x, const HipTensor<T>& weight, const HipTensor<T>& bias, bool with_relu = false) {
+  static_assert(std::is_floating_point<T>::value, "linear is defined for float tensors");
+  HipTensor<T> r(Shape{x.shape[0], weight.shape[0]});
+  const HipTensor<T> wt = weight.transpose(), bb = bias.broadcast(r.shape);
+  if (x.shape[1] != wt.shape[0]) throw std::out_of_range("linear: inner dimensions differ");
+  check(detail::gemm_ex_(x.shape[0], wt.shape[1], x.shape[1], T(1), x.ptr(), x.strides[0], x.strides[1], wt.ptr(),
+                         wt.strides[0], wt.strides[1], T(0), r.ptr(), r.strides[0], r.strides[1],
+                         with_relu ? AM_EPI_BIAS_RELU : AM_EPI_BIAS, bb.ptr(), bb.strides[0], bb.strides[1]));
+  return r;
+}
+
+inline void sync() { check(am_hip_sync()); }
+
+}  // namespace am

@@ -1,0 +1,166 @@
+// C++ twin of the reference's GPU-backend unit tests, driven through am::HipTensor
+// (include/am_hip_tensor.hpp) and therefore through the C ABI. Literals are the ones of
+//   tests/tensor/test_operators_blas_cuda.nim, tests/tensor/test_broadcasting_cuda.nim,
+//   tests/tensor/test_operators_blas.nim (integer cases, strided slices),
+//   src/arraymancer/laser/primitives/matrix_multiplication/gemm.nim:315-567.
+// Exit code 0 = every check passed. Needs an MI355X; run by tests/test_cpp_host_gpu.py.
+#include <cmath>
+#include <cstdio>
+#include <vector>
+
+#include "am_hip_tensor.hpp"
+
+using am::HipTensor;
+using am::Shape;
+using am::toHip;
+
+static int g_failed = 0, g_checked = 0;
+#define CHECK(cond)                                                          \
+  do {                                                                       \
+    ++g_checked;                                                             \
+    if (!(cond)) { ++g_failed; std::printf("FAILED %s:%d  %s\n", __FILE__, __LINE__, #cond); } \
+  } while (0)
+#define EXPECT_THROW(expr, EXC)                                              \
+  do {                                                                       \
+    ++g_checked;                                                             \
+    bool ok_ = false;                                                        \
+    try { (void)(expr); } catch (const EXC&) { ok_ = true; } catch (...) {}  \
+    if (!ok_) { ++g_failed; std::printf("FAILED %s:%d  %s did not throw %s\n", __FILE__, __LINE__, #expr, #EXC); } \
+  } while (0)
+
+template <typename T>
+static bool eq(const HipTensor<T>& t, const std::vector<T>& want) { return t.toCpu() == want; }
+
+template <typename T>
+static void gemm_literals() {
+  // gemm.nim:373-396 / test_operators_blas_cuda.nim:19-35
+  auto a = toHip<T>({1, 2, 3, 4, 5, 6}, {2, 3});
+  auto b = toHip<T>({7, 8, 9, 10, 11, 12}, {3, 2});
+  CHECK(eq(a * b, {58, 64, 139, 154}));
+  // (M x K) * (K x N) with M < N, gemm.nim:398-422
+  auto u = toHip<T>({-2, -3, -1, 3, 0, 4}, {2, 3});
+  auto v = toHip<T>({1, 5, 2, -1, -3, 0, 3, 4, 6, -2, 7, -4}, {3, 4});
+  CHECK(eq(u * v, {1, -8, -20, -6, 27, 7, 34, -19}));
+  // M > N, gemm.nim:424-453
+  auto m1 = toHip<T>({5, 6, 5, 8, 8, 2, 8, 8, 0, 5, 4, 0, 4, 0, 5, 6, 4, 5, 0, 3}, {5, 4});
+  auto m2 = toHip<T>({5, 3, 6, 0, 5, 2, 3, 3, 8, 8, 2, 0, 7, 7, 0, 0}, {4, 4});
+  CHECK(eq(m1 * m2, {151, 123, 58, 18, 170, 148, 70, 6, 57, 42, 23, 15, 102, 94, 34, 0, 66, 43, 39, 15}));
+  // transposed operands, test_operators_blas.nim:133-149
+  auto at = toHip<T>({1, 4, 2, 5, 3, 6}, {3, 2});
+  auto bt = toHip<T>({7, 9, 11, 8, 10, 12}, {2, 3});
+  CHECK(eq(at.transpose() * b, {58, 64, 139, 154}));
+  CHECK(eq(a * bt.transpose(), {58, 64, 139, 154}));
+  CHECK(eq(at.transpose() * bt.transpose(), {58, 64, 139, 154}));
+  // matrix * vector
+  auto d = toHip<T>({1, -1, 2, 0, -3, 1}, {2, 3});
+  auto e = toHip<T>({2, 1, 0}, {3});
+  CHECK(eq(d * e, {1, -3}));
+  // dimension mismatch -> IndexDefect in the reference (test_operators_blas_cuda.nim:100-104)
+  EXPECT_THROW(a * a, std::out_of_range);
+  EXPECT_THROW(e * a, std::invalid_argument);
+  // gemm(alpha, A, B, beta, C) on a strided destination (every other column of a wider buffer)
+  auto wide = toHip<T>(std::vector<T>(8, T(1)), {2, 4});
+  auto cview = wide.slice(1, 0, 2, 2);
+  am::gemm(T(2), a, b, T(3), cview);
+  CHECK(eq(wide, {T(2 * 58 + 3), 1, T(2 * 64 + 3), 1, T(2 * 139 + 3), 1, T(2 * 154 + 3), 1}));
+}
+
+static void integer_slices() {
+  // test_operators_blas.nim:332-365: non-contiguous slices with negative steps
+  auto b = toHip<int64_t>({-87, 44, 13, 1, 8, -16, 8, 91, 6, -2, 56, -56, 82, 70, 34, 23, 52, -70, 0, 53, 35, 94, 39, 36}, {6, 4});
+  auto u = toHip<int64_t>({-91, 81, 69, -75}, {4});
+  CHECK(eq(b * u, {12303, -8297, 7356, -1171, -14377, 4420}));
+  auto b2 = b.slice(0, 4, 2, -2).slice(1, 3, 1, -2);
+  auto u2 = u.slice(0, 2, 0, -2);
+  CHECK(eq(b2 * u2, {10027, -3682}));
+  auto b3 = b.slice(0, 2, 3).slice(1, 3, 1, -2);
+  CHECK(eq(b3 * u2, {-3682, -4783}));
+  // wraparound
+  auto w = toHip<int32_t>({2147483647, 1}, {1, 2});
+  auto x = toHip<int32_t>({2, 3}, {2, 1});
+  CHECK(eq(w * x, {1}));
+}
+
+static void add_sub_scalars() {
+  // test_operators_blas_cuda.nim:121-247
+  auto u = toHip<double>({1, 3, -5}, {3});
+  auto v = toHip<double>({4, -2, -1}, {3});
+  u += v;
+  CHECK(eq(u, {5, 1, -6}));
+  u -= v;
+  CHECK(eq(u + v, {5, 1, -6}) && eq(u - v, {-3, 5, -4}));
+  auto t = toHip<float>({1, 1, 1, 2, 4, 8, 3, 9, 27}, {3, 3});
+  auto z = t.clone().transpose();
+  z += z;
+  CHECK(eq(z, {2, 4, 6, 2, 8, 18, 2, 16, 54}));
+  z += t;
+  CHECK(eq(z, {3, 5, 7, 4, 12, 26, 5, 25, 81}));
+  EXPECT_THROW(z += t.slice(0, 0, 1).slice(1, 0, 1), std::invalid_argument);
+  auto a = toHip<double>({1, 2, 3, 4, 5, 6, 7, 8, 9}, {3, 3});
+  auto a_t = a.transpose();
+  CHECK(eq(a.slice(0, 0, 1).slice(1, 0, 1) + a_t.slice(0, 0, 1).slice(1, 0, 1), {2, 6, 6, 10}));
+  CHECK(eq(a.slice(0, 1, 2).slice(1, 1, 2) - a_t.slice(0, 1, 2).slice(1, 1, 2), {0, -2, 2, 0}));
+  auto s = toHip<double>({2, 6, -10}, {3});
+  CHECK(eq(s / 2.0, {1, 3, -5}));
+  auto f = toHip<float>({1, 3, -5}, {3});
+  CHECK(eq(2.0f * f, {2, 6, -10}) && eq(f * 2.0f, {2, 6, -10}));
+}
+
+template <typename T>
+static void broadcasting() {
+  // test_broadcasting_cuda.nim:18-189 / test_broadcasting.nim:58-240
+  auto a = toHip<T>({0, 10, 20, 30}, {4, 1});
+  auto b = toHip<T>({0, 1, 2}, {1, 3});
+  CHECK(eq(am::bc_add(a, b), {0, 1, 2, 10, 11, 12, 20, 21, 22, 30, 31, 32}));
+  CHECK(eq(am::bc_sub(a, b), {0, -1, -2, 10, 9, 8, 20, 19, 18, 30, 29, 28}));
+  CHECK(eq(am::bc_mul(a, b), {0, 0, 0, 0, 10, 20, 0, 20, 40, 0, 30, 60}));
+  auto c = toHip<T>({100, 10, 20, 30}, {4, 1});
+  auto d = toHip<T>({2, 5, 10}, {1, 3});
+  CHECK(eq(am::bc_div(c, d), {50, 20, 10, 5, 2, 1, 10, 4, 2, 15, 6, 3}));
+  auto e = a.broadcast({4, 3}).clone();
+  e.bc_iadd(b);
+  CHECK(eq(e, {0, 1, 2, 10, 11, 12, 20, 21, 22, 30, 31, 32}));
+  e.bc_isub(b);
+  e.bc_imul(b);
+  CHECK(eq(e, {0, 0, 0, 0, 10, 20, 0, 20, 40, 0, 30, 60}));
+  CHECK(eq(am::bc_add(am::bc_add(T(100), a), T(200)), {300, 310, 320, 330}));
+  CHECK(eq(am::bc_sub(am::bc_sub(T(100), a), T(200)), {-100, -110, -120, -130}));
+  CHECK(eq(am::bc_mul(am::bc_mul(T(10), a), T(20)), {0, 2000, 4000, 6000}));
+  EXPECT_THROW(am::bc_add(toHip<T>(std::vector<T>(8, 0), {4, 2}), b), std::invalid_argument);
+  // explicit broadcast, test_broadcasting.nim:39-56
+  CHECK(eq(toHip<T>({2}, {1, 1}).broadcast({3, 2}).clone(), {2, 2, 2, 2, 2, 2}));
+  CHECK(eq(toHip<T>({1, 2}, {2, 1}).broadcast({2, 2}), {1, 1, 2, 2}));
+}
+
+static void fused_linear() {
+  // nnp_linear.nim:28-29 + relu on small exact values
+  auto x = toHip<float>({1, 2, 3, -1, -2, -3}, {2, 3});
+  auto w = toHip<float>({1, 0, 0, 0, 1, 0, 1, 1, 1, -1, -1, -1}, {4, 3});
+  auto b = toHip<float>({0.5f, -0.5f, 1, 0}, {1, 4});
+  CHECK(eq(am::linear(x, w, b), {1.5f, 1.5f, 7, -6, -0.5f, -2.5f, -5, 6}));
+  CHECK(eq(am::linear(x, w, b, true), {1.5f, 1.5f, 7, 0, 0, 0, 0, 6}));
+  CHECK(eq(am::bias_relu(x, toHip<float>({-2, 0, 2}, {1, 3})), {0, 2, 5, 0, 0, 0}));
+  CHECK(eq(am::relu(x), {1, 2, 3, 0, 0, 0}));
+}
+
+int main() {
+  try {
+    gemm_literals<float>();
+    gemm_literals<double>();
+    gemm_literals<int32_t>();
+    gemm_literals<int64_t>();
+    integer_slices();
+    add_sub_scalars();
+    broadcasting<float>();
+    broadcasting<double>();
+    broadcasting<int32_t>();
+    broadcasting<int64_t>();
+    fused_linear();
+    am::sync();
+  } catch (const std::exception& e) {
+    std::printf("unexpected exception: %s\n", e.what());
+    return 2;
+  }
+  std::printf("%d checks, %d failed\n", g_checked, g_failed);
+  return g_failed ? 1 : 0;
+}
