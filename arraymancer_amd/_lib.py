@@ -55,6 +55,10 @@ def _signatures():
         "am_hip_event_record": (ci, [vp]),
         "am_hip_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),
         "am_hip_event_destroy": (ci, [vp]),
+        "am_hip_graph_begin": (ci, []),
+        "am_hip_graph_end": (ci, [pp]),
+        "am_hip_graph_launch": (ci, [vp]),
+        "am_hip_graph_destroy": (ci, [vp]),
         "am_hip_diag_peak": (ci, [ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
     }
     for sfx, ct in CTYPE.items():

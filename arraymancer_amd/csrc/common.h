@@ -13,6 +13,7 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 // Lazily initialises the device context (device 0 unless am_hip_init chose another).
 int ensure_init();
 hipStream_t stream();
+bool capturing();
 int num_cus();
 
 #define AM_HIP_TRY(expr)                                                                    \

@@ -25,6 +25,12 @@ template <typename T> struct Args {
   const T* bias; int64_t bias_m, bias_n;
   int tiles_m, tiles_n;
   int a_kfast, b_kfast;            // generic loader: 1 = walk k fastest across lanes
+  // Split-K: workgroup (tile, split) multiplies the k range [split * k_chunk, (split + 1) * k_chunk)
+  // and stores its raw partial tile to ws[split][M][N]; splitk_reduce adds the partials in a fixed
+  // order and applies alpha / beta / epilogue. splits == 1: the kernel writes C itself.
+  int splits;
+  int64_t k_chunk;
+  T* ws;
 };
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -104,6 +110,68 @@ static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int6
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
   }
   return best;
+}
+
+// Persistent device workspace for split-K partial sums (runtime.hip): allocated once, on first use
+// outside graph capture; nullptr when `bytes` exceeds its capacity or it cannot be allocated now.
+void* splitk_workspace(size_t bytes);
+
+// Decides the split-K factor for a problem that would otherwise leave most SIMDs idle: small M x N
+// (few tiles) with a long K runs as one serial MFMA / MAC chain per wave, so K is cut into
+// `splits` ranges handled by different workgroups. bk = slab width, waves = wavefronts per tile.
+template <typename T>
+static inline void plan_splitk(Args<T>& g, int bk, int waves_per_tile) {
+  g.splits = 1; g.k_chunk = g.K; g.ws = nullptr;
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  const int64_t simds = (int64_t)num_cus() * 4;
+  const int64_t slabs = (g.K + bk - 1) / bk;
+  if (tiles * waves_per_tile * 2 > simds || slabs < 4) return;
+  int64_t want = simds / (tiles * waves_per_tile);          // one wave per SIMD
+  int64_t max_by_k = slabs / 2;                               // at least two slabs per split
+  int64_t splits = want < max_by_k ? want : max_by_k;
+  if (splits > 32) splits = 32;
+  if (splits < 2) return;
+  const int64_t chunk_slabs = (slabs + splits - 1) / splits;
+  splits = (slabs + chunk_slabs - 1) / chunk_slabs;           // no empty split
+  if (splits < 2) return;
+  const size_t bytes = (size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(T);
+  T* ws = (T*)splitk_workspace(bytes);
+  if (!ws) return;
+  g.splits = (int)splits; g.k_chunk = chunk_slabs * bk; g.ws = ws;
+}
+
+// Second pass of split-K: C <- epilogue(alpha * sum_s ws[s] + beta * C), partials added in
+// ascending s (deterministic). ACC is the type the partials were stored in.
+template <typename T, typename ACC>
+__global__ __launch_bounds__(256) void splitk_reduce(Args<T> p) {
+  const int64_t total = p.M * p.N;
+  const ACC* ws = (const ACC*)p.ws;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    const int64_t row = idx / p.N, col = idx - row * p.N;
+    ACC sum = ws[idx];
+    for (int sidx = 1; sidx < p.splits; ++sidx) sum += ws[(int64_t)sidx * total + idx];
+    T* cp = p.C + row * p.c_m + col * p.c_n;
+    ACC ab = sum;
+    if (p.alpha != (T)1) ab = (ACC)p.alpha * ab;
+    ACC v = ab;
+    if (p.beta != (T)0) {
+      ACC c = (ACC)*cp;
+      if (p.beta != (T)1) c = c * (ACC)p.beta;
+      v = c + ab;
+    }
+    if (p.epilogue & AM_EPI_BIAS) v = v + (ACC)p.bias[row * p.bias_m + col * p.bias_n];
+    if (p.epilogue & AM_EPI_RELU) v = ((ACC)0 >= v) ? (ACC)0 : v;
+    *cp = (T)v;
+  }
+}
+
+template <typename T, typename ACC>
+static int launch_splitk_reduce(const Args<T>& g) {
+  int64_t blocks = (g.M * g.N + 255) / 256;
+  const int64_t cap = (int64_t)num_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL((splitk_reduce<T, ACC>), dim3((unsigned)blocks), dim3(256), 0, stream(), g);
+  return check_launch("splitk_reduce");
 }
 
 // Workgroup id -> (tile_m, tile_n).

@@ -8,13 +8,17 @@ static int run_f32(Args<float>& g) {
   const int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   const int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
   // Candidate workgroup tiles, largest first, with the relative MFMA efficiency of each.
-  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.95}, {64, 64, 0.89}, {256, 128, 0.97}, {128, 64, 0.93}};
-  switch (choose_tile(cand, 5, g.M, g.N, "AM_HIP_GEMM_TILE_F32")) {
+  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.95}, {64, 64, 0.89}, {256, 128, 0.97}, {128, 64, 0.93}, {32, 32, 0.6}, {64, 64, 0.0}, {32, 32, 0.0}, {128, 128, 0.0}};
+  switch (choose_tile(cand, 9, g.M, g.N, "AM_HIP_GEMM_TILE_F32")) {
     case 0: return launch_kinds<float, 256, 256, 16, 2, 4>(g, ak, bk);
     case 1: return launch_kinds<float, 128, 128, 16, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2>(g, ak, bk);
     case 3: return launch_kinds<float, 256, 128, 16, 4, 2>(g, ak, bk);
-    default: return launch_kinds<float, 128, 64, 16, 2, 2>(g, ak, bk);
+    case 4: return launch_kinds<float, 128, 64, 16, 2, 2>(g, ak, bk);
+    case 5: return launch_kinds<float, 32, 32, 16, 1, 1>(g, ak, bk);
+    case 6: return launch_kinds<float, 64, 64, 64, 2, 2>(g, ak, bk);
+    case 7: return launch_kinds<float, 32, 32, 64, 1, 1>(g, ak, bk);
+    default: return launch_kinds<float, 128, 128, 32, 2, 2>(g, ak, bk);
   }
 }
 

@@ -40,13 +40,20 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
   __shared__ __attribute__((aligned(16))) T sA[2][BK * LDA];
   __shared__ __attribute__((aligned(16))) T sB[2][BK * LDB];
 
-  int tile_m, tile_n;
-  tile_of_block((int)blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  int tile_m, tile_n, bid = (int)blockIdx.x, split = 0;
+  if (p.splits > 1) {
+    const int nt = p.tiles_m * p.tiles_n;
+    split = bid / nt;
+    bid -= split * nt;
+  }
+  tile_of_block(bid, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+  const int64_t k_begin = (int64_t)split * p.k_chunk;
+  const int64_t k_end = (k_begin + p.k_chunk < p.K) ? k_begin + p.k_chunk : p.K;
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
 
-  Loader<T, AK, BM, BK, NT, false> la(p.A, p.a_mn, p.a_k, m0, p.M, p.K, p.a_kfast);
-  Loader<T, BKIND, BN, BK, NT, false> lb(p.B, p.b_mn, p.b_k, n0, p.N, p.K, p.b_kfast);
+  Loader<T, AK, BM, BK, NT, false> la(p.A, p.a_mn, p.a_k, m0, p.M, k_end, p.a_kfast);
+  Loader<T, BKIND, BN, BK, NT, false> lb(p.B, p.b_mn, p.b_k, n0, p.N, k_end, p.b_kfast);
 
   ACC acc[TM][TN];
 #pragma unroll
@@ -54,9 +61,9 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = 0;
 
-  const int64_t ktiles = (p.K + BK - 1) / BK;
-  la.fetch(0);
-  lb.fetch(0);
+  const int64_t ktiles = (k_end - k_begin + BK - 1) / BK;
+  la.fetch(k_begin);
+  lb.fetch(k_begin);
   la.commit(sA[0]);
   lb.commit(sB[0]);
   __syncthreads();
@@ -65,8 +72,8 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
     const int cur = (int)(kt & 1);
     const bool more = (kt + 1) < ktiles;
     if (more) {
-      la.fetch((kt + 1) * BK);
-      lb.fetch((kt + 1) * BK);
+      la.fetch(k_begin + (kt + 1) * BK);
+      lb.fetch(k_begin + (kt + 1) * BK);
     }
     const T* a_lds = sA[cur];
     const T* b_lds = sB[cur];
@@ -98,6 +105,20 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
   }
 
   // Epilogue: same case analysis as the reference (gemm_ukernel_generic.nim:53-125), mod 2^w.
+  if (p.splits > 1) {   // split-K: raw partial sums (mod 2^w) to the workspace
+    T* ws = p.ws + (int64_t)split * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int64_t row = m0 + (i / VK) * 16 * VK + ty * VK + (i % VK);
+      if (row >= p.M) continue;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t col = n0 + (j / VK) * 16 * VK + tx * VK + (j % VK);
+        if (col < p.N) ws[row * p.N + col] = (T)(U)acc[i][j];
+      }
+    }
+    return;
+  }
   const U alpha = (U)p.alpha, beta = (U)p.beta;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -127,7 +148,8 @@ static int launch_valu(Args<T>& g, int ak, int bk) {
   g.tiles_n = (int)((g.N + BN - 1) / BN);
   const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
   if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
-  const dim3 grid((unsigned)nb), block(256);
+  plan_splitk(g, BK, 4);
+  const dim3 grid((unsigned)(nb * g.splits)), block(256);
 #define AM_LAUNCH(AKIND, BKIND_) \
   hipLaunchKernelGGL((gemm_valu<T, TM, TN, BK, AKIND, BKIND_>), grid, block, 0, stream(), g)
   switch (ak * 3 + bk) {
@@ -142,7 +164,10 @@ static int launch_valu(Args<T>& g, int ak, int bk) {
     default: AM_LAUNCH(kGeneric, kGeneric); break;
   }
 #undef AM_LAUNCH
-  return check_launch("gemm_valu");
+  AM_TRY(check_launch("gemm_valu"));
+  // ring arithmetic: the reduction runs in the unsigned twin, so it wraps like the main kernel
+  if (g.splits > 1) return launch_splitk_reduce<T, typename UnsignedOf<T>::type>(g);
+  return AM_OK;
 }
 
 }  // namespace gemm

@@ -92,16 +92,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
   __shared__ __attribute__((aligned(16))) T sA[2][A_ELEMS];
   __shared__ __attribute__((aligned(16))) T sB[2][B_ELEMS];
 
-  int tile_m, tile_n;
-  tile_of_block((int)blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  int tile_m, tile_n, bid = (int)blockIdx.x, split = 0;
+  if (p.splits > 1) {
+    const int nt = p.tiles_m * p.tiles_n;
+    split = bid / nt;
+    bid -= split * nt;
+  }
+  tile_of_block(bid, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+  const int64_t k_begin = (int64_t)split * p.k_chunk;
+  const int64_t k_end = (k_begin + p.k_chunk < p.K) ? k_begin + p.k_chunk : p.K;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int lrow = lane % TILE, kl = lane / TILE;
 
-  Loader<T, AK, BM, BK, NT> la(p.A, p.a_mn, p.a_k, m0, p.M, p.K, p.a_kfast);
-  Loader<T, BKIND, BN, BK, NT> lb(p.B, p.b_mn, p.b_k, n0, p.N, p.K, p.b_kfast);
+  Loader<T, AK, BM, BK, NT> la(p.A, p.a_mn, p.a_k, m0, p.M, k_end, p.a_kfast);
+  Loader<T, BKIND, BN, BK, NT> lb(p.B, p.b_mn, p.b_k, n0, p.N, k_end, p.b_kfast);
 
   acc_t acc[TM][TN];
 #pragma unroll
@@ -111,9 +118,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
 #pragma unroll
       for (int r = 0; r < MF::NACC; ++r) acc[i][j][r] = (T)0;
 
-  const int64_t ktiles = (p.K + BK - 1) / BK;
-  la.fetch(0);
-  lb.fetch(0);
+  const int64_t ktiles = (k_end - k_begin + BK - 1) / BK;
+  la.fetch(k_begin);
+  lb.fetch(k_begin);
   la.commit(sA[0]);
   lb.commit(sB[0]);
   __syncthreads();
@@ -122,8 +129,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
     const int cur = (int)(kt & 1);
     const bool more = (kt + 1) < ktiles;
     if (more) {
-      la.fetch((kt + 1) * BK);
-      lb.fetch((kt + 1) * BK);
+      la.fetch(k_begin + (kt + 1) * BK);
+      lb.fetch(k_begin + (kt + 1) * BK);
     }
     const T* a_lds = sA[cur];
     const T* b_lds = sB[cur];
@@ -154,6 +161,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
 
   // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
   // C += alpha * AB, each rounded on its own; then the optional fused bias / ReLU.
+  if (p.splits > 1) {   // split-K: raw partial tile to the workspace, epilogue in splitk_reduce
+    T* ws = p.ws + (int64_t)split * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
+#pragma unroll
+        for (int r = 0; r < MF::NACC; ++r) {
+          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
+          if (row < p.M && col < p.N) ws[row * p.N + col] = acc[i][j][r];
+        }
+      }
+    return;
+  }
   const T alpha = p.alpha, beta = p.beta;
   const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
 #pragma unroll
@@ -189,7 +211,8 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
   g.tiles_n = (int)((g.N + BN - 1) / BN);
   const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
   if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
-  const dim3 grid((unsigned)nb), block(WAVES_M * WAVES_N * 64);
+  plan_splitk(g, BK, WAVES_M * WAVES_N);
+  const dim3 grid((unsigned)(nb * g.splits)), block(WAVES_M * WAVES_N * 64);
 #define AM_LAUNCH(AKIND, BKIND_)                                                                   \
   hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, AKIND, BKIND_>), grid, block, 0, \
                      stream(), g)
@@ -205,7 +228,9 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
     default: AM_LAUNCH(kGeneric, kGeneric); break;
   }
 #undef AM_LAUNCH
-  return check_launch("gemm_mfma");
+  AM_TRY(check_launch("gemm_mfma"));
+  if (g.splits > 1) return launch_splitk_reduce<T, T>(g);
+  return AM_OK;
 }
 
 }  // namespace gemm

@@ -21,6 +21,7 @@ static bool g_ready = false;
 static int g_device = -1;
 static hipStream_t g_stream = nullptr;
 static hipDeviceProp_t g_prop;
+static bool g_capturing = false;   // between am_hip_graph_begin and am_hip_graph_end
 
 static int init_locked(int device) {
   if (g_ready) {
@@ -48,7 +49,23 @@ int ensure_init() {
   return init_locked(0);
 }
 
+// Split-K workspace: one allocation for the life of the process (64 MiB of the 288 GB), so that GEMM
+// calls never allocate (and can be recorded into graphs once it exists).
+static void* g_ws = nullptr;
+static const size_t kWorkspaceBytes = (size_t)64 << 20;
+namespace gemm {
+void* splitk_workspace(size_t bytes) {
+  if (bytes > kWorkspaceBytes) return nullptr;
+  if (!g_ws) {
+    if (g_capturing) return nullptr;
+    if (hipMalloc(&g_ws, kWorkspaceBytes) != hipSuccess) { (void)hipGetLastError(); g_ws = nullptr; }
+  }
+  return g_ws;
+}
+}  // namespace gemm
+
 hipStream_t stream() { return g_stream; }
+bool capturing() { return g_capturing; }
 int num_cus() { return g_ready ? g_prop.multiProcessorCount : 256; }
 
 }  // namespace am
@@ -91,6 +108,7 @@ int am_hip_malloc(size_t bytes, void** out) {
   *out = nullptr;
   if (bytes == 0) return AM_OK;
   AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_malloc: not allowed while a graph is being captured");
   hipError_t e = hipMalloc(out, bytes);
   if (e != hipSuccess) {
     *out = nullptr;
@@ -103,6 +121,7 @@ int am_hip_malloc(size_t bytes, void** out) {
 int am_hip_free(void* dptr) {
   if (!dptr) return AM_OK;
   AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_free: not allowed while a graph is being captured");
   // Work that still reads or writes the buffer is on the library stream: drain it first.
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
   AM_HIP_TRY(hipFree(dptr));
@@ -113,6 +132,7 @@ int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return AM_OK;
   if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_h2d: null pointer");
   AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_memcpy_h2d: not allowed while a graph is being captured");
   AM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
   return AM_OK;
@@ -122,6 +142,7 @@ int am_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return AM_OK;
   if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_d2h: null pointer");
   AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_memcpy_d2h: not allowed while a graph is being captured");
   AM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
   return AM_OK;
@@ -131,6 +152,7 @@ int am_hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return AM_OK;
   if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_d2d: null pointer");
   AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_memcpy_d2d: not allowed while a graph is being captured");
   AM_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
   return AM_OK;
 }
@@ -139,13 +161,55 @@ int am_hip_memset(void* dst, int byte_value, size_t bytes) {
   if (bytes == 0) return AM_OK;
   if (!dst) return fail(AM_E_ARG, "am_hip_memset: null pointer");
   AM_TRY(ensure_init());
+  // Memset nodes are kept out of captured graphs (clear memory with an element-wise kernel instead).
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_memset: not allowed while a graph is being captured");
   AM_HIP_TRY(hipMemsetAsync(dst, byte_value, bytes, g_stream));
   return AM_OK;
 }
 
 int am_hip_sync(void) {
   AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_sync: not allowed while a graph is being captured");
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  return AM_OK;
+}
+
+// ---- HIP graphs: record a sequence of kernel launches once, replay it with one call -------------
+int am_hip_graph_begin(void) {
+  AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_graph_begin: a capture is already in progress");
+  AM_HIP_TRY(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+  g_capturing = true;
+  return AM_OK;
+}
+
+int am_hip_graph_end(void** graph_exec) {
+  if (!graph_exec) return fail(AM_E_ARG, "am_hip_graph_end: null pointer");
+  *graph_exec = nullptr;
+  if (!g_capturing) return fail(AM_E_ARG, "am_hip_graph_end: no capture in progress");
+  g_capturing = false;
+  hipGraph_t graph = nullptr;
+  AM_HIP_TRY(hipStreamEndCapture(g_stream, &graph));
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) return fail(AM_E_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  *graph_exec = (void*)exec;
+  return AM_OK;
+}
+
+int am_hip_graph_launch(void* graph_exec) {
+  if (!graph_exec) return fail(AM_E_ARG, "am_hip_graph_launch: null graph");
+  AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_graph_launch: not allowed while a graph is being captured");
+  AM_HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, g_stream));
+  return AM_OK;
+}
+
+int am_hip_graph_destroy(void* graph_exec) {
+  if (!graph_exec) return AM_OK;
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  AM_HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
   return AM_OK;
 }
 

@@ -265,6 +265,37 @@ def sync() -> None:
     check(_lib.load().am_hip_sync())
 
 
+class Graph:
+    """Records the device operations issued inside `with Graph() as g:` into a HIP graph instead
+    of running them; `g.launch()` replays the sequence with one call. Output tensors must be
+    allocated before the block (allocation is refused during capture), e.g. with `empty` and the
+    `gemm(alpha, A, B, beta, C)` / `apply2` / `_into` forms."""
+
+    def __init__(self):
+        self._exec = ctypes.c_void_p()
+
+    def __enter__(self):
+        check(_lib.load().am_hip_graph_begin())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = _lib.load().am_hip_graph_end(ctypes.byref(self._exec))
+        if exc_type is None:
+            check(rc)
+        return False
+
+    def launch(self):
+        check(_lib.load().am_hip_graph_launch(self._exec))
+
+    def __del__(self):
+        ex, self._exec = getattr(self, "_exec", None), None
+        if ex:
+            try:
+                _lib.load().am_hip_graph_destroy(ex)
+            except Exception:
+                pass
+
+
 # ---------------------------------------------------------------------- checks
 def _same_dtype(*ts):
     d = ts[0].dtype

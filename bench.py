@@ -148,7 +148,45 @@ def other_workloads(am, timer, steps, warmup):
                         value=round(nbytes * steps / wall / 1e9, 1), ms_per_step=round(ev / steps * 1e3, 4),
                         roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                                       frac=round(gbs / HBM_PEAK_GBS, 4))))
+    out.append(bench_chain(am, timer, max(steps, 50), warmup))
     return out
+
+
+def chain_setup(am):
+    """The MNIST-shaped inference chain of BASELINE config 5 (batch 64): conv1 and conv2 as im2col
+    GEMMs, dense + bias + ReLU (fused epilogue), classifier. All outputs are allocated up front so
+    that the four launches can be recorded into a HIP graph. Returns (issue, flops, bytes)."""
+    rng = np.random.default_rng(5001)
+    g = lambda *sh: am.toHip(rng.normal(0, 0.1, sh).astype(np.float32))
+    k1, x1, o1 = g(20, 25), g(25, 36864), am.empty((20, 36864), np.float32)
+    k2, x2, o2 = g(50, 500), g(500, 4096), am.empty((50, 4096), np.float32)
+    x3, w3, b3, h = g(64, 800), g(500, 800), g(1, 500), am.empty((64, 500), np.float32)
+    w4, o4 = g(10, 500), am.empty((64, 10), np.float32)
+    w3t, w4t = w3.transpose(), w4.transpose()
+
+    def issue():
+        am.gemm(1.0, k1, x1, 0.0, o1)
+        am.gemm(1.0, k2, x2, 0.0, o2)
+        am.gemm(1.0, x3, w3t, 0.0, h, epilogue="bias_relu", bias=b3)
+        am.gemm(1.0, h, w4t, 0.0, o4)
+
+    flops = 2.0 * (20 * 25 * 36864 + 50 * 500 * 4096 + 64 * 800 * 500 + 64 * 500 * 10)
+    return issue, flops, 17834080, (k1, x1, o1, k2, x2, o2, x3, w3, b3, h, w4, o4)
+
+
+def bench_chain(am, timer, steps, warmup):
+    issue, flops, nbytes, keep = chain_setup(am)
+    wall_e, ev_e = timer.run(issue, steps, warmup)            # eager: 4 launches per chain from the host
+    with am.Graph() as graph:
+        issue()
+    wall_g, ev_g = timer.run(graph.launch, steps, warmup)     # one graph launch per chain
+    return dict(workload="f32 inference chain: [20x25].[25x36864], [50x500].[500x4096], "
+                         "[64x800].[800x500]+bias+ReLU (fused), [64x500].[500x10]",
+                unit="us per chain", dtype="f32", higher_is_better=False,
+                value=round(ev_g / steps * 1e6, 2), hipgraph_us=round(ev_g / steps * 1e6, 2),
+                eager_us=round(ev_e / steps * 1e6, 2), eager_wall_us=round(wall_e / steps * 1e6, 2),
+                gflops_hipgraph=round(flops / (ev_g / steps) / 1e9, 1),
+                note="launch/latency bound: 2.9e8 FLOP and 17.8 MB per chain; eager figure includes host launch cost")
 
 
 def run_only(am, timer, which, steps, warmup):
@@ -157,6 +195,9 @@ def run_only(am, timer, which, steps, warmup):
     if which == "gemm_f32":
         r = bench_gemm_f32(am, timer, steps, warmup)
         return dict(only=which, ms_per_launch=round(r["ev"] / steps * 1e3, 4), launches=steps + warmup)
+    if which == "chain":
+        r = bench_chain(am, timer, steps, warmup)
+        return dict(only=which, hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"])
     if which == "gemm_i32":
         n = 4096
         A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
@@ -189,7 +230,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy"],
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy", "chain"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:

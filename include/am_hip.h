@@ -70,6 +70,18 @@ int am_hip_event_record(void* ev);
 int am_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* synchronises on `stop` */
 int am_hip_event_destroy(void* ev);
 
+/* HIP graphs on the library stream: between begin and end, GEMM / element-wise calls are recorded
+ * instead of executed (allocation, copies, memset and sync are refused meanwhile); the returned
+ * executable graph replays the whole sequence with one launch. For launch-bound chains of small
+ * kernels such as the reference's per-layer gemm + `+.=` + relu sequence
+ * (src/arraymancer/nn_primitives/nnp_linear.nim:28-29, fallback/conv.nim:99-106). The reference
+ * has no counterpart (one launch per operator, backend/cuda.nim). Buffers recorded in a graph must
+ * stay allocated while it is replayed. */
+int am_hip_graph_begin(void);
+int am_hip_graph_end(void** graph_exec);
+int am_hip_graph_launch(void* graph_exec);
+int am_hip_graph_destroy(void* graph_exec);
+
 /* ---------------------------------------------------------------- GEMM
  * C[M x N] <- alpha * A[M x K] * B[K x N] + beta * C, element X[r,c] = X[r*rsX + c*csX].
  *

@@ -42,6 +42,10 @@ proc am_hip_event_record*(ev: pointer): cint {.importc.}
 proc am_hip_event_elapsed_ms*(start, stop: pointer, ms: ptr cfloat): cint {.importc.}
 proc am_hip_event_destroy*(ev: pointer): cint {.importc.}
 
+proc am_hip_graph_begin*(): cint {.importc.}
+proc am_hip_graph_end*(graph_exec: ptr pointer): cint {.importc.}
+proc am_hip_graph_launch*(graph_exec: pointer): cint {.importc.}
+proc am_hip_graph_destroy*(graph_exec: pointer): cint {.importc.}
 proc am_hip_diag_peak*(kind, iters, waves_per_simd: cint, ops_per_second: ptr cdouble): cint {.importc.}
 
 # ---- GEMM (strides in elements; pointers already offset)
