@@ -220,6 +220,86 @@ __global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T> p) {
   }
 }
 
+// ---- ternary bodies and kernels (map3_inline / apply3_inline) -----------------------------------
+template <typename T, int OP> struct TriOp {
+  typedef typename Traits<T>::U U;
+  static __device__ __forceinline__ T apply(T x, T y, T z) {
+    if constexpr (OP == AM_OP3_MULADD) return (T)((U)x * (U)y + (U)z);
+    else if constexpr (OP == AM_OP3_GRU_CANDIDATE) return dev_tanh(x + y * z);
+    else return ((T)1 - y) * z + y * x;
+  }
+};
+
+template <typename T> struct TriArgs {
+  T* dst; const T* a; const T* b; const T* c;
+  int64_t n;          // generic kernel: total elements
+  int64_t L;          // rows kernel: inner extent
+  uint32_t tiles_per_row, total_tiles;
+  int rank;           // collapsed rank (generic) / number of outer dims (rows)
+  int64_t shape[AM_MAXRANK];
+  int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK], sc[AM_MAXRANK];
+};
+
+// All four operands have unit innermost stride and 16-byte aligned rows (the GRU column slices,
+// plain contiguous tensors): same streaming structure as ew_rows.
+template <typename T, int OP>
+__global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
+  typedef typename Traits<T>::V V;
+  constexpr int VEC = Traits<T>::kVec;
+  constexpr int64_t TILE = (int64_t)kThreads * VEC * kUnroll;
+  for (uint32_t tile = blockIdx.x; tile < p.total_tiles; tile += gridDim.x) {
+    const uint32_t row = tile / p.tiles_per_row;
+    const uint32_t ct = tile - row * p.tiles_per_row;
+    int64_t od = 0, oa = 0, ob = 0, oc = 0;
+    uint32_t rem = row;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      const uint32_t ext = (uint32_t)p.shape[d];
+      const uint32_t q = rem / ext;
+      const int64_t cidx = (int64_t)(rem - q * ext);
+      rem = q;
+      od += cidx * p.sd[d]; oa += cidx * p.sa[d]; ob += cidx * p.sb[d]; oc += cidx * p.sc[d];
+    }
+    T* __restrict__ drow = p.dst + od;
+    const T* __restrict__ arow = p.a + oa;
+    const T* __restrict__ brow = p.b + ob;
+    const T* __restrict__ crow = p.c + oc;
+    const int64_t col0 = (int64_t)ct * TILE + (int64_t)threadIdx.x * VEC;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t col = col0 + (int64_t)u * kThreads * VEC;
+      if (col + VEC <= p.L) {
+        const V av = __builtin_nontemporal_load((const V*)(arow + col));
+        const V bv = __builtin_nontemporal_load((const V*)(brow + col));
+        const V cv = __builtin_nontemporal_load((const V*)(crow + col));
+        V r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r[e] = TriOp<T, OP>::apply(av[e], bv[e], cv[e]);
+        __builtin_nontemporal_store(r, (V*)(drow + col));
+      } else {
+        for (int64_t cc = col; cc < p.L; ++cc) drow[cc] = TriOp<T, OP>::apply(arow[cc], brow[cc], crow[cc]);
+      }
+    }
+  }
+}
+
+template <typename T, int OP, typename IDX>
+__global__ __launch_bounds__(kThreads) void ew3_generic(TriArgs<T> p) {
+  const IDX n = (IDX)p.n;
+  const IDX step = (IDX)gridDim.x * kThreads;
+  for (IDX i = (IDX)blockIdx.x * kThreads + threadIdx.x; i < n; i += step) {
+    IDX rem = i;
+    int64_t od = 0, oa = 0, ob = 0, oc = 0;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      const IDX ext = (IDX)p.shape[d];
+      const IDX q = rem / ext;
+      const int64_t cidx = (int64_t)(rem - q * ext);
+      rem = q;
+      od += cidx * p.sd[d]; oa += cidx * p.sa[d]; ob += cidx * p.sb[d]; oc += cidx * p.sc[d];
+    }
+    p.dst[od] = TriOp<T, OP>::apply(p.a[oa], p.b[ob], p.c[oc]);
+  }
+}
+
 // ---- host side ------------------------------------------------------------------------------
 struct Collapsed {
   int rank;
@@ -439,6 +519,90 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
   }
 }
 
+template <typename T, int OP>
+static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a, const int64_t* sa,
+                const T* b, const int64_t* sb, const T* c, const int64_t* sc) {
+  constexpr int VEC = Traits<T>::kVec;
+  // joint collapse over the four operands
+  TriArgs<T> g;
+  g.dst = dst; g.a = a; g.b = b; g.c = c;
+  int r = 0;
+  int64_t n = 1;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] < 0) return fail(AM_E_ARG, "negative extent in dimension %d", i);
+    n *= shape[i];
+  }
+  if (n == 0) return AM_OK;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] == 1) continue;
+    if (sd[i] == 0) return fail(AM_E_SHAPE, "destination has stride 0 on dimension %d of extent %lld", i, (long long)shape[i]);
+    if (r > 0 && g.sd[r - 1] == shape[i] * sd[i] && g.sa[r - 1] == shape[i] * sa[i] &&
+        g.sb[r - 1] == shape[i] * sb[i] && g.sc[r - 1] == shape[i] * sc[i]) {
+      g.shape[r - 1] *= shape[i];
+      g.sd[r - 1] = sd[i]; g.sa[r - 1] = sa[i]; g.sb[r - 1] = sb[i]; g.sc[r - 1] = sc[i];
+    } else {
+      g.shape[r] = shape[i]; g.sd[r] = sd[i]; g.sa[r] = sa[i]; g.sb[r] = sb[i]; g.sc[r] = sc[i];
+      ++r;
+    }
+  }
+  if (r == 0) { g.shape[0] = 1; g.sd[0] = g.sa[0] = g.sb[0] = g.sc[0] = 1; r = 1; }
+  for (int i = r; i < AM_MAXRANK; ++i) { g.shape[i] = 1; g.sd[i] = g.sa[i] = g.sb[i] = g.sc[i] = 0; }
+  AM_TRY(ensure_init());
+  const int in = r - 1;
+  const int64_t L = g.shape[in];
+  bool ok = g.sd[in] == 1 && g.sa[in] == 1 && g.sb[in] == 1 && g.sc[in] == 1 && aligned16(dst) && aligned16(a) &&
+            aligned16(b) && aligned16(c);
+  for (int d = 0; d < in && ok; ++d)
+    if (g.sd[d] % VEC || g.sa[d] % VEC || g.sb[d] % VEC || g.sc[d] % VEC) ok = false;
+  int64_t rows = 1;
+  for (int d = 0; d < in; ++d) rows *= g.shape[d];
+  const int64_t tile = (int64_t)kThreads * VEC * kUnroll;
+  const int64_t tiles_per_row = (L + tile - 1) / tile;
+  if (ok && rows > 1 && L < tile / 8) ok = false;
+  if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31))) ok = false;
+  g.n = n; g.L = L;
+  if (ok) {
+    g.rank = in;
+    g.tiles_per_row = (uint32_t)tiles_per_row;
+    g.total_tiles = (uint32_t)(tiles_per_row * rows);
+    int64_t blocks = g.total_tiles;
+    const int64_t cap = (int64_t)num_cus() * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((ew3_rows<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+    return check_launch("ew3_rows");
+  }
+  g.rank = r;
+  int64_t blocks = (n + kThreads - 1) / kThreads;
+  const int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  if (n < ((int64_t)1 << 31)) hipLaunchKernelGGL((ew3_generic<T, OP, uint32_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+  else hipLaunchKernelGGL((ew3_generic<T, OP, uint64_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+  return check_launch("ew3_generic");
+}
+
+template <typename T>
+static int ternary(const char* fn, int op, int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a,
+                   const int64_t* sa, const T* b, const int64_t* sb, const T* c, const int64_t* sc) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  if (rank > 0 && (!sb || !sc)) return fail(AM_E_ARG, "%s: null stride array", fn);
+  {
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= shape[i];
+    if (n != 0 && (!b || !c)) return fail(AM_E_ARG, "%s: null data pointer", fn);
+  }
+  constexpr bool F = Traits<T>::kFloat;
+  switch (op) {
+    case AM_OP3_MULADD: return run3<T, AM_OP3_MULADD>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
+    case AM_OP3_GRU_CANDIDATE:
+      if constexpr (F) return run3<T, AM_OP3_GRU_CANDIDATE>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
+      else return fail(AM_E_DTYPE, "%s: tanh(x + y * z) is defined for float tensors only", fn);
+    case AM_OP3_GRU_BLEND:
+      if constexpr (F) return run3<T, AM_OP3_GRU_BLEND>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
+      else return fail(AM_E_DTYPE, "%s: (1 - y) * z + y * x is defined for float tensors only", fn);
+    default: return fail(AM_E_ARG, "%s: unknown ternary op %d", fn, op);
+  }
+}
+
 }  // namespace ew
 }  // namespace am
 
@@ -451,6 +615,12 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
   extern "C" int am_hip_ew_scalar_##SFX(int op, int left, int rank, const int64_t* shape, T* dst,      \
                                         const int64_t* ds, const T* a, const int64_t* as_, T s) {      \
     return ::am::ew::scalar<T>("am_hip_ew_scalar_" #SFX, op, left, rank, shape, dst, ds, a, as_, s);   \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_ternary_##SFX(int op, int rank, const int64_t* shape, T* dst,               \
+                                         const int64_t* ds, const T* a, const int64_t* as_, const T* b, \
+                                         const int64_t* bs, const T* c, const int64_t* cs) {           \
+    return ::am::ew::ternary<T>("am_hip_ew_ternary_" #SFX, op, rank, shape, dst, ds, a, as_, b, bs, c, \
+                                cs);                                                                   \
   }                                                                                                    \
   extern "C" int am_hip_ew_unary_##SFX(int op, int rank, const int64_t* shape, T* dst,                 \
                                        const int64_t* ds, const T* a, const int64_t* as_) {            \

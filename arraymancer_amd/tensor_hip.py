@@ -28,7 +28,7 @@ import numpy as np
 
 from . import _lib
 from . import metadata as md
-from ._lib import CTYPE, EPI, OP, SFX, UOP, check, i64_array
+from ._lib import CTYPE, EPI, OP, OP3, SFX, UOP, check, i64_array
 from .metadata import Layout, Step
 
 
@@ -428,6 +428,36 @@ def apply2(op, dest: HipTensor, src: HipTensor) -> HipTensor:
     _same_dtype(dest, src)
     _check_elementwise(dest, src)
     _binary_into(op, dest, dest, src)
+    return dest
+
+
+def _ternary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor, c: HipTensor):
+    code = OP3[op] if isinstance(op, str) else int(op)
+    check(getattr(_lib.load(), f"am_hip_ew_ternary_{dst.sfx}")(
+        code, dst.rank, i64_array(dst.shape), ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
+        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides), ctypes.c_void_p(b.data_ptr()), i64_array(b.strides),
+        ctypes.c_void_p(c.data_ptr()), i64_array(c.strides)))
+
+
+def map3(op, a: HipTensor, b: HipTensor, c: HipTensor) -> HipTensor:
+    """map3_inline with an enumerated body ("muladd": x*y+z, "gru_candidate": tanh(x+y*z),
+    "gru_blend": (1-y)*z+y*x); src/arraymancer/tensor/higher_order_applymap.nim:122-150."""
+    _same_dtype(a, b, c)
+    _check_elementwise(a, b)
+    _check_elementwise(a, c)
+    out = empty(a.shape, a.dtype)
+    if out.size:
+        _ternary_into(op, out, a, b, c)
+    return out
+
+
+def apply3(op, dest: HipTensor, src1: HipTensor, src2: HipTensor) -> HipTensor:
+    """apply3_inline: dest[i] = op(dest[i], src1[i], src2[i]) through dest's own strides (:58-67)."""
+    _same_dtype(dest, src1, src2)
+    _check_elementwise(dest, src1)
+    _check_elementwise(dest, src2)
+    if dest.size:
+        _ternary_into(op, dest, dest, src1, src2)
     return dest
 
 

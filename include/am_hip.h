@@ -234,6 +234,28 @@ int am_hip_ew_unary_i64(int op, int rank, const int64_t* shape,
                         int64_t* dst, const int64_t* dst_strides,
                         const int64_t* a, const int64_t* a_strides);
 
+/* dst[i] = op(a[i], b[i], c[i]): map3_inline / apply3_inline
+ * (src/arraymancer/tensor/higher_order_applymap.nim:58-67, 122-150) with the enumerated bodies the
+ * reference itself uses on this path (GRU gates over column slices of [batch, 3H] buffers,
+ * src/arraymancer/nn_primitives/nnp_gru.nim:80-88). Every arithmetic step is rounded on its own.
+ * dst may alias any operand exactly. Float tensors: all ops; integer tensors: AM_OP3_MULADD only. */
+#define AM_OP3_MULADD        0   /* x * y + z                                                  */
+#define AM_OP3_GRU_CANDIDATE 1   /* tanh(x + y * z)              apply3_inline(n, r, Uh)       */
+#define AM_OP3_GRU_BLEND     2   /* (1 - y) * z + y * x          apply3_inline(hidden, z, n)   */
+#define AM_OP3_COUNT         3
+int am_hip_ew_ternary_f32(int op, int rank, const int64_t* shape, float* dst, const int64_t* dst_strides,
+                          const float* a, const int64_t* a_strides, const float* b, const int64_t* b_strides,
+                          const float* c, const int64_t* c_strides);
+int am_hip_ew_ternary_f64(int op, int rank, const int64_t* shape, double* dst, const int64_t* dst_strides,
+                          const double* a, const int64_t* a_strides, const double* b, const int64_t* b_strides,
+                          const double* c, const int64_t* c_strides);
+int am_hip_ew_ternary_i32(int op, int rank, const int64_t* shape, int32_t* dst, const int64_t* dst_strides,
+                          const int32_t* a, const int64_t* a_strides, const int32_t* b, const int64_t* b_strides,
+                          const int32_t* c, const int64_t* c_strides);
+int am_hip_ew_ternary_i64(int op, int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides,
+                          const int64_t* a, const int64_t* a_strides, const int64_t* b, const int64_t* b_strides,
+                          const int64_t* c, const int64_t* c_strides);
+
 /* ---------------------------------------------------------------- measurement aid
  * No counterpart in the reference. Register-only micro-benchmarks of the issue ceilings the GEMM
  * kernels are compared with (used by bench.py; the survey's measurement plan asks for a measured

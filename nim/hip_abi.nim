@@ -103,6 +103,19 @@ proc am_hip_ew_scalar_i32*(op, scalar_on_left, rank: cint, shape: ptr int64, dst
 proc am_hip_ew_scalar_i64*(op, scalar_on_left, rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
                            a: ptr int64, a_strides: ptr int64, scalar: int64): cint {.importc.}
 
+proc am_hip_ew_ternary_f32*(op, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
+                            a: ptr cfloat, a_strides: ptr int64, b: ptr cfloat, b_strides: ptr int64,
+                            c: ptr cfloat, c_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_ternary_f64*(op, rank: cint, shape: ptr int64, dst: ptr cdouble, dst_strides: ptr int64,
+                            a: ptr cdouble, a_strides: ptr int64, b: ptr cdouble, b_strides: ptr int64,
+                            c: ptr cdouble, c_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_ternary_i32*(op, rank: cint, shape: ptr int64, dst: ptr int32, dst_strides: ptr int64,
+                            a: ptr int32, a_strides: ptr int64, b: ptr int32, b_strides: ptr int64,
+                            c: ptr int32, c_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_ternary_i64*(op, rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                            a: ptr int64, a_strides: ptr int64, b: ptr int64, b_strides: ptr int64,
+                            c: ptr int64, c_strides: ptr int64): cint {.importc.}
+
 proc am_hip_ew_unary_f32*(op, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
                           a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
 proc am_hip_ew_unary_f64*(op, rank: cint, shape: ptr int64, dst: ptr cdouble, dst_strides: ptr int64,

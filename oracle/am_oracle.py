@@ -28,6 +28,7 @@ _CT = {"f32": ctypes.c_float, "f64": ctypes.c_double, "i32": ctypes.c_int32, "i6
 # op codes of include/am_hip.h
 OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
           relu_bwd=8, max=9, min=10)
+OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
 
 
@@ -55,6 +56,9 @@ def lib() -> ctypes.CDLL:
             f = getattr(L, f"am_oracle_map2_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, p, p, p, p, p, p]
+            f = getattr(L, f"am_oracle_map3_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, p, p, p, p, p, p, p, p]
             f = getattr(L, f"am_oracle_scalar_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, ci, p, p, p, p, p, ct]
@@ -167,6 +171,22 @@ def map2(op, a: np.ndarray, b: np.ndarray, out: np.ndarray | None = None) -> np.
         a.ctypes.data, _i64arr(_estrides(a)), b.ctypes.data, _i64arr(_estrides(b)))
     if rc != 0:
         raise ValueError(f"oracle map2: op {op} not defined for {a.dtype} (rc={rc})")
+    return out
+
+
+def map3(op, a: np.ndarray, b: np.ndarray, c: np.ndarray, out: np.ndarray | None = None) -> np.ndarray:
+    """out[i] = op(a[i], b[i], c[i]); out=a is apply3_inline."""
+    op = OP3[op] if isinstance(op, str) else op
+    assert a.shape == b.shape == c.shape and a.dtype == b.dtype == c.dtype
+    if out is None:
+        out = np.empty(a.shape, dtype=a.dtype)
+    sfx = _sfx(a)
+    rc = getattr(lib(), f"am_oracle_map3_{sfx}")(
+        op, a.ndim, _i64arr(a.shape), out.ctypes.data, _i64arr(_estrides(out)),
+        a.ctypes.data, _i64arr(_estrides(a)), b.ctypes.data, _i64arr(_estrides(b)),
+        c.ctypes.data, _i64arr(_estrides(c)))
+    if rc != 0:
+        raise ValueError(f"oracle map3: op {op} not defined for {a.dtype} (rc={rc})")
     return out
 
 

@@ -264,3 +264,47 @@ def test_config4_8192_bit_exact(hip):
     assert np.array_equal(hip.bc_mul(dY, ds).toCpu(), Y * s)
     say("config4 bias+relu")
     assert np.array_equal(hip.bias_relu(dX, db).toCpu(), np.where(0 >= Y, np.float32(0), Y))
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_gru_cell_gates_on_column_slices(hip, oracle, sfx):
+    """The fused gate bodies of the reference's GRU cell (nn_primitives/nnp_gru.nim:73-88), applied in
+    place to column slices of [batch, 3H] buffers, against the oracle doing the same on NumPy views."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "gru"))
+    batch, H = 48, 256
+    W3x, U3h, hidden = fill(rng, (batch, 3 * H), dt), fill(rng, (batch, 3 * H), dt), fill(rng, (batch, H), dt)
+    dW, dU, dh = hip.toHip(W3x), hip.toHip(U3h), hip.toHip(hidden)
+    sr, sz, srz, s_ = slice(0, H), slice(H, 2 * H), slice(0, 2 * H), slice(2 * H, 3 * H)
+    say("gru step 2", sfx)
+    hip.apply2("add_sigmoid", dW[:, srz], dU[:, srz])
+    oracle.map2("add_sigmoid", W3x[:, srz], U3h[:, srz], out=W3x[:, srz])
+    say("gru step 3", sfx)
+    hip.apply3("gru_candidate", dW[:, s_], dW[:, sr], dU[:, s_])
+    oracle.map3("gru_candidate", W3x[:, s_], W3x[:, sr], U3h[:, s_], out=W3x[:, s_])
+    say("gru step 4", sfx)
+    hip.apply3("gru_blend", dh, dW[:, sz], dW[:, s_])
+    oracle.map3("gru_blend", hidden, W3x[:, sz], W3x[:, s_], out=hidden)
+    tol = 4e-6 if sfx == "f32" else 1e-13
+    np.testing.assert_allclose(dW.toCpu(), W3x, rtol=tol, atol=tol)
+    np.testing.assert_allclose(dh.toCpu(), hidden, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_map3_muladd_bit_exact(hip, oracle, sfx):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "map3"))
+    for shape in [(5,), (33, 1030), (4, 6, 258), (64, 4096)]:
+        a, b, c = fill(rng, shape, dt), fill(rng, shape, dt), fill(rng, shape, dt)
+        say("map3 muladd", sfx, shape)
+        got = hip.map3("muladd", hip.toHip(a), hip.toHip(b), hip.toHip(c)).toCpu()
+        assert np.array_equal(got, oracle.map3("muladd", a, b, c))
+        if len(shape) == 2:   # transposed operand -> generic kernel
+            got = hip.map3("muladd", hip.toHip(a), hip.toHip(np.ascontiguousarray(b.T)).transpose(), hip.toHip(c)).toCpu()
+            assert np.array_equal(got, oracle.map3("muladd", a, b, c))
+    if sfx in INT:
+        with pytest.raises(TypeError):
+            hip.map3("gru_blend", hip.toHip(a), hip.toHip(b), hip.toHip(c))
+    else:
+        x, y, z = (hip.toHip(t) for t in (a, b, c))
+        assert np.array_equal(hip.map3("gru_blend", x, y, z).toCpu(), oracle.map3("gru_blend", a, b, c))

@@ -187,3 +187,25 @@ def test_broadcast_errors(oracle):
         oracle.broadcast(np.zeros((3, 2)), (3, 3))
     with pytest.raises(ValueError):
         oracle.map2("mod", np.zeros(3, np.float32), np.zeros(3, np.float32))
+
+
+def test_map3_bodies_match_numpy(oracle):
+    """x*y+z and (1-y)*z+y*x are sequences of separately rounded IEEE operations: NumPy evaluates the
+    same sequence, so the comparison is bit-exact; tanh(x+y*z) is checked to libm accuracy."""
+    rng = np.random.default_rng(9)
+    for dt in (np.float32, np.float64):
+        base = rng.uniform(-2, 2, (3, 40, 48)).astype(dt)
+        x, y, z = base[0][:, 0:16], base[1][:, 16:32], base[2].T[8:24].T   # column slices, like the GRU gates
+        assert np.array_equal(oracle.map3("muladd", x, y, z), x * y + z)
+        assert np.array_equal(oracle.map3("gru_blend", x, y, z), (dt(1) - y) * z + y * x)
+        np.testing.assert_allclose(oracle.map3("gru_candidate", x, y, z), np.tanh((x + y * z).astype(np.float64)),
+                                   rtol=2e-6 if dt == np.float32 else 1e-14, atol=1e-7 if dt == np.float32 else 1e-15)
+        # apply3: destination is the first operand, written through its own strides
+        dst = base[0].copy()
+        want = dst.copy(); want[:, 0:16] = want[:, 0:16] * y + z
+        oracle.map3("muladd", dst[:, 0:16], y, z, out=dst[:, 0:16])
+        assert np.array_equal(dst, want)
+    a = np.array([2**31 - 1, -5, 7], dtype=np.int32)
+    assert oracle.map3("muladd", a, a, a).tolist() == [(((2**31 - 1) ** 2 + 2**31 - 1 + 2**31) % 2**32) - 2**31, 20, 56]
+    with pytest.raises(ValueError):
+        oracle.map3("gru_blend", a, a, a)
