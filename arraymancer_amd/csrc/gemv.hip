@@ -1,0 +1,259 @@
+// Matrix-vector product and dot product for gfx950 (HBM-bound): am_hip_gemv_*, am_hip_dot_*.
+//
+// y[M] <- alpha * A[M x N] * x[N] + beta * y      (src/arraymancer/tensor/operators_blas_l2l3.nim:24-56,
+//                                                 integer fallback fallback/naive_l2_gemv.nim:24-57)
+// dot(x, y)                                       (src/arraymancer/tensor/operators_blas_l1.nim:27-38)
+//
+// Every byte of A is needed once, so the kernels are shaped around the unit-stride direction of A:
+//   gemv_rows  A has unit column stride: one wavefront per row, lanes stride along the row with
+//              16-byte loads of A and x, 64-lane shuffle reduction at the end.
+//   gemv_cols  A has unit row stride (a transposed view): a lane owns VEC consecutive rows and
+//              walks the columns with 16-byte loads (coalesced along m); x[j] is one scalar load.
+//              The column range is cut over gridDim.y so the chip fills for short, wide matrices;
+//              partial vectors go through the split-K workspace and the shared reduce kernel.
+// Anything else (both strides non-unit, tiny M) runs as an N = 1 GEMM, which handles all strides.
+// Integer arithmetic wraps (unsigned twin); float partial sums are combined in a fixed order.
+#include "gemm_common.h"
+#include "gemm_loader.h"
+
+using namespace am;
+using namespace am::gemm;
+
+extern "C" int am_hip_gemm_f32(int64_t, int64_t, int64_t, float, const float*, int64_t, int64_t, const float*, int64_t, int64_t, float, float*, int64_t, int64_t);
+extern "C" int am_hip_gemm_f64(int64_t, int64_t, int64_t, double, const double*, int64_t, int64_t, const double*, int64_t, int64_t, double, double*, int64_t, int64_t);
+extern "C" int am_hip_gemm_i32(int64_t, int64_t, int64_t, int32_t, const int32_t*, int64_t, int64_t, const int32_t*, int64_t, int64_t, int32_t, int32_t*, int64_t, int64_t);
+extern "C" int am_hip_gemm_i64(int64_t, int64_t, int64_t, int64_t, const int64_t*, int64_t, int64_t, const int64_t*, int64_t, int64_t, int64_t, int64_t*, int64_t, int64_t);
+
+namespace {
+
+template <typename T> struct Acc { typedef T type; };
+template <> struct Acc<int32_t> { typedef uint32_t type; };
+template <> struct Acc<int64_t> { typedef uint64_t type; };
+
+template <typename U> __device__ __forceinline__ U wave_sum(U v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;   // lane 0 holds the total
+}
+template <> __device__ __forceinline__ uint32_t wave_sum<uint32_t>(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += (uint32_t)__shfl_down((int)v, off, 64);
+  return v;
+}
+template <> __device__ __forceinline__ uint64_t wave_sum<uint64_t>(uint64_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += (uint64_t)__shfl_down((long long)v, off, 64);
+  return v;
+}
+
+template <typename T> struct GemvArgs {
+  int64_t M, N;
+  T alpha, beta;
+  const T* A; int64_t rsA, csA;
+  const T* x; int64_t incx;
+  T* y; int64_t incy;
+  T* ws; int splits; int64_t n_chunk;
+};
+
+template <typename T, typename U>
+__device__ __forceinline__ void store_y(const GemvArgs<T>& p, int64_t row, U sum) {
+  T* yp = p.y + row * p.incy;
+  U v = (U)p.alpha * sum;
+  if (p.beta != (T)0) v += (U)p.beta * (U)*yp;
+  *yp = (T)v;
+}
+
+// A row-contiguous. VECLOAD: rows and x are 16-byte aligned and x has unit stride.
+template <typename T, bool VECLOAD>
+__global__ __launch_bounds__(256) void gemv_rows(GemvArgs<T> p) {
+  typedef typename Acc<T>::type U;
+  typedef typename VecTraits<T>::vec_t vec_t;
+  constexpr int VEC = VecTraits<T>::VK;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.M; row += (int64_t)gridDim.x * 4) {
+    const T* __restrict__ a = p.A + row * p.rsA;
+    U acc0 = 0, acc1 = 0;
+    if constexpr (VECLOAD) {
+      const int64_t nvec = p.N / VEC;
+      int64_t j = lane;
+      for (; j + 64 < nvec; j += 128) {
+        const vec_t a0 = __builtin_nontemporal_load((const vec_t*)a + j), a1 = __builtin_nontemporal_load((const vec_t*)a + j + 64);
+        const vec_t x0 = *((const vec_t*)p.x + j), x1 = *((const vec_t*)p.x + j + 64);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { acc0 += (U)a0[e] * (U)x0[e]; acc1 += (U)a1[e] * (U)x1[e]; }
+      }
+      for (; j < nvec; j += 64) {
+        const vec_t a0 = __builtin_nontemporal_load((const vec_t*)a + j);
+        const vec_t x0 = *((const vec_t*)p.x + j);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc0 += (U)a0[e] * (U)x0[e];
+      }
+      for (int64_t c = nvec * VEC + lane; c < p.N; c += 64) acc1 += (U)a[c] * (U)p.x[c];
+    } else {
+      for (int64_t c = lane; c < p.N; c += 64) acc0 += (U)a[c] * (U)p.x[c * p.incx];
+    }
+    const U total = wave_sum<U>(acc0 + acc1);
+    if (lane == 0) store_y<T, U>(p, row, total);
+  }
+}
+
+// A column-contiguous (unit row stride), rows and column starts 16-byte aligned, M % VEC == 0.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_cols(GemvArgs<T> p) {
+  typedef typename Acc<T>::type U;
+  typedef typename VecTraits<T>::vec_t vec_t;
+  constexpr int VEC = VecTraits<T>::VK;
+  const int64_t m = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (m >= p.M) return;
+  const int64_t j0 = (int64_t)blockIdx.y * p.n_chunk;
+  const int64_t j1 = (j0 + p.n_chunk < p.N) ? j0 + p.n_chunk : p.N;
+  U acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0;
+  const T* __restrict__ a = p.A + m;
+  int64_t j = j0;
+  for (; j + 4 <= j1; j += 4) {
+    vec_t v[4];
+    U xs[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      v[u] = __builtin_nontemporal_load((const vec_t*)(a + (j + u) * p.csA));
+      xs[u] = (U)p.x[(j + u) * p.incx];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] += (U)v[u][e] * xs[u];
+  }
+  for (; j < j1; ++j) {
+    const vec_t v = *(const vec_t*)(a + j * p.csA);
+    const U xj = (U)p.x[j * p.incx];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] += (U)v[e] * xj;
+  }
+  if (p.splits > 1) {
+    T* ws = p.ws + (int64_t)blockIdx.y * p.M + m;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ws[e] = (T)acc[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) store_y<T, U>(p, m + e, acc[e]);
+  }
+}
+
+// Per-workgroup partial dot products, one slot each, in the workspace.
+template <typename T>
+__global__ __launch_bounds__(256) void dot_partial(int64_t n, const T* x, int64_t incx, const T* y, int64_t incy, T* ws) {
+  typedef typename Acc<T>::type U;
+  __shared__ U part[4];
+  U acc = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    acc += (U)x[i * incx] * (U)y[i * incy];
+  acc = wave_sum<U>(acc);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) ws[blockIdx.x] = (T)(part[0] + part[1] + part[2] + part[3]);
+}
+
+template <typename T>
+int gemm_fallback(int64_t M, int64_t N, T alpha, const T* A, int64_t rsA, int64_t csA, const T* x, int64_t incx, T beta, T* y, int64_t incy);
+#define AM_GEMV_FALLBACK(T, SFX)                                                                                   \
+  template <> int gemm_fallback<T>(int64_t M, int64_t N, T alpha, const T* A, int64_t rsA, int64_t csA, const T* x, \
+                                   int64_t incx, T beta, T* y, int64_t incy) {                                     \
+    return am_hip_gemm_##SFX(M, 1, N, alpha, A, rsA, csA, x, incx, 1, beta, y, incy, 1);                            \
+  }
+AM_GEMV_FALLBACK(float, f32)
+AM_GEMV_FALLBACK(double, f64)
+AM_GEMV_FALLBACK(int32_t, i32)
+AM_GEMV_FALLBACK(int64_t, i64)
+
+template <typename T>
+int gemv(const char* fn, int64_t M, int64_t N, T alpha, const T* A, int64_t rsA, int64_t csA, const T* x,
+         int64_t incx, T beta, T* y, int64_t incy) {
+  typedef typename Acc<T>::type U;
+  constexpr int VEC = VecTraits<T>::VK;
+  if (M < 0 || N < 0) return fail(AM_E_ARG, "%s: negative dimension", fn);
+  if (M == 0) return AM_OK;
+  if (!y || (N > 0 && (!A || !x))) return fail(AM_E_ARG, "%s: null pointer", fn);
+  if (M > 1 && incy == 0) return fail(AM_E_SHAPE, "%s: y has stride 0", fn);
+  if (N == 0) return AM_OK;   // same convention as GEMM with K == 0: nothing runs, y untouched
+  AM_TRY(ensure_init());
+  GemvArgs<T> g;
+  g.M = M; g.N = N; g.alpha = alpha; g.beta = beta; g.A = A; g.rsA = rsA; g.csA = csA;
+  g.x = x; g.incx = incx; g.y = y; g.incy = incy; g.ws = nullptr; g.splits = 1; g.n_chunk = N;
+
+  if (csA == 1 && M >= 64) {
+    const bool vec = aligned16(A) && aligned16(x) && incx == 1 && (rsA % VEC == 0);
+    int64_t blocks = (M + 3) / 4;
+    const int64_t cap = (int64_t)num_cus() * 16;
+    if (blocks > cap) blocks = cap;
+    if (vec) hipLaunchKernelGGL((gemv_rows<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream(), g);
+    else hipLaunchKernelGGL((gemv_rows<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream(), g);
+    return check_launch("gemv_rows");
+  }
+  if (rsA == 1 && M % VEC == 0 && csA % VEC == 0 && csA >= 0 && aligned16(A) && M >= 256) {
+    const int64_t blocks_m = (M / VEC + 255) / 256;
+    int64_t splits = ((int64_t)num_cus() * 2 + blocks_m - 1) / blocks_m;
+    if (splits > N / 32) splits = N / 32;
+    if (splits > 64) splits = 64;
+    if (splits >= 2) {
+      const int64_t chunk = (N + splits - 1) / splits;
+      splits = (N + chunk - 1) / chunk;
+      T* ws = (T*)splitk_workspace((size_t)splits * M * sizeof(T));
+      if (ws && splits >= 2) { g.ws = ws; g.splits = (int)splits; g.n_chunk = chunk; }
+    }
+    hipLaunchKernelGGL((gemv_cols<T>), dim3((unsigned)blocks_m, (unsigned)g.splits), dim3(256), 0, stream(), g);
+    AM_TRY(check_launch("gemv_cols"));
+    if (g.splits > 1) {
+      Args<T> r;
+      memset(&r, 0, sizeof(r));
+      r.M = M; r.N = 1; r.K = N; r.alpha = alpha; r.beta = beta; r.C = y; r.c_m = incy; r.c_n = 0;
+      r.epilogue = AM_EPI_NONE; r.splits = g.splits; r.ws = g.ws;
+      return launch_splitk_reduce<T, U>(r);
+    }
+    return AM_OK;
+  }
+  return gemm_fallback<T>(M, N, alpha, A, rsA, csA, x, incx, beta, y, incy);
+}
+
+template <typename T>
+int dot(const char* fn, int64_t n, const T* x, int64_t incx, const T* y, int64_t incy, T* result) {
+  typedef typename Acc<T>::type U;
+  if (!result) return fail(AM_E_ARG, "%s: null result pointer", fn);
+  *result = (T)0;
+  if (n < 0) return fail(AM_E_ARG, "%s: negative length", fn);
+  if (n == 0) return AM_OK;
+  if (!x || !y) return fail(AM_E_ARG, "%s: null pointer", fn);
+  AM_TRY(ensure_init());
+  if (capturing()) return fail(AM_E_ARG, "%s: returns a value to the host, not allowed while a graph is being captured", fn);
+  int64_t blocks = (n + 1023) / 1024;
+  const int64_t cap = (int64_t)num_cus() * 4;
+  if (blocks > cap) blocks = cap;
+  T* ws = (T*)splitk_workspace((size_t)(blocks + 1) * sizeof(T));
+  if (!ws) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
+  hipLaunchKernelGGL((dot_partial<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), n, x, incx, y, incy, ws);
+  AM_TRY(check_launch("dot_partial"));
+  Args<T> r;
+  memset(&r, 0, sizeof(r));
+  r.M = 1; r.N = 1; r.K = n; r.alpha = (T)1; r.beta = (T)0; r.C = ws + blocks; r.c_m = 1; r.c_n = 1;
+  r.epilogue = AM_EPI_NONE; r.splits = (int)blocks; r.ws = ws;
+  AM_TRY((launch_splitk_reduce<T, U>(r)));
+  AM_HIP_TRY(hipMemcpyAsync(result, ws + blocks, sizeof(T), hipMemcpyDeviceToHost, stream()));
+  AM_HIP_TRY(hipStreamSynchronize(stream()));
+  return AM_OK;
+}
+
+}  // namespace
+
+#define AM_GEMV_ENTRY(T, SFX)                                                                                      \
+  extern "C" int am_hip_gemv_##SFX(int64_t M, int64_t N, T alpha, const T* A, int64_t rsA, int64_t csA, const T* x, \
+                                   int64_t incx, T beta, T* y, int64_t incy) {                                     \
+    return gemv<T>("am_hip_gemv_" #SFX, M, N, alpha, A, rsA, csA, x, incx, beta, y, incy);                         \
+  }                                                                                                                \
+  extern "C" int am_hip_dot_##SFX(int64_t n, const T* x, int64_t incx, const T* y, int64_t incy, T* result) {      \
+    return dot<T>("am_hip_dot_" #SFX, n, x, incx, y, incy, result);                                                \
+  }
+AM_GEMV_ENTRY(float, f32)
+AM_GEMV_ENTRY(double, f64)
+AM_GEMV_ENTRY(int32_t, i32)
+AM_GEMV_ENTRY(int64_t, i64)

@@ -367,12 +367,40 @@ def matmul(a: HipTensor, b: HipTensor) -> HipTensor:
             raise IndexError(f"Number of columns in the matrix: {a.shape[1]}, must be the same as the "
                              f"number of rows in the vector: {b.shape[0]}")
         out = empty((a.shape[0],), a.dtype)
-        bcol = HipTensor(Layout((b.shape[0], 1), (b.strides[0], 1), b.offset), b.storage, b.dtype)
-        ocol = HipTensor(Layout((a.shape[0], 1), (1, 1), 0), out.storage, out.dtype)
-        gemm(1, a, bcol, 0, ocol)
-        return out
+        return gemv(1, a, b, 0, out)
     raise ValueError("Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a "
                      "Matrix and second is a Matrix or Vector")
+
+
+def gemv(alpha, A: HipTensor, x: HipTensor, beta, y: HipTensor) -> HipTensor:
+    """y <- alpha * A * x + beta * y (src/arraymancer/tensor/operators_blas_l2l3.nim:24-56)."""
+    _same_dtype(A, x, y)
+    if A.rank != 2 or x.rank != 1 or y.rank != 1:
+        raise ValueError("gemv: A must be a matrix, x and y vectors")
+    if A.shape[1] != x.shape[0]:   # check_matvec, p_checks.nim:169-178
+        raise IndexError(f"Number of columns in the matrix: {A.shape[1]}, must be the same as the number "
+                         f"of rows in the vector: {x.shape[0]}")
+    if y.shape[0] != A.shape[0]:
+        raise IndexError(f"gemv: y has {y.shape[0]} elements, expected {A.shape[0]}")
+    ct = CTYPE[y.sfx]
+    check(getattr(_lib.load(), f"am_hip_gemv_{y.sfx}")(
+        A.shape[0], A.shape[1], ct(alpha), ctypes.c_void_p(A.data_ptr()), A.strides[0], A.strides[1],
+        ctypes.c_void_p(x.data_ptr()), x.strides[0], ct(beta), ctypes.c_void_p(y.data_ptr()), y.strides[0]))
+    return y
+
+
+def dot(a: HipTensor, b: HipTensor):
+    """Vector-vector scalar product, returned to the host
+    (src/arraymancer/tensor/operators_blas_l1.nim:27-38)."""
+    _same_dtype(a, b)
+    if a.rank != 1 or b.rank != 1 or a.shape != b.shape:
+        raise ValueError(f"dot: both operands must be vectors of the same length, got {list(a.shape)} and {list(b.shape)}")
+    ct = CTYPE[a.sfx]
+    out = ct()
+    check(getattr(_lib.load(), f"am_hip_dot_{a.sfx}")(
+        a.shape[0], ctypes.c_void_p(a.data_ptr()), a.strides[0], ctypes.c_void_p(b.data_ptr()), b.strides[0],
+        ctypes.byref(out)))
+    return a.dtype.type(out.value)
 
 
 def linear(x: HipTensor, weight: HipTensor, bias: HipTensor | None = None, relu: bool = False) -> HipTensor:

@@ -141,6 +141,26 @@ int am_hip_gemm_ex_f64(int64_t M, int64_t N, int64_t K, double alpha,
                        double beta, double* C, int64_t rsC, int64_t csC,
                        int epilogue, const double* bias, int64_t bias_rs, int64_t bias_cs);
 
+/* ---------------------------------------------------------------- GEMV and dot
+ * y[M] <- alpha * A[M x N] * x[N] + beta * y, any strides (elements).
+ * Replaces gemv (src/arraymancer/tensor/operators_blas_l2l3.nim:24-56; integer fallback
+ * fallback/naive_l2_gemv.nim:24-57; CUDA: operators_blas_l2l3_cuda.nim:20-41, which requires a
+ * contiguous A). N == 0 leaves y untouched, like K == 0 in GEMM. Integers wrap. */
+int am_hip_gemv_f32(int64_t M, int64_t N, float alpha, const float* A, int64_t rsA, int64_t csA,
+                    const float* x, int64_t incx, float beta, float* y, int64_t incy);
+int am_hip_gemv_f64(int64_t M, int64_t N, double alpha, const double* A, int64_t rsA, int64_t csA,
+                    const double* x, int64_t incx, double beta, double* y, int64_t incy);
+int am_hip_gemv_i32(int64_t M, int64_t N, int32_t alpha, const int32_t* A, int64_t rsA, int64_t csA,
+                    const int32_t* x, int64_t incx, int32_t beta, int32_t* y, int64_t incy);
+int am_hip_gemv_i64(int64_t M, int64_t N, int64_t alpha, const int64_t* A, int64_t rsA, int64_t csA,
+                    const int64_t* x, int64_t incx, int64_t beta, int64_t* y, int64_t incy);
+/* *result (HOST pointer) <- sum_i x[i * incx] * y[i * incy]; blocking.
+ * Replaces dot (src/arraymancer/tensor/operators_blas_l1.nim:27-38; CUDA: operators_blas_l1_cuda.nim:28-34). */
+int am_hip_dot_f32(int64_t n, const float* x, int64_t incx, const float* y, int64_t incy, float* result);
+int am_hip_dot_f64(int64_t n, const double* x, int64_t incx, const double* y, int64_t incy, double* result);
+int am_hip_dot_i32(int64_t n, const int32_t* x, int64_t incx, const int32_t* y, int64_t incy, int32_t* result);
+int am_hip_dot_i64(int64_t n, const int64_t* x, int64_t incx, const int64_t* y, int64_t incy, int64_t* result);
+
 /* ---------------------------------------------------------------- element-wise / broadcast / map
  * dst[i] = op(a[i], b[i]) over a common `shape` of `rank` dims (0 <= rank <= 6); each operand
  * is traversed in C order through its own strides (elements; 0 = broadcast, negative allowed

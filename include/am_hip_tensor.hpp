@@ -65,6 +65,19 @@ namespace detail {
                     const int64_t* sa) {                                                                 \
     return am_hip_ew_unary_##SFX(op, rank, sh, d, sd, a, sa);                                             \
   }
+#define AM_HPP_BIND2(T, SFX)                                                                             \
+  inline int gemv_(int64_t M, int64_t N, T al, const T* A, int64_t ra, int64_t ca, const T* x, int64_t ix, \
+                   T be, T* y, int64_t iy) {                                                              \
+    return am_hip_gemv_##SFX(M, N, al, A, ra, ca, x, ix, be, y, iy);                                      \
+  }                                                                                                      \
+  inline int dot_(int64_t n, const T* x, int64_t ix, const T* y, int64_t iy, T* r) {                     \
+    return am_hip_dot_##SFX(n, x, ix, y, iy, r);                                                          \
+  }
+AM_HPP_BIND2(float, f32)
+AM_HPP_BIND2(double, f64)
+AM_HPP_BIND2(int32_t, i32)
+AM_HPP_BIND2(int64_t, i64)
+#undef AM_HPP_BIND2
 AM_HPP_BIND(float, f32)
 AM_HPP_BIND(double, f64)
 AM_HPP_BIND(int32_t, i32)
@@ -308,7 +321,27 @@ void gemm(T alpha, const HipTensor<T>& A, const HipTensor<T>& B, T beta, HipTens
                       B.strides[0], B.strides[1], beta, C.ptr(), C.strides[0], C.strides[1]));
 }
 
-// `*` (operators_blas_l2l3.nim:88-100): matrix-matrix, or matrix-vector (run as an N = 1 product).
+// y <- alpha A x + beta y (operators_blas_l2l3.nim:24-56)
+template <typename T>
+void gemv(T alpha, const HipTensor<T>& A, const HipTensor<T>& x, T beta, HipTensor<T>& y) {
+  if (A.rank() != 2 || x.rank() != 1 || y.rank() != 1) throw std::invalid_argument("gemv: A must be a matrix, x and y vectors");
+  if (A.shape[1] != x.shape[0] || A.shape[0] != y.shape[0])
+    throw std::out_of_range("Number of columns in the matrix: " + std::to_string(A.shape[1]) +
+                            ", must be the same as the number of rows in the vector: " + std::to_string(x.shape[0]));
+  check(detail::gemv_(A.shape[0], A.shape[1], alpha, A.ptr(), A.strides[0], A.strides[1], x.ptr(), x.strides[0], beta,
+                      y.ptr(), y.strides[0]));
+}
+
+// Scalar product, returned to the host (operators_blas_l1.nim:27-38).
+template <typename T>
+T dot(const HipTensor<T>& a, const HipTensor<T>& b) {
+  if (a.rank() != 1 || b.rank() != 1 || a.shape != b.shape) throw std::invalid_argument("dot: vectors of equal length expected");
+  T r{};
+  check(detail::dot_(a.shape[0], a.ptr(), a.strides[0], b.ptr(), b.strides[0], &r));
+  return r;
+}
+
+// `*` (operators_blas_l2l3.nim:88-100): matrix-matrix, or matrix-vector.
 template <typename T>
 HipTensor<T> operator*(const HipTensor<T>& a, const HipTensor<T>& b) {
   if (a.rank() == 2 && b.rank() == 2) {
@@ -321,10 +354,7 @@ HipTensor<T> operator*(const HipTensor<T>& a, const HipTensor<T>& b) {
   }
   if (a.rank() == 2 && b.rank() == 1) {
     HipTensor<T> r(Shape{a.shape[0]});
-    HipTensor<T> bcol = b, ocol = r;
-    bcol.shape.push_back(1); bcol.strides.push_back(1);
-    ocol.shape.push_back(1); ocol.strides.push_back(1);
-    gemm(T(1), a, bcol, T(0), ocol);
+    gemv(T(1), a, b, T(0), r);
     return r;
   }
   throw std::invalid_argument("Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a Matrix "

@@ -62,6 +62,19 @@ proc am_hip_gemm_i64*(M, N, K: int64, alpha: int64, A: ptr int64, rsA, csA: int6
                       B: ptr int64, rsB, csB: int64, beta: int64,
                       C: ptr int64, rsC, csC: int64): cint {.importc.}
 
+proc am_hip_gemv_f32*(M, N: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64, x: ptr cfloat, incx: int64,
+                      beta: cfloat, y: ptr cfloat, incy: int64): cint {.importc.}
+proc am_hip_gemv_f64*(M, N: int64, alpha: cdouble, A: ptr cdouble, rsA, csA: int64, x: ptr cdouble, incx: int64,
+                      beta: cdouble, y: ptr cdouble, incy: int64): cint {.importc.}
+proc am_hip_gemv_i32*(M, N: int64, alpha: int32, A: ptr int32, rsA, csA: int64, x: ptr int32, incx: int64,
+                      beta: int32, y: ptr int32, incy: int64): cint {.importc.}
+proc am_hip_gemv_i64*(M, N: int64, alpha: int64, A: ptr int64, rsA, csA: int64, x: ptr int64, incx: int64,
+                      beta: int64, y: ptr int64, incy: int64): cint {.importc.}
+proc am_hip_dot_f32*(n: int64, x: ptr cfloat, incx: int64, y: ptr cfloat, incy: int64, res: ptr cfloat): cint {.importc.}
+proc am_hip_dot_f64*(n: int64, x: ptr cdouble, incx: int64, y: ptr cdouble, incy: int64, res: ptr cdouble): cint {.importc.}
+proc am_hip_dot_i32*(n: int64, x: ptr int32, incx: int64, y: ptr int32, incy: int64, res: ptr int32): cint {.importc.}
+proc am_hip_dot_i64*(n: int64, x: ptr int64, incx: int64, y: ptr int64, incy: int64, res: ptr int64): cint {.importc.}
+
 const
   AM_EPI_NONE* = 0.cint
   AM_EPI_BIAS* = 1.cint

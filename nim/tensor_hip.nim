@@ -281,18 +281,31 @@ proc gemm*[T: HipScalar](alpha: T, A, B: HipTensor[T], beta: T, C: var HipTensor
   elif T is int32: call am_hip_gemm_i32
   else: call am_hip_gemm_i64
 
+proc gemv*[T: HipScalar](alpha: T, A, x: HipTensor[T], beta: T, y: var HipTensor[T]) =
+  ## y <- alpha A x + beta y (operators_blas_l2l3.nim:24-56)
+  template call(f: untyped) =
+    check f(int64 A.shape[0], int64 A.shape[1], alpha, A.get_offset_ptr, int64 A.strides[0], int64 A.strides[1],
+            x.get_offset_ptr, int64 x.strides[0], beta, y.get_offset_ptr, int64 y.strides[0])
+  when T is float32: call am_hip_gemv_f32
+  elif T is float64: call am_hip_gemv_f64
+  elif T is int32: call am_hip_gemv_i32
+  else: call am_hip_gemv_i64
+
+proc dot*[T: HipScalar](a, b: HipTensor[T]): T =
+  ## operators_blas_l1.nim:27-38
+  when T is float32: check am_hip_dot_f32(int64 a.shape[0], a.get_offset_ptr, int64 a.strides[0], b.get_offset_ptr, int64 b.strides[0], result.addr)
+  elif T is float64: check am_hip_dot_f64(int64 a.shape[0], a.get_offset_ptr, int64 a.strides[0], b.get_offset_ptr, int64 b.strides[0], result.addr)
+  elif T is int32: check am_hip_dot_i32(int64 a.shape[0], a.get_offset_ptr, int64 a.strides[0], b.get_offset_ptr, int64 b.strides[0], result.addr)
+  else: check am_hip_dot_i64(int64 a.shape[0], a.get_offset_ptr, int64 a.strides[0], b.get_offset_ptr, int64 b.strides[0], result.addr)
+
 proc `*`*[T: HipScalar](a, b: HipTensor[T]): HipTensor[T] =
-  ## Matrix-matrix product (operators_blas_l2l3.nim:88-100). Matrix-vector runs as an N = 1 product.
+  ## Matrix-matrix product (operators_blas_l2l3.nim:88-100); matrix-vector goes to gemv.
   if a.rank == 2 and b.rank == 2:
     result = newHipTensor[T]([a.shape[0], b.shape[1]])
     gemm(T(1), a, b, T(0), result)
   elif a.rank == 2 and b.rank == 1:
     result = newHipTensor[T]([a.shape[0]])
-    var bcol = b
-    bcol.shape.add 1; bcol.strides.add 1
-    var ocol = result
-    ocol.shape.add 1; ocol.strides.add 1
-    gemm(T(1), a, bcol, T(0), ocol)
+    gemv(T(1), a, b, T(0), result)
   else:
     raise newException(ValueError, "Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a Matrix and second is a Matrix or Vector")
 

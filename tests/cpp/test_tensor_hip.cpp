@@ -75,6 +75,9 @@ static void integer_slices() {
   CHECK(eq(b2 * u2, {10027, -3682}));
   auto b3 = b.slice(0, 2, 3).slice(1, 3, 1, -2);
   CHECK(eq(b3 * u2, {-3682, -4783}));
+  // dot, test_operators_blas.nim:195-201
+  CHECK(am::dot(toHip<int64_t>({1, 3, -5}, {3}), toHip<int64_t>({4, -2, -1}, {3})) == 3);
+  CHECK(am::dot(toHip<double>({1, 3, -5}, {3}), toHip<double>({4, -2, -1}, {3})) == 3.0);
   // wraparound
   auto w = toHip<int32_t>({2147483647, 1}, {1, 2});
   auto x = toHip<int32_t>({2, 3}, {2, 1});
