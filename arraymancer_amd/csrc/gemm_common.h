@@ -31,6 +31,11 @@ template <typename T> struct Args {
   int splits;
   int64_t k_chunk;
   T* ws;
+  // Strided batch: workgroups with blockIdx.y = z work on A + z * batch_a, B + z * batch_b,
+  // C + z * batch_c (elements); the bias is shared by the whole batch.
+  int batch;
+  int64_t batch_a, batch_b, batch_c;
+  bool swapped;                    // prepare() exchanged the roles of A and B (column-major C)
 };
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -83,6 +88,8 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   }
   g.K = K; g.alpha = alpha; g.beta = beta; g.C = C;
   g.epilogue = epilogue; g.bias = bias;
+  g.batch = 1; g.batch_a = g.batch_b = g.batch_c = 0;
+  g.swapped = swap;
   g.a_kfast = iabs64(g.a_k) <= iabs64(g.a_mn);
   g.b_kfast = iabs64(g.b_k) < iabs64(g.b_mn);
   return AM_OK;
@@ -93,7 +100,7 @@ struct TileChoice { int bm, bn; double eff; };
 
 // Picks the candidate with the least estimated time: rounds of one block per CU, each round
 // costing bm*bn/eff. Ragged edges and under-filled rounds are priced by construction.
-static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int64_t N, const char* env) {
+static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int64_t N, const char* env, int64_t batch = 1) {
   const char* forced = getenv(env);
   if (forced && *forced) {
     int idx = atoi(forced);
@@ -104,7 +111,7 @@ static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int6
   double best_cost = 0;
   for (int i = 0; i < ncand; ++i) {
     if (cand[i].eff <= 0) continue;   // experimental shape: only when forced
-    const int64_t tiles = ((M + cand[i].bm - 1) / cand[i].bm) * ((N + cand[i].bn - 1) / cand[i].bn);
+    const int64_t tiles = ((M + cand[i].bm - 1) / cand[i].bm) * ((N + cand[i].bn - 1) / cand[i].bn) * batch;
     const int64_t rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * cand[i].bm * cand[i].bn / cand[i].eff;
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
@@ -122,6 +129,7 @@ void* splitk_workspace(size_t bytes);
 template <typename T>
 static inline void plan_splitk(Args<T>& g, int bk, int waves_per_tile) {
   g.splits = 1; g.k_chunk = g.K; g.ws = nullptr;
+  if (g.batch > 1) return;   // a batch already supplies the parallelism
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
   const int64_t simds = (int64_t)num_cus() * 4;
   const int64_t slabs = (g.K + bk - 1) / bk;

@@ -5,11 +5,14 @@ using namespace am;
 using namespace am::gemm;
 
 static int run_f32(Args<float>& g) {
-  const int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
-  const int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
+  constexpr int64_t VK = 16 / (int64_t)sizeof(float);
+  int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
+  int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
+  if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;   // every batch member must stay 16-byte aligned
+  if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
   // Candidate workgroup tiles, largest first, with the relative MFMA efficiency of each.
   static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.95}, {64, 64, 0.89}, {256, 128, 0.97}, {128, 64, 0.93}, {32, 32, 0.6}, {64, 64, 0.0}, {32, 32, 0.0}, {128, 128, 0.0}};
-  switch (choose_tile(cand, 9, g.M, g.N, "AM_HIP_GEMM_TILE_F32")) {
+  switch (choose_tile(cand, 9, g.M, g.N, "AM_HIP_GEMM_TILE_F32", g.batch)) {
     case 0: return launch_kinds<float, 256, 256, 16, 2, 4>(g, ak, bk);
     case 1: return launch_kinds<float, 128, 128, 16, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2>(g, ak, bk);
@@ -40,4 +43,24 @@ extern "C" int am_hip_gemm_f32(int64_t M, int64_t N, int64_t K, float alpha, con
                                int64_t rsC, int64_t csC) {
   return am_hip_gemm_ex_f32(M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC, AM_EPI_NONE,
                             nullptr, 0, 0);
+}
+
+extern "C" int am_hip_gemm_batched_f32(int64_t batch, int64_t M, int64_t N, int64_t K, float alpha, const float* A,
+                                       int64_t rsA, int64_t csA, int64_t bsA, const float* B, int64_t rsB, int64_t csB,
+                                       int64_t bsB, float beta, float* C, int64_t rsC, int64_t csC, int64_t bsC,
+                                       int epilogue, const float* bias, int64_t bias_rs, int64_t bias_cs) {
+  if (batch < 0 || batch > 65535) return fail(AM_E_ARG, "am_hip_gemm_batched_f32: batch %lld outside 0..65535", (long long)batch);
+  if (batch == 0) return AM_OK;
+  Args<float> g;
+  const int rc = prepare<float>("am_hip_gemm_batched_f32", M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC,
+                            epilogue, bias, bias_rs, bias_cs, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  if (batch > 1 && bsC == 0) return fail(AM_E_SHAPE, "am_hip_gemm_batched_f32: C has batch stride 0");
+  g.batch = (int)batch;
+  g.batch_a = g.swapped ? bsB : bsA;
+  g.batch_b = g.swapped ? bsA : bsB;
+  g.batch_c = bsC;
+  AM_TRY(ensure_init());
+  return run_f32(g);
 }

@@ -4,6 +4,19 @@
 using namespace am;
 using namespace am::gemm;
 
+static int run_i32(Args<int32_t>& g) {
+  constexpr int64_t VK = 16 / (int64_t)sizeof(int32_t);
+  int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
+  int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
+  if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;
+  if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
+  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 1.0}};
+  switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_GEMM_TILE_I32", g.batch)) {
+    case 0: return launch_valu<int32_t, 8, 8, 16>(g, ak, bk);
+    default: return launch_valu<int32_t, 4, 4, 16>(g, ak, bk);
+  }
+}
+
 extern "C" int am_hip_gemm_i32(int64_t M, int64_t N, int64_t K, int32_t alpha, const int32_t* A, int64_t rsA,
                                int64_t csA, const int32_t* B, int64_t rsB, int64_t csB, int32_t beta, int32_t* C,
                                int64_t rsC, int64_t csC) {
@@ -13,11 +26,28 @@ extern "C" int am_hip_gemm_i32(int64_t M, int64_t N, int64_t K, int32_t alpha, c
   if (rc > 0) return AM_OK;
   if (rc < 0) return rc;
   AM_TRY(ensure_init());
-  const int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
-  const int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
-  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 1.0}};
-  switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_GEMM_TILE_I32")) {
-    case 0: return launch_valu<int32_t, 8, 8, 16>(g, ak, bk);
-    default: return launch_valu<int32_t, 4, 4, 16>(g, ak, bk);
-  }
+  return run_i32(g);
+}
+
+// Integer batched product: no fused epilogue (pass AM_EPI_NONE; add a bias with the element-wise ops).
+extern "C" int am_hip_gemm_batched_i32(int64_t batch, int64_t M, int64_t N, int64_t K, int32_t alpha, const int32_t* A,
+                                       int64_t rsA, int64_t csA, int64_t bsA, const int32_t* B, int64_t rsB, int64_t csB,
+                                       int64_t bsB, int32_t beta, int32_t* C, int64_t rsC, int64_t csC, int64_t bsC,
+                                       int epilogue, const int32_t* bias, int64_t bias_rs, int64_t bias_cs) {
+  (void)bias; (void)bias_rs; (void)bias_cs;
+  if (epilogue != AM_EPI_NONE) return fail(AM_E_DTYPE, "am_hip_gemm_batched_i32: fused epilogues are defined for float tensors");
+  if (batch < 0 || batch > 65535) return fail(AM_E_ARG, "am_hip_gemm_batched_i32: batch %lld outside 0..65535", (long long)batch);
+  if (batch == 0) return AM_OK;
+  Args<int32_t> g;
+  const int rc = prepare<int32_t>("am_hip_gemm_batched_i32", M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC,
+                            AM_EPI_NONE, nullptr, 0, 0, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  if (batch > 1 && bsC == 0) return fail(AM_E_SHAPE, "am_hip_gemm_batched_i32: C has batch stride 0");
+  g.batch = (int)batch;
+  g.batch_a = g.swapped ? bsB : bsA;
+  g.batch_b = g.swapped ? bsA : bsB;
+  g.batch_c = bsC;
+  AM_TRY(ensure_init());
+  return run_i32(g);
 }

@@ -47,6 +47,12 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
     bid -= split * nt;
   }
   tile_of_block(bid, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  if (p.batch > 1) {
+    const int64_t z = blockIdx.y;
+    p.A += z * p.batch_a;
+    p.B += z * p.batch_b;
+    p.C += z * p.batch_c;
+  }
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
   const int64_t k_begin = (int64_t)split * p.k_chunk;
   const int64_t k_end = (k_begin + p.k_chunk < p.K) ? k_begin + p.k_chunk : p.K;
@@ -149,7 +155,7 @@ static int launch_valu(Args<T>& g, int ak, int bk) {
   const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
   if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
   plan_splitk(g, BK, 4);
-  const dim3 grid((unsigned)(nb * g.splits)), block(256);
+  const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(256);
 #define AM_LAUNCH(AKIND, BKIND_) \
   hipLaunchKernelGGL((gemm_valu<T, TM, TN, BK, AKIND, BKIND_>), grid, block, 0, stream(), g)
   switch (ak * 3 + bk) {

@@ -403,6 +403,77 @@ def dot(a: HipTensor, b: HipTensor):
     return a.dtype.type(out.value)
 
 
+def gemm_batched(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none", bias: HipTensor | None = None):
+    """C[z] <- alpha * A[z] * B[z] + beta * C[z] for rank-3 operands [batch, rows, cols] in one
+    launch. A or B of rank 2 is shared by the whole batch (batch stride 0)."""
+    dtype = _same_dtype(A, B, C)
+    if C.rank != 3 or A.rank not in (2, 3) or B.rank not in (2, 3):
+        raise ValueError("gemm_batched: C must be [batch, M, N]; A and B [batch, ., .] or shared matrices")
+    batch, M, N = C.shape
+    a_sh, a_st, a_b = (A.shape[-2:], A.strides[-2:], A.strides[0] if A.rank == 3 else 0)
+    b_sh, b_st, b_b = (B.shape[-2:], B.strides[-2:], B.strides[0] if B.rank == 3 else 0)
+    if (A.rank == 3 and A.shape[0] != batch) or (B.rank == 3 and B.shape[0] != batch):
+        raise IndexError("gemm_batched: batch sizes differ")
+    K = a_sh[1]
+    if a_sh[0] != M or b_sh != (K, N):
+        raise IndexError(f"gemm_batched: shapes {list(A.shape)} x {list(B.shape)} -> {list(C.shape)} do not agree")
+    sfx, ct = C.sfx, CTYPE[C.sfx]
+    epi = EPI[epilogue] if isinstance(epilogue, str) else int(epilogue)
+    bptr, brs, bcs = None, 0, 0
+    if epi & 1:
+        if bias is None:
+            raise ValueError("bias epilogue needs a bias tensor")
+        bb = bias.broadcast((M, N))
+        bptr, brs, bcs = ctypes.c_void_p(bb.data_ptr()), bb.strides[0], bb.strides[1]
+    check(getattr(_lib.load(), f"am_hip_gemm_batched_{sfx}")(
+        batch, M, N, K, ct(alpha), ctypes.c_void_p(A.data_ptr()), a_st[0], a_st[1], a_b,
+        ctypes.c_void_p(B.data_ptr()), b_st[0], b_st[1], b_b, ct(beta),
+        ctypes.c_void_p(C.data_ptr()), C.strides[1], C.strides[2], C.strides[0], epi, bptr, brs, bcs))
+    return C
+
+
+def im2col(x: HipTensor, kernel_size, padding=(0, 0), stride=(1, 1)) -> HipTensor:
+    """[N, C, H, W] -> [N, C*kH*kW, H_out*W_out] on the device, whole batch in one launch
+    (src/arraymancer/nn_primitives/fallback/conv.nim:18-54 does one image per call on the host)."""
+    if x.rank != 4:
+        raise ValueError("im2col: input must be [N, C, H, W]")
+    N, C, H, W = x.shape
+    (kh, kw), (ph, pw), (sh, sw) = kernel_size, padding, stride
+    ho, wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    col = empty((N, C * kh * kw, ho * wo), x.dtype)
+    check(getattr(_lib.load(), f"am_hip_im2col_{x.sfx}")(
+        N, C, H, W, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(x.data_ptr()), *x.strides, ctypes.c_void_p(col.data_ptr())))
+    return col
+
+
+def conv2d(x: HipTensor, kernel: HipTensor, bias: HipTensor | None = None, padding=(0, 0), stride=(1, 1),
+           relu: bool = False) -> HipTensor:
+    """im2colgemm_conv2d (src/arraymancer/nn_primitives/fallback/conv.nim:81-106) in two launches:
+    device im2col of the batch, then one strided-batched GEMM kernel_col[C_out, C*kH*kW] * col[n]
+    written straight into the NCHW result, with the bias [C_out, 1, 1] (and an optional ReLU) fused
+    into its epilogue for float tensors."""
+    _same_dtype(x, kernel)
+    N, C, H, W = x.shape
+    co, ci, kh, kw = kernel.shape
+    if ci != C:
+        raise ValueError(f"conv2d: kernel expects {ci} input channels, input has {C}")
+    col = im2col(x, (kh, kw), padding, stride)
+    ho, wo = (H + 2 * padding[0] - kh) // stride[0] + 1, (W + 2 * padding[1] - kw) // stride[1] + 1
+    out = empty((N, co, ho, wo), x.dtype)
+    out3 = out.reshape(N, co, ho * wo)
+    kcol = kernel.reshape(co, ci * kh * kw)
+    is_float = x.dtype.kind == "f"
+    if bias is not None and is_float:
+        gemm_batched(1, kcol, col, 0, out3, epilogue="bias_relu" if relu else "bias", bias=bias.reshape(co, 1))
+    else:
+        gemm_batched(1, kcol, col, 0, out3, epilogue="relu" if (relu and is_float) else "none")
+        if bias is not None:
+            out3.bc_iadd(bias.reshape(1, co, 1))
+        if relu and not is_float:
+            _unary_into("relu", out3, out3)
+    return out
+
+
 def linear(x: HipTensor, weight: HipTensor, bias: HipTensor | None = None, relu: bool = False) -> HipTensor:
     """out = x * weight.transpose (+ bias) (then ReLU) in ONE kernel — the three passes of
     src/arraymancer/nn_primitives/nnp_linear.nim:20-29 + nnp_activation.nim:35-36 fused into the

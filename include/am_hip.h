@@ -141,6 +141,46 @@ int am_hip_gemm_ex_f64(int64_t M, int64_t N, int64_t K, double alpha,
                        double beta, double* C, int64_t rsC, int64_t csC,
                        int epilogue, const double* bias, int64_t bias_rs, int64_t bias_cs);
 
+/* Strided-batched GEMM: for z in 0..batch-1, C + z*batch_stride_C <- alpha * (A + z*batch_stride_A)
+ * * (B + z*batch_stride_B) + beta * C_z, one launch. A batch stride of 0 shares the operand (the
+ * convolution kernel matrix). The bias is shared by the batch. Integer types: epilogue must be
+ * AM_EPI_NONE. Replaces the per-image GEMM loop of the reference's convolution
+ * (src/arraymancer/nn_primitives/fallback/conv.nim:99-103, "TODO: batch matmul"); the CUDA backend
+ * wraps cublas gemmStridedBatched for the same purpose (backend/cublas.nim:172-208). */
+int am_hip_gemm_batched_f32(int64_t batch, int64_t M, int64_t N, int64_t K, float alpha,
+                            const float* A, int64_t rsA, int64_t csA, int64_t batch_stride_A,
+                            const float* B, int64_t rsB, int64_t csB, int64_t batch_stride_B,
+                            float beta, float* C, int64_t rsC, int64_t csC, int64_t batch_stride_C,
+                            int epilogue, const float* bias, int64_t bias_rs, int64_t bias_cs);
+int am_hip_gemm_batched_f64(int64_t batch, int64_t M, int64_t N, int64_t K, double alpha,
+                            const double* A, int64_t rsA, int64_t csA, int64_t batch_stride_A,
+                            const double* B, int64_t rsB, int64_t csB, int64_t batch_stride_B,
+                            double beta, double* C, int64_t rsC, int64_t csC, int64_t batch_stride_C,
+                            int epilogue, const double* bias, int64_t bias_rs, int64_t bias_cs);
+int am_hip_gemm_batched_i32(int64_t batch, int64_t M, int64_t N, int64_t K, int32_t alpha,
+                            const int32_t* A, int64_t rsA, int64_t csA, int64_t batch_stride_A,
+                            const int32_t* B, int64_t rsB, int64_t csB, int64_t batch_stride_B,
+                            int32_t beta, int32_t* C, int64_t rsC, int64_t csC, int64_t batch_stride_C,
+                            int epilogue, const int32_t* bias, int64_t bias_rs, int64_t bias_cs);
+int am_hip_gemm_batched_i64(int64_t batch, int64_t M, int64_t N, int64_t K, int64_t alpha,
+                            const int64_t* A, int64_t rsA, int64_t csA, int64_t batch_stride_A,
+                            const int64_t* B, int64_t rsB, int64_t csB, int64_t batch_stride_B,
+                            int64_t beta, int64_t* C, int64_t rsC, int64_t csC, int64_t batch_stride_C,
+                            int epilogue, const int64_t* bias, int64_t bias_rs, int64_t bias_cs);
+
+/* col[n][c*kH*kW + kh*kW + kw][h*W_out + w] <- padded input patch element, for the whole batch in
+ * one launch; `in` is addressed through its four NCHW strides (elements), `col` is a contiguous
+ * [N, C*kH*kW, H_out*W_out] buffer. H_out = (H + 2 padH - kH) / strideH + 1, W_out alike.
+ * Replaces im2col (src/arraymancer/nn_primitives/fallback/conv.nim:18-54). */
+int am_hip_im2col_f32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const float* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, float* col);
+int am_hip_im2col_f64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const double* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, double* col);
+int am_hip_im2col_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const int32_t* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, int32_t* col);
+int am_hip_im2col_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const int64_t* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, int64_t* col);
+
 /* ---------------------------------------------------------------- GEMV and dot
  * y[M] <- alpha * A[M x N] * x[N] + beta * y, any strides (elements).
  * Replaces gemv (src/arraymancer/tensor/operators_blas_l2l3.nim:24-56; integer fallback

@@ -216,6 +216,42 @@ def unary(op, a: np.ndarray, out: np.ndarray | None = None) -> np.ndarray:
     return out
 
 
+def im2col(img: np.ndarray, kernel_size, padding=(0, 0), stride=(1, 1)) -> np.ndarray:
+    """im2col of ONE image [C, H, W] -> [C*kH*kW, H_out*W_out], loop for loop as the reference
+    (src/arraymancer/nn_primitives/fallback/conv.nim:18-54)."""
+    C, H, W = img.shape
+    (kh, kw), (ph, pw), (sh, sw) = kernel_size, padding, stride
+    hc, wc = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    out = np.zeros((C * kh * kw, hc * wc), dtype=img.dtype)
+    flat = img.reshape(-1)
+    for c in range(C * kh * kw):
+        w_off, h_off, c_off = c % kw - pw, (c // kw) % kh - ph, (c // kw) // kh
+        for h in range(hc):
+            row = h_off + h * sh
+            for w in range(wc):
+                col = w_off + w * sw
+                if 0 <= row < H and 0 <= col < W:
+                    out[c, h * wc + w] = flat[c_off * H * W + row * W + col]
+    return out
+
+
+def conv2d(x: np.ndarray, kernel: np.ndarray, bias: np.ndarray | None, padding=(0, 0), stride=(1, 1)) -> np.ndarray:
+    """im2colgemm_conv2d (fallback/conv.nim:81-106): per image im2col, gemm(1, kernel_col, input_col,
+    0, out_view) through the restated laser GEMM, then result +.= bias.unsqueeze(0)."""
+    N, C, H, W = x.shape
+    co, _, kh, kw = kernel.shape
+    ho, wo = (H + 2 * padding[0] - kh) // stride[0] + 1, (W + 2 * padding[1] - kw) // stride[1] + 1
+    kcol = np.ascontiguousarray(kernel.reshape(co, C * kh * kw))
+    out = np.empty((N, co, ho, wo), dtype=x.dtype)
+    for n in range(N):
+        col = im2col(np.ascontiguousarray(x[n]), (kh, kw), padding, stride)
+        gemm_strided(1, kcol, col, 0, out[n].reshape(co, ho * wo))
+    if bias is not None:
+        b = broadcast(bias.reshape(1, co, 1, 1), out.shape)
+        map2("add", out, b, out=out)
+    return out
+
+
 # ----------------------------------------------------------------------------- closed forms
 def closed_gemm_int(alpha, A, B, beta, C):
     """Exact integer result of alpha*A*B + beta*C reduced modulo 2^w (w = bit width of the dtype).

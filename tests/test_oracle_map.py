@@ -209,3 +209,15 @@ def test_map3_bodies_match_numpy(oracle):
     assert oracle.map3("muladd", a, a, a).tolist() == [(((2**31 - 1) ** 2 + 2**31 - 1 + 2**31) % 2**32) - 2**31, 20, 56]
     with pytest.raises(ValueError):
         oracle.map3("gru_blend", a, a, a)
+
+
+def test_reference_conv_vectors(vectors, oracle):
+    """im2col + GEMM + bias against the reference's convolution literals
+    (tests/nn_primitives/test_nnp_convolution.nim:21-134)."""
+    for case in vectors["conv_im2col"]:
+        for dt in (np.float32, np.int64, np.float64, np.int32):
+            x = np.array(case["input"], dtype=dt)
+            k = np.array(case["kernel"], dtype=dt)
+            b = np.array(case["bias"], dtype=dt)
+            got = oracle.conv2d(x, k, b, tuple(case["padding"]), tuple(case["stride"]))
+            assert np.array_equal(got, np.array(case["target"], dtype=dt)), case["name"]
