@@ -153,7 +153,7 @@ def other_workloads(am, timer, steps, warmup):
 
 
 def chain_setup(am):
-    """The MNIST-shaped inference chain of BASELINE config 5 (batch 64): conv1 and conv2 as im2col
+    """The MNIST-shaped inference chain (batch 64): conv1 and conv2 as im2col
     GEMMs, dense + bias + ReLU (fused epilogue), classifier. All outputs are allocated up front so
     that the four launches can be recorded into a HIP graph. Returns (issue, flops, bytes)."""
     rng = np.random.default_rng(5001)

@@ -318,8 +318,8 @@ int am_hip_ew_ternary_i64(int op, int rank, const int64_t* shape, int64_t* dst, 
 
 /* ---------------------------------------------------------------- measurement aid
  * No counterpart in the reference. Register-only micro-benchmarks of the issue ceilings the GEMM
- * kernels are compared with (used by bench.py; the survey's measurement plan asks for a measured
- * VALU integer multiply-add peak because 32/64-bit integers have no matrix instruction).
+ * kernels are compared with (used by bench.py: 32/64-bit integers have no matrix instruction and no
+ * published VALU multiply-add peak, so the integer GEMM is priced against a measured one).
  *   kind 0: MFMA f32 32x32x2 (FLOP/s)      kind 1: MFMA f64 16x16x4 (FLOP/s)
  *   kind 2: VALU int32 wrapping multiply-add, 8x8 register tile (integer op/s, 2 per MAC)
  *   kind 3: VALU int64 multiply-add

@@ -5,7 +5,7 @@
 ## arbitrary strides everywhere. All device work goes through hip_abi.nim; there is no inline
 ## device code and no C++ backend requirement (`nim c` is enough).
 ##
-## Hook-up inside Arraymancer (see INTEGRATION.md):
+## Hook-up inside Arraymancer:
 ##   tensor.nim:77-79      add  `when defined(hip): import ./tensor/tensor_hip; export tensor_hip`
 ##
 ## NOT COMPILED in the environment this repository is built in (no Nim toolchain there). The

@@ -250,7 +250,7 @@ def test_errors(hip):
     assert (empty + empty).shape == (0, 5)
 
 
-# ------------------------------------------------------------------ BASELINE config 4, full size
+# ------------------------------------------------------------------ the 8192 x 8192 broadcast configuration, full size
 def test_config4_8192_bit_exact(hip):
     X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
     b = np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32)

@@ -1,5 +1,5 @@
 """GEMM parity on the GPU: the HIP kernels (through the C ABI) against the CPU oracle, the
-reference's known-answer vectors, and size-independent properties at the full BASELINE sizes.
+reference's known-answer vectors, and size-independent properties at the full benchmark sizes.
 
 Bars: integers bit-exact; float32 <= 1e-4, float64 <= 1e-12 relative Frobenius error."""
 import numpy as np
@@ -240,7 +240,7 @@ def test_fused_epilogue(hip, oracle, sfx):
     assert_parity(oracle, sfx, o.toCpu(), oracle.matmul(x, W.T) + bcol, "col bias")
 
 
-# ------------------------------------------------------------------ BASELINE configs
+# ------------------------------------------------------------------ the benchmark configurations
 def test_config1_f32_1024(hip, oracle):
     rng_a, rng_b = np.random.default_rng(1001), np.random.default_rng(1002)
     A = rng_a.uniform(-1, 1, (1024, 1024)).astype(np.float32)
