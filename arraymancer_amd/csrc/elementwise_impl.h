@@ -220,6 +220,65 @@ __global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T> p) {
   }
 }
 
+// ---- 2-D tiled kernel: operands whose unit stride runs along the OTHER axis than dst's ------------
+// (a + b.transpose, clone of a transposed view, in-place update of a transposed tensor ...).
+// After normalisation dst has unit stride along axis 1. An operand with unit stride along axis 0 is
+// read in ITS contiguous direction (coalesced) into a padded 64 x 64 LDS tile and consumed
+// transposed; operands laid out like dst (or broadcast) are read directly. Every global access of
+// a wavefront is therefore a contiguous run, which ew_generic cannot offer for these layouts.
+constexpr int kTile2d = 64;
+
+template <typename T> struct TiledArgs {
+  T* dst; const T* a; const T* b;
+  T scalar;
+  int64_t R, C;                 // extents of axis 0 and axis 1
+  int64_t d0;                   // dst stride along axis 0 (axis 1 is unit)
+  int64_t a0, a1, b0, b1;       // operand strides
+  int a_t, b_t;                 // operand has unit stride along axis 0: go through LDS
+  int tiles_c;
+};
+
+template <typename T, int CODE, bool BCONST, bool SWAP>
+__global__ __launch_bounds__(256) void ew_tiled(TiledArgs<T> p) {
+  typedef typename OpSel<T, CODE>::type Op;
+  __shared__ T ta[kTile2d][kTile2d + 1];
+  __shared__ T tb[BCONST ? 1 : kTile2d][kTile2d + 1];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int tile_r = blockIdx.x / p.tiles_c, tile_c = blockIdx.x - tile_r * p.tiles_c;
+  const int64_t r0 = (int64_t)tile_r * kTile2d, c0 = (int64_t)tile_c * kTile2d;
+  if (p.a_t) {
+#pragma unroll 4
+    for (int i = 0; i < kTile2d / 4; ++i) {
+      const int cl = ty + 4 * i;                       // local column; lanes run along axis 0
+      const int64_t r = r0 + tx, c = c0 + cl;
+      if (r < p.R && c < p.C) ta[cl][tx] = p.a[r * p.a0 + c * p.a1];
+    }
+  }
+  if constexpr (!BCONST) {
+    if (p.b_t) {
+#pragma unroll 4
+      for (int i = 0; i < kTile2d / 4; ++i) {
+        const int cl = ty + 4 * i;
+        const int64_t r = r0 + tx, c = c0 + cl;
+        if (r < p.R && c < p.C) tb[cl][tx] = p.b[r * p.b0 + c * p.b1];
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (int i = 0; i < kTile2d / 4; ++i) {
+    const int rl = ty + 4 * i;
+    const int64_t r = r0 + rl, c = c0 + tx;
+    if (r < p.R && c < p.C) {
+      const T x = p.a_t ? ta[tx][rl] : p.a[r * p.a0 + c * p.a1];
+      T y;
+      if constexpr (BCONST) y = p.scalar;
+      else y = p.b_t ? tb[tx][rl] : p.b[r * p.b0 + c * p.b1];
+      p.dst[r * p.d0 + c] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+    }
+  }
+}
+
 // ---- ternary bodies and kernels (map3_inline / apply3_inline) -----------------------------------
 template <typename T, int OP> struct TriOp {
   typedef typename Traits<T>::U U;
@@ -394,7 +453,31 @@ static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const 
   // Short rows would leave most lanes of a tile idle: those shapes go to the generic kernel.
   if (ok && rows > 1 && L < tile / 4) ok = false;
   if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31) || rows >= ((int64_t)1 << 31))) ok = false;
-  if (!ok) return launch_generic<T, CODE, BCONST, SWAP>(c, dst, a, b, scalar);
+  if (!ok) {
+    // Two collapsed dims with unit strides on different axes: the LDS-tiled kernel.
+    if (c.rank == 2 && c.shape[0] < ((int64_t)1 << 31) && c.shape[1] < ((int64_t)1 << 31)) {
+      int ax = -1;                      // axis along which dst has unit stride
+      if (c.sd[1] == 1) ax = 1; else if (c.sd[0] == 1) ax = 0;
+      if (ax >= 0) {
+        const int o = 1 - ax;
+        TiledArgs<T> t;
+        t.dst = dst; t.a = a; t.b = b; t.scalar = scalar;
+        t.R = c.shape[o]; t.C = c.shape[ax]; t.d0 = c.sd[o];
+        t.a0 = c.sa[o]; t.a1 = c.sa[ax]; t.b0 = BCONST ? 0 : c.sb[o]; t.b1 = BCONST ? 0 : c.sb[ax];
+        auto direct = [](int64_t s1) { return s1 == 0 || s1 == 1; };
+        t.a_t = (!direct(t.a1) && t.a0 == 1) ? 1 : 0;
+        t.b_t = (!BCONST && !direct(t.b1) && t.b0 == 1) ? 1 : 0;
+        const bool a_ok = direct(t.a1) || t.a_t, b_ok = BCONST || direct(t.b1) || t.b_t;
+        const int64_t tr = (t.R + kTile2d - 1) / kTile2d, tc = (t.C + kTile2d - 1) / kTile2d;
+        if (a_ok && b_ok && (t.a_t || t.b_t || ax == 0) && tr * tc < ((int64_t)1 << 31) && t.R >= 16 && t.C >= 16) {
+          t.tiles_c = (int)tc;
+          hipLaunchKernelGGL((ew_tiled<T, CODE, BCONST, SWAP>), dim3((unsigned)(tr * tc)), dim3(256), 0, stream(), t);
+          return check_launch("ew_tiled");
+        }
+      }
+    }
+    return launch_generic<T, CODE, BCONST, SWAP>(c, dst, a, b, scalar);
+  }
 
   RowsArgs<T> r;
   r.dst = dst; r.a = a; r.b = b; r.scalar = scalar; r.L = L;

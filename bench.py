@@ -67,6 +67,17 @@ class Timer:
         return wall, ms.value / 1e3     # seconds: wall clock for all steps, event time for all steps
 
 
+def measured_ceilings(L):
+    """Issue ceilings of this chip from register-only micro-benchmarks (no memory traffic): what a
+    perfect kernel could reach at the clocks the device sustains. T(FL)OP/s."""
+    out = {}
+    for kind, name, iters in [(0, "mfma_f32", 20000), (1, "mfma_f64", 20000), (2, "valu_int32_mac", 20000), (3, "valu_int64_mac", 5000)]:
+        v = ctypes.c_double()
+        if L.am_hip_diag_peak(kind, iters, 2, ctypes.byref(v)) == 0:
+            out[name] = round(v.value / 1e12, 2)
+    return out
+
+
 def load_traffic(key):
     try:
         with open(TRAFFIC_FILE) as f:
@@ -105,7 +116,7 @@ def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
                        f"oracle/laser_gemm.c (laser blocking, 6x16 AVX2+FMA register tile, OpenMP)")
 
 
-def other_workloads(am, timer, steps, warmup):
+def other_workloads(am, timer, steps, warmup, ceilings):
     out = []
     # --- int32 GEMM 4096^3, entries in [-100, 100], wraparound accumulate (VALU bound)
     n = 4096
@@ -114,8 +125,13 @@ def other_workloads(am, timer, steps, warmup):
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
     k = max(3, steps // 4)
     wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+    tops = 2.0 * n ** 3 / (ev / k) / 1e12
+    peak = ceilings.get("valu_int32_mac")
     out.append(dict(workload="i32 GEMM 4096^3 (wraparound, VALU)", unit="Top/s", dtype="i32",
-                    value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4)))
+                    value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                    roofline=dict(bound="valu (measured int32 multiply-add ceiling; no matrix instruction for int32)",
+                                  achieved=round(tops, 3), peak=peak, unit="Top/s",
+                                  frac=round(tops / peak, 4) if peak else None)))
     del dA, dB, dC
     # --- float64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C), M=2048 N=3072 K=1024
     pa = np.random.default_rng(3001).standard_normal((1024, 2048))
@@ -266,7 +282,9 @@ def main():
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_gemm_f32(*r["host"])
     if not args.no_others:
-        line["others"] = other_workloads(am, timer, args.steps, args.warmup)
+        ceilings = measured_ceilings(L)
+        line["measured_ceilings"] = dict(ceilings, unit="T(FL)OP/s", how="am_hip_diag_peak: register-only MFMA / VALU chains")
+        line["others"] = other_workloads(am, timer, args.steps, args.warmup, ceilings)
     print(json.dumps(line))
 
 

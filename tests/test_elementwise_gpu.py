@@ -308,3 +308,34 @@ def test_map3_muladd_bit_exact(hip, oracle, sfx):
     else:
         x, y, z = (hip.toHip(t) for t in (a, b, c))
         assert np.array_equal(hip.map3("gru_blend", x, y, z).toCpu(), oracle.map3("gru_blend", a, b, c))
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("shape", [(16, 16), (130, 67), (257, 1031), (1024, 512)])
+def test_mixed_unit_stride_axes(hip, oracle, sfx, shape):
+    """Operands whose unit stride is on different axes (the LDS-tiled 2-D kernel): transposed inputs,
+    transposed destinations, a broadcast vector beside a transposed matrix, scalar and unary forms."""
+    dt = DTYPES[sfx]
+    R, C = shape
+    rng = np.random.default_rng(seed_of(sfx, "tiled", shape))
+    A, Bt, v = fill(rng, (R, C), dt), fill(rng, (C, R), dt), fill(rng, (1, C), dt)
+    dA, dBt, dv = hip.toHip(A), hip.toHip(Bt), hip.toHip(v)
+    say("tiled a + b^T", sfx, shape)
+    assert np.array_equal(hip.map2("add", dA, dBt.transpose()).toCpu(), A + Bt.T)
+    assert np.array_equal(hip.map2("sub", dBt.transpose(), dA).toCpu(), Bt.T - A)
+    say("tiled both transposed", sfx, shape)
+    assert np.array_equal(hip.map2("mul", dBt.transpose(), dBt.transpose()).toCpu(), oracle.map2("mul", Bt.T, Bt.T))
+    say("tiled clone / unary / scalar of a transposed view", sfx, shape)
+    assert np.array_equal(dBt.transpose().clone().toCpu(), Bt.T)
+    assert np.array_equal(hip.unary("neg", dBt.transpose()).toCpu(), oracle.unary("neg", Bt.T))
+    assert np.array_equal(hip.scalar_op("sub", dBt.transpose(), 3, scalar_on_left=True).toCpu(),
+                          oracle.scalar_op("sub", Bt.T, 3, scalar_on_left=True))
+    say("tiled broadcast row vector + transposed", sfx, shape)
+    assert np.array_equal(hip.bc_add(dBt.transpose(), dv).toCpu(), Bt.T + v)
+    say("tiled in place on a transposed destination", sfx, shape)
+    dD = hip.toHip(Bt)
+    dDt = dD.transpose()
+    dDt += dA
+    assert np.array_equal(dD.toCpu(), (Bt.T + A).T)
+    dDt.bc_imul(dv)
+    assert np.array_equal(dD.toCpu(), ((Bt.T + A) * v).T)
