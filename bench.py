@@ -205,6 +205,93 @@ def bench_chain(am, timer, steps, warmup):
                 note="launch/latency bound: 2.9e8 FLOP and 17.8 MB per chain; eager figure includes host launch cost")
 
 
+def config_report(am, timer, L):
+    """One JSON line per configuration of the path: GPU time / rate / fraction of its bound, the CPU
+    port (oracle, all host cores) timed beside it on the same inputs, and the parity result of the
+    GPU output against the CPU output at full size. Not the default mode (the default prints one
+    line); run as `python bench.py --report`."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import am_oracle
+    from arraymancer_amd import tensor_hip as th
+    ceil = measured_ceilings(L)
+    threads = am_oracle.num_threads()
+
+    def cpu_time(fn, budget=4.0, max_runs=5):
+        fn()
+        ts = []
+        end = time.perf_counter() + budget
+        while not ts or (time.perf_counter() < end and len(ts) < max_runs):
+            t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
+        return min(ts)
+
+    def emit(**kw):
+        print(json.dumps(kw), flush=True)
+
+    def gemm_case(config, sfx, M, N, K, A, B, dA, dB, alpha=1, beta=0, C0=None, peak=None, peak_used="", unit="TFLOP/s", steps=20):
+        dt = A.dtype
+        C_host = C0.copy() if C0 is not None else np.zeros((M, N), dt)
+        dC = am.toHip(C_host)
+        am.gemm(alpha, dA, dB, beta, dC)
+        got = dC.toCpu().copy()
+        want = am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy())
+        if beta == 0:
+            _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3)
+        else:   # accumulating into C: keep the values bounded by restoring nothing, only time it
+            _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3)
+        gpu_s = ev / steps
+        cpu_s = cpu_time(lambda: am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy() if beta != 0 else C_host))
+        ops = 2.0 * M * N * K
+        row = dict(config=config, dtype=sfx, shape=[M, N, K], gpu_ms=round(gpu_s * 1e3, 4),
+                   gpu_rate=round(ops / gpu_s / 1e12, 3), rate_unit=unit,
+                   pct_peak=round(100 * ops / gpu_s / 1e12 / peak, 1) if peak else None, peak_used=peak_used,
+                   cpu_impl="oracle/laser_gemm.c (port of laser gemm_strided, OpenMP)", cpu_threads=threads,
+                   cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1))
+        if dt.kind == "f":
+            row["rel_frobenius_vs_cpu"] = am_oracle.rel_frobenius(got, want)
+        else:
+            row["bit_exact"] = bool(np.array_equal(got, want))
+        emit(**row)
+
+    rng = np.random.default_rng
+    for n in (1024, 4096):
+        A = rng(1001).uniform(-1, 1, (n, n)).astype(np.float32); B = rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
+        gemm_case(f"f32 GEMM {n}^3", "f32", n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_F32_PEAK_TFLOPS,
+                  peak_used="MFMA fp32 157.3 TFLOP/s", steps=50 if n == 1024 else 20)
+    for sfx, dt, key in (("i32", np.int32, "valu_int32_mac"), ("i64", np.int64, "valu_int64_mac")):
+        for n in (1500, 4096):
+            A = rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(dt)
+            B = rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(dt)
+            gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100]", sfx, n, n, n, A, B, am.toHip(A), am.toHip(B),
+                      peak=ceil.get(key), peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s",
+                      unit="Top/s", steps=10)
+    pa = rng(3001).standard_normal((1024, 2048)); pb = rng(3002).standard_normal((1024, 6144))
+    C0 = rng(3003).standard_normal((2048, 3072))
+    gemm_case("f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C)", "f64", 2048, 3072, 1024, pa.T, pb[:, ::2],
+              am.toHip(pa).transpose(), am.toHip(pb)[:, ::2], alpha=1.5, beta=0.5, C0=C0, peak=MFMA_F64_PEAK_TFLOPS,
+              peak_used="MFMA fp64 78.6 TFLOP/s", steps=1)
+    # broadcast ops
+    X = rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
+    b = rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32); sc = rng(4003).uniform(-1, 1, (8192, 1)).astype(np.float32)
+    dX, db, ds, dY = am.toHip(X), am.toHip(b), am.toHip(sc), am.empty((8192, 8192), np.float32)
+    nbytes = 2 * 8192 * 8192 * 4 + 8192 * 4
+    for name, op, dv, hv in (("X +. b[1,8192]", "add", db, b), ("X *. s[8192,1]", "mul", ds, sc), ("map2(X, b, max(0, x+y))", "add_relu", db, b)):
+        bv = dv.broadcast((8192, 8192))
+        _, ev = timer.run(lambda: th._binary_into(op, dY, dX, bv), 50, 5)
+        got = dY.toCpu().copy()
+        hb = am_oracle.broadcast(hv, X.shape)
+        out = np.empty_like(X)
+        cpu_s = cpu_time(lambda: am_oracle.map2(op, X, hb, out=out))
+        gpu_s = ev / 50
+        emit(config=f"f32 8192x8192 {name}", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
+             gpu_rate=round(nbytes / gpu_s / 1e9, 1), rate_unit="GB/s", pct_peak=round(100 * nbytes / gpu_s / 1e9 / HBM_PEAK_GBS, 1),
+             peak_used="HBM 8000 GB/s", cpu_impl="oracle/strided_map.c (port of map2_inline + strided iteration, OpenMP blocks)",
+             cpu_threads=threads, cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1),
+             bit_exact=bool(np.array_equal(got, out)))
+    r = bench_chain(am, timer, 200, 20)
+    emit(config="f32 inference chain (4 GEMMs, fused bias+ReLU)", dtype="f32", hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"],
+         note=r["note"])
+
+
 def run_only(am, timer, which, steps, warmup):
     """One workload, nothing else on the stream: what the rocprofv3 summaries under profiles/ time."""
     from arraymancer_amd import tensor_hip as th
@@ -246,6 +333,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--report", action="store_true",
+                    help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
     ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy", "chain"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
@@ -262,6 +351,9 @@ def main():
 
     if args.only:
         print(json.dumps(run_only(am, timer, args.only, args.steps, args.warmup)))
+        return
+    if args.report:
+        config_report(am, timer, L)
         return
 
     r = bench_gemm_f32(am, timer, args.steps, args.warmup)
