@@ -1,6 +1,7 @@
 // Host-side pieces shared by the MFMA (f32/f64) and VALU (i32/i64) GEMM families: the kernel
 // argument block, argument validation, operand classification and the tile-shape choice.
 #pragma once
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 #include "common.h"
@@ -95,6 +96,12 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   return AM_OK;
 }
 
+// AM_HIP_GEMM_TRACE=1 in the environment: every GEMM call prints the tile / split it chose to stderr.
+static inline bool trace_choices() {
+  static const bool on = [] { const char* e = getenv("AM_HIP_GEMM_TRACE"); return e && *e && *e != '0'; }();
+  return on;
+}
+
 // One candidate tile shape and the relative speed of a CU that runs it.
 struct TileChoice { int bm, bn; double eff; };
 
@@ -148,37 +155,131 @@ static inline void plan_splitk(Args<T>& g, int bk, int waves_per_tile) {
   g.splits = (int)splits; g.k_chunk = chunk_slabs * bk; g.ws = ws;
 }
 
+// Cuts K into `want` ranges (fewer if K has too few slabs or the workspace is too small / cannot
+// be allocated now). want <= 1 leaves the problem whole.
+template <typename T>
+static inline void apply_splitk(Args<T>& g, int bk, int64_t want) {
+  g.splits = 1; g.k_chunk = g.K; g.ws = nullptr;
+  if (want <= 1 || g.batch > 1) return;
+  const int64_t slabs = (g.K + bk - 1) / bk;
+  if (want > slabs) want = slabs;
+  const int64_t chunk_slabs = (slabs + want - 1) / want;
+  const int64_t splits = (slabs + chunk_slabs - 1) / chunk_slabs;   // no empty split
+  if (splits < 2) return;
+  const size_t bytes = (size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(T);
+  T* ws = (T*)splitk_workspace(bytes);
+  if (!ws) return;
+  g.splits = (int)splits; g.k_chunk = chunk_slabs * bk; g.ws = ws;
+}
+
+// Joint choice of workgroup tile and split-K factor for the exact (ring arithmetic) integer
+// products, where cutting K changes no bit of the result. Estimated time of a candidate =
+// rounds of two workgroups per CU x time of one workgroup, plus the second pass that adds the
+// partial sums (its launch and its HBM traffic). mac_per_us: multiply-adds one CU sustains.
+struct TileSplit { int tile; int splits; };
+template <typename T>
+static inline TileSplit choose_tile_split(const TileChoice* cand, int ncand, int64_t M, int64_t N, int64_t K, int bk,
+                                          double mac_per_us, const char* env, int64_t batch) {
+  TileSplit best = {0, 1};
+  int forced_tile = -1;
+  const char* forced = getenv(env);
+  if (forced && *forced) { const int idx = atoi(forced); if (idx >= 0 && idx < ncand) forced_tile = idx; }
+  int forced_splits = 0;
+  const char* fs = getenv("AM_HIP_GEMM_SPLITK");
+  if (fs && *fs) forced_splits = atoi(fs);
+  const int64_t cus = num_cus();
+  const int64_t slabs = (K + bk - 1) / bk;
+  double best_cost = -1;
+  for (int i = 0; i < ncand; ++i) {
+    if (cand[i].eff <= 0 || (forced_tile >= 0 && i != forced_tile)) continue;
+    const int64_t tiles = ((M + cand[i].bm - 1) / cand[i].bm) * ((N + cand[i].bn - 1) / cand[i].bn) * batch;
+    const double slab_us = (double)cand[i].bm * cand[i].bn * bk / (mac_per_us * cand[i].eff);
+    for (int64_t want = 1; want <= 16; ++want) {
+      if (forced_splits > 0 && want != forced_splits) continue;
+      if (want > 1 && (batch > 1 || want > slabs / 2)) break;
+      const int64_t chunk = (slabs + want - 1) / want;
+      const int64_t sp = (slabs + chunk - 1) / chunk;
+      if (sp != want) continue;
+      if (sp > 1 && (double)sp * M * N * sizeof(T) > 64.0 * 1024 * 1024) break;
+      // Two workgroups fit on a CU and share it at full speed; a workgroup alone on its CU runs
+      // at about two thirds of the CU's rate (one wavefront per SIMD: latencies are exposed).
+      const int64_t wgs = tiles * sp, slots = 2 * cus;
+      const int64_t full = wgs / slots, rem = wgs - full * slots;
+      const double wg_us = (double)chunk * slab_us;
+      double cost = (double)full * 2.0 * wg_us + (rem == 0 ? 0.0 : rem <= cus ? wg_us / 0.66 : 2.0 * wg_us);
+      if (sp > 1) cost += 3.0 + (2.0 * sp + 1.0) * (double)M * N * sizeof(T) / 4.0e6;   // second pass at ~4 TB/s
+      if (best_cost < 0 || cost < best_cost) { best_cost = cost; best.tile = i; best.splits = (int)sp; }
+    }
+  }
+  if (trace_choices()) fprintf(stderr, "am_hip gemm: M=%lld N=%lld K=%lld tile %d (%dx%d) splits %d est %.1f us\n", (long long)M, (long long)N, (long long)K, best.tile, cand[best.tile].bm, cand[best.tile].bn, best.splits, best_cost);
+  return best;
+}
+
 // Second pass of split-K: C <- epilogue(alpha * sum_s ws[s] + beta * C), partials added in
-// ascending s (deterministic). ACC is the type the partials were stored in.
-template <typename T, typename ACC>
+// ascending s (deterministic). ACC is the type the partials were stored in. One thread per group
+// of VEC consecutive columns of one row (blockIdx.y walks the rows): VEC = 16 bytes / element when
+// N is a multiple of it (the partials are then read as 16-byte vectors), else 1.
+template <typename T, typename ACC, int VEC>
 __global__ __launch_bounds__(256) void splitk_reduce(Args<T> p) {
+  typedef ACC vec_t __attribute__((ext_vector_type(VEC)));
   const int64_t total = p.M * p.N;
   const ACC* ws = (const ACC*)p.ws;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-    const int64_t row = idx / p.N, col = idx - row * p.N;
-    ACC sum = ws[idx];
-    for (int sidx = 1; sidx < p.splits; ++sidx) sum += ws[(int64_t)sidx * total + idx];
-    T* cp = p.C + row * p.c_m + col * p.c_n;
-    ACC ab = sum;
-    if (p.alpha != (T)1) ab = (ACC)p.alpha * ab;
-    ACC v = ab;
-    if (p.beta != (T)0) {
-      ACC c = (ACC)*cp;
-      if (p.beta != (T)1) c = c * (ACC)p.beta;
-      v = c + ab;
+  const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (col >= p.N) return;
+  for (int64_t row = blockIdx.y; row < p.M; row += gridDim.y) {
+    const int64_t idx = row * p.N + col;
+    ACC sum[VEC];
+    {
+      const vec_t v = *(const vec_t*)(ws + idx);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum[e] = v[e];
     }
-    if (p.epilogue & AM_EPI_BIAS) v = v + (ACC)p.bias[row * p.bias_m + col * p.bias_n];
-    if (p.epilogue & AM_EPI_RELU) v = ((ACC)0 >= v) ? (ACC)0 : v;
-    *cp = (T)v;
+    for (int sidx = 1; sidx < p.splits; ++sidx) {
+      const vec_t v = *(const vec_t*)(ws + (int64_t)sidx * total + idx);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum[e] += v[e];
+    }
+    T* cp = p.C + row * p.c_m + col * p.c_n;
+    ACC cold[VEC], bias[VEC];
+    if (p.beta != (T)0) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) cold[e] = (ACC)cp[e * p.c_n];
+    }
+    if (p.epilogue & AM_EPI_BIAS) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) bias[e] = (ACC)p.bias[row * p.bias_m + (col + e) * p.bias_n];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      ACC ab = sum[e];
+      if (p.alpha != (T)1) ab = (ACC)p.alpha * ab;
+      ACC v = ab;
+      if (p.beta != (T)0) {
+        ACC c = cold[e];
+        if (p.beta != (T)1) c = c * (ACC)p.beta;
+        v = c + ab;
+      }
+      if (p.epilogue & AM_EPI_BIAS) v = v + bias[e];
+      if (p.epilogue & AM_EPI_RELU) v = ((ACC)0 >= v) ? (ACC)0 : v;
+      cp[e * p.c_n] = (T)v;
+    }
   }
 }
 
 template <typename T, typename ACC>
 static int launch_splitk_reduce(const Args<T>& g) {
-  int64_t blocks = (g.M * g.N + 255) / 256;
-  const int64_t cap = (int64_t)num_cus() * 8;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL((splitk_reduce<T, ACC>), dim3((unsigned)blocks), dim3(256), 0, stream(), g);
+  constexpr int VEC = 16 / (int)sizeof(ACC);
+  const bool vec = (g.N % VEC == 0);   // the workspace itself is 256-byte aligned and row pitch N
+  const int64_t cols = vec ? g.N / VEC : g.N;
+  const int64_t bx = (cols + 255) / 256;
+  int64_t by = g.M;
+  const int64_t cap = (int64_t)num_cus() * 16;
+  if (bx * by > cap) by = (cap + bx - 1) / bx;
+  if (by > 65535) by = 65535;
+  if (by < 1) by = 1;
+  const dim3 grid((unsigned)bx, (unsigned)by), block(256);
+  if (vec) hipLaunchKernelGGL((splitk_reduce<T, ACC, VEC>), grid, block, 0, stream(), g);
+  else hipLaunchKernelGGL((splitk_reduce<T, ACC, 1>), grid, block, 0, stream(), g);
   return check_launch("splitk_reduce");
 }
 

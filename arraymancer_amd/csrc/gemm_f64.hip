@@ -10,14 +10,16 @@ static int run_f64(Args<double>& g) {
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
   if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;   // every batch member must stay 16-byte aligned
   if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
-  // Candidate workgroup tiles, largest first, with the relative MFMA efficiency of each.
-  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.98}, {32, 32, 0.8}, {256, 128, 0.96}, {128, 64, 0.97}};
+  // Candidate workgroup tiles with the relative MFMA efficiency of each. The 128 x 128 tile runs
+  // with 8 wavefronts (64 x 32 each) and the 256 x 128 one without fragment prefetch: a 64 x 64
+  // wavefront tile of doubles (128 accumulator registers) leaves no room for a second fragment set.
+  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.93}, {32, 32, 0.7}, {256, 128, 1.0}, {128, 64, 0.98}};
   switch (choose_tile(cand, 5, g.M, g.N, "AM_HIP_GEMM_TILE_F64", g.batch)) {
-    case 0: return launch_kinds<double, 128, 128, 16, 2, 2>(g, ak, bk);
-    case 1: return launch_kinds<double, 64, 64, 16, 2, 2>(g, ak, bk);
-    case 2: return launch_kinds<double, 32, 32, 16, 2, 2>(g, ak, bk);
-    case 3: return launch_kinds<double, 256, 128, 16, 4, 2>(g, ak, bk);
-    default: return launch_kinds<double, 128, 64, 16, 2, 2>(g, ak, bk);
+    case 0: return launch_kinds<double, 128, 128, 16, 2, 4>(g, ak, bk);
+    case 1: return launch_kinds<double, 64, 64, 16, 2, 2, 2>(g, ak, bk);
+    case 2: return launch_kinds<double, 32, 32, 16, 2, 2, 2>(g, ak, bk);
+    case 3: return launch_kinds<double, 256, 128, 16, 4, 2, 1, false>(g, ak, bk);
+    default: return launch_kinds<double, 128, 64, 16, 2, 2, 2>(g, ak, bk);
   }
 }
 

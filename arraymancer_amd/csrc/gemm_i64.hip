@@ -10,10 +10,13 @@ static int run_i64(Args<int64_t>& g) {
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
   if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;
   if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
-  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 1.0}};
-  switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_GEMM_TILE_I64", g.batch)) {
-    case 0: return launch_valu<int64_t, 8, 8, 16>(g, ak, bk);
-    default: return launch_valu<int64_t, 4, 4, 16>(g, ak, bk);
+  // 8 x 8 and 4 x 4 results per lane; the small tile re-reads LDS twice as often per multiply-add.
+  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.85}};
+  // 34.0e3 multiply-adds per microsecond and CU: the measured VALU ceiling of this element type.
+  const TileSplit ts = choose_tile_split<int64_t>(cand, 2, g.M, g.N, g.K, 16, 34.0e3, "AM_HIP_GEMM_TILE_I64", g.batch);
+  switch (ts.tile) {
+    case 0: return launch_valu<int64_t, 8, 8, 16>(g, ak, bk, ts.splits);
+    default: return launch_valu<int64_t, 4, 4, 16>(g, ak, bk, ts.splits);
   }
 }
 

@@ -70,8 +70,8 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
   const int64_t ktiles = (k_end - k_begin + BK - 1) / BK;
   la.fetch(k_begin);
   lb.fetch(k_begin);
-  la.commit(sA[0]);
-  lb.commit(sB[0]);
+  la.commit(sA[0], k_begin);
+  lb.commit(sB[0], k_begin);
   __syncthreads();
 
   for (int64_t kt = 0; kt < ktiles; ++kt) {
@@ -104,8 +104,8 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
         for (int j = 0; j < TN; ++j) acc[i][j] += (ACC)a[i] * (ACC)b[j];
     }
     if (more) {
-      la.commit(sA[cur ^ 1]);
-      lb.commit(sB[cur ^ 1]);
+      la.commit(sA[cur ^ 1], k_begin + (kt + 1) * BK);
+      lb.commit(sB[cur ^ 1], k_begin + (kt + 1) * BK);
     }
     __syncthreads();
   }
@@ -130,31 +130,36 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
   for (int i = 0; i < TM; ++i) {
     const int64_t row = m0 + (i / VK) * 16 * VK + ty * VK + (i % VK);
     if (row >= p.M) continue;
+    // all loads of this row of C first, then the arithmetic and the stores: a load issued after a
+    // store would wait for that store (one memory counter orders both)
+    U cv[TN];
+    if (beta != 0) {
 #pragma unroll
-    for (int cj = 0; cj < CN; ++cj) {
-      const int64_t col0 = n0 + cj * 16 * VK + tx * VK;
+      for (int j = 0; j < TN; ++j) {
+        const int64_t col = n0 + (j / VK) * 16 * VK + tx * VK + (j % VK);
+        cv[j] = (col < p.N) ? (U)p.C[row * p.c_m + col * p.c_n] : (U)0;
+      }
+    }
 #pragma unroll
-      for (int e = 0; e < VK; ++e) {
-        const int64_t col = col0 + e;
-        if (col < p.N) {
-          T* cp = p.C + row * p.c_m + col * p.c_n;
-          U v = alpha * (U)acc[i][cj * VK + e];
-          if (beta != 0) v += beta * (U)(*cp);
-          *cp = (T)v;
-        }
+    for (int j = 0; j < TN; ++j) {
+      const int64_t col = n0 + (j / VK) * 16 * VK + tx * VK + (j % VK);
+      if (col < p.N) {
+        U v = alpha * (U)acc[i][j];
+        if (beta != 0) v += beta * cv[j];
+        p.C[row * p.c_m + col * p.c_n] = (T)v;
       }
     }
   }
 }
 
 template <typename T, int TM, int TN, int BK>
-static int launch_valu(Args<T>& g, int ak, int bk) {
+static int launch_valu(Args<T>& g, int ak, int bk, int want_splits) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
   g.tiles_m = (int)((g.M + BM - 1) / BM);
   g.tiles_n = (int)((g.N + BN - 1) / BN);
   const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
   if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
-  plan_splitk(g, BK, 4);
+  apply_splitk(g, BK, want_splits);
   const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(256);
 #define AM_LAUNCH(AKIND, BKIND_) \
   hipLaunchKernelGGL((gemm_valu<T, TM, TN, BK, AKIND, BKIND_>), grid, block, 0, stream(), g)

@@ -31,120 +31,165 @@ template <typename T, int KIND, int BMN, int BK, bool KG = true> struct Slab {
   static constexpr int ELEMS = (KIND == kKContig && KG) ? (BK / VK) * LDKG * VK : BK * LDMN;
 };
 
-// Moves one operand slab global -> registers (fetch) -> LDS (commit).
-template <typename T, int KIND, int BMN, int BK, int NT, bool KG = true> struct Loader;
+// Moves one operand slab global -> registers (fetch) -> LDS (commit). PF register stages let PF
+// slabs be in flight at once: fetch<S> fills stage S, commit<S> writes stage S to LDS.
+//
+// fetch is branch-free and unconditional: every lane always loads, from an address clamped into
+// the operand. (Loads under a branch would keep the compiler from counting the loads in flight,
+// and every wait would then be a wait for all of them, including those just issued for a later
+// slab.) What the clamping brings in is dealt with as follows:
+//   * rows / columns past the edge of the operand (edge tiles) repeat the last valid one; they
+//     only ever reach rows / columns of C past its edge, which the store masks;
+//   * k values past the end of the k range can only occur in a range's last slab; commit zeroes
+//     them in both operands, so that 0 * Inf never arises. A slab wholly past the end is not
+//     fetched at all (wave-uniform test) and commits as zeros. MASK = false versions of fetch and
+//     commit skip the k clamping and zeroing: for slabs known to lie wholly inside the k range.
+template <typename T, int KIND, int BMN, int BK, int NT, bool KG = true, int PF = 1> struct Loader;
 
-template <typename T, int BMN, int BK, int NT, bool KG> struct Loader<T, kKContig, BMN, BK, NT, KG> {
+template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kKContig, BMN, BK, NT, KG, PF> {
   typedef typename VecTraits<T>::vec_t vec_t;
   static constexpr int VK = VecTraits<T>::VK;
   static constexpr int QN = BK / VK;               // vectors per row
   static constexpr int NV = BMN * QN / NT;         // vectors per thread
   static_assert(BMN * QN % NT == 0 && NV >= 1, "slab must divide evenly over the workgroup");
   const T* ptr[NV];
-  bool rowok[NV];
   int64_t K;
-  vec_t reg[NV];
+  vec_t reg[PF][NV];
   __device__ __forceinline__ Loader(const T* X, int64_t ld_mn, int64_t, int64_t mn0, int64_t MN, int64_t K_, int) : K(K_) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = threadIdx.x + i * NT;
       const int q = v % QN, mn = v / QN;
-      rowok[i] = (mn0 + mn) < MN;
-      ptr[i] = X + (mn0 + mn) * ld_mn + q * VK;
+      ptr[i] = X + ((mn0 + mn) < MN ? mn0 + mn : MN - 1) * ld_mn + q * VK;
     }
   }
-  __device__ __forceinline__ void fetch(int64_t k0) {
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
+    if (MASK && k0 >= K) return;   // slab wholly past the end: commit writes zeros without these registers
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int q = (threadIdx.x + i * NT) % QN;
-      vec_t z = {};
-      reg[i] = (rowok[i] && (k0 + q * VK) < K) ? *(const vec_t*)(ptr[i] + k0) : z;
+      if constexpr (MASK) reg[S][i] = *(const vec_t*)(ptr[i] + ((k0 + q * VK) < K ? k0 : (int64_t)(-q * VK)));
+      else reg[S][i] = *(const vec_t*)(ptr[i] + k0);
     }
   }
-  __device__ __forceinline__ void commit(T* lds) const {
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
+    if (MASK && k0 >= K) {   // nothing was fetched: zeros, without waiting for any load
+#pragma unroll
+      for (int i = 0; i < NV; ++i) { vec_t z = {}; reg[S][i] = z; }
+    } else if (MASK && k0 + BK > K) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int q = (threadIdx.x + i * NT) % QN;
+        vec_t z = {};
+        if ((k0 + q * VK) >= K) reg[S][i] = z;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = threadIdx.x + i * NT;
       const int q = v % QN, mn = v / QN;
       if constexpr (KG) {
         constexpr int LD = Slab<T, kKContig, BMN, BK, true>::LDKG;
-        *(vec_t*)(lds + (q * LD + mn) * VK) = reg[i];
+        *(vec_t*)(lds + (q * LD + mn) * VK) = reg[S][i];
       } else {  // k-row layout wanted: scatter the VK k values of this row
         constexpr int LD = Slab<T, kKContig, BMN, BK, false>::LDMN;
 #pragma unroll
-        for (int s = 0; s < VK; ++s) lds[(q * VK + s) * LD + mn] = reg[i][s];
+        for (int s = 0; s < VK; ++s) lds[(q * VK + s) * LD + mn] = reg[S][i][s];
       }
     }
   }
 };
 
-template <typename T, int BMN, int BK, int NT, bool KG> struct Loader<T, kMNContig, BMN, BK, NT, KG> {
+template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kMNContig, BMN, BK, NT, KG, PF> {
   typedef typename VecTraits<T>::vec_t vec_t;
   static constexpr int VK = VecTraits<T>::VK;
   static constexpr int CN = BMN / VK;              // vectors per k row
   static constexpr int NV = CN * BK / NT;
   static_assert(CN * BK % NT == 0 && NV >= 1, "slab must divide evenly over the workgroup");
   const T* ptr[NV];
-  bool colok[NV];
   int64_t K, ld_k;
-  vec_t reg[NV];
+  vec_t reg[PF][NV];
   __device__ __forceinline__ Loader(const T* X, int64_t, int64_t ld_k_, int64_t mn0, int64_t MN, int64_t K_, int) : K(K_), ld_k(ld_k_) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = threadIdx.x + i * NT;
       const int c = v % CN, k = v / CN;
-      colok[i] = (mn0 + c * VK) < MN;
-      ptr[i] = X + (mn0 + c * VK) + k * ld_k;
+      ptr[i] = X + ((mn0 + c * VK) < MN ? mn0 + c * VK : 0) + k * ld_k;
     }
   }
-  __device__ __forceinline__ void fetch(int64_t k0) {
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
+    if (MASK && k0 >= K) return;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int k = (threadIdx.x + i * NT) / CN;
-      vec_t z = {};
-      reg[i] = (colok[i] && (k0 + k) < K) ? *(const vec_t*)(ptr[i] + k0 * ld_k) : z;
+      if constexpr (MASK) reg[S][i] = *(const vec_t*)(ptr[i] + ((k0 + k) < K ? k0 : (int64_t)(-k)) * ld_k);
+      else reg[S][i] = *(const vec_t*)(ptr[i] + k0 * ld_k);
     }
   }
-  __device__ __forceinline__ void commit(T* lds) const {
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
     constexpr int LD = Slab<T, kMNContig, BMN, BK>::LDMN;
+    if (MASK && k0 >= K) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) { vec_t z = {}; reg[S][i] = z; }
+    } else if (MASK && k0 + BK > K) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int k = (threadIdx.x + i * NT) / CN;
+        vec_t z = {};
+        if ((k0 + k) >= K) reg[S][i] = z;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = threadIdx.x + i * NT;
       const int c = v % CN, k = v / CN;
-      *(vec_t*)(lds + k * LD + c * VK) = reg[i];
+      *(vec_t*)(lds + k * LD + c * VK) = reg[S][i];
     }
   }
 };
 
-template <typename T, int BMN, int BK, int NT, bool KG> struct Loader<T, kGeneric, BMN, BK, NT, KG> {
+template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kGeneric, BMN, BK, NT, KG, PF> {
   static constexpr int NE = BMN * BK / NT;         // elements per thread
   static_assert(BMN * BK % NT == 0 && NE >= 1, "slab must divide evenly over the workgroup");
   const T* X;
   int64_t ld_mn, ld_k, mn0, MN, K;
   int kfast;
-  T reg[NE];
+  T reg[PF][NE];
   __device__ __forceinline__ Loader(const T* X_, int64_t ld_mn_, int64_t ld_k_, int64_t mn0_, int64_t MN_, int64_t K_, int kfast_)
       : X(X_), ld_mn(ld_mn_), ld_k(ld_k_), mn0(mn0_), MN(MN_), K(K_), kfast(kfast_) {}
   __device__ __forceinline__ void coords(int i, int& mn, int& k) const {
     const int e = threadIdx.x + i * NT;
     if (kfast) { k = e % BK; mn = e / BK; } else { mn = e % BMN; k = e / BMN; }
   }
-  __device__ __forceinline__ void fetch(int64_t k0) {
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
+    if (MASK && k0 >= K) return;
 #pragma unroll
     for (int i = 0; i < NE; ++i) {
       int mn, k;
       coords(i, mn, k);
-      const bool ok = (mn0 + mn) < MN && (k0 + k) < K;
-      reg[i] = ok ? X[(mn0 + mn) * ld_mn + (k0 + k) * ld_k] : (T)0;
+      const int64_t cm = (mn0 + mn) < MN ? mn0 + mn : MN - 1;
+      const int64_t ck = (!MASK || (k0 + k) < K) ? k0 + k : K - 1;
+      reg[S][i] = X[cm * ld_mn + ck * ld_k];
     }
   }
-  __device__ __forceinline__ void commit(T* lds) const {
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
     constexpr int LD = Slab<T, kGeneric, BMN, BK>::LDMN;
+    if (MASK && k0 >= K) {
+#pragma unroll
+      for (int i = 0; i < NE; ++i) reg[S][i] = (T)0;
+    } else if (MASK && k0 + BK > K) {
+#pragma unroll
+      for (int i = 0; i < NE; ++i) {
+        int mn, k;
+        coords(i, mn, k);
+        if ((k0 + k) >= K) reg[S][i] = (T)0;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NE; ++i) {
       int mn, k;
       coords(i, mn, k);
-      lds[k * LD + mn] = reg[i];
+      lds[k * LD + mn] = reg[S][i];
     }
   }
 };

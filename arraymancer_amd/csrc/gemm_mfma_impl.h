@@ -27,6 +27,7 @@
 //   * out-of-range rows/columns/k are zero-filled on load (the reference zero-pads its packed
 //     panels the same way, gemm_packing.nim:54-55, 98-99) and masked on store.
 #pragma once
+#include <type_traits>
 #include "gemm_loader.h"
 
 namespace am {
@@ -79,8 +80,15 @@ __device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, 
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int AK, int BKIND>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p) {
+// Second __launch_bounds__ argument: two wavefronts per SIMD whatever the workgroup size, i.e. at
+// most 256 registers per lane, all of them architectural VGPRs. Allowed more, the compiler spreads
+// a large tile's accumulators over VGPRs and AGPRs and copies them back and forth in every loop
+// trip (measured: f64 128 x 128 falls from 61 to 48 TFLOP/s).
+constexpr int mfma_min_blocks(int nt) { return nt <= 256 ? 2 : 1; }
+
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF, bool FPF, int AK, int BKIND>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 : 1))
+void gemm_mfma(Args<T> p) {
   typedef Mfma<T> MF;
   typedef typename MF::acc_t acc_t;
   constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -89,8 +97,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
   static_assert(BK % KSTEP == 0 && WM % TILE == 0 && WN % TILE == 0, "tile shape");
   constexpr int A_ELEMS = Slab<T, AK, BM, BK>::ELEMS, B_ELEMS = Slab<T, BKIND, BN, BK>::ELEMS;
 
-  __shared__ __attribute__((aligned(16))) T sA[2][A_ELEMS];
-  __shared__ __attribute__((aligned(16))) T sB[2][B_ELEMS];
+  static_assert((BK / KSTEP) % 2 == 0, "fragment double buffering needs an even number of k-steps per slab");
+  __shared__ __attribute__((aligned(16))) T sA[3][A_ELEMS];
+  __shared__ __attribute__((aligned(16))) T sB[3][B_ELEMS];
 
   int tile_m, tile_n, bid = (int)blockIdx.x, split = 0;
   if (p.splits > 1) {
@@ -113,8 +122,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int lrow = lane % TILE, kl = lane / TILE;
 
-  Loader<T, AK, BM, BK, NT> la(p.A, p.a_mn, p.a_k, m0, p.M, k_end, p.a_kfast);
-  Loader<T, BKIND, BN, BK, NT> lb(p.B, p.b_mn, p.b_k, n0, p.N, k_end, p.b_kfast);
+  Loader<T, AK, BM, BK, NT, true, PF> la(p.A, p.a_mn, p.a_k, m0, p.M, k_end, p.a_kfast);
+  Loader<T, BKIND, BN, BK, NT, true, PF> lb(p.B, p.b_mn, p.b_k, n0, p.N, k_end, p.b_kfast);
 
   acc_t acc[TM][TN];
 #pragma unroll
@@ -124,45 +133,111 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
 #pragma unroll
       for (int r = 0; r < MF::NACC; ++r) acc[i][j][r] = (T)0;
 
+  // Software pipeline over the K slabs; nothing but the barrier itself is left between the MFMA
+  // streams of consecutive slabs.
+  //   global --fetch--> register stage (PF of them) --commit--> LDS ring of 3 slabs --> fragments
+  // Iteration t multiplies slab t out of LDS buffer t % 3. During its last k-step it
+  //   * reads the first fragments of slab t + 1 (buffer (t+1) % 3, complete since the barrier that
+  //     ended iteration t - 1), so the next iteration starts with its operands in registers
+  //     (FPF = true: fragments are double-buffered in registers and always read one k-step ahead;
+  //     FPF = false, for shapes whose accumulators leave no room: read at the k-step's start);
+  //   * commits slab t + 2 from register stage t % PF to buffer (t+2) % 3 (last read in iteration
+  //     t - 1, i.e. before the previous barrier), then refills that stage with slab t + 2 + PF:
+  //     a global load has PF whole slabs of MFMA work to arrive.
+  // The LDS writes of iteration t are waited for at the barrier that ends it, having had a
+  // k-step of MFMAs to drain.
+  // The loop body is straight-line code on purpose (no test for "is there a next slab"): fetches
+  // and commits past the end of the k range are clamped / zero-filled by the loader and land in
+  // registers or LDS buffers whose contents are multiplied by nothing or are zeros. Only then can
+  // the compiler count the loads in flight and wait for the oldest stage alone. With PF = 2 the
+  // slab count is rounded up to even; the extra slab multiplies zeros.
+  constexpr int NKS = BK / KSTEP;
   const int64_t ktiles = (k_end - k_begin + BK - 1) / BK;
-  la.fetch(k_begin);
-  lb.fetch(k_begin);
-  la.commit(sA[0]);
-  lb.commit(sB[0]);
-  __syncthreads();
+  const int64_t kt_run = (ktiles + PF - 1) / PF * PF;
+  const int64_t full_slabs = (k_end - k_begin) / BK;
 
-  for (int64_t kt = 0; kt < ktiles; ++kt) {
-    const int cur = (int)(kt & 1);
-    const bool more = (kt + 1) < ktiles;
-    if (more) {
-      la.fetch(k_begin + (kt + 1) * BK);
-      lb.fetch(k_begin + (kt + 1) * BK);
-    }
-    const T* a_lds = sA[cur];
-    const T* b_lds = sB[cur];
+  T af[2][TM][VK], bf[2][TN][VK];
+  auto read_frags = [&](auto parity_tag, const T* a_lds, const T* b_lds, int ks) {
+    constexpr int P = decltype(parity_tag)::value;
 #pragma unroll
-    for (int ks = 0; ks < BK / KSTEP; ++ks) {
-      T af[TM][VK], bf[TN][VK];
+    for (int i = 0; i < TM; ++i) read_frag<T, AK, BM, BK>(a_lds, wave_m * WM + i * TILE + lrow, ks, kl, af[P][i]);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) read_frag<T, AK, BM, BK>(a_lds, wave_m * WM + i * TILE + lrow, ks, kl, af[i]);
+    for (int j = 0; j < TN; ++j) read_frag<T, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[P][j]);
+  };
+
+  // Prologue: slabs 0 and 1 into LDS, slabs 2 .. 2 + PF - 1 into the register stages.
+  la.template fetch<0>(k_begin);
+  lb.template fetch<0>(k_begin);
+  if constexpr (PF > 1) {
+    la.template fetch<1>(k_begin + BK);
+    lb.template fetch<1>(k_begin + BK);
+    la.template commit<0>(sA[0], k_begin);
+    lb.template commit<0>(sB[0], k_begin);
+    la.template commit<1>(sA[1], k_begin + BK);
+    lb.template commit<1>(sB[1], k_begin + BK);
+    la.template fetch<0>(k_begin + 2 * BK);
+    lb.template fetch<0>(k_begin + 2 * BK);
+    la.template fetch<1>(k_begin + 3 * BK);
+    lb.template fetch<1>(k_begin + 3 * BK);
+  } else {
+    la.template commit<0>(sA[0], k_begin);
+    lb.template commit<0>(sB[0], k_begin);
+    la.template fetch<0>(k_begin + BK);
+    lb.template fetch<0>(k_begin + BK);
+    la.template commit<0>(sA[1], k_begin + BK);
+    lb.template commit<0>(sB[1], k_begin + BK);
+    la.template fetch<0>(k_begin + 2 * BK);
+    lb.template fetch<0>(k_begin + 2 * BK);
+  }
+  __syncthreads();
+  if constexpr (FPF) read_frags(std::integral_constant<int, 0>(), sA[0], sB[0], 0);
+
+  int cur = 0;   // ring position of the slab being multiplied
+  auto slab = [&](auto stage_tag, auto mask_tag, int64_t kt) {
+    constexpr int S = decltype(stage_tag)::value;
+    constexpr bool MASK = decltype(mask_tag)::value;
+    const int nxt = (cur == 2) ? 0 : cur + 1;
+    const int nxt2 = (nxt == 2) ? 0 : nxt + 1;
 #pragma unroll
-      for (int j = 0; j < TN; ++j) read_frag<T, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[j]);
-      // The other LDS buffer has been free since the barrier that ended the previous slab, so the
-      // next slab is written into it in the middle of this slab's MFMA stream (before the last
-      // k-step) instead of after it: the wait for the global loads and the LDS writes then overlap
-      // with matrix-core work still queued, and only the barrier is left at the end of the slab.
-      if (ks == BK / KSTEP - 1 && more) {
-        la.commit(sA[cur ^ 1]);
-        lb.commit(sB[cur ^ 1]);
+    for (int ks = 0; ks < NKS; ++ks) {
+      // fragments for the k-step after this one: next k-step of this slab, or first of the next slab
+      if constexpr (!FPF) read_frags(std::integral_constant<int, 0>(), sA[cur], sB[cur], ks);
+      if (ks + 1 < NKS) {
+        if constexpr (FPF) {
+          if (ks & 1) read_frags(std::integral_constant<int, 0>(), sA[cur], sB[cur], ks + 1);
+          else read_frags(std::integral_constant<int, 1>(), sA[cur], sB[cur], ks + 1);
+        }
+      } else {
+        if constexpr (FPF) read_frags(std::integral_constant<int, 0>(), sA[nxt], sB[nxt], 0);   // NKS is even
+        la.template commit<S, MASK>(sA[nxt2], k_begin + (kt + 2) * BK);
+        lb.template commit<S, MASK>(sB[nxt2], k_begin + (kt + 2) * BK);
+        la.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
+        lb.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
       }
+      // The instruction scheduler would otherwise sink these reads and loads down to their first
+      // use; they have to be issued here, ahead of the MFMAs that cover their latency.
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s = 0; s < VK; ++s)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[i][s], bf[j][s], acc[i][j]);
+          for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[FPF ? (ks & 1) : 0][i][s], bf[FPF ? (ks & 1) : 0][j][s], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
+    cur = nxt;
+  };
+  // Steady state: every slab this iteration fetches or commits lies wholly inside the k range,
+  // so no clamping or zeroing is compiled in. The last few slabs run the masked version.
+  int64_t kt = 0;
+  for (; kt + (PF - 1) + 2 + PF < full_slabs; kt += PF) {
+    slab(std::integral_constant<int, 0>(), std::false_type(), kt);
+    if constexpr (PF > 1) slab(std::integral_constant<int, 1>(), std::false_type(), kt + 1);
+  }
+  for (; kt < kt_run; kt += PF) {
+    slab(std::integral_constant<int, 0>(), std::true_type(), kt);
+    if constexpr (PF > 1) slab(std::integral_constant<int, 1>(), std::true_type(), kt + 1);
   }
 
   // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
@@ -184,8 +259,35 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
   }
   const T alpha = p.alpha, beta = p.beta;
   const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
+  // One row of accumulator tiles at a time: first every load of C and of the bias for that row is
+  // issued, then the arithmetic and the stores follow. Interleaving load / store per element would
+  // make each load wait for the store before it (one memory counter orders both), i.e. one
+  // round trip to HBM per element.
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
+    T cv[TN][MF::NACC], bv[TN][MF::NACC];
+    if (beta != (T)0) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
+#pragma unroll
+        for (int r = 0; r < MF::NACC; ++r) {
+          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
+          cv[j][r] = (row < p.M && col < p.N) ? p.C[row * p.c_m + col * p.c_n] : (T)0;
+        }
+      }
+    }
+    if (has_bias) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
+#pragma unroll
+        for (int r = 0; r < MF::NACC; ++r) {
+          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
+          bv[j][r] = (row < p.M && col < p.N) ? p.bias[row * p.bias_m + col * p.bias_n] : (T)0;
+        }
+      }
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
@@ -193,25 +295,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 2) void gemm_mfma(Args<T> p)
       for (int r = 0; r < MF::NACC; ++r) {
         const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
         if (row < p.M && col < p.N) {
-          T* cp = p.C + row * p.c_m + col * p.c_n;
           T ab = acc[i][j][r];
           if (alpha != (T)1) ab = alpha * ab;
           T v = ab;
           if (beta != (T)0) {
-            T c = *cp;
+            T c = cv[j][r];
             if (beta != (T)1) c = c * beta;
             v = c + ab;
           }
-          if (has_bias) v = v + p.bias[row * p.bias_m + col * p.bias_n];
+          if (has_bias) v = v + bv[j][r];
           if (relu) v = ((T)0 >= v) ? (T)0 : v;
-          *cp = v;
+          p.C[row * p.c_m + col * p.c_n] = v;
         }
       }
     }
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true>
 static int launch_kinds(Args<T>& g, int ak, int bk) {
   g.tiles_m = (int)((g.M + BM - 1) / BM);
   g.tiles_n = (int)((g.N + BN - 1) / BN);
@@ -220,7 +321,7 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
   plan_splitk(g, BK, WAVES_M * WAVES_N);
   const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(WAVES_M * WAVES_N * 64);
 #define AM_LAUNCH(AKIND, BKIND_)                                                                   \
-  hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, AKIND, BKIND_>), grid, block, 0, \
+  hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, AKIND, BKIND_>), grid, block, 0, \
                      stream(), g)
   switch (ak * 3 + bk) {
     case 0: AM_LAUNCH(kKContig, kKContig); break;

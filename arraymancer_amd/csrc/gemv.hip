@@ -207,7 +207,8 @@ int gemv(const char* fn, int64_t M, int64_t N, T alpha, const T* A, int64_t rsA,
     if (g.splits > 1) {
       Args<T> r;
       memset(&r, 0, sizeof(r));
-      r.M = M; r.N = 1; r.K = N; r.alpha = alpha; r.beta = beta; r.C = y; r.c_m = incy; r.c_n = 0;
+      // y seen as one row of M columns: the reduction kernel spreads threads over columns
+      r.M = 1; r.N = M; r.K = N; r.alpha = alpha; r.beta = beta; r.C = y; r.c_m = 0; r.c_n = incy;
       r.epilogue = AM_EPI_NONE; r.splits = g.splits; r.ws = g.ws;
       return launch_splitk_reduce<T, U>(r);
     }

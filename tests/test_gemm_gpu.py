@@ -100,11 +100,13 @@ def test_edge_shapes_vs_oracle(hip, oracle, sfx, shape):
 
 
 @pytest.mark.parametrize("sfx", ALL)
-@pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4"])
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4", "5"])
 def test_every_tile_shape(hip, oracle, sfx, tile, monkeypatch):
     """Forces each workgroup tile candidate on a ragged problem."""
     if sfx in ("i32", "i64") and int(tile) >= 2:
         pytest.skip("integer path has two tile candidates")
+    if sfx == "f64" and int(tile) >= 5:
+        pytest.skip("float64 path has five tile candidates")
     monkeypatch.setenv(f"AM_HIP_GEMM_TILE_{sfx.upper()}", tile)
     dt = DTYPES[sfx]
     rng = np.random.default_rng(int(tile) + 17)
@@ -406,3 +408,40 @@ def test_small_mn_long_k_split_k(hip, oracle, sfx, shape):
     dCt = hip.toHip(np.zeros((N, M), dtype=dt)).transpose()
     hip.gemm(1, hip.toHip(np.ascontiguousarray(A.T)).transpose(), dB, 0, dCt)
     assert_parity(oracle, sfx, dCt.toCpu(), oracle.matmul(A, B), f"{shape} views")
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+@pytest.mark.parametrize("tile", ["0", "1"])
+@pytest.mark.parametrize("splits", ["1", "2", "3", "5", "16"])
+def test_integer_forced_split_k(hip, oracle, sfx, tile, splits, monkeypatch):
+    """Integer products may cut K into any number of ranges (ring arithmetic: no bit changes). Every
+    tile candidate with forced split factors on ragged shapes, wrapping values, alpha/beta and a
+    strided destination."""
+    monkeypatch.setenv(f"AM_HIP_GEMM_TILE_{sfx.upper()}", tile)
+    monkeypatch.setenv("AM_HIP_GEMM_SPLITK", splits)
+    dt = DTYPES[sfx]
+    info = np.iinfo(dt)
+    for shape in [(150, 130, 333), (129, 257, 40), (64, 64, 16), (300, 5, 1000)]:
+        M, N, K = shape
+        rng = np.random.default_rng(seed_of("forced-splitk", sfx, shape, tile, splits))
+        A, B, C = fill(rng, (M, K), dt, info.min, info.max), fill(rng, (K, N), dt, info.min, info.max), fill(rng, (M, 2 * N), dt, info.min, info.max)
+        say("forced split-k", sfx, tile, splits, shape)
+        want = C.copy()
+        oracle.gemm_strided(-3, A, B, 7, want[:, ::2])
+        dC = hip.toHip(C)
+        hip.gemm(-3, hip.toHip(A), hip.toHip(B), 7, dC[:, ::2])
+        assert np.array_equal(dC.toCpu(), want), f"{shape} tile {tile} splits {splits}"
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+def test_integer_mid_size_balanced_split(hip, oracle, sfx):
+    """Sizes whose tile count does not fill the CUs evenly: the library cuts K on its own."""
+    dt = DTYPES[sfx]
+    for shape in [(1000, 900, 1100), (640, 640, 2048), (1500, 1500, 160)]:
+        M, N, K = shape
+        rng = np.random.default_rng(seed_of("balanced", sfx, shape))
+        A, B = fill(rng, (M, K), dt, -1000, 1000), fill(rng, (K, N), dt, -1000, 1000)
+        say("balanced split-k", sfx, shape)
+        dC = hip.empty((M, N), dt)
+        hip.gemm(1, hip.toHip(A), hip.toHip(B), 0, dC)
+        assert np.array_equal(dC.toCpu(), oracle.matmul(A, B))
