@@ -234,7 +234,19 @@ __global__ __launch_bounds__(256) void splitk_reduce(Args<T> p) {
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sum[e] = v[e];
     }
-    for (int sidx = 1; sidx < p.splits; ++sidx) {
+    // eight partials in flight at a time (the loads are independent; the additions stay in
+    // ascending s): with one load per trip the pass is a chain of memory round trips
+    int sidx = 1;
+    for (; sidx + 8 <= p.splits; sidx += 8) {
+      vec_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *(const vec_t*)(ws + (int64_t)(sidx + u) * total + idx);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) sum[e] += v[u][e];
+    }
+    for (; sidx < p.splits; ++sidx) {
       const vec_t v = *(const vec_t*)(ws + (int64_t)sidx * total + idx);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sum[e] += v[e];
