@@ -19,6 +19,7 @@ OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh
 OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
 EPI = dict(none=0, bias=1, relu=2, bias_relu=3)
+RED = dict(sum=0, product=1, min=2, max=3)
 
 SFX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64",
        np.dtype(np.int32): "i32", np.dtype(np.int64): "i64"}
@@ -76,6 +77,11 @@ def _signatures():
         sig[f"am_hip_ew_scalar_{sfx}"] = (ci, [ci, ci, ci, vp, vp, vp, vp, vp, ct])
         sig[f"am_hip_ew_ternary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp, vp, vp, vp, vp])
         sig[f"am_hip_ew_unary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp])
+        sig[f"am_hip_reduce_axis_{sfx}"] = (ci, [ci, ci, vp, ci, vp, vp, vp, vp])
+        sig[f"am_hip_reduce_all_{sfx}"] = (ci, [ci, ci, vp, vp, vp, ctypes.POINTER(ct)])
+        sig[f"am_hip_maxpool2d_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp])
+        if sfx in ("f32", "f64"):
+            sig[f"am_hip_softmax_rows_{sfx}"] = (ci, [i64, i64, vp, i64, i64, vp, i64, i64])
     return sig
 
 

@@ -1,0 +1,644 @@
+// Reductions, row softmax and 2-D max pooling on device memory.
+//
+//   am_hip_reduce_axis_*   sum / product / min / max along one axis of a strided tensor
+//                          (reduce_axis_inline, src/arraymancer/tensor/higher_order_foldreduce.nim:46-61,
+//                           used by sum/product/min/max(axis), src/arraymancer/tensor/aggregate.nim:38-113)
+//   am_hip_reduce_all_*    the same over every element, result to the host
+//                          (reduce_inline, higher_order_foldreduce.nim:22-31; aggregate.nim:33-36,46-49,89-106)
+//   am_hip_softmax_rows_*  exp(x - max) / sum(exp(x - max)) per row
+//                          (src/arraymancer/nn_primitives/nnp_softmax.nim:18-38, private/p_logsumexp.nim:30-62)
+//   am_hip_maxpool2d_*     NCHW max pooling with the flat argmax indices the backward pass needs
+//                          (src/arraymancer/nn_primitives/nnp_maxpooling.nim:19-66)
+//
+// All of it is HBM-bound. Two kernels cover the axis reductions:
+//   * reduce_seq  one lane per output element, walking the axis front to back: consecutive lanes
+//                 read consecutive outputs, so it streams whenever some other dimension has unit
+//                 stride (e.g. sum over the rows of a row-major matrix). The fold order is the
+//                 reference's (first slice, then each following slice), so float sums agree with a
+//                 serial CPU fold bit for bit as long as the axis is not cut into chunks (below).
+//   * reduce_row  one wavefront per output element, lanes striding along the axis (16-byte loads
+//                 when it has unit stride), then a butterfly over the wavefront. Used when the
+//                 axis itself is the unit-stride dimension. Float results differ from a serial fold
+//                 by reassociation only.
+// When there are too few outputs to fill the chip, the axis is cut into chunks whose partial
+// results go to the library's workspace and are folded by a second pass.
+#include <limits>
+#include <string.h>
+#include "common.h"
+
+namespace am {
+namespace gemm { void* splitk_workspace(size_t bytes); }
+namespace red {
+
+constexpr int kMaxDims = AM_MAXRANK;
+
+template <typename T, int OP> struct Fold;
+template <typename T> struct Fold<T, AM_RED_SUM> { static __device__ __forceinline__ T apply(T x, T y) { return x + y; } };
+template <typename T> struct Fold<T, AM_RED_PROD> { static __device__ __forceinline__ T apply(T x, T y) { return x * y; } };
+// Nim's min / max on ordered types: `if x <= y: x else: y` / `if y <= x: x else: y`.
+template <typename T> struct Fold<T, AM_RED_MIN> { static __device__ __forceinline__ T apply(T x, T y) { return (x <= y) ? x : y; } };
+template <typename T> struct Fold<T, AM_RED_MAX> { static __device__ __forceinline__ T apply(T x, T y) { return (y <= x) ? x : y; } };
+
+// Integer sums and products wrap (two's complement), like the reference's `+=` / `*=` compiled
+// without overflow checks (-d:danger) and like the integer GEMM: fold in the unsigned twin.
+template <> struct Fold<int32_t, AM_RED_SUM> { static __device__ __forceinline__ int32_t apply(int32_t x, int32_t y) { return (int32_t)((uint32_t)x + (uint32_t)y); } };
+template <> struct Fold<int64_t, AM_RED_SUM> { static __device__ __forceinline__ int64_t apply(int64_t x, int64_t y) { return (int64_t)((uint64_t)x + (uint64_t)y); } };
+template <> struct Fold<int32_t, AM_RED_PROD> { static __device__ __forceinline__ int32_t apply(int32_t x, int32_t y) { return (int32_t)((uint32_t)x * (uint32_t)y); } };
+template <> struct Fold<int64_t, AM_RED_PROD> { static __device__ __forceinline__ int64_t apply(int64_t x, int64_t y) { return (int64_t)((uint64_t)x * (uint64_t)y); } };
+
+// The output elements: up to kMaxDims collapsed dimensions, slowest first.
+template <typename T> struct Args {
+  const T* a;
+  T* dst;            // final destination (strided)
+  T* ws;             // partial results [chunk][outputs] when chunks > 1
+  int ndim;
+  int64_t extent[kMaxDims], a_stride[kMaxDims], d_stride[kMaxDims];
+  int64_t outputs;   // product of the extents
+  int64_t L, a_axis_stride;   // reduced axis
+  int chunks;
+  int64_t chunk_len;
+};
+
+template <typename T>
+__device__ __forceinline__ void decode(const Args<T>& p, int64_t o, int64_t& a_off, int64_t& d_off) {
+  a_off = 0; d_off = 0;
+#pragma unroll
+  for (int d = kMaxDims - 1; d >= 0; --d) {
+    if (d < p.ndim) {
+      const int64_t q = o / p.extent[d], r = o - q * p.extent[d];
+      a_off += r * p.a_stride[d];
+      d_off += r * p.d_stride[d];
+      o = q;
+    }
+  }
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(256) void reduce_seq(Args<T> p) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= p.outputs) return;
+  int64_t a_off, d_off;
+  decode(p, o, a_off, d_off);
+  const int64_t l0 = (int64_t)blockIdx.y * p.chunk_len;
+  const int64_t l1 = (l0 + p.chunk_len < p.L) ? l0 + p.chunk_len : p.L;
+  const T* src = p.a + a_off + l0 * p.a_axis_stride;
+  T acc = *src;
+  int64_t l = l0 + 1;
+  // four loads in flight, folded in axis order
+  for (; l + 4 <= l1; l += 4) {
+    const T v0 = p.a[a_off + l * p.a_axis_stride], v1 = p.a[a_off + (l + 1) * p.a_axis_stride];
+    const T v2 = p.a[a_off + (l + 2) * p.a_axis_stride], v3 = p.a[a_off + (l + 3) * p.a_axis_stride];
+    acc = Fold<T, OP>::apply(acc, v0);
+    acc = Fold<T, OP>::apply(acc, v1);
+    acc = Fold<T, OP>::apply(acc, v2);
+    acc = Fold<T, OP>::apply(acc, v3);
+  }
+  for (; l < l1; ++l) acc = Fold<T, OP>::apply(acc, p.a[a_off + l * p.a_axis_stride]);
+  if (p.chunks > 1) p.ws[(int64_t)blockIdx.y * p.outputs + o] = acc;
+  else p.dst[d_off] = acc;
+}
+
+// Butterfly over the 64 lanes; lanes without an element (has == false) are skipped, so no
+// identity value is ever mixed in (a sum of negative zeros stays a negative zero).
+template <typename T, int OP>
+__device__ __forceinline__ void wave_fold(T& acc, bool& has) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    const T other = __shfl_xor(acc, d, 64);
+    const int other_has = __shfl_xor((int)has, d, 64);
+    // a fixed pairing and operand order: the result is the same on every run
+    const bool low = ((threadIdx.x & 63) & d) == 0;
+    if (other_has) {
+      if (has) acc = low ? Fold<T, OP>::apply(acc, other) : Fold<T, OP>::apply(other, acc);
+      else acc = other;
+      has = true;
+    }
+  }
+}
+
+template <typename T, int OP, bool VEC>
+__global__ __launch_bounds__(256) void reduce_row(Args<T> p) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const int lane = threadIdx.x & 63;
+  // one wavefront per (output, chunk) pair
+  const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (unit >= p.outputs * p.chunks) return;
+  const int64_t chunk = unit / p.outputs, o = unit - chunk * p.outputs;
+  int64_t a_off, d_off;
+  decode(p, o, a_off, d_off);
+  const int64_t l0 = chunk * p.chunk_len;
+  const int64_t l1 = (l0 + p.chunk_len < p.L) ? l0 + p.chunk_len : p.L;
+  T acc = (T)0;
+  bool has = false;
+  auto take = [&](T x) { acc = has ? Fold<T, OP>::apply(acc, x) : x; has = true; };
+  auto take_vec = [&](vec_t x) {
+    T part = x[0];
+#pragma unroll
+    for (int e = 1; e < V; ++e) part = Fold<T, OP>::apply(part, x[e]);
+    take(part);
+  };
+  if constexpr (VEC) {   // unit stride along the axis, every chunk start 16-byte aligned
+    const vec_t* src = (const vec_t*)(p.a + a_off + l0);
+    const int64_t nvec = (l1 - l0) / V;
+    int64_t v = lane;
+    for (; v + 192 < nvec; v += 256) {   // four 16-byte loads in flight per lane
+      const vec_t x0 = src[v], x1 = src[v + 64], x2 = src[v + 128], x3 = src[v + 192];
+      take_vec(x0); take_vec(x1); take_vec(x2); take_vec(x3);
+    }
+    for (; v < nvec; v += 64) take_vec(src[v]);
+    for (int64_t l = l0 + nvec * V + lane; l < l1; l += 64) take(p.a[a_off + l]);
+  } else {
+    for (int64_t l = l0 + lane; l < l1; l += 64) take(p.a[a_off + l * p.a_axis_stride]);
+  }
+  wave_fold<T, OP>(acc, has);
+  if (lane == 0) {
+    if (p.chunks > 1) p.ws[chunk * p.outputs + o] = acc;
+    else p.dst[d_off] = acc;
+  }
+}
+
+// ws_off: bytes at the start of the library workspace that the caller keeps for itself (the
+// chunk partials of this call go after them).
+template <typename T, int OP>
+static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
+  constexpr int64_t V = 16 / (int64_t)sizeof(T);
+  const int64_t cus = num_cus();
+  // Enough independent work for the whole chip: if the outputs alone do not supply it, cut the axis.
+  const int64_t units = row_kernel ? g.outputs : (g.outputs + 255) / 256;   // wavefronts resp. workgroups
+  const int64_t want_units = row_kernel ? cus * 32 : cus * 2;
+  const int64_t min_chunk = row_kernel ? 4096 : 64;
+  int64_t chunks = 1;
+  if (units < want_units && g.L >= 2 * min_chunk) {
+    chunks = (want_units + units - 1) / units;
+    if (chunks > g.L / min_chunk) chunks = g.L / min_chunk;
+    if (chunks > 8192) chunks = 8192;
+  }
+  g.chunks = 1; g.chunk_len = g.L; g.ws = nullptr;
+  if (chunks > 1) {
+    int64_t len = (g.L + chunks - 1) / chunks;
+    len = (len + V - 1) / V * V;                    // chunk starts stay 16-byte aligned
+    chunks = (g.L + len - 1) / len;
+    char* base = (chunks > 1) ? (char*)gemm::splitk_workspace(ws_off + (size_t)chunks * (size_t)g.outputs * sizeof(T)) : nullptr;
+    if (base) { g.chunks = (int)chunks; g.chunk_len = len; g.ws = (T*)(base + ws_off); }
+  }
+  if (row_kernel) {
+    bool vec = g.a_axis_stride == 1 && ((uintptr_t)g.a % 16 == 0);
+    for (int d = 0; d < g.ndim && vec; ++d) vec = (g.a_stride[d] % V == 0) || g.extent[d] == 1;
+    const int64_t bx = (g.outputs * g.chunks + 3) / 4;
+    if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "reduce: too many output elements");
+    const dim3 grid((unsigned)bx), block(256);
+    if (vec) hipLaunchKernelGGL((reduce_row<T, OP, true>), grid, block, 0, stream(), g);
+    else hipLaunchKernelGGL((reduce_row<T, OP, false>), grid, block, 0, stream(), g);
+  } else {
+    const int64_t bx = (g.outputs + 255) / 256;
+    if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "reduce: too many output elements");
+    hipLaunchKernelGGL((reduce_seq<T, OP>), dim3((unsigned)bx, (unsigned)g.chunks), dim3(256), 0, stream(), g);
+  }
+  AM_TRY(check_launch("reduce"));
+  if (g.chunks > 1) {   // fold the partials [chunk][outputs] front to back into dst
+    Args<T> r = g;
+    r.a = g.ws;
+    r.L = g.chunks; r.a_axis_stride = g.outputs;
+    int64_t s = 1;
+    for (int d = g.ndim - 1; d >= 0; --d) { r.a_stride[d] = s; s *= g.extent[d]; }
+    r.chunks = 1; r.chunk_len = r.L; r.ws = nullptr;
+    if (g.outputs < 1024 && g.chunks >= 64) {   // few outputs, many partials: a wavefront per output
+      const int64_t bx = (g.outputs + 3) / 4;
+      hipLaunchKernelGGL((reduce_row<T, OP, false>), dim3((unsigned)bx), dim3(256), 0, stream(), r);
+    } else {
+      const int64_t bx = (g.outputs + 255) / 256;
+      hipLaunchKernelGGL((reduce_seq<T, OP>), dim3((unsigned)bx, 1), dim3(256), 0, stream(), r);
+    }
+    AM_TRY(check_launch("reduce (second pass)"));
+  }
+  return AM_OK;
+}
+
+template <typename T>
+static int dispatch(int op, Args<T>& g, bool row_kernel, size_t ws_off) {
+  switch (op) {
+    case AM_RED_SUM: return launch<T, AM_RED_SUM>(g, row_kernel, ws_off);
+    case AM_RED_PROD: return launch<T, AM_RED_PROD>(g, row_kernel, ws_off);
+    case AM_RED_MIN: return launch<T, AM_RED_MIN>(g, row_kernel, ws_off);
+    default: return launch<T, AM_RED_MAX>(g, row_kernel, ws_off);
+  }
+}
+
+// Fills the output dimensions of `g` from every dimension but `axis`, merging neighbours that are
+// contiguous with each other in both the source and the destination.
+template <typename T>
+static void set_outputs(Args<T>& g, int rank, const int64_t* shape, int axis, const int64_t* sa, const int64_t* sd) {
+  g.ndim = 0; g.outputs = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (d == axis || shape[d] == 1) continue;
+    const int64_t ds = sd ? sd[d] : 0;
+    if (g.ndim > 0 && g.a_stride[g.ndim - 1] == sa[d] * shape[d] && (!sd || g.d_stride[g.ndim - 1] == ds * shape[d])) {
+      g.extent[g.ndim - 1] *= shape[d];
+      g.a_stride[g.ndim - 1] = sa[d];
+      g.d_stride[g.ndim - 1] = ds;
+    } else {
+      g.extent[g.ndim] = shape[d]; g.a_stride[g.ndim] = sa[d]; g.d_stride[g.ndim] = ds;
+      ++g.ndim;
+    }
+    g.outputs *= shape[d];
+  }
+  for (int d = g.ndim; d < kMaxDims; ++d) { g.extent[d] = 1; g.a_stride[d] = 0; g.d_stride[d] = 0; }
+}
+
+static inline int64_t iabs64(int64_t v) { return v < 0 ? -v : v; }
+
+template <typename T>
+static int reduce_axis(const char* fn, int op, int rank, const int64_t* shape, int axis, T* dst, const int64_t* sd,
+                       const T* a, const int64_t* sa) {
+  if (op < AM_RED_SUM || op > AM_RED_MAX) return fail(AM_E_ARG, "%s: unknown reduction %d", fn, op);
+  if (rank < 1 || rank > AM_MAXRANK) return fail(AM_E_SHAPE, "%s: rank %d outside 1..%d", fn, rank, AM_MAXRANK);
+  if (!shape || !sd || !sa) return fail(AM_E_ARG, "%s: null shape or strides", fn);
+  // IndexDefect of reduce_axis_inline (higher_order_foldreduce.nim:50-54)
+  if (axis < 0 || axis >= rank) return fail(AM_E_SHAPE, "%s: axis %d outside the tensor's rank %d", fn, axis, rank);
+  int64_t size = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+    size *= shape[d];
+  }
+  if (size == 0) return AM_OK;   // returnEmptyIfEmpty (aggregate.nim:40)
+  if (!dst || !a) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  Args<T> g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.dst = dst;
+  set_outputs(g, rank, shape, axis, sa, sd);
+  g.L = shape[axis]; g.a_axis_stride = sa[axis];
+  // The wavefront-per-output kernel when the axis is the cheapest direction to walk and long
+  // enough to feed 64 lanes; else one lane per output.
+  int64_t best_other = -1;
+  for (int d = 0; d < g.ndim; ++d) if (best_other < 0 || iabs64(g.a_stride[d]) < best_other) best_other = iabs64(g.a_stride[d]);
+  const bool row_kernel = g.L >= 64 && (best_other < 0 || iabs64(g.a_axis_stride) < best_other || g.outputs < 1024);
+  return dispatch<T>(op, g, row_kernel, 0);
+}
+
+template <typename T>
+static int reduce_all(const char* fn, int op, int rank, const int64_t* shape, const T* a, const int64_t* sa, T* result) {
+  if (!result) return fail(AM_E_ARG, "%s: null result pointer", fn);
+  if (op < AM_RED_SUM || op > AM_RED_MAX) return fail(AM_E_ARG, "%s: unknown reduction %d", fn, op);
+  if (rank < 0 || rank > AM_MAXRANK) return fail(AM_E_SHAPE, "%s: rank %d outside 0..%d", fn, rank, AM_MAXRANK);
+  if (rank > 0 && (!shape || !sa)) return fail(AM_E_ARG, "%s: null shape or strides", fn);
+  int64_t size = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+    size *= shape[d];
+  }
+  // reduce_inline starts from the first element: nothing to start from in an empty tensor
+  if (size == 0) return fail(AM_E_SHAPE, "%s: reduction of an empty tensor", fn);
+  if (!a) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  if (capturing()) return fail(AM_E_ARG, "%s: returns a value to the host, not allowed while a graph is being captured", fn);
+  // Dimensions merged where contiguous; a tensor that is one run of memory is a single "row".
+  Args<T> g;
+  memset(&g, 0, sizeof(g));
+  set_outputs(g, rank, shape, -1, sa, nullptr);
+  // workspace layout: [0, 256) the result; [256, 256 + tmp) one partial per run of a strided
+  // tensor; then the chunk partials of whichever step is running
+  T* out = (T*)gemm::splitk_workspace(256);
+  if (!out) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
+  Args<T> r;
+  memset(&r, 0, sizeof(r));
+  r.dst = out; r.ndim = 0; r.outputs = 1;
+  for (int d = 0; d < kMaxDims; ++d) r.extent[d] = 1;
+  if (g.ndim <= 1) {
+    r.a = a;
+    r.L = g.ndim == 1 ? g.extent[0] : 1;
+    r.a_axis_stride = g.ndim == 1 ? g.a_stride[0] : 1;
+    AM_TRY(dispatch<T>(op, r, r.L >= 64, 256));
+  } else {
+    // several runs of memory: fold the last (collapsed) dimension of each run into a temporary in
+    // the workspace, then fold that contiguous temporary
+    const int last = g.ndim - 1;
+    const int64_t rows = g.outputs / g.extent[last];
+    const size_t tmp_bytes = ((size_t)rows * sizeof(T) + 255) / 256 * 256;
+    if (tmp_bytes > (size_t)16 * 1024 * 1024)
+      return fail(AM_E_ALLOC, "%s: a non-contiguous tensor with %lld separate runs is too large for the reduction scratch; "
+                  "reduce a contiguous copy", fn, (long long)rows);
+    char* base = (char*)gemm::splitk_workspace(256 + tmp_bytes);
+    if (!base) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
+    T* tmp = (T*)(base + 256);
+    Args<T> s;
+    memset(&s, 0, sizeof(s));
+    s.a = a; s.dst = tmp;
+    s.ndim = last; s.outputs = rows;
+    int64_t cs = 1;
+    for (int d = last - 1; d >= 0; --d) { s.extent[d] = g.extent[d]; s.a_stride[d] = g.a_stride[d]; s.d_stride[d] = cs; cs *= g.extent[d]; }
+    for (int d = last; d < kMaxDims; ++d) { s.extent[d] = 1; s.a_stride[d] = 0; s.d_stride[d] = 0; }
+    s.L = g.extent[last]; s.a_axis_stride = g.a_stride[last];
+    AM_TRY(dispatch<T>(op, s, s.L >= 64, 256 + tmp_bytes));
+    r.a = tmp; r.L = rows; r.a_axis_stride = 1;
+    AM_TRY(dispatch<T>(op, r, r.L >= 64, 256 + tmp_bytes));
+  }
+  AM_HIP_TRY(hipMemcpyAsync(result, out, sizeof(T), hipMemcpyDeviceToHost, stream()));
+  AM_HIP_TRY(hipStreamSynchronize(stream()));
+  return AM_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Row softmax. One wavefront per row up to 4096 columns, one workgroup per row beyond. The row is
+// read three times (maximum, sum of exponentials, output); the second and third reads come from
+// cache. max and sum are what the reference's streaming pass arrives at, up to rounding of the sum.
+template <typename T> struct SoftmaxArgs {
+  const T* src; T* dst;
+  int64_t rows, cols, s_rs, s_cs, d_rs, d_cs;
+};
+
+template <typename T> __device__ __forceinline__ T dev_exp(T x);
+template <> __device__ __forceinline__ float dev_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double dev_exp<double>(double x) { return exp(x); }
+
+template <typename T, bool BLOCK>
+__global__ __launch_bounds__(256) void softmax_rows(SoftmaxArgs<T> p) {
+  constexpr int W = BLOCK ? 256 : 64;            // lanes working on one row
+  __shared__ T part[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = BLOCK ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+  const bool active = row < p.rows;
+  const int me = BLOCK ? (int)threadIdx.x : lane;
+  const T* src = p.src + (active ? row : 0) * p.s_rs;
+  // `x <= max` is false for the first element against -Inf only if x is NaN; NaN rows give NaN
+  T mx = -std::numeric_limits<T>::infinity();
+  if (active) for (int64_t c = me; c < p.cols; c += W) { const T x = src[c * p.s_cs]; mx = (x <= mx) ? mx : x; }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) { const T o = __shfl_xor(mx, d, 64); mx = (o <= mx) ? mx : o; }
+  if constexpr (BLOCK) {
+    if (lane == 0) part[wave] = mx;
+    __syncthreads();
+    mx = part[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = (part[w] <= mx) ? mx : part[w];
+    __syncthreads();
+  }
+  T sum = (T)0;
+  if (active) for (int64_t c = me; c < p.cols; c += W) sum += dev_exp<T>(src[c * p.s_cs] - mx);
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d, 64);
+  if constexpr (BLOCK) {
+    if (lane == 0) part[wave] = sum;
+    __syncthreads();
+    sum = ((part[0] + part[1]) + part[2]) + part[3];
+  }
+  if (!active) return;
+  T* dst = p.dst + row * p.d_rs;
+  for (int64_t c = me; c < p.cols; c += W) dst[c * p.d_cs] = dev_exp<T>(src[c * p.s_cs] - mx) / sum;   // stable_softmax
+}
+
+// Contiguous rows that fit in registers: each lane keeps NV 16-byte vectors of its row, so the
+// row is read from memory once and written once. W lanes per row (64: four rows per workgroup;
+// 256: one row per workgroup). Requires unit column strides, cols a multiple of the vector width
+// and 16-byte aligned rows; cols <= W * NV * VEC.
+template <typename T, int W, int NV>
+__global__ __launch_bounds__(256) void softmax_rows_reg(SoftmaxArgs<T> p) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  __shared__ T part[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (W == 256) ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+  const bool active = row < p.rows;
+  const int me = (W == 256) ? (int)threadIdx.x : lane;
+  const int64_t nvec = p.cols / V;
+  const vec_t* src = (const vec_t*)(p.src + (active ? row : 0) * p.s_rs);
+  const T ninf = -std::numeric_limits<T>::infinity();
+  vec_t x[NV];
+  T mx = ninf;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int64_t v = (int64_t)i * W + me;
+    if (active && v < nvec) {
+      x[i] = src[v];
+#pragma unroll
+      for (int e = 0; e < V; ++e) mx = (x[i][e] <= mx) ? mx : x[i][e];
+    }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) { const T o = __shfl_xor(mx, d, 64); mx = (o <= mx) ? mx : o; }
+  if constexpr (W == 256) {
+    if (lane == 0) part[wave] = mx;
+    __syncthreads();
+    mx = part[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = (part[w] <= mx) ? mx : part[w];
+    __syncthreads();
+  }
+  T sum = (T)0;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int64_t v = (int64_t)i * W + me;
+    if (active && v < nvec) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) { x[i][e] = dev_exp<T>(x[i][e] - mx); sum += x[i][e]; }
+    }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d, 64);
+  if constexpr (W == 256) {
+    if (lane == 0) part[wave] = sum;
+    __syncthreads();
+    sum = ((part[0] + part[1]) + part[2]) + part[3];
+  }
+  if (!active) return;
+  vec_t* dst = (vec_t*)(p.dst + row * p.d_rs);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int64_t v = (int64_t)i * W + me;
+    if (v < nvec) {
+      vec_t y;
+#pragma unroll
+      for (int e = 0; e < V; ++e) y[e] = x[i][e] / sum;
+      __builtin_nontemporal_store(y, dst + v);
+    }
+  }
+}
+
+template <typename T, int W>
+static void launch_softmax_reg(const SoftmaxArgs<T>& p, int nv, dim3 grid) {
+  switch (nv) {
+    case 1: hipLaunchKernelGGL((softmax_rows_reg<T, W, 1>), grid, dim3(256), 0, stream(), p); break;
+    case 2: hipLaunchKernelGGL((softmax_rows_reg<T, W, 2>), grid, dim3(256), 0, stream(), p); break;
+    case 4: hipLaunchKernelGGL((softmax_rows_reg<T, W, 4>), grid, dim3(256), 0, stream(), p); break;
+    default: hipLaunchKernelGGL((softmax_rows_reg<T, W, 8>), grid, dim3(256), 0, stream(), p); break;
+  }
+}
+
+template <typename T>
+static int softmax(const char* fn, int64_t rows, int64_t cols, T* dst, int64_t d_rs, int64_t d_cs, const T* src,
+                   int64_t s_rs, int64_t s_cs) {
+  constexpr int64_t V = 16 / (int64_t)sizeof(T);
+  if (rows < 0 || cols < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+  if (rows == 0 || cols == 0) return AM_OK;
+  if (!dst || !src) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  if (rows >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many rows", fn);
+  AM_TRY(ensure_init());
+  SoftmaxArgs<T> p = {src, dst, rows, cols, s_rs, s_cs, d_rs, d_cs};
+  const bool vec = s_cs == 1 && d_cs == 1 && cols % V == 0 && (rows == 1 || (s_rs % V == 0 && d_rs % V == 0)) &&
+                   (uintptr_t)src % 16 == 0 && (uintptr_t)dst % 16 == 0;
+  const int64_t nvec = cols / V;
+  if (vec && nvec <= 64 * 8) {          // a wavefront per row
+    int nv = 1;
+    while (64 * nv < nvec) nv *= 2;
+    launch_softmax_reg<T, 64>(p, nv, dim3((unsigned)((rows + 3) / 4)));
+  } else if (vec && nvec <= 256 * 8) {  // a workgroup per row
+    int nv = 1;
+    while (256 * nv < nvec) nv *= 2;
+    launch_softmax_reg<T, 256>(p, nv, dim3((unsigned)rows));
+  } else if (cols > 4096) {
+    hipLaunchKernelGGL((softmax_rows<T, true>), dim3((unsigned)rows), dim3(256), 0, stream(), p);
+  } else {
+    hipLaunchKernelGGL((softmax_rows<T, false>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream(), p);
+  }
+  return check_launch("softmax_rows");
+}
+
+// ------------------------------------------------------------------------------------------------
+// Max pooling, one lane per output element; same scan order, strict `>` and starting values as
+// the reference, so values and argmax indices are identical (first maximum wins; a window that
+// lies wholly in the padding yields lowest(T) and the lowest index).
+template <typename T> struct Lowest { static __device__ __forceinline__ T value() { return std::numeric_limits<T>::lowest(); } };
+// low(float) in Nim is -Inf
+template <> struct Lowest<float> { static __device__ __forceinline__ float value() { return -std::numeric_limits<float>::infinity(); } };
+template <> struct Lowest<double> { static __device__ __forceinline__ double value() { return -std::numeric_limits<double>::infinity(); } };
+
+// IDX: uint32_t when both tensors have fewer than 2^32 elements (64-bit division is slow).
+template <typename T, typename IDX>
+__global__ __launch_bounds__(256) void maxpool2d(const T* in, T* out, int64_t* argmax, int64_t total, int C, int H, int W,
+                                                 int kH, int kW, int padH, int padW, int sH, int sW, int outH, int outW) {
+  const int64_t oidx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (oidx >= total) return;
+  const IDX oi = (IDX)oidx;
+  const int w = (int)(oi % (IDX)outW);
+  const IDX t = oi / (IDX)outW;
+  const int h = (int)(t % (IDX)outH);
+  const int64_t nc = (int64_t)(t / (IDX)outH);   // n * C + c
+  T mx = Lowest<T>::value();
+  int64_t arg = std::numeric_limits<int64_t>::lowest();
+  for (int ph = 0; ph < kH; ++ph) {
+    const int row = h * sH + ph - padH;
+    if (row < 0 || row >= H) continue;
+    for (int pw = 0; pw < kW; ++pw) {
+      const int col = w * sW + pw - padW;
+      if (col < 0 || col >= W) continue;
+      const int64_t iidx = col + (int64_t)W * (row + (int64_t)H * nc);
+      const T v = in[iidx];
+      if (v > mx) { mx = v; arg = iidx; }
+    }
+  }
+  out[oidx] = mx;
+  if (argmax) argmax[oidx] = arg;
+}
+
+// The common 2-wide, stride-2, unpadded-in-width pooling with 16-byte aligned rows: one lane makes
+// V = 16 / sizeof(T) neighbouring outputs from two 16-byte loads per window row, and stores them
+// (and their indices) as vectors. Window scan order and comparisons as in the kernel above.
+template <typename T>
+__global__ __launch_bounds__(256) void maxpool2d_w2(const T* in, T* out, int64_t* argmax, int64_t total_vec, int H, int W,
+                                                    int kH, int padH, int sH, int outH, int outWv) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  typedef int64_t idx2_t __attribute__((ext_vector_type(2)));
+  const int64_t ov = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ov >= total_vec) return;
+  const uint32_t o32 = (uint32_t)ov;           // the launcher guarantees total_vec < 2^32
+  const int wv = (int)(o32 % (uint32_t)outWv);
+  const uint32_t t = o32 / (uint32_t)outWv;
+  const int h = (int)(t % (uint32_t)outH);
+  const int64_t nc = (int64_t)(t / (uint32_t)outH);
+  T mx[V];
+  int64_t arg[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) { mx[j] = Lowest<T>::value(); arg[j] = std::numeric_limits<int64_t>::lowest(); }
+  for (int ph = 0; ph < kH; ++ph) {
+    const int row = h * sH + ph - padH;
+    if (row < 0 || row >= H) continue;
+    const int64_t base = (int64_t)W * (row + (int64_t)H * nc) + (int64_t)wv * 2 * V;
+    const vec_t lo = *(const vec_t*)(in + base), hi = *(const vec_t*)(in + base + V);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+#pragma unroll
+      for (int pw = 0; pw < 2; ++pw) {
+        const int e = 2 * j + pw;
+        const T v = (e < V) ? lo[e] : hi[e - V];
+        if (v > mx[j]) { mx[j] = v; arg[j] = base + e; }
+      }
+    }
+  }
+  vec_t r;
+#pragma unroll
+  for (int j = 0; j < V; ++j) r[j] = mx[j];
+  __builtin_nontemporal_store(r, (vec_t*)(out + ov * V));
+  if (argmax) {
+#pragma unroll
+    for (int j = 0; j < V; j += 2) {
+      idx2_t a2 = {arg[j], arg[j + 1]};
+      __builtin_nontemporal_store(a2, (idx2_t*)(argmax + ov * V + j));
+    }
+  }
+}
+
+template <typename T>
+static int maxpool(const char* fn, int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
+                   const T* in, T* out, int64_t* argmax) {
+  if (N < 0 || C < 0 || H < 0 || W < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+  if (kH < 1 || kW < 1 || sH < 1 || sW < 1 || padH < 0 || padW < 0) return fail(AM_E_ARG, "%s: kernel and stride must be >= 1, padding >= 0", fn);
+  const int64_t outH = ((int64_t)H + 2 * padH - kH) / sH + 1, outW = ((int64_t)W + 2 * padW - kW) / sW + 1;
+  if ((int64_t)H + 2 * padH < kH || (int64_t)W + 2 * padW < kW) return fail(AM_E_SHAPE, "%s: kernel larger than the padded input", fn);
+  const int64_t total = N * C * outH * outW;
+  if (total == 0) return AM_OK;
+  if (!in || !out) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  constexpr int64_t V = 16 / (int64_t)sizeof(T);
+  if (kW == 2 && sW == 2 && padW == 0 && W % (2 * V) == 0 && total / V < ((int64_t)1 << 32) && (uintptr_t)in % 16 == 0 &&
+      (uintptr_t)out % 16 == 0 && (uintptr_t)argmax % 16 == 0) {
+    const int64_t total_vec = total / V;
+    hipLaunchKernelGGL((maxpool2d_w2<T>), dim3((unsigned)((total_vec + 255) / 256)), dim3(256), 0, stream(), in, out, argmax,
+                       total_vec, H, W, kH, padH, sH, (int)outH, (int)(outW / V));
+    return check_launch("maxpool2d_w2");
+  }
+  const int64_t bx = (total + 255) / 256;
+  if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many output elements", fn);
+  if (total < ((int64_t)1 << 32))
+    hipLaunchKernelGGL((maxpool2d<T, uint32_t>), dim3((unsigned)bx), dim3(256), 0, stream(), in, out, argmax, total, C, H, W,
+                       kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
+  else
+    hipLaunchKernelGGL((maxpool2d<T, uint64_t>), dim3((unsigned)bx), dim3(256), 0, stream(), in, out, argmax, total, C, H, W,
+                       kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
+  return check_launch("maxpool2d");
+}
+
+}  // namespace red
+}  // namespace am
+
+using namespace am;
+
+#define AM_RED_ENTRY_POINTS(T, SFX)                                                                                    \
+  extern "C" int am_hip_reduce_axis_##SFX(int op, int rank, const int64_t* shape, int axis, T* dst,                    \
+                                          const int64_t* dst_strides, const T* a, const int64_t* a_strides) {          \
+    return red::reduce_axis<T>("am_hip_reduce_axis_" #SFX, op, rank, shape, axis, dst, dst_strides, a, a_strides);     \
+  }                                                                                                                    \
+  extern "C" int am_hip_reduce_all_##SFX(int op, int rank, const int64_t* shape, const T* a, const int64_t* a_strides, \
+                                         T* result) {                                                                  \
+    return red::reduce_all<T>("am_hip_reduce_all_" #SFX, op, rank, shape, a, a_strides, result);                       \
+  }                                                                                                                    \
+  extern "C" int am_hip_maxpool2d_##SFX(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW,            \
+                                        int strideH, int strideW, const T* input, T* output, int64_t* argmax) {        \
+    return red::maxpool<T>("am_hip_maxpool2d_" #SFX, N, C, H, W, kH, kW, padH, padW, strideH, strideW, input, output,  \
+                           argmax);                                                                                    \
+  }
+
+AM_RED_ENTRY_POINTS(float, f32)
+AM_RED_ENTRY_POINTS(double, f64)
+AM_RED_ENTRY_POINTS(int32_t, i32)
+AM_RED_ENTRY_POINTS(int64_t, i64)
+
+extern "C" int am_hip_softmax_rows_f32(int64_t rows, int64_t cols, float* dst, int64_t dst_rs, int64_t dst_cs,
+                                       const float* src, int64_t src_rs, int64_t src_cs) {
+  return red::softmax<float>("am_hip_softmax_rows_f32", rows, cols, dst, dst_rs, dst_cs, src, src_rs, src_cs);
+}
+extern "C" int am_hip_softmax_rows_f64(int64_t rows, int64_t cols, double* dst, int64_t dst_rs, int64_t dst_cs,
+                                       const double* src, int64_t src_rs, int64_t src_cs) {
+  return red::softmax<double>("am_hip_softmax_rows_f64", rows, cols, dst, dst_rs, dst_cs, src, src_rs, src_cs);
+}

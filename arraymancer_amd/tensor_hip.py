@@ -28,7 +28,7 @@ import numpy as np
 
 from . import _lib
 from . import metadata as md
-from ._lib import CTYPE, EPI, OP, OP3, SFX, UOP, check, i64_array
+from ._lib import CTYPE, EPI, OP, OP3, RED, SFX, UOP, check, i64_array
 from .metadata import Layout, Step
 
 
@@ -627,3 +627,89 @@ def bias_relu(x: HipTensor, b: HipTensor) -> HipTensor:
 OPERATORS = {"+.": bc_add, "-.": bc_sub, "*.": bc_mul, "/.": bc_div, "mod": bc_mod,
              "+.=": HipTensor.bc_iadd, "-.=": HipTensor.bc_isub, "*.=": HipTensor.bc_imul,
              "/.=": HipTensor.bc_idiv}
+
+
+# ---------------------------------------------------------------- reductions, softmax, pooling
+def reduce_axis(op, t: HipTensor, axis: int) -> HipTensor:
+    """reduce_axis_inline (src/arraymancer/tensor/higher_order_foldreduce.nim:46-61): fold along
+    `axis`; the result keeps that axis with extent 1. An empty tensor comes back empty
+    (returnEmptyIfEmpty, aggregate.nim:40); an axis outside the rank raises IndexError."""
+    if not 0 <= axis < t.rank:
+        raise IndexError(f"Input tensor rank ({t.rank}) must be greater than reduction axis ({axis})")
+    if t.size == 0:
+        return empty(t.shape, t.dtype)
+    shape = list(t.shape)
+    shape[axis] = 1
+    out = empty(shape, t.dtype)
+    check(getattr(_lib.load(), f"am_hip_reduce_axis_{t.sfx}")(
+        RED[op], t.rank, i64_array(t.shape), axis, ctypes.c_void_p(out.data_ptr()), i64_array(out.strides),
+        ctypes.c_void_p(t.data_ptr()), i64_array(t.strides)))
+    return out
+
+
+def reduce_all(op, t: HipTensor):
+    """reduce_inline (higher_order_foldreduce.nim:22-31): fold of every element, returned to the host."""
+    out = CTYPE[t.sfx]()
+    check(getattr(_lib.load(), f"am_hip_reduce_all_{t.sfx}")(
+        RED[op], t.rank, i64_array(t.shape), ctypes.c_void_p(t.data_ptr()), i64_array(t.strides), ctypes.byref(out)))
+    return t.dtype.type(out.value)
+
+
+def _aggregate(op):
+    def f(t: HipTensor, axis: int | None = None):
+        return reduce_all(op, t) if axis is None else reduce_axis(op, t, axis)
+    f.__name__ = op
+    f.__doc__ = f"{op} of all elements (scalar on the host) or along `axis` (src/arraymancer/tensor/aggregate.nim:33-113)."
+    return f
+
+
+# exported by the package as sum / product / min / max (the reference's names); other names here
+# so that this module's own use of the builtins stays intact
+tsum = _aggregate("sum")
+tproduct = _aggregate("product")
+tmin = _aggregate("min")
+tmax = _aggregate("max")
+
+
+def mean(t: HipTensor, axis: int | None = None):
+    """aggregate.nim:58-86: the sum divided by the element count; integer tensors use `div`."""
+    if axis is None:
+        s = reduce_all("sum", t)
+        if t.dtype.kind == "f":
+            return t.dtype.type(s / t.dtype.type(t.size))
+        q = abs(int(s)) // t.size               # truncation towards zero, like Nim's div
+        return t.dtype.type(q if int(s) >= 0 else -q)
+    if t.size == 0:
+        return empty(t.shape, t.dtype)
+    return scalar_op("div", reduce_axis("sum", t, axis), t.dtype.type(t.shape[axis]))
+
+
+def softmax(t: HipTensor) -> HipTensor:
+    """Row softmax of a [batch_size, number_of_classes] matrix
+    (src/arraymancer/nn_primitives/nnp_softmax.nim:18-38)."""
+    if t.rank != 2:
+        raise ValueError("softmax: input must be [batch_size, number_of_classes]")
+    if t.dtype.kind != "f":
+        raise TypeError("softmax is defined for float tensors")
+    out = empty(t.shape, t.dtype)
+    check(getattr(_lib.load(), f"am_hip_softmax_rows_{t.sfx}")(
+        t.shape[0], t.shape[1], ctypes.c_void_p(out.data_ptr()), *out.strides, ctypes.c_void_p(t.data_ptr()), *t.strides))
+    return out
+
+
+def maxpool2d(x: HipTensor, kernel, padding=(0, 0), stride=(1, 1)):
+    """(max_indices, maxpooled) of a C-contiguous [N, C, H, W] tensor
+    (src/arraymancer/nn_primitives/nnp_maxpooling.nim:19-66; the reference asserts contiguity too).
+    max_indices is a device int64 vector of flat input indices."""
+    if x.rank != 4 or not x.is_C_contiguous:
+        raise ValueError("maxpool2d: input must be a C-contiguous [N, C, H, W] tensor")
+    N, C, H, W = x.shape
+    (kh, kw), (ph, pw), (sh, sw) = kernel, padding, stride
+    ho, wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    out = empty((N, C, ho, wo), x.dtype)
+    idx = empty((N * C * ho * wo,), np.int64)
+    check(getattr(_lib.load(), f"am_hip_maxpool2d_{x.sfx}")(
+        N, C, H, W, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+        ctypes.c_void_p(idx.data_ptr())))
+    return idx, out
+

@@ -316,6 +316,62 @@ int am_hip_ew_ternary_i64(int op, int rank, const int64_t* shape, int64_t* dst, 
                           const int64_t* a, const int64_t* a_strides, const int64_t* b, const int64_t* b_strides,
                           const int64_t* c, const int64_t* c_strides);
 
+/* ---------------------------------------------------------------- reductions, softmax, pooling
+ * dst <- fold of `a` along `axis` with op (AM_RED_*). `shape` / `a_strides` describe `a` (rank
+ * 1..AM_MAXRANK, element strides, any sign); dst has the same rank with extent 1 along `axis`
+ * (dst_strides[axis] is ignored), exactly what reduce_axis_inline returns
+ * (src/arraymancer/tensor/higher_order_foldreduce.nim:46-61; sum/product/min/max(axis),
+ * src/arraymancer/tensor/aggregate.nim:38-113). The fold starts from the first slice and takes the
+ * following ones in order. Integer sums/products wrap; min/max are Nim's (`if x <= y: x else: y`).
+ * An empty tensor returns AM_OK without touching dst (returnEmptyIfEmpty); axis outside the rank:
+ * AM_E_SHAPE (the reference's IndexDefect). Float sums along a unit-stride axis are reassociated
+ * (tree over a wavefront, chunked for very long axes): equal to a serial fold up to rounding. */
+#define AM_RED_SUM  0
+#define AM_RED_PROD 1
+#define AM_RED_MIN  2
+#define AM_RED_MAX  3
+int am_hip_reduce_axis_f32(int op, int rank, const int64_t* shape, int axis, float* dst, const int64_t* dst_strides,
+                           const float* a, const int64_t* a_strides);
+int am_hip_reduce_axis_f64(int op, int rank, const int64_t* shape, int axis, double* dst, const int64_t* dst_strides,
+                           const double* a, const int64_t* a_strides);
+int am_hip_reduce_axis_i32(int op, int rank, const int64_t* shape, int axis, int32_t* dst, const int64_t* dst_strides,
+                           const int32_t* a, const int64_t* a_strides);
+int am_hip_reduce_axis_i64(int op, int rank, const int64_t* shape, int axis, int64_t* dst, const int64_t* dst_strides,
+                           const int64_t* a, const int64_t* a_strides);
+
+/* *result (HOST pointer) <- fold of every element of `a` (rank 0..AM_MAXRANK); blocks until the
+ * value has arrived; not allowed during graph capture. Replaces reduce_inline and sum / product /
+ * min / max without axis (higher_order_foldreduce.nim:22-31, aggregate.nim:33-36,46-49,89-106).
+ * An empty tensor has no first element to start from: AM_E_SHAPE. */
+int am_hip_reduce_all_f32(int op, int rank, const int64_t* shape, const float* a, const int64_t* a_strides, float* result);
+int am_hip_reduce_all_f64(int op, int rank, const int64_t* shape, const double* a, const int64_t* a_strides, double* result);
+int am_hip_reduce_all_i32(int op, int rank, const int64_t* shape, const int32_t* a, const int64_t* a_strides, int32_t* result);
+int am_hip_reduce_all_i64(int op, int rank, const int64_t* shape, const int64_t* a, const int64_t* a_strides, int64_t* result);
+
+/* dst[i, j] <- exp(src[i, j] - max_i) / sum_j exp(src[i, j] - max_i) for a [rows, cols] matrix
+ * with element strides (rs, cs) on both sides; dst may be src. Replaces softmax
+ * (src/arraymancer/nn_primitives/nnp_softmax.nim:18-38: streaming_max_sumexp + stable_softmax,
+ * private/p_logsumexp.nim:30-62); the row sum is accumulated in a different order than the
+ * reference's streaming pass, the result agrees to rounding. */
+int am_hip_softmax_rows_f32(int64_t rows, int64_t cols, float* dst, int64_t dst_rs, int64_t dst_cs,
+                            const float* src, int64_t src_rs, int64_t src_cs);
+int am_hip_softmax_rows_f64(int64_t rows, int64_t cols, double* dst, int64_t dst_rs, int64_t dst_cs,
+                            const double* src, int64_t src_rs, int64_t src_cs);
+
+/* Max pooling of a C-contiguous [N, C, H, W] input into a C-contiguous [N, C, outH, outW] output,
+ * outH = (H + 2 padH - kH) / strideH + 1 (outW alike), plus, when argmax != NULL, the flat input
+ * index of each maximum (what maxpool2d_backward scatters through). Same window scan order,
+ * strict `>` and starting values as maxpool2d
+ * (src/arraymancer/nn_primitives/nnp_maxpooling.nim:19-66): identical values and indices. */
+int am_hip_maxpool2d_f32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                         const float* input, float* output, int64_t* argmax);
+int am_hip_maxpool2d_f64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                         const double* input, double* output, int64_t* argmax);
+int am_hip_maxpool2d_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                         const int32_t* input, int32_t* output, int64_t* argmax);
+int am_hip_maxpool2d_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                         const int64_t* input, int64_t* output, int64_t* argmax);
+
 /* ---------------------------------------------------------------- measurement aid
  * No counterpart in the reference. Register-only micro-benchmarks of the issue ceilings the GEMM
  * kernels are compared with (used by bench.py: 32/64-bit integers have no matrix instruction and no

@@ -72,6 +72,17 @@ namespace detail {
   }                                                                                                      \
   inline int dot_(int64_t n, const T* x, int64_t ix, const T* y, int64_t iy, T* r) {                     \
     return am_hip_dot_##SFX(n, x, ix, y, iy, r);                                                          \
+  }                                                                                                      \
+  inline int reduce_axis_(int op, int rank, const int64_t* sh, int axis, T* d, const int64_t* sd, const T* a, \
+                          const int64_t* sa) {                                                            \
+    return am_hip_reduce_axis_##SFX(op, rank, sh, axis, d, sd, a, sa);                                    \
+  }                                                                                                      \
+  inline int reduce_all_(int op, int rank, const int64_t* sh, const T* a, const int64_t* sa, T* r) {      \
+    return am_hip_reduce_all_##SFX(op, rank, sh, a, sa, r);                                               \
+  }                                                                                                      \
+  inline int maxpool2d_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,    \
+                        const T* in, T* out, int64_t* idx) {                                              \
+    return am_hip_maxpool2d_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, in, out, idx);                      \
   }
 AM_HPP_BIND2(float, f32)
 AM_HPP_BIND2(double, f64)
@@ -92,6 +103,13 @@ inline int gemm_ex_(int64_t M, int64_t N, int64_t K, double al, const double* A,
                     const double* B, int64_t rb, int64_t cb, double be, double* C, int64_t rc, int64_t cc, int epi,
                     const double* bias, int64_t brs, int64_t bcs) {
   return am_hip_gemm_ex_f64(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc, epi, bias, brs, bcs);
+}
+
+inline int softmax_(int64_t r, int64_t c, float* d, int64_t drs, int64_t dcs, const float* s, int64_t srs, int64_t scs) {
+  return am_hip_softmax_rows_f32(r, c, d, drs, dcs, s, srs, scs);
+}
+inline int softmax_(int64_t r, int64_t c, double* d, int64_t drs, int64_t dcs, const double* s, int64_t srs, int64_t scs) {
+  return am_hip_softmax_rows_f64(r, c, d, drs, dcs, s, srs, scs);
 }
 
 inline std::string str(const Shape& s) {
@@ -371,6 +389,69 @@ HipTensor<T> linear(const HipTensor<T>& x, const HipTensor<T>& weight, const Hip
   check(detail::gemm_ex_(x.shape[0], wt.shape[1], x.shape[1], T(1), x.ptr(), x.strides[0], x.strides[1], wt.ptr(),
                          wt.strides[0], wt.strides[1], T(0), r.ptr(), r.strides[0], r.strides[1],
                          with_relu ? AM_EPI_BIAS_RELU : AM_EPI_BIAS, bb.ptr(), bb.strides[0], bb.strides[1]));
+  return r;
+}
+
+// Fold along `axis`; the result keeps the axis with extent 1 (reduce_axis_inline,
+// higher_order_foldreduce.nim:46-61). op: AM_RED_SUM / PROD / MIN / MAX.
+template <typename T>
+HipTensor<T> reduce_axis(int op, const HipTensor<T>& t, int axis) {
+  if (axis < 0 || axis >= t.rank())
+    throw std::out_of_range("Input tensor rank (" + std::to_string(t.rank()) + ") must be greater than reduction axis (" +
+                            std::to_string(axis) + ")");
+  if (t.size() == 0) return HipTensor<T>(t.shape);   // returnEmptyIfEmpty
+  Shape sh = t.shape;
+  sh[axis] = 1;
+  HipTensor<T> r(sh);
+  check(detail::reduce_axis_(op, t.rank(), t.shape.data(), axis, r.ptr(), r.strides.data(), t.ptr(), t.strides.data()));
+  return r;
+}
+
+// Fold of every element, returned to the host (reduce_inline, higher_order_foldreduce.nim:22-31).
+template <typename T>
+T reduce_all(int op, const HipTensor<T>& t) {
+  T r{};
+  check(detail::reduce_all_(op, t.rank(), t.shape.data(), t.ptr(), t.strides.data(), &r));
+  return r;
+}
+
+// aggregate.nim:33-113
+template <typename T> T sum(const HipTensor<T>& t) { return reduce_all(AM_RED_SUM, t); }
+template <typename T> HipTensor<T> sum(const HipTensor<T>& t, int axis) { return reduce_axis(AM_RED_SUM, t, axis); }
+template <typename T> T product(const HipTensor<T>& t) { return reduce_all(AM_RED_PROD, t); }
+template <typename T> HipTensor<T> product(const HipTensor<T>& t, int axis) { return reduce_axis(AM_RED_PROD, t, axis); }
+template <typename T> T min(const HipTensor<T>& t) { return reduce_all(AM_RED_MIN, t); }
+template <typename T> HipTensor<T> min(const HipTensor<T>& t, int axis) { return reduce_axis(AM_RED_MIN, t, axis); }
+template <typename T> T max(const HipTensor<T>& t) { return reduce_all(AM_RED_MAX, t); }
+template <typename T> HipTensor<T> max(const HipTensor<T>& t, int axis) { return reduce_axis(AM_RED_MAX, t, axis); }
+// integers: C++ `/` truncates towards zero like Nim's `div`
+template <typename T> T mean(const HipTensor<T>& t) { return sum(t) / static_cast<T>(t.size()); }
+template <typename T> HipTensor<T> mean(const HipTensor<T>& t, int axis) {
+  HipTensor<T> s = sum(t, axis);
+  if (s.size() == 0) return s;
+  return scalar_op(AM_OP_DIV, s, static_cast<T>(t.shape[axis]));
+}
+
+// Row softmax of a [batch_size, number_of_classes] matrix (nnp_softmax.nim:18-38).
+template <typename T>
+HipTensor<T> softmax(const HipTensor<T>& t) {
+  static_assert(std::is_floating_point<T>::value, "softmax is defined for float tensors");
+  if (t.rank() != 2) throw std::invalid_argument("softmax: input must be [batch_size, number_of_classes]");
+  HipTensor<T> r(t.shape);
+  check(detail::softmax_(t.shape[0], t.shape[1], r.ptr(), r.strides[0], r.strides[1], t.ptr(), t.strides[0], t.strides[1]));
+  return r;
+}
+
+// maxpool2d (nnp_maxpooling.nim:19-66): values and the flat input index of each maximum.
+template <typename T> struct MaxPooled { HipTensor<int64_t> max_indices; HipTensor<T> maxpooled; };
+template <typename T>
+MaxPooled<T> maxpool2d(const HipTensor<T>& x, int kH, int kW, int padH = 0, int padW = 0, int strideH = 1, int strideW = 1) {
+  if (x.rank() != 4 || !x.is_C_contiguous()) throw std::invalid_argument("maxpool2d: input must be a C-contiguous [N, C, H, W] tensor");
+  const int64_t N = x.shape[0], C = x.shape[1], H = x.shape[2], W = x.shape[3];
+  const int64_t oh = (H + 2 * padH - kH) / strideH + 1, ow = (W + 2 * padW - kW) / strideW + 1;
+  MaxPooled<T> r{HipTensor<int64_t>(Shape{N * C * oh * ow}), HipTensor<T>(Shape{N, C, oh, ow})};
+  check(detail::maxpool2d_(N, (int)C, (int)H, (int)W, kH, kW, padH, padW, strideH, strideW, x.ptr(), r.maxpooled.ptr(),
+                           r.max_indices.ptr()));
   return r;
 }
 

@@ -95,6 +95,28 @@ proc am_hip_dot_f64*(n: int64, x: ptr cdouble, incx: int64, y: ptr cdouble, incy
 proc am_hip_dot_i32*(n: int64, x: ptr int32, incx: int64, y: ptr int32, incy: int64, res: ptr int32): cint {.importc.}
 proc am_hip_dot_i64*(n: int64, x: ptr int64, incx: int64, y: ptr int64, incy: int64, res: ptr int64): cint {.importc.}
 
+# reductions, softmax, pooling — reduce_axis_inline / reduce_inline (higher_order_foldreduce.nim:22-61),
+# softmax (nn_primitives/nnp_softmax.nim:18-38), maxpool2d (nn_primitives/nnp_maxpooling.nim:19-66)
+const
+  AM_RED_SUM* = 0.cint
+  AM_RED_PROD* = 1.cint
+  AM_RED_MIN* = 2.cint
+  AM_RED_MAX* = 3.cint
+proc am_hip_reduce_axis_f32*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr cfloat, dst_strides: ptr int64, a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
+proc am_hip_reduce_axis_f64*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr cdouble, dst_strides: ptr int64, a: ptr cdouble, a_strides: ptr int64): cint {.importc.}
+proc am_hip_reduce_axis_i32*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr int32, dst_strides: ptr int64, a: ptr int32, a_strides: ptr int64): cint {.importc.}
+proc am_hip_reduce_axis_i64*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr int64, dst_strides: ptr int64, a: ptr int64, a_strides: ptr int64): cint {.importc.}
+proc am_hip_reduce_all_f32*(op, rank: cint, shape: ptr int64, a: ptr cfloat, a_strides: ptr int64, res: ptr cfloat): cint {.importc.}
+proc am_hip_reduce_all_f64*(op, rank: cint, shape: ptr int64, a: ptr cdouble, a_strides: ptr int64, res: ptr cdouble): cint {.importc.}
+proc am_hip_reduce_all_i32*(op, rank: cint, shape: ptr int64, a: ptr int32, a_strides: ptr int64, res: ptr int32): cint {.importc.}
+proc am_hip_reduce_all_i64*(op, rank: cint, shape: ptr int64, a: ptr int64, a_strides: ptr int64, res: ptr int64): cint {.importc.}
+proc am_hip_softmax_rows_f32*(rows, cols: int64, dst: ptr cfloat, dst_rs, dst_cs: int64, src: ptr cfloat, src_rs, src_cs: int64): cint {.importc.}
+proc am_hip_softmax_rows_f64*(rows, cols: int64, dst: ptr cdouble, dst_rs, dst_cs: int64, src: ptr cdouble, src_rs, src_cs: int64): cint {.importc.}
+proc am_hip_maxpool2d_f32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cfloat, outp: ptr cfloat, argmax: ptr int64): cint {.importc.}
+proc am_hip_maxpool2d_f64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cdouble, outp: ptr cdouble, argmax: ptr int64): cint {.importc.}
+proc am_hip_maxpool2d_i32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr int32, outp: ptr int32, argmax: ptr int64): cint {.importc.}
+proc am_hip_maxpool2d_i64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr int64, outp: ptr int64, argmax: ptr int64): cint {.importc.}
+
 const
   AM_EPI_NONE* = 0.cint
   AM_EPI_BIAS* = 1.cint

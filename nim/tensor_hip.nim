@@ -328,3 +328,71 @@ proc linear*[T: float32 | float64](x, weight, bias: HipTensor[T], relu = false):
       wt.get_offset_ptr, int64 wt.strides[0], int64 wt.strides[1], 0'f64,
       result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
       epi, bb.get_offset_ptr, int64 bb.strides[0], int64 bb.strides[1])
+
+# ---------------------------------------------------------------- reductions, softmax, pooling
+proc reduce_axis[T: HipScalar](op: cint, t: HipTensor[T], axis: int): HipTensor[T] =
+  ## reduce_axis_inline (higher_order_foldreduce.nim:46-61): the result keeps `axis` with extent 1.
+  if axis < 0 or axis >= t.rank:
+    raise newException(IndexDefect, "Input tensor rank (" & $t.rank & ") must be greater than reduction axis (" & $axis & ")")
+  if t.size == 0: return newHipTensor[T](t.shape.toSeq)     # returnEmptyIfEmpty
+  var oshape = t.shape.toSeq
+  oshape[axis] = 1
+  result = newHipTensor[T](oshape)
+  var sh = i64s(t.shape)
+  var sd = i64s(result.strides)
+  var sa = i64s(t.strides)
+  when T is float32: check am_hip_reduce_axis_f32(op, cint t.rank, sh[0].addr, cint axis, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+  elif T is float64: check am_hip_reduce_axis_f64(op, cint t.rank, sh[0].addr, cint axis, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+  elif T is int32: check am_hip_reduce_axis_i32(op, cint t.rank, sh[0].addr, cint axis, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+  else: check am_hip_reduce_axis_i64(op, cint t.rank, sh[0].addr, cint axis, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+
+proc reduce_all[T: HipScalar](op: cint, t: HipTensor[T]): T =
+  ## reduce_inline (higher_order_foldreduce.nim:22-31), value returned to the host.
+  var sh = i64s(t.shape)
+  var sa = i64s(t.strides)
+  when T is float32: check am_hip_reduce_all_f32(op, cint t.rank, sh[0].addr, t.get_offset_ptr, sa[0].addr, result.addr)
+  elif T is float64: check am_hip_reduce_all_f64(op, cint t.rank, sh[0].addr, t.get_offset_ptr, sa[0].addr, result.addr)
+  elif T is int32: check am_hip_reduce_all_i32(op, cint t.rank, sh[0].addr, t.get_offset_ptr, sa[0].addr, result.addr)
+  else: check am_hip_reduce_all_i64(op, cint t.rank, sh[0].addr, t.get_offset_ptr, sa[0].addr, result.addr)
+
+# aggregate.nim:33-113
+proc sum*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_SUM, t)
+proc sum*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[T] = reduce_axis(AM_RED_SUM, t, axis)
+proc product*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_PROD, t)
+proc product*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[T] = reduce_axis(AM_RED_PROD, t, axis)
+proc min*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_MIN, t)
+proc min*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[T] = reduce_axis(AM_RED_MIN, t, axis)
+proc max*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_MAX, t)
+proc max*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[T] = reduce_axis(AM_RED_MAX, t, axis)
+proc mean*[T: int32 | int64](t: HipTensor[T]): T = t.sum div T(t.size)
+proc mean*[T: float32 | float64](t: HipTensor[T]): T = t.sum / T(t.size)
+proc mean*[T: int32 | int64](t: HipTensor[T], axis: int): HipTensor[T] = t.sum(axis) / T(t.shape[axis])   # opDiv truncates like `div` on integers
+proc mean*[T: float32 | float64](t: HipTensor[T], axis: int): HipTensor[T] = t.sum(axis) / T(t.shape[axis])
+
+proc softmax*[T: float32 | float64](input: HipTensor[T]): HipTensor[T] =
+  ## nn_primitives/nnp_softmax.nim:18-38 on a [batch_size, number_of_classes] matrix.
+  result = newHipTensor[T](input.shape.toSeq)
+  when T is float32:
+    check am_hip_softmax_rows_f32(int64 input.shape[0], int64 input.shape[1], result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
+      input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1])
+  else:
+    check am_hip_softmax_rows_f64(int64 input.shape[0], int64 input.shape[1], result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
+      input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1])
+
+proc maxpool2d*[T: HipScalar](input: HipTensor[T], kernel: tuple[height, width: int], padding = (0, 0), stride = (1, 1)):
+    tuple[max_indices: HipTensor[int64], maxpooled: HipTensor[T]] =
+  ## nn_primitives/nnp_maxpooling.nim:19-66 (the reference asserts a C-contiguous rank-4 input too).
+  assert input.rank == 4 and input.is_C_contiguous
+  let (N, C, H, W) = (input.shape[0], input.shape[1], input.shape[2], input.shape[3])
+  let outH = (H + 2 * padding[0] - kernel.height) div stride[0] + 1
+  let outW = (W + 2 * padding[1] - kernel.width) div stride[1] + 1
+  result.max_indices = newHipTensor[int64]([N * C * outH * outW])
+  result.maxpooled = newHipTensor[T]([N, C, outH, outW])
+  template call(f: untyped) =
+    check f(int64 N, cint C, cint H, cint W, cint kernel.height, cint kernel.width, cint padding[0], cint padding[1],
+            cint stride[0], cint stride[1], input.get_offset_ptr, result.maxpooled.get_offset_ptr, result.max_indices.get_offset_ptr)
+  when T is float32: call am_hip_maxpool2d_f32
+  elif T is float64: call am_hip_maxpool2d_f64
+  elif T is int32: call am_hip_maxpool2d_i32
+  else: call am_hip_maxpool2d_i64
+

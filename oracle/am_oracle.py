@@ -65,6 +65,19 @@ def lib() -> ctypes.CDLL:
             f = getattr(L, f"am_oracle_unary_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, p, p, p, p]
+            f = getattr(L, f"am_oracle_reduce_axis_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, ci, p, p, p, p]
+            f = getattr(L, f"am_oracle_reduce_all_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, p, p, p]
+            f = getattr(L, f"am_oracle_maxpool2d_{sfx}")
+            f.restype = ci
+            f.argtypes = [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, p, p, p, ct]
+        for sfx in ("f32", "f64"):
+            f = getattr(L, f"am_oracle_softmax_rows_{sfx}")
+            f.restype = ci
+            f.argtypes = [i64, i64, p, i64, i64, p, i64, i64]
         L.am_oracle_num_threads.restype = ci
         L.am_oracle_set_num_threads.argtypes = [ci]
         _lib = L
@@ -253,6 +266,77 @@ def conv2d(x: np.ndarray, kernel: np.ndarray, bias: np.ndarray | None, padding=(
 
 
 # ----------------------------------------------------------------------------- closed forms
+RED = {"sum": 0, "product": 1, "min": 2, "max": 3}
+
+
+def reduce_axis(op, a: np.ndarray, axis: int) -> np.ndarray:
+    """reduce_axis_inline (higher_order_foldreduce.nim:46-61): fold along `axis` starting from the
+    first slice; the result keeps the axis with extent 1. Any strides."""
+    sfx = _sfx(a)
+    if not 0 <= axis < a.ndim:
+        raise IndexError(f"axis {axis} outside rank {a.ndim}")
+    out_shape = list(a.shape)
+    out_shape[axis] = 1
+    out = np.empty(out_shape, dtype=a.dtype)
+    if a.size == 0:
+        return np.empty(a.shape, dtype=a.dtype)
+    rc = getattr(lib(), f"am_oracle_reduce_axis_{sfx}")(
+        RED[op], a.ndim, _i64arr(a.shape), axis, out.ctypes.data, _i64arr(_estrides(out)), a.ctypes.data, _i64arr(_estrides(a)))
+    if rc != 0:
+        raise ValueError(f"oracle reduce_axis failed ({rc})")
+    return out
+
+
+def reduce_all(op, a: np.ndarray):
+    """reduce_inline (higher_order_foldreduce.nim:22-31): C-order fold from the first element."""
+    sfx = _sfx(a)
+    if a.size == 0:
+        raise ValueError("reduction of an empty tensor")
+    res = np.empty(1, dtype=a.dtype)
+    rc = getattr(lib(), f"am_oracle_reduce_all_{sfx}")(RED[op], a.ndim, _i64arr(a.shape), a.ctypes.data, _i64arr(_estrides(a)), res.ctypes.data)
+    if rc != 0:
+        raise ValueError(f"oracle reduce_all failed ({rc})")
+    return res[0]
+
+
+def mean(a: np.ndarray, axis: int | None = None):
+    """aggregate.nim:58-80: sum divided by the element count; integers use `div` (truncation)."""
+    if axis is None:
+        s, n = reduce_all("sum", a), a.size
+    else:
+        s, n = reduce_axis("sum", a, axis), a.shape[axis]
+    if a.dtype.kind == "f":
+        return (s / a.dtype.type(n)).astype(a.dtype) if isinstance(s, np.ndarray) else a.dtype.type(s / a.dtype.type(n))
+    q = _trunc_div(np.asarray(s), np.asarray(n, dtype=a.dtype))
+    return q if axis is not None else q.dtype.type(q)
+
+
+def softmax(x: np.ndarray) -> np.ndarray:
+    """nnp_softmax.nim:18-38 on a [batch, classes] matrix (streaming max / sum of exponentials per
+    row, then exp(x - max) / sumexp)."""
+    sfx = _sfx(x)
+    assert x.ndim == 2 and sfx in ("f32", "f64")
+    out = np.empty(x.shape, dtype=x.dtype)
+    xs, os_ = _estrides(x), _estrides(out)
+    getattr(lib(), f"am_oracle_softmax_rows_{sfx}")(x.shape[0], x.shape[1], out.ctypes.data, os_[0], os_[1], x.ctypes.data, xs[0], xs[1])
+    return out
+
+
+def maxpool2d(x: np.ndarray, kernel, padding=(0, 0), stride=(1, 1)):
+    """nnp_maxpooling.nim:19-66: (max_indices [N*C*outH*outW] int64, maxpooled [N, C, outH, outW])."""
+    sfx = _sfx(x)
+    x = np.ascontiguousarray(x)
+    N, C, H, W = x.shape
+    outH = (H + 2 * padding[0] - kernel[0]) // stride[0] + 1
+    outW = (W + 2 * padding[1] - kernel[1]) // stride[1] + 1
+    out = np.empty((N, C, outH, outW), dtype=x.dtype)
+    idx = np.empty(N * C * outH * outW, dtype=np.int64)
+    lowest = -np.inf if x.dtype.kind == "f" else np.iinfo(x.dtype).min   # low(T)
+    getattr(lib(), f"am_oracle_maxpool2d_{sfx}")(N, C, H, W, kernel[0], kernel[1], padding[0], padding[1], stride[0], stride[1],
+                                                 x.ctypes.data, out.ctypes.data, idx.ctypes.data, _CT[sfx](lowest))
+    return idx, out
+
+
 def closed_gemm_int(alpha, A, B, beta, C):
     """Exact integer result of alpha*A*B + beta*C reduced modulo 2^w (w = bit width of the dtype).
     Ring arithmetic is order independent, so this fixes every bit of the result. Uses Python

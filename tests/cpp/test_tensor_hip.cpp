@@ -146,6 +146,51 @@ static void fused_linear() {
   CHECK(eq(am::relu(x), {1, 2, 3, 0, 0, 0}));
 }
 
+template <typename T>
+static void aggregates() {
+  // tests/tensor/test_aggregate.nim:20-84
+  auto t = toHip<T>({0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11}, {4, 3});
+  CHECK(am::sum(t) == T(66));
+  CHECK(eq(am::sum(t, 0), {18, 22, 26}));
+  CHECK(eq(am::sum(t, 1), {3, 12, 21, 30}));
+  CHECK(am::sum(t, 0).shape == (am::Shape{1, 3}) && am::sum(t, 1).shape == (am::Shape{4, 1}));
+  CHECK(am::product(t) == T(0));
+  auto a = toHip<T>({1, 2, 4, 8, 16, 32}, {2, 3});
+  CHECK(am::product(a) == T(32768));
+  CHECK(eq(am::product(a, 0), {8, 32, 128}));
+  CHECK(eq(am::product(a, 1), {8, 4096}));
+  auto v = toHip<T>({2, -1, 3, -3, 5, 0}, {6});
+  CHECK(am::min(v) == T(-3) && am::max(v) == T(5));
+  auto b = toHip<T>({1, 2, 3, -4, 0, 4, -2, 5}, {2, 4});
+  CHECK(eq(am::min(b, 0), {0, 2, -2, -4}));
+  CHECK(eq(am::min(b, 1), {-4, -2}));
+  CHECK(eq(am::max(b, 0), {1, 4, 3, 5}));
+  CHECK(eq(am::max(b, 1), {3, 5}));
+  CHECK(eq(am::sum(t.transpose(), 0), {3, 12, 21, 30}));
+  EXPECT_THROW(am::sum(t, 2), std::out_of_range);
+  if (std::is_floating_point<T>::value) {
+    CHECK(am::mean(t) == T(5.5));
+    CHECK(eq(am::mean(t, 0), {T(4.5), T(5.5), T(6.5)}));
+    CHECK(eq(am::mean(t, 1), {1, 4, 7, 10}));
+  } else {
+    CHECK(am::mean(t) == T(5));
+    CHECK(am::mean(toHip<T>({-7, 2, 1}, {3})) == T(-1));
+  }
+  // tests/nn_primitives/test_nnp_maxpool.nim:20-31
+  auto img = toHip<T>({1, 1, 2, 4, 5, 6, 7, 8, 3, 2, 1, 0, 1, 2, 3, 4}, {1, 1, 4, 4});
+  auto mp = am::maxpool2d(img, 2, 2, 0, 0, 2, 2);
+  CHECK(eq(mp.maxpooled, {6, 8, 3, 4}));
+  CHECK(mp.max_indices.toCpu() == (std::vector<int64_t>{5, 7, 8, 15}));
+}
+
+static void softmax_rows() {
+  auto x = toHip<double>({1, 2, 3, 1000, 1000, 1000}, {2, 3});
+  const std::vector<double> s = am::softmax(x).toCpu();
+  const double e1 = std::exp(1.0), e2 = std::exp(2.0), e3 = std::exp(3.0), z = e1 + e2 + e3;
+  CHECK(std::fabs(s[0] - e1 / z) < 1e-15 && std::fabs(s[1] - e2 / z) < 1e-15 && std::fabs(s[2] - e3 / z) < 1e-15);
+  CHECK(std::fabs(s[3] - 1.0 / 3) < 1e-15 && std::fabs(s[4] - 1.0 / 3) < 1e-15 && std::fabs(s[5] - 1.0 / 3) < 1e-15);
+}
+
 int main() {
   try {
     gemm_literals<float>();
@@ -159,6 +204,11 @@ int main() {
     broadcasting<int32_t>();
     broadcasting<int64_t>();
     fused_linear();
+    aggregates<float>();
+    aggregates<double>();
+    aggregates<int32_t>();
+    aggregates<int64_t>();
+    softmax_rows();
     am::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());

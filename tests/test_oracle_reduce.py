@@ -1,0 +1,153 @@
+"""Pins the CPU restatement of reductions, softmax and max pooling (oracle/reduce_pool.c):
+the reference's literal vectors, then NumPy / exact arithmetic on random strided inputs."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from conftest import DTYPES, seed_of, view_of, VIEW_KINDS, PARENT_SHAPE
+
+NP_OPS = {"sum": np.add, "product": np.multiply, "min": np.minimum, "max": np.maximum}
+
+
+@pytest.mark.parametrize("sfx", list(DTYPES))
+def test_reference_aggregate_vectors(vectors, oracle, sfx):
+    g = vectors["aggregate"]
+    dt = DTYPES[sfx]
+    t = np.array(g["t"], dtype=dt)
+    assert oracle.reduce_all("sum", t) == g["sum"]
+    assert np.array_equal(oracle.reduce_axis("sum", t, 0), np.array(g["sum_axis0"], dtype=dt))
+    assert np.array_equal(oracle.reduce_axis("sum", t, 1), np.array(g["sum_axis1"], dtype=dt))
+    assert oracle.reduce_all("product", t) == g["product_t"]
+    a = np.array(g["a"], dtype=dt)
+    assert oracle.reduce_all("product", a) == g["product_a"]
+    assert np.array_equal(oracle.reduce_axis("product", a, 0), np.array(g["product_a_axis0"], dtype=dt))
+    assert np.array_equal(oracle.reduce_axis("product", a, 1), np.array(g["product_a_axis1"], dtype=dt))
+    v, b = np.array(g["v"], dtype=dt), np.array(g["b"], dtype=dt)
+    assert oracle.reduce_all("min", v) == g["min_v"] and oracle.reduce_all("max", v) == g["max_v"]
+    for op in ("min", "max"):
+        for ax in (0, 1):
+            assert np.array_equal(oracle.reduce_axis(op, b, ax), np.array(g[f"{op}_b_axis{ax}"], dtype=dt))
+    if np.dtype(dt).kind == "f":
+        assert oracle.mean(t) == g["mean_float"]
+        assert np.array_equal(oracle.mean(t, 0), np.array(g["mean_axis0"], dtype=dt))
+        assert np.array_equal(oracle.mean(t, 1), np.array(g["mean_axis1"], dtype=dt))
+
+
+def test_reference_maxpool_vectors(vectors, oracle):
+    g = vectors["maxpool"]
+    for dt in DTYPES.values():
+        x = np.array(g["input"], dtype=dt).reshape(g["input_shape"])
+        idx, pooled = oracle.maxpool2d(x, g["kernel"], g["padding"], g["stride"])
+        assert np.array_equal(pooled, np.array(g["pooled"], dtype=dt).reshape(g["pooled_shape"]))
+        assert np.array_equal(idx, np.array(g["max_indices"], dtype=np.int64))
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+@pytest.mark.parametrize("kind", VIEW_KINDS)
+def test_integer_reductions_against_numpy(oracle, sfx, kind):
+    """Wrapping sums / products and min / max of integer views: NumPy's ufunc.reduce wraps the same
+    way and is order independent for these operations."""
+    dt = DTYPES[sfx]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(seed_of("red-int", sfx, kind))
+    shape = (13, 21)
+    parent = rng.integers(info.min, info.max, size=PARENT_SHAPE[kind](*shape), endpoint=True).astype(dt)
+    v = view_of(parent, kind, shape)
+    for op, uf in NP_OPS.items():
+        with np.errstate(over="ignore"):
+            assert oracle.reduce_all(op, v) == uf.reduce(v, axis=None, dtype=dt)
+            for ax in range(v.ndim):
+                assert np.array_equal(oracle.reduce_axis(op, v, ax), uf.reduce(v, axis=ax, dtype=dt, keepdims=True)), (op, ax)
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_float_sum_is_the_serial_fold(oracle, sfx):
+    """A float sum is pinned by its order: the restatement must equal a left-to-right Python fold
+    in the tensor's own precision, element order = C order of the view (not of memory)."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("fold", sfx))
+    parent = rng.uniform(-1, 1, (7, 9, 5)).astype(dt)
+    for v in (parent, parent.transpose(2, 0, 1), parent[::2, ::-1, 1:4]):
+        acc = None
+        for x in v.reshape(-1):          # reshape of a view copies in C order
+            acc = x if acc is None else dt(acc + x)
+        assert oracle.reduce_all("sum", v) == acc
+        for ax in range(3):
+            want = np.take(v, 0, axis=ax).copy()
+            for l in range(1, v.shape[ax]):
+                want = (want + np.take(v, l, axis=ax)).astype(dt)
+            assert np.array_equal(oracle.reduce_axis("sum", v, ax), np.expand_dims(want, ax))
+
+
+def test_float_sum_close_to_exact(oracle):
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, 2000)
+    exact = sum(Fraction(float(v)) for v in x)
+    assert abs(Fraction(float(oracle.reduce_all("sum", x))) - exact) < Fraction(1, 10**12)
+
+
+def test_integer_mean_truncates(oracle):
+    for dt in (np.int32, np.int64):
+        assert oracle.mean(np.array([-7, 2, 1], dtype=dt)) == -1          # -4 div 3
+        assert oracle.mean(np.array([7, -2, -1], dtype=dt)) == 1
+        m = oracle.mean(np.array([[-7, 5], [2, 2]], dtype=dt), 0)
+        assert np.array_equal(m, np.array([[-2, 3]], dtype=dt))           # -5 div 2 = -2
+
+
+def test_empty_and_bad_axis(oracle):
+    e = np.empty((0, 3), dtype=np.float32)
+    assert oracle.reduce_axis("sum", e, 0).shape == (0, 3)               # returnEmptyIfEmpty
+    with pytest.raises(ValueError):
+        oracle.reduce_all("sum", e)
+    with pytest.raises(IndexError):
+        oracle.reduce_axis("sum", np.zeros((2, 2), np.float32), 2)
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_softmax_closed_form(oracle, sfx):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("softmax", sfx))
+    x = (rng.standard_normal((9, 37)) * 5).astype(dt)
+    got = oracle.softmax(x)
+    xl = x.astype(np.longdouble)
+    e = np.exp(xl - xl.max(1, keepdims=True))
+    want = e / e.sum(1, keepdims=True)
+    tol = 5e-7 if sfx == "f32" else 1e-15
+    assert np.max(np.abs(got - want) / want) < tol * 10
+    assert np.allclose(got.sum(1), 1, atol=tol * 40)
+    # shift invariance (exact up to rounding of x + c) and large magnitudes without overflow
+    assert np.allclose(oracle.softmax((x + dt(3)).astype(dt)), got, rtol=1e-4 if sfx == "f32" else 1e-12)
+    big = np.array([[1000, 1001, 999], [-1000, -1001, -999]], dtype=dt)
+    sb = oracle.softmax(big)
+    assert np.all(np.isfinite(sb)) and np.allclose(sb[0], sb[1][[0, 1, 2]] if False else sb[0])
+    # strided input (transposed view)
+    xt = np.ascontiguousarray(x.T).T
+    assert np.array_equal(oracle.softmax(xt), got)
+
+
+@pytest.mark.parametrize("sfx", list(DTYPES))
+def test_maxpool_against_bruteforce(oracle, sfx):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("maxpool", sfx))
+    x = rng.integers(-50, 50, (2, 3, 7, 9)).astype(dt)
+    for kernel, pad, stride in [((2, 2), (0, 0), (2, 2)), ((3, 3), (1, 1), (1, 1)), ((3, 2), (1, 0), (2, 3)), ((2, 2), (2, 2), (1, 1))]:
+        idx, out = oracle.maxpool2d(x, kernel, pad, stride)
+        low = -np.inf if np.dtype(dt).kind == "f" else np.iinfo(dt).min
+        N, C, H, W = x.shape
+        oh, ow = out.shape[2:]
+        flat = x.reshape(-1)
+        for n in range(N):
+            for c in range(C):
+                for h in range(oh):
+                    for w in range(ow):
+                        best, arg = low, np.iinfo(np.int64).min
+                        for ph in range(kernel[0]):
+                            for pw in range(kernel[1]):
+                                r, q = h * stride[0] + ph - pad[0], w * stride[1] + pw - pad[1]
+                                if 0 <= r < H and 0 <= q < W and x[n, c, r, q] > best:
+                                    best, arg = x[n, c, r, q], q + W * (r + H * (c + n * C))
+                        o = w + ow * (h + oh * (c + n * C))
+                        assert out[n, c, h, w] == best and idx[o] == arg
+                        if arg >= 0:
+                            assert flat[arg] == best

@@ -1,0 +1,224 @@
+"""Reductions, row softmax and max pooling on the GPU through the C ABI: the reference's literal
+vectors, oracle parity on strided views of every rank, chunked long axes, edge cases.
+
+Bars: integers bit-exact (wrapping sums and products are order independent); float min / max
+bit-exact; float sums along a non-unit-stride axis bit-exact (one lane folds the axis in the
+reference's order); float sums that the device reassociates (unit-stride axis, whole tensor) within
+1e-5 (f32) / 1e-13 (f64) of the serial fold relative to sum(|x|); softmax within 8e-6 / 4e-14
+relative per element of the closed form; pooling identical values and indices."""
+import numpy as np
+import pytest
+
+from conftest import DTYPES, seed_of
+
+pytestmark = pytest.mark.gpu
+ALL = ["f32", "f64", "i32", "i64"]
+SUM_TOL = {"f32": 1e-5, "f64": 1e-13}
+OPS = ["sum", "product", "min", "max"]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def fill(rng, shape, dt, op="sum"):
+    if np.dtype(dt).kind == "f":
+        if op == "product":      # keep products finite and away from zero
+            return rng.uniform(0.9, 1.1, size=shape).astype(dt) * rng.choice([-1, 1], size=shape).astype(dt)
+        return rng.uniform(-1, 1, size=shape).astype(dt)
+    info = np.iinfo(dt)
+    return rng.integers(info.min, info.max, size=shape, endpoint=True).astype(dt)
+
+
+def close(sfx, op, got, want, ref_abs):
+    """got vs the serial fold `want`; ref_abs = fold of |x| (scale of the rounding error)."""
+    if sfx in ("i32", "i64") or op in ("min", "max"):
+        return np.array_equal(got, want)
+    if op == "product":
+        return np.allclose(got, want, rtol=1e-4 if sfx == "f32" else 1e-12)
+    return np.all(np.abs(np.asarray(got, dtype=np.float64) - np.asarray(want, dtype=np.float64)) <= SUM_TOL[sfx] * np.asarray(ref_abs, dtype=np.float64))
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_reference_aggregate_vectors(hip, vectors, sfx):
+    g = vectors["aggregate"]
+    dt = DTYPES[sfx]
+    t = hip.toHip(np.array(g["t"], dtype=dt))
+    assert hip.sum(t) == g["sum"]
+    assert np.array_equal(hip.sum(t, axis=0).toCpu(), np.array(g["sum_axis0"], dtype=dt))
+    assert np.array_equal(hip.sum(t, axis=1).toCpu(), np.array(g["sum_axis1"], dtype=dt))
+    assert hip.product(t) == g["product_t"]
+    a = hip.toHip(np.array(g["a"], dtype=dt))
+    assert hip.product(a) == g["product_a"]
+    assert np.array_equal(hip.product(a, 0).toCpu(), np.array(g["product_a_axis0"], dtype=dt))
+    assert np.array_equal(hip.product(a, 1).toCpu(), np.array(g["product_a_axis1"], dtype=dt))
+    v, b = hip.toHip(np.array(g["v"], dtype=dt)), hip.toHip(np.array(g["b"], dtype=dt))
+    assert hip.min(v) == g["min_v"] and hip.max(v) == g["max_v"]
+    for op in ("min", "max"):
+        for ax in (0, 1):
+            assert np.array_equal(getattr(hip, op)(b, ax).toCpu(), np.array(g[f"{op}_b_axis{ax}"], dtype=dt))
+    if np.dtype(dt).kind == "f":
+        assert hip.mean(t) == g["mean_float"]
+        assert np.array_equal(hip.mean(t, 0).toCpu(), np.array(g["mean_axis0"], dtype=dt))
+        assert np.array_equal(hip.mean(t, 1).toCpu(), np.array(g["mean_axis1"], dtype=dt))
+    else:
+        assert hip.mean(t) == 5                                    # 66 div 12
+        assert hip.mean(hip.toHip(np.array([-7, 2, 1], dtype=dt))) == -1
+        assert np.array_equal(hip.mean(hip.toHip(np.array([[-7, 5], [2, 2]], dtype=dt)), 0).toCpu(), np.array([[-2, 3]], dtype=dt))
+
+
+def views(x):
+    """(name, numpy view, function producing the same view of a HipTensor)."""
+    out = [("C", x, lambda d: d)]
+    if x.ndim >= 2:
+        perm = tuple(range(x.ndim - 1, -1, -1))
+        out.append(("reversed-axes", x.transpose(perm), lambda d: d.transpose() if d.rank == 2 else None))
+    sl = tuple(slice(None, None, 2) if i % 2 == 0 else slice(1, None) for i in range(x.ndim))
+    out.append(("stepped", x[sl], lambda d: d[sl]))
+    neg = tuple(slice(None, None, -1) for _ in range(x.ndim))
+    out.append(("negative", x[neg], lambda d: d[neg]))
+    return out
+
+
+SHAPES = [(1,), (63,), (64,), (1000,), (5, 7), (64, 64), (1, 300), (300, 1), (129, 257), (7, 5, 9), (3, 4, 5, 6), (2, 3, 2, 3, 2, 3)]
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("shape", SHAPES)
+def test_reductions_vs_oracle(hip, oracle, sfx, shape):
+    dt = DTYPES[sfx]
+    for op in OPS:
+        rng = np.random.default_rng(seed_of("reduce", sfx, shape, op))
+        x = fill(rng, shape, dt, op)
+        dx = hip.toHip(x)
+        for name, v, mk in views(x):
+            dv = mk(dx)
+            if dv is None or v.size == 0:
+                continue
+            say("reduce", sfx, shape, op, name)
+            assert dv.shape == v.shape
+            absv = np.abs(v)
+            assert close(sfx, op, getattr(hip, op)(dv), oracle.reduce_all(op, v), oracle.reduce_all("sum", absv) if op == "sum" else None), (op, name, "all")
+            for ax in range(v.ndim):
+                got = getattr(hip, op)(dv, ax).toCpu()
+                want = oracle.reduce_axis(op, v, ax)
+                assert got.shape == want.shape
+                assert close(sfx, op, got, want, oracle.reduce_axis("sum", absv, ax) if op == "sum" else None), (op, name, ax)
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_sum_over_non_unit_stride_axis_is_the_serial_fold(hip, oracle, sfx):
+    """Sum over the leading axis of a row-major tensor with enough outputs to fill the chip on their
+    own (no chunking of the axis): one lane per output walks the axis in order, so the result equals
+    the CPU's serial fold bit for bit. (With few outputs the axis is cut up and the sum is
+    reassociated: covered with a tolerance by the other tests.)"""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("rowsum", sfx))
+    for shape in [(64, 200_000), (300, 150_000), (20, 400, 500), (63, 131_072)]:
+        x = rng.uniform(-1, 1, shape).astype(dt)
+        say("serial-order sum", sfx, shape)
+        assert np.array_equal(hip.sum(hip.toHip(x), 0).toCpu(), oracle.reduce_axis("sum", x, 0))
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_long_axes_are_chunked(hip, oracle, sfx):
+    """Few outputs, long axis: the axis is cut into chunks folded by a second pass."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("chunked", sfx))
+    for shape, ax in [((3, 1 << 20), 1), ((1 << 20, 3), 0), ((1, 3_000_001), 1), ((200_000, 17), 0), ((2, 70_000, 2), 1)]:
+        x = fill(rng, shape, dt)
+        dx = hip.toHip(x)
+        for op in ("sum", "max"):
+            say("chunked", sfx, shape, ax, op)
+            got = getattr(hip, op)(dx, ax).toCpu()
+            want = oracle.reduce_axis(op, x, ax)
+            assert close(sfx, op, got, want, oracle.reduce_axis("sum", np.abs(x), ax))
+            assert close(sfx, op, getattr(hip, op)(dx), oracle.reduce_all(op, x), oracle.reduce_all("sum", np.abs(x)))
+
+
+@pytest.mark.parametrize("sfx", ["f32", "i32"])
+def test_full_size_sum_8192(hip, oracle, sfx):
+    """8192 x 8192: column sums, row sums and the total, against the oracle; and the total as the
+    sum of the column sums computed on the device (two different kernels agree)."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("sum8192", sfx))
+    x = fill(rng, (8192, 8192), dt) if sfx == "i32" else rng.uniform(0, 1, (8192, 8192)).astype(dt)
+    dx = hip.toHip(x)
+    say("8192 col sums", sfx)
+    cols = hip.sum(dx, 0)
+    assert close(sfx, "sum", cols.toCpu(), oracle.reduce_axis("sum", x, 0), oracle.reduce_axis("sum", np.abs(x), 0))
+    say("8192 row sums", sfx)
+    rows = hip.sum(dx, 1)
+    assert close(sfx, "sum", rows.toCpu(), oracle.reduce_axis("sum", x, 1), oracle.reduce_axis("sum", np.abs(x), 1))
+    say("8192 total", sfx)
+    total = hip.sum(dx)
+    if sfx == "i32":
+        assert total == hip.sum(cols) == hip.sum(rows) == oracle.reduce_all("sum", x)
+    else:
+        exact = float(np.sum(x, dtype=np.float64))
+        for t in (total, hip.sum(cols), hip.sum(rows)):
+            assert abs(float(t) - exact) <= 1e-5 * exact
+
+
+def test_edge_cases(hip):
+    e = hip.empty((0, 3), np.float32)
+    assert hip.sum(e, 0).shape == (0, 3)                       # returnEmptyIfEmpty
+    with pytest.raises(ValueError):
+        hip.sum(e)                                             # nothing to start the fold from
+    with pytest.raises(IndexError):
+        hip.sum(hip.zeros((2, 2), np.float32), 2)
+    z = hip.toHip(np.array([-0.0, -0.0, -0.0] * 50, dtype=np.float32))
+    assert np.signbit(hip.sum(z)) and np.signbit(hip.sum(z.reshape(3, 50), 1).toCpu()).all()   # no +0 identity mixed in
+    one = hip.toHip(np.array([[4.5]], dtype=np.float64))
+    assert hip.sum(one) == 4.5 and hip.max(one, 0).toCpu()[0, 0] == 4.5
+    inf = hip.toHip(np.array([1.0, np.inf, -3.0], dtype=np.float32))
+    assert hip.max(inf) == np.inf and hip.min(inf) == -3.0
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_softmax_vs_oracle(hip, oracle, sfx):
+    dt = DTYPES[sfx]
+    tol = 2e-6 if sfx == "f32" else 1e-14
+    rng = np.random.default_rng(seed_of("softmax-gpu", sfx))
+    for shape in [(1, 1), (3, 5), (64, 10), (256, 1000), (7, 4096), (5, 4097), (3, 50_000), (1000, 3)]:
+        x = (rng.standard_normal(shape) * 4).astype(dt)
+        say("softmax", sfx, shape)
+        want = oracle.softmax(x)
+        got = hip.softmax(hip.toHip(x)).toCpu()
+        # closed form in extended precision: the tight bar
+        xl = x.astype(np.longdouble)
+        e = np.exp(xl - xl.max(1, keepdims=True))
+        exact = e / e.sum(1, keepdims=True)
+        assert np.max(np.abs(got - exact) / exact) <= tol * 4, shape
+        # the oracle sums the row serially in the tensor's precision: its own rounding error grows
+        # with the row length, so the bar against it does too
+        assert np.max(np.abs(got - want) / want) <= max(tol * 8, shape[1] * np.finfo(dt).eps), shape
+        assert np.allclose(got.sum(1), 1, atol=1e-5 if sfx == "f32" else 1e-13)
+        # transposed view in (strided path of the kernel), same values out up to the order of the row sum
+        xt = hip.toHip(np.ascontiguousarray(x.T)).transpose()
+        assert np.max(np.abs(hip.softmax(xt).toCpu() - exact) / exact) <= tol * 4, shape
+    big = np.array([[1000, 1001, 999], [-1000, -1001, -999]], dtype=dt)
+    assert np.allclose(hip.softmax(hip.toHip(big)).toCpu(), oracle.softmax(big), rtol=tol * 8)
+    with pytest.raises(TypeError):
+        hip.softmax(hip.zeros((2, 2), np.int32))
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_maxpool_vs_oracle(hip, oracle, vectors, sfx):
+    dt = DTYPES[sfx]
+    g = vectors["maxpool"]
+    x = np.array(g["input"], dtype=dt).reshape(g["input_shape"])
+    idx, pooled = hip.maxpool2d(hip.toHip(x), g["kernel"], g["padding"], g["stride"])
+    assert np.array_equal(pooled.toCpu(), np.array(g["pooled"], dtype=dt).reshape(g["pooled_shape"]))
+    assert np.array_equal(idx.toCpu(), np.array(g["max_indices"], dtype=np.int64))
+    rng = np.random.default_rng(seed_of("maxpool-gpu", sfx))
+    cases = [((2, 3, 7, 9), (2, 2), (0, 0), (2, 2)), ((4, 20, 24, 24), (2, 2), (0, 0), (2, 2)), ((3, 5, 13, 11), (3, 3), (1, 1), (1, 1)),
+             ((2, 2, 9, 8), (3, 2), (1, 0), (2, 3)), ((1, 1, 5, 5), (2, 2), (2, 2), (1, 1)), ((64, 50, 8, 8), (2, 2), (0, 0), (2, 2))]
+    for shape, kernel, pad, stride in cases:
+        x = rng.integers(-5, 5, shape).astype(dt)        # ties are frequent: the first maximum must win
+        say("maxpool", sfx, shape, kernel, pad, stride)
+        want_idx, want = oracle.maxpool2d(x, kernel, pad, stride)
+        idx, got = hip.maxpool2d(hip.toHip(x), kernel, pad, stride)
+        assert np.array_equal(got.toCpu(), want) and np.array_equal(idx.toCpu(), want_idx)
+    with pytest.raises(ValueError):
+        hip.maxpool2d(hip.zeros((2, 3, 4, 4), dt).transpose() if False else hip.zeros((4, 4), dt), (2, 2))
