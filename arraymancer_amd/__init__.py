@@ -7,6 +7,7 @@ does, and raises if it is missing (there is no CPU fallback).
 """
 from ._lib import HipAllocError, HipError, load as load_library
 from .metadata import Layout, Step
+from .io_npy import read_npy, write_npy
 from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3, map3, bc_add, bc_div, bc_mod, bc_mul,
                          bc_sub, bias_relu, conv2d, dot, empty, gemm, gemm_batched, gemv, im2col, linear, map2, matmul, relu, scalar_op,
                          sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
@@ -17,5 +18,5 @@ __all__ = [
     "toHip", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "conv2d", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
     "unary", "relu", "sigmoid", "bias_relu", "bc_add", "bc_sub", "bc_mul", "bc_div", "bc_mod",
     "reduce_axis", "reduce_all", "sum", "product", "min", "max", "mean", "softmax", "maxpool2d",
-    "load_library",
+    "read_npy", "write_npy", "load_library",
 ]

@@ -701,7 +701,7 @@ def maxpool2d(x: HipTensor, kernel, padding=(0, 0), stride=(1, 1)):
     """(max_indices, maxpooled) of a C-contiguous [N, C, H, W] tensor
     (src/arraymancer/nn_primitives/nnp_maxpooling.nim:19-66; the reference asserts contiguity too).
     max_indices is a device int64 vector of flat input indices."""
-    if x.rank != 4 or not x.is_C_contiguous:
+    if x.rank != 4 or not x.is_C_contiguous():
         raise ValueError("maxpool2d: input must be a C-contiguous [N, C, H, W] tensor")
     N, C, H, W = x.shape
     (kh, kw), (ph, pw), (sh, sw) = kernel, padding, stride

@@ -22,6 +22,8 @@
 #pragma once
 #include <cstdint>
 #include <cstdlib>
+#include <cstring>
+#include <fstream>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -162,6 +164,14 @@ class HipTensor {
   bool is_C_contiguous() const {
     int64_t cur = 1;
     for (int i = rank() - 1; i >= 0; --i) {
+      if (shape[i] != 1 && strides[i] != cur) return false;
+      cur *= shape[i];
+    }
+    return true;
+  }
+  bool is_F_contiguous() const {
+    int64_t cur = 1;
+    for (int i = 0; i < rank(); ++i) {
       if (shape[i] != 1 && strides[i] != cur) return false;
       cur *= shape[i];
     }
@@ -453,6 +463,107 @@ MaxPooled<T> maxpool2d(const HipTensor<T>& x, int kH, int kW, int padH = 0, int 
   check(detail::maxpool2d_(N, (int)C, (int)H, (int)W, kH, kW, padH, padW, strideH, strideW, x.ptr(), r.maxpooled.ptr(),
                            r.max_indices.ptr()));
   return r;
+}
+
+// ---- .npy files (src/arraymancer/io/io_npy.nim:64-183) -----------------------------------------
+namespace detail {
+template <typename S, typename T>
+inline void npy_convert(const unsigned char* raw, size_t n, bool big_endian, std::vector<T>& out) {
+  out.resize(n);
+  for (size_t i = 0; i < n; ++i) {
+    unsigned char b[sizeof(S)];
+    for (size_t k = 0; k < sizeof(S); ++k) b[k] = raw[i * sizeof(S) + (big_endian ? sizeof(S) - 1 - k : k)];   // to little endian
+    S v;
+    std::memcpy(&v, b, sizeof(S));
+    out[i] = static_cast<T>(v);   // `stream.readXxx.T`: float -> integer truncates
+  }
+}
+}  // namespace detail
+
+// read_npy[T](path): versions 1.0 / 2.0; <f4 >f4 <f8 >f8 <i4 >i4 <i8 >i8 <u4 >u4 <u8 >u8 converted
+// element by element to T; a Fortran-ordered file gives a column-major tensor.
+template <typename T>
+HipTensor<T> read_npy(const std::string& path) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) throw std::ios_base::failure(".npy file \"" + path + "\" does not exist");
+  char magic[8];
+  f.read(magic, 8);
+  if (f.gcount() != 8 || std::memcmp(magic, "\x93NUMPY", 6) != 0) throw std::invalid_argument("This file is not a Numpy file");
+  const int major = (unsigned char)magic[6], minor = (unsigned char)magic[7];
+  if (!((major == 1 || major == 2) && minor == 0)) throw std::invalid_argument("Unsupported .npy format: only 1.0 or 2.0 files can be loaded");
+  unsigned char lb[4] = {0, 0, 0, 0};
+  f.read((char*)lb, major == 1 ? 2 : 4);
+  const size_t header_len = (size_t)lb[0] | ((size_t)lb[1] << 8) | ((size_t)lb[2] << 16) | ((size_t)lb[3] << 24);
+  std::string header(header_len, '\0');
+  f.read(&header[0], (std::streamsize)header_len);
+  auto field = [&](const std::string& key, const std::string& until) {
+    const size_t a = header.find(key);
+    if (a == std::string::npos) throw std::invalid_argument("Error while parsing .npy header " + header);
+    const size_t b = header.find(until, a + key.size());
+    if (b == std::string::npos) throw std::invalid_argument("Error while parsing .npy header " + header);
+    return header.substr(a + key.size(), b - a - key.size());
+  };
+  const std::string descr = field("'descr': '", "'"), fortran = field("'fortran_order': ", ","), shp = field("'shape': (", ")");
+  if (fortran != "False" && fortran != "True") throw std::invalid_argument("Invalid token '" + fortran + "' in numpy description " + header);
+  Shape shape;
+  for (size_t i = 0; i < shp.size();) {
+    if (shp[i] == ' ' || shp[i] == ',') { ++i; continue; }
+    if (shp[i] < '0' || shp[i] > '9') throw std::invalid_argument(std::string("Invalid token '") + shp[i] + "' in numpy shape (" + shp + ")");
+    int64_t v = 0;
+    while (i < shp.size() && shp[i] >= '0' && shp[i] <= '9') v = v * 10 + (shp[i++] - '0');
+    shape.push_back(v);
+  }
+  if (descr.size() != 3 || (descr[0] != '<' && descr[0] != '>') || std::string("fiu").find(descr[1]) == std::string::npos ||
+      (descr[2] != '4' && descr[2] != '8'))
+    throw std::invalid_argument("Numpy type not supported: " + descr + " in file.");
+  size_t n = 1;
+  for (auto e : shape) n *= (size_t)e;
+  const size_t width = (size_t)(descr[2] - '0');
+  std::vector<unsigned char> raw(n * width);
+  f.read((char*)raw.data(), (std::streamsize)raw.size());
+  if ((size_t)f.gcount() != raw.size()) throw std::invalid_argument("truncated .npy file " + path);
+  const bool be = descr[0] == '>';
+  std::vector<T> host;
+  if (descr[1] == 'f' && width == 4) detail::npy_convert<float, T>(raw.data(), n, be, host);
+  else if (descr[1] == 'f') detail::npy_convert<double, T>(raw.data(), n, be, host);
+  else if (descr[1] == 'i' && width == 4) detail::npy_convert<int32_t, T>(raw.data(), n, be, host);
+  else if (descr[1] == 'i') detail::npy_convert<int64_t, T>(raw.data(), n, be, host);
+  else if (width == 4) detail::npy_convert<uint32_t, T>(raw.data(), n, be, host);
+  else detail::npy_convert<uint64_t, T>(raw.data(), n, be, host);
+  if (fortran == "False") return toHip(host, shape);
+  // column-major sequence in the file: upload as is, describe with column-major strides
+  HipTensor<T> t = toHip(host, Shape{(int64_t)n});
+  t.shape = shape;
+  t.strides.assign(shape.size(), 0);
+  int64_t acc = 1;
+  for (size_t i = 0; i < shape.size(); ++i) { t.strides[i] = acc; acc *= shape[i]; }
+  return t;
+}
+
+// t.write_npy(path): a contiguous copy, in Fortran order when the tensor is column-major, version
+// 1.0 header (2.0 past 16 bits) padded so that the data starts on a 16-byte boundary: the same
+// bytes NumPy's own writer produced for the reference's test files. Little-endian hosts.
+template <typename T>
+void write_npy(const HipTensor<T>& t, const std::string& path) {
+  if (t.rank() == 0) throw std::invalid_argument("write_npy: rank-0 tensors are not supported");
+  const bool fortran = t.rank() > 1 && t.is_F_contiguous() && !t.is_C_contiguous();
+  const std::vector<T> host = fortran ? t.transpose().toCpu() : t.toCpu();   // column-major sequence = C order of the transpose
+  std::string header = std::string("{'descr': '<") + (std::is_floating_point<T>::value ? "f" : "i") + std::to_string(sizeof(T)) +
+                       "', 'fortran_order': " + (fortran ? "True" : "False") + ", 'shape': (";
+  for (int i = 0; i < t.rank(); ++i) header += (i ? ", " : "") + std::to_string(t.shape[i]);
+  header += t.rank() == 1 ? ",), }" : "), }";
+  size_t meta = 6 + 4 + header.size() + 1;
+  const bool v1 = meta <= 0xFFFF;
+  if (!v1) meta += 2;
+  header += std::string((16 - (meta & 15)) & 15, ' ') + "\n";
+  std::ofstream f(path, std::ios::binary | std::ios::trunc);
+  if (!f) throw std::ios_base::failure("cannot open " + path + " for writing");
+  f.write("\x93NUMPY", 6);
+  const size_t hl = header.size();
+  if (v1) { const unsigned char b[4] = {1, 0, (unsigned char)(hl & 255), (unsigned char)(hl >> 8)}; f.write((const char*)b, 4); }
+  else { const unsigned char b[6] = {2, 0, (unsigned char)(hl & 255), (unsigned char)((hl >> 8) & 255), (unsigned char)((hl >> 16) & 255), (unsigned char)(hl >> 24)}; f.write((const char*)b, 6); }
+  f.write(header.data(), (std::streamsize)hl);
+  f.write((const char*)host.data(), (std::streamsize)(host.size() * sizeof(T)));
 }
 
 inline void sync() { check(am_hip_sync()); }

@@ -18,6 +18,9 @@ import arraymancer/laser/tensor/datatypes          # Tensor[T], KnownSupportsCop
 import arraymancer/tensor/data_structure            # shape_to_strides, is_C_contiguous, get_offset_ptr
 import arraymancer/tensor/init_cpu                  # newTensorUninit
 import arraymancer/tensor/shapeshifting             # asContiguous (host side, upload only)
+import arraymancer/io/io_npy                        # read_npy / write_npy on host tensors
+import arraymancer/tensor/private/p_display         # prettyImpl
+import std/typetraits                               # type names for `pretty`
 
 type
   HipScalar* = float32 | float64 | int32 | int64
@@ -395,4 +398,24 @@ proc maxpool2d*[T: HipScalar](input: HipTensor[T], kernel: tuple[height, width: 
   elif T is float64: call am_hip_maxpool2d_f64
   elif T is int32: call am_hip_maxpool2d_i32
   else: call am_hip_maxpool2d_i64
+
+# ---------------------------------------------------------------- .npy files and display
+# The file parsing and the pretty printer are the reference's own host code (io/io_npy.nim:64-183,
+# tensor/private/p_display.nim); the device tensor goes through a host copy, exactly as
+# display_cuda.nim:19-36 does for CudaTensor.
+proc read_npy_hip*[T: HipScalar](npyPath: string): HipTensor[T] =
+  read_npy[T](npyPath).toHip
+
+proc write_npy*[T: HipScalar](t: HipTensor[T], npyPath: string) =
+  t.toCpu.write_npy(npyPath)
+
+proc pretty*[T](t: HipTensor[T], precision = -1): string =
+  var desc = t.type.name & " of shape \"" & $t.shape & "\" on backend \"" & "Hip" & "\""
+  if t.storage.isNil: return "Uninitialized " & $desc
+  let cpu_t = t.toCpu
+  if cpu_t.size() == 0: return desc & "\n    [] (empty)"
+  elif cpu_t.rank == 1: return desc & "\n    " & cpu_t.prettyImpl(precision = precision)
+  else: return desc & "\n" & cpu_t.prettyImpl(precision = precision)
+
+proc `$`*[T](t: HipTensor[T]): string = t.pretty()
 

@@ -6,6 +6,9 @@
 // Exit code 0 = every check passed. Needs an MI355X; run by tests/test_cpp_host_gpu.py.
 #include <cmath>
 #include <cstdio>
+#include <fstream>
+#include <iterator>
+#include <string>
 #include <vector>
 
 #include "am_hip_tensor.hpp"
@@ -191,7 +194,40 @@ static void softmax_rows() {
   CHECK(std::fabs(s[3] - 1.0 / 3) < 1e-15 && std::fabs(s[4] - 1.0 / 3) < 1e-15 && std::fabs(s[5] - 1.0 / 3) < 1e-15);
 }
 
-int main() {
+// tests/io/test_numpy.nim:15-96 on the data files of the reference's own test
+static void npy_files(const std::string& dir) {
+  const std::vector<int64_t> e1 = {1, 2, 3, 4}, e2 = {1, 2, 3, 4, 5, 6, 7, 8};
+  for (const char* stem : {"int", "f32LE", "u64BE"}) {
+    const std::string s = dir + "/" + stem;
+    CHECK(am::read_npy<int64_t>(s + ".npy").toCpu() == e1);
+    auto c = am::read_npy<int64_t>(s + "_2D_c.npy"), f = am::read_npy<int64_t>(s + "_2D_f.npy");
+    CHECK(c.shape == (am::Shape{2, 4}) && c.toCpu() == e2 && c.is_C_contiguous());
+    CHECK(f.shape == (am::Shape{2, 4}) && f.toCpu() == e2 && f.is_F_contiguous() && !f.is_C_contiguous());
+    CHECK(eq(am::read_npy<float>(s + "_2D_f.npy"), {1, 2, 3, 4, 5, 6, 7, 8}));
+  }
+  auto same = [](const std::string& a, const std::string& b) {
+    std::ifstream fa(a, std::ios::binary), fb(b, std::ios::binary);
+    const std::string ca((std::istreambuf_iterator<char>(fa)), std::istreambuf_iterator<char>());
+    const std::string cb((std::istreambuf_iterator<char>(fb)), std::istreambuf_iterator<char>());
+    return !ca.empty() && ca == cb;
+  };
+  const std::string out = "/tmp/am_hip_test_write.npy";
+  am::write_npy(toHip<int64_t>({1, 2, 3, 4}, {4}), out);
+  CHECK(same(out, dir + "/int.npy"));
+  auto t2 = toHip<int64_t>({1, 2, 3, 4, 5, 6, 7, 8}, {2, 4});
+  am::write_npy(t2, out);
+  CHECK(same(out, dir + "/int_2D_c.npy"));
+  am::write_npy(toHip<int64_t>({1, 5, 2, 6, 3, 7, 4, 8}, {4, 2}).transpose(), out);   // column-major [2, 4]
+  CHECK(same(out, dir + "/int_2D_f.npy"));
+  am::write_npy(toHip<float>({1, 2, 3, 4, 5, 6, 7, 8}, {2, 4}), out);
+  CHECK(same(out, dir + "/f32LE_2D_c.npy"));
+  am::write_npy(toHip<float>({1, 5, 2, 6, 3, 7, 4, 8}, {4, 2}).transpose(), out);
+  CHECK(same(out, dir + "/f32LE_2D_f.npy"));
+  EXPECT_THROW(am::read_npy<float>(dir + "/does_not_exist.npy"), std::ios_base::failure);
+  std::remove(out.c_str());
+}
+
+int main(int argc, char** argv) {
   try {
     gemm_literals<float>();
     gemm_literals<double>();
@@ -209,6 +245,7 @@ int main() {
     aggregates<int32_t>();
     aggregates<int64_t>();
     softmax_rows();
+    if (argc > 1) npy_files(argv[1]);
     am::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());

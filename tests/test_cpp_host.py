@@ -20,7 +20,7 @@ def test_cpp_host_layer_builds():
 def test_cpp_host_layer_on_device(hip):
     if not os.path.exists(BIN):
         pytest.fail("tests/cpp/test_tensor_hip is not built (python -c 'import __graft_entry__ as g; g.build()')")
-    res = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+    res = subprocess.run([BIN, os.path.join(ROOT, "tests", "golden", "npy")], capture_output=True, text=True, timeout=120)
     print(res.stdout)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-1000:]
     assert " 0 failed" in res.stdout

@@ -221,4 +221,6 @@ def test_maxpool_vs_oracle(hip, oracle, vectors, sfx):
         idx, got = hip.maxpool2d(hip.toHip(x), kernel, pad, stride)
         assert np.array_equal(got.toCpu(), want) and np.array_equal(idx.toCpu(), want_idx)
     with pytest.raises(ValueError):
-        hip.maxpool2d(hip.zeros((2, 3, 4, 4), dt).transpose() if False else hip.zeros((4, 4), dt), (2, 2))
+        hip.maxpool2d(hip.zeros((4, 4), dt), (2, 2))                       # rank
+    with pytest.raises(ValueError):
+        hip.maxpool2d(hip.zeros((2, 3, 4, 4), dt).transpose(), (2, 2))     # not C-contiguous (the reference asserts)
