@@ -27,7 +27,8 @@ template <typename T, int KIND, int BMN, int BK, bool KG = true> struct Slab {
   // the banks (measured on f64: +7 % over a padding that is a multiple of 4).
   static constexpr int QN_ = BK / VK;
   static constexpr int LDKG = BMN + (QN_ >= 8 ? 1 : 8 / QN_);   // 16-byte slots per k-group plane
-  static constexpr int LDMN = BMN + 8;   // k-row layout: elements per k row
+  static constexpr int LDMN = BMN + 4;   // k-row layout: elements per k row (4 * LDMN mod 32 banks = 16: the
+                                         // four k-rows a transposing write touches fall on two bank halves, not one)
   static constexpr int ELEMS = (KIND == kKContig && KG) ? (BK / VK) * LDKG * VK : BK * LDMN;
 };
 

@@ -259,38 +259,31 @@ void gemm_mfma(Args<T> p) {
   }
   const T alpha = p.alpha, beta = p.beta;
   const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
-  // One row of accumulator tiles at a time: first every load of C and of the bias for that row is
-  // issued, then the arithmetic and the stores follow. Interleaving load / store per element would
-  // make each load wait for the store before it (one memory counter orders both), i.e. one
-  // round trip to HBM per element.
+  // One accumulator tile at a time: first every load of C and of the bias for that tile is issued,
+  // then the arithmetic and the stores follow. Interleaving load / store per element would make
+  // each load wait for the store before it (one memory counter orders both), i.e. one round trip
+  // to HBM per element. (A whole row of tiles at once needs more registers than the largest tile
+  // shapes have left next to their accumulators.)
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    T cv[TN][MF::NACC], bv[TN][MF::NACC];
-    if (beta != (T)0) {
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
-#pragma unroll
-        for (int r = 0; r < MF::NACC; ++r) {
-          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
-          cv[j][r] = (row < p.M && col < p.N) ? p.C[row * p.c_m + col * p.c_n] : (T)0;
-        }
-      }
-    }
-    if (has_bias) {
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
-#pragma unroll
-        for (int r = 0; r < MF::NACC; ++r) {
-          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
-          bv[j][r] = (row < p.M && col < p.N) ? p.bias[row * p.bias_m + col * p.bias_n] : (T)0;
-        }
-      }
-    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
+      T cv[MF::NACC], bv[MF::NACC];
+      if (beta != (T)0) {
+#pragma unroll
+        for (int r = 0; r < MF::NACC; ++r) {
+          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
+          cv[r] = (row < p.M && col < p.N) ? p.C[row * p.c_m + col * p.c_n] : (T)0;
+        }
+      }
+      if (has_bias) {
+#pragma unroll
+        for (int r = 0; r < MF::NACC; ++r) {
+          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
+          bv[r] = (row < p.M && col < p.N) ? p.bias[row * p.bias_m + col * p.bias_n] : (T)0;
+        }
+      }
 #pragma unroll
       for (int r = 0; r < MF::NACC; ++r) {
         const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
@@ -299,11 +292,11 @@ void gemm_mfma(Args<T> p) {
           if (alpha != (T)1) ab = alpha * ab;
           T v = ab;
           if (beta != (T)0) {
-            T c = cv[j][r];
+            T c = cv[r];
             if (beta != (T)1) c = c * beta;
             v = c + ab;
           }
-          if (has_bias) v = v + bv[j][r];
+          if (has_bias) v = v + bv[r];
           if (relu) v = ((T)0 >= v) ? (T)0 : v;
           p.C[row * p.c_m + col * p.c_n] = v;
         }
