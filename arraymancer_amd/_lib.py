@@ -53,6 +53,8 @@ def _signatures():
         "am_hip_memset": (ci, [vp, ci, sz]),
         "am_hip_sync": (ci, []),
         "am_hip_stream": (vp, []),
+        "am_hip_empty_cache": (ci, []),
+        "am_hip_memory_stats": (ci, [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
         "am_hip_event_create": (ci, [pp]),
         "am_hip_event_record": (ci, [vp]),
         "am_hip_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),

@@ -1,6 +1,10 @@
 // Device context, stream, memory and timing entry points of the C ABI.
+#include <map>
 #include <mutex>
 #include <stdarg.h>
+#include <stdlib.h>
+#include <unordered_map>
+#include <vector>
 #include <string.h>
 #include "common.h"
 
@@ -64,6 +68,40 @@ void* splitk_workspace(size_t bytes) {
 }
 }  // namespace gemm
 
+// ---- caching allocator -------------------------------------------------------------------------
+// Every operator of the host layers that returns a tensor allocates its result, and hipFree
+// synchronises the device: freed blocks are therefore kept in per-size free lists and handed out
+// again. A block freed while kernels still use it may be reused at once, because whoever receives
+// it next can only touch it through the library stream, i.e. after those kernels. Blocks go back
+// to the driver only from am_hip_empty_cache, when the cache exceeds its limit, or when hipMalloc
+// fails (cache emptied, one retry); each of those drains the stream first.
+static std::mutex g_alloc_mu;
+static std::unordered_map<void*, size_t> g_live;            // blocks handed out -> rounded size
+static std::map<size_t, std::vector<void*>> g_free_blocks;   // rounded size -> cached blocks
+static size_t g_live_bytes = 0, g_cached_bytes = 0;
+
+static size_t cache_limit() {   // AM_HIP_CACHE_LIMIT_MB (default 32768, 0 disables caching)
+  static const size_t limit = [] {
+    const char* e = getenv("AM_HIP_CACHE_LIMIT_MB");
+    return (size_t)((e && *e) ? strtoull(e, nullptr, 10) : 32768ull) << 20;
+  }();
+  return limit;
+}
+
+// 512-byte granules below 1 MiB, 2 MiB granules above: a freed block fits any later request of
+// the same rounded size (no splitting, so no fragmentation inside blocks).
+static size_t round_size(size_t bytes) {
+  const size_t g = bytes < ((size_t)1 << 20) ? 512 : ((size_t)2 << 20);
+  return (bytes + g - 1) / g * g;
+}
+
+static void release_cached_locked() {
+  for (auto& kv : g_free_blocks)
+    for (void* p : kv.second) (void)hipFree(p);
+  g_free_blocks.clear();
+  g_cached_bytes = 0;
+}
+
 hipStream_t stream() { return g_stream; }
 bool capturing() { return g_capturing; }
 int num_cus() { return g_ready ? g_prop.multiProcessorCount : 256; }
@@ -109,12 +147,29 @@ int am_hip_malloc(size_t bytes, void** out) {
   if (bytes == 0) return AM_OK;
   AM_TRY(ensure_init());
   if (g_capturing) return fail(AM_E_ARG, "am_hip_malloc: not allowed while a graph is being captured");
-  hipError_t e = hipMalloc(out, bytes);
-  if (e != hipSuccess) {
-    *out = nullptr;
-    (void)hipGetLastError();
-    return fail(AM_E_ALLOC, "hipMalloc(%zu bytes) failed: %s", bytes, hipGetErrorString(e));
+  const size_t rounded = round_size(bytes);
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  auto it = g_free_blocks.find(rounded);
+  if (it != g_free_blocks.end() && !it->second.empty()) {
+    *out = it->second.back();
+    it->second.pop_back();
+    g_cached_bytes -= rounded;
+  } else {
+    hipError_t e = hipMalloc(out, rounded);
+    if (e != hipSuccess && g_cached_bytes > 0) {   // give the cache back and try once more
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(g_stream);
+      release_cached_locked();
+      e = hipMalloc(out, rounded);
+    }
+    if (e != hipSuccess) {
+      *out = nullptr;
+      (void)hipGetLastError();
+      return fail(AM_E_ALLOC, "hipMalloc(%zu bytes) failed: %s", rounded, hipGetErrorString(e));
+    }
   }
+  g_live[*out] = rounded;
+  g_live_bytes += rounded;
   return AM_OK;
 }
 
@@ -122,9 +177,36 @@ int am_hip_free(void* dptr) {
   if (!dptr) return AM_OK;
   AM_TRY(ensure_init());
   if (g_capturing) return fail(AM_E_ARG, "am_hip_free: not allowed while a graph is being captured");
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  auto it = g_live.find(dptr);
+  if (it == g_live.end()) return fail(AM_E_ARG, "am_hip_free: %p was not allocated by am_hip_malloc (or freed twice)", dptr);
+  const size_t rounded = it->second;
+  g_live.erase(it);
+  g_live_bytes -= rounded;
+  if (g_cached_bytes + rounded <= cache_limit()) {
+    g_free_blocks[rounded].push_back(dptr);
+    g_cached_bytes += rounded;
+    return AM_OK;
+  }
   // Work that still reads or writes the buffer is on the library stream: drain it first.
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
   AM_HIP_TRY(hipFree(dptr));
+  return AM_OK;
+}
+
+int am_hip_empty_cache(void) {
+  AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_empty_cache: not allowed while a graph is being captured");
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  release_cached_locked();
+  return AM_OK;
+}
+
+int am_hip_memory_stats(size_t* live_bytes, size_t* cached_bytes) {
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  if (live_bytes) *live_bytes = g_live_bytes;
+  if (cached_bytes) *cached_bytes = g_cached_bytes;
   return AM_OK;
 }
 

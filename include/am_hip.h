@@ -54,8 +54,17 @@ int am_hip_device_count(int* count);
 int am_hip_device_info(char* name, size_t name_cap, int* compute_units, int* clock_khz,
                        size_t* hbm_bytes, int* lds_bytes_per_cu);
 
+/* Device memory (newCudaStorage / deallocCuda, src/arraymancer/tensor/backend/cuda.nim:23-57). Freed
+ * blocks are cached per size and reused: freeing does not synchronise the device, and a block may be
+ * handed out again while earlier work on the library stream still uses it (whatever touches it next
+ * goes through that stream too). am_hip_free only accepts pointers from am_hip_malloc. */
 int am_hip_malloc(size_t bytes, void** out);   /* bytes == 0 -> *out = NULL, AM_OK */
 int am_hip_free(void* dptr);                   /* NULL is a no-op */
+/* No counterpart in the reference (it cudaMallocs / cudaFrees per tensor): returns every cached
+ * block to the driver (drains the stream first); byte counts of the blocks in use and in the cache.
+ * Cache size limit: environment variable AM_HIP_CACHE_LIMIT_MB (default 32768; 0 = no caching). */
+int am_hip_empty_cache(void);
+int am_hip_memory_stats(size_t* live_bytes, size_t* cached_bytes);
 int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes);  /* host buffer reusable on return */
 int am_hip_memcpy_d2h(void* dst, const void* src, size_t bytes);  /* blocking, ordered after prior work */
 int am_hip_memcpy_d2d(void* dst, const void* src, size_t bytes);  /* stream ordered */

@@ -30,6 +30,8 @@ proc am_hip_device_count*(count: ptr cint): cint {.importc.}
 proc am_hip_device_info*(name: cstring, name_cap: csize_t, compute_units, clock_khz: ptr cint,
                          hbm_bytes: ptr csize_t, lds_bytes_per_cu: ptr cint): cint {.importc.}
 proc am_hip_malloc*(bytes: csize_t, dptr: ptr pointer): cint {.importc.}
+proc am_hip_empty_cache*(): cint {.importc.}   # freed blocks are cached for reuse; this returns them to the driver
+proc am_hip_memory_stats*(live_bytes, cached_bytes: ptr csize_t): cint {.importc.}
 proc am_hip_free*(dptr: pointer): cint {.importc.}
 proc am_hip_memcpy_h2d*(dst, src: pointer, bytes: csize_t): cint {.importc.}
 proc am_hip_memcpy_d2h*(dst, src: pointer, bytes: csize_t): cint {.importc.}

@@ -116,3 +116,42 @@ def test_conv_as_im2col_gemm(hip, vectors):
             out = hip.toHip(k.reshape(Co, -1)) * hip.toHip(col)
             out.bc_iadd(hip.toHip(np.array(case["bias"], dtype=dt).reshape(Co, 1)))
             assert np.array_equal(out.toCpu().reshape(1, Co, Ho, Wo), np.array(case["target"], dtype=dt)), case["name"]
+
+
+def test_caching_allocator(hip):
+    """Freed device blocks are reused without a device synchronisation; results stay right when a
+    block is handed out again while earlier kernels on the stream still read it."""
+    import ctypes
+    L = hip.load_library()
+    live, cached = ctypes.c_size_t(), ctypes.c_size_t()
+
+    def stats():
+        assert L.am_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached)) == 0
+        return live.value, cached.value
+
+    assert L.am_hip_empty_cache() == 0
+    live0, cached0 = stats()
+    assert cached0 == 0
+    t = hip.empty((1000, 1000), np.float32)          # 4 000 000 B -> one 2 MiB-granule block of 4 MiB
+    ptr = t.storage.ptr
+    assert stats()[0] == live0 + 4 * 1024 * 1024
+    del t
+    assert stats() == (live0, 4 * 1024 * 1024)
+    u = hip.empty((1024, 1024), np.float32)          # same rounded size: the cached block comes back
+    assert u.storage.ptr == ptr and stats() == (live0 + 4 * 1024 * 1024, 0)
+    del u
+    small = hip.empty((3,), np.int32)                # 512-byte granule
+    assert stats()[0] == live0 + 512
+    del small
+    # immediate reuse under load: each result of the chain frees its operand while the next kernel is queued
+    rng = np.random.default_rng(11)
+    x = rng.uniform(-1, 1, (512, 512)).astype(np.float32)
+    d = hip.toHip(x)
+    want = x.copy()
+    for i in range(50):
+        d = d + d if i % 2 == 0 else hip.scalar_op("mul", d, np.float32(0.5))
+        want = want + want if i % 2 == 0 else want * np.float32(0.5)
+    assert np.array_equal(d.toCpu(), want)
+    assert L.am_hip_empty_cache() == 0 and stats()[1] == 0
+    # a foreign pointer is rejected, not handed to the driver
+    assert L.am_hip_free(ctypes.c_void_p(0x1000)) != 0
