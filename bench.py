@@ -287,6 +287,30 @@ def config_report(am, timer, L):
              peak_used="HBM 8000 GB/s", cpu_impl="oracle/strided_map.c (port of map2_inline + strided iteration, OpenMP blocks)",
              cpu_threads=threads, cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1),
              bit_exact=bool(np.array_equal(got, out)))
+    # reductions, softmax, pooling (rows beyond the headline configurations)
+    def hbm_case(config, fn_gpu, fn_cpu, nbytes, check):
+        got = fn_gpu()
+        want = fn_cpu()
+        _, ev = timer.run(fn_gpu, 50, 5)
+        cpu_s = cpu_time(fn_cpu, budget=2.0)
+        gpu_s = ev / 50
+        emit(config=config, dtype="f32", gpu_ms=round(gpu_s * 1e3, 4), gpu_rate=round(nbytes / gpu_s / 1e9, 1), rate_unit="GB/s",
+             pct_peak=round(100 * nbytes / gpu_s / 1e9 / HBM_PEAK_GBS, 1), peak_used="HBM 8000 GB/s",
+             cpu_impl="oracle/reduce_pool.c (serial port of the reference's fold / softmax / maxpool2d)", cpu_threads=1,
+             cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1), **check(got, want))
+    n2 = 8192 * 8192 * 4
+    absX = np.abs(X)
+    hbm_case("f32 8192x8192 sum(axis=1)", lambda: am.sum(dX, 1), lambda: am_oracle.reduce_axis("sum", X, 1), n2,
+             lambda g, w: dict(max_err_rel_to_sum_abs=float(np.max(np.abs(g.toCpu().astype(np.float64) - w) / am_oracle.reduce_axis("sum", absX, 1)))))
+    hbm_case("f32 8192x8192 sum(axis=0)", lambda: am.sum(dX, 0), lambda: am_oracle.reduce_axis("sum", X, 0), n2,
+             lambda g, w: dict(max_err_rel_to_sum_abs=float(np.max(np.abs(g.toCpu().astype(np.float64) - w) / am_oracle.reduce_axis("sum", absX, 0)))))
+    hbm_case("f32 8192x8192 softmax (rows)", lambda: am.softmax(dX), lambda: am_oracle.softmax(X), 2 * n2,
+             lambda g, w: dict(max_rel_err=float(np.max(np.abs(g.toCpu() - w) / w))))
+    P = rng(4005).uniform(-1, 1, (64, 64, 112, 112)).astype(np.float32)
+    dP = am.toHip(P)
+    hbm_case("f32 maxpool2d 64x64x112x112, 2x2 stride 2", lambda: am.maxpool2d(dP, (2, 2), (0, 0), (2, 2)),
+             lambda: am_oracle.maxpool2d(P, (2, 2), (0, 0), (2, 2)), P.nbytes + P.nbytes // 4 + P.size // 4 * 8,
+             lambda g, w: dict(bit_exact=bool(np.array_equal(g[1].toCpu(), w[1]) and np.array_equal(g[0].toCpu(), w[0]))))
     r = bench_chain(am, timer, 200, 20)
     emit(config="f32 inference chain (4 GEMMs, fused bias+ReLU)", dtype="f32", hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"],
          note=r["note"])
@@ -313,6 +337,12 @@ def run_only(am, timer, which, steps, warmup):
         dA, dB = am.toHip(pa).transpose(), am.toHip(pb)[:, ::2]
         dC = am.toHip(np.random.default_rng(3003).standard_normal((2048, 3072)))
         fn = lambda: am.gemm(1.5, dA, dB, 0.5, dC)
+    elif which in ("sum_rows", "sum_cols", "softmax"):
+        dX = am.toHip(np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32))
+        fn = {"sum_rows": lambda: am.sum(dX, 1), "sum_cols": lambda: am.sum(dX, 0), "softmax": lambda: am.softmax(dX)}[which]
+    elif which == "maxpool":
+        dX = am.toHip(np.random.default_rng(4005).uniform(-1, 1, (256, 64, 112, 112)).astype(np.float32))
+        fn = lambda: am.maxpool2d(dX, (2, 2), (0, 0), (2, 2))
     else:
         X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
         dX, dY = am.toHip(X), am.empty((8192, 8192), np.float32)
@@ -335,7 +365,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true",
                     help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy", "chain"],
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy", "chain", "sum_rows", "sum_cols", "softmax", "maxpool"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -114,7 +114,7 @@ def test_sum_over_non_unit_stride_axis_is_the_serial_fold(hip, oracle, sfx):
     reassociated: covered with a tolerance by the other tests.)"""
     dt = DTYPES[sfx]
     rng = np.random.default_rng(seed_of("rowsum", sfx))
-    for shape in [(64, 200_000), (300, 150_000), (20, 400, 500), (63, 131_072)]:
+    for shape in [(64, 1_100_000), (20, 1100, 1000), (63, 1_048_576), (5, 3, 1_200_000)]:
         x = rng.uniform(-1, 1, shape).astype(dt)
         say("serial-order sum", sfx, shape)
         assert np.array_equal(hip.sum(hip.toHip(x), 0).toCpu(), oracle.reduce_axis("sum", x, 0))
