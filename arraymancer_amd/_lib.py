@@ -16,7 +16,7 @@ AM_MAXRANK = 6
 
 OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
           relu_bwd=8, max=9, min=10)
-OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2)
+OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2, addmul=3)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
 EPI = dict(none=0, bias=1, relu=2, bias_relu=3)
 RED = dict(sum=0, product=1, min=2, max=3)

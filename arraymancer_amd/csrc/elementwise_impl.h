@@ -284,6 +284,7 @@ template <typename T, int OP> struct TriOp {
   typedef typename Traits<T>::U U;
   static __device__ __forceinline__ T apply(T x, T y, T z) {
     if constexpr (OP == AM_OP3_MULADD) return (T)((U)x * (U)y + (U)z);
+    else if constexpr (OP == AM_OP3_ADDMUL) return (T)(((U)x + (U)y) * (U)z);
     else if constexpr (OP == AM_OP3_GRU_CANDIDATE) return dev_tanh(x + y * z);
     else return ((T)1 - y) * z + y * x;
   }
@@ -295,12 +296,15 @@ template <typename T> struct TriArgs {
   int64_t L;          // rows kernel: inner extent
   uint32_t tiles_per_row, total_tiles;
   int rank;           // collapsed rank (generic) / number of outer dims (rows)
+  int a_const, b_const, c_const;   // rows kernel: operand has inner stride 0 (one value per row)
+  int a_keep, b_keep, c_keep;      // rows kernel: the same row is re-read for every output row: cached loads
   int64_t shape[AM_MAXRANK];
   int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK], sc[AM_MAXRANK];
 };
 
-// All four operands have unit innermost stride and 16-byte aligned rows (the GRU column slices,
-// plain contiguous tensors): same streaming structure as ew_rows.
+// Every operand has unit innermost stride and 16-byte aligned rows (the GRU column slices, plain
+// contiguous tensors, row vectors broadcast over the rows) or innermost stride 0 (a column vector
+// broadcast along the rows: one scalar per row): same streaming structure as ew_rows.
 template <typename T, int OP>
 __global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
   typedef typename Traits<T>::V V;
@@ -327,15 +331,17 @@ __global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t col = col0 + (int64_t)u * kThreads * VEC;
       if (col + VEC <= p.L) {
-        const V av = __builtin_nontemporal_load((const V*)(arow + col));
-        const V bv = __builtin_nontemporal_load((const V*)(brow + col));
-        const V cv = __builtin_nontemporal_load((const V*)(crow + col));
+        V av, bv, cv;
+        if (p.a_const) { for (int e = 0; e < VEC; ++e) av[e] = arow[0]; } else av = p.a_keep ? *(const V*)(arow + col) : __builtin_nontemporal_load((const V*)(arow + col));
+        if (p.b_const) { for (int e = 0; e < VEC; ++e) bv[e] = brow[0]; } else bv = p.b_keep ? *(const V*)(brow + col) : __builtin_nontemporal_load((const V*)(brow + col));
+        if (p.c_const) { for (int e = 0; e < VEC; ++e) cv[e] = crow[0]; } else cv = p.c_keep ? *(const V*)(crow + col) : __builtin_nontemporal_load((const V*)(crow + col));
         V r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) r[e] = TriOp<T, OP>::apply(av[e], bv[e], cv[e]);
         __builtin_nontemporal_store(r, (V*)(drow + col));
       } else {
-        for (int64_t cc = col; cc < p.L; ++cc) drow[cc] = TriOp<T, OP>::apply(arow[cc], brow[cc], crow[cc]);
+        for (int64_t cc = col; cc < p.L; ++cc)
+          drow[cc] = TriOp<T, OP>::apply(arow[p.a_const ? 0 : cc], brow[p.b_const ? 0 : cc], crow[p.c_const ? 0 : cc]);
       }
     }
   }
@@ -633,10 +639,13 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
   AM_TRY(ensure_init());
   const int in = r - 1;
   const int64_t L = g.shape[in];
-  bool ok = g.sd[in] == 1 && g.sa[in] == 1 && g.sb[in] == 1 && g.sc[in] == 1 && aligned16(dst) && aligned16(a) &&
-            aligned16(b) && aligned16(c);
+  g.a_const = g.sa[in] == 0; g.b_const = g.sb[in] == 0; g.c_const = g.sc[in] == 0;
+  g.a_keep = g.b_keep = g.c_keep = in > 0;
+  for (int d = 0; d < in; ++d) { g.a_keep &= g.sa[d] == 0; g.b_keep &= g.sb[d] == 0; g.c_keep &= g.sc[d] == 0; }
+  bool ok = g.sd[in] == 1 && (g.sa[in] == 1 || g.a_const) && (g.sb[in] == 1 || g.b_const) && (g.sc[in] == 1 || g.c_const) &&
+            aligned16(dst) && (g.a_const || aligned16(a)) && (g.b_const || aligned16(b)) && (g.c_const || aligned16(c));
   for (int d = 0; d < in && ok; ++d)
-    if (g.sd[d] % VEC || g.sa[d] % VEC || g.sb[d] % VEC || g.sc[d] % VEC) ok = false;
+    if (g.sd[d] % VEC || (!g.a_const && g.sa[d] % VEC) || (!g.b_const && g.sb[d] % VEC) || (!g.c_const && g.sc[d] % VEC)) ok = false;
   int64_t rows = 1;
   for (int d = 0; d < in; ++d) rows *= g.shape[d];
   const int64_t tile = (int64_t)kThreads * VEC * kUnroll;
@@ -676,6 +685,7 @@ static int ternary(const char* fn, int op, int rank, const int64_t* shape, T* ds
   constexpr bool F = Traits<T>::kFloat;
   switch (op) {
     case AM_OP3_MULADD: return run3<T, AM_OP3_MULADD>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
+    case AM_OP3_ADDMUL: return run3<T, AM_OP3_ADDMUL>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
     case AM_OP3_GRU_CANDIDATE:
       if constexpr (F) return run3<T, AM_OP3_GRU_CANDIDATE>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
       else return fail(AM_E_DTYPE, "%s: tanh(x + y * z) is defined for float tensors only", fn);

@@ -248,6 +248,11 @@ def config_report(am, timer, L):
                    cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1))
         if dt.kind == "f":
             row["rel_frobenius_vs_cpu"] = am_oracle.rel_frobenius(got, want)
+            # the reference's float `*` goes through CBLAS: NumPy's bundled BLAS as the stand-in for it
+            # (a copy of each view first, as the reference makes: p_operator_blas_l2l3.nim:151-152)
+            blas_s = cpu_time(lambda: alpha * (np.ascontiguousarray(A) @ np.ascontiguousarray(B)) + beta * C_host)
+            row["cpu_blas_impl"] = "NumPy bundled BLAS, alpha * (A @ B) + beta * C on contiguous copies (stand-in for the reference's CBLAS path)"
+            row["cpu_blas_ms"] = round(blas_s * 1e3, 2)
         else:
             row["bit_exact"] = bool(np.array_equal(got, want))
         emit(**row)
@@ -287,6 +292,15 @@ def config_report(am, timer, L):
              peak_used="HBM 8000 GB/s", cpu_impl="oracle/strided_map.c (port of map2_inline + strided iteration, OpenMP blocks)",
              cpu_threads=threads, cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1),
              bit_exact=bool(np.array_equal(got, out)))
+    # (X +. b) *. s fused into one pass (same bytes moved once instead of twice)
+    bb, sb = db.broadcast((8192, 8192)), ds.broadcast((8192, 8192))
+    _, ev = timer.run(lambda: th._ternary_into("addmul", dY, dX, bb, sb), 50, 5)
+    gpu_s = ev / 50
+    two_pass = ((X + b) * sc)
+    emit(config="f32 8192x8192 (X +. b) *. s fused (one pass)", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
+         gpu_rate=round((nbytes + 8192 * 4) / gpu_s / 1e9, 1), rate_unit="GB/s",
+         pct_peak=round(100 * (nbytes + 8192 * 4) / gpu_s / 1e9 / HBM_PEAK_GBS, 1), peak_used="HBM 8000 GB/s",
+         bit_exact=bool(np.array_equal(dY.toCpu(), two_pass)), note="equals the two separate broadcast passes bit for bit")
     # reductions, softmax, pooling (rows beyond the headline configurations)
     def hbm_case(config, fn_gpu, fn_cpu, nbytes, check):
         got = fn_gpu()

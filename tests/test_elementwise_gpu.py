@@ -302,6 +302,12 @@ def test_map3_muladd_bit_exact(hip, oracle, sfx):
         if len(shape) == 2:   # transposed operand -> generic kernel
             got = hip.map3("muladd", hip.toHip(a), hip.toHip(np.ascontiguousarray(b.T)).transpose(), hip.toHip(c)).toCpu()
             assert np.array_equal(got, oracle.map3("muladd", a, b, c))
+    # (X +. b) *. s in one pass equals the two broadcast passes bit for bit (each step rounded on its own)
+    X, r, col = fill(rng, (300, 1030), dt), fill(rng, (1, 1030), dt), fill(rng, (300, 1), dt)
+    dX, dr, dc = hip.toHip(X), hip.toHip(r), hip.toHip(col)
+    fused = hip.map3("addmul", dX, dr.broadcast(X.shape), dc.broadcast(X.shape)).toCpu()
+    assert np.array_equal(fused, hip.bc_mul(hip.bc_add(dX, dr), dc).toCpu())
+    assert np.array_equal(fused, oracle.map3("addmul", X, np.broadcast_to(r, X.shape), np.broadcast_to(col, X.shape)))
     if sfx in INT:
         with pytest.raises(TypeError):
             hip.map3("gru_blend", hip.toHip(a), hip.toHip(b), hip.toHip(c))

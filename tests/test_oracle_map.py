@@ -197,6 +197,7 @@ def test_map3_bodies_match_numpy(oracle):
         base = rng.uniform(-2, 2, (3, 40, 48)).astype(dt)
         x, y, z = base[0][:, 0:16], base[1][:, 16:32], base[2].T[8:24].T   # column slices, like the GRU gates
         assert np.array_equal(oracle.map3("muladd", x, y, z), x * y + z)
+        assert np.array_equal(oracle.map3("addmul", x, y, z), (x + y) * z)
         assert np.array_equal(oracle.map3("gru_blend", x, y, z), (dt(1) - y) * z + y * x)
         np.testing.assert_allclose(oracle.map3("gru_candidate", x, y, z), np.tanh((x + y * z).astype(np.float64)),
                                    rtol=2e-6 if dt == np.float32 else 1e-14, atol=1e-7 if dt == np.float32 else 1e-15)
@@ -207,6 +208,7 @@ def test_map3_bodies_match_numpy(oracle):
         assert np.array_equal(dst, want)
     a = np.array([2**31 - 1, -5, 7], dtype=np.int32)
     assert oracle.map3("muladd", a, a, a).tolist() == [(((2**31 - 1) ** 2 + 2**31 - 1 + 2**31) % 2**32) - 2**31, 20, 56]
+    assert oracle.map3("addmul", a, a, a).tolist() == [(((2**32 - 2) * (2**31 - 1)) % 2**32 + 2**31) % 2**32 - 2**31, 50, 98]
     with pytest.raises(ValueError):
         oracle.map3("gru_blend", a, a, a)
 
