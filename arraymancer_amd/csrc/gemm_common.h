@@ -176,11 +176,11 @@ static inline void apply_splitk(Args<T>& g, int bk, int64_t want) {
 // products, where cutting K changes no bit of the result. Estimated time of a candidate =
 // rounds of two workgroups per CU x time of one workgroup, plus the second pass that adds the
 // partial sums (its launch and its HBM traffic). mac_per_us: multiply-adds one CU sustains.
-struct TileSplit { int tile; int splits; };
+struct TileSplit { int tile; int splits; double est_us; };
 template <typename T>
 static inline TileSplit choose_tile_split(const TileChoice* cand, int ncand, int64_t M, int64_t N, int64_t K, int bk,
                                           double mac_per_us, const char* env, int64_t batch) {
-  TileSplit best = {0, 1};
+  TileSplit best = {0, 1, 0.0};
   int forced_tile = -1;
   const char* forced = getenv(env);
   if (forced && *forced) { const int idx = atoi(forced); if (idx >= 0 && idx < ncand) forced_tile = idx; }
@@ -212,6 +212,7 @@ static inline TileSplit choose_tile_split(const TileChoice* cand, int ncand, int
     }
   }
   if (trace_choices()) fprintf(stderr, "am_hip gemm: M=%lld N=%lld K=%lld tile %d (%dx%d) splits %d est %.1f us\n", (long long)M, (long long)N, (long long)K, best.tile, cand[best.tile].bm, cand[best.tile].bn, best.splits, best_cost);
+  best.est_us = best_cost;
   return best;
 }
 

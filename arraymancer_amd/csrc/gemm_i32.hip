@@ -1,11 +1,14 @@
-// int32 GEMM entry point (VALU path, wraparound arithmetic): am_hip_gemm_i32.
+// int32 GEMM entry points (wraparound arithmetic): large products run on the int8 matrix cores by
+// digit slicing, the others on the vector ALU.
 #include "gemm_int_impl.h"
+#include "gemm_i8_digits.h"
 
 using namespace am;
 using namespace am::gemm;
 
 static int run_i32(Args<int32_t>& g) {
   constexpr int64_t VK = 16 / (int64_t)sizeof(int32_t);
+
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
   if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;
@@ -14,6 +17,16 @@ static int run_i32(Args<int32_t>& g) {
   static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.85}};
   // 119.0e3 multiply-adds per microsecond and CU: the measured VALU ceiling of this element type.
   const TileSplit ts = choose_tile_split<int32_t>(cand, 2, g.M, g.N, g.K, 16, 119.0e3, "AM_HIP_GEMM_TILE_I32", g.batch);
+  // The same product on the int8 matrix cores (digit slicing) when that is estimated to be faster.
+  // The VALU estimate is optimistic by about a fifth on mid-sized products (measured), hence the 1.2.
+  if (const int may = i8::applicable(g)) {
+    const i8::Plan pl = i8::plan(g);
+    if (may == 2 || pl.est_us < 1.2 * ts.est_us) {
+      if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path, %s tiles, est %.1f us (VALU est %.1f us)\n", pl.big ? "256x256" : "256x128", pl.est_us, ts.est_us);
+      const int rc = i8::run(g, pl);
+      if (rc <= 0) return rc;   // > 0: no scratch memory for the digit planes, take the VALU kernel
+    }
+  }
   switch (ts.tile) {
     case 0: return launch_valu<int32_t, 8, 8, 16>(g, ak, bk, ts.splits);
     default: return launch_valu<int32_t, 4, 4, 16>(g, ak, bk, ts.splits);

@@ -1,0 +1,358 @@
+// Exact int32 GEMM on the int8 matrix cores of gfx950 by digit slicing.
+//
+// An int32 is written in four balanced base-256 digits, x = d0 + 2^8 d1 + 2^16 d2 + 2^24 d3 (mod 2^32),
+// each d in [-128, 127]. Modulo 2^32 the product of two such numbers only needs the ten digit pairs
+// with i + j <= 3, so
+//     A * B  =  sum_{s=0..3} 2^(8s) * sum_{i+j=s} A_i * B_j          (mod 2^32)
+// where every A_i * B_j is an int8 x int8 -> int32 matrix product, which v_mfma_i32_32x32x32_i8
+// computes exactly; its accumulator wraps modulo 2^32, and a wrapped partial sum shifted left by 8s
+// is still right modulo 2^32. Ring arithmetic: the result has the same bits as the wrapping VALU
+// kernel and as the reference's integer micro-kernels
+// (src/arraymancer/laser/primitives/matrix_multiplication/gemm_ukernel_avx2.nim:15-16), whatever
+// the order of the additions. Ten int8 products cost 10 x 2MNK int8 operations at 5 POP/s of matrix
+// throughput against 2MNK multiply-adds at the 61 Top/s the vector ALU sustains.
+//
+// Two passes:
+//   split_digits   strided int32 operand (any view) -> four int8 planes [digit][row][k], k contiguous,
+//                  rows padded to the tile size and k to the slab size with zeros (a 32 x 128 tile
+//                  goes through LDS so that both the strided read and the k-contiguous write are
+//                  coalesced);
+//   gemm_i8_digits one workgroup of eight wavefronts per 256 x 256 (or 256 x 128) tile of C. For
+//                  s = 3..0 it walks the pairs (i, s - i) whose planes are not empty (split_digits
+//                  flags the planes that hold a non-zero digit: entries within +-127 need one pair
+//                  instead of ten) and the k slabs of each pair as one long k loop (LDS ring of 3 slabs, fragments double-buffered in registers, as in the
+//                  float kernels); between two values of s the accumulators are shifted left by 8
+//                  (Horner form of the sum over s). Padded planes mean no bounds tests in the loop.
+#pragma once
+#include <type_traits>
+#include "gemm_common.h"
+
+extern "C" int am_hip_malloc(size_t bytes, void** out);
+extern "C" int am_hip_free(void* dptr);
+
+namespace am {
+namespace gemm {
+namespace i8 {
+
+constexpr int kRowPad = 256;   // operand planes are padded to this many rows (largest tile edge) ...
+constexpr int kKPad = 128;     // ... and to this many k (largest slab)
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// The four balanced digits of four neighbouring k, packed as one 32-bit word per plane.
+__device__ __forceinline__ void digits_of4(const int32_t (&x)[4], uint32_t (&w)[4]) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) w[d] = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    uint32_t ux = (uint32_t)x[e];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int32_t dig = (int32_t)(int8_t)(ux & 0xFFu);
+      w[d] |= ((uint32_t)dig & 0xFFu) << (8 * e);
+      ux = (ux - (uint32_t)dig) >> 8;
+    }
+  }
+}
+
+// X(mn, k) = X[mn * ld_mn + k * ld_k]  ->  planes P[d][mn][k] (mn < MNp, k < Kp), zero padded.
+// One workgroup moves a 32 (mn) x 128 (k) tile through LDS: the read walks whichever of the two
+// directions is the faster one in memory (kfast), the write is 16 bytes per lane and plane, eight
+// lanes to a 128-byte row segment.
+// flags[d] is set to 1 when plane d holds a non-zero digit anywhere (the product kernel skips the
+// digit pairs of empty planes: operands with small entries have only one or two non-empty planes).
+__global__ __launch_bounds__(256) void split_digits(const int32_t* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t K,
+                                                    int8_t* P, int64_t MNp, int64_t Kp, int kfast, uint32_t* flags) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  __shared__ int32_t tile[32][129];
+  const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int e = threadIdx.x + i * 256;
+    int mn, k;
+    if (kfast) { k = e & 127; mn = e >> 7; } else { mn = e & 31; k = e >> 5; }
+    const bool ok = (mn0 + mn) < MN && (k0 + k) < K;
+    tile[mn][k] = ok ? X[(mn0 + mn) * ld_mn + (k0 + k) * ld_k] : 0;
+  }
+  __syncthreads();
+  const int64_t plane = MNp * Kp;
+  const int k16 = threadIdx.x & 7, mn = threadIdx.x >> 3;
+  u4 out[4];
+  uint32_t nz[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int32_t xs[4] = {tile[mn][k16 * 16 + g * 4], tile[mn][k16 * 16 + g * 4 + 1], tile[mn][k16 * 16 + g * 4 + 2],
+                           tile[mn][k16 * 16 + g * 4 + 3]};
+    uint32_t w[4];   // one 4-byte word (4 consecutive k) per digit plane
+    digits_of4(xs, w);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) { out[d][g] = w[d]; nz[d] |= w[d]; }
+  }
+  int8_t* dst = P + (mn0 + mn) * Kp + k0 + k16 * 16;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) *(u4*)(dst + d * plane) = out[d];
+#pragma unroll
+  for (int d = 0; d < 4; ++d)   // at most one atomic per wavefront and plane, none once the flag is up
+    if (__ballot(nz[d] != 0) != 0 && (threadIdx.x & 63) == 0 && flags[d] == 0) atomicOr(&flags[d], 1u);
+}
+
+struct DigitArgs {
+  const int8_t* PA; const int8_t* PB;   // [4][Mp][Kp], [4][Np][Kp]
+  const uint32_t* flags;                // [0..3]: planes of A that are not all zero, [4..7]: planes of B
+  int64_t Mp, Np, Kp;
+  int32_t* C; int64_t c_m, c_n;
+  int64_t M, N;
+  int32_t alpha, beta;
+  int tiles_m, tiles_n;
+};
+
+// WAVES_M x WAVES_N wavefronts, each with TM x TN accumulator tiles of 32 x 32; BK k (bytes) per slab.
+// The digit sums are evaluated in Horner form, s = 3 first: after the pairs of one s the accumulators
+// are shifted left by 8 and go on accumulating the pairs of s - 1, so one accumulator set suffices
+// (everything modulo 2^32, which both the shift and the matrix cores respect).
+template <int WAVES_M, int WAVES_N, int TM, int TN, int BK>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(DigitArgs p) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int WM = TM * 32, WN = TN * 32, BM = WAVES_M * WM, BN = WAVES_N * WN, NKS = BK / 32, QN = BK / 16;
+  constexpr int LDA = BM + (QN >= 8 ? 1 : 8 / QN), LDB = BN + (QN >= 8 ? 1 : 8 / QN);   // 16-byte slots per k-group plane
+  constexpr int SLAB_A = QN * LDA * 16, SLAB_B = QN * LDB * 16;
+  static_assert(NKS % 2 == 0 && (BM * QN) % NT == 0 && (BN * QN) % NT == 0, "tile shape");
+  __shared__ __attribute__((aligned(16))) int8_t sA[3][SLAB_A];
+  __shared__ __attribute__((aligned(16))) int8_t sB[3][SLAB_B];
+
+  int tile_m, tile_n;
+  tile_of_block((int)blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+  const int lrow = lane & 31, kg = lane >> 5;
+
+  // global -> register -> LDS: rows x QN sixteen-byte vectors per operand slab; QN neighbouring
+  // lanes cover one BK-byte row segment.
+  constexpr int NVA = BM * QN / NT, NVB = BN * QN / NT;
+  const int64_t planeA = p.Mp * p.Kp, planeB = p.Np * p.Kp;
+  const int8_t* ga[NVA]; const int8_t* gb[NVB];
+  int lds_a[NVA], lds_b[NVB];
+#pragma unroll
+  for (int i = 0; i < NVA; ++i) {
+    const int v = threadIdx.x + i * NT;
+    const int q = v % QN, mn = v / QN;
+    ga[i] = p.PA + (m0 + mn) * p.Kp + q * 16;
+    lds_a[i] = (q * LDA + mn) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < NVB; ++i) {
+    const int v = threadIdx.x + i * NT;
+    const int q = v % QN, mn = v / QN;
+    gb[i] = p.PB + (n0 + mn) * p.Kp + q * 16;
+    lds_b[i] = (q * LDB + mn) * 16;
+  }
+  // The digit pairs to multiply: (s, i) with i + j = s <= 3, s = 3 first, restricted to planes
+  // that hold something. tab_shift[pr] = how far the accumulators move left before pair pr (the
+  // Horner steps between its s and the previous pair's), tab_shift[n_pairs] = the final shift.
+  __shared__ int tab_a[10], tab_b[10], tab_shift[11], tab_n;
+  if (threadIdx.x == 0) {
+    int n = 0, prev_s = -1;
+    for (int s = 3; s >= 0; --s)
+      for (int i = 0; i <= s; ++i)
+        if (p.flags[i] != 0 && p.flags[4 + s - i] != 0) {
+          tab_a[n] = i; tab_b[n] = s - i;
+          tab_shift[n] = prev_s < 0 ? 0 : 8 * (prev_s - s);
+          prev_s = s;
+          ++n;
+        }
+    tab_shift[n] = prev_s < 0 ? 0 : 8 * prev_s;
+    tab_n = n;
+  }
+  __syncthreads();
+  const int n_pairs = tab_n;
+  const int64_t slabs_per_pair = p.Kp / BK;
+  const int64_t total = (int64_t)n_pairs * slabs_per_pair;
+  // slab number -> offsets of its A and B slabs
+  auto offsets = [&](int64_t t, int64_t& oa, int64_t& ob) {
+    int64_t pr = t / slabs_per_pair;
+    const int64_t k0 = (t - pr * slabs_per_pair) * BK;
+    if (pr > n_pairs - 1) pr = n_pairs - 1;   // slabs fetched past the end re-read the last pair (never multiplied)
+    oa = tab_a[pr] * planeA + k0;
+    ob = tab_b[pr] * planeB + k0;
+  };
+  v4i ra[NVA], rb[NVB];
+  auto fetch = [&](int64_t t) {
+    int64_t oa, ob;
+    offsets(t, oa, ob);
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) ra[i] = *(const v4i*)(ga[i] + oa);
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) rb[i] = *(const v4i*)(gb[i] + ob);
+  };
+  auto commit = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) *(v4i*)(sA[buf] + lds_a[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) *(v4i*)(sB[buf] + lds_b[i]) = rb[i];
+  };
+  v4i af[2][TM], bf[2][TN];
+  auto read_frags = [&](auto parity_tag, int buf, int ks) {
+    constexpr int P = decltype(parity_tag)::value;
+    const int q = ks * 2 + kg;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[P][i] = *(const v4i*)(sA[buf] + (q * LDA + wave_m * WM + i * 32 + lrow) * 16);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bf[P][j] = *(const v4i*)(sB[buf] + (q * LDB + wave_n * WN + j * 32 + lrow) * 16);
+  };
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  auto shift_acc = [&](int sh) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = (int)((uint32_t)acc[i][j][r] << sh);
+  };
+
+  if (total > 0) {   // (every plane of an operand empty: the product is zero)
+  // prologue: slabs 0 and 1 in LDS, slab 2 in registers
+  fetch(0); commit(0);
+  fetch(1); commit(1);
+  fetch(2);
+  __syncthreads();
+  read_frags(std::integral_constant<int, 0>(), 0, 0);
+
+  int cur = 0;
+  int64_t next_pair = slabs_per_pair;   // first slab of the next pair
+  int pr = 0;
+  for (int64_t t = 0; t < total; ++t) {
+    const int nxt = cur == 2 ? 0 : cur + 1, nxt2 = nxt == 2 ? 0 : nxt + 1;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (ks + 1 < NKS) {
+        if (ks & 1) read_frags(std::integral_constant<int, 0>(), cur, ks + 1);
+        else read_frags(std::integral_constant<int, 1>(), cur, ks + 1);
+      } else {
+        read_frags(std::integral_constant<int, 0>(), nxt, 0);   // NKS is even
+        commit(nxt2);                                            // slab t + 2
+        fetch(t + 3);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+    cur = nxt;
+    if (t + 1 == next_pair) {   // a pair is done: Horner step(s) down to the next pair's s (or to s = 0 at the end)
+      ++pr;
+      next_pair += slabs_per_pair;
+      const int sh = tab_shift[pr];
+      if (sh != 0) shift_acc(sh);
+    }
+  }
+  }
+
+  // C <- alpha * AB + beta * C in the ring of 32-bit integers (same case analysis as the other kernels)
+  const uint32_t alpha = (uint32_t)p.alpha, beta = (uint32_t)p.beta;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int64_t col = n0 + wave_n * WN + j * 32 + lrow;
+      uint32_t cv[16];
+      if (beta != 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t row = m0 + wave_m * WM + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
+          cv[r] = (row < p.M && col < p.N) ? (uint32_t)p.C[row * p.c_m + col * p.c_n] : 0u;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t row = m0 + wave_m * WM + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
+        if (row < p.M && col < p.N) {
+          uint32_t v = alpha * (uint32_t)acc[i][j][r];
+          if (beta != 0) v += beta * cv[r];
+          p.C[row * p.c_m + col * p.c_n] = (int32_t)v;
+        }
+      }
+    }
+}
+
+// Padded operand extents and the estimated time of the digit-sliced product for both tile shapes
+// (rounds of one workgroup per CU x measured time per tile and k, plus the two splitting passes).
+struct Plan { int64_t Mp, Np, Kp; bool big; double est_us; };
+static inline Plan plan(const Args<int32_t>& g) {
+  Plan pl;
+  pl.Mp = (g.M + kRowPad - 1) / kRowPad * kRowPad;
+  pl.Np = (g.N + kRowPad - 1) / kRowPad * kRowPad;
+  pl.Kp = (g.K + kKPad - 1) / kKPad * kKPad;
+  const int64_t cus = num_cus();
+  const int64_t tb = (pl.Mp / 256) * (pl.Np / 256), ts = (pl.Mp / 256) * (pl.Np / 128);
+  // microseconds per k for one tile (all ten digit pairs), measured at 4096^3: 0.162 (256 x 256), 0.098 (256 x 128)
+  const double cost_big = (double)((tb + cus - 1) / cus) * 0.162 * pl.Kp, cost_small = (double)((ts + cus - 1) / cus) * 0.098 * pl.Kp;
+  pl.big = cost_big <= cost_small;
+  const char* force = getenv("AM_HIP_GEMM_TILE_I8");   // 1: 256 x 256 tiles, 0: 256 x 128 (tests)
+  if (force && *force) pl.big = atoi(force) != 0;
+  const double split_us = 2 * 5.0 + 8.0 * (double)(pl.Mp + pl.Np) * pl.Kp / 2.8e6;   // reads 4 B, writes 4 B per element
+  pl.est_us = (pl.big ? cost_big : cost_small) + split_us;
+  return pl;
+}
+
+// Whether the digit-sliced path may take this product at all: not part of a batch, not being
+// recorded into a graph (it allocates its planes). AM_HIP_GEMM_I32_PATH = "valu" / "mfma" forces a
+// path (tests, benchmarks); returns 0 = no, 1 = if estimated faster, 2 = forced.
+static inline int applicable(const Args<int32_t>& g) {
+  const char* e = getenv("AM_HIP_GEMM_I32_PATH");
+  if (e && *e == 'v') return 0;
+  if (g.batch > 1 || capturing()) return 0;
+  if (e && *e == 'm') return 2;
+  return (g.M >= 64 && g.N >= 64 && g.K >= 256) ? 1 : 0;
+}
+
+static int run(const Args<int32_t>& g, const Plan& pl) {
+  const int64_t Mp = pl.Mp, Np = pl.Np, Kp = pl.Kp;
+  const bool big = pl.big;   // 256 x 256 tiles: a 128 x 64 tile per wavefront, fewest LDS reads per matrix instruction
+  if (Mp / 64 >= ((int64_t)1 << 31) || Np / 64 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return 1;
+  const int64_t tiles_m = Mp / 256, tiles_n = big ? Np / 256 : Np / 128;
+  if (tiles_m * tiles_n >= ((int64_t)1 << 31)) return 1;
+  void* ws = nullptr;
+  const size_t plane_bytes = (size_t)4 * (size_t)(Mp + Np) * (size_t)Kp;
+  if (am_hip_malloc(plane_bytes + 256, &ws) != AM_OK) return 1;
+  int8_t* PA = (int8_t*)ws;
+  int8_t* PB = PA + 4 * Mp * Kp;
+  uint32_t* flags = (uint32_t*)((char*)ws + plane_bytes);
+  if (hipMemsetAsync(flags, 0, 8 * sizeof(uint32_t), stream()) != hipSuccess) { (void)hipGetLastError(); (void)am_hip_free(ws); return 1; }
+  auto split = [&](const int32_t* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t MNp, int kfast, int8_t* P, uint32_t* fl) {
+    hipLaunchKernelGGL(split_digits, dim3((unsigned)(MNp / 32), (unsigned)(Kp / 128)), dim3(256), 0, stream(), X, ld_mn, ld_k, MN,
+                       g.K, P, MNp, Kp, kfast, fl);
+  };
+  split(g.A, g.a_mn, g.a_k, g.M, Mp, g.a_kfast, PA, flags);
+  split(g.B, g.b_mn, g.b_k, g.N, Np, g.b_kfast, PB, flags + 4);
+  DigitArgs d;
+  d.PA = PA; d.PB = PB; d.flags = flags; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
+  d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
+  d.alpha = g.alpha; d.beta = g.beta;
+  d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
+  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
+  if (big) hipLaunchKernelGGL((gemm_i8_digits<2, 4, 4, 2, 64>), grid, block, 0, stream(), d);
+  else hipLaunchKernelGGL((gemm_i8_digits<4, 2, 2, 2, 128>), grid, block, 0, stream(), d);
+  const int rc = check_launch("gemm_i8_digits");
+  // The planes go back to the allocator's cache at once: whoever gets the block next reaches it
+  // through the same stream, after this product.
+  (void)am_hip_free(ws);
+  return rc;
+}
+
+}  // namespace i8
+}  // namespace gemm
+}  // namespace am

@@ -29,6 +29,7 @@ sys.path.insert(0, ROOT)
 MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix peak: 256 CU x 256 FLOP/clk x 2.4 GHz
 MFMA_F64_PEAK_TFLOPS = 78.6
 HBM_PEAK_GBS = 8000.0
+MFMA_I8_PEAK_TOPS = 5000.0     # MI355X dense int8 matrix peak (5.0 POP/s)
 # Measured separately with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), see profiles/; None = not measured.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
@@ -118,7 +119,8 @@ def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
 
 def other_workloads(am, timer, steps, warmup, ceilings):
     out = []
-    # --- int32 GEMM 4096^3, entries in [-100, 100], wraparound accumulate (VALU bound)
+    # --- int32 GEMM 4096^3, entries in [-100, 100], wraparound accumulate: digit-sliced on the int8
+    # matrix cores (the library's choice at this size), and the VALU kernel beside it
     n = 4096
     A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
     B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
@@ -126,12 +128,23 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     k = max(3, steps // 4)
     wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
     tops = 2.0 * n ** 3 / (ev / k) / 1e12
+    os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
+    try:
+        _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+    finally:
+        del os.environ["AM_HIP_GEMM_I32_PATH"]
+    valu_tops = 2.0 * n ** 3 / (ev_valu / k) / 1e12
     peak = ceilings.get("valu_int32_mac")
-    out.append(dict(workload="i32 GEMM 4096^3 (wraparound, VALU)", unit="Top/s", dtype="i32",
-                    value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
-                    roofline=dict(bound="valu (measured int32 multiply-add ceiling; no matrix instruction for int32)",
-                                  achieved=round(tops, 3), peak=peak, unit="Top/s",
-                                  frac=round(tops / peak, 4) if peak else None)))
+    out.append(dict(workload="i32 GEMM 4096^3 (wraparound; ten int8 digit-pair products on the matrix cores, incl. the digit-splitting passes)",
+                    unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                    roofline=dict(bound="mfma", achieved=round(10 * tops, 1), peak=MFMA_I8_PEAK_TOPS,
+                                  unit="int8 TOP/s executed (20*M*N*K per product: 10 digit pairs)",
+                                  frac=round(10 * tops / MFMA_I8_PEAK_TOPS, 4)),
+                    valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / k * 1e3, 4),
+                                     roofline=dict(bound="valu (measured int32 multiply-add ceiling; no matrix instruction for int32)",
+                                                   achieved=round(valu_tops, 3), peak=peak, unit="Top/s",
+                                                   frac=round(valu_tops / peak, 4) if peak else None)),
+                    speedup_over_valu_ceiling=round(tops / peak, 2) if peak else None))
     del dA, dB, dC
     # --- float64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C), M=2048 N=3072 K=1024
     pa = np.random.default_rng(3001).standard_normal((1024, 2048))
@@ -266,9 +279,18 @@ def config_report(am, timer, L):
         for n in (1500, 4096):
             A = rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(dt)
             B = rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(dt)
-            gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100]", sfx, n, n, n, A, B, am.toHip(A), am.toHip(B),
-                      peak=ceil.get(key), peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s",
-                      unit="Top/s", steps=10)
+            if sfx == "i32":   # the library's own choice (int8 matrix cores at these sizes), then the VALU kernel
+                gemm_case(f"i32 GEMM {n}^3, entries in [-100, 100] (library's choice: digit-sliced int8 MFMA)", sfx, n, n, n, A, B,
+                          am.toHip(A), am.toHip(B), peak=ceil.get(key),
+                          peak_used=f"measured VALU i32 multiply-add ceiling {ceil.get(key)} Top/s (the matrix-core path may exceed it)",
+                          unit="Top/s", steps=10)
+                os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
+            try:
+                gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100]" + (" (VALU kernel)" if sfx == "i32" else ""), sfx, n, n, n, A, B,
+                          am.toHip(A), am.toHip(B), peak=ceil.get(key),
+                          peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s", unit="Top/s", steps=10)
+            finally:
+                os.environ.pop("AM_HIP_GEMM_I32_PATH", None)
     pa = rng(3001).standard_normal((1024, 2048)); pb = rng(3002).standard_normal((1024, 6144))
     C0 = rng(3003).standard_normal((2048, 3072))
     gemm_case("f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C)", "f64", 2048, 3072, 1024, pa.T, pb[:, ::2],
@@ -339,7 +361,9 @@ def run_only(am, timer, which, steps, warmup):
     if which == "chain":
         r = bench_chain(am, timer, steps, warmup)
         return dict(only=which, hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"])
-    if which == "gemm_i32":
+    if which in ("gemm_i32", "gemm_i32_valu"):
+        if which == "gemm_i32_valu":
+            os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"   # the vector-ALU kernel instead of the digit-sliced matrix-core path
         n = 4096
         A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
         B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
@@ -379,7 +403,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true",
                     help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_f64", "bcast_add", "copy", "chain", "sum_rows", "sum_cols", "softmax", "maxpool"],
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "sum_rows", "sum_cols", "softmax", "maxpool"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -445,3 +445,63 @@ def test_integer_mid_size_balanced_split(hip, oracle, sfx):
         dC = hip.empty((M, N), dt)
         hip.gemm(1, hip.toHip(A), hip.toHip(B), 0, dC)
         assert np.array_equal(dC.toCpu(), oracle.matmul(A, B))
+
+
+@pytest.mark.parametrize("tile", ["0", "1"])
+def test_int32_digit_sliced_matrix_core_path(hip, oracle, tile, monkeypatch):
+    """int32 products on the int8 matrix cores (four balanced base-256 digits, ten digit-pair
+    products, Horner recombination modulo 2^32), forced on for every shape and both tile shapes:
+    digit boundaries (±127, ±128, ±129 in every byte position), INT_MIN / INT_MAX, full-range random
+    values with long K (accumulators wrap many times), ragged M / N / K, strided and transposed
+    operands, column-major and strided destinations, every alpha / beta case. Bit-exact."""
+    monkeypatch.setenv("AM_HIP_GEMM_I32_PATH", "mfma")
+    monkeypatch.setenv("AM_HIP_GEMM_TILE_I8", tile)
+    dt = np.int32
+    info = np.iinfo(dt)
+    edge = np.array([0, 1, -1, 127, 128, 129, -127, -128, -129, 255, 256, -255, -256, 32767, 32768, -32768, -32769,
+                     2**23 - 1, 2**23, -2**23, 2**24 + 127, 2**24 + 128, -(2**24) - 129, info.max, info.min, info.max - 128,
+                     info.min + 128, 0x7F7F7F7F, -0x7F7F7F80, 0x00800080 - 2**31], dtype=np.int64).astype(dt)
+    rng = np.random.default_rng(seed_of("digits", tile))
+    for shape in [(30, 30, 30), (1, 1, 1), (257, 129, 300), (64, 500, 1000), (300, 257, 4099), (513, 511, 129)]:
+        M, N, K = shape
+        say("digit path", tile, shape)
+        A = rng.choice(edge, size=(M, K)) if K <= 300 else fill(rng, (M, K), dt, info.min, info.max)
+        B = rng.choice(edge, size=(K, N)) if K <= 300 else fill(rng, (K, N), dt, info.min, info.max)
+        C = fill(rng, (M, N), dt, info.min, info.max)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        for alpha, beta in [(1, 0), (1, 1), (-3, 7), (info.min, info.max)]:
+            want = oracle.gemm_strided(alpha, A, B, beta, C.copy())
+            assert np.array_equal(want, oracle.closed_gemm_int_fast(alpha, A, B, beta, C)) or K > 300
+            dC = hip.toHip(C)
+            hip.gemm(alpha, dA, dB, beta, dC)
+            assert np.array_equal(dC.toCpu(), want), f"{shape} a={alpha} b={beta}"
+        # transposed / stepped operands, column-major and stepped destinations
+        dAt = hip.toHip(np.ascontiguousarray(A.T)).transpose()
+        B2 = fill(rng, (K, 2 * N), dt, info.min, info.max)
+        dCt = hip.toHip(np.zeros((N, M), dtype=dt)).transpose()
+        hip.gemm(1, dAt, hip.toHip(B2)[:, ::2], 0, dCt)
+        assert np.array_equal(dCt.toCpu(), oracle.matmul(A, np.ascontiguousarray(B2[:, ::2]))), f"{shape} views"
+        wide = fill(rng, (M, 2 * N), dt, info.min, info.max)
+        dW = hip.toHip(wide)
+        want = wide.copy()
+        oracle.gemm_strided(5, A, B, -2, want[:, ::2])
+        hip.gemm(5, dA, dB, -2, dW[:, ::2])
+        assert np.array_equal(dW.toCpu(), want), f"{shape} stepped destination"
+
+
+def test_int32_paths_agree_at_size(hip, oracle, monkeypatch):
+    """2048^3 and a ragged 1500 x 1300 x 1700 product: the automatic choice, the matrix-core path
+    and the VALU path give the same bits (and those of the CPU oracle)."""
+    rng = np.random.default_rng(77)
+    for shape in [(2048, 2048, 2048), (1500, 1300, 1700)]:
+        M, N, K = shape
+        A, B = fill(rng, (M, K), np.int32, -2**31, 2**31 - 1), fill(rng, (K, N), np.int32, -2**31, 2**31 - 1)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        want = oracle.matmul(A, B)
+        for path in (None, "mfma", "valu"):
+            say("i32 paths", shape, path)
+            if path is None:
+                monkeypatch.delenv("AM_HIP_GEMM_I32_PATH", raising=False)
+            else:
+                monkeypatch.setenv("AM_HIP_GEMM_I32_PATH", path)
+            assert np.array_equal((dA * dB).toCpu(), want), f"{shape} path {path}"
