@@ -1,4 +1,4 @@
-// Exact int32 GEMM on the int8 matrix cores of gfx950 by digit slicing.
+// Exact int32 and int64 GEMM on the int8 matrix cores of gfx950 by digit slicing.
 //
 // An int32 is written in four balanced base-256 digits, x = d0 + 2^8 d1 + 2^16 d2 + 2^24 d3 (mod 2^32),
 // each d in [-128, 127]. Modulo 2^32 the product of two such numbers only needs the ten digit pairs
@@ -23,6 +23,10 @@
 //                  instead of ten) and the k slabs of each pair as one long k loop (LDS ring of 3 slabs, fragments double-buffered in registers, as in the
 //                  float kernels); between two values of s the accumulators are shifted left by 8
 //                  (Horner form of the sum over s). Padded planes mean no bounds tests in the loop.
+//
+// int64 works the same way with eight digits and the 36 pairs i + j <= 7. The matrix cores
+// accumulate in 32 bits, which holds one pair's sum over k exactly while k * 2^14 < 2^31; after each
+// pair the 32-bit accumulators are sign-extended into a 64-bit set, which takes the Horner shifts.
 #pragma once
 #include <type_traits>
 #include "gemm_common.h"
@@ -40,18 +44,21 @@ constexpr int kKPad = 128;     // ... and to this many k (largest slab)
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-// The four balanced digits of four neighbouring k, packed as one 32-bit word per plane.
-__device__ __forceinline__ void digits_of4(const int32_t (&x)[4], uint32_t (&w)[4]) {
+// The balanced digits of four neighbouring k, packed as one 32-bit word per plane.
+template <typename T>
+__device__ __forceinline__ void digits_of4(const T (&x)[4], uint32_t (&w)[sizeof(T)]) {
+  constexpr int ND = (int)sizeof(T);
+  using U = std::make_unsigned_t<T>;
 #pragma unroll
-  for (int d = 0; d < 4; ++d) w[d] = 0;
+  for (int d = 0; d < ND; ++d) w[d] = 0;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    uint32_t ux = (uint32_t)x[e];
+    U ux = (U)x[e];
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
+    for (int d = 0; d < ND; ++d) {
       const int32_t dig = (int32_t)(int8_t)(ux & 0xFFu);
       w[d] |= ((uint32_t)dig & 0xFFu) << (8 * e);
-      ux = (ux - (uint32_t)dig) >> 8;
+      ux = (ux - (U)(T)dig) >> 8;
     }
   }
 }
@@ -62,10 +69,12 @@ __device__ __forceinline__ void digits_of4(const int32_t (&x)[4], uint32_t (&w)[
 // lanes to a 128-byte row segment.
 // flags[d] is set to 1 when plane d holds a non-zero digit anywhere (the product kernel skips the
 // digit pairs of empty planes: operands with small entries have only one or two non-empty planes).
-__global__ __launch_bounds__(256) void split_digits(const int32_t* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t K,
+template <typename T>
+__global__ __launch_bounds__(256) void split_digits(const T* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t K,
                                                     int8_t* P, int64_t MNp, int64_t Kp, int kfast, uint32_t* flags) {
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-  __shared__ int32_t tile[32][129];
+  constexpr int ND = (int)sizeof(T);
+  __shared__ T tile[32][129];
   const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
@@ -78,41 +87,48 @@ __global__ __launch_bounds__(256) void split_digits(const int32_t* X, int64_t ld
   __syncthreads();
   const int64_t plane = MNp * Kp;
   const int k16 = threadIdx.x & 7, mn = threadIdx.x >> 3;
-  u4 out[4];
-  uint32_t nz[4] = {0, 0, 0, 0};
+  u4 out[ND];
+  uint32_t nz[ND];
+#pragma unroll
+  for (int d = 0; d < ND; ++d) nz[d] = 0;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const int32_t xs[4] = {tile[mn][k16 * 16 + g * 4], tile[mn][k16 * 16 + g * 4 + 1], tile[mn][k16 * 16 + g * 4 + 2],
+    const T xs[4] = {tile[mn][k16 * 16 + g * 4], tile[mn][k16 * 16 + g * 4 + 1], tile[mn][k16 * 16 + g * 4 + 2],
                            tile[mn][k16 * 16 + g * 4 + 3]};
-    uint32_t w[4];   // one 4-byte word (4 consecutive k) per digit plane
-    digits_of4(xs, w);
+    uint32_t w[ND];   // one 4-byte word (4 consecutive k) per digit plane
+    digits_of4<T>(xs, w);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) { out[d][g] = w[d]; nz[d] |= w[d]; }
+    for (int d = 0; d < ND; ++d) { out[d][g] = w[d]; nz[d] |= w[d]; }
   }
   int8_t* dst = P + (mn0 + mn) * Kp + k0 + k16 * 16;
 #pragma unroll
-  for (int d = 0; d < 4; ++d) *(u4*)(dst + d * plane) = out[d];
+  for (int d = 0; d < ND; ++d) *(u4*)(dst + d * plane) = out[d];
 #pragma unroll
-  for (int d = 0; d < 4; ++d)   // at most one atomic per wavefront and plane, none once the flag is up
+  for (int d = 0; d < ND; ++d)   // at most one atomic per wavefront and plane, none once the flag is up
     if (__ballot(nz[d] != 0) != 0 && (threadIdx.x & 63) == 0 && flags[d] == 0) atomicOr(&flags[d], 1u);
 }
 
+template <typename T>
 struct DigitArgs {
-  const int8_t* PA; const int8_t* PB;   // [4][Mp][Kp], [4][Np][Kp]
-  const uint32_t* flags;                // [0..3]: planes of A that are not all zero, [4..7]: planes of B
+  const int8_t* PA; const int8_t* PB;   // [ND][Mp][Kp], [ND][Np][Kp] with ND = sizeof(T) digits
+  const uint32_t* flags;                // [0..ND-1]: planes of A that are not all zero, [ND..2ND-1]: planes of B
   int64_t Mp, Np, Kp;
-  int32_t* C; int64_t c_m, c_n;
+  T* C; int64_t c_m, c_n;
   int64_t M, N;
-  int32_t alpha, beta;
+  T alpha, beta;
   int tiles_m, tiles_n;
 };
 
 // WAVES_M x WAVES_N wavefronts, each with TM x TN accumulator tiles of 32 x 32; BK k (bytes) per slab.
-// The digit sums are evaluated in Horner form, s = 3 first: after the pairs of one s the accumulators
-// are shifted left by 8 and go on accumulating the pairs of s - 1, so one accumulator set suffices
-// (everything modulo 2^32, which both the shift and the matrix cores respect).
-template <int WAVES_M, int WAVES_N, int TM, int TN, int BK>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(DigitArgs p) {
+// The digit sums are evaluated in Horner form, the highest s first: after the pairs of one s the
+// accumulators are shifted left by 8 and go on accumulating the pairs of s - 1, so one accumulator set
+// suffices (int32: everything modulo 2^32, which both the shift and the matrix cores respect; int64:
+// the 32-bit accumulators of one pair are exact and are added into 64-bit ones when the pair ends).
+template <typename T, int WAVES_M, int WAVES_N, int TM, int TN, int BK>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(DigitArgs<T> p) {
+  using U = std::make_unsigned_t<T>;
+  constexpr int ND = (int)sizeof(T), NPAIRS = ND * (ND + 1) / 2;
+  constexpr bool WIDE = sizeof(T) == 8;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int WM = TM * 32, WN = TN * 32, BM = WAVES_M * WM, BN = WAVES_N * WN, NKS = BK / 32, QN = BK / 16;
   constexpr int LDA = BM + (QN >= 8 ? 1 : 8 / QN), LDB = BN + (QN >= 8 ? 1 : 8 / QN);   // 16-byte slots per k-group plane
@@ -148,15 +164,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
     gb[i] = p.PB + (n0 + mn) * p.Kp + q * 16;
     lds_b[i] = (q * LDB + mn) * 16;
   }
-  // The digit pairs to multiply: (s, i) with i + j = s <= 3, s = 3 first, restricted to planes
+  // The digit pairs to multiply: (s, i) with i + j = s <= ND - 1, the highest s first, restricted to planes
   // that hold something. tab_shift[pr] = how far the accumulators move left before pair pr (the
   // Horner steps between its s and the previous pair's), tab_shift[n_pairs] = the final shift.
-  __shared__ int tab_a[10], tab_b[10], tab_shift[11], tab_n;
+  __shared__ int tab_a[NPAIRS], tab_b[NPAIRS], tab_shift[NPAIRS + 1], tab_n;
   if (threadIdx.x == 0) {
     int n = 0, prev_s = -1;
-    for (int s = 3; s >= 0; --s)
+    for (int s = ND - 1; s >= 0; --s)
       for (int i = 0; i <= s; ++i)
-        if (p.flags[i] != 0 && p.flags[4 + s - i] != 0) {
+        if (p.flags[i] != 0 && p.flags[ND + s - i] != 0) {
           tab_a[n] = i; tab_b[n] = s - i;
           tab_shift[n] = prev_s < 0 ? 0 : 8 * (prev_s - s);
           prev_s = s;
@@ -169,22 +185,28 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
   const int n_pairs = tab_n;
   const int64_t slabs_per_pair = p.Kp / BK;
   const int64_t total = (int64_t)n_pairs * slabs_per_pair;
-  // slab number -> offsets of its A and B slabs
-  auto offsets = [&](int64_t t, int64_t& oa, int64_t& ob) {
-    int64_t pr = t / slabs_per_pair;
-    const int64_t k0 = (t - pr * slabs_per_pair) * BK;
-    if (pr > n_pairs - 1) pr = n_pairs - 1;   // slabs fetched past the end re-read the last pair (never multiplied)
-    oa = tab_a[pr] * planeA + k0;
-    ob = tab_b[pr] * planeB + k0;
-  };
+  // Slabs are fetched in order; (f_oa, f_ob) are the offsets of the next one's A and B parts.
+  // Fetches past the last slab re-read it (never multiplied).
+  int f_pr = 0;
+  int64_t f_k = 0;
+  int64_t f_oa = n_pairs > 0 ? tab_a[0] * planeA : 0, f_ob = n_pairs > 0 ? tab_b[0] * planeB : 0;
   v4i ra[NVA], rb[NVB];
-  auto fetch = [&](int64_t t) {
-    int64_t oa, ob;
-    offsets(t, oa, ob);
+  auto fetch = [&]() {
 #pragma unroll
-    for (int i = 0; i < NVA; ++i) ra[i] = *(const v4i*)(ga[i] + oa);
+    for (int i = 0; i < NVA; ++i) ra[i] = *(const v4i*)(ga[i] + f_oa + f_k);
 #pragma unroll
-    for (int i = 0; i < NVB; ++i) rb[i] = *(const v4i*)(gb[i] + ob);
+    for (int i = 0; i < NVB; ++i) rb[i] = *(const v4i*)(gb[i] + f_ob + f_k);
+    f_k += BK;
+    if (f_k == p.Kp) {
+      if (f_pr + 1 < n_pairs) {
+        ++f_pr;
+        f_k = 0;
+        f_oa = tab_a[f_pr] * planeA;
+        f_ob = tab_b[f_pr] * planeB;
+      } else {
+        f_k -= BK;
+      }
+    }
   };
   auto commit = [&](int buf) {
 #pragma unroll
@@ -210,79 +232,100 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  auto shift_acc = [&](int sh) {
+  uint64_t wide[WIDE ? TM : 1][WIDE ? TN : 1][WIDE ? 16 : 1];
+  if constexpr (WIDE) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = (int)((uint32_t)acc[i][j][r] << sh);
+        for (int r = 0; r < 16; ++r) wide[i][j][r] = 0;
+  }
+  // End of a pair: int64 moves the pair's exact 32-bit sums into the 64-bit accumulators; then the
+  // Horner shift (0 when the next pair has the same s).
+  auto end_pair = [&](int sh) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if constexpr (WIDE) {
+            wide[i][j][r] = (wide[i][j][r] + (uint64_t)(int64_t)acc[i][j][r]) << sh;
+            acc[i][j][r] = 0;
+          } else {
+            acc[i][j][r] = (int)((uint32_t)acc[i][j][r] << sh);
+          }
+        }
   };
 
   if (total > 0) {   // (every plane of an operand empty: the product is zero)
   // prologue: slabs 0 and 1 in LDS, slab 2 in registers
-  fetch(0); commit(0);
-  fetch(1); commit(1);
-  fetch(2);
+  fetch(); commit(0);
+  fetch(); commit(1);
+  fetch();
   __syncthreads();
   read_frags(std::integral_constant<int, 0>(), 0, 0);
 
   int cur = 0;
-  int64_t next_pair = slabs_per_pair;   // first slab of the next pair
-  int pr = 0;
-  for (int64_t t = 0; t < total; ++t) {
-    const int nxt = cur == 2 ? 0 : cur + 1, nxt2 = nxt == 2 ? 0 : nxt + 1;
+  int64_t t = 0;
+  // One inner loop per pair keeps the end-of-pair arithmetic out of the slab loop's body (as a
+  // branch inside one flat loop the compiler turns it into selects executed for every slab).
+  for (int pr = 0; pr < n_pairs; ++pr) {
+    const int64_t t_end = t + slabs_per_pair;
+    for (; t < t_end; ++t) {
+      const int nxt = cur == 2 ? 0 : cur + 1, nxt2 = nxt == 2 ? 0 : nxt + 1;
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      if (ks + 1 < NKS) {
-        if (ks & 1) read_frags(std::integral_constant<int, 0>(), cur, ks + 1);
-        else read_frags(std::integral_constant<int, 1>(), cur, ks + 1);
-      } else {
-        read_frags(std::integral_constant<int, 0>(), nxt, 0);   // NKS is even
-        commit(nxt2);                                            // slab t + 2
-        fetch(t + 3);
+      for (int ks = 0; ks < NKS; ++ks) {
+        if (ks + 1 < NKS) {
+          if (ks & 1) read_frags(std::integral_constant<int, 0>(), cur, ks + 1);
+          else read_frags(std::integral_constant<int, 1>(), cur, ks + 1);
+        } else {
+          read_frags(std::integral_constant<int, 0>(), nxt, 0);   // NKS is even
+          commit(nxt2);                                            // slab t + 2
+          fetch();                                                 // slab t + 3
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      cur = nxt;
     }
-    __syncthreads();
-    cur = nxt;
-    if (t + 1 == next_pair) {   // a pair is done: Horner step(s) down to the next pair's s (or to s = 0 at the end)
-      ++pr;
-      next_pair += slabs_per_pair;
-      const int sh = tab_shift[pr];
-      if (sh != 0) shift_acc(sh);
-    }
+    // the pair is done: Horner step(s) down to the next pair's s (or to s = 0 after the last one)
+    const int sh = tab_shift[pr + 1];
+    if (WIDE || sh != 0) end_pair(sh);
   }
   }
 
-  // C <- alpha * AB + beta * C in the ring of 32-bit integers (same case analysis as the other kernels)
-  const uint32_t alpha = (uint32_t)p.alpha, beta = (uint32_t)p.beta;
+  // C <- alpha * AB + beta * C in the ring of integers modulo 2^32 / 2^64 (same case analysis as the other kernels)
+  const U alpha = (U)p.alpha, beta = (U)p.beta;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int64_t col = n0 + wave_n * WN + j * 32 + lrow;
-      uint32_t cv[16];
+      U cv[16];
       if (beta != 0) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int64_t row = m0 + wave_m * WM + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
-          cv[r] = (row < p.M && col < p.N) ? (uint32_t)p.C[row * p.c_m + col * p.c_n] : 0u;
+          cv[r] = (row < p.M && col < p.N) ? (U)p.C[row * p.c_m + col * p.c_n] : (U)0;
         }
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t row = m0 + wave_m * WM + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
         if (row < p.M && col < p.N) {
-          uint32_t v = alpha * (uint32_t)acc[i][j][r];
+          U v;
+          if constexpr (WIDE) v = alpha * (U)wide[i][j][r];
+          else v = alpha * (U)(uint32_t)acc[i][j][r];
           if (beta != 0) v += beta * cv[r];
-          p.C[row * p.c_m + col * p.c_n] = (int32_t)v;
+          p.C[row * p.c_m + col * p.c_n] = (T)v;
         }
       }
     }
@@ -290,62 +333,80 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
 
 // Padded operand extents and the estimated time of the digit-sliced product for both tile shapes
 // (rounds of one workgroup per CU x measured time per tile and k, plus the two splitting passes).
+// The estimate is for operands that use every digit; the kernel itself skips empty planes.
 struct Plan { int64_t Mp, Np, Kp; bool big; double est_us; };
-static inline Plan plan(const Args<int32_t>& g) {
+template <typename T>
+static inline Plan plan(const Args<T>& g) {
+  constexpr bool WIDE = sizeof(T) == 8;
   Plan pl;
   pl.Mp = (g.M + kRowPad - 1) / kRowPad * kRowPad;
   pl.Np = (g.N + kRowPad - 1) / kRowPad * kRowPad;
   pl.Kp = (g.K + kKPad - 1) / kKPad * kKPad;
   const int64_t cus = num_cus();
   const int64_t tb = (pl.Mp / 256) * (pl.Np / 256), ts = (pl.Mp / 256) * (pl.Np / 128);
-  // microseconds per k for one tile (all ten digit pairs), measured at 4096^3: 0.162 (256 x 256), 0.098 (256 x 128)
-  const double cost_big = (double)((tb + cus - 1) / cus) * 0.162 * pl.Kp, cost_small = (double)((ts + cus - 1) / cus) * 0.098 * pl.Kp;
-  pl.big = cost_big <= cost_small;
-  const char* force = getenv("AM_HIP_GEMM_TILE_I8");   // 1: 256 x 256 tiles, 0: 256 x 128 (tests)
-  if (force && *force) pl.big = atoi(force) != 0;
-  const double split_us = 2 * 5.0 + 8.0 * (double)(pl.Mp + pl.Np) * pl.Kp / 2.8e6;   // reads 4 B, writes 4 B per element
+  // microseconds per k for one tile, measured at 4096^3. int32 (ten pairs): 0.162 (256 x 256), 0.098 (256 x 128);
+  // int64 (36 pairs, 256 x 128 only: the 64-bit accumulators leave no registers for the larger tile): 0.38.
+  const double cost_big = (double)((tb + cus - 1) / cus) * 0.162 * pl.Kp;
+  const double cost_small = (double)((ts + cus - 1) / cus) * (WIDE ? 0.38 : 0.098) * pl.Kp;
+  pl.big = !WIDE && cost_big <= cost_small;
+  if (!WIDE) {
+    const char* force = getenv("AM_HIP_GEMM_TILE_I8");   // 1: 256 x 256 tiles, 0: 256 x 128 (tests)
+    if (force && *force) pl.big = atoi(force) != 0;
+  }
+  // the splitting passes read sizeof(T) and write sizeof(T) bytes per element, at about 2.8 TB/s
+  const double split_us = 2 * 5.0 + 2.0 * sizeof(T) * (double)(pl.Mp + pl.Np) * pl.Kp / 2.8e6;
   pl.est_us = (pl.big ? cost_big : cost_small) + split_us;
   return pl;
 }
 
 // Whether the digit-sliced path may take this product at all: not part of a batch, not being
-// recorded into a graph (it allocates its planes). AM_HIP_GEMM_I32_PATH = "valu" / "mfma" forces a
-// path (tests, benchmarks); returns 0 = no, 1 = if estimated faster, 2 = forced.
-static inline int applicable(const Args<int32_t>& g) {
-  const char* e = getenv("AM_HIP_GEMM_I32_PATH");
+// recorded into a graph (it allocates its planes), and for int64 k small enough that one pair's
+// sum over k fits the 32-bit accumulators of the matrix cores (k * 2^14 < 2^31).
+// AM_HIP_GEMM_I32_PATH / AM_HIP_GEMM_I64_PATH = "valu" / "mfma" forces a path (tests, benchmarks);
+// returns 0 = no, 1 = if estimated faster, 2 = forced.
+template <typename T>
+static inline int applicable(const Args<T>& g) {
+  const char* e = getenv(sizeof(T) == 8 ? "AM_HIP_GEMM_I64_PATH" : "AM_HIP_GEMM_I32_PATH");
   if (e && *e == 'v') return 0;
   if (g.batch > 1 || capturing()) return 0;
+  if (sizeof(T) == 8 && g.K > 131071) return 0;
   if (e && *e == 'm') return 2;
   return (g.M >= 64 && g.N >= 64 && g.K >= 256) ? 1 : 0;
 }
 
-static int run(const Args<int32_t>& g, const Plan& pl) {
+template <typename T>
+static int run(const Args<T>& g, const Plan& pl) {
+  constexpr int ND = (int)sizeof(T);
   const int64_t Mp = pl.Mp, Np = pl.Np, Kp = pl.Kp;
   const bool big = pl.big;   // 256 x 256 tiles: a 128 x 64 tile per wavefront, fewest LDS reads per matrix instruction
-  if (Mp / 64 >= ((int64_t)1 << 31) || Np / 64 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return 1;
+  if (Mp / 32 >= ((int64_t)1 << 31) || Np / 32 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return 1;
   const int64_t tiles_m = Mp / 256, tiles_n = big ? Np / 256 : Np / 128;
   if (tiles_m * tiles_n >= ((int64_t)1 << 31)) return 1;
   void* ws = nullptr;
-  const size_t plane_bytes = (size_t)4 * (size_t)(Mp + Np) * (size_t)Kp;
+  const size_t plane_bytes = (size_t)ND * (size_t)(Mp + Np) * (size_t)Kp;
   if (am_hip_malloc(plane_bytes + 256, &ws) != AM_OK) return 1;
   int8_t* PA = (int8_t*)ws;
-  int8_t* PB = PA + 4 * Mp * Kp;
+  int8_t* PB = PA + (int64_t)ND * Mp * Kp;
   uint32_t* flags = (uint32_t*)((char*)ws + plane_bytes);
-  if (hipMemsetAsync(flags, 0, 8 * sizeof(uint32_t), stream()) != hipSuccess) { (void)hipGetLastError(); (void)am_hip_free(ws); return 1; }
-  auto split = [&](const int32_t* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t MNp, int kfast, int8_t* P, uint32_t* fl) {
-    hipLaunchKernelGGL(split_digits, dim3((unsigned)(MNp / 32), (unsigned)(Kp / 128)), dim3(256), 0, stream(), X, ld_mn, ld_k, MN,
+  if (hipMemsetAsync(flags, 0, 2 * ND * sizeof(uint32_t), stream()) != hipSuccess) { (void)hipGetLastError(); (void)am_hip_free(ws); return 1; }
+  auto split = [&](const T* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t MNp, int kfast, int8_t* P, uint32_t* fl) {
+    hipLaunchKernelGGL(split_digits<T>, dim3((unsigned)(MNp / 32), (unsigned)(Kp / 128)), dim3(256), 0, stream(), X, ld_mn, ld_k, MN,
                        g.K, P, MNp, Kp, kfast, fl);
   };
   split(g.A, g.a_mn, g.a_k, g.M, Mp, g.a_kfast, PA, flags);
-  split(g.B, g.b_mn, g.b_k, g.N, Np, g.b_kfast, PB, flags + 4);
-  DigitArgs d;
+  split(g.B, g.b_mn, g.b_k, g.N, Np, g.b_kfast, PB, flags + ND);
+  DigitArgs<T> d;
   d.PA = PA; d.PB = PB; d.flags = flags; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
   d.alpha = g.alpha; d.beta = g.beta;
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
-  if (big) hipLaunchKernelGGL((gemm_i8_digits<2, 4, 4, 2, 64>), grid, block, 0, stream(), d);
-  else hipLaunchKernelGGL((gemm_i8_digits<4, 2, 2, 2, 128>), grid, block, 0, stream(), d);
+  if constexpr (sizeof(T) == 8) {
+    hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64>), grid, block, 0, stream(), d);
+  } else {
+    if (big) hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 4, 2, 64>), grid, block, 0, stream(), d);
+    else hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 128>), grid, block, 0, stream(), d);
+  }
   const int rc = check_launch("gemm_i8_digits");
   // The planes go back to the allocator's cache at once: whoever gets the block next reaches it
   // through the same stream, after this product.

@@ -117,34 +117,75 @@ def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
                        f"oracle/laser_gemm.c (laser blocking, 6x16 AVX2+FMA register tile, OpenMP)")
 
 
+def digit_pairs(A, B):
+    """How many of the ten digit-pair products (i + j <= 3) the digit-sliced int32 GEMM runs for these
+    operands: a balanced base-256 digit plane that is zero everywhere is skipped."""
+    def planes(X):
+        x = X.astype(np.int64)
+        flags = []
+        for _ in range(4):
+            d = ((x + 128) & 255) - 128
+            flags.append(bool(d.any()))
+            x = (x - d) >> 8
+        return flags
+    fa, fb = planes(A), planes(B)
+    return sum(1 for i in range(4) for j in range(4 - i) if fa[i] and fb[j])
+
+
 def other_workloads(am, timer, steps, warmup, ceilings):
     out = []
-    # --- int32 GEMM 4096^3, entries in [-100, 100], wraparound accumulate: digit-sliced on the int8
-    # matrix cores (the library's choice at this size), and the VALU kernel beside it
+    # --- int32 GEMM 4096^3, wraparound accumulate: digit-sliced on the int8 matrix cores (the
+    # library's choice at this size) with the VALU kernel beside it. Entries in [-100, 100] fit one
+    # base-256 digit, so one of the ten digit-pair products runs; entries over the whole int32 range
+    # need all ten.
     n = 4096
-    A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
-    B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
-    dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
     k = max(3, steps // 4)
-    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
-    tops = 2.0 * n ** 3 / (ev / k) / 1e12
-    os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
-    try:
-        _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
-    finally:
-        del os.environ["AM_HIP_GEMM_I32_PATH"]
-    valu_tops = 2.0 * n ** 3 / (ev_valu / k) / 1e12
     peak = ceilings.get("valu_int32_mac")
-    out.append(dict(workload="i32 GEMM 4096^3 (wraparound; ten int8 digit-pair products on the matrix cores, incl. the digit-splitting passes)",
-                    unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
-                    roofline=dict(bound="mfma", achieved=round(10 * tops, 1), peak=MFMA_I8_PEAK_TOPS,
-                                  unit="int8 TOP/s executed (20*M*N*K per product: 10 digit pairs)",
-                                  frac=round(10 * tops / MFMA_I8_PEAK_TOPS, 4)),
-                    valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / k * 1e3, 4),
-                                     roofline=dict(bound="valu (measured int32 multiply-add ceiling; no matrix instruction for int32)",
-                                                   achieved=round(valu_tops, 3), peak=peak, unit="Top/s",
-                                                   frac=round(valu_tops / peak, 4) if peak else None)),
-                    speedup_over_valu_ceiling=round(tops / peak, 2) if peak else None))
+    for label, lo, hi in (("entries in [-100, 100]", -100, 100), ("entries over the whole int32 range", -2 ** 31, 2 ** 31 - 1)):
+        A = np.random.default_rng(2001).integers(lo, hi, (n, n), endpoint=True).astype(np.int32)
+        B = np.random.default_rng(2002).integers(lo, hi, (n, n), endpoint=True).astype(np.int32)
+        pairs = digit_pairs(A, B)
+        dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
+        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+        tops = 2.0 * n ** 3 / (ev / k) / 1e12
+        entry = dict(workload=f"i32 GEMM 4096^3, {label} (wraparound; {pairs} of 10 int8 digit-pair products on the matrix cores, "
+                              "timed with the two digit-splitting passes)",
+                     unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                     roofline=dict(bound="mfma", achieved=round(pairs * tops, 1), peak=MFMA_I8_PEAK_TOPS,
+                                   unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, splitting passes included",
+                                   frac=round(pairs * tops / MFMA_I8_PEAK_TOPS, 4)),
+                     speedup_over_valu_ceiling=round(tops / peak, 2) if peak else None)
+        if lo == -100:
+            os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
+            try:
+                _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+            finally:
+                del os.environ["AM_HIP_GEMM_I32_PATH"]
+            valu_tops = 2.0 * n ** 3 / (ev_valu / k) / 1e12
+            entry["valu_kernel"] = dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / k * 1e3, 4),
+                                        roofline=dict(bound="valu (measured int32 multiply-add ceiling; no matrix instruction for int32)",
+                                                      achieved=round(valu_tops, 3), peak=peak, unit="Top/s",
+                                                      frac=round(valu_tops / peak, 4) if peak else None))
+        out.append(entry)
+        del dA, dB, dC
+    # --- int64 GEMM 4096^3, entries in [-100, 100]: eight digits, 36 pairs at most, one of them here
+    A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
+    B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
+    dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int64)
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+    os.environ["AM_HIP_GEMM_I64_PATH"] = "valu"
+    try:
+        _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), 3, 1)
+    finally:
+        del os.environ["AM_HIP_GEMM_I64_PATH"]
+    peak64 = ceilings.get("valu_int64_mac")
+    valu_tops = 2.0 * n ** 3 / (ev_valu / 3) / 1e12
+    out.append(dict(workload="i64 GEMM 4096^3, entries in [-100, 100] (wraparound; 1 of 36 int8 digit-pair products on the matrix cores, "
+                             "timed with the two digit-splitting passes)",
+                    unit="Top/s", dtype="i64", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                    valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / 3 * 1e3, 4),
+                                     roofline=dict(bound="valu (measured int64 multiply-add ceiling)", achieved=round(valu_tops, 3),
+                                                   peak=peak64, unit="Top/s", frac=round(valu_tops / peak64, 4) if peak64 else None))))
     del dA, dB, dC
     # --- float64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C), M=2048 N=3072 K=1024
     pa = np.random.default_rng(3001).standard_normal((1024, 2048))
@@ -279,18 +320,29 @@ def config_report(am, timer, L):
         for n in (1500, 4096):
             A = rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(dt)
             B = rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(dt)
-            if sfx == "i32":   # the library's own choice (int8 matrix cores at these sizes), then the VALU kernel
-                gemm_case(f"i32 GEMM {n}^3, entries in [-100, 100] (library's choice: digit-sliced int8 MFMA)", sfx, n, n, n, A, B,
-                          am.toHip(A), am.toHip(B), peak=ceil.get(key),
-                          peak_used=f"measured VALU i32 multiply-add ceiling {ceil.get(key)} Top/s (the matrix-core path may exceed it)",
-                          unit="Top/s", steps=10)
-                os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
+            env = f"AM_HIP_GEMM_{sfx.upper()}_PATH"
+            # the library's own choice (digit slicing on the int8 matrix cores at these sizes), then the VALU kernel
+            gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100] (library's choice: digit-sliced int8 MFMA)", sfx, n, n, n, A, B,
+                      am.toHip(A), am.toHip(B), peak=ceil.get(key),
+                      peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s (the matrix-core path may exceed it)",
+                      unit="Top/s", steps=10)
+            os.environ[env] = "valu"
             try:
-                gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100]" + (" (VALU kernel)" if sfx == "i32" else ""), sfx, n, n, n, A, B,
+                gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100] (VALU kernel)", sfx, n, n, n, A, B,
                           am.toHip(A), am.toHip(B), peak=ceil.get(key),
                           peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s", unit="Top/s", steps=10)
             finally:
-                os.environ.pop("AM_HIP_GEMM_I32_PATH", None)
+                os.environ.pop(env, None)
+    n = 4096
+    for sfx, dt, key in (("i32", np.int32, "valu_int32_mac"), ("i64", np.int64, "valu_int64_mac")):
+        info = np.iinfo(dt)
+        A = rng(2001).integers(info.min, info.max, (n, n), endpoint=True).astype(dt)
+        B = rng(2002).integers(info.min, info.max, (n, n), endpoint=True).astype(dt)
+        gemm_case(f"{sfx} GEMM {n}^3, entries over the whole {sfx} range (library's choice: digit-sliced int8 MFMA, all "
+                  f"{10 if sfx == 'i32' else 36} digit pairs)",
+                  sfx, n, n, n, A, B, am.toHip(A), am.toHip(B), peak=ceil.get(key),
+                  peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s (the matrix-core path may exceed it)",
+                  unit="Top/s", steps=10)
     pa = rng(3001).standard_normal((1024, 2048)); pb = rng(3002).standard_normal((1024, 6144))
     C0 = rng(3003).standard_normal((2048, 3072))
     gemm_case("f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C)", "f64", 2048, 3072, 1024, pa.T, pb[:, ::2],

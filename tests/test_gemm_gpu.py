@@ -505,3 +505,91 @@ def test_int32_paths_agree_at_size(hip, oracle, monkeypatch):
             else:
                 monkeypatch.setenv("AM_HIP_GEMM_I32_PATH", path)
             assert np.array_equal((dA * dB).toCpu(), want), f"{shape} path {path}"
+
+
+def test_int64_digit_sliced_matrix_core_path(hip, oracle, monkeypatch):
+    """int64 products on the int8 matrix cores (eight balanced base-256 digits, 36 digit-pair
+    products, each pair's exact 32-bit sums widened to 64 bits before the Horner shifts), forced on
+    for every shape: digit boundaries in every byte position, INT64_MIN / INT64_MAX, full-range
+    random values, ragged M / N / K, strided and transposed operands and destinations, every
+    alpha / beta case. Bit-exact."""
+    monkeypatch.setenv("AM_HIP_GEMM_I64_PATH", "mfma")
+    dt = np.int64
+    info = np.iinfo(dt)
+    base = [0, 1, -1, 127, 128, 129, -127, -128, -129, 255, 256, -255, -256, 32767, 32768, -32768, -32769]
+    edge = list(base) + [info.max, info.min, info.max - 128, info.min + 128, 0x7F7F7F7F7F7F7F7F, 0x7F7F7F7F7F7F7F80,
+                         -0x7F7F7F7F7F7F7F80, 0x0080008000800080]
+    for byte in range(1, 8):
+        edge += [sgn * (v << (8 * byte)) + off for sgn in (1, -1) for v in (127, 128, 129) for off in (0, 127, -128)
+                 if info.min <= sgn * (v << (8 * byte)) + off <= info.max]
+    edge = np.array(edge, dtype=dt)
+    rng = np.random.default_rng(seed_of("digits64"))
+    for shape in [(30, 30, 30), (1, 1, 1), (257, 129, 300), (64, 500, 1000), (300, 257, 4099), (513, 511, 129)]:
+        M, N, K = shape
+        say("int64 digit path", shape)
+        A = rng.choice(edge, size=(M, K)) if K <= 300 else fill(rng, (M, K), dt, info.min, info.max)
+        B = rng.choice(edge, size=(K, N)) if K <= 300 else fill(rng, (K, N), dt, info.min, info.max)
+        C = fill(rng, (M, N), dt, info.min, info.max)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        for alpha, beta in [(1, 0), (1, 1), (-3, 7), (info.min, info.max)]:
+            want = oracle.gemm_strided(alpha, A, B, beta, C.copy())
+            assert np.array_equal(want, oracle.closed_gemm_int_fast(alpha, A, B, beta, C)) or K > 300
+            dC = hip.toHip(C)
+            hip.gemm(alpha, dA, dB, beta, dC)
+            assert np.array_equal(dC.toCpu(), want), f"{shape} a={alpha} b={beta}"
+        dAt = hip.toHip(np.ascontiguousarray(A.T)).transpose()
+        B2 = fill(rng, (K, 2 * N), dt, info.min, info.max)
+        dCt = hip.toHip(np.zeros((N, M), dtype=dt)).transpose()
+        hip.gemm(1, dAt, hip.toHip(B2)[:, ::2], 0, dCt)
+        assert np.array_equal(dCt.toCpu(), oracle.matmul(A, np.ascontiguousarray(B2[:, ::2]))), f"{shape} views"
+        wide = fill(rng, (M, 2 * N), dt, info.min, info.max)
+        dW = hip.toHip(wide)
+        want = wide.copy()
+        oracle.gemm_strided(5, A, B, -2, want[:, ::2])
+        hip.gemm(5, dA, dB, -2, dW[:, ::2])
+        assert np.array_equal(dW.toCpu(), want), f"{shape} stepped destination"
+
+
+def test_int64_digit_path_accumulator_limit(hip, oracle, monkeypatch):
+    """Every digit of every entry is -128 and k = 131071: each pair's sum over k is 131071 * 2^14, the
+    largest a 32-bit accumulator can be asked to hold exactly. One k more and the product is handed to
+    the VALU kernel, forced or not. Entries with few digits take the same code with most planes skipped."""
+    monkeypatch.setenv("AM_HIP_GEMM_I64_PATH", "mfma")
+    v = np.array([0x7F7F7F7F7F7F7F80], dtype=np.int64)[0]    # = -128 * (1 + 2^8 + ... + 2^56) modulo 2^64
+    for K in (131071, 131072):
+        say("int64 digit path, accumulator limit", K)
+        A = np.full((64, K), v, dtype=np.int64)
+        B = np.full((K, 64), v, dtype=np.int64)
+        B[::7, 3] = -1
+        A[5, ::3] = 127
+        got = (hip.toHip(A) * hip.toHip(B)).toCpu()
+        assert np.array_equal(got, oracle.matmul(A, B)), K
+    rng = np.random.default_rng(seed_of("digits64-small"))
+    for lo, hi in [(-100, 100), (-40000, 40000), (-2**40, 2**40)]:
+        say("int64 digit path, few digits", lo, hi)
+        A, B = fill(rng, (300, 700), np.int64, lo, hi), fill(rng, (700, 260), np.int64, lo, hi)
+        B[:, 5] = 0
+        assert np.array_equal((hip.toHip(A) * hip.toHip(B)).toCpu(), oracle.matmul(A, B)), (lo, hi)
+    Z = np.zeros((128, 512), dtype=np.int64)
+    C = fill(rng, (128, 128), np.int64, -9, 9)
+    dC = hip.toHip(C)
+    hip.gemm(3, hip.toHip(Z), hip.toHip(fill(rng, (512, 128), np.int64, -9, 9)), 2, dC)     # all planes of A empty
+    assert np.array_equal(dC.toCpu(), 2 * C)
+
+
+def test_int64_paths_agree_at_size(hip, oracle, monkeypatch):
+    """2048 x 1024 x 2048 and a ragged 1500 x 1300 x 1700 product: the automatic choice, the
+    matrix-core path and the VALU path give the same bits (and those of the CPU oracle)."""
+    rng = np.random.default_rng(78)
+    for shape in [(2048, 1024, 2048), (1500, 1300, 1700)]:
+        M, N, K = shape
+        A, B = fill(rng, (M, K), np.int64, -2**63, 2**63 - 1), fill(rng, (K, N), np.int64, -2**63, 2**63 - 1)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        want = oracle.matmul(A, B)
+        for path in (None, "mfma", "valu"):
+            say("i64 paths", shape, path)
+            if path is None:
+                monkeypatch.delenv("AM_HIP_GEMM_I64_PATH", raising=False)
+            else:
+                monkeypatch.setenv("AM_HIP_GEMM_I64_PATH", path)
+            assert np.array_equal((dA * dB).toCpu(), want), f"{shape} path {path}"
