@@ -12,15 +12,16 @@
 // the order of the additions. Ten int8 products cost 10 x 2MNK int8 operations at 5 POP/s of matrix
 // throughput against 2MNK multiply-adds at the 61 Top/s the vector ALU sustains.
 //
-// Two passes:
+// Three passes:
+//   scan_digits    marks the digit planes of both operands that hold a non-zero digit anywhere (entries
+//                  within +-127 have one such plane, the others are neither written nor multiplied);
 //   split_digits   strided int32 operand (any view) -> four int8 planes [digit][row][k], k contiguous,
 //                  rows padded to the tile size and k to the slab size with zeros (a 32 x 128 tile
 //                  goes through LDS so that both the strided read and the k-contiguous write are
 //                  coalesced);
 //   gemm_i8_digits one workgroup of eight wavefronts per 256 x 256 (or 256 x 128) tile of C. For
-//                  s = 3..0 it walks the pairs (i, s - i) whose planes are not empty (split_digits
-//                  flags the planes that hold a non-zero digit: entries within +-127 need one pair
-//                  instead of ten) and the k slabs of each pair as one long k loop (LDS ring of 3 slabs, fragments double-buffered in registers, as in the
+//                  s = 3..0 it walks the pairs (i, s - i) whose planes are not empty (entries within
+//                  +-127 need one pair instead of ten) and the k slabs of each pair as one long k loop (LDS ring of 3 slabs, fragments double-buffered in registers, as in the
 //                  float kernels); between two values of s the accumulators are shifted left by 8
 //                  (Horner form of the sum over s). Padded planes mean no bounds tests in the loop.
 //
@@ -44,74 +45,182 @@ constexpr int kKPad = 128;     // ... and to this many k (largest slab)
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-// The balanced digits of four neighbouring k, packed as one 32-bit word per plane.
+// All balanced base-256 digits of x at once, one per byte: digit d is ((x + 128 (1 + 2^8 + .. + 2^(8d))) >> 8d)
+// mod 256 - 128 (the carry of "x - digit" into the next byte is that of adding 128 to it), and adding
+// the higher bytes of the constant does not reach byte d; subtracting 128 from a byte is flipping its top bit.
+template <typename T>
+__device__ __forceinline__ std::make_unsigned_t<T> balanced_digits(T x) {
+  using U = std::make_unsigned_t<T>;
+  constexpr U C = (U)0x8080808080808080ull;
+  return ((U)x + C) ^ C;
+}
+
+// The digits of four neighbouring k, packed as one 32-bit word per plane (a 4 x 4 byte transpose per
+// 32 bits of element width; v_perm_b32 picks bytes 0-3 from its second and 4-7 from its first operand).
 template <typename T>
 __device__ __forceinline__ void digits_of4(const T (&x)[4], uint32_t (&w)[sizeof(T)]) {
-  constexpr int ND = (int)sizeof(T);
   using U = std::make_unsigned_t<T>;
+  U y[4];
 #pragma unroll
-  for (int d = 0; d < ND; ++d) w[d] = 0;
+  for (int e = 0; e < 4; ++e) y[e] = balanced_digits<T>(x[e]);
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    U ux = (U)x[e];
+  for (int h = 0; h < (int)sizeof(T) / 4; ++h) {
+    uint32_t v[4];
 #pragma unroll
-    for (int d = 0; d < ND; ++d) {
-      const int32_t dig = (int32_t)(int8_t)(ux & 0xFFu);
-      w[d] |= ((uint32_t)dig & 0xFFu) << (8 * e);
-      ux = (ux - (U)(T)dig) >> 8;
+    for (int e = 0; e < 4; ++e) v[e] = (uint32_t)(y[e] >> (h * 32 % (8 * (int)sizeof(T))));
+    const uint32_t a = __builtin_amdgcn_perm(v[1], v[0], 0x05010400u), b = __builtin_amdgcn_perm(v[1], v[0], 0x07030602u);
+    const uint32_t c = __builtin_amdgcn_perm(v[3], v[2], 0x05010400u), d = __builtin_amdgcn_perm(v[3], v[2], 0x07030602u);
+    w[4 * h + 0] = __builtin_amdgcn_perm(c, a, 0x05040100u);
+    w[4 * h + 1] = __builtin_amdgcn_perm(c, a, 0x07060302u);
+    w[4 * h + 2] = __builtin_amdgcn_perm(d, b, 0x05040100u);
+    w[4 * h + 3] = __builtin_amdgcn_perm(d, b, 0x07060302u);
+  }
+}
+
+// Both operands of one product, as the two splitting passes see them: X(mn, k) = X[mn * ld_mn + k * ld_k],
+// planes P[d][mn][k] (mn < MNp, k < Kp). flags[op * ND + d] == gen says that plane d of operand op
+// holds a non-zero digit somewhere; gen is a number that grows with every product, so the flags of
+// earlier products read as unset and the flag words never need clearing.
+template <typename T>
+struct SplitArgs {
+  const T* X[2];
+  int64_t ld_mn[2], ld_k[2], MN[2], MNp[2];
+  int kfast[2];
+  int mode[2];      // 0: element loads; 1 / 2: 16-byte loads along k / along mn (unit stride there, 16-byte aligned lines)
+  int8_t* P[2];
+  int64_t K, Kp;
+  uint32_t* flags;
+  uint32_t gen;
+};
+
+// The 32 (mn) x 128 (k) tile at (mn0, k0) of operand op, 16 elements per lane of a 256-lane workgroup:
+// every load is issued before f(mn, k, value) sees the first element (zeros outside the operand).
+template <typename T, typename F>
+__device__ __forceinline__ void visit_tile(const SplitArgs<T>& a, int op, int64_t mn0, int64_t k0, F&& f) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(VEC)));
+  const T* X = a.X[op];
+  const int64_t ld_mn = a.ld_mn[op], ld_k = a.ld_k[op], MN = a.MN[op], K = a.K;
+  const int mode = a.mode[op];
+  const int t = (int)threadIdx.x;
+  if (mode == 1) {
+    constexpr int KV = 128 / VEC, ROWS = 256 / KV, PASSES = 32 / ROWS;
+    vec_t v[PASSES];
+    const int k = (t % KV) * VEC;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const int mn = t / KV + i * ROWS;
+      const T* src = X + (mn0 + mn) * ld_mn + (k0 + k);
+      if ((mn0 + mn) < MN && (k0 + k + VEC) <= K) {
+        v[i] = *(const vec_t*)src;
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[i][e] = ((mn0 + mn) < MN && (k0 + k + e) < K) ? src[e] : (T)0;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) f(t / KV + i * ROWS, k + e, v[i][e]);
+  } else if (mode == 2) {
+    constexpr int MV = 32 / VEC, ROWS = 256 / MV, PASSES = 128 / ROWS;
+    vec_t v[PASSES];
+    const int mn = (t % MV) * VEC;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const int k = t / MV + i * ROWS;
+      const T* src = X + (mn0 + mn) + (k0 + k) * ld_k;
+      if ((k0 + k) < K && (mn0 + mn + VEC) <= MN) {
+        v[i] = *(const vec_t*)src;
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[i][e] = ((k0 + k) < K && (mn0 + mn + e) < MN) ? src[e] : (T)0;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) f(mn + e, t / MV + i * ROWS, v[i][e]);
+  } else {
+    const int kfast = a.kfast[op];
+    T x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int e = t + i * 256;
+      int mn, k;
+      if (kfast) { k = e & 127; mn = e >> 7; } else { mn = e & 31; k = e >> 5; }
+      const bool ok = (mn0 + mn) < MN && (k0 + k) < K;
+      x[i] = ok ? X[(mn0 + mn) * ld_mn + (k0 + k) * ld_k] : (T)0;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int e = t + i * 256;
+      int mn, k;
+      if (kfast) { k = e & 127; mn = e >> 7; } else { mn = e & 31; k = e >> 5; }
+      f(mn, k, x[i]);
     }
   }
 }
 
-// X(mn, k) = X[mn * ld_mn + k * ld_k]  ->  planes P[d][mn][k] (mn < MNp, k < Kp), zero padded.
-// One workgroup moves a 32 (mn) x 128 (k) tile through LDS: the read walks whichever of the two
-// directions is the faster one in memory (kfast), the write is 16 bytes per lane and plane, eight
-// lanes to a 128-byte row segment.
-// flags[d] is set to 1 when plane d holds a non-zero digit anywhere (the product kernel skips the
-// digit pairs of empty planes: operands with small entries have only one or two non-empty planes).
+// First pass (reads only): marks the digit planes that hold anything. Operands with small entries
+// have one or two such planes; the others are neither written by split_digits nor multiplied.
+// blockIdx.z picks the operand; one workgroup looks at a 32 (mn) x 128 (k) tile.
 template <typename T>
-__global__ __launch_bounds__(256) void split_digits(const T* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t K,
-                                                    int8_t* P, int64_t MNp, int64_t Kp, int kfast, uint32_t* flags) {
-  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void scan_digits(SplitArgs<T> a) {
   constexpr int ND = (int)sizeof(T);
-  __shared__ T tile[32][129];
+  using U = std::make_unsigned_t<T>;
+  const int op = (int)blockIdx.z;
   const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int e = threadIdx.x + i * 256;
-    int mn, k;
-    if (kfast) { k = e & 127; mn = e >> 7; } else { mn = e & 31; k = e >> 5; }
-    const bool ok = (mn0 + mn) < MN && (k0 + k) < K;
-    tile[mn][k] = ok ? X[(mn0 + mn) * ld_mn + (k0 + k) * ld_k] : 0;
-  }
-  __syncthreads();
-  const int64_t plane = MNp * Kp;
-  const int k16 = threadIdx.x & 7, mn = threadIdx.x >> 3;
-  u4 out[ND];
+  if (mn0 >= a.MN[op]) return;
+  U seen = 0;   // byte d: OR of the digits d of this lane's elements
+  visit_tile<T>(a, op, mn0, k0, [&](int, int, T x) { seen |= balanced_digits<T>(x); });
   uint32_t nz[ND];
 #pragma unroll
-  for (int d = 0; d < ND; ++d) nz[d] = 0;
+  for (int d = 0; d < ND; ++d) nz[d] = (uint32_t)(seen >> (8 * d)) & 0xFFu;
+  uint32_t* flags = a.flags + op * ND;
+#pragma unroll
+  for (int d = 0; d < ND; ++d)   // every writer stores the same value; at most one store per wavefront and plane
+    if (__ballot(nz[d] != 0) != 0 && (threadIdx.x & 63) == 0 && flags[d] != a.gen) flags[d] = a.gen;
+}
+
+// Second pass: writes the marked planes, zero padded to MNp x Kp. One workgroup moves a 32 (mn) x
+// 128 (k) tile through LDS: the read walks whichever of the two directions is the faster one in
+// memory (kfast), the write is 16 bytes per lane and plane, eight lanes to a 128-byte row segment.
+template <typename T>
+__global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  constexpr int ND = (int)sizeof(T);
+  __shared__ __attribute__((aligned(16))) T tile[32][128 + 16 / sizeof(T)];   // rows stay 16-byte aligned
+  const int op = (int)blockIdx.z;
+  const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
+  const int64_t MNp = a.MNp[op];
+  if (mn0 >= MNp) return;
+  visit_tile<T>(a, op, mn0, k0, [&](int mn, int k, T x) { tile[mn][k] = x; });
+  __syncthreads();
+  const int64_t plane = MNp * a.Kp;
+  const int k16 = threadIdx.x & 7, mn = threadIdx.x >> 3;
+  u4 out[ND];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const T xs[4] = {tile[mn][k16 * 16 + g * 4], tile[mn][k16 * 16 + g * 4 + 1], tile[mn][k16 * 16 + g * 4 + 2],
-                           tile[mn][k16 * 16 + g * 4 + 3]};
+                     tile[mn][k16 * 16 + g * 4 + 3]};
     uint32_t w[ND];   // one 4-byte word (4 consecutive k) per digit plane
     digits_of4<T>(xs, w);
 #pragma unroll
-    for (int d = 0; d < ND; ++d) { out[d][g] = w[d]; nz[d] |= w[d]; }
+    for (int d = 0; d < ND; ++d) out[d][g] = w[d];
   }
-  int8_t* dst = P + (mn0 + mn) * Kp + k0 + k16 * 16;
+  int8_t* dst = a.P[op] + (mn0 + mn) * a.Kp + k0 + k16 * 16;
+  const uint32_t* flags = a.flags + op * ND;
 #pragma unroll
-  for (int d = 0; d < ND; ++d) *(u4*)(dst + d * plane) = out[d];
-#pragma unroll
-  for (int d = 0; d < ND; ++d)   // at most one atomic per wavefront and plane, none once the flag is up
-    if (__ballot(nz[d] != 0) != 0 && (threadIdx.x & 63) == 0 && flags[d] == 0) atomicOr(&flags[d], 1u);
+  for (int d = 0; d < ND; ++d)
+    if (flags[d] == a.gen) *(u4*)(dst + d * plane) = out[d];
 }
 
 template <typename T>
 struct DigitArgs {
   const int8_t* PA; const int8_t* PB;   // [ND][Mp][Kp], [ND][Np][Kp] with ND = sizeof(T) digits
-  const uint32_t* flags;                // [0..ND-1]: planes of A that are not all zero, [ND..2ND-1]: planes of B
+  const uint32_t* flags;                // [0..ND-1]: planes of A, [ND..2ND-1]: planes of B; == gen: not all zero
+  uint32_t gen;
   int64_t Mp, Np, Kp;
   T* C; int64_t c_m, c_n;
   int64_t M, N;
@@ -172,7 +281,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
     int n = 0, prev_s = -1;
     for (int s = ND - 1; s >= 0; --s)
       for (int i = 0; i <= s; ++i)
-        if (p.flags[i] != 0 && p.flags[ND + s - i] != 0) {
+        if (p.flags[i] == p.gen && p.flags[ND + s - i] == p.gen) {
           tab_a[n] = i; tab_b[n] = s - i;
           tab_shift[n] = prev_s < 0 ? 0 : 8 * (prev_s - s);
           prev_s = s;
@@ -382,21 +491,42 @@ static int run(const Args<T>& g, const Plan& pl) {
   if (Mp / 32 >= ((int64_t)1 << 31) || Np / 32 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return 1;
   const int64_t tiles_m = Mp / 256, tiles_n = big ? Np / 256 : Np / 128;
   if (tiles_m * tiles_n >= ((int64_t)1 << 31)) return 1;
+  // Flag words live as long as the process: every product uses a new generation number, so they are
+  // cleared only once (and again should the 32-bit counter ever wrap).
+  static uint32_t* flags = nullptr;
+  static uint32_t gen = 0;
+  if (!flags) {
+    void* f = nullptr;
+    if (am_hip_malloc(256, &f) != AM_OK) return 1;
+    flags = (uint32_t*)f;
+    gen = 0;
+  }
+  if (gen == 0 || gen == 0xFFFFFFFFu) {
+    if (hipMemsetAsync(flags, 0, 256, stream()) != hipSuccess) { (void)hipGetLastError(); return 1; }
+    gen = 0;
+  }
+  ++gen;
   void* ws = nullptr;
   const size_t plane_bytes = (size_t)ND * (size_t)(Mp + Np) * (size_t)Kp;
-  if (am_hip_malloc(plane_bytes + 256, &ws) != AM_OK) return 1;
+  if (am_hip_malloc(plane_bytes, &ws) != AM_OK) return 1;
   int8_t* PA = (int8_t*)ws;
   int8_t* PB = PA + (int64_t)ND * Mp * Kp;
-  uint32_t* flags = (uint32_t*)((char*)ws + plane_bytes);
-  if (hipMemsetAsync(flags, 0, 2 * ND * sizeof(uint32_t), stream()) != hipSuccess) { (void)hipGetLastError(); (void)am_hip_free(ws); return 1; }
-  auto split = [&](const T* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t MNp, int kfast, int8_t* P, uint32_t* fl) {
-    hipLaunchKernelGGL(split_digits<T>, dim3((unsigned)(MNp / 32), (unsigned)(Kp / 128)), dim3(256), 0, stream(), X, ld_mn, ld_k, MN,
-                       g.K, P, MNp, Kp, kfast, fl);
-  };
-  split(g.A, g.a_mn, g.a_k, g.M, Mp, g.a_kfast, PA, flags);
-  split(g.B, g.b_mn, g.b_k, g.N, Np, g.b_kfast, PB, flags + ND);
+  SplitArgs<T> sp;
+  sp.X[0] = g.A; sp.ld_mn[0] = g.a_mn; sp.ld_k[0] = g.a_k; sp.MN[0] = g.M; sp.MNp[0] = Mp; sp.kfast[0] = g.a_kfast; sp.P[0] = PA;
+  sp.X[1] = g.B; sp.ld_mn[1] = g.b_mn; sp.ld_k[1] = g.b_k; sp.MN[1] = g.N; sp.MNp[1] = Np; sp.kfast[1] = g.b_kfast; sp.P[1] = PB;
+  sp.K = g.K; sp.Kp = Kp; sp.flags = flags; sp.gen = gen;
+  constexpr int64_t VEC = 16 / (int64_t)sizeof(T);
+  for (int op = 0; op < 2; ++op) {
+    const bool aligned = ((uintptr_t)sp.X[op] & 15) == 0;
+    sp.mode[op] = (aligned && sp.ld_k[op] == 1 && sp.ld_mn[op] % VEC == 0)   ? 1
+                  : (aligned && sp.ld_mn[op] == 1 && sp.ld_k[op] % VEC == 0) ? 2
+                                                                             : 0;
+  }
+  const int64_t mx = g.M > g.N ? g.M : g.N, mxp = Mp > Np ? Mp : Np;
+  hipLaunchKernelGGL(scan_digits<T>, dim3((unsigned)((mx + 31) / 32), (unsigned)((g.K + 127) / 128), 2), dim3(256), 0, stream(), sp);
+  hipLaunchKernelGGL(split_digits<T>, dim3((unsigned)(mxp / 32), (unsigned)(Kp / 128), 2), dim3(256), 0, stream(), sp);
   DigitArgs<T> d;
-  d.PA = PA; d.PB = PB; d.flags = flags; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
+  d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
   d.alpha = g.alpha; d.beta = g.beta;
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;

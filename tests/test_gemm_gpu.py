@@ -593,3 +593,31 @@ def test_int64_paths_agree_at_size(hip, oracle, monkeypatch):
             else:
                 monkeypatch.setenv("AM_HIP_GEMM_I64_PATH", path)
             assert np.array_equal((dA * dB).toCpu(), want), f"{shape} path {path}"
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+def test_digit_path_window_views(hip, oracle, sfx, monkeypatch):
+    """Operands that are windows of larger 16-byte aligned buffers, with extents that are not
+    multiples of the 16-byte load width: the vector loads of the digit-splitting passes must stop at
+    the window's edge (what lies beyond is made large so that reading it would change the result)."""
+    monkeypatch.setenv(f"AM_HIP_GEMM_{sfx.upper()}_PATH", "mfma")
+    dt = DTYPES[sfx]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(seed_of("windows", sfx))
+    for (M, N, K) in [(61, 67, 131), (130, 35, 257), (33, 129, 62)]:
+        say("digit path windows", sfx, (M, N, K))
+        bigA = fill(rng, (M + 8, K + 24), dt, info.min, info.max)
+        bigB = fill(rng, (K + 8, N + 24), dt, info.min, info.max)
+        A_small = fill(rng, (M, K), dt, -100, 100)
+        B_small = fill(rng, (K, N), dt, -100, 100)
+        for r0, c0 in [(0, 0), (4, 8), (3, 4)]:
+            hostA, hostB = bigA.copy(), bigB.copy()
+            hostA[r0:r0 + M, c0:c0 + K] = A_small
+            hostB[r0:r0 + K, c0:c0 + N] = B_small
+            dA = hip.toHip(hostA)[r0:r0 + M, c0:c0 + K]
+            dB = hip.toHip(hostB)[r0:r0 + K, c0:c0 + N]
+            assert np.array_equal((dA * dB).toCpu(), oracle.matmul(A_small, B_small)), (M, N, K, r0, c0)
+            # the same windows transposed: unit stride along the other direction
+            dAt = hip.toHip(np.ascontiguousarray(hostA.T))[c0:c0 + K, r0:r0 + M].transpose()
+            dBt = hip.toHip(np.ascontiguousarray(hostB.T))[c0:c0 + N, r0:r0 + K].transpose()
+            assert np.array_equal((dAt * dBt).toCpu(), oracle.matmul(A_small, B_small)), (M, N, K, r0, c0, "T")
