@@ -15,15 +15,18 @@
 // Three passes:
 //   scan_digits    marks the digit planes of both operands that hold a non-zero digit anywhere (entries
 //                  within +-127 have one such plane, the others are neither written nor multiplied);
-//   split_digits   strided int32 operand (any view) -> four int8 planes [digit][row][k], k contiguous,
-//                  rows padded to the tile size and k to the slab size with zeros (a 32 x 128 tile
-//                  goes through LDS so that both the strided read and the k-contiguous write are
-//                  coalesced);
+//   split_digits   strided operand (any view) -> its marked int8 planes, rows padded to the tile size
+//                  and k to the slab size with zeros, stored as 1 KiB blocks of 32 rows x 32 k in the
+//                  register layout of the matrix instruction (a 32 x 128 tile goes through LDS so that
+//                  both the strided read and the block write are coalesced);
 //   gemm_i8_digits one workgroup of eight wavefronts per 256 x 256 (or 256 x 128) tile of C. For
-//                  s = 3..0 it walks the pairs (i, s - i) whose planes are not empty (entries within
-//                  +-127 need one pair instead of ten) and the k slabs of each pair as one long k loop (LDS ring of 3 slabs, fragments double-buffered in registers, as in the
-//                  float kernels); between two values of s the accumulators are shifted left by 8
-//                  (Horner form of the sum over s). Padded planes mean no bounds tests in the loop.
+//                  s = 3..0 it walks the pairs (i, s - i) whose planes are not empty and the k slabs
+//                  of each pair as one long k loop: blocks go from global memory straight into an
+//                  LDS ring (global_load_lds_dwordx4, no register stage, no LDS write instructions),
+//                  several slabs ahead; fragments are double-buffered in registers. Between two
+//                  values of s the accumulators are shifted left by 8 (Horner form of the sum over
+//                  s). Padded planes mean no bounds tests in the loop. The kernel is bound by LDS
+//                  reads (six 1 KiB fragment reads per eight matrix instructions and wavefront).
 //
 // int64 works the same way with eight digits and the 36 pairs i + j <= 7. The matrix cores
 // accumulate in 32 bits, which holds one pair's sum over k exactly while k * 2^14 < 2^31; after each
@@ -209,7 +212,10 @@ __global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
 #pragma unroll
     for (int d = 0; d < ND; ++d) out[d][g] = w[d];
   }
-  int8_t* dst = a.P[op] + (mn0 + mn) * a.Kp + k0 + k16 * 16;
+  // Planes are stored in the order the matrix instruction wants them: one 1 KiB block per 32 rows x 32 k,
+  // lane (row % 32) + 32 * ((k % 32) / 16) of a wavefront owning 16 consecutive k. The product kernel moves
+  // whole blocks from global memory into LDS without passing through registers.
+  int8_t* dst = a.P[op] + ((((mn0 >> 5) * (a.Kp >> 5) + (k0 >> 5) + (k16 >> 1)) * 64 + (k16 & 1) * 32 + mn) << 4);
   const uint32_t* flags = a.flags + op * ND;
 #pragma unroll
   for (int d = 0; d < ND; ++d)
@@ -218,7 +224,7 @@ __global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
 
 template <typename T>
 struct DigitArgs {
-  const int8_t* PA; const int8_t* PB;   // [ND][Mp][Kp], [ND][Np][Kp] with ND = sizeof(T) digits
+  const int8_t* PA; const int8_t* PB;   // ND = sizeof(T) digit planes each, in 1 KiB fragment blocks [rows/32][Kp/32][64 lanes][16]
   const uint32_t* flags;                // [0..ND-1]: planes of A, [ND..2ND-1]: planes of B; == gen: not all zero
   uint32_t gen;
   int64_t Mp, Np, Kp;
@@ -233,45 +239,44 @@ struct DigitArgs {
 // accumulators are shifted left by 8 and go on accumulating the pairs of s - 1, so one accumulator set
 // suffices (int32: everything modulo 2^32, which both the shift and the matrix cores respect; int64:
 // the 32-bit accumulators of one pair are exact and are added into 64-bit ones when the pair ends).
-template <typename T, int WAVES_M, int WAVES_N, int TM, int TN, int BK>
+template <typename T, int WAVES_M, int WAVES_N, int TM, int TN, int BK, int RING>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(DigitArgs<T> p) {
   using U = std::make_unsigned_t<T>;
   constexpr int ND = (int)sizeof(T), NPAIRS = ND * (ND + 1) / 2;
   constexpr bool WIDE = sizeof(T) == 8;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int WM = TM * 32, WN = TN * 32, BM = WAVES_M * WM, BN = WAVES_N * WN, NKS = BK / 32, QN = BK / 16;
-  constexpr int LDA = BM + (QN >= 8 ? 1 : 8 / QN), LDB = BN + (QN >= 8 ? 1 : 8 / QN);   // 16-byte slots per k-group plane
-  constexpr int SLAB_A = QN * LDA * 16, SLAB_B = QN * LDB * 16;
-  static_assert(NKS % 2 == 0 && (BM * QN) % NT == 0 && (BN * QN) % NT == 0, "tile shape");
-  __shared__ __attribute__((aligned(16))) int8_t sA[3][SLAB_A];
-  __shared__ __attribute__((aligned(16))) int8_t sB[3][SLAB_B];
+  // One slab = NKS k-steps of 32; its blocks in LDS: A's (BM / 32) x NKS, then B's (BN / 32) x NKS, 1 KiB each.
+  constexpr int NW = WAVES_M * WAVES_N, NBA = BM / 32 * NKS, NBB = BN / 32 * NKS;
+  constexpr int LPA = NBA / NW, LPB = NBB / NW;            // block loads per wavefront and slab
+  constexpr int SLAB = (NBA + NBB) * 1024;   // RING slabs in LDS: the one being multiplied and RING - 1 on their way
+  static_assert(NKS % 2 == 0 && NBA % NW == 0 && NBB % NW == 0 && QN > 0 && RING >= 3 && (RING - 2) * (LPA + LPB) <= 15, "tile shape");
+  __shared__ __attribute__((aligned(1024))) int8_t sbuf[RING][SLAB];
 
   int tile_m, tile_n;
   tile_of_block((int)blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int lrow = lane & 31, kg = lane >> 5;
 
-  // global -> register -> LDS: rows x QN sixteen-byte vectors per operand slab; QN neighbouring
-  // lanes cover one BK-byte row segment.
-  constexpr int NVA = BM * QN / NT, NVB = BN * QN / NT;
+  // global -> LDS without registers: a wavefront's load instruction moves one block, lane l's 16 bytes to
+  // LDS offset 16 l of the block. Wavefront w takes blocks w, w + NW, ... of each operand.
   const int64_t planeA = p.Mp * p.Kp, planeB = p.Np * p.Kp;
-  const int8_t* ga[NVA]; const int8_t* gb[NVB];
-  int lds_a[NVA], lds_b[NVB];
+  const int64_t kb32 = p.Kp >> 5;
+  const int8_t* ga[LPA]; const int8_t* gb[LPB];
+  int lds_a[LPA], lds_b[LPB];
 #pragma unroll
-  for (int i = 0; i < NVA; ++i) {
-    const int v = threadIdx.x + i * NT;
-    const int q = v % QN, mn = v / QN;
-    ga[i] = p.PA + (m0 + mn) * p.Kp + q * 16;
-    lds_a[i] = (q * LDA + mn) * 16;
+  for (int i = 0; i < LPA; ++i) {
+    const int b = wave + i * NW;
+    ga[i] = p.PA + ((((m0 >> 5) + b / NKS) * kb32 + b % NKS) << 10) + lane * 16;
+    lds_a[i] = b * 1024;
   }
 #pragma unroll
-  for (int i = 0; i < NVB; ++i) {
-    const int v = threadIdx.x + i * NT;
-    const int q = v % QN, mn = v / QN;
-    gb[i] = p.PB + (n0 + mn) * p.Kp + q * 16;
-    lds_b[i] = (q * LDB + mn) * 16;
+  for (int i = 0; i < LPB; ++i) {
+    const int b = wave + i * NW;
+    gb[i] = p.PB + ((((n0 >> 5) + b / NKS) * kb32 + b % NKS) << 10) + lane * 16;
+    lds_b[i] = (NBA + b) * 1024;
   }
   // The digit pairs to multiply: (s, i) with i + j = s <= ND - 1, the highest s first, restricted to planes
   // that hold something. tab_shift[pr] = how far the accumulators move left before pair pr (the
@@ -294,43 +299,43 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
   const int n_pairs = tab_n;
   const int64_t slabs_per_pair = p.Kp / BK;
   const int64_t total = (int64_t)n_pairs * slabs_per_pair;
-  // Slabs are fetched in order; (f_oa, f_ob) are the offsets of the next one's A and B parts.
-  // Fetches past the last slab re-read it (never multiplied).
+  // Slabs are fetched in order, RING - 1 ahead of the one being multiplied; (f_oa, f_ob) + f_k are the
+  // offsets of the next one's A and B blocks. Fetches past the last slab re-read it (never multiplied).
   int f_pr = 0;
-  int64_t f_k = 0;
+  int64_t f_k = 0;   // in bytes of a block row: 1024 per k-step of 32
   int64_t f_oa = n_pairs > 0 ? tab_a[0] * planeA : 0, f_ob = n_pairs > 0 ? tab_b[0] * planeB : 0;
-  v4i ra[NVA], rb[NVB];
-  auto fetch = [&]() {
+  // The load is written as inline assembly: the compiler's own wait-count pass would otherwise drain
+  // every outstanding load (vmcnt(0)) before the next LDS read, which undoes the prefetch. The waits
+  // that order these loads before the reads of their slab are the explicit s_waitcnt before each barrier.
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(&sbuf[0][0]);
+  auto block_to_lds = [&](const int8_t* src, int lds_off) {
+    const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)lds_off);
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0) : "memory", "m0");
+  };
+  auto fetch = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < NVA; ++i) ra[i] = *(const v4i*)(ga[i] + f_oa + f_k);
+    for (int i = 0; i < LPA; ++i) block_to_lds(ga[i] + f_oa + f_k, buf * SLAB + lds_a[i]);
 #pragma unroll
-    for (int i = 0; i < NVB; ++i) rb[i] = *(const v4i*)(gb[i] + f_ob + f_k);
-    f_k += BK;
-    if (f_k == p.Kp) {
+    for (int i = 0; i < LPB; ++i) block_to_lds(gb[i] + f_ob + f_k, buf * SLAB + lds_b[i]);
+    f_k += NKS * 1024;
+    if (f_k == (kb32 << 10)) {
       if (f_pr + 1 < n_pairs) {
         ++f_pr;
         f_k = 0;
         f_oa = tab_a[f_pr] * planeA;
         f_ob = tab_b[f_pr] * planeB;
       } else {
-        f_k -= BK;
+        f_k -= NKS * 1024;
       }
     }
-  };
-  auto commit = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < NVA; ++i) *(v4i*)(sA[buf] + lds_a[i]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < NVB; ++i) *(v4i*)(sB[buf] + lds_b[i]) = rb[i];
   };
   v4i af[2][TM], bf[2][TN];
   auto read_frags = [&](auto parity_tag, int buf, int ks) {
     constexpr int P = decltype(parity_tag)::value;
-    const int q = ks * 2 + kg;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) af[P][i] = *(const v4i*)(sA[buf] + (q * LDA + wave_m * WM + i * 32 + lrow) * 16);
+    for (int i = 0; i < TM; ++i) af[P][i] = *(const v4i*)(sbuf[buf] + (((wave_m * TM + i) * NKS + ks) << 10) + lane * 16);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) bf[P][j] = *(const v4i*)(sB[buf] + (q * LDB + wave_n * WN + j * 32 + lrow) * 16);
+    for (int j = 0; j < TN; ++j) bf[P][j] = *(const v4i*)(sbuf[buf] + ((NBA + (wave_n * TN + j) * NKS + ks) << 10) + lane * 16);
   };
 
   v16i acc[TM][TN];
@@ -369,10 +374,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
   };
 
   if (total > 0) {   // (every plane of an operand empty: the product is zero)
-  // prologue: slabs 0 and 1 in LDS, slab 2 in registers
-  fetch(); commit(0);
-  fetch(); commit(1);
-  fetch();
+  // prologue: slabs 0 and 1 on their way into LDS; slab 0 must have landed
+#pragma unroll
+  for (int r = 0; r < RING - 1; ++r) fetch(r);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | ((RING - 2) * (LPA + LPB)));   // all but the loads of the later slabs: slab 0 is in
   __syncthreads();
   read_frags(std::integral_constant<int, 0>(), 0, 0);
 
@@ -383,16 +388,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
   for (int pr = 0; pr < n_pairs; ++pr) {
     const int64_t t_end = t + slabs_per_pair;
     for (; t < t_end; ++t) {
-      const int nxt = cur == 2 ? 0 : cur + 1, nxt2 = nxt == 2 ? 0 : nxt + 1;
+      const int nxt = cur == RING - 1 ? 0 : cur + 1, last = cur == 0 ? RING - 1 : cur - 1;
+      fetch(last);   // slab t + RING - 1; its buffer held slab t - 1, which every wavefront left before the last barrier
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         if (ks + 1 < NKS) {
           if (ks & 1) read_frags(std::integral_constant<int, 0>(), cur, ks + 1);
           else read_frags(std::integral_constant<int, 1>(), cur, ks + 1);
         } else {
+          // Slab t + 1 was requested RING - 2 slabs ago: wait for this wavefront's part of it (vmcnt <= the
+          // loads of the later slabs) and for its own outstanding reads of slab t (lgkmcnt 0: the matrix
+          // instructions below need them anyway), then for everyone's. A bare barrier: the fence of
+          // __syncthreads would drain the later slabs' loads as well.
+          __builtin_amdgcn_s_waitcnt(0x0070 | ((RING - 2) * (LPA + LPB)));
+          __builtin_amdgcn_s_barrier();
           read_frags(std::integral_constant<int, 0>(), nxt, 0);   // NKS is even
-          commit(nxt2);                                            // slab t + 2
-          fetch();                                                 // slab t + 3
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -402,7 +412,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
-      __syncthreads();
       cur = nxt;
     }
     // the pair is done: Horner step(s) down to the next pair's s (or to s = 0 after the last one)
@@ -532,10 +541,10 @@ static int run(const Args<T>& g, const Plan& pl) {
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
   if constexpr (sizeof(T) == 8) {
-    hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64>), grid, block, 0, stream(), d);
+    hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 5>), grid, block, 0, stream(), d);
   } else {
-    if (big) hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 4, 2, 64>), grid, block, 0, stream(), d);
-    else hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 128>), grid, block, 0, stream(), d);
+    if (big) hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 4, 2, 64, 4>), grid, block, 0, stream(), d);
+    else hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 5>), grid, block, 0, stream(), d);
   }
   const int rc = check_launch("gemm_i8_digits");
   // The planes go back to the allocator's cache at once: whoever gets the block next reaches it
