@@ -21,6 +21,10 @@ import os
 import sys
 import time
 
+# The CPU legs use OpenMP: their worker threads should sleep, not spin, once a parallel region is
+# over, or they compete with the thread that launches the GPU kernels timed right afterwards.
+os.environ.setdefault("OMP_WAIT_POLICY", "passive")
+
 import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -118,18 +122,17 @@ def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
 
 
 def digit_pairs(A, B):
-    """How many of the ten digit-pair products (i + j <= 3) the digit-sliced int32 GEMM runs for these
-    operands: a balanced base-256 digit plane that is zero everywhere is skipped."""
-    def planes(X):
-        x = X.astype(np.int64)
-        flags = []
-        for _ in range(4):
-            d = ((x + 128) & 255) - 128
-            flags.append(bool(d.any()))
-            x = (x - d) >> 8
-        return flags
+    """How many of the digit-pair products (i + j < number of bytes: ten for int32, 36 for int64) the
+    digit-sliced integer GEMM runs for these operands: a balanced base-256 digit plane that is zero
+    everywhere is skipped."""
+    nd = A.dtype.itemsize
+    mask = np.uint64(0x8080808080808080 >> (8 * (8 - nd)))
+    def planes(X):   # digit d of x is byte d of (x + 0x80..80) ^ 0x80..80, modulo 2^(8 nd)
+        y = X.astype(np.int64).view(np.uint64)
+        y = (y + mask) ^ mask
+        return [bool(((y >> np.uint64(8 * d)) & np.uint64(0xFF)).any()) for d in range(nd)]
     fa, fb = planes(A), planes(B)
-    return sum(1 for i in range(4) for j in range(4 - i) if fa[i] and fb[j])
+    return sum(1 for i in range(nd) for j in range(nd - i) if fa[i] and fb[j])
 
 
 def other_workloads(am, timer, steps, warmup, ceilings):
@@ -149,10 +152,10 @@ def other_workloads(am, timer, steps, warmup, ceilings):
         wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
         tops = 2.0 * n ** 3 / (ev / k) / 1e12
         entry = dict(workload=f"i32 GEMM 4096^3, {label} (wraparound; {pairs} of 10 int8 digit-pair products on the matrix cores, "
-                              "timed with the two digit-splitting passes)",
+                              "timed with the scan and split passes)",
                      unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
                      roofline=dict(bound="mfma", achieved=round(pairs * tops, 1), peak=MFMA_I8_PEAK_TOPS,
-                                   unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, splitting passes included",
+                                   unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, scan and split passes included",
                                    frac=round(pairs * tops / MFMA_I8_PEAK_TOPS, 4)),
                      speedup_over_valu_ceiling=round(tops / peak, 2) if peak else None)
         if lo == -100:
@@ -181,8 +184,11 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     peak64 = ceilings.get("valu_int64_mac")
     valu_tops = 2.0 * n ** 3 / (ev_valu / 3) / 1e12
     out.append(dict(workload="i64 GEMM 4096^3, entries in [-100, 100] (wraparound; 1 of 36 int8 digit-pair products on the matrix cores, "
-                             "timed with the two digit-splitting passes)",
+                             "timed with the scan and split passes)",
                     unit="Top/s", dtype="i64", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                    roofline=dict(bound="mfma", achieved=round(2.0 * n ** 3 / (ev / k) / 1e12, 1), peak=MFMA_I8_PEAK_TOPS,
+                                  unit="int8 TOP/s executed (1 digit pair x 2*M*N*K) over the whole call, scan and split passes included",
+                                  frac=round(2.0 * n ** 3 / (ev / k) / 1e12 / MFMA_I8_PEAK_TOPS, 4)),
                     valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / 3 * 1e3, 4),
                                      roofline=dict(bound="valu (measured int64 multiply-add ceiling)", achieved=round(valu_tops, 3),
                                                    peak=peak64, unit="Top/s", frac=round(valu_tops / peak64, 4) if peak64 else None))))
@@ -287,12 +293,10 @@ def config_report(am, timer, L):
         dC = am.toHip(C_host)
         am.gemm(alpha, dA, dB, beta, dC)
         got = dC.toCpu().copy()
-        want = am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy())
-        if beta == 0:
-            _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3)
-        else:   # accumulating into C: keep the values bounded by restoring nothing, only time it
-            _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3)
+        # (with beta != 0 the timed calls go on accumulating into C: only their time is used)
+        _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3)
         gpu_s = ev / steps
+        want = am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy())
         cpu_s = cpu_time(lambda: am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy() if beta != 0 else C_host))
         ops = 2.0 * M * N * K
         row = dict(config=config, dtype=sfx, shape=[M, N, K], gpu_ms=round(gpu_s * 1e3, 4),
@@ -322,10 +326,11 @@ def config_report(am, timer, L):
             B = rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(dt)
             env = f"AM_HIP_GEMM_{sfx.upper()}_PATH"
             # the library's own choice (digit slicing on the int8 matrix cores at these sizes), then the VALU kernel
-            gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100] (library's choice: digit-sliced int8 MFMA)", sfx, n, n, n, A, B,
-                      am.toHip(A), am.toHip(B), peak=ceil.get(key),
-                      peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s (the matrix-core path may exceed it)",
-                      unit="Top/s", steps=10)
+            pairs = digit_pairs(A, B)
+            gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100] (library's choice: digit-sliced int8 MFMA, {pairs} digit pair)", sfx, n, n, n,
+                      A, B, am.toHip(A), am.toHip(B), peak=MFMA_I8_PEAK_TOPS / pairs,
+                      peak_used=f"int8 MFMA 5000 TOP/s / {pairs} digit-pair product(s) executed; whole call incl. the scan and split passes",
+                      unit="Top/s", steps=20)
             os.environ[env] = "valu"
             try:
                 gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100] (VALU kernel)", sfx, n, n, n, A, B,
@@ -338,10 +343,10 @@ def config_report(am, timer, L):
         info = np.iinfo(dt)
         A = rng(2001).integers(info.min, info.max, (n, n), endpoint=True).astype(dt)
         B = rng(2002).integers(info.min, info.max, (n, n), endpoint=True).astype(dt)
-        gemm_case(f"{sfx} GEMM {n}^3, entries over the whole {sfx} range (library's choice: digit-sliced int8 MFMA, all "
-                  f"{10 if sfx == 'i32' else 36} digit pairs)",
-                  sfx, n, n, n, A, B, am.toHip(A), am.toHip(B), peak=ceil.get(key),
-                  peak_used=f"measured VALU {sfx} multiply-add ceiling {ceil.get(key)} Top/s (the matrix-core path may exceed it)",
+        pairs = digit_pairs(A, B)
+        gemm_case(f"{sfx} GEMM {n}^3, entries over the whole {sfx} range (library's choice: digit-sliced int8 MFMA, all {pairs} digit pairs)",
+                  sfx, n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_I8_PEAK_TOPS / pairs,
+                  peak_used=f"int8 MFMA 5000 TOP/s / {pairs} digit-pair products executed; whole call incl. the scan and split passes",
                   unit="Top/s", steps=10)
     pa = rng(3001).standard_normal((1024, 2048)); pb = rng(3002).standard_normal((1024, 6144))
     C0 = rng(3003).standard_normal((2048, 3072))
