@@ -109,6 +109,11 @@ int am_hip_graph_destroy(void* graph_exec);
  *   - K == 0 (or M == 0 or N == 0) leaves C untouched, beta is NOT applied.
  *   - integer types wrap modulo 2^32 / 2^64.
  * C must not overlap itself (no zero stride on a dimension of extent > 1) nor A or B.
+ *
+ * Large integer products run on the int8 matrix cores (the operands are split into base-256
+ * digit planes in scratch device memory taken from the block cache behind am_hip_malloc; ring
+ * arithmetic, so the bits are those of the vector-ALU kernel); small ones, batched ones and
+ * calls made while a graph is being captured use the vector-ALU kernel and allocate nothing.
  */
 int am_hip_gemm_f32(int64_t M, int64_t N, int64_t K, float alpha,
                     const float* A, int64_t rsA, int64_t csA,
