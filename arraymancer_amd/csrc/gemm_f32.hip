@@ -1,10 +1,12 @@
 // float32 GEMM entry points (MFMA path): am_hip_gemm_f32, am_hip_gemm_ex_f32.
 #include "gemm_mfma_impl.h"
+#include "gemm_small_impl.h"
 
 using namespace am;
 using namespace am::gemm;
 
 static int run_f32(Args<float>& g) {
+  if (small::applicable(g)) return small::run(g);   // few rows or columns: no LDS staging, no second kernel
   constexpr int64_t VK = 16 / (int64_t)sizeof(float);
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);

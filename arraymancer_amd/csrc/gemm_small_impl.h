@@ -1,0 +1,239 @@
+// Float GEMM for products with at most 64 rows (or, through the transposed problem, at most 64
+// columns) and a modest amount of work: the dense layers of small-batch inference, e.g.
+// [64 x 800] * [800 x 500] (src/arraymancer/nn_primitives/nnp_linear.nim:20-29) or the im2col
+// products of a small convolution (nn_primitives/fallback/conv.nim:81-106).
+//
+// The tiled kernel handles such shapes with 32 x 32 tiles, one wavefront each, a split of k
+// over workgroups and a second kernel that adds the partial tiles: a chain of global -> LDS ->
+// register round trips whose latency nothing overlaps, 10 to 14 microseconds per product. Here
+// there is no LDS staging and no second kernel:
+//   - a workgroup of W wavefronts (1..4) owns one 16 x 16 tile of C; wavefront w multiplies a
+//     contiguous share of the k range with v_mfma_*_16x16x4, loading its operand elements
+//     straight from global memory in the register layout of the instruction (lane (i, g) =
+//     (lane % 16, lane / 16) supplies A[m0 + i][k] and B[k][n0 + i] for one k per group g);
+//   - within a block of 16 k, group g takes k = 4 g + s for step s = 0..3, so an operand with unit
+//     stride along k is read with one 16-byte load per lane and block; any bijection between
+//     (step, group) and k is legal as long as A and B use the same one;
+//   - the W partial tiles are added in a fixed order through LDS and the first wavefront applies
+//     alpha / beta / bias / ReLU exactly as the tiled kernel does.
+// A wavefront keeps the loads of the next chunk of k in flight while it multiplies the current one.
+#pragma once
+#include "gemm_common.h"
+
+namespace am {
+namespace gemm {
+namespace small {
+
+template <typename T> struct M16;
+template <> struct M16<float> {
+  typedef float acc_t __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  // v_mfma_f32_16x16x4: register r of lane group g = lane / 16 holds row 4 g + r (column = lane % 16).
+  static __device__ __forceinline__ int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+template <> struct M16<double> {
+  typedef double acc_t __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  // v_mfma_f64_16x16x4: register r of lane group g holds row 4 r + g.
+  static __device__ __forceinline__ int acc_row(int r, int lane) { return 4 * r + (lane >> 4); }
+};
+
+constexpr int kMaxWaves = 4;
+
+// The four values lane group g feeds to the four steps of the 16-k block at kb: X[x + (kb + 4 g + s) * ld_k].
+template <typename T, bool VEC>
+__device__ __forceinline__ void load4(const T* x, int64_t ld_k, int64_t k, T (&out)[4]) {
+  if constexpr (VEC) {
+    constexpr int VK = 16 / (int)sizeof(T);
+    typedef T vec_t __attribute__((ext_vector_type(VK)));
+#pragma unroll
+    for (int v = 0; v < 4 / VK; ++v) {
+      const vec_t t = *(const vec_t*)(x + k + v * VK);
+#pragma unroll
+      for (int e = 0; e < VK; ++e) out[v * VK + e] = t[e];
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) out[s] = x[(k + s) * ld_k];
+  }
+}
+
+// MAXW: most wavefronts per workgroup this instantiation is launched with (it sets the register budget);
+// CHUNK: blocks of 16 k whose loads are issued together. The chunks of a wavefront's share are double
+// buffered: the loads of chunk c + 1 are in flight while chunk c is multiplied.
+template <typename T, bool AVEC, bool BVEC, int MAXW, int CHUNK>
+__global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
+  typedef typename M16<T>::acc_t acc_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][256] partial tiles, W > 1 only
+  T (*red)[256] = reinterpret_cast<T (*)[256]>(red_raw);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int i = lane & 15, g = lane >> 4;
+  const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * 16;
+  // rows / columns past the edge read the last valid one; their results are not stored
+  const int64_t arow = (m0 + i < p.M) ? m0 + i : p.M - 1, bcol = (n0 + i < p.N) ? n0 + i : p.N - 1;
+  const T* a = p.A + arow * p.a_mn;
+  const T* b = p.B + bcol * p.b_mn;
+
+  // blocks of 16 k: nfull whole ones and possibly a partial one; wavefront w takes a contiguous share
+  const int64_t nfull = p.K >> 4, nblk = (p.K + 15) >> 4;
+  const int64_t per = (nblk + nw - 1) / nw;
+  const int64_t blk0 = (int64_t)wave * per;
+  int64_t blk1 = blk0 + per;
+  if (blk1 > nblk) blk1 = nblk;
+  const int64_t full1 = blk1 < nfull ? blk1 : nfull;   // end of this wavefront's whole blocks
+
+  acc_t acc = {0, 0, 0, 0};
+  T av[2][CHUNK][4], bv[2][CHUNK][4];
+  auto load_chunk = [&](int set, int64_t first_blk) {   // set is a constant after unrolling
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u) {
+      const int64_t k = ((first_blk + u) << 4) + 4 * g;
+      load4<T, AVEC>(a, p.a_k, k, av[set][u]);
+      load4<T, BVEC>(b, p.b_k, k, bv[set][u]);
+    }
+  };
+  auto mma_chunk = [&](int set) {
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) acc = M16<T>::mma(av[set][u][s], bv[set][u][s], acc);
+  };
+  const int64_t nchunks = (full1 - blk0) / CHUNK;
+  int64_t blk = blk0;
+  if (nchunks > 0) {
+    load_chunk(0, blk0);
+    int64_t c = 0;
+    for (; c + 2 <= nchunks; c += 2) {
+      load_chunk(1, blk0 + (c + 1) * CHUNK);
+      mma_chunk(0);
+      const int64_t nxt = c + 2 < nchunks ? c + 2 : nchunks - 1;   // past the end: a harmless reload
+      load_chunk(0, blk0 + nxt * CHUNK);
+      mma_chunk(1);
+    }
+    if (c < nchunks) mma_chunk(0);
+    blk = blk0 + nchunks * CHUNK;
+  }
+  // what is left of the whole blocks (fewer than CHUNK): halving groups, loads before matrix instructions
+#pragma unroll
+  for (int grp = CHUNK / 2; grp >= 1; grp /= 2) {
+    if (blk + grp <= full1) {
+#pragma unroll
+      for (int u = 0; u < grp; ++u) {
+        const int64_t k = ((blk + u) << 4) + 4 * g;
+        load4<T, AVEC>(a, p.a_k, k, av[0][u]);
+        load4<T, BVEC>(b, p.b_k, k, bv[0][u]);
+      }
+#pragma unroll
+      for (int u = 0; u < grp; ++u)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc = M16<T>::mma(av[0][u][s], bv[0][u][s], acc);
+      blk += grp;
+    }
+  }
+  if (blk < blk1) {   // the partial last block: elements past K count as zero
+    const int64_t k = (blk << 4) + 4 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const bool ok = k + s < p.K;
+      const int64_t kk = ok ? k + s : p.K - 1;
+      const T x = a[kk * p.a_k], y = b[kk * p.b_k];
+      acc = M16<T>::mma(ok ? x : (T)0, ok ? y : (T)0, acc);
+    }
+  }
+
+  if (nw > 1) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][r * 64 + lane] = acc[r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      T sum = red[0][r * 64 + lane];
+      for (int w = 1; w < nw; ++w) sum += red[w][r * 64 + lane];   // fixed order: the result does not depend on timing
+      acc[r] = sum;
+    }
+  }
+
+  // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
+  // C += alpha * AB, each rounded on its own; then the optional fused bias / ReLU.
+  const T alpha = p.alpha, beta = p.beta;
+  const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
+  const int64_t col = n0 + i;
+  T cv[4], bias[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int64_t row = m0 + M16<T>::acc_row(r, lane);
+    const bool ok = row < p.M && col < p.N;
+    cv[r] = (ok && beta != (T)0) ? p.C[row * p.c_m + col * p.c_n] : (T)0;
+    bias[r] = (ok && has_bias) ? p.bias[row * p.bias_m + col * p.bias_n] : (T)0;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int64_t row = m0 + M16<T>::acc_row(r, lane);
+    if (row < p.M && col < p.N) {
+      T ab = acc[r];
+      if (alpha != (T)1) ab = alpha * ab;
+      T v = ab;
+      if (beta != (T)0) {
+        T c = cv[r];
+        if (beta != (T)1) c = c * beta;
+        v = c + ab;
+      }
+      if (has_bias) v = v + bias[r];
+      if (relu) v = ((T)0 >= v) ? (T)0 : v;
+      p.C[row * p.c_m + col * p.c_n] = v;
+    }
+  }
+}
+
+// Whether this product belongs here: few rows or few columns, little work, not a batch member.
+// AM_HIP_GEMM_SMALL = 0 / 1 in the environment turns the path off / forces it where its limits allow (tests).
+template <typename T>
+static inline bool applicable(const Args<T>& g) {
+  const char* e = getenv("AM_HIP_GEMM_SMALL");
+  const int forced = (e && *e) ? atoi(e) : -1;
+  if (forced == 0 || g.batch > 1) return false;
+  const int64_t mn = g.M < g.N ? g.M : g.N;
+  if (mn > 64) return false;
+  if (forced == 1) return true;
+  const double macs = (double)g.M * (double)g.N * (double)g.K;
+  return macs <= 268435456.0 && g.K <= 8192;
+}
+
+template <typename T>
+static int run(const Args<T>& g_in) {
+  constexpr int64_t VK = 16 / (int64_t)sizeof(T);
+  Args<T> g = g_in;
+  if (g.M > 64) {   // few columns: the transposed problem C^T = B^T A^T has few rows
+    g.M = g_in.N; g.N = g_in.M;
+    g.A = g_in.B; g.a_mn = g_in.b_mn; g.a_k = g_in.b_k;
+    g.B = g_in.A; g.b_mn = g_in.a_mn; g.b_k = g_in.a_k;
+    g.c_m = g_in.c_n; g.c_n = g_in.c_m;
+    g.bias_m = g_in.bias_n; g.bias_n = g_in.bias_m;
+  }
+  const int64_t tiles_m = (g.M + 15) / 16, tiles_n = (g.N + 15) / 16;
+  if (tiles_n >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
+  // Wavefronts per tile: about one per SIMD over the chip and at most four (measured: starting more
+  // wavefronts costs more than the latency they would hide), every one with at least two blocks of 16 k.
+  const int64_t tiles = tiles_m * tiles_n, nblk = (g.K + 15) / 16;
+  int64_t want = (int64_t)num_cus() * 4 / tiles;
+  if (want > nblk / 2) want = nblk / 2;
+  int nw = 1;
+  while (nw * 2 <= want && nw * 2 <= kMaxWaves) nw *= 2;
+  if (const char* e = getenv("AM_HIP_GEMM_SMALL_W")) { const int w = atoi(e); if (w >= 1 && w <= kMaxWaves) nw = w; }   // tests
+  const size_t lds = nw > 1 ? (size_t)nw * 256 * sizeof(T) : 0;
+  const bool avec = g.a_k == 1 && aligned16(g.A) && (g.a_mn % VK == 0 || g.M == 1);
+  const bool bvec = g.b_k == 1 && aligned16(g.B) && (g.b_mn % VK == 0 || g.N == 1);
+  const dim3 grid((unsigned)tiles_n, (unsigned)tiles_m), block((unsigned)nw * 64);
+  if (trace_choices()) fprintf(stderr, "am_hip gemm: small path, %lld x %lld tiles of 16 x 16, %d wavefronts per tile\n", (long long)tiles_m, (long long)tiles_n, nw);
+  constexpr int CH = sizeof(T) == 4 ? 4 : 2;
+  if (avec && bvec) hipLaunchKernelGGL((gemm_rows16<T, true, true, kMaxWaves, CH>), grid, block, lds, stream(), g);
+  else if (avec) hipLaunchKernelGGL((gemm_rows16<T, true, false, kMaxWaves, CH>), grid, block, lds, stream(), g);
+  else if (bvec) hipLaunchKernelGGL((gemm_rows16<T, false, true, kMaxWaves, CH>), grid, block, lds, stream(), g);
+  else hipLaunchKernelGGL((gemm_rows16<T, false, false, kMaxWaves, CH>), grid, block, lds, stream(), g);
+  return check_launch("gemm_rows16");
+}
+
+}  // namespace small
+}  // namespace gemm
+}  // namespace am

@@ -619,3 +619,86 @@ def test_digit_path_window_views(hip, oracle, sfx, monkeypatch):
             dAt = hip.toHip(np.ascontiguousarray(hostA.T))[c0:c0 + K, r0:r0 + M].transpose()
             dBt = hip.toHip(np.ascontiguousarray(hostB.T))[c0:c0 + N, r0:r0 + K].transpose()
             assert np.array_equal((dAt * dBt).toCpu(), oracle.matmul(A_small, B_small)), (M, N, K, r0, c0, "T")
+
+
+SMALL_SHAPES = [(1, 1, 1), (20, 36864 // 64, 25), (50, 300, 500), (64, 500, 800), (64, 10, 500), (7, 33, 15), (16, 16, 16),
+                (17, 47, 17), (64, 64, 4099), (33, 200, 1000), (3, 5, 8191), (500, 10, 64), (4096, 3, 129), (300, 64, 77)]
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_small_row_path(hip, oracle, sfx, monkeypatch):
+    """Products with at most 64 rows or columns on the kernel that loads matrix-instruction operands
+    straight from global memory (forced on): every k tail (K < 16, K % 16 != 0, K % 4 != 0), ragged
+    M and N, one to four wavefronts per tile, both orientations, every alpha / beta case, against
+    the oracle and against the tiled kernel on the same inputs."""
+    dt = DTYPES[sfx]
+    eps = np.finfo(dt).eps
+    rng = np.random.default_rng(seed_of("small", sfx))
+    for (M, N, K) in SMALL_SHAPES:
+        A, B, C = fill(rng, (M, K), dt), fill(rng, (K, N), dt), fill(rng, (M, N), dt)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        for alpha, beta in [(1, 0), (1, 1), (-0.75, 0.5), (2, -1)]:
+            say("small path", sfx, (M, N, K), alpha, beta)
+            want = oracle.closed_gemm_float(alpha, A, B, beta, C).astype(dt)
+            got = {}
+            for mode in ("1", "0"):
+                monkeypatch.setenv("AM_HIP_GEMM_SMALL", mode)
+                dC = hip.toHip(C)
+                hip.gemm(alpha, dA, dB, beta, dC)
+                got[mode] = dC.toCpu().copy()
+                assert_parity(oracle, sfx, got[mode], want, f"{(M, N, K)} a={alpha} b={beta} small={mode}")
+            scale = np.abs(alpha) * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + np.abs(beta * C)
+            assert np.all(np.abs(got["1"].astype(np.float64) - want) <= 4 * (K + 4) * eps * scale + np.finfo(dt).tiny), (M, N, K)
+    monkeypatch.setenv("AM_HIP_GEMM_SMALL", "1")
+    # beta == 0 must not read C: NaN there never reaches the result
+    C = np.full((20, 70), np.nan, dtype=dt)
+    A, B = fill(rng, (20, 40), dt), fill(rng, (40, 70), dt)
+    dC = hip.toHip(C)
+    hip.gemm(1, hip.toHip(A), hip.toHip(B), 0, dC)
+    assert np.isfinite(dC.toCpu()).all()
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_small_row_path_views_and_epilogue(hip, oracle, sfx, monkeypatch):
+    """The same kernel on transposed, stepped, reversed and broadcast operands, strided and
+    column-major destinations, and with the fused bias / ReLU epilogue (row and column bias)."""
+    monkeypatch.setenv("AM_HIP_GEMM_SMALL", "1")
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("small-views", sfx))
+    for (M, N, K) in [(64, 500, 800), (20, 300, 25), (50, 96, 500), (300, 20, 123)]:
+        say("small path views", sfx, (M, N, K))
+        A, B = fill(rng, (M, K), dt), fill(rng, (K, N), dt)
+        want = oracle.matmul(A, B)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        dAt = hip.toHip(np.ascontiguousarray(A.T)).transpose()          # unit stride along m
+        dBt = hip.toHip(np.ascontiguousarray(B.T)).transpose()          # unit stride along k
+        for a, b, what in [(dA, dBt, "C * F"), (dAt, dB, "F * C"), (dAt, dBt, "F * F")]:
+            assert_parity(oracle, sfx, (a * b).toCpu(), want, f"{(M, N, K)} {what}")
+        A2, B2 = fill(rng, (2 * M, K), dt), fill(rng, (K, 2 * N), dt)
+        got = (hip.toHip(A2)[::2] * hip.toHip(B2)[:, ::2]).toCpu()
+        assert_parity(oracle, sfx, got, oracle.matmul(np.ascontiguousarray(A2[::2]), np.ascontiguousarray(B2[:, ::2])), "stepped")
+        got = (hip.toHip(A)[::-1] * dB).toCpu()
+        assert_parity(oracle, sfx, got, oracle.matmul(np.ascontiguousarray(A[::-1]), B), "reversed rows")
+        row = fill(rng, (1, K), dt)
+        got = (hip.toHip(row).broadcast((M, K)) * dB).toCpu()
+        assert_parity(oracle, sfx, got, oracle.matmul(np.ascontiguousarray(np.broadcast_to(row, (M, K))), B), "broadcast rows")
+        # destinations: column-major, and every second column of a wider buffer
+        dCt = hip.toHip(np.zeros((N, M), dtype=dt)).transpose()
+        hip.gemm(1, dA, dB, 0, dCt)
+        assert_parity(oracle, sfx, dCt.toCpu(), want, "column-major C")
+        wide = fill(rng, (M, 2 * N), dt)
+        dW = hip.toHip(wide)
+        ref = wide.copy()
+        ref[:, ::2] = oracle.closed_gemm_float(2, A, B, 0.5, wide[:, ::2]).astype(dt)
+        hip.gemm(2, dA, dB, 0.5, dW[:, ::2])
+        assert_parity(oracle, sfx, dW.toCpu(), ref, "stepped C")
+        assert np.array_equal(dW.toCpu()[:, 1::2], wide[:, 1::2])
+        # fused epilogue
+        brow, bcol = fill(rng, (1, N), dt), fill(rng, (M, 1), dt)
+        for bias, epi in [(brow, "bias"), (brow, "bias_relu"), (bcol, "bias_relu"), (None, "relu")]:
+            o = hip.empty((M, N), dt)
+            hip.gemm(1, dA, dB, 0, o, epilogue=epi, bias=None if bias is None else hip.toHip(bias))
+            ref = want + (0 if bias is None else bias)
+            if "relu" in epi:
+                ref = np.where(0 >= ref, 0, ref)
+            assert_parity(oracle, sfx, o.toCpu(), ref.astype(dt), f"{(M, N, K)} {epi}")
