@@ -650,6 +650,15 @@ def test_small_row_path(hip, oracle, sfx, monkeypatch):
             scale = np.abs(alpha) * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + np.abs(beta * C)
             assert np.all(np.abs(got["1"].astype(np.float64) - want) <= 4 * (K + 4) * eps * scale + np.finfo(dt).tiny), (M, N, K)
     monkeypatch.setenv("AM_HIP_GEMM_SMALL", "1")
+    # every number of wavefronts per tile on shares of k that are whole chunks, part chunks and a tail
+    for (M, N, K) in [(40, 100, 1000), (64, 64, 333), (5, 20, 40)]:
+        A, B = fill(rng, (M, K), dt), fill(rng, (K, N), dt)
+        want = oracle.closed_gemm_float(1, A, B, 0, None).astype(dt)
+        for w in ("1", "2", "4"):
+            say("small path, wavefronts per tile", sfx, (M, N, K), w)
+            monkeypatch.setenv("AM_HIP_GEMM_SMALL_W", w)
+            assert_parity(oracle, sfx, (hip.toHip(A) * hip.toHip(B)).toCpu(), want, f"{(M, N, K)} W={w}")
+    monkeypatch.delenv("AM_HIP_GEMM_SMALL_W")
     # beta == 0 must not read C: NaN there never reaches the result
     C = np.full((20, 70), np.nan, dtype=dt)
     A, B = fill(rng, (20, 40), dt), fill(rng, (40, 70), dt)
