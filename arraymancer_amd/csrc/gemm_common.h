@@ -4,6 +4,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <type_traits>
 #include "common.h"
 
 namespace am {
@@ -37,7 +38,27 @@ template <typename T> struct Args {
   int batch;
   int64_t batch_a, batch_b, batch_c;
   bool swapped;                    // prepare() exchanged the roles of A and B (column-major C)
+  // Integer products launched behind the digit-sliced path as its alternative: when gate_flags is
+  // set, the vector-ALU kernels leave at once if the operands have at most gate_max_pairs non-empty
+  // digit pairs (the digit-sliced kernel, launched just before with the same limit, has then
+  // written C); otherwise the digit-sliced kernel has left and they do the work.
+  const uint32_t* gate_flags;
+  uint32_t gate_gen;
+  int gate_max_pairs;
 };
+
+// Digit pairs (i, j), i + j < ND, whose planes are both marked non-empty: flags[i] == gen for A's
+// plane i, flags[ND + j] == gen for B's plane j. Uniform over the workgroup.
+template <int ND>
+__device__ __forceinline__ int live_digit_pairs(const uint32_t* flags, uint32_t gen) {
+  int n = 0, live_b = 0;
+#pragma unroll
+  for (int i = ND - 1; i >= 0; --i) {          // live_b counts B's live planes j <= ND - 1 - i
+    live_b += flags[ND + (ND - 1 - i)] == gen ? 1 : 0;
+    n += flags[i] == gen ? live_b : 0;
+  }
+  return n;
+}
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
@@ -90,6 +111,7 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   g.K = K; g.alpha = alpha; g.beta = beta; g.C = C;
   g.epilogue = epilogue; g.bias = bias;
   g.batch = 1; g.batch_a = g.batch_b = g.batch_c = 0;
+  g.gate_flags = nullptr; g.gate_gen = 0; g.gate_max_pairs = 0;
   g.swapped = swap;
   g.a_kfast = iabs64(g.a_k) <= iabs64(g.a_mn);
   g.b_kfast = iabs64(g.b_k) < iabs64(g.b_mn);
@@ -223,6 +245,7 @@ static inline TileSplit choose_tile_split(const TileChoice* cand, int ncand, int
 template <typename T, typename ACC, int VEC>
 __global__ __launch_bounds__(256) void splitk_reduce(Args<T> p) {
   typedef ACC vec_t __attribute__((ext_vector_type(VEC)));
+  if (std::is_integral<T>::value && p.gate_flags != nullptr && live_digit_pairs<(int)sizeof(T)>(p.gate_flags, p.gate_gen) <= p.gate_max_pairs) return;
   const int64_t total = p.M * p.N;
   const ACC* ws = (const ACC*)p.ws;
   const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;

@@ -16,15 +16,10 @@ static int run_i64(Args<int64_t>& g) {
   static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.85}};
   // 34.0e3 multiply-adds per microsecond and CU: the measured VALU ceiling of this element type.
   const TileSplit ts = choose_tile_split<int64_t>(cand, 2, g.M, g.N, g.K, 16, 34.0e3, "AM_HIP_GEMM_TILE_I64", g.batch);
-  // The same product on the int8 matrix cores (digit slicing) when that is estimated to be faster.
-  if (const int may = i8::applicable(g)) {
-    const i8::Plan pl = i8::plan(g);
-    if (may == 2 || pl.est_us < 1.2 * ts.est_us) {
-      if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path (int64), est %.1f us (VALU est %.1f us)\n", pl.est_us, ts.est_us);
-      const int rc = i8::run(g, pl);
-      if (rc <= 0) return rc;   // > 0: no scratch memory for the digit planes, take the VALU kernel
-    }
-  }
+  // The same product on the int8 matrix cores (digit slicing) when that is estimated to be faster,
+  // or when it would be for operands with few non-empty digit planes (then the data decides on the device).
+  int rc = AM_OK;
+  if (!i8::try_digits(g, ts.est_us, &rc)) return rc;
   switch (ts.tile) {
     case 0: return launch_valu<int64_t, 8, 8, 16>(g, ak, bk, ts.splits);
     default: return launch_valu<int64_t, 4, 4, 16>(g, ak, bk, ts.splits);

@@ -94,6 +94,7 @@ struct SplitArgs {
   int64_t K, Kp;
   uint32_t* flags;
   uint32_t gen;
+  int max_pairs;    // split_digits writes nothing when more digit pairs than this are live (the product then runs elsewhere)
 };
 
 // The 32 (mn) x 128 (k) tile at (mn0, k0) of operand op, 16 elements per lane of a 256-lane workgroup:
@@ -198,6 +199,7 @@ __global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
   const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
   const int64_t MNp = a.MNp[op];
   if (mn0 >= MNp) return;
+  if (live_digit_pairs<ND>(a.flags, a.gen) > a.max_pairs) return;
   visit_tile<T>(a, op, mn0, k0, [&](int mn, int k, T x) { tile[mn][k] = x; });
   __syncthreads();
   const int64_t plane = MNp * a.Kp;
@@ -227,6 +229,7 @@ struct DigitArgs {
   const int8_t* PA; const int8_t* PB;   // ND = sizeof(T) digit planes each, in 1 KiB fragment blocks [rows/32][Kp/32][64 lanes][16]
   const uint32_t* flags;                // [0..ND-1]: planes of A, [ND..2ND-1]: planes of B; == gen: not all zero
   uint32_t gen;
+  int max_pairs;                        // the kernel leaves at once when more digit pairs than this are live
   int64_t Mp, Np, Kp;
   T* C; int64_t c_m, c_n;
   int64_t M, N;
@@ -297,6 +300,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
   }
   __syncthreads();
   const int n_pairs = tab_n;
+  if (n_pairs > p.max_pairs) return;   // uniform: the vector-ALU kernel launched behind this one takes the product
   const int64_t slabs_per_pair = p.Kp / BK;
   const int64_t total = (int64_t)n_pairs * slabs_per_pair;
   // Slabs are fetched in order, RING - 1 ahead of the one being multiplied; (f_oa, f_ob) + f_k are the
@@ -452,7 +456,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
 // Padded operand extents and the estimated time of the digit-sliced product for both tile shapes
 // (rounds of one workgroup per CU x measured time per tile and k, plus the two splitting passes).
 // The estimate is for operands that use every digit; the kernel itself skips empty planes.
-struct Plan { int64_t Mp, Np, Kp; bool big; double est_us; };
+struct Plan { int64_t Mp, Np, Kp; bool big; double est_us, main_us, split_us; };
 template <typename T>
 static inline Plan plan(const Args<T>& g) {
   constexpr bool WIDE = sizeof(T) == 8;
@@ -473,7 +477,9 @@ static inline Plan plan(const Args<T>& g) {
   }
   // the splitting passes read sizeof(T) and write sizeof(T) bytes per element, at about 2.8 TB/s
   const double split_us = 2 * 5.0 + 2.0 * sizeof(T) * (double)(pl.Mp + pl.Np) * pl.Kp / 2.8e6;
-  pl.est_us = (pl.big ? cost_big : cost_small) + split_us;
+  pl.main_us = pl.big ? cost_big : cost_small;
+  pl.split_us = split_us;
+  pl.est_us = pl.main_us + split_us;
   return pl;
 }
 
@@ -481,7 +487,7 @@ static inline Plan plan(const Args<T>& g) {
 // recorded into a graph (it allocates its planes), and for int64 k small enough that one pair's
 // sum over k fits the 32-bit accumulators of the matrix cores (k * 2^14 < 2^31).
 // AM_HIP_GEMM_I32_PATH / AM_HIP_GEMM_I64_PATH = "valu" / "mfma" forces a path (tests, benchmarks);
-// returns 0 = no, 1 = if estimated faster, 2 = forced.
+// returns 0 = no, 1 = if estimated faster, 2 = forced, 3 = forced as a data-dependent choice.
 template <typename T>
 static inline int applicable(const Args<T>& g) {
   const char* e = getenv(sizeof(T) == 8 ? "AM_HIP_GEMM_I64_PATH" : "AM_HIP_GEMM_I32_PATH");
@@ -489,11 +495,15 @@ static inline int applicable(const Args<T>& g) {
   if (g.batch > 1 || capturing()) return 0;
   if (sizeof(T) == 8 && g.K > 131071) return 0;
   if (e && *e == 'm') return 2;
+  if (e && *e == 's') return 3;   // "spec": both kernels behind the scan, the data decides (tests)
   return (g.M >= 64 && g.N >= 64 && g.K >= 256) ? 1 : 0;
 }
 
+// max_pairs < all pairs: the product is left alone when the operands turn out to have more live digit
+// pairs; *gate_flags / *gate_gen then tell the caller what to hand to the kernels it launches next.
 template <typename T>
-static int run(const Args<T>& g, const Plan& pl) {
+static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const uint32_t** gate_flags = nullptr,
+               uint32_t* gate_gen = nullptr) {
   constexpr int ND = (int)sizeof(T);
   const int64_t Mp = pl.Mp, Np = pl.Np, Kp = pl.Kp;
   const bool big = pl.big;   // 256 x 256 tiles: a 128 x 64 tile per wavefront, fewest LDS reads per matrix instruction
@@ -523,7 +533,9 @@ static int run(const Args<T>& g, const Plan& pl) {
   SplitArgs<T> sp;
   sp.X[0] = g.A; sp.ld_mn[0] = g.a_mn; sp.ld_k[0] = g.a_k; sp.MN[0] = g.M; sp.MNp[0] = Mp; sp.kfast[0] = g.a_kfast; sp.P[0] = PA;
   sp.X[1] = g.B; sp.ld_mn[1] = g.b_mn; sp.ld_k[1] = g.b_k; sp.MN[1] = g.N; sp.MNp[1] = Np; sp.kfast[1] = g.b_kfast; sp.P[1] = PB;
-  sp.K = g.K; sp.Kp = Kp; sp.flags = flags; sp.gen = gen;
+  sp.K = g.K; sp.Kp = Kp; sp.flags = flags; sp.gen = gen; sp.max_pairs = max_pairs;
+  if (gate_flags) *gate_flags = flags;
+  if (gate_gen) *gate_gen = gen;
   constexpr int64_t VEC = 16 / (int64_t)sizeof(T);
   for (int op = 0; op < 2; ++op) {
     const bool aligned = ((uintptr_t)sp.X[op] & 15) == 0;
@@ -535,7 +547,7 @@ static int run(const Args<T>& g, const Plan& pl) {
   hipLaunchKernelGGL(scan_digits<T>, dim3((unsigned)((mx + 31) / 32), (unsigned)((g.K + 127) / 128), 2), dim3(256), 0, stream(), sp);
   hipLaunchKernelGGL(split_digits<T>, dim3((unsigned)(mxp / 32), (unsigned)(Kp / 128), 2), dim3(256), 0, stream(), sp);
   DigitArgs<T> d;
-  d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
+  d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.max_pairs = max_pairs; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
   d.alpha = g.alpha; d.beta = g.beta;
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
@@ -551,6 +563,42 @@ static int run(const Args<T>& g, const Plan& pl) {
   // through the same stream, after this product.
   (void)am_hip_free(ws);
   return rc;
+}
+
+// The integer product on the matrix cores, decided in three steps. (1) Estimated faster than the
+// vector-ALU kernel even if every digit pair is needed: taken outright. (2) Not, but faster when
+// few pairs are live (operands with small entries): scan, split and the digit kernel are launched with
+// the largest pair count that still wins; the caller then launches the vector-ALU kernel gated on the
+// same flags, and whichever of the two the data rules out leaves at once. (3) Otherwise not taken.
+// Returns 0 when the product is done or a launch failed (rc), 1 when the caller has to launch the
+// vector-ALU kernel (g.gate_* set for case 2).
+template <typename T>
+static int try_digits(Args<T>& g, double valu_est_us, int* rc) {
+  constexpr int ND = (int)sizeof(T), NPAIRS = ND * (ND + 1) / 2;
+  *rc = AM_OK;
+  const int may = applicable(g);
+  if (!may) return 1;
+  const Plan pl = plan(g);
+  if (may == 2 || (may == 1 && pl.est_us < 1.2 * valu_est_us)) {
+    if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path, %s tiles, est %.1f us (VALU est %.1f us)\n", pl.big ? "256x256" : "256x128", pl.est_us, valu_est_us);
+    const int r = run(g, pl);
+    if (r <= 0) { *rc = r; return 0; }
+    return 1;   // no scratch memory for the digit planes
+  }
+  // the scan and an early-leaving kernel or two cost about 10 us when the data says no
+  const double per_pair = pl.main_us / NPAIRS, fixed = pl.split_us * 0.6 + 10.0;
+  int max_pairs = (int)((0.8 * valu_est_us - fixed) / per_pair);
+  if (const char* e = getenv("AM_HIP_GEMM_SPEC_PAIRS")) max_pairs = atoi(e);   // tests
+  if (max_pairs > NPAIRS) max_pairs = NPAIRS;
+  if (may != 3 && (max_pairs < 1 || valu_est_us < 40.0)) return 1;
+  if (max_pairs < 0) max_pairs = 0;
+  if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path if at most %d digit pairs are live, else VALU (est %.1f us)\n", max_pairs, valu_est_us);
+  const uint32_t* flags = nullptr;
+  uint32_t gen = 0;
+  const int r = run(g, pl, max_pairs, &flags, &gen);
+  if (r < 0) { *rc = r; return 0; }
+  if (r == 0) { g.gate_flags = flags; g.gate_gen = gen; g.gate_max_pairs = max_pairs; }
+  return 1;
 }
 
 }  // namespace i8

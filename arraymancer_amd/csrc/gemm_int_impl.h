@@ -40,6 +40,7 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
   __shared__ __attribute__((aligned(16))) T sA[2][BK * LDA];
   __shared__ __attribute__((aligned(16))) T sB[2][BK * LDB];
 
+  if (p.gate_flags != nullptr && live_digit_pairs<(int)sizeof(T)>(p.gate_flags, p.gate_gen) <= p.gate_max_pairs) return;
   int tile_m, tile_n, bid = (int)blockIdx.x, split = 0;
   if (p.splits > 1) {
     const int nt = p.tiles_m * p.tiles_n;

@@ -711,3 +711,32 @@ def test_small_row_path_views_and_epilogue(hip, oracle, sfx, monkeypatch):
             if "relu" in epi:
                 ref = np.where(0 >= ref, 0, ref)
             assert_parity(oracle, sfx, o.toCpu(), ref.astype(dt), f"{(M, N, K)} {epi}")
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+def test_integer_data_dependent_path(hip, oracle, sfx, monkeypatch):
+    """Both integer kernels launched behind the digit scan, the one the data rules out leaving at
+    once: for every limit on the number of live digit pairs and operands with one, a few and all
+    digit planes in use, with and without a split of k in the vector-ALU kernel, with beta != 0
+    (a product computed twice, or by neither kernel, would show). Bit-exact."""
+    monkeypatch.setenv(f"AM_HIP_GEMM_{sfx.upper()}_PATH", "spec")
+    dt = DTYPES[sfx]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(seed_of("spec", sfx))
+    M, N, K = 300, 260, 700
+    C = fill(rng, (M, N), dt, -1000, 1000)
+    for lo, hi in [(-100, 100), (-40000, 40000), (info.min, info.max), (0, 0)]:
+        A, B = fill(rng, (M, K), dt, lo, hi), fill(rng, (K, N), dt, lo, hi)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        want = oracle.gemm_strided(3, A, B, -2, C.copy())
+        for limit in ("0", "1", "2", "4", "9", "10", "35", "36"):
+            for splitk in (None, "3"):
+                say("data-dependent integer path", sfx, (lo, hi), limit, splitk)
+                monkeypatch.setenv("AM_HIP_GEMM_SPEC_PAIRS", limit)
+                if splitk:
+                    monkeypatch.setenv("AM_HIP_GEMM_SPLITK", splitk)
+                else:
+                    monkeypatch.delenv("AM_HIP_GEMM_SPLITK", raising=False)
+                dC = hip.toHip(C)
+                hip.gemm(3, dA, dB, -2, dC)
+                assert np.array_equal(dC.toCpu(), want), (lo, hi, limit, splitk)
