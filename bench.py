@@ -259,10 +259,12 @@ def bench_chain(am, timer, steps, warmup):
     return dict(workload="f32 inference chain: [20x25].[25x36864], [50x500].[500x4096], "
                          "[64x800].[800x500]+bias+ReLU (fused), [64x500].[500x10]",
                 unit="us per chain", dtype="f32", higher_is_better=False,
-                value=round(ev_g / steps * 1e6, 2), hipgraph_us=round(ev_g / steps * 1e6, 2),
+                value=round(min(ev_g, ev_e) / steps * 1e6, 2), value_is="eager" if ev_e <= ev_g else "hipgraph",
+                hipgraph_us=round(ev_g / steps * 1e6, 2),
                 eager_us=round(ev_e / steps * 1e6, 2), eager_wall_us=round(wall_e / steps * 1e6, 2),
-                gflops_hipgraph=round(flops / (ev_g / steps) / 1e9, 1),
-                note="launch/latency bound: 2.9e8 FLOP and 17.8 MB per chain; eager figure includes host launch cost")
+                gflops=round(flops / (min(ev_g, ev_e) / steps) / 1e9, 1),
+                note="launch/latency bound: 2.9e8 FLOP and 17.8 MB per chain; four kernels of 5-10 us; the eager figure "
+                     "includes the host's launch cost, the replayed graph pays more between its nodes")
 
 
 def config_report(am, timer, L):
