@@ -25,8 +25,9 @@
 //                  LDS ring (global_load_lds_dwordx4, no register stage, no LDS write instructions),
 //                  several slabs ahead; fragments are double-buffered in registers. Between two
 //                  values of s the accumulators are shifted left by 8 (Horner form of the sum over
-//                  s). Padded planes mean no bounds tests in the loop. The kernel is bound by LDS
-//                  reads (six 1 KiB fragment reads per eight matrix instructions and wavefront).
+//                  s). Padded planes mean no bounds tests in the loop. Of 72 us for one pair at
+//                  4096^3, 31 are the matrix instructions, 10 the store of C, 15 the operand fetch
+//                  from L2 that the prefetch does not hide, the rest fragment reads and barriers.
 //
 // int64 works the same way with eight digits and the 36 pairs i + j <= 7. The matrix cores
 // accumulate in 32 bits, which holds one pair's sum over k exactly while k * 2^14 < 2^31; after each
