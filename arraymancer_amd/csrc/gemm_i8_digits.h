@@ -13,12 +13,13 @@
 // throughput against 2MNK multiply-adds at the 61 Top/s the vector ALU sustains.
 //
 // Three passes:
-//   scan_digits    marks the digit planes of both operands that hold a non-zero digit anywhere (entries
-//                  within +-127 have one such plane, the others are neither written nor multiplied);
-//   split_digits   strided operand (any view) -> its marked int8 planes, rows padded to the tile size
-//                  and k to the slab size with zeros, stored as 1 KiB blocks of 32 rows x 32 k in the
-//                  register layout of the matrix instruction (a 32 x 128 tile goes through LDS so that
-//                  both the strided read and the block write are coalesced);
+//   split_digits<first>   reads both operands (any strided view), marks the digit planes that hold a
+//                  non-zero digit anywhere and writes plane 0 of each: int8 planes with rows padded to
+//                  the tile size and k to the slab size with zeros, stored as 1 KiB blocks of 32 rows x
+//                  32 k in the register layout of the matrix instruction (a 32 x 128 tile goes through
+//                  LDS so that both the strided read and the block write are coalesced);
+//   split_digits<second>  writes the marked planes above plane 0. Entries within +-127 have none (the
+//                  pass leaves at once, the operands were read only once, one pair instead of ten runs);
 //   gemm_i8_digits one workgroup of eight wavefronts per 256 x 256 (or 256 x 128) tile of C. For
 //                  s = 3..0 it walks the pairs (i, s - i) whose planes are not empty and the k slabs
 //                  of each pair as one long k loop: blocks go from global memory straight into an
@@ -95,7 +96,7 @@ struct SplitArgs {
   int64_t K, Kp;
   uint32_t* flags;
   uint32_t gen;
-  int max_pairs;    // split_digits writes nothing when more digit pairs than this are live (the product then runs elsewhere)
+  int max_pairs;    // the second splitting pass writes nothing when more digit pairs than this are live (the product then runs elsewhere)
 };
 
 // The 32 (mn) x 128 (k) tile at (mn0, k0) of operand op, 16 elements per lane of a 256-lane workgroup:
@@ -167,62 +168,99 @@ __device__ __forceinline__ void visit_tile(const SplitArgs<T>& a, int op, int64_
   }
 }
 
-// First pass (reads only): marks the digit planes that hold anything. Operands with small entries
-// have one or two such planes; the others are neither written by split_digits nor multiplied.
-// blockIdx.z picks the operand; one workgroup looks at a 32 (mn) x 128 (k) tile.
-template <typename T>
-__global__ __launch_bounds__(256) void scan_digits(SplitArgs<T> a) {
-  constexpr int ND = (int)sizeof(T);
-  using U = std::make_unsigned_t<T>;
-  const int op = (int)blockIdx.z;
-  const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
-  if (mn0 >= a.MN[op]) return;
-  U seen = 0;   // byte d: OR of the digits d of this lane's elements
-  visit_tile<T>(a, op, mn0, k0, [&](int, int, T x) { seen |= balanced_digits<T>(x); });
-  uint32_t nz[ND];
-#pragma unroll
-  for (int d = 0; d < ND; ++d) nz[d] = (uint32_t)(seen >> (8 * d)) & 0xFFu;
-  uint32_t* flags = a.flags + op * ND;
-#pragma unroll
-  for (int d = 0; d < ND; ++d)   // every writer stores the same value; at most one store per wavefront and plane
-    if (__ballot(nz[d] != 0) != 0 && (threadIdx.x & 63) == 0 && flags[d] != a.gen) flags[d] = a.gen;
-}
-
-// Second pass: writes the marked planes, zero padded to MNp x Kp. One workgroup moves a 32 (mn) x
-// 128 (k) tile through LDS: the read walks whichever of the two directions is the faster one in
-// memory (kfast), the write is 16 bytes per lane and plane, eight lanes to a 128-byte row segment.
-template <typename T>
+// The two splitting passes. A workgroup moves one 32 (mn) x 128 (k) tile of an operand at a time through
+// LDS: the read walks whichever of the two directions is the faster one in memory, the write is
+// 16 bytes per lane and plane into the 1 KiB blocks the product kernel wants (32 rows x 32 k in the
+// register layout of the matrix instruction: lane (row % 32) + 32 * ((k % 32) / 16) owns 16 consecutive k).
+//   FIRST = true : marks the digit planes that hold anything (flags) and writes plane 0, which
+//                  practically every operand needs. Operands with entries within +-127 need nothing else:
+//                  the second pass then leaves at once and the operand has been read only once.
+//   FIRST = false: writes the marked planes above plane 0 (nothing if there is none, or if the product
+//                  has more live digit pairs than max_pairs and therefore runs on the vector ALU).
+template <typename T, bool FIRST>
 __global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
   constexpr int ND = (int)sizeof(T);
-  __shared__ __attribute__((aligned(16))) T tile[32][128 + 16 / sizeof(T)];   // rows stay 16-byte aligned
-  const int op = (int)blockIdx.z;
-  const int64_t mn0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 128;
+  using U = std::make_unsigned_t<T>;
+  // the tile in LDS: whole elements for the second pass, only their lowest digit for the first (rows stay 16-byte aligned)
+  typedef std::conditional_t<FIRST, int8_t, T> tile_t;
+  __shared__ __attribute__((aligned(16))) tile_t tile[32][128 + 16 / sizeof(tile_t)];
+  bool live[2][ND];   // second pass: which planes were marked (one round trip for all the flag words)
+  bool any_high[2] = {false, false};
+  if constexpr (!FIRST) {
+    uint32_t fl[2 * ND];
+#pragma unroll
+    for (int i = 0; i < 2 * ND; ++i) fl[i] = a.flags[i];
+    int pairs = 0, live_b = 0;
+#pragma unroll
+    for (int i = ND - 1; i >= 0; --i) {
+      live_b += fl[ND + (ND - 1 - i)] == a.gen ? 1 : 0;
+      pairs += fl[i] == a.gen ? live_b : 0;
+    }
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        live[o][d] = fl[o * ND + d] == a.gen;
+        if (d > 0) any_high[o] |= live[o][d];
+      }
+    if (pairs > a.max_pairs || !(any_high[0] || any_high[1])) return;
+  }
+  // a few workgroups per CU walk the tiles of both operands (a second pass with nothing to do ends quickly)
+  const int64_t kt = a.Kp >> 7, t0 = (a.MNp[0] >> 5) * kt, t1 = (a.MNp[1] >> 5) * kt;
+  for (int64_t t = blockIdx.x; t < t0 + t1; t += gridDim.x) {
+  const int op = t < t0 ? 0 : 1;
+  const int64_t tt = t - (op ? t0 : 0);
+  const int64_t mn0 = (tt / kt) * 32, k0 = (tt % kt) * 128;
   const int64_t MNp = a.MNp[op];
-  if (mn0 >= MNp) return;
-  if (live_digit_pairs<ND>(a.flags, a.gen) > a.max_pairs) return;
-  visit_tile<T>(a, op, mn0, k0, [&](int mn, int k, T x) { tile[mn][k] = x; });
+  uint32_t* flags = a.flags + op * ND;
+  if constexpr (!FIRST) {
+    if (!any_high[op]) {   // nothing above plane 0 in this operand: go to the other one, or leave
+      if (op == 1) return;
+      t += (t0 - 1 - tt) / gridDim.x * gridDim.x;   // the last tile of this workgroup's walk that is still in operand 0
+      continue;
+    }
+  }
+  U seen = 0;   // byte d: OR of the digits d of this lane's elements
+  visit_tile<T>(a, op, mn0, k0, [&](int mn, int k, T x) {
+    if constexpr (FIRST) {
+      const U y = balanced_digits<T>(x);
+      seen |= y;
+      tile[mn][k] = (int8_t)(y & 0xFFu);
+    } else {
+      tile[mn][k] = x;
+    }
+  });
+  if constexpr (FIRST) {
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {   // every writer stores the same value; at most one store per wavefront and plane
+      const bool nz = ((uint32_t)(seen >> (8 * d)) & 0xFFu) != 0;
+      if (__ballot(nz) != 0 && (threadIdx.x & 63) == 0 && flags[d] != a.gen) flags[d] = a.gen;
+    }
+  }
   __syncthreads();
   const int64_t plane = MNp * a.Kp;
   const int k16 = threadIdx.x & 7, mn = threadIdx.x >> 3;
-  u4 out[ND];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const T xs[4] = {tile[mn][k16 * 16 + g * 4], tile[mn][k16 * 16 + g * 4 + 1], tile[mn][k16 * 16 + g * 4 + 2],
-                     tile[mn][k16 * 16 + g * 4 + 3]};
-    uint32_t w[ND];   // one 4-byte word (4 consecutive k) per digit plane
-    digits_of4<T>(xs, w);
-#pragma unroll
-    for (int d = 0; d < ND; ++d) out[d][g] = w[d];
-  }
-  // Planes are stored in the order the matrix instruction wants them: one 1 KiB block per 32 rows x 32 k,
-  // lane (row % 32) + 32 * ((k % 32) / 16) of a wavefront owning 16 consecutive k. The product kernel moves
-  // whole blocks from global memory into LDS without passing through registers.
   int8_t* dst = a.P[op] + ((((mn0 >> 5) * (a.Kp >> 5) + (k0 >> 5) + (k16 >> 1)) * 64 + (k16 & 1) * 32 + mn) << 4);
-  const uint32_t* flags = a.flags + op * ND;
+  if constexpr (FIRST) {
+    *(u4*)dst = *(const u4*)&tile[mn][k16 * 16];
+  } else {
+    u4 out[ND];
 #pragma unroll
-  for (int d = 0; d < ND; ++d)
-    if (flags[d] == a.gen) *(u4*)(dst + d * plane) = out[d];
+    for (int g = 0; g < 4; ++g) {
+      const T xs[4] = {tile[mn][k16 * 16 + g * 4], tile[mn][k16 * 16 + g * 4 + 1], tile[mn][k16 * 16 + g * 4 + 2],
+                       tile[mn][k16 * 16 + g * 4 + 3]};
+      uint32_t w[ND];   // one 4-byte word (4 consecutive k) per digit plane
+      digits_of4<T>(xs, w);
+#pragma unroll
+      for (int d = 0; d < ND; ++d) out[d][g] = w[d];
+    }
+#pragma unroll
+    for (int d = 1; d < ND; ++d)
+      if (op == 0 ? live[0][d] : live[1][d]) *(u4*)(dst + d * plane) = out[d];
+  }
+  __syncthreads();   // the tile buffer is reused
+  }
 }
 
 template <typename T>
@@ -496,7 +534,7 @@ static inline int applicable(const Args<T>& g) {
   if (g.batch > 1 || capturing()) return 0;
   if (sizeof(T) == 8 && g.K > 131071) return 0;
   if (e && *e == 'm') return 2;
-  if (e && *e == 's') return 3;   // "spec": both kernels behind the scan, the data decides (tests)
+  if (e && *e == 's') return 3;   // "spec": both kernels behind the first splitting pass, the data decides (tests)
   return (g.M >= 64 && g.N >= 64 && g.K >= 256) ? 1 : 0;
 }
 
@@ -544,9 +582,10 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
                   : (aligned && sp.ld_mn[op] == 1 && sp.ld_k[op] % VEC == 0) ? 2
                                                                              : 0;
   }
-  const int64_t mx = g.M > g.N ? g.M : g.N, mxp = Mp > Np ? Mp : Np;
-  hipLaunchKernelGGL(scan_digits<T>, dim3((unsigned)((mx + 31) / 32), (unsigned)((g.K + 127) / 128), 2), dim3(256), 0, stream(), sp);
-  hipLaunchKernelGGL(split_digits<T>, dim3((unsigned)(mxp / 32), (unsigned)(Kp / 128), 2), dim3(256), 0, stream(), sp);
+  const int64_t stiles = (Mp + Np) / 32 * (Kp / 128), smax = (int64_t)num_cus() * 16;
+  const dim3 sgrid((unsigned)(stiles < smax ? stiles : smax));
+  hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
+  hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
   DigitArgs<T> d;
   d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.max_pairs = max_pairs; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
@@ -568,7 +607,7 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
 
 // The integer product on the matrix cores, decided in three steps. (1) Estimated faster than the
 // vector-ALU kernel even if every digit pair is needed: taken outright. (2) Not, but faster when
-// few pairs are live (operands with small entries): scan, split and the digit kernel are launched with
+// few pairs are live (operands with small entries): the splitting passes and the digit kernel are launched with
 // the largest pair count that still wins; the caller then launches the vector-ALU kernel gated on the
 // same flags, and whichever of the two the data rules out leaves at once. (3) Otherwise not taken.
 // Returns 0 when the product is done or a launch failed (rc), 1 when the caller has to launch the
@@ -586,7 +625,7 @@ static int try_digits(Args<T>& g, double valu_est_us, int* rc) {
     if (r <= 0) { *rc = r; return 0; }
     return 1;   // no scratch memory for the digit planes
   }
-  // the scan and an early-leaving kernel or two cost about 10 us when the data says no
+  // the first splitting pass and an early-leaving kernel or two cost about 10 us when the data says no
   const double per_pair = pl.main_us / NPAIRS, fixed = pl.split_us * 0.6 + 10.0;
   int max_pairs = (int)((0.8 * valu_est_us - fixed) / per_pair);
   if (const char* e = getenv("AM_HIP_GEMM_SPEC_PAIRS")) max_pairs = atoi(e);   // tests

@@ -152,10 +152,10 @@ def other_workloads(am, timer, steps, warmup, ceilings):
         wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
         tops = 2.0 * n ** 3 / (ev / k) / 1e12
         entry = dict(workload=f"i32 GEMM 4096^3, {label} (wraparound; {pairs} of 10 int8 digit-pair products on the matrix cores, "
-                              "timed with the scan and split passes)",
+                              "timed with the two digit-splitting passes)",
                      unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
                      roofline=dict(bound="mfma", achieved=round(pairs * tops, 1), peak=MFMA_I8_PEAK_TOPS,
-                                   unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, scan and split passes included",
+                                   unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, two digit-splitting passes included",
                                    frac=round(pairs * tops / MFMA_I8_PEAK_TOPS, 4)),
                      speedup_over_valu_ceiling=round(tops / peak, 2) if peak else None)
         if lo == -100:
@@ -184,10 +184,10 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     peak64 = ceilings.get("valu_int64_mac")
     valu_tops = 2.0 * n ** 3 / (ev_valu / 3) / 1e12
     out.append(dict(workload="i64 GEMM 4096^3, entries in [-100, 100] (wraparound; 1 of 36 int8 digit-pair products on the matrix cores, "
-                             "timed with the scan and split passes)",
+                             "timed with the two digit-splitting passes)",
                     unit="Top/s", dtype="i64", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
                     roofline=dict(bound="mfma", achieved=round(2.0 * n ** 3 / (ev / k) / 1e12, 1), peak=MFMA_I8_PEAK_TOPS,
-                                  unit="int8 TOP/s executed (1 digit pair x 2*M*N*K) over the whole call, scan and split passes included",
+                                  unit="int8 TOP/s executed (1 digit pair x 2*M*N*K) over the whole call, two digit-splitting passes included",
                                   frac=round(2.0 * n ** 3 / (ev / k) / 1e12 / MFMA_I8_PEAK_TOPS, 4)),
                     valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / 3 * 1e3, 4),
                                      roofline=dict(bound="valu (measured int64 multiply-add ceiling)", achieved=round(valu_tops, 3),
@@ -331,7 +331,7 @@ def config_report(am, timer, L):
             pairs = digit_pairs(A, B)
             gemm_case(f"{sfx} GEMM {n}^3, entries in [-100, 100] (library's choice: digit-sliced int8 MFMA, {pairs} digit pair)", sfx, n, n, n,
                       A, B, am.toHip(A), am.toHip(B), peak=MFMA_I8_PEAK_TOPS / pairs,
-                      peak_used=f"int8 MFMA 5000 TOP/s / {pairs} digit-pair product(s) executed; whole call incl. the scan and split passes",
+                      peak_used=f"int8 MFMA 5000 TOP/s / {pairs} digit-pair product(s) executed; whole call incl. the two digit-splitting passes",
                       unit="Top/s", steps=20)
             os.environ[env] = "valu"
             try:
@@ -348,7 +348,7 @@ def config_report(am, timer, L):
         pairs = digit_pairs(A, B)
         gemm_case(f"{sfx} GEMM {n}^3, entries over the whole {sfx} range (library's choice: digit-sliced int8 MFMA, all {pairs} digit pairs)",
                   sfx, n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_I8_PEAK_TOPS / pairs,
-                  peak_used=f"int8 MFMA 5000 TOP/s / {pairs} digit-pair products executed; whole call incl. the scan and split passes",
+                  peak_used=f"int8 MFMA 5000 TOP/s / {pairs} digit-pair products executed; whole call incl. the two digit-splitting passes",
                   unit="Top/s", steps=10)
     pa = rng(3001).standard_normal((1024, 2048)); pb = rng(3002).standard_normal((1024, 6144))
     C0 = rng(3003).standard_normal((2048, 3072))
