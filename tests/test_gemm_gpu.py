@@ -740,3 +740,27 @@ def test_integer_data_dependent_path(hip, oracle, sfx, monkeypatch):
                 dC = hip.toHip(C)
                 hip.gemm(3, dA, dB, -2, dC)
                 assert np.array_equal(dC.toCpu(), want), (lo, hi, limit, splitk)
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+def test_digit_path_broadcast_and_reversed_operands(hip, oracle, sfx, monkeypatch):
+    """Zero and negative strides reach the digit-splitting passes as element loads: a row broadcast
+    over all rows of A, B with its rows and columns reversed, and both at once."""
+    monkeypatch.setenv(f"AM_HIP_GEMM_{sfx.upper()}_PATH", "mfma")
+    dt = DTYPES[sfx]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(seed_of("digit-bcast", sfx))
+    M, N, K = 70, 130, 300
+    row = fill(rng, (1, K), dt, info.min, info.max)
+    B = fill(rng, (K, N), dt, info.min, info.max)
+    A = fill(rng, (M, K), dt, -300, 300)
+    dB = hip.toHip(B)
+    say("digit path, broadcast A", sfx)
+    got = (hip.toHip(row).broadcast((M, K)) * dB).toCpu()
+    assert np.array_equal(got, oracle.matmul(np.ascontiguousarray(np.broadcast_to(row, (M, K))), B))
+    say("digit path, reversed B", sfx)
+    got = (hip.toHip(A) * dB[::-1, ::-1]).toCpu()
+    assert np.array_equal(got, oracle.matmul(A, np.ascontiguousarray(B[::-1, ::-1])))
+    say("digit path, both", sfx)
+    got = (hip.toHip(row).broadcast((M, K)) * dB[::-1, ::-1]).toCpu()
+    assert np.array_equal(got, oracle.matmul(np.ascontiguousarray(np.broadcast_to(row, (M, K))), np.ascontiguousarray(B[::-1, ::-1])))
