@@ -764,3 +764,29 @@ def test_digit_path_broadcast_and_reversed_operands(hip, oracle, sfx, monkeypatc
     say("digit path, both", sfx)
     got = (hip.toHip(row).broadcast((M, K)) * dB[::-1, ::-1]).toCpu()
     assert np.array_equal(got, oracle.matmul(np.ascontiguousarray(np.broadcast_to(row, (M, K))), np.ascontiguousarray(B[::-1, ::-1])))
+
+
+def test_random_products_all_routes(hip, oracle):
+    """120 seeded random products: element type, extents from 1 to 700 (log-uniform, so that the
+    small-product, tiled, split-k, VALU and digit-sliced routes all get picked by the library on its
+    own), layout of A, B and C, alpha / beta. Integers bit-exact, floats within the tolerance."""
+    from conftest import strided_view, view_of
+    rng = np.random.default_rng(20240607)
+    dest_kinds = ["C", "F", "rowstep2", "colstep2", "inner_block"]
+    for case in range(120):
+        sfx = ALL[case % len(ALL)]
+        dt = DTYPES[sfx]
+        M, N, K = (int(round(np.exp(rng.uniform(0, np.log(700))))) for _ in range(3))
+        ka, kb = rng.choice(VIEW_KINDS), rng.choice(VIEW_KINDS)
+        kc = rng.choice(dest_kinds)
+        alpha, beta = [(1, 0), (1, 1), (2, -1), (-3, 2), (0, 1)][int(rng.integers(0, 5))]
+        A, pa = strided_view(rng, (M, K), dt, ka)
+        B, pb = strided_view(rng, (K, N), dt, kb)
+        Cv, pc = strided_view(rng, (M, N), dt, kc)
+        say("random product", case, sfx, (M, N, K), ka, kb, kc, alpha, beta)
+        dA, dB = device_view(hip, pa, ka, (M, K)), device_view(hip, pb, kb, (K, N))
+        dC = device_view(hip, pc, kc, (M, N))
+        hip.gemm(alpha, dA, dB, beta, dC)
+        oracle.gemm_strided(alpha, A, B, beta, Cv)          # through the NumPy view into `pc`
+        after = hip.HipTensor(hip.Layout(pc.shape, tuple(st // pc.itemsize for st in pc.strides), 0), dC.storage, dC.dtype).toCpu()
+        assert_parity(oracle, sfx, view_of(after, kc, (M, N)), Cv, f"case {case}: {sfx} {(M, N, K)} {ka} {kb} {kc} a={alpha} b={beta}")
