@@ -447,12 +447,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
           __builtin_amdgcn_s_barrier();
           read_frags(std::integral_constant<int, 0>(), nxt, 0);   // NKS is even
         }
-        __builtin_amdgcn_sched_barrier(0);
+        // the fragment reads above are for the next k-step: they are spread between this step's matrix
+        // instructions (a wavefront issues in order; in front of them they would only delay them)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int m = 0; m < TM * TN; ++m) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+          __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);   // address arithmetic
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       cur = nxt;

@@ -214,15 +214,29 @@ void gemm_mfma(Args<T> p) {
         la.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
         lb.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
       }
-      // The instruction scheduler would otherwise sink these reads and loads down to their first
-      // use; they have to be issued here, ahead of the MFMAs that cover their latency.
-      __builtin_amdgcn_sched_barrier(0);
+      // Left alone, the instruction scheduler sinks the reads and loads above down to their first use.
+      // With fragment prefetch (the operands of this k-step are already in registers) they are spread
+      // between this k-step's matrix instructions instead: a wavefront issues in order, so whatever
+      // stands in front of its matrix instructions delays them (measured: +15 % on 64 x 64 tiles with one
+      // wavefront per SIMD, +2 to 7 % on the large ones). Without prefetch they have to come first.
+      constexpr bool ILV = FPF;
+      if constexpr (!ILV) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s = 0; s < VK; ++s)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[FPF ? (ks & 1) : 0][i][s], bf[FPF ? (ks & 1) : 0][j][s], acc[i][j]);
+      if constexpr (ILV) {
+#pragma unroll
+        for (int m = 0; m < VK * TM * TN; ++m) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // LDS reads
+          __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);   // LDS writes
+          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);   // global loads
+          __builtin_amdgcn_sched_group_barrier(0x006, 8, 0);   // address arithmetic
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
