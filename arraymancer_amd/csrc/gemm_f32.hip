@@ -14,7 +14,7 @@ static int run_f32(Args<float>& g) {
   if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
   // Candidate workgroup tiles with the relative MFMA efficiency of each (measured on 2048^3 and
   // 4096^3). PF = 2 (two slabs of global loads in flight) on the tiles whose slab is short.
-  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.85}, {64, 64, 0.70}, {256, 128, 0.97}, {128, 64, 0.82}, {32, 32, 0.5}};
+  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.94}, {64, 64, 0.88}, {256, 128, 0.97}, {128, 64, 0.92}, {32, 32, 0.74}};
   switch (choose_tile(cand, 6, g.M, g.N, "AM_HIP_GEMM_TILE_F32", g.batch)) {
     case 0: return launch_kinds<float, 256, 256, 16, 2, 4>(g, ak, bk);
     case 1: return launch_kinds<float, 128, 128, 16, 2, 2, 2>(g, ak, bk);
