@@ -220,13 +220,36 @@ void gemm_mfma(Args<T> p) {
       // stands in front of its matrix instructions delays them (measured: +15 % on 64 x 64 tiles with one
       // wavefront per SIMD, +2 to 7 % on the large ones). Without prefetch they have to come first.
       constexpr bool ILV = FPF;
-      if constexpr (!ILV) __builtin_amdgcn_sched_barrier(0);
+      if constexpr (ILV) {
 #pragma unroll
-      for (int s = 0; s < VK; ++s)
+        for (int s = 0; s < VK; ++s)
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[ks & 1][i][s], bf[ks & 1][j][s], acc[i][j]);
+      } else {
+        // No prefetch: this k-step's own fragments were requested just above. Row block by row block,
+        // so that the matrix instructions of block i can start once the B fragments and A fragment i
+        // are in, while the reads of the later A fragments and everything else go on between them.
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[FPF ? (ks & 1) : 0][i][s], bf[FPF ? (ks & 1) : 0][j][s], acc[i][j]);
+          for (int s = 0; s < VK; ++s)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[0][i][s], bf[0][j][s], acc[i][j]);
+        constexpr int RA = AK == kKContig ? 1 : VK, RB = BKIND == kKContig ? 1 : VK;   // LDS reads per fragment
+        __builtin_amdgcn_sched_group_barrier(0x100, TN * RB + RA, 0);   // the B fragments and A fragment 0
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int m = 0; m < VK * TN; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (m == 0 && i + 1 < TM) __builtin_amdgcn_sched_group_barrier(0x100, RA, 0);   // A fragment i + 1
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);
+          }
+      }
       if constexpr (ILV) {
 #pragma unroll
         for (int m = 0; m < VK * TM * TN; ++m) {
