@@ -16,7 +16,7 @@ static int run_f32(Args<float>& g) {
   // 4096^3). PF = 2 (two slabs of global loads in flight) on the tiles whose slab is short.
   static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.94}, {64, 64, 0.88}, {256, 128, 0.97}, {128, 64, 0.92}, {32, 32, 0.74}};
   switch (choose_tile(cand, 6, g.M, g.N, "AM_HIP_GEMM_TILE_F32", g.batch)) {
-    case 0: return launch_kinds<float, 256, 256, 16, 2, 4>(g, ak, bk);
+    case 0: return launch_kinds<float, 256, 256, 16, 2, 4, 1, true, false>(g, ak, bk);   // its loop is long enough: unrolling it over the ring costs 4 %
     case 1: return launch_kinds<float, 128, 128, 16, 2, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2, 2>(g, ak, bk);
     case 3: return launch_kinds<float, 256, 128, 16, 4, 2>(g, ak, bk);

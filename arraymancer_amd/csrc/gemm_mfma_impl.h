@@ -86,7 +86,7 @@ __device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, 
 // trip (measured: f64 128 x 128 falls from 61 to 48 TFLOP/s).
 constexpr int mfma_min_blocks(int nt) { return nt <= 256 ? 2 : 1; }
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF, bool FPF, int AK, int BKIND>
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF, bool FPF, bool RU, int AK, int BKIND>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 : 1))
 void gemm_mfma(Args<T> p) {
   typedef Mfma<T> MF;
@@ -193,19 +193,24 @@ void gemm_mfma(Args<T> p) {
   if constexpr (FPF) read_frags(std::integral_constant<int, 0>(), sA[0], sB[0], 0);
 
   int cur = 0;   // ring position of the slab being multiplied
-  auto slab = [&](auto stage_tag, auto mask_tag, int64_t kt) {
+  // cur_tag >= 0: the ring position is known at compile time (the steady-state loop is unrolled over the
+  // ring), so every LDS address of the slab is a constant offset and no address arithmetic stands
+  // between the matrix instructions and the fragment reads; -1: taken from `cur` (the last few slabs).
+  auto slab = [&](auto stage_tag, auto mask_tag, auto cur_tag, int64_t kt) {
     constexpr int S = decltype(stage_tag)::value;
     constexpr bool MASK = decltype(mask_tag)::value;
-    const int nxt = (cur == 2) ? 0 : cur + 1;
+    constexpr int CT = decltype(cur_tag)::value;
+    const int here = CT >= 0 ? CT : cur;
+    const int nxt = (here == 2) ? 0 : here + 1;
     const int nxt2 = (nxt == 2) ? 0 : nxt + 1;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       // fragments for the k-step after this one: next k-step of this slab, or first of the next slab
-      if constexpr (!FPF) read_frags(std::integral_constant<int, 0>(), sA[cur], sB[cur], ks);
+      if constexpr (!FPF) read_frags(std::integral_constant<int, 0>(), sA[here], sB[here], ks);
       if (ks + 1 < NKS) {
         if constexpr (FPF) {
-          if (ks & 1) read_frags(std::integral_constant<int, 0>(), sA[cur], sB[cur], ks + 1);
-          else read_frags(std::integral_constant<int, 1>(), sA[cur], sB[cur], ks + 1);
+          if (ks & 1) read_frags(std::integral_constant<int, 0>(), sA[here], sB[here], ks + 1);
+          else read_frags(std::integral_constant<int, 1>(), sA[here], sB[here], ks + 1);
         }
       } else {
         if constexpr (FPF) read_frags(std::integral_constant<int, 0>(), sA[nxt], sB[nxt], 0);   // NKS is even
@@ -268,13 +273,32 @@ void gemm_mfma(Args<T> p) {
   // Steady state: every slab this iteration fetches or commits lies wholly inside the k range,
   // so no clamping or zeroing is compiled in. The last few slabs run the masked version.
   int64_t kt = 0;
+  typedef std::integral_constant<int, 0> c0;
+  typedef std::integral_constant<int, 1> c1;
+  typedef std::integral_constant<int, 2> c2;
+  typedef std::integral_constant<int, -1> dyn;
+  constexpr int UNR = PF == 1 ? 3 : 6;   // whole turns of the ring, a whole number of register stages
+  for (; RU && kt + (UNR - 1) + 2 + PF < full_slabs; kt += UNR) {   // starts and ends at ring position 0
+    if constexpr (PF == 1) {
+      slab(c0(), std::false_type(), c0(), kt);
+      slab(c0(), std::false_type(), c1(), kt + 1);
+      slab(c0(), std::false_type(), c2(), kt + 2);
+    } else {
+      slab(c0(), std::false_type(), c0(), kt);
+      slab(c1(), std::false_type(), c1(), kt + 1);
+      slab(c0(), std::false_type(), c2(), kt + 2);
+      slab(c1(), std::false_type(), c0(), kt + 3);
+      slab(c0(), std::false_type(), c1(), kt + 4);
+      slab(c1(), std::false_type(), c2(), kt + 5);
+    }
+  }
   for (; kt + (PF - 1) + 2 + PF < full_slabs; kt += PF) {
-    slab(std::integral_constant<int, 0>(), std::false_type(), kt);
-    if constexpr (PF > 1) slab(std::integral_constant<int, 1>(), std::false_type(), kt + 1);
+    slab(c0(), std::false_type(), dyn(), kt);
+    if constexpr (PF > 1) slab(c1(), std::false_type(), dyn(), kt + 1);
   }
   for (; kt < kt_run; kt += PF) {
-    slab(std::integral_constant<int, 0>(), std::true_type(), kt);
-    if constexpr (PF > 1) slab(std::integral_constant<int, 1>(), std::true_type(), kt + 1);
+    slab(c0(), std::true_type(), dyn(), kt);
+    if constexpr (PF > 1) slab(c1(), std::true_type(), dyn(), kt + 1);
   }
 
   // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
@@ -342,7 +366,8 @@ void gemm_mfma(Args<T> p) {
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true>
+// PF: register stages of global loads; FPF: fragment prefetch; RU: steady-state loop unrolled over the LDS ring.
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true, bool RU = true>
 static int launch_kinds(Args<T>& g, int ak, int bk) {
   g.tiles_m = (int)((g.M + BM - 1) / BM);
   g.tiles_n = (int)((g.N + BN - 1) / BN);
@@ -351,7 +376,7 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
   plan_splitk(g, BK, WAVES_M * WAVES_N);
   const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(WAVES_M * WAVES_N * 64);
 #define AM_LAUNCH(AKIND, BKIND_)                                                                   \
-  hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, AKIND, BKIND_>), grid, block, 0, \
+  hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, AKIND, BKIND_>), grid, block, 0, \
                      stream(), g)
   switch (ak * 3 + bk) {
     case 0: AM_LAUNCH(kKContig, kKContig); break;
