@@ -18,7 +18,7 @@ static int run_f64(Args<double>& g) {
   // 128 x 192 (8 wavefronts of 64 x 48) exists for shapes that the others cut into a number of
   // tiles just above a multiple of the CU count: 2048 x 3072 is 384 tiles of 128 x 128 (two rounds,
   // the second half empty) but exactly 256 of 128 x 192.
-  static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.95}, {32, 32, 0.78}, {256, 128, 0.95}, {128, 64, 0.98}, {128, 192, 1.0}};
+  static const TileChoice cand[] = {{128, 128, 0.97}, {64, 64, 0.93}, {32, 32, 0.76}, {256, 128, 1.0}, {128, 64, 0.96}, {128, 192, 0.98}};
   switch (choose_tile(cand, 6, g.M, g.N, "AM_HIP_GEMM_TILE_F64", g.batch)) {
     case 0: return launch_kinds<double, 128, 128, 16, 2, 4>(g, ak, bk);
     case 1: return launch_kinds<double, 64, 64, 16, 2, 2, 2>(g, ak, bk);
