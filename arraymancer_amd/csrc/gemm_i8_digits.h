@@ -45,7 +45,7 @@ namespace gemm {
 namespace i8 {
 
 constexpr int kRowPad = 256;   // operand planes are padded to this many rows (largest tile edge) ...
-constexpr int kKPad = 128;     // ... and to this many k (largest slab)
+constexpr int kKPad = 256;     // ... and to this many k (a whole turn of the LDS ring: four slabs of 64)
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -424,45 +424,87 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
   __syncthreads();
   read_frags(std::integral_constant<int, 0>(), 0, 0);
 
-  int cur = 0;
-  int64_t t = 0;
   // One inner loop per pair keeps the end-of-pair arithmetic out of the slab loop's body (as a
-  // branch inside one flat loop the compiler turns it into selects executed for every slab).
-  for (int pr = 0; pr < n_pairs; ++pr) {
-    const int64_t t_end = t + slabs_per_pair;
-    for (; t < t_end; ++t) {
-      const int nxt = cur == RING - 1 ? 0 : cur + 1, last = cur == 0 ? RING - 1 : cur - 1;
-      fetch(last);   // slab t + RING - 1; its buffer held slab t - 1, which every wavefront left before the last barrier
+  // branch inside one flat loop the compiler turns it into selects executed for every slab). The
+  // planes are padded to a whole number of turns of the ring per pair, so the loop can be unrolled over
+  // the ring: the ring position is then a compile-time constant and every LDS address a constant offset
+  // (the lambda below). That pays for the 256 x 128 tile (int64: 96 -> 90 us per pair at 4096^3); the
+  // 256 x 256 tile is faster with the rolled loop further down (69 against 74 us), the same steps with the
+  // position in `cur`.
+  int cur = 0;   // ring position of the slab being multiplied (rolled loop)
+  auto slab = [&](auto cur_tag) {
+    constexpr int CUR = decltype(cur_tag)::value;
+    constexpr int NXT = CUR == RING - 1 ? 0 : CUR + 1, LAST = CUR == 0 ? RING - 1 : CUR - 1;
+    fetch(LAST);   // slab t + RING - 1; its buffer held slab t - 1, which every wavefront left before the last barrier
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        if (ks + 1 < NKS) {
-          if (ks & 1) read_frags(std::integral_constant<int, 0>(), cur, ks + 1);
-          else read_frags(std::integral_constant<int, 1>(), cur, ks + 1);
-        } else {
-          // Slab t + 1 was requested RING - 2 slabs ago: wait for this wavefront's part of it (vmcnt <= the
-          // loads of the later slabs) and for its own outstanding reads of slab t (lgkmcnt 0: the matrix
-          // instructions below need them anyway), then for everyone's. A bare barrier: the fence of
-          // __syncthreads would drain the later slabs' loads as well.
-          __builtin_amdgcn_s_waitcnt(0x0070 | ((RING - 2) * (LPA + LPB)));
-          __builtin_amdgcn_s_barrier();
-          read_frags(std::integral_constant<int, 0>(), nxt, 0);   // NKS is even
-        }
-        // the fragment reads above are for the next k-step: they are spread between this step's matrix
-        // instructions (a wavefront issues in order; in front of them they would only delay them)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
-#pragma unroll
-        for (int m = 0; m < TM * TN; ++m) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-          __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);   // address arithmetic
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (ks + 1 < NKS) {
+        if (ks & 1) read_frags(std::integral_constant<int, 0>(), CUR, ks + 1);
+        else read_frags(std::integral_constant<int, 1>(), CUR, ks + 1);
+      } else {
+        // Slab t + 1 was requested RING - 2 slabs ago: wait for this wavefront's part of it (vmcnt <= the
+        // loads of the later slabs) and for its own outstanding reads of slab t (lgkmcnt 0: the matrix
+        // instructions below need them anyway), then for everyone's. A bare barrier: the fence of
+        // __syncthreads would drain the later slabs' loads as well.
+        __builtin_amdgcn_s_waitcnt(0x0070 | ((RING - 2) * (LPA + LPB)));
+        __builtin_amdgcn_s_barrier();
+        read_frags(std::integral_constant<int, 0>(), NXT, 0);   // NKS is even
       }
-      cur = nxt;
+      // the fragment reads above are for the next k-step: they are spread between this step's matrix
+      // instructions (a wavefront issues in order; in front of them they would only delay them)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int m = 0; m < TM * TN; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);   // address arithmetic
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  static_assert(RING == 4, "the slab loop below is written out for a ring of four");
+  constexpr bool UNROLL_RING = BM * BN < 256 * 256;
+  for (int pr = 0; pr < n_pairs; ++pr) {
+    if constexpr (UNROLL_RING) {
+      for (int64_t t = 0; t < slabs_per_pair; t += RING) {   // slabs_per_pair is a multiple of RING (kKPad)
+        slab(std::integral_constant<int, 0>());
+        slab(std::integral_constant<int, 1>());
+        slab(std::integral_constant<int, 2>());
+        slab(std::integral_constant<int, 3>());
+      }
+    } else {
+      for (int64_t t = 0; t < slabs_per_pair; ++t) {
+        const int nxt = cur == RING - 1 ? 0 : cur + 1, last = cur == 0 ? RING - 1 : cur - 1;
+        fetch(last);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          if (ks + 1 < NKS) {
+            if (ks & 1) read_frags(std::integral_constant<int, 0>(), cur, ks + 1);
+            else read_frags(std::integral_constant<int, 1>(), cur, ks + 1);
+          } else {
+            __builtin_amdgcn_s_waitcnt(0x0070 | ((RING - 2) * (LPA + LPB)));
+            __builtin_amdgcn_s_barrier();
+            read_frags(std::integral_constant<int, 0>(), nxt, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
+#pragma unroll
+          for (int m = 0; m < TM * TN; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        cur = nxt;
+      }
     }
     // the pair is done: Horner step(s) down to the next pair's s (or to s = 0 after the last one)
     const int sh = tab_shift[pr + 1];
@@ -600,10 +642,10 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
   if constexpr (sizeof(T) == 8) {
-    hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 5>), grid, block, 0, stream(), d);
+    hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 4>), grid, block, 0, stream(), d);
   } else {
     if (big) hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 4, 2, 64, 4>), grid, block, 0, stream(), d);
-    else hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 5>), grid, block, 0, stream(), d);
+    else hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 4>), grid, block, 0, stream(), d);
   }
   const int rc = check_launch("gemm_i8_digits");
   // The planes go back to the allocator's cache at once: whoever gets the block next reaches it
