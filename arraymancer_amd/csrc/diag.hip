@@ -47,6 +47,28 @@ __global__ __launch_bounds__(256) void peak_mfma_f64(int iters, double* out) {
   if (s == 12345.678) out[0] = s;
 }
 
+// int8 matrix instruction of the digit-sliced integer GEMM; operands with mixed byte values (the power
+// drawn, and with it the clock the chip settles at, depends on how many bits toggle).
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256) void peak_mfma_i8(int iters, int* out) {
+  v16i acc[4];   // four chains: 64 accumulator registers, 32 cycles apart
+  for (int c = 0; c < 4; ++c)
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0;
+  const int t = (int)threadIdx.x;
+  const v4i a = {0x5a3c9671 + t * 0x01010101, 0x1234fedc ^ t, (int)0x9e3779b9 * (t + 1), 0x7f80017f};
+  const v4i b = {(int)0x85ebca6b * (t + 3), 0x0badf00d + t, 0x13579bdf ^ (t << 8), (int)0xc2b2ae35};
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc[c]) : "v"(a), "v"(b));
+  }
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  int s = 0;
+  for (int c = 0; c < 4; ++c) s += acc[c][0] + acc[c][15];
+  if (s == 0x12345678) out[0] = s;
+}
+
 // 8 x 8 register tile of wrapping 32-bit multiply-accumulates per step: the inner body of the
 // integer GEMM kernel without its LDS reads.
 template <typename U>
@@ -75,7 +97,8 @@ __global__ __launch_bounds__(256) void peak_valu_mac(int iters, U* out, U seed) 
 }  // namespace
 
 // kind: 0 = MFMA f32 32x32x2 (FLOP/s), 1 = MFMA f64 16x16x4 (FLOP/s),
-//       2 = VALU int32 multiply-add (integer op/s, 2 per MAC), 3 = VALU int64 multiply-add.
+//       2 = VALU int32 multiply-add (integer op/s, 2 per MAC), 3 = VALU int64 multiply-add,
+//       4 = MFMA i32 32x32x32 int8 (integer op/s).
 // Launches `waves_per_simd` wavefronts on every SIMD of the device, `iters` loop trips each.
 extern "C" int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second) {
   if (!ops_per_second || iters <= 0 || waves_per_simd < 1 || waves_per_simd > 8)
@@ -106,6 +129,10 @@ extern "C" int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double*
       case 3:
         hipLaunchKernelGGL(peak_valu_mac<uint64_t>, dim3(blocks), dim3(256), 0, stream(), iters, (uint64_t*)scratch, (uint64_t)12345);
         ops_per_launch = (double)blocks * 256 * iters * 64 * 2.0;
+        break;
+      case 4:
+        hipLaunchKernelGGL(peak_mfma_i8, dim3(blocks), dim3(256), 0, stream(), iters, (int*)scratch);
+        ops_per_launch = (double)blocks * 4 * iters * 4 * (32.0 * 32 * 32 * 2);
         break;
       default:
         (void)hipFree(scratch);

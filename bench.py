@@ -76,7 +76,8 @@ def measured_ceilings(L):
     """Issue ceilings of this chip from register-only micro-benchmarks (no memory traffic): what a
     perfect kernel could reach at the clocks the device sustains. T(FL)OP/s."""
     out = {}
-    for kind, name, iters in [(0, "mfma_f32", 20000), (1, "mfma_f64", 20000), (2, "valu_int32_mac", 20000), (3, "valu_int64_mac", 5000)]:
+    for kind, name, iters in [(0, "mfma_f32", 20000), (1, "mfma_f64", 20000), (2, "valu_int32_mac", 20000), (3, "valu_int64_mac", 5000),
+                              (4, "mfma_i8", 20000)]:
         v = ctypes.c_double()
         if L.am_hip_diag_peak(kind, iters, 2, ctypes.byref(v)) == 0:
             out[name] = round(v.value / 1e12, 2)

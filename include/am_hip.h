@@ -394,6 +394,7 @@ int am_hip_maxpool2d_i64(int64_t N, int C, int H, int W, int kH, int kW, int pad
  *   kind 0: MFMA f32 32x32x2 (FLOP/s)      kind 1: MFMA f64 16x16x4 (FLOP/s)
  *   kind 2: VALU int32 wrapping multiply-add, 8x8 register tile (integer op/s, 2 per MAC)
  *   kind 3: VALU int64 multiply-add
+ *   kind 4: MFMA int8 32x32x32 (integer op/s), the instruction of the digit-sliced integer GEMM
  * waves_per_simd wavefronts are resident on every SIMD (1..8); iters loop trips each. */
 int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second);
 
