@@ -166,7 +166,7 @@ static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
   const int64_t cus = num_cus();
   // Enough independent work for the whole chip: if the outputs alone do not supply it, cut the axis.
   const int64_t units = row_kernel ? g.outputs : (g.outputs + 255) / 256;   // wavefronts resp. workgroups
-  const int64_t want_units = row_kernel ? cus * 32 : cus * 2;
+  const int64_t want_units = row_kernel ? cus * 32 : cus * 8;
   const int64_t min_chunk = row_kernel ? 4096 : 64;
   int64_t chunks = 1;
   if (units < want_units && g.L >= 2 * min_chunk) {
