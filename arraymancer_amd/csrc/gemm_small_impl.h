@@ -83,6 +83,21 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   const int64_t full1 = blk1 < nfull ? blk1 : nfull;   // end of this wavefront's whole blocks
 
   acc_t acc = {0, 0, 0, 0};
+  // The partial last block of the k range (elements past K count as zero), if this wavefront owns it:
+  // requested first, multiplied last, so that its round trip to memory runs beside the whole blocks'.
+  const bool has_tail = blk0 <= nfull && nfull < blk1;   // nfull is the number of the partial block, if there is one
+  T tail_a[4] = {0, 0, 0, 0}, tail_b[4] = {0, 0, 0, 0};
+  if (has_tail) {
+    const int64_t k = (nfull << 4) + 4 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const bool ok = k + s < p.K;
+      const int64_t kk = ok ? k + s : p.K - 1;
+      const T x = a[kk * p.a_k], y = b[kk * p.b_k];
+      tail_a[s] = ok ? x : (T)0;
+      tail_b[s] = ok ? y : (T)0;
+    }
+  }
   T av[2][CHUNK][4], bv[2][CHUNK][4];
   auto load_chunk = [&](int set, int64_t first_blk) {   // set is a constant after unrolling
 #pragma unroll
@@ -130,15 +145,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
       blk += grp;
     }
   }
-  if (blk < blk1) {   // the partial last block: elements past K count as zero
-    const int64_t k = (blk << 4) + 4 * g;
+  if (has_tail) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const bool ok = k + s < p.K;
-      const int64_t kk = ok ? k + s : p.K - 1;
-      const T x = a[kk * p.a_k], y = b[kk * p.b_k];
-      acc = M16<T>::mma(ok ? x : (T)0, ok ? y : (T)0, acc);
-    }
+    for (int s = 0; s < 4; ++s) acc = M16<T>::mma(tail_a[s], tail_b[s], acc);
   }
 
   if (nw > 1) {
@@ -226,11 +235,21 @@ static int run(const Args<T>& g_in) {
   const bool bvec = g.b_k == 1 && aligned16(g.B) && (g.b_mn % VK == 0 || g.N == 1);
   const dim3 grid((unsigned)tiles_n, (unsigned)tiles_m), block((unsigned)nw * 64);
   if (trace_choices()) fprintf(stderr, "am_hip gemm: small path, %lld x %lld tiles of 16 x 16, %d wavefronts per tile\n", (long long)tiles_m, (long long)tiles_n, nw);
+  // Chunks of four (float) or two (double) blocks of 16 k where a wavefront has that many; one block at a
+  // time where its share of k is one or two blocks: that instantiation needs a third of the registers,
+  // so all the wavefronts of a product with many tiles and a short k are resident at once.
   constexpr int CH = sizeof(T) == 4 ? 4 : 2;
-  if (avec && bvec) hipLaunchKernelGGL((gemm_rows16<T, true, true, kMaxWaves, CH>), grid, block, lds, stream(), g);
-  else if (avec) hipLaunchKernelGGL((gemm_rows16<T, true, false, kMaxWaves, CH>), grid, block, lds, stream(), g);
-  else if (bvec) hipLaunchKernelGGL((gemm_rows16<T, false, true, kMaxWaves, CH>), grid, block, lds, stream(), g);
-  else hipLaunchKernelGGL((gemm_rows16<T, false, false, kMaxWaves, CH>), grid, block, lds, stream(), g);
+  const bool short_k = (nblk + nw - 1) / nw <= 2;
+#define AM_SMALL_LAUNCH(AV, BV)                                                                              \
+  do {                                                                                                       \
+    if (short_k) hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, 1>), grid, block, lds, stream(), g);   \
+    else hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, CH>), grid, block, lds, stream(), g);          \
+  } while (0)
+  if (avec && bvec) AM_SMALL_LAUNCH(true, true);
+  else if (avec) AM_SMALL_LAUNCH(true, false);
+  else if (bvec) AM_SMALL_LAUNCH(false, true);
+  else AM_SMALL_LAUNCH(false, false);
+#undef AM_SMALL_LAUNCH
   return check_launch("gemm_rows16");
 }
 
