@@ -75,8 +75,14 @@ template <typename T, int OP> struct BinOp {
       return (x <= (T)0) ? (T)0 : y;
     } else if constexpr (OP == AM_OP_MAX) {
       return (y <= x) ? x : y;
-    } else {  // AM_OP_MIN
+    } else if constexpr (OP == AM_OP_MIN) {
       return (x <= y) ? x : y;
+    } else if constexpr (OP == AM_OP_SIGMOID_BWD) {
+      if constexpr (Traits<T>::kFloat) return x * ((T)1 - x) * y;
+      else return (T)((U)x * ((U)1 - (U)x) * (U)y);
+    } else {  // AM_OP_TANH_BWD
+      if constexpr (Traits<T>::kFloat) return y * ((T)1 - x * x);
+      else return (T)((U)y * ((U)1 - (U)x * (U)x));
     }
   }
 };
@@ -545,6 +551,7 @@ static int binary(const char* fn, int op, int rank, const int64_t* shape, T* dst
 #define AM_CASE(code) case code: return run<T, code, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0)
     AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
     AM_CASE(AM_OP_ADD_RELU); AM_CASE(AM_OP_RELU_BWD); AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN);
+    AM_CASE(AM_OP_SIGMOID_BWD); AM_CASE(AM_OP_TANH_BWD);
 #undef AM_CASE
     case AM_OP_MOD:
       if constexpr (!F) return run<T, AM_OP_MOD, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);

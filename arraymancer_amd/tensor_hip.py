@@ -483,6 +483,18 @@ def linear(x: HipTensor, weight: HipTensor, bias: HipTensor | None = None, relu:
     return gemm(1, x, weight.transpose(), 0, out, epilogue=epi, bias=bias)
 
 
+def linear_backward(input: HipTensor, weight: HipTensor, gradOutput: HipTensor, with_bias: bool = True):
+    """(gradInput, gradWeight[, gradBias]) of src/arraymancer/nn_primitives/nnp_linear.nim:39-66:
+    gradInput = gradOutput * weight, gradWeight = gradOutput.transpose * input (the transposed
+    view goes to the GEMM as strides), gradBias = sum(gradOutput, axis=0) of shape
+    [1, out_features]."""
+    grad_input = matmul(gradOutput, weight)
+    grad_weight = matmul(gradOutput.transpose(), input)
+    if not with_bias:
+        return grad_input, grad_weight
+    return grad_input, grad_weight, tsum(gradOutput, axis=0)
+
+
 # ---------------------------------------------------------------------- element-wise
 def _binary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor):
     sfx = dst.sfx
@@ -622,6 +634,27 @@ def sigmoid(t: HipTensor) -> HipTensor:
 def bias_relu(x: HipTensor, b: HipTensor) -> HipTensor:
     """map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass."""
     return _bc("add_relu", x, b)
+
+
+def tanh(t: HipTensor) -> HipTensor:
+    """src/arraymancer/nn_primitives/nnp_activation.nim:38-39."""
+    return unary("tanh", t)
+
+
+def relu_backward(gradient: HipTensor, cached_tensor: HipTensor) -> HipTensor:
+    """map2_inline(cached_tensor, gradient): if x <= 0: 0 else: y
+    (src/arraymancer/nn_primitives/nnp_activation.nim:65-70)."""
+    return map2("relu_bwd", cached_tensor, gradient)
+
+
+def sigmoid_backward(gradient: HipTensor, cached_tensor: HipTensor) -> HipTensor:
+    """map2_inline(cached_tensor, gradient): x * (1 - x) * y (nnp_activation.nim:61-63)."""
+    return map2("sigmoid_bwd", cached_tensor, gradient)
+
+
+def tanh_backward(gradient: HipTensor, cached_tensor: HipTensor) -> HipTensor:
+    """map2_inline(cached_tensor, gradient): y * (1 - x * x) (nnp_activation.nim:72-74)."""
+    return map2("tanh_bwd", cached_tensor, gradient)
 
 
 OPERATORS = {"+.": bc_add, "-.": bc_sub, "*.": bc_mul, "/.": bc_div, "mod": bc_mod,

@@ -243,10 +243,12 @@ int am_hip_dot_i64(int64_t n, const int64_t* x, int64_t incx, const int64_t* y, 
 #define AM_OP_ADD_RELU    5   /* t = a + b; (0 >= t) ? 0 : t        (fused bias + ReLU)              */
 #define AM_OP_ADD_SIGMOID 6   /* floats: 1 / (1 + exp(-(a + b)))    (GRU gates, nnp_gru.nim:78)      */
 #define AM_OP_ADD_TANH    7   /* floats: tanh(a + b)                                                */
-#define AM_OP_RELU_BWD    8   /* (a <= 0) ? 0 : b                   (nnp_activation.nim:61-74)       */
+#define AM_OP_RELU_BWD    8   /* (a <= 0) ? 0 : b                   (nnp_activation.nim:65-70)       */
 #define AM_OP_MAX         9
 #define AM_OP_MIN        10
-#define AM_OP_BINARY_COUNT 11
+#define AM_OP_SIGMOID_BWD 11  /* a * (1 - a) * b   a = cached sigmoid output (nnp_activation.nim:61-63)  */
+#define AM_OP_TANH_BWD   12   /* b * (1 - a * a)   a = cached tanh output    (nnp_activation.nim:72-74)  */
+#define AM_OP_BINARY_COUNT 13
 
 int am_hip_ew_binary_f32(int op, int rank, const int64_t* shape,
                          float* dst, const int64_t* dst_strides,

@@ -335,6 +335,10 @@ template <typename T> HipTensor<T> bc_div(const HipTensor<T>& t, T s) { return s
 template <typename T> HipTensor<T> bc_div(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_DIV, t, s, true); }
 // map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass
 template <typename T> HipTensor<T> bias_relu(const HipTensor<T>& x, const HipTensor<T>& b) { return map2(AM_OP_ADD_RELU, x, b.broadcast(x.shape)); }
+// Activation backward passes: map2_inline(cached_tensor, gradient) bodies of nnp_activation.nim:61-74.
+template <typename T> HipTensor<T> relu_backward(const HipTensor<T>& gradient, const HipTensor<T>& cached) { return map2(AM_OP_RELU_BWD, cached, gradient); }
+template <typename T> HipTensor<T> sigmoid_backward(const HipTensor<T>& gradient, const HipTensor<T>& cached) { return map2(AM_OP_SIGMOID_BWD, cached, gradient); }
+template <typename T> HipTensor<T> tanh_backward(const HipTensor<T>& gradient, const HipTensor<T>& cached) { return map2(AM_OP_TANH_BWD, cached, gradient); }
 
 // ---- GEMM -----------------------------------------------------------------------------------------
 // C <- alpha A B + beta C (operators_blas_l2l3.nim:58-81); any strides on A, B and C.
@@ -434,6 +438,14 @@ template <typename T> T min(const HipTensor<T>& t) { return reduce_all(AM_RED_MI
 template <typename T> HipTensor<T> min(const HipTensor<T>& t, int axis) { return reduce_axis(AM_RED_MIN, t, axis); }
 template <typename T> T max(const HipTensor<T>& t) { return reduce_all(AM_RED_MAX, t); }
 template <typename T> HipTensor<T> max(const HipTensor<T>& t, int axis) { return reduce_axis(AM_RED_MAX, t, axis); }
+
+// gradInput = gradOutput * weight, gradWeight = gradOutput^T * input (the transposed view reaches
+// the GEMM as strides), gradBias = sum(gradOutput, axis 0): nnp_linear.nim:39-66.
+template <typename T> struct LinearGrads { HipTensor<T> input, weight, bias; };
+template <typename T>
+LinearGrads<T> linear_backward(const HipTensor<T>& input, const HipTensor<T>& weight, const HipTensor<T>& grad_output) {
+  return {grad_output * weight, grad_output.transpose() * input, sum(grad_output, 0)};
+}
 // integers: C++ `/` truncates towards zero like Nim's `div`
 template <typename T> T mean(const HipTensor<T>& t) { return sum(t) / static_cast<T>(t.size()); }
 template <typename T> HipTensor<T> mean(const HipTensor<T>& t, int axis) {

@@ -265,6 +265,16 @@ proc biasRelu*[T: float32 | float64](x, b: HipTensor[T]): HipTensor[T] =
   ## map2_inline(x, b.broadcast(x.shape), max(0.T, x + y)) in one pass.
   map2(x, opAddRelu, b.broadcast(x.shape.toSeq))
 
+proc relu_backward*[T: HipScalar](gradient, cached_tensor: HipTensor[T]): HipTensor[T] =
+  ## nnp_activation.nim:65-70
+  map2(cached_tensor, opReluBwd, gradient)
+proc sigmoid_backward*[T: HipScalar](gradient, cached_tensor: HipTensor[T]): HipTensor[T] =
+  ## x * (1 - x) * y, nnp_activation.nim:61-63
+  map2(cached_tensor, opSigmoidBwd, gradient)
+proc tanh_backward*[T: HipScalar](gradient, cached_tensor: HipTensor[T]): HipTensor[T] =
+  ## y * (1 - x * x), nnp_activation.nim:72-74
+  map2(cached_tensor, opTanhBwd, gradient)
+
 # ---------------------------------------------------------------- GEMM
 proc gemm*[T: HipScalar](alpha: T, A, B: HipTensor[T], beta: T, C: var HipTensor[T]) =
   ## C <- alpha A B + beta C (operators_blas_l2l3.nim:58-81). Any strides; no host copy.
@@ -361,6 +371,19 @@ proc reduce_all[T: HipScalar](op: cint, t: HipTensor[T]): T =
 # aggregate.nim:33-113
 proc sum*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_SUM, t)
 proc sum*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[T] = reduce_axis(AM_RED_SUM, t, axis)
+
+proc linear_backward*[T: HipScalar](input, weight, gradOutput: HipTensor[T],
+                                    gradInput, gradWeight, gradBias: var HipTensor[T]) =
+  ## nnp_linear.nim:39-55; the transposed view reaches the GEMM as strides.
+  gradInput = gradOutput * weight
+  gradWeight = gradOutput.transpose * input
+  gradBias = sum(gradOutput, axis = 0)
+
+proc linear_backward*[T: HipScalar](input, weight, gradOutput: HipTensor[T],
+                                    gradInput, gradWeight: var HipTensor[T]) =
+  ## nnp_linear.nim:57-66
+  gradInput = gradOutput * weight
+  gradWeight = gradOutput.transpose * input
 proc product*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_PROD, t)
 proc product*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[T] = reduce_axis(AM_RED_PROD, t, axis)
 proc min*[T: HipScalar](t: HipTensor[T]): T = reduce_all(AM_RED_MIN, t)

@@ -27,7 +27,7 @@ _CT = {"f32": ctypes.c_float, "f64": ctypes.c_double, "i32": ctypes.c_int32, "i6
 
 # op codes of include/am_hip.h
 OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
-          relu_bwd=8, max=9, min=10)
+          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12)
 OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2, addmul=3)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
 
@@ -424,6 +424,10 @@ def closed_map2(op, a, b):
             return np.where(b <= a, a, b)
         if name == "min":
             return np.where(a <= b, a, b)
+        if name == "sigmoid_bwd":
+            return a * (1 - a) * b
+        if name == "tanh_bwd":
+            return b * (1 - a * a)
     raise KeyError(name)
 
 

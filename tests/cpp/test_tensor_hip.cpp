@@ -147,6 +147,16 @@ static void fused_linear() {
   CHECK(eq(am::linear(x, w, b, true), {1.5f, 1.5f, 7, 0, 0, 0, 0, 6}));
   CHECK(eq(am::bias_relu(x, toHip<float>({-2, 0, 2}, {1, 3})), {0, 2, 5, 0, 0, 0}));
   CHECK(eq(am::relu(x), {1, 2, 3, 0, 0, 0}));
+  // nnp_linear.nim:39-55 on values small enough to be exact
+  auto g = toHip<float>({1, 0, 2, -1, 0, 1, 0, 1}, {2, 4});
+  auto grads = am::linear_backward(x, w, g);
+  CHECK(eq(grads.input, {4, 3, 3, -1, 0, -1}));
+  CHECK(eq(grads.weight, {1, 2, 3, -1, -2, -3, 2, 4, 6, -2, -4, -6}));
+  CHECK(grads.bias.shape == (Shape{1, 4}) && eq(grads.bias, {1, 1, 2, 0}));
+  // nnp_activation.nim:61-74
+  CHECK(eq(am::relu_backward(toHip<float>({1, 2, 3, 4, 5, 6}, {2, 3}), x), {1, 2, 3, 0, 0, 0}));
+  CHECK(eq(am::sigmoid_backward(toHip<float>({4, 16}, {2}), toHip<float>({0.5f, 0.25f}, {2})), {1, 3}));
+  CHECK(eq(am::tanh_backward(toHip<float>({4, 8}, {2}), toHip<float>({0.5f, -0.5f}, {2})), {3, 6}));
 }
 
 template <typename T>

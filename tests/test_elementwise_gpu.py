@@ -107,7 +107,7 @@ def test_reference_map2_bool(hip, vectors):
 
 # ------------------------------------------------------------------ oracle / NumPy parity
 SHAPES = [(1,), (3,), (1000,), (4099,), (7, 13), (64, 4096), (33, 4100), (5, 6, 7), (2, 3, 4, 5, 6, 2), (300, 1), (1, 300)]
-BIN_OPS = ["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min"]
+BIN_OPS = ["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min", "sigmoid_bwd", "tanh_bwd"]
 
 
 @pytest.mark.parametrize("sfx", ALL)
@@ -345,3 +345,29 @@ def test_mixed_unit_stride_axes(hip, oracle, sfx, shape):
     assert np.array_equal(dD.toCpu(), (Bt.T + A).T)
     dDt.bc_imul(dv)
     assert np.array_equal(dD.toCpu(), ((Bt.T + A) * v).T)
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_activation_backward(hip, oracle, sfx):
+    """relu / sigmoid / tanh backward (nnp_activation.nim:61-74): map2 over (cached output,
+    gradient), bit-exact against the oracle and the NumPy statement; sigmoid and tanh backward
+    agree with central differences of the device forward pass."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(77)
+    x, g = fill(rng, (33, 130), dt), fill(rng, (33, 130), dt)
+    dx, dg = hip.toHip(x), hip.toHip(g)
+    say("activation backward", sfx)
+    assert np.array_equal(hip.relu_backward(dg, dx).toCpu(), np.where(x <= 0, dt(0), g))
+    s, t = hip.sigmoid(dx), hip.tanh(dx)
+    cs, ct = s.toCpu(), t.toCpu()
+    assert np.array_equal(hip.sigmoid_backward(dg, s).toCpu(), cs * (1 - cs) * g)
+    assert np.array_equal(hip.tanh_backward(dg, t).toCpu(), g * (1 - ct * ct))
+    assert np.array_equal(hip.sigmoid_backward(dg, s).toCpu(), oracle.map2("sigmoid_bwd", cs, g))
+    assert np.array_equal(hip.tanh_backward(dg, t.transpose().clone().transpose()).toCpu(), oracle.map2("tanh_bwd", ct, g))
+    if sfx == "f64":
+        h = 1e-6
+        up, dn = hip.toHip(x + h), hip.toHip(x - h)
+        num = (hip.sigmoid(up).toCpu() - hip.sigmoid(dn).toCpu()) / (2 * h) * g
+        assert np.allclose(num, hip.sigmoid_backward(dg, s).toCpu(), rtol=1e-6, atol=1e-9)
+        num = (hip.tanh(up).toCpu() - hip.tanh(dn).toCpu()) / (2 * h) * g
+        assert np.allclose(num, hip.tanh_backward(dg, t).toCpu(), rtol=1e-6, atol=1e-9)

@@ -207,6 +207,48 @@ def test_empty_extents_leave_c_untouched(hip, sfx):
     assert (hip.empty((0, 3), dt) * hip.empty((3, 4), dt)).shape == (0, 4)
 
 
+@pytest.mark.parametrize("sfx", ALL)
+def test_linear_backward(hip, oracle, sfx):
+    """gradInput = gradOutput * weight, gradWeight = gradOutput.transpose * input,
+    gradBias = sum(gradOutput, axis=0) (nnp_linear.nim:39-66) against the oracle's GEMM and fold,
+    at the dense layer of the MNIST chain and at a ragged shape."""
+    dt = DTYPES[sfx]
+    for batch, fin, fout in ((64, 800, 500), (37, 129, 61)):
+        rng = np.random.default_rng(batch)
+        x, W, g = fill(rng, (batch, fin), dt), fill(rng, (fout, fin), dt), fill(rng, (batch, fout), dt)
+        say("linear_backward", sfx, batch, fin, fout)
+        gi, gw, gb = hip.linear_backward(hip.toHip(x), hip.toHip(W), hip.toHip(g))
+        assert gi.shape == (batch, fin) and gw.shape == (fout, fin) and gb.shape == (1, fout)
+        assert_parity(oracle, sfx, gi.toCpu(), oracle.matmul(g, W), "gradInput")
+        assert_parity(oracle, sfx, gw.toCpu(), oracle.matmul(g.T, x), "gradWeight")
+        assert_parity(oracle, sfx, gb.toCpu(), oracle.reduce_axis("sum", g, 0), "gradBias")
+        gi2, gw2 = hip.linear_backward(hip.toHip(x), hip.toHip(W), hip.toHip(g), with_bias=False)
+        assert np.array_equal(gi2.toCpu(), gi.toCpu()) and np.array_equal(gw2.toCpu(), gw.toCpu())
+
+
+def test_linear_backward_is_the_gradient_of_linear(hip):
+    """Central differences of L = sum(linear(x, W, b) *. G) through the device forward pass agree
+    with linear_backward (float64, so the difference quotient is good to ~1e-9)."""
+    rng = np.random.default_rng(5)
+    x, W, b, G = (rng.standard_normal(s) for s in ((5, 7), (4, 7), (1, 4), (5, 4)))
+    dG = hip.toHip(G)
+
+    def loss(x_, W_, b_):
+        return hip.sum(hip.bc_mul(hip.linear(hip.toHip(x_), hip.toHip(W_), hip.toHip(b_)), dG))
+
+    gi, gw, gb = (t.toCpu() for t in hip.linear_backward(hip.toHip(x), hip.toHip(W), dG))
+    h = 1e-5
+    for arr, grad, pos in ((x, gi, 0), (W, gw, 1), (b, gb, 2)):
+        num = np.zeros_like(arr)
+        for idx in np.ndindex(arr.shape):
+            args = [x.copy(), W.copy(), b.copy()]
+            args[pos][idx] += h
+            up = loss(*args)
+            args[pos][idx] -= 2 * h
+            num[idx] = (up - loss(*args)) / (2 * h)
+        assert np.allclose(num, grad, rtol=1e-7, atol=1e-8), pos
+
+
 def test_int_wrap_known_answers(hip):
     A = hip.toHip(np.array([[2**31 - 1, 1]], dtype=np.int32))
     B = hip.toHip(np.array([[2], [3]], dtype=np.int32))

@@ -146,7 +146,8 @@ def _make(rng, shape, dt, spec):
 
 @settings(max_examples=120, deadline=None)
 @given(strided_pair(), st.sampled_from(["f32", "f64", "i32", "i64"]),
-       st.sampled_from(["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min"]), st.integers(0, 2**31))
+       st.sampled_from(["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min", "sigmoid_bwd", "tanh_bwd"]),
+       st.integers(0, 2**31))
 def test_random_strides_match_numpy(oracle, spec, sfx, op, seed):
     shape, views = spec
     dt = DTYPES[sfx]
