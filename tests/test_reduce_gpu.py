@@ -136,6 +136,32 @@ def test_long_axes_are_chunked(hip, oracle, sfx):
             assert close(sfx, op, getattr(hip, op)(dx), oracle.reduce_all(op, x), oracle.reduce_all("sum", np.abs(x)))
 
 
+@pytest.mark.parametrize("sfx", ALL)
+def test_column_walks_with_16_byte_lanes(hip, oracle, sfx):
+    """Walks across a unit-stride dimension take 16 bytes of adjacent outputs per lane when extents,
+    strides and base addresses allow it, and one output per lane otherwise; both fold every output
+    front to back, so without chunking floats equal the serial fold bit for bit."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("colvec", sfx))
+    cases = [((4096, 2048), 0, True), ((70, 4100), 0, False), ((70, 4098), 0, False), ((120, 6, 512), 0, False),
+             ((300, 600, 8), 1, True), ((9, 2048, 4), 0, False)]
+    for shape, ax, chunked in cases:
+        lead = (slice(None),) * (len(shape) - 1)
+        for op in OPS:
+            x = fill(rng, shape, dt, op)
+            dx = hip.toHip(x)
+            for name, sl in (("whole", ()), ("every other slice", (slice(None, None, 2),)), ("columns from 4", lead + (slice(4, None),)),
+                             ("columns from 1", lead + (slice(1, None),)), ("columns reversed", lead + (slice(None, None, -1),))):
+                v, dv = x[sl], dx[sl] if sl else dx
+                say("column walk", sfx, shape, ax, name, op)
+                got = getattr(hip, op)(dv, ax).toCpu()
+                want = oracle.reduce_axis(op, v, ax)
+                if sfx in ("i32", "i64") or op in ("min", "max") or not chunked:
+                    assert np.array_equal(got, want), (shape, ax, name, op)
+                else:
+                    assert close(sfx, op, got, want, oracle.reduce_axis("sum", np.abs(v), ax)), (shape, ax, name, op)
+
+
 @pytest.mark.parametrize("sfx", ["f32", "i32"])
 def test_full_size_sum_8192(hip, oracle, sfx):
     """8192 x 8192: column sums, row sums and the total, against the oracle; and the total as the
