@@ -544,7 +544,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
 // Padded operand extents and the estimated time of the digit-sliced product for both tile shapes
 // (rounds of one workgroup per CU x measured time per tile and k, plus the two splitting passes).
 // The estimate is for operands that use every digit; the kernel itself skips empty planes.
-struct Plan { int64_t Mp, Np, Kp; bool big; double est_us, main_us, split_us; };
+// Estimated times of the digit path in microseconds: the two splitting passes, the product kernel with
+// every digit pair live (main_us, of which fixed_us do not depend on the number of pairs), and their sum.
+struct Plan { int64_t Mp, Np, Kp; bool big; double est_us, main_us, fixed_us, first_us, second_us; };
+
+// Time of the product kernel for `tiles` workgroup tiles, one per CU and round. A tile's time per k
+// grows with the share of the chip that is busy (the tiles compete for L2 and fabric bandwidth):
+// c0 * (1 + a * load^2), fitted to kernel times at 512^3 ... 4096^3 with all pairs live.
+static inline double main_us_per_k(int64_t tiles, int64_t cus, double c0, double a) {
+  const int64_t full = tiles / cus, rem = tiles - full * cus;
+  const double load = (double)rem / (double)cus;
+  return (double)full * c0 * (1.0 + a) + (rem ? c0 * (1.0 + a * load * load) : 0.0);
+}
+
 template <typename T>
 static inline Plan plan(const Args<T>& g) {
   constexpr bool WIDE = sizeof(T) == 8;
@@ -554,20 +566,25 @@ static inline Plan plan(const Args<T>& g) {
   pl.Kp = (g.K + kKPad - 1) / kKPad * kKPad;
   const int64_t cus = num_cus();
   const int64_t tb = (pl.Mp / 256) * (pl.Np / 256), ts = (pl.Mp / 256) * (pl.Np / 128);
-  // microseconds per k for one tile, measured at 4096^3. int32 (ten pairs): 0.162 (256 x 256), 0.098 (256 x 128);
-  // int64 (36 pairs, 256 x 128 only: the 64-bit accumulators leave no registers for the larger tile): 0.38.
-  const double cost_big = (double)((tb + cus - 1) / cus) * 0.162 * pl.Kp;
-  const double cost_small = (double)((ts + cus - 1) / cus) * (WIDE ? 0.38 : 0.098) * pl.Kp;
+  // microseconds per k of one tile on an otherwise idle chip (c0) and its growth to a full chip (a).
+  // int32 (ten pairs): 256 x 128 tiles 0.054 -> 0.089, 256 x 256 tiles 0.093 -> 0.157;
+  // int64 (36 pairs, 256 x 128 only: the 64-bit accumulators leave no registers for the larger tile): 0.205 -> 0.29.
+  const double cost_big = main_us_per_k(tb, cus, 0.093, 0.69) * pl.Kp;
+  const double cost_small = main_us_per_k(ts, cus, WIDE ? 0.205 : 0.054, WIDE ? 0.42 : 0.65) * pl.Kp;
   pl.big = !WIDE && cost_big <= cost_small;
   if (!WIDE) {
     const char* force = getenv("AM_HIP_GEMM_TILE_I8");   // 1: 256 x 256 tiles, 0: 256 x 128 (tests)
     if (force && *force) pl.big = atoi(force) != 0;
   }
-  // the splitting passes read sizeof(T) and write sizeof(T) bytes per element, at about 2.8 TB/s
-  const double split_us = 2 * 5.0 + 2.0 * sizeof(T) * (double)(pl.Mp + pl.Np) * pl.Kp / 2.8e6;
-  pl.main_us = pl.big ? cost_big : cost_small;
-  pl.split_us = split_us;
-  pl.est_us = pl.main_us + split_us;
+  // launch, pair table, the result's round trip (int64: one widening per pair on top)
+  pl.fixed_us = WIDE ? 15.0 : 5.0;
+  pl.main_us = pl.fixed_us + (pl.big ? cost_big : cost_small);
+  // The first pass reads every element and writes its lowest digit; the second reads it again (mostly
+  // from the memory-side cache) and writes the other planes.
+  const double elems = (double)(pl.Mp + pl.Np) * pl.Kp, sz = (double)sizeof(T);
+  pl.first_us = 4.5 + elems * (sz + 1.0) / (WIDE ? 5.5e6 : 6.2e6);
+  pl.second_us = 4.5 + elems * (2.0 * sz - 1.0) / 7.0e6;
+  pl.est_us = pl.main_us + pl.first_us + pl.second_us;
   return pl;
 }
 
@@ -634,7 +651,8 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
   const int64_t stiles = (Mp + Np) / 32 * (Kp / 128), smax = (int64_t)num_cus() * 16;
   const dim3 sgrid((unsigned)(stiles < smax ? stiles : smax));
   hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
-  hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
+  // with at most one live pair allowed there is nothing above plane 0 that could be needed
+  if (max_pairs >= 2) hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
   DigitArgs<T> d;
   d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.max_pairs = max_pairs; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
@@ -668,20 +686,24 @@ static int try_digits(Args<T>& g, double valu_est_us, int* rc) {
   const int may = applicable(g);
   if (!may) return 1;
   const Plan pl = plan(g);
-  if (may == 2 || (may == 1 && pl.est_us < 1.2 * valu_est_us)) {
-    if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path, %s tiles, est %.1f us (VALU est %.1f us)\n", pl.big ? "256x256" : "256x128", pl.est_us, valu_est_us);
+  // What the vector-ALU kernel takes in practice: its tile model leaves out launch and tail effects
+  // (fitted to the same sizes as the digit path's model).
+  const double valu_us = (sizeof(T) == 8 ? 1.15 : 1.3) * valu_est_us + 5.0;
+  if (may == 2 || (may == 1 && pl.est_us < 1.1 * valu_us)) {
+    if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path, %s tiles, est %.1f us (VALU est %.1f us)\n", pl.big ? "256x256" : "256x128", pl.est_us, valu_us);
     const int r = run(g, pl);
     if (r <= 0) { *rc = r; return 0; }
     return 1;   // no scratch memory for the digit planes
   }
-  // the first splitting pass and an early-leaving kernel or two cost about 10 us when the data says no
-  const double per_pair = pl.main_us / NPAIRS, fixed = pl.split_us * 0.6 + 10.0;
-  int max_pairs = (int)((0.8 * valu_est_us - fixed) / per_pair);
+  // When the data says no, the first splitting pass and two kernels that leave at once have been paid
+  // for nothing (about 10 us at small sizes): only worth risking on products that take a few times that.
+  const double per_pair = (pl.main_us - pl.fixed_us) / NPAIRS, fixed = pl.first_us + 4.5 + 3.0 + pl.fixed_us;   // + a second pass and a product kernel that leave at once
+  int max_pairs = (int)((0.85 * valu_us - fixed) / per_pair);
   if (const char* e = getenv("AM_HIP_GEMM_SPEC_PAIRS")) max_pairs = atoi(e);   // tests
   if (max_pairs > NPAIRS) max_pairs = NPAIRS;
-  if (may != 3 && (max_pairs < 1 || valu_est_us < 40.0)) return 1;
+  if (may != 3 && (max_pairs < 1 || valu_us < 32.0)) return 1;
   if (max_pairs < 0) max_pairs = 0;
-  if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path if at most %d digit pairs are live, else VALU (est %.1f us)\n", max_pairs, valu_est_us);
+  if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path if at most %d digit pairs are live, else VALU (est %.1f us)\n", max_pairs, valu_us);
   const uint32_t* flags = nullptr;
   uint32_t gen = 0;
   const int r = run(g, pl, max_pairs, &flags, &gen);
