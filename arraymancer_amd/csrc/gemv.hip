@@ -8,7 +8,8 @@
 //   gemv_rows  A has unit column stride: one wavefront per row, lanes stride along the row with
 //              16-byte loads of A and x, 64-lane shuffle reduction at the end.
 //   gemv_cols  A has unit row stride (a transposed view): a lane owns VEC consecutive rows and
-//              walks the columns with 16-byte loads (coalesced along m); x[j] is one scalar load.
+//              walks the columns with 16-byte loads (coalesced along m), UN of them in flight; x[j] is
+//              one scalar load.
 //              The column range is cut over gridDim.y so the chip fills for short, wide matrices;
 //              partial vectors go through the split-K workspace and the shared reduce kernel.
 // Anything else (both strides non-unit, tiny M) runs as an N = 1 GEMM, which handles all strides.
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(256) void gemv_rows(GemvArgs<T> p) {
 }
 
 // A column-contiguous (unit row stride), rows and column starts 16-byte aligned, M % VEC == 0.
-template <typename T>
+template <typename T, int UN>
 __global__ __launch_bounds__(256) void gemv_cols(GemvArgs<T> p) {
   typedef typename Acc<T>::type U;
   typedef typename VecTraits<T>::vec_t vec_t;
@@ -112,16 +113,16 @@ __global__ __launch_bounds__(256) void gemv_cols(GemvArgs<T> p) {
   for (int e = 0; e < VEC; ++e) acc[e] = 0;
   const T* __restrict__ a = p.A + m;
   int64_t j = j0;
-  for (; j + 4 <= j1; j += 4) {
-    vec_t v[4];
-    U xs[4];
+  for (; j + UN <= j1; j += UN) {
+    vec_t v[UN];
+    U xs[UN];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UN; ++u) {
       v[u] = __builtin_nontemporal_load((const vec_t*)(a + (j + u) * p.csA));
       xs[u] = (U)p.x[(j + u) * p.incx];
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < UN; ++u)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) acc[e] += (U)v[u][e] * xs[u];
   }
@@ -193,7 +194,8 @@ int gemv(const char* fn, int64_t M, int64_t N, T alpha, const T* A, int64_t rsA,
   }
   if (rsA == 1 && M % VEC == 0 && csA % VEC == 0 && csA >= 0 && aligned16(A) && M >= 256) {
     const int64_t blocks_m = (M / VEC + 255) / 256;
-    int64_t splits = ((int64_t)num_cus() * 2 + blocks_m - 1) / blocks_m;
+    // one workgroup per CU: fewer, longer column walks (and fewer partial vectors) measured fastest
+    int64_t splits = ((int64_t)num_cus() + blocks_m - 1) / blocks_m;
     if (splits > N / 32) splits = N / 32;
     if (splits > 64) splits = 64;
     if (splits >= 2) {
@@ -202,7 +204,7 @@ int gemv(const char* fn, int64_t M, int64_t N, T alpha, const T* A, int64_t rsA,
       T* ws = (T*)splitk_workspace((size_t)splits * M * sizeof(T));
       if (ws && splits >= 2) { g.ws = ws; g.splits = (int)splits; g.n_chunk = chunk; }
     }
-    hipLaunchKernelGGL((gemv_cols<T>), dim3((unsigned)blocks_m, (unsigned)g.splits), dim3(256), 0, stream(), g);
+    hipLaunchKernelGGL((gemv_cols<T, 8>), dim3((unsigned)blocks_m, (unsigned)g.splits), dim3(256), 0, stream(), g);
     AM_TRY(check_launch("gemv_cols"));
     if (g.splits > 1) {
       Args<T> r;
