@@ -443,7 +443,8 @@ __global__ __launch_bounds__(256) void softmax_rows(SoftmaxArgs<T> p) {
   }
   if (!active) return;
   T* dst = p.dst + row * p.d_rs;
-  for (int64_t c = me; c < p.cols; c += W) dst[c * p.d_cs] = dev_exp<T>(src[c * p.s_cs] - mx) / sum;   // stable_softmax
+  const T inv = (T)1 / sum;
+  for (int64_t c = me; c < p.cols; c += W) dst[c * p.d_cs] = dev_exp<T>(src[c * p.s_cs] - mx) * inv;   // stable_softmax
 }
 
 // Contiguous rows that fit in registers: each lane keeps NV 16-byte vectors of its row, so the
@@ -501,13 +502,14 @@ __global__ __launch_bounds__(256) void softmax_rows_reg(SoftmaxArgs<T> p) {
   }
   if (!active) return;
   vec_t* dst = (vec_t*)(p.dst + row * p.d_rs);
+  const T inv = (T)1 / sum;   // one division per row; every element is then within 1.5 ulp of exp / sum
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int64_t v = (int64_t)i * W + me;
     if (v < nvec) {
       vec_t y;
 #pragma unroll
-      for (int e = 0; e < V; ++e) y[e] = x[i][e] / sum;
+      for (int e = 0; e < V; ++e) y[e] = x[i][e] * inv;
       __builtin_nontemporal_store(y, dst + v);
     }
   }
@@ -519,7 +521,8 @@ static void launch_softmax_reg(const SoftmaxArgs<T>& p, int nv, dim3 grid) {
     case 1: hipLaunchKernelGGL((softmax_rows_reg<T, W, 1>), grid, dim3(256), 0, stream(), p); break;
     case 2: hipLaunchKernelGGL((softmax_rows_reg<T, W, 2>), grid, dim3(256), 0, stream(), p); break;
     case 4: hipLaunchKernelGGL((softmax_rows_reg<T, W, 4>), grid, dim3(256), 0, stream(), p); break;
-    default: hipLaunchKernelGGL((softmax_rows_reg<T, W, 8>), grid, dim3(256), 0, stream(), p); break;
+    case 8: hipLaunchKernelGGL((softmax_rows_reg<T, W, 8>), grid, dim3(256), 0, stream(), p); break;
+    default: hipLaunchKernelGGL((softmax_rows_reg<T, W, 16>), grid, dim3(256), 0, stream(), p); break;
   }
 }
 
@@ -540,7 +543,7 @@ static int softmax(const char* fn, int64_t rows, int64_t cols, T* dst, int64_t d
     int nv = 1;
     while (64 * nv < nvec) nv *= 2;
     launch_softmax_reg<T, 64>(p, nv, dim3((unsigned)((rows + 3) / 4)));
-  } else if (vec && nvec <= 256 * 8) {  // a workgroup per row
+  } else if (vec && nvec <= 256 * 16) {  // a workgroup per row (up to 64 registers of row per lane)
     int nv = 1;
     while (256 * nv < nvec) nv *= 2;
     launch_softmax_reg<T, 256>(p, nv, dim3((unsigned)rows));

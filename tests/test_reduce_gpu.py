@@ -206,7 +206,8 @@ def test_softmax_vs_oracle(hip, oracle, sfx):
     dt = DTYPES[sfx]
     tol = 2e-6 if sfx == "f32" else 1e-14
     rng = np.random.default_rng(seed_of("softmax-gpu", sfx))
-    for shape in [(1, 1), (3, 5), (64, 10), (256, 1000), (7, 4096), (5, 4097), (3, 50_000), (1000, 3)]:
+    for shape in [(1, 1), (3, 5), (64, 10), (256, 1000), (7, 4096), (5, 4097), (3, 8192), (4, 12288), (3, 16384), (3, 50_000),
+                  (1000, 3)]:
         x = (rng.standard_normal(shape) * 4).astype(dt)
         say("softmax", sfx, shape)
         want = oracle.softmax(x)
