@@ -43,6 +43,8 @@ template <> struct Traits<int64_t> {
 
 __device__ __forceinline__ float dev_exp(float x) { return expf(x); }
 __device__ __forceinline__ double dev_exp(double x) { return exp(x); }
+__device__ __forceinline__ float dev_sqrt(float x) { return sqrtf(x); }
+__device__ __forceinline__ double dev_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float dev_tanh(float x) { return tanhf(x); }
 __device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
 
@@ -80,9 +82,12 @@ template <typename T, int OP> struct BinOp {
     } else if constexpr (OP == AM_OP_SIGMOID_BWD) {
       if constexpr (Traits<T>::kFloat) return x * ((T)1 - x) * y;
       else return (T)((U)x * ((U)1 - (U)x) * (U)y);
-    } else {  // AM_OP_TANH_BWD
+    } else if constexpr (OP == AM_OP_TANH_BWD) {
       if constexpr (Traits<T>::kFloat) return y * ((T)1 - x * x);
       else return (T)((U)y * ((U)1 - (U)x * (U)x));
+    } else {  // AM_OP_SQDIFF
+      if constexpr (Traits<T>::kFloat) { const T d = x - y; return d * d; }
+      else { const U d = (U)x - (U)y; return (T)(d * d); }
     }
   }
 };
@@ -99,6 +104,11 @@ template <typename T, int UOP> struct UnOp {
     else if constexpr (UOP == AM_UOP_SIGMOID) return (T)1 / ((T)1 + dev_exp(-x));
     else if constexpr (UOP == AM_UOP_TANH) return dev_tanh(x);
     else if constexpr (UOP == AM_UOP_EXP) return dev_exp(x);
+    else if constexpr (UOP == AM_UOP_SQRT) {
+      if constexpr (Traits<T>::kFloat) return dev_sqrt(x); else return x;   // never dispatched for integers
+    } else if constexpr (UOP == AM_UOP_SQUARE) {
+      if constexpr (Traits<T>::kFloat) return x * x; else return (T)((U)x * (U)x);
+    }
     else {  // ABS
       if constexpr (Traits<T>::kFloat) return __builtin_fabs(x);
       else return (x < 0) ? (T)((U)0 - (U)x) : x;
@@ -551,7 +561,7 @@ static int binary(const char* fn, int op, int rank, const int64_t* shape, T* dst
 #define AM_CASE(code) case code: return run<T, code, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0)
     AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
     AM_CASE(AM_OP_ADD_RELU); AM_CASE(AM_OP_RELU_BWD); AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN);
-    AM_CASE(AM_OP_SIGMOID_BWD); AM_CASE(AM_OP_TANH_BWD);
+    AM_CASE(AM_OP_SIGMOID_BWD); AM_CASE(AM_OP_TANH_BWD); AM_CASE(AM_OP_SQDIFF);
 #undef AM_CASE
     case AM_OP_MOD:
       if constexpr (!F) return run<T, AM_OP_MOD, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
@@ -599,7 +609,7 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
   constexpr bool F = Traits<T>::kFloat;
   switch (op) {
 #define AM_CASE(code) case code: return run<T, kUnaryBase + code, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0)
-    AM_CASE(AM_UOP_COPY); AM_CASE(AM_UOP_NEG); AM_CASE(AM_UOP_RELU); AM_CASE(AM_UOP_ABS);
+    AM_CASE(AM_UOP_COPY); AM_CASE(AM_UOP_NEG); AM_CASE(AM_UOP_RELU); AM_CASE(AM_UOP_ABS); AM_CASE(AM_UOP_SQUARE);
 #undef AM_CASE
     case AM_UOP_SIGMOID:
       if constexpr (F) return run<T, kUnaryBase + AM_UOP_SIGMOID, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
@@ -610,6 +620,9 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
     case AM_UOP_EXP:
       if constexpr (F) return run<T, kUnaryBase + AM_UOP_EXP, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
       else return fail(AM_E_DTYPE, "%s: exp is defined for float tensors only", fn);
+    case AM_UOP_SQRT:
+      if constexpr (F) return run<T, kUnaryBase + AM_UOP_SQRT, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
+      else return fail(AM_E_DTYPE, "%s: sqrt is defined for float tensors only", fn);
     default:
       return fail(AM_E_ARG, "%s: unknown unary op %d", fn, op);
   }

@@ -717,6 +717,47 @@ def mean(t: HipTensor, axis: int | None = None):
     return scalar_op("div", reduce_axis("sum", t, axis), t.dtype.type(t.shape[axis]))
 
 
+def variance(t: HipTensor, axis: int | None = None):
+    """Sample variance, normalised by n - 1 (src/arraymancer/tensor/aggregate.nim:115-146): the mean,
+    then the sum of square(y - mean) (one fused map, one fold), divided by n - 1. Floats only."""
+    if t.dtype.kind != "f":
+        raise TypeError("variance is defined for float tensors")
+    if axis is None:
+        m = mean(t)
+        sq = empty(t.shape, t.dtype)
+        _scalar_sqdiff(sq, t, m)
+        return t.dtype.type(reduce_all("sum", sq) / t.dtype.type(t.size - 1))
+    if t.size == 0:
+        return empty(t.shape, t.dtype)
+    m = mean(t, axis)
+    sq = map2("sqdiff", t, m.broadcast(t.shape))
+    return scalar_op("div", reduce_axis("sum", sq, axis), t.dtype.type(t.shape[axis] - 1))
+
+
+def _scalar_sqdiff(dst: HipTensor, t: HipTensor, m):
+    """dst = square(t - m) for a host scalar m: a subtraction pass, then the square in place."""
+    _scalar_into("sub", dst, t, m, False)
+    _unary_into("square", dst, dst)
+
+
+def std(t: HipTensor, axis: int | None = None):
+    """sqrt of the variance (aggregate.nim:148-158)."""
+    v = variance(t, axis)
+    if axis is None:
+        return t.dtype.type(np.sqrt(v))
+    return unary("sqrt", v) if v.size else v
+
+
+def sqrt(t: HipTensor) -> HipTensor:
+    """src/arraymancer/tensor/ufunc.nim:91."""
+    return unary("sqrt", t)
+
+
+def square(t: HipTensor) -> HipTensor:
+    """src/arraymancer/tensor/math_functions.nim:218-222."""
+    return unary("square", t)
+
+
 def softmax(t: HipTensor) -> HipTensor:
     """Row softmax of a [batch_size, number_of_classes] matrix
     (src/arraymancer/nn_primitives/nnp_softmax.nim:18-38)."""

@@ -248,7 +248,8 @@ int am_hip_dot_i64(int64_t n, const int64_t* x, int64_t incx, const int64_t* y, 
 #define AM_OP_MIN        10
 #define AM_OP_SIGMOID_BWD 11  /* a * (1 - a) * b   a = cached sigmoid output (nnp_activation.nim:61-63)  */
 #define AM_OP_TANH_BWD   12   /* b * (1 - a * a)   a = cached tanh output    (nnp_activation.nim:72-74)  */
-#define AM_OP_BINARY_COUNT 13
+#define AM_OP_SQDIFF     13   /* (a - b) * (a - b): the fold body of variance (tensor/aggregate.nim:115-146) */
+#define AM_OP_BINARY_COUNT 14
 
 int am_hip_ew_binary_f32(int op, int rank, const int64_t* shape,
                          float* dst, const int64_t* dst_strides,
@@ -296,7 +297,9 @@ int am_hip_ew_scalar_i64(int op, int scalar_on_left, int rank, const int64_t* sh
 #define AM_UOP_TANH    4   /* floats only      */
 #define AM_UOP_EXP     5   /* floats only      */
 #define AM_UOP_ABS     6
-#define AM_UOP_COUNT   7
+#define AM_UOP_SQRT    7   /* floats only: IEEE square root (tensor/ufunc.nim:91)        */
+#define AM_UOP_SQUARE  8   /* x * x (tensor/math_functions.nim:218-222); integers wrap   */
+#define AM_UOP_COUNT   9
 int am_hip_ew_unary_f32(int op, int rank, const int64_t* shape,
                         float* dst, const int64_t* dst_strides,
                         const float* a, const int64_t* a_strides);

@@ -454,6 +454,26 @@ template <typename T> HipTensor<T> mean(const HipTensor<T>& t, int axis) {
   return scalar_op(AM_OP_DIV, s, static_cast<T>(t.shape[axis]));
 }
 
+template <typename T> HipTensor<T> sqrt(const HipTensor<T>& t) { return unary(AM_UOP_SQRT, t); }      // ufunc.nim:91
+template <typename T> HipTensor<T> square(const HipTensor<T>& t) { return unary(AM_UOP_SQUARE, t); }  // math_functions.nim:218-222
+// Sample variance, normalised by n - 1, and its square root (aggregate.nim:115-158): the mean, then the
+// sum of square(y - mean).
+template <typename T> T variance(const HipTensor<T>& t) {
+  static_assert(std::is_floating_point<T>::value, "variance is defined for float tensors");
+  return sum(square(scalar_op(AM_OP_SUB, t, mean(t)))) / static_cast<T>(t.size() - 1);
+}
+template <typename T> HipTensor<T> variance(const HipTensor<T>& t, int axis) {
+  static_assert(std::is_floating_point<T>::value, "variance is defined for float tensors");
+  HipTensor<T> m = mean(t, axis);
+  if (m.size() == 0) return m;
+  return scalar_op(AM_OP_DIV, sum(map2(AM_OP_SQDIFF, t, m.broadcast(t.shape)), axis), static_cast<T>(t.shape[axis] - 1));
+}
+template <typename T> T stddev(const HipTensor<T>& t) { return std::sqrt(variance(t)); }
+template <typename T> HipTensor<T> stddev(const HipTensor<T>& t, int axis) {
+  HipTensor<T> v = variance(t, axis);
+  return v.size() == 0 ? v : sqrt(v);
+}
+
 // Row softmax of a [batch_size, number_of_classes] matrix (nnp_softmax.nim:18-38).
 template <typename T>
 HipTensor<T> softmax(const HipTensor<T>& t) {

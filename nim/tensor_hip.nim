@@ -21,6 +21,7 @@ import arraymancer/tensor/shapeshifting             # asContiguous (host side, u
 import arraymancer/io/io_npy                        # read_npy / write_npy on host tensors
 import arraymancer/tensor/private/p_display         # prettyImpl
 import std/typetraits                               # type names for `pretty`
+import std/math                                     # scalar sqrt for `std`
 
 type
   HipScalar* = float32 | float64 | int32 | int64
@@ -394,6 +395,28 @@ proc mean*[T: int32 | int64](t: HipTensor[T]): T = t.sum div T(t.size)
 proc mean*[T: float32 | float64](t: HipTensor[T]): T = t.sum / T(t.size)
 proc mean*[T: int32 | int64](t: HipTensor[T], axis: int): HipTensor[T] = t.sum(axis) / T(t.shape[axis])   # opDiv truncates like `div` on integers
 proc mean*[T: float32 | float64](t: HipTensor[T], axis: int): HipTensor[T] = t.sum(axis) / T(t.shape[axis])
+
+proc sqrt*[T: float32 | float64](t: HipTensor[T]): HipTensor[T] =
+  ## ufunc.nim:91
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewUnary(T, uopSqrt, result, t)
+proc square*[T: HipScalar](t: HipTensor[T]): HipTensor[T] =
+  ## math_functions.nim:218-222
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewUnary(T, uopSquare, result, t)
+
+proc variance*[T: float32 | float64](t: HipTensor[T]): T =
+  ## aggregate.nim:115-129: the mean, then the sum of square(y - mean), over n - 1
+  square(t -. t.mean).sum / T(t.size - 1)
+proc variance*[T: float32 | float64](t: HipTensor[T], axis: int): HipTensor[T] =
+  ## aggregate.nim:131-146
+  if t.size == 0: return t
+  let m = t.mean(axis)
+  map2(t, opSqDiff, m.broadcast(t.shape.toSeq)).sum(axis) / T(t.shape[axis] - 1)
+proc std*[T: float32 | float64](t: HipTensor[T]): T = math.sqrt(t.variance)                        ## aggregate.nim:148-151
+proc std*[T: float32 | float64](t: HipTensor[T], axis: int): HipTensor[T] =                   ## aggregate.nim:153-158
+  if t.size == 0: return t
+  sqrt(t.variance(axis))
 
 proc softmax*[T: float32 | float64](input: HipTensor[T]): HipTensor[T] =
   ## nn_primitives/nnp_softmax.nim:18-38 on a [batch_size, number_of_classes] matrix.

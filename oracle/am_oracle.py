@@ -27,9 +27,9 @@ _CT = {"f32": ctypes.c_float, "f64": ctypes.c_double, "i32": ctypes.c_int32, "i6
 
 # op codes of include/am_hip.h
 OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
-          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12)
+          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12, sqdiff=13)
 OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2, addmul=3)
-UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6)
+UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6, sqrt=7, square=8)
 
 
 def build(force: bool = False) -> str:
@@ -311,6 +311,23 @@ def mean(a: np.ndarray, axis: int | None = None):
     return q if axis is not None else q.dtype.type(q)
 
 
+def variance(a: np.ndarray, axis: int | None = None):
+    """aggregate.nim:115-146: mean, then the serial fold of square(y - mean) in the tensor's own
+    precision, divided by n - 1."""
+    m = mean(a, axis)
+    d = a - m                      # m broadcasts: it keeps the reduced axis with extent 1
+    sq = (d * d).astype(a.dtype)
+    if axis is None:
+        return a.dtype.type(reduce_all("sum", sq) / a.dtype.type(a.size - 1))
+    return (reduce_axis("sum", sq, axis) / a.dtype.type(a.shape[axis] - 1)).astype(a.dtype)
+
+
+def std(a: np.ndarray, axis: int | None = None):
+    """aggregate.nim:148-158."""
+    v = variance(a, axis)
+    return np.sqrt(v).astype(a.dtype) if axis is not None else a.dtype.type(np.sqrt(v))
+
+
 def softmax(x: np.ndarray) -> np.ndarray:
     """nnp_softmax.nim:18-38 on a [batch, classes] matrix (streaming max / sum of exponentials per
     row, then exp(x - max) / sumexp)."""
@@ -428,6 +445,8 @@ def closed_map2(op, a, b):
             return a * (1 - a) * b
         if name == "tanh_bwd":
             return b * (1 - a * a)
+        if name == "sqdiff":
+            return (a - b) * (a - b)
     raise KeyError(name)
 
 

@@ -81,6 +81,7 @@ static inline void iter_advance(strided_iter* it) {
 #define IS_FLOAT 1
 #define F_EXP expf
 #define F_TANH tanhf
+#define F_SQRT sqrtf
 #include "strided_map_impl.inc"
 #undef T
 #undef UT
@@ -88,6 +89,7 @@ static inline void iter_advance(strided_iter* it) {
 #undef IS_FLOAT
 #undef F_EXP
 #undef F_TANH
+#undef F_SQRT
 
 #define T double
 #define UT double
@@ -95,6 +97,7 @@ static inline void iter_advance(strided_iter* it) {
 #define IS_FLOAT 1
 #define F_EXP exp
 #define F_TANH tanh
+#define F_SQRT sqrt
 #include "strided_map_impl.inc"
 #undef T
 #undef UT
@@ -102,6 +105,7 @@ static inline void iter_advance(strided_iter* it) {
 #undef IS_FLOAT
 #undef F_EXP
 #undef F_TANH
+#undef F_SQRT
 
 #define T int32_t
 #define UT uint32_t

@@ -138,6 +138,21 @@ static void broadcasting() {
   CHECK(eq(toHip<T>({1, 2}, {2, 1}).broadcast({2, 2}), {1, 1, 2, 2}));
 }
 
+static void variance_std() {
+  // tests/tensor/test_aggregate.nim:88-110
+  auto a = toHip<double>({-3, -2, -1, 0, 1, 2, 3}, {7});
+  CHECK(std::fabs(am::variance(a) - 4.6666666666667) < 1e-8);
+  CHECK(std::fabs(am::stddev(a) - 2.1602468994693) < 1e-8);
+  auto b = toHip<double>({1, 2, 3, -4, 0, 4, -2, 5}, {2, 4});
+  CHECK(eq(am::variance(b, 0), {0.5, 2.0, 12.5, 40.5}));
+  auto v1 = am::variance(b, 1).toCpu();
+  CHECK(v1.size() == 2 && std::fabs(v1[0] - 9.666666666666666) + std::fabs(v1[1] - 10.91666666666667) < 1e-8);
+  auto s0 = am::stddev(b, 0).toCpu();
+  CHECK(std::fabs(s0[0] - 0.7071067811865476) + std::fabs(s0[3] - 6.363961030678928) < 1e-8);
+  CHECK(eq(am::sqrt(toHip<float>({4, 9, 0.25f}, {3})), {2, 3, 0.5f}));
+  CHECK(eq(am::square(toHip<int32_t>({-3, 65536, 7}, {3})), {9, 0, 49}));
+}
+
 static void fused_linear() {
   // nnp_linear.nim:28-29 + relu on small exact values
   auto x = toHip<float>({1, 2, 3, -1, -2, -3}, {2, 3});
@@ -250,6 +265,7 @@ int main(int argc, char** argv) {
     broadcasting<int32_t>();
     broadcasting<int64_t>();
     fused_linear();
+    variance_std();
     aggregates<float>();
     aggregates<double>();
     aggregates<int32_t>();

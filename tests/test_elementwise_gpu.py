@@ -107,7 +107,7 @@ def test_reference_map2_bool(hip, vectors):
 
 # ------------------------------------------------------------------ oracle / NumPy parity
 SHAPES = [(1,), (3,), (1000,), (4099,), (7, 13), (64, 4096), (33, 4100), (5, 6, 7), (2, 3, 4, 5, 6, 2), (300, 1), (1, 300)]
-BIN_OPS = ["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min", "sigmoid_bwd", "tanh_bwd"]
+BIN_OPS = ["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min", "sigmoid_bwd", "tanh_bwd", "sqdiff"]
 
 
 @pytest.mark.parametrize("sfx", ALL)
@@ -192,10 +192,12 @@ def test_scalar_and_unary(hip, oracle, sfx):
             say("scalar", sfx, op, left)
             got = hip.scalar_op(op, da, 3, scalar_on_left=left).toCpu()
             assert np.array_equal(got, oracle.scalar_op(op, a, 3, scalar_on_left=left)), (op, left)
-    for op in ["copy", "neg", "relu", "abs"]:
+    for op in ["copy", "neg", "relu", "abs", "square"] + (["sqrt"] if sfx in FLT else []):
         say("unary", sfx, op)
-        assert np.array_equal(hip.unary(op, da).toCpu(), oracle.unary(op, a)), op
-        assert np.array_equal(hip.unary(op, da.transpose()).toCpu(), oracle.unary(op, a.T)), op
+        nan_ok = op == "sqrt"   # negative entries
+        with np.errstate(invalid="ignore"):
+            assert np.array_equal(hip.unary(op, da).toCpu(), oracle.unary(op, a), equal_nan=nan_ok), op
+            assert np.array_equal(hip.unary(op, da.transpose()).toCpu(), oracle.unary(op, a.T), equal_nan=nan_ok), op
     assert np.array_equal((da * 2).toCpu(), a * dt(2))
     assert np.array_equal((2 * da).toCpu(), a * dt(2))
     assert np.array_equal((-da).toCpu(), -a)
@@ -220,6 +222,21 @@ def test_transcendental_bodies(hip, oracle, sfx):
         np.testing.assert_allclose(hip.map2(op, la, lb).toCpu(), oracle.map2(op, ba, bb), rtol=rtol, atol=rtol)
     for op in ("sigmoid", "tanh", "exp"):
         np.testing.assert_allclose(hip.unary(op, da).toCpu(), oracle.unary(op, a), rtol=rtol, atol=rtol)
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_sqrt_is_correctly_rounded(hip, sfx):
+    """IEEE square root: the same bits as NumPy's, NaN for negative input, signed zeros kept."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "sqrt"))
+    x = np.concatenate([rng.uniform(0, 1e6, 4093), 10.0 ** rng.uniform(-40, 38, 2000), [0.0, -0.0, np.inf, 1.0, 4.0, 2.0]]).astype(dt)
+    got = hip.sqrt(hip.toHip(x)).toCpu()
+    assert np.array_equal(got, np.sqrt(x))
+    assert np.signbit(got[-5]) and got[-5] == 0
+    with np.errstate(invalid="ignore"):
+        assert np.isnan(hip.sqrt(hip.toHip(np.array([-1.0, np.nan], dtype=dt))).toCpu()).all()
+    with pytest.raises(TypeError):
+        hip.sqrt(hip.zeros((4,), np.int32))
 
 
 def test_relu_special_values(hip):

@@ -146,7 +146,7 @@ def _make(rng, shape, dt, spec):
 
 @settings(max_examples=120, deadline=None)
 @given(strided_pair(), st.sampled_from(["f32", "f64", "i32", "i64"]),
-       st.sampled_from(["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min", "sigmoid_bwd", "tanh_bwd"]),
+       st.sampled_from(["add", "sub", "mul", "div", "add_relu", "relu_bwd", "max", "min", "sigmoid_bwd", "tanh_bwd", "sqdiff"]),
        st.integers(0, 2**31))
 def test_random_strides_match_numpy(oracle, spec, sfx, op, seed):
     shape, views = spec
@@ -179,6 +179,22 @@ def test_transcendental_bodies_close_to_numpy(oracle):
         b = rng.uniform(-3, 3, (33, 17)).astype(dt)
         np.testing.assert_allclose(oracle.map2("add_sigmoid", a, b), 1 / (1 + np.exp(-(a + b).astype(np.float64))), rtol=tol)
         np.testing.assert_allclose(oracle.map2("add_tanh", a, b), np.tanh((a + b).astype(np.float64)), rtol=tol, atol=tol)
+
+
+def test_sqrt_and_square_bodies(oracle):
+    """sqrt is one correctly rounded IEEE operation, square one multiplication (wrapping for
+    integers): NumPy computes the same bits."""
+    rng = np.random.default_rng(4)
+    for dt in (np.float32, np.float64):
+        x = rng.uniform(0, 1e6, (33, 17)).astype(dt)
+        assert np.array_equal(oracle.unary("sqrt", x), np.sqrt(x))
+        assert np.array_equal(oracle.unary("square", x.T), (x * x).T)
+    for dt in (np.int32, np.int64):
+        info = np.iinfo(dt)
+        x = rng.integers(info.min, info.max, (9, 31), endpoint=True).astype(dt)
+        assert np.array_equal(oracle.unary("square", x), x * x)
+        with pytest.raises(ValueError):
+            oracle.unary("sqrt", x)
 
 
 def test_broadcast_errors(oracle):

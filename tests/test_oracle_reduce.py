@@ -34,6 +34,34 @@ def test_reference_aggregate_vectors(vectors, oracle, sfx):
         assert np.array_equal(oracle.mean(t, 1), np.array(g["mean_axis1"], dtype=dt))
 
 
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_reference_variance_std_vectors(vectors, oracle, sfx):
+    """tests/tensor/test_aggregate.nim:88-110 (its bar is 1e-8 in float64)."""
+    g = vectors["aggregate_float"]
+    dt = DTYPES[sfx]
+    tol = 1e-8 if sfx == "f64" else 2e-6
+    a, b = np.array(g["a"], dtype=dt), np.array(g["b"], dtype=dt)
+    assert abs(oracle.variance(a) - g["variance_a"]) < tol * 5
+    assert abs(oracle.std(a) - g["std_a"]) < tol * 5
+    for ax in (0, 1):
+        assert np.abs(oracle.variance(b, ax) - np.array(g[f"variance_b_axis{ax}"])).sum() < tol * 50
+        assert np.abs(oracle.std(b, ax) - np.array(g[f"std_b_axis{ax}"])).sum() < tol * 10
+    assert np.array_equal(oracle.variance(b.astype(dt), 0), np.array(g["variance_b_axis0"], dtype=dt))   # exact in the reference's test
+
+
+def test_variance_against_float64_closed_form(oracle):
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((37, 53)).astype(np.float32) * 3 + 1
+    assert abs(oracle.variance(x) - np.var(x.astype(np.float64), ddof=1)) < 1e-4
+    for ax in (0, 1):
+        want = np.var(x.astype(np.float64), axis=ax, ddof=1, keepdims=True)
+        got = oracle.variance(x, ax)
+        assert got.shape == want.shape and np.allclose(got, want, rtol=1e-5)
+        assert np.allclose(oracle.std(x, ax), np.sqrt(want), rtol=1e-5)
+    x64 = x.astype(np.float64)
+    assert np.allclose(oracle.variance(x64.T, 0), np.var(x64.T, axis=0, ddof=1, keepdims=True), rtol=1e-12)
+
+
 def test_reference_maxpool_vectors(vectors, oracle):
     g = vectors["maxpool"]
     for dt in DTYPES.values():

@@ -136,6 +136,38 @@ def test_long_axes_are_chunked(hip, oracle, sfx):
             assert close(sfx, op, getattr(hip, op)(dx), oracle.reduce_all(op, x), oracle.reduce_all("sum", np.abs(x)))
 
 
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_variance_and_std(hip, oracle, vectors, sfx):
+    """variance / std (aggregate.nim:115-158): the reference's own literals, then the oracle on
+    larger tensors and views, along every axis and over all elements."""
+    dt = DTYPES[sfx]
+    g = vectors["aggregate_float"]
+    tol = 1e-8 if sfx == "f64" else 2e-6
+    a, b = hip.toHip(np.array(g["a"], dtype=dt)), hip.toHip(np.array(g["b"], dtype=dt))
+    assert abs(hip.variance(a) - g["variance_a"]) < tol * 5 and abs(hip.std(a) - g["std_a"]) < tol * 5
+    assert np.array_equal(hip.variance(b, 0).toCpu(), np.array(g["variance_b_axis0"], dtype=dt))
+    for ax in (0, 1):
+        assert np.abs(hip.variance(b, ax).toCpu() - np.array(g[f"variance_b_axis{ax}"])).sum() < tol * 50
+        assert np.abs(hip.std(b, ax).toCpu() - np.array(g[f"std_b_axis{ax}"])).sum() < tol * 10
+    rng = np.random.default_rng(seed_of("variance", sfx))
+    rtol = 2e-5 if sfx == "f32" else 1e-12
+    for shape in [(300, 70), (5, 2048), (4100, 3), (6, 50, 7)]:
+        x = (rng.standard_normal(shape) * 3 + 1).astype(dt)
+        dx = hip.toHip(x)
+        say("variance", sfx, shape)
+        assert np.isclose(hip.variance(dx), oracle.variance(x), rtol=rtol)
+        assert np.isclose(hip.std(dx), oracle.std(x), rtol=rtol)
+        for ax in range(len(shape)):
+            got = hip.variance(dx, ax).toCpu()
+            assert got.shape == oracle.variance(x, ax).shape
+            assert np.allclose(got, oracle.variance(x, ax), rtol=rtol)
+            assert np.allclose(hip.std(dx, ax).toCpu(), oracle.std(x, ax), rtol=rtol)
+        if len(shape) == 2:
+            assert np.allclose(hip.variance(dx.transpose(), 0).toCpu(), oracle.variance(x.T, 0), rtol=rtol)
+    with pytest.raises(TypeError):
+        hip.variance(hip.zeros((3, 3), np.int32))
+
+
 @pytest.mark.parametrize("sfx", ALL)
 def test_column_walks_with_16_byte_lanes(hip, oracle, sfx):
     """Walks across a unit-stride dimension take 16 bytes of adjacent outputs per lane when extents,
