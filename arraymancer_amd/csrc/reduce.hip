@@ -398,6 +398,138 @@ static int reduce_all(const char* fn, int op, int rank, const int64_t* shape, co
 }
 
 // ------------------------------------------------------------------------------------------------
+// Index and value of the first maximum (or minimum) along an axis: argmax_max / argmin_min of the
+// reference (src/arraymancer/tensor/aggregate.nim:159-193, 216-250). It starts from slice 0 and
+// replaces the running value only on a strict `>` (`<`), so ties keep the lowest index, a NaN in
+// slice 0 stays (nothing compares greater than it) and a NaN elsewhere is never taken.
+template <typename T> struct ArgArgs {
+  const T* a; T* val; int64_t* idx;
+  int ndim;
+  int64_t extent[kMaxDims], a_stride[kMaxDims], v_stride[kMaxDims], i_stride[kMaxDims];
+  int64_t outputs, L, a_axis_stride;
+};
+
+template <typename T>
+__device__ __forceinline__ void decode3(const ArgArgs<T>& p, int64_t o, int64_t& a_off, int64_t& v_off, int64_t& i_off) {
+  a_off = 0; v_off = 0; i_off = 0;
+#pragma unroll
+  for (int d = kMaxDims - 1; d >= 0; --d) {
+    if (d < p.ndim) {
+      const int64_t q = o / p.extent[d], r = o - q * p.extent[d];
+      a_off += r * p.a_stride[d];
+      v_off += r * p.v_stride[d];
+      i_off += r * p.i_stride[d];
+      o = q;
+    }
+  }
+}
+
+template <typename T, bool MAXOP> __device__ __forceinline__ bool beats(T x, T cur) { return MAXOP ? (x > cur) : (x < cur); }
+
+// One lane per output element walks the axis front to back.
+template <typename T, bool MAXOP>
+__global__ __launch_bounds__(256) void argreduce_seq(ArgArgs<T> p) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= p.outputs) return;
+  int64_t a_off, v_off, i_off;
+  decode3(p, o, a_off, v_off, i_off);
+  const T* src = p.a + a_off;
+  T best = src[0];
+  int64_t at = 0;
+  int64_t l = 1;
+  for (; l + 4 <= p.L; l += 4) {   // four loads in flight, compared in axis order
+    const T v0 = src[l * p.a_axis_stride], v1 = src[(l + 1) * p.a_axis_stride];
+    const T v2 = src[(l + 2) * p.a_axis_stride], v3 = src[(l + 3) * p.a_axis_stride];
+    if (beats<T, MAXOP>(v0, best)) { best = v0; at = l; }
+    if (beats<T, MAXOP>(v1, best)) { best = v1; at = l + 1; }
+    if (beats<T, MAXOP>(v2, best)) { best = v2; at = l + 2; }
+    if (beats<T, MAXOP>(v3, best)) { best = v3; at = l + 3; }
+  }
+  for (; l < p.L; ++l) {
+    const T v = src[l * p.a_axis_stride];
+    if (beats<T, MAXOP>(v, best)) { best = v; at = l; }
+  }
+  p.val[v_off] = best;
+  p.idx[i_off] = at;
+}
+
+// One wavefront per output element, lanes striding along the axis. A lane keeps the first best of its
+// own positions among the values that are not NaN; the butterfly keeps the better value and, between
+// equal values, the lower position; slice 0 holding a NaN overrides everything, as in the serial walk.
+template <typename T, bool MAXOP>
+__global__ __launch_bounds__(256) void argreduce_row(ArgArgs<T> p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t o = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (o >= p.outputs) return;
+  int64_t a_off, v_off, i_off;
+  decode3(p, o, a_off, v_off, i_off);
+  const T* src = p.a + a_off;
+  T best = (T)0;
+  int64_t at = 0;
+  bool has = false;
+  for (int64_t l = lane; l < p.L; l += 64) {
+    const T v = src[l * p.a_axis_stride];
+    if (v == v && (!has || beats<T, MAXOP>(v, best))) { best = v; at = l; has = true; }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    const T ov = __shfl_xor(best, d, 64);
+    const int64_t oa = (int64_t)__shfl_xor((long long)at, d, 64);
+    const bool oh = __shfl_xor((int)has, d, 64) != 0;
+    if (oh && (!has || beats<T, MAXOP>(ov, best) || (ov == best && oa < at))) { best = ov; at = oa; has = true; }
+  }
+  if (lane == 0) {
+    const T first = src[0];
+    if (!(first == first) || !has) { best = first; at = 0; }
+    p.val[v_off] = best;
+    p.idx[i_off] = at;
+  }
+}
+
+template <typename T>
+static int argreduce(const char* fn, int op, int rank, const int64_t* shape, int axis, int64_t* idx, const int64_t* si,
+                     T* val, const int64_t* sv, const T* a, const int64_t* sa) {
+  if (op != AM_RED_MAX && op != AM_RED_MIN) return fail(AM_E_ARG, "%s: op must be AM_RED_MAX or AM_RED_MIN", fn);
+  if (rank < 1 || rank > AM_MAXRANK) return fail(AM_E_SHAPE, "%s: rank %d outside 1..%d", fn, rank, AM_MAXRANK);
+  if (!shape || !si || !sv || !sa) return fail(AM_E_ARG, "%s: null shape or strides", fn);
+  if (axis < 0 || axis >= rank) return fail(AM_E_SHAPE, "%s: axis %d outside the tensor's rank %d", fn, axis, rank);
+  int64_t size = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+    size *= shape[d];
+  }
+  if (size == 0) return AM_OK;
+  if (!idx || !val || !a) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  ArgArgs<T> g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.val = val; g.idx = idx;
+  g.outputs = 1;
+  int64_t best_other = -1;
+  for (int d = 0; d < rank; ++d) {
+    if (d == axis || shape[d] == 1) continue;
+    g.extent[g.ndim] = shape[d]; g.a_stride[g.ndim] = sa[d]; g.v_stride[g.ndim] = sv[d]; g.i_stride[g.ndim] = si[d];
+    ++g.ndim;
+    g.outputs *= shape[d];
+    if (best_other < 0 || iabs64(sa[d]) < best_other) best_other = iabs64(sa[d]);
+  }
+  for (int d = g.ndim; d < kMaxDims; ++d) g.extent[d] = 1;
+  g.L = shape[axis]; g.a_axis_stride = sa[axis];
+  const bool row_kernel = g.L >= 64 && (best_other < 0 || iabs64(g.a_axis_stride) < best_other || g.outputs < 1024);
+  const int64_t bx = row_kernel ? (g.outputs + 3) / 4 : (g.outputs + 255) / 256;
+  if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many output elements", fn);
+  const dim3 grid((unsigned)bx), block(256);
+  if (row_kernel) {
+    if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_row<T, true>), grid, block, 0, stream(), g);
+    else hipLaunchKernelGGL((argreduce_row<T, false>), grid, block, 0, stream(), g);
+  } else {
+    if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_seq<T, true>), grid, block, 0, stream(), g);
+    else hipLaunchKernelGGL((argreduce_seq<T, false>), grid, block, 0, stream(), g);
+  }
+  return check_launch("argreduce");
+}
+
+// ------------------------------------------------------------------------------------------------
 // Row softmax. One wavefront per row up to 4096 columns, one workgroup per row beyond. The row is
 // read three times (maximum, sum of exponentials, output); the second and third reads come from
 // cache. max and sum are what the reference's streaming pass arrives at, up to rounding of the sum.
@@ -683,6 +815,12 @@ using namespace am;
   extern "C" int am_hip_reduce_all_##SFX(int op, int rank, const int64_t* shape, const T* a, const int64_t* a_strides, \
                                          T* result) {                                                                  \
     return red::reduce_all<T>("am_hip_reduce_all_" #SFX, op, rank, shape, a, a_strides, result);                       \
+  }                                                                                                                    \
+  extern "C" int am_hip_argreduce_##SFX(int op, int rank, const int64_t* shape, int axis, int64_t* idx,                \
+                                        const int64_t* idx_strides, T* val, const int64_t* val_strides, const T* a,    \
+                                        const int64_t* a_strides) {                                                    \
+    return red::argreduce<T>("am_hip_argreduce_" #SFX, op, rank, shape, axis, idx, idx_strides, val, val_strides, a,   \
+                             a_strides);                                                                               \
   }                                                                                                                    \
   extern "C" int am_hip_maxpool2d_##SFX(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW,            \
                                         int strideH, int strideW, const T* input, T* output, int64_t* argmax) {        \

@@ -680,6 +680,41 @@ def reduce_axis(op, t: HipTensor, axis: int) -> HipTensor:
     return out
 
 
+def _argreduce(op, t: HipTensor, axis: int):
+    if not 0 <= axis < t.rank:
+        raise IndexError(f"Input tensor rank ({t.rank}) must be greater than reduction axis ({axis})")
+    if t.size == 0:
+        return empty(t.shape, np.int64), empty(t.shape, t.dtype)
+    shape = list(t.shape)
+    shape[axis] = 1
+    idx, val = empty(shape, np.int64), empty(shape, t.dtype)
+    check(getattr(_lib.load(), f"am_hip_argreduce_{t.sfx}")(
+        RED[op], t.rank, i64_array(t.shape), axis, ctypes.c_void_p(idx.data_ptr()), i64_array(idx.strides),
+        ctypes.c_void_p(val.data_ptr()), i64_array(val.strides), ctypes.c_void_p(t.data_ptr()), i64_array(t.strides)))
+    return idx, val
+
+
+def argmax_max(t: HipTensor, axis: int):
+    """(indices, maxes) along an axis (src/arraymancer/tensor/aggregate.nim:159-193): the first
+    maximum wins; indices are int64, both results keep the axis with extent 1."""
+    return _argreduce("max", t, axis)
+
+
+def argmax(t: HipTensor, axis: int) -> HipTensor:
+    """aggregate.nim:195-214."""
+    return _argreduce("max", t, axis)[0]
+
+
+def argmin_min(t: HipTensor, axis: int):
+    """(indices, mins) along an axis (aggregate.nim:216-250): the first minimum wins."""
+    return _argreduce("min", t, axis)
+
+
+def argmin(t: HipTensor, axis: int) -> HipTensor:
+    """aggregate.nim:252-271."""
+    return _argreduce("min", t, axis)[0]
+
+
 def reduce_all(op, t: HipTensor):
     """reduce_inline (higher_order_foldreduce.nim:22-31): fold of every element, returned to the host."""
     out = CTYPE[t.sfx]()

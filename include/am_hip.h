@@ -359,6 +359,22 @@ int am_hip_reduce_axis_i32(int op, int rank, const int64_t* shape, int axis, int
 int am_hip_reduce_axis_i64(int op, int rank, const int64_t* shape, int axis, int64_t* dst, const int64_t* dst_strides,
                            const int64_t* a, const int64_t* a_strides);
 
+/* idx, val <- position along `axis` and value of the first maximum (op = AM_RED_MAX) or minimum
+ * (AM_RED_MIN) of `a` along that axis; both outputs have a's rank with extent 1 along `axis`
+ * (their strides along it are ignored); idx is the reference's Tensor[int] (int64). Replaces
+ * argmax_max / argmin_min (src/arraymancer/tensor/aggregate.nim:159-193, 216-250; argmax / argmin
+ * :195-214, 252-271 keep the indices only): the walk starts from slice 0 and moves on a strict
+ * `>` / `<` only, so ties keep the lowest position, a NaN in slice 0 stays and a NaN elsewhere
+ * is never taken. An empty tensor returns AM_OK without touching the outputs. */
+int am_hip_argreduce_f32(int op, int rank, const int64_t* shape, int axis, int64_t* idx, const int64_t* idx_strides,
+                         float* val, const int64_t* val_strides, const float* a, const int64_t* a_strides);
+int am_hip_argreduce_f64(int op, int rank, const int64_t* shape, int axis, int64_t* idx, const int64_t* idx_strides,
+                         double* val, const int64_t* val_strides, const double* a, const int64_t* a_strides);
+int am_hip_argreduce_i32(int op, int rank, const int64_t* shape, int axis, int64_t* idx, const int64_t* idx_strides,
+                         int32_t* val, const int64_t* val_strides, const int32_t* a, const int64_t* a_strides);
+int am_hip_argreduce_i64(int op, int rank, const int64_t* shape, int axis, int64_t* idx, const int64_t* idx_strides,
+                         int64_t* val, const int64_t* val_strides, const int64_t* a, const int64_t* a_strides);
+
 /* *result (HOST pointer) <- fold of every element of `a` (rank 0..AM_MAXRANK); blocks until the
  * value has arrived; not allowed during graph capture. Replaces reduce_inline and sum / product /
  * min / max without axis (higher_order_foldreduce.nim:22-31, aggregate.nim:33-36,46-49,89-106).

@@ -79,6 +79,10 @@ namespace detail {
                           const int64_t* sa) {                                                            \
     return am_hip_reduce_axis_##SFX(op, rank, sh, axis, d, sd, a, sa);                                    \
   }                                                                                                      \
+  inline int argreduce_(int op, int rank, const int64_t* sh, int axis, int64_t* i, const int64_t* si, T* v, \
+                        const int64_t* sv, const T* a, const int64_t* sa) {                                \
+    return am_hip_argreduce_##SFX(op, rank, sh, axis, i, si, v, sv, a, sa);                               \
+  }                                                                                                      \
   inline int reduce_all_(int op, int rank, const int64_t* sh, const T* a, const int64_t* sa, T* r) {      \
     return am_hip_reduce_all_##SFX(op, rank, sh, a, sa, r);                                               \
   }                                                                                                      \
@@ -453,6 +457,27 @@ template <typename T> HipTensor<T> mean(const HipTensor<T>& t, int axis) {
   if (s.size() == 0) return s;
   return scalar_op(AM_OP_DIV, s, static_cast<T>(t.shape[axis]));
 }
+
+// (indices, values) of the first maximum / minimum along an axis (argmax_max / argmin_min,
+// aggregate.nim:159-193, 216-250); indices are int64, both keep the axis with extent 1.
+template <typename T>
+std::pair<HipTensor<int64_t>, HipTensor<T>> argreduce(int op, const HipTensor<T>& t, int axis) {
+  if (axis < 0 || axis >= t.rank())
+    throw std::out_of_range("Input tensor rank (" + std::to_string(t.rank()) + ") must be greater than reduction axis (" +
+                            std::to_string(axis) + ")");
+  Shape shape = t.shape;
+  if (t.size() != 0) shape[axis] = 1;
+  HipTensor<int64_t> idx(shape);
+  HipTensor<T> val(shape);
+  if (t.size() != 0)
+    check(detail::argreduce_(op, t.rank(), t.shape.data(), axis, idx.ptr(), idx.strides.data(), val.ptr(), val.strides.data(),
+                             t.ptr(), t.strides.data()));
+  return {idx, val};
+}
+template <typename T> std::pair<HipTensor<int64_t>, HipTensor<T>> argmax_max(const HipTensor<T>& t, int axis) { return argreduce(AM_RED_MAX, t, axis); }
+template <typename T> std::pair<HipTensor<int64_t>, HipTensor<T>> argmin_min(const HipTensor<T>& t, int axis) { return argreduce(AM_RED_MIN, t, axis); }
+template <typename T> HipTensor<int64_t> argmax(const HipTensor<T>& t, int axis) { return argreduce(AM_RED_MAX, t, axis).first; }
+template <typename T> HipTensor<int64_t> argmin(const HipTensor<T>& t, int axis) { return argreduce(AM_RED_MIN, t, axis).first; }
 
 template <typename T> HipTensor<T> sqrt(const HipTensor<T>& t) { return unary(AM_UOP_SQRT, t); }      // ufunc.nim:91
 template <typename T> HipTensor<T> square(const HipTensor<T>& t) { return unary(AM_UOP_SQUARE, t); }  // math_functions.nim:218-222

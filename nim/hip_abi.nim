@@ -104,6 +104,10 @@ const
   AM_RED_PROD* = 1.cint
   AM_RED_MIN* = 2.cint
   AM_RED_MAX* = 3.cint
+proc am_hip_argreduce_f32*(op, rank: cint, shape: ptr int64, axis: cint, idx: ptr int64, idx_strides: ptr int64, val: ptr cfloat, val_strides: ptr int64, a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
+proc am_hip_argreduce_f64*(op, rank: cint, shape: ptr int64, axis: cint, idx: ptr int64, idx_strides: ptr int64, val: ptr cdouble, val_strides: ptr int64, a: ptr cdouble, a_strides: ptr int64): cint {.importc.}
+proc am_hip_argreduce_i32*(op, rank: cint, shape: ptr int64, axis: cint, idx: ptr int64, idx_strides: ptr int64, val: ptr int32, val_strides: ptr int64, a: ptr int32, a_strides: ptr int64): cint {.importc.}
+proc am_hip_argreduce_i64*(op, rank: cint, shape: ptr int64, axis: cint, idx: ptr int64, idx_strides: ptr int64, val: ptr int64, val_strides: ptr int64, a: ptr int64, a_strides: ptr int64): cint {.importc.}
 proc am_hip_reduce_axis_f32*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr cfloat, dst_strides: ptr int64, a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
 proc am_hip_reduce_axis_f64*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr cdouble, dst_strides: ptr int64, a: ptr cdouble, a_strides: ptr int64): cint {.importc.}
 proc am_hip_reduce_axis_i32*(op, rank: cint, shape: ptr int64, axis: cint, dst: ptr int32, dst_strides: ptr int64, a: ptr int32, a_strides: ptr int64): cint {.importc.}

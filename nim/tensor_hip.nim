@@ -360,6 +360,33 @@ proc reduce_axis[T: HipScalar](op: cint, t: HipTensor[T], axis: int): HipTensor[
   elif T is int32: check am_hip_reduce_axis_i32(op, cint t.rank, sh[0].addr, cint axis, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
   else: check am_hip_reduce_axis_i64(op, cint t.rank, sh[0].addr, cint axis, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
 
+proc argreduce[T: HipScalar](op: cint, t: HipTensor[T], axis: int): tuple[indices: HipTensor[int64], values: HipTensor[T]] =
+  ## argmax_max / argmin_min (aggregate.nim:159-193, 216-250); the indices are the reference's Tensor[int].
+  if axis < 0 or axis >= t.rank:
+    raise newException(IndexDefect, "Input tensor rank (" & $t.rank & ") must be greater than reduction axis (" & $axis & ")")
+  var oshape = t.shape.toSeq
+  if t.size != 0: oshape[axis] = 1
+  result.indices = newHipTensor[int64](oshape)
+  result.values = newHipTensor[T](oshape)
+  if t.size == 0: return
+  var sh = i64s(t.shape)
+  var si = i64s(result.indices.strides)
+  var sv = i64s(result.values.strides)
+  var sa = i64s(t.strides)
+  when T is float32: check am_hip_argreduce_f32(op, cint t.rank, sh[0].addr, cint axis, result.indices.get_offset_ptr, si[0].addr, result.values.get_offset_ptr, sv[0].addr, t.get_offset_ptr, sa[0].addr)
+  elif T is float64: check am_hip_argreduce_f64(op, cint t.rank, sh[0].addr, cint axis, result.indices.get_offset_ptr, si[0].addr, result.values.get_offset_ptr, sv[0].addr, t.get_offset_ptr, sa[0].addr)
+  elif T is int32: check am_hip_argreduce_i32(op, cint t.rank, sh[0].addr, cint axis, result.indices.get_offset_ptr, si[0].addr, result.values.get_offset_ptr, sv[0].addr, t.get_offset_ptr, sa[0].addr)
+  else: check am_hip_argreduce_i64(op, cint t.rank, sh[0].addr, cint axis, result.indices.get_offset_ptr, si[0].addr, result.values.get_offset_ptr, sv[0].addr, t.get_offset_ptr, sa[0].addr)
+
+proc argmax_max*[T: HipScalar](t: HipTensor[T], axis: int): tuple[indices: HipTensor[int64], maxes: HipTensor[T]] =
+  let r = argreduce(AM_RED_MAX, t, axis)
+  (indices: r.indices, maxes: r.values)
+proc argmax*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[int64] = argreduce(AM_RED_MAX, t, axis).indices   ## aggregate.nim:195-214
+proc argmin_min*[T: HipScalar](t: HipTensor[T], axis: int): tuple[indices: HipTensor[int64], mins: HipTensor[T]] =
+  let r = argreduce(AM_RED_MIN, t, axis)
+  (indices: r.indices, mins: r.values)
+proc argmin*[T: HipScalar](t: HipTensor[T], axis: int): HipTensor[int64] = argreduce(AM_RED_MIN, t, axis).indices   ## aggregate.nim:252-271
+
 proc reduce_all[T: HipScalar](op: cint, t: HipTensor[T]): T =
   ## reduce_inline (higher_order_foldreduce.nim:22-31), value returned to the host.
   var sh = i64s(t.shape)

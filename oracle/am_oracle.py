@@ -68,6 +68,9 @@ def lib() -> ctypes.CDLL:
             f = getattr(L, f"am_oracle_reduce_axis_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, ci, p, p, p, p]
+            f = getattr(L, f"am_oracle_argreduce_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, ci, p, p, p, p, p, p]
             f = getattr(L, f"am_oracle_reduce_all_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, p, p, p]
@@ -285,6 +288,25 @@ def reduce_axis(op, a: np.ndarray, axis: int) -> np.ndarray:
     if rc != 0:
         raise ValueError(f"oracle reduce_axis failed ({rc})")
     return out
+
+
+def argreduce(op, a: np.ndarray, axis: int):
+    """argmax_max (op "max") / argmin_min (op "min") of tensor/aggregate.nim:159-193, 216-250:
+    (indices as int64, values), both with extent 1 along `axis`."""
+    sfx = _sfx(a)
+    if not 0 <= axis < a.ndim:
+        raise IndexError(f"axis {axis} outside rank {a.ndim}")
+    out_shape = list(a.shape)
+    out_shape[axis] = 1
+    if a.size == 0:
+        return np.empty(a.shape, dtype=np.int64), np.empty(a.shape, dtype=a.dtype)
+    idx, val = np.empty(out_shape, dtype=np.int64), np.empty(out_shape, dtype=a.dtype)
+    rc = getattr(lib(), f"am_oracle_argreduce_{sfx}")(
+        RED[op], a.ndim, _i64arr(a.shape), axis, idx.ctypes.data, _i64arr(_estrides(idx)), val.ctypes.data,
+        _i64arr(_estrides(val)), a.ctypes.data, _i64arr(_estrides(a)))
+    if rc != 0:
+        raise ValueError(f"oracle argreduce failed ({rc})")
+    return idx, val
 
 
 def reduce_all(op, a: np.ndarray):

@@ -10,13 +10,14 @@
  *                                              slice along the axis, fold slices 1 .. n-1 in order;
  *                                              the result keeps the axis with extent 1
  *   tensor/aggregate.nim:33-113                sum, product, min, max (+ mean = sum div / n)
+ *   tensor/aggregate.nim:159-271               argmax_max / argmin_min: first strict maximum / minimum
  *   nn_primitives/private/p_logsumexp.nim:30-62   streaming_max_sumexp, stable_softmax
  *   nn_primitives/nnp_softmax.nim:18-38        softmax over the rows of a [batch, classes] matrix
  *   nn_primitives/nnp_maxpooling.nim:19-66     maxpool2d (values + flat argmax indices)
  * Op codes are AM_RED_* of include/am_hip.h.
  *
  * Pinned by tests/test_oracle_reduce.py against the reference's literal vectors
- * (tests/tensor/test_aggregate.nim:20-84, tests/nn_primitives/test_nnp_maxpool.nim:20-31) and
+ * (tests/tensor/test_aggregate.nim:20-215, tests/nn_primitives/test_nnp_maxpool.nim:20-31) and
  * against NumPy / exact rational arithmetic on random strided inputs. Softmax has no vector in the
  * reference's tests: it is pinned on the closed form exp(x) / sum(exp(x)) in extended precision,
  * on shift invariance and on rows summing to one.
@@ -50,6 +51,36 @@ enum { RED_SUM = 0, RED_PROD = 1, RED_MIN = 2, RED_MAX = 3 };
       T acc = a[a_off];                                                                              \
       for (int64_t l = 1; l < shape[axis]; l++) acc = fold_##SFX(op, acc, a[a_off + l * sa[axis]]);  \
       dst[d_off] = acc;                                                                              \
+      for (int d = rank - 1; d >= 0; d--) {                                                          \
+        if (d == axis) continue;                                                                     \
+        if (++coord[d] < shape[d]) break;                                                            \
+        coord[d] = 0;                                                                                \
+      }                                                                                              \
+    }                                                                                                \
+    return 0;                                                                                        \
+  }                                                                                                  \
+  /* argmax_max / argmin_min (tensor/aggregate.nim:159-193, 216-250): values start as slice 0,      \
+     positions as 0; slices 1 .. n-1 in order replace them on a strict > (op RED_MAX) or < */        \
+  int am_oracle_argreduce_##SFX(int op, int rank, const int64_t* shape, int axis, int64_t* idx,         \
+                             const int64_t* si, T* val, const int64_t* sv, const T* a,               \
+                             const int64_t* sa) {                                                    \
+    if (rank < 1 || rank > AM_MAXRANK || axis < 0 || axis >= rank) return -2;                        \
+    if (op != RED_MAX && op != RED_MIN) return -2;                                                   \
+    int64_t outputs = 1;                                                                             \
+    for (int d = 0; d < rank; d++) { if (shape[d] == 0) return 0; if (d != axis) outputs *= shape[d]; } \
+    int64_t coord[AM_MAXRANK] = {0};                                                                 \
+    for (int64_t o = 0; o < outputs; o++) {                                                          \
+      int64_t a_off = 0, v_off = 0, i_off = 0;                                                       \
+      for (int d = 0; d < rank; d++)                                                                 \
+        if (d != axis) { a_off += coord[d] * sa[d]; v_off += coord[d] * sv[d]; i_off += coord[d] * si[d]; } \
+      T best = a[a_off];                                                                             \
+      int64_t at = 0;                                                                                \
+      for (int64_t l = 1; l < shape[axis]; l++) {                                                    \
+        const T v = a[a_off + l * sa[axis]];                                                         \
+        if (op == RED_MAX ? (v > best) : (v < best)) { best = v; at = l; }                           \
+      }                                                                                              \
+      val[v_off] = best;                                                                             \
+      idx[i_off] = at;                                                                               \
       for (int d = rank - 1; d >= 0; d--) {                                                          \
         if (d == axis) continue;                                                                     \
         if (++coord[d] < shape[d]) break;                                                            \

@@ -153,6 +153,17 @@ static void variance_std() {
   CHECK(eq(am::square(toHip<int32_t>({-3, 65536, 7}, {3})), {9, 0, 49}));
 }
 
+static void argmax_argmin() {
+  // tests/tensor/test_aggregate.nim:112-119, 158-166
+  auto a = toHip<int32_t>({0, 4, 7, 1, 9, 5, 3, 4, 1}, {3, 3});
+  CHECK(eq(am::argmax(a, 0), std::vector<int64_t>{2, 1, 0}));
+  CHECK(eq(am::argmax(a, 1), std::vector<int64_t>{2, 1, 1}));
+  CHECK(eq(am::argmin(a, 0), std::vector<int64_t>{0, 0, 2}));
+  CHECK(eq(am::argmin(a, 1), std::vector<int64_t>{0, 0, 2}));
+  auto r = am::argmax_max(toHip<float>({1, 5, 5, 2}, {1, 4}), 1);
+  CHECK(eq(r.first, std::vector<int64_t>{1}) && eq(r.second, {5.0f}) && r.first.shape == (Shape{1, 1}));
+}
+
 static void fused_linear() {
   // nnp_linear.nim:28-29 + relu on small exact values
   auto x = toHip<float>({1, 2, 3, -1, -2, -3}, {2, 3});
@@ -266,6 +277,7 @@ int main(int argc, char** argv) {
     broadcasting<int64_t>();
     fused_linear();
     variance_std();
+    argmax_argmin();
     aggregates<float>();
     aggregates<double>();
     aggregates<int32_t>();

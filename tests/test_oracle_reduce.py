@@ -62,6 +62,39 @@ def test_variance_against_float64_closed_form(oracle):
     assert np.allclose(oracle.variance(x64.T, 0), np.var(x64.T, axis=0, ddof=1, keepdims=True), rtol=1e-12)
 
 
+@pytest.mark.parametrize("sfx", list(DTYPES))
+def test_reference_argmax_argmin_vectors(vectors, oracle, sfx):
+    """tests/tensor/test_aggregate.nim:112-215."""
+    dt = DTYPES[sfx]
+    for case in vectors["argmax_argmin"]["cases"]:
+        a = np.array(case["a"], dtype=dt)
+        for name, op in (("argmax", "max"), ("argmin", "min")):
+            for ax, want in case[name].items():
+                idx, val = oracle.argreduce(op, a, int(ax))
+                assert idx.dtype == np.int64 and np.array_equal(idx, np.array(want)), (name, ax)
+                assert np.array_equal(val, np.take_along_axis(a, idx, int(ax)))
+
+
+def test_argreduce_first_extremum_and_nan_rules(oracle):
+    """Ties keep the lowest position (NumPy's argmax / argmin agree on NaN-free data); a NaN in slice 0
+    stays, a NaN elsewhere is never taken (what `if val > dmax` does, aggregate.nim:191, 248)."""
+    rng = np.random.default_rng(3)
+    for dt in DTYPES.values():
+        x = rng.integers(-4, 5, (7, 33, 5)).astype(dt)      # many ties
+        for v in (x, x.transpose(2, 0, 1), x[::-1, ::2]):
+            for ax in range(3):
+                for op, ref in (("max", np.argmax), ("min", np.argmin)):
+                    idx, val = oracle.argreduce(op, v, ax)
+                    assert np.array_equal(idx, np.expand_dims(ref(v, axis=ax), ax))
+                    assert np.array_equal(val, np.take_along_axis(v, idx, ax))
+    nan = np.nan
+    x = np.array([[nan, 1, 2], [1, nan, 3], [1, nan, 0], [nan, nan, nan], [2, 2, nan]], dtype=np.float64)
+    idx, val = oracle.argreduce("max", x, 1)
+    assert idx.ravel().tolist() == [0, 2, 0, 0, 0] and np.isnan(val[0, 0]) and val[1, 0] == 3 and np.isnan(val[3, 0])
+    idx, val = oracle.argreduce("min", x, 1)
+    assert idx.ravel().tolist() == [0, 0, 2, 0, 0] and val[2, 0] == 0
+
+
 def test_reference_maxpool_vectors(vectors, oracle):
     g = vectors["maxpool"]
     for dt in DTYPES.values():

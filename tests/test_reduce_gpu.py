@@ -169,6 +169,62 @@ def test_variance_and_std(hip, oracle, vectors, sfx):
 
 
 @pytest.mark.parametrize("sfx", ALL)
+def test_argmax_argmin(hip, oracle, vectors, sfx):
+    """argmax_max / argmin_min (aggregate.nim:159-271): the reference's literals, then the oracle on
+    tie-heavy and random data, along every axis, over views, through both kernels (one lane per
+    output; one wavefront per output for long axes), bit-exact in positions and values."""
+    dt = DTYPES[sfx]
+    for case in vectors["argmax_argmin"]["cases"]:
+        a = hip.toHip(np.array(case["a"], dtype=dt))
+        for name in ("argmax", "argmin"):
+            for ax, want in case[name].items():
+                got = getattr(hip, name)(a, int(ax))
+                assert got.dtype == np.int64 and np.array_equal(got.toCpu(), np.array(want)), (name, ax)
+    rng = np.random.default_rng(seed_of("argmax", sfx))
+    for shape in [(7, 33, 5), (300, 70), (5, 5000), (5000, 5), (64, 10), (3, 2, 4, 3, 2, 3), (1, 1), (2100, 1100)]:
+        for ties in (True, False):
+            x = rng.integers(-4, 5, shape).astype(dt) if ties else fill(rng, shape, dt)
+            dx = hip.toHip(x)
+            for name, v, mk in views(x):
+                dv = mk(dx)
+                if dv is None or v.size == 0:
+                    continue
+                for ax in range(v.ndim):
+                    for op, fn in (("max", hip.argmax_max), ("min", hip.argmin_min)):
+                        say("argreduce", sfx, shape, ties, name, ax, op)
+                        gi, gv = fn(dv, ax)
+                        wi, wv = oracle.argreduce(op, v, ax)
+                        assert gi.shape == wi.shape and np.array_equal(gi.toCpu(), wi), (shape, name, ax, op)
+                        assert np.array_equal(gv.toCpu(), wv), (shape, name, ax, op)
+    with pytest.raises(IndexError):
+        hip.argmax(hip.zeros((2, 2), dt), 2)
+    assert hip.argmax(hip.empty((0, 3), dt), 0).shape == (0, 3)
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_argmax_nan_rules(hip, oracle, sfx):
+    """A NaN in slice 0 stays, a NaN elsewhere is never taken — also when the axis is long enough for
+    the wavefront kernel, whose lanes each see only every 64th element."""
+    dt = DTYPES[sfx]
+    nan = np.nan
+    x = np.array([[nan, 1, 2], [1, nan, 3], [1, nan, 0], [nan, nan, nan], [2, 2, nan]], dtype=dt)
+    for op, fn in (("max", hip.argmax_max), ("min", hip.argmin_min)):
+        gi, gv = fn(hip.toHip(x), 1)
+        wi, wv = oracle.argreduce(op, x, 1)
+        assert np.array_equal(gi.toCpu(), wi) and np.array_equal(gv.toCpu(), wv, equal_nan=True)
+    rng = np.random.default_rng(seed_of("argmax-nan", sfx))
+    y = rng.standard_normal((6, 1000)).astype(dt)
+    y[0, 0] = nan; y[1, 500] = nan; y[2, ::3] = nan; y[3, 1:] = nan; y[4, :] = nan; y[5, 64] = nan; y[5, 0] = y[5].max()
+    for v, dv in ((y, hip.toHip(y)), (y.T, hip.toHip(np.ascontiguousarray(y.T)))):
+        ax = 1 if v is y else 0
+        for op, fn in (("max", hip.argmax_max), ("min", hip.argmin_min)):
+            gi, gv = fn(dv, ax)
+            wi, wv = oracle.argreduce(op, v, ax)
+            assert np.array_equal(gi.toCpu(), wi), (op, ax)
+            assert np.array_equal(gv.toCpu(), wv, equal_nan=True), (op, ax)
+
+
+@pytest.mark.parametrize("sfx", ALL)
 def test_column_walks_with_16_byte_lanes(hip, oracle, sfx):
     """Walks across a unit-stride dimension take 16 bytes of adjacent outputs per lane when extents,
     strides and base addresses allow it, and one output per lane otherwise; both fold every output
