@@ -13,14 +13,14 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, maxpool2d, tanh, relu_backward, sigmoid_backward,
                          tanh_backward, linear_backward, variance, std, sqrt, square, argmax_max, argmax,
-                         argmin_min, argmin)
+                         argmin_min, argmin, maxpool2d_backward)
 
 __all__ = [
     "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
     "toHip", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "conv2d", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
     "unary", "relu", "sigmoid", "bias_relu", "bc_add", "bc_sub", "bc_mul", "bc_div", "bc_mod",
     "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward",
-    "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin",
+    "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin", "maxpool2d_backward",
     "reduce_axis", "reduce_all", "sum", "product", "min", "max", "mean", "softmax", "maxpool2d",
     "read_npy", "write_npy", "load_library",
 ]

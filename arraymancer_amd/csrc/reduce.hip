@@ -802,6 +802,55 @@ static int maxpool(const char* fn, int64_t N, int C, int H, int W, int kH, int k
   return check_launch("maxpool2d");
 }
 
+// Backward pass of max pooling: grad_in[argmax[i]] = grad_out[i] over zeros, the LAST i winning where
+// overlapping windows picked the same input element (the serial order of
+// src/arraymancer/nn_primitives/nnp_maxpooling.nim:68-83). Run as a gather so that nothing races: one
+// lane per input element looks through the windows that contain it, highest output index first, and
+// takes the first whose recorded maximum is this element.
+template <typename T>
+__global__ __launch_bounds__(256) void maxpool2d_backward(const int64_t* argmax, const T* grad_out, T* grad_in, int64_t total,
+                                                          int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
+                                                          int outH, int outW) {
+  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (p >= total) return;
+  const int col = (int)(p % W);
+  const int64_t t = p / W;
+  const int row = (int)(t % H);
+  const int64_t nc = t / H;
+  // windows h with h * sH - padH <= row < h * sH - padH + kH
+  const int rh = row + padH, rw = col + padW;
+  int h_hi = rh / sH, w_hi = rw / sW;
+  int h_lo = rh - kH + 1 <= 0 ? 0 : (rh - kH + sH) / sH, w_lo = rw - kW + 1 <= 0 ? 0 : (rw - kW + sW) / sW;
+  if (h_hi > outH - 1) h_hi = outH - 1;
+  if (w_hi > outW - 1) w_hi = outW - 1;
+  T g = (T)0;
+  bool found = false;
+  for (int h = h_hi; h >= h_lo && !found; --h)
+    for (int w = w_hi; w >= w_lo; --w) {
+      const int64_t o = w + (int64_t)outW * (h + (int64_t)outH * nc);
+      if (argmax[o] == p) { g = grad_out[o]; found = true; break; }
+    }
+  grad_in[p] = g;
+}
+
+template <typename T>
+static int maxpool_backward(const char* fn, int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
+                            const int64_t* argmax, const T* grad_out, T* grad_in) {
+  if (N < 0 || C < 0 || H < 0 || W < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+  if (kH < 1 || kW < 1 || sH < 1 || sW < 1 || padH < 0 || padW < 0) return fail(AM_E_ARG, "%s: kernel and stride must be >= 1, padding >= 0", fn);
+  if ((int64_t)H + 2 * padH < kH || (int64_t)W + 2 * padW < kW) return fail(AM_E_SHAPE, "%s: kernel larger than the padded input", fn);
+  const int64_t outH = ((int64_t)H + 2 * padH - kH) / sH + 1, outW = ((int64_t)W + 2 * padW - kW) / sW + 1;
+  const int64_t total = N * C * (int64_t)H * W;
+  if (total == 0) return AM_OK;
+  if (!argmax || !grad_out || !grad_in) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  const int64_t bx = (total + 255) / 256;
+  if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many input elements", fn);
+  hipLaunchKernelGGL((maxpool2d_backward<T>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in, total, H, W,
+                     kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
+  return check_launch("maxpool2d_backward");
+}
+
 }  // namespace red
 }  // namespace am
 
@@ -826,6 +875,12 @@ using namespace am;
                                         int strideH, int strideW, const T* input, T* output, int64_t* argmax) {        \
     return red::maxpool<T>("am_hip_maxpool2d_" #SFX, N, C, H, W, kH, kW, padH, padW, strideH, strideW, input, output,  \
                            argmax);                                                                                    \
+  }                                                                                                                    \
+  extern "C" int am_hip_maxpool2d_backward_##SFX(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW,   \
+                                                 int strideH, int strideW, const int64_t* argmax, const T* grad_output, \
+                                                 T* grad_input) {                                                      \
+    return red::maxpool_backward<T>("am_hip_maxpool2d_backward_" #SFX, N, C, H, W, kH, kW, padH, padW, strideH,        \
+                                    strideW, argmax, grad_output, grad_input);                                         \
   }
 
 AM_RED_ENTRY_POINTS(float, f32)

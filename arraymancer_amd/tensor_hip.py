@@ -63,7 +63,7 @@ def _dtype_sfx(dtype) -> str:
 
 
 class HipTensor:
-    __slots__ = ("layout", "storage", "dtype")
+    __slots__ = ("layout", "storage", "dtype", "pool_geometry")
 
     def __init__(self, layout: Layout, storage: HipStorage, dtype):
         self.layout = layout
@@ -820,5 +820,34 @@ def maxpool2d(x: HipTensor, kernel, padding=(0, 0), stride=(1, 1)):
     check(getattr(_lib.load(), f"am_hip_maxpool2d_{x.sfx}")(
         N, C, H, W, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(out.data_ptr()),
         ctypes.c_void_p(idx.data_ptr())))
+    idx.pool_geometry = ((kh, kw), (ph, pw), (sh, sw))   # what maxpool2d_backward needs besides the indices
     return idx, out
+
+
+def maxpool2d_backward(cached_input_shape, cached_max_indices: HipTensor, gradOutput: HipTensor, kernel=None,
+                       padding=None, stride=None) -> HipTensor:
+    """gradInput = zeros(cached_input_shape) with gradInput[max_indices[i]] = gradOutput[i]
+    (src/arraymancer/nn_primitives/nnp_maxpooling.nim:68-83). The device runs the scatter as a gather
+    over the pooling windows and therefore needs kernel, padding and stride: they are taken from
+    the indices returned by maxpool2d of this module, or passed explicitly."""
+    geom = getattr(cached_max_indices, "pool_geometry", None)
+    if kernel is not None:
+        geom = (tuple(kernel), tuple(padding or (0, 0)), tuple(stride or (1, 1)))
+    if geom is None:
+        raise ValueError("maxpool2d_backward: pass kernel, padding and stride (the indices do not come from maxpool2d)")
+    shape = tuple(int(s) for s in cached_input_shape)
+    if len(shape) != 4:
+        raise ValueError("maxpool2d_backward: cached_input_shape must be [N, C, H, W]")
+    (kh, kw), (ph, pw), (sh, sw) = geom
+    N, C, H, W = shape
+    ho, wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    if gradOutput.size != cached_max_indices.size or gradOutput.size != N * C * ho * wo:
+        raise ValueError("maxpool2d_backward: gradOutput, the indices and the pooling geometry do not match")
+    if cached_max_indices.dtype != np.int64 or not cached_max_indices.is_C_contiguous() or not gradOutput.is_C_contiguous():
+        raise ValueError("maxpool2d_backward: indices must be a contiguous int64 tensor, gradOutput contiguous")
+    out = empty(shape, gradOutput.dtype)
+    check(getattr(_lib.load(), f"am_hip_maxpool2d_backward_{gradOutput.sfx}")(
+        N, C, H, W, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(cached_max_indices.data_ptr()),
+        ctypes.c_void_p(gradOutput.data_ptr()), ctypes.c_void_p(out.data_ptr())))
+    return out
 

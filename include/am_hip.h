@@ -408,6 +408,22 @@ int am_hip_maxpool2d_i32(int64_t N, int C, int H, int W, int kH, int kW, int pad
 int am_hip_maxpool2d_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
                          const int64_t* input, int64_t* output, int64_t* argmax);
 
+/* grad_input[N, C, H, W] <- zeros, then grad_input[argmax[i]] = grad_output[i] for the outputs i in
+ * ascending order (where overlapping windows recorded the same input element, the last one wins):
+ * maxpool2d_backward (src/arraymancer/nn_primitives/nnp_maxpooling.nim:68-83; the reference runs this
+ * loop under OpenMP, so its own result for such duplicates depends on thread timing; the serial order
+ * is reproduced here). argmax is what am_hip_maxpool2d_* wrote for the same geometry, which the
+ * reference's signature does not carry and this one needs: the scatter is run as a race-free gather,
+ * every input element looking through the windows that contain it. All tensors C-contiguous. */
+int am_hip_maxpool2d_backward_f32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH,
+                                  int strideW, const int64_t* argmax, const float* grad_output, float* grad_input);
+int am_hip_maxpool2d_backward_f64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH,
+                                  int strideW, const int64_t* argmax, const double* grad_output, double* grad_input);
+int am_hip_maxpool2d_backward_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH,
+                                  int strideW, const int64_t* argmax, const int32_t* grad_output, int32_t* grad_input);
+int am_hip_maxpool2d_backward_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH,
+                                  int strideW, const int64_t* argmax, const int64_t* grad_output, int64_t* grad_input);
+
 /* ---------------------------------------------------------------- measurement aid
  * No counterpart in the reference. Register-only micro-benchmarks of the issue ceilings the GEMM
  * kernels are compared with (used by bench.py: 32/64-bit integers have no matrix instruction and no

@@ -86,6 +86,10 @@ namespace detail {
   inline int reduce_all_(int op, int rank, const int64_t* sh, const T* a, const int64_t* sa, T* r) {      \
     return am_hip_reduce_all_##SFX(op, rank, sh, a, sa, r);                                               \
   }                                                                                                      \
+  inline int maxpool2d_backward_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW, \
+                                 const int64_t* idx, const T* go, T* gi) {                                \
+    return am_hip_maxpool2d_backward_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, idx, go, gi);              \
+  }                                                                                                      \
   inline int maxpool2d_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,    \
                         const T* in, T* out, int64_t* idx) {                                              \
     return am_hip_maxpool2d_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, in, out, idx);                      \
@@ -519,6 +523,25 @@ MaxPooled<T> maxpool2d(const HipTensor<T>& x, int kH, int kW, int padH = 0, int 
   MaxPooled<T> r{HipTensor<int64_t>(Shape{N * C * oh * ow}), HipTensor<T>(Shape{N, C, oh, ow})};
   check(detail::maxpool2d_(N, (int)C, (int)H, (int)W, kH, kW, padH, padW, strideH, strideW, x.ptr(), r.maxpooled.ptr(),
                            r.max_indices.ptr()));
+  return r;
+}
+
+// maxpool2d_backward (nnp_maxpooling.nim:68-83): zeros of the cached input shape with
+// gradInput[max_indices[i]] = gradOutput[i]. The device runs the scatter as a gather over the pooling
+// windows, so the geometry of the forward pass is passed again.
+template <typename T>
+HipTensor<T> maxpool2d_backward(const Shape& cached_input_shape, const HipTensor<int64_t>& cached_max_indices,
+                                const HipTensor<T>& grad_output, int kH, int kW, int padH = 0, int padW = 0,
+                                int strideH = 1, int strideW = 1) {
+  if (cached_input_shape.size() != 4) throw std::invalid_argument("maxpool2d_backward: cached_input_shape must be [N, C, H, W]");
+  const int64_t N = cached_input_shape[0], C = cached_input_shape[1], H = cached_input_shape[2], W = cached_input_shape[3];
+  const int64_t oh = (H + 2 * padH - kH) / strideH + 1, ow = (W + 2 * padW - kW) / strideW + 1;
+  if (grad_output.size() != cached_max_indices.size() || grad_output.size() != N * C * oh * ow ||
+      !grad_output.is_C_contiguous() || !cached_max_indices.is_C_contiguous())
+    throw std::invalid_argument("maxpool2d_backward: gradOutput, the indices and the pooling geometry do not match");
+  HipTensor<T> r(cached_input_shape);
+  check(detail::maxpool2d_backward_(N, (int)C, (int)H, (int)W, kH, kW, padH, padW, strideH, strideW, cached_max_indices.ptr(),
+                                    grad_output.ptr(), r.ptr()));
   return r;
 }
 

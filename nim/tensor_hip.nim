@@ -472,6 +472,23 @@ proc maxpool2d*[T: HipScalar](input: HipTensor[T], kernel: tuple[height, width: 
   elif T is int32: call am_hip_maxpool2d_i32
   else: call am_hip_maxpool2d_i64
 
+proc maxpool2d_backward*[T: HipScalar](cached_input_shape: openArray[int], cached_max_indices: HipTensor[int64],
+                                       gradOutput: HipTensor[T], kernel: tuple[height, width: int],
+                                       padding = (0, 0), stride = (1, 1)): HipTensor[T] =
+  ## nn_primitives/nnp_maxpooling.nim:68-83. The device runs the scatter as a gather over the pooling
+  ## windows, so kernel, padding and stride of the forward pass are passed again.
+  assert cached_input_shape.len == 4 and gradOutput.size == cached_max_indices.size
+  assert gradOutput.is_C_contiguous and cached_max_indices.is_C_contiguous
+  let (N, C, H, W) = (cached_input_shape[0], cached_input_shape[1], cached_input_shape[2], cached_input_shape[3])
+  result = newHipTensor[T]([N, C, H, W])
+  template call(f: untyped) =
+    check f(int64 N, cint C, cint H, cint W, cint kernel.height, cint kernel.width, cint padding[0], cint padding[1],
+            cint stride[0], cint stride[1], cached_max_indices.get_offset_ptr, gradOutput.get_offset_ptr, result.get_offset_ptr)
+  when T is float32: call am_hip_maxpool2d_backward_f32
+  elif T is float64: call am_hip_maxpool2d_backward_f64
+  elif T is int32: call am_hip_maxpool2d_backward_i32
+  else: call am_hip_maxpool2d_backward_i64
+
 # ---------------------------------------------------------------- .npy files and display
 # The file parsing and the pretty printer are the reference's own host code (io/io_npy.nim:64-183,
 # tensor/private/p_display.nim); the device tensor goes through a host copy, exactly as

@@ -74,6 +74,9 @@ def lib() -> ctypes.CDLL:
             f = getattr(L, f"am_oracle_reduce_all_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, p, p, p]
+            f = getattr(L, f"am_oracle_maxpool2d_backward_{sfx}")
+            f.restype = ci
+            f.argtypes = [i64, i64, p, p, p]
             f = getattr(L, f"am_oracle_maxpool2d_{sfx}")
             f.restype = ci
             f.argtypes = [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, p, p, p, ct]
@@ -374,6 +377,18 @@ def maxpool2d(x: np.ndarray, kernel, padding=(0, 0), stride=(1, 1)):
     getattr(lib(), f"am_oracle_maxpool2d_{sfx}")(N, C, H, W, kernel[0], kernel[1], padding[0], padding[1], stride[0], stride[1],
                                                  x.ctypes.data, out.ctypes.data, idx.ctypes.data, _CT[sfx](lowest))
     return idx, out
+
+
+def maxpool2d_backward(cached_input_shape, cached_max_indices: np.ndarray, grad_output: np.ndarray) -> np.ndarray:
+    """nnp_maxpooling.nim:68-83, serial: zeros(cached_input_shape), then result[idx[i]] = gradOutput[i]
+    for i in order."""
+    sfx = _sfx(grad_output)
+    go = np.ascontiguousarray(grad_output).reshape(-1)
+    idx = np.ascontiguousarray(cached_max_indices, dtype=np.int64).reshape(-1)
+    assert go.size == idx.size
+    out = np.empty(tuple(cached_input_shape), dtype=grad_output.dtype)
+    getattr(lib(), f"am_oracle_maxpool2d_backward_{sfx}")(out.size, go.size, idx.ctypes.data, go.ctypes.data, out.ctypes.data)
+    return out
 
 
 def closed_gemm_int(alpha, A, B, beta, C):

@@ -14,6 +14,7 @@
  *   nn_primitives/private/p_logsumexp.nim:30-62   streaming_max_sumexp, stable_softmax
  *   nn_primitives/nnp_softmax.nim:18-38        softmax over the rows of a [batch, classes] matrix
  *   nn_primitives/nnp_maxpooling.nim:19-66     maxpool2d (values + flat argmax indices)
+ *   nn_primitives/nnp_maxpooling.nim:68-83     maxpool2d_backward (scatter through the indices)
  * Op codes are AM_RED_* of include/am_hip.h.
  *
  * Pinned by tests/test_oracle_reduce.py against the reference's literal vectors
@@ -138,6 +139,22 @@ enum { RED_SUM = 0, RED_PROD = 1, RED_MIN = 2, RED_MAX = 3 };
           }                                                                                          \
     return 0;                                                                                        \
   }
+
+/* maxpool2d_backward (nnp_maxpooling.nim:68-83), serial: zeros, then rdata[cmidata[i]] = godata[i] in order */
+#define DEFINE_POOL_BACKWARD(T, SFX)                                                                 \
+  int am_oracle_maxpool2d_backward_##SFX(int64_t n_in, int64_t n_out, const int64_t* argmax,            \
+                                      const T* grad_out, T* grad_in) {                               \
+    memset(grad_in, 0, (size_t)n_in * sizeof(T));                                                    \
+    for (int64_t i = 0; i < n_out; i++) {                                                            \
+      if (argmax[i] < 0 || argmax[i] >= n_in) continue;   /* a window made of padding only */          \
+      grad_in[argmax[i]] = grad_out[i];                                                              \
+    }                                                                                                \
+    return 0;                                                                                        \
+  }
+DEFINE_POOL_BACKWARD(float, f32)
+DEFINE_POOL_BACKWARD(double, f64)
+DEFINE_POOL_BACKWARD(int32_t, i32)
+DEFINE_POOL_BACKWARD(int64_t, i64)
 
 DEFINE_FOLD(float, float, f32, 0)
 DEFINE_FOLD(double, double, f64, 0)

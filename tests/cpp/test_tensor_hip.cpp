@@ -164,6 +164,15 @@ static void argmax_argmin() {
   CHECK(eq(r.first, std::vector<int64_t>{1}) && eq(r.second, {5.0f}) && r.first.shape == (Shape{1, 1}));
 }
 
+static void maxpool_backward() {
+  // tests/nn_primitives/test_nnp_maxpool.nim:20-45
+  auto a = toHip<float>({1, 1, 2, 4, 5, 6, 7, 8, 3, 2, 1, 0, 1, 2, 3, 4}, {1, 1, 4, 4});
+  auto p = am::maxpool2d(a, 2, 2, 0, 0, 2, 2);
+  CHECK(eq(p.maxpooled, {6, 8, 3, 4}) && eq(p.max_indices, std::vector<int64_t>{5, 7, 8, 15}));
+  auto g = am::maxpool2d_backward(a.shape, p.max_indices, p.maxpooled, 2, 2, 0, 0, 2, 2);
+  CHECK(eq(g, {0, 0, 0, 0, 0, 6, 0, 8, 3, 0, 0, 0, 0, 0, 0, 4}));
+}
+
 static void fused_linear() {
   // nnp_linear.nim:28-29 + relu on small exact values
   auto x = toHip<float>({1, 2, 3, -1, -2, -3}, {2, 3});
@@ -278,6 +287,7 @@ int main(int argc, char** argv) {
     fused_linear();
     variance_std();
     argmax_argmin();
+    maxpool_backward();
     aggregates<float>();
     aggregates<double>();
     aggregates<int32_t>();

@@ -102,6 +102,32 @@ def test_reference_maxpool_vectors(vectors, oracle):
         idx, pooled = oracle.maxpool2d(x, g["kernel"], g["padding"], g["stride"])
         assert np.array_equal(pooled, np.array(g["pooled"], dtype=dt).reshape(g["pooled_shape"]))
         assert np.array_equal(idx, np.array(g["max_indices"], dtype=np.int64))
+        # backward with gradOutput = pooled (tests/nn_primitives/test_nnp_maxpool.nim:34-45)
+        grad = oracle.maxpool2d_backward(x.shape, idx, pooled)
+        assert np.array_equal(grad.reshape(4, 4), np.array(g["backward"]["grad_input"], dtype=dt))
+
+
+def test_maxpool_backward_is_the_serial_scatter(oracle):
+    """Overlapping windows record the same input element several times: the last output in index
+    order wins (a NumPy fancy assignment applies the same rule); without overlap the result is the
+    gradient of sum(maxpooled * G), checked by differences on a tie-free input."""
+    rng = np.random.default_rng(8)
+    x = rng.integers(-3, 4, (2, 3, 7, 6)).astype(np.float64)
+    idx, pooled = oracle.maxpool2d(x, (3, 3), (1, 1), (1, 1))
+    g = rng.standard_normal(pooled.shape)
+    want = np.zeros(x.size)
+    want[idx] = g.reshape(-1)
+    assert np.array_equal(oracle.maxpool2d_backward(x.shape, idx, g).reshape(-1), want)
+    x = rng.permutation(2 * 2 * 6 * 6).reshape(2, 2, 6, 6).astype(np.float64)   # no ties
+    idx, pooled = oracle.maxpool2d(x, (2, 2), (0, 0), (2, 2))
+    g = rng.standard_normal(pooled.shape)
+    grad = oracle.maxpool2d_backward(x.shape, idx, g)
+    h = 1e-3
+    for pos in [(0, 0, 0, 0), (1, 1, 3, 2), (0, 1, 5, 5), (1, 0, 2, 4)]:
+        xp, xm = x.copy(), x.copy()
+        xp[pos] += h; xm[pos] -= h
+        num = ((oracle.maxpool2d(xp, (2, 2), (0, 0), (2, 2))[1] - oracle.maxpool2d(xm, (2, 2), (0, 0), (2, 2))[1]) * g).sum() / (2 * h)
+        assert abs(num - grad[pos]) < 1e-9
 
 
 @pytest.mark.parametrize("sfx", ["i32", "i64"])

@@ -323,6 +323,7 @@ def test_maxpool_vs_oracle(hip, oracle, vectors, sfx):
     dt = DTYPES[sfx]
     g = vectors["maxpool"]
     x = np.array(g["input"], dtype=dt).reshape(g["input_shape"])
+    x0 = x
     idx, pooled = hip.maxpool2d(hip.toHip(x), g["kernel"], g["padding"], g["stride"])
     assert np.array_equal(pooled.toCpu(), np.array(g["pooled"], dtype=dt).reshape(g["pooled_shape"]))
     assert np.array_equal(idx.toCpu(), np.array(g["max_indices"], dtype=np.int64))
@@ -335,6 +336,17 @@ def test_maxpool_vs_oracle(hip, oracle, vectors, sfx):
         want_idx, want = oracle.maxpool2d(x, kernel, pad, stride)
         idx, got = hip.maxpool2d(hip.toHip(x), kernel, pad, stride)
         assert np.array_equal(got.toCpu(), want) and np.array_equal(idx.toCpu(), want_idx)
+        # backward: the serial scatter of the reference, overlapping windows included (last output wins)
+        go = rng.integers(-99, 100, want.shape).astype(dt)
+        want_grad = oracle.maxpool2d_backward(shape, want_idx, go)
+        grad = hip.maxpool2d_backward(shape, idx, hip.toHip(go))
+        assert grad.shape == tuple(shape) and np.array_equal(grad.toCpu(), want_grad), ("backward", shape, kernel, pad, stride)
+        bare = hip.toHip(want_idx)                                          # indices that did not come from maxpool2d
+        assert np.array_equal(hip.maxpool2d_backward(shape, bare, hip.toHip(go), kernel, pad, stride).toCpu(), want_grad)
+        with pytest.raises(ValueError):
+            hip.maxpool2d_backward(shape, bare, hip.toHip(go))
+    gb = hip.maxpool2d_backward(g["input_shape"], *hip.maxpool2d(hip.toHip(x0), g["kernel"], g["padding"], g["stride"]))
+    assert np.array_equal(gb.toCpu().reshape(4, 4), np.array(g["backward"]["grad_input"], dtype=dt))
     with pytest.raises(ValueError):
         hip.maxpool2d(hip.zeros((4, 4), dt), (2, 2))                       # rank
     with pytest.raises(ValueError):
