@@ -407,6 +407,9 @@ template <typename T> struct ArgArgs {
   int ndim;
   int64_t extent[kMaxDims], a_stride[kMaxDims], v_stride[kMaxDims], i_stride[kMaxDims];
   int64_t outputs, L, a_axis_stride;
+  // the axis cut into chunks (one-lane-per-output kernel, too few outputs to fill the chip): partial
+  // values and positions [chunk][output] in the workspace, position -1 = nothing but NaN in the chunk
+  int chunks; int64_t chunk_len; T* ws_val; int64_t* ws_idx;
 };
 
 template <typename T>
@@ -426,7 +429,8 @@ __device__ __forceinline__ void decode3(const ArgArgs<T>& p, int64_t o, int64_t&
 
 template <typename T, bool MAXOP> __device__ __forceinline__ bool beats(T x, T cur) { return MAXOP ? (x > cur) : (x < cur); }
 
-// One lane per output element walks the axis front to back.
+// One lane per output element walks the axis (or its chunk of it) front to back. The chunk that holds
+// slice 0 starts from that slice whatever it is; later chunks skip NaN, which the serial walk never takes.
 template <typename T, bool MAXOP>
 __global__ __launch_bounds__(256) void argreduce_seq(ArgArgs<T> p) {
   const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -434,30 +438,56 @@ __global__ __launch_bounds__(256) void argreduce_seq(ArgArgs<T> p) {
   int64_t a_off, v_off, i_off;
   decode3(p, o, a_off, v_off, i_off);
   const T* src = p.a + a_off;
-  T best = src[0];
-  int64_t at = 0;
-  int64_t l = 1;
-  for (; l + 4 <= p.L; l += 4) {   // four loads in flight, compared in axis order
+  const int64_t l0 = (int64_t)blockIdx.y * p.chunk_len;
+  const int64_t l1 = (l0 + p.chunk_len < p.L) ? l0 + p.chunk_len : p.L;
+  T best = src[l0 * p.a_axis_stride];
+  int64_t at = l0;
+  bool has = (blockIdx.y == 0) || (best == best);
+  auto take = [&](T v, int64_t l) {
+    if (has ? beats<T, MAXOP>(v, best) : (v == v)) { best = v; at = l; has = true; }
+  };
+  int64_t l = l0 + 1;
+  for (; l + 4 <= l1; l += 4) {   // four loads in flight, compared in axis order
     const T v0 = src[l * p.a_axis_stride], v1 = src[(l + 1) * p.a_axis_stride];
     const T v2 = src[(l + 2) * p.a_axis_stride], v3 = src[(l + 3) * p.a_axis_stride];
-    if (beats<T, MAXOP>(v0, best)) { best = v0; at = l; }
-    if (beats<T, MAXOP>(v1, best)) { best = v1; at = l + 1; }
-    if (beats<T, MAXOP>(v2, best)) { best = v2; at = l + 2; }
-    if (beats<T, MAXOP>(v3, best)) { best = v3; at = l + 3; }
+    take(v0, l); take(v1, l + 1); take(v2, l + 2); take(v3, l + 3);
   }
-  for (; l < p.L; ++l) {
-    const T v = src[l * p.a_axis_stride];
-    if (beats<T, MAXOP>(v, best)) { best = v; at = l; }
+  for (; l < l1; ++l) take(src[l * p.a_axis_stride], l);
+  if (p.chunks > 1) {
+    p.ws_val[(int64_t)blockIdx.y * p.outputs + o] = best;
+    p.ws_idx[(int64_t)blockIdx.y * p.outputs + o] = has ? at : -1;
+  } else {
+    p.val[v_off] = best;
+    p.idx[i_off] = at;
+  }
+}
+
+// Second pass of the chunked walk: the chunks' results in axis order under the same strict comparison.
+template <typename T, bool MAXOP>
+__global__ __launch_bounds__(256) void argreduce_merge(ArgArgs<T> p) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= p.outputs) return;
+  int64_t a_off, v_off, i_off;
+  decode3(p, o, a_off, v_off, i_off);
+  T best = p.ws_val[o];
+  int64_t at = p.ws_idx[o];       // chunk 0 always has a position
+  for (int c = 1; c < p.chunks; ++c) {
+    const T v = p.ws_val[(int64_t)c * p.outputs + o];
+    const int64_t i = p.ws_idx[(int64_t)c * p.outputs + o];
+    if (i >= 0 && beats<T, MAXOP>(v, best)) { best = v; at = i; }
   }
   p.val[v_off] = best;
   p.idx[i_off] = at;
 }
 
-// One wavefront per output element, lanes striding along the axis. A lane keeps the first best of its
-// own positions among the values that are not NaN; the butterfly keeps the better value and, between
-// equal values, the lower position; slice 0 holding a NaN overrides everything, as in the serial walk.
-template <typename T, bool MAXOP>
+// One wavefront per output element, lanes striding along the axis (16-byte loads when it has unit
+// stride). A lane keeps the first best of its own positions among the values that are not NaN; the
+// butterfly keeps the better value and, between equal values, the lower position; slice 0 holding a
+// NaN overrides everything, as in the serial walk.
+template <typename T, bool MAXOP, bool VEC>
 __global__ __launch_bounds__(256) void argreduce_row(ArgArgs<T> p) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
   const int lane = threadIdx.x & 63;
   const int64_t o = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (o >= p.outputs) return;
@@ -467,9 +497,32 @@ __global__ __launch_bounds__(256) void argreduce_row(ArgArgs<T> p) {
   T best = (T)0;
   int64_t at = 0;
   bool has = false;
-  for (int64_t l = lane; l < p.L; l += 64) {
-    const T v = src[l * p.a_axis_stride];
+  auto take = [&](T v, int64_t l) {
     if (v == v && (!has || beats<T, MAXOP>(v, best))) { best = v; at = l; has = true; }
+  };
+  if constexpr (VEC) {
+    const vec_t* vs = (const vec_t*)src;
+    const int64_t nvec = p.L / V;
+    int64_t v = lane;
+    for (; v + 192 < nvec; v += 256) {   // four 16-byte loads in flight per lane, taken in position order
+      const vec_t x0 = vs[v], x1 = vs[v + 64], x2 = vs[v + 128], x3 = vs[v + 192];
+#pragma unroll
+      for (int e = 0; e < V; ++e) take(x0[e], v * V + e);
+#pragma unroll
+      for (int e = 0; e < V; ++e) take(x1[e], (v + 64) * V + e);
+#pragma unroll
+      for (int e = 0; e < V; ++e) take(x2[e], (v + 128) * V + e);
+#pragma unroll
+      for (int e = 0; e < V; ++e) take(x3[e], (v + 192) * V + e);
+    }
+    for (; v < nvec; v += 64) {
+      const vec_t x0 = vs[v];
+#pragma unroll
+      for (int e = 0; e < V; ++e) take(x0[e], v * V + e);
+    }
+    for (int64_t l = nvec * V + lane; l < p.L; l += 64) take(src[l], l);
+  } else {
+    for (int64_t l = lane; l < p.L; l += 64) take(src[l * p.a_axis_stride], l);
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) {
@@ -518,13 +571,41 @@ static int argreduce(const char* fn, int op, int rank, const int64_t* shape, int
   const bool row_kernel = g.L >= 64 && (best_other < 0 || iabs64(g.a_axis_stride) < best_other || g.outputs < 1024);
   const int64_t bx = row_kernel ? (g.outputs + 3) / 4 : (g.outputs + 255) / 256;
   if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many output elements", fn);
-  const dim3 grid((unsigned)bx), block(256);
+  g.chunks = 1; g.chunk_len = g.L; g.ws_val = nullptr; g.ws_idx = nullptr;
+  const dim3 block(256);
   if (row_kernel) {
-    if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_row<T, true>), grid, block, 0, stream(), g);
-    else hipLaunchKernelGGL((argreduce_row<T, false>), grid, block, 0, stream(), g);
+    constexpr int64_t V = 16 / (int64_t)sizeof(T);
+    bool vec = g.a_axis_stride == 1 && ((uintptr_t)g.a % 16 == 0);
+    for (int d = 0; d < g.ndim && vec; ++d) vec = g.a_stride[d] % V == 0;
+    const dim3 grid((unsigned)bx);
+    if (op == AM_RED_MAX) {
+      if (vec) hipLaunchKernelGGL((argreduce_row<T, true, true>), grid, block, 0, stream(), g);
+      else hipLaunchKernelGGL((argreduce_row<T, true, false>), grid, block, 0, stream(), g);
+    } else {
+      if (vec) hipLaunchKernelGGL((argreduce_row<T, false, true>), grid, block, 0, stream(), g);
+      else hipLaunchKernelGGL((argreduce_row<T, false, false>), grid, block, 0, stream(), g);
+    }
   } else {
+    // too few outputs to fill the chip: cut the axis (eight workgroups per CU, at least 64 slices per chunk)
+    const int64_t want = (int64_t)num_cus() * 8;
+    if (bx < want && g.L >= 128) {
+      int64_t chunks = (want + bx - 1) / bx;
+      if (chunks > g.L / 64) chunks = g.L / 64;
+      if (chunks > 1024) chunks = 1024;
+      const int64_t len = (g.L + chunks - 1) / chunks;
+      chunks = (g.L + len - 1) / len;
+      const size_t val_bytes = ((size_t)chunks * (size_t)g.outputs * sizeof(T) + 255) / 256 * 256;
+      char* base = chunks > 1 ? (char*)gemm::splitk_workspace(val_bytes + (size_t)chunks * (size_t)g.outputs * sizeof(int64_t)) : nullptr;
+      if (base) { g.chunks = (int)chunks; g.chunk_len = len; g.ws_val = (T*)base; g.ws_idx = (int64_t*)(base + val_bytes); }
+    }
+    const dim3 grid((unsigned)bx, (unsigned)g.chunks);
     if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_seq<T, true>), grid, block, 0, stream(), g);
     else hipLaunchKernelGGL((argreduce_seq<T, false>), grid, block, 0, stream(), g);
+    if (g.chunks > 1) {
+      AM_TRY(check_launch("argreduce"));
+      if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_merge<T, true>), dim3((unsigned)bx), block, 0, stream(), g);
+      else hipLaunchKernelGGL((argreduce_merge<T, false>), dim3((unsigned)bx), block, 0, stream(), g);
+    }
   }
   return check_launch("argreduce");
 }
@@ -807,16 +888,17 @@ static int maxpool(const char* fn, int64_t N, int C, int H, int W, int kH, int k
 // src/arraymancer/nn_primitives/nnp_maxpooling.nim:68-83). Run as a gather so that nothing races: one
 // lane per input element looks through the windows that contain it, highest output index first, and
 // takes the first whose recorded maximum is this element.
-template <typename T>
+template <typename T, typename IDX>
 __global__ __launch_bounds__(256) void maxpool2d_backward(const int64_t* argmax, const T* grad_out, T* grad_in, int64_t total,
                                                           int H, int W, int kH, int kW, int padH, int padW, int sH, int sW,
                                                           int outH, int outW) {
-  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (p >= total) return;
-  const int col = (int)(p % W);
-  const int64_t t = p / W;
-  const int row = (int)(t % H);
-  const int64_t nc = t / H;
+  const int64_t p64 = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (p64 >= total) return;
+  const IDX p = (IDX)p64;             // 32-bit index arithmetic whenever the tensor allows it
+  const int col = (int)(p % (IDX)W);
+  const IDX t = p / (IDX)W;
+  const int row = (int)(t % (IDX)H);
+  const IDX nc = t / (IDX)H;
   // windows h with h * sH - padH <= row < h * sH - padH + kH
   const int rh = row + padH, rw = col + padW;
   int h_hi = rh / sH, w_hi = rw / sW;
@@ -828,9 +910,47 @@ __global__ __launch_bounds__(256) void maxpool2d_backward(const int64_t* argmax,
   for (int h = h_hi; h >= h_lo && !found; --h)
     for (int w = w_hi; w >= w_lo; --w) {
       const int64_t o = w + (int64_t)outW * (h + (int64_t)outH * nc);
-      if (argmax[o] == p) { g = grad_out[o]; found = true; break; }
+      if (argmax[o] == p64) { g = grad_out[o]; found = true; break; }
     }
-  grad_in[p] = g;
+  grad_in[p64] = g;
+}
+
+// Windows two wide with stride two and no padding in width (W a multiple of the 16-byte vector): a lane
+// owns V consecutive input columns, i.e. V / 2 windows per candidate row of windows, read and written
+// as vectors.
+template <typename T>
+__global__ __launch_bounds__(256) void maxpool2d_backward_w2(const int64_t* argmax, const T* grad_out, T* grad_in,
+                                                             uint32_t total_vec, int H, int Wv, int kH, int padH, int sH,
+                                                             int outH) {
+  constexpr int V = 16 / (int)sizeof(T), NO = V / 2;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  typedef T go_t __attribute__((ext_vector_type(NO)));
+  typedef int64_t ix_t __attribute__((ext_vector_type(NO)));
+  const uint32_t q = blockIdx.x * 256u + threadIdx.x;
+  if (q >= total_vec) return;
+  const uint32_t cv = q % (uint32_t)Wv, t = q / (uint32_t)Wv;
+  const int row = (int)(t % (uint32_t)H);
+  const uint32_t nc = t / (uint32_t)H;
+  const int64_t p0 = (int64_t)q * V;               // flat index of the lane's first input element
+  const int outW = Wv * NO;
+  const int rh = row + padH;
+  int h_hi = rh / sH;
+  const int h_lo = rh - kH + 1 <= 0 ? 0 : (rh - kH + sH) / sH;
+  if (h_hi > outH - 1) h_hi = outH - 1;
+  vec_t g;
+  bool found[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) { g[e] = (T)0; found[e] = false; }
+  for (int h = h_hi; h >= h_lo; --h) {
+    const int64_t o = (int64_t)cv * NO + (int64_t)outW * (h + (int64_t)outH * nc);
+    const ix_t ix = *(const ix_t*)(argmax + o);
+    const go_t go = *(const go_t*)(grad_out + o);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      if (!found[e] && ix[e / 2] == p0 + e) { g[e] = go[e / 2]; found[e] = true; }
+    }
+  }
+  *(vec_t*)(grad_in + p0) = g;
 }
 
 template <typename T>
@@ -844,10 +964,22 @@ static int maxpool_backward(const char* fn, int64_t N, int C, int H, int W, int 
   if (total == 0) return AM_OK;
   if (!argmax || !grad_out || !grad_in) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
   AM_TRY(ensure_init());
+  constexpr int64_t V = 16 / (int64_t)sizeof(T);
+  if (kW == 2 && sW == 2 && padW == 0 && W % (2 * V) == 0 && total / V < ((int64_t)1 << 32) && (uintptr_t)argmax % 16 == 0 &&
+      (uintptr_t)grad_out % 16 == 0 && (uintptr_t)grad_in % 16 == 0) {
+    const int64_t total_vec = total / V;
+    hipLaunchKernelGGL((maxpool2d_backward_w2<T>), dim3((unsigned)((total_vec + 255) / 256)), dim3(256), 0, stream(), argmax,
+                       grad_out, grad_in, (uint32_t)total_vec, H, (int)(W / V), kH, padH, sH, (int)outH);
+    return check_launch("maxpool2d_backward_w2");
+  }
   const int64_t bx = (total + 255) / 256;
   if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many input elements", fn);
-  hipLaunchKernelGGL((maxpool2d_backward<T>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in, total, H, W,
-                     kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
+  if (total < ((int64_t)1 << 32))
+    hipLaunchKernelGGL((maxpool2d_backward<T, uint32_t>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in,
+                       total, H, W, kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
+  else
+    hipLaunchKernelGGL((maxpool2d_backward<T, uint64_t>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in,
+                       total, H, W, kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
   return check_launch("maxpool2d_backward");
 }
 

@@ -213,6 +213,13 @@ def test_argmax_nan_rules(hip, oracle, sfx):
         wi, wv = oracle.argreduce(op, x, 1)
         assert np.array_equal(gi.toCpu(), wi) and np.array_equal(gv.toCpu(), wv, equal_nan=True)
     rng = np.random.default_rng(seed_of("argmax-nan", sfx))
+    z = rng.standard_normal((2000, 1100)).astype(dt)     # many outputs, long axis: the walk is cut into chunks
+    z[0, 0] = nan; z[1:, 1] = nan; z[::7, 2] = nan; z[:, 3] = nan; z[0, 4] = 99; z[63:70, 5] = nan; z[1000:, 6] = nan; z[:1000, 7] = nan
+    z[0, 7] = -99
+    for op, fn in (("max", hip.argmax_max), ("min", hip.argmin_min)):
+        gi, gv = fn(hip.toHip(z), 0)
+        wi, wv = oracle.argreduce(op, z, 0)
+        assert np.array_equal(gi.toCpu(), wi) and np.array_equal(gv.toCpu(), wv, equal_nan=True), op
     y = rng.standard_normal((6, 1000)).astype(dt)
     y[0, 0] = nan; y[1, 500] = nan; y[2, ::3] = nan; y[3, 1:] = nan; y[4, :] = nan; y[5, 64] = nan; y[5, 0] = y[5].max()
     for v, dv in ((y, hip.toHip(y)), (y.T, hip.toHip(np.ascontiguousarray(y.T)))):
