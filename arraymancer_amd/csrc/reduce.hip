@@ -86,8 +86,8 @@ __global__ __launch_bounds__(256) void reduce_seq(Args<T> p) {
   int64_t l = l0 + 1;
   // four loads in flight, folded in axis order
   for (; l + 4 <= l1; l += 4) {
-    const T v0 = p.a[a_off + l * p.a_axis_stride], v1 = p.a[a_off + (l + 1) * p.a_axis_stride];
-    const T v2 = p.a[a_off + (l + 2) * p.a_axis_stride], v3 = p.a[a_off + (l + 3) * p.a_axis_stride];
+    const T v0 = __builtin_nontemporal_load(p.a + a_off + l * p.a_axis_stride), v1 = __builtin_nontemporal_load(p.a + a_off + (l + 1) * p.a_axis_stride);
+    const T v2 = __builtin_nontemporal_load(p.a + a_off + (l + 2) * p.a_axis_stride), v3 = __builtin_nontemporal_load(p.a + a_off + (l + 3) * p.a_axis_stride);
     acc = Fold<T, OP>::apply(acc, v0);
     acc = Fold<T, OP>::apply(acc, v1);
     acc = Fold<T, OP>::apply(acc, v2);
@@ -98,6 +98,8 @@ __global__ __launch_bounds__(256) void reduce_seq(Args<T> p) {
   else p.dst[d_off] = acc;
 }
 
+// (Column walks load non-temporally: measured 10 % faster, also when the tensor would fit the memory-side
+// cache; the wavefront-per-output kernels are faster with ordinary loads.)
 // The same walk with one lane per 16 bytes of adjacent outputs (the innermost output dimension has
 // unit stride in the source and the destination): 16-byte loads, eight in flight, every output
 // still folded front to back along the axis, so the results are those of reduce_seq bit for bit.
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(256) void reduce_seq_vec(Args<T> p) {
   for (; l + U <= l1; l += U) {
     vec_t x[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) x[u] = *(const vec_t*)(src + (l + u) * p.a_axis_stride);
+    for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load((const vec_t*)(src + (l + u) * p.a_axis_stride));
 #pragma unroll
     for (int u = 0; u < U; ++u) fold(x[u]);
   }
@@ -149,7 +151,7 @@ __device__ __forceinline__ void wave_fold(T& acc, bool& has) {
   }
 }
 
-template <typename T, int OP, bool VEC>
+template <typename T, int OP, bool VEC, bool STREAM>
 __global__ __launch_bounds__(256) void reduce_row(Args<T> p) {
   constexpr int V = 16 / (int)sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(V)));
@@ -176,7 +178,13 @@ __global__ __launch_bounds__(256) void reduce_row(Args<T> p) {
     const int64_t nvec = (l1 - l0) / V;
     int64_t v = lane;
     for (; v + 192 < nvec; v += 256) {   // four 16-byte loads in flight per lane
-      const vec_t x0 = src[v], x1 = src[v + 64], x2 = src[v + 128], x3 = src[v + 192];
+      vec_t x0, x1, x2, x3;
+      if constexpr (STREAM) {   // a template parameter: a run-time branch is merged back into ordinary loads
+        x0 = __builtin_nontemporal_load(src + v); x1 = __builtin_nontemporal_load(src + v + 64);
+        x2 = __builtin_nontemporal_load(src + v + 128); x3 = __builtin_nontemporal_load(src + v + 192);
+      } else {
+        x0 = src[v]; x1 = src[v + 64]; x2 = src[v + 128]; x3 = src[v + 192];
+      }
       take_vec(x0); take_vec(x1); take_vec(x2); take_vec(x3);
     }
     for (; v < nvec; v += 64) take_vec(src[v]);
@@ -227,6 +235,9 @@ static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
     if (chunks > 8192) chunks = 8192;
   }
   g.chunks = 1; g.chunk_len = g.L; g.ws = nullptr;
+  // 8192 x 8192 f64 row sums: 98 us with ordinary loads, 88 us with non-temporal ones; at half the size
+  // (which the 256 MB memory-side cache can hold from the producing kernel) it is the other way round
+  const bool stream_loads = (double)g.outputs * (double)g.L * sizeof(T) > 384.0 * 1024 * 1024;
   if (chunks > 1) {
     int64_t len = (g.L + chunks - 1) / chunks;
     len = (len + V - 1) / V * V;                    // chunk starts stay 16-byte aligned
@@ -240,8 +251,9 @@ static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
     const int64_t bx = (g.outputs * g.chunks + 3) / 4;
     if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "reduce: too many output elements");
     const dim3 grid((unsigned)bx), block(256);
-    if (vec) hipLaunchKernelGGL((reduce_row<T, OP, true>), grid, block, 0, stream(), g);
-    else hipLaunchKernelGGL((reduce_row<T, OP, false>), grid, block, 0, stream(), g);
+    if (vec && stream_loads) hipLaunchKernelGGL((reduce_row<T, OP, true, true>), grid, block, 0, stream(), g);
+    else if (vec) hipLaunchKernelGGL((reduce_row<T, OP, true, false>), grid, block, 0, stream(), g);
+    else hipLaunchKernelGGL((reduce_row<T, OP, false, false>), grid, block, 0, stream(), g);
   } else if (seq_vec) {
     const int64_t bx = (g.outputs / V + 255) / 256;
     hipLaunchKernelGGL((reduce_seq_vec<T, OP>), dim3((unsigned)bx, (unsigned)g.chunks), dim3(256), 0, stream(), g);
@@ -260,7 +272,7 @@ static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
     r.chunks = 1; r.chunk_len = r.L; r.ws = nullptr;
     if (g.outputs < 1024 && g.chunks >= 64) {   // few outputs, many partials: a wavefront per output
       const int64_t bx = (g.outputs + 3) / 4;
-      hipLaunchKernelGGL((reduce_row<T, OP, false>), dim3((unsigned)bx), dim3(256), 0, stream(), r);
+      hipLaunchKernelGGL((reduce_row<T, OP, false, false>), dim3((unsigned)bx), dim3(256), 0, stream(), r);
     } else if (seq_vec) {   // the partials are laid out like the outputs, so the same test holds for them
       const int64_t bx = (g.outputs / V + 255) / 256;
       hipLaunchKernelGGL((reduce_seq_vec<T, OP>), dim3((unsigned)bx, 1), dim3(256), 0, stream(), r);
@@ -448,8 +460,8 @@ __global__ __launch_bounds__(256) void argreduce_seq(ArgArgs<T> p) {
   };
   int64_t l = l0 + 1;
   for (; l + 4 <= l1; l += 4) {   // four loads in flight, compared in axis order
-    const T v0 = src[l * p.a_axis_stride], v1 = src[(l + 1) * p.a_axis_stride];
-    const T v2 = src[(l + 2) * p.a_axis_stride], v3 = src[(l + 3) * p.a_axis_stride];
+    const T v0 = __builtin_nontemporal_load(src + l * p.a_axis_stride), v1 = __builtin_nontemporal_load(src + (l + 1) * p.a_axis_stride);
+    const T v2 = __builtin_nontemporal_load(src + (l + 2) * p.a_axis_stride), v3 = __builtin_nontemporal_load(src + (l + 3) * p.a_axis_stride);
     take(v0, l); take(v1, l + 1); take(v2, l + 2); take(v3, l + 3);
   }
   for (; l < l1; ++l) take(src[l * p.a_axis_stride], l);
