@@ -101,7 +101,7 @@ struct SplitArgs {
 
 // The 32 (mn) x 128 (k) tile at (mn0, k0) of operand op, 16 elements per lane of a 256-lane workgroup:
 // every load is issued before f(mn, k, value) sees the first element (zeros outside the operand).
-template <typename T, typename F>
+template <typename T, bool STREAM, typename F>
 __device__ __forceinline__ void visit_tile(const SplitArgs<T>& a, int op, int64_t mn0, int64_t k0, F&& f) {
   constexpr int VEC = 16 / (int)sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
@@ -118,7 +118,7 @@ __device__ __forceinline__ void visit_tile(const SplitArgs<T>& a, int op, int64_
       const int mn = t / KV + i * ROWS;
       const T* src = X + (mn0 + mn) * ld_mn + (k0 + k);
       if ((mn0 + mn) < MN && (k0 + k + VEC) <= K) {
-        v[i] = *(const vec_t*)src;
+        if constexpr (STREAM) v[i] = __builtin_nontemporal_load((const vec_t*)src); else v[i] = *(const vec_t*)src;
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v[i][e] = ((mn0 + mn) < MN && (k0 + k + e) < K) ? src[e] : (T)0;
@@ -137,7 +137,7 @@ __device__ __forceinline__ void visit_tile(const SplitArgs<T>& a, int op, int64_
       const int k = t / MV + i * ROWS;
       const T* src = X + (mn0 + mn) + (k0 + k) * ld_k;
       if ((k0 + k) < K && (mn0 + mn + VEC) <= MN) {
-        v[i] = *(const vec_t*)src;
+        if constexpr (STREAM) v[i] = __builtin_nontemporal_load((const vec_t*)src); else v[i] = *(const vec_t*)src;
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v[i][e] = ((k0 + k) < K && (mn0 + mn + e) < MN) ? src[e] : (T)0;
@@ -177,7 +177,7 @@ __device__ __forceinline__ void visit_tile(const SplitArgs<T>& a, int op, int64_
 //                  the second pass then leaves at once and the operand has been read only once.
 //   FIRST = false: writes the marked planes above plane 0 (nothing if there is none, or if the product
 //                  has more live digit pairs than max_pairs and therefore runs on the vector ALU).
-template <typename T, bool FIRST>
+template <typename T, bool FIRST, bool STREAM_LOADS = false>
 __global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
   constexpr int ND = (int)sizeof(T);
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void split_digits(SplitArgs<T> a) {
     }
   }
   U seen = 0;   // byte d: OR of the digits d of this lane's elements
-  visit_tile<T>(a, op, mn0, k0, [&](int mn, int k, T x) {
+  visit_tile<T, FIRST && STREAM_LOADS>(a, op, mn0, k0, [&](int mn, int k, T x) {
     if constexpr (FIRST) {
       const U y = balanced_digits<T>(x);
       seen |= y;
@@ -650,7 +650,11 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
   }
   const int64_t stiles = (Mp + Np) / 32 * (Kp / 128), smax = (int64_t)num_cus() * 16;
   const dim3 sgrid((unsigned)(stiles < smax ? stiles : smax));
-  hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
+  // Operands beyond what the memory-side cache may still hold from their producer are read with non-temporal
+  // loads (int64 4096^3, 256 MiB of operands: first pass 65 -> 46 us); smaller ones are faster with ordinary loads.
+  const bool stream_loads = (double)(g.M + g.N) * (double)g.K * sizeof(T) > 192.0 * 1024 * 1024;
+  if (stream_loads) hipLaunchKernelGGL((split_digits<T, true, true>), sgrid, dim3(256), 0, stream(), sp);
+  else hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
   // with at most one live pair allowed there is nothing above plane 0 that could be needed
   if (max_pairs >= 2) hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
   DigitArgs<T> d;
