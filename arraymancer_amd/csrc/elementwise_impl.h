@@ -146,6 +146,14 @@ template <typename T> struct GenericArgs {
   int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK];
 };
 
+// Hides a pointer's origin from the optimiser (no instruction is emitted); the result is typed as a pointer to
+// global memory, which the optimiser can no longer infer for it.
+template <typename P> __device__ __forceinline__ const __attribute__((address_space(1))) P* launder(const P* ptr) {
+  auto g = (const __attribute__((address_space(1))) P*)ptr;
+  asm("" : "+v"(g));
+  return g;
+}
+
 template <typename T, int CODE, int AK, int BK, bool SWAP>
 __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
   typedef typename Traits<T>::V V;
@@ -180,14 +188,29 @@ __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
     V av[kUnroll], bv[kUnroll];
     bool full[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t col = col0 + (int64_t)u * kThreads * VEC;
-      full[u] = (col + VEC <= p.L);
-      if (full[u]) {
-        if constexpr (AK == kVecOperand)
-          av[u] = p.a_stream ? __builtin_nontemporal_load((const V*)(arow + col)) : *(const V*)(arow + col);
-        if constexpr (BK == kVecOperand)
-          bv[u] = p.b_stream ? __builtin_nontemporal_load((const V*)(brow + col)) : *(const V*)(brow + col);
+    for (int u = 0; u < kUnroll; ++u) full[u] = (col0 + (int64_t)u * kThreads * VEC + VEC <= p.L);
+    // One branch per operand around its loads: a select between a non-temporal and an ordinary load of the
+    // same address is merged into an ordinary load by the compiler, hence also the laundered pointer.
+    if constexpr (AK == kVecOperand) {
+      if (p.a_stream) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          if (full[u]) av[u] = __builtin_nontemporal_load(launder((const V*)(arow + col0 + (int64_t)u * kThreads * VEC)));
+      } else {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          if (full[u]) av[u] = *(const V*)(arow + col0 + (int64_t)u * kThreads * VEC);
+      }
+    }
+    if constexpr (BK == kVecOperand) {
+      if (p.b_stream) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          if (full[u]) bv[u] = __builtin_nontemporal_load(launder((const V*)(brow + col0 + (int64_t)u * kThreads * VEC)));
+      } else {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          if (full[u]) bv[u] = *(const V*)(brow + col0 + (int64_t)u * kThreads * VEC);
       }
     }
 #pragma unroll
@@ -513,6 +536,14 @@ static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const 
     if (c.sb[d] != 0) r.b_stream = 1;
   }
   if (in == 0) { r.a_stream = 1; r.b_stream = 1; }
+  // Non-temporal loads pay once the operands read once exceed what the 256 MB memory-side cache can still hold
+  // from the kernel that produced them (f32 8192 x 8192: X + Y 142 -> 128 us); below that ordinary loads are
+  // faster (copy of one 256 MB operand: 63 us against 87 us).
+  {
+    const double operand_bytes = (double)rows * (double)L * sizeof(T);
+    const int streamed = (ia == 1 ? r.a_stream : 0) + (!BCONST && ib == 1 ? r.b_stream : 0);
+    if (!(streamed * operand_bytes > 384.0 * 1024 * 1024)) { r.a_stream = 0; r.b_stream = 0; }
+  }
   for (int d = 0; d < kMaxOuter; ++d) {
     r.oshape[d] = d < in ? c.shape[d] : 1;
     r.od[d] = d < in ? c.sd[d] : 0;
