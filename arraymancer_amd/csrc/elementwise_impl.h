@@ -154,6 +154,12 @@ template <typename P> __device__ __forceinline__ const __attribute__((address_sp
   return g;
 }
 
+// An ordinary or a non-temporal 16-byte load, as two branches (see ew_rows).
+template <typename V> __device__ __forceinline__ V load_as(bool keep, const V* ptr) {
+  if (keep) return *ptr;
+  return __builtin_nontemporal_load(launder(ptr));
+}
+
 template <typename T, int CODE, int AK, int BK, bool SWAP>
 __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
   typedef typename Traits<T>::V V;
@@ -336,7 +342,8 @@ template <typename T> struct TriArgs {
   uint32_t tiles_per_row, total_tiles;
   int rank;           // collapsed rank (generic) / number of outer dims (rows)
   int a_const, b_const, c_const;   // rows kernel: operand has inner stride 0 (one value per row)
-  int a_keep, b_keep, c_keep;      // rows kernel: the same row is re-read for every output row: cached loads
+  int a_keep, b_keep, c_keep;      // rows kernel: ordinary loads (a row re-read for every output row, or operands small
+                                   // enough for the memory-side cache); 0 = non-temporal loads
   int64_t shape[AM_MAXRANK];
   int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK], sc[AM_MAXRANK];
 };
@@ -371,9 +378,9 @@ __global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
       const int64_t col = col0 + (int64_t)u * kThreads * VEC;
       if (col + VEC <= p.L) {
         V av, bv, cv;
-        if (p.a_const) { for (int e = 0; e < VEC; ++e) av[e] = arow[0]; } else av = p.a_keep ? *(const V*)(arow + col) : __builtin_nontemporal_load((const V*)(arow + col));
-        if (p.b_const) { for (int e = 0; e < VEC; ++e) bv[e] = brow[0]; } else bv = p.b_keep ? *(const V*)(brow + col) : __builtin_nontemporal_load((const V*)(brow + col));
-        if (p.c_const) { for (int e = 0; e < VEC; ++e) cv[e] = crow[0]; } else cv = p.c_keep ? *(const V*)(crow + col) : __builtin_nontemporal_load((const V*)(crow + col));
+        if (p.a_const) { for (int e = 0; e < VEC; ++e) av[e] = arow[0]; } else av = load_as(p.a_keep != 0, (const V*)(arow + col));
+        if (p.b_const) { for (int e = 0; e < VEC; ++e) bv[e] = brow[0]; } else bv = load_as(p.b_keep != 0, (const V*)(brow + col));
+        if (p.c_const) { for (int e = 0; e < VEC; ++e) cv[e] = crow[0]; } else cv = load_as(p.c_keep != 0, (const V*)(crow + col));
         V r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) r[e] = TriOp<T, OP>::apply(av[e], bv[e], cv[e]);
@@ -704,6 +711,10 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
   if (ok && rows > 1 && L < tile / 8) ok = false;
   if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31))) ok = false;
   g.n = n; g.L = L;
+  {  // same rule as the two-operand kernel: non-temporal loads only when the operands read once exceed 384 MiB
+    const int streamed = (!g.a_const && !g.a_keep) + (!g.b_const && !g.b_keep) + (!g.c_const && !g.c_keep);
+    if (!(streamed * (double)rows * (double)L * sizeof(T) > 384.0 * 1024 * 1024)) g.a_keep = g.b_keep = g.c_keep = 1;
+  }
   if (ok) {
     g.rank = in;
     g.tiles_per_row = (uint32_t)tiles_per_row;
