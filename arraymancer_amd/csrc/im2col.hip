@@ -37,6 +37,38 @@ __global__ __launch_bounds__(256) void im2col_kernel(Im2colArgs p, const T* __re
   }
 }
 
+// One lane per 16 bytes of one row of the column matrix (V consecutive output pixels of one (n, c)):
+// 32-bit index arithmetic, five divisions per lane instead of seven 64-bit ones per element, one
+// 16-byte store. Needs H_out * W_out to be a multiple of V and fewer than 2^32 vectors.
+template <typename T, bool STREAM>
+__global__ __launch_bounds__(256) void im2col_vec(Im2colArgs p, const T* __restrict__ in, T* __restrict__ col, uint32_t total_vec) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const uint32_t Pv = (uint32_t)(p.Hout * p.Wout) / V;
+  const uint32_t CK = (uint32_t)(p.C * p.kH * p.kW);
+  for (uint32_t q = blockIdx.x * 256u + threadIdx.x; q < total_vec; q += gridDim.x * 256u) {
+    const uint32_t rid = q / Pv, pv = q - rid * Pv;          // row of the column matrix over all images, vector in it
+    const uint32_t n = rid / CK, c = rid - n * CK;
+    const uint32_t ck = c / (uint32_t)p.kW;
+    const int w_off = (int)(c - ck * (uint32_t)p.kW) - p.padW;
+    const uint32_t c_off = ck / (uint32_t)p.kH;
+    const int h_off = (int)(ck - c_off * (uint32_t)p.kH) - p.padH;
+    const uint32_t pix0 = pv * V;
+    int h = (int)(pix0 / (uint32_t)p.Wout), w = (int)(pix0 - (uint32_t)h * (uint32_t)p.Wout);
+    const T* __restrict__ base = in + (int64_t)n * p.in_n + (int64_t)c_off * p.in_c;
+    vec_t v;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const int row = h_off + h * p.strideH, cc = w_off + w * p.strideW;
+      v[e] = (row >= 0 && cc >= 0 && row < p.H && cc < p.W) ? base[(int64_t)row * p.in_h + (int64_t)cc * p.in_w] : (T)0;
+      if (++w == p.Wout) { w = 0; ++h; }
+    }
+    // a column matrix beyond the memory-side cache is written past it; a smaller one stays there for the GEMM
+    if constexpr (STREAM) __builtin_nontemporal_store(v, (vec_t*)(col + (int64_t)q * V));
+    else *(vec_t*)(col + (int64_t)q * V) = v;
+  }
+}
+
 template <typename T>
 int im2col(const char* fn, int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH,
            int strideW, const T* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, T* col) {
@@ -52,8 +84,19 @@ int im2col(const char* fn, int64_t N, int C, int H, int W, int kH, int kW, int p
   a.C = C; a.H = H; a.W = W; a.kH = kH; a.kW = kW; a.padH = padH; a.padW = padW;
   a.strideH = strideH; a.strideW = strideW; a.Hout = Hout; a.Wout = Wout;
   a.in_n = in_n; a.in_c = in_c; a.in_h = in_h; a.in_w = in_w;
-  int64_t blocks = (a.total + 255) / 256;
+  constexpr int64_t V = 16 / (int64_t)sizeof(T);
   const int64_t cap = (int64_t)num_cus() * 32;
+  if (((int64_t)Hout * Wout) % V == 0 && a.total / V < ((int64_t)1 << 32) && (int64_t)C * kH * kW < ((int64_t)1 << 31) &&
+      (uintptr_t)col % 16 == 0) {
+    int64_t blocks = (a.total / V + 255) / 256;
+    if (blocks > cap) blocks = cap;
+    if ((double)a.total * sizeof(T) > 384.0 * 1024 * 1024)
+      hipLaunchKernelGGL((im2col_vec<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream(), a, in, col, (uint32_t)(a.total / V));
+    else
+      hipLaunchKernelGGL((im2col_vec<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream(), a, in, col, (uint32_t)(a.total / V));
+    return check_launch("im2col");
+  }
+  int64_t blocks = (a.total + 255) / 256;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL((im2col_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), a, in, col);
   return check_launch("im2col");

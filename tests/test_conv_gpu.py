@@ -43,6 +43,8 @@ GEOMS = [  # N, C, H, W, C_out, kH, kW, pad, stride
     (8, 3, 16, 16, 8, 5, 5, (2, 2), (1, 1)),
     (64, 1, 28, 28, 20, 5, 5, (0, 0), (1, 1)),      # MNIST conv1 of the reference's example (24 x 24 = 576 outputs)
     (16, 20, 12, 12, 50, 5, 5, (0, 0), (1, 1)),     # conv2 (8 x 8 = 64 outputs)
+    (2, 3, 4, 8, 2, 3, 3, (0, 0), (1, 1)),          # 2 x 6 outputs: 16-byte groups of pixels straddle the output rows
+    (4, 2, 16, 16, 3, 3, 3, (1, 1), (2, 2)),        # stride 2 with padding, 8 x 8 outputs
 ]
 
 
