@@ -18,7 +18,7 @@
  * Op codes are AM_RED_* of include/am_hip.h.
  *
  * Pinned by tests/test_oracle_reduce.py against the reference's literal vectors
- * (tests/tensor/test_aggregate.nim:20-215, tests/nn_primitives/test_nnp_maxpool.nim:20-31) and
+ * (tests/tensor/test_aggregate.nim:20-215, tests/nn_primitives/test_nnp_maxpool.nim:20-45) and
  * against NumPy / exact rational arithmetic on random strided inputs. Softmax has no vector in the
  * reference's tests: it is pinned on the closed form exp(x) / sum(exp(x)) in extended precision,
  * on shift invariance and on rows summing to one.

@@ -12,11 +12,15 @@
  *   private/p_accessors.nim:378-413    dualStridedIteration (the per-operand walk)
  *   operators_broadcasted.nim:28-194, operators_blas_l1.nim:44-136   the operator bodies
  *   nn_primitives/nnp_activation.nim:35-36, private/p_activation.nim:17-18   relu, sigmoid
+ *   nn_primitives/nnp_activation.nim:61-74   relu / sigmoid / tanh backward bodies
+ *   ufunc.nim:91, math_functions.nim:218-222, aggregate.nim:115-146   sqrt, square, square(y - mean)
  * Op codes are those of include/am_hip.h (AM_OP_*, AM_UOP_*).
  *
  * Pinned by tests/test_oracle_map.py against the reference's literal vectors
  * (tests/tensor/test_broadcasting.nim, test_operators_blas.nim:294-303, test_higherorder.nim)
- * and against NumPy broadcasting / as_strided on random shapes and strides.
+ * and against NumPy broadcasting / as_strided on random shapes and strides. The backward bodies, sqrt,
+ * square and the squared difference have no vector in the reference's tests: each is a short sequence of
+ * separately rounded IEEE (or ring) operations and is held bit for bit to NumPy evaluating the same sequence.
  * Unpinned (no run of the reference possible, Nim stdlib absent): NaN / -0 behaviour of
  * Nim's `max` inside relu; the (0 >= x) ? 0 : x form is adopted.
  */
