@@ -26,6 +26,14 @@ def test_header_and_binding_agree():
     assert sorted(_lib.SIGNATURES) == syms
 
 
+def test_nim_and_cpp_host_layers_bind_every_declared_symbol():
+    """nim/hip_abi.nim imports each entry point the header declares; the C++ host layer includes the header itself."""
+    nim = open(os.path.join(ROOT, "nim", "hip_abi.nim")).read()
+    for s in declared_symbols():
+        assert re.search(rf"\bproc {s}\*\(", nim), f"{s} has no importc declaration in nim/hip_abi.nim"
+    assert '#include "am_hip.h"' in open(os.path.join(ROOT, "include", "am_hip_tensor.hpp")).read()
+
+
 def test_library_exports_every_declared_symbol():
     L = ctypes.CDLL(_lib.LIB_PATH)
     for s in declared_symbols():
