@@ -143,17 +143,58 @@ __global__ __launch_bounds__(256) void gemv_cols(GemvArgs<T> p) {
 }
 
 // Per-workgroup partial dot products, one slot each, in the workspace.
-template <typename T>
+template <typename T, bool VECLOAD, bool STREAM>
 __global__ __launch_bounds__(256) void dot_partial(int64_t n, const T* x, int64_t incx, const T* y, int64_t incy, T* ws) {
   typedef typename Acc<T>::type U;
+  typedef typename VecTraits<T>::vec_t vec_t;
+  constexpr int VEC = VecTraits<T>::VK;
   __shared__ U part[4];
   U acc = 0;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
-    acc += (U)x[i * incx] * (U)y[i * incy];
+  if constexpr (VECLOAD) {   // unit strides, 16-byte aligned: two 16-byte loads per vector and lane, two vectors in flight
+    const int64_t nvec = n / VEC, stride = (int64_t)gridDim.x * 256;
+    U acc1 = 0;
+    int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (; v + stride < nvec; v += 2 * stride) {
+      vec_t x0, y0, x1, y1;
+      if constexpr (STREAM) {   // vectors beyond the memory-side cache
+        x0 = __builtin_nontemporal_load((const vec_t*)x + v); y0 = __builtin_nontemporal_load((const vec_t*)y + v);
+        x1 = __builtin_nontemporal_load((const vec_t*)x + v + stride); y1 = __builtin_nontemporal_load((const vec_t*)y + v + stride);
+      } else {
+        x0 = *((const vec_t*)x + v); y0 = *((const vec_t*)y + v);
+        x1 = *((const vec_t*)x + v + stride); y1 = *((const vec_t*)y + v + stride);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { acc += (U)x0[e] * (U)y0[e]; acc1 += (U)x1[e] * (U)y1[e]; }
+    }
+    for (; v < nvec; v += stride) {
+      const vec_t x0 = *((const vec_t*)x + v), y0 = *((const vec_t*)y + v);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc += (U)x0[e] * (U)y0[e];
+    }
+    acc += acc1;
+    for (int64_t i = nvec * VEC + (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) acc += (U)x[i] * (U)y[i];
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+      acc += (U)x[i * incx] * (U)y[i * incy];
+  }
   acc = wave_sum<U>(acc);
   if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
   __syncthreads();
   if (threadIdx.x == 0) ws[blockIdx.x] = (T)(part[0] + part[1] + part[2] + part[3]);
+}
+
+// The per-workgroup partials into one value: a lane adds every 256th partial, then the lanes are combined
+// in a fixed order (one thread walking a thousand partials costs 20 us of dependent loads).
+template <typename T>
+__global__ __launch_bounds__(256) void dot_final(int count, const T* ws, T* out) {
+  typedef typename Acc<T>::type U;
+  __shared__ U part[4];
+  U acc = 0;
+  for (int i = threadIdx.x; i < count; i += 256) acc += (U)ws[i];
+  acc = wave_sum<U>(acc);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) *out = (T)(part[0] + part[1] + part[2] + part[3]);
 }
 
 template <typename T>
@@ -232,18 +273,18 @@ int dot(const char* fn, int64_t n, const T* x, int64_t incx, const T* y, int64_t
   int64_t blocks = (n + 1023) / 1024;
   const int64_t cap = (int64_t)num_cus() * 4;
   if (blocks > cap) blocks = cap;
+  const bool vec = incx == 1 && incy == 1 && aligned16(x) && aligned16(y);
+  const bool stream_loads = 2.0 * (double)n * sizeof(T) > 384.0 * 1024 * 1024;
   T* ws = (T*)splitk_workspace((size_t)(blocks + 1) * sizeof(T));
   if (!ws) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
-  hipLaunchKernelGGL((dot_partial<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), n, x, incx, y, incy, ws);
+  const dim3 grid((unsigned)blocks), block(256);
+  if (vec && stream_loads) hipLaunchKernelGGL((dot_partial<T, true, true>), grid, block, 0, stream(), n, x, incx, y, incy, ws);
+  else if (vec) hipLaunchKernelGGL((dot_partial<T, true, false>), grid, block, 0, stream(), n, x, incx, y, incy, ws);
+  else hipLaunchKernelGGL((dot_partial<T, false, false>), grid, block, 0, stream(), n, x, incx, y, incy, ws);
   AM_TRY(check_launch("dot_partial"));
-  Args<T> r;
-  memset(&r, 0, sizeof(r));
-  r.M = 1; r.N = 1; r.K = n; r.alpha = (T)1; r.beta = (T)0; r.C = ws + blocks; r.c_m = 1; r.c_n = 1;
-  r.epilogue = AM_EPI_NONE; r.splits = (int)blocks; r.ws = ws;
-  AM_TRY((launch_splitk_reduce<T, U>(r)));
-  AM_HIP_TRY(hipMemcpyAsync(result, ws + blocks, sizeof(T), hipMemcpyDeviceToHost, stream()));
-  AM_HIP_TRY(hipStreamSynchronize(stream()));
-  return AM_OK;
+  hipLaunchKernelGGL((dot_final<T>), dim3(1), block, 0, stream(), (int)blocks, ws, ws + blocks);
+  AM_TRY(check_launch("dot_final"));
+  return fetch_result(result, ws + blocks, sizeof(T));
 }
 
 }  // namespace

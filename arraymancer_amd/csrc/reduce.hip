@@ -272,7 +272,9 @@ static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
     r.chunks = 1; r.chunk_len = r.L; r.ws = nullptr;
     if (g.outputs < 1024 && g.chunks >= 64) {   // few outputs, many partials: a wavefront per output
       const int64_t bx = (g.outputs + 3) / 4;
-      hipLaunchKernelGGL((reduce_row<T, OP, false, false>), dim3((unsigned)bx), dim3(256), 0, stream(), r);
+      // a single output: its partials are one run of memory, read 16 bytes per lane
+      if (g.outputs == 1 && (uintptr_t)r.a % 16 == 0) hipLaunchKernelGGL((reduce_row<T, OP, true, false>), dim3((unsigned)bx), dim3(256), 0, stream(), r);
+      else hipLaunchKernelGGL((reduce_row<T, OP, false, false>), dim3((unsigned)bx), dim3(256), 0, stream(), r);
     } else if (seq_vec) {   // the partials are laid out like the outputs, so the same test holds for them
       const int64_t bx = (g.outputs / V + 255) / 256;
       hipLaunchKernelGGL((reduce_seq_vec<T, OP>), dim3((unsigned)bx, 1), dim3(256), 0, stream(), r);
@@ -404,9 +406,7 @@ static int reduce_all(const char* fn, int op, int rank, const int64_t* shape, co
     r.a = tmp; r.L = rows; r.a_axis_stride = 1;
     AM_TRY(dispatch<T>(op, r, r.L >= 64, 256 + tmp_bytes));
   }
-  AM_HIP_TRY(hipMemcpyAsync(result, out, sizeof(T), hipMemcpyDeviceToHost, stream()));
-  AM_HIP_TRY(hipStreamSynchronize(stream()));
-  return AM_OK;
+  return fetch_result(result, out, sizeof(T));
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -220,6 +220,21 @@ int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
   return AM_OK;
 }
 
+}  // extern "C"
+
+namespace am {
+int fetch_result(void* host_dst, const void* dev_src, size_t bytes) {
+  static void* pinned = nullptr;
+  if (bytes > 256) return fail(AM_E_ARG, "fetch_result: %zu bytes", bytes);
+  if (!pinned) AM_HIP_TRY(hipHostMalloc(&pinned, 256, hipHostMallocDefault));
+  AM_HIP_TRY(hipMemcpyAsync(pinned, dev_src, bytes, hipMemcpyDeviceToHost, g_stream));
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  memcpy(host_dst, pinned, bytes);
+  return AM_OK;
+}
+}  // namespace am
+
+extern "C" {
 int am_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return AM_OK;
   if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_d2h: null pointer");
