@@ -48,6 +48,31 @@ __device__ __forceinline__ double dev_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float dev_tanh(float x) { return tanhf(x); }
 __device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
 
+// The reference's tests compare `^.` results with == (tests/tensor/test_broadcasting.nim:130-146), and the
+// host's powf is correctly rounded in all but rare cases while the device's is not exact even for 2^19.
+// Evaluated in double and rounded once, the float result is the correctly rounded one except where the
+// exact value lies within 2^-52 (relative) of a rounding boundary.
+__device__ __forceinline__ float dev_pow(float x, float y) { return (float)pow((double)x, (double)y); }
+__device__ __forceinline__ double dev_pow(double x, double y) { return pow(x, y); }
+
+// The C math library's function for a universal-function op code (tensor/ufunc.nim:82-130), in
+// the precision of T. Only instantiated for float and double.
+template <int UOP, typename T> __device__ __forceinline__ T dev_math(T x) {
+#define AM_MATH1(code, fn) \
+  if constexpr (UOP == code) { if constexpr (std::is_same<T, float>::value) return fn##f(x); else return fn(x); } else
+  AM_MATH1(AM_UOP_LN, log) AM_MATH1(AM_UOP_LOG10, log10) AM_MATH1(AM_UOP_LOG2, log2)
+  AM_MATH1(AM_UOP_SIN, sin) AM_MATH1(AM_UOP_COS, cos) AM_MATH1(AM_UOP_TAN, tan)
+  AM_MATH1(AM_UOP_SINH, sinh) AM_MATH1(AM_UOP_COSH, cosh)
+  AM_MATH1(AM_UOP_ARCSIN, asin) AM_MATH1(AM_UOP_ARCCOS, acos) AM_MATH1(AM_UOP_ARCTAN, atan)
+  AM_MATH1(AM_UOP_ARCSINH, asinh) AM_MATH1(AM_UOP_ARCCOSH, acosh) AM_MATH1(AM_UOP_ARCTANH, atanh)
+  AM_MATH1(AM_UOP_CBRT, cbrt) AM_MATH1(AM_UOP_ERF, erf) AM_MATH1(AM_UOP_ERFC, erfc)
+  AM_MATH1(AM_UOP_GAMMA, tgamma) AM_MATH1(AM_UOP_LGAMMA, lgamma)
+  AM_MATH1(AM_UOP_FLOOR, floor) AM_MATH1(AM_UOP_CEIL, ceil) AM_MATH1(AM_UOP_TRUNC, trunc)
+  AM_MATH1(AM_UOP_ROUND, round)
+  { static_assert(UOP == AM_UOP_RECIPROCAL, "not a universal-function op code"); return (T)1 / x; }
+#undef AM_MATH1
+}
+
 // ---- binary op bodies. Integer arithmetic is carried out in the unsigned twin so that it wraps.
 template <typename T, int OP> struct BinOp {
   typedef typename Traits<T>::U U;
@@ -85,6 +110,8 @@ template <typename T, int OP> struct BinOp {
     } else if constexpr (OP == AM_OP_TANH_BWD) {
       if constexpr (Traits<T>::kFloat) return y * ((T)1 - x * x);
       else return (T)((U)y * ((U)1 - (U)x * (U)x));
+    } else if constexpr (OP == AM_OP_POW) {
+      if constexpr (Traits<T>::kFloat) return dev_pow(x, y); else return x;   // never dispatched for integers
     } else {  // AM_OP_SQDIFF
       if constexpr (Traits<T>::kFloat) { const T d = x - y; return d * d; }
       else { const U d = (U)x - (U)y; return (T)(d * d); }
@@ -108,6 +135,9 @@ template <typename T, int UOP> struct UnOp {
       if constexpr (Traits<T>::kFloat) return dev_sqrt(x); else return x;   // never dispatched for integers
     } else if constexpr (UOP == AM_UOP_SQUARE) {
       if constexpr (Traits<T>::kFloat) return x * x; else return (T)((U)x * (U)x);
+    }
+    else if constexpr (UOP >= AM_UOP_LN) {
+      if constexpr (Traits<T>::kFloat) return dev_math<UOP>(x); else return x;   // never dispatched for integers
     }
     else {  // ABS
       if constexpr (Traits<T>::kFloat) return __builtin_fabs(x);
@@ -610,6 +640,9 @@ static int binary(const char* fn, int op, int rank, const int64_t* shape, T* dst
     case AM_OP_ADD_TANH:
       if constexpr (F) return run<T, AM_OP_ADD_TANH, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
       else return fail(AM_E_DTYPE, "%s: add_tanh is defined for float tensors only", fn);
+    case AM_OP_POW:
+      if constexpr (F) return run<T, AM_OP_POW, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
+      else return fail(AM_E_DTYPE, "%s: pow is defined for float tensors only", fn);
     default:
       return fail(AM_E_ARG, "%s: unknown op %d", fn, op);
   }
@@ -635,6 +668,9 @@ static int scalar(const char* fn, int op, int left, int rank, const int64_t* sha
     case AM_OP_MOD:
       if constexpr (!F) return scalar_lr<T, AM_OP_MOD>(left != 0, rank, shape, dst, sd, a, sa, s);
       else return fail(AM_E_DTYPE, "%s: mod is defined for integer tensors only", fn);
+    case AM_OP_POW:
+      if constexpr (F) return scalar_lr<T, AM_OP_POW>(left != 0, rank, shape, dst, sd, a, sa, s);
+      else return fail(AM_E_DTYPE, "%s: pow is defined for float tensors only", fn);
     default:
       return fail(AM_E_ARG, "%s: op %d has no tensor-scalar form", fn, op);
   }
@@ -661,6 +697,16 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
     case AM_UOP_SQRT:
       if constexpr (F) return run<T, kUnaryBase + AM_UOP_SQRT, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
       else return fail(AM_E_DTYPE, "%s: sqrt is defined for float tensors only", fn);
+#define AM_CASE(code) \
+    case code: \
+      if constexpr (F) return run<T, kUnaryBase + code, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0); \
+      else return fail(AM_E_DTYPE, "%s: unary op %d is defined for float tensors only", fn, op)
+    AM_CASE(AM_UOP_LN); AM_CASE(AM_UOP_LOG10); AM_CASE(AM_UOP_LOG2); AM_CASE(AM_UOP_SIN); AM_CASE(AM_UOP_COS);
+    AM_CASE(AM_UOP_TAN); AM_CASE(AM_UOP_SINH); AM_CASE(AM_UOP_COSH); AM_CASE(AM_UOP_ARCSIN); AM_CASE(AM_UOP_ARCCOS);
+    AM_CASE(AM_UOP_ARCTAN); AM_CASE(AM_UOP_ARCSINH); AM_CASE(AM_UOP_ARCCOSH); AM_CASE(AM_UOP_ARCTANH);
+    AM_CASE(AM_UOP_CBRT); AM_CASE(AM_UOP_ERF); AM_CASE(AM_UOP_ERFC); AM_CASE(AM_UOP_GAMMA); AM_CASE(AM_UOP_LGAMMA);
+    AM_CASE(AM_UOP_FLOOR); AM_CASE(AM_UOP_CEIL); AM_CASE(AM_UOP_TRUNC); AM_CASE(AM_UOP_ROUND); AM_CASE(AM_UOP_RECIPROCAL);
+#undef AM_CASE
     default:
       return fail(AM_E_ARG, "%s: unknown unary op %d", fn, op);
   }

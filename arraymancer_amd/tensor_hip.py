@@ -229,6 +229,14 @@ class HipTensor:
     def bc_idiv(self, other):
         return _bc_inplace("div", self, other)
 
+    def bc_ipow(self, exponent):
+        """`^.=`: in-place pow(x, exponent), float tensors, scalar exponent
+        (src/arraymancer/tensor/operators_broadcasted.nim:178-182)."""
+        _float_scalar("^.=", self, exponent)
+        if self.size:
+            _scalar_into("pow", self, self, exponent, False)
+        return self
+
 
 # ---------------------------------------------------------------------- construction
 def empty(shape: Sequence[int], dtype) -> HipTensor:
@@ -585,6 +593,24 @@ def bc_div(a, b): return _bc_or_scalar("div", a, b)
 def bc_mod(a, b): return _bc_or_scalar("mod", a, b)
 
 
+def bc_pow(a, b):
+    """`^.`: tensor ^. scalar = pow(x, exponent), scalar ^. tensor = pow(base, x); float tensors
+    only, one operand a scalar (src/arraymancer/tensor/operators_broadcasted.nim:153-161)."""
+    ta, tb = isinstance(a, HipTensor), isinstance(b, HipTensor)
+    if ta == tb:
+        raise TypeError("`^.` takes one tensor and one scalar")
+    t, s = (a, b) if ta else (b, a)
+    _float_scalar("^.", t, s)
+    return scalar_op("pow", t, s, scalar_on_left=tb)
+
+
+def _float_scalar(name, t: HipTensor, scalar):
+    if t.dtype.kind != "f":
+        raise TypeError(f"{name} is defined for float tensors only")
+    if isinstance(scalar, HipTensor):
+        raise TypeError(f"{name} takes a scalar")
+
+
 def _bc_or_scalar(op, a, b):
     """`+.` and friends: tensor-tensor with implicit broadcasting, tensor-scalar, scalar-tensor
     (src/arraymancer/tensor/operators_broadcasted.nim:28-60, 107-161)."""
@@ -658,8 +684,42 @@ def tanh_backward(gradient: HipTensor, cached_tensor: HipTensor) -> HipTensor:
 
 
 OPERATORS = {"+.": bc_add, "-.": bc_sub, "*.": bc_mul, "/.": bc_div, "mod": bc_mod,
+             "^.": bc_pow,
              "+.=": HipTensor.bc_iadd, "-.=": HipTensor.bc_isub, "*.=": HipTensor.bc_imul,
-             "/.=": HipTensor.bc_idiv}
+             "/.=": HipTensor.bc_idiv, "^.=": HipTensor.bc_ipow}
+
+
+# The universal functions of src/arraymancer/tensor/ufunc.nim:82-130 (makeUniversal: map_inline of
+# the math library's function of the same name) and reciprocal (math_functions.nim:52-58).
+UFUNCS = ("ln", "log10", "log2", "exp", "sqrt", "cbrt", "sin", "cos", "tan", "sinh", "cosh", "tanh",
+          "arcsin", "arccos", "arctan", "arcsinh", "arccosh", "arctanh", "erf", "erfc", "gamma", "lgamma",
+          "floor", "ceil", "trunc", "round", "reciprocal")
+
+
+def _make_ufunc(name):
+    def f(t: HipTensor) -> HipTensor:
+        if t.dtype.kind != "f":
+            raise TypeError(f"{name} is defined for float tensors only")
+        return unary(name, t)
+    f.__name__ = name
+    f.__doc__ = f"Element-wise {name} of a float tensor (src/arraymancer/tensor/ufunc.nim:56-130)."
+    return f
+
+
+ln, log10, log2, exp, cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, arcsinh, arccosh, arctanh, \
+    erf, erfc, gamma, lgamma, floor, ceil, trunc, reciprocal = (_make_ufunc(n) for n in (
+        "ln", "log10", "log2", "exp", "cbrt", "sin", "cos", "tan", "sinh", "cosh", "arcsin", "arccos", "arctan",
+        "arcsinh", "arccosh", "arctanh", "erf", "erfc", "gamma", "lgamma", "floor", "ceil", "trunc", "reciprocal"))
+tround = _make_ufunc("round")
+
+
+def mreciprocal(t: HipTensor) -> HipTensor:
+    """In-place 1 / x (src/arraymancer/tensor/math_functions.nim:56-58)."""
+    if t.dtype.kind != "f":
+        raise TypeError("mreciprocal is defined for float tensors only")
+    if t.size:
+        _unary_into("reciprocal", t, t)
+    return t
 
 
 # ---------------------------------------------------------------- reductions, softmax, pooling

@@ -249,7 +249,8 @@ int am_hip_dot_i64(int64_t n, const int64_t* x, int64_t incx, const int64_t* y, 
 #define AM_OP_SIGMOID_BWD 11  /* a * (1 - a) * b   a = cached sigmoid output (nnp_activation.nim:61-63)  */
 #define AM_OP_TANH_BWD   12   /* b * (1 - a * a)   a = cached tanh output    (nnp_activation.nim:72-74)  */
 #define AM_OP_SQDIFF     13   /* (a - b) * (a - b): the fold body of variance (tensor/aggregate.nim:115-146) */
-#define AM_OP_BINARY_COUNT 14
+#define AM_OP_POW        14   /* floats only: pow(a, b); `^.` and `^.=` (operators_broadcasted.nim:153-161, 178-182) */
+#define AM_OP_BINARY_COUNT 15
 
 int am_hip_ew_binary_f32(int op, int rank, const int64_t* shape,
                          float* dst, const int64_t* dst_strides,
@@ -269,7 +270,7 @@ int am_hip_ew_binary_i64(int op, int rank, const int64_t* shape,
                          const int64_t* b, const int64_t* b_strides);
 
 /* dst[i] = scalar_on_left ? op(scalar, a[i]) : op(a[i], scalar); ops AM_OP_ADD..AM_OP_MOD,
- * AM_OP_MAX, AM_OP_MIN. Replaces the tensor-scalar forms
+ * AM_OP_MAX, AM_OP_MIN, AM_OP_POW (`t ^. exponent`, `base ^. t`). Replaces the tensor-scalar forms
  *   src/arraymancer/tensor/operators_broadcasted.nim:107-194, operators_blas_l1.nim:66-136
  * (GPU precedent: cuda_apply_rscal / _lscal / _scal, incl_higher_order_cuda.nim:121-229).
  * dst may alias a exactly (the in-place `+.=`, `*=` ... forms). */
@@ -299,7 +300,36 @@ int am_hip_ew_scalar_i64(int op, int scalar_on_left, int rank, const int64_t* sh
 #define AM_UOP_ABS     6
 #define AM_UOP_SQRT    7   /* floats only: IEEE square root (tensor/ufunc.nim:91)        */
 #define AM_UOP_SQUARE  8   /* x * x (tensor/math_functions.nim:218-222); integers wrap   */
-#define AM_UOP_COUNT   9
+/* The universal functions of tensor/ufunc.nim:82-130 (map_inline of the C math library's
+ * function of the same name) and `reciprocal` (tensor/math_functions.nim:52-58). Floats only.
+ * The device math library evaluates the transcendental ones: a few units in the last place from
+ * the host's libm, not the same bits. floor / ceil / trunc / round (half away from zero) and
+ * reciprocal (one IEEE division) are exact. */
+#define AM_UOP_LN          9
+#define AM_UOP_LOG10      10
+#define AM_UOP_LOG2       11
+#define AM_UOP_SIN        12
+#define AM_UOP_COS        13
+#define AM_UOP_TAN        14
+#define AM_UOP_SINH       15
+#define AM_UOP_COSH       16
+#define AM_UOP_ARCSIN     17
+#define AM_UOP_ARCCOS     18
+#define AM_UOP_ARCTAN     19
+#define AM_UOP_ARCSINH    20
+#define AM_UOP_ARCCOSH    21
+#define AM_UOP_ARCTANH    22
+#define AM_UOP_CBRT       23
+#define AM_UOP_ERF        24
+#define AM_UOP_ERFC       25
+#define AM_UOP_GAMMA      26   /* the gamma function itself (C tgamma) */
+#define AM_UOP_LGAMMA     27
+#define AM_UOP_FLOOR      28
+#define AM_UOP_CEIL       29
+#define AM_UOP_TRUNC      30
+#define AM_UOP_ROUND      31   /* halfway cases away from zero (C round) */
+#define AM_UOP_RECIPROCAL 32   /* 1 / x */
+#define AM_UOP_COUNT      33
 int am_hip_ew_unary_f32(int op, int rank, const int64_t* shape,
                         float* dst, const int64_t* dst_strides,
                         const float* a, const int64_t* a_strides);

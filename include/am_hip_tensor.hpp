@@ -15,6 +15,8 @@
 //   s * t, t * s, t / s               same
 //   a +. b, a -. b, a *. b, a /. b    am::bc_add / bc_sub / bc_mul / bc_div   (also tensor-scalar)
 //   a +.= b ...                       a.bc_iadd(b) / bc_isub / bc_imul / bc_idiv
+//   t ^. e, b ^. t, t ^.= e           am::bc_pow(t, e), am::bc_pow(b, t), t.bc_ipow(e)
+//   ln(t), cos(t), floor(t) ...       am::ln(t), am::cos(t), am::floor(t) ...
 //   t.transpose, t[a..b|s, ...]       t.transpose(), t.slice(axis, first, last, step)
 //   t.broadcast(shape)                t.broadcast(shape)
 // Errors: std::invalid_argument where the reference raises ValueError, std::out_of_range where it
@@ -245,6 +247,8 @@ class HipTensor {
   HipTensor& bc_isub(const HipTensor& b) { return apply2(AM_OP_SUB, b.broadcast(shape)); }
   HipTensor& bc_imul(const HipTensor& b) { return apply2(AM_OP_MUL, b.broadcast(shape)); }
   HipTensor& bc_idiv(const HipTensor& b) { return apply2(AM_OP_DIV, b.broadcast(shape)); }
+  // `^.=`: pow(x, exponent) in place, float tensors (operators_broadcasted.nim:178-182)
+  HipTensor& bc_ipow(T exponent) { return apply_scalar(AM_OP_POW, exponent); }
 
   // apply2_inline (higher_order_applymap.nim:40-47) with an enumerated body.
   HipTensor& apply2(int op, const HipTensor& src) {
@@ -341,6 +345,22 @@ template <typename T> HipTensor<T> bc_mul(const HipTensor<T>& t, T s) { return s
 template <typename T> HipTensor<T> bc_mul(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_MUL, t, s, true); }
 template <typename T> HipTensor<T> bc_div(const HipTensor<T>& t, T s) { return scalar_op(AM_OP_DIV, t, s); }
 template <typename T> HipTensor<T> bc_div(T s, const HipTensor<T>& t) { return scalar_op(AM_OP_DIV, t, s, true); }
+// `^.`: tensor ^. exponent and base ^. tensor, float tensors (operators_broadcasted.nim:153-161)
+template <typename T> HipTensor<T> bc_pow(const HipTensor<T>& t, T exponent) { return scalar_op(AM_OP_POW, t, exponent); }
+template <typename T> HipTensor<T> bc_pow(T base, const HipTensor<T>& t) { return scalar_op(AM_OP_POW, t, base, true); }
+// The universal functions (ufunc.nim:82-130) and reciprocal (math_functions.nim:52-58), float tensors.
+#define AM_HIP_UFUNC(name, code) \
+  template <typename T> HipTensor<T> name(const HipTensor<T>& t) { return unary(code, t); }
+AM_HIP_UFUNC(ln, AM_UOP_LN) AM_HIP_UFUNC(log10, AM_UOP_LOG10) AM_HIP_UFUNC(log2, AM_UOP_LOG2) AM_HIP_UFUNC(exp, AM_UOP_EXP)
+AM_HIP_UFUNC(sin, AM_UOP_SIN) AM_HIP_UFUNC(cos, AM_UOP_COS) AM_HIP_UFUNC(tan, AM_UOP_TAN)
+AM_HIP_UFUNC(sinh, AM_UOP_SINH) AM_HIP_UFUNC(cosh, AM_UOP_COSH) AM_HIP_UFUNC(tanh, AM_UOP_TANH)
+AM_HIP_UFUNC(arcsin, AM_UOP_ARCSIN) AM_HIP_UFUNC(arccos, AM_UOP_ARCCOS) AM_HIP_UFUNC(arctan, AM_UOP_ARCTAN)
+AM_HIP_UFUNC(arcsinh, AM_UOP_ARCSINH) AM_HIP_UFUNC(arccosh, AM_UOP_ARCCOSH) AM_HIP_UFUNC(arctanh, AM_UOP_ARCTANH)
+AM_HIP_UFUNC(cbrt, AM_UOP_CBRT) AM_HIP_UFUNC(erf, AM_UOP_ERF) AM_HIP_UFUNC(erfc, AM_UOP_ERFC)
+AM_HIP_UFUNC(gamma, AM_UOP_GAMMA) AM_HIP_UFUNC(lgamma, AM_UOP_LGAMMA)
+AM_HIP_UFUNC(floor, AM_UOP_FLOOR) AM_HIP_UFUNC(ceil, AM_UOP_CEIL) AM_HIP_UFUNC(trunc, AM_UOP_TRUNC)
+AM_HIP_UFUNC(round, AM_UOP_ROUND) AM_HIP_UFUNC(reciprocal, AM_UOP_RECIPROCAL)
+#undef AM_HIP_UFUNC
 // map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass
 template <typename T> HipTensor<T> bias_relu(const HipTensor<T>& x, const HipTensor<T>& b) { return map2(AM_OP_ADD_RELU, x, b.broadcast(x.shape)); }
 // Activation backward passes: map2_inline(cached_tensor, gradient) bodies of nnp_activation.nim:61-74.

@@ -146,9 +146,14 @@ proc am_hip_gemm_ex_f64*(M, N, K: int64, alpha: cdouble, A: ptr cdouble, rsA, cs
 type
   AmBinaryOp* {.size: sizeof(cint).} = enum
     opAdd = 0, opSub = 1, opMul = 2, opDiv = 3, opMod = 4, opAddRelu = 5, opAddSigmoid = 6,
-    opAddTanh = 7, opReluBwd = 8, opMax = 9, opMin = 10, opSigmoidBwd = 11, opTanhBwd = 12, opSqDiff = 13
+    opAddTanh = 7, opReluBwd = 8, opMax = 9, opMin = 10, opSigmoidBwd = 11, opTanhBwd = 12, opSqDiff = 13,
+    opPow = 14
   AmUnaryOp* {.size: sizeof(cint).} = enum
-    uopCopy = 0, uopNeg = 1, uopRelu = 2, uopSigmoid = 3, uopTanh = 4, uopExp = 5, uopAbs = 6, uopSqrt = 7, uopSquare = 8
+    uopCopy = 0, uopNeg = 1, uopRelu = 2, uopSigmoid = 3, uopTanh = 4, uopExp = 5, uopAbs = 6, uopSqrt = 7, uopSquare = 8,
+    uopLn = 9, uopLog10 = 10, uopLog2 = 11, uopSin = 12, uopCos = 13, uopTan = 14, uopSinh = 15, uopCosh = 16,
+    uopArcsin = 17, uopArccos = 18, uopArctan = 19, uopArcsinh = 20, uopArccosh = 21, uopArctanh = 22, uopCbrt = 23,
+    uopErf = 24, uopErfc = 25, uopGamma = 26, uopLgamma = 27, uopFloor = 28, uopCeil = 29, uopTrunc = 30,
+    uopRound = 31, uopReciprocal = 32
 
 proc am_hip_ew_binary_f32*(op: cint, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
                            a: ptr cfloat, a_strides: ptr int64, b: ptr cfloat, b_strides: ptr int64): cint {.importc.}

@@ -258,6 +258,54 @@ proc `/.`*[T](s: T, t: HipTensor[T]): HipTensor[T] =
   result = newHipTensor[T](t.shape)
   if result.size > 0: ewScalar(T, opDiv, true, result, t, s)
 
+proc `^.`*[T: float32 | float64](t: HipTensor[T], exponent: T): HipTensor[T] =
+  ## operators_broadcasted.nim:153-156
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opPow, false, result, t, exponent)
+proc `^.`*[T: float32 | float64](base: T, t: HipTensor[T]): HipTensor[T] =
+  ## operators_broadcasted.nim:158-161
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opPow, true, result, t, base)
+proc `^.=`*[T: float32 | float64](t: var HipTensor[T], exponent: T) =
+  ## operators_broadcasted.nim:178-182
+  if t.size > 0: ewScalar(T, opPow, false, t, t, exponent)
+
+template makeHipUniversal(name: untyped, code: AmUnaryOp) =
+  ## The device twin of makeUniversal (ufunc.nim:56-68): `name` applied element-wise.
+  proc name*[T: float32 | float64](t: HipTensor[T]): HipTensor[T] =
+    result = newHipTensor[T](t.shape)
+    if result.size > 0: ewUnary(T, code, result, t)
+
+makeHipUniversal(ln, uopLn)
+makeHipUniversal(log10, uopLog10)
+makeHipUniversal(log2, uopLog2)
+makeHipUniversal(exp, uopExp)
+makeHipUniversal(sin, uopSin)
+makeHipUniversal(cos, uopCos)
+makeHipUniversal(tan, uopTan)
+makeHipUniversal(sinh, uopSinh)
+makeHipUniversal(cosh, uopCosh)
+makeHipUniversal(tanh, uopTanh)
+makeHipUniversal(arcsin, uopArcsin)
+makeHipUniversal(arccos, uopArccos)
+makeHipUniversal(arctan, uopArctan)
+makeHipUniversal(arcsinh, uopArcsinh)
+makeHipUniversal(arccosh, uopArccosh)
+makeHipUniversal(arctanh, uopArctanh)
+makeHipUniversal(cbrt, uopCbrt)
+makeHipUniversal(erf, uopErf)
+makeHipUniversal(erfc, uopErfc)
+makeHipUniversal(gamma, uopGamma)
+makeHipUniversal(lgamma, uopLgamma)
+makeHipUniversal(floor, uopFloor)
+makeHipUniversal(ceil, uopCeil)
+makeHipUniversal(trunc, uopTrunc)
+makeHipUniversal(round, uopRound)
+makeHipUniversal(reciprocal, uopReciprocal)   # math_functions.nim:52-54
+proc mreciprocal*[T: float32 | float64](t: var HipTensor[T]) =
+  ## math_functions.nim:56-58
+  if t.size > 0: ewUnary(T, uopReciprocal, t, t)
+
 proc relu*[T: float32 | float64](t: HipTensor[T]): HipTensor[T] =
   result = newHipTensor[T](t.shape)
   if result.size > 0: ewUnary(T, uopRelu, result, t)

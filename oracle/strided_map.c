@@ -14,6 +14,8 @@
  *   nn_primitives/nnp_activation.nim:35-36, private/p_activation.nim:17-18   relu, sigmoid
  *   nn_primitives/nnp_activation.nim:61-74   relu / sigmoid / tanh backward bodies
  *   ufunc.nim:91, math_functions.nim:218-222, aggregate.nim:115-146   sqrt, square, square(y - mean)
+ *   ufunc.nim:82-130, math_functions.nim:52-58, operators_broadcasted.nim:153-182
+ *                                      the universal functions (this host's libm), reciprocal, `^.`
  * Op codes are those of include/am_hip.h (AM_OP_*, AM_UOP_*).
  *
  * Pinned by tests/test_oracle_map.py against the reference's literal vectors
@@ -21,6 +23,10 @@
  * and against NumPy broadcasting / as_strided on random shapes and strides. The backward bodies, sqrt,
  * square and the squared difference have no vector in the reference's tests: each is a short sequence of
  * separately rounded IEEE (or ring) operations and is held bit for bit to NumPy evaluating the same sequence.
+ * The universal functions and pow are this host's libm, which is what the reference's map_inline bodies call:
+ * pinned on the reference's literals (test_ufunc.nim:38-44 cos / ln, test_broadcasting.nim:130-146 `^.`,
+ * test_math_functions.nim:20-30 reciprocal), on NumPy's own evaluation within 2 units in the last place, and
+ * on closed forms (floor / ceil / trunc / round on halves and integers, gamma at integers, erf + erfc = 1).
  * Unpinned (no run of the reference possible, Nim stdlib absent): NaN / -0 behaviour of
  * Nim's `max` inside relu; the (0 >= x) ? 0 : x form is adopted.
  */
@@ -86,6 +92,7 @@ static inline void iter_advance(strided_iter* it) {
 #define F_EXP expf
 #define F_TANH tanhf
 #define F_SQRT sqrtf
+#define F_M(name) name##f
 #include "strided_map_impl.inc"
 #undef T
 #undef UT
@@ -94,6 +101,7 @@ static inline void iter_advance(strided_iter* it) {
 #undef F_EXP
 #undef F_TANH
 #undef F_SQRT
+#undef F_M
 
 #define T double
 #define UT double
@@ -102,6 +110,7 @@ static inline void iter_advance(strided_iter* it) {
 #define F_EXP exp
 #define F_TANH tanh
 #define F_SQRT sqrt
+#define F_M(name) name
 #include "strided_map_impl.inc"
 #undef T
 #undef UT
@@ -110,6 +119,7 @@ static inline void iter_advance(strided_iter* it) {
 #undef F_EXP
 #undef F_TANH
 #undef F_SQRT
+#undef F_M
 
 #define T int32_t
 #define UT uint32_t

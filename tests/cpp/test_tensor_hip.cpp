@@ -153,6 +153,37 @@ static void variance_std() {
   CHECK(eq(am::square(toHip<int32_t>({-3, 65536, 7}, {3})), {9, 0, 49}));
 }
 
+static void pow_and_universal_functions() {
+  // tests/tensor/test_broadcasting.nim:130-146, 340-362: `^.`, `^.=`
+  auto a = toHip<double>({1, 10, 20, 30}, {4, 1});
+  CHECK(eq(am::bc_pow(a, 2.0), {1, 100, 400, 900}));
+  auto inv = am::bc_pow(a, -1.0).toCpu();
+  auto p2 = am::bc_pow(2.0, a).toCpu();
+  const double want_inv[4] = {1.0, 1.0 / 10.0, 1.0 / 20.0, 1.0 / 30.0};
+  const double want_p2[4] = {2.0, 1024.0, 1048576.0, 1073741824.0};
+  for (int i = 0; i < 4; ++i) {
+    CHECK(std::fabs(inv[i] - want_inv[i]) <= 4e-16 * want_inv[i]);
+    CHECK(std::fabs(p2[i] - want_p2[i]) <= 4e-16 * want_p2[i]);
+  }
+  auto b = a.clone();
+  b.bc_ipow(2.0);
+  CHECK(eq(b, {1, 100, 400, 900}));
+  // tests/tensor/test_math_functions.nim:20-45: reciprocal is one IEEE division
+  CHECK(eq(am::reciprocal(a), {1.0, 1.0 / 10.0, 1.0 / 20.0, 1.0 / 30.0}));
+  // tests/tensor/test_ufunc.nim:31-44: cos and ln against the scalar functions
+  auto c = am::cos(toHip<double>({1, 2, 3, 4, 5, 6}, {2, 3})).toCpu();
+  auto l = am::ln(toHip<double>({7, 8, 9, 10, 11, 12}, {3, 2})).toCpu();
+  for (int i = 0; i < 6; ++i) {
+    CHECK(std::fabs(c[i] - std::cos(1.0 + i)) <= 1e-15);
+    CHECK(std::fabs(l[i] - std::log(7.0 + i)) <= 1e-15);
+  }
+  CHECK(eq(am::floor(toHip<float>({-1.5f, -0.5f, 0.5f, 2.0f}, {4})), {-2, -1, 0, 2}));
+  CHECK(eq(am::ceil(toHip<float>({-1.5f, -0.5f, 0.5f, 2.0f}, {4})), {-1, -0.0f, 1, 2}));
+  CHECK(eq(am::trunc(toHip<float>({-1.5f, -0.5f, 0.5f, 2.0f}, {4})), {-1, -0.0f, 0, 2}));
+  CHECK(eq(am::round(toHip<float>({-1.5f, -0.5f, 0.5f, 2.5f}, {4})), {-2, -1, 1, 3}));
+  EXPECT_THROW(am::unary(AM_UOP_LN, toHip<int32_t>({1, 2}, {2})), std::invalid_argument);
+}
+
 static void argmax_argmin() {
   // tests/tensor/test_aggregate.nim:112-119, 158-166
   auto a = toHip<int32_t>({0, 4, 7, 1, 9, 5, 3, 4, 1}, {3, 3});
@@ -286,6 +317,7 @@ int main(int argc, char** argv) {
     broadcasting<int64_t>();
     fused_linear();
     variance_std();
+    pow_and_universal_functions();
     argmax_argmin();
     maxpool_backward();
     aggregates<float>();

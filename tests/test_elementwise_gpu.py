@@ -388,3 +388,138 @@ def test_activation_backward(hip, oracle, sfx):
         assert np.allclose(num, hip.sigmoid_backward(dg, s).toCpu(), rtol=1e-6, atol=1e-9)
         num = (hip.tanh(up).toCpu() - hip.tanh(dn).toCpu()) / (2 * h) * g
         assert np.allclose(num, hip.tanh_backward(dg, t).toCpu(), rtol=1e-6, atol=1e-9)
+
+
+# ------------------------------------------------------------------ `^.` and the universal functions
+_UFUNC_DOMAIN = dict(ln=(1e-3, 1e3), log10=(1e-3, 1e3), log2=(1e-3, 1e3), arcsin=(-1, 1), arccos=(-1, 1),
+                     arccosh=(1, 50), arctanh=(-0.999, 0.999), sinh=(-20, 20), cosh=(-20, 20), gamma=(-3.9, 12),
+                     lgamma=(-3.9, 30), cbrt=(-1e3, 1e3))
+_EXACT_UFUNCS = ("floor", "ceil", "trunc", "round", "reciprocal", "sqrt")
+# Units in the last place allowed between the device math library and the host's libm (both are a few
+# ulp from the true value; the reference's result is the host libm's).
+_UFUNC_ULPS = dict(gamma=16, lgamma=16, erfc=8, tan=8)
+
+
+def test_reference_pow_and_ufunc_vectors(hip, vectors):
+    """The reference's literals for `^.`, `^.=`, reciprocal, cos and ln. The reference compares pow
+    results with ==; the device pow is held to 2 units in the last place here, and the cases whose
+    result the device also hits exactly are asserted as such."""
+    import math
+    v = vectors["pow_and_ufunc"]
+    a = np.array(v["a"])
+    da = hip.toHip(a)
+    quot = np.array([[n / q] for n, q in v["pow_m1_as_quotients"]])
+    say("pow literals")
+    assert np.array_equal(hip.OPERATORS["^."](da, 2.0).toCpu(), np.array(v["pow_2"]))
+    np.testing.assert_allclose(hip.OPERATORS["^."](da, -1.0).toCpu(), quot, rtol=2 ** -51, atol=0)
+    np.testing.assert_allclose(hip.OPERATORS["^."](2.0, da).toCpu(), np.array(v["two_pow_a"]), rtol=2 ** -51, atol=0)
+    b = da.clone()
+    assert hip.OPERATORS["^.="](b, 2.0) is b
+    assert np.array_equal(b.toCpu(), np.array(v["pow_2"]))
+    assert np.array_equal(hip.reciprocal(da).toCpu(), quot)
+    c = da.clone()
+    hip.mreciprocal(c)
+    assert np.array_equal(c.toCpu(), quot)
+    ci, li = np.array(v["cos_input"]), np.array(v["ln_input"])
+    assert np.abs(hip.cos(hip.toHip(ci)).toCpu() - np.vectorize(math.cos)(ci)).mean() <= 1e-15
+    np.testing.assert_allclose(hip.ln(hip.toHip(li)).toCpu(), np.vectorize(math.log)(li), rtol=2 ** -52, atol=0)
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_universal_functions(hip, oracle, sfx):
+    """Every function of tensor/ufunc.nim against the oracle (the host's libm, which the reference
+    calls): exact for the rounding functions and reciprocal, within a few units in the last place for
+    the device math library's transcendental ones; contiguous, transposed and column-slice operands."""
+    dt = DTYPES[sfx]
+    ulp = np.finfo(dt).eps
+    rng = np.random.default_rng(seed_of(sfx, "ufunc"))
+    for name in hip.UFUNCS:
+        lo, hi = _UFUNC_DOMAIN.get(name, (-8, 8))
+        if name == "sqrt":
+            lo, hi = 0, 1e6
+        a = rng.uniform(lo, hi, (96, 1030)).astype(dt)
+        da = hip.toHip(a)
+        say("ufunc", sfx, name)
+        want = oracle.unary(name, a)
+        got = getattr(hip, name if name != "round" else "round")(da).toCpu()
+        got_t = hip.unary(name, da.transpose()).toCpu()
+        got_s = hip.unary(name, da[:, 3:900]).toCpu()
+        if name in _EXACT_UFUNCS:
+            assert np.array_equal(got, want), name
+        else:
+            floor = 1.0 if name == "lgamma" else float(np.finfo(dt).tiny)
+            tol = _UFUNC_ULPS.get(name, 4) * ulp * np.maximum(np.abs(want), floor)
+            err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+            assert np.all(err <= tol), (name, float((err / tol).max()))
+        # the same kernel body whatever the strides: transposed and sliced operands give the same bits
+        assert np.array_equal(got_t, got.T, equal_nan=True), name
+        assert np.array_equal(got_s, got[:, 3:900], equal_nan=True), name
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_rounding_functions_special_values(hip, sfx):
+    dt = DTYPES[sfx]
+    x = np.array([-2.5, -1.5, -0.5, -0.25, -0.0, 0.0, 0.25, 0.5, 1.5, 2.5, 1e30, -1e30, np.inf, -np.inf,
+                  np.nextafter(dt(0.5), dt(0))], dtype=dt)
+    d = hip.toHip(x)
+    for name, fn in (("floor", np.floor), ("ceil", np.ceil), ("trunc", np.trunc)):
+        got = hip.unary(name, d).toCpu()
+        assert np.array_equal(got, fn(x)) and np.array_equal(np.signbit(got), np.signbit(fn(x))), name
+    r = np.trunc(x)
+    with np.errstate(invalid="ignore"):
+        want = np.where(np.abs(x - r) >= 0.5, r + np.copysign(dt(1), x), r).astype(dt)   # halves away from zero
+    got = hip.round(d).toCpu()
+    assert np.array_equal(got, want) and np.array_equal(np.signbit(got), np.signbit(x))
+    assert np.isnan(hip.floor(hip.toHip(np.array([np.nan], dtype=dt))).toCpu()[0])
+    with np.errstate(divide="ignore"):
+        assert np.array_equal(hip.reciprocal(d).toCpu(), dt(1) / x)
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_pow_forms(hip, oracle, sfx):
+    """pow as tensor ^. scalar, scalar ^. tensor, in place, and as a map2 body over broadcast operands."""
+    dt = DTYPES[sfx]
+    ulp = np.finfo(dt).eps
+    rng = np.random.default_rng(seed_of(sfx, "pow"))
+    base = rng.uniform(0.1, 6, (64, 1030)).astype(dt)
+    expo = rng.uniform(-3, 3, (1, 1030)).astype(dt)
+    db, de = hip.toHip(base), hip.toHip(expo)
+
+    def close(got, want, what):
+        # float32 pow is evaluated in double on the device and rounded once: the host's bits except at
+        # rare near-ties; float64 pow is the device math library's, a few units in the last place off
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        lim = (1 if sfx == "f32" else 4) * ulp * np.abs(want)
+        assert np.all(err <= lim), (what, float((err / (ulp * np.abs(want))).max()))
+        if sfx == "f32":
+            assert np.mean(got == want) >= 0.999, (what, float(np.mean(got == want)))
+
+    say("pow", sfx)
+    close(hip.bc_pow(db, 2.5).toCpu(), oracle.scalar_op("pow", base, 2.5), "t ^. s")
+    close(hip.bc_pow(1.5, db).toCpu(), oracle.scalar_op("pow", base, 1.5, scalar_on_left=True), "s ^. t")
+    close(hip.bc_pow(db.transpose(), -0.5).toCpu(), oracle.scalar_op("pow", base.T, -0.5), "transposed")
+    ba, bb = oracle.broadcast2(base, expo)
+    close(hip.map2("pow", db, de.broadcast(base.shape)).toCpu(), oracle.map2("pow", ba, bb), "map2")
+    c = db.clone()
+    c.bc_ipow(2.0)
+    close(c.toCpu(), oracle.scalar_op("pow", base, 2.0), "^.=")
+    ints = np.arange(0, 24, dtype=dt)
+    if sfx == "f32":
+        assert np.array_equal(hip.bc_pow(2.0, hip.toHip(ints)).toCpu(), 2.0 ** ints)
+        assert np.array_equal(c.toCpu(), base * base)        # pow(x, 2) correctly rounded = the rounded square
+    else:
+        close(hip.bc_pow(2.0, hip.toHip(ints)).toCpu(), 2.0 ** ints, "2 ^. n")
+    with np.errstate(invalid="ignore"):
+        sp = hip.bc_pow(hip.toHip(np.array([-8.0, 0.0, np.inf, -1.0], dtype=dt)), 0.5).toCpu()
+    assert np.isnan(sp[0]) and sp[1] == 0 and sp[2] == np.inf and np.isnan(sp[3])
+    assert hip.bc_pow(hip.empty((0, 3), dt), 2.0).shape == (0, 3)
+
+
+def test_pow_and_ufunc_errors(hip):
+    ti = hip.toHip(np.arange(6, dtype=np.int32))
+    tf = hip.toHip(np.arange(6, dtype=np.float32))
+    for call in (lambda: hip.bc_pow(ti, 2), lambda: hip.bc_pow(tf, tf), lambda: hip.bc_pow(2.0, 3.0),
+                 lambda: hip.ln(ti), lambda: hip.unary("floor", ti), lambda: hip.scalar_op("pow", ti, 2),
+                 lambda: hip.map2("pow", ti, ti), lambda: ti.bc_ipow(2), lambda: hip.mreciprocal(ti)):
+        with pytest.raises(TypeError):
+            call()

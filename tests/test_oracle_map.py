@@ -240,3 +240,76 @@ def test_reference_conv_vectors(vectors, oracle):
             b = np.array(case["bias"], dtype=dt)
             got = oracle.conv2d(x, k, b, tuple(case["padding"]), tuple(case["stride"]))
             assert np.array_equal(got, np.array(case["target"], dtype=dt)), case["name"]
+
+
+_UFUNC_NUMPY = dict(ln=np.log, log10=np.log10, log2=np.log2, sin=np.sin, cos=np.cos, tan=np.tan, sinh=np.sinh,
+                    cosh=np.cosh, arcsin=np.arcsin, arccos=np.arccos, arctan=np.arctan, arcsinh=np.arcsinh,
+                    arccosh=np.arccosh, arctanh=np.arctanh, cbrt=np.cbrt, floor=np.floor, ceil=np.ceil,
+                    trunc=np.trunc)
+_UFUNC_DOMAIN = dict(ln=(1e-3, 1e3), log10=(1e-3, 1e3), log2=(1e-3, 1e3), arcsin=(-1, 1), arccos=(-1, 1),
+                     arccosh=(1, 50), arctanh=(-0.999, 0.999), sinh=(-20, 20), cosh=(-20, 20))
+
+
+def test_reference_pow_and_ufunc_vectors(vectors, oracle):
+    """`^.` / `^.=`, reciprocal, cos and ln on the reference's own literals. The reference compares
+    pow with ==: so does this test (the host's pow is correctly rounded on these inputs)."""
+    v = vectors["pow_and_ufunc"]
+    a = np.array(v["a"])
+    assert np.array_equal(oracle.scalar_op("pow", a, 2.0), np.array(v["pow_2"]))
+    quot = np.array([[n / q] for n, q in v["pow_m1_as_quotients"]])
+    assert np.array_equal(oracle.scalar_op("pow", a, -1.0), quot)
+    assert np.array_equal(oracle.unary("reciprocal", a), quot)
+    assert np.array_equal(oracle.scalar_op("pow", a, 2.0, scalar_on_left=True), np.array(v["two_pow_a"]))
+    inplace = a.copy()
+    oracle.scalar_op("pow", inplace, 2.0, out=inplace)
+    assert np.array_equal(inplace, np.array(v["pow_2"]))
+    import math
+    c, l = np.array(v["cos_input"]), np.array(v["ln_input"])
+    assert np.abs(oracle.unary("cos", c) - np.vectorize(math.cos)(c)).mean() <= 1e-15
+    assert np.array_equal(oracle.unary("ln", l), np.vectorize(math.log)(l))
+
+
+def test_ufunc_bodies_against_numpy_and_closed_forms(oracle):
+    """Every universal function is the host libm's function of that name. Pinned against NumPy's own
+    evaluation (2 units in the last place: NumPy may use its SIMD routines), against Python's math
+    module for the ones NumPy lacks, and against closed forms a wrong function name would break."""
+    import math
+    rng = np.random.default_rng(11)
+    for dt, ulp in ((np.float32, 2 ** -23), (np.float64, 2 ** -52)):
+        for name, fn in _UFUNC_NUMPY.items():
+            lo, hi = _UFUNC_DOMAIN.get(name, (-8, 8))
+            x = rng.uniform(lo, hi, (13, 29)).astype(dt)
+            got, want = oracle.unary(name, x.T), fn(x.T)
+            assert got.dtype == dt
+            if name in ("floor", "ceil", "trunc"):
+                assert np.array_equal(got, want), name
+            else:
+                assert np.all(np.abs(got - want) <= 2 * ulp * np.maximum(np.abs(want), np.finfo(dt).tiny)), (name, dt)
+        x = rng.uniform(-3, 3, 200).astype(dt)
+        for name, fn in (("erf", math.erf), ("erfc", math.erfc), ("gamma", math.gamma), ("lgamma", math.lgamma)):
+            want = np.array([fn(float(v)) for v in x])
+            np.testing.assert_allclose(oracle.unary(name, x), want, rtol=8 * ulp, atol=8 * ulp, err_msg=name)
+        # closed forms
+        halves = np.array([-2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 0.49999997, -0.0, 3.0], dtype=dt)
+        assert np.array_equal(oracle.unary("round", halves), np.array([-3, -2, -1, 1, 2, 3, 0, -0.0, 3], dtype=dt))
+        assert np.signbit(oracle.unary("round", np.array([-0.25], dtype=dt)))[0]
+        ints = np.arange(1, 11, dtype=dt)
+        np.testing.assert_allclose(oracle.unary("gamma", ints), [math.factorial(int(i) - 1) for i in ints], rtol=2 * ulp)
+        np.testing.assert_allclose(oracle.unary("cbrt", ints ** 3), ints, rtol=2 * ulp)
+        assert np.array_equal(oracle.unary("log2", 2.0 ** ints), ints)
+        assert np.array_equal(oracle.unary("reciprocal", x), dt(1) / x)
+        np.testing.assert_allclose(oracle.unary("erf", x) + oracle.unary("erfc", x), 1, rtol=4 * ulp)
+        s, c = oracle.unary("sin", x), oracle.unary("cos", x)
+        np.testing.assert_allclose(s * s + c * c, 1, rtol=8 * ulp)
+        # pow: tensor-tensor, both scalar sides; exact where the result is representable
+        y = rng.uniform(-3, 3, x.shape).astype(dt)
+        b = np.abs(x) + dt(0.5)
+        want = np.power(b, y)
+        assert np.all(np.abs(oracle.map2("pow", b, y) - want) <= 2 * ulp * np.abs(want))
+        assert np.array_equal(oracle.scalar_op("pow", ints, 2), ints * ints)
+        assert np.array_equal(oracle.scalar_op("pow", ints, 2, scalar_on_left=True), 2.0 ** ints)
+    for dt in (np.int32, np.int64):
+        with pytest.raises(ValueError):
+            oracle.unary("ln", np.arange(4, dtype=dt))
+        with pytest.raises(ValueError):
+            oracle.map2("pow", np.arange(4, dtype=dt), np.arange(4, dtype=dt))
