@@ -88,8 +88,12 @@ template <typename T, int OP> struct BinOp {
         return x / y;
       }
     } else if constexpr (OP == AM_OP_MOD) {
-      if (y == 0 || y == (T)-1) return 0;
-      return x % y;
+      if constexpr (std::is_same<T, float>::value) return fmodf(x, y);      // Nim's float `mod` is C fmod: exact
+      else if constexpr (std::is_same<T, double>::value) return fmod(x, y);
+      else {
+        if (y == 0 || y == (T)-1) return 0;
+        return x % y;
+      }
     } else if constexpr (OP == AM_OP_ADD_RELU) {
       T t = (T)((U)x + (U)y);
       return ((T)0 >= t) ? (T)0 : t;
@@ -629,11 +633,8 @@ static int binary(const char* fn, int op, int rank, const int64_t* shape, T* dst
 #define AM_CASE(code) case code: return run<T, code, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0)
     AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
     AM_CASE(AM_OP_ADD_RELU); AM_CASE(AM_OP_RELU_BWD); AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN);
-    AM_CASE(AM_OP_SIGMOID_BWD); AM_CASE(AM_OP_TANH_BWD); AM_CASE(AM_OP_SQDIFF);
+    AM_CASE(AM_OP_SIGMOID_BWD); AM_CASE(AM_OP_TANH_BWD); AM_CASE(AM_OP_SQDIFF); AM_CASE(AM_OP_MOD);
 #undef AM_CASE
-    case AM_OP_MOD:
-      if constexpr (!F) return run<T, AM_OP_MOD, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
-      else return fail(AM_E_DTYPE, "%s: mod is defined for integer tensors only", fn);
     case AM_OP_ADD_SIGMOID:
       if constexpr (F) return run<T, AM_OP_ADD_SIGMOID, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
       else return fail(AM_E_DTYPE, "%s: add_sigmoid is defined for float tensors only", fn);
@@ -663,11 +664,8 @@ static int scalar(const char* fn, int op, int left, int rank, const int64_t* sha
   switch (op) {
 #define AM_CASE(code) case code: return scalar_lr<T, code>(left != 0, rank, shape, dst, sd, a, sa, s)
     AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
-    AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN);
+    AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN); AM_CASE(AM_OP_MOD);
 #undef AM_CASE
-    case AM_OP_MOD:
-      if constexpr (!F) return scalar_lr<T, AM_OP_MOD>(left != 0, rank, shape, dst, sd, a, sa, s);
-      else return fail(AM_E_DTYPE, "%s: mod is defined for integer tensors only", fn);
     case AM_OP_POW:
       if constexpr (F) return scalar_lr<T, AM_OP_POW>(left != 0, rank, shape, dst, sd, a, sa, s);
       else return fail(AM_E_DTYPE, "%s: pow is defined for float tensors only", fn);

@@ -239,7 +239,7 @@ int am_hip_dot_i64(int64_t n, const int64_t* x, int64_t incx, const int64_t* y, 
 #define AM_OP_SUB         1
 #define AM_OP_MUL         2
 #define AM_OP_DIV         3   /* floats: IEEE /; integers: truncating `div`; x div 0 -> 0 on device */
-#define AM_OP_MOD         4   /* integers only: C `%` (sign of dividend), x mod 0 -> 0 on device     */
+#define AM_OP_MOD         4   /* integers: C `%` (sign of dividend), x mod 0 -> 0 on device; floats: C fmod */
 #define AM_OP_ADD_RELU    5   /* t = a + b; (0 >= t) ? 0 : t        (fused bias + ReLU)              */
 #define AM_OP_ADD_SIGMOID 6   /* floats: 1 / (1 + exp(-(a + b)))    (GRU gates, nnp_gru.nim:78)      */
 #define AM_OP_ADD_TANH    7   /* floats: tanh(a + b)                                                */

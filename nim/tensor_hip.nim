@@ -232,9 +232,9 @@ proc `*.`*[T](a, b: HipTensor[T]): HipTensor[T] =
 proc `/.`*[T](a, b: HipTensor[T]): HipTensor[T] =
   let (ta, tb) = broadcast2(a, b)
   map2(ta, opDiv, tb)       # integers: truncating `div`
-proc `mod`*[T: int32 | int64](a, b: HipTensor[T]): HipTensor[T] =
+proc `mod`*[T: HipScalar](a, b: HipTensor[T]): HipTensor[T] =
   let (ta, tb) = broadcast2(a, b)
-  map2(ta, opMod, tb)
+  map2(ta, opMod, tb)       # integers: sign of the dividend; floats: C fmod, like std/math `mod`
 
 proc `+.=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opAdd, b.broadcast(a.shape.toSeq))
 proc `-.=`*[T](a: var HipTensor[T], b: HipTensor[T]) = apply2(a, opSub, b.broadcast(a.shape.toSeq))

@@ -258,8 +258,6 @@ def test_errors(hip):
     with pytest.raises(ValueError):
         hip.bc_add(a, hip.toHip(np.zeros((1, 3), np.float32)))
     with pytest.raises(TypeError):
-        hip.bc_mod(a, a)
-    with pytest.raises(TypeError):
         hip.map2("add_tanh", hip.toHip(np.zeros(3, np.int32)), hip.toHip(np.zeros(3, np.int32)))
     with pytest.raises(ValueError):   # zero-stride destination
         hip.apply2("add", hip.toHip(np.zeros((1, 2), np.float32)).broadcast((4, 2)), a)
@@ -513,6 +511,27 @@ def test_pow_forms(hip, oracle, sfx):
         sp = hip.bc_pow(hip.toHip(np.array([-8.0, 0.0, np.inf, -1.0], dtype=dt)), 0.5).toCpu()
     assert np.isnan(sp[0]) and sp[1] == 0 and sp[2] == np.inf and np.isnan(sp[3])
     assert hip.bc_pow(hip.empty((0, 3), dt), 2.0).shape == (0, 3)
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_float_mod(hip, oracle, sfx):
+    """`mod` on float tensors (C fmod) is exact: the oracle's bits in every form, special values included."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "fmod"))
+    x = (rng.uniform(-1e4, 1e4, (64, 1030)) * 10.0 ** rng.integers(-3, 4, (64, 1030))).astype(dt)
+    y = rng.uniform(-50, 50, (1, 1030)).astype(dt)
+    dx, dy = hip.toHip(x), hip.toHip(y)
+    say("float mod", sfx)
+    bx, by = oracle.broadcast2(x, y)
+    assert np.array_equal(hip.bc_mod(dx, dy).toCpu(), oracle.map2("mod", bx, by))
+    assert np.array_equal(hip.bc_mod(dx, 3.5).toCpu(), oracle.scalar_op("mod", x, 3.5))
+    assert np.array_equal(hip.bc_mod(3.5, dx.transpose()).toCpu(), oracle.scalar_op("mod", x.T, 3.5, scalar_on_left=True))
+    a, b = np.array([5.5, -5.5, 1.0, np.inf, -0.0, 7.0], dtype=dt), np.array([2.0, 2.0, 0.0, 2.0, 3.0, np.inf], dtype=dt)
+    with np.errstate(invalid="ignore"):
+        want = np.fmod(a, b)
+    got = hip.bc_mod(hip.toHip(a), hip.toHip(b)).toCpu()
+    ok = ~np.isnan(want)                         # the sign of a NaN is not specified
+    assert np.array_equal(got, want, equal_nan=True) and np.array_equal(np.signbit(got)[ok], np.signbit(want)[ok])
 
 
 def test_pow_and_ufunc_errors(hip):

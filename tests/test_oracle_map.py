@@ -202,8 +202,25 @@ def test_broadcast_errors(oracle):
         oracle.broadcast2(np.zeros((3, 2)), np.zeros((2, 2)))
     with pytest.raises(ValueError):
         oracle.broadcast(np.zeros((3, 2)), (3, 3))
-    with pytest.raises(ValueError):
-        oracle.map2("mod", np.zeros(3, np.float32), np.zeros(3, np.float32))
+
+
+def test_float_mod_is_fmod(oracle):
+    """`mod` on float tensors is Nim's std/math `mod`, C fmod: an exact operation (no rounding), result
+    with the dividend's sign. Pinned on NumPy's fmod, on the exact identity x = trunc(x / y) * y + r for
+    small integer-valued operands, and on the special values."""
+    rng = np.random.default_rng(21)
+    for dt in (np.float32, np.float64):
+        x = (rng.uniform(-1e4, 1e4, (17, 33)) * 10.0 ** rng.integers(-3, 4, (17, 33))).astype(dt)
+        y = rng.uniform(-50, 50, (17, 33)).astype(dt)
+        assert np.array_equal(oracle.map2("mod", x, y), np.fmod(x, y))
+        assert np.array_equal(oracle.scalar_op("mod", x, 3.5), np.fmod(x, dt(3.5)))
+        assert np.array_equal(oracle.scalar_op("mod", y, 3.5, scalar_on_left=True), np.fmod(dt(3.5), y))
+        xi, yi = rng.integers(-1000, 1000, 500).astype(dt), rng.integers(1, 40, 500).astype(dt)
+        r = oracle.map2("mod", xi, yi)
+        assert np.array_equal(np.trunc(xi / yi) * yi + r, xi) and np.all(np.abs(r) < yi)
+        with np.errstate(invalid="ignore"):
+            sp = oracle.map2("mod", np.array([5.5, -5.5, 1.0, np.inf, -0.0], dtype=dt), np.array([2.0, 2.0, 0.0, 2.0, 3.0], dtype=dt))
+        assert sp[0] == 1.5 and sp[1] == -1.5 and np.isnan(sp[2]) and np.isnan(sp[3]) and sp[4] == 0 and np.signbit(sp[4])
 
 
 def test_map3_bodies_match_numpy(oracle):
