@@ -13,7 +13,7 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, maxpool2d, tanh, relu_backward, sigmoid_backward,
                          tanh_backward, linear_backward, variance, std, sqrt, square, argmax_max, argmax,
-                         argmin_min, argmin, maxpool2d_backward, bc_pow, mreciprocal, UFUNCS, ln, log10, log2, exp,
+                         argmin_min, argmin, maxpool2d_backward, bc_pow, mreciprocal, clamp, mclamp, UFUNCS, ln, log10, log2, exp,
                          cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, arcsinh, arccosh, arctanh, erf, erfc,
                          gamma, lgamma, floor, ceil, trunc, reciprocal, tround as round)
 
@@ -24,7 +24,7 @@ __all__ = [
     "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward",
     "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin", "maxpool2d_backward",
     "reduce_axis", "reduce_all", "sum", "product", "min", "max", "mean", "softmax", "maxpool2d",
-    "bc_pow", "mreciprocal", "UFUNCS", "ln", "log10", "log2", "exp", "cbrt", "sin", "cos", "tan", "sinh", "cosh",
+    "bc_pow", "mreciprocal", "clamp", "mclamp", "UFUNCS", "ln", "log10", "log2", "exp", "cbrt", "sin", "cos", "tan", "sinh", "cosh",
     "arcsin", "arccos", "arctan", "arcsinh", "arccosh", "arctanh", "erf", "erfc", "gamma", "lgamma", "floor", "ceil",
     "trunc", "reciprocal", "round",
     "read_npy", "write_npy", "load_library",

@@ -365,6 +365,7 @@ template <typename T, int OP> struct TriOp {
     if constexpr (OP == AM_OP3_MULADD) return (T)((U)x * (U)y + (U)z);
     else if constexpr (OP == AM_OP3_ADDMUL) return (T)(((U)x + (U)y) * (U)z);
     else if constexpr (OP == AM_OP3_GRU_CANDIDATE) return dev_tanh(x + y * z);
+    else if constexpr (OP == AM_OP3_CLAMP) return (x < y) ? y : ((x > z) ? z : x);   // a NaN x stays, like Nim's clamp
     else return ((T)1 - y) * z + y * x;
   }
 };
@@ -792,6 +793,7 @@ static int ternary(const char* fn, int op, int rank, const int64_t* shape, T* ds
   switch (op) {
     case AM_OP3_MULADD: return run3<T, AM_OP3_MULADD>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
     case AM_OP3_ADDMUL: return run3<T, AM_OP3_ADDMUL>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
+    case AM_OP3_CLAMP: return run3<T, AM_OP3_CLAMP>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
     case AM_OP3_GRU_CANDIDATE:
       if constexpr (F) return run3<T, AM_OP3_GRU_CANDIDATE>(rank, shape, dst, sd, a, sa, b, sb, c, sc);
       else return fail(AM_E_DTYPE, "%s: tanh(x + y * z) is defined for float tensors only", fn);

@@ -713,6 +713,31 @@ ln, log10, log2, exp, cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, a
 tround = _make_ufunc("round")
 
 
+def _clamp_into(dst: HipTensor, t: HipTensor, lo, hi):
+    # min and max travel as a two-element device tensor, each seen through all-zero strides (the
+    # reference's scalar broadcast is the same: one element, strides 0, private/p_shapeshifting.nim:136-176)
+    bounds = toHip(np.array([lo, hi], dtype=t.dtype))
+    zero = md.Layout(tuple(t.shape), (0,) * t.rank, 0)
+    one = md.Layout(tuple(t.shape), (0,) * t.rank, 1)
+    _ternary_into("clamp", dst, t, HipTensor(zero, bounds.storage, t.dtype), HipTensor(one, bounds.storage, t.dtype))
+
+
+def clamp(t: HipTensor, min, max) -> HipTensor:
+    """map_inline(clamp(x, min, max)): min where x < min, max where x > max, else x
+    (src/arraymancer/tensor/math_functions.nim:146-148). One pass."""
+    out = empty(t.shape, t.dtype)
+    if out.size:
+        _clamp_into(out, t, min, max)
+    return out
+
+
+def mclamp(t: HipTensor, min, max) -> HipTensor:
+    """In-place clamp (math_functions.nim:150-152)."""
+    if t.size:
+        _clamp_into(t, t, min, max)
+    return t
+
+
 def mreciprocal(t: HipTensor) -> HipTensor:
     """In-place 1 / x (src/arraymancer/tensor/math_functions.nim:56-58)."""
     if t.dtype.kind != "f":

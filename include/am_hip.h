@@ -347,12 +347,15 @@ int am_hip_ew_unary_i64(int op, int rank, const int64_t* shape,
  * (src/arraymancer/tensor/higher_order_applymap.nim:58-67, 122-150) with the enumerated bodies the
  * reference itself uses on this path (GRU gates over column slices of [batch, 3H] buffers,
  * src/arraymancer/nn_primitives/nnp_gru.nim:80-88). Every arithmetic step is rounded on its own.
- * dst may alias any operand exactly. Float tensors: all ops; integer tensors: AM_OP3_MULADD and AM_OP3_ADDMUL (wrapping). */
+ * dst may alias any operand exactly. Float tensors: all ops; integer tensors: AM_OP3_MULADD and AM_OP3_ADDMUL (wrapping), AM_OP3_CLAMP. */
 #define AM_OP3_MULADD        0   /* x * y + z                                                  */
 #define AM_OP3_GRU_CANDIDATE 1   /* tanh(x + y * z)              apply3_inline(n, r, Uh)       */
 #define AM_OP3_GRU_BLEND     2   /* (1 - y) * z + y * x          apply3_inline(hidden, z, n)   */
 #define AM_OP3_ADDMUL        3   /* (x + y) * z: `(X +. b) *. s` in one pass, each step rounded   */
-#define AM_OP3_COUNT         4
+#define AM_OP3_CLAMP         4   /* (x < y) ? y : (x > z) ? z : x: clamp(x, min, max), any element type
+                                    (tensor/math_functions.nim:146-152); min and max as one-element operands
+                                    with all strides 0 */
+#define AM_OP3_COUNT         5
 int am_hip_ew_ternary_f32(int op, int rank, const int64_t* shape, float* dst, const int64_t* dst_strides,
                           const float* a, const int64_t* a_strides, const float* b, const int64_t* b_strides,
                           const float* c, const int64_t* c_strides);

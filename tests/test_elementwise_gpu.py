@@ -542,3 +542,26 @@ def test_pow_and_ufunc_errors(hip):
                  lambda: hip.map2("pow", ti, ti), lambda: ti.bc_ipow(2), lambda: hip.mreciprocal(ti)):
         with pytest.raises(TypeError):
             call()
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_clamp(hip, oracle, sfx):
+    """clamp / mclamp in one pass (bounds as zero-stride operands), any element type, any strides."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of(sfx, "clamp"))
+    x = rng.uniform(-100, 100, (70, 1030)).astype(dt)
+    dx = hip.toHip(x)
+    say("clamp", sfx)
+    want = oracle.map3("clamp", x, np.broadcast_to(dt(-25), x.shape), np.broadcast_to(dt(40), x.shape))
+    assert np.array_equal(want, np.clip(x, -25, 40))
+    assert np.array_equal(hip.clamp(dx, -25, 40).toCpu(), want)
+    assert np.array_equal(hip.clamp(dx.transpose(), -25, 40).toCpu(), want.T)
+    assert np.array_equal(hip.clamp(dx[:, 5:77], -25, 40).toCpu(), want[:, 5:77])
+    v = dx[:, 4:1028]
+    assert hip.mclamp(v, -25, 40) is v
+    got = dx.toCpu()
+    assert np.array_equal(got[:, 4:1028], want[:, 4:1028]) and np.array_equal(got[:, :4], x[:, :4])
+    assert hip.clamp(hip.empty((0, 4), dt), 0, 1).shape == (0, 4)
+    if sfx in FLT:
+        s = hip.clamp(hip.toHip(np.array([np.nan, -np.inf, np.inf, -0.0, 5.0], dtype=dt)), 0, 1).toCpu()
+        assert np.isnan(s[0]) and s[1] == 0 and s[2] == 1 and s[3] == 0 and np.signbit(s[3]) and s[4] == 1

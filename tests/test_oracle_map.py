@@ -330,3 +330,16 @@ def test_ufunc_bodies_against_numpy_and_closed_forms(oracle):
             oracle.unary("ln", np.arange(4, dtype=dt))
         with pytest.raises(ValueError):
             oracle.map2("pow", np.arange(4, dtype=dt), np.arange(4, dtype=dt))
+
+
+def test_clamp_body(oracle):
+    """clamp(x, min, max) = min where x < min, max where x > max, else x (math_functions.nim:146-152; the
+    comparisons of Nim's clamp): NumPy's clip computes the same on non-NaN input; a NaN stays a NaN."""
+    rng = np.random.default_rng(31)
+    for dt in (np.float32, np.float64, np.int32, np.int64):
+        x = (rng.uniform(-100, 100, (19, 23))).astype(dt)
+        lo, hi = np.broadcast_to(dt(-25), x.shape), np.broadcast_to(dt(40), x.shape)
+        assert np.array_equal(oracle.map3("clamp", x.T, lo.T, hi.T), np.clip(x, -25, 40).T)
+    x = np.array([np.nan, -np.inf, np.inf, -0.0, 5.0])
+    got = oracle.map3("clamp", x, np.broadcast_to(0.0, x.shape), np.broadcast_to(1.0, x.shape))
+    assert np.isnan(got[0]) and got[1] == 0 and got[2] == 1 and got[3] == 0 and np.signbit(got[3]) and got[4] == 1
