@@ -71,6 +71,8 @@ def _signatures():
     for sfx, ct in CTYPE.items():
         gemm = [i64, i64, i64, ct, vp, i64, i64, vp, i64, i64, ct, vp, i64, i64]
         sig[f"am_hip_gemm_{sfx}"] = (ci, gemm)
+        if sfx == "f32":
+            sig["am_hip_gemm_noalloc_f32"] = (ci, gemm)
         if sfx in ("f32", "f64"):
             sig[f"am_hip_gemm_ex_{sfx}"] = (ci, gemm + [ci, vp, i64, i64])
         sig[f"am_hip_gemm_batched_{sfx}"] = (ci, [i64, i64, i64, i64, ct, vp, i64, i64, i64, vp, i64, i64, i64, ct,

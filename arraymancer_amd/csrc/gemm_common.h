@@ -45,6 +45,11 @@ template <typename T> struct Args {
   const uint32_t* gate_flags;
   uint32_t gate_gen;
   int gate_max_pairs;
+  // Allocation-free entry point: split-K partials go to the library's static device array instead
+  // of the hipMalloc'ed workspace; a plan that needs more than the array holds is recorded in
+  // static_ws_short (bytes it would have needed) and the call is refused.
+  bool static_ws;
+  size_t static_ws_short;
 };
 
 // Digit pairs (i, j), i + j < ND, whose planes are both marked non-empty: flags[i] == gen for A's
@@ -112,6 +117,7 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   g.epilogue = epilogue; g.bias = bias;
   g.batch = 1; g.batch_a = g.batch_b = g.batch_c = 0;
   g.gate_flags = nullptr; g.gate_gen = 0; g.gate_max_pairs = 0;
+  g.static_ws = false; g.static_ws_short = 0;
   g.swapped = swap;
   g.a_kfast = iabs64(g.a_k) <= iabs64(g.a_mn);
   g.b_kfast = iabs64(g.b_k) < iabs64(g.b_mn);
@@ -151,6 +157,9 @@ static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int6
 // Persistent device workspace for split-K partial sums (runtime.hip): allocated once, on first use
 // outside graph capture; nullptr when `bytes` exceeds its capacity or it cannot be allocated now.
 void* splitk_workspace(size_t bytes);
+// The static device array behind the allocation-free entry point (runtime.hip): its device address
+// (looked up once when the library initialised the device) and its size. Never allocates.
+void* static_scratch(size_t* capacity);
 
 // Decides the split-K factor for a problem that would otherwise leave most SIMDs idle: small M x N
 // (few tiles) with a long K runs as one serial MFMA / MAC chain per wave, so K is cut into
@@ -172,7 +181,14 @@ static inline void plan_splitk(Args<T>& g, int bk, int waves_per_tile) {
   splits = (slabs + chunk_slabs - 1) / chunk_slabs;           // no empty split
   if (splits < 2) return;
   const size_t bytes = (size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(T);
-  T* ws = (T*)splitk_workspace(bytes);
+  T* ws;
+  if (g.static_ws) {
+    size_t cap = 0;
+    ws = (T*)static_scratch(&cap);
+    if (!ws || bytes > cap) { g.static_ws_short = bytes; return; }
+  } else {
+    ws = (T*)splitk_workspace(bytes);
+  }
   if (!ws) return;
   g.splits = (int)splits; g.k_chunk = chunk_slabs * bk; g.ws = ws;
 }

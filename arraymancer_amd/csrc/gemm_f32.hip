@@ -45,6 +45,21 @@ extern "C" int am_hip_gemm_f32(int64_t M, int64_t N, int64_t K, float alpha, con
                             nullptr, 0, 0);
 }
 
+// am_hip_gemm_f32 for callers that cannot allocate: same kernels, split-K partials in the library's
+// static device array. Calls no hipMalloc / hipFree and no routine that allocates.
+extern "C" int am_hip_gemm_noalloc_f32(int64_t M, int64_t N, int64_t K, float alpha, const float* A, int64_t rsA,
+                                       int64_t csA, const float* B, int64_t rsB, int64_t csB, float beta, float* C,
+                                       int64_t rsC, int64_t csC) {
+  Args<float> g;
+  const int rc = prepare<float>("am_hip_gemm_noalloc_f32", M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC,
+                                AM_EPI_NONE, nullptr, 0, 0, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  g.static_ws = true;
+  return run_f32(g);
+}
+
 extern "C" int am_hip_gemm_batched_f32(int64_t batch, int64_t M, int64_t N, int64_t K, float alpha, const float* A,
                                        int64_t rsA, int64_t csA, int64_t bsA, const float* B, int64_t rsB, int64_t csB,
                                        int64_t bsB, float beta, float* C, int64_t rsC, int64_t csC, int64_t bsC,

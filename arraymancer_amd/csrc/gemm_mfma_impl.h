@@ -374,6 +374,13 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
   const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
   if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
   plan_splitk(g, BK, WAVES_M * WAVES_N);
+  if (g.static_ws_short) {
+    size_t cap = 0;
+    (void)static_scratch(&cap);
+    return fail(AM_E_SHAPE, "am_hip_gemm_noalloc_f32: M=%lld N=%lld K=%lld needs %zu bytes of split-K scratch, the static "
+                "buffer holds %zu; call am_hip_gemm_f32 for this product", (long long)g.M, (long long)g.N, (long long)g.K,
+                g.static_ws_short, cap);
+  }
   const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(WAVES_M * WAVES_N * 64);
 #define AM_LAUNCH(AKIND, BKIND_)                                                                   \
   hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, AKIND, BKIND_>), grid, block, 0, \

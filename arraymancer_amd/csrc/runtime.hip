@@ -20,6 +20,16 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// Scratch of the allocation-free entry point (am_hip_gemm_noalloc_f32): the split-K partial tiles go
+// here instead of into the workspace that splitk_workspace() takes from hipMalloc. The array lives
+// in the code object, so every device the library runs on holds its own copy, at its own address,
+// until the process ends. Host code never uses the array's name as an address: init_locked() asks
+// the runtime for the device address once, with the device current, and everything afterwards
+// (kernel arguments) uses that pointer.
+static constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr = nullptr;   // device address of `scratch` on g_device (the library binds one device per process)
+
 static std::mutex g_mu;
 static bool g_ready = false;
 static int g_device = -1;
@@ -42,6 +52,7 @@ static int init_locked(int device) {
   if (strncmp(g_prop.gcnArchName, "gfx950", 6) != 0)
     return fail(AM_E_NODEVICE, "device %d is %s; this library carries gfx950 code only", device, g_prop.gcnArchName);
   AM_HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  AM_HIP_TRY(hipGetSymbolAddress((void**)&g_scratch_ptr, HIP_SYMBOL(scratch)));
   g_device = device;
   g_ready = true;
   return AM_OK;
@@ -65,6 +76,10 @@ void* splitk_workspace(size_t bytes) {
     if (hipMalloc(&g_ws, kWorkspaceBytes) != hipSuccess) { (void)hipGetLastError(); g_ws = nullptr; }
   }
   return g_ws;
+}
+void* static_scratch(size_t* capacity) {
+  if (capacity) *capacity = kStaticScratchBytes;
+  return g_ready ? g_scratch_ptr : nullptr;
 }
 }  // namespace gemm
 

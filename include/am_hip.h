@@ -132,6 +132,24 @@ int am_hip_gemm_i64(int64_t M, int64_t N, int64_t K, int64_t alpha,
                     const int64_t* B, int64_t rsB, int64_t csB,
                     int64_t beta, int64_t* C, int64_t rsC, int64_t csC);
 
+/* am_hip_gemm_f32 for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
+ * arguments, kernels and result bits as am_hip_gemm_f32; the difference is where the split-K partial
+ * tiles go (products with few output tiles and a long K are cut along K over several workgroups):
+ * am_hip_gemm_f32 takes a workspace from hipMalloc on first use, this entry point uses a 16 MiB
+ * array that is part of the library's device code and calls no hipMalloc / hipFree nor any routine
+ * that allocates. Each device the library runs on holds that array until the process ends.
+ * Limit: a product whose plan needs more than 16 MiB of partials (splits * M * N * 4 bytes, splits
+ * <= 32; only products of fewer than 512 wavefront tiles are split at all, so M * N <= 131072 always
+ * fits and large products need none) is refused with AM_E_SHAPE and a message that says so.
+ * All calls on a device share the array, which keeps the last call's contents (every partial is
+ * written before it is read, so nothing has to be cleared). Calls that overlap on one device would
+ * race on it; the library's contract (one calling thread at a time, one stream) rules that out. */
+int am_hip_gemm_noalloc_f32(int64_t M, int64_t N, int64_t K, float alpha,
+                            const float* A, int64_t rsA, int64_t csA,
+                            const float* B, int64_t rsB, int64_t csB,
+                            float beta, float* C, int64_t rsC, int64_t csC);
+
 /* GEMM with a fused element-wise epilogue:
  *   C <- act( alpha*A*B + beta*C + bias ),  bias[r,c] = bias[r*bias_rs + c*bias_cs]
  * (bias_rs = 0, bias_cs = 1 is the [1,N] row vector of `linear`).

@@ -54,6 +54,9 @@ proc am_hip_diag_peak*(kind, iters, waves_per_simd: cint, ops_per_second: ptr cd
 proc am_hip_gemm_f32*(M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64,
                       B: ptr cfloat, rsB, csB: int64, beta: cfloat,
                       C: ptr cfloat, rsC, csC: int64): cint {.importc.}
+proc am_hip_gemm_noalloc_f32*(M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64,
+                              B: ptr cfloat, rsB, csB: int64, beta: cfloat,
+                              C: ptr cfloat, rsC, csC: int64): cint {.importc.}   # allocates nothing: split-K partials in a 16 MiB static device array
 proc am_hip_gemm_f64*(M, N, K: int64, alpha: cdouble, A: ptr cdouble, rsA, csA: int64,
                       B: ptr cdouble, rsB, csB: int64, beta: cdouble,
                       C: ptr cdouble, rsC, csC: int64): cint {.importc.}
