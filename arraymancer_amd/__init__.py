@@ -15,7 +15,8 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          tanh_backward, linear_backward, variance, std, sqrt, square, argmax_max, argmax,
                          argmin_min, argmin, maxpool2d_backward, bc_pow, mreciprocal, clamp, mclamp, UFUNCS, ln, log10, log2, exp,
                          cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, arcsinh, arccosh, arctanh, erf, erfc,
-                         gamma, lgamma, floor, ceil, trunc, reciprocal, tround as round)
+                         gamma, lgamma, floor, ceil, trunc, reciprocal, tround as round, bc_eq, bc_ne, bc_lt, bc_le, bc_gt,
+                         bc_ge, isNaN, isNotNaN, classify, FLOAT_CLASS, sgn, floorMod, copySign, mcopySign, degToRad, radToDeg)
 
 __all__ = [
     "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
@@ -27,5 +28,7 @@ __all__ = [
     "bc_pow", "mreciprocal", "clamp", "mclamp", "UFUNCS", "ln", "log10", "log2", "exp", "cbrt", "sin", "cos", "tan", "sinh", "cosh",
     "arcsin", "arccos", "arctan", "arcsinh", "arccosh", "arctanh", "erf", "erfc", "gamma", "lgamma", "floor", "ceil",
     "trunc", "reciprocal", "round",
+    "bc_eq", "bc_ne", "bc_lt", "bc_le", "bc_gt", "bc_ge", "isNaN", "isNotNaN", "classify", "FLOAT_CLASS", "sgn", "floorMod",
+    "copySign", "mcopySign", "degToRad", "radToDeg",
     "read_npy", "write_npy", "load_library",
 ]

@@ -15,12 +15,14 @@ AM_OK, AM_E_ARG, AM_E_SHAPE, AM_E_DTYPE, AM_E_ALLOC, AM_E_HIP, AM_E_NODEVICE = 0
 AM_MAXRANK = 6
 
 OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
-          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12, sqdiff=13, pow=14)
+          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12, sqdiff=13, pow=14, floormod=15, copysign=16)
+CMP = {"==": 0, "!=": 1, "<": 2, "<=": 3, ">": 4, ">=": 5, "mod_is_zero": 6}
+PRED = dict(isnan=0, isnotnan=1, classify=2)
 OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2, addmul=3, clamp=4)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6, sqrt=7, square=8,
            ln=9, log10=10, log2=11, sin=12, cos=13, tan=14, sinh=15, cosh=16, arcsin=17,
            arccos=18, arctan=19, arcsinh=20, arccosh=21, arctanh=22, cbrt=23, erf=24, erfc=25, gamma=26,
-           lgamma=27, floor=28, ceil=29, trunc=30, round=31, reciprocal=32)
+           lgamma=27, floor=28, ceil=29, trunc=30, round=31, reciprocal=32, degtorad=33, radtodeg=34)
 EPI = dict(none=0, bias=1, relu=2, bias_relu=3)
 RED = dict(sum=0, product=1, min=2, max=3)
 
@@ -84,6 +86,12 @@ def _signatures():
         sig[f"am_hip_ew_scalar_{sfx}"] = (ci, [ci, ci, ci, vp, vp, vp, vp, vp, ct])
         sig[f"am_hip_ew_ternary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp, vp, vp, vp, vp])
         sig[f"am_hip_ew_unary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp])
+        sig[f"am_hip_ew_compare_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp, vp, vp])
+        sig[f"am_hip_ew_compare_scalar_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp, ct])
+        sig[f"am_hip_ew_sgn_{sfx}"] = (ci, [ci, vp, vp, vp, vp, vp])
+        sig[f"am_hip_ew_clamp_{sfx}"] = (ci, [ci, vp, vp, vp, vp, vp, ct, ct])
+        if sfx in ("f32", "f64"):
+            sig[f"am_hip_ew_predicate_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp])
         sig[f"am_hip_reduce_axis_{sfx}"] = (ci, [ci, ci, vp, ci, vp, vp, vp, vp])
         sig[f"am_hip_argreduce_{sfx}"] = (ci, [ci, ci, vp, ci, vp, vp, vp, vp, vp, vp])
         sig[f"am_hip_reduce_all_{sfx}"] = (ci, [ci, ci, vp, vp, vp, ctypes.POINTER(ct)])

@@ -116,6 +116,20 @@ template <typename T, int OP> struct BinOp {
       else return (T)((U)y * ((U)1 - (U)x * (U)x));
     } else if constexpr (OP == AM_OP_POW) {
       if constexpr (Traits<T>::kFloat) return dev_pow(x, y); else return x;   // never dispatched for integers
+    } else if constexpr (OP == AM_OP_FLOORMOD) {
+      // Nim's floorMod: r = x mod y, moved by y when r and y have opposite signs (a zero r stays, -0.0 included)
+      T r;
+      if constexpr (std::is_same<T, float>::value) r = fmodf(x, y);
+      else if constexpr (std::is_same<T, double>::value) r = fmod(x, y);
+      else r = (y == 0 || y == (T)-1) ? (T)0 : (T)(x % y);
+      if ((r > (T)0 && y < (T)0) || (r < (T)0 && y > (T)0)) {
+        if constexpr (Traits<T>::kFloat) r = r + y; else r = (T)((U)r + (U)y);
+      }
+      return r;
+    } else if constexpr (OP == AM_OP_COPYSIGN) {
+      if constexpr (std::is_same<T, float>::value) return copysignf(x, y);
+      else if constexpr (std::is_same<T, double>::value) return copysign(x, y);
+      else return x;   // never dispatched for integers
     } else {  // AM_OP_SQDIFF
       if constexpr (Traits<T>::kFloat) { const T d = x - y; return d * d; }
       else { const U d = (U)x - (U)y; return (T)(d * d); }
@@ -140,6 +154,11 @@ template <typename T, int UOP> struct UnOp {
     } else if constexpr (UOP == AM_UOP_SQUARE) {
       if constexpr (Traits<T>::kFloat) return x * x; else return (T)((U)x * (U)x);
     }
+    else if constexpr (UOP == AM_UOP_DEGTORAD) {   // Nim: d * RadPerDeg, RadPerDeg = PI / 180 rounded to T
+      if constexpr (Traits<T>::kFloat) return x * (T)(3.14159265358979323846 / 180.0); else return x;
+    } else if constexpr (UOP == AM_UOP_RADTODEG) {   // Nim: d / RadPerDeg
+      if constexpr (Traits<T>::kFloat) return x / (T)(3.14159265358979323846 / 180.0); else return x;
+    }
     else if constexpr (UOP >= AM_UOP_LN) {
       if constexpr (Traits<T>::kFloat) return dev_math<UOP>(x); else return x;   // never dispatched for integers
     }
@@ -150,8 +169,49 @@ template <typename T, int UOP> struct UnOp {
   }
 };
 
+// Bodies whose result type differs from the operands' (the reference's map templates infer it:
+// src/arraymancer/tensor/higher_order_applymap.nim:92-120). Comparisons give Nim's bool as one byte
+// (0 / 1): `==.` `!=.` `<.` `<=.` `>.` `>=.` (src/arraymancer/tensor/operators_comparison.nim:41-146)
+// and `x mod y == 0`, the body of the reference's own fixture (tests/tensor/test_higherorder.nim:103-112).
+constexpr int kCmpBase = 200;
+template <typename T, int CMP> struct CmpOp {
+  static __device__ __forceinline__ uint8_t apply(T x, T y) {
+    if constexpr (CMP == AM_CMP_EQ) return x == y;
+    else if constexpr (CMP == AM_CMP_NE) return x != y;
+    else if constexpr (CMP == AM_CMP_LT) return x < y;
+    else if constexpr (CMP == AM_CMP_LE) return x <= y;
+    else if constexpr (CMP == AM_CMP_GT) return x > y;
+    else if constexpr (CMP == AM_CMP_GE) return x >= y;
+    else return BinOp<T, AM_OP_MOD>::apply(x, y) == (T)0;   // AM_CMP_MOD_IS_ZERO
+  }
+};
+
+// Predicates and classifiers of one operand: isNaN / isNotNaN (operators_comparison.nim:192-206: x != x,
+// x == x), classify (tensor/math_functions.nim:264-276, the ordinal of Nim's FloatClass in one byte) and
+// sgn (math_functions.nim:110-117: Tensor[int], i.e. int64; -1, 0, 1, a NaN gives 0).
+constexpr int kPredBase = 300;
+template <typename T, int PRED> struct PredOp {
+  static __device__ __forceinline__ auto apply(T x, T) {
+    if constexpr (PRED == AM_PRED_ISNAN) return (uint8_t)(x != x);
+    else if constexpr (PRED == AM_PRED_ISNOTNAN) return (uint8_t)(x == x);
+    else if constexpr (PRED == AM_PRED_SGN) return (int64_t)((T)0 < x) - (int64_t)(x < (T)0);
+    else {   // AM_PRED_CLASSIFY: fcNormal, fcSubnormal, fcZero, fcNegZero, fcNan, fcInf, fcNegInf = 0..6
+      if constexpr (Traits<T>::kFloat) {
+        if (x != x) return (uint8_t)4;
+        if (x == (T)0) return (uint8_t)(__builtin_signbit(x) ? 3 : 2);
+        const T ax = __builtin_fabs(x);
+        if (ax == (T)__builtin_inf()) return (uint8_t)(x > (T)0 ? 5 : 6);
+        constexpr T tiny = std::is_same<T, float>::value ? (T)1.17549435e-38f : (T)2.2250738585072014e-308;
+        return (uint8_t)(ax < tiny ? 1 : 0);
+      } else return (uint8_t)0;   // never dispatched for integers
+    }
+  }
+};
+
 template <typename T, int CODE> struct OpSel {
-  typedef typename std::conditional<(CODE >= kUnaryBase), UnOp<T, CODE - kUnaryBase>, BinOp<T, CODE>>::type type;
+  typedef typename std::conditional<(CODE >= kPredBase), PredOp<T, CODE - kPredBase>,
+          typename std::conditional<(CODE >= kCmpBase), CmpOp<T, CODE - kCmpBase>,
+          typename std::conditional<(CODE >= kUnaryBase), UnOp<T, CODE - kUnaryBase>, BinOp<T, CODE>>::type>::type>::type type;
 };
 
 // ---- layouts passed to kernels by value
@@ -159,8 +219,9 @@ constexpr int kMaxOuter = AM_MAXRANK - 1;
 
 enum Kind : int { kVecOperand = 0, kRowScalar = 1, kConst = 2 };
 
-template <typename T> struct RowsArgs {
-  T* dst; const T* a; const T* b;
+// T: element type of the operands, D: of the destination (the same except for comparisons and predicates).
+template <typename T, typename D = T> struct RowsArgs {
+  D* dst; const T* a; const T* b;
   T scalar;               // the kConst operand
   int a_stream, b_stream; // 1: operand is read once (non-temporal loads); 0: re-read per row, keep cached
   int64_t L;              // inner extent (elements)
@@ -171,8 +232,8 @@ template <typename T> struct RowsArgs {
   int64_t od[kMaxOuter], oa[kMaxOuter], ob[kMaxOuter];  // outer strides per operand (elements)
 };
 
-template <typename T> struct GenericArgs {
-  T* dst; const T* a; const T* b;
+template <typename T, typename D = T> struct GenericArgs {
+  D* dst; const T* a; const T* b;
   T scalar;
   int64_t n;
   int rank;
@@ -194,9 +255,10 @@ template <typename V> __device__ __forceinline__ V load_as(bool keep, const V* p
   return __builtin_nontemporal_load(launder(ptr));
 }
 
-template <typename T, int CODE, int AK, int BK, bool SWAP>
-__global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
+template <typename T, typename D, int CODE, int AK, int BK, bool SWAP>
+__global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T, D> p) {
   typedef typename Traits<T>::V V;
+  typedef D DV __attribute__((ext_vector_type(Traits<T>::kVec)));   // one result per operand element of a 16-byte vector
   typedef typename OpSel<T, CODE>::type Op;
   constexpr int VEC = Traits<T>::kVec;
   constexpr int64_t TILE = (int64_t)kThreads * VEC * kUnroll;
@@ -217,7 +279,7 @@ __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
         if constexpr (BK != kConst) offb += c * p.ob[d];
       }
     }
-    T* __restrict__ drow = p.dst + offd;
+    D* __restrict__ drow = p.dst + offd;
     const T* __restrict__ arow = p.a + offa;
     const T* __restrict__ brow = (BK != kConst) ? p.b + offb : nullptr;
     T asc = (T)0, bsc = p.scalar;
@@ -257,27 +319,27 @@ __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T> p) {
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t col = col0 + (int64_t)u * kThreads * VEC;
       if (full[u]) {
-        V r;
+        DV r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const T x = (AK == kVecOperand) ? av[u][e] : asc;
           const T y = (BK == kVecOperand) ? bv[u][e] : bsc;
-          r[e] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+          r[e] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
         }
-        __builtin_nontemporal_store(r, (V*)(drow + col));
+        __builtin_nontemporal_store(r, (DV*)(drow + col));
       } else {
         for (int64_t c = col; c < p.L; ++c) {   // ragged end of the row (< VEC elements)
           const T x = (AK == kVecOperand) ? arow[c] : asc;
           const T y = (BK == kVecOperand) ? brow[c] : bsc;
-          drow[c] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+          drow[c] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
         }
       }
     }
   }
 }
 
-template <typename T, int CODE, bool BCONST, bool SWAP, typename IDX>
-__global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T> p) {
+template <typename T, typename D, int CODE, bool BCONST, bool SWAP, typename IDX>
+__global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T, D> p) {
   typedef typename OpSel<T, CODE>::type Op;
   const IDX n = (IDX)p.n;
   const IDX step = (IDX)gridDim.x * kThreads;
@@ -295,7 +357,7 @@ __global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T> p) {
     }
     const T x = p.a[offa];
     const T y = BCONST ? p.scalar : p.b[offb];
-    p.dst[offd] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+    p.dst[offd] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
   }
 }
 
@@ -307,8 +369,8 @@ __global__ __launch_bounds__(kThreads) void ew_generic(GenericArgs<T> p) {
 // a wavefront is therefore a contiguous run, which ew_generic cannot offer for these layouts.
 constexpr int kTile2d = 64;
 
-template <typename T> struct TiledArgs {
-  T* dst; const T* a; const T* b;
+template <typename T, typename D = T> struct TiledArgs {
+  D* dst; const T* a; const T* b;
   T scalar;
   int64_t R, C;                 // extents of axis 0 and axis 1
   int64_t d0;                   // dst stride along axis 0 (axis 1 is unit)
@@ -317,8 +379,8 @@ template <typename T> struct TiledArgs {
   int tiles_c;
 };
 
-template <typename T, int CODE, bool BCONST, bool SWAP>
-__global__ __launch_bounds__(256) void ew_tiled(TiledArgs<T> p) {
+template <typename T, typename D, int CODE, bool BCONST, bool SWAP>
+__global__ __launch_bounds__(256) void ew_tiled(TiledArgs<T, D> p) {
   typedef typename OpSel<T, CODE>::type Op;
   __shared__ T ta[kTile2d][kTile2d + 1];
   __shared__ T tb[BCONST ? 1 : kTile2d][kTile2d + 1];
@@ -353,7 +415,7 @@ __global__ __launch_bounds__(256) void ew_tiled(TiledArgs<T> p) {
       T y;
       if constexpr (BCONST) y = p.scalar;
       else y = p.b_t ? tb[tx][rl] : p.b[r * p.b0 + c * p.b1];
-      p.dst[r * p.d0 + c] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+      p.dst[r * p.d0 + c] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
     }
   }
 }
@@ -379,6 +441,8 @@ template <typename T> struct TriArgs {
   int a_const, b_const, c_const;   // rows kernel: operand has inner stride 0 (one value per row)
   int a_keep, b_keep, c_keep;      // rows kernel: ordinary loads (a row re-read for every output row, or operands small
                                    // enough for the memory-side cache); 0 = non-temporal loads
+  int bc_imm;                      // operands b and c are the values b_imm and c_imm (clamp bounds passed by value)
+  T b_imm, c_imm;
   int64_t shape[AM_MAXRANK];
   int64_t sd[AM_MAXRANK], sa[AM_MAXRANK], sb[AM_MAXRANK], sc[AM_MAXRANK];
 };
@@ -414,15 +478,19 @@ __global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
       if (col + VEC <= p.L) {
         V av, bv, cv;
         if (p.a_const) { for (int e = 0; e < VEC; ++e) av[e] = arow[0]; } else av = load_as(p.a_keep != 0, (const V*)(arow + col));
-        if (p.b_const) { for (int e = 0; e < VEC; ++e) bv[e] = brow[0]; } else bv = load_as(p.b_keep != 0, (const V*)(brow + col));
-        if (p.c_const) { for (int e = 0; e < VEC; ++e) cv[e] = crow[0]; } else cv = load_as(p.c_keep != 0, (const V*)(crow + col));
+        if (p.bc_imm) { for (int e = 0; e < VEC; ++e) { bv[e] = p.b_imm; cv[e] = p.c_imm; } }
+        else {
+          if (p.b_const) { for (int e = 0; e < VEC; ++e) bv[e] = brow[0]; } else bv = load_as(p.b_keep != 0, (const V*)(brow + col));
+          if (p.c_const) { for (int e = 0; e < VEC; ++e) cv[e] = crow[0]; } else cv = load_as(p.c_keep != 0, (const V*)(crow + col));
+        }
         V r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) r[e] = TriOp<T, OP>::apply(av[e], bv[e], cv[e]);
         __builtin_nontemporal_store(r, (V*)(drow + col));
       } else {
         for (int64_t cc = col; cc < p.L; ++cc)
-          drow[cc] = TriOp<T, OP>::apply(arow[p.a_const ? 0 : cc], brow[p.b_const ? 0 : cc], crow[p.c_const ? 0 : cc]);
+          drow[cc] = TriOp<T, OP>::apply(arow[p.a_const ? 0 : cc], p.bc_imm ? p.b_imm : brow[p.b_const ? 0 : cc],
+                                         p.bc_imm ? p.c_imm : crow[p.c_const ? 0 : cc]);
       }
     }
   }
@@ -442,7 +510,7 @@ __global__ __launch_bounds__(kThreads) void ew3_generic(TriArgs<T> p) {
       rem = q;
       od += cidx * p.sd[d]; oa += cidx * p.sa[d]; ob += cidx * p.sb[d]; oc += cidx * p.sc[d];
     }
-    p.dst[od] = TriOp<T, OP>::apply(p.a[oa], p.b[ob], p.c[oc]);
+    p.dst[od] = TriOp<T, OP>::apply(p.a[oa], p.bc_imm ? p.b_imm : p.b[ob], p.bc_imm ? p.c_imm : p.c[oc]);
   }
 }
 
@@ -488,9 +556,9 @@ static inline int collapse(int rank, const int64_t* shape, const int64_t* sd, co
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-template <typename T, int CODE, bool BCONST, bool SWAP>
-static int launch_generic(const Collapsed& c, T* dst, const T* a, const T* b, T scalar) {
-  GenericArgs<T> g;
+template <typename T, int CODE, bool BCONST, bool SWAP, typename D = T>
+static int launch_generic(const Collapsed& c, D* dst, const T* a, const T* b, T scalar) {
+  GenericArgs<T, D> g;
   g.dst = dst; g.a = a; g.b = b; g.scalar = scalar; g.n = c.n; g.rank = c.rank;
   for (int i = 0; i < AM_MAXRANK; ++i) {
     g.shape[i] = i < c.rank ? c.shape[i] : 1;
@@ -502,19 +570,20 @@ static int launch_generic(const Collapsed& c, T* dst, const T* a, const T* b, T 
   const int64_t cap = (int64_t)num_cus() * 16;
   if (blocks > cap) blocks = cap;
   if (c.n < ((int64_t)1 << 31)) {
-    hipLaunchKernelGGL((ew_generic<T, CODE, BCONST, SWAP, uint32_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+    hipLaunchKernelGGL((ew_generic<T, D, CODE, BCONST, SWAP, uint32_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
   } else {
-    hipLaunchKernelGGL((ew_generic<T, CODE, BCONST, SWAP, uint64_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+    hipLaunchKernelGGL((ew_generic<T, D, CODE, BCONST, SWAP, uint64_t>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
   }
   return check_launch("ew_generic");
 }
 
 // Runs dst = op(a, b) (BCONST: b is `scalar`). Chooses the streaming kernel when every
 // operand's innermost collapsed stride is 1 (or 0 for a/b) and rows start 16-byte aligned.
-template <typename T, int CODE, bool BCONST, bool SWAP>
-static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a,
+template <typename T, int CODE, bool BCONST, bool SWAP, typename D = T>
+static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const T* a,
                const int64_t* sa, const T* b, const int64_t* sb, T scalar) {
   constexpr int VEC = Traits<T>::kVec;
+  constexpr uintptr_t kDstAlign = VEC * sizeof(D) < 16 ? VEC * sizeof(D) : 16;   // one vector store of VEC results
   Collapsed c;
   AM_TRY(collapse(rank, shape, sd, sa, BCONST ? nullptr : sb, &c));
   if (c.n == 0) return AM_OK;
@@ -526,7 +595,7 @@ static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const 
   bool ok = (id == 1) && (ia == 0 || ia == 1) && (ib == 0 || ib == 1) && !(ia == 0 && ib == 0 && !BCONST);
   if (BCONST && ia == 0) ok = false;
   if (ok) {
-    ok = aligned16(dst) && (ia == 0 || aligned16(a)) && (BCONST || ib == 0 || aligned16(b));
+    ok = ((uintptr_t)dst % kDstAlign == 0) && (ia == 0 || aligned16(a)) && (BCONST || ib == 0 || aligned16(b));
     for (int d = 0; d < in && ok; ++d) {
       if (c.sd[d] % VEC != 0) ok = false;
       if (ia == 1 && c.sa[d] % VEC != 0) ok = false;
@@ -547,7 +616,7 @@ static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const 
       if (c.sd[1] == 1) ax = 1; else if (c.sd[0] == 1) ax = 0;
       if (ax >= 0) {
         const int o = 1 - ax;
-        TiledArgs<T> t;
+        TiledArgs<T, D> t;
         t.dst = dst; t.a = a; t.b = b; t.scalar = scalar;
         t.R = c.shape[o]; t.C = c.shape[ax]; t.d0 = c.sd[o];
         t.a0 = c.sa[o]; t.a1 = c.sa[ax]; t.b0 = BCONST ? 0 : c.sb[o]; t.b1 = BCONST ? 0 : c.sb[ax];
@@ -558,15 +627,15 @@ static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const 
         const int64_t tr = (t.R + kTile2d - 1) / kTile2d, tc = (t.C + kTile2d - 1) / kTile2d;
         if (a_ok && b_ok && (t.a_t || t.b_t || ax == 0) && tr * tc < ((int64_t)1 << 31) && t.R >= 16 && t.C >= 16) {
           t.tiles_c = (int)tc;
-          hipLaunchKernelGGL((ew_tiled<T, CODE, BCONST, SWAP>), dim3((unsigned)(tr * tc)), dim3(256), 0, stream(), t);
+          hipLaunchKernelGGL((ew_tiled<T, D, CODE, BCONST, SWAP>), dim3((unsigned)(tr * tc)), dim3(256), 0, stream(), t);
           return check_launch("ew_tiled");
         }
       }
     }
-    return launch_generic<T, CODE, BCONST, SWAP>(c, dst, a, b, scalar);
+    return launch_generic<T, CODE, BCONST, SWAP, D>(c, dst, a, b, scalar);
   }
 
-  RowsArgs<T> r;
+  RowsArgs<T, D> r;
   r.dst = dst; r.a = a; r.b = b; r.scalar = scalar; r.L = L;
   r.tiles_per_row = (uint32_t)tiles_per_row;
   r.total_tiles = (uint32_t)(tiles_per_row * rows);
@@ -597,11 +666,11 @@ static int run(int rank, const int64_t* shape, T* dst, const int64_t* sd, const 
   if (blocks > cap) blocks = cap;
   const dim3 grid((unsigned)blocks), block(kThreads);
   if constexpr (BCONST) {
-    hipLaunchKernelGGL((ew_rows<T, CODE, kVecOperand, kConst, SWAP>), grid, block, 0, stream(), r);
+    hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kConst, SWAP>), grid, block, 0, stream(), r);
   } else {
-    if (ia == 1 && ib == 1) hipLaunchKernelGGL((ew_rows<T, CODE, kVecOperand, kVecOperand, false>), grid, block, 0, stream(), r);
-    else if (ia == 1) hipLaunchKernelGGL((ew_rows<T, CODE, kVecOperand, kRowScalar, false>), grid, block, 0, stream(), r);
-    else hipLaunchKernelGGL((ew_rows<T, CODE, kRowScalar, kVecOperand, false>), grid, block, 0, stream(), r);
+    if (ia == 1 && ib == 1) hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kVecOperand, false>), grid, block, 0, stream(), r);
+    else if (ia == 1) hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kRowScalar, false>), grid, block, 0, stream(), r);
+    else hipLaunchKernelGGL((ew_rows<T, D, CODE, kRowScalar, kVecOperand, false>), grid, block, 0, stream(), r);
   }
   return check_launch("ew_rows");
 }
@@ -645,6 +714,10 @@ static int binary(const char* fn, int op, int rank, const int64_t* shape, T* dst
     case AM_OP_POW:
       if constexpr (F) return run<T, AM_OP_POW, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
       else return fail(AM_E_DTYPE, "%s: pow is defined for float tensors only", fn);
+    case AM_OP_FLOORMOD: return run<T, AM_OP_FLOORMOD, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
+    case AM_OP_COPYSIGN:
+      if constexpr (F) return run<T, AM_OP_COPYSIGN, false, false>(rank, shape, dst, sd, a, sa, b, sb, (T)0);
+      else return fail(AM_E_DTYPE, "%s: copySign is defined for float tensors only", fn);
     default:
       return fail(AM_E_ARG, "%s: unknown op %d", fn, op);
   }
@@ -665,7 +738,7 @@ static int scalar(const char* fn, int op, int left, int rank, const int64_t* sha
   switch (op) {
 #define AM_CASE(code) case code: return scalar_lr<T, code>(left != 0, rank, shape, dst, sd, a, sa, s)
     AM_CASE(AM_OP_ADD); AM_CASE(AM_OP_SUB); AM_CASE(AM_OP_MUL); AM_CASE(AM_OP_DIV);
-    AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN); AM_CASE(AM_OP_MOD);
+    AM_CASE(AM_OP_MAX); AM_CASE(AM_OP_MIN); AM_CASE(AM_OP_MOD); AM_CASE(AM_OP_FLOORMOD);
 #undef AM_CASE
     case AM_OP_POW:
       if constexpr (F) return scalar_lr<T, AM_OP_POW>(left != 0, rank, shape, dst, sd, a, sa, s);
@@ -705,19 +778,76 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
     AM_CASE(AM_UOP_ARCTAN); AM_CASE(AM_UOP_ARCSINH); AM_CASE(AM_UOP_ARCCOSH); AM_CASE(AM_UOP_ARCTANH);
     AM_CASE(AM_UOP_CBRT); AM_CASE(AM_UOP_ERF); AM_CASE(AM_UOP_ERFC); AM_CASE(AM_UOP_GAMMA); AM_CASE(AM_UOP_LGAMMA);
     AM_CASE(AM_UOP_FLOOR); AM_CASE(AM_UOP_CEIL); AM_CASE(AM_UOP_TRUNC); AM_CASE(AM_UOP_ROUND); AM_CASE(AM_UOP_RECIPROCAL);
+    AM_CASE(AM_UOP_DEGTORAD); AM_CASE(AM_UOP_RADTODEG);
 #undef AM_CASE
     default:
       return fail(AM_E_ARG, "%s: unknown unary op %d", fn, op);
   }
 }
 
+// dst (one byte per element, 0 / 1) = cmp(a, b): the broadcast comparison family and any other
+// map2 body with a bool result.
+template <typename T>
+static int compare(const char* fn, int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* sd,
+                   const T* a, const int64_t* sa, const T* b, const int64_t* sb) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  if (rank > 0 && !sb) return fail(AM_E_ARG, "%s: null stride array", fn);
+  {
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= shape[i];
+    if (n != 0 && !b) return fail(AM_E_ARG, "%s: null data pointer", fn);
+  }
+  switch (op) {
+#define AM_CASE(code) case code: return run<T, kCmpBase + code, false, false, uint8_t>(rank, shape, dst, sd, a, sa, b, sb, (T)0)
+    AM_CASE(AM_CMP_EQ); AM_CASE(AM_CMP_NE); AM_CASE(AM_CMP_LT); AM_CASE(AM_CMP_LE); AM_CASE(AM_CMP_GT); AM_CASE(AM_CMP_GE);
+    AM_CASE(AM_CMP_MOD_IS_ZERO);
+#undef AM_CASE
+    default: return fail(AM_E_ARG, "%s: unknown comparison %d", fn, op);
+  }
+}
+
+template <typename T>
+static int compare_scalar(const char* fn, int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* sd,
+                          const T* a, const int64_t* sa, T s) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  switch (op) {
+#define AM_CASE(code) case code: return run<T, kCmpBase + code, true, false, uint8_t>(rank, shape, dst, sd, a, sa, nullptr, nullptr, s)
+    AM_CASE(AM_CMP_EQ); AM_CASE(AM_CMP_NE); AM_CASE(AM_CMP_LT); AM_CASE(AM_CMP_LE); AM_CASE(AM_CMP_GT); AM_CASE(AM_CMP_GE);
+    AM_CASE(AM_CMP_MOD_IS_ZERO);
+#undef AM_CASE
+    default: return fail(AM_E_ARG, "%s: unknown comparison %d", fn, op);
+  }
+}
+
+template <typename T>
+static int predicate(const char* fn, int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* sd,
+                     const T* a, const int64_t* sa) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  if constexpr (!Traits<T>::kFloat) return fail(AM_E_DTYPE, "%s: defined for float tensors only", fn);
+  else switch (op) {
+#define AM_CASE(code) case code: return run<T, kPredBase + code, true, false, uint8_t>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0)
+    AM_CASE(AM_PRED_ISNAN); AM_CASE(AM_PRED_ISNOTNAN); AM_CASE(AM_PRED_CLASSIFY);
+#undef AM_CASE
+    default: return fail(AM_E_ARG, "%s: unknown predicate %d", fn, op);
+  }
+}
+
+template <typename T>
+static int sgn(const char* fn, int rank, const int64_t* shape, int64_t* dst, const int64_t* sd, const T* a, const int64_t* sa) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  return run<T, kPredBase + AM_PRED_SGN, true, false, int64_t>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
+}
+
 template <typename T, int OP>
 static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a, const int64_t* sa,
-                const T* b, const int64_t* sb, const T* c, const int64_t* sc) {
+                const T* b, const int64_t* sb, const T* c, const int64_t* sc, const T* imm = nullptr) {
   constexpr int VEC = Traits<T>::kVec;
   // joint collapse over the four operands
   TriArgs<T> g;
   g.dst = dst; g.a = a; g.b = b; g.c = c;
+  g.bc_imm = imm != nullptr; g.b_imm = imm ? imm[0] : (T)0; g.c_imm = imm ? imm[1] : (T)0;
+  static const int64_t zero_strides[AM_MAXRANK] = {0, 0, 0, 0, 0, 0};
+  if (imm) { sb = zero_strides; sc = zero_strides; }
   int r = 0;
   int64_t n = 1;
   for (int i = 0; i < rank; ++i) {
@@ -780,6 +910,13 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
 }
 
 template <typename T>
+static int clamp(const char* fn, int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a, const int64_t* sa, T lo, T hi) {
+  AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
+  const T imm[2] = {lo, hi};
+  return run3<T, AM_OP3_CLAMP>(rank, shape, dst, sd, a, sa, nullptr, nullptr, nullptr, nullptr, imm);
+}
+
+template <typename T>
 static int ternary(const char* fn, int op, int rank, const int64_t* shape, T* dst, const int64_t* sd, const T* a,
                    const int64_t* sa, const T* b, const int64_t* sb, const T* c, const int64_t* sc) {
   AM_TRY(check_common(fn, rank, shape, dst, sd, a, sa));
@@ -826,4 +963,27 @@ static int ternary(const char* fn, int op, int rank, const int64_t* shape, T* ds
   extern "C" int am_hip_ew_unary_##SFX(int op, int rank, const int64_t* shape, T* dst,                 \
                                        const int64_t* ds, const T* a, const int64_t* as_) {            \
     return ::am::ew::unary<T>("am_hip_ew_unary_" #SFX, op, rank, shape, dst, ds, a, as_);              \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_compare_##SFX(int op, int rank, const int64_t* shape, uint8_t* dst,         \
+                                         const int64_t* ds, const T* a, const int64_t* as_,            \
+                                         const T* b, const int64_t* bs) {                              \
+    return ::am::ew::compare<T>("am_hip_ew_compare_" #SFX, op, rank, shape, dst, ds, a, as_, b, bs);   \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_compare_scalar_##SFX(int op, int rank, const int64_t* shape, uint8_t* dst,  \
+                                                const int64_t* ds, const T* a, const int64_t* as_, T s) { \
+    return ::am::ew::compare_scalar<T>("am_hip_ew_compare_scalar_" #SFX, op, rank, shape, dst, ds, a, as_, s); \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_clamp_##SFX(int rank, const int64_t* shape, T* dst, const int64_t* ds,      \
+                                       const T* a, const int64_t* as_, T lo, T hi) {                   \
+    return ::am::ew::clamp<T>("am_hip_ew_clamp_" #SFX, rank, shape, dst, ds, a, as_, lo, hi);          \
+  }                                                                                                    \
+  extern "C" int am_hip_ew_sgn_##SFX(int rank, const int64_t* shape, int64_t* dst, const int64_t* ds,  \
+                                     const T* a, const int64_t* as_) {                                 \
+    return ::am::ew::sgn<T>("am_hip_ew_sgn_" #SFX, rank, shape, dst, ds, a, as_);                      \
+  }
+
+#define AM_EW_DEFINE_FLOAT_ENTRY_POINTS(T, SFX)                                                        \
+  extern "C" int am_hip_ew_predicate_##SFX(int op, int rank, const int64_t* shape, uint8_t* dst,       \
+                                           const int64_t* ds, const T* a, const int64_t* as_) {        \
+    return ::am::ew::predicate<T>("am_hip_ew_predicate_" #SFX, op, rank, shape, dst, ds, a, as_);      \
   }

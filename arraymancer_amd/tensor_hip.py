@@ -28,7 +28,7 @@ import numpy as np
 
 from . import _lib
 from . import metadata as md
-from ._lib import CTYPE, EPI, OP, OP3, RED, SFX, UOP, check, i64_array
+from ._lib import CMP, CTYPE, EPI, OP, OP3, PRED, RED, SFX, UOP, check, i64_array
 from .metadata import Layout, Step
 
 
@@ -62,6 +62,11 @@ def _dtype_sfx(dtype) -> str:
         raise TypeError(f"HipTensor supports float32, float64, int32 and int64, not {dtype}")
 
 
+# Element types a HipTensor can hold as the RESULT of a map whose body changes the type (Tensor[bool] of the
+# comparisons, one byte per element; classify's FloatClass ordinals): views and toCpu work, arithmetic does not.
+_RESULT_ONLY = (np.dtype(np.bool_), np.dtype(np.uint8))
+
+
 class HipTensor:
     __slots__ = ("layout", "storage", "dtype", "pool_geometry")
 
@@ -93,7 +98,10 @@ class HipTensor:
 
     @property
     def sfx(self) -> str:
-        return SFX[self.dtype]
+        try:
+            return SFX[self.dtype]
+        except KeyError:
+            raise TypeError(f"no arithmetic is defined on a HipTensor of {self.dtype}")
 
     def data_ptr(self) -> int:
         """Device address of element [0, 0, ...] (get_offset_ptr, data_structure.nim:206-211)."""
@@ -110,6 +118,16 @@ class HipTensor:
 
     def __repr__(self):
         return f"HipTensor[{self.dtype}](shape={list(self.shape)}, strides={list(self.strides)}, offset={self.offset})"
+
+    def pretty(self, precision: int = -1, specifier: str = "") -> str:
+        """The reference's `pretty` / `$` for a device tensor (src/arraymancer/tensor/display_cuda.nim:19-36):
+        a host copy laid out by the CPU printer (display.nim:19-115), under a header that names this
+        type and backend. `specifier`: "" (table), "||", "[]", "[:]", "<>", "<:>" and their header forms."""
+        from . import display
+        return display.pretty_array(np.ascontiguousarray(self.toCpu()), "HipTensor", "Hip", precision, specifier)
+
+    def __str__(self):
+        return self.pretty()
 
     # ------------------------------------------------------------------ views (no data movement)
     def transpose(self) -> "HipTensor":
@@ -242,7 +260,8 @@ class HipTensor:
 def empty(shape: Sequence[int], dtype) -> HipTensor:
     """newTensorUninit on the device: row-major, uninitialised."""
     dtype = np.dtype(dtype)
-    _dtype_sfx(dtype)
+    if dtype not in _RESULT_ONLY:
+        _dtype_sfx(dtype)
     lay = md.contiguous(shape)
     return HipTensor(lay, HipStorage(lay.size, dtype.itemsize), dtype)
 
@@ -537,6 +556,11 @@ def map2(op, a: HipTensor, b: HipTensor) -> HipTensor:
     already have equal shapes (src/arraymancer/tensor/higher_order_applymap.nim:92-120)."""
     _same_dtype(a, b)
     _check_elementwise(a, b)
+    if op in CMP:   # a body with a bool result: the output type follows the body, like the reference's template
+        out = empty(a.shape, np.bool_)
+        if out.size:
+            _compare_into(op, out, a, b)
+        return out
     out = empty(a.shape, a.dtype)
     _binary_into(op, out, a, b)
     return out
@@ -548,6 +572,12 @@ def apply2(op, dest: HipTensor, src: HipTensor) -> HipTensor:
     _check_elementwise(dest, src)
     _binary_into(op, dest, dest, src)
     return dest
+
+
+def _compare_into(cmp, dst: HipTensor, a: HipTensor, b: HipTensor):
+    check(getattr(_lib.load(), f"am_hip_ew_compare_{a.sfx}")(
+        CMP[cmp], dst.rank, i64_array(dst.shape), ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
+        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides), ctypes.c_void_p(b.data_ptr()), i64_array(b.strides)))
 
 
 def _ternary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor, c: HipTensor):
@@ -591,6 +621,101 @@ def bc_sub(a, b): return _bc_or_scalar("sub", a, b)
 def bc_mul(a, b): return _bc_or_scalar("mul", a, b)
 def bc_div(a, b): return _bc_or_scalar("div", a, b)
 def bc_mod(a, b): return _bc_or_scalar("mod", a, b)
+
+
+def floorMod(a, b):
+    """floorMod(tensor, tensor) (equal shapes: map2_inline without broadcasting), floorMod(tensor, scalar),
+    floorMod(scalar, tensor) (src/arraymancer/tensor/math_functions.nim:134-144)."""
+    ta, tb = isinstance(a, HipTensor), isinstance(b, HipTensor)
+    if ta and tb:
+        return map2("floormod", a, b)
+    return _bc_or_scalar("floormod", a, b)
+
+
+def copySign(t1: HipTensor, t2: HipTensor) -> HipTensor:
+    """Magnitudes of t1 with the signs of t2, float tensors (math_functions.nim:119-125)."""
+    if t1.dtype.kind != "f":
+        raise TypeError("copySign is defined for float tensors only")
+    return map2("copysign", t1, t2)
+
+
+def mcopySign(t1: HipTensor, t2: HipTensor) -> HipTensor:
+    """In-place copySign (math_functions.nim:127-132)."""
+    if t1.dtype.kind != "f":
+        raise TypeError("mcopySign is defined for float tensors only")
+    return apply2("copysign", t1, t2)
+
+
+# ---- comparisons: `==.` `!=.` `<.` `<=.` `>.` `>=.` (src/arraymancer/tensor/operators_comparison.nim:41-185)
+_MIRROR = {"==": "==", "!=": "!=", "<": ">", "<=": ">=", ">": "<", ">=": "<="}
+
+
+def _bc_compare(cmp, a, b) -> HipTensor:
+    """Tensor-tensor with implicit broadcasting, tensor-scalar, or scalar-tensor (which the reference
+    rewrites into the mirrored tensor-scalar comparison, :150-185). Result: a bool tensor."""
+    ta, tb = isinstance(a, HipTensor), isinstance(b, HipTensor)
+    if ta and tb:
+        _same_dtype(a, b)
+        la, lb = md.broadcast2(a.layout, b.layout)
+        return map2(cmp, HipTensor(la, a.storage, a.dtype), HipTensor(lb, b.storage, b.dtype))
+    if not (ta or tb):
+        raise TypeError("at least one operand must be a HipTensor")
+    t, value, cmp = (a, b, cmp) if ta else (b, a, _MIRROR[cmp])
+    out = empty(t.shape, np.bool_)      # returnEmptyIfEmpty: an empty tensor comes back empty
+    if out.size:
+        check(getattr(_lib.load(), f"am_hip_ew_compare_scalar_{t.sfx}")(
+            CMP[cmp], out.rank, i64_array(out.shape), ctypes.c_void_p(out.data_ptr()), i64_array(out.strides),
+            ctypes.c_void_p(t.data_ptr()), i64_array(t.strides), CTYPE[t.sfx](value)))
+    return out
+
+
+def bc_eq(a, b): return _bc_compare("==", a, b)
+def bc_ne(a, b): return _bc_compare("!=", a, b)
+def bc_lt(a, b): return _bc_compare("<", a, b)
+def bc_le(a, b): return _bc_compare("<=", a, b)
+def bc_gt(a, b): return _bc_compare(">", a, b)
+def bc_ge(a, b): return _bc_compare(">=", a, b)
+
+
+def _predicate(op, t: HipTensor, out_dtype) -> HipTensor:
+    if t.dtype.kind != "f":
+        raise TypeError(f"{op} is defined for float tensors only")
+    out = empty(t.shape, out_dtype)
+    if out.size:
+        check(getattr(_lib.load(), f"am_hip_ew_predicate_{t.sfx}")(
+            PRED[op], out.rank, i64_array(out.shape), ctypes.c_void_p(out.data_ptr()), i64_array(out.strides),
+            ctypes.c_void_p(t.data_ptr()), i64_array(t.strides)))
+    return out
+
+
+def isNaN(t: HipTensor) -> HipTensor:
+    """Bool tensor, true where x != x (operators_comparison.nim:192-198)."""
+    return _predicate("isnan", t, np.bool_)
+
+
+def isNotNaN(t: HipTensor) -> HipTensor:
+    """Bool tensor, true where x == x (operators_comparison.nim:200-206)."""
+    return _predicate("isnotnan", t, np.bool_)
+
+
+# Ordinals of Nim's FloatClass, the element type of classify's result (math_functions.nim:264-276).
+FLOAT_CLASS = ("fcNormal", "fcSubnormal", "fcZero", "fcNegZero", "fcNan", "fcInf", "fcNegInf")
+
+
+def classify(t: HipTensor) -> HipTensor:
+    """uint8 tensor of FloatClass ordinals (index into FLOAT_CLASS)."""
+    return _predicate("classify", t, np.uint8)
+
+
+def sgn(t: HipTensor) -> HipTensor:
+    """int64 tensor (the reference's Tensor[int]) of -1 / 0 / 1; zeros and NaN give 0
+    (src/arraymancer/tensor/math_functions.nim:110-117)."""
+    out = empty(t.shape, np.int64)
+    if out.size:
+        check(getattr(_lib.load(), f"am_hip_ew_sgn_{t.sfx}")(
+            out.rank, i64_array(out.shape), ctypes.c_void_p(out.data_ptr()), i64_array(out.strides),
+            ctypes.c_void_p(t.data_ptr()), i64_array(t.strides)))
+    return out
 
 
 def bc_pow(a, b):
@@ -685,6 +810,7 @@ def tanh_backward(gradient: HipTensor, cached_tensor: HipTensor) -> HipTensor:
 
 OPERATORS = {"+.": bc_add, "-.": bc_sub, "*.": bc_mul, "/.": bc_div, "mod": bc_mod,
              "^.": bc_pow,
+             "==.": bc_eq, "!=.": bc_ne, "<.": bc_lt, "<=.": bc_le, ">.": bc_gt, ">=.": bc_ge,
              "+.=": HipTensor.bc_iadd, "-.=": HipTensor.bc_isub, "*.=": HipTensor.bc_imul,
              "/.=": HipTensor.bc_idiv, "^.=": HipTensor.bc_ipow}
 
@@ -713,13 +839,26 @@ ln, log10, log2, exp, cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, a
 tround = _make_ufunc("round")
 
 
+def degToRad(t: HipTensor) -> HipTensor:
+    """x * (PI / 180) (src/arraymancer/tensor/ufunc.nim:129)."""
+    if t.dtype.kind != "f":
+        raise TypeError("degToRad is defined for float tensors only")
+    return unary("degtorad", t)
+
+
+def radToDeg(t: HipTensor) -> HipTensor:
+    """x / (PI / 180) (src/arraymancer/tensor/ufunc.nim:130)."""
+    if t.dtype.kind != "f":
+        raise TypeError("radToDeg is defined for float tensors only")
+    return unary("radtodeg", t)
+
+
 def _clamp_into(dst: HipTensor, t: HipTensor, lo, hi):
-    # min and max travel as a two-element device tensor, each seen through all-zero strides (the
-    # reference's scalar broadcast is the same: one element, strides 0, private/p_shapeshifting.nim:136-176)
-    bounds = toHip(np.array([lo, hi], dtype=t.dtype))
-    zero = md.Layout(tuple(t.shape), (0,) * t.rank, 0)
-    one = md.Layout(tuple(t.shape), (0,) * t.rank, 1)
-    _ternary_into("clamp", dst, t, HipTensor(zero, bounds.storage, t.dtype), HipTensor(one, bounds.storage, t.dtype))
+    # both bounds travel by value: no device allocation, no copy, no synchronisation, recordable into a graph
+    ct = CTYPE[t.sfx]
+    check(getattr(_lib.load(), f"am_hip_ew_clamp_{t.sfx}")(
+        dst.rank, i64_array(dst.shape), ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
+        ctypes.c_void_p(t.data_ptr()), i64_array(t.strides), ct(lo), ct(hi)))
 
 
 def clamp(t: HipTensor, min, max) -> HipTensor:

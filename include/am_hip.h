@@ -268,7 +268,10 @@ int am_hip_dot_i64(int64_t n, const int64_t* x, int64_t incx, const int64_t* y, 
 #define AM_OP_TANH_BWD   12   /* b * (1 - a * a)   a = cached tanh output    (nnp_activation.nim:72-74)  */
 #define AM_OP_SQDIFF     13   /* (a - b) * (a - b): the fold body of variance (tensor/aggregate.nim:115-146) */
 #define AM_OP_POW        14   /* floats only: pow(a, b); `^.` and `^.=` (operators_broadcasted.nim:153-161, 178-182) */
-#define AM_OP_BINARY_COUNT 15
+#define AM_OP_FLOORMOD   15   /* Nim's floorMod: r = a mod b, plus b when r and b have opposite signs
+                                 (tensor/math_functions.nim:134-144; std/math floorMod). Integers: b == 0 -> 0 */
+#define AM_OP_COPYSIGN   16   /* floats only: magnitude of a, sign of b (copySign / mcopySign, math_functions.nim:119-132) */
+#define AM_OP_BINARY_COUNT 17
 
 int am_hip_ew_binary_f32(int op, int rank, const int64_t* shape,
                          float* dst, const int64_t* dst_strides,
@@ -347,7 +350,9 @@ int am_hip_ew_scalar_i64(int op, int scalar_on_left, int rank, const int64_t* sh
 #define AM_UOP_TRUNC      30
 #define AM_UOP_ROUND      31   /* halfway cases away from zero (C round) */
 #define AM_UOP_RECIPROCAL 32   /* 1 / x */
-#define AM_UOP_COUNT      33
+#define AM_UOP_DEGTORAD   33   /* x * (PI / 180), the constant rounded to the element type (Nim's degToRad, ufunc.nim:129) */
+#define AM_UOP_RADTODEG   34   /* x / (PI / 180)                                           (Nim's radToDeg, ufunc.nim:130) */
+#define AM_UOP_COUNT      35
 int am_hip_ew_unary_f32(int op, int rank, const int64_t* shape,
                         float* dst, const int64_t* dst_strides,
                         const float* a, const int64_t* a_strides);
@@ -360,6 +365,60 @@ int am_hip_ew_unary_i32(int op, int rank, const int64_t* shape,
 int am_hip_ew_unary_i64(int op, int rank, const int64_t* shape,
                         int64_t* dst, const int64_t* dst_strides,
                         const int64_t* a, const int64_t* a_strides);
+
+/* Map bodies whose result type differs from the operands': the reference's map templates infer the
+ * type of the result (src/arraymancer/tensor/higher_order_applymap.nim:69-120, its own fixture:
+ * tests/tensor/test_higherorder.nim:103-112, `x mod y == 0` -> Tensor[bool]).
+ *
+ * dst[i] (one byte per element, 0 or 1: Nim's bool) = a[i] cmp b[i]. Replaces the broadcast comparison
+ * family `==.` `!=.` `<.` `<=.` `>.` `>=.` (src/arraymancer/tensor/operators_comparison.nim:41-94:
+ * broadcast2 then map2_inline) and, in the scalar form, :111-146 (map_inline of `x cmp value`; the
+ * reversed forms `value cmp t` are the mirrored comparison of `t`, :150-185). Same traversal, strides
+ * and dimension collapsing as am_hip_ew_binary_*; dst strides count bytes = elements. Floats compare
+ * like IEEE (every comparison with a NaN is false except `!=`). */
+#define AM_CMP_EQ 0
+#define AM_CMP_NE 1
+#define AM_CMP_LT 2
+#define AM_CMP_LE 3
+#define AM_CMP_GT 4
+#define AM_CMP_GE 5
+#define AM_CMP_MOD_IS_ZERO 6   /* (a mod b) == 0 with AM_OP_MOD's `mod` */
+#define AM_CMP_COUNT 7
+int am_hip_ew_compare_f32(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                          const float* a, const int64_t* a_strides, const float* b, const int64_t* b_strides);
+int am_hip_ew_compare_f64(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                          const double* a, const int64_t* a_strides, const double* b, const int64_t* b_strides);
+int am_hip_ew_compare_i32(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                          const int32_t* a, const int64_t* a_strides, const int32_t* b, const int64_t* b_strides);
+int am_hip_ew_compare_i64(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                          const int64_t* a, const int64_t* a_strides, const int64_t* b, const int64_t* b_strides);
+int am_hip_ew_compare_scalar_f32(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                                 const float* a, const int64_t* a_strides, float scalar);
+int am_hip_ew_compare_scalar_f64(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                                 const double* a, const int64_t* a_strides, double scalar);
+int am_hip_ew_compare_scalar_i32(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                                 const int32_t* a, const int64_t* a_strides, int32_t scalar);
+int am_hip_ew_compare_scalar_i64(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                                 const int64_t* a, const int64_t* a_strides, int64_t scalar);
+
+/* dst[i] (one byte) = predicate(a[i]) for float tensors: isNaN (x != x) and isNotNaN (x == x),
+ * src/arraymancer/tensor/operators_comparison.nim:192-206; classify, src/arraymancer/tensor/
+ * math_functions.nim:264-276, as the ordinal of Nim's FloatClass: 0 fcNormal, 1 fcSubnormal, 2 fcZero,
+ * 3 fcNegZero, 4 fcNan, 5 fcInf, 6 fcNegInf. */
+#define AM_PRED_ISNAN    0
+#define AM_PRED_ISNOTNAN 1
+#define AM_PRED_CLASSIFY 2
+#define AM_PRED_SGN      3   /* only through am_hip_ew_sgn_*: its destination is int64 */
+int am_hip_ew_predicate_f32(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                            const float* a, const int64_t* a_strides);
+int am_hip_ew_predicate_f64(int op, int rank, const int64_t* shape, uint8_t* dst, const int64_t* dst_strides,
+                            const double* a, const int64_t* a_strides);
+/* dst[i] (int64: the reference's Tensor[int]) = -1, 0 or 1, the sign of a[i]; zeros of either sign and
+ * NaN give 0 (sgn, src/arraymancer/tensor/math_functions.nim:110-117). */
+int am_hip_ew_sgn_f32(int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides, const float* a, const int64_t* a_strides);
+int am_hip_ew_sgn_f64(int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides, const double* a, const int64_t* a_strides);
+int am_hip_ew_sgn_i32(int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides, const int32_t* a, const int64_t* a_strides);
+int am_hip_ew_sgn_i64(int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides, const int64_t* a, const int64_t* a_strides);
 
 /* dst[i] = op(a[i], b[i], c[i]): map3_inline / apply3_inline
  * (src/arraymancer/tensor/higher_order_applymap.nim:58-67, 122-150) with the enumerated bodies the
@@ -386,6 +445,19 @@ int am_hip_ew_ternary_i32(int op, int rank, const int64_t* shape, int32_t* dst, 
 int am_hip_ew_ternary_i64(int op, int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides,
                           const int64_t* a, const int64_t* a_strides, const int64_t* b, const int64_t* b_strides,
                           const int64_t* c, const int64_t* c_strides);
+
+/* dst[i] = (a[i] < lo) ? lo : (a[i] > hi) ? hi : a[i] with both bounds passed by value: clamp / mclamp
+ * (src/arraymancer/tensor/math_functions.nim:146-152, map_inline / apply_inline of Nim's clamp). One
+ * pass, no device memory for the bounds, no copy, so it can be recorded into a graph like every other
+ * element-wise call. dst may alias a exactly. A NaN element stays NaN. */
+int am_hip_ew_clamp_f32(int rank, const int64_t* shape, float* dst, const int64_t* dst_strides,
+                        const float* a, const int64_t* a_strides, float lo, float hi);
+int am_hip_ew_clamp_f64(int rank, const int64_t* shape, double* dst, const int64_t* dst_strides,
+                        const double* a, const int64_t* a_strides, double lo, double hi);
+int am_hip_ew_clamp_i32(int rank, const int64_t* shape, int32_t* dst, const int64_t* dst_strides,
+                        const int32_t* a, const int64_t* a_strides, int32_t lo, int32_t hi);
+int am_hip_ew_clamp_i64(int rank, const int64_t* shape, int64_t* dst, const int64_t* dst_strides,
+                        const int64_t* a, const int64_t* a_strides, int64_t lo, int64_t hi);
 
 /* ---------------------------------------------------------------- reductions, softmax, pooling
  * dst <- fold of `a` along `axis` with op (AM_RED_*). `shape` / `a_strides` describe `a` (rank

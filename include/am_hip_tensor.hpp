@@ -16,6 +16,10 @@
 //   a +. b, a -. b, a *. b, a /. b    am::bc_add / bc_sub / bc_mul / bc_div   (also tensor-scalar)
 //   a +.= b ...                       a.bc_iadd(b) / bc_isub / bc_imul / bc_idiv
 //   t ^. e, b ^. t, t ^.= e           am::bc_pow(t, e), am::bc_pow(b, t), t.bc_ipow(e)
+//   a ==. b, a <. b, t >=. s ...      am::bc_eq / bc_ne / bc_lt / bc_le / bc_gt / bc_ge  -> HipTensor<uint8_t> (bool)
+//   map2_inline(a, b, x mod y == 0)   am::map2_bool(AM_CMP_MOD_IS_ZERO, a, b)
+//   isNaN, classify, sgn, clamp       am::isNaN, am::classify, am::sgn, am::clamp / t.mclamp(lo, hi)
+//   echo t, t.pretty(precision)       std::cout << t, am::pretty(t, precision, specifier)
 //   ln(t), cos(t), floor(t) ...       am::ln(t), am::cos(t), am::floor(t) ...
 //   t.transpose, t[a..b|s, ...]       t.transpose(), t.slice(axis, first, last, step)
 //   t.broadcast(shape)                t.broadcast(shape)
@@ -25,8 +29,11 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
+#include <cstdio>
 #include <fstream>
 #include <memory>
+#include <ostream>
 #include <stdexcept>
 #include <string>
 #include <type_traits>
@@ -68,6 +75,22 @@ namespace detail {
   inline int unary_(int op, int rank, const int64_t* sh, T* d, const int64_t* sd, const T* a,            \
                     const int64_t* sa) {                                                                 \
     return am_hip_ew_unary_##SFX(op, rank, sh, d, sd, a, sa);                                             \
+  }                                                                                                      \
+  inline int compare_(int op, int rank, const int64_t* sh, uint8_t* d, const int64_t* sd, const T* a,    \
+                      const int64_t* sa, const T* b, const int64_t* sb) {                                \
+    return am_hip_ew_compare_##SFX(op, rank, sh, d, sd, a, sa, b, sb);                                    \
+  }                                                                                                      \
+  inline int compare_scalar_(int op, int rank, const int64_t* sh, uint8_t* d, const int64_t* sd,         \
+                             const T* a, const int64_t* sa, T s) {                                       \
+    return am_hip_ew_compare_scalar_##SFX(op, rank, sh, d, sd, a, sa, s);                                 \
+  }                                                                                                      \
+  inline int sgn_(int rank, const int64_t* sh, int64_t* d, const int64_t* sd, const T* a,                \
+                  const int64_t* sa) {                                                                   \
+    return am_hip_ew_sgn_##SFX(rank, sh, d, sd, a, sa);                                                   \
+  }                                                                                                      \
+  inline int clamp_(int rank, const int64_t* sh, T* d, const int64_t* sd, const T* a, const int64_t* sa, \
+                    T lo, T hi) {                                                                        \
+    return am_hip_ew_clamp_##SFX(rank, sh, d, sd, a, sa, lo, hi);                                         \
   }
 #define AM_HPP_BIND2(T, SFX)                                                                             \
   inline int gemv_(int64_t M, int64_t N, T al, const T* A, int64_t ra, int64_t ca, const T* x, int64_t ix, \
@@ -117,6 +140,13 @@ inline int gemm_ex_(int64_t M, int64_t N, int64_t K, double al, const double* A,
   return am_hip_gemm_ex_f64(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc, epi, bias, brs, bcs);
 }
 
+inline int predicate_(int op, int rank, const int64_t* sh, uint8_t* d, const int64_t* sd, const float* a, const int64_t* sa) {
+  return am_hip_ew_predicate_f32(op, rank, sh, d, sd, a, sa);
+}
+inline int predicate_(int op, int rank, const int64_t* sh, uint8_t* d, const int64_t* sd, const double* a, const int64_t* sa) {
+  return am_hip_ew_predicate_f64(op, rank, sh, d, sd, a, sa);
+}
+
 inline int softmax_(int64_t r, int64_t c, float* d, int64_t drs, int64_t dcs, const float* s, int64_t srs, int64_t scs) {
   return am_hip_softmax_rows_f32(r, c, d, drs, dcs, s, srs, scs);
 }
@@ -149,9 +179,12 @@ struct HipStorage {
 
 template <typename T>
 class HipTensor {
+  // uint8_t holds the result of a map whose body changes the type: Tensor[bool] of the comparisons (one
+  // byte per element, 0 / 1) and classify's FloatClass ordinals. Such a tensor can be viewed and copied to
+  // the host; no arithmetic is defined on it.
   static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value ||
-                    std::is_same<T, int32_t>::value || std::is_same<T, int64_t>::value,
-                "HipTensor supports float, double, int32_t and int64_t");
+                    std::is_same<T, int32_t>::value || std::is_same<T, int64_t>::value || std::is_same<T, uint8_t>::value,
+                "HipTensor supports float, double, int32_t and int64_t (and uint8_t as a result type)");
 
  public:
   Shape shape, strides;     // elements
@@ -226,6 +259,8 @@ class HipTensor {
   // ---- transfers ----------------------------------------------------------------------------
   // Blocking copy of the logical contents in C order (a device-side gather first if strided).
   std::vector<T> toCpu() const {
+    if (std::is_same<T, uint8_t>::value && !is_C_contiguous())
+      throw std::invalid_argument("toCpu: a strided view of a bool / uint8 tensor cannot be gathered on the device");
     const HipTensor c = is_C_contiguous() ? *this : clone();
     std::vector<T> host((size_t)size());
     if (!host.empty()) check(am_hip_memcpy_d2h(host.data(), c.ptr(), host.size() * sizeof(T)));
@@ -233,8 +268,18 @@ class HipTensor {
   }
   HipTensor clone() const {
     HipTensor r(shape);
-    if (size() > 0) check(detail::unary_(AM_UOP_COPY, rank(), shape.data(), r.ptr(), r.strides.data(), ptr(), strides.data()));
+    if constexpr (std::is_same<T, uint8_t>::value) {
+      if (!is_C_contiguous()) throw std::invalid_argument("clone: a strided view of a bool / uint8 tensor cannot be gathered on the device");
+      if (size() > 0) check(am_hip_memcpy_d2d(r.ptr(), ptr(), (size_t)size()));
+    } else {
+      if (size() > 0) check(detail::unary_(AM_UOP_COPY, rank(), shape.data(), r.ptr(), r.strides.data(), ptr(), strides.data()));
+    }
     return r;
+  }
+  // In-place clamp to [lo, hi] (mclamp, math_functions.nim:150-152); the bounds travel by value.
+  HipTensor& mclamp(T lo, T hi) {
+    if (size() > 0) check(detail::clamp_(rank(), shape.data(), ptr(), strides.data(), ptr(), strides.data(), lo, hi));
+    return *this;
   }
 
   // ---- in-place forms -------------------------------------------------------------------------
@@ -348,6 +393,67 @@ template <typename T> HipTensor<T> bc_div(T s, const HipTensor<T>& t) { return s
 // `^.`: tensor ^. exponent and base ^. tensor, float tensors (operators_broadcasted.nim:153-161)
 template <typename T> HipTensor<T> bc_pow(const HipTensor<T>& t, T exponent) { return scalar_op(AM_OP_POW, t, exponent); }
 template <typename T> HipTensor<T> bc_pow(T base, const HipTensor<T>& t) { return scalar_op(AM_OP_POW, t, base, true); }
+// ---- map bodies whose result type differs from the operands' --------------------------------------
+// The reference's map templates infer the result type (higher_order_applymap.nim:69-120); a bool result
+// is a HipTensor<uint8_t> here (one byte per element, 0 / 1).
+template <typename T>
+HipTensor<uint8_t> map2_bool(int cmp, const HipTensor<T>& a, const HipTensor<T>& b) {
+  if (a.shape != b.shape)
+    throw std::invalid_argument("Both Tensors should have the same shape. Left-hand side has shape " +
+                                detail::str(a.shape) + " while right-hand side has shape " + detail::str(b.shape));
+  HipTensor<uint8_t> r(a.shape);
+  if (r.size() > 0)
+    check(detail::compare_(cmp, r.rank(), r.shape.data(), r.ptr(), r.strides.data(), a.ptr(), a.strides.data(), b.ptr(), b.strides.data()));
+  return r;
+}
+template <typename T>
+HipTensor<uint8_t> compare_scalar(int cmp, const HipTensor<T>& t, T value) {
+  HipTensor<uint8_t> r(t.shape);   // returnEmptyIfEmpty: an empty tensor comes back empty
+  if (r.size() > 0)
+    check(detail::compare_scalar_(cmp, r.rank(), r.shape.data(), r.ptr(), r.strides.data(), t.ptr(), t.strides.data(), value));
+  return r;
+}
+// `==.` `!=.` `<.` `<=.` `>.` `>=.` (operators_comparison.nim:41-185): tensor-tensor with implicit
+// broadcasting, tensor-scalar, and scalar-tensor (the mirrored tensor-scalar comparison, as in the reference).
+#define AM_HIP_COMPARISON(name, code, mirrored)                                                                  \
+  template <typename T> HipTensor<uint8_t> name(const HipTensor<T>& a, const HipTensor<T>& b) {                  \
+    auto p = broadcast2(a, b);                                                                                   \
+    return map2_bool(code, p.first, p.second);                                                                   \
+  }                                                                                                              \
+  template <typename T> HipTensor<uint8_t> name(const HipTensor<T>& t, T value) { return compare_scalar(code, t, value); } \
+  template <typename T> HipTensor<uint8_t> name(T value, const HipTensor<T>& t) { return compare_scalar(mirrored, t, value); }
+AM_HIP_COMPARISON(bc_eq, AM_CMP_EQ, AM_CMP_EQ) AM_HIP_COMPARISON(bc_ne, AM_CMP_NE, AM_CMP_NE)
+AM_HIP_COMPARISON(bc_lt, AM_CMP_LT, AM_CMP_GT) AM_HIP_COMPARISON(bc_le, AM_CMP_LE, AM_CMP_GE)
+AM_HIP_COMPARISON(bc_gt, AM_CMP_GT, AM_CMP_LT) AM_HIP_COMPARISON(bc_ge, AM_CMP_GE, AM_CMP_LE)
+#undef AM_HIP_COMPARISON
+template <typename T> HipTensor<uint8_t> predicate(int op, const HipTensor<T>& t) {
+  static_assert(std::is_floating_point<T>::value, "isNaN / isNotNaN / classify are defined for float tensors");
+  HipTensor<uint8_t> r(t.shape);
+  if (r.size() > 0) check(detail::predicate_(op, r.rank(), r.shape.data(), r.ptr(), r.strides.data(), t.ptr(), t.strides.data()));
+  return r;
+}
+template <typename T> HipTensor<uint8_t> isNaN(const HipTensor<T>& t) { return predicate(AM_PRED_ISNAN, t); }        // operators_comparison.nim:192-198
+template <typename T> HipTensor<uint8_t> isNotNaN(const HipTensor<T>& t) { return predicate(AM_PRED_ISNOTNAN, t); }  // :200-206
+// Ordinals of Nim's FloatClass: 0 fcNormal, 1 fcSubnormal, 2 fcZero, 3 fcNegZero, 4 fcNan, 5 fcInf, 6 fcNegInf (math_functions.nim:264-276)
+template <typename T> HipTensor<uint8_t> classify(const HipTensor<T>& t) { return predicate(AM_PRED_CLASSIFY, t); }
+// -1 / 0 / 1 as the reference's Tensor[int]; zeros and NaN give 0 (math_functions.nim:110-117)
+template <typename T> HipTensor<int64_t> sgn(const HipTensor<T>& t) {
+  HipTensor<int64_t> r(t.shape);
+  if (r.size() > 0) check(detail::sgn_(r.rank(), r.shape.data(), r.ptr(), r.strides.data(), t.ptr(), t.strides.data()));
+  return r;
+}
+// clamp (math_functions.nim:146-148): one pass, bounds by value
+template <typename T> HipTensor<T> clamp(const HipTensor<T>& t, T lo, T hi) {
+  HipTensor<T> r(t.shape);
+  if (r.size() > 0) check(detail::clamp_(r.rank(), r.shape.data(), r.ptr(), r.strides.data(), t.ptr(), t.strides.data(), lo, hi));
+  return r;
+}
+// floorMod (math_functions.nim:134-144) and copySign (:119-125)
+template <typename T> HipTensor<T> floorMod(const HipTensor<T>& a, const HipTensor<T>& b) { return map2(AM_OP_FLOORMOD, a, b); }
+template <typename T> HipTensor<T> floorMod(const HipTensor<T>& t, T value) { return scalar_op(AM_OP_FLOORMOD, t, value); }
+template <typename T> HipTensor<T> floorMod(T value, const HipTensor<T>& t) { return scalar_op(AM_OP_FLOORMOD, t, value, true); }
+template <typename T> HipTensor<T> copySign(const HipTensor<T>& a, const HipTensor<T>& b) { return map2(AM_OP_COPYSIGN, a, b); }
+
 // The universal functions (ufunc.nim:82-130) and reciprocal (math_functions.nim:52-58), float tensors.
 #define AM_HIP_UFUNC(name, code) \
   template <typename T> HipTensor<T> name(const HipTensor<T>& t) { return unary(code, t); }
@@ -360,6 +466,7 @@ AM_HIP_UFUNC(cbrt, AM_UOP_CBRT) AM_HIP_UFUNC(erf, AM_UOP_ERF) AM_HIP_UFUNC(erfc,
 AM_HIP_UFUNC(gamma, AM_UOP_GAMMA) AM_HIP_UFUNC(lgamma, AM_UOP_LGAMMA)
 AM_HIP_UFUNC(floor, AM_UOP_FLOOR) AM_HIP_UFUNC(ceil, AM_UOP_CEIL) AM_HIP_UFUNC(trunc, AM_UOP_TRUNC)
 AM_HIP_UFUNC(round, AM_UOP_ROUND) AM_HIP_UFUNC(reciprocal, AM_UOP_RECIPROCAL)
+AM_HIP_UFUNC(degToRad, AM_UOP_DEGTORAD) AM_HIP_UFUNC(radToDeg, AM_UOP_RADTODEG)
 #undef AM_HIP_UFUNC
 // map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass
 template <typename T> HipTensor<T> bias_relu(const HipTensor<T>& x, const HipTensor<T>& b) { return map2(AM_OP_ADD_RELU, x, b.broadcast(x.shape)); }
@@ -665,6 +772,188 @@ void write_npy(const HipTensor<T>& t, const std::string& path) {
   f.write(header.data(), (std::streamsize)hl);
   f.write((const char*)host.data(), (std::streamsize)(host.size() * sizeof(T)));
 }
+
+// ---- display (src/arraymancer/tensor/display_cuda.nim:19-36 over display.nim:19-115, private/p_display.nim:152-485) ----
+// A device tensor prints as its host copy laid out by the reference's CPU printer: table mode (specifier ""
+// or "||" / "<|>" / "<>||": last two dimensions as rows between `|`, odd dimensions side by side under their
+// index, even dimensions stacked with their index on the left), or array modes ("[]" one line, "[:]" one row
+// per line; "<>" / "<:>" / "<>[]" / "<>[:]" with a compact header). Floats print like printf's %g
+// (precision -1) or %#.{precision}g. Everything below formats host data; nothing runs on the device.
+namespace detail {
+inline std::string nim_type_name(float) { return "float32"; }
+inline std::string nim_type_name(double) { return "float"; }     // Nim's float is the 64-bit one
+inline std::string nim_type_name(int32_t) { return "int32"; }
+inline std::string nim_type_name(int64_t) { return "int"; }      // Nim's int is the 64-bit one here
+inline std::string nim_type_name(uint8_t) { return "bool"; }
+
+template <typename T> std::string disp_element(T v, int precision) {
+  char buf[64];
+  if constexpr (std::is_floating_point<T>::value) {
+    if (v != v) return "nan";
+    if (precision >= 0) std::snprintf(buf, sizeof(buf), "%#.*g", precision, (double)v);
+    else std::snprintf(buf, sizeof(buf), "%g", (double)v);
+    return buf;
+  } else if constexpr (std::is_same<T, uint8_t>::value) {
+    return v ? "true" : "false";
+  } else {
+    return std::to_string((long long)v);
+  }
+}
+inline std::vector<std::string> split_lines(const std::string& s) {   // "a\nb\n" -> {"a", "b", ""}
+  std::vector<std::string> out(1);
+  for (char c : s) { if (c == '\n') out.emplace_back(); else out.back() += c; }
+  return out;
+}
+inline std::string center(const std::string& s, size_t width) {       // the smaller padding on the left
+  if (width <= s.size()) return s;
+  const size_t left = (width - s.size()) / 2;
+  return std::string(left, ' ') + s + std::string(width - s.size() - left, ' ');
+}
+inline std::string strip(const std::string& s) {
+  const char* ws = " \t\n\r";
+  const size_t a = s.find_first_not_of(ws);
+  if (a == std::string::npos) return "";
+  return s.substr(a, s.find_last_not_of(ws) - a + 1);
+}
+inline std::string zip_strings(const std::string& s1, const std::string& s2, const std::string& sep, bool allow_empty) {
+  const auto a = split_lines(s1), b = split_lines(s2);
+  if (a.size() == 1) return s2;
+  if (b.size() == 1) return s1;
+  std::string out;
+  for (size_t i = 0; i < std::min(a.size(), b.size()); ++i) {
+    if (!allow_empty && a[i].empty() && b[i].empty()) continue;
+    out += a[i] + sep + b[i] + "\n";
+  }
+  return out;
+}
+inline std::string gen_sep(int rank, size_t line_len = 0, bool xaxis = false) {
+  std::string out;
+  for (int i = 2; i < rank; ++i) {
+    if (i % 2 == 0) out += xaxis ? std::string(line_len, '-') : std::string(" ");
+    else out += xaxis ? std::string(line_len, ' ') : std::string(" | ");
+    if (xaxis) out += "\n";
+  }
+  return out;
+}
+inline std::string left_idx(const std::string& ax, const std::string& s) {
+  const std::string c = center(ax + " ", split_lines(s).size());
+  std::vector<std::string> tmp(1);
+  for (char ch : c) { if (ch == ' ') tmp.emplace_back(); else tmp.back() += ch; }
+  std::string out;
+  const size_t high = tmp.size() - 1;
+  for (size_t i = 0; i < high; ++i) {
+    out += tmp[i].empty() ? std::string(ax.size(), ' ') + " " : tmp[i] + " ";
+    if (i + 1 < high) out += "\n";
+  }
+  return out;
+}
+inline std::string pad_left(const std::string& v, int w) { return (int)v.size() >= w ? v : std::string(w - v.size(), ' ') + v; }
+inline std::string pad_right(const std::string& v, int w) { return (int)v.size() >= w ? v : v + std::string(w - v.size(), ' '); }
+
+// `data` holds the elements of a tensor of `shape` in C order.
+template <typename T>
+std::string disp_table(const T* data, Shape shape, int input_rank, int align_by, int precision) {
+  const int align_spacing = 4;
+  int64_t n = 1;
+  for (auto e : shape) n *= e;
+  if (input_rank == 0) {
+    input_rank = (int)shape.size();
+    size_t largest = 0;
+    for (int64_t i = 0; i < n; ++i) largest = std::max(largest, disp_element(data[i], precision).size());
+    align_by = std::max(6, (int)largest + align_spacing);
+  }
+  if (shape.size() <= 2) {
+    std::string out;
+    const int64_t cols = shape.size() == 2 ? shape[1] : 0;
+    for (int64_t idx = 1; idx <= n; ++idx) {
+      const std::string val = disp_element(data[idx - 1], precision);
+      if (cols == 0) out += pad_left(val, align_by);
+      else if (idx % cols == 0) out += cols == 1 ? "|" + pad_left(val, align_by - align_spacing) + "|\n" : pad_left(val, align_by) + "|\n";
+      else if (idx % cols == 1) out += "|" + pad_right(val, align_by - align_spacing);
+      else out += pad_left(val, align_by);
+    }
+    return strip(out);
+  }
+  const int rank = (int)shape.size();
+  const bool odd = rank % 2 != 0;
+  Shape sub(shape.begin() + 1, shape.end());
+  sub.erase(std::remove(sub.begin(), sub.end(), (int64_t)1), sub.end());   // squeeze
+  if (sub.empty()) sub.push_back(1);
+  const int64_t sub_n = n / shape[0];
+  std::string res;
+  for (int64_t ax = 0; ax < shape[0]; ++ax) {
+    std::string part = disp_table(data + ax * sub_n, sub, input_rank, align_by, precision);
+    if (odd) {
+      part = center(std::to_string(ax), split_lines(part)[0].size()) + "\n" + part;
+      res = zip_strings(res, part, gen_sep(rank), false);
+    } else {
+      res += zip_strings(left_idx(std::to_string(ax), part), part, "", true);
+    }
+  }
+  if (odd && rank != input_rank) res += gen_sep(rank, split_lines(res)[0].size(), true);
+  return res;
+}
+
+template <typename T>
+std::string disp_array(const T* data, Shape shape, int precision, const std::string& row_sep) {
+  if (shape.size() <= 1) {
+    const int64_t n = shape.empty() ? 1 : shape[0];
+    std::string out = "[";
+    for (int64_t i = 0; i < n; ++i) out += (i ? ", " : "") + disp_element(data[i], precision);
+    return out + "]";
+  }
+  int64_t sub_n = 1;
+  for (size_t i = 1; i < shape.size(); ++i) sub_n *= shape[i];
+  const Shape sub(shape.begin() + 1, shape.end());
+  std::string out = "[";
+  for (int64_t i = 0; i < shape[0]; ++i) {
+    if (i) out += ", " + row_sep;
+    out += disp_array(data + i * sub_n, sub, precision, row_sep);
+  }
+  return out + "]";
+}
+}  // namespace detail
+
+// prettyImpl for host data of `shape` in C order; `type_name` / `backend` go into the header.
+template <typename T>
+std::string pretty_host(const std::vector<T>& host, const Shape& shape, const std::string& type_name, const std::string& backend,
+                        int precision = -1, const std::string& specifier = "") {
+  int mode;      // 0 table, 1 single line, 2 one row per line
+  bool header;
+  if (specifier == "" || specifier == "<|>" || specifier == "<>||") { mode = 0; header = true; }
+  else if (specifier == "||") { mode = 0; header = false; }
+  else if (specifier == "[]") { mode = 1; header = false; }
+  else if (specifier == "<>[]" || specifier == "<>") { mode = 1; header = true; }
+  else if (specifier == "[:]") { mode = 2; header = false; }
+  else if (specifier == "<>[:]" || specifier == "<:>") { mode = 2; header = true; }
+  else throw std::invalid_argument("Invalid tensor format specifier (" + specifier + ")");
+  const std::string elem = detail::nim_type_name(T());
+  if (mode != 0) {
+    std::string compact = type_name + "[" + elem + "]<";
+    for (size_t i = 0; i < shape.size(); ++i) compact += (i ? "," : "") + std::to_string(shape[i]);
+    compact += ">";
+    if (mode == 1) return (header ? compact + ":" : "") + detail::disp_array(host.data(), shape, precision, "");
+    std::string body;
+    for (const std::string& line : detail::split_lines(detail::disp_array(host.data(), shape, precision, "\n"))) {
+      const size_t brackets = line.find_first_not_of('[') == std::string::npos ? line.size() : line.find_first_not_of('[');
+      body += (line.empty() ? "" : std::string(shape.size() > brackets ? shape.size() - brackets : 0, ' ')) + line + "\n";
+    }
+    while (!body.empty() && (body.back() == '\n' || body.back() == ' ')) body.pop_back();
+    return (header ? compact + ":\n" : "") + body;
+  }
+  const std::string desc = header ? type_name + "[system." + elem + "] of shape \"" + detail::str(shape) + "\" on backend \"" + backend + "\"\n" : "";
+  if (host.empty()) return desc + "    [] (empty)";
+  if (shape.size() == 1) return desc + "    " + detail::disp_table(host.data(), shape, 0, 0, precision);
+  return desc + detail::disp_table(host.data(), shape, 0, 0, precision);
+}
+
+// t.pretty(precision) / `$t` for a device tensor.
+template <typename T>
+std::string pretty(const HipTensor<T>& t, int precision = -1, const std::string& specifier = "") {
+  return pretty_host(t.toCpu(), t.shape, "HipTensor", "Hip", precision, specifier);
+}
+template <typename T>
+std::ostream& operator<<(std::ostream& os, const HipTensor<T>& t) { return os << pretty(t); }
 
 inline void sync() { check(am_hip_sync()); }
 

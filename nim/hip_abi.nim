@@ -150,13 +150,17 @@ type
   AmBinaryOp* {.size: sizeof(cint).} = enum
     opAdd = 0, opSub = 1, opMul = 2, opDiv = 3, opMod = 4, opAddRelu = 5, opAddSigmoid = 6,
     opAddTanh = 7, opReluBwd = 8, opMax = 9, opMin = 10, opSigmoidBwd = 11, opTanhBwd = 12, opSqDiff = 13,
-    opPow = 14
+    opPow = 14, opFloorMod = 15, opCopySign = 16
+  AmCompareOp* {.size: sizeof(cint).} = enum   # results are Tensor[bool]: one byte per element
+    cmpEq = 0, cmpNe = 1, cmpLt = 2, cmpLe = 3, cmpGt = 4, cmpGe = 5, cmpModIsZero = 6
+  AmPredicate* {.size: sizeof(cint).} = enum
+    predIsNaN = 0, predIsNotNaN = 1, predClassify = 2
   AmUnaryOp* {.size: sizeof(cint).} = enum
     uopCopy = 0, uopNeg = 1, uopRelu = 2, uopSigmoid = 3, uopTanh = 4, uopExp = 5, uopAbs = 6, uopSqrt = 7, uopSquare = 8,
     uopLn = 9, uopLog10 = 10, uopLog2 = 11, uopSin = 12, uopCos = 13, uopTan = 14, uopSinh = 15, uopCosh = 16,
     uopArcsin = 17, uopArccos = 18, uopArctan = 19, uopArcsinh = 20, uopArccosh = 21, uopArctanh = 22, uopCbrt = 23,
     uopErf = 24, uopErfc = 25, uopGamma = 26, uopLgamma = 27, uopFloor = 28, uopCeil = 29, uopTrunc = 30,
-    uopRound = 31, uopReciprocal = 32
+    uopRound = 31, uopReciprocal = 32, uopDegToRad = 33, uopRadToDeg = 34
 
 proc am_hip_ew_binary_f32*(op: cint, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
                            a: ptr cfloat, a_strides: ptr int64, b: ptr cfloat, b_strides: ptr int64): cint {.importc.}
@@ -197,6 +201,44 @@ proc am_hip_ew_unary_i32*(op, rank: cint, shape: ptr int64, dst: ptr int32, dst_
                           a: ptr int32, a_strides: ptr int64): cint {.importc.}
 proc am_hip_ew_unary_i64*(op, rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
                           a: ptr int64, a_strides: ptr int64): cint {.importc.}
+
+# map bodies whose result type differs from the operands' (comparisons -> bool, sgn -> int), clamp with bounds by value
+proc am_hip_ew_compare_f32*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                            a: ptr cfloat, a_strides: ptr int64, b: ptr cfloat, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_compare_f64*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                            a: ptr cdouble, a_strides: ptr int64, b: ptr cdouble, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_compare_i32*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                            a: ptr int32, a_strides: ptr int64, b: ptr int32, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_compare_i64*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                            a: ptr int64, a_strides: ptr int64, b: ptr int64, b_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_compare_scalar_f32*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                                   a: ptr cfloat, a_strides: ptr int64, scalar: cfloat): cint {.importc.}
+proc am_hip_ew_compare_scalar_f64*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                                   a: ptr cdouble, a_strides: ptr int64, scalar: cdouble): cint {.importc.}
+proc am_hip_ew_compare_scalar_i32*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                                   a: ptr int32, a_strides: ptr int64, scalar: int32): cint {.importc.}
+proc am_hip_ew_compare_scalar_i64*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                                   a: ptr int64, a_strides: ptr int64, scalar: int64): cint {.importc.}
+proc am_hip_ew_predicate_f32*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                              a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_predicate_f64*(op, rank: cint, shape: ptr int64, dst: ptr uint8, dst_strides: ptr int64,
+                              a: ptr cdouble, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_sgn_f32*(rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                        a: ptr cfloat, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_sgn_f64*(rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                        a: ptr cdouble, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_sgn_i32*(rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                        a: ptr int32, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_sgn_i64*(rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                        a: ptr int64, a_strides: ptr int64): cint {.importc.}
+proc am_hip_ew_clamp_f32*(rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
+                          a: ptr cfloat, a_strides: ptr int64, lo, hi: cfloat): cint {.importc.}
+proc am_hip_ew_clamp_f64*(rank: cint, shape: ptr int64, dst: ptr cdouble, dst_strides: ptr int64,
+                          a: ptr cdouble, a_strides: ptr int64, lo, hi: cdouble): cint {.importc.}
+proc am_hip_ew_clamp_i32*(rank: cint, shape: ptr int64, dst: ptr int32, dst_strides: ptr int64,
+                          a: ptr int32, a_strides: ptr int64, lo, hi: int32): cint {.importc.}
+proc am_hip_ew_clamp_i64*(rank: cint, shape: ptr int64, dst: ptr int64, dst_strides: ptr int64,
+                          a: ptr int64, a_strides: ptr int64, lo, hi: int64): cint {.importc.}
 
 {.pop.}
 

@@ -25,17 +25,20 @@ import std/math                                     # scalar sqrt for `std`
 
 type
   HipScalar* = float32 | float64 | int32 | int64
+  HipElem* = HipScalar | bool | uint8
+    ## what a HipTensor can hold: the four arithmetic types, plus bool (one byte, the result of the
+    ## comparison family) and uint8 (FloatClass ordinals of `classify`) as result-only element types
 
-  HipRefTrackerObj*[T: HipScalar] = object
+  HipRefTrackerObj*[T: HipElem] = object
     value*: ptr UncheckedArray[T]
   HipRefTracker*[T] = ref HipRefTrackerObj[T]
 
-  HipStorage*[T: HipScalar] = object
+  HipStorage*[T: HipElem] = object
     Flen*: int
     Fdata*: ptr UncheckedArray[T]
     Fref_tracking*: HipRefTracker[T]
 
-  HipTensor*[T: HipScalar] = object
+  HipTensor*[T: HipElem] = object
     ## Same fields as Tensor / CudaTensor: views share `storage`; shape, strides, offset in elements.
     shape*: Metadata
     strides*: Metadata
@@ -47,7 +50,7 @@ proc `=destroy`*[T](p: HipRefTrackerObj[T]) =
     discard am_hip_free(p.value)
 
 # ---------------------------------------------------------------- allocation / metadata
-proc newHipStorage[T: HipScalar](length: int): HipStorage[T] =
+proc newHipStorage[T: HipElem](length: int): HipStorage[T] =
   result.Flen = length
   new result.Fref_tracking
   var p: pointer
@@ -58,7 +61,7 @@ proc newHipStorage[T: HipScalar](length: int): HipStorage[T] =
 proc size*(t: HipTensor): int {.inline.} = t.shape.product
 proc rank*(t: HipTensor): int {.inline.} = t.shape.len
 
-proc newHipTensor*[T: HipScalar](shape: varargs[int] | Metadata): HipTensor[T] =
+proc newHipTensor*[T: HipElem](shape: varargs[int] | Metadata): HipTensor[T] =
   ## Row-major, uninitialised.
   result.shape.copyFrom(shape)
   shape_to_strides(result.shape, rowMajor, result.strides)
@@ -201,6 +204,122 @@ proc clone*[T](t: HipTensor[T]): HipTensor[T] =
   result = newHipTensor[T](t.shape)
   if result.size > 0: ewUnary(T, uopCopy, result, t)
 
+# ---------------------------------------------------------------- map bodies with another result type
+# map_inline / map2_inline infer the result type from the body (higher_order_applymap.nim:69-120); over a C ABI
+# the bodies are enumerated: the comparison family -> Tensor[bool], sgn -> Tensor[int], classify -> FloatClass.
+template ewCompare(T: typedesc, op: AmCompareOp, dst, a, b: untyped) =
+  var sh = i64s(dst.shape)
+  var sd = i64s(dst.strides)
+  var sa = i64s(a.strides)
+  var sb = i64s(b.strides)
+  let d = cast[ptr uint8](dst.get_offset_ptr)
+  when T is float32:
+    check am_hip_ew_compare_f32(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+  elif T is float64:
+    check am_hip_ew_compare_f64(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+  elif T is int32:
+    check am_hip_ew_compare_i32(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+  else:
+    check am_hip_ew_compare_i64(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, b.get_offset_ptr, sb[0].addr)
+
+template ewCompareScalar(T: typedesc, op: AmCompareOp, dst, a: untyped, s: untyped) =
+  var sh = i64s(dst.shape)
+  var sd = i64s(dst.strides)
+  var sa = i64s(a.strides)
+  let d = cast[ptr uint8](dst.get_offset_ptr)
+  when T is float32:
+    check am_hip_ew_compare_scalar_f32(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+  elif T is float64:
+    check am_hip_ew_compare_scalar_f64(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+  elif T is int32:
+    check am_hip_ew_compare_scalar_i32(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+  else:
+    check am_hip_ew_compare_scalar_i64(cint(op), cint(dst.rank), sh[0].addr, d, sd[0].addr, a.get_offset_ptr, sa[0].addr, s)
+
+proc map2*[T: HipScalar](a: HipTensor[T], op: AmCompareOp, b: HipTensor[T]): HipTensor[bool] =
+  ## map2_inline with a bool-valued body, e.g. `map2(a, cmpModIsZero, b)` for `x mod y == 0`
+  ## (tests/tensor/test_higherorder.nim:103-112).
+  check_elementwise(a, b)
+  result = newHipTensor[bool](a.shape)
+  if result.size > 0: ewCompare(T, op, result, a, b)
+
+proc compareScalar[T: HipScalar](t: HipTensor[T], op: AmCompareOp, value: T): HipTensor[bool] =
+  result = newHipTensor[bool](t.shape)          # returnEmptyIfEmpty: an empty tensor comes back empty
+  if result.size > 0: ewCompareScalar(T, op, result, t, value)
+
+template genComparison(opName: untyped, code, mirrored: AmCompareOp) =
+  ## operators_comparison.nim:41-94 (tensor, tensor: broadcast2 then map2_inline), :111-146 (tensor, scalar),
+  ## :150-185 (scalar, tensor: the mirrored comparison of the tensor)
+  proc opName*[T: HipScalar](a, b: HipTensor[T]): HipTensor[bool] =
+    let (x, y) = broadcast2(a, b)
+    map2(x, code, y)
+  proc opName*[T: HipScalar](t: HipTensor[T], value: T): HipTensor[bool] = compareScalar(t, code, value)
+  proc opName*[T: HipScalar](value: T, t: HipTensor[T]): HipTensor[bool] = compareScalar(t, mirrored, value)
+
+genComparison(`==.`, cmpEq, cmpEq)
+genComparison(`!=.`, cmpNe, cmpNe)
+genComparison(`<.`, cmpLt, cmpGt)
+genComparison(`<=.`, cmpLe, cmpGe)
+genComparison(`>.`, cmpGt, cmpLt)
+genComparison(`>=.`, cmpGe, cmpLe)
+
+proc predicate[T: float32 | float64; D: bool | uint8](t: HipTensor[T], op: AmPredicate): HipTensor[D] =
+  result = newHipTensor[D](t.shape)
+  if result.size > 0:
+    var sh = i64s(t.shape)
+    var sd = i64s(result.strides)
+    var sa = i64s(t.strides)
+    let d = cast[ptr uint8](result.get_offset_ptr)
+    when T is float32:
+      check am_hip_ew_predicate_f32(cint(op), cint(t.rank), sh[0].addr, d, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+    else:
+      check am_hip_ew_predicate_f64(cint(op), cint(t.rank), sh[0].addr, d, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+
+proc isNaN*[T: float32 | float64](t: HipTensor[T]): HipTensor[bool] = predicate[T, bool](t, predIsNaN)        ## operators_comparison.nim:192-198
+proc isNotNaN*[T: float32 | float64](t: HipTensor[T]): HipTensor[bool] = predicate[T, bool](t, predIsNotNaN)  ## :200-206
+proc classify*[T: float32 | float64](t: HipTensor[T]): HipTensor[uint8] = predicate[T, uint8](t, predClassify)
+  ## ord(FloatClass) per element (math_functions.nim:264-276); `FloatClass(v)` converts a copied-back value
+
+proc sgn*[T: HipScalar](t: HipTensor[T]): HipTensor[int64] =
+  ## math_functions.nim:110-117: -1 / 0 / 1, zeros of either sign and NaN give 0
+  result = newHipTensor[int64](t.shape)
+  if result.size > 0:
+    var sh = i64s(t.shape)
+    var sd = i64s(result.strides)
+    var sa = i64s(t.strides)
+    when T is float32: check am_hip_ew_sgn_f32(cint(t.rank), sh[0].addr, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+    elif T is float64: check am_hip_ew_sgn_f64(cint(t.rank), sh[0].addr, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+    elif T is int32: check am_hip_ew_sgn_i32(cint(t.rank), sh[0].addr, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+    else: check am_hip_ew_sgn_i64(cint(t.rank), sh[0].addr, result.get_offset_ptr, sd[0].addr, t.get_offset_ptr, sa[0].addr)
+
+template ewClamp(T: typedesc, dst, a: untyped, lo, hi: untyped) =
+  var sh = i64s(dst.shape)
+  var sd = i64s(dst.strides)
+  var sa = i64s(a.strides)
+  when T is float32: check am_hip_ew_clamp_f32(cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, lo, hi)
+  elif T is float64: check am_hip_ew_clamp_f64(cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, lo, hi)
+  elif T is int32: check am_hip_ew_clamp_i32(cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, lo, hi)
+  else: check am_hip_ew_clamp_i64(cint(dst.rank), sh[0].addr, dst.get_offset_ptr, sd[0].addr, a.get_offset_ptr, sa[0].addr, lo, hi)
+
+proc clamp*[T: HipScalar](t: HipTensor[T], min, max: T): HipTensor[T] =
+  ## math_functions.nim:146-148; both bounds travel by value, one pass
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewClamp(T, result, t, min, max)
+
+proc mclamp*[T: HipScalar](t: var HipTensor[T], min, max: T) =
+  ## math_functions.nim:150-152
+  if t.size > 0: ewClamp(T, t, t, min, max)
+
+proc floorMod*[T: HipScalar](t1, t2: HipTensor[T]): HipTensor[T] = map2(t1, opFloorMod, t2)      ## math_functions.nim:134-136
+proc floorMod*[T: HipScalar](t: HipTensor[T], val: T): HipTensor[T] =                              ## :138-140
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opFloorMod, false, result, t, val)
+proc floorMod*[T: HipScalar](val: T, t: HipTensor[T]): HipTensor[T] =                              ## :142-144
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewScalar(T, opFloorMod, true, result, t, val)
+proc copySign*[T: float32 | float64](t1, t2: HipTensor[T]): HipTensor[T] = map2(t1, opCopySign, t2)   ## :119-125
+proc mcopySign*[T: float32 | float64](t1: var HipTensor[T], t2: HipTensor[T]) = apply2(t1, opCopySign, t2)   ## :127-132
+
 # ---------------------------------------------------------------- BLAS L1-like operators
 proc `+`*[T](a, b: HipTensor[T]): HipTensor[T] = map2(a, opAdd, b)
 proc `-`*[T](a, b: HipTensor[T]): HipTensor[T] = map2(a, opSub, b)
@@ -302,6 +421,8 @@ makeHipUniversal(ceil, uopCeil)
 makeHipUniversal(trunc, uopTrunc)
 makeHipUniversal(round, uopRound)
 makeHipUniversal(reciprocal, uopReciprocal)   # math_functions.nim:52-54
+makeHipUniversal(degToRad, uopDegToRad)       # ufunc.nim:129
+makeHipUniversal(radToDeg, uopRadToDeg)       # ufunc.nim:130
 proc mreciprocal*[T: float32 | float64](t: var HipTensor[T]) =
   ## math_functions.nim:56-58
   if t.size > 0: ewUnary(T, uopReciprocal, t, t)

@@ -27,12 +27,14 @@ _CT = {"f32": ctypes.c_float, "f64": ctypes.c_double, "i32": ctypes.c_int32, "i6
 
 # op codes of include/am_hip.h
 OP = dict(add=0, sub=1, mul=2, div=3, mod=4, add_relu=5, add_sigmoid=6, add_tanh=7,
-          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12, sqdiff=13, pow=14)
+          relu_bwd=8, max=9, min=10, sigmoid_bwd=11, tanh_bwd=12, sqdiff=13, pow=14, floormod=15, copysign=16)
+CMP = {"==": 0, "!=": 1, "<": 2, "<=": 3, ">": 4, ">=": 5, "mod_is_zero": 6}
+PRED = dict(isnan=0, isnotnan=1, classify=2)
 OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2, addmul=3, clamp=4)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6, sqrt=7, square=8,
            ln=9, log10=10, log2=11, sin=12, cos=13, tan=14, sinh=15, cosh=16, arcsin=17,
            arccos=18, arctan=19, arcsinh=20, arccosh=21, arctanh=22, cbrt=23, erf=24, erfc=25, gamma=26,
-           lgamma=27, floor=28, ceil=29, trunc=30, round=31, reciprocal=32)
+           lgamma=27, floor=28, ceil=29, trunc=30, round=31, reciprocal=32, degtorad=33, radtodeg=34)
 
 
 def build(force: bool = False) -> str:
@@ -68,6 +70,12 @@ def lib() -> ctypes.CDLL:
             f = getattr(L, f"am_oracle_unary_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, p, p, p, p]
+            f = getattr(L, f"am_oracle_compare_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, p, p, p, p, p, p]
+            f = getattr(L, f"am_oracle_sgn_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, p, p, p, p, p]
             f = getattr(L, f"am_oracle_reduce_axis_{sfx}")
             f.restype = ci
             f.argtypes = [ci, ci, p, ci, p, p, p, p]
@@ -84,6 +92,9 @@ def lib() -> ctypes.CDLL:
             f.restype = ci
             f.argtypes = [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, p, p, p, ct]
         for sfx in ("f32", "f64"):
+            f = getattr(L, f"am_oracle_predicate_{sfx}")
+            f.restype = ci
+            f.argtypes = [ci, ci, p, p, p, p, p]
             f = getattr(L, f"am_oracle_softmax_rows_{sfx}")
             f.restype = ci
             f.argtypes = [i64, i64, p, i64, i64, p, i64, i64]
@@ -193,6 +204,41 @@ def map2(op, a: np.ndarray, b: np.ndarray, out: np.ndarray | None = None) -> np.
         a.ctypes.data, _i64arr(_estrides(a)), b.ctypes.data, _i64arr(_estrides(b)))
     if rc != 0:
         raise ValueError(f"oracle map2: op {op} not defined for {a.dtype} (rc={rc})")
+    return out
+
+
+def compare(cmp, a: np.ndarray, b) -> np.ndarray:
+    """Bool tensor of a[i] cmp b[i] (equal shapes, or b a scalar seen through zero strides): the broadcast
+    comparison family and `x mod y == 0`."""
+    if not isinstance(b, np.ndarray):
+        b = np.broadcast_to(np.asarray(b, dtype=a.dtype), a.shape)
+    assert a.shape == b.shape and a.dtype == b.dtype
+    out = np.empty(a.shape, dtype=np.uint8)
+    rc = getattr(lib(), f"am_oracle_compare_{_sfx(a)}")(
+        CMP[cmp], a.ndim, _i64arr(a.shape), out.ctypes.data, _i64arr(_estrides(out)),
+        a.ctypes.data, _i64arr(_estrides(a)), b.ctypes.data, _i64arr(_estrides(b)))
+    if rc != 0:
+        raise ValueError(f"oracle compare: rc={rc}")
+    return out.view(np.bool_)
+
+
+def predicate(pred, a: np.ndarray) -> np.ndarray:
+    """isnan / isnotnan (bool) or classify (uint8 ordinals of Nim's FloatClass) of a float tensor."""
+    out = np.empty(a.shape, dtype=np.uint8)
+    rc = getattr(lib(), f"am_oracle_predicate_{_sfx(a)}")(
+        PRED[pred], a.ndim, _i64arr(a.shape), out.ctypes.data, _i64arr(_estrides(out)),
+        a.ctypes.data, _i64arr(_estrides(a)))
+    if rc != 0:
+        raise ValueError(f"oracle predicate: rc={rc}")
+    return out if pred == "classify" else out.view(np.bool_)
+
+
+def sgn(a: np.ndarray) -> np.ndarray:
+    out = np.empty(a.shape, dtype=np.int64)
+    rc = getattr(lib(), f"am_oracle_sgn_{_sfx(a)}")(
+        a.ndim, _i64arr(a.shape), out.ctypes.data, _i64arr(_estrides(out)), a.ctypes.data, _i64arr(_estrides(a)))
+    if rc != 0:
+        raise ValueError(f"oracle sgn: rc={rc}")
     return out
 
 

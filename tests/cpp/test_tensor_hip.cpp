@@ -262,6 +262,65 @@ static void aggregates() {
   CHECK(mp.max_indices.toCpu() == (std::vector<int64_t>{5, 7, 8, 15}));
 }
 
+static void comparisons_and_predicates() {
+  using U8 = std::vector<uint8_t>;
+  // tests/tensor/test_higherorder.nim:103-112: a map body with a bool result, one device pass
+  auto a = toHip<int64_t>({10, 2, 4, 12}, {4});
+  auto b = toHip<int64_t>({4, 4, 4, 4}, {4});
+  CHECK(am::map2_bool(AM_CMP_MOD_IS_ZERO, a, b).toCpu() == (U8{0, 0, 1, 1}));
+  // tests/tensor/test_operators_comparison.nim:57-79
+  auto x = toHip<int32_t>({0, 1, 2, 3}, {4});
+  auto y = toHip<int32_t>({0, 2, 1, 3}, {4});
+  CHECK(am::bc_eq(x, y).toCpu() == (U8{1, 0, 0, 1}));
+  CHECK(am::bc_lt(x, y).toCpu() == (U8{0, 1, 0, 0}));
+  CHECK(am::bc_ge(x, 2).toCpu() == (U8{0, 0, 1, 1}));
+  CHECK(am::bc_le(2, x).toCpu() == (U8{0, 0, 1, 1}));
+  // implicit broadcasting [4,1] vs [1,3]
+  auto c = toHip<double>({0, 1, 2, 3}, {4, 1});
+  auto d = toHip<double>({0, 1, 2}, {1, 3});
+  auto gt = am::bc_gt(c, d);
+  CHECK(gt.shape == (Shape{4, 3}) && gt.toCpu() == (U8{0, 0, 0, 1, 0, 0, 1, 1, 0, 1, 1, 1}));
+  EXPECT_THROW(am::bc_eq(toHip<double>(std::vector<double>(8, 0), {4, 2}), d), std::invalid_argument);
+  // tests/tensor/test_math_functions.nim:115-164
+  auto s = toHip<double>({-5.3, 42.0, -0.0, 0.01, 10.7, -0.001, 0.9, -125.3}, {8});
+  CHECK(am::sgn(s).toCpu() == (std::vector<int64_t>{-1, 1, 0, 1, 1, -1, 1, -1}));
+  const double inf = 1.0 / 0.0, nan = std::nan("");
+  auto f = toHip<double>({0.0, -0.0, inf, -inf, nan}, {5});
+  CHECK(am::isNaN(f).toCpu() == (U8{0, 0, 0, 0, 1}) && am::isNotNaN(f).toCpu() == (U8{1, 1, 1, 1, 0}));
+  CHECK(am::classify(f).toCpu() == (U8{2, 3, 5, 6, 4}));   // fcZero, fcNegZero, fcInf, fcNegInf, fcNan
+  // test_math_functions.nim:62-68 clamp / mclamp
+  auto k = toHip<int64_t>({-5, 2, 3, 5, 10, 0, 1, -1}, {8});
+  CHECK(eq(am::clamp(k, int64_t(-2), int64_t(2)), {-2, 2, 2, 2, 2, 0, 1, -1}));
+  k.mclamp(-2, 2);
+  CHECK(eq(k, {-2, 2, 2, 2, 2, 0, 1, -1}));
+  // :125-130 floorMod on arange(-70.7, 50.0, 34.7), :119-123 copySign
+  auto m = toHip<double>({-70.7, -36.0, -1.3, 33.4}, {4});
+  const std::vector<double> ts = am::floorMod(m, 3.0).toCpu(), st = am::floorMod(3.0, m).toCpu();
+  const double wts[4] = {1.3, -0.0, 1.7, 0.4}, wst[4] = {-67.7, -33.0, -0.9, 3.0};
+  for (int i = 0; i < 4; ++i) CHECK(std::fabs(ts[i] - wts[i]) < 1e-9 && std::fabs(st[i] - wst[i]) < 1e-9);
+  CHECK(eq(am::copySign(toHip<double>({-5.3, 42.0, 0.9}, {3}), toHip<double>({-4.0, -3.0, 2.0}, {3})), {-5.3, -42.0, 0.9}));
+  CHECK(eq(am::degToRad(toHip<double>({180.0, 0.0}, {2})), {3.14159265358979323846, 0.0}));
+}
+
+static void display() {
+  // tests/tensor/test_display.nim:143-151 (3D table) and :85-92 (single column), on device tensors
+  std::vector<int64_t> v(24);
+  for (int i = 0; i < 24; ++i) v[i] = i + 1;
+  const std::string got = am::pretty(toHip<int64_t>(v, {2, 3, 4}));
+  const std::string want =
+      "HipTensor[system.int] of shape \"[2, 3, 4]\" on backend \"Hip\"\n"
+      "          0                      1           \n"
+      "|1      2     3     4| |13    14    15    16|\n"
+      "|5      6     7     8| |17    18    19    20|\n"
+      "|9     10    11    12| |21    22    23    24|\n";
+  CHECK(got == want);
+  auto col = toHip<int64_t>({1, 2, 3, 4, 5}, {1, 5}).transpose();   // a strided view: gathered on the device first
+  CHECK(am::pretty(col, -1, "||") == "| 1|\n| 2|\n| 3|\n| 4|\n| 5|");
+  CHECK(am::pretty(col, -1, "<>") == "HipTensor[int]<5,1>:[[1], [2], [3], [4], [5]]");
+  CHECK(am::pretty(am::bc_ge(toHip<float>({0.5f, 2.0f}, {2}), 1.0f), -1, "<>") == "HipTensor[bool]<2>:[false, true]");
+  CHECK(am::pretty(toHip<float>({0.9532932f, 0.12945823f}, {2}), 4, "[]") == "[0.9533, 0.1295]");
+}
+
 static void softmax_rows() {
   auto x = toHip<double>({1, 2, 3, 1000, 1000, 1000}, {2, 3});
   const std::vector<double> s = am::softmax(x).toCpu();
@@ -325,6 +384,8 @@ int main(int argc, char** argv) {
     aggregates<int32_t>();
     aggregates<int64_t>();
     softmax_rows();
+    comparisons_and_predicates();
+    display();
     if (argc > 1) npy_files(argv[1]);
     am::sync();
   } catch (const std::exception& e) {

@@ -34,6 +34,99 @@ def test_nim_and_cpp_host_layers_bind_every_declared_symbol():
     assert '#include "am_hip.h"' in open(os.path.join(ROOT, "include", "am_hip_tensor.hpp")).read()
 
 
+_C2NIM = {"int": "cint", "int64_t": "int64", "int32_t": "int32", "uint8_t": "uint8", "float": "cfloat", "double": "cdouble",
+          "size_t": "csize_t", "void*": "pointer", "char*": "cstring", "void**": "ptr pointer"}
+
+
+def _c_type_as_nim(ctype: str) -> str:
+    t = re.sub(r"\bconst\b", "", ctype).replace(" ", "")
+    if t in _C2NIM:
+        return _C2NIM[t]
+    if t.endswith("*"):
+        return "ptr " + _c_type_as_nim(t[:-1])
+    raise AssertionError(f"no Nim spelling known for C type {ctype!r}")
+
+
+def c_prototypes():
+    """name -> (result type, [parameter types]) of every prototype in include/am_hip.h, spelled as Nim types."""
+    text = open(os.path.join(ROOT, "include", "am_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^\s*#[^\n]*$", "", text, flags=re.M)                    # preprocessor lines
+    text = text.replace('extern "C" {', "")
+    out = {}
+    for stmt in text.split(";"):
+        m = re.match(r"^([\w\s\*]+?)\b(am_hip_\w+)\s*\(([^)]*)\)\s*$", stmt.strip(), flags=re.S)
+        if not m:
+            continue
+        res, name, params = m.group(1).strip(), m.group(2), m.group(3).strip()
+        types = []
+        if params != "void":
+            for prm in params.split(","):
+                pm = re.match(r"^(.*?)(\w+)$", prm.strip(), flags=re.S)   # the type is everything before the parameter's name
+                types.append(_c_type_as_nim(pm.group(1)))
+        out[name] = (_c_type_as_nim(res), types)
+    return out
+
+
+def nim_prototypes():
+    """name -> (result type, [parameter types]) of every importc proc in nim/hip_abi.nim."""
+    text = open(os.path.join(ROOT, "nim", "hip_abi.nim")).read()
+    text = re.sub(r"#[^\n]*", "", text)
+    out = {}
+    for m in re.finditer(r"proc (am_hip_\w+)\*\(([^)]*)\)\s*(?::\s*([\w ]+?))?\s*\{\.importc\.\}", text, flags=re.S):
+        name, params, res = m.group(1), m.group(2), (m.group(3) or "void").strip()
+        types, pending = [], 0
+        for piece in re.split(r"[;,]", params):
+            piece = piece.strip()
+            if not piece:
+                continue
+            if ":" in piece:            # `a, b, c: T` declares three parameters of type T
+                types.extend([" ".join(piece.split(":", 1)[1].split())] * (pending + 1))
+                pending = 0
+            else:
+                pending += 1
+        assert pending == 0, name
+        out[name] = (res, types)
+    return out
+
+
+def test_nim_binding_matches_the_header_type_for_type():
+    """Arity and the C type of every parameter and result of nim/hip_abi.nim against include/am_hip.h (the Nim
+    file cannot be compiled here, so this is the check that a swapped or mistyped parameter fails)."""
+    c, nim = c_prototypes(), nim_prototypes()
+    assert sorted(c) == declared_symbols()
+    assert sorted(nim) == sorted(c)
+    for name, (res, types) in c.items():
+        nres, ntypes = nim[name]
+        assert len(ntypes) == len(types), f"{name}: {len(ntypes)} parameters in Nim, {len(types)} in C"
+        for i, (a, b) in enumerate(zip(types, ntypes)):
+            assert a == b, f"{name}: parameter {i} is {b} in Nim, {a} in C"
+        assert nres == res, f"{name}: result {nres} in Nim, {res} in C"
+
+
+def test_ctypes_binding_matches_the_header_arity():
+    c = c_prototypes()
+    for name, (res, args) in _lib.SIGNATURES.items():
+        assert len(args) == len(c[name][1]), name
+        for i, (ct, nt) in enumerate(zip(args, c[name][1])):
+            is_ptr = nt.startswith("ptr ") or nt in ("pointer", "cstring")
+            got_ptr = ct in (ctypes.c_void_p, ctypes.c_char_p) or hasattr(ct, "contents")
+            assert is_ptr == got_ptr, f"{name}: parameter {i} is {nt} in C, {ct} in ctypes"
+            if not is_ptr:
+                want = {"cint": ctypes.c_int, "int64": ctypes.c_int64, "int32": ctypes.c_int32, "cfloat": ctypes.c_float,
+                        "cdouble": ctypes.c_double, "csize_t": ctypes.c_size_t}[nt]
+                assert ct is want, f"{name}: parameter {i} is {nt} in C, {ct} in ctypes"
+
+
+def test_header_is_plain_c99(tmp_path):
+    import subprocess
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "am_hip.h"\nint main(void) { return am_hip_version() == 0; }\n')
+    res = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(src)],
+                         capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+
+
 def test_library_exports_every_declared_symbol():
     L = ctypes.CDLL(_lib.LIB_PATH)
     for s in declared_symbols():

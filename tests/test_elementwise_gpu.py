@@ -99,10 +99,58 @@ def test_reference_inplace_on_transposed(hip, vectors):
 
 
 def test_reference_map2_bool(hip, vectors):
+    """The reference's fixture for a map body whose result type differs from the input's: x mod y == 0
+    as ONE device pass that returns a bool tensor."""
     c = vectors["map2_bool"]
-    a, b = hip.toHip(np.array(c["a"], dtype=np.int64)), hip.toHip(np.array(c["b"], dtype=np.int64))
-    m = hip.map2("mod", a, b).toCpu()
-    assert np.array_equal(m == 0, np.array(c["expect"]))
+    for dt in (np.int64, np.int32):
+        a, b = hip.toHip(np.array(c["a"], dtype=dt)), hip.toHip(np.array(c["b"], dtype=dt))
+        m = hip.map2("mod_is_zero", a, b)
+        assert m.dtype == np.bool_ and m.shape == (4,)
+        assert np.array_equal(m.toCpu(), np.array(c["expect"]))
+        assert np.array_equal(hip.map2("mod", a, b).toCpu(), np.array(c["expect_mod"], dtype=dt))
+
+
+def test_reference_comparison_vectors(hip, vectors):
+    c = vectors["comparison"]
+    for sfx in ALL:
+        dt = DTYPES[sfx]
+        a, b = hip.toHip(np.array(c["a"], dtype=dt)), hip.toHip(np.array(c["b"], dtype=dt))
+        for case in c["tensor_tensor"]:
+            say("compare vector", sfx, case["cmp"])
+            got = hip.OPERATORS[case["cmp"] + "."](a, b)
+            assert got.dtype == np.bool_ and np.array_equal(got.toCpu(), np.array(case["expect"]))
+        for case in c["tensor_scalar"]:
+            f = hip.OPERATORS[case["cmp"] + "."]
+            got = f(case["scalar"], a) if case["scalar_on_left"] else f(a, case["scalar"])
+            assert np.array_equal(got.toCpu(), np.array(case["expect"])), case
+
+
+def test_reference_math_function_vectors(hip, vectors):
+    m = vectors["math_functions"]
+    for sfx in FLT:
+        dt = DTYPES[sfx]
+        s = m["sgn"]
+        got = hip.sgn(hip.toHip(np.array(s["a"], dtype=dt)))
+        assert got.dtype == np.int64 and got.toCpu().tolist() == s["expect"]
+        cs = m["copysign"]
+        a = hip.toHip(np.array(cs["a"], dtype=dt))
+        want = np.array(cs["expect"], dtype=dt)
+        hip.mcopySign(a, hip.toHip(np.array(cs["signs"], dtype=dt)))
+        assert np.array_equal(a.toCpu(), want) and np.array_equal(np.signbit(a.toCpu()), np.signbit(want))
+        c = m["classify"]
+        x = hip.toHip(np.array([float(v) for v in c["a"]], dtype=dt))
+        assert np.array_equal(hip.isNaN(x).toCpu(), np.array(c["isnan"]))
+        assert np.array_equal(hip.isNotNaN(x).toCpu(), ~np.array(c["isnan"]))
+        assert [hip.FLOAT_CLASS[k] for k in hip.classify(x).toCpu()] == c["classes"]
+    mm = m["minmax"]
+    for sfx in INT:
+        a, b = hip.toHip(np.array(mm["a"], dtype=DTYPES[sfx])), hip.toHip(np.array(mm["b"], dtype=DTYPES[sfx]))
+        assert hip.map2("min", a, b).toCpu().tolist() == mm["min"] and hip.map2("max", a, b).toCpu().tolist() == mm["max"]
+    f = m["floormod"]
+    a = np.array([f["start"] + i * f["step"] for i in range(f["count"])])
+    ts, st = hip.floorMod(hip.toHip(a), 3.0).toCpu(), hip.floorMod(3.0, hip.toHip(a)).toCpu()
+    assert np.mean(np.abs(ts - np.array(f["tensor_scalar_3"]))) < 1e-9 and np.signbit(ts[1])
+    assert np.mean(np.abs(st - np.array(f["scalar_3_tensor"]))) < 1e-9
 
 
 # ------------------------------------------------------------------ oracle / NumPy parity
@@ -149,6 +197,121 @@ def test_broadcast_ops_bit_exact(hip, oracle, sfx, shapes):
     ba, bb = oracle.broadcast2(a, b)
     assert np.array_equal(hip.bc_div(da, db).toCpu(), oracle.map2("div", ba, bb))
     assert np.array_equal(hip.bias_relu(da, db).toCpu(), oracle.map2("add_relu", ba, bb))
+
+
+CMPS = ["==", "!=", "<", "<=", ">", ">="]
+_NP_CMP = {"==": np.equal, "!=": np.not_equal, "<": np.less, "<=": np.less_equal, ">": np.greater, ">=": np.greater_equal}
+
+
+def _with_specials(a, b, sfx):
+    if sfx in FLT:   # NaN, infinities and signed zeros on both sides, some of them facing each other
+        sp = np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, np.nan], dtype=a.dtype)
+        a.ravel()[: min(6, a.size)] = sp[: min(6, a.size)]
+        b.ravel()[: min(6, b.size)] = sp[::-1][: min(6, b.size)]
+    return a, b
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("shapes", BC_CASES + [((4099,), (4099,)), ((33, 4100), (33, 4100))])
+def test_broadcast_comparisons_bit_exact(hip, oracle, sfx, shapes):
+    """`==.` ... `>=.` with implicit broadcasting and in the scalar forms: each output byte is one comparison,
+    so NumPy fixes it; the oracle's strided walk is compared as well. Small value range, so that equal
+    elements occur."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("cmp", sfx, shapes))
+    a = rng.integers(-3, 3, shapes[0], endpoint=True).astype(dt)
+    b = rng.integers(-3, 3, shapes[1], endpoint=True).astype(dt)
+    a, b = _with_specials(a, b, sfx)
+    da, db = hip.toHip(a), hip.toHip(b)
+    ba, bb = oracle.broadcast2(a, b)
+    for cmp in CMPS:
+        say("compare", sfx, shapes, cmp)
+        got = hip.OPERATORS[cmp + "."](da, db)
+        assert got.dtype == np.bool_ and got.is_C_contiguous()
+        g = got.toCpu()
+        with np.errstate(invalid="ignore"):
+            assert np.array_equal(g, _NP_CMP[cmp](a, b)), cmp
+        assert np.array_equal(g, oracle.compare(cmp, ba, bb)), cmp
+        with np.errstate(invalid="ignore"):
+            assert np.array_equal(hip.OPERATORS[cmp + "."](da, 1).toCpu(), _NP_CMP[cmp](a, dt(1))), cmp
+            assert np.array_equal(hip.OPERATORS[cmp + "."](1, da).toCpu(), _NP_CMP[cmp](dt(1), a)), cmp
+    if sfx in INT:
+        b2 = b.copy(); b2[b2 == 0] = 2
+        got = hip.map2("mod_is_zero", hip.toHip(ba.copy()), hip.toHip(np.broadcast_to(b2, ba.shape).copy())).toCpu()
+        assert np.array_equal(got, np.fmod(ba, np.broadcast_to(b2, ba.shape)) == 0)
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_comparisons_and_predicates_on_strided_views(hip, oracle, sfx):
+    """Transposed, stepped, reversed and column-sliced operands (the generic and the LDS-tiled kernels with a
+    one-byte destination), plus sgn / isNaN / classify on the same views."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("cmp-strided", sfx))
+    P = rng.integers(-2, 2, (96, 80), endpoint=True).astype(dt)
+    Q = rng.integers(-2, 2, (80, 96), endpoint=True).astype(dt)
+    P, Q = _with_specials(P, Q, sfx)
+    if sfx in FLT:
+        P[5, 7:12] = [np.finfo(dt).tiny / 2, -np.finfo(dt).tiny / 8, np.finfo(dt).tiny, -1e-30, 3.5]
+    dP, dQ = hip.toHip(P), hip.toHip(Q)
+    cases = [("transposed b", dP, P, dQ.transpose(), Q.T),
+             ("both stepped", dP[::2, ::2], P[::2, ::2], dQ.transpose()[::2, ::2], Q.T[::2, ::2]),
+             ("reversed", dP[::-1, ::-1], P[::-1, ::-1], dQ.transpose(), Q.T),
+             ("column block", dP[:, 16:48], P[:, 16:48], dP[:, 48:80], P[:, 48:80])]
+    for name, da, a, db, b in cases:
+        for cmp in ("==", "<", ">="):
+            say("compare strided", sfx, name, cmp)
+            assert np.array_equal(hip.map2(cmp, da, db).toCpu(), oracle.compare(cmp, a, b)), (name, cmp)
+        assert np.array_equal(hip.sgn(da).toCpu(), oracle.sgn(a)), name
+        if sfx in FLT:
+            for pred, f in (("isnan", hip.isNaN), ("isnotnan", hip.isNotNaN), ("classify", hip.classify)):
+                assert np.array_equal(f(da).toCpu(), oracle.predicate(pred, a)), (name, pred)
+    with pytest.raises(TypeError):
+        hip.map2("add", hip.map2("==", dP, dP), hip.map2("==", dP, dP))     # no arithmetic on bool tensors
+    if sfx in INT:
+        with pytest.raises(TypeError):
+            hip.isNaN(dP)
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_floormod_clamp_by_value_and_angle_conversions(hip, oracle, sfx):
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("floormod", sfx))
+    a, b = fill(rng, (37, 1028), dt), fill(rng, (37, 1028), dt, lo=-9, hi=9)
+    b[b == 0] = 4
+    da, db = hip.toHip(a), hip.toHip(b)
+    assert np.array_equal(hip.floorMod(da, db).toCpu(), oracle.map2("floormod", a, b))
+    assert np.array_equal(hip.floorMod(da, 3).toCpu(), oracle.scalar_op("floormod", a, 3))
+    assert np.array_equal(hip.floorMod(-3, da.transpose()).toCpu(), oracle.scalar_op("floormod", a.T, -3, scalar_on_left=True))
+    if sfx in INT:
+        assert np.array_equal(hip.floorMod(da, db).toCpu(), np.mod(a, b))       # Python's %: sign of the divisor
+    # clamp with both bounds by value, out of place on a view and in place
+    lo, hi = (dt(-1.5), dt(2.25)) if sfx in FLT else (dt(-7), dt(11))
+    assert np.array_equal(hip.clamp(da, lo, hi).toCpu(), np.clip(a, lo, hi))
+    assert np.array_equal(hip.clamp(da.transpose()[::2], lo, hi).toCpu(), np.clip(a.T[::2], lo, hi))
+    dc = hip.toHip(a)
+    hip.mclamp(dc[:, 16:48], lo, hi)
+    want = a.copy(); want[:, 16:48] = np.clip(a[:, 16:48], lo, hi)
+    assert np.array_equal(dc.toCpu(), want)
+    if sfx in FLT:
+        x = np.concatenate([a.ravel()[:4000] * 90, [0.0, 180.0, -360.0, 1e-30]]).astype(dt)
+        assert np.array_equal(hip.degToRad(hip.toHip(x)).toCpu(), oracle.unary("degtorad", x))
+        assert np.array_equal(hip.radToDeg(hip.toHip(x)).toCpu(), oracle.unary("radtodeg", x))
+        assert np.array_equal(hip.copySign(da, db).toCpu(), np.copysign(a, b))
+        nan_clamped = hip.clamp(hip.toHip(np.array([np.nan, -9, 9], dtype=dt)), lo, hi).toCpu()
+        assert np.isnan(nan_clamped[0]) and nan_clamped[1] == lo and nan_clamped[2] == hi
+
+
+def test_clamp_inside_a_graph(hip):
+    """Bounds by value: the call allocates nothing and copies nothing, so it can be recorded."""
+    x = np.random.default_rng(5).uniform(-4, 4, (64, 4096)).astype(np.float32)
+    dx, out = hip.toHip(x), hip.empty((64, 4096), np.float32)
+    from arraymancer_amd import tensor_hip as th
+    with hip.Graph() as g:
+        th._clamp_into(out, dx, -1.0, 1.0)
+    for _ in range(3):
+        g.launch()
+        assert np.array_equal(out.toCpu(), np.clip(x, -1, 1))
+        th._unary_into("neg", out, out)   # eager work between replays
 
 
 @pytest.mark.parametrize("sfx", ALL)

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 from hypothesis import given, settings, strategies as st
 
-from conftest import DTYPES
+from conftest import DTYPES, seed_of
 
 INT = ["i32", "i64"]
 FLT = ["f32", "f64"]
@@ -89,6 +89,90 @@ def test_reference_map2_bool(vectors, oracle):
     m = oracle.map2("mod", a, b)
     assert np.array_equal(m, np.array(c["expect_mod"]))
     assert np.array_equal(m == 0, np.array(c["expect"]))
+    got = oracle.compare("mod_is_zero", a, b)      # the whole body, with its bool result
+    assert got.dtype == np.bool_ and np.array_equal(got, np.array(c["expect"]))
+
+
+_NP_CMP = {"==": np.equal, "!=": np.not_equal, "<": np.less, "<=": np.less_equal, ">": np.greater, ">=": np.greater_equal}
+
+
+def test_reference_comparison_vectors(vectors, oracle):
+    c = vectors["comparison"]
+    for dt in (np.int32, np.int64, np.float32, np.float64):
+        a, b = np.array(c["a"], dtype=dt), np.array(c["b"], dtype=dt)
+        for case in c["tensor_tensor"]:
+            assert np.array_equal(oracle.compare(case["cmp"], a, b), np.array(case["expect"]))
+        for case in c["tensor_scalar"]:
+            cmp = {"<=": ">=", ">=": "<=", "<": ">", ">": "<"}.get(case["cmp"], case["cmp"]) if case["scalar_on_left"] else case["cmp"]
+            assert np.array_equal(oracle.compare(cmp, a, case["scalar"]), np.array(case["expect"]))
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.float32, np.float64])
+def test_comparisons_against_numpy_on_strided_operands(oracle, dt):
+    """Each output element is one comparison: NumPy's broadcasting comparison fixes it, NaN included."""
+    rng = np.random.default_rng(seed_of("cmp", str(dt)))
+    a = rng.integers(-3, 3, (7, 1, 5)).astype(dt)
+    b = rng.integers(-3, 3, (1, 6, 5)).astype(dt)
+    if np.dtype(dt).kind == "f":
+        a[0, 0, :3] = [np.nan, np.inf, -0.0]
+        b[0, :3, 0] = [np.nan, 0.0, np.inf]
+    ba, bb = oracle.broadcast2(a, b)
+    for cmp, f in _NP_CMP.items():
+        with np.errstate(invalid="ignore"):
+            assert np.array_equal(oracle.compare(cmp, ba, bb), f(a, b)), cmp
+            assert np.array_equal(oracle.compare(cmp, ba[::-1].transpose(2, 0, 1), bb[::-1].transpose(2, 0, 1)),
+                                  f(a, b)[::-1].transpose(2, 0, 1)), cmp
+            assert np.array_equal(oracle.compare(cmp, ba, 1), f(a, dt(1)) & np.ones(ba.shape, bool)), cmp
+
+
+def test_reference_math_function_vectors(vectors, oracle):
+    m = vectors["math_functions"]
+    for dt in (np.float32, np.float64):
+        s = m["sgn"]
+        assert np.array_equal(oracle.sgn(np.array(s["a"], dtype=dt)), np.array(s["expect"], dtype=np.int64))
+        cs = m["copysign"]
+        got = oracle.map2("copysign", np.array(cs["a"], dtype=dt), np.array(cs["signs"], dtype=dt))
+        want = np.array(cs["expect"], dtype=dt)
+        assert np.array_equal(got, want) and np.array_equal(np.signbit(got), np.signbit(want))
+        c = m["classify"]
+        x = np.array([float(v) for v in c["a"]], dtype=dt)
+        assert np.array_equal(oracle.predicate("isnan", x), np.array(c["isnan"]))
+        assert np.array_equal(oracle.predicate("isnotnan", x), ~np.array(c["isnan"]))
+        names = ("fcNormal", "fcSubnormal", "fcZero", "fcNegZero", "fcNan", "fcInf", "fcNegInf")
+        assert [names[k] for k in oracle.predicate("classify", x)] == c["classes"]
+        tiny = np.finfo(dt).tiny
+        assert oracle.predicate("classify", np.array([tiny, tiny / 2, -tiny / 4, 1.0, -3.5], dtype=dt)).tolist() == [0, 1, 1, 0, 0]
+    for dt in (np.int32, np.int64):
+        assert oracle.sgn(np.array([-7, 0, 9, np.iinfo(dt).min], dtype=dt)).tolist() == [-1, 0, 1, -1]
+        mm = m["minmax"]
+        a, b = np.array(mm["a"], dtype=dt), np.array(mm["b"], dtype=dt)
+        assert oracle.map2("min", a, b).tolist() == mm["min"] and oracle.map2("max", a, b).tolist() == mm["max"]
+    f = m["floormod"]
+    a = np.array([f["start"] + i * f["step"] for i in range(f["count"])])       # arange(-70.7, 50.0, 34.7)
+    ts, st = oracle.scalar_op("floormod", a, 3.0), oracle.scalar_op("floormod", a, 3.0, scalar_on_left=True)
+    assert np.mean(np.abs(ts - np.array(f["tensor_scalar_3"]))) < 1e-9 and np.signbit(ts[1])
+    assert np.mean(np.abs(st - np.array(f["scalar_3_tensor"]))) < 1e-9
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.float64])
+def test_floormod_is_python_modulo(oracle, dt):
+    """floorMod's result takes the divisor's sign: for integers it is Python's %, for floats np.mod
+    wherever that is exact (it is np.fmod moved by one divisor)."""
+    rng = np.random.default_rng(seed_of("floormod", str(dt)))
+    a = rng.integers(-50, 50, 400).astype(dt)
+    b = rng.integers(-9, 9, 400).astype(dt)
+    b[b == 0] = 4
+    got = oracle.map2("floormod", a, b)
+    assert np.array_equal(got, np.array([int(x) % int(y) for x, y in zip(a, b)], dtype=dt))
+
+
+def test_deg_rad_conversions(oracle):
+    for dt in (np.float32, np.float64):
+        x = np.array([0, 30, 45, 90, 180, -360, 1e-3], dtype=dt)
+        r = oracle.unary("degtorad", x)
+        np.testing.assert_allclose(r, np.deg2rad(x.astype(np.float64)), rtol=4 * np.finfo(dt).eps)
+        np.testing.assert_allclose(oracle.unary("radtodeg", r), x, rtol=4 * np.finfo(dt).eps)
+    assert oracle.unary("degtorad", np.array([180.0]))[0] == np.pi
 
 
 def test_int_division_truncates_toward_zero(oracle):

@@ -155,3 +155,23 @@ def test_caching_allocator(hip):
     assert L.am_hip_empty_cache() == 0 and stats()[1] == 0
     # a foreign pointer is rejected, not handed to the driver
     assert L.am_hip_free(ctypes.c_void_p(0x1000)) != 0
+
+
+def test_display_of_device_tensors(hip):
+    """`$t` / pretty on real device tensors, views included: the reference's table layout under a header that
+    names this backend (format pinned on the reference's literals in tests/test_display.py)."""
+    t = hip.toHip(np.arange(1, 25, dtype=np.int64).reshape(2, 3, 4))
+    want = ('HipTensor[system.int] of shape "[2, 3, 4]" on backend "Hip"\n'
+            "          0                      1\n"
+            "|1      2     3     4| |13    14    15    16|\n"
+            "|5      6     7     8| |17    18    19    20|\n"
+            "|9     10    11    12| |21    22    23    24|")
+    got = str(t)
+    assert [l.rstrip() for l in got.rstrip("\n").split("\n")] == want.split("\n")
+    v = hip.toHip(np.arange(1, 6, dtype=np.int32).reshape(1, 5)).transpose()
+    assert v.pretty(specifier="||") == "| 1|\n| 2|\n| 3|\n| 4|\n| 5|"
+    sl = hip.toHip(np.arange(12, dtype=np.float32).reshape(3, 4))[::2, 1::2]          # strided view
+    assert sl.pretty(specifier="<>") == "HipTensor[float32]<2,2>:[[1, 3], [9, 11]]"
+    assert hip.bc_ge(sl, 3.0).pretty(specifier="<>") == "HipTensor[bool]<2,2>:[[false, true], [true, true]]"
+    assert hip.toHip(np.array([0.9532932, 0.12945823])).pretty(precision=4, specifier="[]") == "[0.9533, 0.1295]"
+    assert str(hip.empty((0, 3), np.float64)) == 'HipTensor[system.float] of shape "[0, 3]" on backend "Hip"\n    [] (empty)'
