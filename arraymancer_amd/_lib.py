@@ -69,6 +69,9 @@ def _signatures():
         "am_hip_graph_launch": (ci, [vp]),
         "am_hip_graph_destroy": (ci, [vp]),
         "am_hip_diag_peak": (ci, [ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
+        "am_hip_diag_clock_begin": (ci, []),
+        "am_hip_diag_clock_end": (ci, [ctypes.POINTER(ctypes.c_double)]),
+        "am_hip_diag_hbm": (ci, [ci, sz, ci, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
     }
     for sfx, ct in CTYPE.items():
         gemm = [i64, i64, i64, ct, vp, i64, i64, vp, i64, i64, ct, vp, i64, i64]

@@ -19,6 +19,25 @@ bool capturing();
 // memory is staged by the runtime and costs about 10 us more.
 int fetch_result(void* host_dst, const void* dev_src, size_t bytes);
 int num_cus();
+// Device buffer the matrix-core kernels add their shader-cycle / constant-rate-tick counts to while
+// am_hip_diag_clock_begin .. _end is open; nullptr otherwise (the kernels then read no counter).
+long long* clock_probe_buffer();
+
+// In a kernel: reads both counters at construction; finish() has the first lane of workgroup 0 add the
+// differences to out[0] (shader cycles) and out[1] (ticks). Does nothing when `out` is null.
+struct ClockProbe {
+  long long c0, w0;
+  long long* out;
+  __device__ __forceinline__ explicit ClockProbe(long long* o) : c0(0), w0(0), out(o) {
+    if (out) { c0 = clock64(); w0 = wall_clock64(); }
+  }
+  __device__ __forceinline__ void finish() const {
+    if (out && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+      out[0] += clock64() - c0;
+      out[1] += wall_clock64() - w0;
+    }
+  }
+};
 
 #define AM_HIP_TRY(expr)                                                                    \
   do {                                                                                      \

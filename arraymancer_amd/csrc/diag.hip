@@ -94,7 +94,164 @@ __global__ __launch_bounds__(256) void peak_valu_mac(int iters, U* out, U seed) 
   if (s == (U)0x1234567) out[0] = s;
 }
 
+// ---- HBM streams: what the memory system delivers to a kernel that does nothing else --------------
+// One workgroup walks tiles of 256 lanes x UNROLL x 16 bytes (every load instruction of a wavefront
+// covers 1 KiB of consecutive addresses, UNROLL of them in flight per lane), grid-stride over the
+// buffer. KIND 0 reads (folds into a register, stores nothing), 1 writes a constant, 2 copies.
+// NTL / NTS: non-temporal loads / stores. CHUNKED: a workgroup owns one contiguous run of tiles
+// instead of every gridDim.x-th tile.
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+template <int KIND, int UNROLL, bool NTL, bool NTS, bool CHUNKED>
+__global__ __launch_bounds__(256) void hbm_stream(const v4u* __restrict__ src, v4u* __restrict__ dst, uint64_t ntiles, uint32_t* sink) {
+  constexpr uint64_t TILE_V = 256ull * UNROLL;   // 16-byte vectors per tile
+  v4u fold = {0u, 0u, 0u, 0u};
+  uint64_t first = blockIdx.x, last = ntiles, step = gridDim.x;
+  if (CHUNKED) {
+    const uint64_t per = (ntiles + gridDim.x - 1) / gridDim.x;
+    first = per * blockIdx.x;
+    last = first + per < ntiles ? first + per : ntiles;
+    step = 1;
+  }
+  for (uint64_t tile = first; tile < last; tile += step) {
+    const uint64_t base = tile * TILE_V + threadIdx.x;
+    v4u v[UNROLL];
+    if (KIND != 1) {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if (NTL) v[u] = __builtin_nontemporal_load(src + base + (uint64_t)u * 256);
+        else v[u] = src[base + (uint64_t)u * 256];
+      }
+    }
+    if (KIND == 0) {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) fold ^= v[u];
+    } else {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const v4u w = KIND == 1 ? v4u{(uint32_t)tile, 1u, 2u, 3u} : v[u];
+        if (NTS) __builtin_nontemporal_store(w, dst + base + (uint64_t)u * 256);
+        else dst[base + (uint64_t)u * 256] = w;
+      }
+    }
+  }
+  if (KIND == 0 && (fold[0] ^ fold[1] ^ fold[2] ^ fold[3]) == 0x9e3779b9u) sink[0] = fold[0];   // keeps the loads alive
+}
+
+template <int KIND, int UNROLL>
+static void launch_hbm(bool ntl, bool nts, bool chunked, unsigned blocks, const v4u* src, v4u* dst, uint64_t ntiles, uint32_t* sink) {
+#define AM_HBM(L, S, C) hipLaunchKernelGGL((hbm_stream<KIND, UNROLL, L, S, C>), dim3(blocks), dim3(256), 0, stream(), src, dst, ntiles, sink)
+  const int sel = (ntl ? 4 : 0) | (nts ? 2 : 0) | (chunked ? 1 : 0);
+  switch (sel) {
+    case 0: AM_HBM(false, false, false); break;
+    case 1: AM_HBM(false, false, true); break;
+    case 2: AM_HBM(false, true, false); break;
+    case 3: AM_HBM(false, true, true); break;
+    case 4: AM_HBM(true, false, false); break;
+    case 5: AM_HBM(true, false, true); break;
+    case 6: AM_HBM(true, true, false); break;
+    default: AM_HBM(true, true, true); break;
+  }
+#undef AM_HBM
+}
+
+template <int KIND>
+static void launch_hbm_u(int unroll, bool ntl, bool nts, bool chunked, unsigned blocks, const v4u* src, v4u* dst, uint64_t bytes, uint32_t* sink) {
+  switch (unroll) {
+    case 1: launch_hbm<KIND, 1>(ntl, nts, chunked, blocks, src, dst, bytes / (4096ull * 1), sink); break;
+    case 2: launch_hbm<KIND, 2>(ntl, nts, chunked, blocks, src, dst, bytes / (4096ull * 2), sink); break;
+    case 8: launch_hbm<KIND, 8>(ntl, nts, chunked, blocks, src, dst, bytes / (4096ull * 8), sink); break;
+    default: launch_hbm<KIND, 4>(ntl, nts, chunked, blocks, src, dst, bytes / (4096ull * 4), sink); break;
+  }
+}
+
 }  // namespace
+
+// HBM stream ceilings. kind: 0 read, 1 write, 2 copy. Each launch moves `bytes` (a multiple of 32 KiB) of
+// a window that rotates through `windows` disjoint buffers (windows * bytes should exceed the 256 MB
+// memory-side cache several times over, so that no launch finds its input there); blocks_per_cu x CUs
+// workgroups; `unroll` (1, 2, 4, 8) 16-byte accesses in flight per lane; flags: bit 0 non-temporal loads,
+// bit 1 non-temporal stores, bit 2 a contiguous run of tiles per workgroup. Returns bytes moved per second
+// (read + written) averaged over `launches` launches after `windows` untimed ones.
+extern "C" int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_per_cu, int unroll, int flags, int launches,
+                               double* bytes_per_second) {
+  if (!bytes_per_second || kind < 0 || kind > 2 || bytes == 0 || bytes % 32768 != 0 || windows < 1 || windows > 64 ||
+      blocks_per_cu < 1 || blocks_per_cu > 64 || (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8) || launches < 1)
+    return fail(AM_E_ARG, "am_hip_diag_hbm: bad argument");
+  AM_TRY(ensure_init());
+  char *src = nullptr, *dst = nullptr;
+  uint32_t* sink = nullptr;
+  const size_t total = bytes * (size_t)windows;
+  AM_HIP_TRY(hipMalloc((void**)&sink, 256));
+  if (kind != 1) {
+    if (hipMalloc((void**)&src, total) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(sink); return fail(AM_E_ALLOC, "am_hip_diag_hbm: %zu bytes", total); }
+    AM_HIP_TRY(hipMemsetAsync(src, 0x5a, total, stream()));
+  }
+  if (kind != 0) {
+    if (hipMalloc((void**)&dst, total) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(src); (void)hipFree(sink); return fail(AM_E_ALLOC, "am_hip_diag_hbm: %zu bytes", total); }
+    AM_HIP_TRY(hipMemsetAsync(dst, 0, total, stream()));
+  }
+  const unsigned blocks = (unsigned)(num_cus() * blocks_per_cu);
+  hipEvent_t e0, e1;
+  AM_HIP_TRY(hipEventCreate(&e0));
+  AM_HIP_TRY(hipEventCreate(&e1));
+  auto one = [&](int i) {
+    const size_t off = (size_t)(i % windows) * bytes;
+    const v4u* s = (const v4u*)(src ? src + off : nullptr);
+    v4u* d = (v4u*)(dst ? dst + off : nullptr);
+    const bool ntl = flags & 1, nts = flags & 2, chunked = flags & 4;
+    if (kind == 0) launch_hbm_u<0>(unroll, ntl, nts, chunked, blocks, s, d, bytes, sink);
+    else if (kind == 1) launch_hbm_u<1>(unroll, ntl, nts, chunked, blocks, s, d, bytes, sink);
+    else launch_hbm_u<2>(unroll, ntl, nts, chunked, blocks, s, d, bytes, sink);
+  };
+  for (int i = 0; i < windows; ++i) one(i);
+  AM_HIP_TRY(hipEventRecord(e0, stream()));
+  for (int i = 0; i < launches; ++i) one(windows + i);
+  AM_HIP_TRY(hipEventRecord(e1, stream()));
+  AM_HIP_TRY(hipEventSynchronize(e1));
+  float ms = 0;
+  AM_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+  AM_HIP_TRY(hipEventDestroy(e0));
+  AM_HIP_TRY(hipEventDestroy(e1));
+  (void)hipFree(src); (void)hipFree(dst); (void)hipFree(sink);
+  AM_TRY(check_launch("hbm_stream"));
+  *bytes_per_second = (double)bytes * (kind == 2 ? 2.0 : 1.0) * launches / (ms * 1e-3);
+  return AM_OK;
+}
+
+// ---- shader clock sustained by the matrix kernels themselves --------------------------------------
+// While armed, the matrix-core GEMM kernels (gemm_mfma, gemm_i8_digits) have the first lane of workgroup 0
+// read the shader-cycle counter and the constant-rate counter when it starts and when it ends, and add the
+// two differences to this buffer: cycles / ticks x the constant rate is the shader clock averaged over the
+// kernels that ran, measured inside them (a second kernel running beside them to watch the clock takes a CU
+// from a launch of exactly one workgroup per CU and doubles its time).
+namespace {
+long long* g_clock_buf = nullptr;   // device: [0] shader cycles, [1] constant-rate ticks
+bool g_clock_armed = false;
+}  // namespace
+namespace am {
+long long* clock_probe_buffer() { return g_clock_armed ? g_clock_buf : nullptr; }
+}
+
+extern "C" int am_hip_diag_clock_begin(void) {
+  AM_TRY(ensure_init());
+  if (capturing()) return fail(AM_E_ARG, "am_hip_diag_clock_begin: not allowed while a graph is being captured");
+  if (!g_clock_buf) AM_HIP_TRY(hipMalloc((void**)&g_clock_buf, 256));
+  AM_HIP_TRY(hipMemsetAsync(g_clock_buf, 0, 256, stream()));
+  g_clock_armed = true;
+  return AM_OK;
+}
+
+extern "C" int am_hip_diag_clock_end(double* shader_mhz) {
+  if (!shader_mhz) return fail(AM_E_ARG, "am_hip_diag_clock_end: null pointer");
+  if (!g_clock_armed) return fail(AM_E_ARG, "am_hip_diag_clock_end: am_hip_diag_clock_begin was not called");
+  g_clock_armed = false;
+  long long h[2] = {0, 0};
+  AM_TRY(fetch_result(h, g_clock_buf, sizeof(h)));
+  int khz = 100000;
+  (void)hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, 0);
+  *shader_mhz = h[1] > 0 ? (double)h[0] / (double)h[1] * (khz / 1e3) : 0.0;
+  return AM_OK;
+}
 
 // kind: 0 = MFMA f32 32x32x2 (FLOP/s), 1 = MFMA f64 16x16x4 (FLOP/s),
 //       2 = VALU int32 multiply-add (integer op/s, 2 per MAC), 3 = VALU int64 multiply-add,

@@ -14,6 +14,7 @@
 // (src/arraymancer/tensor/private/p_accessors.nim:181-208, 378-413); both kernels compute the
 // same element correspondence in closed form instead of carrying coordinates.
 #pragma once
+#include <stdlib.h>
 #include <type_traits>
 #include "common.h"
 
@@ -217,7 +218,10 @@ template <typename T, int CODE> struct OpSel {
 // ---- layouts passed to kernels by value
 constexpr int kMaxOuter = AM_MAXRANK - 1;
 
-enum Kind : int { kVecOperand = 0, kRowScalar = 1, kConst = 2 };
+// How ew_rows sees an operand: a vector stream with its own row offset (kVecOperand), one row re-used for
+// every output row (kRowVector: all outer strides zero, loaded once per workgroup and kept in registers), one
+// value per row (kRowScalar: inner stride zero) or the scalar argument (kConst).
+enum Kind : int { kVecOperand = 0, kRowScalar = 1, kConst = 2, kRowVector = 3 };
 
 // T: element type of the operands, D: of the destination (the same except for comparisons and predicates).
 template <typename T, typename D = T> struct RowsArgs {
@@ -226,7 +230,9 @@ template <typename T, typename D = T> struct RowsArgs {
   int a_stream, b_stream; // 1: operand is read once (non-temporal loads); 0: re-read per row, keep cached
   int64_t L;              // inner extent (elements)
   uint32_t tiles_per_row; // ceil(L / tile)
-  uint32_t total_tiles;   // rows * tiles_per_row
+  uint32_t rows;          // product of the outer extents
+  uint32_t col_blocks;    // workgroups side by side along a row: workgroup (c, g) = blockIdx.x % col_blocks, / col_blocks
+                          // takes the column tiles c, c + col_blocks, ... of the rows g, g + gridDim.x / col_blocks, ...
   int outer_rank;         // 0..5 collapsed outer dims (row-major over them = row index)
   int64_t oshape[kMaxOuter];
   int64_t od[kMaxOuter], oa[kMaxOuter], ob[kMaxOuter];  // outer strides per operand (elements)
@@ -262,79 +268,103 @@ __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T, D> p) {
   typedef typename OpSel<T, CODE>::type Op;
   constexpr int VEC = Traits<T>::kVec;
   constexpr int64_t TILE = (int64_t)kThreads * VEC * kUnroll;
+  constexpr bool A_ROW = AK == kVecOperand || AK == kRowVector, B_ROW = BK == kVecOperand || BK == kRowVector;
 
-  for (uint32_t tile = blockIdx.x; tile < p.total_tiles; tile += gridDim.x) {
-    const uint32_t row = tile / p.tiles_per_row;
-    const uint32_t ct = tile - row * p.tiles_per_row;
-    int64_t offd = 0, offa = 0, offb = 0;
-    {
-      uint32_t rem = row;
-      for (int d = p.outer_rank - 1; d >= 0; --d) {
-        const uint32_t ext = (uint32_t)p.oshape[d];
-        const uint32_t q = rem / ext;
-        const int64_t c = (int64_t)(rem - q * ext);
-        rem = q;
-        offd += c * p.od[d];
-        offa += c * p.oa[d];
-        if constexpr (BK != kConst) offb += c * p.ob[d];
-      }
-    }
-    D* __restrict__ drow = p.dst + offd;
-    const T* __restrict__ arow = p.a + offa;
-    const T* __restrict__ brow = (BK != kConst) ? p.b + offb : nullptr;
-    T asc = (T)0, bsc = p.scalar;
-    if constexpr (AK == kRowScalar) asc = arow[0];
-    if constexpr (BK == kRowScalar) bsc = brow[0];
-
+  const uint32_t cb = blockIdx.x % p.col_blocks, g0 = blockIdx.x / p.col_blocks, gstep = gridDim.x / p.col_blocks;
+  // A workgroup keeps its column tile while it walks down the rows: the column offsets and a row vector that
+  // every output row re-uses (the bias of `X +. b`) are computed / loaded once per column tile instead of once
+  // per row. WHOLE: the tile lies wholly inside the row (every column tile but a ragged last one), so that
+  // the loop body is straight-line code: loads under a branch are waited for one by one.
+  auto column_tile = [&](auto whole_tag, uint32_t ct) {
+    constexpr bool WHOLE = decltype(whole_tag)::value;
     const int64_t col0 = (int64_t)ct * TILE + (int64_t)threadIdx.x * VEC;
-    V av[kUnroll], bv[kUnroll];
+    // Ragged tile: every lane still loads all its vectors, those past the end of the row from the row's first
+    // vector instead (the host sends rows shorter than one vector elsewhere), and only the stores are
+    // conditional. Loads under a branch would be waited for one at a time.
     bool full[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) full[u] = (col0 + (int64_t)u * kThreads * VEC + VEC <= p.L);
-    // One branch per operand around its loads: a select between a non-temporal and an ordinary load of the
-    // same address is merged into an ordinary load by the compiler, hence also the laundered pointer.
-    if constexpr (AK == kVecOperand) {
-      if (p.a_stream) {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-          if (full[u]) av[u] = __builtin_nontemporal_load(launder((const V*)(arow + col0 + (int64_t)u * kThreads * VEC)));
-      } else {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-          if (full[u]) av[u] = *(const V*)(arow + col0 + (int64_t)u * kThreads * VEC);
-      }
-    }
-    if constexpr (BK == kVecOperand) {
-      if (p.b_stream) {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-          if (full[u]) bv[u] = __builtin_nontemporal_load(launder((const V*)(brow + col0 + (int64_t)u * kThreads * VEC)));
-      } else {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-          if (full[u]) bv[u] = *(const V*)(brow + col0 + (int64_t)u * kThreads * VEC);
-      }
-    }
+    int64_t lcol[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t col = col0 + (int64_t)u * kThreads * VEC;
-      if (full[u]) {
+      full[u] = WHOLE || (col + VEC <= p.L);
+      lcol[u] = full[u] ? col : 0;
+    }
+    V av[kUnroll], bv[kUnroll];
+    if constexpr (AK == kRowVector) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) av[u] = *(const V*)(p.a + lcol[u]);
+    }
+    if constexpr (BK == kRowVector) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) bv[u] = *(const V*)(p.b + lcol[u]);
+    }
+    for (uint32_t row = g0; row < p.rows; row += gstep) {
+      int64_t offd = 0, offa = 0, offb = 0;
+      {
+        uint32_t rem = row;
+        for (int d = p.outer_rank - 1; d >= 0; --d) {
+          const uint32_t ext = (uint32_t)p.oshape[d];
+          const uint32_t q = rem / ext;
+          const int64_t c = (int64_t)(rem - q * ext);
+          rem = q;
+          offd += c * p.od[d];
+          if constexpr (AK != kRowVector) offa += c * p.oa[d];
+          if constexpr (BK != kConst && BK != kRowVector) offb += c * p.ob[d];
+        }
+      }
+      D* __restrict__ drow = p.dst + offd;
+      const T* __restrict__ arow = p.a + offa;
+      const T* __restrict__ brow = (BK != kConst) ? p.b + offb : nullptr;
+      T asc = (T)0, bsc = p.scalar;
+      if constexpr (AK == kRowScalar) asc = arow[0];
+      if constexpr (BK == kRowScalar) bsc = brow[0];
+
+      // One branch per operand around its loads: a select between a non-temporal and an ordinary load of the
+      // same address is merged into an ordinary load by the compiler, hence also the laundered pointer.
+      if constexpr (AK == kVecOperand) {
+        if (p.a_stream) {
+#pragma unroll
+          for (int u = 0; u < kUnroll; ++u) av[u] = __builtin_nontemporal_load(launder((const V*)(arow + lcol[u])));
+        } else {
+#pragma unroll
+          for (int u = 0; u < kUnroll; ++u) av[u] = *(const V*)(arow + lcol[u]);
+        }
+      }
+      if constexpr (BK == kVecOperand) {
+        if (p.b_stream) {
+#pragma unroll
+          for (int u = 0; u < kUnroll; ++u) bv[u] = __builtin_nontemporal_load(launder((const V*)(brow + lcol[u])));
+        } else {
+#pragma unroll
+          for (int u = 0; u < kUnroll; ++u) bv[u] = *(const V*)(brow + lcol[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
         DV r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const T x = (AK == kVecOperand) ? av[u][e] : asc;
-          const T y = (BK == kVecOperand) ? bv[u][e] : bsc;
+          const T x = A_ROW ? av[u][e] : asc;
+          const T y = B_ROW ? bv[u][e] : bsc;
           r[e] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
         }
-        __builtin_nontemporal_store(r, (DV*)(drow + col));
-      } else {
-        for (int64_t c = col; c < p.L; ++c) {   // ragged end of the row (< VEC elements)
-          const T x = (AK == kVecOperand) ? arow[c] : asc;
-          const T y = (BK == kVecOperand) ? brow[c] : bsc;
-          drow[c] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
+        if (full[u]) __builtin_nontemporal_store(r, (DV*)(drow + lcol[u]));
+      }
+      if constexpr (!WHOLE) {   // the row's last L mod VEC elements, one lane
+        const int64_t tail = p.L - p.L % VEC;
+        if (threadIdx.x == 0 && tail < p.L && tail >= (int64_t)ct * TILE) {
+          for (int64_t c = tail; c < p.L; ++c) {
+            const T x = A_ROW ? (AK == kRowVector ? p.a[c] : arow[c]) : asc;
+            const T y = B_ROW ? (BK == kRowVector ? p.b[c] : brow[c]) : bsc;
+            drow[c] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
+          }
         }
       }
     }
+  };
+  for (uint32_t ct = cb; ct < p.tiles_per_row; ct += p.col_blocks) {
+    if ((int64_t)(ct + 1) * TILE <= p.L) column_tile(std::true_type(), ct);
+    else column_tile(std::false_type(), ct);
   }
 }
 
@@ -606,8 +636,9 @@ static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const 
   for (int d = 0; d < in; ++d) rows *= c.shape[d];
   const int64_t tile = (int64_t)kThreads * VEC * kUnroll;
   const int64_t tiles_per_row = (L + tile - 1) / tile;
-  // Short rows would leave most lanes of a tile idle: those shapes go to the generic kernel.
-  if (ok && rows > 1 && L < tile / 4) ok = false;
+  // Short rows would leave most lanes of a tile idle: those shapes go to the generic kernel (and so does a
+  // row shorter than one 16-byte vector, which the streaming kernel's clamped loads would overrun).
+  if (ok && ((rows > 1 && L < tile / 4) || L < VEC)) ok = false;
   if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31) || rows >= ((int64_t)1 << 31))) ok = false;
   if (!ok) {
     // Two collapsed dims with unit strides on different axes: the LDS-tiled kernel.
@@ -638,7 +669,7 @@ static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const 
   RowsArgs<T, D> r;
   r.dst = dst; r.a = a; r.b = b; r.scalar = scalar; r.L = L;
   r.tiles_per_row = (uint32_t)tiles_per_row;
-  r.total_tiles = (uint32_t)(tiles_per_row * rows);
+  r.rows = (uint32_t)rows;
   r.outer_rank = in;
   // An operand whose outer strides are all zero is one row re-read `rows` times: keep it cached.
   r.a_stream = 0; r.b_stream = 0;
@@ -647,13 +678,17 @@ static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const 
     if (c.sb[d] != 0) r.b_stream = 1;
   }
   if (in == 0) { r.a_stream = 1; r.b_stream = 1; }
-  // Non-temporal loads pay once the operands read once exceed what the 256 MB memory-side cache can still hold
-  // from the kernel that produced them (f32 8192 x 8192: X + Y 142 -> 128 us); below that ordinary loads are
-  // faster (copy of one 256 MB operand: 63 us against 87 us).
+  // Operands that are read once are loaded non-temporally unless they are small enough to be served by the
+  // XCDs' L2 (32 MB together). What a previous kernel wrote with non-temporal stores is not in the memory-side
+  // cache, so a chain of passes reads every byte from HBM, and from HBM non-temporal loads are the faster ones:
+  // f32 8192 x 8192, X +. b then *. s over rotating buffers 183 -> 175 us (the second pass in place: 198 -> 174),
+  // one pass 88 -> 86.5 us. (Ordinary loads win only where the same input is read again and again with nothing in
+  // between, 77 us: the memory-side cache then still holds part of it.) AM_HIP_EW_NT = 0 | 1 forces the kind.
   {
     const double operand_bytes = (double)rows * (double)L * sizeof(T);
     const int streamed = (ia == 1 ? r.a_stream : 0) + (!BCONST && ib == 1 ? r.b_stream : 0);
-    if (!(streamed * operand_bytes > 384.0 * 1024 * 1024)) { r.a_stream = 0; r.b_stream = 0; }
+    if (!(streamed * operand_bytes > 32.0 * 1024 * 1024)) { r.a_stream = 0; r.b_stream = 0; }
+    if (const char* e = getenv("AM_HIP_EW_NT")) { if (*e == '1') { r.a_stream = (ia == 1); r.b_stream = (ib == 1); } else if (*e == '0') { r.a_stream = r.b_stream = 0; } }
   }
   for (int d = 0; d < kMaxOuter; ++d) {
     r.oshape[d] = d < in ? c.shape[d] : 1;
@@ -661,14 +696,27 @@ static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const 
     r.oa[d] = d < in ? c.sa[d] : 0;
     r.ob[d] = d < in ? c.sb[d] : 0;
   }
-  int64_t blocks = r.total_tiles;
   const int64_t cap = (int64_t)num_cus() * 32;
-  if (blocks > cap) blocks = cap;
-  const dim3 grid((unsigned)blocks), block(kThreads);
+  const int64_t col_blocks = tiles_per_row < cap ? tiles_per_row : cap;
+  int64_t row_groups = cap / col_blocks;
+  if (row_groups > rows) row_groups = rows;
+  if (row_groups < 1) row_groups = 1;
+  r.col_blocks = (uint32_t)col_blocks;
+  const dim3 grid((unsigned)(col_blocks * row_groups)), block(kThreads);
+  // a vector operand whose outer strides are all zero is the same row for every output row: kept in registers
+  bool a_rowvec = ia == 1 && in > 0, b_rowvec = !BCONST && ib == 1 && in > 0;
+  for (int d = 0; d < in; ++d) {
+    if (c.sa[d] != 0) a_rowvec = false;
+    if (BCONST || c.sb[d] != 0) b_rowvec = false;
+  }
   if constexpr (BCONST) {
     hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kConst, SWAP>), grid, block, 0, stream(), r);
   } else {
-    if (ia == 1 && ib == 1) hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kVecOperand, false>), grid, block, 0, stream(), r);
+    if (ia == 1 && ib == 1) {
+      if (b_rowvec && !a_rowvec) hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kRowVector, false>), grid, block, 0, stream(), r);
+      else if (a_rowvec && !b_rowvec) hipLaunchKernelGGL((ew_rows<T, D, CODE, kRowVector, kVecOperand, false>), grid, block, 0, stream(), r);
+      else hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kVecOperand, false>), grid, block, 0, stream(), r);
+    }
     else if (ia == 1) hipLaunchKernelGGL((ew_rows<T, D, CODE, kVecOperand, kRowScalar, false>), grid, block, 0, stream(), r);
     else hipLaunchKernelGGL((ew_rows<T, D, CODE, kRowScalar, kVecOperand, false>), grid, block, 0, stream(), r);
   }
@@ -886,9 +934,10 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
   if (ok && rows > 1 && L < tile / 8) ok = false;
   if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31))) ok = false;
   g.n = n; g.L = L;
-  {  // same rule as the two-operand kernel: non-temporal loads only when the operands read once exceed 384 MiB
+  {  // same rule as the two-operand kernel: non-temporal loads once the operands read once exceed what the L2s hold
     const int streamed = (!g.a_const && !g.a_keep) + (!g.b_const && !g.b_keep) + (!g.c_const && !g.c_keep);
-    if (!(streamed * (double)rows * (double)L * sizeof(T) > 384.0 * 1024 * 1024)) g.a_keep = g.b_keep = g.c_keep = 1;
+    if (!(streamed * (double)rows * (double)L * sizeof(T) > 32.0 * 1024 * 1024)) g.a_keep = g.b_keep = g.c_keep = 1;
+    if (const char* e = getenv("AM_HIP_EW_NT")) { if (*e == '1') { g.a_keep = g.b_keep = g.c_keep = 0; } else if (*e == '0') { g.a_keep = g.b_keep = g.c_keep = 1; } }
   }
   if (ok) {
     g.rank = in;

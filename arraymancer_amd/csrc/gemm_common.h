@@ -50,6 +50,7 @@ template <typename T> struct Args {
   // static_ws_short (bytes it would have needed) and the call is refused.
   bool static_ws;
   size_t static_ws_short;
+  long long* clock_out;            // where the matrix-core kernels add their cycle counts while a clock window is open
 };
 
 // Digit pairs (i, j), i + j < ND, whose planes are both marked non-empty: flags[i] == gen for A's
@@ -118,6 +119,7 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   g.batch = 1; g.batch_a = g.batch_b = g.batch_c = 0;
   g.gate_flags = nullptr; g.gate_gen = 0; g.gate_max_pairs = 0;
   g.static_ws = false; g.static_ws_short = 0;
+  g.clock_out = clock_probe_buffer();
   g.swapped = swap;
   g.a_kfast = iabs64(g.a_k) <= iabs64(g.a_mn);
   g.b_kfast = iabs64(g.b_k) < iabs64(g.b_mn);

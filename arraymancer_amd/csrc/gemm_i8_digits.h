@@ -274,6 +274,7 @@ struct DigitArgs {
   int64_t M, N;
   T alpha, beta;
   int tiles_m, tiles_n;
+  long long* clock_out;                 // see ClockProbe (common.h)
 };
 
 // WAVES_M x WAVES_N wavefronts, each with TM x TN accumulator tiles of 32 x 32; BK k (bytes) per slab.
@@ -284,6 +285,7 @@ struct DigitArgs {
 template <typename T, int WAVES_M, int WAVES_N, int TM, int TN, int BK, int RING>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(DigitArgs<T> p) {
   using U = std::make_unsigned_t<T>;
+  const ClockProbe probe(p.clock_out);
   constexpr int ND = (int)sizeof(T), NPAIRS = ND * (ND + 1) / 2;
   constexpr bool WIDE = sizeof(T) == 8;
   constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -539,6 +541,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
         }
       }
     }
+  probe.finish();
 }
 
 // Padded operand extents and the estimated time of the digit-sliced product for both tile shapes
@@ -659,7 +662,7 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
   if (max_pairs >= 2) hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
   DigitArgs<T> d;
   d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.max_pairs = max_pairs; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
-  d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N;
+  d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N; d.clock_out = g.clock_out;
   d.alpha = g.alpha; d.beta = g.beta;
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);

@@ -91,6 +91,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
 void gemm_mfma(Args<T> p) {
   typedef Mfma<T> MF;
   typedef typename MF::acc_t acc_t;
+  const ClockProbe probe(p.clock_out);
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int TILE = MF::TILE, VK = MF::VK, KL = MF::KL, KSTEP = VK * KL;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / TILE, TN = WN / TILE;
@@ -316,6 +317,7 @@ void gemm_mfma(Args<T> p) {
           if (row < p.M && col < p.N) ws[row * p.N + col] = acc[i][j][r];
         }
       }
+    probe.finish();
     return;
   }
   const T alpha = p.alpha, beta = p.beta;
@@ -364,6 +366,7 @@ void gemm_mfma(Args<T> p) {
       }
     }
   }
+  probe.finish();
 }
 
 // PF: register stages of global loads; FPF: fragment prefetch; RU: steady-state loop unrolled over the LDS ring.

@@ -57,9 +57,13 @@ class Timer:
         L.am_hip_event_create(ctypes.byref(self.e1))
 
     def run(self, fn, steps, warmup):
+        """Times `steps` calls of fn after `warmup` untimed ones. While the timed steps run, the matrix-core
+        GEMM kernels count shader cycles against the constant-rate counter (am_hip_diag_clock_*):
+        self.sclk_mhz is the shader clock they sustained (None when no such kernel ran)."""
         for _ in range(warmup):
             fn()
         self.am.sync()
+        armed = self.L.am_hip_diag_clock_begin() == 0
         t0 = time.perf_counter()
         self.L.am_hip_event_record(self.e0)
         for _ in range(steps):
@@ -69,6 +73,11 @@ class Timer:
         wall = time.perf_counter() - t0
         ms = ctypes.c_float()
         self.L.am_hip_event_elapsed_ms(self.e0, self.e1, ctypes.byref(ms))
+        self.sclk_mhz = None
+        if armed:
+            mhz = ctypes.c_double()
+            if self.L.am_hip_diag_clock_end(ctypes.byref(mhz)) == 0 and mhz.value > 0:
+                self.sclk_mhz = round(mhz.value, 0)
         return wall, ms.value / 1e3     # seconds: wall clock for all steps, event time for all steps
 
 
@@ -90,22 +99,46 @@ def run_rotating(timer, fns, rounds, warm_rounds=1):
 
 def measured_ceilings(L):
     """Issue ceilings of this chip from register-only micro-benchmarks (no memory traffic): what a
-    perfect kernel could reach at the clocks the device sustains. T(FL)OP/s."""
+    perfect kernel could reach at the clocks the device sustains, T(FL)OP/s; and what HBM delivers to
+    kernels that only stream (read, write, copy of 256 MiB per launch over six rotating buffers = 1.5 GiB
+    per direction, so every byte comes from HBM; 16-byte non-temporal accesses, four in flight per lane;
+    the best of a few grid sizes), TB/s."""
     out = {}
     for kind, name, iters in [(0, "mfma_f32", 20000), (1, "mfma_f64", 20000), (2, "valu_int32_mac", 20000), (3, "valu_int64_mac", 5000),
                               (4, "mfma_i8", 20000)]:
         v = ctypes.c_double()
         if L.am_hip_diag_peak(kind, iters, 2, ctypes.byref(v)) == 0:
             out[name] = round(v.value / 1e12, 2)
+    for kind, name in [(0, "hbm_read"), (1, "hbm_write"), (2, "hbm_copy")]:
+        best = 0.0
+        for blocks_per_cu in (2, 8, 32):
+            for flags in ((1,) if kind == 0 else (2, 0) if kind == 1 else (3,)):
+                v = ctypes.c_double()
+                if L.am_hip_diag_hbm(kind, 256 << 20, 6, blocks_per_cu, 4, flags, 24, ctypes.byref(v)) == 0:
+                    best = max(best, v.value)
+        if best:
+            out[name + "_tbs"] = round(best / 1e12, 3)
     return out
 
 
 def load_traffic(key):
+    """(bytes per launch from the committed rocprofv3 --pmc passes, where those were taken) - the figure is not
+    re-measured by this run: counters need the profiler."""
     try:
         with open(TRAFFIC_FILE) as f:
-            return json.load(f).get(key)
+            d = json.load(f)
+        return d.get(key), d.get("_source")
     except (OSError, ValueError):
-        return None
+        return None, None
+
+
+def at_clock(roof, peak, sclk_mhz, nominal_mhz=2400.0):
+    """Adds the sustained shader clock and the fraction of the peak scaled to that clock (the published
+    matrix peaks are CUs x ops per clock x 2.4 GHz)."""
+    if sclk_mhz:
+        roof["sclk_mhz"] = sclk_mhz
+        roof["frac_of_peak_at_sclk"] = round(roof["achieved"] / (peak * sclk_mhz / nominal_mhz), 4)
+    return roof
 
 
 def bench_gemm_f32(am, timer, steps, warmup, n=4096):
@@ -114,7 +147,7 @@ def bench_gemm_f32(am, timer, steps, warmup, n=4096):
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.float32)
     wall, ev = timer.run(lambda: am.gemm(1.0, dA, dB, 0.0, dC), steps, warmup)
     flops = 2.0 * n ** 3
-    return dict(wall=wall, ev=ev, flops=flops, host=(A, B))
+    return dict(wall=wall, ev=ev, flops=flops, host=(A, B), sclk_mhz=timer.sclk_mhz)
 
 
 def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
@@ -167,13 +200,14 @@ def other_workloads(am, timer, steps, warmup, ceilings):
         pairs = digit_pairs(A, B)
         dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
         wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+        sclk = timer.sclk_mhz
         tops = 2.0 * n ** 3 / (ev / k) / 1e12
         entry = dict(workload=f"i32 GEMM 4096^3, {label} (wraparound; {pairs} of 10 int8 digit-pair products on the matrix cores, "
                               "timed with the two digit-splitting passes)",
                      unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
-                     roofline=dict(bound="mfma", achieved=round(pairs * tops, 1), peak=MFMA_I8_PEAK_TOPS,
-                                   unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, two digit-splitting passes included",
-                                   frac=round(pairs * tops / MFMA_I8_PEAK_TOPS, 4)),
+                     roofline=at_clock(dict(bound="mfma", achieved=round(pairs * tops, 1), peak=MFMA_I8_PEAK_TOPS,
+                                            unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, two digit-splitting passes included",
+                                            frac=round(pairs * tops / MFMA_I8_PEAK_TOPS, 4)), MFMA_I8_PEAK_TOPS, sclk),
                      speedup_over_valu_ceiling=round(tops / peak, 2) if peak else None)
         if lo == -100:
             os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
@@ -193,6 +227,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int64)
     wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+    sclk = timer.sclk_mhz
     os.environ["AM_HIP_GEMM_I64_PATH"] = "valu"
     try:
         _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), 3, 1)
@@ -203,9 +238,9 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     out.append(dict(workload="i64 GEMM 4096^3, entries in [-100, 100] (wraparound; 1 of 36 int8 digit-pair products on the matrix cores, "
                              "timed with the two digit-splitting passes)",
                     unit="Top/s", dtype="i64", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
-                    roofline=dict(bound="mfma", achieved=round(2.0 * n ** 3 / (ev / k) / 1e12, 1), peak=MFMA_I8_PEAK_TOPS,
-                                  unit="int8 TOP/s executed (1 digit pair x 2*M*N*K) over the whole call, two digit-splitting passes included",
-                                  frac=round(2.0 * n ** 3 / (ev / k) / 1e12 / MFMA_I8_PEAK_TOPS, 4)),
+                    roofline=at_clock(dict(bound="mfma", achieved=round(2.0 * n ** 3 / (ev / k) / 1e12, 1), peak=MFMA_I8_PEAK_TOPS,
+                                           unit="int8 TOP/s executed (1 digit pair x 2*M*N*K) over the whole call, two digit-splitting passes included",
+                                           frac=round(2.0 * n ** 3 / (ev / k) / 1e12 / MFMA_I8_PEAK_TOPS, 4)), MFMA_I8_PEAK_TOPS, sclk),
                     valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / 3 * 1e3, 4),
                                      roofline=dict(bound="valu (measured int64 multiply-add ceiling)", achieved=round(valu_tops, 3),
                                                    peak=peak64, unit="Top/s", frac=round(valu_tops / peak64, 4) if peak64 else None))))
@@ -219,8 +254,9 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     fl = 2.0 * 2048 * 3072 * 1024
     out.append(dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", unit="TFLOP/s",
                     dtype="f64", value=round(fl * steps / wall / 1e12, 3), ms_per_step=round(ev / steps * 1e3, 4),
-                    roofline=dict(bound="mfma", achieved=round(fl / (ev / steps) / 1e12, 3), peak=MFMA_F64_PEAK_TFLOPS,
-                                  unit="TFLOP/s", frac=round(fl / (ev / steps) / 1e12 / MFMA_F64_PEAK_TFLOPS, 4))))
+                    roofline=at_clock(dict(bound="mfma", achieved=round(fl / (ev / steps) / 1e12, 3), peak=MFMA_F64_PEAK_TFLOPS,
+                                           unit="TFLOP/s", frac=round(fl / (ev / steps) / 1e12 / MFMA_F64_PEAK_TFLOPS, 4)),
+                                      MFMA_F64_PEAK_TFLOPS, timer.sclk_mhz)))
     del dA, dB, dC
     # --- broadcast ops on X[8192, 8192] f32 (HBM bound): 536 903 680 algorithmic bytes per op
     X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
@@ -234,20 +270,24 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     bb = db.broadcast((8192, 8192))
     sb = ds.broadcast((8192, 8192))
     nbytes = 2 * 8192 * 8192 * 4 + 8192 * 4
-    # `value`: the same X and Y every step, like every other entry; the 256 MiB input is then re-read from the
-    # 256 MB memory-side cache, so this rate can exceed what HBM delivers. `roofline`: five buffer sets round
-    # robin (2.5 GiB), every byte from HBM.
+    # Five buffer sets round robin (2.5 GiB), so that every byte of every launch comes from HBM: both `value`
+    # and `roofline` are that figure. The same-buffer time is listed beside it (part of a 256 MiB input that is
+    # read again at once can still be in the 256 MB memory-side cache).
+    copy_ceiling = ceilings.get("hbm_copy_tbs")
     for name, op, rhs in [("X +. b[1,8192]", "add", bb), ("Y *. s[8192,1]", "mul", sb),
                           ("map2(X, b, max(0, x+y)) (fused bias+ReLU)", "add_relu", bb)]:
-        wall, ev = timer.run(lambda: th._binary_into(op, dY, dX, rhs), steps, warmup)
-        cold = run_rotating(timer, [(lambda i=i: th._binary_into(op, dYs[i], dXs[i], rhs)) for i in range(ROTATE)], max(steps // ROTATE, 4))
+        _, ev = timer.run(lambda: th._binary_into(op, dY, dX, rhs), steps, warmup)
+        rounds = max(steps // ROTATE, 4)
+        t0 = time.perf_counter()
+        cold = run_rotating(timer, [(lambda i=i: th._binary_into(op, dYs[i], dXs[i], rhs)) for i in range(ROTATE)], rounds)
         gbs = nbytes / cold / 1e9
-        out.append(dict(workload=f"f32 8192x8192 {name}", unit="GB/s", dtype="f32",
-                        value=round(nbytes * steps / wall / 1e9, 1), ms_per_step=round(ev / steps * 1e3, 4),
-                        value_is="same buffers every step: the input is re-read from the 256 MB memory-side cache",
-                        roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                                      frac=round(gbs / HBM_PEAK_GBS, 4), ms_per_launch=round(cold * 1e3, 4),
-                                      protocol=f"{ROTATE} buffer sets round robin (2.5 GiB): every byte from HBM")))
+        roof = dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4),
+                    ms_per_launch=round(cold * 1e3, 4), protocol=f"{ROTATE} buffer sets round robin (2.5 GiB): every byte from HBM")
+        if copy_ceiling:
+            roof["measured_copy_ceiling_gbs"] = round(copy_ceiling * 1e3, 1)
+            roof["frac_of_measured_copy_ceiling"] = round(gbs / (copy_ceiling * 1e3), 4)
+        out.append(dict(workload=f"f32 8192x8192 {name}", unit="GB/s", dtype="f32", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 4),
+                        same_buffers_every_step_ms=round(ev / steps * 1e3, 4), roofline=roof))
     del dXs, dYs
     out.append(bench_chain(am, timer, max(steps, 50), warmup))
     return out
@@ -524,6 +564,7 @@ def main():
     r = bench_gemm_f32(am, timer, args.steps, args.warmup)
     tflops = r["flops"] * args.steps / r["wall"] / 1e12
     kern_tflops = r["flops"] / (r["ev"] / args.steps) / 1e12
+    traffic, traffic_src = load_traffic("gemm_f32_4096")
     line = {
         "metric": "GEMM TFLOP/s (%MFMA peak) fp32/int32 4096^3; broadcast op HBM GB/s (%peak)",
         "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -531,9 +572,9 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "f32 GEMM C=A*B, M=N=K=4096, row-major contiguous, uniform[-1,1) seeds 1001/1002 "
                                "(the 4096^3 size the metric is quoted on)"},
-        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": MFMA_F32_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(kern_tflops / MFMA_F32_PEAK_TFLOPS, 4),
-                     "traffic": load_traffic("gemm_f32_4096")},
+        "roofline": at_clock({"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": MFMA_F32_PEAK_TFLOPS,
+                              "unit": "TFLOP/s", "frac": round(kern_tflops / MFMA_F32_PEAK_TFLOPS, 4),
+                              "traffic": traffic, "traffic_source": traffic_src}, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"]),
         "device": info,
     }
     if not args.no_cpu:

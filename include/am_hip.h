@@ -557,6 +557,23 @@ int am_hip_maxpool2d_backward_i64(int64_t N, int C, int H, int W, int kH, int kW
  *   kind 4: MFMA int8 32x32x32 (integer op/s), the instruction of the digit-sliced integer GEMM
  * waves_per_simd wavefronts are resident on every SIMD (1..8); iters loop trips each. */
 int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second);
+/* What HBM delivers to a kernel that only streams: kind 0 reads, 1 writes, 2 copies `bytes` (a multiple of
+ * 32 KiB) per launch with 16-byte accesses, `unroll` (1, 2, 4, 8) of them in flight per lane, from
+ * blocks_per_cu x CUs workgroups of 256 lanes. Launches rotate through `windows` disjoint buffers of `bytes`
+ * each (allocated and freed inside the call), so that with windows * bytes several times the 256 MB
+ * memory-side cache every byte comes from HBM. flags: bit 0 non-temporal loads, bit 1 non-temporal stores,
+ * bit 2 one contiguous run of tiles per workgroup instead of every n-th tile. Result: bytes read plus bytes
+ * written per second, averaged over `launches` launches. The HBM-bound kernels are priced against the
+ * published 8 TB/s; this is the measured ceiling shown beside it. */
+int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_per_cu, int unroll, int flags, int launches,
+                    double* bytes_per_second);
+/* The shader clock the device sustains under the matrix-core GEMM kernels: between _begin and _end the first
+ * lane of workgroup 0 of every gemm_mfma / gemm_i8_digits launch compares the shader-cycle counter with the
+ * constant-rate counter over the kernel's own lifetime; _end (blocking) returns cycles / ticks as MHz, averaged
+ * over those launches (0 if none ran). The matrix peaks are quoted at 2.4 GHz; a power-limited kernel settles
+ * lower, and its fraction of peak is read against that. */
+int am_hip_diag_clock_begin(void);
+int am_hip_diag_clock_end(double* shader_mhz);
 
 #ifdef __cplusplus
 }

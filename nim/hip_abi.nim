@@ -49,6 +49,10 @@ proc am_hip_graph_end*(graph_exec: ptr pointer): cint {.importc.}
 proc am_hip_graph_launch*(graph_exec: pointer): cint {.importc.}
 proc am_hip_graph_destroy*(graph_exec: pointer): cint {.importc.}
 proc am_hip_diag_peak*(kind, iters, waves_per_simd: cint, ops_per_second: ptr cdouble): cint {.importc.}
+proc am_hip_diag_clock_begin*(): cint {.importc.}
+proc am_hip_diag_clock_end*(shader_mhz: ptr cdouble): cint {.importc.}
+proc am_hip_diag_hbm*(kind: cint, bytes: csize_t, windows, blocks_per_cu, unroll, flags, launches: cint,
+                      bytes_per_second: ptr cdouble): cint {.importc.}
 
 # ---- GEMM (strides in elements; pointers already offset)
 proc am_hip_gemm_f32*(M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64,
