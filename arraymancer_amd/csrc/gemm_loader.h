@@ -149,28 +149,42 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
   }
 };
 
+// Any strides (zero, negative, stepped): one element per load. Each lane keeps the address of its NE
+// elements of slab 0 (row / column clamped into the operand); a slab's loads are those addresses plus
+// k0 * ld_k, one 64-bit product per slab shared by all of them, instead of two per element.
 template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kGeneric, BMN, BK, NT, KG, PF> {
   static constexpr int NE = BMN * BK / NT;         // elements per thread
   static_assert(BMN * BK % NT == 0 && NE >= 1, "slab must divide evenly over the workgroup");
-  const T* X;
-  int64_t ld_mn, ld_k, mn0, MN, K;
+  const T* ptr[NE];
+  int64_t ld_k, K;
   int kfast;
   T reg[PF][NE];
-  __device__ __forceinline__ Loader(const T* X_, int64_t ld_mn_, int64_t ld_k_, int64_t mn0_, int64_t MN_, int64_t K_, int kfast_)
-      : X(X_), ld_mn(ld_mn_), ld_k(ld_k_), mn0(mn0_), MN(MN_), K(K_), kfast(kfast_) {}
   __device__ __forceinline__ void coords(int i, int& mn, int& k) const {
     const int e = threadIdx.x + i * NT;
     if (kfast) { k = e % BK; mn = e / BK; } else { mn = e % BMN; k = e / BMN; }
   }
-  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
-    if (MASK && k0 >= K) return;
+  __device__ __forceinline__ Loader(const T* X, int64_t ld_mn, int64_t ld_k_, int64_t mn0, int64_t MN, int64_t K_, int kfast_)
+      : ld_k(ld_k_), K(K_), kfast(kfast_) {
 #pragma unroll
     for (int i = 0; i < NE; ++i) {
       int mn, k;
       coords(i, mn, k);
       const int64_t cm = (mn0 + mn) < MN ? mn0 + mn : MN - 1;
-      const int64_t ck = (!MASK || (k0 + k) < K) ? k0 + k : K - 1;
-      reg[S][i] = X[cm * ld_mn + ck * ld_k];
+      ptr[i] = X + cm * ld_mn + (int64_t)k * ld_k;
+    }
+  }
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
+    if (MASK && k0 >= K) return;
+    const int64_t step = k0 * ld_k;
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+      if constexpr (MASK) {
+        int mn, k;
+        coords(i, mn, k);
+        reg[S][i] = ptr[i][(k0 + k) < K ? step : (K - 1 - k) * ld_k];   // past the end: the last valid k (zeroed at commit)
+      } else {
+        reg[S][i] = ptr[i][step];
+      }
     }
   }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {

@@ -56,13 +56,25 @@ class Timer:
         L.am_hip_event_create(ctypes.byref(self.e0))
         L.am_hip_event_create(ctypes.byref(self.e1))
 
-    def run(self, fn, steps, warmup):
+    def run(self, fn, steps, warmup, min_warm_s=0.0):
         """Times `steps` calls of fn after `warmup` untimed ones. While the timed steps run, the matrix-core
         GEMM kernels count shader cycles against the constant-rate counter (am_hip_diag_clock_*):
-        self.sclk_mhz is the shader clock they sustained (None when no such kernel ran)."""
+        self.sclk_mhz is the shader clock they sustained (None when no such kernel ran).
+        min_warm_s: go on warming up until the untimed calls have kept the device busy for that long. The
+        shader clock needs 20-50 ms under load to climb from about 2.1 GHz to the 2.39 GHz it then holds (and as
+        long to recover after a power-limited kernel); a figure taken inside that ramp is 10 % low."""
+        self.L.am_hip_event_record(self.e0)
         for _ in range(warmup):
             fn()
+        self.L.am_hip_event_record(self.e1)
         self.am.sync()
+        if min_warm_s > 0 and warmup > 0:
+            ms = ctypes.c_float()
+            self.L.am_hip_event_elapsed_ms(self.e0, self.e1, ctypes.byref(ms))
+            per_call = max(ms.value / 1e3 / warmup, 1e-6)
+            for _ in range(min(int((min_warm_s - ms.value / 1e3) / per_call) + 1, 20000) if ms.value / 1e3 < min_warm_s else 0):
+                fn()
+            self.am.sync()
         armed = self.L.am_hip_diag_clock_begin() == 0
         t0 = time.perf_counter()
         self.L.am_hip_event_record(self.e0)
@@ -84,6 +96,9 @@ class Timer:
 ROTATE = 5   # buffer sets of the rotating protocol: together far beyond the 256 MB memory-side cache
 
 
+WARM_S = 0.05   # device-busy time before every timed region of the secondary workloads (see Timer.run)
+
+
 def run_rotating(timer, fns, rounds, warm_rounds=1):
     """The same operation on len(fns) disjoint buffer sets, issued round robin, so that no byte of an
     input is still in the memory-side cache when it is read again: every byte comes from HBM.
@@ -93,7 +108,7 @@ def run_rotating(timer, fns, rounds, warm_rounds=1):
     def step():
         fns[state["i"] % len(fns)]()
         state["i"] += 1
-    _, ev = timer.run(step, rounds * len(fns), warm_rounds * len(fns))
+    _, ev = timer.run(step, rounds * len(fns), warm_rounds * len(fns), WARM_S)
     return ev / (rounds * len(fns))
 
 
@@ -141,10 +156,22 @@ def at_clock(roof, peak, sclk_mhz, nominal_mhz=2400.0):
     return roof
 
 
-def bench_gemm_f32(am, timer, steps, warmup, n=4096):
-    A = np.random.default_rng(1001).uniform(-1, 1, (n, n)).astype(np.float32)
-    B = np.random.default_rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
+def spin_up(L, seconds=0.08):
+    """Keeps the matrix cores busy for `seconds` with the register-only MFMA chain (no memory traffic, not
+    the workload): the shader clock climbs from the 2.1 GHz of an idle device to the 2.39 GHz it holds under
+    sustained load."""
+    t_end = time.perf_counter() + seconds
+    v = ctypes.c_double()
+    while time.perf_counter() < t_end:
+        L.am_hip_diag_peak(0, 20000, 2, ctypes.byref(v))
+
+
+def bench_gemm_f32(am, timer, steps, warmup, n=4096, host=None, device_warm_s=0.0):
+    A, B = host or (np.random.default_rng(1001).uniform(-1, 1, (n, n)).astype(np.float32),
+                    np.random.default_rng(1002).uniform(-1, 1, (n, n)).astype(np.float32))
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.float32)
+    if device_warm_s > 0:
+        spin_up(timer.L, device_warm_s)
     wall, ev = timer.run(lambda: am.gemm(1.0, dA, dB, 0.0, dC), steps, warmup)
     flops = 2.0 * n ** 3
     return dict(wall=wall, ev=ev, flops=flops, host=(A, B), sclk_mhz=timer.sclk_mhz)
@@ -199,7 +226,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
         B = np.random.default_rng(2002).integers(lo, hi, (n, n), endpoint=True).astype(np.int32)
         pairs = digit_pairs(A, B)
         dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
-        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, WARM_S)
         sclk = timer.sclk_mhz
         tops = 2.0 * n ** 3 / (ev / k) / 1e12
         entry = dict(workload=f"i32 GEMM 4096^3, {label} (wraparound; {pairs} of 10 int8 digit-pair products on the matrix cores, "
@@ -212,7 +239,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
         if lo == -100:
             os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"
             try:
-                _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+                _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, WARM_S)
             finally:
                 del os.environ["AM_HIP_GEMM_I32_PATH"]
             valu_tops = 2.0 * n ** 3 / (ev_valu / k) / 1e12
@@ -226,11 +253,11 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
     B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int64)
-    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2)
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, WARM_S)
     sclk = timer.sclk_mhz
     os.environ["AM_HIP_GEMM_I64_PATH"] = "valu"
     try:
-        _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), 3, 1)
+        _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), 3, 1, WARM_S)
     finally:
         del os.environ["AM_HIP_GEMM_I64_PATH"]
     peak64 = ceilings.get("valu_int64_mac")
@@ -250,7 +277,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     pb = np.random.default_rng(3002).standard_normal((1024, 6144))
     C = np.random.default_rng(3003).standard_normal((2048, 3072))
     dA, dB, dC = am.toHip(pa).transpose(), am.toHip(pb)[:, ::2], am.toHip(C)
-    wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, warmup)
+    wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, warmup, WARM_S)
     fl = 2.0 * 2048 * 3072 * 1024
     out.append(dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", unit="TFLOP/s",
                     dtype="f64", value=round(fl * steps / wall / 1e12, 3), ms_per_step=round(ev / steps * 1e3, 4),
@@ -276,7 +303,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     copy_ceiling = ceilings.get("hbm_copy_tbs")
     for name, op, rhs in [("X +. b[1,8192]", "add", bb), ("Y *. s[8192,1]", "mul", sb),
                           ("map2(X, b, max(0, x+y)) (fused bias+ReLU)", "add_relu", bb)]:
-        _, ev = timer.run(lambda: th._binary_into(op, dY, dX, rhs), steps, warmup)
+        _, ev = timer.run(lambda: th._binary_into(op, dY, dX, rhs), steps, warmup, WARM_S)
         rounds = max(steps // ROTATE, 4)
         t0 = time.perf_counter()
         cold = run_rotating(timer, [(lambda i=i: th._binary_into(op, dYs[i], dXs[i], rhs)) for i in range(ROTATE)], rounds)
@@ -317,10 +344,10 @@ def chain_setup(am):
 
 def bench_chain(am, timer, steps, warmup):
     issue, flops, nbytes, keep = chain_setup(am)
-    wall_e, ev_e = timer.run(issue, steps, warmup)            # eager: 4 launches per chain from the host
+    wall_e, ev_e = timer.run(issue, steps, warmup, WARM_S)    # eager: 4 launches per chain from the host
     with am.Graph() as graph:
         issue()
-    wall_g, ev_g = timer.run(graph.launch, steps, warmup)     # one graph launch per chain
+    wall_g, ev_g = timer.run(graph.launch, steps, warmup, WARM_S)     # one graph launch per chain
     return dict(workload="f32 inference chain: [20x25].[25x36864], [50x500].[500x4096], "
                          "[64x800].[800x500]+bias+ReLU (fused), [64x500].[500x10]",
                 unit="us per chain", dtype="f32", higher_is_better=False,
@@ -361,7 +388,7 @@ def config_report(am, timer, L):
         am.gemm(alpha, dA, dB, beta, dC)
         got = dC.toCpu().copy()
         # (with beta != 0 the timed calls go on accumulating into C: only their time is used)
-        _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3)
+        _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3, WARM_S)
         gpu_s = ev / steps
         want = am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy())
         cpu_s = cpu_time(lambda: am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy() if beta != 0 else C_host))
@@ -435,7 +462,7 @@ def config_report(am, timer, L):
     # HBM-bound rows: timed over five buffer sets round robin, so that every byte comes from HBM
     for name, op, dv, hv in (("X +. b[1,8192]", "add", db, b), ("X *. s[8192,1]", "mul", ds, sc), ("map2(X, b, max(0, x+y))", "add_relu", db, b)):
         bv = dv.broadcast((8192, 8192))
-        _, ev = timer.run(lambda: th._binary_into(op, dY, dX, bv), 50, 5)
+        _, ev = timer.run(lambda: th._binary_into(op, dY, dX, bv), 50, 5, WARM_S)
         gpu_s = run_rotating(timer, [(lambda i=i: th._binary_into(op, dYs[i], dXs[i], bv)) for i in range(ROTATE)], 10)
         got = dYs[ROTATE - 1].toCpu().copy()
         hb = am_oracle.broadcast(hv, X.shape)
@@ -448,7 +475,7 @@ def config_report(am, timer, L):
              bit_exact=bool(np.array_equal(got, out)), note=warm_note(ev / 50, nbytes))
     # (X +. b) *. s fused into one pass (same bytes moved once instead of twice)
     bb, sb = db.broadcast((8192, 8192)), ds.broadcast((8192, 8192))
-    _, ev = timer.run(lambda: th._ternary_into("addmul", dY, dX, bb, sb), 50, 5)
+    _, ev = timer.run(lambda: th._ternary_into("addmul", dY, dX, bb, sb), 50, 5, WARM_S)
     gpu_s = run_rotating(timer, [(lambda i=i: th._ternary_into("addmul", dYs[i], dXs[i], bb, sb)) for i in range(ROTATE)], 10)
     two_pass = ((X + b) * sc)
     emit(config="f32 8192x8192 (X +. b) *. s fused (one pass)", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
@@ -462,7 +489,7 @@ def config_report(am, timer, L):
         """fn_gpu(x) on each of the rotating inputs (every byte from HBM); the warm figure goes into the note."""
         got = fn_gpu(inputs[0])
         want = fn_cpu()
-        _, ev = timer.run(lambda: fn_gpu(inputs[0]), 50, 5)
+        _, ev = timer.run(lambda: fn_gpu(inputs[0]), 50, 5, WARM_S)
         gpu_s = run_rotating(timer, [(lambda x=x: fn_gpu(x)) for x in inputs], 10)
         cpu_s = cpu_time(fn_cpu, budget=2.0)
         emit(config=config, dtype="f32", gpu_ms=round(gpu_s * 1e3, 4), gpu_rate=round(nbytes / gpu_s / 1e9, 1), rate_unit="GB/s",
@@ -527,7 +554,7 @@ def run_only(am, timer, which, steps, warmup):
             b = am.toHip(np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32))
             bb = b.broadcast((8192, 8192))
             fn = lambda: th._binary_into("add", dY, dX, bb)
-    wall, ev = timer.run(fn, steps, warmup)
+    wall, ev = timer.run(fn, steps, warmup, WARM_S)
     return dict(only=which, ms_per_launch=round(ev / steps * 1e3, 4), launches=steps + warmup)
 
 
@@ -561,7 +588,12 @@ def main():
         config_report(am, timer, L)
         return
 
-    r = bench_gemm_f32(am, timer, args.steps, args.warmup)
+    # The same W warm-up steps + K timed steps twice: straight from the idle device (`from_idle`: the shader
+    # clock is still climbing then), and again right after 80 ms of register-only matrix-core work that is not
+    # the workload (`value`: the clock the device holds under sustained load, printed beside it).
+    idle = bench_gemm_f32(am, timer, args.steps, args.warmup)
+    r = bench_gemm_f32(am, timer, args.steps, args.warmup, host=idle["host"], device_warm_s=0.08)
+    ceilings = measured_ceilings(L)
     tflops = r["flops"] * args.steps / r["wall"] / 1e12
     kern_tflops = r["flops"] / (r["ev"] / args.steps) / 1e12
     traffic, traffic_src = load_traffic("gemm_f32_4096")
@@ -575,13 +607,18 @@ def main():
         "roofline": at_clock({"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": MFMA_F32_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(kern_tflops / MFMA_F32_PEAK_TFLOPS, 4),
                               "traffic": traffic, "traffic_source": traffic_src}, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"]),
+        "from_idle": {"value": round(idle["flops"] * args.steps / idle["wall"] / 1e12, 3), "unit": "TFLOP/s",
+                      "ms_per_step": round(idle["wall"] / args.steps * 1e3, 4), "sclk_mhz": idle["sclk_mhz"],
+                      "what": "the same warm-up and timed steps started on the idle device, before anything else ran: the shader "
+                              "clock needs 20-50 ms under load to reach the frequency it then holds. `value` is taken right "
+                              "after 80 ms of register-only matrix-core work (am_hip_diag_peak, not the workload)"},
         "device": info,
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_gemm_f32(*r["host"])
     if not args.no_others:
-        ceilings = measured_ceilings(L)
-        line["measured_ceilings"] = dict(ceilings, unit="T(FL)OP/s", how="am_hip_diag_peak: register-only MFMA / VALU chains")
+        line["measured_ceilings"] = dict(ceilings, unit="T(FL)OP/s (hbm_*: TB/s)",
+                                         how="am_hip_diag_peak: register-only MFMA / VALU chains; am_hip_diag_hbm: streaming kernels over rotating buffers")
         line["others"] = other_workloads(am, timer, args.steps, args.warmup, ceilings)
     print(json.dumps(line))
 
