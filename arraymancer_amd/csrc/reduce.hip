@@ -388,12 +388,21 @@ static int reduce_all(const char* fn, int op, int rank, const int64_t* shape, co
     const int last = g.ndim - 1;
     const int64_t rows = g.outputs / g.extent[last];
     const size_t tmp_bytes = ((size_t)rows * sizeof(T) + 255) / 256 * 256;
-    if (tmp_bytes > (size_t)16 * 1024 * 1024)
-      return fail(AM_E_ALLOC, "%s: a non-contiguous tensor with %lld separate runs is too large for the reduction scratch; "
-                  "reduce a contiguous copy", fn, (long long)rows);
-    char* base = (char*)gemm::splitk_workspace(256 + tmp_bytes);
-    if (!base) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
-    T* tmp = (T*)(base + 256);
+    // The per-run partials live in the workspace while they fit beside the chunk partials; a tensor of very
+    // many short runs (a stepped slice [4M, k], a tall transposed view) takes them from the block cache
+    // instead and gives them back once the value is on the host.
+    const bool in_ws = tmp_bytes <= (size_t)16 * 1024 * 1024;
+    void* big = nullptr;
+    T* tmp;
+    if (in_ws) {
+      char* base = (char*)gemm::splitk_workspace(256 + tmp_bytes);
+      if (!base) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
+      tmp = (T*)(base + 256);
+    } else {
+      AM_TRY(am_hip_malloc(tmp_bytes, &big));
+      tmp = (T*)big;
+    }
+    const size_t ws_off = in_ws ? 256 + tmp_bytes : 256;
     Args<T> s;
     memset(&s, 0, sizeof(s));
     s.a = a; s.dst = tmp;
@@ -402,9 +411,14 @@ static int reduce_all(const char* fn, int op, int rank, const int64_t* shape, co
     for (int d = last - 1; d >= 0; --d) { s.extent[d] = g.extent[d]; s.a_stride[d] = g.a_stride[d]; s.d_stride[d] = cs; cs *= g.extent[d]; }
     for (int d = last; d < kMaxDims; ++d) { s.extent[d] = 1; s.a_stride[d] = 0; s.d_stride[d] = 0; }
     s.L = g.extent[last]; s.a_axis_stride = g.a_stride[last];
-    AM_TRY(dispatch<T>(op, s, s.L >= 64, 256 + tmp_bytes));
-    r.a = tmp; r.L = rows; r.a_axis_stride = 1;
-    AM_TRY(dispatch<T>(op, r, r.L >= 64, 256 + tmp_bytes));
+    int rc = dispatch<T>(op, s, s.L >= 64, ws_off);
+    if (rc == AM_OK) {
+      r.a = tmp; r.L = rows; r.a_axis_stride = 1;
+      rc = dispatch<T>(op, r, r.L >= 64, ws_off);
+    }
+    if (rc == AM_OK) rc = fetch_result(result, out, sizeof(T));   // blocking: the partials are no longer in use afterwards
+    if (big) (void)am_hip_free(big);
+    return rc;
   }
   return fetch_result(result, out, sizeof(T));
 }

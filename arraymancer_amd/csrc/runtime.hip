@@ -110,6 +110,30 @@ static size_t round_size(size_t bytes) {
   return (bytes + g - 1) / g * g;
 }
 
+// Blocks freed while a graph is being captured: the recorded kernels may use them (a temporary that a
+// host layer allocated before the capture and dropped inside it), so they stay allocated, owned by the
+// graph, and go back to the cache when the graph is destroyed.
+static std::vector<void*> g_capture_freed;
+static std::unordered_map<void*, std::vector<void*>> g_graph_blocks;   // executable graph -> blocks it keeps alive
+
+// Hands a live block back: to the cache, or to the driver when the cache is full. g_alloc_mu held.
+static int free_block_locked(void* dptr) {
+  auto it = g_live.find(dptr);
+  if (it == g_live.end()) return fail(AM_E_ARG, "am_hip_free: %p was not allocated by am_hip_malloc (or freed twice)", dptr);
+  const size_t rounded = it->second;
+  g_live.erase(it);
+  g_live_bytes -= rounded;
+  if (g_cached_bytes + rounded <= cache_limit()) {
+    g_free_blocks[rounded].push_back(dptr);
+    g_cached_bytes += rounded;
+    return AM_OK;
+  }
+  // Work that still reads or writes the buffer is on the library stream: drain it first.
+  AM_HIP_TRY(hipStreamSynchronize(g_stream));
+  AM_HIP_TRY(hipFree(dptr));
+  return AM_OK;
+}
+
 static void release_cached_locked() {
   for (auto& kv : g_free_blocks)
     for (void* p : kv.second) (void)hipFree(p);
@@ -191,22 +215,16 @@ int am_hip_malloc(size_t bytes, void** out) {
 int am_hip_free(void* dptr) {
   if (!dptr) return AM_OK;
   AM_TRY(ensure_init());
-  if (g_capturing) return fail(AM_E_ARG, "am_hip_free: not allowed while a graph is being captured");
   std::lock_guard<std::mutex> lk(g_alloc_mu);
-  auto it = g_live.find(dptr);
-  if (it == g_live.end()) return fail(AM_E_ARG, "am_hip_free: %p was not allocated by am_hip_malloc (or freed twice)", dptr);
-  const size_t rounded = it->second;
-  g_live.erase(it);
-  g_live_bytes -= rounded;
-  if (g_cached_bytes + rounded <= cache_limit()) {
-    g_free_blocks[rounded].push_back(dptr);
-    g_cached_bytes += rounded;
+  if (g_capturing) {   // kept for the graph being recorded, see g_capture_freed
+    if (g_live.find(dptr) == g_live.end())
+      return fail(AM_E_ARG, "am_hip_free: %p was not allocated by am_hip_malloc (or freed twice)", dptr);
+    for (void* q : g_capture_freed)
+      if (q == dptr) return fail(AM_E_ARG, "am_hip_free: %p freed twice", dptr);
+    g_capture_freed.push_back(dptr);
     return AM_OK;
   }
-  // Work that still reads or writes the buffer is on the library stream: drain it first.
-  AM_HIP_TRY(hipStreamSynchronize(g_stream));
-  AM_HIP_TRY(hipFree(dptr));
-  return AM_OK;
+  return free_block_locked(dptr);
 }
 
 int am_hip_empty_cache(void) {
@@ -301,11 +319,21 @@ int am_hip_graph_end(void** graph_exec) {
   if (!g_capturing) return fail(AM_E_ARG, "am_hip_graph_end: no capture in progress");
   g_capturing = false;
   hipGraph_t graph = nullptr;
-  AM_HIP_TRY(hipStreamEndCapture(g_stream, &graph));
   hipGraphExec_t exec = nullptr;
-  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-  (void)hipGraphDestroy(graph);
-  if (e != hipSuccess) return fail(AM_E_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  hipError_t e = hipStreamEndCapture(g_stream, &graph);
+  if (e == hipSuccess) {
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+  }
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  if (e != hipSuccess) {   // no graph will replay anything: the blocks freed meanwhile go back now
+    for (void* q : g_capture_freed) (void)free_block_locked(q);
+    g_capture_freed.clear();
+    (void)hipGetLastError();
+    return fail(AM_E_HIP, "ending the capture failed: %s", hipGetErrorString(e));
+  }
+  if (!g_capture_freed.empty()) g_graph_blocks[(void*)exec] = std::move(g_capture_freed);
+  g_capture_freed.clear();
   *graph_exec = (void*)exec;
   return AM_OK;
 }
@@ -322,6 +350,12 @@ int am_hip_graph_destroy(void* graph_exec) {
   if (!graph_exec) return AM_OK;
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
   AM_HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  auto it = g_graph_blocks.find(graph_exec);
+  if (it != g_graph_blocks.end()) {   // what was freed during its capture is free now
+    for (void* q : it->second) (void)free_block_locked(q);
+    g_graph_blocks.erase(it);
+  }
   return AM_OK;
 }
 

@@ -50,9 +50,12 @@ class HipStorage:
         ptr, self.ptr = getattr(self, "ptr", 0), 0
         if ptr:
             try:
-                _lib.load().am_hip_free(ctypes.c_void_p(ptr))
+                rc = _lib.load().am_hip_free(ctypes.c_void_p(ptr))
             except Exception:  # interpreter shutdown
-                pass
+                return
+            if rc != 0:        # a destructor cannot raise: say so instead of leaking silently
+                import warnings
+                warnings.warn(f"am_hip_free failed ({rc}): {_lib.last_error()}", ResourceWarning)
 
 
 def _dtype_sfx(dtype) -> str:
@@ -296,7 +299,10 @@ class Graph:
     """Records the device operations issued inside `with Graph() as g:` into a HIP graph instead
     of running them; `g.launch()` replays the sequence with one call. Output tensors must be
     allocated before the block (allocation is refused during capture), e.g. with `empty` and the
-    `gemm(alpha, A, B, beta, C)` / `apply2` / `_into` forms."""
+    `gemm(alpha, A, B, beta, C)` / `apply2` / `_into` forms. A tensor that goes out of scope inside the
+    block is kept alive by the graph (the library holds its block until the graph is destroyed); tensors
+    recorded in the graph and dropped after the block must outlive the replays - pass them to `keep()`
+    to tie their lifetime to the graph's."""
 
     def __init__(self):
         self._exec = ctypes.c_void_p()
@@ -313,6 +319,11 @@ class Graph:
 
     def launch(self):
         check(_lib.load().am_hip_graph_launch(self._exec))
+
+    def keep(self, *tensors):
+        """Holds a reference to the storage of each tensor for as long as this graph exists."""
+        self._kept = getattr(self, "_kept", []) + [t.storage for t in tensors]
+        return self
 
     def __del__(self):
         ex, self._exec = getattr(self, "_exec", None), None

@@ -59,7 +59,9 @@ int am_hip_device_info(char* name, size_t name_cap, int* compute_units, int* clo
  * handed out again while earlier work on the library stream still uses it (whatever touches it next
  * goes through that stream too). am_hip_free only accepts pointers from am_hip_malloc. */
 int am_hip_malloc(size_t bytes, void** out);   /* bytes == 0 -> *out = NULL, AM_OK */
-int am_hip_free(void* dptr);                   /* NULL is a no-op */
+int am_hip_free(void* dptr);                   /* NULL is a no-op. While a graph is being captured the block is not
+                                                  released but kept for that graph (its kernels may use it) until
+                                                  am_hip_graph_destroy; it counts as live meanwhile. */
 /* No counterpart in the reference (it cudaMallocs / cudaFrees per tensor): returns every cached
  * block to the driver (drains the stream first); byte counts of the blocks in use and in the cache.
  * Cache size limit: environment variable AM_HIP_CACHE_LIMIT_MB (default 32768; 0 = no caching). */
@@ -85,7 +87,8 @@ int am_hip_event_destroy(void* ev);
  * kernels such as the reference's per-layer gemm + `+.=` + relu sequence
  * (src/arraymancer/nn_primitives/nnp_linear.nim:28-29, fallback/conv.nim:99-106). The reference
  * has no counterpart (one launch per operator, backend/cuda.nim). Buffers recorded in a graph must
- * stay allocated while it is replayed. */
+ * stay allocated while it is replayed: a block freed DURING the capture is kept alive by the graph itself,
+ * one freed after am_hip_graph_end is the caller's responsibility. */
 int am_hip_graph_begin(void);
 int am_hip_graph_end(void** graph_exec);
 int am_hip_graph_launch(void* graph_exec);

@@ -172,7 +172,9 @@ struct HipStorage {
     check(am_hip_malloc((size_t)n * sizeof(T), &p));
     data = static_cast<T*>(p);
   }
-  ~HipStorage() { am_hip_free(data); }
+  // am_hip_free does not fail for a block of am_hip_malloc (inside a graph capture the library keeps the
+  // block for the graph instead of releasing it); a destructor could not report it anyway.
+  ~HipStorage() { (void)am_hip_free(data); }
   HipStorage(const HipStorage&) = delete;
   HipStorage& operator=(const HipStorage&) = delete;
 };

@@ -10,10 +10,13 @@ CPP_DIR = os.path.join(ROOT, "tests", "cpp")
 BIN = os.path.join(CPP_DIR, "test_tensor_hip")
 
 
+BIN_ASAN = os.path.join(CPP_DIR, "test_tensor_hip_asan")
+
+
 def test_cpp_host_layer_builds():
-    res = subprocess.run(["make", "-C", CPP_DIR, "-B", "test_tensor_hip"], capture_output=True, text=True)
+    res = subprocess.run(["make", "-C", CPP_DIR, "-B", "test_tensor_hip", "test_tensor_hip_asan"], capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-3000:]
-    assert os.path.exists(BIN)
+    assert os.path.exists(BIN) and os.path.exists(BIN_ASAN)
 
 
 @pytest.mark.gpu
@@ -24,3 +27,17 @@ def test_cpp_host_layer_on_device(hip):
     print(res.stdout)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-1000:]
     assert " 0 failed" in res.stdout
+
+
+@pytest.mark.gpu
+def test_cpp_host_layer_on_device_under_sanitizers(hip):
+    """The same program with its host side (tensor ownership, views, printing, the test code) under
+    AddressSanitizer + UndefinedBehaviorSanitizer. Leak detection is off: the HIP runtime keeps its own
+    allocations until the process ends."""
+    if not os.path.exists(BIN_ASAN):
+        pytest.fail("tests/cpp/test_tensor_hip_asan is not built (python -c 'import __graft_entry__ as g; g.build()')")
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:protect_shadow_gap=0", UBSAN_OPTIONS="halt_on_error=1:print_stacktrace=1")
+    res = subprocess.run([BIN_ASAN, os.path.join(ROOT, "tests", "golden", "npy")], capture_output=True, text=True, timeout=180, env=env)
+    print(res.stdout)
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
+    assert " 0 failed" in res.stdout and "AddressSanitizer" not in res.stderr and "runtime error" not in res.stderr

@@ -728,3 +728,31 @@ def test_clamp(hip, oracle, sfx):
     if sfx in FLT:
         s = hip.clamp(hip.toHip(np.array([np.nan, -np.inf, np.inf, -0.0, 5.0], dtype=dt)), 0, 1).toCpu()
         assert np.isnan(s[0]) and s[1] == 0 and s[2] == 1 and s[3] == 0 and np.signbit(s[3]) and s[4] == 1
+
+
+def test_more_than_2_pow_31_elements(hip):
+    """A destination of 2^31 + 2^20 int32 elements (8 GiB): the streaming kernel's row / tile counters and the
+    generic kernel's switch from 32- to 64-bit element indices are both past 2^31 here. Written through
+    zero-stride (broadcast) operands and checked by folds on the device, so nothing of that size is copied."""
+    n_rows, L = (1 << 15) + 16, 1 << 16                      # 32784 x 65536 = 2^31 + 2^20 elements
+    col = np.arange(n_rows, dtype=np.int32).reshape(n_rows, 1) % 7 - 3
+    row = (np.arange(L, dtype=np.int32).reshape(1, L) % 5) * 11
+    dcol, drow = hip.toHip(col), hip.toHip(row)
+    say("8 GiB destination, streaming kernel")
+    big = hip.bc_add(dcol, drow)                             # [n_rows, L], rows kernel (row vector + one scalar per row)
+    assert big.size > 2**31
+    want_sum = int(col.astype(np.int64).sum()) * L + int(row.astype(np.int64).sum()) * n_rows
+    wrap = lambda v: ((v + 2**31) % 2**32) - 2**31
+    assert int(hip.sum(big)) == wrap(want_sum)               # int32 sums wrap
+    assert int(hip.max(big)) == int(col.max() + row.max()) and int(hip.min(big)) == int(col.min() + row.min())
+    # the first and the last row, each through a small device-side gather (toCpu of a view copies its whole storage)
+    assert np.array_equal(big[:1, :].clone().toCpu(), col[:1] + row)
+    assert np.array_equal(big[n_rows - 1:, :].clone().toCpu(), col[n_rows - 1:] + row)
+    del big
+    say("8 GiB destination, generic kernel (64-bit element index)")
+    # inner stride -1 on an operand sends the same shape to the generic kernel
+    rrow = hip.toHip(row[:, ::-1].copy())[:, ::-1]           # the same values seen through a reversed view
+    big2 = hip.bc_add(dcol, rrow)
+    assert int(hip.sum(big2)) == wrap(want_sum)
+    assert np.array_equal(big2[n_rows - 1:, :].clone().toCpu(), col[n_rows - 1:] + row)
+    assert np.array_equal(big2[:1, :].clone().toCpu(), col[:1] + row)

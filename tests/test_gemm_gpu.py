@@ -303,8 +303,9 @@ def test_config2_i32_1500_bit_exact(hip, oracle):
 
 @pytest.mark.parametrize("sfx", ["i32", "i64"])
 def test_config2_4096_ring_checksum(hip, oracle, sfx):
-    """Full size, checked through a property that holds exactly in Z / 2^w:
-    (A B) v == A (B v) for any v, plus a bit-exact block against the oracle."""
+    """Full size: every one of the 4096 x 4096 outputs against the oracle's blocked gemm_strided, and, as a
+    second check that shares nothing with it, a property that holds exactly in Z / 2^w:
+    (A B) v == A (B v) for any v."""
     dt = DTYPES[sfx]
     n = 4096
     A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(dt)
@@ -318,8 +319,27 @@ def test_config2_4096_ring_checksum(hip, oracle, sfx):
         rhs = U(A) @ (U(B) @ v)
     mask = np.uint64(0xFFFFFFFF) if sfx == "i32" else np.uint64(0xFFFFFFFFFFFFFFFF)
     assert np.array_equal(lhs & mask, rhs & mask)
-    rows = slice(1000, 1192)
-    assert np.array_equal(C[rows], oracle.matmul(A[rows], B))
+    assert np.array_equal(C, oracle.matmul(A, B))            # the whole matrix
+
+
+def test_i64_4096_whole_range_all_digit_pairs(hip, oracle):
+    """int64 4096^3 with entries over the whole int64 range: all 36 digit pairs of the matrix-core path are
+    live and every accumulator wraps many times. Whole matrix through the ring checksum, a block of rows
+    against the closed form in unsigned 64-bit arithmetic (NumPy's uint64 product wraps modulo 2^64) and
+    against the oracle's blocked kernel."""
+    n = 4096
+    info = np.iinfo(np.int64)
+    A = np.random.default_rng(2011).integers(info.min, info.max, (n, n), endpoint=True).astype(np.int64)
+    B = np.random.default_rng(2012).integers(info.min, info.max, (n, n), endpoint=True).astype(np.int64)
+    say("i64 4096^3 whole range")
+    C = (hip.toHip(A) * hip.toHip(B)).toCpu()
+    U = lambda x: x.view(np.uint64)
+    v = np.random.default_rng(6).integers(info.min, info.max, (n, 1)).astype(np.int64)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(U(C) @ U(v), U(A) @ (U(B) @ U(v)))
+        rows = slice(3000, 3256)
+        assert np.array_equal(U(C[rows]), U(np.ascontiguousarray(A[rows])) @ U(B))
+    assert np.array_equal(C[rows], oracle.matmul(np.ascontiguousarray(A[rows]), B))
 
 
 def test_config3_f64_views(hip, oracle):
@@ -362,13 +382,17 @@ def test_config5_inference_chain(hip, oracle):
 
 
 def test_fp32_4096_properties(hip, oracle):
-    """Full headline size: linearity in alpha and agreement of a row block with float64."""
+    """Full headline size: the whole 4096 x 4096 result against the oracle's gemm_strided (<= 1e-4 relative
+    Frobenius error, the float32 bar of the path) and against the float64 product, a row block on its own, and
+    linearity in alpha."""
     n = 4096
     A = np.random.default_rng(1001).uniform(-1, 1, (n, n)).astype(np.float32)
     B = np.random.default_rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
     dA, dB = hip.toHip(A), hip.toHip(B)
     say("f32 4096^3")
     C1 = (dA * dB).toCpu()
+    assert oracle.rel_frobenius(C1, oracle.matmul(A, B)) <= 1e-4                          # the whole matrix
+    assert oracle.rel_frobenius(C1, A.astype(np.float64) @ B.astype(np.float64)) <= 1e-4
     rows = slice(2048, 2048 + 128)
     assert oracle.rel_frobenius(C1[rows], A[rows].astype(np.float64) @ B.astype(np.float64)) <= 1e-4
     dC = hip.empty((n, n), np.float32)

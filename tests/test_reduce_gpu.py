@@ -358,3 +358,20 @@ def test_maxpool_vs_oracle(hip, oracle, vectors, sfx):
         hip.maxpool2d(hip.zeros((4, 4), dt), (2, 2))                       # rank
     with pytest.raises(ValueError):
         hip.maxpool2d(hip.zeros((2, 3, 4, 4), dt).transpose(), (2, 2))     # not C-contiguous (the reference asserts)
+
+
+def test_reduce_all_of_a_view_with_millions_of_runs(hip, oracle):
+    """Whole-tensor folds of a strided view whose per-run partials (one per row here: 4.5 M rows x 8 bytes = 36 MB)
+    exceed what the library keeps in its workspace: the partials then come from the block cache."""
+    rows = 4_500_000
+    rng = np.random.default_rng(seed_of("reduce-many-runs"))
+    parent = rng.integers(-3, 3, (rows, 4), endpoint=True).astype(np.int64)
+    d = hip.toHip(parent)
+    view, host = d[:, 1:3], parent[:, 1:3]                     # [4.5 M, 2] with row stride 4: 4.5 M runs of 2
+    say("reduce_all, strided view with 4.5 M runs")
+    assert hip.sum(view) == host.sum()
+    assert hip.max(view) == host.max() and hip.min(view) == host.min()
+    f = hip.toHip(parent.astype(np.float64))[::1, 0:3:2]       # columns 0 and 2: inner stride 2
+    want = parent[:, 0:3:2].astype(np.float64)
+    assert abs(hip.sum(f) - want.sum()) <= 1e-9 * np.abs(want).sum()
+    assert hip.mean(f) == pytest.approx(want.mean(), rel=1e-12)

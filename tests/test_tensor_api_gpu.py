@@ -175,3 +175,42 @@ def test_display_of_device_tensors(hip):
     assert hip.bc_ge(sl, 3.0).pretty(specifier="<>") == "HipTensor[bool]<2,2>:[[false, true], [true, true]]"
     assert hip.toHip(np.array([0.9532932, 0.12945823])).pretty(precision=4, specifier="[]") == "[0.9533, 0.1295]"
     assert str(hip.empty((0, 3), np.float64)) == 'HipTensor[system.float] of shape "[0, 3]" on backend "Hip"\n    [] (empty)'
+
+
+def test_free_during_graph_capture_is_deferred_to_the_graph(hip):
+    """A tensor dropped inside `with Graph()` is neither leaked nor handed out again while the graph can
+    still replay the kernels that use it: the block stays live until the graph is destroyed, then goes back
+    to the cache. Live / cached byte counts balance across the whole capture."""
+    import ctypes
+    import gc
+    L = hip.load_library()
+    live, cached = ctypes.c_size_t(), ctypes.c_size_t()
+
+    def stats():
+        assert L.am_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached)) == 0
+        return live.value, cached.value
+
+    x = np.random.default_rng(3).uniform(-1, 1, (256, 1024)).astype(np.float32)
+    dx, out = hip.toHip(x), hip.empty((256, 1024), np.float32)
+    assert L.am_hip_empty_cache() == 0
+    live0, _ = stats()
+    tmp = hip.toHip(2 * x)                      # 1 MiB of data, allocated before the capture
+    live_tmp, _ = stats()
+    assert live_tmp > live0
+    from arraymancer_amd import tensor_hip as th
+    with hip.Graph() as g:
+        th._binary_into("add", out, dx, tmp)    # the graph reads tmp ...
+        del tmp                                 # ... and tmp goes out of scope inside the capture
+        gc.collect()
+    assert stats() == (live_tmp, 0)             # still live: the graph owns it; nothing was cached
+    other = hip.empty((256, 1024), np.float32)  # must not receive tmp's block
+    th._unary_into("copy", other, dx)
+    for _ in range(3):
+        g.launch()
+        assert np.array_equal(out.toCpu(), x + 2 * x)
+        th._unary_into("neg", out, out)
+    del other
+    del g
+    gc.collect()
+    assert L.am_hip_empty_cache() == 0
+    assert stats() == (live0, 0)                # the deferred block came back when the graph went away
