@@ -68,11 +68,15 @@ __device__ __forceinline__ int live_digit_pairs(const uint32_t* flags, uint32_t 
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+// An operand with a unit stride is moved in 16-byte vectors whatever its row pitch, extent or base address
+// (the loaders take care of vectors that straddle an edge); a row shorter than one vector, a negative pitch
+// along the vectors' direction... everything else is gathered element by element.
 template <typename T>
 static inline int classify(const T* X, int64_t ld_mn, int64_t ld_k, int64_t MN, int64_t K) {
   constexpr int64_t VK = 16 / (int64_t)sizeof(T);
-  if (ld_k == 1 && K % VK == 0 && (ld_mn % VK == 0 || MN == 1) && ld_mn >= 0 && aligned16(X)) return kKContig;
-  if (ld_mn == 1 && MN % VK == 0 && (ld_k % VK == 0 || K == 1) && ld_k >= 0 && aligned16(X)) return kMNContig;
+  (void)X;
+  if (ld_k == 1 && K >= VK && ld_mn >= 0) return kKContig;
+  if (ld_mn == 1 && MN >= VK && (MN % VK == 0 ? ld_k >= 0 : ld_k >= MN)) return kMNContig;   // ragged rows must not overlap
   return kGeneric;
 }
 

@@ -7,11 +7,8 @@ using namespace am::gemm;
 
 static int run_f32(Args<float>& g) {
   if (small::applicable(g)) return small::run(g);   // few rows or columns: no LDS staging, no second kernel
-  constexpr int64_t VK = 16 / (int64_t)sizeof(float);
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
-  if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;   // every batch member must stay 16-byte aligned
-  if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
   // Candidate workgroup tiles with the relative MFMA efficiency of each (measured on 2048^3 and
   // 4096^3). PF = 2 (two slabs of global loads in flight) on the tiles whose slab is short.
   static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.94}, {64, 64, 0.88}, {256, 128, 0.97}, {128, 64, 0.92}, {32, 32, 0.74}};

@@ -7,11 +7,8 @@ using namespace am::gemm;
 
 static int run_f64(Args<double>& g) {
   if (small::applicable(g)) return small::run(g);   // few rows or columns: no LDS staging, no second kernel
-  constexpr int64_t VK = 16 / (int64_t)sizeof(double);
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
-  if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;   // every batch member must stay 16-byte aligned
-  if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
   // Candidate workgroup tiles with the relative MFMA efficiency of each. The 128 x 128 tile runs
   // with 8 wavefronts (64 x 32 each) and the 256 x 128 one without fragment prefetch: a 64 x 64
   // wavefront tile of doubles (128 accumulator registers) leaves no room for a second fragment set.

@@ -7,11 +7,8 @@ using namespace am;
 using namespace am::gemm;
 
 static int run_i64(Args<int64_t>& g) {
-  constexpr int64_t VK = 16 / (int64_t)sizeof(int64_t);
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
-  if (g.batch > 1 && g.batch_a % VK != 0) ak = kGeneric;
-  if (g.batch > 1 && g.batch_b % VK != 0) bk = kGeneric;
   // 8 x 8 and 4 x 4 results per lane; the small tile re-reads LDS twice as often per multiply-add.
   static const TileChoice cand[] = {{128, 128, 1.0}, {64, 64, 0.85}};
   // 34.0e3 multiply-adds per microsecond and CU: the measured VALU ceiling of this element type.

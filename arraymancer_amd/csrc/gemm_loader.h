@@ -12,11 +12,15 @@
 namespace am {
 namespace gemm {
 
+// vec_t: a 16-byte vector in registers / LDS. gvec_t: the same vector as it sits in global memory, where only
+// the element's own alignment is promised (a row of 4095 floats starts 4 bytes off every 16): the hardware
+// serves a 16-byte global load from any dword-aligned address, so an operand with a unit stride is moved in
+// 16-byte pieces whatever its row pitch, extent or base address.
 template <typename T> struct VecTraits;
-template <> struct VecTraits<float> { static constexpr int VK = 4; typedef float vec_t __attribute__((ext_vector_type(4))); };
-template <> struct VecTraits<double> { static constexpr int VK = 2; typedef double vec_t __attribute__((ext_vector_type(2))); };
-template <> struct VecTraits<int32_t> { static constexpr int VK = 4; typedef int32_t vec_t __attribute__((ext_vector_type(4))); };
-template <> struct VecTraits<int64_t> { static constexpr int VK = 2; typedef int64_t vec_t __attribute__((ext_vector_type(2))); };
+template <> struct VecTraits<float> { static constexpr int VK = 4; typedef float vec_t __attribute__((ext_vector_type(4))); typedef vec_t gvec_t __attribute__((aligned(4))); };
+template <> struct VecTraits<double> { static constexpr int VK = 2; typedef double vec_t __attribute__((ext_vector_type(2))); typedef vec_t gvec_t __attribute__((aligned(8))); };
+template <> struct VecTraits<int32_t> { static constexpr int VK = 4; typedef int32_t vec_t __attribute__((ext_vector_type(4))); typedef vec_t gvec_t __attribute__((aligned(4))); };
+template <> struct VecTraits<int64_t> { static constexpr int VK = 2; typedef int64_t vec_t __attribute__((ext_vector_type(2))); typedef vec_t gvec_t __attribute__((aligned(8))); };
 
 // LDS geometry of one operand slab (BMN rows/cols x BK k values).
 template <typename T, int KIND, int BMN, int BK, bool KG = true> struct Slab {
@@ -49,6 +53,7 @@ template <typename T, int KIND, int BMN, int BK, int NT, bool KG = true, int PF 
 
 template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kKContig, BMN, BK, NT, KG, PF> {
   typedef typename VecTraits<T>::vec_t vec_t;
+  typedef typename VecTraits<T>::gvec_t gvec_t;
   static constexpr int VK = VecTraits<T>::VK;
   static constexpr int QN = BK / VK;               // vectors per row
   static constexpr int NV = BMN * QN / NT;         // vectors per thread
@@ -64,13 +69,35 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
       ptr[i] = X + ((mn0 + mn) < MN ? mn0 + mn : MN - 1) * ld_mn + q * VK;
     }
   }
+  __device__ __forceinline__ bool tail_guard() const { return false; }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
     if (MASK && k0 >= K) return;   // slab wholly past the end: commit writes zeros without these registers
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int q = (threadIdx.x + i * NT) % QN;
-      if constexpr (MASK) reg[S][i] = *(const vec_t*)(ptr[i] + ((k0 + q * VK) < K ? k0 : (int64_t)(-q * VK)));
-      else reg[S][i] = *(const vec_t*)(ptr[i] + k0);
+      if constexpr (MASK) {
+        // A vector that straddles the end of the k range (K not a multiple of VK) is read from where it
+        // ends at K instead and moved into place (what lies past K is zeroed): nothing past the last element
+        // of a row is ever touched. A vector wholly past the end repeats the row's first one. (The host sends
+        // k ranges shorter than one vector to the element-wise loader.)
+        const int64_t kv = k0 + q * VK;
+        const int64_t over = kv + VK - K;                       // elements past the end, if positive
+        const bool straddles = (K % VK != 0) && over > 0 && over < VK;   // first test uniform: nothing to do for whole vectors
+        const vec_t v = *(const gvec_t*)(ptr[i] + (kv >= K ? (int64_t)(-q * VK) : straddles ? k0 - over : k0));
+        vec_t r = v;
+        if (straddles) {
+#pragma unroll
+          for (int e = 0; e < VK; ++e) {
+            T x = (T)0;
+#pragma unroll
+            for (int f = 0; f < VK; ++f) x = (e + over == f) ? v[f] : x;
+            r[e] = x;
+          }
+        }
+        reg[S][i] = r;
+      } else {
+        reg[S][i] = *(const gvec_t*)(ptr[i] + k0);
+      }
     }
   }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
@@ -81,8 +108,9 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int q = (threadIdx.x + i * NT) % QN;
-        vec_t z = {};
-        if ((k0 + q * VK) >= K) reg[S][i] = z;
+#pragma unroll
+        for (int e = 0; e < VK; ++e)
+          if ((k0 + q * VK + e) >= K) reg[S][i][e] = (T)0;
       }
     }
 #pragma unroll
@@ -103,28 +131,57 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
 
 template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kMNContig, BMN, BK, NT, KG, PF> {
   typedef typename VecTraits<T>::vec_t vec_t;
+  typedef typename VecTraits<T>::gvec_t gvec_t;
   static constexpr int VK = VecTraits<T>::VK;
   static constexpr int CN = BMN / VK;              // vectors per k row
   static constexpr int NV = CN * BK / NT;
   static_assert(CN * BK % NT == 0 && NV >= 1, "slab must divide evenly over the workgroup");
   const T* ptr[NV];
   int64_t K, ld_k;
+  // The one vector per k row that straddles the edge of the operand (MN not a multiple of VK; edge tiles only)
+  // reads up to VK - 1 elements past the end of its row. In every k row but the operand's last one those are
+  // the first elements of the next row (the host sends operands whose rows overlap elsewhere), and what they
+  // hold only reaches columns of C past its edge. The last row must not be overrun: the MASK = true versions,
+  // which the kernel runs for the slab that holds it (tail_guard), read that vector from where it ends at MN,
+  // `shift` elements back, and move it into place in registers.
+  int shift[NV];
+  bool shift_any;   // uniform over the workgroup
   vec_t reg[PF][NV];
   __device__ __forceinline__ Loader(const T* X, int64_t, int64_t ld_k_, int64_t mn0, int64_t MN, int64_t K_, int) : K(K_), ld_k(ld_k_) {
+    shift_any = (MN % VK != 0) && (mn0 + BMN > MN);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = threadIdx.x + i * NT;
       const int c = v % CN, k = v / CN;
-      ptr[i] = X + ((mn0 + c * VK) < MN ? mn0 + c * VK : 0) + k * ld_k;
+      const int64_t col = mn0 + c * VK;
+      const int64_t over = col + VK - MN;          // elements past the edge, if positive
+      shift[i] = (over > 0 && over < VK) ? (int)over : 0;
+      ptr[i] = X + (col < MN ? col : 0) + k * ld_k;
     }
   }
+  // True when the unmasked fetch must not be used for the slab that holds the last k row.
+  __device__ __forceinline__ bool tail_guard() const { return shift_any; }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
     if (MASK && k0 >= K) return;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int k = (threadIdx.x + i * NT) / CN;
-      if constexpr (MASK) reg[S][i] = *(const vec_t*)(ptr[i] + ((k0 + k) < K ? k0 : (int64_t)(-k)) * ld_k);
-      else reg[S][i] = *(const vec_t*)(ptr[i] + k0 * ld_k);
+      if constexpr (MASK) {
+        const vec_t v = *(const gvec_t*)(ptr[i] - shift[i] + ((k0 + k) < K ? k0 : (int64_t)(-k)) * ld_k);
+        vec_t r = v;
+        if (shift_any) {
+#pragma unroll
+          for (int e = 0; e < VK; ++e) {
+            T x = v[e];
+#pragma unroll
+            for (int f = 0; f < VK; ++f) x = (shift[i] != 0 && e + shift[i] == f) ? v[f] : x;
+            r[e] = x;
+          }
+        }
+        reg[S][i] = r;
+      } else {
+        reg[S][i] = *(const gvec_t*)(ptr[i] + k0 * ld_k);
+      }
     }
   }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
@@ -173,6 +230,7 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
       ptr[i] = X + cm * ld_mn + (int64_t)k * ld_k;
     }
   }
+  __device__ __forceinline__ bool tail_guard() const { return false; }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
     if (MASK && k0 >= K) return;
     const int64_t step = k0 * ld_k;

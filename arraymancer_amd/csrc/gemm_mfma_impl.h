@@ -155,7 +155,9 @@ void gemm_mfma(Args<T> p) {
   constexpr int NKS = BK / KSTEP;
   const int64_t ktiles = (k_end - k_begin + BK - 1) / BK;
   const int64_t kt_run = (ktiles + PF - 1) / PF * PF;
-  const int64_t full_slabs = (k_end - k_begin) / BK;
+  // Slabs that the unmasked (steady-state) loop may fetch: those wholly inside the k range, less the last
+  // one when a loader must not run its unmasked fetch on the operand's last k row (see tail_guard).
+  const int64_t full_slabs = (k_end - k_begin) / BK - ((la.tail_guard() || lb.tail_guard()) ? 1 : 0);
 
   T af[2][TM][VK], bf[2][TN][VK];
   auto read_frags = [&](auto parity_tag, const T* a_lds, const T* b_lds, int ks) {

@@ -414,8 +414,14 @@ def config_report(am, timer, L):
         A = rng(1001).uniform(-1, 1, (n, n)).astype(np.float32); B = rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
         gemm_case(f"f32 GEMM {n}^3", "f32", n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_F32_PEAK_TFLOPS,
                   peak_used="MFMA fp32 157.3 TFLOP/s", steps=50 if n == 1024 else 20)
+    # extents that are not a multiple of the 16-byte vector, beside their aligned neighbour (4096): unit-stride
+    # operands are moved in 16-byte pieces whatever their pitch; 4097 pays for a second, nearly empty round of tiles
+    for n in (4095, 4097):
+        A = rng(1001).uniform(-1, 1, (n, n)).astype(np.float32); B = rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
+        gemm_case(f"f32 GEMM {n}^3 (ragged extents)", "f32", n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_F32_PEAK_TFLOPS,
+                  peak_used="MFMA fp32 157.3 TFLOP/s", steps=20)
     for sfx, dt, key in (("i32", np.int32, "valu_int32_mac"), ("i64", np.int64, "valu_int64_mac")):
-        for n in (1500, 4096):
+        for n in (1500, 1501, 4096) if sfx == "i32" else (1500, 4096):
             A = rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(dt)
             B = rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(dt)
             env = f"AM_HIP_GEMM_{sfx.upper()}_PATH"

@@ -117,6 +117,44 @@ def test_every_tile_shape(hip, oracle, sfx, tile, monkeypatch):
     assert_parity(oracle, sfx, dC.toCpu(), want, f"tile {tile}")
 
 
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("layout", ["CC", "FC", "CF", "FF"])
+def test_unit_stride_operands_of_any_pitch_and_alignment(hip, oracle, sfx, layout):
+    """Operands with a unit stride are moved in 16-byte vectors whatever their row pitch, extent and base
+    address: extents that are not a multiple of the vector (k, m and n all ragged), pitches that put every
+    row at another offset within 16 bytes, base addresses one element off, and views that end exactly at the
+    end of their allocation (so that a vector read past the last row would leave it)."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("ragged", sfx, layout))
+    vk = 16 // np.dtype(dt).itemsize
+    for (M, N, K) in [(259, 131, 67), (64 + 1, 4 * vk + 1, vk + 1), (300, 257, 2 * vk - 1)]:
+        # parents sized to a whole number of 512-byte allocation granules, views that drop the FIRST row and
+        # column: the view's last element is the allocation's last element
+        def parent_and_view(rows, cols, fortran):
+            pr, pc = (cols + 1, rows + 1) if fortran else (rows + 1, cols + 1)
+            pad = (-(pr * pc * np.dtype(dt).itemsize)) % 512 // np.dtype(dt).itemsize
+            return fill(rng, (pad + pr * pc,), dt), pad, pr, pc
+        views_np, views_dev = [], []
+        for (rows, cols), fortran in (((M, K), layout[0] == "F"), ((K, N), layout[1] == "F")):
+            flat, pad, pr, pc = parent_and_view(rows, cols, fortran)
+            host = flat[pad:].reshape(pr, pc)[1:, 1:]
+            dflat = hip.toHip(flat)
+            from arraymancer_amd import metadata as md
+            from arraymancer_amd.tensor_hip import HipTensor
+            dev = HipTensor(md.Layout((pr - 1, pc - 1), (pc, 1), pad + pc + 1), dflat.storage, dflat.dtype)
+            if fortran:
+                host, dev = host.T, dev.transpose()
+            assert host.shape == (rows, cols) and dev.shape == (rows, cols)
+            views_np.append(host); views_dev.append(dev)
+        C = fill(rng, (M, N), dt)
+        for alpha, beta in ((1, 0), (2, 1)):
+            say("ragged", sfx, layout, (M, N, K), alpha, beta)
+            want = oracle.gemm_strided(alpha, views_np[0], views_np[1], beta, C.copy())
+            dC = hip.toHip(C)
+            hip.gemm(alpha, views_dev[0], views_dev[1], beta, dC)
+            assert_parity(oracle, sfx, dC.toCpu(), want, f"{layout} {(M, N, K)}")
+
+
 # ------------------------------------------------------------------ strided / transposed views
 def device_view(hip, parent_np, kind, shape):
     """The same geometry as conftest.strided_view, built with view ops on the device tensor."""
