@@ -317,6 +317,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
                         same_buffers_every_step_ms=round(ev / steps * 1e3, 4), roofline=roof))
     del dXs, dYs
     out.append(bench_chain(am, timer, max(steps, 50), warmup))
+    out.append(bench_ex02(am, timer, max(steps, 50), warmup))
     return out
 
 
@@ -355,8 +356,32 @@ def bench_chain(am, timer, steps, warmup):
                 hipgraph_us=round(ev_g / steps * 1e6, 2),
                 eager_us=round(ev_e / steps * 1e6, 2), eager_wall_us=round(wall_e / steps * 1e6, 2),
                 gflops=round(flops / (min(ev_g, ev_e) / steps) / 1e9, 1),
-                note="launch/latency bound: 2.9e8 FLOP and 17.8 MB per chain; four kernels of 5-10 us; the eager figure "
-                     "includes the host's launch cost, the replayed graph pays more between its nodes")
+                note="kernel-time bound: 2.9e8 FLOP and 17.8 MB per chain in four kernels of 5-10 us whose durations sum to the eager "
+                     "figure; a graph replay adds about 3 us per launch of the graph on this runtime and removes about 1 us of "
+                     "host gap per kernel, so it pays from about six kernels per graph (the eight-launch forward pass below), "
+                     "not on these four")
+
+
+def bench_ex02(am, timer, steps, warmup, batch=64):
+    """The whole forward pass of the reference's example 2 (conv - ReLU - maxpool twice, two dense layers) at batch 64:
+    eight launches per pass issued from the host, and the same eight replayed from one HIP graph."""
+    from arraymancer_amd import ex02
+    rng = np.random.default_rng(5002)
+    net = ex02.DemoNet(batch, ex02.random_params(rng), np.float32)
+    dx = am.toHip(rng.uniform(0, 1, (batch, 1, 28, 28)).astype(np.float32))
+    wall_e, ev_e = timer.run(lambda: net.forward(dx), steps, warmup, WARM_S)
+    graph = net.capture(dx)
+    wall_g, ev_g = timer.run(graph.launch, steps, warmup, WARM_S)
+    flops = 2.0 * batch * (20 * 25 * 576 + 50 * 500 * 64 + 800 * 500 + 500 * 10)
+    best = min(ev_e, ev_g)
+    return dict(workload=f"f32 example-2 forward pass, batch {batch}: conv(1->20,5x5)+ReLU, maxpool 2x2, conv(20->50,5x5)+ReLU, "
+                         "maxpool 2x2, flatten, linear(800->500)+ReLU, linear(500->10); 8 launches",
+                unit="us per pass", dtype="f32", higher_is_better=False, value=round(best / steps * 1e6, 2),
+                value_is="eager" if ev_e <= ev_g else "hipgraph", eager_us=round(ev_e / steps * 1e6, 2),
+                eager_wall_us=round(wall_e / steps * 1e6, 2), hipgraph_us=round(ev_g / steps * 1e6, 2),
+                images_per_s=round(batch / (best / steps), 0), gflops=round(flops / (best / steps) / 1e9, 1),
+                note="3.0e8 FLOP per pass over eight kernels of 4-17 us whose durations sum to about 61 us: the graph replay runs "
+                     "them back to back, the eager pass leaves about 1 us of host launch gap after each")
 
 
 def config_report(am, timer, L):
@@ -531,6 +556,9 @@ def run_only(am, timer, which, steps, warmup):
     if which == "chain":
         r = bench_chain(am, timer, steps, warmup)
         return dict(only=which, hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"])
+    if which == "ex02":
+        r = bench_ex02(am, timer, steps, warmup)
+        return dict(only=which, hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"])
     if which in ("gemm_i32", "gemm_i32_valu"):
         if which == "gemm_i32_valu":
             os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"   # the vector-ALU kernel instead of the digit-sliced matrix-core path
@@ -539,6 +567,27 @@ def run_only(am, timer, which, steps, warmup):
         B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
         dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
         fn = lambda: am.gemm(1, dA, dB, 0, dC)
+    elif which in ("gemm_f32_1024", "gemm_f32_2048"):
+        n = int(which.rsplit("_", 1)[1])
+        dA = am.toHip(np.random.default_rng(1001).standard_normal((n, n)).astype(np.float32))
+        dB = am.toHip(np.random.default_rng(1002).standard_normal((n, n)).astype(np.float32))
+        dC = am.empty((n, n), np.float32)
+        fn = lambda: am.gemm(1, dA, dB, 0, dC)
+    elif which == "gemm_i32_1500":
+        n = 1500
+        dA = am.toHip(np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32))
+        dB = am.toHip(np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32))
+        dC = am.empty((n, n), np.int32)
+        fn = lambda: am.gemm(1, dA, dB, 0, dC)
+    elif which == "bcast_add_rotating":      # five buffer sets round robin: every byte of every launch comes from HBM
+        X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
+        b = am.toHip(np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32))
+        bb = b.broadcast((8192, 8192))
+        dXs = [am.toHip(X) for _ in range(ROTATE)]
+        dYs = [am.empty((8192, 8192), np.float32) for _ in range(ROTATE)]
+        rounds = max(steps // ROTATE, 4)
+        per = run_rotating(timer, [(lambda i=i: th._binary_into("add", dYs[i], dXs[i], bb)) for i in range(ROTATE)], rounds)
+        return dict(only=which, ms_per_launch=round(per * 1e3, 4), launches=(rounds + 1) * ROTATE)
     elif which == "gemm_f64":
         pa = np.random.default_rng(3001).standard_normal((1024, 2048))
         pb = np.random.default_rng(3002).standard_normal((1024, 6144))
@@ -573,7 +622,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true",
                     help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "sum_rows", "sum_cols", "softmax", "maxpool"],
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool",
+                                      "gemm_f32_1024", "gemm_f32_2048", "gemm_i32_1500", "bcast_add_rotating"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
