@@ -81,20 +81,24 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
         // of a row is ever touched. A vector wholly past the end repeats the row's first one. (The host sends
         // k ranges shorter than one vector to the element-wise loader.)
         const int64_t kv = k0 + q * VK;
-        const int64_t over = kv + VK - K;                       // elements past the end, if positive
-        const bool straddles = (K % VK != 0) && over > 0 && over < VK;   // first test uniform: nothing to do for whole vectors
-        const vec_t v = *(const gvec_t*)(ptr[i] + (kv >= K ? (int64_t)(-q * VK) : straddles ? k0 - over : k0));
-        vec_t r = v;
-        if (straddles) {
+        if (K % VK != 0) {   // uniform
+          const int64_t over = kv + VK - K;                       // elements past the end, if positive
+          const bool straddles = over > 0 && over < VK;
+          const vec_t v = *(const gvec_t*)(ptr[i] + (kv >= K ? (int64_t)(-q * VK) : straddles ? k0 - over : k0));
+          vec_t r = v;
+          if (straddles) {
 #pragma unroll
-          for (int e = 0; e < VK; ++e) {
-            T x = (T)0;
+            for (int e = 0; e < VK; ++e) {
+              T x = (T)0;
 #pragma unroll
-            for (int f = 0; f < VK; ++f) x = (e + over == f) ? v[f] : x;
-            r[e] = x;
+              for (int f = 0; f < VK; ++f) x = (e + over == f) ? v[f] : x;
+              r[e] = x;
+            }
           }
+          reg[S][i] = r;
+        } else {
+          reg[S][i] = *(const gvec_t*)(ptr[i] + (kv >= K ? (int64_t)(-q * VK) : k0));
         }
-        reg[S][i] = r;
       } else {
         reg[S][i] = *(const gvec_t*)(ptr[i] + k0);
       }

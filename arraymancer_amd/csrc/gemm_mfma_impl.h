@@ -86,6 +86,13 @@ __device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, 
 // trip (measured: f64 128 x 128 falls from 61 to 48 TFLOP/s).
 constexpr int mfma_min_blocks(int nt) { return nt <= 256 ? 2 : 1; }
 
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>());
+    static_for<I + 1, N>(f);
+  }
+}
+
 template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF, bool FPF, bool RU, int AK, int BKIND>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 : 1))
 void gemm_mfma(Args<T> p) {
@@ -168,30 +175,39 @@ void gemm_mfma(Args<T> p) {
     for (int j = 0; j < TN; ++j) read_frag<T, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[P][j]);
   };
 
-  // Prologue: slabs 0 and 1 into LDS, slabs 2 .. 2 + PF - 1 into the register stages.
-  la.template fetch<0>(k_begin);
-  lb.template fetch<0>(k_begin);
-  if constexpr (PF > 1) {
-    la.template fetch<1>(k_begin + BK);
-    lb.template fetch<1>(k_begin + BK);
-    la.template commit<0>(sA[0], k_begin);
-    lb.template commit<0>(sB[0], k_begin);
-    la.template commit<1>(sA[1], k_begin + BK);
-    lb.template commit<1>(sB[1], k_begin + BK);
-    la.template fetch<0>(k_begin + 2 * BK);
-    lb.template fetch<0>(k_begin + 2 * BK);
-    la.template fetch<1>(k_begin + 3 * BK);
-    lb.template fetch<1>(k_begin + 3 * BK);
-  } else {
-    la.template commit<0>(sA[0], k_begin);
-    lb.template commit<0>(sB[0], k_begin);
-    la.template fetch<0>(k_begin + BK);
-    lb.template fetch<0>(k_begin + BK);
-    la.template commit<0>(sA[1], k_begin + BK);
-    lb.template commit<0>(sB[1], k_begin + BK);
-    la.template fetch<0>(k_begin + 2 * BK);
-    lb.template fetch<0>(k_begin + 2 * BK);
-  }
+  // Prologue: slabs 0 and 1 into LDS, slabs 2 .. 2 + PF - 1 into the register stages (stage s holds slab 2 + s).
+  // When all of them lie wholly inside the k range (any but a very short one) the unmasked loads do: a few
+  // instructions each, where the masked ones compute clamped addresses per vector.
+  auto prologue = [&](auto mask_tag) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+    if constexpr (PF > 1) {
+      la.template fetch<0, MASK>(k_begin);
+      lb.template fetch<0, MASK>(k_begin);
+      la.template fetch<1, MASK>(k_begin + BK);
+      lb.template fetch<1, MASK>(k_begin + BK);
+      la.template commit<0, MASK>(sA[0], k_begin);
+      lb.template commit<0, MASK>(sB[0], k_begin);
+      la.template commit<1, MASK>(sA[1], k_begin + BK);
+      lb.template commit<1, MASK>(sB[1], k_begin + BK);
+      static_for<0, PF>([&](auto st) {
+        la.template fetch<decltype(st)::value, MASK>(k_begin + (2 + decltype(st)::value) * BK);
+        lb.template fetch<decltype(st)::value, MASK>(k_begin + (2 + decltype(st)::value) * BK);
+      });
+    } else {
+      la.template fetch<0, MASK>(k_begin);
+      lb.template fetch<0, MASK>(k_begin);
+      la.template commit<0, MASK>(sA[0], k_begin);
+      lb.template commit<0, MASK>(sB[0], k_begin);
+      la.template fetch<0, MASK>(k_begin + BK);
+      lb.template fetch<0, MASK>(k_begin + BK);
+      la.template commit<0, MASK>(sA[1], k_begin + BK);
+      lb.template commit<0, MASK>(sB[1], k_begin + BK);
+      la.template fetch<0, MASK>(k_begin + 2 * BK);
+      lb.template fetch<0, MASK>(k_begin + 2 * BK);
+    }
+  };
+  if (full_slabs >= 2 + PF) prologue(std::false_type());
+  else prologue(std::true_type());
   __syncthreads();
   if constexpr (FPF) read_frags(std::integral_constant<int, 0>(), sA[0], sB[0], 0);
 
@@ -276,33 +292,17 @@ void gemm_mfma(Args<T> p) {
   // Steady state: every slab this iteration fetches or commits lies wholly inside the k range,
   // so no clamping or zeroing is compiled in. The last few slabs run the masked version.
   int64_t kt = 0;
-  typedef std::integral_constant<int, 0> c0;
-  typedef std::integral_constant<int, 1> c1;
-  typedef std::integral_constant<int, 2> c2;
   typedef std::integral_constant<int, -1> dyn;
-  constexpr int UNR = PF == 1 ? 3 : 6;   // whole turns of the ring, a whole number of register stages
-  for (; RU && kt + (UNR - 1) + 2 + PF < full_slabs; kt += UNR) {   // starts and ends at ring position 0
-    if constexpr (PF == 1) {
-      slab(c0(), std::false_type(), c0(), kt);
-      slab(c0(), std::false_type(), c1(), kt + 1);
-      slab(c0(), std::false_type(), c2(), kt + 2);
-    } else {
-      slab(c0(), std::false_type(), c0(), kt);
-      slab(c1(), std::false_type(), c1(), kt + 1);
-      slab(c0(), std::false_type(), c2(), kt + 2);
-      slab(c1(), std::false_type(), c0(), kt + 3);
-      slab(c0(), std::false_type(), c1(), kt + 4);
-      slab(c1(), std::false_type(), c2(), kt + 5);
-    }
-  }
-  for (; kt + (PF - 1) + 2 + PF < full_slabs; kt += PF) {
-    slab(c0(), std::false_type(), dyn(), kt);
-    if constexpr (PF > 1) slab(c1(), std::false_type(), dyn(), kt + 1);
-  }
-  for (; kt < kt_run; kt += PF) {
-    slab(c0(), std::true_type(), dyn(), kt);
-    if constexpr (PF > 1) slab(c1(), std::true_type(), dyn(), kt + 1);
-  }
+  constexpr int UNR = PF % 3 == 0 ? PF : 3 * PF;   // whole turns of the ring, a whole number of register stages
+  for (; RU && kt + (UNR - 1) + 2 + PF < full_slabs; kt += UNR)   // starts and ends at ring position 0
+    static_for<0, UNR>([&](auto i) {
+      constexpr int I = decltype(i)::value;
+      slab(std::integral_constant<int, I % PF>(), std::false_type(), std::integral_constant<int, I % 3>(), kt + I);
+    });
+  for (; kt + (PF - 1) + 2 + PF < full_slabs; kt += PF)
+    static_for<0, PF>([&](auto i) { slab(i, std::false_type(), dyn(), kt + decltype(i)::value); });
+  for (; kt < kt_run; kt += PF)
+    static_for<0, PF>([&](auto i) { slab(i, std::true_type(), dyn(), kt + decltype(i)::value); });
 
   // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
   // C += alpha * AB, each rounded on its own; then the optional fused bias / ReLU.
@@ -324,49 +324,75 @@ void gemm_mfma(Args<T> p) {
   }
   const T alpha = p.alpha, beta = p.beta;
   const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
+  // Accumulator register r of tile (i, j) holds C(row0 + i * TILE + acc_row(r, 0), col0 + j * TILE): one 64-bit
+  // address product per lane, every other offset is a compile-time multiple of a stride (scalar arithmetic).
+  const int64_t row0 = m0 + wave_m * WM + MF::acc_row(0, lane), col0 = n0 + wave_n * WN + lrow;
+  T* const c0 = p.C + row0 * p.c_m + col0 * p.c_n;
+  const T* const b0 = has_bias ? p.bias + row0 * p.bias_m + col0 * p.bias_n : nullptr;
   // One accumulator tile at a time: first every load of C and of the bias for that tile is issued,
   // then the arithmetic and the stores follow. Interleaving load / store per element would make
   // each load wait for the store before it (one memory counter orders both), i.e. one round trip
   // to HBM per element. (A whole row of tiles at once needs more registers than the largest tile
-  // shapes have left next to their accumulators.)
+  // shapes have left next to their accumulators.) INTERIOR: the workgroup's tile lies wholly inside C,
+  // nothing is tested per element. PLAIN: C <- AB (alpha = 1, beta = 0, no fused epilogue), stores only.
+  auto write_out = [&](auto interior_tag, auto plain_tag) {
+    constexpr bool INTERIOR = decltype(interior_tag)::value;
+    constexpr bool PLAIN = decltype(plain_tag)::value;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int64_t col = n0 + wave_n * WN + j * TILE + lrow;
-      T cv[MF::NACC], bv[MF::NACC];
-      if (beta != (T)0) {
+      for (int j = 0; j < TN; ++j) {
+        const bool col_ok = INTERIOR || col0 + j * TILE < p.N;
+        T cv[MF::NACC], bv[MF::NACC];
+        if constexpr (PLAIN) {
 #pragma unroll
-        for (int r = 0; r < MF::NACC; ++r) {
-          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
-          cv[r] = (row < p.M && col < p.N) ? p.C[row * p.c_m + col * p.c_n] : (T)0;
-        }
-      }
-      if (has_bias) {
-#pragma unroll
-        for (int r = 0; r < MF::NACC; ++r) {
-          const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
-          bv[r] = (row < p.M && col < p.N) ? p.bias[row * p.bias_m + col * p.bias_n] : (T)0;
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < MF::NACC; ++r) {
-        const int64_t row = m0 + wave_m * WM + i * TILE + MF::acc_row(r, lane);
-        if (row < p.M && col < p.N) {
-          T ab = acc[i][j][r];
-          if (alpha != (T)1) ab = alpha * ab;
-          T v = ab;
-          if (beta != (T)0) {
-            T c = cv[r];
-            if (beta != (T)1) c = c * beta;
-            v = c + ab;
+          for (int r = 0; r < MF::NACC; ++r) {
+            const int dr = i * TILE + MF::acc_row(r, 0);
+            if (INTERIOR || (col_ok && row0 + dr < p.M)) c0[dr * p.c_m + j * TILE * p.c_n] = acc[i][j][r];
           }
-          if (has_bias) v = v + bv[r];
-          if (relu) v = ((T)0 >= v) ? (T)0 : v;
-          p.C[row * p.c_m + col * p.c_n] = v;
+          continue;
+        }
+        if (beta != (T)0) {
+#pragma unroll
+          for (int r = 0; r < MF::NACC; ++r) {
+            const int dr = i * TILE + MF::acc_row(r, 0);
+            cv[r] = (INTERIOR || (col_ok && row0 + dr < p.M)) ? c0[dr * p.c_m + j * TILE * p.c_n] : (T)0;
+          }
+        }
+        if (has_bias) {
+#pragma unroll
+          for (int r = 0; r < MF::NACC; ++r) {
+            const int dr = i * TILE + MF::acc_row(r, 0);
+            bv[r] = (INTERIOR || (col_ok && row0 + dr < p.M)) ? b0[dr * p.bias_m + j * TILE * p.bias_n] : (T)0;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < MF::NACC; ++r) {
+          const int dr = i * TILE + MF::acc_row(r, 0);
+          if (INTERIOR || (col_ok && row0 + dr < p.M)) {
+            T ab = acc[i][j][r];
+            if (alpha != (T)1) ab = alpha * ab;
+            T v = ab;
+            if (beta != (T)0) {
+              T c = cv[r];
+              if (beta != (T)1) c = c * beta;
+              v = c + ab;
+            }
+            if (has_bias) v = v + bv[r];
+            if (relu) v = ((T)0 >= v) ? (T)0 : v;
+            c0[dr * p.c_m + j * TILE * p.c_n] = v;
+          }
         }
       }
     }
+  };
+  const bool interior = m0 + BM <= p.M && n0 + BN <= p.N;
+  if (alpha == (T)1 && beta == (T)0 && p.epilogue == 0) {
+    if (interior) write_out(std::true_type(), std::true_type());
+    else write_out(std::false_type(), std::true_type());
+  } else {
+    if (interior) write_out(std::true_type(), std::false_type());
+    else write_out(std::false_type(), std::false_type());
   }
   probe.finish();
 }
