@@ -154,14 +154,11 @@ void gemm_mfma(Args<T> p) {
   //     a global load has PF whole slabs of MFMA work to arrive.
   // The LDS writes of iteration t are waited for at the barrier that ends it, having had a
   // k-step of MFMAs to drain.
-  // The loop body is straight-line code on purpose (no test for "is there a next slab"): fetches
-  // and commits past the end of the k range are clamped / zero-filled by the loader and land in
-  // registers or LDS buffers whose contents are multiplied by nothing or are zeros. Only then can
-  // the compiler count the loads in flight and wait for the oldest stage alone. With PF = 2 the
-  // slab count is rounded up to even; the extra slab multiplies zeros.
+  // The loop body is straight-line code on purpose (no test for "is there a next slab"): only then can
+  // the compiler count the loads in flight and wait for the oldest stage alone. The slabs near the end of
+  // the k range, whose fetches or commits would pass it, run other instances of the same body (see below).
   constexpr int NKS = BK / KSTEP;
   const int64_t ktiles = (k_end - k_begin + BK - 1) / BK;
-  const int64_t kt_run = (ktiles + PF - 1) / PF * PF;
   // Slabs that the unmasked (steady-state) loop may fetch: those wholly inside the k range, less the last
   // one when a loader must not run its unmasked fetch on the operand's last k row (see tail_guard).
   const int64_t full_slabs = (k_end - k_begin) / BK - ((la.tail_guard() || lb.tail_guard()) ? 1 : 0);
@@ -215,9 +212,15 @@ void gemm_mfma(Args<T> p) {
   // cur_tag >= 0: the ring position is known at compile time (the steady-state loop is unrolled over the
   // ring), so every LDS address of the slab is a constant offset and no address arithmetic stands
   // between the matrix instructions and the fragment reads; -1: taken from `cur` (the last few slabs).
-  auto slab = [&](auto stage_tag, auto mask_tag, auto cur_tag, int64_t kt) {
+  // What a slab's last k-step moves besides multiplying: kSteady commits slab kt + 2 and fetches slab kt + 2 + PF, both
+  // wholly inside the k range (nothing clamped or zeroed); kMasked does the same with clamping and zero fill; kCommit
+  // commits a whole slab and fetches nothing (slab kt + 2 + PF does not exist); kIdle moves nothing (slab kt + 2 does
+  // not exist either).
+  constexpr int kSteady = 0, kMasked = 1, kCommit = 2, kIdle = 3;
+  auto slab = [&](auto stage_tag, auto mode_tag, auto cur_tag, int64_t kt) {
     constexpr int S = decltype(stage_tag)::value;
-    constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr bool MASK = MODE == kMasked;
     constexpr int CT = decltype(cur_tag)::value;
     const int here = CT >= 0 ? CT : cur;
     const int nxt = (here == 2) ? 0 : here + 1;
@@ -233,10 +236,14 @@ void gemm_mfma(Args<T> p) {
         }
       } else {
         if constexpr (FPF) read_frags(std::integral_constant<int, 0>(), sA[nxt], sB[nxt], 0);   // NKS is even
-        la.template commit<S, MASK>(sA[nxt2], k_begin + (kt + 2) * BK);
-        lb.template commit<S, MASK>(sB[nxt2], k_begin + (kt + 2) * BK);
-        la.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
-        lb.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
+        if constexpr (MODE != kIdle) {
+          la.template commit<S, MASK>(sA[nxt2], k_begin + (kt + 2) * BK);
+          lb.template commit<S, MASK>(sB[nxt2], k_begin + (kt + 2) * BK);
+        }
+        if constexpr (MODE == kSteady || MODE == kMasked) {
+          la.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
+          lb.template fetch<S, MASK>(k_begin + (kt + 2 + PF) * BK);
+        }
       }
       // Left alone, the instruction scheduler sinks the reads and loads above down to their first use.
       // With fragment prefetch (the operands of this k-step are already in registers) they are spread
@@ -290,19 +297,32 @@ void gemm_mfma(Args<T> p) {
     cur = nxt;
   };
   // Steady state: every slab this iteration fetches or commits lies wholly inside the k range,
-  // so no clamping or zeroing is compiled in. The last few slabs run the masked version.
+  // so no clamping or zeroing is compiled in. The last 2 + PF slabs (more when the range ends in a partial slab)
+  // run the masked form or, slab by slab, the cheapest form that is correct for them.
   int64_t kt = 0;
   typedef std::integral_constant<int, -1> dyn;
+  typedef std::integral_constant<int, kSteady> steady;
   constexpr int UNR = PF % 3 == 0 ? PF : 3 * PF;   // whole turns of the ring, a whole number of register stages
   for (; RU && kt + (UNR - 1) + 2 + PF < full_slabs; kt += UNR)   // starts and ends at ring position 0
     static_for<0, UNR>([&](auto i) {
       constexpr int I = decltype(i)::value;
-      slab(std::integral_constant<int, I % PF>(), std::false_type(), std::integral_constant<int, I % 3>(), kt + I);
+      slab(std::integral_constant<int, I % PF>(), steady(), std::integral_constant<int, I % 3>(), kt + I);
     });
   for (; kt + (PF - 1) + 2 + PF < full_slabs; kt += PF)
-    static_for<0, PF>([&](auto i) { slab(i, std::false_type(), dyn(), kt + decltype(i)::value); });
-  for (; kt < kt_run; kt += PF)
-    static_for<0, PF>([&](auto i) { slab(i, std::true_type(), dyn(), kt + decltype(i)::value); });
+    static_for<0, PF>([&](auto i) { slab(i, steady(), dyn(), kt + decltype(i)::value); });
+  // The cheaper forms only where a wavefront owns one or two accumulator tiles: there the last slabs are a
+  // visible share of a short K loop. The large tiles, whose registers are all taken, run the masked form throughout
+  // (more instances of their loop body cost them spills, and their K loops are long).
+  constexpr bool CHEAP_TAIL = TM * TN <= 2;
+  const int64_t whole = (k_end - k_begin) / BK;   // slabs wholly inside the k range
+  for (; kt < ktiles; kt += PF)
+    static_for<0, PF>([&](auto i) {
+      const int64_t k = kt + decltype(i)::value;
+      if (k >= ktiles) return;                                  // uniform, like every test below
+      if (CHEAP_TAIL && k + 2 >= ktiles) slab(i, std::integral_constant<int, CHEAP_TAIL ? kIdle : kMasked>(), dyn(), k);
+      else if (CHEAP_TAIL && k + 2 < whole && k + 2 + PF >= ktiles) slab(i, std::integral_constant<int, CHEAP_TAIL ? kCommit : kMasked>(), dyn(), k);
+      else slab(i, std::integral_constant<int, kMasked>(), dyn(), k);
+    });
 
   // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
   // C += alpha * AB, each rounded on its own; then the optional fused bias / ReLU.
