@@ -141,9 +141,10 @@ struct TileChoice { int bm, bn; double eff; };
 
 // Picks the candidate with the least estimated time: rounds of one block per CU, each round
 // costing bm*bn/eff. Ragged edges and under-filled rounds are priced by construction.
-static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int64_t N, const char* env, int64_t batch = 1) {
+static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int64_t N, const char* env, int64_t batch = 1,
+                              double* cost_out = nullptr) {
   const char* forced = getenv(env);
-  if (forced && *forced) {
+  if (forced && *forced && !cost_out) {
     int idx = atoi(forced);
     if (idx >= 0 && idx < ncand) return idx;
   }
@@ -157,7 +158,48 @@ static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int6
     const double cost = (double)rounds * cand[i].bm * cand[i].bn / cand[i].eff;
     if (i == 0 || cost < best_cost) { best = i; best_cost = cost; }
   }
+  if (cost_out) *cost_out = best_cost;
   return best;
+}
+
+// The sub-problem C[r0:r1, c0:c1] of g (rows of A, columns of B, the block of C and of the bias).
+template <typename T>
+static inline Args<T> sub_problem(const Args<T>& g, int64_t r0, int64_t r1, int64_t c0, int64_t c1) {
+  Args<T> s = g;
+  s.M = r1 - r0; s.N = c1 - c0;
+  s.A = g.A + r0 * g.a_mn;
+  s.B = g.B + c0 * g.b_mn;
+  s.C = g.C + r0 * g.c_m + c0 * g.c_n;
+  if (g.bias) s.bias = g.bias + r0 * g.bias_m + c0 * g.bias_n;
+  return s;
+}
+
+// A matrix whose extent is a few rows or columns more than a multiple of the tile edge costs a whole extra
+// round of tiles for those few (4097^2 outputs: 289 tiles of 256 x 256 on 256 CUs, two rounds for what is
+// 1.0005 rounds of work). Such a product is cut into the aligned block, run by the tiled kernel, and strips of
+// at most 16 rows / columns, run as the skinny products they are (they stream the other operand once).
+// Returns the number of rows (*rm) and columns (*rn) to cut off, both 0 when the product is better left whole:
+// the estimate compares rounds x tile area (choose_tile's cost) with and without the cut, and prices a strip
+// by the bytes it streams.
+template <typename T>
+static inline void plan_peel(const Args<T>& g, const TileChoice* cand, int ncand, const char* env, double flops_per_cu_us,
+                             int64_t* rm, int64_t* rn) {
+  *rm = *rn = 0;
+  if (g.batch > 1 || g.static_ws) return;   // (the allocation-free entry point refuses a product as a whole or not at all)
+  const char* e = getenv("AM_HIP_GEMM_PEEL");   // "0": never cut; "1": cut whenever the shape allows it (tests)
+  if (e && *e == '0') return;
+  const int64_t pm = g.M % 64, pn = g.N % 64;
+  const bool cm = pm > 0 && pm <= 16 && g.M >= 512, cn = pn > 0 && pn <= 16 && g.N >= 512;
+  if (!cm && !cn) return;
+  double whole = 0, cut = 0;
+  (void)choose_tile(cand, ncand, g.M, g.N, env, 1, &whole);
+  const int64_t M0 = cm ? g.M - pm : g.M, N0 = cn ? g.N - pn : g.N;
+  (void)choose_tile(cand, ncand, M0, N0, env, 1, &cut);
+  const double us_per_cost = 2.0 * (double)g.K / flops_per_cu_us;          // time of one output element's K loop on one CU
+  // a strip: one launch, and the other operand streamed once at ~3 TB/s
+  const double strips = (cm ? 6.0 + (double)g.K * (double)g.N * sizeof(T) / 3.0e6 : 0.0) +
+                        (cn ? 6.0 + (double)g.K * (double)M0 * sizeof(T) / 3.0e6 : 0.0);
+  if ((e && *e == '1') || cut * us_per_cost + strips < 0.92 * whole * us_per_cost) { *rm = cm ? pm : 0; *rn = cn ? pn : 0; }
 }
 
 // Persistent device workspace for split-K partial sums (runtime.hip): allocated once, on first use

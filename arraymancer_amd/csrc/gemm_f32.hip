@@ -5,14 +5,33 @@
 using namespace am;
 using namespace am::gemm;
 
+static int run_whole_f32(Args<float>& g);
+static const TileChoice* candidates_f32(int* n);
+
+// The product as the caller stated it: whole, or as an aligned block plus strips (plan_peel).
 static int run_f32(Args<float>& g) {
+  int nc = 0;
+  const TileChoice* cand = candidates_f32(&nc);
+  int64_t rm = 0, rn = 0;
+  if (!small::applicable(g)) plan_peel(g, cand, nc, "AM_HIP_GEMM_TILE_F32", 157.3e6 / 256, &rm, &rn);
+  if (rm == 0 && rn == 0) return run_whole_f32(g);
+  const int64_t M0 = g.M - rm, N0 = g.N - rn;
+  Args<float> part = sub_problem(g, 0, M0, 0, N0);
+  AM_TRY(run_whole_f32(part));
+  if (rm) { part = sub_problem(g, M0, g.M, 0, g.N); AM_TRY(run_whole_f32(part)); }   // bottom strip, full width
+  if (rn) { part = sub_problem(g, 0, M0, N0, g.N); AM_TRY(run_whole_f32(part)); }   // right strip above it
+  return AM_OK;
+}
+
+static int run_whole_f32(Args<float>& g) {
   if (small::applicable(g)) return small::run(g);   // few rows or columns: no LDS staging, no second kernel
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
   // Candidate workgroup tiles with the relative MFMA efficiency of each (measured on 2048^3 and
   // 4096^3). PF = 2 (two slabs of global loads in flight) on the tiles whose slab is short.
-  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.94}, {64, 64, 0.88}, {256, 128, 0.97}, {128, 64, 0.92}, {32, 32, 0.74}};
-  switch (choose_tile(cand, 6, g.M, g.N, "AM_HIP_GEMM_TILE_F32", g.batch)) {
+  int nc = 0;
+  const TileChoice* cand = candidates_f32(&nc);
+  switch (choose_tile(cand, nc, g.M, g.N, "AM_HIP_GEMM_TILE_F32", g.batch)) {
     case 0: return launch_kinds<float, 256, 256, 16, 2, 4, 1, true, false>(g, ak, bk);   // its loop is long enough: unrolling it over the ring costs 4 %
     case 1: return launch_kinds<float, 128, 128, 16, 2, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2, 2>(g, ak, bk);
@@ -20,6 +39,12 @@ static int run_f32(Args<float>& g) {
     case 4: return launch_kinds<float, 128, 64, 16, 2, 2, 2>(g, ak, bk);
     default: return launch_kinds<float, 32, 32, 16, 1, 1, 2>(g, ak, bk);
   }
+}
+
+static const TileChoice* candidates_f32(int* n) {
+  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.94}, {64, 64, 0.88}, {256, 128, 0.97}, {128, 64, 0.92}, {32, 32, 0.74}};
+  *n = (int)(sizeof(cand) / sizeof(cand[0]));
+  return cand;
 }
 
 extern "C" int am_hip_gemm_ex_f32(int64_t M, int64_t N, int64_t K, float alpha, const float* A, int64_t rsA,

@@ -5,7 +5,25 @@
 using namespace am;
 using namespace am::gemm;
 
+static int run_whole_f64(Args<double>& g);
+static const TileChoice* candidates_f64(int* n);
+
+// The product as the caller stated it: whole, or as an aligned block plus strips (plan_peel).
 static int run_f64(Args<double>& g) {
+  int nc = 0;
+  const TileChoice* cand = candidates_f64(&nc);
+  int64_t rm = 0, rn = 0;
+  if (!small::applicable(g)) plan_peel(g, cand, nc, "AM_HIP_GEMM_TILE_F64", 78.6e6 / 256, &rm, &rn);
+  if (rm == 0 && rn == 0) return run_whole_f64(g);
+  const int64_t M0 = g.M - rm, N0 = g.N - rn;
+  Args<double> part = sub_problem(g, 0, M0, 0, N0);
+  AM_TRY(run_whole_f64(part));
+  if (rm) { part = sub_problem(g, M0, g.M, 0, g.N); AM_TRY(run_whole_f64(part)); }   // bottom strip, full width
+  if (rn) { part = sub_problem(g, 0, M0, N0, g.N); AM_TRY(run_whole_f64(part)); }   // right strip above it
+  return AM_OK;
+}
+
+static int run_whole_f64(Args<double>& g) {
   if (small::applicable(g)) return small::run(g);   // few rows or columns: no LDS staging, no second kernel
   int ak = classify(g.A, g.a_mn, g.a_k, g.M, g.K);
   int bk = classify(g.B, g.b_mn, g.b_k, g.N, g.K);
@@ -15,8 +33,9 @@ static int run_f64(Args<double>& g) {
   // 128 x 192 (8 wavefronts of 64 x 48) exists for shapes that the others cut into a number of
   // tiles just above a multiple of the CU count: 2048 x 3072 is 384 tiles of 128 x 128 (two rounds,
   // the second half empty) but exactly 256 of 128 x 192.
-  static const TileChoice cand[] = {{128, 128, 0.97}, {64, 64, 0.93}, {32, 32, 0.76}, {256, 128, 1.0}, {128, 64, 0.96}, {128, 192, 0.98}};
-  switch (choose_tile(cand, 6, g.M, g.N, "AM_HIP_GEMM_TILE_F64", g.batch)) {
+  int nc = 0;
+  const TileChoice* cand = candidates_f64(&nc);
+  switch (choose_tile(cand, nc, g.M, g.N, "AM_HIP_GEMM_TILE_F64", g.batch)) {
     case 0: return launch_kinds<double, 128, 128, 16, 2, 4>(g, ak, bk);
     case 1: return launch_kinds<double, 64, 64, 16, 2, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<double, 32, 32, 16, 2, 2, 2>(g, ak, bk);
@@ -24,6 +43,12 @@ static int run_f64(Args<double>& g) {
     case 4: return launch_kinds<double, 128, 64, 16, 2, 2, 2>(g, ak, bk);
     default: return launch_kinds<double, 128, 192, 16, 2, 4, 1, false>(g, ak, bk);
   }
+}
+
+static const TileChoice* candidates_f64(int* n) {
+  static const TileChoice cand[] = {{128, 128, 0.97}, {64, 64, 0.93}, {32, 32, 0.76}, {256, 128, 1.0}, {128, 64, 0.96}, {128, 192, 0.98}};
+  *n = (int)(sizeof(cand) / sizeof(cand[0]));
+  return cand;
 }
 
 extern "C" int am_hip_gemm_ex_f64(int64_t M, int64_t N, int64_t K, double alpha, const double* A, int64_t rsA,

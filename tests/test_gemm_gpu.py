@@ -155,6 +155,38 @@ def test_unit_stride_operands_of_any_pitch_and_alignment(hip, oracle, sfx, layou
             assert_parity(oracle, sfx, dC.toCpu(), want, f"{layout} {(M, N, K)}")
 
 
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_extents_just_above_a_tile_multiple(hip, oracle, sfx, monkeypatch):
+    """A float product with a few rows / columns more than a multiple of the tile edge runs as the aligned block
+    plus strips of those rows and columns (three or two launches): every block of C, the bias and the views must
+    be cut at the same place. Compared with the oracle and with the same product run whole (the cut is forced: the
+    library's own estimate only cuts where a round of tiles is saved)."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("peel", sfx))
+    for (M, N, K), trans in [((1030, 520, 300), ""), ((512 + 16, 2048 + 1, 96), "AB"), ((1024, 1024 + 3, 130), "B"), ((1024 + 2, 640, 77), "A")]:
+        A = fill(rng, (K, M) if "A" in trans else (M, K), dt)
+        B = fill(rng, (N, K) if "B" in trans else (K, N), dt)
+        C, bias = fill(rng, (M, N), dt), fill(rng, (1, N), dt)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        vA, vB = (dA.transpose(), A.T) if "A" in trans else (dA, A), (dB.transpose(), B.T) if "B" in trans else (dB, B)
+        results = {}
+        for peel in ("1", "0"):
+            monkeypatch.setenv("AM_HIP_GEMM_PEEL", peel)
+            say("peel", sfx, (M, N, K), trans, "cut" if peel == "1" else "whole")
+            dC = hip.toHip(C)
+            hip.gemm(1.5, vA[0], vB[0], 0.5, dC, epilogue="bias_relu", bias=hip.toHip(bias))
+            results[peel] = dC.toCpu()
+            dP = hip.empty((M, N), dt)
+            hip.gemm(1, vA[0], vB[0], 0, dP)
+            results[peel + "plain"] = dP.toCpu()
+        want = oracle.gemm_strided(1.5, vA[1], vB[1], 0.5, C.copy())
+        want = oracle.map2("add_relu", want, oracle.broadcast(bias, want.shape))
+        assert_parity(oracle, sfx, results["1"], want, f"cut {(M, N, K)} {trans}")
+        assert_parity(oracle, sfx, results["1plain"], oracle.matmul(vA[1], vB[1]), f"cut, plain {(M, N, K)} {trans}")
+        assert oracle.rel_frobenius(results["1"], results["0"]) <= TOL[sfx]
+        assert oracle.rel_frobenius(results["1plain"], results["0plain"]) <= TOL[sfx]
+
+
 # ------------------------------------------------------------------ strided / transposed views
 def device_view(hip, parent_np, kind, shape):
     """The same geometry as conftest.strided_view, built with view ops on the device tensor."""
