@@ -69,6 +69,31 @@ __global__ __launch_bounds__(256) void peak_mfma_i8(int iters, int* out) {
   if (s == 0x12345678) out[0] = s;
 }
 
+// LDS read rate: every wavefront reads 16 bytes per lane (ds_read_b128, consecutive lanes at consecutive
+// addresses: no bank conflicts), eight independent reads in flight per trip, each wavefront from its own 8 KiB.
+// Written as inline assembly so that the loop is the eight reads, one wait and the loop counter.
+__global__ __launch_bounds__(256) void peak_lds_read(int iters, int* out) {
+  __shared__ __attribute__((aligned(16))) int buf[8192];
+  for (int i = threadIdx.x; i < 8192; i += 256) buf[i] = i * 0x9e3779b9;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t addr = (uint32_t)reinterpret_cast<uintptr_t>(buf) + (uint32_t)(wave * 8192 + lane * 16);
+  v4i v0, v1, v2, v3, v4, v5, v6, v7;
+  int s = 0;
+  for (int i = 0; i < iters; ++i) {
+    asm volatile(
+        "ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:1024\n\tds_read_b128 %2, %8 offset:2048\n\t"
+        "ds_read_b128 %3, %8 offset:3072\n\tds_read_b128 %4, %8 offset:4096\n\tds_read_b128 %5, %8 offset:5120\n\t"
+        "ds_read_b128 %6, %8 offset:6144\n\tds_read_b128 %7, %8 offset:7168\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
+        : "v"(addr)
+        : "memory");
+    s ^= v0[0] ^ v7[3];
+  }
+  s ^= v1[1] ^ v2[2] ^ v3[3] ^ v4[0] ^ v5[1] ^ v6[2];
+  if (s == 0x12345678) out[0] = s;
+}
+
 // 8 x 8 register tile of wrapping 32-bit multiply-accumulates per step: the inner body of the
 // integer GEMM kernel without its LDS reads.
 template <typename U>
@@ -255,7 +280,7 @@ extern "C" int am_hip_diag_clock_end(double* shader_mhz) {
 
 // kind: 0 = MFMA f32 32x32x2 (FLOP/s), 1 = MFMA f64 16x16x4 (FLOP/s),
 //       2 = VALU int32 multiply-add (integer op/s, 2 per MAC), 3 = VALU int64 multiply-add,
-//       4 = MFMA i32 32x32x32 int8 (integer op/s).
+//       4 = MFMA i32 32x32x32 int8 (integer op/s), 5 = LDS reads of 16 bytes per lane (bytes/s).
 // Launches `waves_per_simd` wavefronts on every SIMD of the device, `iters` loop trips each.
 extern "C" int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second) {
   if (!ops_per_second || iters <= 0 || waves_per_simd < 1 || waves_per_simd > 8)
@@ -290,6 +315,10 @@ extern "C" int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double*
       case 4:
         hipLaunchKernelGGL(peak_mfma_i8, dim3(blocks), dim3(256), 0, stream(), iters, (int*)scratch);
         ops_per_launch = (double)blocks * 4 * iters * 4 * (32.0 * 32 * 32 * 2);
+        break;
+      case 5:
+        hipLaunchKernelGGL(peak_lds_read, dim3(blocks), dim3(256), 0, stream(), iters, (int*)scratch);
+        ops_per_launch = (double)blocks * 256 * iters * 8 * 16.0;   // bytes
         break;
       default:
         (void)hipFree(scratch);

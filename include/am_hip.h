@@ -558,6 +558,7 @@ int am_hip_maxpool2d_backward_i64(int64_t N, int C, int H, int W, int kH, int kW
  *   kind 2: VALU int32 wrapping multiply-add, 8x8 register tile (integer op/s, 2 per MAC)
  *   kind 3: VALU int64 multiply-add
  *   kind 4: MFMA int8 32x32x32 (integer op/s), the instruction of the digit-sliced integer GEMM
+ *   kind 5: LDS reads of 16 bytes per lane, no bank conflicts (bytes/s over the whole device)
  * waves_per_simd wavefronts are resident on every SIMD (1..8); iters loop trips each. */
 int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second);
 /* What HBM delivers to a kernel that only streams: kind 0 reads, 1 writes, 2 copies `bytes` (a multiple of
