@@ -37,7 +37,9 @@ static int run_whole_f32(Args<float>& g) {
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2, 2>(g, ak, bk);
     case 3: return launch_kinds<float, 256, 128, 16, 4, 2>(g, ak, bk);
     case 4: return launch_kinds<float, 128, 64, 16, 2, 2, 2>(g, ak, bk);
-    default: return launch_kinds<float, 32, 32, 16, 1, 1, 2>(g, ak, bk);
+    // four wavefronts of 16 x 16 each (one per SIMD) where one of 32 x 32 would run alone on its CU: 64 batched
+    // [50 x 500] . [500 x 64] products 13.3 -> 7.2 us
+    default: return launch_kinds<float, 32, 32, 32, 2, 2, 2, true, true, MfmaF32x16>(g, ak, bk);
   }
 }
 

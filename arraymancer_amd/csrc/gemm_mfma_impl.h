@@ -49,6 +49,23 @@ template <> struct Mfma<float> {
   static __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 };
 
+// float32 with the 16 x 16 x 4 instruction (8 passes, the same rate per cycle as 32 x 32 x 2): a quarter of the
+// accumulator registers per tile, so a small workgroup tile can be spread over four wavefronts, one per SIMD,
+// where the large instruction would leave it to a single one.
+struct MfmaF32x16 {
+  static constexpr int TILE = 16;
+  static constexpr int KL = 4;
+  static constexpr int VK = 4;
+  static constexpr int NACC = 4;
+  typedef float acc_t __attribute__((ext_vector_type(4)));
+  typedef float vec_t __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  // Register r of lane group g = lane / 16 holds row 4 * g + r (column = lane % 16).
+  static __device__ __forceinline__ int acc_row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+
 template <> struct Mfma<double> {
   static constexpr int TILE = 16;
   static constexpr int KL = 4;
@@ -64,10 +81,10 @@ template <> struct Mfma<double> {
 };
 
 // Reads the VK k values that `lane` feeds to the MFMA steps of k-step `ks` for row/col `mn`.
-template <typename T, int KIND, int BMN, int BK>
-__device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, T (&out)[Mfma<T>::VK]) {
-  typedef typename Mfma<T>::vec_t vec_t;
-  constexpr int VK = Mfma<T>::VK, KL = Mfma<T>::KL;
+template <typename T, typename MF, int KIND, int BMN, int BK>
+__device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, T (&out)[MF::VK]) {
+  typedef typename MF::vec_t vec_t;
+  constexpr int VK = MF::VK, KL = MF::KL;
   if constexpr (KIND == kKContig) {
     constexpr int LD = Slab<T, KIND, BMN, BK>::LDKG;
     const vec_t v = *(const vec_t*)(lds + ((ks * KL + kl) * LD + mn) * VK);
@@ -93,10 +110,9 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
   }
 }
 
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF, bool FPF, bool RU, int AK, int BKIND>
+template <typename T, typename MF, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF, bool FPF, bool RU, int AK, int BKIND>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 : 1))
 void gemm_mfma(Args<T> p) {
-  typedef Mfma<T> MF;
   typedef typename MF::acc_t acc_t;
   const ClockProbe probe(p.clock_out);
   constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -167,9 +183,9 @@ void gemm_mfma(Args<T> p) {
   auto read_frags = [&](auto parity_tag, const T* a_lds, const T* b_lds, int ks) {
     constexpr int P = decltype(parity_tag)::value;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) read_frag<T, AK, BM, BK>(a_lds, wave_m * WM + i * TILE + lrow, ks, kl, af[P][i]);
+    for (int i = 0; i < TM; ++i) read_frag<T, MF, AK, BM, BK>(a_lds, wave_m * WM + i * TILE + lrow, ks, kl, af[P][i]);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) read_frag<T, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[P][j]);
+    for (int j = 0; j < TN; ++j) read_frag<T, MF, BKIND, BN, BK>(b_lds, wave_n * WN + j * TILE + lrow, ks, kl, bf[P][j]);
   };
 
   // Prologue: slabs 0 and 1 into LDS, slabs 2 .. 2 + PF - 1 into the register stages (stage s holds slab 2 + s).
@@ -418,7 +434,8 @@ void gemm_mfma(Args<T> p) {
 }
 
 // PF: register stages of global loads; FPF: fragment prefetch; RU: steady-state loop unrolled over the LDS ring.
-template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true, bool RU = true>
+// MF: the matrix instruction (Mfma<T>, or MfmaF32x16 for small float tiles).
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true, bool RU = true, typename MF = Mfma<T>>
 static int launch_kinds(Args<T>& g, int ak, int bk) {
   g.tiles_m = (int)((g.M + BM - 1) / BM);
   g.tiles_n = (int)((g.N + BN - 1) / BN);
@@ -434,7 +451,7 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
   }
   const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(WAVES_M * WAVES_N * 64);
 #define AM_LAUNCH(AKIND, BKIND_)                                                                   \
-  hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, AKIND, BKIND_>), grid, block, 0, \
+  hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, AKIND, BKIND_>), grid, block, 0, \
                      stream(), g)
   switch (ak * 3 + bk) {
     case 0: AM_LAUNCH(kKContig, kKContig); break;
