@@ -422,7 +422,7 @@ def config_report(am, timer, L):
                    gpu_rate=round(ops / gpu_s / 1e12, 3), rate_unit=unit,
                    pct_peak=round(100 * ops / gpu_s / 1e12 / peak, 1) if peak else None, peak_used=peak_used,
                    cpu_impl="oracle/laser_gemm.c (port of laser gemm_strided, OpenMP)", cpu_threads=threads,
-                   cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1))
+                   cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1), sclk_mhz=timer.sclk_mhz)
         if dt.kind == "f":
             row["rel_frobenius_vs_cpu"] = am_oracle.rel_frobenius(got, want)
             # the reference's float `*` goes through CBLAS: NumPy's bundled BLAS as the stand-in for it
@@ -435,12 +435,12 @@ def config_report(am, timer, L):
         emit(**row)
 
     rng = np.random.default_rng
-    for n in (1024, 4096):
+    for n in (1024, 2048, 4096):
         A = rng(1001).uniform(-1, 1, (n, n)).astype(np.float32); B = rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
         gemm_case(f"f32 GEMM {n}^3", "f32", n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_F32_PEAK_TFLOPS,
-                  peak_used="MFMA fp32 157.3 TFLOP/s", steps=50 if n == 1024 else 20)
+                  peak_used="MFMA fp32 157.3 TFLOP/s", steps=50 if n <= 2048 else 20)
     # extents that are not a multiple of the 16-byte vector, beside their aligned neighbour (4096): unit-stride
-    # operands are moved in 16-byte pieces whatever their pitch; 4097 pays for a second, nearly empty round of tiles
+    # operands are moved in 16-byte pieces whatever their pitch; 4097 runs as the 4096^3 block plus two skinny strips
     for n in (4095, 4097):
         A = rng(1001).uniform(-1, 1, (n, n)).astype(np.float32); B = rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
         gemm_case(f"f32 GEMM {n}^3 (ragged extents)", "f32", n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_F32_PEAK_TFLOPS,
@@ -544,6 +544,9 @@ def config_report(am, timer, L):
     del dPs
     r = bench_chain(am, timer, 200, 20)
     emit(config="f32 inference chain (4 GEMMs, fused bias+ReLU)", dtype="f32", hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"],
+         note=r["note"])
+    r = bench_ex02(am, timer, 200, 20)
+    emit(config="f32 example-2 forward pass, batch 64 (8 kernels)", dtype="f32", hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"],
          note=r["note"])
 
 
