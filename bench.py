@@ -380,8 +380,8 @@ def bench_ex02(am, timer, steps, warmup, batch=64):
                 value_is="eager" if ev_e <= ev_g else "hipgraph", eager_us=round(ev_e / steps * 1e6, 2),
                 eager_wall_us=round(wall_e / steps * 1e6, 2), hipgraph_us=round(ev_g / steps * 1e6, 2),
                 images_per_s=round(batch / (best / steps), 0), gflops=round(flops / (best / steps) / 1e9, 1),
-                note="3.0e8 FLOP per pass over eight kernels of 4-17 us whose durations sum to about 61 us: the graph replay runs "
-                     "them back to back, the eager pass leaves about 1 us of host launch gap after each")
+                note="3.0e8 FLOP per pass over eight kernels of 3-10 us each: the graph replay runs them back to back (its time is "
+                     "the sum of their durations), the eager pass adds the host's launch gap after each")
 
 
 def config_report(am, timer, L):
