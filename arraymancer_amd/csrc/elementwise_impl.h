@@ -466,11 +466,9 @@ template <typename T> struct TriArgs {
   T* dst; const T* a; const T* b; const T* c;
   int64_t n;          // generic kernel: total elements
   int64_t L;          // rows kernel: inner extent
-  uint32_t tiles_per_row, total_tiles;
+  uint32_t tiles_per_row, rows, col_blocks;   // rows kernel: see RowsArgs
   int rank;           // collapsed rank (generic) / number of outer dims (rows)
-  int a_const, b_const, c_const;   // rows kernel: operand has inner stride 0 (one value per row)
-  int a_keep, b_keep, c_keep;      // rows kernel: ordinary loads (a row re-read for every output row, or operands small
-                                   // enough for the memory-side cache); 0 = non-temporal loads
+  int a_mode, b_mode, c_mode;      // rows kernel: how each operand is read (kTriVec ... kTriImm)
   int bc_imm;                      // operands b and c are the values b_imm and c_imm (clamp bounds passed by value)
   T b_imm, c_imm;
   int64_t shape[AM_MAXRANK];
@@ -479,50 +477,101 @@ template <typename T> struct TriArgs {
 
 // Every operand has unit innermost stride and 16-byte aligned rows (the GRU column slices, plain
 // contiguous tensors, row vectors broadcast over the rows) or innermost stride 0 (a column vector
-// broadcast along the rows: one scalar per row): same streaming structure as ew_rows.
+// broadcast along the rows: one scalar per row): same streaming structure as ew_rows. A workgroup keeps
+// its column tile while it walks down the rows; an operand that is one row for every output row is
+// loaded once per column tile and kept in registers; the loads of a row are unconditional (from
+// addresses clamped into the row) and sit in one workgroup-uniform branch per operand and kind of load.
+// How each operand is read: kTriVec (16-byte loads), kTriVecNt (non-temporal ones), kTriRowVector (one row
+// for all output rows), kTriRowScalar (one value per row), kTriImm (a value in the kernel arguments).
+enum { kTriVec = 0, kTriVecNt = 1, kTriRowVector = 2, kTriRowScalar = 3, kTriImm = 4 };
+
 template <typename T, int OP>
 __global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
   typedef typename Traits<T>::V V;
   constexpr int VEC = Traits<T>::kVec;
   constexpr int64_t TILE = (int64_t)kThreads * VEC * kUnroll;
-  for (uint32_t tile = blockIdx.x; tile < p.total_tiles; tile += gridDim.x) {
-    const uint32_t row = tile / p.tiles_per_row;
-    const uint32_t ct = tile - row * p.tiles_per_row;
-    int64_t od = 0, oa = 0, ob = 0, oc = 0;
-    uint32_t rem = row;
-    for (int d = p.rank - 1; d >= 0; --d) {
-      const uint32_t ext = (uint32_t)p.shape[d];
-      const uint32_t q = rem / ext;
-      const int64_t cidx = (int64_t)(rem - q * ext);
-      rem = q;
-      od += cidx * p.sd[d]; oa += cidx * p.sa[d]; ob += cidx * p.sb[d]; oc += cidx * p.sc[d];
-    }
-    T* __restrict__ drow = p.dst + od;
-    const T* __restrict__ arow = p.a + oa;
-    const T* __restrict__ brow = p.b + ob;
-    const T* __restrict__ crow = p.c + oc;
+  const uint32_t cb = blockIdx.x % p.col_blocks, g0 = blockIdx.x / p.col_blocks, gstep = gridDim.x / p.col_blocks;
+  const int am = p.a_mode, bm = p.b_mode, cm = p.c_mode;
+  auto column_tile = [&](auto whole_tag, uint32_t ct) {
+    constexpr bool WHOLE = decltype(whole_tag)::value;
     const int64_t col0 = (int64_t)ct * TILE + (int64_t)threadIdx.x * VEC;
+    bool full[kUnroll];
+    int64_t lcol[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t col = col0 + (int64_t)u * kThreads * VEC;
-      if (col + VEC <= p.L) {
-        V av, bv, cv;
-        if (p.a_const) { for (int e = 0; e < VEC; ++e) av[e] = arow[0]; } else av = load_as(p.a_keep != 0, (const V*)(arow + col));
-        if (p.bc_imm) { for (int e = 0; e < VEC; ++e) { bv[e] = p.b_imm; cv[e] = p.c_imm; } }
-        else {
-          if (p.b_const) { for (int e = 0; e < VEC; ++e) bv[e] = brow[0]; } else bv = load_as(p.b_keep != 0, (const V*)(brow + col));
-          if (p.c_const) { for (int e = 0; e < VEC; ++e) cv[e] = crow[0]; } else cv = load_as(p.c_keep != 0, (const V*)(crow + col));
+      full[u] = WHOLE || (col + VEC <= p.L);
+      lcol[u] = full[u] ? col : 0;   // (the host sends rows shorter than one vector elsewhere)
+    }
+    V av[kUnroll], bv[kUnroll], cv[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) { av[u] = V{}; bv[u] = V{}; cv[u] = V{}; }
+    if (am == kTriRowVector) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) av[u] = *(const V*)(p.a + lcol[u]);
+    }
+    if (bm == kTriRowVector) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) bv[u] = *(const V*)(p.b + lcol[u]);
+    }
+    if (cm == kTriRowVector) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) cv[u] = *(const V*)(p.c + lcol[u]);
+    }
+    for (uint32_t row = g0; row < p.rows; row += gstep) {
+      int64_t od = 0, oa = 0, ob = 0, oc = 0;
+      uint32_t rem = row;
+      // constant indices into the argument arrays (a loop with a run-time bound would move them to scratch memory)
+#pragma unroll
+      for (int d = AM_MAXRANK - 2; d >= 0; --d) {
+        if (d < p.rank) {
+          const uint32_t ext = (uint32_t)p.shape[d];
+          const uint32_t q = rem / ext;
+          const int64_t cidx = (int64_t)(rem - q * ext);
+          rem = q;
+          od += cidx * p.sd[d]; oa += cidx * p.sa[d]; ob += cidx * p.sb[d]; oc += cidx * p.sc[d];
         }
+      }
+      T* __restrict__ drow = p.dst + od;
+      const T* __restrict__ arow = p.a + oa;
+      const T* __restrict__ brow = p.b + ob;
+      const T* __restrict__ crow = p.c + oc;
+      const T asc = am == kTriRowScalar ? arow[0] : (T)0;
+      const T bsc = bm == kTriRowScalar ? brow[0] : p.b_imm;
+      const T csc = cm == kTriRowScalar ? crow[0] : p.c_imm;
+#define AM_TRI_LOADS(mode, vec, rowptr)                                                                                  \
+      if (mode == kTriVecNt) {                                                                                            \
+        _Pragma("unroll") for (int u = 0; u < kUnroll; ++u) vec[u] = __builtin_nontemporal_load(launder((const V*)(rowptr + lcol[u]))); \
+      } else if (mode == kTriVec) {                                                                                       \
+        _Pragma("unroll") for (int u = 0; u < kUnroll; ++u) vec[u] = *(const V*)(rowptr + lcol[u]);                       \
+      }
+      AM_TRI_LOADS(am, av, arow)
+      AM_TRI_LOADS(bm, bv, brow)
+      AM_TRI_LOADS(cm, cv, crow)
+#undef AM_TRI_LOADS
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
         V r;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) r[e] = TriOp<T, OP>::apply(av[e], bv[e], cv[e]);
-        __builtin_nontemporal_store(r, (V*)(drow + col));
-      } else {
-        for (int64_t cc = col; cc < p.L; ++cc)
-          drow[cc] = TriOp<T, OP>::apply(arow[p.a_const ? 0 : cc], p.bc_imm ? p.b_imm : brow[p.b_const ? 0 : cc],
-                                         p.bc_imm ? p.c_imm : crow[p.c_const ? 0 : cc]);
+        for (int e = 0; e < VEC; ++e)
+          r[e] = TriOp<T, OP>::apply(am >= kTriRowScalar ? asc : av[u][e], bm >= kTriRowScalar ? bsc : bv[u][e],
+                                     cm >= kTriRowScalar ? csc : cv[u][e]);
+        if (full[u]) __builtin_nontemporal_store(r, (V*)(drow + lcol[u]));
+      }
+      if constexpr (!WHOLE) {   // the row's last L mod VEC elements, one lane
+        const int64_t tail = p.L - p.L % VEC;
+        if (threadIdx.x == 0 && tail < p.L && tail >= (int64_t)ct * TILE) {
+          for (int64_t cc = tail; cc < p.L; ++cc)
+            drow[cc] = TriOp<T, OP>::apply(am >= kTriRowScalar ? asc : (am == kTriRowVector ? p.a[cc] : arow[cc]),
+                                           bm >= kTriRowScalar ? bsc : (bm == kTriRowVector ? p.b[cc] : brow[cc]),
+                                           cm >= kTriRowScalar ? csc : (cm == kTriRowVector ? p.c[cc] : crow[cc]));
+        }
       }
     }
+  };
+  for (uint32_t ct = cb; ct < p.tiles_per_row; ct += p.col_blocks) {
+    if ((int64_t)(ct + 1) * TILE <= p.L) column_tile(std::true_type(), ct);
+    else column_tile(std::false_type(), ct);
   }
 }
 
@@ -920,33 +969,41 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
   AM_TRY(ensure_init());
   const int in = r - 1;
   const int64_t L = g.shape[in];
-  g.a_const = g.sa[in] == 0; g.b_const = g.sb[in] == 0; g.c_const = g.sc[in] == 0;
-  g.a_keep = g.b_keep = g.c_keep = in > 0;
-  for (int d = 0; d < in; ++d) { g.a_keep &= g.sa[d] == 0; g.b_keep &= g.sb[d] == 0; g.c_keep &= g.sc[d] == 0; }
-  bool ok = g.sd[in] == 1 && (g.sa[in] == 1 || g.a_const) && (g.sb[in] == 1 || g.b_const) && (g.sc[in] == 1 || g.c_const) &&
-            aligned16(dst) && (g.a_const || aligned16(a)) && (g.b_const || aligned16(b)) && (g.c_const || aligned16(c));
+  const bool a_const = g.sa[in] == 0, b_const = g.sb[in] == 0, c_const = g.sc[in] == 0;
+  // an operand whose outer strides are all zero is one row for every output row
+  bool a_rowvec = in > 0 && !a_const, b_rowvec = in > 0 && !b_const, c_rowvec = in > 0 && !c_const;
+  for (int d = 0; d < in; ++d) { a_rowvec &= g.sa[d] == 0; b_rowvec &= g.sb[d] == 0; c_rowvec &= g.sc[d] == 0; }
+  bool ok = g.sd[in] == 1 && (g.sa[in] == 1 || a_const) && (g.sb[in] == 1 || b_const) && (g.sc[in] == 1 || c_const) &&
+            aligned16(dst) && (a_const || aligned16(a)) && (b_const || aligned16(b)) && (c_const || aligned16(c));
   for (int d = 0; d < in && ok; ++d)
-    if (g.sd[d] % VEC || (!g.a_const && g.sa[d] % VEC) || (!g.b_const && g.sb[d] % VEC) || (!g.c_const && g.sc[d] % VEC)) ok = false;
+    if (g.sd[d] % VEC || (!a_const && g.sa[d] % VEC) || (!b_const && g.sb[d] % VEC) || (!c_const && g.sc[d] % VEC)) ok = false;
   int64_t rows = 1;
   for (int d = 0; d < in; ++d) rows *= g.shape[d];
   const int64_t tile = (int64_t)kThreads * VEC * kUnroll;
   const int64_t tiles_per_row = (L + tile - 1) / tile;
-  if (ok && rows > 1 && L < tile / 8) ok = false;
-  if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31))) ok = false;
+  // (rows shorter than one vector: the streaming kernel's clamped loads would overrun them)
+  if (ok && ((rows > 1 && L < tile / 8) || L < VEC)) ok = false;
+  if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31) || rows >= ((int64_t)1 << 31))) ok = false;
   g.n = n; g.L = L;
-  {  // same rule as the two-operand kernel: non-temporal loads once the operands read once exceed what the L2s hold
-    const int streamed = (!g.a_const && !g.a_keep) + (!g.b_const && !g.b_keep) + (!g.c_const && !g.c_keep);
-    if (!(streamed * (double)rows * (double)L * sizeof(T) > 32.0 * 1024 * 1024)) g.a_keep = g.b_keep = g.c_keep = 1;
-    if (const char* e = getenv("AM_HIP_EW_NT")) { if (*e == '1') { g.a_keep = g.b_keep = g.c_keep = 0; } else if (*e == '0') { g.a_keep = g.b_keep = g.c_keep = 1; } }
-  }
   if (ok) {
+    // same rule as the two-operand kernel: non-temporal loads once the operands read once exceed what the L2s hold
+    const int streamed = (!a_const && !a_rowvec) + (!imm && !b_const && !b_rowvec) + (!imm && !c_const && !c_rowvec);
+    bool nt = streamed * (double)rows * (double)L * sizeof(T) > 32.0 * 1024 * 1024;
+    if (const char* e = getenv("AM_HIP_EW_NT")) { if (*e == '1') nt = true; else if (*e == '0') nt = false; }
+    auto mode = [&](bool is_const, bool rowvec) { return is_const ? kTriRowScalar : rowvec ? kTriRowVector : nt ? kTriVecNt : kTriVec; };
+    g.a_mode = mode(a_const, a_rowvec);
+    g.b_mode = imm ? kTriImm : mode(b_const, b_rowvec);
+    g.c_mode = imm ? kTriImm : mode(c_const, c_rowvec);
     g.rank = in;
     g.tiles_per_row = (uint32_t)tiles_per_row;
-    g.total_tiles = (uint32_t)(tiles_per_row * rows);
-    int64_t blocks = g.total_tiles;
+    g.rows = (uint32_t)rows;
     const int64_t cap = (int64_t)num_cus() * 32;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL((ew3_rows<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), g);
+    const int64_t col_blocks = tiles_per_row < cap ? tiles_per_row : cap;
+    int64_t row_groups = cap / col_blocks;
+    if (row_groups > rows) row_groups = rows;
+    if (row_groups < 1) row_groups = 1;
+    g.col_blocks = (uint32_t)col_blocks;
+    hipLaunchKernelGGL((ew3_rows<T, OP>), dim3((unsigned)(col_blocks * row_groups)), dim3(kThreads), 0, stream(), g);
     return check_launch("ew3_rows");
   }
   g.rank = r;
