@@ -23,6 +23,10 @@ int num_cus();
 // am_hip_diag_clock_begin .. _end is open; nullptr otherwise (the kernels then read no counter).
 long long* clock_probe_buffer();
 
+// Inputs larger than this are read with non-temporal loads by the streaming kernels outside the element-wise
+// family (experiments: AM_HIP_NT_MB in the environment, in MiB).
+double nt_threshold_bytes();
+
 // In a kernel: reads both counters at construction; finish() has the first lane of workgroup 0 add the
 // differences to out[0] (shader cycles) and out[1] (ticks). Does nothing when `out` is null.
 struct ClockProbe {

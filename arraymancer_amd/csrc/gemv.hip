@@ -274,7 +274,7 @@ int dot(const char* fn, int64_t n, const T* x, int64_t incx, const T* y, int64_t
   const int64_t cap = (int64_t)num_cus() * 4;
   if (blocks > cap) blocks = cap;
   const bool vec = incx == 1 && incy == 1 && aligned16(x) && aligned16(y);
-  const bool stream_loads = 2.0 * (double)n * sizeof(T) > 384.0 * 1024 * 1024;
+  const bool stream_loads = 2.0 * (double)n * sizeof(T) > nt_threshold_bytes();
   T* ws = (T*)splitk_workspace((size_t)(blocks + 1) * sizeof(T));
   if (!ws) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
   const dim3 grid((unsigned)blocks), block(256);

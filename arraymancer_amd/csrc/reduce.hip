@@ -235,9 +235,10 @@ static int launch(Args<T>& g, bool row_kernel, size_t ws_off) {
     if (chunks > 8192) chunks = 8192;
   }
   g.chunks = 1; g.chunk_len = g.L; g.ws = nullptr;
-  // 8192 x 8192 f64 row sums: 98 us with ordinary loads, 88 us with non-temporal ones; at half the size
-  // (which the 256 MB memory-side cache can hold from the producing kernel) it is the other way round
-  const bool stream_loads = (double)g.outputs * (double)g.L * sizeof(T) > 384.0 * 1024 * 1024;
+  // Inputs beyond what the L2s hold are read with non-temporal loads: 8192 x 8192 f32 row sums over rotating
+  // buffers (every byte from HBM) 47.2 -> 42.8 us; the same buffer every launch, which the memory-side cache
+  // partly holds, 40.4 -> 41.7 us.
+  bool stream_loads = (double)g.outputs * (double)g.L * sizeof(T) > nt_threshold_bytes();
   if (chunks > 1) {
     int64_t len = (g.L + chunks - 1) / chunks;
     len = (len + V - 1) / V * V;                    // chunk starts stay 16-byte aligned
@@ -690,7 +691,7 @@ __global__ __launch_bounds__(256) void softmax_rows(SoftmaxArgs<T> p) {
 // row is read from memory once and written once. W lanes per row (64: four rows per workgroup;
 // 256: one row per workgroup). Requires unit column strides, cols a multiple of the vector width
 // and 16-byte aligned rows; cols <= W * NV * VEC.
-template <typename T, int W, int NV>
+template <typename T, int W, int NV, bool STREAM>
 __global__ __launch_bounds__(256) void softmax_rows_reg(SoftmaxArgs<T> p) {
   constexpr int V = 16 / (int)sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(V)));
@@ -704,11 +705,18 @@ __global__ __launch_bounds__(256) void softmax_rows_reg(SoftmaxArgs<T> p) {
   const T ninf = -std::numeric_limits<T>::infinity();
   vec_t x[NV];
   T mx = ninf;
+  // every load of the row is issued before the first use, unconditionally (vectors past the end of the row read
+  // its first one): loads under a per-lane test are waited for one by one
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int64_t v = (int64_t)i * W + me;
+    const vec_t* at = src + (v < nvec ? v : 0);
+    if constexpr (STREAM) x[i] = __builtin_nontemporal_load(at); else x[i] = *at;
+  }
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int64_t v = (int64_t)i * W + me;
     if (active && v < nvec) {
-      x[i] = src[v];
 #pragma unroll
       for (int e = 0; e < V; ++e) mx = (x[i][e] <= mx) ? mx : x[i][e];
     }
@@ -754,14 +762,14 @@ __global__ __launch_bounds__(256) void softmax_rows_reg(SoftmaxArgs<T> p) {
   }
 }
 
-template <typename T, int W>
+template <typename T, int W, bool STREAM>
 static void launch_softmax_reg(const SoftmaxArgs<T>& p, int nv, dim3 grid) {
   switch (nv) {
-    case 1: hipLaunchKernelGGL((softmax_rows_reg<T, W, 1>), grid, dim3(256), 0, stream(), p); break;
-    case 2: hipLaunchKernelGGL((softmax_rows_reg<T, W, 2>), grid, dim3(256), 0, stream(), p); break;
-    case 4: hipLaunchKernelGGL((softmax_rows_reg<T, W, 4>), grid, dim3(256), 0, stream(), p); break;
-    case 8: hipLaunchKernelGGL((softmax_rows_reg<T, W, 8>), grid, dim3(256), 0, stream(), p); break;
-    default: hipLaunchKernelGGL((softmax_rows_reg<T, W, 16>), grid, dim3(256), 0, stream(), p); break;
+    case 1: hipLaunchKernelGGL((softmax_rows_reg<T, W, 1, STREAM>), grid, dim3(256), 0, stream(), p); break;
+    case 2: hipLaunchKernelGGL((softmax_rows_reg<T, W, 2, STREAM>), grid, dim3(256), 0, stream(), p); break;
+    case 4: hipLaunchKernelGGL((softmax_rows_reg<T, W, 4, STREAM>), grid, dim3(256), 0, stream(), p); break;
+    case 8: hipLaunchKernelGGL((softmax_rows_reg<T, W, 8, STREAM>), grid, dim3(256), 0, stream(), p); break;
+    default: hipLaunchKernelGGL((softmax_rows_reg<T, W, 16, STREAM>), grid, dim3(256), 0, stream(), p); break;
   }
 }
 
@@ -781,11 +789,13 @@ static int softmax(const char* fn, int64_t rows, int64_t cols, T* dst, int64_t d
   if (vec && nvec <= 64 * 8) {          // a wavefront per row
     int nv = 1;
     while (64 * nv < nvec) nv *= 2;
-    launch_softmax_reg<T, 64>(p, nv, dim3((unsigned)((rows + 3) / 4)));
+    launch_softmax_reg<T, 64, false>(p, nv, dim3((unsigned)((rows + 3) / 4)));
   } else if (vec && nvec <= 256 * 16) {  // a workgroup per row (up to 64 registers of row per lane)
     int nv = 1;
     while (256 * nv < nvec) nv *= 2;
-    launch_softmax_reg<T, 256>(p, nv, dim3((unsigned)rows));
+    // rows this long make an input beyond the L2s at a few thousand rows: read it with non-temporal loads then
+    if ((double)rows * (double)cols * sizeof(T) > nt_threshold_bytes()) launch_softmax_reg<T, 256, true>(p, nv, dim3((unsigned)rows));
+    else launch_softmax_reg<T, 256, false>(p, nv, dim3((unsigned)rows));
   } else if (cols > 4096) {
     hipLaunchKernelGGL((softmax_rows<T, true>), dim3((unsigned)rows), dim3(256), 0, stream(), p);
   } else {

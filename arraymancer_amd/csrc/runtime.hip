@@ -12,6 +12,11 @@ namespace am {
 
 static thread_local char g_err[512] = "";
 
+double nt_threshold_bytes() {
+  static const double mb = [] { const char* e = getenv("AM_HIP_NT_MB"); return (e && *e) ? atof(e) : 32.0; }();
+  return mb * 1024.0 * 1024.0;
+}
+
 int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
