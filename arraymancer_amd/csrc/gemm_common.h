@@ -14,7 +14,19 @@ namespace gemm {
 enum LoadKind : int {
   kKContig = 0,   // ld_k == 1: 16-byte vectors along k
   kMNContig = 1,  // ld_mn == 1: 16-byte vectors along m (A) or n (B)
-  kGeneric = 2    // any strides (zero, negative, non-unit): scalar gathers
+  kGeneric = 2,   // any strides (zero, negative, non-unit): scalar gathers
+  kGather = 3     // B only: the column matrix of a convolution, read straight from the image (ConvGeom)
+};
+
+// Geometry of a convolution whose column matrix col(k, j) = image[c, oh * sh - ph + kh, ow * sw - pw + kw]
+// (k = (c * kH + kh) * kW + kw, j = oh * Wo + ow; zero where the window leaves the image) is the B operand of
+// a GEMM without ever being written to memory (fallback/conv.nim:18-54 writes it, one image at a time).
+// k is decoded with two multiply-high divisions by kH * kW and kW (multipliers from the host, exact while
+// K * kH * kW < 2^32).
+struct ConvGeom {
+  int H, W, kH, kW, Wo, ph, pw, sh, sw;
+  uint32_t magic_khw, magic_kw;   // ceil(2^32 / (kH * kW)), ceil(2^32 / kW); 0 where the divisor is 1
+  int64_t in_c, in_h, in_w;       // strides of the image (elements); the image pointer is the GEMM's B
 };
 
 template <typename T> struct Args {
@@ -51,6 +63,7 @@ template <typename T> struct Args {
   bool static_ws;
   size_t static_ws_short;
   long long* clock_out;            // where the matrix-core kernels add their cycle counts while a clock window is open
+  ConvGeom conv;                   // read by the kGather loader only
 };
 
 // Digit pairs (i, j), i + j < ND, whose planes are both marked non-empty: flags[i] == gen for A's
@@ -160,6 +173,35 @@ static inline int choose_tile(const TileChoice* cand, int ncand, int64_t M, int6
   }
   if (cost_out) *cost_out = best_cost;
   return best;
+}
+
+// Fills the GEMM view of a convolution (fallback/conv.nim:81-106: out[n] = kernel_col * col[n] + bias) whose column
+// matrix is gathered by the kGather loader: M = C_out, N = H_out * W_out, K = C * kH * kW, one batch member per image.
+// Returns 1 when there is nothing to do, a negative code on bad arguments.
+template <typename T>
+static int prepare_conv(const char* fn, int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH,
+                        int strideW, const T* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, const T* kernel,
+                        int64_t kernel_rs, int epilogue, const T* bias, int64_t bias_s, T* out, Args<T>* g_out) {
+  if (N < 0 || C < 0 || H < 0 || W < 0 || Cout < 0 || kH <= 0 || kW <= 0 || padH < 0 || padW < 0 || strideH <= 0 || strideW <= 0)
+    return fail(AM_E_ARG, "%s: bad geometry", fn);
+  if (N > 65535) return fail(AM_E_SHAPE, "%s: more than 65535 images in one call", fn);
+  const int64_t Ho = ((int64_t)H + 2 * padH - kH) / strideH + 1, Wo = ((int64_t)W + 2 * padW - kW) / strideW + 1;
+  if ((int64_t)H + 2 * padH < kH || (int64_t)W + 2 * padW < kW) return fail(AM_E_SHAPE, "%s: kernel larger than the padded image", fn);
+  if (N == 0 || C == 0 || Cout == 0 || Ho <= 0 || Wo <= 0) return 1;
+  const int64_t K = (int64_t)C * kH * kW, P = Ho * Wo;
+  if (K < 16 / (int64_t)sizeof(T) || K * kH * kW >= ((int64_t)1 << 32) || P >= ((int64_t)1 << 31))
+    return fail(AM_E_SHAPE, "%s: C * kH * kW = %lld outside what the fused kernel takes (use im2col + gemm_batched)", fn, (long long)K);
+  if (!in || !kernel || !out) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  const int rc = prepare<T>(fn, Cout, P, K, (T)1, kernel, kernel_rs, 1, in, 0, 1, (T)0, out, P, 1, epilogue, bias, bias_s, 0, g_out);
+  if (rc != AM_OK) return rc;
+  Args<T>& g = *g_out;
+  g.batch = (int)N; g.batch_a = 0; g.batch_b = in_n; g.batch_c = (int64_t)Cout * P;
+  ConvGeom& cg = g.conv;
+  cg.H = H; cg.W = W; cg.kH = kH; cg.kW = kW; cg.Wo = (int)Wo; cg.ph = padH; cg.pw = padW; cg.sh = strideH; cg.sw = strideW;
+  cg.in_c = in_c; cg.in_h = in_h; cg.in_w = in_w;
+  auto magic = [](int d) { return d == 1 ? 0u : (uint32_t)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d); };
+  cg.magic_khw = magic(kH * kW); cg.magic_kw = magic(kW);
+  return AM_OK;
 }
 
 // The sub-problem C[r0:r1, c0:c1] of g (rows of A, columns of B, the block of C and of the bias).

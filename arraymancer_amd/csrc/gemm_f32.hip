@@ -103,3 +103,22 @@ extern "C" int am_hip_gemm_batched_f32(int64_t batch, int64_t M, int64_t N, int6
   AM_TRY(ensure_init());
   return run_f32(g);
 }
+
+// im2colgemm_conv2d (src/arraymancer/nn_primitives/fallback/conv.nim:81-106) in one launch: the column matrix is never
+// written, the GEMM's B loader gathers it from the images; bias and ReLU in the epilogue.
+extern "C" int am_hip_conv2d_f32(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH,
+                                 int strideW, const float* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                                 const float* kernel, int64_t kernel_rs, int epilogue, const float* bias, int64_t bias_s, float* out) {
+  Args<float> g;
+  const int rc = prepare_conv<float>("am_hip_conv2d_f32", N, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW, in, in_n, in_c,
+                                    in_h, in_w, kernel, kernel_rs, epilogue, bias, bias_s, out, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  // (a 128 x 128 tile, eight gathered elements per lane and slab, measured half as fast as 64 x 64 with four)
+  static const TileChoice cand[] = {{64, 64, 0.88}, {32, 32, 0.60}};
+  switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_CONV_TILE_F32", g.batch)) {
+    case 0: return launch_conv<float, 64, 64, 16, 2, 2, 2>(g);
+    default: return launch_conv<float, 32, 32, 32, 2, 2, 2, true, true, MfmaF32x16>(g);
+  }
+}

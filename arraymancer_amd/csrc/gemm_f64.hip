@@ -90,3 +90,21 @@ extern "C" int am_hip_gemm_batched_f64(int64_t batch, int64_t M, int64_t N, int6
   AM_TRY(ensure_init());
   return run_f64(g);
 }
+
+// im2colgemm_conv2d (src/arraymancer/nn_primitives/fallback/conv.nim:81-106) in one launch: the column matrix is never
+// written, the GEMM's B loader gathers it from the images; bias and ReLU in the epilogue.
+extern "C" int am_hip_conv2d_f64(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH,
+                                 int strideW, const double* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                                 const double* kernel, int64_t kernel_rs, int epilogue, const double* bias, int64_t bias_s, double* out) {
+  Args<double> g;
+  const int rc = prepare_conv<double>("am_hip_conv2d_f64", N, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW, in, in_n, in_c,
+                                    in_h, in_w, kernel, kernel_rs, epilogue, bias, bias_s, out, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  static const TileChoice cand[] = {{64, 64, 0.93}, {32, 32, 0.62}};
+  switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_CONV_TILE_F64", g.batch)) {
+    case 0: return launch_conv<double, 64, 64, 16, 2, 2, 2>(g);
+    default: return launch_conv<double, 32, 32, 16, 2, 2, 2>(g);
+  }
+}

@@ -147,7 +147,7 @@ void gemm_mfma(Args<T> p) {
   const int lrow = lane % TILE, kl = lane / TILE;
 
   Loader<T, AK, BM, BK, NT, true, PF> la(p.A, p.a_mn, p.a_k, m0, p.M, k_end, p.a_kfast);
-  Loader<T, BKIND, BN, BK, NT, true, PF> lb(p.B, p.b_mn, p.b_k, n0, p.N, k_end, p.b_kfast);
+  Loader<T, BKIND, BN, BK, NT, true, PF> lb(p.B, p.b_mn, p.b_k, n0, p.N, k_end, p.b_kfast, &p.conv);
 
   acc_t acc[TM][TN];
 #pragma unroll
@@ -466,6 +466,22 @@ static int launch_kinds(Args<T>& g, int ak, int bk) {
   }
 #undef AM_LAUNCH
   AM_TRY(check_launch("gemm_mfma"));
+  if (g.splits > 1) return launch_splitk_reduce<T, T>(g);
+  return AM_OK;
+}
+
+// A convolution as one batched GEMM whose B operand is gathered from the images (kGather): A = the kernel matrix
+// [C_out, C * kH * kW] with unit stride along k, one batch member per image.
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true, bool RU = true, typename MF = Mfma<T>>
+static int launch_conv(Args<T>& g) {
+  g.tiles_m = (int)((g.M + BM - 1) / BM);
+  g.tiles_n = (int)((g.N + BN - 1) / BN);
+  const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
+  if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "conv2d: too many tiles");
+  plan_splitk(g, BK, WAVES_M * WAVES_N);
+  const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(WAVES_M * WAVES_N * 64);
+  hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, kKContig, kGather>), grid, block, 0, stream(), g);
+  AM_TRY(check_launch("gemm_mfma (convolution)"));
   if (g.splits > 1) return launch_splitk_reduce<T, T>(g);
   return AM_OK;
 }

@@ -5,11 +5,11 @@ composed from the device operators of this package:
     cv1 = Conv2D(1 -> 20, 5x5)   mp1 = MaxPool2D(2x2, stride 2)   cv2 = Conv2D(20 -> 50, 5x5)   mp2 = MaxPool2D(2x2, stride 2)
     fl = Flatten                 hidden = Linear(800 -> 500)      classifier = Linear(500 -> 10)
 
-Each convolution is the reference's im2col + GEMM (nn_primitives/fallback/conv.nim:81-106) as one device
-im2col of the whole batch and one strided-batched GEMM with the bias and the ReLU that follows it fused into
+Each convolution is the reference's im2col + GEMM (nn_primitives/fallback/conv.nim:81-106) as ONE batched GEMM
+whose B loader gathers the column matrix from the images, with the bias and the ReLU that follows it fused into
 the epilogue; each dense layer is one GEMM with fused bias (+ ReLU) (nn_primitives/nnp_linear.nim:20-29); max
 pooling is nn_primitives/nnp_maxpooling.nim:19-66. Every buffer is allocated once in the constructor, so that
-`forward` issues eight kernel launches and nothing else and can be recorded into a HIP graph.
+`forward` issues six kernel launches and nothing else and can be recorded into a HIP graph.
 """
 from __future__ import annotations
 
@@ -19,7 +19,7 @@ import numpy as np
 
 from . import _lib
 from ._lib import check
-from .tensor_hip import Graph, HipTensor, empty, gemm, gemm_batched, toHip
+from .tensor_hip import Graph, HipTensor, conv2d_into, empty, gemm, toHip
 
 
 class DemoNet:
@@ -36,23 +36,13 @@ class DemoNet:
         h2, w2 = hp1 - k2 + 1, wp1 - k2 + 1             # 8 x 8
         hp2, wp2 = h2 // 2, w2 // 2                     # 4 x 4
         e = lambda *shape: empty(shape, dtype)
-        self.col1, self.a1 = e(batch, 1 * k1 * k1, h1 * w1), e(batch, c1, h1, w1)
+        self.a1 = e(batch, c1, h1, w1)
         self.pool1, self.idx1 = e(batch, c1, hp1, wp1), empty((batch * c1 * hp1 * wp1,), np.int64)
-        self.col2, self.a2 = e(batch, c1 * k2 * k2, h2 * w2), e(batch, c2, h2, w2)
+        self.a2 = e(batch, c2, h2, w2)
         self.pool2, self.idx2 = e(batch, c2, hp2, wp2), empty((batch * c2 * hp2 * wp2,), np.int64)
         self.hidden, self.logits = e(batch, self.p["hidden_w"].shape[0]), e(batch, self.p["classifier_w"].shape[0])
         if c2 * hp2 * wp2 != self.p["hidden_w"].shape[1]:
             raise ValueError("hidden layer width does not match the flattened pooling output")
-
-    # one convolution stage: device im2col of the batch, then kernel_col [C_out, C kH kW] x col[n] for every image in
-    # one strided-batched GEMM that writes the NCHW result and applies bias + ReLU in its epilogue
-    def _conv_relu(self, x: HipTensor, w: HipTensor, b: HipTensor, col: HipTensor, out: HipTensor):
-        N, C, H, W = x.shape
-        co, _, kh, kw = w.shape
-        check(getattr(_lib.load(), f"am_hip_im2col_{x.sfx}")(
-            N, C, H, W, kh, kw, 0, 0, 1, 1, ctypes.c_void_p(x.data_ptr()), *x.strides, ctypes.c_void_p(col.data_ptr())))
-        gemm_batched(1, w.reshape(co, C * kh * kw), col, 0, out.reshape(N, co, out.shape[2] * out.shape[3]),
-                     epilogue="bias_relu", bias=b.reshape(co, 1))
 
     def _maxpool(self, x: HipTensor, out: HipTensor, idx: HipTensor):
         N, C, H, W = x.shape
@@ -63,9 +53,9 @@ class DemoNet:
     def forward(self, x: HipTensor) -> HipTensor:
         """x: [batch, 1, 28, 28] on the device. Returns the [batch, 10] logits (a buffer of this object)."""
         p = self.p
-        self._conv_relu(x, p["cv1_w"], p["cv1_b"], self.col1, self.a1)
+        conv2d_into(self.a1, x, p["cv1_w"], p["cv1_b"], relu=True)
         self._maxpool(self.a1, self.pool1, self.idx1)
-        self._conv_relu(self.pool1, p["cv2_w"], p["cv2_b"], self.col2, self.a2)
+        conv2d_into(self.a2, self.pool1, p["cv2_w"], p["cv2_b"], relu=True)
         self._maxpool(self.a2, self.pool2, self.idx2)
         flat = self.pool2.reshape(self.batch, self.pool2.size // self.batch)          # Flatten: metadata only
         gemm(1, flat, p["hidden_w"].transpose(), 0, self.hidden, epilogue="bias_relu", bias=p["hidden_b"])

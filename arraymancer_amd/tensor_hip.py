@@ -484,23 +484,48 @@ def im2col(x: HipTensor, kernel_size, padding=(0, 0), stride=(1, 1)) -> HipTenso
     return col
 
 
+def conv2d_into(out: HipTensor, x: HipTensor, kernel: HipTensor, bias: HipTensor | None = None, padding=(0, 0), stride=(1, 1),
+                relu: bool = False) -> HipTensor:
+    """The fused convolution of `conv2d` written into an existing C-contiguous [N, C_out, H_out, W_out] tensor: one
+    launch, nothing allocated (what a captured graph needs). Float tensors, kernel rows with unit stride."""
+    _same_dtype(x, kernel, out)
+    N, C, H, W = x.shape
+    co, ci, kh, kw = kernel.shape
+    kcol = kernel.reshape(co, ci * kh * kw)
+    if kcol.strides[1] != 1 or not out.is_C_contiguous():
+        raise ValueError("conv2d_into: the kernel needs unit stride within a row and the result must be C-contiguous")
+    epi = EPI[("bias_relu" if relu else "bias") if bias is not None else ("relu" if relu else "none")]
+    bptr, bs = (ctypes.c_void_p(bias.data_ptr()), bias.reshape(co).strides[0]) if bias is not None else (None, 0)
+    check(getattr(_lib.load(), f"am_hip_conv2d_{x.sfx}")(
+        N, C, H, W, co, kh, kw, padding[0], padding[1], stride[0], stride[1], ctypes.c_void_p(x.data_ptr()), *x.strides,
+        ctypes.c_void_p(kcol.data_ptr()), kcol.strides[0], epi, bptr, bs, ctypes.c_void_p(out.data_ptr())))
+    return out
+
+
 def conv2d(x: HipTensor, kernel: HipTensor, bias: HipTensor | None = None, padding=(0, 0), stride=(1, 1),
-           relu: bool = False) -> HipTensor:
-    """im2colgemm_conv2d (src/arraymancer/nn_primitives/fallback/conv.nim:81-106) in two launches:
-    device im2col of the batch, then one strided-batched GEMM kernel_col[C_out, C*kH*kW] * col[n]
-    written straight into the NCHW result, with the bias [C_out, 1, 1] (and an optional ReLU) fused
-    into its epilogue for float tensors."""
+           relu: bool = False, fused: bool | None = None) -> HipTensor:
+    """im2colgemm_conv2d (src/arraymancer/nn_primitives/fallback/conv.nim:81-106). Float tensors: ONE launch, a
+    batched GEMM kernel_col[C_out, C*kH*kW] * col[n] whose B loader gathers the column matrix from the images
+    (it is never written), with the bias [C_out, 1, 1] (and an optional ReLU) in its epilogue. Integer tensors, and
+    `fused=False`: device im2col of the batch, then one strided-batched GEMM written straight into the NCHW result."""
     _same_dtype(x, kernel)
     N, C, H, W = x.shape
     co, ci, kh, kw = kernel.shape
     if ci != C:
         raise ValueError(f"conv2d: kernel expects {ci} input channels, input has {C}")
-    col = im2col(x, (kh, kw), padding, stride)
     ho, wo = (H + 2 * padding[0] - kh) // stride[0] + 1, (W + 2 * padding[1] - kw) // stride[1] + 1
+    is_float = x.dtype.kind == "f"
+    if fused is None:
+        # up to about a hundred output channels the gathered form wins (no column matrix is written and read back);
+        # beyond, the two-launch form's vector loads and larger tiles do (32 x 128 x 28 x 28 -> 128, 3 x 3: 139 against 117 us)
+        fused = is_float and ci * kh * kw * x.dtype.itemsize >= 16 and N <= 65535 and co <= 96
+    if fused:
+        k = kernel if kernel.reshape(co, ci * kh * kw).strides[1] == 1 else kernel.clone()
+        return conv2d_into(empty((N, co, ho, wo), x.dtype), x, k, bias, padding, stride, relu)
+    col = im2col(x, (kh, kw), padding, stride)
     out = empty((N, co, ho, wo), x.dtype)
     out3 = out.reshape(N, co, ho * wo)
     kcol = kernel.reshape(co, ci * kh * kw)
-    is_float = x.dtype.kind == "f"
     if bias is not None and is_float:
         gemm_batched(1, kcol, col, 0, out3, epilogue="bias_relu" if relu else "bias", bias=bias.reshape(co, 1))
     else:

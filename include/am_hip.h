@@ -216,6 +216,22 @@ int am_hip_im2col_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, 
 int am_hip_im2col_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
                       const int64_t* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, int64_t* col);
 
+/* out[n][co][h*W_out + w] <- sum over (c, kh, kw) of kernel[co][c*kH*kW + kh*kW + kw] * (padded input patch element)
+ * (+ bias[co]) (then ReLU), for the whole batch in ONE launch: the column matrix of im2col is never written, the
+ * GEMM's B loader gathers it from the images. `in` is addressed through its four NCHW strides (elements); `kernel` is
+ * the [C_out, C*kH*kW] matrix of a [C_out, C, kH, kW] tensor, rows `kernel_rs` apart, unit stride within a row;
+ * `bias` (epilogue AM_EPI_BIAS / AM_EPI_BIAS_RELU) has C_out elements `bias_s` apart; `out` is a contiguous
+ * [N, C_out, H_out, W_out] tensor. Float types; N <= 65535; C*kH*kW must hold one 16-byte vector at least
+ * (AM_E_SHAPE otherwise: run am_hip_im2col_* + am_hip_gemm_batched_* then).
+ * Replaces im2colgemm_conv2d (src/arraymancer/nn_primitives/fallback/conv.nim:81-106: per image im2col, gemm,
+ * then the bias broadcast added) followed by relu (nnp_activation.nim:35-36) where asked for. */
+int am_hip_conv2d_f32(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const float* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                      const float* kernel, int64_t kernel_rs, int epilogue, const float* bias, int64_t bias_s, float* out);
+int am_hip_conv2d_f64(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const double* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                      const double* kernel, int64_t kernel_rs, int epilogue, const double* bias, int64_t bias_s, double* out);
+
 /* ---------------------------------------------------------------- GEMV and dot
  * y[M] <- alpha * A[M x N] * x[N] + beta * y, any strides (elements).
  * Replaces gemv (src/arraymancer/tensor/operators_blas_l2l3.nim:24-56; integer fallback

@@ -45,6 +45,9 @@ GEOMS = [  # N, C, H, W, C_out, kH, kW, pad, stride
     (16, 20, 12, 12, 50, 5, 5, (0, 0), (1, 1)),     # conv2 (8 x 8 = 64 outputs)
     (2, 3, 4, 8, 2, 3, 3, (0, 0), (1, 1)),          # 2 x 6 outputs: 16-byte groups of pixels straddle the output rows
     (4, 2, 16, 16, 3, 3, 3, (1, 1), (2, 2)),        # stride 2 with padding, 8 x 8 outputs
+    (2, 5, 11, 13, 70, 1, 1, (0, 0), (1, 1)),       # 1 x 1 kernel (k is the channel alone), more output channels than a small tile
+    (3, 8, 20, 20, 130, 3, 5, (2, 3), (1, 2)),      # padding wider than the kernel's reach on one side, 130 output channels
+    (2, 16, 40, 40, 32, 3, 3, (1, 1), (1, 1)),      # 1600 outputs per image: the larger tiles
 ]
 
 
@@ -62,14 +65,20 @@ def test_im2col_and_conv_vs_oracle(hip, oracle, sfx, geom):
         assert np.array_equal(col[n], oracle.im2col(x[n], (kh, kw), pad, stride))
     say("conv2d", sfx, geom)
     want = oracle.conv2d(x, k, b, pad, stride)
-    got = hip.conv2d(dx, hip.toHip(k), hip.toHip(b), pad, stride).toCpu()
-    check(oracle, sfx, got, want, "conv + bias")
-    got = hip.conv2d(dx, hip.toHip(k), hip.toHip(b), pad, stride, relu=True).toCpu()
-    check(oracle, sfx, got, np.where(0 >= want, np.zeros_like(want), want), "conv + bias + relu")
-    # a channel-sliced (strided) input goes through the same kernel
-    if C > 1:
-        got = hip.conv2d(dx[:, ::-1], hip.toHip(np.ascontiguousarray(k[:, ::-1])), None, pad, stride).toCpu()
-        check(oracle, sfx, got, oracle.conv2d(x, k, None, pad, stride), "reversed channels")
+    # floats: the one-launch form (column matrix gathered by the GEMM's loader) and the im2col + batched GEMM form;
+    # integers only have the second
+    forms = (True, False, None) if sfx in ("f32", "f64") and C * kh * kw * np.dtype(dt).itemsize >= 16 else (False, None)
+    for fused in forms:
+        got = hip.conv2d(dx, hip.toHip(k), hip.toHip(b), pad, stride, fused=fused).toCpu()
+        check(oracle, sfx, got, want, f"conv + bias, fused={fused}")
+        got = hip.conv2d(dx, hip.toHip(k), hip.toHip(b), pad, stride, relu=True, fused=fused).toCpu()
+        check(oracle, sfx, got, np.where(0 >= want, np.zeros_like(want), want), f"conv + bias + relu, fused={fused}")
+        got = hip.conv2d(dx, hip.toHip(k), None, pad, stride, fused=fused).toCpu()
+        check(oracle, sfx, got, oracle.conv2d(x, k, None, pad, stride), f"conv, fused={fused}")
+        # a channel-sliced (strided) input goes through the same kernel
+        if C > 1:
+            got = hip.conv2d(dx[:, ::-1], hip.toHip(np.ascontiguousarray(k[:, ::-1])), None, pad, stride, fused=fused).toCpu()
+            check(oracle, sfx, got, oracle.conv2d(x, k, None, pad, stride), f"reversed channels, fused={fused}")
 
 
 @pytest.mark.parametrize("sfx", ALL)
