@@ -185,6 +185,12 @@ def test_extents_just_above_a_tile_multiple(hip, oracle, sfx, monkeypatch):
         assert_parity(oracle, sfx, results["1plain"], oracle.matmul(vA[1], vB[1]), f"cut, plain {(M, N, K)} {trans}")
         assert oracle.rel_frobenius(results["1"], results["0"]) <= TOL[sfx]
         assert oracle.rel_frobenius(results["1plain"], results["0plain"]) <= TOL[sfx]
+        # a column-major destination (the library multiplies the transposed problem: the cut must follow the swap)
+        monkeypatch.setenv("AM_HIP_GEMM_PEEL", "1")
+        dCt = hip.toHip(np.ascontiguousarray(C.T))
+        hip.gemm(1.5, vA[0], vB[0], 0.5, dCt.transpose(), epilogue="bias", bias=hip.toHip(bias))
+        want_cm = oracle.map2("add", oracle.gemm_strided(1.5, vA[1], vB[1], 0.5, C.copy()), oracle.broadcast(bias, C.shape))
+        assert_parity(oracle, sfx, dCt.toCpu().T, want_cm, f"cut, column-major C {(M, N, K)} {trans}")
 
 
 # ------------------------------------------------------------------ strided / transposed views
