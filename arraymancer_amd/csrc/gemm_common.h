@@ -26,7 +26,12 @@ enum LoadKind : int {
 struct ConvGeom {
   int H, W, kH, kW, Wo, ph, pw, sh, sw;
   uint32_t magic_khw, magic_kw;   // ceil(2^32 / (kH * kW)), ceil(2^32 / kW); 0 where the divisor is 1
-  int64_t in_c, in_h, in_w;       // strides of the image (elements); the image pointer is the GEMM's B
+  // Strides of the image in BYTES, and the distance in bytes from the lowest address any of its elements has to
+  // its element (0, 0, 0): every element's offset from that lowest address is then a non-negative 32-bit number
+  // (the host refuses images that span 4 GiB or more), which is what a load with a scalar base and a 32-bit
+  // vector offset takes. The image pointer is the GEMM's B.
+  int in_c, in_h, in_w;
+  uint32_t origin;
 };
 
 template <typename T> struct Args {
@@ -198,7 +203,18 @@ static int prepare_conv(const char* fn, int64_t N, int C, int H, int W, int Cout
   g.batch = (int)N; g.batch_a = 0; g.batch_b = in_n; g.batch_c = (int64_t)Cout * P;
   ConvGeom& cg = g.conv;
   cg.H = H; cg.W = W; cg.kH = kH; cg.kW = kW; cg.Wo = (int)Wo; cg.ph = padH; cg.pw = padW; cg.sh = strideH; cg.sw = strideW;
-  cg.in_c = in_c; cg.in_h = in_h; cg.in_w = in_w;
+  {
+    const int64_t sz = (int64_t)sizeof(T);
+    const int64_t ext[3] = {C, H, W}, str[3] = {in_c, in_h, in_w};
+    int64_t lowest = 0, highest = 0;     // element offsets of the image's lowest and highest address
+    for (int d = 0; d < 3; ++d) {
+      if (str[d] < 0) lowest += str[d] * (ext[d] - 1); else highest += str[d] * (ext[d] - 1);
+    }
+    if ((highest - lowest + 1) * sz >= ((int64_t)1 << 32))
+      return fail(AM_E_SHAPE, "%s: one image spans 4 GiB or more (use im2col + gemm_batched)", fn);
+    cg.in_c = (int)(in_c * sz); cg.in_h = (int)(in_h * sz); cg.in_w = (int)(in_w * sz);
+    cg.origin = (uint32_t)(-lowest * sz);
+  }
   auto magic = [](int d) { return d == 1 ? 0u : (uint32_t)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d); };
   cg.magic_khw = magic(kH * kW); cg.magic_kw = magic(kW);
   return AM_OK;

@@ -273,58 +273,57 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
 
 // The column matrix of a convolution as the B operand, gathered from the image (ConvGeom): element (k, j) is one
 // image element or zero. A lane owns one column j (one output pixel: its window origin is decoded once) and NE k
-// values per slab, NT / BMN apart; every load is unconditional from an address clamped into the image and
-// what the padding or the end of the k range rules out is replaced by zero before the commit. k-row LDS layout.
+// values per slab, NT / BMN apart. k is decoded into (c, kh, kw) by two multiply-high divisions - scalar arithmetic
+// where the slab is 64 columns wide or more, since the lanes of a wavefront then share k; an element's address is a
+// uniform base plus a non-negative 32-bit byte offset. Every load is unconditional (what the padding or the end of
+// the k range rules out is loaded from the image's lowest address instead) and replaced by zero before the commit.
+// The loader is bound by the instructions it issues, not by its loads: each of these choices removes some.
+// k-row LDS layout.
 template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kGather, BMN, BK, NT, KG, PF> {
   static constexpr int NE = BMN * BK / NT;         // elements per thread
   static constexpr int KSTRIDE = NT / BMN;         // distance in k between a lane's elements
   static_assert(BMN * BK % NT == 0 && NE >= 1 && NT % BMN == 0, "a lane must own one column of the slab");
-  const T* img;
-  int64_t noff;          // offset of the window origin (may lie in the padding: negative coordinates)
+  const char* low;       // the image's lowest address
+  uint32_t noff;         // byte offset of the window origin from `low` (modulo 2^32: it may lie in the padding)
   int ih0, iw0, kbase;
   int64_t K;
   ConvGeom g;
   T reg[PF][NE];
-  uint32_t ok[PF];       // bit i: element i of the stage is a real image element
+  bool ok[PF][NE];       // the element is a real image element
   __device__ __forceinline__ Loader(const T* X, int64_t, int64_t, int64_t mn0, int64_t MN, int64_t K_, int, const ConvGeom* geom)
-      : img(X), K(K_), g(*geom) {
+      : K(K_), g(*geom) {
+    low = (const char*)X - g.origin;
     const int64_t j = mn0 + (int)(threadIdx.x % BMN);
     const int jj = (int)(j < MN ? j : MN - 1);      // columns past the edge repeat the last one (masked at the store)
     const int oh = jj / g.Wo, ow = jj - oh * g.Wo;
     ih0 = oh * g.sh - g.ph;
     iw0 = ow * g.sw - g.pw;
-    noff = (int64_t)ih0 * g.in_h + (int64_t)iw0 * g.in_w;
+    noff = g.origin + (uint32_t)(ih0 * g.in_h) + (uint32_t)(iw0 * g.in_w);
     kbase = (int)(threadIdx.x / BMN);
   }
   __device__ __forceinline__ bool tail_guard() const { return false; }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
     if (MASK && k0 >= K) return;
-    uint32_t bits = 0;
+    const uint32_t kb = (BMN % 64 == 0) ? (uint32_t)__builtin_amdgcn_readfirstlane(kbase) : (uint32_t)kbase;
 #pragma unroll
     for (int i = 0; i < NE; ++i) {
-      // (a slab column of 64 lanes or more: the lanes of a wavefront share k, so its decoding is scalar arithmetic)
-      const uint32_t kb = (BMN % 64 == 0) ? (uint32_t)__builtin_amdgcn_readfirstlane(kbase) : (uint32_t)kbase;
       const uint32_t k = (uint32_t)k0 + kb + (uint32_t)(i * KSTRIDE);
       const uint32_t c = g.magic_khw ? __umulhi(k, g.magic_khw) : k;        // (multiplier 0: the divisor is 1)
       const uint32_t r = k - c * (uint32_t)(g.kH * g.kW);
       const uint32_t kh = g.magic_kw ? __umulhi(r, g.magic_kw) : r;
       const uint32_t kw = r - kh * (uint32_t)g.kW;
+      const uint32_t koff = c * (uint32_t)g.in_c + kh * (uint32_t)g.in_h + kw * (uint32_t)g.in_w;   // modulo 2^32, like noff
       const bool valid = (!MASK || (int64_t)k < K) && (uint32_t)(ih0 + (int)kh) < (uint32_t)g.H && (uint32_t)(iw0 + (int)kw) < (uint32_t)g.W;
-      const int64_t off = (int64_t)c * g.in_c + (int64_t)kh * g.in_h + (int64_t)kw * g.in_w + noff;
-      reg[S][i] = img[valid ? off : 0];
-      bits |= valid ? (1u << i) : 0u;
+      ok[S][i] = valid;
+      reg[S][i] = *(const T*)(low + (valid ? noff + koff : 0u));
     }
-    ok[S] = bits;
   }
   template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
     constexpr int LD = Slab<T, kGather, BMN, BK>::LDMN;
     const bool none = MASK && k0 >= K;     // nothing was fetched
     const int mn = (int)(threadIdx.x % BMN);
 #pragma unroll
-    for (int i = 0; i < NE; ++i) {
-      const T v = (!none && ((ok[S] >> i) & 1u)) ? reg[S][i] : (T)0;
-      lds[(kbase + i * KSTRIDE) * LD + mn] = v;
-    }
+    for (int i = 0; i < NE; ++i) lds[(kbase + i * KSTRIDE) * LD + mn] = (!none && ok[S][i]) ? reg[S][i] : (T)0;
   }
 };
 

@@ -517,7 +517,7 @@ def conv2d(x: HipTensor, kernel: HipTensor, bias: HipTensor | None = None, paddi
     is_float = x.dtype.kind == "f"
     if fused is None:
         # up to about a hundred output channels the gathered form wins (no column matrix is written and read back);
-        # beyond, the two-launch form's vector loads and larger tiles do (32 x 128 x 28 x 28 -> 128, 3 x 3: 139 against 117 us)
+        # beyond, the two-launch form's vector loads and larger tiles catch up (32 x 128 x 28 x 28 -> 128, 3 x 3: 122 against 116 us)
         fused = is_float and ci * kh * kw * x.dtype.itemsize >= 16 and N <= 65535 and co <= 96
     if fused:
         k = kernel if kernel.reshape(co, ci * kh * kw).strides[1] == 1 else kernel.clone()
