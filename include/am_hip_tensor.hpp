@@ -118,6 +118,16 @@ namespace detail {
   inline int maxpool2d_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW,    \
                         const T* in, T* out, int64_t* idx) {                                              \
     return am_hip_maxpool2d_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, in, out, idx);                      \
+  }                                                                                                      \
+  inline int im2col_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW, const T* in, \
+                     int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, T* col) {                     \
+    return am_hip_im2col_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, col);      \
+  }                                                                                                      \
+  inline int gemm_batched_(int64_t batch, int64_t M, int64_t N, int64_t K, T al, const T* A, int64_t ra, int64_t ca, \
+                           int64_t ba, const T* B, int64_t rb, int64_t cb, int64_t bb, T be, T* C, int64_t rc,     \
+                           int64_t cc, int64_t bc, int epi, const T* bias, int64_t brs, int64_t bcs) {            \
+    return am_hip_gemm_batched_##SFX(batch, M, N, K, al, A, ra, ca, ba, B, rb, cb, bb, be, C, rc, cc, bc, epi,    \
+                                     bias, brs, bcs);                                                      \
   }
 AM_HPP_BIND2(float, f32)
 AM_HPP_BIND2(double, f64)
@@ -140,6 +150,16 @@ inline int gemm_ex_(int64_t M, int64_t N, int64_t K, double al, const double* A,
   return am_hip_gemm_ex_f64(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc, epi, bias, brs, bcs);
 }
 
+inline int conv2d_(int64_t N, int C, int H, int W, int Co, int kH, int kW, int pH, int pW, int sH, int sW, const float* in,
+                   int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, const float* k, int64_t k_rs, int epi,
+                   const float* bias, int64_t bias_s, float* out) {
+  return am_hip_conv2d_f32(N, C, H, W, Co, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, k, k_rs, epi, bias, bias_s, out);
+}
+inline int conv2d_(int64_t N, int C, int H, int W, int Co, int kH, int kW, int pH, int pW, int sH, int sW, const double* in,
+                   int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, const double* k, int64_t k_rs, int epi,
+                   const double* bias, int64_t bias_s, double* out) {
+  return am_hip_conv2d_f64(N, C, H, W, Co, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, k, k_rs, epi, bias, bias_s, out);
+}
 inline int predicate_(int op, int rank, const int64_t* sh, uint8_t* d, const int64_t* sd, const float* a, const int64_t* sa) {
   return am_hip_ew_predicate_f32(op, rank, sh, d, sd, a, sa);
 }
@@ -640,6 +660,51 @@ HipTensor<T> softmax(const HipTensor<T>& t) {
   HipTensor<T> r(t.shape);
   check(detail::softmax_(t.shape[0], t.shape[1], r.ptr(), r.strides[0], r.strides[1], t.ptr(), t.strides[0], t.strides[1]));
   return r;
+}
+
+// conv2d = im2colgemm_conv2d (nn_primitives/fallback/conv.nim:81-106), bias [C_out] or [C_out, 1, 1], optionally
+// followed by relu. Float tensors with `fused`: one launch, the GEMM's B loader gathers the column matrix from the
+// images. Otherwise (integer tensors, or asked for): device im2col of the batch, then one strided-batched GEMM
+// written straight into the NCHW result.
+template <typename T>
+HipTensor<T> conv2d(const HipTensor<T>& x, const HipTensor<T>& kernel, const HipTensor<T>* bias = nullptr, int padH = 0,
+                    int padW = 0, int strideH = 1, int strideW = 1, bool with_relu = false, bool fused = true) {
+  if (x.rank() != 4 || kernel.rank() != 4) throw std::invalid_argument("conv2d: input must be [N, C, H, W], kernel [C_out, C, kH, kW]");
+  if (kernel.shape[1] != x.shape[1])
+    throw std::invalid_argument("conv2d: kernel expects " + std::to_string(kernel.shape[1]) + " input channels, input has " + std::to_string(x.shape[1]));
+  const int64_t N = x.shape[0], C = x.shape[1], H = x.shape[2], W = x.shape[3];
+  const int64_t co = kernel.shape[0], kH = kernel.shape[2], kW = kernel.shape[3], K = C * kH * kW;
+  const int64_t oh = (H + 2 * padH - kH) / strideH + 1, ow = (W + 2 * padW - kW) / strideW + 1, P = oh * ow;
+  if (bias && bias->size() != co) throw std::invalid_argument("conv2d: bias must have one element per output channel");
+  const HipTensor<T> kc = kernel.is_C_contiguous() ? kernel : kernel.clone();
+  int64_t bias_s = 0;
+  if (bias) for (int d = 0; d < bias->rank(); ++d) if (bias->shape[d] == co) { bias_s = bias->strides[d]; break; }
+  constexpr bool F = std::is_floating_point<T>::value;
+  const int epi = F ? ((bias ? AM_EPI_BIAS : 0) | (with_relu ? AM_EPI_RELU : 0)) : AM_EPI_NONE;
+  HipTensor<T> out(Shape{N, co, oh, ow});
+  if (out.size() == 0) return out;
+  if constexpr (F) {
+    if (fused && K * (int64_t)sizeof(T) >= 16 && N <= 65535) {
+      check(detail::conv2d_(N, (int)C, (int)H, (int)W, (int)co, (int)kH, (int)kW, padH, padW, strideH, strideW, x.ptr(), x.strides[0],
+                            x.strides[1], x.strides[2], x.strides[3], kc.ptr(), K, epi, bias ? bias->ptr() : nullptr, bias_s, out.ptr()));
+      return out;
+    }
+  }
+  HipTensor<T> col(Shape{N, K, P});
+  check(detail::im2col_(N, (int)C, (int)H, (int)W, (int)kH, (int)kW, padH, padW, strideH, strideW, x.ptr(), x.strides[0], x.strides[1],
+                        x.strides[2], x.strides[3], col.ptr()));
+  check(detail::gemm_batched_(N, co, P, K, T(1), kc.ptr(), K, 1, 0, col.ptr(), P, 1, K * P, T(0), out.ptr(), P, 1, co * P, epi,
+                              (F && bias) ? bias->ptr() : nullptr, bias_s, 0));
+  if constexpr (!F) {   // integer tensors have no fused epilogue: result +.= bias.unsqueeze(0), then relu
+    if (bias) {
+      HipTensor<T> b3 = *bias;
+      b3.shape = Shape{1, co, 1, 1};
+      b3.strides = Shape{0, bias_s, 0, 0};
+      out.bc_iadd(b3);
+    }
+    if (with_relu) out = unary(AM_UOP_RELU, out);
+  }
+  return out;
 }
 
 // maxpool2d (nnp_maxpooling.nim:19-66): values and the flat input index of each maximum.

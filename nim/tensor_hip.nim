@@ -624,6 +624,25 @@ proc softmax*[T: float32 | float64](input: HipTensor[T]): HipTensor[T] =
     check am_hip_softmax_rows_f64(int64 input.shape[0], int64 input.shape[1], result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
       input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1])
 
+proc conv2d*[T: SomeFloat](input, kernel, bias: HipTensor[T], padding = (0, 0), stride = (1, 1), relu = false): HipTensor[T] =
+  ## im2colgemm_conv2d (nn_primitives/fallback/conv.nim:81-106), optionally followed by relu, in one launch: the GEMM's
+  ## B loader gathers the column matrix from the images. input [N, C, H, W], kernel [C_out, C, kH, kW] (C-contiguous),
+  ## bias [C_out, 1, 1].
+  assert input.rank == 4 and kernel.rank == 4 and kernel.shape[1] == input.shape[1]
+  let kc = if kernel.is_C_contiguous: kernel else: kernel.clone()
+  let (N, C, H, W) = (input.shape[0], input.shape[1], input.shape[2], input.shape[3])
+  let (co, kH, kW) = (kernel.shape[0], kernel.shape[2], kernel.shape[3])
+  let outH = (H + 2 * padding[0] - kH) div stride[0] + 1
+  let outW = (W + 2 * padding[1] - kW) div stride[1] + 1
+  result = newHipTensor[T]([N, co, outH, outW])
+  let epilogue = cint(if relu: AM_EPI_BIAS_RELU else: AM_EPI_BIAS)
+  template call(f: untyped) =
+    check f(int64 N, cint C, cint H, cint W, cint co, cint kH, cint kW, cint padding[0], cint padding[1], cint stride[0], cint stride[1],
+            input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1], int64 input.strides[2], int64 input.strides[3],
+            kc.get_offset_ptr, int64(C * kH * kW), epilogue, bias.get_offset_ptr, int64 bias.strides[0], result.get_offset_ptr)
+  when T is float32: call am_hip_conv2d_f32
+  else: call am_hip_conv2d_f64
+
 proc maxpool2d*[T: HipScalar](input: HipTensor[T], kernel: tuple[height, width: int], padding = (0, 0), stride = (1, 1)):
     tuple[max_indices: HipTensor[int64], maxpooled: HipTensor[T]] =
   ## nn_primitives/nnp_maxpooling.nim:19-66 (the reference asserts a C-contiguous rank-4 input too).

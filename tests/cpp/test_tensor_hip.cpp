@@ -195,6 +195,33 @@ static void argmax_argmin() {
   CHECK(eq(r.first, std::vector<int64_t>{1}) && eq(r.second, {5.0f}) && r.first.shape == (Shape{1, 1}));
 }
 
+template <typename T> static void conv_literals() {
+  // tests/nn_primitives/test_nnp_convolution.nim:21-46 and :54-134: the convolution as one launch (float types) and as
+  // im2col + batched GEMM (every type)
+  {  // simple_pad1
+    auto x = toHip<T>({1, 2, 0, 0, 5, 3, 0, 4, 0, 0, 0, 7, 9, 3, 0, 0}, {1, 1, 4, 4});
+    auto k = toHip<T>({1, 1, 1, 1, 1, 0, 1, 0, 0}, {1, 1, 3, 3});
+    auto b = toHip<T>(std::vector<T>{0}, {1});   // ({0} alone would be a null pointer)
+    const std::vector<T> want = {1, 8, 5, 0, 8, 11, 5, 4, 8, 17, 10, 11, 9, 12, 10, 7};
+    CHECK(eq(am::conv2d(x, k, &b, 1, 1, 1, 1), want));
+    CHECK(eq(am::conv2d(x, k, &b, 1, 1, 1, 1, false, false), want));   // im2col + batched GEMM
+    std::vector<T> clipped = want;
+    for (auto& v : clipped) v = v > T(0) ? v : T(0);
+    CHECK(eq(am::conv2d(x, k, &b, 1, 1, 1, 1, true), clipped));
+  }
+  {  // strided_pad1_stride2
+    auto x = toHip<T>({2, 2, 0, 2, 1, 0, 1, 1, 0, 2, 1, 2, 1, 2, 1, 2, 2, 0, 0, 2, 2, 1, 1, 1, 2, 2, 0, 1, 1, 1, 2, 2, 0, 0, 2, 2, 2, 1, 0, 0, 1, 1, 2, 2, 0, 2, 1, 1, 1, 0, 0, 1, 2, 2, 0, 1, 1, 1, 1, 0, 2, 1, 2, 2, 0, 0, 2, 2, 2, 1, 0, 0, 2, 2, 1}, {1, 3, 5, 5});
+    auto k = toHip<T>({-1, -1, -1, 1, 0, 1, 0, -1, 0, 1, 0, -1, 1, -1, 1, 0, 1, 0, 0, 0, 1, -1, -1, -1, -1, 0, 0, 0, 1, 0, 1, -1, -1, 1, 1, -1, -1, 0, 1, -1, -1, 1, 1, 1, 0, 0, 1, 1, -1, 1, -1, -1, -1, 0}, {2, 3, 3, 3});
+    auto b = toHip<T>({1, 0}, {2});
+    const std::vector<T> want = {2, -2, 0, -3, 2, -5, -2, -1, 0, -7, 1, 0, 3, -3, 2, 1, 3, -2};
+    CHECK(eq(am::conv2d(x, k, &b, 1, 1, 2, 2), want));
+    CHECK(eq(am::conv2d(x, k, &b, 1, 1, 2, 2, false, false), want));   // im2col + batched GEMM
+    std::vector<T> clipped = want;
+    for (auto& v : clipped) v = v > T(0) ? v : T(0);
+    CHECK(eq(am::conv2d(x, k, &b, 1, 1, 2, 2, true), clipped));
+  }
+}
+
 static void maxpool_backward() {
   // tests/nn_primitives/test_nnp_maxpool.nim:20-45
   auto a = toHip<float>({1, 1, 2, 4, 5, 6, 7, 8, 3, 2, 1, 0, 1, 2, 3, 4}, {1, 1, 4, 4});
@@ -378,7 +405,11 @@ int main(int argc, char** argv) {
     variance_std();
     pow_and_universal_functions();
     argmax_argmin();
-    maxpool_backward();
+    conv_literals<float>();
+  conv_literals<double>();
+  conv_literals<int32_t>();
+  conv_literals<int64_t>();
+  maxpool_backward();
     aggregates<float>();
     aggregates<double>();
     aggregates<int32_t>();
