@@ -233,19 +233,20 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     # base-256 digit, so one of the ten digit-pair products runs; entries over the whole int32 range
     # need all ten.
     n = 4096
-    k = max(3, steps // 4)
+    k = max(3, steps // 4)       # launches of the VALU kernels (2.5 - 8 ms each)
+    kd = max(20, steps)          # launches of the digit-sliced products (0.1 - 0.7 ms each)
     peak = ceilings.get("valu_int32_mac")
     for label, lo, hi in (("entries in [-100, 100]", -100, 100), ("entries over the whole int32 range", -2 ** 31, 2 ** 31 - 1)):
         A = np.random.default_rng(2001).integers(lo, hi, (n, n), endpoint=True).astype(np.int32)
         B = np.random.default_rng(2002).integers(lo, hi, (n, n), endpoint=True).astype(np.int32)
         pairs = digit_pairs(A, B)
         dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
-        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, WARM_S)
+        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), kd, 2, WARM_S)
         sclk = timer.sclk_mhz
-        tops = 2.0 * n ** 3 / (ev / k) / 1e12
+        tops = 2.0 * n ** 3 / (ev / kd) / 1e12
         entry = dict(workload=f"i32 GEMM 4096^3, {label} (wraparound; {pairs} of 10 int8 digit-pair products on the matrix cores, "
                               "timed with the two digit-splitting passes)",
-                     unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                     unit="Top/s", dtype="i32", value=round(2.0 * n ** 3 * kd / wall / 1e12, 3), ms_per_step=round(ev / kd * 1e3, 4),
                      roofline=at_clock(dict(bound="mfma", achieved=round(pairs * tops, 1), peak=MFMA_I8_PEAK_TOPS,
                                             unit=f"int8 TOP/s executed ({pairs} digit pairs x 2*M*N*K) over the whole call, two digit-splitting passes included",
                                             frac=round(pairs * tops / MFMA_I8_PEAK_TOPS, 4)), MFMA_I8_PEAK_TOPS, sclk),
@@ -267,7 +268,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
     B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int64)
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int64)
-    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, WARM_S)
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), kd, 2, WARM_S)
     sclk = timer.sclk_mhz
     os.environ["AM_HIP_GEMM_I64_PATH"] = "valu"
     try:
@@ -278,10 +279,10 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     valu_tops = 2.0 * n ** 3 / (ev_valu / 3) / 1e12
     out.append(dict(workload="i64 GEMM 4096^3, entries in [-100, 100] (wraparound; 1 of 36 int8 digit-pair products on the matrix cores, "
                              "timed with the two digit-splitting passes)",
-                    unit="Top/s", dtype="i64", value=round(2.0 * n ** 3 * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
-                    roofline=at_clock(dict(bound="mfma", achieved=round(2.0 * n ** 3 / (ev / k) / 1e12, 1), peak=MFMA_I8_PEAK_TOPS,
+                    unit="Top/s", dtype="i64", value=round(2.0 * n ** 3 * kd / wall / 1e12, 3), ms_per_step=round(ev / kd * 1e3, 4),
+                    roofline=at_clock(dict(bound="mfma", achieved=round(2.0 * n ** 3 / (ev / kd) / 1e12, 1), peak=MFMA_I8_PEAK_TOPS,
                                            unit="int8 TOP/s executed (1 digit pair x 2*M*N*K) over the whole call, two digit-splitting passes included",
-                                           frac=round(2.0 * n ** 3 / (ev / k) / 1e12 / MFMA_I8_PEAK_TOPS, 4)), MFMA_I8_PEAK_TOPS, sclk),
+                                           frac=round(2.0 * n ** 3 / (ev / kd) / 1e12 / MFMA_I8_PEAK_TOPS, 4)), MFMA_I8_PEAK_TOPS, sclk),
                     valu_kernel=dict(value=round(valu_tops, 3), unit="Top/s", ms_per_step=round(ev_valu / 3 * 1e3, 4),
                                      roofline=dict(bound="valu (measured int64 multiply-add ceiling)", achieved=round(valu_tops, 3),
                                                    peak=peak64, unit="Top/s", frac=round(valu_tops / peak64, 4) if peak64 else None))))
