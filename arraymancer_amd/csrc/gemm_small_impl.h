@@ -195,6 +195,164 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   }
 }
 
+// The same product when B has unit stride along n (a row-major [k x n] operand, e.g. x * W with W stored
+// [in x out]): a workgroup owns 16 rows x 16 VN columns (VN = elements per 16 bytes), i.e. VN tiles that share
+// one A fragment. Lane (i, g) reads B[k][n0 + VN i .. n0 + VN i + VN - 1] with one 16-byte load per k and gives
+// element j to tile j, so tile j holds the columns n0 + VN i + j: a permutation of the block's columns under which
+// a lane ends up with VN consecutive columns of each of its rows, stored with one 16-byte store when C has unit
+// stride along n. Against gemm_rows16 on the same operand: a quarter of the load instructions (an eighth for A),
+// 16-byte instead of 64-byte runs on both B and C, and VN independent accumulator chains per wavefront.
+// Requires N % VN == 0 (no vector crosses the end of a row of B).
+template <typename T, bool AVEC, int MAXW, int CHUNK>
+__global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
+  typedef typename M16<T>::acc_t acc_t;
+  constexpr int VN = 16 / (int)sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(VN)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][VN][256] partial tiles, W > 1 only
+  T (*red)[VN * 256] = reinterpret_cast<T (*)[VN * 256]>(red_raw);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int i = lane & 15, g = lane >> 4;
+  const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * (16 * VN);
+  // rows / column vectors past the edge read the last valid one; their results are not stored
+  const int64_t arow = (m0 + i < p.M) ? m0 + i : p.M - 1;
+  const int64_t col0 = n0 + VN * i, bcol = (col0 < p.N) ? col0 : p.N - VN;
+  const T* a = p.A + arow * p.a_mn;
+  const T* b = p.B + bcol;
+
+  const int64_t nfull = p.K >> 4, nblk = (p.K + 15) >> 4;
+  const int64_t per = (nblk + nw - 1) / nw;
+  const int64_t blk0 = (int64_t)wave * per;
+  int64_t blk1 = blk0 + per;
+  if (blk1 > nblk) blk1 = nblk;
+  const int64_t full1 = blk1 < nfull ? blk1 : nfull;
+
+  acc_t acc[VN];
+#pragma unroll
+  for (int j = 0; j < VN; ++j) acc[j] = acc_t{0, 0, 0, 0};
+  const bool has_tail = blk0 <= nfull && nfull < blk1;
+  T tail_a[4] = {0, 0, 0, 0};
+  vec_t tail_b[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) tail_b[s] = vec_t{};
+  if (has_tail) {
+    const int64_t k = (nfull << 4) + 4 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const bool ok = k + s < p.K;
+      const int64_t kk = ok ? k + s : p.K - 1;
+      const T x = a[kk * p.a_k];
+      const vec_t y = *(const vec_t*)(b + kk * p.b_k);
+      tail_a[s] = ok ? x : (T)0;
+      tail_b[s] = ok ? y : vec_t{};
+    }
+  }
+  T av[2][CHUNK][4];
+  vec_t bv[2][CHUNK][4];
+  auto load_blocks = [&](int set, int64_t first_blk, int count) {   // set and count are constants after unrolling
+#pragma unroll
+    for (int u = 0; u < count; ++u) {
+      const int64_t k = ((first_blk + u) << 4) + 4 * g;
+      load4<T, AVEC>(a, p.a_k, k, av[set][u]);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) bv[set][u][s] = *(const vec_t*)(b + (k + s) * p.b_k);
+    }
+  };
+  auto mma_blocks = [&](int set, int count) {
+#pragma unroll
+    for (int u = 0; u < count; ++u)
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int j = 0; j < VN; ++j) acc[j] = M16<T>::mma(av[set][u][s], bv[set][u][s][j], acc[j]);
+  };
+  const int64_t nchunks = (full1 - blk0) / CHUNK;
+  int64_t blk = blk0;
+  if (nchunks > 0) {
+    load_blocks(0, blk0, CHUNK);
+    int64_t c = 0;
+    for (; c + 2 <= nchunks; c += 2) {
+      load_blocks(1, blk0 + (c + 1) * CHUNK, CHUNK);
+      mma_blocks(0, CHUNK);
+      const int64_t nxt = c + 2 < nchunks ? c + 2 : nchunks - 1;   // past the end: a harmless reload
+      load_blocks(0, blk0 + nxt * CHUNK, CHUNK);
+      mma_blocks(1, CHUNK);
+    }
+    if (c < nchunks) mma_blocks(0, CHUNK);
+    blk = blk0 + nchunks * CHUNK;
+  }
+#pragma unroll
+  for (int grp = CHUNK / 2; grp >= 1; grp /= 2) {
+    if (blk + grp <= full1) {
+      load_blocks(0, blk, grp);
+      mma_blocks(0, grp);
+      blk += grp;
+    }
+  }
+  if (has_tail) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int j = 0; j < VN; ++j) acc[j] = M16<T>::mma(tail_a[s], tail_b[s][j], acc[j]);
+  }
+
+  if (nw > 1) {
+#pragma unroll
+    for (int j = 0; j < VN; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][(j * 4 + r) * 64 + lane] = acc[j][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int j = 0; j < VN; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        T sum = red[0][(j * 4 + r) * 64 + lane];
+        for (int w = 1; w < nw; ++w) sum += red[w][(j * 4 + r) * 64 + lane];   // fixed order
+        acc[j][r] = sum;
+      }
+  }
+
+  // Epilogue: the same steps, each rounded on its own, as gemm_rows16 (gemm_ukernel_generic.nim:53-125)
+  const T alpha = p.alpha, beta = p.beta;
+  const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
+  const bool cvec = p.c_n == 1;
+  if (col0 >= p.N) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int64_t row = m0 + M16<T>::acc_row(r, lane);
+    if (row >= p.M) continue;
+    T* c = p.C + row * p.c_m + col0 * p.c_n;
+    vec_t old = vec_t{};
+    if (beta != (T)0) {
+      if (cvec) old = *(const vec_t*)c;
+      else {
+#pragma unroll
+        for (int j = 0; j < VN; ++j) old[j] = c[j * p.c_n];
+      }
+    }
+    vec_t out;
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      T ab = acc[j][r];
+      if (alpha != (T)1) ab = alpha * ab;
+      T v = ab;
+      if (beta != (T)0) {
+        T cc = old[j];
+        if (beta != (T)1) cc = cc * beta;
+        v = cc + ab;
+      }
+      if (has_bias) v = v + p.bias[row * p.bias_m + (col0 + j) * p.bias_n];
+      if (relu) v = ((T)0 >= v) ? (T)0 : v;
+      out[j] = v;
+    }
+    if (cvec) *(vec_t*)c = out;
+    else {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) c[j * p.c_n] = out[j];
+    }
+  }
+}
+
 // Whether this product belongs here: few rows or few columns, little work, not a batch member.
 // AM_HIP_GEMM_SMALL = 0 / 1 in the environment turns the path off / forces it where its limits allow (tests).
 template <typename T>
@@ -220,7 +378,18 @@ static int run(const Args<T>& g_in) {
     g.c_m = g_in.c_n; g.c_n = g_in.c_m;
     g.bias_m = g_in.bias_n; g.bias_n = g_in.bias_m;
   }
-  const int64_t tiles_m = (g.M + 15) / 16, tiles_n = (g.N + 15) / 16;
+  // B with unit stride along n (and no unit stride along k): the kernel whose wavefronts own VK tiles side by side
+  // Measured: it wins (6.1 -> 5.2 us on [20 x 25] * [25 x 36864], 7.9 -> 5.8 on [16 x 64] * [64 x 65536], float64 15.2 -> 9.1
+  // on [64 x 256] * [256 x 8192]) where its fewer, wider tiles still give every SIMD of the chip a wavefront, and loses
+  // below that (a wavefront's chain of load round trips is what such a product costs, and fewer wavefronts means longer
+  // chains). AM_HIP_GEMM_SMALL_NVEC = 0 / 2 in the environment turns it off / forces it where it is legal (tests).
+  const char* nv = getenv("AM_HIP_GEMM_SMALL_NVEC");
+  const int nvec_mode = (nv && *nv) ? atoi(nv) : 1;
+  const bool nvec_legal = g.b_mn == 1 && g.b_k != 1 && g.N % VK == 0 && g.N >= 8 * VK;
+  const bool nvec = nvec_legal && nvec_mode != 0 &&
+                    (nvec_mode == 2 || ((g.M + 15) / 16) * ((g.N + 16 * VK - 1) / (16 * VK)) >= (int64_t)num_cus() * 4);
+  const int64_t tile_cols = nvec ? 16 * VK : 16;
+  const int64_t tiles_m = (g.M + 15) / 16, tiles_n = (g.N + tile_cols - 1) / tile_cols;
   if (tiles_n >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "gemm: too many tiles");
   // Wavefronts per tile: about one per SIMD over the chip and at most four (measured: starting more
   // wavefronts costs more than the latency they would hide), every one with at least two blocks of 16 k.
@@ -230,7 +399,7 @@ static int run(const Args<T>& g_in) {
   int nw = 1;
   while (nw * 2 <= want && nw * 2 <= kMaxWaves) nw *= 2;
   if (const char* e = getenv("AM_HIP_GEMM_SMALL_W")) { const int w = atoi(e); if (w >= 1 && w <= kMaxWaves) nw = w; }   // tests
-  const size_t lds = nw > 1 ? (size_t)nw * 256 * sizeof(T) : 0;
+  const size_t lds = nw > 1 ? (size_t)nw * 256 * sizeof(T) * (nvec ? VK : 1) : 0;
   const bool avec = g.a_k == 1 && aligned16(g.A) && (g.a_mn % VK == 0 || g.M == 1);
   const bool bvec = g.b_k == 1 && aligned16(g.B) && (g.b_mn % VK == 0 || g.N == 1);
   const dim3 grid((unsigned)tiles_n, (unsigned)tiles_m), block((unsigned)nw * 64);
@@ -240,6 +409,18 @@ static int run(const Args<T>& g_in) {
   // so all the wavefronts of a product with many tiles and a short k are resident at once.
   constexpr int CH = sizeof(T) == 4 ? 4 : 2;
   const bool short_k = (nblk + nw - 1) / nw <= 2;
+  if (nvec) {
+    if (trace_choices()) fprintf(stderr, "am_hip gemm: small path, B in 16-byte vectors along n\n");
+    constexpr int CHN = 2;
+    if (short_k) {
+      if (avec) hipLaunchKernelGGL((gemm_rows16n<T, true, kMaxWaves, 1>), grid, block, lds, stream(), g);
+      else hipLaunchKernelGGL((gemm_rows16n<T, false, kMaxWaves, 1>), grid, block, lds, stream(), g);
+    } else {
+      if (avec) hipLaunchKernelGGL((gemm_rows16n<T, true, kMaxWaves, CHN>), grid, block, lds, stream(), g);
+      else hipLaunchKernelGGL((gemm_rows16n<T, false, kMaxWaves, CHN>), grid, block, lds, stream(), g);
+    }
+    return check_launch("gemm_rows16n");
+  }
 #define AM_SMALL_LAUNCH(AV, BV)                                                                              \
   do {                                                                                                       \
     if (short_k) hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, 1>), grid, block, lds, stream(), g);   \

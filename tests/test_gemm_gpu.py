@@ -764,15 +764,20 @@ def test_digit_path_window_views(hip, oracle, sfx, monkeypatch):
 
 
 SMALL_SHAPES = [(1, 1, 1), (20, 36864 // 64, 25), (50, 300, 500), (64, 500, 800), (64, 10, 500), (7, 33, 15), (16, 16, 16),
-                (17, 47, 17), (64, 64, 4099), (33, 200, 1000), (3, 5, 8191), (500, 10, 64), (4096, 3, 129), (300, 64, 77)]
+                (17, 47, 17), (64, 64, 4099), (33, 200, 1000), (3, 5, 8191), (500, 10, 64), (4096, 3, 129), (300, 64, 77),
+                (37, 132, 40), (9, 70, 33), (16, 1028, 16)]
 
 
+@pytest.mark.parametrize("nvec", ["0", "2"])
 @pytest.mark.parametrize("sfx", ["f32", "f64"])
-def test_small_row_path(hip, oracle, sfx, monkeypatch):
+def test_small_row_path(hip, oracle, sfx, nvec, monkeypatch):
     """Products with at most 64 rows or columns on the kernel that loads matrix-instruction operands
     straight from global memory (forced on): every k tail (K < 16, K % 16 != 0, K % 4 != 0), ragged
     M and N, one to four wavefronts per tile, both orientations, every alpha / beta case, against
-    the oracle and against the tiled kernel on the same inputs."""
+    the oracle and against the tiled kernel on the same inputs. nvec: the variant for a B with unit
+    stride along n (16-byte loads along n, several tiles per wavefront) switched off / forced wherever
+    the operand allows it."""
+    monkeypatch.setenv("AM_HIP_GEMM_SMALL_NVEC", nvec)
     dt = DTYPES[sfx]
     eps = np.finfo(dt).eps
     rng = np.random.default_rng(seed_of("small", sfx))
@@ -809,11 +814,13 @@ def test_small_row_path(hip, oracle, sfx, monkeypatch):
     assert np.isfinite(dC.toCpu()).all()
 
 
+@pytest.mark.parametrize("nvec", ["0", "2"])
 @pytest.mark.parametrize("sfx", ["f32", "f64"])
-def test_small_row_path_views_and_epilogue(hip, oracle, sfx, monkeypatch):
-    """The same kernel on transposed, stepped, reversed and broadcast operands, strided and
+def test_small_row_path_views_and_epilogue(hip, oracle, sfx, nvec, monkeypatch):
+    """The same kernels on transposed, stepped, reversed and broadcast operands, strided and
     column-major destinations, and with the fused bias / ReLU epilogue (row and column bias)."""
     monkeypatch.setenv("AM_HIP_GEMM_SMALL", "1")
+    monkeypatch.setenv("AM_HIP_GEMM_SMALL_NVEC", nvec)
     dt = DTYPES[sfx]
     rng = np.random.default_rng(seed_of("small-views", sfx))
     for (M, N, K) in [(64, 500, 800), (20, 300, 25), (50, 96, 500), (300, 20, 123)]:
