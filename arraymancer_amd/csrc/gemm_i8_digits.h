@@ -549,15 +549,42 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
 // The estimate is for operands that use every digit; the kernel itself skips empty planes.
 // Estimated times of the digit path in microseconds: the two splitting passes, the product kernel with
 // every digit pair live (main_us, of which fixed_us do not depend on the number of pairs), and their sum.
-struct Plan { int64_t Mp, Np, Kp; bool big; double est_us, main_us, fixed_us, first_us, second_us; };
+struct Plan { int64_t Mp, Np, Kp; int tile; double est_us, main_us, fixed_us, first_us, second_us; };
 
-// Time of the product kernel for `tiles` workgroup tiles, one per CU and round. A tile's time per k
-// grows with the share of the chip that is busy (the tiles compete for L2 and fabric bandwidth):
-// c0 * (1 + a * load^2), fitted to kernel times at 512^3 ... 4096^3 with all pairs live.
-static inline double main_us_per_k(int64_t tiles, int64_t cus, double c0, double a) {
-  const int64_t full = tiles / cus, rem = tiles - full * cus;
-  const double load = (double)rem / (double)cus;
-  return (double)full * c0 * (1.0 + a) + (rem ? c0 * (1.0 + a * load * load) : 0.0);
+// Workgroup tiles of the product kernel: 256 x 128 (8 wavefronts of 64 x 64), 256 x 256 (8 of 128 x 64: fewest LDS
+// reads per matrix instruction; int32 only, the 64-bit accumulators of int64 leave no registers for it), 128 x 128
+// (8 of 64 x 32) and 64 x 64 (4 of 32 x 32) for products that the large tiles spread over a fraction of the chip.
+constexpr int kTileCount = 4;
+constexpr int kTileRows[kTileCount] = {256, 256, 128, 64}, kTileCols[kTileCount] = {128, 256, 128, 64};
+static inline const char* tile_name(int t) { static const char* n[kTileCount] = {"256x128", "256x256", "128x128", "64x64"}; return n[t]; }
+
+// Microseconds per k (all digit pairs live) of the product kernel for `tiles` workgroup tiles, fitted to kernel times
+// (rocprofv3) at 512^3 ... 4096^3. `slots` workgroups of a tile shape share a CU (LDS: 128 / 64 / 32 KiB per workgroup
+// for the two large, the 128 x 128 and the 64 x 64 tile). Whole rounds of slots x CUs tiles take c_full each. A last,
+// partial round of r tiles: up to one per CU a tile's time grows with the share of the chip that is busy (the tiles
+// compete for L2 and fabric bandwidth), c0 (1 + a (r / CUs)^2); from there to a whole round it grows linearly to c_full.
+struct TileFit { double c0, a, c_full; int slots; };
+static inline TileFit tile_fit(int tile, bool wide) {
+  //                                           256 x 128                256 x 256               128 x 128                64 x 64
+  static const TileFit i32[kTileCount] = {{0.048, 0.58, 0.076, 1}, {0.090, 0.34, 0.121, 1}, {0.029, 0.31, 0.0755, 2}, {0.0215, 0.0, 0.059, 4}};
+  static const TileFit i64[kTileCount] = {{0.205, 0.42, 0.291, 1}, {0.0, 0.0, 0.0, 1}, {0.118, 0.30, 0.296, 2}, {0.083, 0.0, 0.231, 4}};
+  return wide ? i64[tile] : i32[tile];
+}
+static inline double main_us_per_k(int tile, bool wide, int64_t tiles, int64_t cus) {
+  const TileFit f = tile_fit(tile, wide);
+  const int64_t round = cus * f.slots, full = tiles / round, r = tiles - full * round;
+  double us = (double)full * f.c_full;
+  if (r > 0) {
+    const double one_per_cu = f.c0 * (1.0 + f.a);
+    if (r <= cus) { const double load = (double)r / (double)cus; us += f.c0 * (1.0 + f.a * load * load); }
+    else us += one_per_cu + (f.c_full - one_per_cu) * (double)(r - cus) / (double)(round - cus);
+  }
+  return us;
+}
+// Launch, prologue (pair table, filling the ring) and the store of the result.
+static inline double fixed_us(int tile, bool wide, double c_bytes) {
+  static const double base[kTileCount] = {11.0, 13.0, 8.0, 5.5};
+  return base[tile] + c_bytes / (wide ? 1.0e7 : 6.0e6);
 }
 
 template <typename T>
@@ -568,20 +595,21 @@ static inline Plan plan(const Args<T>& g) {
   pl.Np = (g.N + kRowPad - 1) / kRowPad * kRowPad;
   pl.Kp = (g.K + kKPad - 1) / kKPad * kKPad;
   const int64_t cus = num_cus();
-  const int64_t tb = (pl.Mp / 256) * (pl.Np / 256), ts = (pl.Mp / 256) * (pl.Np / 128);
-  // microseconds per k of one tile on an otherwise idle chip (c0) and its growth to a full chip (a).
-  // int32 (ten pairs): 256 x 128 tiles 0.054 -> 0.089, 256 x 256 tiles 0.093 -> 0.157;
-  // int64 (36 pairs, 256 x 128 only: the 64-bit accumulators leave no registers for the larger tile): 0.205 -> 0.29.
-  const double cost_big = main_us_per_k(tb, cus, 0.093, 0.69) * pl.Kp;
-  const double cost_small = main_us_per_k(ts, cus, WIDE ? 0.205 : 0.054, WIDE ? 0.42 : 0.65) * pl.Kp;
-  pl.big = !WIDE && cost_big <= cost_small;
-  if (!WIDE) {
-    const char* force = getenv("AM_HIP_GEMM_TILE_I8");   // 1: 256 x 256 tiles, 0: 256 x 128 (tests)
-    if (force && *force) pl.big = atoi(force) != 0;
+  const double c_bytes = (double)g.M * (double)g.N * sizeof(T);
+  int best = 0;
+  double best_us = 0.0;
+  for (int t = 0; t < kTileCount; ++t) {
+    if (WIDE && t == 1) continue;
+    const int64_t tiles = (pl.Mp / kTileRows[t]) * (pl.Np / kTileCols[t]);
+    const double us = fixed_us(t, WIDE, c_bytes) + main_us_per_k(t, WIDE, tiles, cus) * (double)pl.Kp;
+    if (t == 0 || us < best_us) { best = t; best_us = us; }
   }
-  // launch, pair table, the result's round trip (int64: one widening per pair on top)
-  pl.fixed_us = WIDE ? 15.0 : 5.0;
-  pl.main_us = pl.fixed_us + (pl.big ? cost_big : cost_small);
+  if (const char* force = getenv("AM_HIP_GEMM_TILE_I8")) {   // tests: 0 ... 3, see kTileRows / kTileCols
+    if (*force) { const int t = atoi(force); if (t >= 0 && t < kTileCount && !(WIDE && t == 1)) best = t; }
+  }
+  pl.tile = best;
+  pl.fixed_us = fixed_us(best, WIDE, c_bytes);
+  pl.main_us = pl.fixed_us + main_us_per_k(best, WIDE, (pl.Mp / kTileRows[best]) * (pl.Np / kTileCols[best]), cus) * (double)pl.Kp;
   // The first pass reads every element and writes its lowest digit; the second reads it again (mostly
   // from the memory-side cache) and writes the other planes.
   const double elems = (double)(pl.Mp + pl.Np) * pl.Kp, sz = (double)sizeof(T);
@@ -614,9 +642,8 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
                uint32_t* gate_gen = nullptr) {
   constexpr int ND = (int)sizeof(T);
   const int64_t Mp = pl.Mp, Np = pl.Np, Kp = pl.Kp;
-  const bool big = pl.big;   // 256 x 256 tiles: a 128 x 64 tile per wavefront, fewest LDS reads per matrix instruction
   if (Mp / 32 >= ((int64_t)1 << 31) || Np / 32 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return 1;
-  const int64_t tiles_m = Mp / 256, tiles_n = big ? Np / 256 : Np / 128;
+  const int64_t tiles_m = Mp / kTileRows[pl.tile], tiles_n = Np / kTileCols[pl.tile];
   if (tiles_m * tiles_n >= ((int64_t)1 << 31)) return 1;
   // Flag words live as long as the process: every product uses a new generation number, so they are
   // cleared only once (and again should the 32-bit counter ever wrap).
@@ -665,12 +692,14 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N; d.clock_out = g.clock_out;
   d.alpha = g.alpha; d.beta = g.beta;
   d.tiles_m = (int)tiles_m; d.tiles_n = (int)tiles_n;
-  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
-  if constexpr (sizeof(T) == 8) {
-    hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 4>), grid, block, 0, stream(), d);
-  } else {
-    if (big) hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 4, 2, 64, 4>), grid, block, 0, stream(), d);
-    else hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 4>), grid, block, 0, stream(), d);
+  const dim3 grid((unsigned)(tiles_m * tiles_n));
+  switch (pl.tile) {
+    case 1:
+      if constexpr (sizeof(T) == 4) { hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 4, 2, 64, 4>), grid, dim3(512), 0, stream(), d); break; }
+      [[fallthrough]];   // int64 has no 256 x 256 tile (plan() never picks it)
+    default: hipLaunchKernelGGL((gemm_i8_digits<T, 4, 2, 2, 2, 64, 4>), grid, dim3(512), 0, stream(), d); break;
+    case 2: hipLaunchKernelGGL((gemm_i8_digits<T, 2, 4, 2, 1, 64, 4>), grid, dim3(512), 0, stream(), d); break;
+    case 3: hipLaunchKernelGGL((gemm_i8_digits<T, 2, 2, 1, 1, 64, 4>), grid, dim3(256), 0, stream(), d); break;
   }
   const int rc = check_launch("gemm_i8_digits");
   // The planes go back to the allocator's cache at once: whoever gets the block next reaches it
@@ -697,7 +726,7 @@ static int try_digits(Args<T>& g, double valu_est_us, int* rc) {
   // (fitted to the same sizes as the digit path's model).
   const double valu_us = (sizeof(T) == 8 ? 1.15 : 1.3) * valu_est_us + 5.0;
   if (may == 2 || (may == 1 && pl.est_us < 1.1 * valu_us)) {
-    if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path, %s tiles, est %.1f us (VALU est %.1f us)\n", pl.big ? "256x256" : "256x128", pl.est_us, valu_us);
+    if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path, %s tiles, est %.1f us (VALU est %.1f us)\n", tile_name(pl.tile), pl.est_us, valu_us);
     const int r = run(g, pl);
     if (r <= 0) { *rc = r; return 0; }
     return 1;   // no scratch memory for the digit planes

@@ -587,10 +587,11 @@ def test_integer_mid_size_balanced_split(hip, oracle, sfx):
         assert np.array_equal(dC.toCpu(), oracle.matmul(A, B))
 
 
-@pytest.mark.parametrize("tile", ["0", "1"])
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3"])
 def test_int32_digit_sliced_matrix_core_path(hip, oracle, tile, monkeypatch):
     """int32 products on the int8 matrix cores (four balanced base-256 digits, ten digit-pair
-    products, Horner recombination modulo 2^32), forced on for every shape and both tile shapes:
+    products, Horner recombination modulo 2^32), forced on for every shape and all four tile shapes
+    (256 x 128, 256 x 256, 128 x 128, 64 x 64):
     digit boundaries (±127, ±128, ±129 in every byte position), INT_MIN / INT_MAX, full-range random
     values with long K (accumulators wrap many times), ragged M / N / K, strided and transposed
     operands, column-major and strided destinations, every alpha / beta case. Bit-exact."""
@@ -647,13 +648,15 @@ def test_int32_paths_agree_at_size(hip, oracle, monkeypatch):
             assert np.array_equal((dA * dB).toCpu(), want), f"{shape} path {path}"
 
 
-def test_int64_digit_sliced_matrix_core_path(hip, oracle, monkeypatch):
+@pytest.mark.parametrize("tile", ["0", "2", "3"])
+def test_int64_digit_sliced_matrix_core_path(hip, oracle, tile, monkeypatch):
     """int64 products on the int8 matrix cores (eight balanced base-256 digits, 36 digit-pair
     products, each pair's exact 32-bit sums widened to 64 bits before the Horner shifts), forced on
-    for every shape: digit boundaries in every byte position, INT64_MIN / INT64_MAX, full-range
+    for every shape and each of its three tile shapes (256 x 128, 128 x 128, 64 x 64): digit boundaries in every byte position, INT64_MIN / INT64_MAX, full-range
     random values, ragged M / N / K, strided and transposed operands and destinations, every
     alpha / beta case. Bit-exact."""
     monkeypatch.setenv("AM_HIP_GEMM_I64_PATH", "mfma")
+    monkeypatch.setenv("AM_HIP_GEMM_TILE_I8", tile)
     dt = np.int64
     info = np.iinfo(dt)
     base = [0, 1, -1, 127, 128, 129, -127, -128, -129, 255, 256, -255, -256, 32767, 32768, -32768, -32769]
@@ -663,10 +666,10 @@ def test_int64_digit_sliced_matrix_core_path(hip, oracle, monkeypatch):
         edge += [sgn * (v << (8 * byte)) + off for sgn in (1, -1) for v in (127, 128, 129) for off in (0, 127, -128)
                  if info.min <= sgn * (v << (8 * byte)) + off <= info.max]
     edge = np.array(edge, dtype=dt)
-    rng = np.random.default_rng(seed_of("digits64"))
+    rng = np.random.default_rng(seed_of("digits64", tile))
     for shape in [(30, 30, 30), (1, 1, 1), (257, 129, 300), (64, 500, 1000), (300, 257, 4099), (513, 511, 129)]:
         M, N, K = shape
-        say("int64 digit path", shape)
+        say("int64 digit path", tile, shape)
         A = rng.choice(edge, size=(M, K)) if K <= 300 else fill(rng, (M, K), dt, info.min, info.max)
         B = rng.choice(edge, size=(K, N)) if K <= 300 else fill(rng, (K, N), dt, info.min, info.max)
         C = fill(rng, (M, N), dt, info.min, info.max)
