@@ -44,8 +44,8 @@ namespace am {
 namespace gemm {
 namespace i8 {
 
-constexpr int kRowPad = 256;   // operand planes are padded to this many rows (largest tile edge) ...
-constexpr int kKPad = 256;     // ... and to this many k (a whole turn of the LDS ring: four slabs of 64)
+constexpr int kKPad = 256;     // operand planes are padded to a multiple of the workgroup tile in rows and to this many k
+                               // (a whole turn of the LDS ring: four slabs of 64)
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -591,25 +591,27 @@ template <typename T>
 static inline Plan plan(const Args<T>& g) {
   constexpr bool WIDE = sizeof(T) == 8;
   Plan pl;
-  pl.Mp = (g.M + kRowPad - 1) / kRowPad * kRowPad;
-  pl.Np = (g.N + kRowPad - 1) / kRowPad * kRowPad;
   pl.Kp = (g.K + kKPad - 1) / kKPad * kKPad;
   const int64_t cus = num_cus();
   const double c_bytes = (double)g.M * (double)g.N * sizeof(T);
+  // rows and columns are padded to the chosen tile only (1280 is 20 tiles of 64, not 24)
+  auto padded = [](int64_t x, int64_t to) { return (x + to - 1) / to * to; };
+  auto tiles_of = [&](int t) { return (padded(g.M, kTileRows[t]) / kTileRows[t]) * (padded(g.N, kTileCols[t]) / kTileCols[t]); };
   int best = 0;
   double best_us = 0.0;
   for (int t = 0; t < kTileCount; ++t) {
     if (WIDE && t == 1) continue;
-    const int64_t tiles = (pl.Mp / kTileRows[t]) * (pl.Np / kTileCols[t]);
-    const double us = fixed_us(t, WIDE, c_bytes) + main_us_per_k(t, WIDE, tiles, cus) * (double)pl.Kp;
+    const double us = fixed_us(t, WIDE, c_bytes) + main_us_per_k(t, WIDE, tiles_of(t), cus) * (double)pl.Kp;
     if (t == 0 || us < best_us) { best = t; best_us = us; }
   }
   if (const char* force = getenv("AM_HIP_GEMM_TILE_I8")) {   // tests: 0 ... 3, see kTileRows / kTileCols
     if (*force) { const int t = atoi(force); if (t >= 0 && t < kTileCount && !(WIDE && t == 1)) best = t; }
   }
   pl.tile = best;
+  pl.Mp = padded(g.M, kTileRows[best]);
+  pl.Np = padded(g.N, kTileCols[best]);
   pl.fixed_us = fixed_us(best, WIDE, c_bytes);
-  pl.main_us = pl.fixed_us + main_us_per_k(best, WIDE, (pl.Mp / kTileRows[best]) * (pl.Np / kTileCols[best]), cus) * (double)pl.Kp;
+  pl.main_us = pl.fixed_us + main_us_per_k(best, WIDE, tiles_of(best), cus) * (double)pl.Kp;
   // The first pass reads every element and writes its lowest digit; the second reads it again (mostly
   // from the memory-side cache) and writes the other planes.
   const double elems = (double)(pl.Mp + pl.Np) * pl.Kp, sz = (double)sizeof(T);
