@@ -407,6 +407,7 @@ template <typename T, typename D = T> struct TiledArgs {
   int64_t a0, a1, b0, b1;       // operand strides
   int a_t, b_t;                 // operand has unit stride along axis 0: go through LDS
   int tiles_c;
+  int tiles_r, stream;          // vector kernel: tile rows; non-temporal loads (operands beyond what the caches hold)
 };
 
 template <typename T, typename D, int CODE, bool BCONST, bool SWAP>
@@ -447,6 +448,171 @@ __global__ __launch_bounds__(256) void ew_tiled(TiledArgs<T, D> p) {
       else y = p.b_t ? tb[tx][rl] : p.b[r * p.b0 + c * p.b1];
       p.dst[r * p.d0 + c] = (D)(SWAP ? Op::apply(y, x) : Op::apply(x, y));
     }
+  }
+}
+
+// The same scheme for operands and results of one width whose runs are 16-byte aligned, at full memory speed:
+// tiles of 512 bytes x 512 bytes (128 x 128 four-byte, 64 x 64 eight-byte elements: a wavefront's access is then two
+// whole 512-byte runs instead of one of 256 bytes), 16-byte global loads and stores, all of a tile's loads issued before
+// the first is needed, non-temporal stores (and loads, beyond what the caches hold), and tiles numbered in bands of
+// eight tile rows walked column by column, so that the workgroups running at the same time read and write neighbouring
+// runs (4 KiB of every touched row of the transposed operand together, instead of 512 bytes each 8192 columns apart).
+// Measured, clone of a transposed 8192 x 8192 float32 view, every byte from HBM: 64 x 64 tiles with element accesses
+// 125 us, this form 95 us = 5.6 TB/s against 86 us for a plain copy. A tile that reaches over the edge takes the
+// element-wise path of the same layout. LDS rows are padded by one vector: rows stay 16-byte aligned for the
+// output's vector reads; the transposing writes then conflict on banks, which costs nothing measurable here
+// (an XOR swizzle without conflicts ran at the same speed).
+// Bodies whose library code keeps a table in private memory (the argument reduction of sin / cos / tan, gamma) stay on
+// the element kernel: there the table lives in registers; here, beside a tile's worth of loads, it goes to scratch.
+constexpr bool tiled_vec_body(int code) {
+  return !(code == kUnaryBase + AM_UOP_SIN || code == kUnaryBase + AM_UOP_COS || code == kUnaryBase + AM_UOP_TAN ||
+           code == kUnaryBase + AM_UOP_GAMMA);
+}
+
+template <typename T> struct Tile2dVec {
+  static constexpr int TS = 512 / (int)sizeof(T), VEC = 16 / (int)sizeof(T), LD = TS + VEC;
+  static constexpr int Q = TS / VEC, RPP = 256 / Q, PASSES = TS / RPP;
+  static constexpr size_t kTileBytes = (size_t)TS * LD * sizeof(T);
+};
+
+template <typename T, int CODE, bool BCONST, bool SWAP>
+__global__ __launch_bounds__(256) void ew_tiled_vec(TiledArgs<T, T> p) {
+  typedef typename OpSel<T, CODE>::type Op;
+  typedef Tile2dVec<T> G;
+  constexpr int TS = G::TS, VEC = G::VEC, LD = G::LD, Q = G::Q, RPP = G::RPP, PASSES = G::PASSES;
+  typedef T V __attribute__((ext_vector_type(VEC)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char tile_mem[];
+  T* ta = reinterpret_cast<T*>(tile_mem);
+  T* tb = ta + (p.a_t ? TS * LD : 0);
+  const int band = blockIdx.x / (8 * p.tiles_c), in = blockIdx.x - band * 8 * p.tiles_c;
+  const int h = p.tiles_r - 8 * band < 8 ? p.tiles_r - 8 * band : 8;
+  const int tile_r = 8 * band + in % h, tile_c = in / h;
+  const int64_t r0 = (int64_t)tile_r * TS, c0 = (int64_t)tile_c * TS;
+  const bool b_t = !BCONST && p.b_t;
+
+  if (r0 + TS > p.R || c0 + TS > p.C) {   // a tile over the edge: one element at a time, same layout
+    const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
+    constexpr int STEP = 256 / TS;
+    for (int cl = ty; cl < TS; cl += STEP) {
+      const int64_t r = r0 + tx, c = c0 + cl;
+      if (r < p.R && c < p.C) {
+        if (p.a_t) ta[tx * LD + cl] = p.a[r + c * p.a1];
+        if (b_t) tb[tx * LD + cl] = p.b[r + c * p.b1];
+      }
+    }
+    __syncthreads();
+    for (int rl = ty; rl < TS; rl += STEP) {
+      const int64_t r = r0 + rl, c = c0 + tx;
+      if (r < p.R && c < p.C) {
+        const T x = p.a_t ? ta[rl * LD + tx] : p.a[r * p.a0 + c * p.a1];
+        T y;
+        if constexpr (BCONST) y = p.scalar;
+        else y = b_t ? tb[rl * LD + tx] : p.b[r * p.b0 + c * p.b1];
+        p.dst[r * p.d0 + c] = SWAP ? Op::apply(y, x) : Op::apply(x, y);
+      }
+    }
+    return;
+  }
+
+  const int q = threadIdx.x % Q, rr = threadIdx.x / Q;
+  V va[PASSES], vb[BCONST ? 1 : PASSES];
+  // the transposed operands: lane (q, rr) reads VEC elements along axis 0 of column c0 + rr + RPP pass
+  if (p.a_t) {
+    const T* src = p.a + r0 + VEC * q + (c0 + rr) * p.a1;
+    if (p.stream) {
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i) va[i] = __builtin_nontemporal_load(launder((const V*)(src + (int64_t)i * RPP * p.a1)));
+    } else {
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i) va[i] = *(const V*)(src + (int64_t)i * RPP * p.a1);
+    }
+  }
+  if constexpr (!BCONST) {
+    if (b_t) {
+      const T* src = p.b + r0 + VEC * q + (c0 + rr) * p.b1;
+      if (p.stream) {
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) vb[i] = __builtin_nontemporal_load(launder((const V*)(src + (int64_t)i * RPP * p.b1)));
+      } else {
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) vb[i] = *(const V*)(src + (int64_t)i * RPP * p.b1);
+      }
+    }
+  }
+  if (p.a_t) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) ta[(VEC * q + j) * LD + rr + i * RPP] = va[i][j];
+  }
+  if constexpr (!BCONST) {
+    if (b_t) {
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) tb[(VEC * q + j) * LD + rr + i * RPP] = vb[i][j];
+    }
+  }
+  __syncthreads();
+  // output: lane (q, rr) owns VEC consecutive columns of row r0 + rr + RPP pass; operands laid out like the result are
+  // read here (unit stride along axis 1: a vector; stride 0: one value for the row)
+  const int64_t col = c0 + VEC * q;
+  if (!p.a_t) {
+    if (p.a1 == 1) {
+      const T* src = p.a + (r0 + rr) * p.a0 + col;
+      if (p.stream) {
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) va[i] = __builtin_nontemporal_load(launder((const V*)(src + (int64_t)i * RPP * p.a0)));
+      } else {
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) va[i] = *(const V*)(src + (int64_t)i * RPP * p.a0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i) {
+        const T x = p.a[(r0 + rr + i * RPP) * p.a0];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) va[i][j] = x;
+      }
+    }
+  }
+  if constexpr (!BCONST) {
+    if (!b_t) {
+      if (p.b1 == 1) {
+        const T* src = p.b + (r0 + rr) * p.b0 + col;
+        if (p.stream) {
+#pragma unroll
+          for (int i = 0; i < PASSES; ++i) vb[i] = __builtin_nontemporal_load(launder((const V*)(src + (int64_t)i * RPP * p.b0)));
+        } else {
+#pragma unroll
+          for (int i = 0; i < PASSES; ++i) vb[i] = *(const V*)(src + (int64_t)i * RPP * p.b0);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+          const T y = p.b[(r0 + rr + i * RPP) * p.b0];
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) vb[i][j] = y;
+        }
+      }
+    }
+  }
+  T* out = p.dst + (r0 + rr) * p.d0 + col;
+#pragma unroll
+  for (int i = 0; i < PASSES; ++i) {
+    const int rl = rr + i * RPP;
+    const V x = p.a_t ? *(const V*)&ta[rl * LD + VEC * q] : va[i];
+    V y;
+    if constexpr (BCONST) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) y[j] = p.scalar;
+    } else {
+      y = b_t ? *(const V*)&tb[rl * LD + VEC * q] : vb[i];
+    }
+    V res;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) res[j] = SWAP ? Op::apply(y[j], x[j]) : Op::apply(x[j], y[j]);
+    __builtin_nontemporal_store(res, (V*)(out + (int64_t)i * RPP * p.d0));
   }
 }
 
@@ -706,6 +872,33 @@ static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const 
         const bool a_ok = direct(t.a1) || t.a_t, b_ok = BCONST || direct(t.b1) || t.b_t;
         const int64_t tr = (t.R + kTile2d - 1) / kTile2d, tc = (t.C + kTile2d - 1) / kTile2d;
         if (a_ok && b_ok && (t.a_t || t.b_t || ax == 0) && tr * tc < ((int64_t)1 << 31) && t.R >= 16 && t.C >= 16) {
+          if constexpr (std::is_same_v<T, D> && tiled_vec_body(CODE)) {
+            // 16-byte runs everywhere and at least one whole tile each way: the vector form
+            typedef Tile2dVec<T> G;
+            auto vec_ok = [&](const void* base, int64_t s_axis0, int64_t s_axis1, bool transposed) {
+              if (transposed) return aligned16(base) && s_axis1 % VEC == 0;
+              if (s_axis1 == 1) return aligned16(base) && s_axis0 % VEC == 0;
+              return s_axis1 == 0;
+            };
+            static const bool tiled_vec_on = [] { const char* e = getenv("AM_HIP_EW_TILED_VEC"); return !(e && *e == '0'); }();
+            if (tiled_vec_on && t.R >= G::TS && t.C >= G::TS && aligned16(dst) && t.d0 % VEC == 0 && vec_ok(a, t.a0, t.a1, t.a_t != 0) &&
+                (BCONST || vec_ok(b, t.b0, t.b1, t.b_t != 0))) {
+              const int64_t vr = (t.R + G::TS - 1) / G::TS, vc = (t.C + G::TS - 1) / G::TS;
+              t.tiles_r = (int)vr; t.tiles_c = (int)vc;
+              const double bytes = (double)t.R * (double)t.C * sizeof(T) * (BCONST ? 1.0 : 2.0);
+              t.stream = bytes > nt_threshold_bytes() ? 1 : 0;
+              const size_t lds = G::kTileBytes * (size_t)((t.a_t ? 1 : 0) + (t.b_t ? 1 : 0));
+              auto kernel = ew_tiled_vec<T, CODE, BCONST, SWAP>;
+              static bool lds_set = false;   // one flag per instantiation: more than 64 KiB of dynamic LDS has to be asked for
+              if (!lds_set) {
+                if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * G::kTileBytes)) != hipSuccess)
+                  return fail(AM_E_HIP, "hipFuncSetAttribute(ew_tiled_vec) failed");
+                lds_set = true;
+              }
+              hipLaunchKernelGGL(kernel, dim3((unsigned)(vr * vc)), dim3(256), lds, stream(), t);
+              return check_launch("ew_tiled_vec");
+            }
+          }
           t.tiles_c = (int)tc;
           hipLaunchKernelGGL((ew_tiled<T, D, CODE, BCONST, SWAP>), dim3((unsigned)(tr * tc)), dim3(256), 0, stream(), t);
           return check_launch("ew_tiled");

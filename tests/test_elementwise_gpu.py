@@ -495,10 +495,12 @@ def test_map3_muladd_bit_exact(hip, oracle, sfx):
 
 
 @pytest.mark.parametrize("sfx", ALL)
-@pytest.mark.parametrize("shape", [(16, 16), (130, 67), (257, 1031), (1024, 512)])
+@pytest.mark.parametrize("shape", [(16, 16), (130, 67), (257, 1031), (1024, 512), (128, 128), (260, 392), (136, 1028)])
 def test_mixed_unit_stride_axes(hip, oracle, sfx, shape):
-    """Operands whose unit stride is on different axes (the LDS-tiled 2-D kernel): transposed inputs,
-    transposed destinations, a broadcast vector beside a transposed matrix, scalar and unary forms."""
+    """Operands whose unit stride is on different axes (the LDS-tiled 2-D kernels: the element form for small,
+    odd or unaligned extents, the 16-byte-vector form with whole and ragged tiles otherwise): transposed inputs,
+    transposed destinations, a broadcast row or column vector beside a transposed matrix, scalar and unary
+    forms, windows of larger tensors."""
     dt = DTYPES[sfx]
     R, C = shape
     rng = np.random.default_rng(seed_of(sfx, "tiled", shape))
@@ -516,6 +518,14 @@ def test_mixed_unit_stride_axes(hip, oracle, sfx, shape):
                           oracle.scalar_op("sub", Bt.T, 3, scalar_on_left=True))
     say("tiled broadcast row vector + transposed", sfx, shape)
     assert np.array_equal(hip.bc_add(dBt.transpose(), dv).toCpu(), Bt.T + v)
+    col = fill(rng, (R, 1), dt)
+    assert np.array_equal(hip.bc_mul(dBt.transpose(), hip.toHip(col)).toCpu(), oracle.map2("mul", Bt.T, np.broadcast_to(col, (R, C))))
+    if R > 24 and C > 24:
+        say("tiled windows", sfx, shape)
+        for r_lo, c_lo in [(8, 4), (4, 8), (1, 3)]:    # the last one breaks the 16-byte alignment: element form
+            got = hip.map2("add", dA[r_lo:, c_lo:], dBt.transpose()[r_lo:, c_lo:]).toCpu()
+            assert np.array_equal(got, A[r_lo:, c_lo:] + Bt.T[r_lo:, c_lo:]), (r_lo, c_lo)
+            assert np.array_equal(dBt.transpose()[r_lo:, c_lo:].clone().toCpu(), Bt.T[r_lo:, c_lo:])
     say("tiled in place on a transposed destination", sfx, shape)
     dD = hip.toHip(Bt)
     dDt = dD.transpose()
