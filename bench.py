@@ -517,6 +517,21 @@ def config_report(am, timer, L):
          pct_peak=round(100 * (nbytes + 8192 * 4) / gpu_s / 1e9 / HBM_PEAK_GBS, 1), peak_used="HBM 8000 GB/s",
          bit_exact=bool(np.array_equal(dYs[ROTATE - 1].toCpu(), two_pass)),
          note="equals the two separate broadcast passes bit for bit; " + warm_note(ev / 50, nbytes + 8192 * 4))
+    # operands whose unit stride lies on the other axis than the result's (strided iteration, p_accessors.nim:181-208)
+    Xt = np.ascontiguousarray(X.T)
+    for name, launch, nb, want, cpu_fn in (
+            ("clone of a transposed view", lambda i: th._unary_into("copy", dYs[i], dXs[i].transpose()), 2 * X.nbytes, Xt,
+             lambda: np.copyto(out, X.T)),
+            ("X + X^T (transposed operand)", lambda i: th._binary_into("add", dYs[i], dXs[i], dXs[(i + 1) % ROTATE].transpose()), 3 * X.nbytes,
+             X + Xt, lambda: am_oracle.map2("add", X, X.T, out=out))):
+        gpu_s = run_rotating(timer, [(lambda i=i: launch(i)) for i in range(ROTATE)], 10)
+        cpu_s = cpu_time(cpu_fn, budget=2.0)
+        emit(config=f"f32 8192x8192 {name}", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
+             gpu_rate=round(nb / gpu_s / 1e9, 1), rate_unit="GB/s", pct_peak=round(100 * nb / gpu_s / 1e9 / HBM_PEAK_GBS, 1),
+             peak_used="HBM 8000 GB/s", cpu_impl="NumPy strided copy" if "clone" in name else "oracle/strided_map.c (strided iteration, OpenMP blocks)",
+             cpu_threads=1 if "clone" in name else threads, cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1),
+             bit_exact=bool(np.array_equal(dYs[ROTATE - 1].toCpu(), want)),
+             note="16-byte-vector tiled kernel: both operands read and the result written along their own unit-stride axis")
     del dYs
     # reductions, softmax, pooling (rows beyond the headline configurations)
     def hbm_case(config, fn_gpu, fn_cpu, nbytes, check, inputs):

@@ -177,7 +177,10 @@ def test_same_shape_ops_bit_exact(hip, oracle, sfx, shape):
 
 BC_CASES = [((64, 4096), (1, 4096)), ((64, 4096), (64, 1)), ((1, 4096), (64, 4096)), ((64, 1), (64, 4096)),
             ((4, 1), (1, 3)), ((5, 1, 7), (1, 6, 1)), ((2, 3, 2048), (2, 1, 2048)), ((3, 1, 4096), (1, 5, 1)),
-            ((1, 1), (9, 1031))]
+            ((1, 1), (9, 1031)),
+            # rows far shorter than a column tile, whole 16-byte vectors per row: the flat form of the row kernel
+            ((300, 64), (1, 64)), ((300, 64), (300, 1)), ((1, 64), (300, 64)), ((300, 1), (300, 64)), ((17, 8, 36), (1, 8, 1)),
+            ((17, 8, 36), (17, 1, 36)), ((6, 5, 4, 24), (1, 5, 1, 1)), ((6, 5, 4, 24), (6, 1, 4, 1))]
 
 
 @pytest.mark.parametrize("sfx", ALL)
@@ -239,6 +242,40 @@ def test_broadcast_comparisons_bit_exact(hip, oracle, sfx, shapes):
         b2 = b.copy(); b2[b2 == 0] = 2
         got = hip.map2("mod_is_zero", hip.toHip(ba.copy()), hip.toHip(np.broadcast_to(b2, ba.shape).copy())).toCpu()
         assert np.array_equal(got, np.fmod(ba, np.broadcast_to(b2, ba.shape)) == 0)
+
+
+@pytest.mark.parametrize("sfx", ALL)
+def test_short_rows_in_wider_buffers(hip, oracle, sfx):
+    """Column windows of wider buffers whose rows are a few vectors long (the flat form of the row kernel, with row
+    strides that differ between the operands): two windows, window and row / column vector, scalar and unary forms,
+    comparisons, in place; a window that starts off a 16-byte boundary takes the generic kernel and must agree."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("short-rows", sfx))
+    P, Q = fill(rng, (257, 200), dt), fill(rng, (257, 136), dt)
+    dP, dQ = hip.toHip(P), hip.toHip(Q)
+    row, col = fill(rng, (1, 72), dt), fill(rng, (257, 1), dt)
+    drow, dcol = hip.toHip(row), hip.toHip(col)
+    for lo_p, lo_q in [(8, 16), (64, 0), (3, 5)]:
+        a, b = P[:, lo_p:lo_p + 72], Q[:, lo_q:lo_q + 72]
+        da, db = dP[:, lo_p:lo_p + 72], dQ[:, lo_q:lo_q + 72]
+        say("short rows", sfx, lo_p, lo_q)
+        with np.errstate(over="ignore"):
+            assert np.array_equal(hip.map2("sub", da, db).toCpu(), a - b)
+            assert np.array_equal(hip.bc_add(da, drow).toCpu(), a + row)
+            assert np.array_equal(hip.bc_mul(dcol, db).toCpu(), col * b)
+            assert np.array_equal(hip.scalar_op("sub", da, 3, scalar_on_left=True).toCpu(), dt(3) - a)
+            assert np.array_equal(hip.unary("neg", db).toCpu(), -b)
+        assert np.array_equal(hip.bc_lt(da, db).toCpu(), a < b)
+        assert np.array_equal(hip.bc_ge(da, dcol).toCpu(), a >= col)
+    # in place on a window: the columns outside it stay as they were
+    want = P.copy()
+    with np.errstate(over="ignore"):
+        want[:, 8:80] += Q[:, 16:88]
+        want[:, 8:80] *= row
+    w = dP[:, 8:80]
+    w += dQ[:, 16:88]
+    w.bc_imul(drow)
+    assert np.array_equal(dP.toCpu(), want)
 
 
 @pytest.mark.parametrize("sfx", ALL)
