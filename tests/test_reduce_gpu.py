@@ -136,6 +136,41 @@ def test_long_axes_are_chunked(hip, oracle, sfx):
             assert close(sfx, op, getattr(hip, op)(dx), oracle.reduce_all(op, x), oracle.reduce_all("sum", np.abs(x)))
 
 
+@pytest.mark.parametrize("sfx", ALL)
+def test_tall_skinny_reductions(hip, oracle, sfx):
+    """Matrices with many rows and few columns, both ways: down the rows (the bias gradient of a dense layer: the
+    workgroup-wide walk with a second pass over chunk partials, also on column windows of wider buffers) and along
+    short rows (several rows per wavefront, row lengths that fill their lane group and that do not), on 2-D and 3-D
+    tensors. Integers, min and max exactly; float sums and products against the serial fold with the usual bound."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("tall-skinny", sfx))
+    cases = [((70_000, 64), 0, None), ((5_000, 512), 0, None), ((3_000, 128), 0, (slice(None), slice(16, 80))), ((600, 8), 0, None),
+             ((70_000, 64), 1, None), ((300_000, 16), 1, None), ((100_000, 24), 1, None), ((5_000, 8, 32), 2, None),
+             ((9_000, 128), 1, (slice(None), slice(8, 72))), ((4_100, 4), 1, None)]
+    for shape, ax, window in cases:
+        for op in OPS:
+            if op == "product" and sfx in ("f32", "f64") and shape[ax] > 3000:
+                continue   # thousands of factors near 1 leave the normal range: nothing to compare
+            x = fill(rng, shape, dt, op)
+            dx = hip.toHip(x)
+            v, dv = (x[window], dx[window]) if window else (x, dx)
+            say("tall-skinny", sfx, shape, ax, op, "window" if window else "whole")
+            got = getattr(hip, op)(dv, ax).toCpu()
+            want = oracle.reduce_axis(op, v, ax)
+            assert got.shape == want.shape
+            if sfx in ("i32", "i64") or op in ("min", "max"):
+                assert np.array_equal(got, want), (shape, ax, op)
+            else:
+                assert close(sfx, op, got, want, oracle.reduce_axis("sum", np.abs(v), ax) if op == "sum" else None), (shape, ax, op)
+    if sfx in ("f32", "f64"):   # mean and variance ride the same kernels
+        x = rng.uniform(-1, 1, (50_000, 32)).astype(dt)
+        dx = hip.toHip(x)
+        rtol = 2e-5 if sfx == "f32" else 1e-12
+        for ax in (0, 1):
+            assert np.allclose(hip.mean(dx, ax).toCpu(), x.astype(np.float64).mean(ax, keepdims=True), rtol=rtol, atol=rtol)
+            assert np.allclose(hip.variance(dx, ax).toCpu(), oracle.variance(x, ax), rtol=rtol * 10)
+
+
 @pytest.mark.parametrize("sfx", ["f32", "f64"])
 def test_variance_and_std(hip, oracle, vectors, sfx):
     """variance / std (aggregate.nim:115-158): the reference's own literals, then the oracle on
@@ -301,8 +336,11 @@ def test_softmax_vs_oracle(hip, oracle, sfx):
     dt = DTYPES[sfx]
     tol = 2e-6 if sfx == "f32" else 1e-14
     rng = np.random.default_rng(seed_of("softmax-gpu", sfx))
+    # (rows, cols): a wavefront, a workgroup or sixteen wavefronts per row by length; from 1024 rows on, several short
+    # rows per wavefront (whole vectors per row) or a lane per row (any length up to 64)
     for shape in [(1, 1), (3, 5), (64, 10), (256, 1000), (7, 4096), (5, 4097), (3, 8192), (4, 12288), (3, 16384), (3, 50_000),
-                  (1000, 3)]:
+                  (1000, 3), (3, 65536), (2, 40_000), (2, 70_000), (5000, 64), (3000, 16), (2000, 24), (1030, 4), (1500, 128),
+                  (20_000, 10), (1100, 63), (3, 300_000), (70, 131_072)]:
         x = (rng.standard_normal(shape) * 4).astype(dt)
         say("softmax", sfx, shape)
         want = oracle.softmax(x)
