@@ -50,6 +50,7 @@ template <typename T> struct Args {
   int splits;
   int64_t k_chunk;
   T* ws;
+  int want_splits;                 // > 0: the split factor the tile chooser decided on (plan_splitk then takes it as is)
   // Strided batch: workgroups with blockIdx.y = z work on A + z * batch_a, B + z * batch_b,
   // C + z * batch_c (elements); the bias is shared by the whole batch.
   int batch;
@@ -141,6 +142,7 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   g.batch = 1; g.batch_a = g.batch_b = g.batch_c = 0;
   g.gate_flags = nullptr; g.gate_gen = 0; g.gate_max_pairs = 0;
   g.static_ws = false; g.static_ws_short = 0;
+  g.want_splits = 0;
   g.clock_out = clock_probe_buffer();
   g.swapped = swap;
   g.a_kfast = iabs64(g.a_k) <= iabs64(g.a_mn);
@@ -154,8 +156,9 @@ static inline bool trace_choices() {
   return on;
 }
 
-// One candidate tile shape and the relative speed of a CU that runs it.
-struct TileChoice { int bm, bn; double eff; };
+// One candidate tile shape and the relative speed of a CU that runs it; bk / waves (slab width, wavefronts per
+// workgroup; 0 = 16 / 4) are what the split-K estimate of choose_tile_and_split needs.
+struct TileChoice { int bm, bn; double eff; int bk, waves; };
 
 // Picks the candidate with the least estimated time: rounds of one block per CU, each round
 // costing bm*bn/eff. Ragged edges and under-filled rounds are priced by construction.
@@ -270,18 +273,35 @@ void* static_scratch(size_t* capacity);
 // Decides the split-K factor for a problem that would otherwise leave most SIMDs idle: small M x N
 // (few tiles) with a long K runs as one serial MFMA / MAC chain per wave, so K is cut into
 // `splits` ranges handled by different workgroups. bk = slab width, waves = wavefronts per tile.
+// The split factors worth considering for `tiles` workgroup tiles of `waves` wavefronts and `slabs` slabs of k:
+// *base = one wavefront per SIMD over the chip, at least two slabs per split, at most 32 (1 when the tiles already
+// fill half the chip or k is short); *deep = up to four wavefronts per SIMD while every split keeps eight slabs, at most
+// 128: worth it for a very long k on tiles large enough that the matrix cores, not the round trips of a slab, set
+// a split's time (0 when it offers nothing beyond *base).
+static inline void splitk_factors(int64_t tiles, int waves, int64_t slabs, int64_t* base, int64_t* deep) {
+  *base = 1; *deep = 0;
+  const int64_t simds = (int64_t)num_cus() * 4;
+  if (tiles * waves * 2 > simds || slabs < 4) return;
+  int64_t want = simds / (tiles * waves);
+  if (want > slabs / 2) want = slabs / 2;
+  if (want > 32) want = 32;
+  if (want >= 2) *base = want;
+  int64_t d = 4 * simds / (tiles * waves);
+  if (d > slabs / 8) d = slabs / 8;
+  if (d > 128) d = 128;
+  if (d > *base) *deep = d;
+}
+
 template <typename T>
 static inline void plan_splitk(Args<T>& g, int bk, int waves_per_tile) {
   g.splits = 1; g.k_chunk = g.K; g.ws = nullptr;
   if (g.batch > 1) return;   // a batch already supplies the parallelism
   const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-  const int64_t simds = (int64_t)num_cus() * 4;
   const int64_t slabs = (g.K + bk - 1) / bk;
-  if (tiles * waves_per_tile * 2 > simds || slabs < 4) return;
-  int64_t want = simds / (tiles * waves_per_tile);          // one wave per SIMD
-  int64_t max_by_k = slabs / 2;                               // at least two slabs per split
-  int64_t splits = want < max_by_k ? want : max_by_k;
-  if (splits > 32) splits = 32;
+  int64_t splits, deep;
+  splitk_factors(tiles, waves_per_tile, slabs, &splits, &deep);
+  if (g.want_splits > 0) splits = g.want_splits;
+  if (splits > slabs) splits = slabs;
   if (splits < 2) return;
   const int64_t chunk_slabs = (slabs + splits - 1) / splits;
   splits = (slabs + chunk_slabs - 1) / chunk_slabs;           // no empty split
@@ -297,6 +317,75 @@ static inline void plan_splitk(Args<T>& g, int bk, int waves_per_tile) {
   }
   if (!ws) return;
   g.splits = (int)splits; g.k_chunk = chunk_slabs * bk; g.ws = ws;
+}
+
+// Tile AND split factor of a float product together. Where the tiles alone fill the chip this is choose_tile (rounds of
+// one workgroup per CU x tile area / efficiency). Where they do not, choose_tile's answer is the smallest tile (most
+// workgroups), whose matrix instructions wait on LDS and whose operands cross L2 most often, although a split of k can
+// supply the workgroups instead: [500 x 65536] * [65536 x 800] as 32 x 32 tiles 630 us, as 128 x 128 tiles x 9 splits
+// 440 us. So every candidate is priced with its own split factor (both kinds, see splitk_factors):
+//   rounds x slabs per split x time of a slab  +  the second pass (launch, and the partials read eight at a time by
+//   however many lanes the result offers)  +  a workgroup's fixed cost.
+// flops_per_cu_us: what one CU sustains (peak / CUs). Sets g.want_splits.
+template <typename T>
+static inline int choose_tile_and_split(Args<T>& g, const TileChoice* cand, int ncand, const char* env, double flops_per_cu_us) {
+  g.want_splits = 0;
+  const int by_rounds = choose_tile(cand, ncand, g.M, g.N, env, g.batch);
+  const char* forced = getenv(env);
+  if ((forced && *forced) || g.batch > 1 || g.static_ws) return by_rounds;
+  static const bool joint = [] { const char* e = getenv("AM_HIP_GEMM_JOINT"); return !(e && *e == '0'); }();
+  if (!joint) return by_rounds;
+  const int64_t cus = num_cus();
+  // choose_tile's answer priced the same way is the bar; the other tiles enter with their split factors only (without
+  // a split they have lost against it already), and one of them has to beat the bar by a tenth.
+  auto price = [&](int i, int64_t sp_in, int64_t* sp_out) {
+    const TileChoice& c = cand[i];
+    const int bk = c.bk ? c.bk : 16;
+    const int64_t tiles = ((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn);
+    const int64_t slabs = (g.K + bk - 1) / bk;
+    const int64_t chunk = (slabs + sp_in - 1) / sp_in;
+    const int64_t sp = (slabs + chunk - 1) / chunk;
+    *sp_out = sp;
+    if (sp > 1 && (double)sp * g.M * g.N * sizeof(T) > 48.0 * 1024 * 1024) return -1.0;
+    // a slab's time: the matrix instructions; a workgroup alone on its CU cannot go below what its chain of LDS and
+    // barrier waits allows (measured on the 32 x 32 tile: 0.23 us per slab of 32 k)
+    double slab_us = 2.0 * c.bm * c.bn * bk / (flops_per_cu_us * c.eff);
+    if ((sp > 1 || tiles < cus) && slab_us < 0.22) slab_us = 0.22;
+    const int64_t rounds = (tiles * sp + cus - 1) / cus;
+    double us = 4.0 + (double)rounds * (double)chunk * slab_us;
+    if (sp > 1) {
+      const double lanes = (double)g.M * (double)g.N / (16.0 / sizeof(T));
+      const double passes = (double)((sp + (sp >= 32 ? 31 : 7)) / (sp >= 32 ? 32 : 8));   // 8 partials in flight per lane, x 4 wavefronts
+      const double latency = passes * 1.0, bandwidth = (double)(sp + 1) * g.M * g.N * sizeof(T) / 4.0e6;
+      us += 5.0 + (lanes >= (double)cus * 1024 ? bandwidth : (latency > bandwidth ? latency : bandwidth));
+    }
+    return us;
+  };
+  int best = by_rounds;
+  int64_t best_splits = 0;
+  double best_us = -1, bar_us = -1;
+  for (int i = 0; i < ncand; ++i) {
+    const TileChoice& c = cand[i];
+    if (c.eff <= 0) continue;
+    const int bk = c.bk ? c.bk : 16, waves = c.waves ? c.waves : 4;
+    const int64_t tiles = ((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn);
+    int64_t opt[2];
+    splitk_factors(tiles, waves, (g.K + bk - 1) / bk, &opt[0], &opt[1]);
+    for (int o = 0; o < 2; ++o) {
+      if (opt[o] < 1 || (opt[o] < 2 && i != by_rounds)) continue;
+      int64_t sp;
+      const double us = price(i, opt[o], &sp);
+      if (us < 0) continue;
+      if (i == by_rounds && o == 0) bar_us = us;
+      if (best_us < 0 || us < best_us) { best_us = us; best = i; best_splits = sp; }
+    }
+  }
+  if (best != by_rounds && bar_us >= 0 && best_us > 0.85 * bar_us) { best = by_rounds; best_splits = 0; best_us = bar_us; }
+  g.want_splits = (int)best_splits;
+  if (trace_choices())
+    fprintf(stderr, "am_hip gemm: M=%lld N=%lld K=%lld tile %dx%d with %lld splits of k, est %.1f us (by rounds alone: %dx%d)\n", (long long)g.M,
+            (long long)g.N, (long long)g.K, cand[best].bm, cand[best].bn, (long long)best_splits, best_us, cand[by_rounds].bm, cand[by_rounds].bn);
+  return best;
 }
 
 // Cuts K into `want` ranges (fewer if K has too few slabs or the workspace is too small / cannot
@@ -364,38 +453,57 @@ static inline TileSplit choose_tile_split(const TileChoice* cand, int ncand, int
 // ascending s (deterministic). ACC is the type the partials were stored in. One thread per group
 // of VEC consecutive columns of one row (blockIdx.y walks the rows): VEC = 16 bytes / element when
 // N is a multiple of it (the partials are then read as 16-byte vectors), else 1.
-template <typename T, typename ACC, int VEC>
+// SY = 4 (many partials, few outputs: the pass is then a chain of memory round trips per lane, not bandwidth): the four
+// wavefronts of a workgroup share 64 column groups and take the partials s = w, w + 4, w + 8, ... each; their four sums
+// are added through LDS in the order ((w0 + w1) + w2) + w3 and the first wavefront writes. Needs splits >= 4.
+template <typename T, typename ACC, int VEC, int SY = 1>
 __global__ __launch_bounds__(256) void splitk_reduce(Args<T> p) {
   typedef ACC vec_t __attribute__((ext_vector_type(VEC)));
   if (std::is_integral<T>::value && p.gate_flags != nullptr && live_digit_pairs<(int)sizeof(T)>(p.gate_flags, p.gate_gen) <= p.gate_max_pairs) return;
   const int64_t total = p.M * p.N;
   const ACC* ws = (const ACC*)p.ws;
-  const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
-  if (col >= p.N) return;
+  __shared__ ACC cls[SY > 1 ? SY - 1 : 1][SY > 1 ? 64 * VEC : 1];
+  const int cl = SY > 1 ? (int)(threadIdx.x >> 6) : 0;
+  const int64_t col = SY > 1 ? ((int64_t)blockIdx.x * 64 + (threadIdx.x & 63)) * VEC : ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (SY == 1 && col >= p.N) return;
+  const bool in_range = col < p.N;
   for (int64_t row = blockIdx.y; row < p.M; row += gridDim.y) {
-    const int64_t idx = row * p.N + col;
+    const int64_t idx = row * p.N + (in_range ? col : 0);
     ACC sum[VEC];
     {
-      const vec_t v = *(const vec_t*)(ws + idx);
+      const vec_t v = *(const vec_t*)(ws + (int64_t)cl * total + idx);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sum[e] = v[e];
     }
     // eight partials in flight at a time (the loads are independent; the additions stay in
     // ascending s): with one load per trip the pass is a chain of memory round trips
-    int sidx = 1;
-    for (; sidx + 8 <= p.splits; sidx += 8) {
+    int sidx = cl + SY;
+    for (; sidx + 7 * SY < p.splits; sidx += 8 * SY) {
       vec_t v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = *(const vec_t*)(ws + (int64_t)(sidx + u) * total + idx);
+      for (int u = 0; u < 8; ++u) v[u] = *(const vec_t*)(ws + (int64_t)(sidx + u * SY) * total + idx);
 #pragma unroll
       for (int u = 0; u < 8; ++u)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) sum[e] += v[u][e];
     }
-    for (; sidx < p.splits; ++sidx) {
+    for (; sidx < p.splits; sidx += SY) {
       const vec_t v = *(const vec_t*)(ws + (int64_t)sidx * total + idx);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) sum[e] += v[e];
+    }
+    if constexpr (SY > 1) {
+      if (row != (int64_t)blockIdx.y) __syncthreads();   // the previous row's sums have been read
+      if (cl > 0) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) cls[cl - 1][(threadIdx.x & 63) * VEC + e] = sum[e];
+      }
+      __syncthreads();
+      if (cl > 0 || !in_range) continue;
+#pragma unroll
+      for (int w = 0; w < SY - 1; ++w)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) sum[e] += cls[w][(threadIdx.x & 63) * VEC + e];
     }
     T* cp = p.C + row * p.c_m + col * p.c_n;
     ACC cold[VEC], bias[VEC];
@@ -429,14 +537,17 @@ static int launch_splitk_reduce(const Args<T>& g) {
   constexpr int VEC = 16 / (int)sizeof(ACC);
   const bool vec = (g.N % VEC == 0);   // the workspace itself is 256-byte aligned and row pitch N
   const int64_t cols = vec ? g.N / VEC : g.N;
-  const int64_t bx = (cols + 255) / 256;
+  // many partials of a small result: four wavefronts per 64 column groups, each a quarter of the partials
+  const bool wide = vec && g.splits >= 32 && cols * g.M < (int64_t)num_cus() * 1024;
+  const int64_t bx = wide ? (cols + 63) / 64 : (cols + 255) / 256;
   int64_t by = g.M;
   const int64_t cap = (int64_t)num_cus() * 16;
   if (bx * by > cap) by = (cap + bx - 1) / bx;
   if (by > 65535) by = 65535;
   if (by < 1) by = 1;
   const dim3 grid((unsigned)bx, (unsigned)by), block(256);
-  if (vec) hipLaunchKernelGGL((splitk_reduce<T, ACC, VEC>), grid, block, 0, stream(), g);
+  if (wide) hipLaunchKernelGGL((splitk_reduce<T, ACC, VEC, 4>), grid, block, 0, stream(), g);
+  else if (vec) hipLaunchKernelGGL((splitk_reduce<T, ACC, VEC>), grid, block, 0, stream(), g);
   else hipLaunchKernelGGL((splitk_reduce<T, ACC, 1>), grid, block, 0, stream(), g);
   return check_launch("splitk_reduce");
 }

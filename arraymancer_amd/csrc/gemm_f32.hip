@@ -31,7 +31,7 @@ static int run_whole_f32(Args<float>& g) {
   // 4096^3). PF = 2 (two slabs of global loads in flight) on the tiles whose slab is short.
   int nc = 0;
   const TileChoice* cand = candidates_f32(&nc);
-  switch (choose_tile(cand, nc, g.M, g.N, "AM_HIP_GEMM_TILE_F32", g.batch)) {
+  switch (choose_tile_and_split(g, cand, nc, "AM_HIP_GEMM_TILE_F32", 157.3e6 / 256)) {
     case 0: return launch_kinds<float, 256, 256, 16, 2, 4, 1, true, false>(g, ak, bk);   // its loop is long enough: unrolling it over the ring costs 4 %
     case 1: return launch_kinds<float, 128, 128, 16, 2, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2, 2>(g, ak, bk);
@@ -44,7 +44,9 @@ static int run_whole_f32(Args<float>& g) {
 }
 
 static const TileChoice* candidates_f32(int* n) {
-  static const TileChoice cand[] = {{256, 256, 1.0}, {128, 128, 0.94}, {64, 64, 0.88}, {256, 128, 0.97}, {128, 64, 0.92}, {32, 32, 0.74}};
+  // {rows, columns, efficiency, slab width, wavefronts}
+  static const TileChoice cand[] = {{256, 256, 1.0, 16, 8}, {128, 128, 0.94, 16, 4}, {64, 64, 0.88, 16, 4}, {256, 128, 0.97, 16, 8},
+                                    {128, 64, 0.92, 16, 4},  {32, 32, 0.74, 32, 4}};
   *n = (int)(sizeof(cand) / sizeof(cand[0]));
   return cand;
 }

@@ -35,7 +35,7 @@ static int run_whole_f64(Args<double>& g) {
   // the second half empty) but exactly 256 of 128 x 192.
   int nc = 0;
   const TileChoice* cand = candidates_f64(&nc);
-  switch (choose_tile(cand, nc, g.M, g.N, "AM_HIP_GEMM_TILE_F64", g.batch)) {
+  switch (choose_tile_and_split(g, cand, nc, "AM_HIP_GEMM_TILE_F64", 78.6e6 / 256)) {
     case 0: return launch_kinds<double, 128, 128, 16, 2, 4>(g, ak, bk);
     case 1: return launch_kinds<double, 64, 64, 16, 2, 2, 2>(g, ak, bk);
     case 2: return launch_kinds<double, 32, 32, 16, 2, 2, 2>(g, ak, bk);
@@ -46,7 +46,9 @@ static int run_whole_f64(Args<double>& g) {
 }
 
 static const TileChoice* candidates_f64(int* n) {
-  static const TileChoice cand[] = {{128, 128, 0.97}, {64, 64, 0.93}, {32, 32, 0.76}, {256, 128, 1.0}, {128, 64, 0.96}, {128, 192, 0.98}};
+  // {rows, columns, efficiency, slab width, wavefronts}
+  static const TileChoice cand[] = {{128, 128, 0.97, 16, 8}, {64, 64, 0.93, 16, 4}, {32, 32, 0.76, 16, 4}, {256, 128, 1.0, 16, 8},
+                                    {128, 64, 0.96, 16, 4},  {128, 192, 0.98, 16, 8}};
   *n = (int)(sizeof(cand) / sizeof(cand[0]));
   return cand;
 }

@@ -517,7 +517,10 @@ def test_hip_graph_replays_match_eager(hip, oracle):
         assert np.array_equal(scratch.toCpu(), expect_scratch)
 
 
-SPLITK_SHAPES = [(64, 10, 500), (64, 500, 800), (50, 4096, 500), (33, 47, 2049), (128, 128, 4096), (1, 1, 1000), (7, 300, 257)]
+SPLITK_SHAPES = [(64, 10, 500), (64, 500, 800), (50, 4096, 500), (33, 47, 2049), (128, 128, 4096), (1, 1, 1000), (7, 300, 257),
+                 # k long enough for the deep split factors (up to 128 ranges of k, larger tiles than the tile count alone would
+                 # pick, partials folded by four wavefronts per column group)
+                 (70, 70, 70_000), (128, 96, 100_000), (200, 200, 50_000), (300, 520, 20_000)]
 
 
 @pytest.mark.parametrize("sfx", ALL)
