@@ -621,6 +621,28 @@ def run_only(am, timer, which, steps, warmup):
     elif which == "maxpool":
         dX = am.toHip(np.random.default_rng(4005).uniform(-1, 1, (256, 64, 112, 112)).astype(np.float32))
         fn = lambda: am.maxpool2d(dX, (2, 2), (0, 0), (2, 2))
+    elif which == "transposed_add":   # X + Z^T: operands with unit strides on different axes, three buffer sets round robin
+        X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
+        dXs = [am.toHip(X) for _ in range(3)]
+        dYs = [am.empty((8192, 8192), np.float32) for _ in range(3)]
+        rounds = max(steps // 3, 4)
+        per = run_rotating(timer, [(lambda i=i: th._binary_into("add", dYs[i], dXs[i], dXs[(i + 1) % 3].transpose())) for i in range(3)], rounds)
+        return dict(only=which, ms_per_launch=round(per * 1e3, 4), launches=(rounds + 1) * 3)
+    elif which in ("bias_short_rows", "sum_cols_narrow", "sum_rows_short", "softmax_short_rows"):
+        # tall and skinny: a [batch x features] activation with its bias, the bias gradient, row sums and softmax of short rows
+        rows, cols = (65536, 512) if which in ("bias_short_rows", "sum_cols_narrow") else (1048576, 64)
+        dX = am.toHip(np.random.default_rng(4001).uniform(-1, 1, (rows, cols)).astype(np.float32))
+        if which == "bias_short_rows":
+            dY = am.empty((rows, cols), np.float32)
+            bb = am.toHip(np.random.default_rng(4002).uniform(-1, 1, (1, cols)).astype(np.float32)).broadcast((rows, cols))
+            fn = lambda: th._binary_into("add", dY, dX, bb)
+        else:
+            fn = {"sum_cols_narrow": lambda: am.sum(dX, 0), "sum_rows_short": lambda: am.sum(dX, 1), "softmax_short_rows": lambda: am.softmax(dX)}[which]
+    elif which == "gemm_f32_long_k":   # the weight gradient of a dense layer over a large batch: few tiles, very long k
+        dA = am.toHip(np.random.default_rng(1001).standard_normal((500, 65536)).astype(np.float32))
+        dB = am.toHip(np.random.default_rng(1002).standard_normal((65536, 800)).astype(np.float32))
+        dC = am.empty((500, 800), np.float32)
+        fn = lambda: am.gemm(1, dA, dB, 0, dC)
     else:
         X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
         dX, dY = am.toHip(X), am.empty((8192, 8192), np.float32)
@@ -643,7 +665,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true",
                     help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool",
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool", "transposed_add", "bias_short_rows", "sum_cols_narrow", "sum_rows_short", "softmax_short_rows", "gemm_f32_long_k",
                                       "gemm_f32_1024", "gemm_f32_2048", "gemm_i32_1500", "bcast_add_rotating"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
