@@ -369,18 +369,32 @@ static inline int choose_tile_and_split(Args<T>& g, const TileChoice* cand, int 
     if (c.eff <= 0) continue;
     const int bk = c.bk ? c.bk : 16, waves = c.waves ? c.waves : 4;
     const int64_t tiles = ((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn);
-    int64_t opt[2];
+    // choose_tile's tile also without any split: a second launch for a product of a few microseconds costs more than
+    // the idle SIMDs it fills (256^3: 8.4 us as 4 ranges of k + second pass, 5.5 us whole)
+    int64_t opt[3] = {0, 0, i == by_rounds ? 1 : 0};
     splitk_factors(tiles, waves, (g.K + bk - 1) / bk, &opt[0], &opt[1]);
-    for (int o = 0; o < 2; ++o) {
+    for (int o = 0; o < 3; ++o) {
       if (opt[o] < 1 || (opt[o] < 2 && i != by_rounds)) continue;
       int64_t sp;
       const double us = price(i, opt[o], &sp);
       if (us < 0) continue;
-      if (i == by_rounds && o == 0) bar_us = us;
+      if (i == by_rounds && (bar_us < 0 || us < bar_us)) bar_us = us;
       if (best_us < 0 || us < best_us) { best_us = us; best = i; best_splits = sp; }
     }
   }
-  if (best != by_rounds && bar_us >= 0 && best_us > 0.85 * bar_us) { best = by_rounds; best_splits = 0; best_us = bar_us; }
+  if (best != by_rounds && bar_us >= 0 && best_us > 0.85 * bar_us) {   // not convincingly better: choose_tile's tile, at its own best split
+    best = by_rounds; best_us = -1;
+    const TileChoice& c = cand[best];
+    const int bk = c.bk ? c.bk : 16, waves = c.waves ? c.waves : 4;
+    int64_t opt[3] = {0, 0, 1};
+    splitk_factors(((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn), waves, (g.K + bk - 1) / bk, &opt[0], &opt[1]);
+    for (int o = 0; o < 3; ++o) {
+      if (opt[o] < 1) continue;
+      int64_t sp;
+      const double us = price(best, opt[o], &sp);
+      if (us >= 0 && (best_us < 0 || us < best_us)) { best_us = us; best_splits = sp; }
+    }
+  }
   g.want_splits = (int)best_splits;
   if (trace_choices())
     fprintf(stderr, "am_hip gemm: M=%lld N=%lld K=%lld tile %dx%d with %lld splits of k, est %.1f us (by rounds alone: %dx%d)\n", (long long)g.M,
