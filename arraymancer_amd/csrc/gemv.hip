@@ -47,6 +47,10 @@ template <> __device__ __forceinline__ uint64_t wave_sum<uint64_t>(uint64_t v) {
   return v;
 }
 
+template <typename U> __device__ __forceinline__ U xor_lane(U v, int d) { return __shfl_xor(v, d, 64); }
+template <> __device__ __forceinline__ uint32_t xor_lane<uint32_t>(uint32_t v, int d) { return (uint32_t)__shfl_xor((int)v, d, 64); }
+template <> __device__ __forceinline__ uint64_t xor_lane<uint64_t>(uint64_t v, int d) { return (uint64_t)__shfl_xor((long long)v, d, 64); }
+
 template <typename T> struct GemvArgs {
   int64_t M, N;
   T alpha, beta;
@@ -64,37 +68,150 @@ __device__ __forceinline__ void store_y(const GemvArgs<T>& p, int64_t row, U sum
   *yp = (T)v;
 }
 
-// A row-contiguous. VECLOAD: rows and x are 16-byte aligned and x has unit stride.
+// A row-contiguous. VECLOAD: rows and x are 16-byte aligned and x has unit stride. With p.splits > 1 (few, long
+// rows: a wavefront per row would leave most of the chip idle) a wavefront takes one chunk of one row, columns
+// [chunk * n_chunk, ...), and its sum goes to ws[chunk][row] for the split-K reduce kernel.
 template <typename T, bool VECLOAD>
 __global__ __launch_bounds__(256) void gemv_rows(GemvArgs<T> p) {
   typedef typename Acc<T>::type U;
   typedef typename VecTraits<T>::vec_t vec_t;
   constexpr int VEC = VecTraits<T>::VK;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.M; row += (int64_t)gridDim.x * 4) {
-    const T* __restrict__ a = p.A + row * p.rsA;
+  const int64_t units = p.M * p.splits;
+  for (int64_t unit = (int64_t)blockIdx.x * 4 + wave; unit < units; unit += (int64_t)gridDim.x * 4) {
+    const int64_t chunk = unit / p.M, row = unit - chunk * p.M;
+    const int64_t c0 = chunk * p.n_chunk;
+    const int64_t len = (c0 + p.n_chunk < p.N) ? p.n_chunk : p.N - c0;
+    const T* __restrict__ a = p.A + row * p.rsA + c0;
+    const T* __restrict__ xs = p.x + c0 * p.incx;
     U acc0 = 0, acc1 = 0;
     if constexpr (VECLOAD) {
-      const int64_t nvec = p.N / VEC;
+      const int64_t nvec = len / VEC;
       int64_t j = lane;
-      for (; j + 64 < nvec; j += 128) {
+      for (; j + 192 < nvec; j += 256) {   // four 16-byte loads of A in flight per lane
         const vec_t a0 = __builtin_nontemporal_load((const vec_t*)a + j), a1 = __builtin_nontemporal_load((const vec_t*)a + j + 64);
-        const vec_t x0 = *((const vec_t*)p.x + j), x1 = *((const vec_t*)p.x + j + 64);
+        const vec_t a2 = __builtin_nontemporal_load((const vec_t*)a + j + 128), a3 = __builtin_nontemporal_load((const vec_t*)a + j + 192);
+        const vec_t x0 = *((const vec_t*)xs + j), x1 = *((const vec_t*)xs + j + 64), x2 = *((const vec_t*)xs + j + 128), x3 = *((const vec_t*)xs + j + 192);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) { acc0 += (U)a0[e] * (U)x0[e]; acc1 += (U)a1[e] * (U)x1[e]; }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { acc0 += (U)a2[e] * (U)x2[e]; acc1 += (U)a3[e] * (U)x3[e]; }
       }
       for (; j < nvec; j += 64) {
         const vec_t a0 = __builtin_nontemporal_load((const vec_t*)a + j);
-        const vec_t x0 = *((const vec_t*)p.x + j);
+        const vec_t x0 = *((const vec_t*)xs + j);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc0 += (U)a0[e] * (U)x0[e];
       }
-      for (int64_t c = nvec * VEC + lane; c < p.N; c += 64) acc1 += (U)a[c] * (U)p.x[c];
+      for (int64_t c = nvec * VEC + lane; c < len; c += 64) acc1 += (U)a[c] * (U)xs[c];
     } else {
-      for (int64_t c = lane; c < p.N; c += 64) acc0 += (U)a[c] * (U)p.x[c * p.incx];
+      for (int64_t c = lane; c < len; c += 64) acc0 += (U)a[c] * (U)xs[c * p.incx];
     }
     const U total = wave_sum<U>(acc0 + acc1);
-    if (lane == 0) store_y<T, U>(p, row, total);
+    if (lane == 0) {
+      if (p.splits > 1) p.ws[chunk * p.M + row] = (T)total;
+      else store_y<T, U>(p, row, total);
+    }
+  }
+}
+
+// Many SHORT rows (a [batch x features] matrix times a weight vector, 4 ... 128 features): `lanes` lanes (a power of
+// two <= 32) share a row, one 16-byte vector of A each and their piece of x in registers, so a wavefront's load is one
+// contiguous run of 64 / lanes rows; four row groups in flight; the lanes of a row are summed by a butterfly.
+// Requires unit strides of A's columns and of x, N % VEC == 0, 16-byte aligned rows.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_rows_short(GemvArgs<T> p, int lanes) {
+  typedef typename Acc<T>::type U;
+  typedef typename VecTraits<T>::vec_t vec_t;
+  constexpr int VEC = VecTraits<T>::VK;
+  constexpr int UNR = 4;
+  const int lane = threadIdx.x & 63;
+  const int j = lane & (lanes - 1), sub = lane / lanes, rows_per_step = 64 / lanes;
+  const int64_t nvec = p.N / VEC;
+  const bool mine = j < nvec;
+  const vec_t xv = *((const vec_t*)p.x + (mine ? j : 0));
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t row0 = wave * (int64_t)(UNR * rows_per_step) + sub;
+  vec_t av[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t row = row0 + (int64_t)u * rows_per_step;
+    av[u] = __builtin_nontemporal_load((const vec_t*)(p.A + (row < p.M ? row : 0) * p.rsA) + (mine ? j : 0));
+  }
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t row = row0 + (int64_t)u * rows_per_step;
+    U acc = 0;
+    if (mine) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc += (U)av[u][e] * (U)xv[e];
+    }
+    for (int d = lanes >> 1; d >= 1; d >>= 1) acc += xor_lane<U>(acc, d);
+    if (j == 0 && row < p.M) store_y<T, U>(p, row, acc);
+  }
+}
+
+// A column-contiguous with FEW rows (y = A^T r for a tall [batch x features] matrix: the outputs are the features):
+// the 256 lanes of a workgroup are laid over cxw lanes along the unit-stride direction x 256 / cxw columns, each lane
+// walks every (256 / cxw)-th column of the workgroup's chunk with eight loads in flight, and the column classes are
+// summed through LDS in a fixed order. grid = (chunks of the walk, blocks of cxw lanes along m). With chunks, the
+// partials ws[chunk][M] are folded by a second launch of this kernel over the partials themselves (x == nullptr: every
+// factor is one; 8 lanes wide, so that it spreads over many workgroups), which applies alpha and beta.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_cols_narrow(GemvArgs<T> p, int cxw) {
+  typedef typename Acc<T>::type U;
+  typedef typename VecTraits<T>::vec_t vec_t;
+  constexpr int VEC = VecTraits<T>::VK;
+  constexpr int UN = 8;
+  __shared__ U part[256][VEC];
+  const int ry = 256 / cxw;
+  const int xq = (int)threadIdx.x % cxw, yq = (int)threadIdx.x / cxw;
+  const int64_t m = ((int64_t)blockIdx.y * cxw + xq) * VEC;
+  const bool active = yq < ry && m < p.M;
+  const bool ones = p.x == nullptr;
+  const int64_t j0 = (int64_t)blockIdx.x * p.n_chunk;
+  const int64_t j1 = (j0 + p.n_chunk < p.N) ? j0 + p.n_chunk : p.N;
+  U acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0;
+  if (active) {
+    const T* __restrict__ a = p.A + m;
+    int64_t j = j0 + yq;
+    for (; j + (int64_t)(UN - 1) * ry < j1; j += (int64_t)UN * ry) {
+      vec_t v[UN];
+      U xs[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        v[u] = __builtin_nontemporal_load((const vec_t*)(a + (j + (int64_t)u * ry) * p.csA));
+        xs[u] = ones ? (U)1 : (U)p.x[(j + (int64_t)u * ry) * p.incx];
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += (U)v[u][e] * xs[u];
+    }
+    for (; j < j1; j += ry) {
+      const vec_t v = *(const vec_t*)(a + j * p.csA);
+      const U xj = ones ? (U)1 : (U)p.x[j * p.incx];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] += (U)v[e] * xj;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) part[threadIdx.x][e] = acc[e];
+  __syncthreads();
+  if (active && yq == 0) {
+    for (int yy = 1; yy < ry; ++yy)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] += part[yy * cxw + xq][e];
+    if (p.splits > 1) {
+      T* ws = p.ws + (int64_t)blockIdx.x * p.M + m;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) ws[e] = (T)acc[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) store_y<T, U>(p, m + e, acc[e]);
+    }
   }
 }
 
@@ -224,14 +341,71 @@ int gemv(const char* fn, int64_t M, int64_t N, T alpha, const T* A, int64_t rsA,
   g.M = M; g.N = N; g.alpha = alpha; g.beta = beta; g.A = A; g.rsA = rsA; g.csA = csA;
   g.x = x; g.incx = incx; g.y = y; g.incy = incy; g.ws = nullptr; g.splits = 1; g.n_chunk = N;
 
-  if (csA == 1 && M >= 64) {
+  // y seen as one row of M columns: the split-K reduce kernel adds the partials ws[split][M] in ascending order
+  auto fold_partials = [&]() {
+    Args<T> r;
+    memset(&r, 0, sizeof(r));
+    r.M = 1; r.N = M; r.K = N; r.alpha = alpha; r.beta = beta; r.C = y; r.c_m = 0; r.c_n = incy;
+    r.epilogue = AM_EPI_NONE; r.splits = g.splits; r.ws = g.ws;
+    return launch_splitk_reduce<T, U>(r);
+  };
+  if (csA == 1 && (M >= 64 || N >= 16384)) {
     const bool vec = aligned16(A) && aligned16(x) && incx == 1 && (rsA % VEC == 0);
-    int64_t blocks = (M + 3) / 4;
+    // short rows: several per wavefront
+    if (vec && N % VEC == 0 && N / VEC <= 32 && M >= 4096) {
+      int lanes = 1;
+      while (lanes < N / VEC) lanes *= 2;
+      const int64_t rows_per_wg = 4 * 4 * (64 / lanes);
+      const int64_t blocks = (M + rows_per_wg - 1) / rows_per_wg;
+      if (blocks < ((int64_t)1 << 31)) {
+        hipLaunchKernelGGL((gemv_rows_short<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), g, lanes);
+        return check_launch("gemv_rows_short");
+      }
+    }
+    // few long rows: chunks of a row over several wavefronts (16 wavefronts per CU over the chip, at least 4096 columns each)
+    const int64_t want_waves = (int64_t)num_cus() * 16;
+    if (M < want_waves / 2 && N >= 8192) {
+      int64_t splits = (want_waves + M - 1) / M;
+      if (splits > N / 4096) splits = N / 4096;
+      if (splits > 256) splits = 256;
+      if (splits >= 2) {
+        int64_t chunk = (N + splits - 1) / splits;
+        chunk = (chunk + 255) / 256 * 256;                      // chunk starts stay 16-byte aligned
+        splits = (N + chunk - 1) / chunk;
+        T* ws = splits >= 2 ? (T*)splitk_workspace((size_t)splits * M * sizeof(T)) : nullptr;
+        if (ws) { g.ws = ws; g.splits = (int)splits; g.n_chunk = chunk; }
+      }
+    }
+    int64_t blocks = (M * g.splits + 3) / 4;
     const int64_t cap = (int64_t)num_cus() * 16;
     if (blocks > cap) blocks = cap;
     if (vec) hipLaunchKernelGGL((gemv_rows<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream(), g);
     else hipLaunchKernelGGL((gemv_rows<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream(), g);
-    return check_launch("gemv_rows");
+    AM_TRY(check_launch("gemv_rows"));
+    return g.splits > 1 ? fold_partials() : AM_OK;
+  }
+  if (rsA == 1 && M % VEC == 0 && M / VEC <= 128 && csA % VEC == 0 && csA >= M && aligned16(A) && N >= 512) {
+    // few outputs, a long walk: the workgroup-wide form, the walk cut into chunks (4 workgroups per CU)
+    const int cx = (int)(M / VEC);
+    int64_t splits = (int64_t)num_cus() * 4;
+    if (splits > N / 256) splits = N / 256;
+    if (splits >= 2) {
+      const int64_t chunk = (N + splits - 1) / splits;
+      splits = (N + chunk - 1) / chunk;
+      T* ws = splits >= 2 ? (T*)splitk_workspace((size_t)splits * M * sizeof(T)) : nullptr;
+      if (ws) { g.ws = ws; g.splits = (int)splits; g.n_chunk = chunk; }
+    }
+    hipLaunchKernelGGL((gemv_cols_narrow<T>), dim3((unsigned)g.splits, 1), dim3(256), 0, stream(), g, cx);
+    AM_TRY(check_launch("gemv_cols_narrow"));
+    if (g.splits > 1) {
+      GemvArgs<T> r = g;
+      r.A = g.ws; r.rsA = 1; r.csA = M; r.N = g.splits; r.x = nullptr; r.incx = 0;
+      r.ws = nullptr; r.splits = 1; r.n_chunk = r.N;
+      const int cxw = cx < 8 ? cx : 8;
+      hipLaunchKernelGGL((gemv_cols_narrow<T>), dim3(1, (unsigned)((cx + cxw - 1) / cxw)), dim3(256), 0, stream(), r, cxw);
+      AM_TRY(check_launch("gemv_cols_narrow (second pass)"));
+    }
+    return AM_OK;
   }
   if (rsA == 1 && M % VEC == 0 && csA % VEC == 0 && csA >= 0 && aligned16(A) && M >= 256) {
     const int64_t blocks_m = (M / VEC + 255) / 256;
@@ -247,15 +421,7 @@ int gemv(const char* fn, int64_t M, int64_t N, T alpha, const T* A, int64_t rsA,
     }
     hipLaunchKernelGGL((gemv_cols<T, 8>), dim3((unsigned)blocks_m, (unsigned)g.splits), dim3(256), 0, stream(), g);
     AM_TRY(check_launch("gemv_cols"));
-    if (g.splits > 1) {
-      Args<T> r;
-      memset(&r, 0, sizeof(r));
-      // y seen as one row of M columns: the reduction kernel spreads threads over columns
-      r.M = 1; r.N = M; r.K = N; r.alpha = alpha; r.beta = beta; r.C = y; r.c_m = 0; r.c_n = incy;
-      r.epilogue = AM_EPI_NONE; r.splits = g.splits; r.ws = g.ws;
-      return launch_splitk_reduce<T, U>(r);
-    }
-    return AM_OK;
+    return g.splits > 1 ? fold_partials() : AM_OK;
   }
   return gemm_fallback<T>(M, N, alpha, A, rsA, csA, x, incx, beta, y, incy);
 }

@@ -46,7 +46,10 @@ def test_reference_literals(hip, vectors, sfx):
     assert np.array_equal((b[2:4, 3:0:-2] * uu[2::-2]).toCpu(), np.array([-3682, -4783], dtype=dt))
 
 
-SHAPES = [(1, 1), (3, 5), (64, 64), (65, 129), (256, 33), (300, 1000), (1024, 4096), (4096, 260), (2048, 2050)]
+SHAPES = [(1, 1), (3, 5), (64, 64), (65, 129), (256, 33), (300, 1000), (1024, 4096), (4096, 260), (2048, 2050),
+          # tall and skinny, both ways: several short rows per wavefront (C layout) / the workgroup-wide walk with a second
+          # pass over chunk partials (F layout); few long rows: chunks of a row over several wavefronts
+          (70_000, 64), (9_000, 16), (5_000, 24), (20_000, 128), (64, 70_000), (5, 300_000), (300, 20_000), (512, 9_000)]
 
 
 @pytest.mark.parametrize("sfx", ALL)
