@@ -708,20 +708,26 @@ __global__ __launch_bounds__(256) void argreduce_row(ArgArgs<T> p) {
   constexpr int V = 16 / (int)sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(V)));
   const int lane = threadIdx.x & 63;
-  const int64_t o = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (o >= p.outputs) return;
+  // one wavefront per (output, chunk of the axis): with few outputs and a long axis the axis is cut (chunk starts are
+  // multiples of the vector) and the chunks' results go to the workspace for argreduce_merge
+  const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (unit >= p.outputs * p.chunks) return;
+  const int64_t chunk = unit / p.outputs, o = unit - chunk * p.outputs;
   int64_t a_off, v_off, i_off;
   decode3(p, o, a_off, v_off, i_off);
-  const T* src = p.a + a_off;
+  const int64_t l0 = chunk * p.chunk_len;
+  const int64_t len = (l0 + p.chunk_len < p.L) ? p.chunk_len : p.L - l0;
+  const T* row = p.a + a_off;
+  const T* src = row + l0 * p.a_axis_stride;
   T best = (T)0;
   int64_t at = 0;
   bool has = false;
   auto take = [&](T v, int64_t l) {
-    if (v == v && (!has || beats<T, MAXOP>(v, best))) { best = v; at = l; has = true; }
+    if (v == v && (!has || beats<T, MAXOP>(v, best))) { best = v; at = l0 + l; has = true; }
   };
   if constexpr (VEC) {
     const vec_t* vs = (const vec_t*)src;
-    const int64_t nvec = p.L / V;
+    const int64_t nvec = len / V;
     int64_t v = lane;
     for (; v + 192 < nvec; v += 256) {   // four 16-byte loads in flight per lane, taken in position order
       const vec_t x0 = vs[v], x1 = vs[v + 64], x2 = vs[v + 128], x3 = vs[v + 192];
@@ -739,9 +745,9 @@ __global__ __launch_bounds__(256) void argreduce_row(ArgArgs<T> p) {
 #pragma unroll
       for (int e = 0; e < V; ++e) take(x0[e], v * V + e);
     }
-    for (int64_t l = nvec * V + lane; l < p.L; l += 64) take(src[l], l);
+    for (int64_t l = nvec * V + lane; l < len; l += 64) take(src[l], l);
   } else {
-    for (int64_t l = lane; l < p.L; l += 64) take(src[l * p.a_axis_stride], l);
+    for (int64_t l = lane; l < len; l += 64) take(src[l * p.a_axis_stride], l);
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) {
@@ -751,10 +757,137 @@ __global__ __launch_bounds__(256) void argreduce_row(ArgArgs<T> p) {
     if (oh && (!has || beats<T, MAXOP>(ov, best) || (ov == best && oa < at))) { best = ov; at = oa; has = true; }
   }
   if (lane == 0) {
-    const T first = src[0];
-    if (!(first == first) || !has) { best = first; at = 0; }
-    p.val[v_off] = best;
-    p.idx[i_off] = at;
+    if (chunk == 0) {
+      const T first = row[0];
+      if (!(first == first) || !has) { best = first; at = 0; has = true; }
+    }
+    if (p.chunks > 1) {
+      p.ws_val[chunk * p.outputs + o] = best;
+      p.ws_idx[chunk * p.outputs + o] = has ? at : -1;
+    } else {
+      p.val[v_off] = best;
+      p.idx[i_off] = at;
+    }
+  }
+}
+
+// Many SHORT rows along their unit-stride axis (the class of each row of a [batch x classes] matrix): `lanes` lanes (a
+// power of two <= 32) share a row, one 16-byte vector each; a lane keeps the first best of its elements that are not
+// NaN, the lanes of a row merge by (better value, lower position), and a NaN in position 0 overrides, as above.
+template <typename T, bool MAXOP>
+__global__ __launch_bounds__(256) void argreduce_rows_short(ArgArgs<T> p, int lanes) {
+  constexpr int V = 16 / (int)sizeof(T);
+  constexpr int U = 4;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const int lane = threadIdx.x & 63;
+  const int j = lane & (lanes - 1), sub = lane / lanes, rows_per_step = 64 / lanes;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t row0 = wave * (int64_t)(U * rows_per_step) + sub;
+  const int64_t nvec = p.L / V;
+  vec_t x[U];
+  int64_t v_off[U], i_off[U];
+  bool ok[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t o = row0 + (int64_t)u * rows_per_step;
+    ok[u] = o < p.outputs && j < nvec;
+    int64_t a_off;
+    decode3(p, o < p.outputs ? o : 0, a_off, v_off[u], i_off[u]);
+    x[u] = *((const vec_t*)(p.a + a_off) + (j < nvec ? j : 0));
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    T best = (T)0;
+    int64_t at = 0;
+    bool has = false;
+    if (ok[u]) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const T v = x[u][e];
+        if (v == v && (!has || beats<T, MAXOP>(v, best))) { best = v; at = (int64_t)j * V + e; has = true; }
+      }
+    }
+    const T first = __shfl(x[u][0], lane - j, 64);   // element 0 of the row sits in the group's first lane
+    for (int d = lanes >> 1; d >= 1; d >>= 1) {
+      const T ov = __shfl_xor(best, d, 64);
+      const int64_t oa = (int64_t)__shfl_xor((long long)at, d, 64);
+      const bool oh = __shfl_xor((int)has, d, 64) != 0;
+      if (oh && (!has || beats<T, MAXOP>(ov, best) || (ov == best && oa < at))) { best = ov; at = oa; has = true; }
+    }
+    if (j == 0 && ok[u]) {
+      if (!(first == first) || !has) { best = first; at = 0; }
+      p.val[v_off[u]] = best;
+      p.idx[i_off[u]] = at;
+    }
+  }
+}
+
+// A walk down the rows of a matrix with FEW columns (the outputs are one unit-stride run of at most half a workgroup of
+// 16-byte lanes): lanes over the columns x 256 / cx row classes as in reduce_cols_narrow, every lane VEC outputs with
+// their own (value, position), row classes merged through LDS by (better value, lower position), so any merge order
+// gives the serial walk's answer; NaN is never taken except from row 0 (the chunk that holds it checks). Chunks of the
+// axis over the grid; their results go to the workspace in axis order for argreduce_merge.
+template <typename T, bool MAXOP>
+__global__ __launch_bounds__(256) void argreduce_cols_narrow(ArgArgs<T> p, int cx) {
+  constexpr int V = 16 / (int)sizeof(T);
+  constexpr int U = 4;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  __shared__ T s_val[256][V];
+  __shared__ int64_t s_idx[256][V];
+  const int ry = 256 / cx;
+  const int xq = (int)threadIdx.x % cx, yq = (int)threadIdx.x / cx;
+  const int64_t col = (int64_t)xq * V;
+  const bool active = yq < ry;
+  const int64_t l0 = (int64_t)blockIdx.x * p.chunk_len;
+  const int64_t l1 = (l0 + p.chunk_len < p.L) ? l0 + p.chunk_len : p.L;
+  T best[V];
+  int64_t at[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) { best[e] = (T)0; at[e] = -1; }
+  auto take = [&](const vec_t& v, int64_t l) {
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+      if (v[e] == v[e] && (at[e] < 0 || beats<T, MAXOP>(v[e], best[e]))) { best[e] = v[e]; at[e] = l; }
+  };
+  const T* src = p.a + col;
+  if (active) {
+    int64_t l = l0 + yq;
+    for (; l + (int64_t)(U - 1) * ry < l1; l += (int64_t)U * ry) {
+      vec_t v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load((const vec_t*)(src + (l + (int64_t)u * ry) * p.a_axis_stride));
+#pragma unroll
+      for (int u = 0; u < U; ++u) take(v[u], l + (int64_t)u * ry);
+    }
+    for (; l < l1; l += ry) take(*(const vec_t*)(src + l * p.a_axis_stride), l);
+  }
+#pragma unroll
+  for (int e = 0; e < V; ++e) { s_val[threadIdx.x][e] = best[e]; s_idx[threadIdx.x][e] = at[e]; }
+  __syncthreads();
+  if (active && yq == 0) {
+    for (int yy = 1; yy < ry; ++yy)
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const T ov = s_val[yy * cx + xq][e];
+        const int64_t oa = s_idx[yy * cx + xq][e];
+        if (oa >= 0 && (at[e] < 0 || beats<T, MAXOP>(ov, best[e]) || (ov == best[e] && oa < at[e]))) { best[e] = ov; at[e] = oa; }
+      }
+    if (blockIdx.x == 0) {   // row 0 holding a NaN overrides; a column of nothing but NaN reports row 0 as well
+      const vec_t first = *(const vec_t*)src;
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        if (!(first[e] == first[e]) || at[e] < 0) { best[e] = first[e]; at[e] = 0; }
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      if (p.chunks > 1) {
+        p.ws_val[(int64_t)blockIdx.x * p.outputs + col + e] = best[e];
+        p.ws_idx[(int64_t)blockIdx.x * p.outputs + col + e] = at[e];
+      } else {
+        p.val[(col + e) * p.v_stride[0]] = best[e];
+        p.idx[(col + e) * p.i_stride[0]] = at[e];
+      }
+    }
   }
 }
 
@@ -792,11 +925,69 @@ static int argreduce(const char* fn, int op, int rank, const int64_t* shape, int
   if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many output elements", fn);
   g.chunks = 1; g.chunk_len = g.L; g.ws_val = nullptr; g.ws_idx = nullptr;
   const dim3 block(256);
+  constexpr int64_t V = 16 / (int64_t)sizeof(T);
+  // chunk partials [chunk][output]: values, then positions
+  auto chunk_workspace = [&](int64_t chunks, int64_t len) {
+    const size_t val_bytes = ((size_t)chunks * (size_t)g.outputs * sizeof(T) + 255) / 256 * 256;
+    char* base = chunks > 1 ? (char*)gemm::splitk_workspace(val_bytes + (size_t)chunks * (size_t)g.outputs * sizeof(int64_t)) : nullptr;
+    if (base) { g.chunks = (int)chunks; g.chunk_len = len; g.ws_val = (T*)base; g.ws_idx = (int64_t*)(base + val_bytes); }
+  };
+  auto merge_chunks = [&]() {
+    AM_TRY(check_launch("argreduce"));
+    const dim3 mgrid((unsigned)((g.outputs + 255) / 256));
+    if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_merge<T, true>), mgrid, block, 0, stream(), g);
+    else hipLaunchKernelGGL((argreduce_merge<T, false>), mgrid, block, 0, stream(), g);
+    return check_launch("argreduce_merge");
+  };
+  const bool aligned = (uintptr_t)g.a % 16 == 0;
+  // few columns, a walk down many rows
+  if (g.ndim == 1 && g.a_stride[0] == 1 && iabs64(g.a_axis_stride) > 1 && g.outputs % V == 0 && g.outputs / V <= 128 && g.L >= 512 &&
+      g.a_axis_stride >= g.outputs && g.a_axis_stride % V == 0 && aligned) {
+    int64_t chunks = (int64_t)num_cus() * 2;
+    if (chunks > g.L / 256) chunks = g.L / 256;
+    if (chunks >= 2) {
+      const int64_t len = (g.L + chunks - 1) / chunks;
+      chunk_workspace((g.L + len - 1) / len, len);
+    }
+    const dim3 grid((unsigned)g.chunks);
+    const int cx = (int)(g.outputs / V);
+    if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_cols_narrow<T, true>), grid, block, 0, stream(), g, cx);
+    else hipLaunchKernelGGL((argreduce_cols_narrow<T, false>), grid, block, 0, stream(), g, cx);
+    return g.chunks > 1 ? merge_chunks() : check_launch("argreduce_cols_narrow");
+  }
+  // many short rows along their unit-stride axis
+  if (g.a_axis_stride == 1 && g.L % V == 0 && g.L / V <= 32 && g.outputs >= 4096 && aligned) {
+    bool rows_aligned = true;
+    for (int d = 0; d < g.ndim; ++d) rows_aligned = rows_aligned && g.a_stride[d] % V == 0;
+    if (rows_aligned) {
+      int lanes = 1;
+      while (lanes < g.L / V) lanes *= 2;
+      const int64_t rows_per_wg = 4 * 4 * (64 / lanes);
+      const int64_t sb = (g.outputs + rows_per_wg - 1) / rows_per_wg;
+      if (sb < ((int64_t)1 << 31)) {
+        if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_rows_short<T, true>), dim3((unsigned)sb), block, 0, stream(), g, lanes);
+        else hipLaunchKernelGGL((argreduce_rows_short<T, false>), dim3((unsigned)sb), block, 0, stream(), g, lanes);
+        return check_launch("argreduce_rows_short");
+      }
+    }
+  }
   if (row_kernel) {
-    constexpr int64_t V = 16 / (int64_t)sizeof(T);
-    bool vec = g.a_axis_stride == 1 && ((uintptr_t)g.a % 16 == 0);
+    bool vec = g.a_axis_stride == 1 && aligned;
     for (int d = 0; d < g.ndim && vec; ++d) vec = g.a_stride[d] % V == 0;
-    const dim3 grid((unsigned)bx);
+    // few outputs, a long axis: chunks of the axis over several wavefronts (16 per CU over the chip, 4096 elements or more each)
+    const int64_t want_waves = (int64_t)num_cus() * 16;
+    if (g.outputs < want_waves / 2 && g.L >= 8192) {
+      int64_t chunks = (want_waves + g.outputs - 1) / g.outputs;
+      if (chunks > g.L / 4096) chunks = g.L / 4096;
+      if (chunks > 1024) chunks = 1024;
+      if (chunks >= 2) {
+        int64_t len = (g.L + chunks - 1) / chunks;
+        len = (len + 255) / 256 * 256;
+        chunk_workspace((g.L + len - 1) / len, len);
+      }
+    }
+    const int64_t rb = (g.outputs * g.chunks + 3) / 4;
+    const dim3 grid((unsigned)rb);
     if (op == AM_RED_MAX) {
       if (vec) hipLaunchKernelGGL((argreduce_row<T, true, true>), grid, block, 0, stream(), g);
       else hipLaunchKernelGGL((argreduce_row<T, true, false>), grid, block, 0, stream(), g);
@@ -804,6 +995,7 @@ static int argreduce(const char* fn, int op, int rank, const int64_t* shape, int
       if (vec) hipLaunchKernelGGL((argreduce_row<T, false, true>), grid, block, 0, stream(), g);
       else hipLaunchKernelGGL((argreduce_row<T, false, false>), grid, block, 0, stream(), g);
     }
+    if (g.chunks > 1) return merge_chunks();
   } else {
     // too few outputs to fill the chip: cut the axis (eight workgroups per CU, at least 64 slices per chunk)
     const int64_t want = (int64_t)num_cus() * 8;
@@ -812,19 +1004,12 @@ static int argreduce(const char* fn, int op, int rank, const int64_t* shape, int
       if (chunks > g.L / 64) chunks = g.L / 64;
       if (chunks > 1024) chunks = 1024;
       const int64_t len = (g.L + chunks - 1) / chunks;
-      chunks = (g.L + len - 1) / len;
-      const size_t val_bytes = ((size_t)chunks * (size_t)g.outputs * sizeof(T) + 255) / 256 * 256;
-      char* base = chunks > 1 ? (char*)gemm::splitk_workspace(val_bytes + (size_t)chunks * (size_t)g.outputs * sizeof(int64_t)) : nullptr;
-      if (base) { g.chunks = (int)chunks; g.chunk_len = len; g.ws_val = (T*)base; g.ws_idx = (int64_t*)(base + val_bytes); }
+      chunk_workspace((g.L + len - 1) / len, len);
     }
     const dim3 grid((unsigned)bx, (unsigned)g.chunks);
     if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_seq<T, true>), grid, block, 0, stream(), g);
     else hipLaunchKernelGGL((argreduce_seq<T, false>), grid, block, 0, stream(), g);
-    if (g.chunks > 1) {
-      AM_TRY(check_launch("argreduce"));
-      if (op == AM_RED_MAX) hipLaunchKernelGGL((argreduce_merge<T, true>), dim3((unsigned)bx), block, 0, stream(), g);
-      else hipLaunchKernelGGL((argreduce_merge<T, false>), dim3((unsigned)bx), block, 0, stream(), g);
-    }
+    if (g.chunks > 1) return merge_chunks();
   }
   return check_launch("argreduce");
 }

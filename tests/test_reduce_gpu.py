@@ -267,6 +267,39 @@ def test_argmax_nan_rules(hip, oracle, sfx):
 
 
 @pytest.mark.parametrize("sfx", ALL)
+def test_argmax_tall_skinny_and_long_rows(hip, oracle, sfx):
+    """Positions and values of the first maximum / minimum on shapes away from square: many short rows (lane groups per
+    row), a walk down many rows of few columns (workgroup-wide, chunks merged in axis order), few long rows (chunks of a
+    row over several wavefronts); tie-heavy data, so that 'first' matters across lanes, row classes and chunks, and
+    NaN in row 0, elsewhere, and everywhere for floats. Bit-exact against the serial walk."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("argmax-shapes", sfx))
+    for shape, ax in [((70_000, 64), 1), ((9_000, 16), 1), ((5_000, 24), 1), ((4_100, 128), 1), ((70_000, 64), 0), ((3_000, 512), 0),
+                      ((600, 8), 0), ((5, 300_000), 1), ((64, 20_000), 1), ((300_000, 5), 0)]:
+        for ties in (True, False):
+            x = rng.integers(-3, 4, shape).astype(dt) if ties else fill(rng, shape, dt)
+            if sfx in ("f32", "f64"):
+                other = 1 - ax
+                idx = [slice(None), slice(None)]
+                n_other = shape[other]
+                def at(o, l):
+                    k = [0, 0]; k[other] = o; k[ax] = l; return tuple(k)
+                x[at(0, 0)] = np.nan                       # NaN in position 0: stays
+                if n_other > 1: x[at(1, shape[ax] // 2)] = np.nan   # NaN elsewhere: never taken
+                if n_other > 2:
+                    k = [slice(None), slice(None)]; k[other] = 2; x[tuple(k)] = np.nan      # nothing but NaN
+                if n_other > 3:
+                    k = [slice(None), slice(None)]; k[other] = 3; k[ax] = slice(1, None); x[tuple(k)] = np.nan   # only position 0 is a number
+            dx = hip.toHip(x)
+            for op, fn in (("max", hip.argmax_max), ("min", hip.argmin_min)):
+                say("argreduce shapes", sfx, shape, ax, ties, op)
+                gi, gv = fn(dx, ax)
+                wi, wv = oracle.argreduce(op, x, ax)
+                assert gi.shape == wi.shape and np.array_equal(gi.toCpu(), wi), (shape, ax, ties, op)
+                assert np.array_equal(gv.toCpu(), wv, equal_nan=True), (shape, ax, ties, op)
+
+
+@pytest.mark.parametrize("sfx", ALL)
 def test_column_walks_with_16_byte_lanes(hip, oracle, sfx):
     """Walks across a unit-stride dimension take 16 bytes of adjacent outputs per lane when extents,
     strides and base addresses allow it, and one output per lane otherwise; both fold every output
