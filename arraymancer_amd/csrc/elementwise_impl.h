@@ -368,7 +368,7 @@ __global__ __launch_bounds__(kThreads) void ew_rows(RowsArgs<T, D> p) {
   }
 }
 
-// Rows shorter than a quarter of a column tile (a [batch x features] activation plus its bias with a few hundred
+// Rows shorter than half a column tile (a [batch x features] activation plus its bias with a few hundred
 // features, per-pixel or per-row factors on images) would leave most of ew_rows' lanes idle. Same operand kinds, other
 // decomposition: the problem is the flat sequence of its rows x L / VEC vectors, consecutive lanes take consecutive
 // vectors (so a wavefront's access is one contiguous run wherever the rows themselves are contiguous), and every
@@ -823,6 +823,67 @@ __global__ __launch_bounds__(kThreads) void ew3_rows(TriArgs<T> p) {
   }
 }
 
+// The three-operand bodies on rows shorter than half a column tile (the gate arithmetic of a GRU cell on column slices
+// [_, a ..< b] of [batch x 3 hidden] buffers with a few hundred hidden units, nnp_gru.nim:73-88): the flat form, as
+// ew_short_rows — consecutive lanes take consecutive 16-byte vectors of the rows x L / VEC of them, each vector finds its row
+// and from it every operand's row offset by division. Operand modes as in ew3_rows (a row vector is an ordinary vector
+// operand here: its outer strides are zero). Requires L % VEC == 0; rows x L / VEC < 2^31.
+template <typename T, int OP>
+__global__ __launch_bounds__(kThreads) void ew3_short_rows(TriArgs<T> p, uint32_t lv, uint32_t total) {
+  typedef typename Traits<T>::V V;
+  constexpr int VEC = Traits<T>::kVec;
+  const int am = p.a_mode, bm = p.b_mode, cm = p.c_mode;
+  const uint32_t v0 = blockIdx.x * (uint32_t)(kThreads * kUnroll) + threadIdx.x;
+  bool live[kUnroll];
+  int64_t offd[kUnroll], offa[kUnroll], offb[kUnroll], offc[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const uint32_t v = v0 + (uint32_t)u * kThreads;
+    live[u] = v < total;
+    const uint32_t vv = live[u] ? v : 0;
+    const uint32_t row = vv / lv;
+    const int64_t col = (int64_t)(vv - row * lv) * VEC;
+    int64_t od = col, oa = am >= kTriRowScalar ? 0 : col, ob = bm >= kTriRowScalar ? 0 : col, oc = cm >= kTriRowScalar ? 0 : col;
+    uint32_t rem = row;
+#pragma unroll
+    for (int d = AM_MAXRANK - 2; d >= 0; --d) {
+      if (d < p.rank) {
+        const uint32_t ext = (uint32_t)p.shape[d];
+        const uint32_t q = rem / ext;
+        const int64_t cidx = (int64_t)(rem - q * ext);
+        rem = q;
+        od += cidx * p.sd[d]; oa += cidx * p.sa[d]; ob += cidx * p.sb[d]; oc += cidx * p.sc[d];
+      }
+    }
+    offd[u] = od; offa[u] = oa; offb[u] = ob; offc[u] = oc;
+  }
+  V av[kUnroll], bv[kUnroll], cv[kUnroll];
+  T asc[kUnroll], bsc[kUnroll], csc[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) { av[u] = V{}; bv[u] = V{}; cv[u] = V{}; asc[u] = (T)0; bsc[u] = p.b_imm; csc[u] = p.c_imm; }
+#define AM_TRI_FLAT_LOADS(mode, vec, sc, base, off)                                                                       \
+  if (mode == kTriVecNt) {                                                                                                \
+    _Pragma("unroll") for (int u = 0; u < kUnroll; ++u) vec[u] = __builtin_nontemporal_load(launder((const V*)(base + off[u]))); \
+  } else if (mode == kTriVec || mode == kTriRowVector) {                                                                  \
+    _Pragma("unroll") for (int u = 0; u < kUnroll; ++u) vec[u] = *(const V*)(base + off[u]);                              \
+  } else if (mode == kTriRowScalar) {                                                                                     \
+    _Pragma("unroll") for (int u = 0; u < kUnroll; ++u) sc[u] = base[off[u]];                                             \
+  }
+  AM_TRI_FLAT_LOADS(am, av, asc, p.a, offa)
+  AM_TRI_FLAT_LOADS(bm, bv, bsc, p.b, offb)
+  AM_TRI_FLAT_LOADS(cm, cv, csc, p.c, offc)
+#undef AM_TRI_FLAT_LOADS
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    V r;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+      r[e] = TriOp<T, OP>::apply(am >= kTriRowScalar ? asc[u] : av[u][e], bm >= kTriRowScalar ? bsc[u] : bv[u][e],
+                                 cm >= kTriRowScalar ? csc[u] : cv[u][e]);
+    if (live[u]) __builtin_nontemporal_store(r, (V*)(p.dst + offd[u]));
+  }
+}
+
 template <typename T, int OP, typename IDX>
 __global__ __launch_bounds__(kThreads) void ew3_generic(TriArgs<T> p) {
   const IDX n = (IDX)p.n;
@@ -935,8 +996,8 @@ static int run(int rank, const int64_t* shape, D* dst, const int64_t* sd, const 
   const int64_t tiles_per_row = (L + tile - 1) / tile;
   // Short rows would leave most lanes of a tile idle: whole vectors per row -> the flat form of the kernel, else the
   // generic kernel (and so does a row shorter than one 16-byte vector, which the clamped loads would overrun).
-  const bool short_rows = ok && rows > 1 && L < tile / 4 && L >= VEC && L % VEC == 0 && rows * (L / VEC) < ((int64_t)1 << 31);
-  if (ok && !short_rows && ((rows > 1 && L < tile / 4) || L < VEC)) ok = false;
+  const bool short_rows = ok && rows > 1 && L < tile / 2 && L >= VEC && L % VEC == 0 && rows * (L / VEC) < ((int64_t)1 << 31);
+  if (ok && !short_rows && ((rows > 1 && L < tile / 2) || L < VEC)) ok = false;
   if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31) || rows >= ((int64_t)1 << 31))) ok = false;
   if (!ok) {
     // Two collapsed dims with unit strides on different axes: the LDS-tiled kernel.
@@ -1270,7 +1331,10 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
   const int64_t tile = (int64_t)kThreads * VEC * kUnroll;
   const int64_t tiles_per_row = (L + tile - 1) / tile;
   // (rows shorter than one vector: the streaming kernel's clamped loads would overrun them)
-  if (ok && ((rows > 1 && L < tile / 8) || L < VEC)) ok = false;
+  // rows shorter than half a column tile would leave most lanes idle (a quarter used: 2.7 TB/s): the flat form when a row is
+  // whole vectors, else the generic kernel
+  const bool short_rows = ok && rows > 1 && L < tile / 2 && L >= VEC && L % VEC == 0 && rows * (L / VEC) < ((int64_t)1 << 31);
+  if (ok && !short_rows && ((rows > 1 && L < tile / 2) || L < VEC)) ok = false;
   if (ok && (tiles_per_row * rows >= ((int64_t)1 << 31) || rows >= ((int64_t)1 << 31))) ok = false;
   g.n = n; g.L = L;
   if (ok) {
@@ -1285,6 +1349,11 @@ static int run3(int rank, const int64_t* shape, T* dst, const int64_t* sd, const
     g.rank = in;
     g.tiles_per_row = (uint32_t)tiles_per_row;
     g.rows = (uint32_t)rows;
+    if (short_rows) {
+      const uint32_t lv = (uint32_t)(L / VEC), total = (uint32_t)(rows * (L / VEC));
+      hipLaunchKernelGGL((ew3_short_rows<T, OP>), dim3((total + kThreads * kUnroll - 1) / (kThreads * kUnroll)), dim3(kThreads), 0, stream(), g, lv, total);
+      return check_launch("ew3_short_rows");
+    }
     const int64_t cap = (int64_t)num_cus() * 32;
     const int64_t col_blocks = tiles_per_row < cap ? tiles_per_row : cap;
     int64_t row_groups = cap / col_blocks;
