@@ -304,40 +304,55 @@ static int dispatch_cols_narrow(int op, Args<T>& g) {
   }
 }
 
-// Many SHORT rows folded along their unit-stride axis (row sums of [rows x 16 ... 128] tensors): a wavefront per
-// row would move 64 ... 512 bytes per six-step butterfly, a lane per row reads 16 bytes of every cache line it touches
-// per instruction. Here `lanes` lanes (a power of two <= 32) share a row, one 16-byte vector each, so that a
-// wavefront's load instruction is one contiguous run of 64 / lanes rows; each lane folds its vector in element order,
-// then the lanes of a row fold in a fixed butterfly. Four row groups per wavefront are in flight.
+// Many SHORT rows folded along their unit-stride axis (row sums of [rows x 4 ... 1024] tensors): a wavefront per
+// row would move 16 ... 4096 bytes per six-step butterfly, a lane per row reads 16 bytes of every cache line it touches
+// per instruction. Here `lanes` lanes (a power of two <= 64) share a row, VPL 16-byte vectors each (1, 2 or 4: rows
+// of up to 256 vectors), so that a wavefront's load instruction is one contiguous run of 64 / lanes rows; each lane folds
+// its vectors in element order, then the lanes of a row fold in a fixed butterfly. Several row groups per wavefront are
+// in flight (eight loads per lane).
 // Measured, f32 sum over axis 1: [1048576 x 64] 260 us before (a wavefront per row) -> 48 us; [4194304 x 16] 154 -> 51 us.
-template <typename T, int OP, bool STREAM>
+template <typename T, int OP, bool STREAM, int VPL>
 __global__ __launch_bounds__(256) void reduce_rows_short(Args<T> p, int lanes) {
   constexpr int V = 16 / (int)sizeof(T);
-  constexpr int U = 4;
+  constexpr int U = VPL >= 4 ? 2 : 4;
   typedef T vec_t __attribute__((ext_vector_type(V)));
   const int lane = threadIdx.x & 63;
   const int j = lane & (lanes - 1), sub = lane / lanes, rows_per_step = 64 / lanes;
   const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int64_t row0 = wave * (int64_t)(U * rows_per_step) + sub;
   const int64_t nvec = p.L / V;
-  vec_t x[U];
+  vec_t x[U][VPL];
   bool ok[U];
   int64_t d_off[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int64_t o = row0 + (int64_t)u * rows_per_step;
-    ok[u] = o < p.outputs && j < nvec;
+    ok[u] = o < p.outputs;
     int64_t a_off;
-    decode(p, o < p.outputs ? o : 0, a_off, d_off[u]);
-    const vec_t* at = (const vec_t*)(p.a + a_off) + (j < nvec ? j : 0);   // every lane loads, from inside its row
-    if constexpr (STREAM) x[u] = __builtin_nontemporal_load(at); else x[u] = *at;
+    decode(p, ok[u] ? o : 0, a_off, d_off[u]);
+    const vec_t* row = (const vec_t*)(p.a + a_off);
+#pragma unroll
+    for (int w = 0; w < VPL; ++w) {
+      const int64_t v = j + (int64_t)w * lanes;
+      const vec_t* at = row + (v < nvec ? v : 0);   // every lane loads, from inside its row
+      if constexpr (STREAM) x[u][w] = __builtin_nontemporal_load(at); else x[u][w] = *at;
+    }
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    T acc = x[u][0];
+    T acc = (T)0;
+    bool has = false;
 #pragma unroll
-    for (int e = 1; e < V; ++e) acc = Fold<T, OP>::apply(acc, x[u][e]);
-    bool has = ok[u];
+    for (int w = 0; w < VPL; ++w) {
+      if (j + (int64_t)w * lanes < nvec) {
+        T part = x[u][w][0];
+#pragma unroll
+        for (int e = 1; e < V; ++e) part = Fold<T, OP>::apply(part, x[u][w][e]);
+        acc = has ? Fold<T, OP>::apply(acc, part) : part;
+        has = true;
+      }
+    }
+    has = has && ok[u];
     for (int d = lanes >> 1; d >= 1; d >>= 1) {
       const T other = __shfl_xor(acc, d, 64);
       const int other_has = __shfl_xor((int)has, d, 64);
@@ -352,32 +367,34 @@ __global__ __launch_bounds__(256) void reduce_rows_short(Args<T> p, int lanes) {
   }
 }
 
-// Whether reduce_rows_short applies, and with how many lanes per row.
+// Whether reduce_rows_short applies, and with how many lanes per row (*vpl: 16-byte vectors per lane, 1, 2 or 4).
 template <typename T>
-static int rows_short_lanes(const Args<T>& g) {
+static int rows_short_lanes(const Args<T>& g, int* vpl) {
   constexpr int64_t V = 16 / (int64_t)sizeof(T);
-  if (g.a_axis_stride != 1 || g.L % V != 0 || g.L / V > 32 || g.outputs < 4096) return 0;
+  if (g.a_axis_stride != 1 || g.L % V != 0 || g.L / V > 256 || g.outputs < 4096) return 0;
   if ((uintptr_t)g.a % 16 != 0) return 0;
   for (int d = 0; d < g.ndim; ++d)
     if (g.a_stride[d] % V != 0) return 0;
   int lanes = 1;
-  while (lanes < g.L / V) lanes *= 2;
+  while (lanes < g.L / V && lanes < 64) lanes *= 2;
+  const int64_t per_lane = (g.L / V + lanes - 1) / lanes;
+  *vpl = per_lane <= 1 ? 1 : per_lane <= 2 ? 2 : 4;
   return lanes;
 }
 
-template <typename T>
-static int dispatch_rows_short(int op, Args<T>& g, int lanes) {
-  constexpr int U = 4;
+template <typename T, int VPL>
+static int dispatch_rows_short_vpl(int op, Args<T>& g, int lanes) {
+  constexpr int U = VPL >= 4 ? 2 : 4;
   const int64_t rows_per_wg = 4 * U * (64 / lanes);
   const int64_t bx = (g.outputs + rows_per_wg - 1) / rows_per_wg;
   if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "reduce: too many output elements");
   g.chunks = 1; g.chunk_len = g.L; g.ws = nullptr;
   const bool stream_loads = (double)g.outputs * (double)g.L * sizeof(T) > nt_threshold_bytes();
   const dim3 grid((unsigned)bx), block(256);
-#define AM_ROWS_SHORT(OPC)                                                                                          \
-  do {                                                                                                              \
-    if (stream_loads) hipLaunchKernelGGL((reduce_rows_short<T, OPC, true>), grid, block, 0, stream(), g, lanes);    \
-    else hipLaunchKernelGGL((reduce_rows_short<T, OPC, false>), grid, block, 0, stream(), g, lanes);                \
+#define AM_ROWS_SHORT(OPC)                                                                                               \
+  do {                                                                                                                   \
+    if (stream_loads) hipLaunchKernelGGL((reduce_rows_short<T, OPC, true, VPL>), grid, block, 0, stream(), g, lanes);    \
+    else hipLaunchKernelGGL((reduce_rows_short<T, OPC, false, VPL>), grid, block, 0, stream(), g, lanes);                \
   } while (0)
   switch (op) {
     case AM_RED_SUM: AM_ROWS_SHORT(AM_RED_SUM); break;
@@ -387,6 +404,13 @@ static int dispatch_rows_short(int op, Args<T>& g, int lanes) {
   }
 #undef AM_ROWS_SHORT
   return check_launch("reduce_rows_short");
+}
+
+template <typename T>
+static int dispatch_rows_short(int op, Args<T>& g, int lanes, int vpl) {
+  if (vpl == 1) return dispatch_rows_short_vpl<T, 1>(op, g, lanes);
+  if (vpl == 2) return dispatch_rows_short_vpl<T, 2>(op, g, lanes);
+  return dispatch_rows_short_vpl<T, 4>(op, g, lanes);
 }
 
 // Whether reduce_seq_vec applies: the innermost output dimension is a unit-stride run in the source
@@ -537,7 +561,10 @@ static int reduce_axis(const char* fn, int op, int rank, const int64_t* shape, i
   int64_t best_other = -1;
   for (int d = 0; d < g.ndim; ++d) if (best_other < 0 || iabs64(g.a_stride[d]) < best_other) best_other = iabs64(g.a_stride[d]);
   if (best_other >= 0 && iabs64(g.a_axis_stride) > best_other && cols_narrow_ok(g)) return dispatch_cols_narrow<T>(op, g);
-  if (const int lanes = rows_short_lanes(g)) return dispatch_rows_short<T>(op, g, lanes);
+  {
+    int vpl = 1;
+    if (const int lanes = rows_short_lanes(g, &vpl)) return dispatch_rows_short<T>(op, g, lanes, vpl);
+  }
   const bool row_kernel = g.L >= 64 && (best_other < 0 || iabs64(g.a_axis_stride) < best_other || g.outputs < 1024);
   return dispatch<T>(op, g, row_kernel, 0);
 }

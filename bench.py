@@ -317,7 +317,38 @@ def other_workloads(am, timer, steps, warmup, ceilings):
             roof["frac_of_measured_copy_ceiling"] = round(gbs / (copy_ceiling * 1e3), 4)
         out.append(dict(workload=f"f32 8192x8192 {name}", unit="GB/s", dtype="f32", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 4),
                         same_buffers_every_step_ms=round(ev / steps * 1e3, 4), roofline=roof))
+    # --- the same kinds of pass on operands that are not square row-major matrices: a transposed operand, and the
+    # [batch x features] shapes of a dense layer (bias add, bias gradient, row sums, weight gradient). Three buffer
+    # sets round robin for the HBM-bound ones (0.4 - 0.8 GiB per set).
+    def hbm_entry(workload, launches, nbytes):
+        cold = run_rotating(timer, launches, max(steps // len(launches), 4))
+        gbs = nbytes / cold / 1e9
+        out.append(dict(workload=workload, unit="GB/s", dtype="f32", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 4),
+                        roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4),
+                                      protocol=f"{len(launches)} buffer sets round robin: every byte from HBM")))
+    hbm_entry("f32 8192x8192 X + Z^T (Z a transposed view)",
+              [(lambda i=i: th._binary_into("add", dYs[i], dXs[i], dXs[(i + 1) % 3].transpose())) for i in range(3)], 3 * 8192 * 8192 * 4)
     del dXs, dYs
+    T = np.random.default_rng(4004).uniform(-1, 1, (65536, 512)).astype(np.float32)
+    dTs = [am.toHip(T) for _ in range(3)]
+    dOs = [am.empty((65536, 512), np.float32) for _ in range(3)]
+    bias = am.toHip(np.random.default_rng(4005).uniform(-1, 1, (1, 512)).astype(np.float32)).broadcast((65536, 512))
+    hbm_entry("f32 65536x512 X +. b[1,512] (bias of a dense layer)", [(lambda i=i: th._binary_into("add", dOs[i], dTs[i], bias)) for i in range(3)],
+              2 * T.nbytes + 2048)
+    hbm_entry("f32 sum(X[65536,512], axis=0) (bias gradient)", [(lambda i=i: am.sum(dTs[i], 0)) for i in range(3)], T.nbytes)
+    hbm_entry("f32 sum(X[65536,512], axis=1)", [(lambda i=i: am.sum(dTs[i], 1)) for i in range(3)], T.nbytes)
+    del dTs, dOs
+    dA = am.toHip(np.random.default_rng(1003).standard_normal((500, 65536)).astype(np.float32))
+    dB = am.toHip(np.random.default_rng(1004).standard_normal((65536, 800)).astype(np.float32))
+    dC = am.empty((500, 800), np.float32)
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), max(steps, 20), warmup, WARM_S)
+    fl = 2.0 * 500 * 800 * 65536
+    k = max(steps, 20)
+    out.append(dict(workload="f32 GEMM [500x65536].[65536x800] (weight gradient of a dense layer over a large batch: few tiles, long k)",
+                    unit="TFLOP/s", dtype="f32", value=round(fl * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 4),
+                    roofline=at_clock(dict(bound="mfma", achieved=round(fl / (ev / k) / 1e12, 3), peak=MFMA_F32_PEAK_TFLOPS, unit="TFLOP/s",
+                                           frac=round(fl / (ev / k) / 1e12 / MFMA_F32_PEAK_TFLOPS, 4)), MFMA_F32_PEAK_TFLOPS, timer.sclk_mhz)))
+    del dA, dB, dC
     out.append(bench_chain(am, timer, max(steps, 50), warmup))
     out.append(bench_ex02(am, timer, max(steps, 50), warmup))
     return out

@@ -146,7 +146,8 @@ def test_tall_skinny_reductions(hip, oracle, sfx):
     rng = np.random.default_rng(seed_of("tall-skinny", sfx))
     cases = [((70_000, 64), 0, None), ((5_000, 512), 0, None), ((3_000, 128), 0, (slice(None), slice(16, 80))), ((600, 8), 0, None),
              ((70_000, 64), 1, None), ((300_000, 16), 1, None), ((100_000, 24), 1, None), ((5_000, 8, 32), 2, None),
-             ((9_000, 128), 1, (slice(None), slice(8, 72))), ((4_100, 4), 1, None)]
+             ((9_000, 128), 1, (slice(None), slice(8, 72))), ((4_100, 4), 1, None), ((5_000, 512), 1, None), ((4_200, 1000), 1, None),
+             ((4_100, 264), 1, None), ((4_500, 520), 1, None)]
     for shape, ax, window in cases:
         for op in OPS:
             if op == "product" and sfx in ("f32", "f64") and shape[ax] > 3000:
