@@ -9,7 +9,7 @@ from ._lib import HipAllocError, HipError, load as load_library
 from .metadata import Layout, Step
 from .io_npy import read_npy, write_npy
 from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3, map3, bc_add, bc_div, bc_mod, bc_mul,
-                         bc_sub, bias_relu, conv2d, conv2d_into, dot, empty, gemm, gemm_batched, gemv, im2col, linear, map2, matmul, relu, scalar_op,
+                         bc_sub, bias_relu, conv2d, conv2d_into, conv2d_backward, col2im, im2col_folded, dot, empty, gemm, gemm_batched, gemv, im2col, linear, map2, matmul, relu, scalar_op,
                          sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, maxpool2d, tanh, relu_backward, sigmoid_backward,
                          tanh_backward, linear_backward, variance, std, sqrt, square, argmax_max, argmax,
@@ -20,7 +20,7 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
 
 __all__ = [
     "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
-    "toHip", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "conv2d", "conv2d_into", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
+    "toHip", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "im2col_folded", "col2im", "conv2d", "conv2d_into", "conv2d_backward", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
     "unary", "relu", "sigmoid", "bias_relu", "bc_add", "bc_sub", "bc_mul", "bc_div", "bc_mod",
     "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward",
     "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin", "maxpool2d_backward",

@@ -83,6 +83,8 @@ def _signatures():
         sig[f"am_hip_gemm_batched_{sfx}"] = (ci, [i64, i64, i64, i64, ct, vp, i64, i64, i64, vp, i64, i64, i64, ct,
                                                  vp, i64, i64, i64, ci, vp, i64, i64])
         sig[f"am_hip_im2col_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, i64, i64, i64, i64, vp])
+        sig[f"am_hip_im2col_strided_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, i64, i64, i64, i64, vp, i64, i64])
+        sig[f"am_hip_col2im_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, i64, i64, vp, i64, i64, i64, i64])
         sig[f"am_hip_gemv_{sfx}"] = (ci, [i64, i64, ct, vp, i64, i64, vp, i64, ct, vp, i64])
         sig[f"am_hip_dot_{sfx}"] = (ci, [i64, vp, i64, vp, i64, ctypes.POINTER(ct)])
         sig[f"am_hip_ew_binary_{sfx}"] = (ci, [ci, ci, vp, vp, vp, vp, vp, vp, vp])

@@ -72,6 +72,15 @@ def transpose(l: Layout) -> Layout:
     return Layout(l.shape[::-1], l.strides[::-1], l.offset)
 
 
+def permute(l: Layout, dims: Sequence[int]) -> Layout:
+    """The dimensions in the order `dims` (src/arraymancer/tensor/shapeshifting.nim:207-226): dimension i of the
+    result is dimension dims[i] of the input; no data moves."""
+    dims = tuple(int(d) for d in dims)
+    if sorted(dims) != list(range(len(l.shape))):
+        raise ValueError(f"permute: {dims} is not a permutation of the tensor's {len(l.shape)} dimensions")
+    return Layout(tuple(l.shape[d] for d in dims), tuple(l.strides[d] for d in dims), l.offset)
+
+
 class Step:
     """One slice in the reference's notation: first..last|step with INCLUSIVE ends;
     `first_from_end` / `last_from_end` are the `^n` forms (index = extent - n)."""

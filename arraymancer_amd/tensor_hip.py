@@ -140,6 +140,12 @@ class HipTensor:
     def T(self):
         return self.transpose()
 
+    def permute(self, *dims) -> "HipTensor":
+        """The dimensions in a new order, same data (src/arraymancer/tensor/shapeshifting.nim:207-226)."""
+        if len(dims) == 1 and not isinstance(dims[0], int):
+            dims = tuple(dims[0])
+        return HipTensor(md.permute(self.layout, dims), self.storage, self.dtype)
+
     def __getitem__(self, key) -> "HipTensor":
         return HipTensor(md.py_index(self.layout, key), self.storage, self.dtype)
 
@@ -482,6 +488,82 @@ def im2col(x: HipTensor, kernel_size, padding=(0, 0), stride=(1, 1)) -> HipTenso
     check(getattr(_lib.load(), f"am_hip_im2col_{x.sfx}")(
         N, C, H, W, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(x.data_ptr()), *x.strides, ctypes.c_void_p(col.data_ptr())))
     return col
+
+
+def im2col_folded(x: HipTensor, kernel_size, padding=(0, 0), stride=(1, 1)) -> HipTensor:
+    """[N, C, H, W] -> [C*kH*kW, N * H_out*W_out]: the column matrices of all images side by side (image n's columns
+    from n * H_out*W_out on), so that a product over the whole batch is one GEMM. Same entries as `im2col`."""
+    if x.rank != 4:
+        raise ValueError("im2col: input must be [N, C, H, W]")
+    N, C, H, W = x.shape
+    (kh, kw), (ph, pw), (sh, sw) = kernel_size, padding, stride
+    ho, wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    col = empty((C * kh * kw, N * ho * wo), x.dtype)
+    check(getattr(_lib.load(), f"am_hip_im2col_strided_{x.sfx}")(
+        N, C, H, W, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(x.data_ptr()), *x.strides, ctypes.c_void_p(col.data_ptr()),
+        ho * wo, N * ho * wo))
+    return col
+
+
+def col2im(col: HipTensor, channels: int, height: int, width: int, kernel_size, padding=(0, 0), stride=(1, 1)) -> HipTensor:
+    """col2im (src/arraymancer/nn_primitives/fallback/conv.nim:55-79): [C*kH*kW, H_out*W_out] -> [C, H, W], or for a
+    batch [N, C*kH*kW, H_out*W_out] -> [N, C, H, W] in one launch; pixels covered by several columns are summed."""
+    (kh, kw), (ph, pw), (sh, sw) = kernel_size, padding, stride
+    ho, wo = (height + 2 * ph - kh) // sh + 1, (width + 2 * pw - kw) // sw + 1
+    batched = col.rank == 3
+    c3 = col if batched else col.reshape(1, *col.shape)
+    if c3.rank != 3 or c3.shape[1] != channels * kh * kw or c3.shape[2] != ho * wo:
+        raise ValueError(f"col2im: column matrix of shape {col.shape} does not match the geometry")
+    if c3.strides[2] != 1:
+        c3 = c3.clone()
+    N = c3.shape[0]
+    out = empty((N, channels, height, width), col.dtype)
+    check(getattr(_lib.load(), f"am_hip_col2im_{col.sfx}")(
+        N, channels, height, width, kh, kw, ph, pw, sh, sw, ctypes.c_void_p(c3.data_ptr()), c3.strides[0], c3.strides[1],
+        ctypes.c_void_p(out.data_ptr()), *out.strides))
+    return out if batched else out.reshape(channels, height, width)
+
+
+def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None, padding, stride, grad_output: HipTensor):
+    """(grad_input, grad_weight, grad_bias) of conv2d_backward (src/arraymancer/nn_primitives/nnp_convolution.nim:65-107)
+    over im2colgemm_conv2d_gradient (fallback/conv.nim:107-145). The reference loops over the images (two GEMMs, an
+    im2col and a col2im each); here the batch is folded into the columns, g[C_out, N*P] = grad_output with its first
+    two axes swapped and col[C*kH*kW, N*P] the column matrices side by side, so that the whole pass is
+
+        grad_bias   = row sums of g                      (sum(3).sum(2).sum(0) of the reference)
+        grad_weight = g * col^T                          (one product with k = N*P; the per-image products summed)
+        grad_input  = col2im(kernel_col^T * g)           (one product, one gather)
+
+    Float tensors with unit stride and up to 96 input channels take grad_input as ONE launch instead: the convolution
+    of grad_output with the turned kernel. grad_bias is None when `bias` is."""
+    _same_dtype(input, weight, grad_output)
+    N, C, H, W = input.shape
+    co, ci, kh, kw = weight.shape
+    if ci != C:
+        raise ValueError(f"conv2d_backward: kernel expects {ci} input channels, input has {C}")
+    ho, wo = (H + 2 * padding[0] - kh) // stride[0] + 1, (W + 2 * padding[1] - kw) // stride[1] + 1
+    if grad_output.shape != (N, co, ho, wo):
+        raise ValueError(f"conv2d_backward: grad_output is {grad_output.shape}, the convolution's result is {(N, co, ho, wo)}")
+    P = ho * wo
+    g = grad_output.reshape(N, co, P).permute(1, 0, 2).clone().reshape(co, N * P)
+    grad_bias = tsum(g, axis=1).reshape(*bias.shape) if bias is not None else None
+    col = im2col_folded(input, (kh, kw), padding, stride)
+    kcol = weight.reshape(co, ci * kh * kw)
+    grad_weight = matmul(g, col.transpose()).reshape(co, ci, kh, kw)
+    if (input.dtype.kind == "f" and tuple(stride) == (1, 1) and padding[0] < kh and padding[1] < kw and C <= 96 and N <= 65535
+            and co * kh * kw * input.dtype.itemsize >= 16):
+        # With unit stride the gradient is itself a convolution, of grad_output with the kernel turned by 180 degrees and
+        # its two channel axes swapped, padded by k - 1 - p: one launch of the gathered form instead of a product that
+        # writes the column matrix of the gradient and a pass that reads it back (64 x 64 x 56 x 56, 3 x 3: 416 -> 191 us).
+        turned = weight.permute(1, 0, 2, 3)[:, :, ::-1, ::-1].clone()
+        grad_input = conv2d_into(empty((N, C, H, W), input.dtype), grad_output, turned, None, (kh - 1 - padding[0], kw - 1 - padding[1]))
+        return grad_input, grad_weight, grad_bias
+    gcol = matmul(kcol.transpose(), g)                      # [C*kH*kW, N*P]
+    grad_input = empty((N, C, H, W), input.dtype)
+    check(getattr(_lib.load(), f"am_hip_col2im_{input.sfx}")(
+        N, C, H, W, kh, kw, padding[0], padding[1], stride[0], stride[1], ctypes.c_void_p(gcol.data_ptr()), P, N * P,
+        ctypes.c_void_p(grad_input.data_ptr()), *grad_input.strides))
+    return grad_input, grad_weight, grad_bias
 
 
 def conv2d_into(out: HipTensor, x: HipTensor, kernel: HipTensor, bias: HipTensor | None = None, padding=(0, 0), stride=(1, 1),

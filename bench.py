@@ -287,6 +287,25 @@ def other_workloads(am, timer, steps, warmup, ceilings):
                                      roofline=dict(bound="valu (measured int64 multiply-add ceiling)", achieved=round(valu_tops, 3),
                                                    peak=peak64, unit="Top/s", frac=round(valu_tops / peak64, 4) if peak64 else None))))
     del dA, dB, dC
+    # --- the one figure the reference publishes for this path: `a * b` of two 1500 x 1500 int64 tensors with
+    # entries in [0, 99] (benchmarks/integer_matmul.nim:8-33: 0.14 s on an 18-core i9-9980XE, a whole process
+    # with the random fill, so the ratio is an upper bound on the kernel-to-kernel one)
+    n5 = 1500
+    A = np.random.default_rng(2003).integers(0, 99, (n5, n5), endpoint=True).astype(np.int64)
+    B = np.random.default_rng(2004).integers(0, 99, (n5, n5), endpoint=True).astype(np.int64)
+    dA, dB = am.toHip(A), am.toHip(B)
+    dC = dA * dB
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), max(steps, 50), warmup, WARM_S)
+    k5 = max(steps, 50)
+    want = A[n5 // 2] @ B          # one row of the product (the benchmark prints one element of it)
+    out.append(dict(workload="i64 matmul 1500x1500, entries in [0, 99] (the reference's published integer benchmark: 1 of 36 int8 digit-pair "
+                             "products on the matrix cores, timed with the two digit-splitting passes)",
+                    unit="Top/s", dtype="i64", value=round(2.0 * n5 ** 3 * k5 / wall / 1e12, 3), ms_per_step=round(ev / k5 * 1e3, 4),
+                    row_750_matches_numpy=bool(np.array_equal(dC.toCpu()[n5 // 2], want)),
+                    published=dict(seconds=0.14, gops=round(2.0 * n5 ** 3 / 0.14 / 1e9, 1), hardware="i9-9980XE, 18 cores, -d:danger -d:openmp",
+                                   source="benchmarks/integer_matmul.nim:8-33 (wall time of the whole process: random fill, product, one element printed)",
+                                   ratio_to_this_kernel_time=round(0.14 / (ev / k5), 0))))
+    del dA, dB, dC
     # --- broadcast ops on X[8192, 8192] f32 (HBM bound): 536 903 680 algorithmic bytes per op
     X = np.random.default_rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
     b = np.random.default_rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32)
@@ -351,6 +370,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     del dA, dB, dC
     out.append(bench_chain(am, timer, max(steps, 50), warmup))
     out.append(bench_ex02(am, timer, max(steps, 50), warmup))
+    out.extend(bench_conv_backward(am, timer, steps, warmup))
     return out
 
 
@@ -416,6 +436,32 @@ def bench_ex02(am, timer, steps, warmup, batch=64):
                 images_per_s=round(batch / (best / steps), 0), gflops=round(flops / (best / steps) / 1e9, 1),
                 note="3.0e8 FLOP per pass over six kernels of 3-15 us each: the graph replay runs them back to back (its time is "
                      "the sum of their durations), the eager pass adds the host's launch gap after each")
+
+
+def bench_conv_backward(am, timer, steps, warmup):
+    """conv2d_backward (grad_input, grad_weight, grad_bias) on a ResNet-like layer and on the second convolution of
+    the reference's example 2. FLOP counted: twice the forward pass (one product for each of the two gradients)."""
+    out = []
+    for name, (N, C, H, W, co, k, pad) in (("[64,64,56,56], 64 kernels 3x3, pad 1", (64, 64, 56, 56, 64, 3, 1)),
+                                           ("[64,20,12,12], 50 kernels 5x5 (example 2, conv2)", (64, 20, 12, 12, 50, 5, 0))):
+        rng = np.random.default_rng(6001)
+        ho = H + 2 * pad - k + 1
+        x = am.toHip(rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32))
+        w = am.toHip(rng.uniform(-1, 1, (co, C, k, k)).astype(np.float32))
+        b = am.toHip(rng.uniform(-1, 1, (co, 1, 1)).astype(np.float32))
+        g = am.toHip(rng.uniform(-1, 1, (N, co, ho, ho)).astype(np.float32))
+        _, ev_f = timer.run(lambda: am.conv2d(x, w, b, (pad, pad), (1, 1)), steps, warmup, WARM_S)
+        _, ev_b = timer.run(lambda: am.conv2d_backward(x, w, b, (pad, pad), (1, 1), g), steps, warmup, WARM_S)
+        fl = 2.0 * N * co * ho * ho * C * k * k
+        out.append(dict(workload=f"f32 conv2d_backward {name}", unit="TFLOP/s", dtype="f32", value=round(2 * fl / (ev_b / steps) / 1e12, 2),
+                        ms_per_step=round(ev_b / steps * 1e3, 4), forward_ms=round(ev_f / steps * 1e3, 4),
+                        forward_tflops=round(fl / (ev_f / steps) / 1e12, 2),
+                        roofline=dict(bound="mfma", achieved=round(2 * fl / (ev_b / steps) / 1e12, 2), peak=MFMA_F32_PEAK_TFLOPS, unit="TFLOP/s",
+                                      frac=round(2 * fl / (ev_b / steps) / 1e12 / MFMA_F32_PEAK_TFLOPS, 4)),
+                        note="five launches and a small copy: grad_output with its first two axes swapped, its row sums (grad_bias), "
+                             "the column matrices of the batch side by side, grad_weight as one product over k = N*H_out*W_out, "
+                             "grad_input as one convolution of grad_output with the turned kernel"))
+    return out
 
 
 def config_report(am, timer, L):
@@ -611,6 +657,9 @@ def run_only(am, timer, which, steps, warmup):
     if which == "ex02":
         r = bench_ex02(am, timer, steps, warmup)
         return dict(only=which, hipgraph_us=r["hipgraph_us"], eager_us=r["eager_us"])
+    if which == "conv_backward":
+        r = bench_conv_backward(am, timer, steps, warmup)[0]
+        return dict(only=which, ms_per_step=r["ms_per_step"], tflops=r["value"], forward_ms=r["forward_ms"])
     if which in ("gemm_i32", "gemm_i32_valu"):
         if which == "gemm_i32_valu":
             os.environ["AM_HIP_GEMM_I32_PATH"] = "valu"   # the vector-ALU kernel instead of the digit-sliced matrix-core path
@@ -696,7 +745,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true",
                     help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool", "transposed_add", "bias_short_rows", "sum_cols_narrow", "sum_rows_short", "softmax_short_rows", "gemm_f32_long_k",
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool", "transposed_add", "bias_short_rows", "sum_cols_narrow", "sum_rows_short", "softmax_short_rows", "gemm_f32_long_k", "conv_backward",
                                       "gemm_f32_1024", "gemm_f32_2048", "gemm_i32_1500", "bcast_add_rotating"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()

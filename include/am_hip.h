@@ -216,6 +216,42 @@ int am_hip_im2col_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, 
 int am_hip_im2col_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
                       const int64_t* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, int64_t* col);
 
+/* The same column matrix with image n's row r at col + n*col_n + r*col_c (unit stride along a row; col_c and col_n at
+ * least H_out*W_out). col_n = H_out*W_out, col_c = N*H_out*W_out folds the batch into the columns
+ * ([C*kH*kW][N*H_out*W_out]): the layout in which the backward pass of the convolution is two plain products.
+ * Replaces im2col (src/arraymancer/nn_primitives/fallback/conv.nim:18-54) inside the per-image loop of
+ * im2colgemm_conv2d_gradient (fallback/conv.nim:134-145). */
+int am_hip_im2col_strided_f32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                              const float* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                              float* col, int64_t col_n, int64_t col_c);
+int am_hip_im2col_strided_f64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                              const double* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                              double* col, int64_t col_n, int64_t col_c);
+int am_hip_im2col_strided_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                              const int32_t* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                              int32_t* col, int64_t col_n, int64_t col_c);
+int am_hip_im2col_strided_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                              const int64_t* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                              int64_t* col, int64_t col_n, int64_t col_c);
+
+/* out[n][c][y][x] <- sum over (kh, kw), in increasing order, of the entry of row c*kH*kW + kh*kW + kw of image n's
+ * column matrix that covers pixel (y, x), if any: the reverse of im2col, overlapping patches summed (integers wrap).
+ * `col` is addressed like am_hip_im2col_strided_*'s, `out` through its four NCHW strides (elements); every pixel of
+ * `out` is written. Replaces col2im (src/arraymancer/nn_primitives/fallback/conv.nim:55-79), whose scatter loop
+ * adds the same entries to a pixel in the same order. */
+int am_hip_col2im_f32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const float* col, int64_t col_n, int64_t col_c,
+                      float* out, int64_t out_n, int64_t out_c, int64_t out_h, int64_t out_w);
+int am_hip_col2im_f64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const double* col, int64_t col_n, int64_t col_c,
+                      double* out, int64_t out_n, int64_t out_c, int64_t out_h, int64_t out_w);
+int am_hip_col2im_i32(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const int32_t* col, int64_t col_n, int64_t col_c,
+                      int32_t* out, int64_t out_n, int64_t out_c, int64_t out_h, int64_t out_w);
+int am_hip_col2im_i64(int64_t N, int C, int H, int W, int kH, int kW, int padH, int padW, int strideH, int strideW,
+                      const int64_t* col, int64_t col_n, int64_t col_c,
+                      int64_t* out, int64_t out_n, int64_t out_c, int64_t out_h, int64_t out_w);
+
 /* out[n][co][h*W_out + w] <- sum over (c, kh, kw) of kernel[co][c*kH*kW + kh*kW + kw] * (padded input patch element)
  * (+ bias[co]) (then ReLU), for the whole batch in ONE launch: the column matrix of im2col is never written, the
  * GEMM's B loader gathers it from the images. `in` is addressed through its four NCHW strides (elements); `kernel` is

@@ -123,6 +123,14 @@ namespace detail {
                      int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, T* col) {                     \
     return am_hip_im2col_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, col);      \
   }                                                                                                      \
+  inline int im2col_strided_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW, const T* in, \
+                             int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, T* col, int64_t col_n, int64_t col_c) { \
+    return am_hip_im2col_strided_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, col, col_n, col_c); \
+  }                                                                                                      \
+  inline int col2im_(int64_t N, int C, int H, int W, int kH, int kW, int pH, int pW, int sH, int sW, const T* col, \
+                     int64_t col_n, int64_t col_c, T* out, int64_t on, int64_t oc, int64_t oh, int64_t ow) { \
+    return am_hip_col2im_##SFX(N, C, H, W, kH, kW, pH, pW, sH, sW, col, col_n, col_c, out, on, oc, oh, ow); \
+  }                                                                                                      \
   inline int gemm_batched_(int64_t batch, int64_t M, int64_t N, int64_t K, T al, const T* A, int64_t ra, int64_t ca, \
                            int64_t ba, const T* B, int64_t rb, int64_t cb, int64_t bb, T be, T* C, int64_t rc,     \
                            int64_t cc, int64_t bc, int epi, const T* bias, int64_t brs, int64_t bcs) {            \
@@ -705,6 +713,67 @@ HipTensor<T> conv2d(const HipTensor<T>& x, const HipTensor<T>& kernel, const Hip
     if (with_relu) out = unary(AM_UOP_RELU, out);
   }
   return out;
+}
+
+// col2im (nn_primitives/fallback/conv.nim:55-79) for a batch: [N, C*kH*kW, H_out*W_out] -> [N, C, H, W], pixels
+// covered by several columns summed in the order of the reference's loop.
+template <typename T>
+HipTensor<T> col2im(const HipTensor<T>& col, int64_t C, int64_t H, int64_t W, int kH, int kW, int padH = 0, int padW = 0,
+                    int strideH = 1, int strideW = 1) {
+  const int64_t oh = (H + 2 * padH - kH) / strideH + 1, ow = (W + 2 * padW - kW) / strideW + 1;
+  if (col.rank() != 3 || col.shape[1] != C * kH * kW || col.shape[2] != oh * ow)
+    throw std::invalid_argument("col2im: column matrix of shape " + detail::str(col.shape) + " does not match the geometry");
+  const HipTensor<T> c = col.strides[2] == 1 ? col : col.clone();
+  HipTensor<T> out(Shape{col.shape[0], C, H, W});
+  check(detail::col2im_(col.shape[0], (int)C, (int)H, (int)W, kH, kW, padH, padW, strideH, strideW, c.ptr(), c.strides[0], c.strides[1],
+                        out.ptr(), out.strides[0], out.strides[1], out.strides[2], out.strides[3]));
+  return out;
+}
+
+// conv2d_backward (nn_primitives/nnp_convolution.nim:65-107) over im2colgemm_conv2d_gradient (fallback/conv.nim:107-145).
+// The reference loops over the images; here the batch is folded into the columns: g [C_out, N*P] is grad_output with
+// its first two axes swapped, col [C*kH*kW, N*P] the column matrices side by side, and the pass is
+// grad_bias = row sums of g, grad_weight = g * col^T, grad_input = col2im(kernel_col^T * g). `bias` of the result has
+// shape [C_out, 1, 1]; without with_bias it stays a rank-0 tensor without storage (the reference's "bias.rank == 0").
+template <typename T> struct Conv2dGrads { HipTensor<T> input, weight, bias; };
+template <typename T>
+Conv2dGrads<T> conv2d_backward(const HipTensor<T>& x, const HipTensor<T>& weight, bool with_bias, int padH, int padW, int strideH,
+                               int strideW, const HipTensor<T>& grad_output) {
+  if (x.rank() != 4 || weight.rank() != 4 || weight.shape[1] != x.shape[1])
+    throw std::invalid_argument("conv2d_backward: input must be [N, C, H, W], kernel [C_out, C, kH, kW]");
+  const int64_t N = x.shape[0], C = x.shape[1], H = x.shape[2], W = x.shape[3];
+  const int64_t co = weight.shape[0], kH = weight.shape[2], kW = weight.shape[3], K = C * kH * kW;
+  const int64_t oh = (H + 2 * padH - kH) / strideH + 1, ow = (W + 2 * padW - kW) / strideW + 1, P = oh * ow;
+  if (grad_output.shape != Shape{N, co, oh, ow})
+    throw std::invalid_argument("conv2d_backward: grad_output is " + detail::str(grad_output.shape) + ", the convolution's result is " +
+                                detail::str(Shape{N, co, oh, ow}));
+  const HipTensor<T> go = grad_output.is_C_contiguous() ? grad_output : grad_output.clone();
+  HipTensor<T> gview = go;                       // g[co, n, p] = grad_output[n, co, p]
+  gview.shape = Shape{co, N, P};
+  gview.strides = Shape{P, co * P, 1};
+  HipTensor<T> g = gview.clone();
+  g.shape = Shape{co, N * P};
+  g.strides = Shape{N * P, 1};
+  Conv2dGrads<T> r;
+  if (with_bias) {
+    r.bias = sum(g, 1);
+    r.bias.shape = Shape{co, 1, 1};
+    r.bias.strides = Shape{1, 1, 1};
+  }
+  HipTensor<T> col(Shape{K, N * P});
+  check(detail::im2col_strided_(N, (int)C, (int)H, (int)W, (int)kH, (int)kW, padH, padW, strideH, strideW, x.ptr(), x.strides[0],
+                                x.strides[1], x.strides[2], x.strides[3], col.ptr(), P, N * P));
+  HipTensor<T> kcol = weight.is_C_contiguous() ? weight : weight.clone();
+  kcol.shape = Shape{co, K};
+  kcol.strides = Shape{K, 1};
+  r.weight = g * col.transpose();
+  r.weight.shape = Shape{co, C, kH, kW};
+  r.weight.strides = Shape{K, kH * kW, kW, 1};
+  const HipTensor<T> gcol = kcol.transpose() * g;
+  r.input = HipTensor<T>(Shape{N, C, H, W});
+  check(detail::col2im_(N, (int)C, (int)H, (int)W, (int)kH, (int)kW, padH, padW, strideH, strideW, gcol.ptr(), P, N * P, r.input.ptr(),
+                        r.input.strides[0], r.input.strides[1], r.input.strides[2], r.input.strides[3]));
+  return r;
 }
 
 // maxpool2d (nnp_maxpooling.nim:19-66): values and the flat input index of each maximum.

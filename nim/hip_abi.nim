@@ -76,11 +76,19 @@ proc am_hip_gemm_batched_f32*(batch, M, N, K: int64, alpha: cfloat, A: ptr cfloa
                               epilogue: cint, bias: ptr cfloat, bias_rs, bias_cs: int64): cint {.importc.}
 proc am_hip_im2col_f32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cfloat,
                         in_n, in_c, in_h, in_w: int64, col: ptr cfloat): cint {.importc.}
+proc am_hip_im2col_strided_f32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cfloat,
+                                in_n, in_c, in_h, in_w: int64, col: ptr cfloat, col_n, col_c: int64): cint {.importc.}
+proc am_hip_col2im_f32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, col: ptr cfloat,
+                        col_n, col_c: int64, output: ptr cfloat, out_n, out_c, out_h, out_w: int64): cint {.importc.}
 proc am_hip_gemm_batched_f64*(batch, M, N, K: int64, alpha: cdouble, A: ptr cdouble, rsA, csA, bsA: int64,
                               B: ptr cdouble, rsB, csB, bsB: int64, beta: cdouble, C: ptr cdouble, rsC, csC, bsC: int64,
                               epilogue: cint, bias: ptr cdouble, bias_rs, bias_cs: int64): cint {.importc.}
 proc am_hip_im2col_f64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cdouble,
                         in_n, in_c, in_h, in_w: int64, col: ptr cdouble): cint {.importc.}
+proc am_hip_im2col_strided_f64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cdouble,
+                                in_n, in_c, in_h, in_w: int64, col: ptr cdouble, col_n, col_c: int64): cint {.importc.}
+proc am_hip_col2im_f64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, col: ptr cdouble,
+                        col_n, col_c: int64, output: ptr cdouble, out_n, out_c, out_h, out_w: int64): cint {.importc.}
 proc am_hip_conv2d_f32*(N: int64, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cfloat,
                         in_n, in_c, in_h, in_w: int64, kernel: ptr cfloat, kernel_rs: int64, epilogue: cint,
                         bias: ptr cfloat, bias_s: int64, output: ptr cfloat): cint {.importc.}
@@ -92,11 +100,19 @@ proc am_hip_gemm_batched_i32*(batch, M, N, K: int64, alpha: int32, A: ptr int32,
                               epilogue: cint, bias: ptr int32, bias_rs, bias_cs: int64): cint {.importc.}
 proc am_hip_im2col_i32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr int32,
                         in_n, in_c, in_h, in_w: int64, col: ptr int32): cint {.importc.}
+proc am_hip_im2col_strided_i32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr int32,
+                                in_n, in_c, in_h, in_w: int64, col: ptr int32, col_n, col_c: int64): cint {.importc.}
+proc am_hip_col2im_i32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, col: ptr int32,
+                        col_n, col_c: int64, output: ptr int32, out_n, out_c, out_h, out_w: int64): cint {.importc.}
 proc am_hip_gemm_batched_i64*(batch, M, N, K: int64, alpha: int64, A: ptr int64, rsA, csA, bsA: int64,
                               B: ptr int64, rsB, csB, bsB: int64, beta: int64, C: ptr int64, rsC, csC, bsC: int64,
                               epilogue: cint, bias: ptr int64, bias_rs, bias_cs: int64): cint {.importc.}
 proc am_hip_im2col_i64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr int64,
                         in_n, in_c, in_h, in_w: int64, col: ptr int64): cint {.importc.}
+proc am_hip_im2col_strided_i64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr int64,
+                                in_n, in_c, in_h, in_w: int64, col: ptr int64, col_n, col_c: int64): cint {.importc.}
+proc am_hip_col2im_i64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, col: ptr int64,
+                        col_n, col_c: int64, output: ptr int64, out_n, out_c, out_h, out_w: int64): cint {.importc.}
 proc am_hip_gemv_f32*(M, N: int64, alpha: cfloat, A: ptr cfloat, rsA, csA: int64, x: ptr cfloat, incx: int64,
                       beta: cfloat, y: ptr cfloat, incy: int64): cint {.importc.}
 proc am_hip_gemv_f64*(M, N: int64, alpha: cdouble, A: ptr cdouble, rsA, csA: int64, x: ptr cdouble, incx: int64,

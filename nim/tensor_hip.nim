@@ -643,6 +643,55 @@ proc conv2d*[T: SomeFloat](input, kernel, bias: HipTensor[T], padding = (0, 0), 
   when T is float32: call am_hip_conv2d_f32
   else: call am_hip_conv2d_f64
 
+proc conv2d_backward*[T: HipScalar](input, weight, bias: HipTensor[T], padding, stride: tuple[height, width: int],
+                                    grad_output: HipTensor[T], grad_input, grad_weight, grad_bias: var HipTensor[T]) =
+  ## conv2d_backward (nn_primitives/nnp_convolution.nim:65-107) over im2colgemm_conv2d_gradient
+  ## (fallback/conv.nim:107-145). The reference loops over the images; here the batch is folded into the columns:
+  ## g [C_out, N*P] is grad_output with its first two axes swapped, col [C*kH*kW, N*P] the column matrices side by
+  ## side, and the pass is grad_bias = row sums of g, grad_weight = g * col^T, grad_input = col2im(kernel_col^T * g).
+  assert input.rank == 4 and weight.rank == 4 and weight.shape[1] == input.shape[1]
+  assert bias.rank == 3 or bias.rank == 0
+  let (N, C, H, W) = (input.shape[0], input.shape[1], input.shape[2], input.shape[3])
+  let (co, kH, kW) = (weight.shape[0], weight.shape[2], weight.shape[3])
+  let outH = (H + 2 * padding.height - kH) div stride.height + 1
+  let outW = (W + 2 * padding.width - kW) div stride.width + 1
+  let P = outH * outW
+  assert grad_output.shape[0] == N and grad_output.shape[1] == co and grad_output.shape[2] == outH and grad_output.shape[3] == outW
+  let go = if grad_output.is_C_contiguous: grad_output else: grad_output.clone()
+  # g[co, n, p] = grad_output[n, co, p]: a strided view of the same memory, packed by one copy pass
+  var gview: HipTensor[T]
+  gview.shape.copyFrom([co, N, P]); gview.strides.copyFrom([P, co * P, 1])
+  gview.offset = go.offset; gview.storage = go.storage
+  var g = gview.clone()
+  g.shape.copyFrom([co, N * P]); g.strides.copyFrom([N * P, 1])
+  if bias.rank > 0:
+    grad_bias = sum(g, axis = 1)
+    grad_bias.shape.copyFrom([co, 1, 1]); grad_bias.strides.copyFrom([1, 1, 1])
+  var col = newHipTensor[T]([C * kH * kW, N * P])
+  template unroll(f: untyped) =
+    check f(int64 N, cint C, cint H, cint W, cint kH, cint kW, cint padding.height, cint padding.width, cint stride.height, cint stride.width,
+            input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1], int64 input.strides[2], int64 input.strides[3],
+            col.get_offset_ptr, int64 P, int64(N * P))
+  when T is float32: unroll am_hip_im2col_strided_f32
+  elif T is float64: unroll am_hip_im2col_strided_f64
+  elif T is int32: unroll am_hip_im2col_strided_i32
+  else: unroll am_hip_im2col_strided_i64
+  let wc = if weight.is_C_contiguous: weight else: weight.clone()
+  var kcol = wc
+  kcol.shape.copyFrom([co, C * kH * kW]); kcol.strides.copyFrom([C * kH * kW, 1])
+  grad_weight = g * col.transpose
+  grad_weight.shape.copyFrom([co, C, kH, kW]); grad_weight.strides.copyFrom([C * kH * kW, kH * kW, kW, 1])
+  let gcol = kcol.transpose * g
+  grad_input = newHipTensor[T]([N, C, H, W])
+  template fold(f: untyped) =
+    check f(int64 N, cint C, cint H, cint W, cint kH, cint kW, cint padding.height, cint padding.width, cint stride.height, cint stride.width,
+            gcol.get_offset_ptr, int64 P, int64(N * P), grad_input.get_offset_ptr,
+            int64 grad_input.strides[0], int64 grad_input.strides[1], int64 grad_input.strides[2], int64 grad_input.strides[3])
+  when T is float32: fold am_hip_col2im_f32
+  elif T is float64: fold am_hip_col2im_f64
+  elif T is int32: fold am_hip_col2im_i32
+  else: fold am_hip_col2im_i64
+
 proc maxpool2d*[T: HipScalar](input: HipTensor[T], kernel: tuple[height, width: int], padding = (0, 0), stride = (1, 1)):
     tuple[max_indices: HipTensor[int64], maxpooled: HipTensor[T]] =
   ## nn_primitives/nnp_maxpooling.nim:19-66 (the reference asserts a C-contiguous rank-4 input too).

@@ -320,6 +320,57 @@ def conv2d(x: np.ndarray, kernel: np.ndarray, bias: np.ndarray | None, padding=(
     return out
 
 
+def col2im(col: np.ndarray, channels: int, height: int, width: int, kernel_size, padding=(0, 0), stride=(1, 1)) -> np.ndarray:
+    """col2im of ONE column matrix [C*kH*kW, H_out*W_out] -> [C, H, W], loop for loop as the reference
+    (src/arraymancer/nn_primitives/fallback/conv.nim:55-79): pixels that several columns cover are summed, in
+    the order of the rows of the column matrix."""
+    (kh, kw), (ph, pw), (sh, sw) = kernel_size, padding, stride
+    hc, wc = (height + 2 * ph - kh) // sh + 1, (width + 2 * pw - kw) // sw + 1
+    out = np.zeros((channels, height, width), dtype=col.dtype)
+    with np.errstate(over="ignore"):
+        for c in range(channels * kh * kw):
+            w_off, h_off, c_off = c % kw - pw, (c // kw) % kh - ph, (c // kw) // kh
+            for h in range(hc):
+                row = h_off + h * sh
+                if not 0 <= row < height:
+                    continue
+                for w in range(wc):
+                    cc = w_off + w * sw
+                    if 0 <= cc < width:
+                        out[c_off, row, cc] += col[c, h * wc + w]
+    return out
+
+
+def conv2d_backward(x: np.ndarray, kernel: np.ndarray, bias: np.ndarray | None, padding, stride, grad_output: np.ndarray):
+    """conv2d_backward (src/arraymancer/nn_primitives/nnp_convolution.nim:65-107) over
+    im2colgemm_conv2d_gradient (fallback/conv.nim:107-145): per image grad_input_col = kernel_col^T * grad_output_col,
+    grad_input[n] = col2im(grad_input_col), grad_weight += grad_output_col * input_col^T, all through the restated laser
+    GEMM; grad_bias = grad_output.sum(3).sum(2).sum(0). Returns (grad_input, grad_weight, grad_bias or None)."""
+    N, C, H, W = x.shape
+    co, _, kh, kw = kernel.shape
+    ho, wo = (H + 2 * padding[0] - kh) // stride[0] + 1, (W + 2 * padding[1] - kw) // stride[1] + 1
+    assert grad_output.shape == (N, co, ho, wo)
+    kcol = np.ascontiguousarray(kernel.reshape(co, C * kh * kw))
+    grad_input = np.zeros_like(x)
+    grad_weight = np.zeros((co, C * kh * kw), dtype=x.dtype)
+    for n in range(N):
+        gcol = np.ascontiguousarray(grad_output[n].reshape(co, ho * wo))
+        gin_col = np.empty((C * kh * kw, ho * wo), dtype=x.dtype)
+        gemm_strided(1, kcol.T, gcol, 0, gin_col)
+        grad_input[n] = col2im(gin_col, C, H, W, (kh, kw), padding, stride)
+        col = im2col(np.ascontiguousarray(x[n]), (kh, kw), padding, stride)
+        part = np.empty_like(grad_weight)
+        gemm_strided(1, gcol, col.T, 0, part)
+        map2("add", grad_weight, part, out=grad_weight)
+    grad_bias = None
+    if bias is not None:
+        g = grad_output
+        for ax in (3, 2, 0):
+            g = reduce_axis("sum", np.ascontiguousarray(g), ax)
+        grad_bias = g.reshape(bias.shape)
+    return grad_input, grad_weight.reshape(kernel.shape), grad_bias
+
+
 # ----------------------------------------------------------------------------- closed forms
 RED = {"sum": 0, "product": 1, "min": 2, "max": 3}
 

@@ -222,6 +222,27 @@ template <typename T> static void conv_literals() {
   }
 }
 
+template <typename T> static void conv_backward_known_answer() {
+  // conv2d_backward (nnp_convolution.nim:65-107) on a case worked by hand: two copies of the 3 x 3 image 1..9, one
+  // 2 x 2 kernel {1, 2, 3, 4}, grad_output all ones. grad_weight[kh, kw] sums the image under each kernel entry,
+  // grad_input is the kernel spread over the positions it was applied at, grad_bias counts the outputs.
+  auto x = toHip<T>({1, 2, 3, 4, 5, 6, 7, 8, 9, 1, 2, 3, 4, 5, 6, 7, 8, 9}, {2, 1, 3, 3});
+  auto k = toHip<T>({1, 2, 3, 4}, {1, 1, 2, 2});
+  auto g = toHip<T>({1, 1, 1, 1, 1, 1, 1, 1}, {2, 1, 2, 2});
+  auto r = am::conv2d_backward(x, k, true, 0, 0, 1, 1, g);
+  CHECK(r.weight.shape == (Shape{1, 1, 2, 2}) && eq(r.weight, {24, 32, 48, 56}));
+  CHECK(r.input.shape == (Shape{2, 1, 3, 3}) && eq(r.input, {1, 3, 2, 4, 10, 6, 3, 7, 4, 1, 3, 2, 4, 10, 6, 3, 7, 4}));
+  CHECK(r.bias.shape == (Shape{1, 1, 1}) && eq(r.bias, {8}));
+  auto nb = am::conv2d_backward(x, k, false, 0, 0, 1, 1, g);
+  CHECK(nb.bias.rank() == 0 && eq(nb.weight, {24, 32, 48, 56}));
+  // col2im on its own: the column matrix of ones of that geometry counts the patches over each pixel
+  auto ones = toHip<T>(std::vector<T>(16, T(1)), {1, 4, 4});
+  CHECK(eq(am::col2im(ones, 1, 3, 3, 2, 2), {1, 2, 1, 2, 4, 2, 1, 2, 1}));
+  bool threw = false;
+  try { am::conv2d_backward(x, k, true, 0, 0, 1, 1, x); } catch (const std::invalid_argument&) { threw = true; }
+  CHECK(threw);
+}
+
 static void maxpool_backward() {
   // tests/nn_primitives/test_nnp_maxpool.nim:20-45
   auto a = toHip<float>({1, 1, 2, 4, 5, 6, 7, 8, 3, 2, 1, 0, 1, 2, 3, 4}, {1, 1, 4, 4});
@@ -409,6 +430,10 @@ int main(int argc, char** argv) {
   conv_literals<double>();
   conv_literals<int32_t>();
   conv_literals<int64_t>();
+  conv_backward_known_answer<float>();
+  conv_backward_known_answer<double>();
+  conv_backward_known_answer<int32_t>();
+  conv_backward_known_answer<int64_t>();
   maxpool_backward();
     aggregates<float>();
     aggregates<double>();

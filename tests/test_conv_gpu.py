@@ -102,3 +102,96 @@ def test_gemm_batched(hip, oracle, sfx):
     check(oracle, sfx, dC.toCpu(), want, "shared A")
     with pytest.raises(IndexError):
         hip.gemm_batched(1, hip.toHip(A[:3]), hip.toHip(B), 0, dC)
+
+
+BWD_GEOMS = [  # N, C, H, W, C_out, kH, kW, pad, stride
+    (2, 3, 4, 5, 2, 3, 3, (1, 1), (1, 1)),          # the reference's own backward case (test_nnp_convolution.nim:137-168)
+    (1, 1, 5, 5, 1, 3, 3, (0, 0), (1, 1)),
+    (3, 2, 9, 7, 4, 3, 2, (1, 0), (2, 1)),
+    (4, 2, 16, 16, 3, 3, 3, (1, 1), (2, 2)),        # stride 2 with padding: pixels that no column covers get 0
+    (3, 8, 20, 20, 13, 3, 5, (2, 3), (1, 2)),       # padding wider than the kernel's reach on one side
+    (2, 5, 11, 13, 7, 1, 1, (0, 0), (1, 1)),        # 1 x 1 kernel
+    (2, 3, 9, 9, 4, 2, 2, (0, 0), (3, 3)),          # stride beyond the kernel: rows and columns of the image left out
+    (64, 1, 28, 28, 20, 5, 5, (0, 0), (1, 1)),      # conv1 of the reference's example 2 at batch 64
+    (16, 20, 12, 12, 50, 5, 5, (0, 0), (1, 1)),     # conv2
+    (2, 3, 6, 6, 4, 3, 3, (2, 2), (1, 1)),          # padding k - 1: the gradient as a convolution needs no padding of its own
+    (2, 3, 6, 6, 4, 2, 2, (2, 2), (1, 1)),          # padding k: outputs made of padding alone; not a convolution any more
+    (1, 2, 9, 10, 3, 3, 4, (1, 2), (1, 1)),         # kernel widths 4, 7 and 9 at unit stride
+    (1, 1, 10, 12, 2, 2, 7, (0, 3), (1, 1)),
+    (1, 1, 6, 14, 2, 2, 9, (0, 4), (1, 1)),
+    (2, 100, 8, 8, 6, 3, 3, (1, 1), (1, 1)),        # more input channels than the one-launch form of grad_input takes
+]
+
+
+@pytest.mark.parametrize("sfx", ALL)
+@pytest.mark.parametrize("geom", BWD_GEOMS)
+def test_col2im_and_conv_backward_vs_oracle(hip, oracle, sfx, geom):
+    """col2im and conv2d_backward (fallback/conv.nim:55-79, 107-145; nnp_convolution.nim:65-107) against the oracle's
+    per-image restatement: col2im bit for bit in every type (same entries added in the same order), the gradients bit
+    for bit on integers and within the float GEMM tolerance otherwise."""
+    dt = DTYPES[sfx]
+    N, C, H, W, co, kh, kw, pad, stride = geom
+    rng = np.random.default_rng(seed_of("conv-bwd", sfx, geom))
+    ho, wo = (H + 2 * pad[0] - kh) // stride[0] + 1, (W + 2 * pad[1] - kw) // stride[1] + 1
+    x, k, b = fill(rng, (N, C, H, W), dt), fill(rng, (co, C, kh, kw), dt), fill(rng, (co, 1, 1), dt)
+    g = fill(rng, (N, co, ho, wo), dt)
+    say("col2im", sfx, geom)
+    cols = fill(rng, (N, C * kh * kw, ho * wo), dt)
+    got = hip.col2im(hip.toHip(cols), C, H, W, (kh, kw), pad, stride).toCpu()
+    for n in (0, N - 1):
+        assert np.array_equal(got[n], oracle.col2im(cols[n], C, H, W, (kh, kw), pad, stride)), n
+    one = hip.col2im(hip.toHip(cols[0]), C, H, W, (kh, kw), pad, stride).toCpu()
+    assert one.shape == (C, H, W) and np.array_equal(one, got[0])
+    say("folded im2col", sfx, geom)
+    folded = hip.im2col_folded(hip.toHip(x), (kh, kw), pad, stride).toCpu().reshape(C * kh * kw, N, ho * wo)
+    for n in (0, N - 1):
+        assert np.array_equal(folded[:, n], oracle.im2col(x[n], (kh, kw), pad, stride)), n
+    say("conv2d_backward", sfx, geom)
+    gi, gw, gb = hip.conv2d_backward(hip.toHip(x), hip.toHip(k), hip.toHip(b), pad, stride, hip.toHip(g))
+    wi, ww, wb = oracle.conv2d_backward(x, k, b, pad, stride, g)
+    assert gi.shape == x.shape and gw.shape == k.shape and gb.shape == b.shape
+    check(oracle, sfx, gi.toCpu(), wi, "grad_input")
+    check(oracle, sfx, gw.toCpu(), ww, "grad_weight")
+    check(oracle, sfx, gb.toCpu(), wb, "grad_bias")
+    gi2, gw2, gb2 = hip.conv2d_backward(hip.toHip(x), hip.toHip(k), None, pad, stride, hip.toHip(g))
+    assert gb2 is None and np.array_equal(gi2.toCpu(), gi.toCpu()) and np.array_equal(gw2.toCpu(), gw.toCpu())
+
+
+def test_conv_backward_reference_check(hip, oracle):
+    """The reference's own check (test_nnp_convolution.nim:137-168): float32 gradients for grad_output = ones against
+    the float64 numerical gradient of the forward pass, mean relative error below 1e-6."""
+    rng = np.random.default_rng(seed_of("conv-bwd-reference"))
+    x = rng.uniform(0, 1, (2, 3, 4, 5)).astype(np.float32)
+    k = rng.uniform(0, 1, (2, 3, 3, 3)).astype(np.float32)
+    b = rng.uniform(0, 1, (2, 1, 1)).astype(np.float32)
+    pad, stride = (1, 1), (1, 1)
+    out = hip.conv2d(hip.toHip(x), hip.toHip(k), hip.toHip(b), pad, stride)
+    gi, gw, gb = hip.conv2d_backward(hip.toHip(x), hip.toHip(k), hip.toHip(b), pad, stride, hip.toHip(np.ones(out.shape, np.float32)))
+    x64, k64, b64 = x.astype(np.float64), k.astype(np.float64), b.astype(np.float64)
+
+    def numerical(arr, h=1e-3):
+        grad = np.zeros_like(arr)
+        flat, gf = arr.reshape(-1), grad.reshape(-1)
+        for i in range(flat.size):
+            keep = flat[i]
+            flat[i] = keep + h; up = oracle.conv2d(x64, k64, b64, pad, stride).sum()
+            flat[i] = keep - h; dn = oracle.conv2d(x64, k64, b64, pad, stride).sum()
+            flat[i] = keep
+            gf[i] = (up - dn) / (2 * h)
+        return grad
+
+    for got, arr, name in ((gi, x64, "grad_input"), (gw, k64, "grad_weight"), (gb, b64, "grad_bias")):
+        want = numerical(arr)
+        err = np.mean(np.abs(got.toCpu().astype(np.float64) - want) / np.abs(want))
+        say("conv backward, reference check", name, err)
+        assert err < 1e-6, name
+
+
+def test_conv_backward_errors(hip):
+    x, k = hip.zeros((2, 3, 5, 5), np.float32), hip.zeros((4, 3, 3, 3), np.float32)
+    with pytest.raises(ValueError):
+        hip.conv2d_backward(x, k, None, (0, 0), (1, 1), hip.zeros((2, 4, 4, 4), np.float32))     # wrong output extent
+    with pytest.raises(ValueError):
+        hip.conv2d_backward(x, hip.zeros((4, 2, 3, 3), np.float32), None, (0, 0), (1, 1), hip.zeros((2, 4, 3, 3), np.float32))
+    with pytest.raises(ValueError):
+        hip.col2im(hip.zeros((27, 8), np.float32), 3, 5, 5, (3, 3))                               # 9 columns expected

@@ -41,3 +41,13 @@ def test_cpp_host_layer_on_device_under_sanitizers(hip):
     print(res.stdout)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
     assert " 0 failed" in res.stdout and "AddressSanitizer" not in res.stderr and "runtime error" not in res.stderr
+
+
+def test_division_by_launch_constants_is_exact():
+    """csrc/fastdiv.h (multiply-and-shift division used by the im2col / col2im kernels' index arithmetic), compiled
+    for the host and compared with the machine's division over 4000+ divisors and the dividends where a wrong
+    multiplier or shift would show."""
+    res = subprocess.run(["make", "-C", CPP_DIR, "-B", "test_fastdiv"], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-3000:]
+    res = subprocess.run([os.path.join(CPP_DIR, "test_fastdiv")], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0 and " 0 wrong" in res.stdout, res.stdout[-2000:] + res.stderr[-2000:]

@@ -343,6 +343,104 @@ def test_reference_conv_vectors(vectors, oracle):
             assert np.array_equal(got, np.array(case["target"], dtype=dt)), case["name"]
 
 
+def _conv_direct(x, k, pad, st):
+    """Cross-correlation straight from its definition (no column matrix), in the operands' own type."""
+    N, C, H, W = x.shape
+    co, _, kh, kw = k.shape
+    ho, wo = (H + 2 * pad[0] - kh) // st[0] + 1, (W + 2 * pad[1] - kw) // st[1] + 1
+    xp = np.zeros((N, C, H + 2 * pad[0], W + 2 * pad[1]), dtype=x.dtype)
+    xp[:, :, pad[0]:pad[0] + H, pad[1]:pad[1] + W] = x
+    y = np.zeros((N, co, ho, wo), dtype=x.dtype)
+    for h in range(ho):
+        for w in range(wo):
+            patch = xp[:, :, h * st[0]:h * st[0] + kh, w * st[1]:w * st[1] + kw]
+            y[:, :, h, w] = np.einsum("ncij,ocij->no", patch, k)
+    return y
+
+
+_BWD_GEOMS = [((2, 3, 4, 5), (2, 3, 3, 3), (1, 1), (1, 1)),      # the reference's own backward case (test_nnp_convolution.nim:137-168)
+              ((2, 3, 5, 5), (2, 3, 3, 3), (1, 1), (2, 2)),
+              ((3, 2, 7, 6), (4, 2, 3, 2), (0, 2), (2, 1)),
+              ((1, 1, 6, 9), (3, 1, 2, 4), (2, 0), (1, 3)),
+              ((2, 4, 5, 5), (1, 4, 5, 5), (0, 0), (1, 1))]
+
+
+@pytest.mark.parametrize("geom", _BWD_GEOMS)
+def test_conv_backward_against_numerical_gradient_and_adjoints(oracle, geom):
+    """conv2d_backward the way the reference checks it (tests/nn_primitives/test_nnp_convolution.nim:137-168):
+    against central differences of the pinned forward pass, in float64. The convolution is linear in each argument,
+    so the differences are exact up to rounding. Beside that, with a random grad_output instead of ones: the two
+    adjoint identities <conv(x, k), g> = <x, grad_input> = <k, grad_weight>, which no transposed or shifted index
+    survives, with the forward pass taken from the definition rather than from the column matrix."""
+    xs, ks, pad, st = geom
+    rng = np.random.default_rng(seed_of("conv-bwd-oracle", geom))
+    x, k, b = rng.uniform(-1, 1, xs), rng.uniform(-1, 1, ks), rng.uniform(-1, 1, (ks[0], 1, 1))
+    y = oracle.conv2d(x, k, b, pad, st)
+    assert np.allclose(y, _conv_direct(x, k, pad, st) + b.reshape(1, -1, 1, 1), rtol=0, atol=1e-13)
+    ones = np.ones_like(y)
+    gi, gw, gb = oracle.conv2d_backward(x, k, b, pad, st, ones)
+
+    def numerical(arr, f, h=1e-3):
+        g = np.zeros_like(arr)
+        flat, gf = arr.reshape(-1), g.reshape(-1)
+        for i in range(flat.size):
+            keep = flat[i]
+            flat[i] = keep + h; up = f()
+            flat[i] = keep - h; dn = f()
+            flat[i] = keep
+            gf[i] = (up - dn) / (2 * h)
+        return g
+
+    total = lambda: oracle.conv2d(x, k, b, pad, st).sum()
+    for got, arr in ((gi, x), (gw, k), (gb, b)):
+        want = numerical(arr, total)
+        assert np.mean(np.abs(got - want) / (np.abs(want) + 1e-30)) < 1e-6 or np.max(np.abs(got - want)) < 1e-9
+    for trial in range(3):
+        g = rng.uniform(-1, 1, y.shape)
+        gi, gw, gb = oracle.conv2d_backward(x, k, b, pad, st, g)
+        lhs = np.sum(_conv_direct(x, k, pad, st) * g)
+        assert abs(lhs - np.sum(x * gi)) <= 1e-12 * max(1.0, abs(lhs))
+        assert abs(lhs - np.sum(k * gw)) <= 1e-12 * max(1.0, abs(lhs))
+        assert np.allclose(gb.reshape(-1), g.sum((0, 2, 3)), rtol=0, atol=1e-13)
+        # every entry, not one inner product: grad_input[n, c, y, x] = <conv(e_ncyx, k), g>, grad_weight likewise
+        e = np.zeros_like(x)
+        for idx in [tuple(rng.integers(0, s) for s in xs) for _ in range(6)]:
+            e[idx] = 1.0
+            assert abs(np.sum(_conv_direct(e, k, pad, st) * g) - gi[idx]) <= 1e-12
+            e[idx] = 0.0
+        e = np.zeros_like(k)
+        for idx in [tuple(rng.integers(0, s) for s in ks) for _ in range(6)]:
+            e[idx] = 1.0
+            assert abs(np.sum(_conv_direct(x, e, pad, st) * g) - gw[idx]) <= 1e-12
+            e[idx] = 0.0
+
+
+def test_col2im_is_the_adjoint_of_im2col_and_wraps(oracle):
+    """col2im sums the entries im2col would have read from a pixel: <im2col(x), c> = <x, col2im(c)> exactly on
+    integers (wrapping ones included), and col2im(im2col(ones)) counts the patches that cover each pixel."""
+    rng = np.random.default_rng(seed_of("col2im-oracle"))
+    for (C, H, W, kh, kw, pad, st) in [(2, 5, 6, 3, 3, (1, 1), (1, 1)), (1, 7, 4, 2, 3, (0, 2), (2, 1)), (3, 4, 4, 4, 4, (0, 0), (1, 1)),
+                                       (2, 6, 6, 3, 3, (2, 2), (3, 2))]:
+        x = rng.integers(-50, 50, (C, H, W)).astype(np.int64)
+        col = oracle.im2col(x, (kh, kw), pad, st)
+        c = rng.integers(-50, 50, col.shape).astype(np.int64)
+        back = oracle.col2im(c, C, H, W, (kh, kw), pad, st)
+        assert int(np.sum(col * c)) == int(np.sum(x * back))
+        cover = oracle.col2im(oracle.im2col(np.ones_like(x), (kh, kw), pad, st), C, H, W, (kh, kw), pad, st)
+        hc, wc = (H + 2 * pad[0] - kh) // st[0] + 1, (W + 2 * pad[1] - kw) // st[1] + 1
+        brute = np.zeros((H, W), dtype=np.int64)
+        for h in range(hc):
+            for w in range(wc):
+                for i in range(kh):
+                    for j in range(kw):
+                        r, q = h * st[0] + i - pad[0], w * st[1] + j - pad[1]
+                        if 0 <= r < H and 0 <= q < W:
+                            brute[r, q] += 1
+        assert np.array_equal(cover, np.broadcast_to(brute, (C, H, W)))
+    big = np.full((4, 4), 2**31 - 1, dtype=np.int32)         # a pixel covered by four patches: 4 * INT_MAX wraps to -4
+    assert oracle.col2im(big, 1, 3, 3, (2, 2), (0, 0), (1, 1))[0, 1, 1] == np.int32(-4)
+
+
 _UFUNC_NUMPY = dict(ln=np.log, log10=np.log10, log2=np.log2, sin=np.sin, cos=np.cos, tan=np.tan, sinh=np.sinh,
                     cosh=np.cosh, arcsin=np.arcsin, arccos=np.arccos, arctan=np.arctan, arcsinh=np.arcsinh,
                     arccosh=np.arccosh, arctanh=np.arctanh, cbrt=np.cbrt, floor=np.floor, ceil=np.ceil,
