@@ -1148,6 +1148,72 @@ def softmax(t: HipTensor) -> HipTensor:
     return out
 
 
+def _check_input_target(input: HipTensor, target: HipTensor, sparse: bool):
+    if input.rank != 2 or input.dtype.kind != "f":
+        raise ValueError("softmax cross-entropy: input must be a float [batch_size, number_of_classes] matrix")
+    if sparse:
+        if target.rank != 1 or target.shape[0] != input.shape[0]:
+            raise ValueError(f"sparse softmax cross-entropy: {target.shape[0] if target.rank else 0} labels for {input.shape[0]} rows")
+        if target.dtype != np.dtype(np.int64):
+            raise TypeError("sparse softmax cross-entropy: the labels must be an int64 tensor (the reference's Tensor[int])")
+    else:
+        _same_dtype(input, target)
+        if target.shape != input.shape:     # check_input_target, private/p_nnp_checks.nim
+            raise ValueError(f"softmax cross-entropy: input {input.shape} and target {target.shape} must have the same shape")
+
+
+def softmax_cross_entropy(input: HipTensor, target: HipTensor) -> float:
+    """Softmax + cross-entropy loss in one pass, averaged over the batch
+    (src/arraymancer/nn_primitives/nnp_softmax_cross_entropy.nim:17-86). `target` holds probabilities [batch, classes]."""
+    _check_input_target(input, target, False)
+    loss = _lib.CTYPE[input.sfx]()
+    check(getattr(_lib.load(), f"am_hip_softmax_cross_entropy_{input.sfx}")(
+        input.shape[0], input.shape[1], ctypes.c_void_p(input.data_ptr()), *input.strides,
+        ctypes.c_void_p(target.data_ptr()), *target.strides, ctypes.byref(loss)))
+    return input.dtype.type(loss.value)
+
+
+def sparse_softmax_cross_entropy(input: HipTensor, target: HipTensor) -> float:
+    """The same loss with one int64 class index per row (nnp_softmax_cross_entropy.nim:88-177)."""
+    _check_input_target(input, target, True)
+    loss = _lib.CTYPE[input.sfx]()
+    check(getattr(_lib.load(), f"am_hip_sparse_softmax_cross_entropy_{input.sfx}")(
+        input.shape[0], input.shape[1], ctypes.c_void_p(input.data_ptr()), *input.strides,
+        ctypes.c_void_p(target.data_ptr()), target.strides[0], ctypes.byref(loss)))
+    return input.dtype.type(loss.value)
+
+
+def _scalar_gradient(gradient, dtype):
+    """The reference takes the upstream gradient as a scalar or as a one-element tensor (its first element is used)."""
+    if isinstance(gradient, HipTensor):
+        return dtype.type(gradient.toCpu().reshape(-1)[0])
+    return dtype.type(gradient)
+
+
+def softmax_cross_entropy_backward(gradient, cached_tensor: HipTensor, target: HipTensor) -> HipTensor:
+    """gradient * (softmax(cached_tensor) - target) / batch_size in one launch
+    (nnp_softmax_cross_entropy.nim:186-214)."""
+    _check_input_target(cached_tensor, target, False)
+    out = empty(cached_tensor.shape, cached_tensor.dtype)
+    check(getattr(_lib.load(), f"am_hip_softmax_cross_entropy_backward_{cached_tensor.sfx}")(
+        cached_tensor.shape[0], cached_tensor.shape[1], _lib.CTYPE[cached_tensor.sfx](_scalar_gradient(gradient, cached_tensor.dtype)),
+        ctypes.c_void_p(cached_tensor.data_ptr()), *cached_tensor.strides, ctypes.c_void_p(target.data_ptr()), *target.strides,
+        ctypes.c_void_p(out.data_ptr()), *out.strides))
+    return out
+
+
+def sparse_softmax_cross_entropy_backward(gradient, cached_tensor: HipTensor, target: HipTensor) -> HipTensor:
+    """gradient * (softmax(cached_tensor) - onehot(target)) / batch_size in one launch
+    (nnp_softmax_cross_entropy.nim:217-256)."""
+    _check_input_target(cached_tensor, target, True)
+    out = empty(cached_tensor.shape, cached_tensor.dtype)
+    check(getattr(_lib.load(), f"am_hip_sparse_softmax_cross_entropy_backward_{cached_tensor.sfx}")(
+        cached_tensor.shape[0], cached_tensor.shape[1], _lib.CTYPE[cached_tensor.sfx](_scalar_gradient(gradient, cached_tensor.dtype)),
+        ctypes.c_void_p(cached_tensor.data_ptr()), *cached_tensor.strides, ctypes.c_void_p(target.data_ptr()), target.strides[0],
+        ctypes.c_void_p(out.data_ptr()), *out.strides))
+    return out
+
+
 def maxpool2d(x: HipTensor, kernel, padding=(0, 0), stride=(1, 1)):
     """(max_indices, maxpooled) of a C-contiguous [N, C, H, W] tensor
     (src/arraymancer/nn_primitives/nnp_maxpooling.nim:19-66; the reference asserts contiguity too).

@@ -572,6 +572,41 @@ int am_hip_softmax_rows_f32(int64_t rows, int64_t cols, float* dst, int64_t dst_
 int am_hip_softmax_rows_f64(int64_t rows, int64_t cols, double* dst, int64_t dst_rs, int64_t dst_cs,
                             const double* src, int64_t src_rs, int64_t src_cs);
 
+/* *loss (host) <- (1 / rows) * sum over the rows i of  ln(sum_j exp(input[i, j])) - sum_j input[i, j] * target[i, j]:
+ * softmax and cross-entropy in one pass over `input` [rows, cols] and `target` [rows, cols] (probabilities), element
+ * strides (rs, cs). Blocking; 0 for an empty batch. Replaces softmax_cross_entropy
+ * (src/arraymancer/nn_primitives/nnp_softmax_cross_entropy.nim:17-86); the rows' losses are added in a fixed order
+ * (the reference adds them with an atomic under OpenMP), the result agrees to rounding. */
+int am_hip_softmax_cross_entropy_f32(int64_t rows, int64_t cols, const float* input, int64_t in_rs, int64_t in_cs,
+                                     const float* target, int64_t t_rs, int64_t t_cs, float* loss);
+int am_hip_softmax_cross_entropy_f64(int64_t rows, int64_t cols, const double* input, int64_t in_rs, int64_t in_cs,
+                                     const double* target, int64_t t_rs, int64_t t_cs, double* loss);
+/* The same with one class index per row instead of probabilities: labels[i * labels_s] in [0, cols); the row's term is
+ * ln(sum_j exp(input[i, j])) - input[i, label]. A label outside [0, cols) makes the loss NaN (the reference reads out
+ * of bounds or raises an IndexDefect). Replaces sparse_softmax_cross_entropy (nnp_softmax_cross_entropy.nim:88-177). */
+int am_hip_sparse_softmax_cross_entropy_f32(int64_t rows, int64_t cols, const float* input, int64_t in_rs, int64_t in_cs,
+                                            const int64_t* labels, int64_t labels_s, float* loss);
+int am_hip_sparse_softmax_cross_entropy_f64(int64_t rows, int64_t cols, const double* input, int64_t in_rs, int64_t in_cs,
+                                            const int64_t* labels, int64_t labels_s, double* loss);
+/* result[i, j] <- gradient * (softmax(input[i, :])[j] - target[i, j]) / rows: the gradient of the loss above with respect
+ * to `input`, one launch. Replaces softmax_cross_entropy_backward (nnp_softmax_cross_entropy.nim:186-214) with a scalar
+ * gradient (a one-element gradient tensor is read by the host layer). */
+int am_hip_softmax_cross_entropy_backward_f32(int64_t rows, int64_t cols, float gradient, const float* input, int64_t in_rs,
+                                              int64_t in_cs, const float* target, int64_t t_rs, int64_t t_cs,
+                                              float* result, int64_t r_rs, int64_t r_cs);
+int am_hip_softmax_cross_entropy_backward_f64(int64_t rows, int64_t cols, double gradient, const double* input, int64_t in_rs,
+                                              int64_t in_cs, const double* target, int64_t t_rs, int64_t t_cs,
+                                              double* result, int64_t r_rs, int64_t r_cs);
+/* result[i, j] <- gradient * (softmax(input[i, :])[j] - (j == labels[i] ? 1 : 0)) / rows. A label outside [0, cols)
+ * leaves its row the plain softmax term. Replaces sparse_softmax_cross_entropy_backward
+ * (nnp_softmax_cross_entropy.nim:217-256). */
+int am_hip_sparse_softmax_cross_entropy_backward_f32(int64_t rows, int64_t cols, float gradient, const float* input,
+                                                     int64_t in_rs, int64_t in_cs, const int64_t* labels, int64_t labels_s,
+                                                     float* result, int64_t r_rs, int64_t r_cs);
+int am_hip_sparse_softmax_cross_entropy_backward_f64(int64_t rows, int64_t cols, double gradient, const double* input,
+                                                     int64_t in_rs, int64_t in_cs, const int64_t* labels, int64_t labels_s,
+                                                     double* result, int64_t r_rs, int64_t r_cs);
+
 /* Max pooling of a C-contiguous [N, C, H, W] input into a C-contiguous [N, C, outH, outW] output,
  * outH = (H + 2 padH - kH) / strideH + 1 (outW alike), plus, when argmax != NULL, the flat input
  * index of each maximum (what maxpool2d_backward scatters through). Same window scan order,

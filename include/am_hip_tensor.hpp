@@ -670,6 +670,68 @@ HipTensor<T> softmax(const HipTensor<T>& t) {
   return r;
 }
 
+// Softmax + cross-entropy in one pass, averaged over the batch, and its gradient
+// (nn_primitives/nnp_softmax_cross_entropy.nim:17-86, 88-177, 186-214, 217-256). The dense forms take probabilities
+// [batch_size, classes], the sparse forms one int64 class index per row.
+namespace detail {
+#define AM_HPP_LOSS(T, SFX)                                                                                                   \
+  inline int sce_(int64_t r, int64_t c, const T* x, int64_t xr, int64_t xc, const T* t, int64_t tr, int64_t tc, T* loss) {    \
+    return am_hip_softmax_cross_entropy_##SFX(r, c, x, xr, xc, t, tr, tc, loss);                                              \
+  }                                                                                                                           \
+  inline int sparse_sce_(int64_t r, int64_t c, const T* x, int64_t xr, int64_t xc, const int64_t* l, int64_t ls, T* loss) {   \
+    return am_hip_sparse_softmax_cross_entropy_##SFX(r, c, x, xr, xc, l, ls, loss);                                           \
+  }                                                                                                                           \
+  inline int sce_bwd_(int64_t r, int64_t c, T g, const T* x, int64_t xr, int64_t xc, const T* t, int64_t tr, int64_t tc,      \
+                      T* o, int64_t orr, int64_t oc) {                                                                        \
+    return am_hip_softmax_cross_entropy_backward_##SFX(r, c, g, x, xr, xc, t, tr, tc, o, orr, oc);                            \
+  }                                                                                                                           \
+  inline int sparse_sce_bwd_(int64_t r, int64_t c, T g, const T* x, int64_t xr, int64_t xc, const int64_t* l, int64_t ls,     \
+                             T* o, int64_t orr, int64_t oc) {                                                                 \
+    return am_hip_sparse_softmax_cross_entropy_backward_##SFX(r, c, g, x, xr, xc, l, ls, o, orr, oc);                         \
+  }
+AM_HPP_LOSS(float, f32)
+AM_HPP_LOSS(double, f64)
+#undef AM_HPP_LOSS
+}  // namespace detail
+
+template <typename T>
+T softmax_cross_entropy(const HipTensor<T>& input, const HipTensor<T>& target) {
+  if (input.rank() != 2 || input.shape != target.shape)
+    throw std::invalid_argument("softmax_cross_entropy: input " + detail::str(input.shape) + " and target " + detail::str(target.shape) +
+                                " must be matrices of the same shape");
+  T loss = T(0);
+  check(detail::sce_(input.shape[0], input.shape[1], input.ptr(), input.strides[0], input.strides[1], target.ptr(), target.strides[0],
+                     target.strides[1], &loss));
+  return loss;
+}
+template <typename T>
+T sparse_softmax_cross_entropy(const HipTensor<T>& input, const HipTensor<int64_t>& target) {
+  if (input.rank() != 2 || target.rank() != 1 || target.shape[0] != input.shape[0])
+    throw std::invalid_argument("sparse_softmax_cross_entropy: one label per row of the input is needed");
+  T loss = T(0);
+  check(detail::sparse_sce_(input.shape[0], input.shape[1], input.ptr(), input.strides[0], input.strides[1], target.ptr(),
+                            target.strides[0], &loss));
+  return loss;
+}
+template <typename T>
+HipTensor<T> softmax_cross_entropy_backward(T gradient, const HipTensor<T>& cached_tensor, const HipTensor<T>& target) {
+  if (cached_tensor.rank() != 2 || cached_tensor.shape != target.shape)
+    throw std::invalid_argument("softmax_cross_entropy_backward: input and target must be matrices of the same shape");
+  HipTensor<T> r(cached_tensor.shape);
+  check(detail::sce_bwd_(cached_tensor.shape[0], cached_tensor.shape[1], gradient, cached_tensor.ptr(), cached_tensor.strides[0],
+                         cached_tensor.strides[1], target.ptr(), target.strides[0], target.strides[1], r.ptr(), r.strides[0], r.strides[1]));
+  return r;
+}
+template <typename T>
+HipTensor<T> sparse_softmax_cross_entropy_backward(T gradient, const HipTensor<T>& cached_tensor, const HipTensor<int64_t>& target) {
+  if (cached_tensor.rank() != 2 || target.rank() != 1 || target.shape[0] != cached_tensor.shape[0])
+    throw std::invalid_argument("sparse_softmax_cross_entropy_backward: one label per row of the input is needed");
+  HipTensor<T> r(cached_tensor.shape);
+  check(detail::sparse_sce_bwd_(cached_tensor.shape[0], cached_tensor.shape[1], gradient, cached_tensor.ptr(), cached_tensor.strides[0],
+                                cached_tensor.strides[1], target.ptr(), target.strides[0], r.ptr(), r.strides[0], r.strides[1]));
+  return r;
+}
+
 // conv2d = im2colgemm_conv2d (nn_primitives/fallback/conv.nim:81-106), bias [C_out] or [C_out, 1, 1], optionally
 // followed by relu. Float tensors with `fused`: one launch, the GEMM's B loader gathers the column matrix from the
 // images. Otherwise (integer tensors, or asked for): device im2col of the batch, then one strided-batched GEMM

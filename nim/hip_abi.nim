@@ -147,6 +147,14 @@ proc am_hip_reduce_all_i32*(op, rank: cint, shape: ptr int64, a: ptr int32, a_st
 proc am_hip_reduce_all_i64*(op, rank: cint, shape: ptr int64, a: ptr int64, a_strides: ptr int64, res: ptr int64): cint {.importc.}
 proc am_hip_softmax_rows_f32*(rows, cols: int64, dst: ptr cfloat, dst_rs, dst_cs: int64, src: ptr cfloat, src_rs, src_cs: int64): cint {.importc.}
 proc am_hip_softmax_rows_f64*(rows, cols: int64, dst: ptr cdouble, dst_rs, dst_cs: int64, src: ptr cdouble, src_rs, src_cs: int64): cint {.importc.}
+proc am_hip_softmax_cross_entropy_f32*(rows, cols: int64, input: ptr cfloat, in_rs, in_cs: int64, target: ptr cfloat, t_rs, t_cs: int64, loss: ptr cfloat): cint {.importc.}
+proc am_hip_sparse_softmax_cross_entropy_f32*(rows, cols: int64, input: ptr cfloat, in_rs, in_cs: int64, labels: ptr int64, labels_s: int64, loss: ptr cfloat): cint {.importc.}
+proc am_hip_softmax_cross_entropy_backward_f32*(rows, cols: int64, gradient: cfloat, input: ptr cfloat, in_rs, in_cs: int64, target: ptr cfloat, t_rs, t_cs: int64, res: ptr cfloat, r_rs, r_cs: int64): cint {.importc.}
+proc am_hip_sparse_softmax_cross_entropy_backward_f32*(rows, cols: int64, gradient: cfloat, input: ptr cfloat, in_rs, in_cs: int64, labels: ptr int64, labels_s: int64, res: ptr cfloat, r_rs, r_cs: int64): cint {.importc.}
+proc am_hip_softmax_cross_entropy_f64*(rows, cols: int64, input: ptr cdouble, in_rs, in_cs: int64, target: ptr cdouble, t_rs, t_cs: int64, loss: ptr cdouble): cint {.importc.}
+proc am_hip_sparse_softmax_cross_entropy_f64*(rows, cols: int64, input: ptr cdouble, in_rs, in_cs: int64, labels: ptr int64, labels_s: int64, loss: ptr cdouble): cint {.importc.}
+proc am_hip_softmax_cross_entropy_backward_f64*(rows, cols: int64, gradient: cdouble, input: ptr cdouble, in_rs, in_cs: int64, target: ptr cdouble, t_rs, t_cs: int64, res: ptr cdouble, r_rs, r_cs: int64): cint {.importc.}
+proc am_hip_sparse_softmax_cross_entropy_backward_f64*(rows, cols: int64, gradient: cdouble, input: ptr cdouble, in_rs, in_cs: int64, labels: ptr int64, labels_s: int64, res: ptr cdouble, r_rs, r_cs: int64): cint {.importc.}
 proc am_hip_maxpool2d_backward_f32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, argmax: ptr int64, grad_output: ptr cfloat, grad_input: ptr cfloat): cint {.importc.}
 proc am_hip_maxpool2d_backward_f64*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, argmax: ptr int64, grad_output: ptr cdouble, grad_input: ptr cdouble): cint {.importc.}
 proc am_hip_maxpool2d_backward_i32*(N: int64, C, H, W, kH, kW, padH, padW, strideH, strideW: cint, argmax: ptr int64, grad_output: ptr int32, grad_input: ptr int32): cint {.importc.}

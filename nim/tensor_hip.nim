@@ -624,6 +624,47 @@ proc softmax*[T: float32 | float64](input: HipTensor[T]): HipTensor[T] =
     check am_hip_softmax_rows_f64(int64 input.shape[0], int64 input.shape[1], result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
       input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1])
 
+proc softmax_cross_entropy*[T: float32 | float64](input, target: HipTensor[T]): T =
+  ## nn_primitives/nnp_softmax_cross_entropy.nim:17-86: softmax and cross-entropy in one pass, averaged over the batch.
+  assert input.rank == 2 and input.shape == target.shape
+  template call(f: untyped) =
+    check f(int64 input.shape[0], int64 input.shape[1], input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1],
+            target.get_offset_ptr, int64 target.strides[0], int64 target.strides[1], result.addr)
+  when T is float32: call am_hip_softmax_cross_entropy_f32
+  else: call am_hip_softmax_cross_entropy_f64
+
+proc sparse_softmax_cross_entropy*[T: float32 | float64](input: HipTensor[T], target: HipTensor[int64]): T =
+  ## nnp_softmax_cross_entropy.nim:88-177: one class index per row.
+  assert input.rank == 2 and target.rank == 1 and target.shape[0] == input.shape[0]
+  template call(f: untyped) =
+    check f(int64 input.shape[0], int64 input.shape[1], input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1],
+            target.get_offset_ptr, int64 target.strides[0], result.addr)
+  when T is float32: call am_hip_sparse_softmax_cross_entropy_f32
+  else: call am_hip_sparse_softmax_cross_entropy_f64
+
+proc softmax_cross_entropy_backward*[T: float32 | float64](gradient: T, cached_tensor, target: HipTensor[T]): HipTensor[T] =
+  ## nnp_softmax_cross_entropy.nim:186-214: gradient * (softmax(cached_tensor) - target) / batch_size, one launch.
+  assert cached_tensor.rank == 2 and cached_tensor.shape == target.shape
+  result = newHipTensor[T](cached_tensor.shape)
+  template call(f: untyped) =
+    check f(int64 cached_tensor.shape[0], int64 cached_tensor.shape[1], gradient, cached_tensor.get_offset_ptr,
+            int64 cached_tensor.strides[0], int64 cached_tensor.strides[1], target.get_offset_ptr, int64 target.strides[0],
+            int64 target.strides[1], result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1])
+  when T is float32: call am_hip_softmax_cross_entropy_backward_f32
+  else: call am_hip_softmax_cross_entropy_backward_f64
+
+proc sparse_softmax_cross_entropy_backward*[T: float32 | float64](gradient: T, cached_tensor: HipTensor[T],
+                                                                  target: HipTensor[int64]): HipTensor[T] =
+  ## nnp_softmax_cross_entropy.nim:217-256: gradient * (softmax(cached_tensor) - onehot(target)) / batch_size, one launch.
+  assert cached_tensor.rank == 2 and target.rank == 1 and target.shape[0] == cached_tensor.shape[0]
+  result = newHipTensor[T](cached_tensor.shape)
+  template call(f: untyped) =
+    check f(int64 cached_tensor.shape[0], int64 cached_tensor.shape[1], gradient, cached_tensor.get_offset_ptr,
+            int64 cached_tensor.strides[0], int64 cached_tensor.strides[1], target.get_offset_ptr, int64 target.strides[0],
+            result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1])
+  when T is float32: call am_hip_sparse_softmax_cross_entropy_backward_f32
+  else: call am_hip_sparse_softmax_cross_entropy_backward_f64
+
 proc conv2d*[T: SomeFloat](input, kernel, bias: HipTensor[T], padding = (0, 0), stride = (1, 1), relu = false): HipTensor[T] =
   ## im2colgemm_conv2d (nn_primitives/fallback/conv.nim:81-106), optionally followed by relu, in one launch: the GEMM's
   ## B loader gathers the column matrix from the images. input [N, C, H, W], kernel [C_out, C, kH, kW] (C-contiguous),

@@ -464,6 +464,72 @@ def softmax(x: np.ndarray) -> np.ndarray:
     return out
 
 
+def streaming_max_sumexp(x: np.ndarray):
+    """Row by row the one-pass recurrence of streaming_max_sumexp (src/arraymancer/nn_primitives/private/
+    p_logsumexp.nim:20-31), in the element type: the running maximum and the sum of exp(x - maximum), rescaled whenever
+    the maximum moves. All rows advance together, each through its own elements in order. Returns (max, sumexp)."""
+    dt = x.dtype.type
+    mx = np.full(x.shape[0], -np.inf, dtype=x.dtype)
+    se = np.zeros(x.shape[0], dtype=x.dtype)
+    with np.errstate(over="ignore", invalid="ignore"):
+        for j in range(x.shape[1]):
+            val = x[:, j]
+            le = val <= mx
+            se = np.where(le, se + np.exp(val - mx), se * np.exp(mx - val) + dt(1)).astype(x.dtype)
+            mx = np.where(le, mx, val)
+    return mx, se
+
+
+def softmax_cross_entropy(x: np.ndarray, target: np.ndarray):
+    """softmax_cross_entropy (src/arraymancer/nn_primitives/nnp_softmax_cross_entropy.nim:17-86): per row
+    ln(sumexp) + max - dot(row, target row), summed over the rows in order, divided by the batch size."""
+    dt = x.dtype.type
+    if x.shape[0] == 0:
+        return dt(0)
+    mx, se = streaming_max_sumexp(x)
+    dot = np.zeros(x.shape[0], dtype=x.dtype)
+    for j in range(x.shape[1]):
+        dot = (dot + x[:, j] * target[:, j]).astype(x.dtype)
+    local = (np.log(se) + mx - dot).astype(x.dtype)
+    total = dt(0)
+    for v in local:
+        total = dt(total + v)
+    return dt(total / dt(x.shape[0]))
+
+
+def sparse_softmax_cross_entropy(x: np.ndarray, labels: np.ndarray):
+    """sparse_softmax_cross_entropy (nnp_softmax_cross_entropy.nim:88-177): per row ln(sumexp) + max - row[label]."""
+    dt = x.dtype.type
+    if x.shape[0] == 0:
+        return dt(0)
+    mx, se = streaming_max_sumexp(x)
+    local = ((np.log(se) + mx).astype(x.dtype) - x[np.arange(x.shape[0]), labels.astype(np.int64)]).astype(x.dtype)
+    total = dt(0)
+    for v in local:
+        total = dt(total + v)
+    return dt(total / dt(x.shape[0]))
+
+
+def softmax_cross_entropy_backward(gradient, x: np.ndarray, target: np.ndarray) -> np.ndarray:
+    """softmax_cross_entropy_backward (nnp_softmax_cross_entropy.nim:186-214):
+    grad * (exp(x - max) / sumexp - target) / batch_size, every step rounded in the element type."""
+    dt = x.dtype.type
+    mx, se = streaming_max_sumexp(x)
+    sm = (np.exp(x - mx[:, None]) / se[:, None]).astype(x.dtype)
+    return ((dt(gradient) * (sm - target)).astype(x.dtype) / dt(x.shape[0])).astype(x.dtype)
+
+
+def sparse_softmax_cross_entropy_backward(gradient, x: np.ndarray, labels: np.ndarray) -> np.ndarray:
+    """sparse_softmax_cross_entropy_backward (nnp_softmax_cross_entropy.nim:217-256): the result starts as -1 at each
+    row's label and 0 elsewhere, then grad * (softmax + that) / batch_size."""
+    dt = x.dtype.type
+    mx, se = streaming_max_sumexp(x)
+    sm = (np.exp(x - mx[:, None]) / se[:, None]).astype(x.dtype)
+    start = np.zeros_like(x)
+    start[np.arange(x.shape[0]), labels.astype(np.int64)] = dt(-1)
+    return ((dt(gradient) * (sm + start)).astype(x.dtype) / dt(x.shape[0])).astype(x.dtype)
+
+
 def maxpool2d(x: np.ndarray, kernel, padding=(0, 0), stride=(1, 1)):
     """nnp_maxpooling.nim:19-66: (max_indices [N*C*outH*outW] int64, maxpooled [N, C, outH, outW])."""
     sfx = _sfx(x)

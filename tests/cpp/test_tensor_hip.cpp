@@ -243,6 +243,21 @@ template <typename T> static void conv_backward_known_answer() {
   CHECK(threw);
 }
 
+static void loss_literals() {
+  // tests/nn_primitives/test_nnp_loss.nim:31-44: one row, truth = class 3, loss 0.0709 within 2e-5, dense and sparse
+  auto predicted = toHip<double>({-3.44, 1.16, -0.81, 3.91}, {1, 4});
+  auto truth = toHip<double>({0, 0, 0, 1}, {1, 4});
+  auto sparse_truth = toHip<int64_t>(std::vector<int64_t>{3}, {1});
+  const double dense = am::softmax_cross_entropy(predicted, truth), sparse = am::sparse_softmax_cross_entropy(predicted, sparse_truth);
+  CHECK(std::fabs(dense - 0.0709) <= 2e-5 && std::fabs(sparse - 0.0709) <= 2e-5);
+  // the gradient: softmax - onehot, scaled; its entries sum to zero and only the true class is negative
+  auto g = am::softmax_cross_entropy_backward(1.0, predicted, truth).toCpu();
+  auto gs = am::sparse_softmax_cross_entropy_backward(1.0, predicted, sparse_truth).toCpu();
+  CHECK(std::fabs(g[0] + g[1] + g[2] + g[3]) < 1e-15 && g[3] < 0 && g[0] > 0 && g[1] > 0 && g[2] > 0);
+  CHECK(std::fabs(g[3] - (std::exp(-dense) - 1.0)) < 1e-12);   // softmax of the true class is exp(-loss)
+  for (int i = 0; i < 4; ++i) CHECK(std::fabs(g[i] - gs[i]) < 1e-15);
+}
+
 static void maxpool_backward() {
   // tests/nn_primitives/test_nnp_maxpool.nim:20-45
   auto a = toHip<float>({1, 1, 2, 4, 5, 6, 7, 8, 3, 2, 1, 0, 1, 2, 3, 4}, {1, 1, 4, 4});
@@ -430,6 +445,7 @@ int main(int argc, char** argv) {
   conv_literals<double>();
   conv_literals<int32_t>();
   conv_literals<int64_t>();
+  loss_literals();
   conv_backward_known_answer<float>();
   conv_backward_known_answer<double>();
   conv_backward_known_answer<int32_t>();

@@ -238,3 +238,70 @@ def test_maxpool_against_bruteforce(oracle, sfx):
                         assert out[n, c, h, w] == best and idx[o] == arg
                         if arg >= 0:
                             assert flat[arg] == best
+
+
+def _exact_sce(x, target):
+    """The loss from its definition in extended precision: mean over rows of logsumexp(row) - <row, target row>."""
+    xl, tl = x.astype(np.longdouble), target.astype(np.longdouble)
+    m = xl.max(1, keepdims=True)
+    lse = np.log(np.exp(xl - m).sum(1)) + m[:, 0]
+    return np.mean(lse - (xl * tl).sum(1))
+
+
+def test_cross_entropy_reference_literal(oracle):
+    """tests/nn_primitives/test_nnp_loss.nim:31-44: one row of four scores, the fourth class true: 0.0709 within 2e-5,
+    through the dense and the sparse form."""
+    predicted = np.array([[-3.44, 1.16, -0.81, 3.91]])
+    truth = np.array([[0.0, 0, 0, 1]])
+    assert abs(oracle.softmax_cross_entropy(predicted, truth) - 0.0709) <= 2e-5
+    assert abs(oracle.sparse_softmax_cross_entropy(predicted, np.array([3])) - 0.0709) <= 2e-5
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_cross_entropy_closed_forms_and_gradients(oracle, sfx):
+    """What the mathematics fixes for the restated one-pass recurrence: the loss against its definition in extended
+    precision (random soft targets; one-hot targets = the sparse form), shift invariance, ln(classes) for equal
+    scores, no overflow at +-1000; the backward forms against central differences of the loss (the reference's own
+    check, test_nnp_loss.nim:46-62 and 66-103) and against softmax - target entry by entry."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("sce-oracle", sfx))
+    tol = 2e-6 if sfx == "f32" else 1e-14
+    for rows, cols in ((1, 4), (7, 10), (256, 20), (5, 1), (3, 333)):
+        x = (rng.standard_normal((rows, cols)) * 3).astype(dt)
+        soft = rng.uniform(0, 1, (rows, cols))
+        soft = (soft / soft.sum(1, keepdims=True)).astype(dt)
+        labels = rng.integers(0, cols, rows)
+        onehot = np.zeros((rows, cols), dtype=dt)
+        onehot[np.arange(rows), labels] = 1
+        for target in (soft, onehot):
+            got = oracle.softmax_cross_entropy(x, target)
+            want = _exact_sce(x, target)
+            assert abs(got - want) <= tol * max(1.0, abs(want)) * 8, (rows, cols)
+        assert abs(oracle.sparse_softmax_cross_entropy(x, labels) - _exact_sce(x, onehot)) <= tol * 8 * max(1.0, abs(_exact_sce(x, onehot)))
+        assert abs(oracle.softmax_cross_entropy((x + dt(5)).astype(dt), onehot) - oracle.softmax_cross_entropy(x, onehot)) <= tol * 64
+        # gradients: g * (softmax - target) / rows, and the numerical gradient of the float64 loss
+        xl = x.astype(np.longdouble)
+        e = np.exp(xl - xl.max(1, keepdims=True))
+        sm = e / e.sum(1, keepdims=True)
+        g = dt(0.37)
+        for target, got in ((soft, oracle.softmax_cross_entropy_backward(g, x, soft)),
+                            (onehot, oracle.sparse_softmax_cross_entropy_backward(g, x, labels)),
+                            (onehot, oracle.softmax_cross_entropy_backward(g, x, onehot))):
+            want = np.longdouble(g) * (sm - target.astype(np.longdouble)) / rows
+            assert np.max(np.abs(got - want)) <= tol * 8, (rows, cols)
+        if sfx == "f64" and rows * cols <= 200:
+            num = np.zeros_like(x)
+            for idx in np.ndindex(*x.shape):
+                keep = x[idx]
+                x[idx] = keep + 1e-5; up = oracle.softmax_cross_entropy(x, soft)
+                x[idx] = keep - 1e-5; dn = oracle.softmax_cross_entropy(x, soft)
+                x[idx] = keep
+                num[idx] = (up - dn) / 2e-5
+            assert np.max(np.abs(oracle.softmax_cross_entropy_backward(1.0, x, soft) - num)) < 1e-9
+    flat = np.zeros((3, 8), dtype=dt)
+    assert abs(oracle.sparse_softmax_cross_entropy(flat, np.array([0, 3, 7])) - np.log(8)) <= tol * 8
+    big = np.array([[1000, -1000, 999], [-1000, -1001, -999]], dtype=dt)
+    v = oracle.sparse_softmax_cross_entropy(big, np.array([0, 2]))
+    # ln(sumexp) + max is rounded at the magnitude of the scores before the score of the true class is subtracted
+    assert np.isfinite(v) and abs(v - _exact_sce(big, np.array([[1, 0, 0], [0, 0, 1]], dtype=dt))) <= np.finfo(dt).eps * 1000 * 2
+    assert oracle.softmax_cross_entropy(np.zeros((0, 4), dtype=dt), np.zeros((0, 4), dtype=dt)) == 0
