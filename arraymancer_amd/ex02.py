@@ -1,5 +1,5 @@
-"""The forward pass of the reference's example 2 (examples/ex02_handwritten_digits_recognition.nim:36-46),
-composed from the device operators of this package:
+"""The network of the reference's example 2 (examples/ex02_handwritten_digits_recognition.nim:36-46), its forward pass
+and one step of its learning loop (:58-72), composed from the device operators of this package:
 
     x.cv1.relu.mp1.cv2.relu.mp2.fl.hidden.relu.classifier
     cv1 = Conv2D(1 -> 20, 5x5)   mp1 = MaxPool2D(2x2, stride 2)   cv2 = Conv2D(20 -> 50, 5x5)   mp2 = MaxPool2D(2x2, stride 2)
@@ -19,7 +19,9 @@ import numpy as np
 
 from . import _lib
 from ._lib import check
-from .tensor_hip import Graph, HipTensor, conv2d_into, empty, gemm, toHip
+from .tensor_hip import (Graph, HipTensor, _ternary_into, conv2d_backward, conv2d_into, empty, gemm, linear_backward,
+                         maxpool2d_backward, relu_backward, sparse_softmax_cross_entropy,
+                         sparse_softmax_cross_entropy_backward, toHip)
 
 
 class DemoNet:
@@ -61,6 +63,43 @@ class DemoNet:
         gemm(1, flat, p["hidden_w"].transpose(), 0, self.hidden, epilogue="bias_relu", bias=p["hidden_b"])
         gemm(1, self.hidden, p["classifier_w"].transpose(), 0, self.logits, epilogue="bias", bias=p["classifier_b"])
         return self.logits
+
+    def loss_and_gradients(self, x: HipTensor, labels: HipTensor):
+        """One training pass of the example's learning loop (examples/ex02_handwritten_digits_recognition.nim:58-72)
+        without the update: forward, `sparse_softmax_cross_entropy` against the int64 `labels` [batch], and what
+        `loss.backprop()` walks through, composed from the backward primitives in the order of the forward pass
+        reversed (nnp_softmax_cross_entropy.nim:217-256, nnp_linear.nim:39-66, nnp_activation.nim:65-70,
+        nnp_maxpooling.nim:68-83, nnp_convolution.nim:65-107). Returns (loss, gradients by parameter name)."""
+        p, n = self.p, self.batch
+        logits = self.forward(x)
+        loss = sparse_softmax_cross_entropy(logits, labels)
+        d_logits = sparse_softmax_cross_entropy_backward(1, logits, labels)
+        flat = self.pool2.reshape(n, self.pool2.size // n)
+        d_hidden, g_cw, g_cb = linear_backward(self.hidden, p["classifier_w"], d_logits)
+        d_hidden = relu_backward(d_hidden, self.hidden)
+        d_flat, g_hw, g_hb = linear_backward(flat, p["hidden_w"], d_hidden)
+        pool = dict(kernel=(2, 2), padding=(0, 0), stride=(2, 2))
+        d_a2 = maxpool2d_backward(self.a2.shape, self.idx2, d_flat.reshape(*self.pool2.shape), **pool)
+        d_a2 = relu_backward(d_a2, self.a2)
+        d_pool1, g_k2, g_b2 = conv2d_backward(self.pool1, p["cv2_w"], p["cv2_b"], (0, 0), (1, 1), d_a2)
+        d_a1 = maxpool2d_backward(self.a1.shape, self.idx1, d_pool1, **pool)
+        d_a1 = relu_backward(d_a1, self.a1)
+        _, g_k1, g_b1 = conv2d_backward(x, p["cv1_w"], p["cv1_b"], (0, 0), (1, 1), d_a1)
+        return loss, dict(cv1_w=g_k1, cv1_b=g_b1, cv2_w=g_k2, cv2_b=g_b2, hidden_w=g_hw, hidden_b=g_hb,
+                          classifier_w=g_cw, classifier_b=g_cb)
+
+    def sgd_update(self, gradients: dict, learning_rate: float):
+        """The SGD optimizer's update (src/arraymancer/nn/optimizers/optimizers.nim:35-51: x - lr * y over every parameter)
+        as one pass per parameter: value = grad * (-learning_rate) + value, the same two roundings."""
+        step = toHip(np.array([-learning_rate], dtype=self.dtype))
+        for name, g in gradients.items():
+            w = self.p[name]
+            _ternary_into("muladd", w, g, step.reshape(*([1] * w.rank)).broadcast(w.shape), w)
+
+    def train_step(self, x: HipTensor, labels: HipTensor, learning_rate: float = 0.01):
+        loss, gradients = self.loss_and_gradients(x, labels)
+        self.sgd_update(gradients, learning_rate)
+        return loss
 
     def capture(self, x: HipTensor) -> Graph:
         """Records one forward pass over `x` into a HIP graph (run one eager pass first: the GEMM workspace must

@@ -371,6 +371,7 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     out.append(bench_chain(am, timer, max(steps, 50), warmup))
     out.append(bench_ex02(am, timer, max(steps, 50), warmup))
     out.extend(bench_conv_backward(am, timer, steps, warmup))
+    out.append(bench_ex02_train(am, timer, max(steps, 20), warmup))
     return out
 
 
@@ -436,6 +437,25 @@ def bench_ex02(am, timer, steps, warmup, batch=64):
                 images_per_s=round(batch / (best / steps), 0), gflops=round(flops / (best / steps) / 1e9, 1),
                 note="3.0e8 FLOP per pass over six kernels of 3-15 us each: the graph replay runs them back to back (its time is "
                      "the sum of their durations), the eager pass adds the host's launch gap after each")
+
+
+def bench_ex02_train(am, timer, steps, warmup, batch=64):
+    """One step of example 2's learning loop at batch 64: forward, sparse softmax cross-entropy (read back to the
+    host), the backward primitives, the SGD update of the eight parameters."""
+    from arraymancer_amd import ex02
+    rng = np.random.default_rng(5003)
+    net = ex02.DemoNet(batch, ex02.random_params(rng), np.float32)
+    dx = am.toHip(rng.uniform(0, 1, (batch, 1, 28, 28)).astype(np.float32))
+    dl = am.toHip(rng.integers(0, 10, batch).astype(np.int64))
+    wall, ev = timer.run(lambda: net.train_step(dx, dl, 0.01), steps, warmup, WARM_S)
+    flops = 3 * 2.0 * batch * (20 * 25 * 576 + 50 * 500 * 64 + 800 * 500 + 500 * 10)
+    return dict(workload=f"f32 example-2 training step, batch {batch}: forward, sparse softmax cross-entropy, backward through "
+                         "linear / ReLU / maxpool / conv2d, SGD update of 8 parameters",
+                unit="us per step", dtype="f32", higher_is_better=False, value=round(ev / steps * 1e6, 2),
+                wall_us=round(wall / steps * 1e6, 2), images_per_s=round(batch / (ev / steps), 0),
+                gflops=round(flops / (ev / steps) / 1e9, 1),
+                note="about forty short launches issued one by one from the host (the loss is read back every step, as the "
+                     "example prints it): bound by the host's launch rate, not by the 0.9 GFLOP of arithmetic")
 
 
 def bench_conv_backward(am, timer, steps, warmup):

@@ -79,3 +79,72 @@ def test_ex02_forward(hip, oracle, sfx, batch):
         g.launch()
         hip.sync()
         assert np.array_equal(net.logits.toCpu(), eager), f"replay {rep}"
+
+
+def oracle_backward(oracle, x, labels, p):
+    """Loss and parameter gradients of one learning step through the oracle's primitives, in the reference's order."""
+    st = oracle_stages(oracle, x, p)
+    n = x.shape[0]
+    loss = oracle.sparse_softmax_cross_entropy(st["logits"], labels)
+    d_logits = oracle.sparse_softmax_cross_entropy_backward(1, st["logits"], labels)
+
+    def linear_bwd(inp, w, go):                                   # nnp_linear.nim:39-55
+        return oracle.matmul(go, w), oracle.matmul(go.T, inp), oracle.reduce_axis("sum", go, 0)
+
+    relu_bwd = lambda g, cached: oracle.map2("relu_bwd", cached, g)   # nnp_activation.nim:65-70
+    d_hidden, g_cw, g_cb = linear_bwd(st["hidden"], p["classifier_w"], d_logits)
+    d_hidden = relu_bwd(d_hidden, st["hidden"])
+    d_flat, g_hw, g_hb = linear_bwd(st["pool2"].reshape(n, -1), p["hidden_w"], d_hidden)
+    d_a2 = oracle.maxpool2d_backward(st["a2"].shape, st["idx2"], np.ascontiguousarray(d_flat.reshape(st["pool2"].shape)))
+    d_a2 = relu_bwd(d_a2, st["a2"])
+    d_pool1, g_k2, g_b2 = oracle.conv2d_backward(st["pool1"], p["cv2_w"], p["cv2_b"], (0, 0), (1, 1), d_a2)
+    d_a1 = oracle.maxpool2d_backward(st["a1"].shape, st["idx1"], d_pool1)
+    d_a1 = relu_bwd(d_a1, st["a1"])
+    _, g_k1, g_b1 = oracle.conv2d_backward(x, p["cv1_w"], p["cv1_b"], (0, 0), (1, 1), d_a1)
+    return loss, dict(cv1_w=g_k1, cv1_b=g_b1, cv2_w=g_k2, cv2_b=g_b2, hidden_w=g_hw, hidden_b=g_hb, classifier_w=g_cw, classifier_b=g_cb)
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_ex02_training_step(hip, oracle, sfx):
+    """One step of the example's learning loop (examples/ex02_handwritten_digits_recognition.nim:58-72) on the device:
+    forward, sparse softmax cross-entropy, the backward primitives in reverse order, the SGD update. The gradients
+    against the same chain through the oracle; in float64 also against central differences of the oracle's loss for
+    a few entries of every parameter; the update bit for bit against x - lr * y; and the loss of a fixed batch goes down."""
+    from arraymancer_amd import ex02
+    dt, batch = DT[sfx], 16
+    rng = np.random.default_rng(seed_of("ex02-train", sfx))
+    p = ex02.random_params(rng, dt)
+    x = rng.uniform(0, 1, (batch, 1, 28, 28)).astype(dt)
+    labels = rng.integers(0, 10, batch).astype(np.int64)
+    net = ex02.DemoNet(batch, p, dt)
+    dx, dl = hip.toHip(x), hip.toHip(labels)
+    say("ex02 training step", sfx)
+    loss, grads = net.loss_and_gradients(dx, dl)
+    want_loss, want = oracle_backward(oracle, x, labels, p)
+    assert abs(loss - want_loss) <= (1e-5 if sfx == "f32" else 1e-12) * max(1.0, abs(want_loss))
+    for name, g in grads.items():
+        assert g.shape == p[name].shape, name
+        err = oracle.rel_frobenius(g.toCpu(), want[name].reshape(p[name].shape))
+        say(f"  gradient of {name}: {err:.2e}")
+        assert err <= (2e-4 if sfx == "f32" else 1e-11), name
+    if sfx == "f64":
+        def loss_at():
+            return float(oracle.sparse_softmax_cross_entropy(oracle_stages(oracle, x, p)["logits"], labels))
+        for name in p:
+            flat = p[name].reshape(-1)
+            got = grads[name].toCpu().reshape(-1)
+            for i in rng.choice(flat.size, 3, replace=False):
+                keep = flat[i]
+                flat[i] = keep + 1e-5; up = loss_at()
+                flat[i] = keep - 1e-5; dn = loss_at()
+                flat[i] = keep
+                num = (up - dn) / 2e-5
+                assert abs(got[i] - num) <= 1e-6 * max(1e-3, abs(num)), (name, i, got[i], num)
+    before = {k: v.toCpu().copy() for k, v in net.p.items()}
+    host_grads = {k: g.toCpu().copy() for k, g in grads.items()}
+    net.sgd_update(grads, 0.01)
+    for name in p:
+        assert np.array_equal(net.p[name].toCpu(), before[name] - dt(0.01) * host_grads[name].reshape(before[name].shape)), name
+    losses = [float(loss)] + [float(net.train_step(dx, dl, 0.01)) for _ in range(5)]
+    say("  losses over six steps on one batch:", [round(v, 4) for v in losses])
+    assert losses[-1] < losses[0]
