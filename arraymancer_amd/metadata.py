@@ -81,6 +81,28 @@ def permute(l: Layout, dims: Sequence[int]) -> Layout:
     return Layout(tuple(l.shape[d] for d in dims), tuple(l.strides[d] for d in dims), l.offset)
 
 
+def squeeze(l: Layout, axis: int | None = None) -> Layout:
+    """Drops the dimensions of extent 1 (all of them, keeping rank >= 1, or the one at `axis` if it has extent 1 and the
+    rank is above 1): squeezeImpl, src/arraymancer/tensor/private/p_shapeshifting.nim:157-177."""
+    if axis is None:
+        keep = [i for i, n in enumerate(l.shape) if n != 1] or [len(l.shape) - 1]
+        return Layout(tuple(l.shape[i] for i in keep), tuple(l.strides[i] for i in keep), l.offset)
+    if not 0 <= axis < len(l.shape):
+        raise IndexError(f"squeeze: axis {axis} outside the tensor's rank {len(l.shape)}")
+    if len(l.shape) > 1 and l.shape[axis] == 1:
+        return Layout(l.shape[:axis] + l.shape[axis + 1:], l.strides[:axis] + l.strides[axis + 1:], l.offset)
+    return l
+
+
+def unsqueeze(l: Layout, axis: int) -> Layout:
+    """Inserts a dimension of extent 1 at `axis`, with the stride the reference gives it
+    (unsqueezeImpl, private/p_shapeshifting.nim:179-191)."""
+    if not 0 <= axis <= len(l.shape):
+        raise IndexError(f"unsqueeze: axis {axis} outside 0..{len(l.shape)}")
+    stride = 1 if axis >= len(l.shape) else l.shape[axis] * l.strides[axis]
+    return Layout(l.shape[:axis] + (1,) + l.shape[axis:], l.strides[:axis] + (stride,) + l.strides[axis:], l.offset)
+
+
 class Step:
     """One slice in the reference's notation: first..last|step with INCLUSIVE ends;
     `first_from_end` / `last_from_end` are the `^n` forms (index = extent - n)."""

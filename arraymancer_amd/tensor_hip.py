@@ -140,6 +140,14 @@ class HipTensor:
     def T(self):
         return self.transpose()
 
+    def squeeze(self, axis: int | None = None) -> "HipTensor":
+        """Without the dimensions of extent 1, or without the one at `axis` (shapeshifting.nim:396-413)."""
+        return HipTensor(md.squeeze(self.layout, axis), self.storage, self.dtype)
+
+    def unsqueeze(self, axis: int) -> "HipTensor":
+        """With a dimension of extent 1 inserted at `axis` (shapeshifting.nim:415-424)."""
+        return HipTensor(md.unsqueeze(self.layout, axis), self.storage, self.dtype)
+
     def permute(self, *dims) -> "HipTensor":
         """The dimensions in a new order, same data (src/arraymancer/tensor/shapeshifting.nim:207-226)."""
         if len(dims) == 1 and not isinstance(dims[0], int):
@@ -638,6 +646,80 @@ def linear_backward(input: HipTensor, weight: HipTensor, gradOutput: HipTensor, 
     if not with_bias:
         return grad_input, grad_weight
     return grad_input, grad_weight, tsum(gradOutput, axis=0)
+
+
+# ---------------------------------------------------------------------- gated recurrent unit
+def gru_cell_inference(input: HipTensor, W3: HipTensor, U3: HipTensor, bW3: HipTensor, bU3: HipTensor, hidden: HipTensor) -> HipTensor:
+    """gru_cell_inference (src/arraymancer/nn_primitives/nnp_gru.nim:40-88): h(t) -> h'(t) in place. Two dense layers
+    with the bias in the GEMM epilogue ([batch, 3H] each), then the three gate passes in place on column slices of those
+    buffers: sigmoid(x + y) over the reset and update columns together, tanh(x + y * z) for the candidate,
+    (1 - y) * z + y * x into `hidden`. input [batch, features], W3 [3H, features], U3 [3H, H], biases [1, 3H]."""
+    H = hidden.shape[1]
+    W3x, U3h = linear(input, W3, bW3), linear(hidden, U3, bU3)
+    srz, sr, sz, s_ = slice(0, 2 * H), slice(0, H), slice(H, 2 * H), slice(2 * H, 3 * H)
+    apply2("add_sigmoid", W3x[:, srz], U3h[:, srz])
+    apply3("gru_candidate", W3x[:, s_], W3x[:, sr], U3h[:, s_])
+    apply3("gru_blend", hidden, W3x[:, sz], W3x[:, s_])
+    return hidden
+
+
+def gru_cell_forward(input: HipTensor, W3: HipTensor, U3: HipTensor, bW3: HipTensor, bU3: HipTensor, hidden: HipTensor):
+    """gru_cell_forward (nnp_gru.nim:90-146): like gru_cell_inference, keeping what the backward pass needs. Updates
+    `hidden` in place and returns (r, z, n, Uh), each [batch, H] (r and z are the two halves of one buffer)."""
+    H = hidden.shape[1]
+    W3x, U3h = linear(input, W3, bW3), linear(hidden, U3, bU3)
+    sr, sz, s_ = slice(0, H), slice(H, 2 * H), slice(2 * H, 3 * H)
+    Uh = U3h[:, s_].clone()
+    rz = map2("add_sigmoid", W3x[:, 0:2 * H], U3h[:, 0:2 * H])
+    r, z = rz[:, sr], rz[:, sz]
+    n = map3("gru_candidate", W3x[:, s_], r, U3h[:, s_])
+    apply3("gru_blend", hidden, z, n)
+    return r, z, n, Uh
+
+
+def gru_cell_backward(dnext: HipTensor, x: HipTensor, h: HipTensor, W3: HipTensor, U3: HipTensor,
+                      r: HipTensor, z: HipTensor, n: HipTensor, Uh: HipTensor):
+    """gru_cell_backward (nnp_gru.nim:148-192): (dx, dh, dW3, dU3, dbW3, dbU3) from the gradient `dnext` of the next
+    hidden state, the inputs of the forward pass (h is the hidden state BEFORE it) and the tensors it saved. The
+    reference concatenates the three gate gradients; here they are written into column slices of one [batch, 3H]
+    buffer per dense layer."""
+    B, H = h.shape
+    sr, sz, s_ = slice(0, H), slice(H, 2 * H), slice(2 * H, 3 * H)
+    dW3x, dU3h = empty((B, 3 * H), h.dtype), empty((B, 3 * H), h.dtype)
+    dz = map2("mul", map2("sub", h, n), dnext)                                   # step 4, z part
+    dn = map2("mul", scalar_op("sub", z, 1, scalar_on_left=True), dnext)
+    _binary_into("tanh_bwd", dW3x[:, s_], n, dn)                                 # step 3: dWx = dn * (1 - n * n)
+    dr = map2("mul", Uh, dW3x[:, s_])
+    _binary_into("mul", dU3h[:, s_], r, dW3x[:, s_])                             # dUh = r * dWx
+    _binary_into("sigmoid_bwd", dW3x[:, sz], z, dz)                              # step 2: update gate
+    _binary_into("sigmoid_bwd", dW3x[:, sr], r, dr)                              # step 2: reset gate
+    _unary_into("copy", dU3h[:, 0:2 * H], dW3x[:, 0:2 * H])                      # dUrh = dWrx, dUzh = dWzx
+    dx, dW3, dbW3 = linear_backward(x, W3, dW3x)                                 # step 1
+    dh, dU3, dbU3 = linear_backward(h, U3, dU3h)
+    _ternary_into("muladd", dh, dnext, z, dh)                                    # step 4, h part: dh + dnext * z
+    return dx, dh, dW3, dU3, dbW3, dbU3
+
+
+def gru_inference(input: HipTensor, W3s0: HipTensor, W3sN: HipTensor | None, U3s: HipTensor, bW3s: HipTensor, bU3s: HipTensor,
+                  hidden: HipTensor) -> HipTensor:
+    """gru_inference (nnp_gru.nim:194-262): a stack of GRU layers over a sequence. input [timesteps, batch, features];
+    W3s0 [3H, features]; W3sN [layers - 1, 3H, H] (None or empty for one layer); U3s [layers, 3H, H]; biases
+    [layers, 1, 3H]; hidden [layers, batch, H], updated in place to the state after the last timestep. Returns the
+    output [timesteps, batch, H]: the top layer's hidden state at every timestep."""
+    T, B, F = input.shape
+    H = hidden.shape[2]
+    layers = 1 + (W3sN.shape[0] if W3sN is not None and W3sN.size else 0)
+    if hidden.shape != (layers, B, H) or W3s0.shape != (3 * H, F) or U3s.shape != (layers, 3 * H, H) or \
+            bW3s.shape != (layers, 1, 3 * H) or bU3s.shape != bW3s.shape or (layers > 1 and W3sN.shape != (layers - 1, 3 * H, H)):
+        raise ValueError("gru_inference: shapes of the weights, biases and hidden state do not fit the input")
+    output = empty((T, B, H), input.dtype)
+    for layer in range(layers):
+        W3l = W3s0 if layer == 0 else W3sN[layer - 1].squeeze(0)
+        U3l, bW3l, bU3l, h_l = U3s[layer].squeeze(0), bW3s[layer].squeeze(0), bU3s[layer].squeeze(0), hidden[layer].squeeze(0)
+        for t in range(T):
+            gru_cell_inference((input[t] if layer == 0 else output[t]).squeeze(0), W3l, U3l, bW3l, bU3l, h_l)
+            _unary_into("copy", output[t].squeeze(0), h_l)
+    return output
 
 
 # ---------------------------------------------------------------------- element-wise

@@ -1,0 +1,153 @@
+"""The GRU primitives on the GPU (src/arraymancer/nn_primitives/nnp_gru.nim): the reference's own vectors
+(tests/nn_primitives/test_nnp_gru.nim:10-57 one cell, :178-268 two stacked layers over four timesteps, values it took
+from PyTorch / cuDNN, mean relative error below 1e-8 in float64), the cell's backward pass against the numerical
+gradient of the forward pass as the reference checks it (:78-172, mean absolute error below 1e-8), and larger random
+cells against the same chain through the oracle's operators."""
+import numpy as np
+import pytest
+
+from conftest import seed_of
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+X = [[0.1, 0.2, 0.3, 0.4], [-0.1, -0.2, -0.3, -0.4], [0.5, 0.6, 0.7, 0.8]]
+HIDDEN = [[-1.0, -1.0]] * 3
+W3 = [[0.9, 0.8, 0.7, 0.6], [0.8, 0.7, 0.6, 0.5], [0.7, 0.6, 0.5, 0.4], [0.6, 0.5, 0.4, 0.3], [0.5, 0.4, 0.3, 0.2], [0.4, 0.3, 0.2, 0.1]]
+U3 = [[-0.3, -0.1], [-0.2, 0.0], [-0.3, -0.1], [-0.2, 0.0], [-0.3, -0.1], [-0.2, 0.0]]
+BW3 = [[0.1, 0.2, 0.3, 0.4, 0.5, 0.6]]
+BU3 = [[-0.1, -0.2, -0.3, -0.4, -0.5, -0.6]]
+PYTORCH_CELL = [[-0.5317437280, -0.4752916969], [-0.3930421219, -0.3209550879], [-0.7325259335, -0.6429624731]]
+
+
+def mean_relative_error(got, want):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = np.maximum(np.abs(got), np.abs(want))
+    return np.mean(np.where(d == 0, 0.0, np.abs(got - want) / np.where(d == 0, 1.0, d)))
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float64, 1e-8), (np.float32, 1e-6)])
+def test_cell_reference_vectors(hip, dt, tol):
+    arrs = [np.array(v, dtype=dt) for v in (X, W3, U3, BW3, BU3)]
+    dev = [hip.toHip(a) for a in arrs]
+    h = hip.toHip(np.array(HIDDEN, dtype=dt))
+    assert hip.gru_cell_inference(*dev, h) is h
+    assert mean_relative_error(h.toCpu(), PYTORCH_CELL) < tol
+    h = hip.toHip(np.array(HIDDEN, dtype=dt))
+    r, z, n, Uh = hip.gru_cell_forward(*dev, h)
+    assert mean_relative_error(h.toCpu(), PYTORCH_CELL) < tol
+    assert all(t.shape == (3, 2) for t in (r, z, n, Uh))
+    # what was saved is what the forward pass used: h' = (1 - z) * n + z * h
+    zz, nn = z.toCpu().astype(np.float64), n.toCpu().astype(np.float64)
+    assert np.allclose((1 - zz) * nn + zz * np.array(HIDDEN), PYTORCH_CELL, rtol=0, atol=tol * 10)
+
+
+SEQ_X = [[[0.1, 0.2, 0.3, 0.4, 0.5], [-0.1, -0.2, -0.3, -0.4, -0.5], [0.5, 0.6, 0.7, 0.8, 0.9]],
+         [[-0.1, -0.2, -0.3, -0.4, -0.5], [-0.1, -0.2, -0.3, -0.4, -0.5], [0.5, 0.6, 0.7, 0.8, 0.9]],
+         [[0.1, 0.2, 0.3, 0.4, 0.5], [-0.1, -0.2, -0.3, -0.4, -0.5], [-0.1, -0.2, -0.3, -0.4, -0.5]],
+         [[-0.1, -0.2, -0.3, -0.4, -0.5], [-0.1, -0.2, -0.3, -0.4, -0.5], [-0.1, -0.2, -0.3, -0.4, -0.5]]]
+SEQ_HIDDEN = [[[-1.0, -1.0]] * 3, [[2.0, 3.0]] * 3]
+W3S0 = [[0.9, 0.8, 0.7, 0.6, 0.5], [0.8, 0.7, 0.6, 0.5, 0.4], [0.7, 0.6, 0.5, 0.4, 0.3], [0.6, 0.5, 0.4, 0.3, 0.2],
+        [0.5, 0.4, 0.3, 0.2, 0.1], [0.4, 0.3, 0.2, 0.1, 0.0]]
+W3SN = [[[0.5, 0.6], [0.4, 0.5], [0.3, 0.4], [0.2, 0.3], [0.1, 0.2], [0.0, 0.1]]]
+U3S = [[[-0.3, -0.1], [-0.2, 0.0], [-0.3, -0.1], [-0.2, 0.0], [-0.3, -0.1], [-0.2, 0.0]],
+       [[-0.4, -0.5], [-0.4, 0.5], [-0.4, -0.5], [-0.4, 0.5], [-0.4, -0.5], [-0.4, 0.5]]]
+BW3S = [[[0.1, 0.2, 0.3, 0.4, 0.5, 0.6]], [[0.2, 0.3, 0.4, 0.2, 0.3, 0.4]]]
+BU3S = [[[-0.1, -0.2, -0.3, -0.4, -0.5, -0.6]], [[0.1, 0.2, 0.3, 0.4, 0.5, 0.6]]]
+PY_OUTPUT = [[[0.2564464804, 2.4324064858], [0.3212793315, 2.4821776260], [0.1983539289, 2.3849941275]],
+             [[0.1323593874, 2.1939630024], [0.1591080583, 2.2447442148], [0.0683269257, 2.1121420346]],
+             [[0.1233993158, 1.9977140846], [0.1320258443, 2.0434525564], [0.0904040251, 1.9111566097]],
+             [[0.1355803839, 1.8195602154], [0.1369919053, 1.8612790359], [0.1230976350, 1.7381913793]]]
+PY_HIDDEN_N = [[[0.0155439572, 0.1680427130], [-0.0038861287, 0.1854366532], [-0.0549487103, 0.1189245136]],
+               [[0.1355803839, 1.8195602154], [0.1369919053, 1.8612790359], [0.1230976350, 1.7381913793]]]
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float64, 1e-8), (np.float32, 2e-6)])
+def test_stacked_sequence_reference_vectors(hip, dt, tol):
+    dev = [hip.toHip(np.array(v, dtype=dt)) for v in (SEQ_X, W3S0, W3SN, U3S, BW3S, BU3S)]
+    h = hip.toHip(np.array(SEQ_HIDDEN, dtype=dt))
+    out = hip.gru_inference(*dev, h)
+    assert out.shape == (4, 3, 2)
+    assert mean_relative_error(out.toCpu(), PY_OUTPUT) < tol
+    assert mean_relative_error(h.toCpu(), PY_HIDDEN_N) < tol
+    # one layer alone: W3sN empty or None
+    h1 = hip.toHip(np.array(SEQ_HIDDEN[:1], dtype=dt))
+    one = hip.gru_inference(dev[0], dev[1], None, dev[3][0:1], dev[4][0:1], dev[5][0:1], h1)
+    assert np.array_equal(one.toCpu()[-1], h1.toCpu()[0])
+    assert mean_relative_error(h1.toCpu()[0], PY_HIDDEN_N[0]) < tol
+    with pytest.raises(ValueError):
+        hip.gru_inference(dev[0], dev[1], None, dev[3], dev[4], dev[5], h)
+
+
+def oracle_cell(oracle, x, W3_, U3_, bW3, bU3, h):
+    """gru_cell_inference through the oracle's GEMM and map bodies; returns (h', r, z, n, Uh)."""
+    H = h.shape[1]
+    W3x = oracle.map2("add", oracle.matmul(x, W3_.T), oracle.broadcast(bW3, (x.shape[0], 3 * H)))
+    U3h = oracle.map2("add", oracle.matmul(h, U3_.T), oracle.broadcast(bU3, (x.shape[0], 3 * H)))
+    Uh = U3h[:, 2 * H:].copy()
+    rz = oracle.map2("add_sigmoid", np.ascontiguousarray(W3x[:, :2 * H]), np.ascontiguousarray(U3h[:, :2 * H]))
+    r, z = np.ascontiguousarray(rz[:, :H]), np.ascontiguousarray(rz[:, H:])
+    n = oracle.map3("gru_candidate", np.ascontiguousarray(W3x[:, 2 * H:]), r, Uh)
+    return oracle.map3("gru_blend", h, z, n), r, z, n, Uh
+
+
+@pytest.mark.parametrize("dt,B,F,H", [(np.float64, 3, 4, 2), (np.float64, 64, 100, 96), (np.float32, 128, 256, 512), (np.float32, 5, 7, 3)])
+def test_cell_forward_and_backward(hip, oracle, dt, B, F, H):
+    rng = np.random.default_rng(seed_of("gru-cell", np.dtype(dt).name, B, F, H))
+    scale = 1.0 if F < 50 else 0.1
+    x, h = rng.uniform(0, 1, (B, F)).astype(dt), rng.uniform(0, 1, (B, H)).astype(dt)
+    W3_, U3_ = (rng.uniform(0, 1, (3 * H, F)) * scale).astype(dt), (rng.uniform(0, 1, (3 * H, H)) * scale).astype(dt)
+    bW3, bU3 = rng.uniform(0, 1, (1, 3 * H)).astype(dt), rng.uniform(0, 1, (1, 3 * H)).astype(dt)
+    f32 = dt == np.float32
+    say("gru cell", np.dtype(dt).name, B, F, H)
+    dev = [hip.toHip(a) for a in (x, W3_, U3_, bW3, bU3)]
+    dh = hip.toHip(h)
+    r, z, n, Uh = hip.gru_cell_forward(*dev, dh)
+    want_h, wr, wz, wn, wUh = oracle_cell(oracle, x, W3_, U3_, bW3, bU3, h)
+    tol = 2e-5 if f32 else 1e-12
+    for got, want, name in ((dh, want_h, "h'"), (r, wr, "r"), (z, wz, "z"), (n, wn, "n"), (Uh, wUh, "Uh")):
+        assert np.max(np.abs(got.toCpu() - want)) <= tol * max(1.0, np.max(np.abs(want))), name
+    h2 = hip.toHip(h)
+    hip.gru_cell_inference(*dev, h2)
+    assert np.max(np.abs(h2.toCpu() - dh.toCpu())) <= tol
+    dnext = rng.uniform(0.5, 1.5, (B, H)).astype(dt) if B > 3 else np.ones((B, H), dtype=dt)
+    grads = hip.gru_cell_backward(hip.toHip(dnext), dev[0], hip.toHip(h), dev[1], dev[2], r, z, n, Uh)
+    names = ("dx", "dh", "dW3", "dU3", "dbW3", "dbU3")
+    shapes = (x.shape, h.shape, W3_.shape, U3_.shape, bW3.shape, bU3.shape)
+    for g, name, shape in zip(grads, names, shapes):
+        assert g.shape == shape, name
+    if B * F <= 100 and not f32:
+        # the reference's check: numerical gradient of sum(dnext * h') with respect to every input, float64
+        params = [x, h, W3_, U3_, bW3, bU3]
+
+        def objective():
+            return float(np.sum(dnext * oracle_cell(oracle, params[0], params[2], params[3], params[4], params[5], params[1])[0]))
+
+        for g, arr, name in zip(grads, params, names):
+            num = np.zeros_like(arr)
+            flat, nf = arr.reshape(-1), num.reshape(-1)
+            for i in range(flat.size):
+                keep = flat[i]
+                flat[i] = keep + 1e-5; up = objective()
+                flat[i] = keep - 1e-5; dn = objective()
+                flat[i] = keep
+                nf[i] = (up - dn) / 2e-5
+            err = np.mean(np.abs(g.toCpu() - num))
+            say(f"  {name}: mean absolute error against the numerical gradient {err:.2e}")
+            assert err < 1e-8, name
+    # the same formulas in extended precision from the saved tensors
+    L = np.longdouble
+    rr, zz, nn, uu, hh, dn_ = (a.astype(L) for a in (r.toCpu(), z.toCpu(), n.toCpu(), Uh.toCpu(), h, dnext))
+    dz, dnn = (hh - nn) * dn_, (1 - zz) * dn_
+    dWx = dnn * (1 - nn * nn)
+    dr, dUh = uu * dWx, rr * dWx
+    dWzx, dWrx = zz * (1 - zz) * dz, rr * (1 - rr) * dr
+    dW3x, dU3h = np.concatenate([dWrx, dWzx, dWx], 1), np.concatenate([dWrx, dWzx, dUh], 1)
+    want = (dW3x @ W3_.astype(L), dU3h @ U3_.astype(L) + dn_ * zz, dW3x.T @ x.astype(L), dU3h.T @ hh, dW3x.sum(0, keepdims=True), dU3h.sum(0, keepdims=True))
+    for g, w, name in zip(grads, want, names):
+        rel = np.linalg.norm((g.toCpu().astype(L) - w).astype(np.float64)) / max(np.linalg.norm(w.astype(np.float64)), 1e-30)
+        assert rel <= (1e-4 if f32 else 1e-12), (name, rel)

@@ -104,3 +104,27 @@ def test_extent_in_storage():
     assert md.extent_in_storage(Layout((2, 2), (-8, -2), 19)) == (9, 19)
     assert md.extent_in_storage(Layout((3, 4), (4, 1), 0)) == (0, 11)
     assert md.extent_in_storage(Layout((0, 4), (4, 1), 5)) == (5, 4)
+
+
+def test_permute_squeeze_unsqueeze_match_numpy():
+    """permute / squeeze / unsqueeze (shapeshifting.nim:207-226, 396-424) are metadata only: the same elements as the
+    NumPy view of the same name, and unsqueeze's new stride is the reference's shape[axis] * strides[axis]."""
+    from arraymancer_amd import metadata as md
+    base = np.arange(2 * 1 * 3 * 1 * 4).reshape(2, 1, 3, 1, 4)
+
+    def view(l):
+        return np.lib.stride_tricks.as_strided(base.reshape(-1)[l.offset:], shape=l.shape, strides=tuple(s * base.itemsize for s in l.strides))
+
+    l = md.contiguous(base.shape)
+    assert np.array_equal(view(md.permute(l, (4, 2, 0, 1, 3))), base.transpose(4, 2, 0, 1, 3))
+    with pytest.raises(ValueError):
+        md.permute(l, (0, 1, 2, 3, 3))
+    assert np.array_equal(view(md.squeeze(l)), base.squeeze())
+    assert np.array_equal(view(md.squeeze(l, 1)), base.squeeze(1))
+    assert md.squeeze(l, 0) == l                                      # extent 2: nothing to drop
+    ones = md.contiguous((1, 1))
+    assert md.squeeze(ones).shape == (1,)                             # the rank never drops to 0
+    u = md.unsqueeze(md.contiguous((3, 4)), 1)
+    assert u.shape == (3, 1, 4) and u.strides == (4, 4, 1)
+    assert md.unsqueeze(md.contiguous((3, 4)), 2).strides == (4, 1, 1)
+    assert np.array_equal(view(md.unsqueeze(md.squeeze(l), 0))[0], base.squeeze())
