@@ -649,32 +649,39 @@ def linear_backward(input: HipTensor, weight: HipTensor, gradOutput: HipTensor, 
 
 
 # ---------------------------------------------------------------------- gated recurrent unit
+def _gru_gates_inplace(W3x: HipTensor, U3h: HipTensor, hidden: HipTensor, keep=None):
+    """Steps 2-4 of gru_cell_inference / gru_cell_forward (nnp_gru.nim:72-88, 125-146) as one launch over the two
+    [batch, 3H] products; `hidden` is updated in place. keep = (r, z, n, Uh) receives what the backward pass needs."""
+    B, H = hidden.shape
+    if W3x.shape != (B, 3 * H) or U3h.shape != (B, 3 * H):
+        raise ValueError(f"gru: products of shape {W3x.shape} and {U3h.shape} for a hidden state {hidden.shape}")
+    if W3x.strides[1] != 1 or U3h.strides[1] != 1 or hidden.strides[1] != 1:
+        raise ValueError("gru: the rows of the products and of the hidden state need unit stride")
+    saved = [ctypes.c_void_p(t.data_ptr()) for t in keep] if keep else [None] * 4
+    lds = keep[0].strides[0] if keep else 0
+    if keep and any(t.shape != (B, H) or t.strides != keep[0].strides or t.strides[1] != 1 for t in keep):
+        raise ValueError("gru: r, z, n and Uh must be [batch, H] tensors of one layout")
+    check(getattr(_lib.load(), f"am_hip_gru_gates_{hidden.sfx}")(
+        B, H, ctypes.c_void_p(W3x.data_ptr()), W3x.strides[0], ctypes.c_void_p(U3h.data_ptr()), U3h.strides[0],
+        ctypes.c_void_p(hidden.data_ptr()), hidden.strides[0], *saved, lds))
+
+
 def gru_cell_inference(input: HipTensor, W3: HipTensor, U3: HipTensor, bW3: HipTensor, bU3: HipTensor, hidden: HipTensor) -> HipTensor:
     """gru_cell_inference (src/arraymancer/nn_primitives/nnp_gru.nim:40-88): h(t) -> h'(t) in place. Two dense layers
-    with the bias in the GEMM epilogue ([batch, 3H] each), then the three gate passes in place on column slices of those
-    buffers: sigmoid(x + y) over the reset and update columns together, tanh(x + y * z) for the candidate,
-    (1 - y) * z + y * x into `hidden`. input [batch, features], W3 [3H, features], U3 [3H, H], biases [1, 3H]."""
-    H = hidden.shape[1]
-    W3x, U3h = linear(input, W3, bW3), linear(hidden, U3, bU3)
-    srz, sr, sz, s_ = slice(0, 2 * H), slice(0, H), slice(H, 2 * H), slice(2 * H, 3 * H)
-    apply2("add_sigmoid", W3x[:, srz], U3h[:, srz])
-    apply3("gru_candidate", W3x[:, s_], W3x[:, sr], U3h[:, s_])
-    apply3("gru_blend", hidden, W3x[:, sz], W3x[:, s_])
+    with the bias in the GEMM epilogue ([batch, 3H] each), then the gate arithmetic (sigmoid(x + y) for the reset and update
+    gates, tanh(x + r * u) for the candidate, (1 - z) * n + z * h into `hidden`) as one launch.
+    input [batch, features], W3 [3H, features], U3 [3H, H], biases [1, 3H]."""
+    _gru_gates_inplace(linear(input, W3, bW3), linear(hidden, U3, bU3), hidden)
     return hidden
 
 
 def gru_cell_forward(input: HipTensor, W3: HipTensor, U3: HipTensor, bW3: HipTensor, bU3: HipTensor, hidden: HipTensor):
     """gru_cell_forward (nnp_gru.nim:90-146): like gru_cell_inference, keeping what the backward pass needs. Updates
-    `hidden` in place and returns (r, z, n, Uh), each [batch, H] (r and z are the two halves of one buffer)."""
-    H = hidden.shape[1]
-    W3x, U3h = linear(input, W3, bW3), linear(hidden, U3, bU3)
-    sr, sz, s_ = slice(0, H), slice(H, 2 * H), slice(2 * H, 3 * H)
-    Uh = U3h[:, s_].clone()
-    rz = map2("add_sigmoid", W3x[:, 0:2 * H], U3h[:, 0:2 * H])
-    r, z = rz[:, sr], rz[:, sz]
-    n = map3("gru_candidate", W3x[:, s_], r, U3h[:, s_])
-    apply3("gru_blend", hidden, z, n)
-    return r, z, n, Uh
+    `hidden` in place and returns (r, z, n, Uh), each [batch, H]."""
+    B, H = hidden.shape
+    keep = tuple(empty((B, H), hidden.dtype) for _ in range(4))
+    _gru_gates_inplace(linear(input, W3, bW3), linear(hidden, U3, bU3), hidden, keep)
+    return keep
 
 
 def gru_cell_backward(dnext: HipTensor, x: HipTensor, h: HipTensor, W3: HipTensor, U3: HipTensor,
@@ -716,8 +723,12 @@ def gru_inference(input: HipTensor, W3s0: HipTensor, W3sN: HipTensor | None, U3s
     for layer in range(layers):
         W3l = W3s0 if layer == 0 else W3sN[layer - 1].squeeze(0)
         U3l, bW3l, bU3l, h_l = U3s[layer].squeeze(0), bW3s[layer].squeeze(0), bU3s[layer].squeeze(0), hidden[layer].squeeze(0)
+        # The input side of the layer does not depend on the recurrence: W3 * x + bW3 for ALL timesteps is one product
+        # [T * batch, features] * W3^T (the reference multiplies per timestep; row by row the same dot products).
+        src = input if layer == 0 else output
+        W3x_all = linear(src.reshape(T * B, src.shape[2]), W3l, bW3l).reshape(T, B, 3 * H)
         for t in range(T):
-            gru_cell_inference((input[t] if layer == 0 else output[t]).squeeze(0), W3l, U3l, bW3l, bU3l, h_l)
+            _gru_gates_inplace(W3x_all[t].squeeze(0), linear(h_l, U3l, bU3l), h_l)
             _unary_into("copy", output[t].squeeze(0), h_l)
     return output
 

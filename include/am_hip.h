@@ -572,6 +572,18 @@ int am_hip_softmax_rows_f32(int64_t rows, int64_t cols, float* dst, int64_t dst_
 int am_hip_softmax_rows_f64(int64_t rows, int64_t cols, double* dst, int64_t dst_rs, int64_t dst_cs,
                             const double* src, int64_t src_rs, int64_t src_cs);
 
+/* The gate arithmetic of a GRU cell in one pass over the two [batch, 3H] products w3x = W3 x + bW3 and u3h = U3 h + bU3
+ * (rows ldw resp. ldu apart, unit stride within a row; columns [0, H) reset, [H, 2H) update, [2H, 3H) candidate):
+ *   r = sigmoid(w3x_r + u3h_r), z = sigmoid(w3x_z + u3h_z), n = tanh(w3x_n + r * u3h_n), hidden <- (1 - z) * n + z * hidden
+ * with `hidden` [batch, H] (rows ldh apart) updated in place. When r, z, n and uh are not NULL (all four or none; [batch, H]
+ * each, rows lds apart) they receive r, z, n and u3h_n for the backward pass. Replaces steps 2-4 of gru_cell_inference and
+ * gru_cell_forward (src/arraymancer/nn_primitives/nnp_gru.nim:72-88, 125-146: three apply2 / apply3 passes over column
+ * slices); same expressions, each step rounded on its own. */
+int am_hip_gru_gates_f32(int64_t batch, int64_t H, const float* w3x, int64_t ldw, const float* u3h, int64_t ldu,
+                         float* hidden, int64_t ldh, float* r, float* z, float* n, float* uh, int64_t lds);
+int am_hip_gru_gates_f64(int64_t batch, int64_t H, const double* w3x, int64_t ldw, const double* u3h, int64_t ldu,
+                         double* hidden, int64_t ldh, double* r, double* z, double* n, double* uh, int64_t lds);
+
 /* *loss (host) <- (1 / rows) * sum over the rows i of  ln(sum_j exp(input[i, j])) - sum_j input[i, j] * target[i, j]:
  * softmax and cross-entropy in one pass over `input` [rows, cols] and `target` [rows, cols] (probabilities), element
  * strides (rs, cs). Blocking; 0 for an empty batch. Replaces softmax_cross_entropy

@@ -571,6 +571,35 @@ HipTensor<T> linear(const HipTensor<T>& x, const HipTensor<T>& weight, const Hip
   return r;
 }
 
+// gru_cell_inference (nn_primitives/nnp_gru.nim:40-88): h(t) -> h'(t) in place. Two dense layers with their bias in the
+// GEMM epilogue, then steps 2-4 (three apply2 / apply3 passes over column slices in the reference) as one launch.
+// `saved`, when given, receives {r, z, n, Uh} for the backward pass (gru_cell_forward, nnp_gru.nim:90-146).
+namespace detail {
+inline int gru_gates_(int64_t b, int64_t h, const float* w, int64_t lw, const float* u, int64_t lu, float* hid, int64_t lh, float* r,
+                      float* z, float* n, float* uh, int64_t ls) {
+  return am_hip_gru_gates_f32(b, h, w, lw, u, lu, hid, lh, r, z, n, uh, ls);
+}
+inline int gru_gates_(int64_t b, int64_t h, const double* w, int64_t lw, const double* u, int64_t lu, double* hid, int64_t lh, double* r,
+                      double* z, double* n, double* uh, int64_t ls) {
+  return am_hip_gru_gates_f64(b, h, w, lw, u, lu, hid, lh, r, z, n, uh, ls);
+}
+}  // namespace detail
+template <typename T>
+void gru_cell_inference(const HipTensor<T>& input, const HipTensor<T>& W3, const HipTensor<T>& U3, const HipTensor<T>& bW3,
+                        const HipTensor<T>& bU3, HipTensor<T>& hidden, std::vector<HipTensor<T>>* saved = nullptr) {
+  if (hidden.rank() != 2 || hidden.strides[1] != 1) throw std::invalid_argument("gru_cell_inference: hidden must be [batch, H] with unit-stride rows");
+  const int64_t B = hidden.shape[0], H = hidden.shape[1];
+  if (W3.shape[0] != 3 * H || U3.shape[0] != 3 * H || U3.shape[1] != H) throw std::invalid_argument("gru_cell_inference: weights must be [3H, features] and [3H, H]");
+  const HipTensor<T> W3x = linear(input, W3, bW3), U3h = linear(hidden, U3, bU3);
+  T *r = nullptr, *z = nullptr, *n = nullptr, *uh = nullptr;
+  if (saved) {
+    saved->assign(4, HipTensor<T>());
+    for (auto& t : *saved) t = HipTensor<T>(Shape{B, H});
+    r = (*saved)[0].ptr(); z = (*saved)[1].ptr(); n = (*saved)[2].ptr(); uh = (*saved)[3].ptr();
+  }
+  check(detail::gru_gates_(B, H, W3x.ptr(), W3x.strides[0], U3h.ptr(), U3h.strides[0], hidden.ptr(), hidden.strides[0], r, z, n, uh, H));
+}
+
 // Fold along `axis`; the result keeps the axis with extent 1 (reduce_axis_inline,
 // higher_order_foldreduce.nim:46-61). op: AM_RED_SUM / PROD / MIN / MAX.
 template <typename T>

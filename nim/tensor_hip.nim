@@ -512,6 +512,33 @@ proc linear*[T: float32 | float64](x, weight, bias: HipTensor[T], relu = false):
       result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1],
       epi, bb.get_offset_ptr, int64 bb.strides[0], int64 bb.strides[1])
 
+proc gru_cell_inference*[T: float32 | float64](input, W3, U3, bW3, bU3: HipTensor[T], hidden: var HipTensor[T]) =
+  ## nn_primitives/nnp_gru.nim:40-88: h(t) -> h'(t) in place. The two dense layers carry their bias in the GEMM
+  ## epilogue; steps 2-4 (the three apply2 / apply3 passes over column slices) are one launch.
+  let H = hidden.shape[1]
+  let W3x = linear(input, W3, bW3)
+  let U3h = linear(hidden, U3, bU3)
+  assert hidden.strides[1] == 1
+  template call(f: untyped) =
+    check f(int64 hidden.shape[0], int64 H, W3x.get_offset_ptr, int64 W3x.strides[0], U3h.get_offset_ptr, int64 U3h.strides[0],
+            hidden.get_offset_ptr, int64 hidden.strides[0], nil, nil, nil, nil, 0'i64)
+  when T is float32: call am_hip_gru_gates_f32
+  else: call am_hip_gru_gates_f64
+
+proc gru_cell_forward*[T: float32 | float64](input, W3, U3, bW3, bU3: HipTensor[T], r, z, n, Uh, hidden: var HipTensor[T]) =
+  ## nn_primitives/nnp_gru.nim:90-146: the same cell, keeping r, z, n and the candidate's U3h slice for the backward pass.
+  let H = hidden.shape[1]
+  let W3x = linear(input, W3, bW3)
+  let U3h = linear(hidden, U3, bU3)
+  r = newHipTensor[T]([hidden.shape[0], H]); z = newHipTensor[T]([hidden.shape[0], H])
+  n = newHipTensor[T]([hidden.shape[0], H]); Uh = newHipTensor[T]([hidden.shape[0], H])
+  assert hidden.strides[1] == 1
+  template call(f: untyped) =
+    check f(int64 hidden.shape[0], int64 H, W3x.get_offset_ptr, int64 W3x.strides[0], U3h.get_offset_ptr, int64 U3h.strides[0],
+            hidden.get_offset_ptr, int64 hidden.strides[0], r.get_offset_ptr, z.get_offset_ptr, n.get_offset_ptr, Uh.get_offset_ptr, int64 H)
+  when T is float32: call am_hip_gru_gates_f32
+  else: call am_hip_gru_gates_f64
+
 # ---------------------------------------------------------------- reductions, softmax, pooling
 proc reduce_axis[T: HipScalar](op: cint, t: HipTensor[T], axis: int): HipTensor[T] =
   ## reduce_axis_inline (higher_order_foldreduce.nim:46-61): the result keeps `axis` with extent 1.

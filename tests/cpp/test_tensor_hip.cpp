@@ -243,6 +243,31 @@ template <typename T> static void conv_backward_known_answer() {
   CHECK(threw);
 }
 
+static void gru_cell_literals() {
+  // tests/nn_primitives/test_nnp_gru.nim:10-57: one GRU cell against the values the reference took from PyTorch / cuDNN
+  auto x = toHip<double>({0.1, 0.2, 0.3, 0.4, -0.1, -0.2, -0.3, -0.4, 0.5, 0.6, 0.7, 0.8}, {3, 4});
+  auto W3 = toHip<double>({0.9, 0.8, 0.7, 0.6, 0.8, 0.7, 0.6, 0.5, 0.7, 0.6, 0.5, 0.4, 0.6, 0.5, 0.4, 0.3, 0.5, 0.4, 0.3, 0.2, 0.4, 0.3, 0.2, 0.1}, {6, 4});
+  auto U3 = toHip<double>({-0.3, -0.1, -0.2, 0.0, -0.3, -0.1, -0.2, 0.0, -0.3, -0.1, -0.2, 0.0}, {6, 2});
+  auto bW3 = toHip<double>({0.1, 0.2, 0.3, 0.4, 0.5, 0.6}, {1, 6});
+  auto bU3 = toHip<double>({-0.1, -0.2, -0.3, -0.4, -0.5, -0.6}, {1, 6});
+  const std::vector<double> want = {-0.5317437280, -0.4752916969, -0.3930421219, -0.3209550879, -0.7325259335, -0.6429624731};
+  auto close = [&](const am::HipTensor<double>& h) {
+    const auto got = h.toCpu();
+    double err = 0;
+    for (size_t i = 0; i < want.size(); ++i) err += std::fabs(got[i] - want[i]) / std::fabs(want[i]);
+    return err / want.size() < 1e-8;
+  };
+  auto h = toHip<double>({-1, -1, -1, -1, -1, -1}, {3, 2});
+  am::gru_cell_inference(x, W3, U3, bW3, bU3, h);
+  CHECK(close(h));
+  auto h2 = toHip<double>({-1, -1, -1, -1, -1, -1}, {3, 2});
+  std::vector<am::HipTensor<double>> saved;
+  am::gru_cell_inference(x, W3, U3, bW3, bU3, h2, &saved);
+  CHECK(close(h2) && saved.size() == 4 && saved[0].shape == (Shape{3, 2}));
+  const auto z = saved[1].toCpu(), n = saved[2].toCpu(), hn = h2.toCpu();
+  for (size_t i = 0; i < 6; ++i) CHECK(std::fabs((1 - z[i]) * n[i] + z[i] * -1.0 - hn[i]) < 1e-15);
+}
+
 static void loss_literals() {
   // tests/nn_primitives/test_nnp_loss.nim:31-44: one row, truth = class 3, loss 0.0709 within 2e-5, dense and sparse
   auto predicted = toHip<double>({-3.44, 1.16, -0.81, 3.91}, {1, 4});
@@ -446,6 +471,7 @@ int main(int argc, char** argv) {
   conv_literals<int32_t>();
   conv_literals<int64_t>();
   loss_literals();
+  gru_cell_literals();
   conv_backward_known_answer<float>();
   conv_backward_known_answer<double>();
   conv_backward_known_answer<int32_t>();

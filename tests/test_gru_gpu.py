@@ -151,3 +151,39 @@ def test_cell_forward_and_backward(hip, oracle, dt, B, F, H):
     for g, w, name in zip(grads, want, names):
         rel = np.linalg.norm((g.toCpu().astype(L) - w).astype(np.float64)) / max(np.linalg.norm(w.astype(np.float64)), 1e-30)
         assert rel <= (1e-4 if f32 else 1e-12), (name, rel)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_fused_gates_equal_the_three_passes(hip, dt):
+    """am_hip_gru_gates_* against the three separate bodies of the reference's cell (apply2 sigmoid(x + y) on the reset
+    and update columns, apply3 tanh(x + y * z), apply3 (1 - y) * z + y * x) bit for bit: aligned buffers (16-byte
+    lanes) and products / hidden states that are windows of wider buffers at odd offsets (element lanes)."""
+    from arraymancer_amd import tensor_hip as th
+    rng = np.random.default_rng(seed_of("gru-gates", np.dtype(dt).name))
+    for B, H, pad in ((3, 2, 0), (64, 96, 0), (17, 33, 0), (40, 64, 3), (5, 8, 1)):
+        wide_w = rng.standard_normal((B, 3 * H + 2 * pad)).astype(dt)
+        wide_u = rng.standard_normal((B, 3 * H + 2 * pad)).astype(dt)
+        wide_h = rng.standard_normal((B, H + 2 * pad)).astype(dt)
+        win3, win1 = slice(pad, pad + 3 * H), slice(pad, pad + H)
+        # three passes, in place on copies
+        W, U, h = hip.toHip(wide_w)[:, win3], hip.toHip(wide_u)[:, win3], hip.toHip(wide_h)[:, win1]
+        hip.apply2("add_sigmoid", W[:, 0:2 * H], U[:, 0:2 * H])
+        hip.apply3("gru_candidate", W[:, 2 * H:], W[:, 0:H], U[:, 2 * H:])
+        hip.apply3("gru_blend", h, W[:, H:2 * H], W[:, 2 * H:])
+        # one pass
+        W2, U2 = hip.toHip(wide_w)[:, win3], hip.toHip(wide_u)[:, win3]
+        parent_h = hip.toHip(wide_h)
+        h2 = parent_h[:, win1]
+        keep = tuple(hip.empty((B, H), dt) for _ in range(4))
+        th._gru_gates_inplace(W2, U2, h2, keep)
+        assert np.array_equal(h2.toCpu(), h.toCpu()), (B, H, pad)
+        assert np.array_equal(keep[0].toCpu(), W.toCpu()[:, 0:H]) and np.array_equal(keep[1].toCpu(), W.toCpu()[:, H:2 * H])
+        assert np.array_equal(keep[2].toCpu(), W.toCpu()[:, 2 * H:]) and np.array_equal(keep[3].toCpu(), wide_u[:, pad + 2 * H:pad + 3 * H])
+        assert np.array_equal(W2.toCpu(), wide_w[:, win3])                       # the products are only read
+        full = parent_h.toCpu()
+        assert np.array_equal(full[:, :pad], wide_h[:, :pad]) and np.array_equal(full[:, pad + H:], wide_h[:, pad + H:])
+        h3 = hip.toHip(wide_h)[:, win1]
+        th._gru_gates_inplace(W2, U2, h3)                                        # nothing kept: same hidden state
+        assert np.array_equal(h3.toCpu(), h.toCpu())
+    with pytest.raises(ValueError):
+        th._gru_gates_inplace(hip.zeros((2, 5), dt), hip.zeros((2, 6), dt), hip.zeros((2, 2), dt))
