@@ -1108,7 +1108,15 @@ def reduce_axis(op, t: HipTensor, axis: int) -> HipTensor:
         return empty(t.shape, t.dtype)
     shape = list(t.shape)
     shape[axis] = 1
-    out = empty(shape, t.dtype)
+    return reduce_axis_into(op, empty(shape, t.dtype), t, axis)
+
+
+def reduce_axis_into(op, out: HipTensor, t: HipTensor, axis: int) -> HipTensor:
+    """reduce_axis written into an existing tensor of t's shape with extent 1 along `axis` (any strides): nothing is
+    allocated, which a captured graph or a tight loop needs."""
+    _same_dtype(out, t)
+    if out.rank != t.rank or any(o != (1 if d == axis else n) for d, (o, n) in enumerate(zip(out.shape, t.shape))):
+        raise ValueError(f"reduce_axis_into: result {out.shape} does not fit {t.shape} folded along axis {axis}")
     check(getattr(_lib.load(), f"am_hip_reduce_axis_{t.sfx}")(
         RED[op], t.rank, i64_array(t.shape), axis, ctypes.c_void_p(out.data_ptr()), i64_array(out.strides),
         ctypes.c_void_p(t.data_ptr()), i64_array(t.strides)))

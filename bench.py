@@ -354,8 +354,9 @@ def other_workloads(am, timer, steps, warmup, ceilings):
     bias = am.toHip(np.random.default_rng(4005).uniform(-1, 1, (1, 512)).astype(np.float32)).broadcast((65536, 512))
     hbm_entry("f32 65536x512 X +. b[1,512] (bias of a dense layer)", [(lambda i=i: th._binary_into("add", dOs[i], dTs[i], bias)) for i in range(3)],
               2 * T.nbytes + 2048)
-    hbm_entry("f32 sum(X[65536,512], axis=0) (bias gradient)", [(lambda i=i: am.sum(dTs[i], 0)) for i in range(3)], T.nbytes)
-    hbm_entry("f32 sum(X[65536,512], axis=1)", [(lambda i=i: am.sum(dTs[i], 1)) for i in range(3)], T.nbytes)
+    col_sums, row_sums = am.empty((1, 512), np.float32), am.empty((65536, 1), np.float32)
+    hbm_entry("f32 sum(X[65536,512], axis=0) (bias gradient)", [(lambda i=i: th.reduce_axis_into("sum", col_sums, dTs[i], 0)) for i in range(3)], T.nbytes)
+    hbm_entry("f32 sum(X[65536,512], axis=1)", [(lambda i=i: th.reduce_axis_into("sum", row_sums, dTs[i], 1)) for i in range(3)], T.nbytes)
     del dTs, dOs
     dA = am.toHip(np.random.default_rng(1003).standard_normal((500, 65536)).astype(np.float32))
     dB = am.toHip(np.random.default_rng(1004).standard_normal((65536, 800)).astype(np.float32))
@@ -738,6 +739,11 @@ def run_only(am, timer, which, steps, warmup):
             fn = lambda: th._binary_into("add", dY, dX, bb)
         else:
             fn = {"sum_cols_narrow": lambda: am.sum(dX, 0), "sum_rows_short": lambda: am.sum(dX, 1), "softmax_short_rows": lambda: am.softmax(dX)}[which]
+    elif which in ("sce_forward", "sce_backward"):   # sparse softmax cross-entropy of [65536 x 1000] scores (262 MB)
+        rows, cols = 65536, 1000
+        dX = am.toHip(np.random.default_rng(4006).standard_normal((rows, cols)).astype(np.float32))
+        lab = am.toHip(np.random.default_rng(4007).integers(0, cols, rows).astype(np.int64))
+        fn = (lambda: am.sparse_softmax_cross_entropy(dX, lab)) if which == "sce_forward" else (lambda: am.sparse_softmax_cross_entropy_backward(1.0, dX, lab))
     elif which == "gemm_f32_long_k":   # the weight gradient of a dense layer over a large batch: few tiles, very long k
         dA = am.toHip(np.random.default_rng(1001).standard_normal((500, 65536)).astype(np.float32))
         dB = am.toHip(np.random.default_rng(1002).standard_normal((65536, 800)).astype(np.float32))
@@ -765,7 +771,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true",
                     help="print one JSON line per configuration (GPU vs CPU port, parity at full size) instead of the single benchmark line")
-    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool", "transposed_add", "bias_short_rows", "sum_cols_narrow", "sum_rows_short", "softmax_short_rows", "gemm_f32_long_k", "conv_backward",
+    ap.add_argument("--only", choices=["gemm_f32", "gemm_i32", "gemm_i32_valu", "gemm_f64", "bcast_add", "copy", "chain", "ex02", "sum_rows", "sum_cols", "softmax", "maxpool", "transposed_add", "bias_short_rows", "sum_cols_narrow", "sum_rows_short", "softmax_short_rows", "gemm_f32_long_k", "conv_backward", "sce_forward", "sce_backward",
                                       "gemm_f32_1024", "gemm_f32_2048", "gemm_i32_1500", "bcast_add_rotating"],
                     help="profiling aid: run just this workload's launches and print a short JSON line")
     args = ap.parse_args()
