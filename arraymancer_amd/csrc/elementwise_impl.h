@@ -160,6 +160,15 @@ template <typename T, int UOP> struct UnOp {
     } else if constexpr (UOP == AM_UOP_RADTODEG) {   // Nim: d / RadPerDeg
       if constexpr (Traits<T>::kFloat) return x / (T)(3.14159265358979323846 / 180.0); else return x;
     }
+    else if constexpr (UOP == AM_UOP_FAC) {   // n! from 0! to 20! (what fits 64 bits, the extent of Nim's table)
+      if constexpr (Traits<T>::kFloat) return x;   // never dispatched for floats
+      else {
+        uint64_t f = 1;
+        const bool in_range = x >= 0 && x <= 20;
+        for (int i = 2; i <= 20; ++i) f *= (i <= (int)(in_range ? x : 0)) ? (uint64_t)i : 1u;
+        return in_range ? (T)f : (T)0;
+      }
+    }
     else if constexpr (UOP >= AM_UOP_LN) {
       if constexpr (Traits<T>::kFloat) return dev_math<UOP>(x); else return x;   // never dispatched for integers
     }
@@ -1226,6 +1235,9 @@ static int unary(const char* fn, int op, int rank, const int64_t* shape, T* dst,
     AM_CASE(AM_UOP_FLOOR); AM_CASE(AM_UOP_CEIL); AM_CASE(AM_UOP_TRUNC); AM_CASE(AM_UOP_ROUND); AM_CASE(AM_UOP_RECIPROCAL);
     AM_CASE(AM_UOP_DEGTORAD); AM_CASE(AM_UOP_RADTODEG);
 #undef AM_CASE
+    case AM_UOP_FAC:
+      if constexpr (!F) return run<T, kUnaryBase + AM_UOP_FAC, true, false>(rank, shape, dst, sd, a, sa, nullptr, nullptr, (T)0);
+      else return fail(AM_E_DTYPE, "%s: fac is defined for integer tensors only", fn);
     default:
       return fail(AM_E_ARG, "%s: unknown unary op %d", fn, op);
   }

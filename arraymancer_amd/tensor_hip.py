@@ -1064,6 +1064,17 @@ def radToDeg(t: HipTensor) -> HipTensor:
     return unary("radtodeg", t)
 
 
+def fac(t: HipTensor) -> HipTensor:
+    """The factorial of every element (src/arraymancer/tensor/ufunc.nim:84-85 maps Nim's `fac`, a table of 0! .. 20!
+    that asserts its argument lies inside it): integer tensors, every element in 0 .. 20, else ValueError
+    (the range is checked with two reductions before the pass)."""
+    if t.dtype.kind != "i":
+        raise TypeError("fac is defined for integer tensors only")
+    if t.size and (int(reduce_all("min", t)) < 0 or int(reduce_all("max", t)) > 20):
+        raise ValueError("fac: every element must be a non-negative integer of at most 20")
+    return unary("fac", t)
+
+
 def _clamp_into(dst: HipTensor, t: HipTensor, lo, hi):
     # both bounds travel by value: no device allocation, no copy, no synchronisation, recordable into a graph
     ct = CTYPE[t.sfx]

@@ -407,7 +407,9 @@ int am_hip_ew_scalar_i64(int op, int scalar_on_left, int rank, const int64_t* sh
 #define AM_UOP_RECIPROCAL 32   /* 1 / x */
 #define AM_UOP_DEGTORAD   33   /* x * (PI / 180), the constant rounded to the element type (Nim's degToRad, ufunc.nim:129) */
 #define AM_UOP_RADTODEG   34   /* x / (PI / 180)                                           (Nim's radToDeg, ufunc.nim:130) */
-#define AM_UOP_COUNT      35
+#define AM_UOP_FAC        35   /* integers only: n! for 0 <= n <= 20 (Nim's fac, mapped by tensor/ufunc.nim:84-85), wrapped into the
+                                   element type; 0 outside that range (Nim raises there: the host layers check first) */
+#define AM_UOP_COUNT      36
 int am_hip_ew_unary_f32(int op, int rank, const int64_t* shape,
                         float* dst, const int64_t* dst_strides,
                         const float* a, const int64_t* a_strides);

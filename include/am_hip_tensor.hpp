@@ -498,6 +498,12 @@ AM_HIP_UFUNC(floor, AM_UOP_FLOOR) AM_HIP_UFUNC(ceil, AM_UOP_CEIL) AM_HIP_UFUNC(t
 AM_HIP_UFUNC(round, AM_UOP_ROUND) AM_HIP_UFUNC(reciprocal, AM_UOP_RECIPROCAL)
 AM_HIP_UFUNC(degToRad, AM_UOP_DEGTORAD) AM_HIP_UFUNC(radToDeg, AM_UOP_RADTODEG)
 #undef AM_HIP_UFUNC
+// fac (ufunc.nim:84-85): n! of every element of an integer tensor; Nim's table covers 0 .. 20 and asserts outside it.
+template <typename T> HipTensor<T> fac(const HipTensor<T>& t) {
+  static_assert(std::is_integral<T>::value, "fac is defined for integer tensors");
+  if (t.size() > 0 && (min(t) < T(0) || max(t) > T(20))) throw std::out_of_range("fac: every element must lie in 0 .. 20");
+  return unary(AM_UOP_FAC, t);
+}
 // map2_inline(x, b.broadcast(x.shape), max(0, x + y)) in one pass
 template <typename T> HipTensor<T> bias_relu(const HipTensor<T>& x, const HipTensor<T>& b) { return map2(AM_OP_ADD_RELU, x, b.broadcast(x.shape)); }
 // Activation backward passes: map2_inline(cached_tensor, gradient) bodies of nnp_activation.nim:61-74.

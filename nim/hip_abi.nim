@@ -196,7 +196,7 @@ type
     uopLn = 9, uopLog10 = 10, uopLog2 = 11, uopSin = 12, uopCos = 13, uopTan = 14, uopSinh = 15, uopCosh = 16,
     uopArcsin = 17, uopArccos = 18, uopArctan = 19, uopArcsinh = 20, uopArccosh = 21, uopArctanh = 22, uopCbrt = 23,
     uopErf = 24, uopErfc = 25, uopGamma = 26, uopLgamma = 27, uopFloor = 28, uopCeil = 29, uopTrunc = 30,
-    uopRound = 31, uopReciprocal = 32, uopDegToRad = 33, uopRadToDeg = 34
+    uopRound = 31, uopReciprocal = 32, uopDegToRad = 33, uopRadToDeg = 34, uopFac = 35
 
 proc am_hip_ew_binary_f32*(op: cint, rank: cint, shape: ptr int64, dst: ptr cfloat, dst_strides: ptr int64,
                            a: ptr cfloat, a_strides: ptr int64, b: ptr cfloat, b_strides: ptr int64): cint {.importc.}

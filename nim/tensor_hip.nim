@@ -423,6 +423,12 @@ makeHipUniversal(round, uopRound)
 makeHipUniversal(reciprocal, uopReciprocal)   # math_functions.nim:52-54
 makeHipUniversal(degToRad, uopDegToRad)       # ufunc.nim:129
 makeHipUniversal(radToDeg, uopRadToDeg)       # ufunc.nim:130
+proc fac*[T: int32 | int64](t: HipTensor[T]): HipTensor[T] =
+  ## ufunc.nim:84-85: Nim's `fac` over every element; it asserts 0 <= n <= 20, checked here with two reductions first.
+  if t.size > 0: doAssert t.min >= T(0) and t.max <= T(20), "fac: every element must lie in 0 .. 20"
+  result = newHipTensor[T](t.shape)
+  if result.size > 0: ewUnary(T, uopFac, result, t)
+
 proc mreciprocal*[T: float32 | float64](t: var HipTensor[T]) =
   ## math_functions.nim:56-58
   if t.size > 0: ewUnary(T, uopReciprocal, t, t)

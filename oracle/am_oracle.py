@@ -34,7 +34,7 @@ OP3 = dict(muladd=0, gru_candidate=1, gru_blend=2, addmul=3, clamp=4)
 UOP = dict(copy=0, neg=1, relu=2, sigmoid=3, tanh=4, exp=5, abs=6, sqrt=7, square=8,
            ln=9, log10=10, log2=11, sin=12, cos=13, tan=14, sinh=15, cosh=16, arcsin=17,
            arccos=18, arctan=19, arcsinh=20, arccosh=21, arctanh=22, cbrt=23, erf=24, erfc=25, gamma=26,
-           lgamma=27, floor=28, ceil=29, trunc=30, round=31, reciprocal=32, degtorad=33, radtodeg=34)
+           lgamma=27, floor=28, ceil=29, trunc=30, round=31, reciprocal=32, degtorad=33, radtodeg=34, fac=35)
 
 
 def build(force: bool = False) -> str:

@@ -803,3 +803,29 @@ def test_more_than_2_pow_31_elements(hip):
     assert int(hip.sum(big2)) == wrap(want_sum)
     assert np.array_equal(big2[n_rows - 1:, :].clone().toCpu(), col[n_rows - 1:] + row)
     assert np.array_equal(big2[:1, :].clone().toCpu(), col[:1] + row)
+
+
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+def test_fac(hip, oracle, sfx):
+    """fac (tensor/ufunc.nim:84-85): n! of every element, 0 .. 20, bit for bit against the oracle (int32 wraps from 13!
+    on) on contiguous and strided operands; an element outside the table's range raises, like Nim's assertion."""
+    import math
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("fac", sfx))
+    n = np.arange(0, 21).astype(dt)
+    got = hip.fac(hip.toHip(n)).toCpu()
+    assert got.tolist() == oracle.unary("fac", n).tolist()
+    if sfx == "i64":
+        assert got.tolist() == [math.factorial(int(k)) for k in n]
+    a = rng.integers(0, 21, (257, 130)).astype(dt)
+    da = hip.toHip(a)
+    assert np.array_equal(hip.fac(da).toCpu(), oracle.unary("fac", a))
+    assert np.array_equal(hip.fac(da.transpose()[3:, ::2]).toCpu(), oracle.unary("fac", np.ascontiguousarray(a.T[3:, ::2])))
+    for bad in (-1, 21):
+        b = a.copy()
+        b[100, 7] = bad
+        with pytest.raises(ValueError):
+            hip.fac(hip.toHip(b))
+    with pytest.raises(TypeError):
+        hip.fac(hip.zeros((2, 2), np.float32))
+    assert hip.fac(hip.zeros((0, 3), dt)).shape == (0, 3)

@@ -525,3 +525,16 @@ def test_clamp_body(oracle):
     x = np.array([np.nan, -np.inf, np.inf, -0.0, 5.0])
     got = oracle.map3("clamp", x, np.broadcast_to(0.0, x.shape), np.broadcast_to(1.0, x.shape))
     assert np.isnan(got[0]) and got[1] == 0 and got[2] == 1 and got[3] == 0 and np.signbit(got[3]) and got[4] == 1
+
+
+def test_fac_is_the_factorial(oracle):
+    """fac (tensor/ufunc.nim:84-85 -> Nim's std/math fac): n! for 0 .. 20 against Python's exact integers, wrapped into
+    int32 from 13! on; 0 outside the table's range, where Nim raises."""
+    import math
+    n = np.arange(0, 21, dtype=np.int64)
+    assert oracle.unary("fac", n).tolist() == [math.factorial(int(k)) for k in n]
+    got32 = oracle.unary("fac", n.astype(np.int32))
+    assert got32.tolist() == [((math.factorial(int(k)) + 2**31) % 2**32) - 2**31 for k in n]
+    assert oracle.unary("fac", np.array([-1, 21, 5], dtype=np.int64)).tolist() == [0, 0, 120]
+    with pytest.raises(ValueError):
+        oracle.unary("fac", np.array([1.0, 2.0]))
