@@ -684,15 +684,12 @@ def gru_cell_forward(input: HipTensor, W3: HipTensor, U3: HipTensor, bW3: HipTen
     return keep
 
 
-def gru_cell_backward(dnext: HipTensor, x: HipTensor, h: HipTensor, W3: HipTensor, U3: HipTensor,
-                      r: HipTensor, z: HipTensor, n: HipTensor, Uh: HipTensor):
-    """gru_cell_backward (nnp_gru.nim:148-192): (dx, dh, dW3, dU3, dbW3, dbU3) from the gradient `dnext` of the next
-    hidden state, the inputs of the forward pass (h is the hidden state BEFORE it) and the tensors it saved. The
-    reference concatenates the three gate gradients; here they are written into column slices of one [batch, 3H]
-    buffer per dense layer."""
-    B, H = h.shape
+def _gru_gates_backward_passes(dnext, h, r, z, n, Uh, dW3x, dU3h):
+    """The element-wise part of gru_cell_backward (nnp_gru.nim:165-186) with the reference's separate bodies, written
+    into column slices of the two [batch, 3H] buffers where the reference concatenates. Nine launches; kept as the
+    statement the one-launch kernel is compared with."""
+    H = h.shape[1]
     sr, sz, s_ = slice(0, H), slice(H, 2 * H), slice(2 * H, 3 * H)
-    dW3x, dU3h = empty((B, 3 * H), h.dtype), empty((B, 3 * H), h.dtype)
     dz = map2("mul", map2("sub", h, n), dnext)                                   # step 4, z part
     dn = map2("mul", scalar_op("sub", z, 1, scalar_on_left=True), dnext)
     _binary_into("tanh_bwd", dW3x[:, s_], n, dn)                                 # step 3: dWx = dn * (1 - n * n)
@@ -701,6 +698,24 @@ def gru_cell_backward(dnext: HipTensor, x: HipTensor, h: HipTensor, W3: HipTenso
     _binary_into("sigmoid_bwd", dW3x[:, sz], z, dz)                              # step 2: update gate
     _binary_into("sigmoid_bwd", dW3x[:, sr], r, dr)                              # step 2: reset gate
     _unary_into("copy", dU3h[:, 0:2 * H], dW3x[:, 0:2 * H])                      # dUrh = dWrx, dUzh = dWzx
+
+
+def gru_cell_backward(dnext: HipTensor, x: HipTensor, h: HipTensor, W3: HipTensor, U3: HipTensor,
+                      r: HipTensor, z: HipTensor, n: HipTensor, Uh: HipTensor):
+    """gru_cell_backward (nnp_gru.nim:148-192): (dx, dh, dW3, dU3, dbW3, dbU3) from the gradient `dnext` of the next
+    hidden state, the inputs of the forward pass (h is the hidden state BEFORE it) and the tensors it saved. The
+    element-wise steps and the two concatenations of the reference are one launch that writes the gate gradients into
+    the column slices of one [batch, 3H] buffer per dense layer; then the two linear_backward and dh + dnext * z."""
+    B, H = h.shape
+    dW3x, dU3h = empty((B, 3 * H), h.dtype), empty((B, 3 * H), h.dtype)
+    saved = (dnext, h, r, z, n, Uh)
+    same = all(t.shape == (B, H) and t.strides == dnext.strides and t.strides[1] == 1 for t in saved)
+    if same:
+        check(getattr(_lib.load(), f"am_hip_gru_gates_backward_{h.sfx}")(
+            B, H, *[ctypes.c_void_p(t.data_ptr()) for t in saved], dnext.strides[0],
+            ctypes.c_void_p(dW3x.data_ptr()), 3 * H, ctypes.c_void_p(dU3h.data_ptr()), 3 * H))
+    else:   # operands of different layouts: the separate passes take any strides
+        _gru_gates_backward_passes(dnext, h, r, z, n, Uh, dW3x, dU3h)
     dx, dW3, dbW3 = linear_backward(x, W3, dW3x)                                 # step 1
     dh, dU3, dbU3 = linear_backward(h, U3, dU3h)
     _ternary_into("muladd", dh, dnext, z, dh)                                    # step 4, h part: dh + dnext * z

@@ -586,6 +586,17 @@ int am_hip_gru_gates_f32(int64_t batch, int64_t H, const float* w3x, int64_t ldw
 int am_hip_gru_gates_f64(int64_t batch, int64_t H, const double* w3x, int64_t ldw, const double* u3h, int64_t ldu,
                          double* hidden, int64_t ldh, double* r, double* z, double* n, double* uh, int64_t lds);
 
+/* The element-wise part of the cell's backward pass in one launch: from dnext (the gradient of the next hidden state), h
+ * (the hidden state BEFORE the step) and r, z, n, uh as kept by am_hip_gru_gates_* (all [batch, H], rows ld_in apart), the
+ * gradients of the two products, dw3x = [dWrx | dWzx | dWx] and du3h = [dWrx | dWzx | dUh] ([batch, 3H], rows ldw resp. ldu
+ * apart). Replaces the `-.` / `*.` / tanh_backward / sigmoid_backward passes and the two `concat`s of gru_cell_backward
+ * (src/arraymancer/nn_primitives/nnp_gru.nim:165-186); the two linear_backward calls and the final dh + dnext * z stay
+ * with the caller. */
+int am_hip_gru_gates_backward_f32(int64_t batch, int64_t H, const float* dnext, const float* h, const float* r, const float* z,
+                                  const float* n, const float* uh, int64_t ld_in, float* dw3x, int64_t ldw, float* du3h, int64_t ldu);
+int am_hip_gru_gates_backward_f64(int64_t batch, int64_t H, const double* dnext, const double* h, const double* r, const double* z,
+                                  const double* n, const double* uh, int64_t ld_in, double* dw3x, int64_t ldw, double* du3h, int64_t ldu);
+
 /* *loss (host) <- (1 / rows) * sum over the rows i of  ln(sum_j exp(input[i, j])) - sum_j input[i, j] * target[i, j]:
  * softmax and cross-entropy in one pass over `input` [rows, cols] and `target` [rows, cols] (probabilities), element
  * strides (rs, cs). Blocking; 0 for an empty batch. Replaces softmax_cross_entropy

@@ -187,3 +187,35 @@ def test_fused_gates_equal_the_three_passes(hip, dt):
         assert np.array_equal(h3.toCpu(), h.toCpu())
     with pytest.raises(ValueError):
         th._gru_gates_inplace(hip.zeros((2, 5), dt), hip.zeros((2, 6), dt), hip.zeros((2, 2), dt))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_fused_backward_gates_equal_the_separate_passes(hip, dt):
+    """am_hip_gru_gates_backward_* against the reference's sequence of `-.`, `*.`, tanh_backward, sigmoid_backward and
+    concat (nnp_gru.nim:165-186) run as separate launches: both [batch, 3H] gradients bit for bit, on shapes that take
+    the 16-byte lanes and on ones that take the element lanes."""
+    from arraymancer_amd import tensor_hip as th
+    rng = np.random.default_rng(seed_of("gru-gates-bwd", np.dtype(dt).name))
+    for B, H in ((3, 2), (64, 96), (17, 33), (128, 512)):
+        host = [rng.uniform(-1, 1, (B, H)).astype(dt) for _ in range(6)]          # dnext, h, r, z, n, Uh
+        dev = [hip.toHip(a) for a in host]
+        want_w, want_u = hip.empty((B, 3 * H), dt), hip.empty((B, 3 * H), dt)
+        th._gru_gates_backward_passes(*dev, want_w, want_u)
+        x = hip.toHip(rng.uniform(-1, 1, (B, 5)).astype(dt))
+        W3_, U3_ = hip.toHip(rng.uniform(-1, 1, (3 * H, 5)).astype(dt)), hip.toHip(rng.uniform(-1, 1, (3 * H, H)).astype(dt))
+        dx, dh, dW3, dU3, dbW3, dbU3 = hip.gru_cell_backward(dev[0], x, dev[1], W3_, U3_, *dev[2:])
+        # the dense layers' gradients are functions of the two gate-gradient buffers alone
+        wx, wW, wb = hip.linear_backward(x, W3_, want_w)
+        wh, wU, wbu = hip.linear_backward(dev[1], U3_, want_u)
+        assert np.array_equal(dx.toCpu(), wx.toCpu()) and np.array_equal(dW3.toCpu(), wW.toCpu()) and np.array_equal(dbW3.toCpu(), wb.toCpu())
+        assert np.array_equal(dU3.toCpu(), wU.toCpu()) and np.array_equal(dbU3.toCpu(), wbu.toCpu())
+        assert np.array_equal(dh.toCpu(), (host[0] * host[3] + wh.toCpu()).astype(dt))
+        # and the gate gradients themselves, against NumPy (single IEEE operations in the same order)
+        dnext, h, r, z, n, Uh = host
+        one = dt(1)
+        dz, dn = (h - n) * dnext, (one - z) * dnext
+        dWx = dn * (one - n * n)
+        dr, dUh = Uh * dWx, r * dWx
+        dWzx, dWrx = z * (one - z) * dz, r * (one - r) * dr
+        assert np.array_equal(want_w.toCpu(), np.concatenate([dWrx, dWzx, dWx], 1))
+        assert np.array_equal(want_u.toCpu(), np.concatenate([dWrx, dWzx, dUh], 1))
