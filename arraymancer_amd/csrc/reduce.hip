@@ -25,6 +25,7 @@
 #include <limits>
 #include <string.h>
 #include "common.h"
+#include "fastdiv.h"
 
 namespace am {
 namespace gemm { void* splitk_workspace(size_t bytes); }
@@ -1407,6 +1408,43 @@ __global__ __launch_bounds__(256) void maxpool2d(const T* in, T* out, int64_t* a
 // The common 2-wide, stride-2, unpadded-in-width pooling with 16-byte aligned rows: one lane makes
 // V = 16 / sizeof(T) neighbouring outputs from two 16-byte loads per window row, and stores them
 // (and their indices) as vectors. Window scan order and comparisons as in the kernel above.
+// Windows of a few elements (KH x KW known at compile time, any stride and padding): the KH * KW loads of a window are
+// issued together, from a clamped address where the window reaches into the padding, and compared afterwards in the
+// reference's scan order with its strict `>`; the output index is taken apart with launch-constant dividers. 3 x 3
+// windows with stride 2 and padding 1 on [64, 64, 112, 112] f32: 2.6 -> see the measurement beside the host function.
+template <typename T, int KH, int KW>
+__global__ __launch_bounds__(256) void maxpool2d_small(const T* __restrict__ in, T* __restrict__ out, int64_t* __restrict__ argmax,
+                                                       uint32_t total, int H, int W, int padH, int padW, int sH, int sW,
+                                                       FastDiv by_outw, FastDiv by_outh) {
+  const uint32_t oidx = blockIdx.x * 256u + threadIdx.x;
+  if (oidx >= total) return;
+  uint32_t w, h;
+  const uint32_t nc = by_outh.divmod(by_outw.divmod(oidx, w), h);   // n * C + c
+  const int row0 = (int)h * sH - padH, col0 = (int)w * sW - padW;
+  const int64_t base = (int64_t)nc * H * W;
+  const T* __restrict__ plane = in + base;
+  T v[KH][KW];
+  int off[KH][KW];
+#pragma unroll
+  for (int ph = 0; ph < KH; ++ph)
+#pragma unroll
+    for (int pw = 0; pw < KW; ++pw) {
+      const int row = row0 + ph, col = col0 + pw;
+      const bool ok = (unsigned)row < (unsigned)H && (unsigned)col < (unsigned)W;
+      off[ph][pw] = ok ? row * W + col : -1;
+      v[ph][pw] = plane[ok ? row * W + col : 0];
+    }
+  T mx = Lowest<T>::value();
+  int best = -1;
+#pragma unroll
+  for (int ph = 0; ph < KH; ++ph)
+#pragma unroll
+    for (int pw = 0; pw < KW; ++pw)
+      if (off[ph][pw] >= 0 && v[ph][pw] > mx) { mx = v[ph][pw]; best = off[ph][pw]; }
+  out[oidx] = mx;
+  if (argmax) argmax[oidx] = best >= 0 ? base + best : std::numeric_limits<int64_t>::lowest();
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void maxpool2d_w2(const T* in, T* out, int64_t* argmax, int64_t total_vec, int H, int W,
                                                     int kH, int padH, int sH, int outH, int outWv) {
@@ -1473,6 +1511,16 @@ static int maxpool(const char* fn, int64_t N, int C, int H, int W, int kH, int k
   }
   const int64_t bx = (total + 255) / 256;
   if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many output elements", fn);
+  if (total < ((int64_t)1 << 32) && (int64_t)H * W < ((int64_t)1 << 31) && kH == kW && (kH == 2 || kH == 3)) {
+    const FastDiv by_outw((uint32_t)outW), by_outh((uint32_t)outH);
+    if (kH == 2)
+      hipLaunchKernelGGL((maxpool2d_small<T, 2, 2>), dim3((unsigned)bx), dim3(256), 0, stream(), in, out, argmax, (uint32_t)total, H, W,
+                         padH, padW, sH, sW, by_outw, by_outh);
+    else
+      hipLaunchKernelGGL((maxpool2d_small<T, 3, 3>), dim3((unsigned)bx), dim3(256), 0, stream(), in, out, argmax, (uint32_t)total, H, W,
+                         padH, padW, sH, sW, by_outw, by_outh);
+    return check_launch("maxpool2d_small");
+  }
   if (total < ((int64_t)1 << 32))
     hipLaunchKernelGGL((maxpool2d<T, uint32_t>), dim3((unsigned)bx), dim3(256), 0, stream(), in, out, argmax, total, C, H, W,
                        kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);
@@ -1517,6 +1565,55 @@ __global__ __launch_bounds__(256) void maxpool2d_backward(const int64_t* argmax,
 // Windows two wide with stride two and no padding in width (W a multiple of the 16-byte vector): a lane
 // owns V consecutive input columns, i.e. V / 2 windows per candidate row of windows, read and written
 // as vectors.
+// At most NH x NW windows contain an input element (NH = ceil(kH / sH), NW likewise, known at compile time): their recorded
+// indices and gradients are loaded together (from a clamped position where a window does not exist) and the first match
+// in the order "highest output index first" decides.
+template <typename T, int NH, int NW>
+__global__ __launch_bounds__(256) void maxpool2d_backward_small(const int64_t* __restrict__ argmax, const T* __restrict__ grad_out,
+                                                                T* __restrict__ grad_in, uint32_t total, int H, int W, int kH, int kW,
+                                                                int padH, int padW, int sH, int sW, int outH, int outW,
+                                                                FastDiv by_w, FastDiv by_h, FastDiv by_sh, FastDiv by_sw) {
+  const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+  if (p >= total) return;
+  uint32_t col, row;
+  const uint32_t nc = by_h.divmod(by_w.divmod(p, col), row);
+  const int rh = (int)row + padH, rw = (int)col + padW;
+  int h_hi = (int)by_sh.div((uint32_t)rh), w_hi = (int)by_sw.div((uint32_t)rw);
+  const int h_lo = rh - kH + 1 <= 0 ? 0 : (int)by_sh.div((uint32_t)(rh - kH + sH));
+  const int w_lo = rw - kW + 1 <= 0 ? 0 : (int)by_sw.div((uint32_t)(rw - kW + sW));
+  if (h_hi > outH - 1) h_hi = outH - 1;
+  if (w_hi > outW - 1) w_hi = outW - 1;
+  const int64_t obase = (int64_t)nc * outH * outW;
+  constexpr bool EAGER = NH * NW <= 4;
+  int64_t rec[NH][NW];
+  T gv[NH][NW];
+  bool ok[NH][NW];
+#pragma unroll
+  for (int i = 0; i < NH; ++i)
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const int h = h_hi - i, w = w_hi - j;
+      ok[i][j] = h >= h_lo && w >= w_lo;
+      const int64_t o = obase + (ok[i][j] ? h * outW + w : 0);
+      rec[i][j] = argmax[o];
+      // up to four candidates: the gradients are read with the indices, not after the comparison (one memory round
+      // trip per element: 14 x 14 maps, 2 x 2 / 2: 180 -> 152 us); with nine that costs more than it saves
+      if constexpr (EAGER) gv[i][j] = grad_out[o];
+    }
+  T g = (T)0;
+  int64_t hit = -1;
+#pragma unroll
+  for (int i = 0; i < NH; ++i)
+#pragma unroll
+    for (int j = 0; j < NW; ++j)
+      if (hit < 0 && ok[i][j] && rec[i][j] == (int64_t)p) {
+        hit = obase + (h_hi - i) * outW + (w_hi - j);
+        if constexpr (EAGER) g = gv[i][j];
+      }
+  if constexpr (!EAGER) { if (hit >= 0) g = grad_out[hit]; }
+  grad_in[p] = g;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void maxpool2d_backward_w2(const int64_t* argmax, const T* grad_out, T* grad_in,
                                                              uint32_t total_vec, int H, int Wv, int kH, int padH, int sH,
@@ -1573,6 +1670,24 @@ static int maxpool_backward(const char* fn, int64_t N, int C, int H, int W, int 
   }
   const int64_t bx = (total + 255) / 256;
   if (bx >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many input elements", fn);
+  {
+    const int nh = (kH + sH - 1) / sH, nw = (kW + sW - 1) / sW;   // windows that can contain one element
+    const int64_t outH_ = ((int64_t)H + 2 * padH - kH) / sH + 1, outW_ = ((int64_t)W + 2 * padW - kW) / sW + 1;
+    if (total < ((int64_t)1 << 31) && nh == nw && nh <= 3 && outH_ * outW_ < ((int64_t)1 << 31) &&
+        (int64_t)H + padH < ((int64_t)1 << 30) && (int64_t)W + padW < ((int64_t)1 << 30)) {
+      const FastDiv by_w((uint32_t)W), by_h((uint32_t)H), by_sh((uint32_t)sH), by_sw((uint32_t)sW);
+      if (nh == 1)   // windows that do not overlap (the stride is the window or more): one candidate
+        hipLaunchKernelGGL((maxpool2d_backward_small<T, 1, 1>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in,
+                           (uint32_t)total, H, W, kH, kW, padH, padW, sH, sW, (int)outH_, (int)outW_, by_w, by_h, by_sh, by_sw);
+      else if (nh == 2)
+        hipLaunchKernelGGL((maxpool2d_backward_small<T, 2, 2>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in,
+                           (uint32_t)total, H, W, kH, kW, padH, padW, sH, sW, (int)outH_, (int)outW_, by_w, by_h, by_sh, by_sw);
+      else
+        hipLaunchKernelGGL((maxpool2d_backward_small<T, 3, 3>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in,
+                           (uint32_t)total, H, W, kH, kW, padH, padW, sH, sW, (int)outH_, (int)outW_, by_w, by_h, by_sh, by_sw);
+      return check_launch("maxpool2d_backward_small");
+    }
+  }
   if (total < ((int64_t)1 << 32))
     hipLaunchKernelGGL((maxpool2d_backward<T, uint32_t>), dim3((unsigned)bx), dim3(256), 0, stream(), argmax, grad_out, grad_in,
                        total, H, W, kH, kW, padH, padW, sH, sW, (int)outH, (int)outW);

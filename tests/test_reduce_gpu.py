@@ -408,7 +408,12 @@ def test_maxpool_vs_oracle(hip, oracle, vectors, sfx):
     assert np.array_equal(idx.toCpu(), np.array(g["max_indices"], dtype=np.int64))
     rng = np.random.default_rng(seed_of("maxpool-gpu", sfx))
     cases = [((2, 3, 7, 9), (2, 2), (0, 0), (2, 2)), ((4, 20, 24, 24), (2, 2), (0, 0), (2, 2)), ((3, 5, 13, 11), (3, 3), (1, 1), (1, 1)),
-             ((2, 2, 9, 8), (3, 2), (1, 0), (2, 3)), ((1, 1, 5, 5), (2, 2), (2, 2), (1, 1)), ((64, 50, 8, 8), (2, 2), (0, 0), (2, 2))]
+             ((2, 2, 9, 8), (3, 2), (1, 0), (2, 3)), ((1, 1, 5, 5), (2, 2), (2, 2), (1, 1)), ((64, 50, 8, 8), (2, 2), (0, 0), (2, 2)),
+             # the small-window kernels: 3 x 3 with stride 2 and padding (four windows per element), stride 3 (one), padding
+             # as wide as the reach; 2 x 2 with stride 1 (four), 3 (gaps between the windows) and odd widths (14 x 14 maps)
+             ((3, 4, 16, 16), (3, 3), (1, 1), (2, 2)), ((2, 3, 15, 17), (3, 3), (1, 1), (2, 2)), ((2, 2, 10, 11), (3, 3), (0, 0), (3, 3)),
+             ((1, 2, 6, 7), (3, 3), (2, 2), (1, 1)), ((2, 3, 9, 9), (2, 2), (0, 0), (1, 1)), ((2, 3, 11, 10), (2, 2), (1, 1), (3, 3)),
+             ((8, 16, 14, 14), (2, 2), (0, 0), (2, 2)), ((2, 2, 7, 9), (3, 3), (1, 1), (2, 1)), ((1, 1, 4, 4), (4, 4), (0, 0), (4, 4))]
     for shape, kernel, pad, stride in cases:
         x = rng.integers(-5, 5, shape).astype(dt)        # ties are frequent: the first maximum must win
         say("maxpool", sfx, shape, kernel, pad, stride)
