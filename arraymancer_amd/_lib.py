@@ -65,6 +65,7 @@ def _signatures():
         "am_hip_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),
         "am_hip_event_destroy": (ci, [vp]),
         "am_hip_graph_begin": (ci, []),
+        "am_hip_alloc_hold": (ci, [ci]),
         "am_hip_graph_end": (ci, [pp]),
         "am_hip_graph_launch": (ci, [vp]),
         "am_hip_graph_destroy": (ci, [vp]),

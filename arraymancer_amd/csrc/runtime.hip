@@ -119,6 +119,11 @@ static size_t round_size(size_t bytes) {
 // host layer allocated before the capture and dropped inside it), so they stay allocated, owned by the
 // graph, and go back to the cache when the graph is destroyed.
 static std::vector<void*> g_capture_freed;
+// Rehearsal of a sequence that is about to be captured: while the hold is on, freed blocks are not handed out again
+// but collected here, so that every allocation of the sequence takes a block of its own; switching the hold off puts
+// them all into the cache, where the capture of the same sequence then finds one block per allocation.
+static bool g_hold = false;
+static std::vector<void*> g_held;
 static std::unordered_map<void*, std::vector<void*>> g_graph_blocks;   // executable graph -> blocks it keeps alive
 
 // Hands a live block back: to the cache, or to the driver when the cache is full. g_alloc_mu held.
@@ -190,7 +195,6 @@ int am_hip_malloc(size_t bytes, void** out) {
   *out = nullptr;
   if (bytes == 0) return AM_OK;
   AM_TRY(ensure_init());
-  if (g_capturing) return fail(AM_E_ARG, "am_hip_malloc: not allowed while a graph is being captured");
   const size_t rounded = round_size(bytes);
   std::lock_guard<std::mutex> lk(g_alloc_mu);
   auto it = g_free_blocks.find(rounded);
@@ -198,6 +202,10 @@ int am_hip_malloc(size_t bytes, void** out) {
     *out = it->second.back();
     it->second.pop_back();
     g_cached_bytes -= rounded;
+  } else if (g_capturing) {
+    // The driver cannot be asked for memory while the stream records: a capture is served from the cache alone.
+    return fail(AM_E_ALLOC, "am_hip_malloc: no cached block of %zu bytes while a graph is being captured (run the sequence "
+                "once between am_hip_alloc_hold(1) and am_hip_alloc_hold(0) first: that leaves one cached block per allocation)", rounded);
   } else {
     hipError_t e = hipMalloc(out, rounded);
     if (e != hipSuccess && g_cached_bytes > 0) {   // give the cache back and try once more
@@ -229,7 +237,30 @@ int am_hip_free(void* dptr) {
     g_capture_freed.push_back(dptr);
     return AM_OK;
   }
+  if (g_hold) {   // kept until am_hip_alloc_hold(0), see g_held
+    if (g_live.find(dptr) == g_live.end())
+      return fail(AM_E_ARG, "am_hip_free: %p was not allocated by am_hip_malloc (or freed twice)", dptr);
+    for (void* q : g_held)
+      if (q == dptr) return fail(AM_E_ARG, "am_hip_free: %p freed twice", dptr);
+    g_held.push_back(dptr);
+    return AM_OK;
+  }
   return free_block_locked(dptr);
+}
+
+int am_hip_alloc_hold(int on) {
+  AM_TRY(ensure_init());
+  if (g_capturing) return fail(AM_E_ARG, "am_hip_alloc_hold: not allowed while a graph is being captured");
+  std::lock_guard<std::mutex> lk(g_alloc_mu);
+  if (on) { g_hold = true; return AM_OK; }
+  g_hold = false;
+  int rc = AM_OK;
+  for (void* q : g_held) {
+    const int r = free_block_locked(q);
+    if (r != AM_OK) rc = r;
+  }
+  g_held.clear();
+  return rc;
 }
 
 int am_hip_empty_cache(void) {

@@ -19,7 +19,7 @@ import numpy as np
 
 from . import _lib
 from ._lib import check
-from .tensor_hip import (Graph, HipTensor, _ternary_into, conv2d_backward, conv2d_into, empty, gemm, linear_backward,
+from .tensor_hip import (Graph, HipTensor, _ternary_into, _unary_into, conv2d_backward, conv2d_into, empty, gemm, linear_backward,
                          maxpool2d_backward, relu_backward, sparse_softmax_cross_entropy,
                          sparse_softmax_cross_entropy_backward, toHip)
 
@@ -64,7 +64,7 @@ class DemoNet:
         gemm(1, self.hidden, p["classifier_w"].transpose(), 0, self.logits, epilogue="bias", bias=p["classifier_b"])
         return self.logits
 
-    def loss_and_gradients(self, x: HipTensor, labels: HipTensor):
+    def loss_and_gradients(self, x: HipTensor, labels: HipTensor, with_loss: bool = True):
         """One training pass of the example's learning loop (examples/ex02_handwritten_digits_recognition.nim:58-72)
         without the update: forward, `sparse_softmax_cross_entropy` against the int64 `labels` [batch], and what
         `loss.backprop()` walks through, composed from the backward primitives in the order of the forward pass
@@ -72,7 +72,7 @@ class DemoNet:
         nnp_maxpooling.nim:68-83, nnp_convolution.nim:65-107). Returns (loss, gradients by parameter name)."""
         p, n = self.p, self.batch
         logits = self.forward(x)
-        loss = sparse_softmax_cross_entropy(logits, labels)
+        loss = sparse_softmax_cross_entropy(logits, labels) if with_loss else None
         d_logits = sparse_softmax_cross_entropy_backward(1, logits, labels)
         flat = self.pool2.reshape(n, self.pool2.size // n)
         d_hidden, g_cw, g_cb = linear_backward(self.hidden, p["classifier_w"], d_logits)
@@ -91,10 +91,34 @@ class DemoNet:
     def sgd_update(self, gradients: dict, learning_rate: float):
         """The SGD optimizer's update (src/arraymancer/nn/optimizers/optimizers.nim:35-51: x - lr * y over every parameter)
         as one pass per parameter: value = grad * (-learning_rate) + value, the same two roundings."""
-        step = toHip(np.array([-learning_rate], dtype=self.dtype))
+        step = self._step_tensor(learning_rate)
         for name, g in gradients.items():
             w = self.p[name]
             _ternary_into("muladd", w, g, step.reshape(*([1] * w.rank)).broadcast(w.shape), w)
+
+    def _step_tensor(self, learning_rate: float) -> HipTensor:
+        """-learning_rate as a one-element device tensor, uploaded once per value (an upload cannot be recorded)."""
+        cache = self.__dict__.setdefault("_steps", {})
+        if learning_rate not in cache:
+            cache[learning_rate] = toHip(np.array([-learning_rate], dtype=self.dtype))
+        return cache[learning_rate]
+
+    def gradients(self, x: HipTensor, labels: HipTensor) -> dict:
+        """`loss_and_gradients` without the loss: device work only, so that it can be recorded into a graph."""
+        return self.loss_and_gradients(x, labels, with_loss=False)[1]
+
+    def capture_train_step(self, x: HipTensor, labels: HipTensor, learning_rate: float = 0.01) -> Graph:
+        """One whole learning step (forward, backward, update; the loss is not read back) as ONE graph over the
+        buffers `x` and `labels`: refill them and launch. About forty kernels per replay and no host work in between."""
+        self._step_tensor(learning_rate)
+
+        def step():
+            self.sgd_update(self.gradients(x, labels), learning_rate)
+        before = {k: v.clone() for k, v in self.p.items()}      # the rehearsal and the capture are not steps of the training
+        g = Graph.record(step)
+        for k, v in before.items():
+            _unary_into("copy", self.p[k], v)
+        return g.keep(x, labels)
 
     def train_step(self, x: HipTensor, labels: HipTensor, learning_rate: float = 0.01):
         loss, gradients = self.loss_and_gradients(x, labels)

@@ -311,9 +311,10 @@ def sync() -> None:
 
 class Graph:
     """Records the device operations issued inside `with Graph() as g:` into a HIP graph instead
-    of running them; `g.launch()` replays the sequence with one call. Output tensors must be
-    allocated before the block (allocation is refused during capture), e.g. with `empty` and the
-    `gemm(alpha, A, B, beta, C)` / `apply2` / `_into` forms. A tensor that goes out of scope inside the
+    of running them; `g.launch()` replays the sequence with one call. Allocation during the block is
+    served from the allocator's cache of freed blocks only (`Graph.record(fn)` prepares it with a
+    rehearsal); results that are read after a replay must live in tensors made before the block, e.g. with
+    `empty` and the `gemm(alpha, A, B, beta, C)` / `apply2` / `_into` forms. A tensor that goes out of scope inside the
     block is kept alive by the graph (the library holds its block until the graph is destroyed); tensors
     recorded in the graph and dropped after the block must outlive the replays - pass them to `keep()`
     to tie their lifetime to the graph's."""
@@ -333,6 +334,22 @@ class Graph:
 
     def launch(self):
         check(_lib.load().am_hip_graph_launch(self._exec))
+
+    @staticmethod
+    def record(fn) -> "Graph":
+        """A graph of everything `fn()` issues, temporaries included. `fn` runs twice: once as a rehearsal with the
+        allocator holding back every block that is freed (afterwards its cache has one block per allocation `fn`
+        makes, and the library workspace its final size), then under capture, where allocation is served from that
+        cache. `fn` must only issue device work (no read-backs, uploads or `zeros`) on tensors that outlive the graph."""
+        L = _lib.load()
+        check(L.am_hip_alloc_hold(1))
+        try:
+            fn()
+        finally:
+            check(L.am_hip_alloc_hold(0))
+        with Graph() as g:
+            fn()
+        return g
 
     def keep(self, *tensors):
         """Holds a reference to the storage of each tensor for as long as this graph exists."""

@@ -449,14 +449,20 @@ def bench_ex02_train(am, timer, steps, warmup, batch=64):
     dx = am.toHip(rng.uniform(0, 1, (batch, 1, 28, 28)).astype(np.float32))
     dl = am.toHip(rng.integers(0, 10, batch).astype(np.int64))
     wall, ev = timer.run(lambda: net.train_step(dx, dl, 0.01), steps, warmup, WARM_S)
+    graph = net.capture_train_step(dx, dl, 0.01)
+    wall_g, ev_g = timer.run(graph.launch, steps, warmup, WARM_S)
     flops = 3 * 2.0 * batch * (20 * 25 * 576 + 50 * 500 * 64 + 800 * 500 + 500 * 10)
+    best = min(ev, ev_g)
     return dict(workload=f"f32 example-2 training step, batch {batch}: forward, sparse softmax cross-entropy, backward through "
                          "linear / ReLU / maxpool / conv2d, SGD update of 8 parameters",
-                unit="us per step", dtype="f32", higher_is_better=False, value=round(ev / steps * 1e6, 2),
-                wall_us=round(wall / steps * 1e6, 2), images_per_s=round(batch / (ev / steps), 0),
-                gflops=round(flops / (ev / steps) / 1e9, 1),
-                note="about forty short launches issued one by one from the host (the loss is read back every step, as the "
-                     "example prints it): bound by the host's launch rate, not by the 0.9 GFLOP of arithmetic")
+                unit="us per step", dtype="f32", higher_is_better=False, value=round(best / steps * 1e6, 2),
+                value_is="eager" if ev <= ev_g else "hipgraph", eager_us=round(ev / steps * 1e6, 2),
+                eager_wall_us=round(wall / steps * 1e6, 2), hipgraph_us=round(ev_g / steps * 1e6, 2),
+                images_per_s=round(batch / (best / steps), 0), gflops=round(flops / (best / steps) / 1e9, 1),
+                note="eager: about forty short launches issued one by one from the host, the loss read back every step: bound "
+                     "by the host's launch rate. hipgraph: the same step without the read-back recorded once with its "
+                     "temporaries (a rehearsal leaves the allocator one cached block per allocation, the capture is served "
+                     "from that cache) and replayed with one launch per step")
 
 
 def bench_conv_backward(am, timer, steps, warmup, first_only=False):

@@ -82,7 +82,8 @@ int am_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* synchronises
 int am_hip_event_destroy(void* ev);
 
 /* HIP graphs on the library stream: between begin and end, GEMM / element-wise calls are recorded
- * instead of executed (allocation, copies, memset and sync are refused meanwhile); the returned
+ * instead of executed (copies, memset and sync are refused meanwhile, allocation is served from the cache: see
+ * am_hip_alloc_hold); the returned
  * executable graph replays the whole sequence with one launch. For launch-bound chains of small
  * kernels such as the reference's per-layer gemm + `+.=` + relu sequence
  * (src/arraymancer/nn_primitives/nnp_linear.nim:28-29, fallback/conv.nim:99-106). The reference
@@ -90,6 +91,14 @@ int am_hip_event_destroy(void* ev);
  * stay allocated while it is replayed: a block freed DURING the capture is kept alive by the graph itself,
  * one freed after am_hip_graph_end is the caller's responsibility. */
 int am_hip_graph_begin(void);
+/* Memory for a capture. am_hip_malloc during a capture is served from the library's cache of freed blocks only (the
+ * driver cannot be asked for memory while the stream records) and fails with AM_E_ALLOC when the cache has no block of
+ * that size. am_hip_alloc_hold(1) ... am_hip_alloc_hold(0) around one ordinary run of the sequence prepares that cache:
+ * while the hold is on, freed blocks are set aside instead of being handed out again, so that every allocation of the
+ * sequence gets a block of its own, and switching it off puts them all into the cache. The same sequence recorded right
+ * afterwards then finds one block per allocation (and the library workspace at its final size). No counterpart in the
+ * reference. */
+int am_hip_alloc_hold(int on);
 int am_hip_graph_end(void** graph_exec);
 int am_hip_graph_launch(void* graph_exec);
 int am_hip_graph_destroy(void* graph_exec);

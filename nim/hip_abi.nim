@@ -45,6 +45,7 @@ proc am_hip_event_elapsed_ms*(start, stop: pointer, ms: ptr cfloat): cint {.impo
 proc am_hip_event_destroy*(ev: pointer): cint {.importc.}
 
 proc am_hip_graph_begin*(): cint {.importc.}
+proc am_hip_alloc_hold*(on: cint): cint {.importc.}
 proc am_hip_graph_end*(graph_exec: ptr pointer): cint {.importc.}
 proc am_hip_graph_launch*(graph_exec: pointer): cint {.importc.}
 proc am_hip_graph_destroy*(graph_exec: pointer): cint {.importc.}

@@ -148,3 +148,50 @@ def test_ex02_training_step(hip, oracle, sfx):
     losses = [float(loss)] + [float(net.train_step(dx, dl, 0.01)) for _ in range(5)]
     say("  losses over six steps on one batch:", [round(v, 4) for v in losses])
     assert losses[-1] < losses[0]
+
+
+def test_ex02_training_step_as_one_graph(hip):
+    """The whole learning step (forward, backward, SGD update; about forty kernels with their temporaries) recorded
+    into ONE graph by Graph.record - a rehearsal that leaves the allocator one cached block per allocation, then the
+    capture served from that cache - against the same steps issued one by one: parameters bit for bit after every
+    step, with new images and labels in the same buffers each time; the recording itself must not count as a step."""
+    from arraymancer_amd import ex02
+    dt, batch = np.float32, 32
+    rng = np.random.default_rng(seed_of("ex02-train-graph"))
+    p = ex02.random_params(rng, dt)
+    eager, replayed = ex02.DemoNet(batch, p, dt), ex02.DemoNet(batch, p, dt)
+    x, labels = hip.empty((batch, 1, 28, 28), dt), hip.empty((batch,), np.int64)
+    first_x, first_l = rng.uniform(0, 1, (batch, 1, 28, 28)).astype(dt), rng.integers(0, 10, batch).astype(np.int64)
+    hip.tensor_hip._unary_into("copy", x, hip.toHip(first_x))
+    hip.tensor_hip._unary_into("copy", labels, hip.toHip(first_l))
+    say("ex02 training step as a graph: recording")
+    graph = replayed.capture_train_step(x, labels, 0.05)
+    for name in p:
+        assert np.array_equal(replayed.p[name].toCpu(), np.asarray(p[name], dtype=dt).reshape(replayed.p[name].shape)), name
+    eager._step_tensor(0.05)                     # the eager net's own one-element tensor, kept from its first step on
+    live0, _ = memory(hip)
+    for step in range(4):
+        hx, hl = rng.uniform(0, 1, (batch, 1, 28, 28)).astype(dt), rng.integers(0, 10, batch).astype(np.int64)
+        hip.tensor_hip._unary_into("copy", x, hip.toHip(hx))
+        hip.tensor_hip._unary_into("copy", labels, hip.toHip(hl))
+        eager.train_step(x, labels, 0.05)
+        graph.launch()
+        hip.sync()
+        for name in p:
+            assert np.array_equal(replayed.p[name].toCpu(), eager.p[name].toCpu()), (step, name)
+    live1, _ = memory(hip)
+    assert live1 <= live0, "replays must not allocate"
+    # a sequence that was not rehearsed finds no cached block of an unusual size: a clear error, and the capture ends cleanly
+    del graph, replayed, eager
+    assert hip.load_library().am_hip_empty_cache() == 0
+    with pytest.raises(hip.HipAllocError):
+        with hip.Graph():
+            hip.empty((12345, 77), np.float64)
+    assert hip.empty((4,), dt).shape == (4,)
+
+
+def memory(hip):
+    import ctypes
+    live, cached = ctypes.c_size_t(), ctypes.c_size_t()
+    hip.load_library().am_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached))
+    return live.value, cached.value
