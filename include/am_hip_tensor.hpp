@@ -334,6 +334,14 @@ class HipTensor {
       check(detail::binary_(op, rank(), shape.data(), ptr(), strides.data(), ptr(), strides.data(), src.ptr(), src.strides.data()));
     return *this;
   }
+  // Element-wise copy of a tensor of the same shape into this one's memory, through both tensors' strides
+  // (the reference's copyFrom / slice assignment; a device-side pass, recordable into a graph).
+  HipTensor& copy_from(const HipTensor& src) {
+    if (shape != src.shape)
+      throw std::invalid_argument("copy_from: shapes " + detail::str(shape) + " and " + detail::str(src.shape) + " differ");
+    if (size() > 0) check(detail::unary_(AM_UOP_COPY, rank(), shape.data(), ptr(), strides.data(), src.ptr(), src.strides.data()));
+    return *this;
+  }
   HipTensor& apply_scalar(int op, T s) {
     if (size() > 0) check(detail::scalar_(op, 0, rank(), shape.data(), ptr(), strides.data(), ptr(), strides.data(), s));
     return *this;
@@ -904,6 +912,42 @@ HipTensor<T> maxpool2d_backward(const Shape& cached_input_shape, const HipTensor
                                     grad_output.ptr(), r.ptr()));
   return r;
 }
+
+// ---- HIP graphs ---------------------------------------------------------------------------------
+// A recorded sequence of device operations, replayed with one launch. Graph::record(fn) runs fn twice: once as a
+// rehearsal with the allocator holding back every block that is freed (afterwards its cache has one block per
+// allocation fn makes, and the library workspace its final size), then under capture, where allocation is served from
+// that cache - so fn may create temporaries freely. fn must only issue device work (no toCpu / toHip) on tensors that
+// outlive the graph. The reference has no counterpart (one launch per operator).
+class Graph {
+ public:
+  Graph() = default;
+  Graph(const Graph&) = delete;
+  Graph& operator=(const Graph&) = delete;
+  Graph(Graph&& o) noexcept : exec_(o.exec_) { o.exec_ = nullptr; }
+  Graph& operator=(Graph&& o) noexcept {
+    if (this != &o) { reset(); exec_ = o.exec_; o.exec_ = nullptr; }
+    return *this;
+  }
+  ~Graph() { reset(); }
+
+  template <typename F> static Graph record(F&& fn) {
+    check(am_hip_alloc_hold(1));
+    try { fn(); } catch (...) { (void)am_hip_alloc_hold(0); throw; }
+    check(am_hip_alloc_hold(0));
+    check(am_hip_graph_begin());
+    Graph g;
+    try { fn(); } catch (...) { void* dead = nullptr; (void)am_hip_graph_end(&dead); if (dead) (void)am_hip_graph_destroy(dead); throw; }
+    check(am_hip_graph_end(&g.exec_));
+    return g;
+  }
+  void launch() const { check(am_hip_graph_launch(exec_)); }
+  explicit operator bool() const { return exec_ != nullptr; }
+
+ private:
+  void reset() { if (exec_) { (void)am_hip_graph_destroy(exec_); exec_ = nullptr; } }
+  void* exec_ = nullptr;
+};
 
 // ---- .npy files (src/arraymancer/io/io_npy.nim:64-183) -----------------------------------------
 namespace detail {

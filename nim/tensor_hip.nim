@@ -800,6 +800,36 @@ proc maxpool2d_backward*[T: HipScalar](cached_input_shape: openArray[int], cache
   elif T is int32: call am_hip_maxpool2d_backward_i32
   else: call am_hip_maxpool2d_backward_i64
 
+# ---------------------------------------------------------------- HIP graphs
+type HipGraph* = object
+  ## A recorded sequence of device operations, replayed with one launch (no counterpart in the reference).
+  exec: pointer
+
+proc `=destroy`*(g: HipGraph) =
+  if not g.exec.isNil: discard am_hip_graph_destroy(g.exec)
+
+proc `=copy`*(dst: var HipGraph, src: HipGraph) {.error: "a HipGraph owns its executable graph".}
+
+template recordGraph*(body: untyped): HipGraph =
+  ## Runs `body` twice: once as a rehearsal with the allocator holding back every block that is freed (its cache then
+  ## has one block per allocation of `body`, the library workspace its final size), then under capture, where
+  ## allocation is served from that cache. `body` must only issue device work on tensors that outlive the graph.
+  block:
+    var g: HipGraph
+    check am_hip_alloc_hold(1)
+    try:
+      body
+    finally:
+      check am_hip_alloc_hold(0)
+    check am_hip_graph_begin()
+    try:
+      body
+    finally:
+      check am_hip_graph_end(g.exec.addr)
+    g
+
+proc launch*(g: HipGraph) = check am_hip_graph_launch(g.exec)
+
 # ---------------------------------------------------------------- .npy files and display
 # The file parsing and the pretty printer are the reference's own host code (io/io_npy.nim:64-183,
 # tensor/private/p_display.nim); the device tensor goes through a host copy, exactly as

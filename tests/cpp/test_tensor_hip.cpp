@@ -268,6 +268,29 @@ static void gru_cell_literals() {
   for (size_t i = 0; i < 6; ++i) CHECK(std::fabs((1 - z[i]) * n[i] + z[i] * -1.0 - hn[i]) < 1e-15);
 }
 
+static void graph_with_temporaries() {
+  // A sequence with temporaries recorded as it is: out <- relu(a * w + a) through three operator results that are
+  // dropped inside the recorded function; replays follow new values written into `a`.
+  auto a = toHip<float>({1, -2, 3, -4}, {2, 2});
+  auto w = toHip<float>({1, 0, 0, 1}, {2, 2});
+  am::HipTensor<float> out(Shape{2, 2});
+  auto step = [&]() {
+    auto prod = a * w;            // temporary
+    auto sum = prod + a;          // temporary
+    out.copy_from(am::unary(AM_UOP_RELU, sum));
+  };
+  auto g = am::Graph::record(step);
+  g.launch();
+  CHECK(eq(out, {2, 0, 6, 0}));
+  a.copy_from(toHip<float>({-1, 2, -3, 4}, {2, 2}));
+  g.launch();
+  CHECK(eq(out, {0, 4, 0, 8}));
+  am::Graph moved = std::move(g);
+  CHECK(bool(moved) && !bool(g));
+  moved.launch();
+  CHECK(eq(out, {0, 4, 0, 8}));
+}
+
 static void loss_literals() {
   // tests/nn_primitives/test_nnp_loss.nim:31-44: one row, truth = class 3, loss 0.0709 within 2e-5, dense and sparse
   auto predicted = toHip<double>({-3.44, 1.16, -0.81, 3.91}, {1, 4});
@@ -471,6 +494,7 @@ int main(int argc, char** argv) {
   conv_literals<int32_t>();
   conv_literals<int64_t>();
   loss_literals();
+  graph_with_temporaries();
   gru_cell_literals();
   conv_backward_known_answer<float>();
   conv_backward_known_answer<double>();
