@@ -17,7 +17,7 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          argmin_min, argmin, maxpool2d_backward, bc_pow, mreciprocal, clamp, mclamp, UFUNCS, ln, log10, log2, exp,
                          cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, arcsinh, arccosh, arctanh, erf, erfc,
                          gamma, lgamma, floor, ceil, trunc, reciprocal, tround as round, bc_eq, bc_ne, bc_lt, bc_le, bc_gt,
-                         bc_ge, isNaN, isNotNaN, classify, FLOAT_CLASS, sgn, floorMod, copySign, mcopySign, degToRad, radToDeg, fac)
+                         bc_ge, isNaN, isNotNaN, classify, FLOAT_CLASS, sgn, floorMod, copySign, mcopySign, degToRad, radToDeg, fac, sgd_update)
 
 __all__ = [
     "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
@@ -31,6 +31,6 @@ __all__ = [
     "arcsin", "arccos", "arctan", "arcsinh", "arccosh", "arctanh", "erf", "erfc", "gamma", "lgamma", "floor", "ceil",
     "trunc", "reciprocal", "round",
     "bc_eq", "bc_ne", "bc_lt", "bc_le", "bc_gt", "bc_ge", "isNaN", "isNotNaN", "classify", "FLOAT_CLASS", "sgn", "floorMod",
-    "copySign", "mcopySign", "degToRad", "radToDeg", "fac",
+    "copySign", "mcopySign", "degToRad", "radToDeg", "fac", "sgd_update",
     "read_npy", "write_npy", "load_library",
 ]

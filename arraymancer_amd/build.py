@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libam_hip.so")
 SOURCES = [
     "runtime.hip", "diag.hip",
     "elementwise_f32.hip", "elementwise_f64.hip", "elementwise_i32.hip", "elementwise_i64.hip",
-    "gemm_f32.hip", "gemm_f64.hip", "gemm_i32.hip", "gemm_i64.hip", "gemv.hip", "im2col.hip", "reduce.hip", "loss.hip", "gru.hip",
+    "gemm_f32.hip", "gemm_f64.hip", "gemm_i32.hip", "gemm_i64.hip", "gemv.hip", "im2col.hip", "reduce.hip", "loss.hip", "gru.hip", "optim.hip",
 ]
 
 # -ffp-contract=off: every float operation of an epilogue / map body is rounded on its own, so

@@ -19,9 +19,9 @@ import numpy as np
 
 from . import _lib
 from ._lib import check
-from .tensor_hip import (Graph, HipTensor, _ternary_into, _unary_into, conv2d_backward, conv2d_into, empty, gemm, linear_backward,
+from .tensor_hip import (Graph, HipTensor, _unary_into, conv2d_backward, conv2d_into, empty, gemm, linear_backward,
                          maxpool2d_backward, relu_backward, sparse_softmax_cross_entropy,
-                         sparse_softmax_cross_entropy_backward, toHip)
+                         sparse_softmax_cross_entropy_backward, sgd_update, toHip)
 
 
 class DemoNet:
@@ -84,24 +84,15 @@ class DemoNet:
         d_pool1, g_k2, g_b2 = conv2d_backward(self.pool1, p["cv2_w"], p["cv2_b"], (0, 0), (1, 1), d_a2)
         d_a1 = maxpool2d_backward(self.a1.shape, self.idx1, d_pool1, **pool)
         d_a1 = relu_backward(d_a1, self.a1)
-        _, g_k1, g_b1 = conv2d_backward(x, p["cv1_w"], p["cv1_b"], (0, 0), (1, 1), d_a1)
+        _, g_k1, g_b1 = conv2d_backward(x, p["cv1_w"], p["cv1_b"], (0, 0), (1, 1), d_a1, need_input_grad=False)
         return loss, dict(cv1_w=g_k1, cv1_b=g_b1, cv2_w=g_k2, cv2_b=g_b2, hidden_w=g_hw, hidden_b=g_hb,
                           classifier_w=g_cw, classifier_b=g_cb)
 
     def sgd_update(self, gradients: dict, learning_rate: float):
-        """The SGD optimizer's update (src/arraymancer/nn/optimizers/optimizers.nim:35-51: x - lr * y over every parameter)
-        as one pass per parameter: value = grad * (-learning_rate) + value, the same two roundings."""
-        step = self._step_tensor(learning_rate)
-        for name, g in gradients.items():
-            w = self.p[name]
-            _ternary_into("muladd", w, g, step.reshape(*([1] * w.rank)).broadcast(w.shape), w)
-
-    def _step_tensor(self, learning_rate: float) -> HipTensor:
-        """-learning_rate as a one-element device tensor, uploaded once per value (an upload cannot be recorded)."""
-        cache = self.__dict__.setdefault("_steps", {})
-        if learning_rate not in cache:
-            cache[learning_rate] = toHip(np.array([-learning_rate], dtype=self.dtype))
-        return cache[learning_rate]
+        """The SGD optimizer's update (src/arraymancer/nn/optimizers/optimizers.nim:35-51: x - lr * y over every
+        parameter) as ONE launch over all eight parameters."""
+        names = list(gradients)
+        sgd_update([self.p[k] for k in names], [gradients[k].reshape(*self.p[k].shape) for k in names], learning_rate)
 
     def gradients(self, x: HipTensor, labels: HipTensor) -> dict:
         """`loss_and_gradients` without the loss: device work only, so that it can be recorded into a graph."""
@@ -110,8 +101,6 @@ class DemoNet:
     def capture_train_step(self, x: HipTensor, labels: HipTensor, learning_rate: float = 0.01) -> Graph:
         """One whole learning step (forward, backward, update; the loss is not read back) as ONE graph over the
         buffers `x` and `labels`: refill them and launch. About forty kernels per replay and no host work in between."""
-        self._step_tensor(learning_rate)
-
         def step():
             self.sgd_update(self.gradients(x, labels), learning_rate)
         before = {k: v.clone() for k, v in self.p.items()}      # the rehearsal and the capture are not steps of the training

@@ -549,7 +549,8 @@ def col2im(col: HipTensor, channels: int, height: int, width: int, kernel_size, 
     return out if batched else out.reshape(channels, height, width)
 
 
-def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None, padding, stride, grad_output: HipTensor):
+def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None, padding, stride, grad_output: HipTensor,
+                    need_input_grad: bool = True):
     """(grad_input, grad_weight, grad_bias) of conv2d_backward (src/arraymancer/nn_primitives/nnp_convolution.nim:65-107)
     over im2colgemm_conv2d_gradient (fallback/conv.nim:107-145). The reference loops over the images (two GEMMs, an
     im2col and a col2im each); here the batch is folded into the columns, g[C_out, N*P] = grad_output with its first
@@ -560,7 +561,8 @@ def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None,
         grad_input  = col2im(kernel_col^T * g)           (one product, one gather)
 
     Float tensors with unit stride and up to 96 input channels take grad_input as ONE launch instead: the convolution
-    of grad_output with the turned kernel. grad_bias is None when `bias` is."""
+    of grad_output with the turned kernel. grad_bias is None when `bias` is; grad_input is None (and not computed) when
+    `need_input_grad` is False: the first layer of a network has no use for the gradient of the images."""
     _same_dtype(input, weight, grad_output)
     N, C, H, W = input.shape
     co, ci, kh, kw = weight.shape
@@ -575,6 +577,8 @@ def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None,
     col = im2col_folded(input, (kh, kw), padding, stride)
     kcol = weight.reshape(co, ci * kh * kw)
     grad_weight = matmul(g, col.transpose()).reshape(co, ci, kh, kw)
+    if not need_input_grad:
+        return None, grad_weight, grad_bias
     if (input.dtype.kind == "f" and tuple(stride) == (1, 1) and padding[0] < kh and padding[1] < kw and C <= 96 and N <= 65535
             and co * kh * kw * input.dtype.itemsize >= 16):
         # With unit stride the gradient is itself a convolution, of grad_output with the kernel turned by 180 degrees and
@@ -663,6 +667,30 @@ def linear_backward(input: HipTensor, weight: HipTensor, gradOutput: HipTensor, 
     if not with_bias:
         return grad_input, grad_weight
     return grad_input, grad_weight, tsum(gradOutput, axis=0)
+
+
+# ---------------------------------------------------------------------- optimizer
+def sgd_update(values, gradients, learning_rate: float):
+    """value -= learning_rate * gradient for every (value, gradient) pair in ONE launch: the update of the SGD optimizer
+    (src/arraymancer/nn/optimizers/optimizers.nim:35-51 runs one apply2_inline per parameter). C-contiguous float
+    tensors of one element type; each gradient has its value's shape."""
+    values, gradients = list(values), list(gradients)
+    if len(values) != len(gradients):
+        raise ValueError("sgd_update: one gradient per value")
+    if not values:
+        return
+    _same_dtype(*values, *gradients)
+    if values[0].dtype.kind != "f":
+        raise TypeError("sgd_update is defined for float tensors")
+    for v, g in zip(values, gradients):
+        if v.shape != g.shape:
+            raise ValueError(f"sgd_update: gradient of shape {g.shape} for a value of shape {v.shape}")
+        if not (v.is_C_contiguous() and g.is_C_contiguous()):
+            raise ValueError("sgd_update: values and gradients must be C-contiguous")
+    n = len(values)
+    ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+    check(getattr(_lib.load(), f"am_hip_sgd_update_{values[0].sfx}")(
+        n, ptrs(values), ptrs(gradients), i64_array([v.size for v in values]), _lib.CTYPE[values[0].sfx](learning_rate)))
 
 
 # ---------------------------------------------------------------------- gated recurrent unit

@@ -606,6 +606,12 @@ int am_hip_gru_gates_backward_f32(int64_t batch, int64_t H, const float* dnext, 
 int am_hip_gru_gates_backward_f64(int64_t batch, int64_t H, const double* dnext, const double* h, const double* r, const double* z,
                                   const double* n, const double* uh, int64_t ld_in, double* dw3x, int64_t ldw, double* du3h, int64_t ldu);
 
+/* values[t][i] <- values[t][i] - learning_rate * grads[t][i] for `count` contiguous tensors of sizes[t] elements in ONE
+ * launch (64 tensors per launch beyond that). Replaces the SGD optimizer's update, one apply2_inline per parameter
+ * (src/arraymancer/nn/optimizers/optimizers.nim:35-51); same expression, the product rounded before the subtraction. */
+int am_hip_sgd_update_f32(int count, float* const* values, const float* const* grads, const int64_t* sizes, float learning_rate);
+int am_hip_sgd_update_f64(int count, double* const* values, const double* const* grads, const int64_t* sizes, double learning_rate);
+
 /* *loss (host) <- (1 / rows) * sum over the rows i of  ln(sum_j exp(input[i, j])) - sum_j input[i, j] * target[i, j]:
  * softmax and cross-entropy in one pass over `input` [rows, cols] and `target` [rows, cols] (probabilities), element
  * strides (rs, cs). Blocking; 0 for an empty batch. Replaces softmax_cross_entropy

@@ -829,3 +829,38 @@ def test_fac(hip, oracle, sfx):
     with pytest.raises(TypeError):
         hip.fac(hip.zeros((2, 2), np.float32))
     assert hip.fac(hip.zeros((0, 3), dt)).shape == (0, 3)
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_sgd_update_of_many_tensors_in_one_launch(hip, sfx):
+    """am_hip_sgd_update_*: value - lr * gradient over a list of tensors (optimizers.nim:35-51 runs one pass per
+    parameter) bit for bit against NumPy's same expression: sizes around the 4096-element pieces and the 16-byte
+    vectors, an empty tensor in the list, more tensors than one launch takes, an unaligned window of a wider buffer."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("sgd", sfx))
+    sizes = [1, 3, 4, 5, 500, 4095, 4096, 4097, 8191, 10, 0, 12289, 400_000] + [int(n) for n in rng.integers(1, 300, 70)]
+    vals = [rng.standard_normal(n).astype(dt) for n in sizes]
+    grads = [rng.standard_normal(n).astype(dt) for n in sizes]
+    dv, dg = [hip.toHip(v) for v in vals], [hip.toHip(g) for g in grads]
+    lr = dt(0.0375)
+    hip.sgd_update(dv, dg, float(lr))
+    for v, g, d, n in zip(vals, grads, dv, sizes):
+        assert np.array_equal(d.toCpu(), v - lr * g), n
+    # 2-D parameters and a window that starts at an odd element
+    w, gw = rng.standard_normal((37, 53)).astype(dt), rng.standard_normal((37, 53)).astype(dt)
+    wide = rng.standard_normal(1001).astype(dt)
+    dwide = hip.toHip(wide)
+    gwin = rng.standard_normal(998).astype(dt)
+    dw = hip.toHip(w)
+    hip.sgd_update([dw, dwide[3:]], [hip.toHip(gw), hip.toHip(gwin)], 0.5)
+    assert np.array_equal(dw.toCpu(), w - dt(0.5) * gw)
+    expect = wide.copy()
+    expect[3:] = wide[3:] - dt(0.5) * gwin
+    assert np.array_equal(dwide.toCpu(), expect)
+    with pytest.raises(ValueError):
+        hip.sgd_update([dw], [hip.toHip(gw.T.copy())], 0.1)                 # shapes differ
+    with pytest.raises(ValueError):
+        hip.sgd_update([dw.transpose()], [hip.toHip(gw).transpose()], 0.1)  # not contiguous
+    with pytest.raises(TypeError):
+        hip.sgd_update([hip.zeros((3,), np.int32)], [hip.zeros((3,), np.int32)], 0.1)
+    hip.sgd_update([], [], 0.1)

@@ -168,7 +168,6 @@ def test_ex02_training_step_as_one_graph(hip):
     graph = replayed.capture_train_step(x, labels, 0.05)
     for name in p:
         assert np.array_equal(replayed.p[name].toCpu(), np.asarray(p[name], dtype=dt).reshape(replayed.p[name].shape)), name
-    eager._step_tensor(0.05)                     # the eager net's own one-element tensor, kept from its first step on
     live0, _ = memory(hip)
     for step in range(4):
         hx, hl = rng.uniform(0, 1, (batch, 1, 28, 28)).astype(dt), rng.integers(0, 10, batch).astype(np.int64)
