@@ -13,7 +13,7 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, softmax_cross_entropy, sparse_softmax_cross_entropy,
                          softmax_cross_entropy_backward, sparse_softmax_cross_entropy_backward, maxpool2d, tanh, relu_backward, sigmoid_backward,
-                         tanh_backward, linear_backward, gru_cell_inference, gru_cell_forward, gru_cell_backward, gru_inference, variance, std, sqrt, square, argmax_max, argmax,
+                         tanh_backward, linear_backward, gru_cell_inference, gru_cell_forward, gru_cell_backward, gru_inference, gru_forward, gru_backward, variance, std, sqrt, square, argmax_max, argmax,
                          argmin_min, argmin, maxpool2d_backward, bc_pow, mreciprocal, clamp, mclamp, UFUNCS, ln, log10, log2, exp,
                          cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, arcsinh, arccosh, arctanh, erf, erfc,
                          gamma, lgamma, floor, ceil, trunc, reciprocal, tround as round, bc_eq, bc_ne, bc_lt, bc_le, bc_gt,
@@ -23,7 +23,7 @@ __all__ = [
     "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
     "toHip", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "im2col_folded", "col2im", "conv2d", "conv2d_into", "conv2d_backward", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
     "unary", "relu", "sigmoid", "bias_relu", "bc_add", "bc_sub", "bc_mul", "bc_div", "bc_mod",
-    "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward", "gru_cell_inference", "gru_cell_forward", "gru_cell_backward", "gru_inference",
+    "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward", "gru_cell_inference", "gru_cell_forward", "gru_cell_backward", "gru_inference", "gru_forward", "gru_backward",
     "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin", "maxpool2d_backward",
     "reduce_axis", "reduce_all", "sum", "product", "min", "max", "mean", "softmax", "maxpool2d", "softmax_cross_entropy", "sparse_softmax_cross_entropy",
     "softmax_cross_entropy_backward", "sparse_softmax_cross_entropy_backward",

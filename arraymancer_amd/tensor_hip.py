@@ -793,6 +793,89 @@ def gru_inference(input: HipTensor, W3s0: HipTensor, W3sN: HipTensor | None, U3s
     return output
 
 
+def _gru_layer_weights(layer, W3s0, W3sN, U3s, bW3s=None, bU3s=None):
+    W3l = W3s0 if layer == 0 else W3sN[layer - 1].squeeze(0)
+    out = [W3l, U3s[layer].squeeze(0)]
+    if bW3s is not None:
+        out += [bW3s[layer].squeeze(0), bU3s[layer].squeeze(0)]
+    return out
+
+
+def gru_forward(input: HipTensor, W3s0: HipTensor, W3sN: HipTensor | None, U3s: HipTensor, bW3s: HipTensor, bU3s: HipTensor,
+                hidden: HipTensor):
+    """gru_forward (nnp_gru.nim:263-374): gru_inference that keeps what gru_backward needs. Returns (output, cache);
+    `hidden` [layers, batch, H] is updated in place. The cache holds, per layer, the layer's input [T, batch, features]
+    and, time-major [T, batch, H], the hidden state before every step and the r, z, n, Uh of every step (the reference
+    keeps the same values as seq[Tensor] / [layers, T, batch, H] tensors)."""
+    T, B, F = input.shape
+    H = hidden.shape[2]
+    layers = 1 + (W3sN.shape[0] if W3sN is not None and W3sN.size else 0)
+    if hidden.shape != (layers, B, H) or W3s0.shape != (3 * H, F) or U3s.shape != (layers, 3 * H, H) or \
+            bW3s.shape != (layers, 1, 3 * H) or bU3s.shape != bW3s.shape or (layers > 1 and W3sN.shape != (layers - 1, 3 * H, H)):
+        raise ValueError("gru_forward: shapes of the weights, biases and hidden state do not fit the input")
+    output = empty((T, B, H), input.dtype)
+    cache = []
+    for layer in range(layers):
+        W3l, U3l, bW3l, bU3l = _gru_layer_weights(layer, W3s0, W3sN, U3s, bW3s, bU3s)
+        src = input if layer == 0 else output.clone()
+        W3x_all = linear(src.reshape(T * B, src.shape[2]), W3l, bW3l).reshape(T, B, 3 * H)
+        h_l = hidden[layer].squeeze(0)
+        hs, r, z, n, Uh = (empty((T, B, H), input.dtype) for _ in range(5))
+        for t in range(T):
+            _unary_into("copy", hs[t].squeeze(0), h_l)
+            keep = tuple(a[t].squeeze(0) for a in (r, z, n, Uh))
+            _gru_gates_inplace(W3x_all[t].squeeze(0), linear(h_l, U3l, bU3l), h_l, keep)
+            _unary_into("copy", output[t].squeeze(0), h_l)
+        cache.append(dict(input=src, hiddens=hs, r=r, z=z, n=n, Uh=Uh))
+    return output, cache
+
+
+def gru_backward(dOutput: HipTensor, dHiddenN: HipTensor, cache, W3s0: HipTensor, W3sN: HipTensor | None, U3s: HipTensor):
+    """gru_backward (nnp_gru.nim:376-500): (dInput, dHidden0, dW3s0, dW3sN, dU3s, dbW3s, dbU3s) from the gradients of the
+    output [T, batch, H] and of the last hidden state [layers, batch, H]. Only the recurrence is walked step by step
+    (per step the one-launch gate gradients, one product with U3 and dh + dnext * z); the gradients of the weights, biases
+    and of the layer's input are taken over all timesteps at once afterwards - four products and two column sums per
+    layer where the reference accumulates four products per step (the same sums in another order)."""
+    layers = len(cache)
+    T, B, H = cache[0]["r"].shape
+    dt = dOutput.dtype
+    if dOutput.shape != (T, B, H) or dHiddenN.shape != (layers, B, H):
+        raise ValueError("gru_backward: gradients of shape [T, batch, H] and [layers, batch, H] expected")
+    gflow = dOutput.clone()
+    dHidden0 = empty((layers, B, H), dt)
+    dW3sN = empty(W3sN.shape, dt) if layers > 1 else None
+    dU3s, dbW3s, dbU3s = empty(U3s.shape, dt), empty((layers, 1, 3 * H), dt), empty((layers, 1, 3 * H), dt)
+    dInput = dW3s0 = None
+    for layer in range(layers - 1, -1, -1):
+        W3l, U3l = _gru_layer_weights(layer, W3s0, W3sN, U3s)
+        c = cache[layer]
+        dW3x_all, dU3h_all = empty((T, B, 3 * H), dt), empty((T, B, 3 * H), dt)
+        dht1 = dHiddenN[layer].squeeze(0).clone()
+        for t in range(T - 1, -1, -1):
+            apply2("add", dht1, gflow[t].squeeze(0))
+            saved = (dht1,) + tuple(c[k][t].squeeze(0) for k in ("hiddens", "r", "z", "n", "Uh"))
+            check(getattr(_lib.load(), f"am_hip_gru_gates_backward_{saved[0].sfx}")(
+                B, H, *[ctypes.c_void_p(a.data_ptr()) for a in saved], H,
+                ctypes.c_void_p(dW3x_all[t].data_ptr()), 3 * H, ctypes.c_void_p(dU3h_all[t].data_ptr()), 3 * H))
+            dh = matmul(dU3h_all[t].squeeze(0), U3l)
+            _ternary_into("muladd", dh, dht1, c["z"][t].squeeze(0), dh)
+            dht1 = dh
+        _unary_into("copy", dHidden0[layer].squeeze(0), dht1)
+        X = c["input"].reshape(T * B, c["input"].shape[2])
+        G, GU = dW3x_all.reshape(T * B, 3 * H), dU3h_all.reshape(T * B, 3 * H)
+        dx_all = matmul(G, W3l)
+        dW3 = matmul(G.transpose(), X)
+        if layer == 0:
+            dInput, dW3s0 = dx_all.reshape(T, B, X.shape[1]), dW3
+        else:
+            gflow = dx_all.reshape(T, B, H)
+            _unary_into("copy", dW3sN[layer - 1].squeeze(0), dW3)
+        gemm(1, GU.transpose(), c["hiddens"].reshape(T * B, H), 0, dU3s[layer].squeeze(0))
+        reduce_axis_into("sum", dbW3s[layer].squeeze(0), G, 0)
+        reduce_axis_into("sum", dbU3s[layer].squeeze(0), GU, 0)
+    return dInput, dHidden0, dW3s0, dW3sN, dU3s, dbW3s, dbU3s
+
+
 # ---------------------------------------------------------------------- element-wise
 def _binary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor):
     sfx = dst.sfx

@@ -219,3 +219,64 @@ def test_fused_backward_gates_equal_the_separate_passes(hip, dt):
         dWzx, dWrx = z * (one - z) * dz, r * (one - r) * dr
         assert np.array_equal(want_w.toCpu(), np.concatenate([dWrx, dWzx, dWx], 1))
         assert np.array_equal(want_u.toCpu(), np.concatenate([dWrx, dWzx, dUh], 1))
+
+
+def oracle_gru(oracle, x, W3s0, W3sN, U3s, bW3s, bU3s, hidden):
+    """gru_inference (nnp_gru.nim:194-262) cell by cell through the oracle's operators; returns (output, hiddenN)."""
+    T = x.shape[0]
+    layers = U3s.shape[0]
+    h = hidden.copy()
+    out = np.empty((T, x.shape[1], hidden.shape[2]), dtype=x.dtype)
+    for layer in range(layers):
+        W3l = W3s0 if layer == 0 else W3sN[layer - 1]
+        for t in range(T):
+            src = np.ascontiguousarray(x[t] if layer == 0 else out[t])
+            h[layer] = oracle_cell(oracle, src, W3l, U3s[layer], bW3s[layer], bU3s[layer], np.ascontiguousarray(h[layer]))[0]
+            out[t] = h[layer]
+    return out, h
+
+
+@pytest.mark.parametrize("layers,T", [(1, 1), (1, 4), (2, 1), (2, 3), (3, 2)])
+def test_sequence_forward_and_backward(hip, oracle, layers, T):
+    """gru_forward / gru_backward (nnp_gru.nim:263-500) the way the reference checks them (test_nnp_gru.nim:295-470):
+    forward equal to the inference pass, and every gradient against central differences of
+    sum(wo * output) + sum(wh * hiddenN) through the inference pass, float64, for stacks of one to three layers."""
+    B, F, H = 3, 4, 2
+    rng = np.random.default_rng(seed_of("gru-seq", layers, T))
+    u = lambda *s: rng.uniform(0, 1, s)
+    x, hidden = u(T, B, F), u(layers, B, H)
+    W3s0, W3sN, U3s = u(3 * H, F), u(max(layers - 1, 0), 3 * H, H), u(layers, 3 * H, H)
+    bW3s, bU3s = u(layers, 1, 3 * H), u(layers, 1, 3 * H)
+    wo, wh = u(T, B, H), u(layers, B, H)                   # the gradients flowing back
+    say("gru sequence", layers, "layers", T, "steps")
+    dev = lambda a: hip.toHip(a)
+    dWN = dev(W3sN) if layers > 1 else None
+    h = dev(hidden)
+    out, cache = hip.gru_forward(dev(x), dev(W3s0), dWN, dev(U3s), dev(bW3s), dev(bU3s), h)
+    want_out, want_h = oracle_gru(oracle, x, W3s0, W3sN, U3s, bW3s, bU3s, hidden)
+    assert np.max(np.abs(out.toCpu() - want_out)) < 1e-12 and np.max(np.abs(h.toCpu() - want_h)) < 1e-12
+    h2 = dev(hidden)
+    assert np.max(np.abs(hip.gru_inference(dev(x), dev(W3s0), dWN, dev(U3s), dev(bW3s), dev(bU3s), h2).toCpu() - out.toCpu())) < 1e-13
+    grads = hip.gru_backward(dev(wo), dev(wh), cache, dev(W3s0), dWN, dev(U3s))
+    params = dict(dInput=x, dHidden0=hidden, dW3s0=W3s0, dW3sN=W3sN, dU3s=U3s, dbW3s=bW3s, dbU3s=bU3s)
+
+    def objective():
+        o, hn = oracle_gru(oracle, x, W3s0, W3sN, U3s, bW3s, bU3s, hidden)
+        return float(np.sum(wo * o) + np.sum(wh * hn))
+
+    for got, (name, arr) in zip(grads, params.items()):
+        if arr.size == 0:
+            assert got is None, name
+            continue
+        assert got.shape == arr.shape, name
+        num = np.zeros_like(arr)
+        flat, nf = arr.reshape(-1), num.reshape(-1)
+        for i in range(flat.size):
+            keep = flat[i]
+            flat[i] = keep + 1e-5; up = objective()
+            flat[i] = keep - 1e-5; dn = objective()
+            flat[i] = keep
+            nf[i] = (up - dn) / 2e-5
+        err = np.mean(np.abs(got.toCpu() - num))
+        say(f"  {name}: mean absolute error against the numerical gradient {err:.2e}")
+        assert err < 1e-8, name
