@@ -12,7 +12,8 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          bc_sub, bias_relu, conv2d, conv2d_into, conv2d_backward, col2im, im2col_folded, dot, empty, gemm, gemm_batched, gemv, im2col, linear, map2, matmul, relu, scalar_op,
                          sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, softmax_cross_entropy, sparse_softmax_cross_entropy,
-                         softmax_cross_entropy_backward, sparse_softmax_cross_entropy_backward, maxpool2d, tanh, relu_backward, sigmoid_backward,
+                         softmax_cross_entropy_backward, sparse_softmax_cross_entropy_backward, sigmoid_cross_entropy,
+                         sigmoid_cross_entropy_backward, maxpool2d, tanh, relu_backward, sigmoid_backward,
                          tanh_backward, linear_backward, gru_cell_inference, gru_cell_forward, gru_cell_backward, gru_inference, gru_forward, gru_backward, variance, std, sqrt, square, argmax_max, argmax,
                          argmin_min, argmin, maxpool2d_backward, bc_pow, mreciprocal, clamp, mclamp, UFUNCS, ln, log10, log2, exp,
                          cbrt, sin, cos, tan, sinh, cosh, arcsin, arccos, arctan, arcsinh, arccosh, arctanh, erf, erfc,
@@ -26,7 +27,7 @@ __all__ = [
     "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward", "gru_cell_inference", "gru_cell_forward", "gru_cell_backward", "gru_inference", "gru_forward", "gru_backward",
     "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin", "maxpool2d_backward",
     "reduce_axis", "reduce_all", "sum", "product", "min", "max", "mean", "softmax", "maxpool2d", "softmax_cross_entropy", "sparse_softmax_cross_entropy",
-    "softmax_cross_entropy_backward", "sparse_softmax_cross_entropy_backward",
+    "softmax_cross_entropy_backward", "sparse_softmax_cross_entropy_backward", "sigmoid_cross_entropy", "sigmoid_cross_entropy_backward",
     "bc_pow", "mreciprocal", "clamp", "mclamp", "UFUNCS", "ln", "log10", "log2", "exp", "cbrt", "sin", "cos", "tan", "sinh", "cosh",
     "arcsin", "arccos", "arctan", "arcsinh", "arccosh", "arctanh", "erf", "erfc", "gamma", "lgamma", "floor", "ceil",
     "trunc", "reciprocal", "round",

@@ -110,6 +110,8 @@ def _signatures():
             sig[f"am_hip_gru_gates_{sfx}"] = (ci, [i64, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, i64])
             sig[f"am_hip_gru_gates_backward_{sfx}"] = (ci, [i64, i64, vp, vp, vp, vp, vp, vp, i64, vp, i64, vp, i64])
             sig[f"am_hip_softmax_cross_entropy_{sfx}"] = (ci, [i64, i64, vp, i64, i64, vp, i64, i64, ctypes.POINTER(ct)])
+            sig[f"am_hip_sigmoid_cross_entropy_{sfx}"] = (ci, [i64, i64, vp, i64, i64, vp, i64, i64, ctypes.POINTER(ct)])
+            sig[f"am_hip_sigmoid_cross_entropy_backward_{sfx}"] = (ci, [i64, i64, ct, vp, i64, i64, vp, i64, i64, vp, i64, i64])
             sig[f"am_hip_sparse_softmax_cross_entropy_{sfx}"] = (ci, [i64, i64, vp, i64, i64, vp, i64, ctypes.POINTER(ct)])
             sig[f"am_hip_softmax_cross_entropy_backward_{sfx}"] = (ci, [i64, i64, ct, vp, i64, i64, vp, i64, i64, vp, i64, i64])
             sig[f"am_hip_sparse_softmax_cross_entropy_backward_{sfx}"] = (ci, [i64, i64, ct, vp, i64, i64, vp, i64, vp, i64, i64])

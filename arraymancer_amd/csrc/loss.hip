@@ -1,5 +1,6 @@
 // Softmax + cross-entropy fused, forward and backward: am_hip_softmax_cross_entropy_*,
-// am_hip_sparse_softmax_cross_entropy_* and their _backward forms
+// am_hip_sparse_softmax_cross_entropy_* and their _backward forms; sigmoid + cross-entropy likewise
+// (am_hip_sigmoid_cross_entropy_*, src/arraymancer/nn_primitives/nnp_sigmoid_cross_entropy.nim:23-62)
 // (src/arraymancer/nn_primitives/nnp_softmax_cross_entropy.nim:17-86, 88-177, 186-214, 217-256).
 //
 // The reference walks each row once with a running maximum and a sum of exp(x - maximum) that is rescaled whenever
@@ -202,6 +203,50 @@ __global__ __launch_bounds__(256) void sce_backward(Args<T> p, int lanes) {
   }
 }
 
+// Sigmoid + cross-entropy (nnp_sigmoid_cross_entropy.nim:23-45): the map2 body -y * x + max(x, 0) + ln1p(exp(-|x|)) summed
+// over every element, divided by the batch size. One lane per 8 elements of the C-order traversal (any strides), the
+// workgroup's 2048 terms folded through LDS into one partial; the partials are then added like the rows' losses above.
+template <typename T> __device__ __forceinline__ T dev_log1p(T v);
+template <> __device__ __forceinline__ float dev_log1p<float>(float v) { return log1pf(v); }
+template <> __device__ __forceinline__ double dev_log1p<double>(double v) { return log1p(v); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_ce_partial(Args<T> p, T* __restrict__ partial) {
+  __shared__ T part[256];
+  const int64_t total = p.rows * p.cols;
+  T acc = (T)0;
+  const int64_t base = (int64_t)blockIdx.x * 2048 + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int64_t i = base + (int64_t)u * 256;
+    if (i < total) {
+      const int64_t r = i / p.cols, c = i - r * p.cols;
+      const T x = p.x[r * p.x_rs + c * p.x_cs], y = p.target[r * p.t_rs + c * p.t_cs];
+      const T ax = x < (T)0 ? -x : x;
+      acc += -y * x + (x > (T)0 ? x : (T)0) + dev_log1p<T>(dev_exp<T>(-ax));
+    }
+  }
+  part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int d = 128; d >= 1; d >>= 1) {
+    if ((int)threadIdx.x < d) part[threadIdx.x] += part[threadIdx.x + d];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partial[blockIdx.x] = part[0];
+}
+
+// grad * (sigmoid(x) - y) / batch_size (nnp_sigmoid_cross_entropy.nim:47-62), sigmoid = 1 / (1 + exp(-x)).
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_ce_backward(Args<T> p) {
+  const int64_t total = p.rows * p.cols;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / p.cols, c = i - r * p.cols;
+    const T x = p.x[r * p.x_rs + c * p.x_cs], y = p.target[r * p.t_rs + c * p.t_cs];
+    const T sg = (T)1 / ((T)1 + dev_exp<T>(-x));
+    p.out[r * p.o_rs + c * p.o_cs] = p.grad * (sg - y) / p.batch;
+  }
+}
+
 // Whether the rows can be walked in 16-byte vectors: unit stride along the row, whole vectors, aligned row starts.
 template <typename T>
 static bool vec_ok(const Args<T>& p, bool dense, bool with_out) {
@@ -286,6 +331,56 @@ static int backward(const char* fn, int64_t rows, int64_t cols, T gradient, cons
   return check_launch("sce_backward");
 }
 
+template <typename T>
+static int sigmoid_forward(const char* fn, int64_t rows, int64_t cols, const T* x, int64_t x_rs, int64_t x_cs, const T* target,
+                           int64_t t_rs, int64_t t_cs, T* loss) {
+  if (!loss) return fail(AM_E_ARG, "%s: null result pointer", fn);
+  if (rows < 0 || cols < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+  if (rows == 0) return fail(AM_E_SHAPE, "%s: empty batch (the reference divides by the batch size)", fn);
+  if (cols == 0) { *loss = (T)0; return AM_OK; }
+  if (!x || !target) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  if (capturing()) return fail(AM_E_ARG, "%s: returns a value to the host, not allowed while a graph is being captured", fn);
+  const int64_t total = rows * cols, blocks = (total + 2047) / 2048;
+  if (blocks >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "%s: too many elements", fn);
+  char* ws = (char*)gemm::splitk_workspace(256 + ((size_t)blocks + (size_t)blocks / 4096 + 16) * sizeof(T));
+  if (!ws) return fail(AM_E_ALLOC, "%s: workspace unavailable", fn);
+  Args<T> p = {};
+  p.x = x; p.x_rs = x_rs; p.x_cs = x_cs; p.target = target; p.t_rs = t_rs; p.t_cs = t_cs; p.rows = rows; p.cols = cols;
+  T* partial = (T*)(ws + 256);
+  hipLaunchKernelGGL((sigmoid_ce_partial<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), p, partial);
+  AM_TRY(check_launch("sigmoid_ce_partial"));
+  const T* v = partial;
+  int64_t n = blocks;
+  T* spare = partial + blocks;
+  while (n > 8192) {
+    const int64_t slices = (n + 8191) / 8192;
+    hipLaunchKernelGGL((sum_slices<T>), dim3((unsigned)slices), dim3(256), 0, stream(), v, n, (int64_t)8192, (T)1, spare);
+    AM_TRY(check_launch("sum_slices"));
+    v = spare; n = slices; spare += slices;
+  }
+  hipLaunchKernelGGL((sum_slices<T>), dim3(1), dim3(256), 0, stream(), v, n, n, (T)1 / (T)rows, (T*)ws);
+  AM_TRY(check_launch("sum_slices"));
+  return fetch_result(loss, ws, sizeof(T));
+}
+
+template <typename T>
+static int sigmoid_backward(const char* fn, int64_t rows, int64_t cols, T gradient, const T* x, int64_t x_rs, int64_t x_cs,
+                            const T* target, int64_t t_rs, int64_t t_cs, T* out, int64_t o_rs, int64_t o_cs) {
+  if (rows < 0 || cols < 0) return fail(AM_E_SHAPE, "%s: negative extent", fn);
+  if (rows == 0 || cols == 0) return AM_OK;
+  if (!x || !target || !out) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  AM_TRY(ensure_init());
+  Args<T> p = {};
+  p.x = x; p.x_rs = x_rs; p.x_cs = x_cs; p.target = target; p.t_rs = t_rs; p.t_cs = t_cs; p.rows = rows; p.cols = cols;
+  p.out = out; p.o_rs = o_rs; p.o_cs = o_cs; p.grad = gradient; p.batch = (T)rows;
+  int64_t blocks = (rows * cols + 255) / 256;
+  const int64_t cap = (int64_t)num_cus() * 32;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL((sigmoid_ce_backward<T>), dim3((unsigned)blocks), dim3(256), 0, stream(), p);
+  return check_launch("sigmoid_ce_backward");
+}
+
 }  // namespace loss
 }  // namespace am
 
@@ -314,5 +409,18 @@ using namespace am;
     return loss::backward<T, false>("am_hip_sparse_softmax_cross_entropy_backward_" #SFX, rows, cols, gradient, input, in_rs, \
                                     in_cs, nullptr, 0, 0, labels, labels_s, result, r_rs, r_cs);                            \
   }
+#define AM_SIGMOID_CE_ENTRY_POINTS(T, SFX)                                                                                   \
+  extern "C" int am_hip_sigmoid_cross_entropy_##SFX(int64_t rows, int64_t cols, const T* input, int64_t in_rs, int64_t in_cs, \
+                                                    const T* target, int64_t t_rs, int64_t t_cs, T* loss) {                 \
+    return loss::sigmoid_forward<T>("am_hip_sigmoid_cross_entropy_" #SFX, rows, cols, input, in_rs, in_cs, target, t_rs, t_cs, loss); \
+  }                                                                                                                         \
+  extern "C" int am_hip_sigmoid_cross_entropy_backward_##SFX(int64_t rows, int64_t cols, T gradient, const T* input,        \
+                                                             int64_t in_rs, int64_t in_cs, const T* target, int64_t t_rs,   \
+                                                             int64_t t_cs, T* result, int64_t r_rs, int64_t r_cs) {        \
+    return loss::sigmoid_backward<T>("am_hip_sigmoid_cross_entropy_backward_" #SFX, rows, cols, gradient, input, in_rs, in_cs, \
+                                     target, t_rs, t_cs, result, r_rs, r_cs);                                               \
+  }
+AM_SIGMOID_CE_ENTRY_POINTS(float, f32)
+AM_SIGMOID_CE_ENTRY_POINTS(double, f64)
 AM_LOSS_ENTRY_POINTS(float, f32)
 AM_LOSS_ENTRY_POINTS(double, f64)

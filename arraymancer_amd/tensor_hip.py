@@ -1438,6 +1438,30 @@ def sparse_softmax_cross_entropy(input: HipTensor, target: HipTensor) -> float:
     return input.dtype.type(loss.value)
 
 
+def sigmoid_cross_entropy(input: HipTensor, target: HipTensor) -> float:
+    """Sigmoid + binary cross-entropy in one pass, averaged over the batch
+    (src/arraymancer/nn_primitives/nnp_sigmoid_cross_entropy.nim:23-45)."""
+    _check_input_target(input, target, False)
+    if input.shape[0] == 0:
+        raise ValueError("sigmoid_cross_entropy: empty batch")
+    loss = _lib.CTYPE[input.sfx]()
+    check(getattr(_lib.load(), f"am_hip_sigmoid_cross_entropy_{input.sfx}")(
+        input.shape[0], input.shape[1], ctypes.c_void_p(input.data_ptr()), *input.strides,
+        ctypes.c_void_p(target.data_ptr()), *target.strides, ctypes.byref(loss)))
+    return input.dtype.type(loss.value)
+
+
+def sigmoid_cross_entropy_backward(gradient, cached_tensor: HipTensor, target: HipTensor) -> HipTensor:
+    """gradient * (sigmoid(cached_tensor) - target) / batch_size (nnp_sigmoid_cross_entropy.nim:47-62)."""
+    _check_input_target(cached_tensor, target, False)
+    out = empty(cached_tensor.shape, cached_tensor.dtype)
+    check(getattr(_lib.load(), f"am_hip_sigmoid_cross_entropy_backward_{cached_tensor.sfx}")(
+        cached_tensor.shape[0], cached_tensor.shape[1], _lib.CTYPE[cached_tensor.sfx](_scalar_gradient(gradient, cached_tensor.dtype)),
+        ctypes.c_void_p(cached_tensor.data_ptr()), *cached_tensor.strides, ctypes.c_void_p(target.data_ptr()), *target.strides,
+        ctypes.c_void_p(out.data_ptr()), *out.strides))
+    return out
+
+
 def _scalar_gradient(gradient, dtype):
     """The reference takes the upstream gradient as a scalar or as a one-element tensor (its first element is used)."""
     if isinstance(gradient, HipTensor):

@@ -647,6 +647,23 @@ int am_hip_sparse_softmax_cross_entropy_backward_f64(int64_t rows, int64_t cols,
                                                      int64_t in_rs, int64_t in_cs, const int64_t* labels, int64_t labels_s,
                                                      double* result, int64_t r_rs, int64_t r_cs);
 
+/* *loss (host) <- (1 / rows) * sum over all elements of  -target * input + max(input, 0) + ln1p(exp(-|input|)): sigmoid and
+ * binary cross-entropy in one pass over `input` and `target` [rows, cols] (element strides rs, cs), the terms added in a
+ * fixed order. Blocking. Replaces sigmoid_cross_entropy (src/arraymancer/nn_primitives/nnp_sigmoid_cross_entropy.nim:23-45:
+ * a map2_inline followed by sum). */
+int am_hip_sigmoid_cross_entropy_f32(int64_t rows, int64_t cols, const float* input, int64_t in_rs, int64_t in_cs,
+                                     const float* target, int64_t t_rs, int64_t t_cs, float* loss);
+int am_hip_sigmoid_cross_entropy_f64(int64_t rows, int64_t cols, const double* input, int64_t in_rs, int64_t in_cs,
+                                     const double* target, int64_t t_rs, int64_t t_cs, double* loss);
+/* result[i, j] <- gradient * (sigmoid(input[i, j]) - target[i, j]) / rows. Replaces sigmoid_cross_entropy_backward
+ * (nnp_sigmoid_cross_entropy.nim:47-62) with a scalar gradient. */
+int am_hip_sigmoid_cross_entropy_backward_f32(int64_t rows, int64_t cols, float gradient, const float* input, int64_t in_rs,
+                                              int64_t in_cs, const float* target, int64_t t_rs, int64_t t_cs,
+                                              float* result, int64_t r_rs, int64_t r_cs);
+int am_hip_sigmoid_cross_entropy_backward_f64(int64_t rows, int64_t cols, double gradient, const double* input, int64_t in_rs,
+                                              int64_t in_cs, const double* target, int64_t t_rs, int64_t t_cs,
+                                              double* result, int64_t r_rs, int64_t r_cs);
+
 /* Max pooling of a C-contiguous [N, C, H, W] input into a C-contiguous [N, C, outH, outW] output,
  * outH = (H + 2 padH - kH) / strideH + 1 (outW alike), plus, when argmax != NULL, the flat input
  * index of each maximum (what maxpool2d_backward scatters through). Same window scan order,

@@ -154,6 +154,10 @@ proc am_hip_gru_gates_backward_f32*(batch, H: int64, dnext, h, r, z, n, uh: ptr 
 proc am_hip_gru_gates_backward_f64*(batch, H: int64, dnext, h, r, z, n, uh: ptr cdouble, ld_in: int64, dw3x: ptr cdouble, ldw: int64, du3h: ptr cdouble, ldu: int64): cint {.importc.}
 proc am_hip_sgd_update_f32*(count: cint, values: ptr ptr cfloat, grads: ptr ptr cfloat, sizes: ptr int64, learning_rate: cfloat): cint {.importc.}
 proc am_hip_sgd_update_f64*(count: cint, values: ptr ptr cdouble, grads: ptr ptr cdouble, sizes: ptr int64, learning_rate: cdouble): cint {.importc.}
+proc am_hip_sigmoid_cross_entropy_f32*(rows, cols: int64, input: ptr cfloat, in_rs, in_cs: int64, target: ptr cfloat, t_rs, t_cs: int64, loss: ptr cfloat): cint {.importc.}
+proc am_hip_sigmoid_cross_entropy_backward_f32*(rows, cols: int64, gradient: cfloat, input: ptr cfloat, in_rs, in_cs: int64, target: ptr cfloat, t_rs, t_cs: int64, res: ptr cfloat, r_rs, r_cs: int64): cint {.importc.}
+proc am_hip_sigmoid_cross_entropy_f64*(rows, cols: int64, input: ptr cdouble, in_rs, in_cs: int64, target: ptr cdouble, t_rs, t_cs: int64, loss: ptr cdouble): cint {.importc.}
+proc am_hip_sigmoid_cross_entropy_backward_f64*(rows, cols: int64, gradient: cdouble, input: ptr cdouble, in_rs, in_cs: int64, target: ptr cdouble, t_rs, t_cs: int64, res: ptr cdouble, r_rs, r_cs: int64): cint {.importc.}
 proc am_hip_softmax_cross_entropy_f32*(rows, cols: int64, input: ptr cfloat, in_rs, in_cs: int64, target: ptr cfloat, t_rs, t_cs: int64, loss: ptr cfloat): cint {.importc.}
 proc am_hip_sparse_softmax_cross_entropy_f32*(rows, cols: int64, input: ptr cfloat, in_rs, in_cs: int64, labels: ptr int64, labels_s: int64, loss: ptr cfloat): cint {.importc.}
 proc am_hip_softmax_cross_entropy_backward_f32*(rows, cols: int64, gradient: cfloat, input: ptr cfloat, in_rs, in_cs: int64, target: ptr cfloat, t_rs, t_cs: int64, res: ptr cfloat, r_rs, r_cs: int64): cint {.importc.}

@@ -530,6 +530,25 @@ def sparse_softmax_cross_entropy_backward(gradient, x: np.ndarray, labels: np.nd
     return ((dt(gradient) * (sm + start)).astype(x.dtype) / dt(x.shape[0])).astype(x.dtype)
 
 
+def sigmoid_cross_entropy(x: np.ndarray, target: np.ndarray):
+    """sigmoid_cross_entropy (src/arraymancer/nn_primitives/nnp_sigmoid_cross_entropy.nim:23-45): the map2 body
+    -y * x + max(x, 0) + ln1p(exp(-|x|)) in the element type, summed in C order, divided by the batch size."""
+    dt = x.dtype.type
+    body = (-target * x + np.maximum(x, dt(0)) + np.log1p(np.exp(-np.abs(x)))).astype(x.dtype)
+    total = dt(0)
+    for v in body.reshape(-1):
+        total = dt(total + v)
+    return dt(total / dt(x.shape[0]))
+
+
+def sigmoid_cross_entropy_backward(gradient, x: np.ndarray, target: np.ndarray) -> np.ndarray:
+    """sigmoid_cross_entropy_backward (nnp_sigmoid_cross_entropy.nim:47-62): grad * (sigmoid(x) - y) / batch_size with
+    sigmoid(x) = 1 / (1 + exp(-x)) (nn_primitives/private/p_activation.nim:17-18)."""
+    dt = x.dtype.type
+    sg = (dt(1) / (dt(1) + np.exp(-x))).astype(x.dtype)
+    return ((dt(gradient) * (sg - target)).astype(x.dtype) / dt(x.shape[0])).astype(x.dtype)
+
+
 def maxpool2d(x: np.ndarray, kernel, padding=(0, 0), stride=(1, 1)):
     """nnp_maxpooling.nim:19-66: (max_indices [N*C*outH*outW] int64, maxpooled [N, C, outH, outW])."""
     sfx = _sfx(x)

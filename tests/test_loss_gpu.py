@@ -161,3 +161,42 @@ def test_edge_cases_and_errors(hip):
         hip.sparse_softmax_cross_entropy(hip.zeros((2, 3), f32), hip.toHip(np.zeros(2, np.int32)))
     with pytest.raises((TypeError, ValueError)):
         hip.softmax_cross_entropy(hip.zeros((2, 3), np.int32), hip.zeros((2, 3), np.int32))
+
+
+@pytest.mark.parametrize("sfx", FLT)
+def test_sigmoid_cross_entropy(hip, oracle, sfx):
+    """sigmoid_cross_entropy and its backward form (nnp_sigmoid_cross_entropy.nim:23-62; no vector in the reference's
+    tests: pinned on the definition of binary cross-entropy in extended precision) on small, ragged, large and strided
+    operands: loss within 4e-6 / 1e-13 of the definition relative to max(1, |loss|), gradient entries within 2e-6 / 1e-14,
+    and both against the oracle's restatement where its serial sum is short."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("sigmoid-ce-gpu", sfx))
+    for rows, cols in ((1, 1), (7, 10), (64, 33), (1000, 17), (513, 2049), (4096, 1000)):
+        say("sigmoid cross-entropy", sfx, rows, cols)
+        x = (rng.standard_normal((rows, cols)) * 3).astype(dt)
+        y = rng.uniform(0, 1, (rows, cols)).astype(dt)
+        dx, dy = hip.toHip(x), hip.toHip(y)
+        xl, yl = x.astype(np.longdouble), y.astype(np.longdouble)
+        s = 1 / (1 + np.exp(-xl))
+        exact = float(np.sum(-(yl * np.log(s) + (1 - yl) * np.log1p(-s))) / rows)
+        got = hip.sigmoid_cross_entropy(dx, dy)
+        assert isinstance(got, dt) and abs(got - exact) <= LOSS_TOL[sfx] * max(1.0, abs(exact)), (rows, cols, got, exact)
+        if rows * cols <= 20000:
+            want = oracle.sigmoid_cross_entropy(x, y)
+            assert abs(got - want) <= LOSS_TOL[sfx] * max(1.0, abs(want)) * 4, (rows, cols)
+        g = hip.sigmoid_cross_entropy_backward(dt(1.3), dx, dy).toCpu()
+        assert np.max(np.abs(g - np.longdouble(1.3) * (s - yl) / rows)) <= GRAD_TOL[sfx] * 1.3, (rows, cols)
+        if rows * cols <= 20000:
+            assert np.max(np.abs(g - oracle.sigmoid_cross_entropy_backward(dt(1.3), x, y))) <= GRAD_TOL[sfx] * 1.3
+    # transposed operands: the same value and gradient as their contiguous copies
+    x, y = (rng.standard_normal((37, 21)) * 2).astype(dt), rng.uniform(0, 1, (37, 21)).astype(dt)
+    base = hip.sigmoid_cross_entropy(hip.toHip(x), hip.toHip(y))
+    xt, yt = hip.toHip(np.ascontiguousarray(x.T)).transpose(), hip.toHip(np.ascontiguousarray(y.T)).transpose()
+    assert hip.sigmoid_cross_entropy(xt, yt) == base
+    assert np.array_equal(hip.sigmoid_cross_entropy_backward(1.0, xt, yt).toCpu(), hip.sigmoid_cross_entropy_backward(1.0, hip.toHip(x), hip.toHip(y)).toCpu())
+    big = hip.toHip(np.array([[1000.0, -1000.0]], dtype=dt))
+    assert hip.sigmoid_cross_entropy(big, hip.toHip(np.array([[1.0, 0.0]], dtype=dt))) == 0
+    with pytest.raises(ValueError):
+        hip.sigmoid_cross_entropy(hip.zeros((2, 3), dt), hip.zeros((3, 2), dt))
+    with pytest.raises(ValueError):
+        hip.sigmoid_cross_entropy(hip.zeros((0, 3), dt), hip.zeros((0, 3), dt))

@@ -305,3 +305,38 @@ def test_cross_entropy_closed_forms_and_gradients(oracle, sfx):
     # ln(sumexp) + max is rounded at the magnitude of the scores before the score of the true class is subtracted
     assert np.isfinite(v) and abs(v - _exact_sce(big, np.array([[1, 0, 0], [0, 0, 1]], dtype=dt))) <= np.finfo(dt).eps * 1000 * 2
     assert oracle.softmax_cross_entropy(np.zeros((0, 4), dtype=dt), np.zeros((0, 4), dtype=dt)) == 0
+
+
+@pytest.mark.parametrize("sfx", ["f32", "f64"])
+def test_sigmoid_cross_entropy_closed_forms(oracle, sfx):
+    """No vector in the reference's tests: the restated body -y x + max(x, 0) + ln1p(exp(-|x|)) against the definition of
+    binary cross-entropy, -(y ln s + (1 - y) ln(1 - s)) with s = sigmoid(x), in extended precision (they are the same
+    function; the body is the overflow-free form), ln 2 at x = 0, no overflow at +-1000, and the backward form against
+    (s - y) / batch and central differences of the loss."""
+    dt = DTYPES[sfx]
+    rng = np.random.default_rng(seed_of("sigmoid-ce-oracle", sfx))
+    tol = 4e-6 if sfx == "f32" else 1e-13
+    for rows, cols in ((1, 1), (7, 10), (64, 33)):
+        x = (rng.standard_normal((rows, cols)) * 3).astype(dt)
+        y = rng.uniform(0, 1, (rows, cols)).astype(dt)
+        xl, yl = x.astype(np.longdouble), y.astype(np.longdouble)
+        s = 1 / (1 + np.exp(-xl))
+        want = float(np.sum(-(yl * np.log(s) + (1 - yl) * np.log1p(-s))) / rows)
+        got = oracle.sigmoid_cross_entropy(x, y)
+        assert abs(got - want) <= tol * max(1.0, abs(want)) * cols, (rows, cols)
+        g = oracle.sigmoid_cross_entropy_backward(dt(0.7), x, y)
+        assert np.max(np.abs(g - np.longdouble(0.7) * (s - yl) / rows)) <= tol
+        if sfx == "f64" and rows * cols <= 70:
+            num = np.zeros_like(x)
+            for idx in np.ndindex(*x.shape):
+                keep = x[idx]
+                x[idx] = keep + 1e-5; up = oracle.sigmoid_cross_entropy(x, y)
+                x[idx] = keep - 1e-5; dn = oracle.sigmoid_cross_entropy(x, y)
+                x[idx] = keep
+                num[idx] = (up - dn) / 2e-5
+            assert np.max(np.abs(oracle.sigmoid_cross_entropy_backward(1.0, x, y) - num)) < 1e-9
+    zero = np.zeros((4, 5), dtype=dt)
+    assert abs(oracle.sigmoid_cross_entropy(zero, zero) - 5 * np.log(2)) <= tol * 8
+    big = np.array([[1000.0, -1000.0]], dtype=dt)
+    assert oracle.sigmoid_cross_entropy(big, np.array([[1.0, 0.0]], dtype=dt)) == 0
+    assert oracle.sigmoid_cross_entropy(big, np.array([[0.0, 1.0]], dtype=dt)) == 2000
