@@ -6,7 +6,7 @@
 // The reference walks each row once with a running maximum and a sum of exp(x - maximum) that is rescaled whenever
 // the maximum moves (private/p_logsumexp.nim:20-31), rows in parallel under OpenMP, and adds the rows' losses with an
 // atomic. Here `lanes` lanes (a power of two up to 64) share a row: each runs the same recurrence over every lanes-th
-// element, the lanes' (maximum, sum) pairs are merged in a fixed butterfly (M = max, S = s1 exp(m1 - M) + s2 exp(m2 - M)),
+// element, the lanes' maxima and then their sums, each rescaled once to the row's maximum, are folded in fixed butterflies,
 // so a wavefront covers 64 / lanes rows and a load instruction of the wavefront reads neighbouring elements of them.
 // The rows' losses go to the library workspace and are added there in a fixed order (slices of 8192, then the slices'
 // sums): the result does not depend on timing, unlike the reference's atomic sum. The backward kernels recompute (M, S) the same way and write
@@ -41,10 +41,10 @@ template <> __device__ __forceinline__ double dev_log<double>(double v) { return
 // before the first is used), raises the maximum to that of the group with one rescaling of the sum, then adds the
 // group's exponentials: one exp per element and one per group instead of the reference's data-dependent branch per
 // element.
-template <typename T, bool DENSE, bool VEC>
+template <typename T, bool DENSE, bool VEC, bool SHORT>
 __device__ __forceinline__ void row_max_sumexp(const Args<T>& p, const T* x, const T* t, int j0, int lanes, T& m, T& s, T& dot) {
   constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
-  constexpr int U = VEC ? 4 : 8;
+  constexpr int U = SHORT ? 1 : (VEC ? 4 : 8);   // SHORT: the row has at most one unit per lane
   typedef T vec_t __attribute__((ext_vector_type(V)));
   const T ninf = -std::numeric_limits<T>::infinity();
   m = ninf;
@@ -90,37 +90,48 @@ __device__ __forceinline__ void row_max_sumexp(const Args<T>& p, const T* x, con
       }
     s += add;
   }
+  // The lanes of the row: first their maxima (a butterfly of comparisons), then every lane's sum rescaled once to the
+  // row's maximum, then the sums (a butterfly of additions). One exp per lane instead of two per butterfly step, which
+  // on rows of a few vectors was most of the kernel's arithmetic.
+  T M = m;
   for (int d = lanes >> 1; d >= 1; d >>= 1) {
-    const T om = __shfl_xor(m, d, 64), os = __shfl_xor(s, d, 64);
-    const T M = (om <= m) ? m : om;
-    // a lane without elements holds (-inf, 0): its share is 0 whatever M is (exp(-inf - -inf) would be NaN)
-    const T mine = (s == (T)0) ? (T)0 : s * dev_exp<T>(m - M);
-    const T theirs = (os == (T)0) ? (T)0 : os * dev_exp<T>(om - M);
-    s = mine + theirs;
-    m = M;
+    const T om = __shfl_xor(M, d, 64);
+    M = (om <= M) ? M : om;
+  }
+  // a lane without elements holds (-inf, 0): its share is 0 whatever M is (exp(-inf - -inf) would be NaN)
+  s = (s == (T)0) ? (T)0 : s * dev_exp<T>(m - M);
+  m = M;
+  for (int d = lanes >> 1; d >= 1; d >>= 1) {
+    s += __shfl_xor(s, d, 64);
     if constexpr (DENSE) dot += __shfl_xor(dot, d, 64);
   }
 }
 
-template <typename T, bool DENSE, bool VEC>
+template <typename T, bool DENSE, bool VEC, bool SHORT>
 __global__ __launch_bounds__(256) void sce_forward(Args<T> p, int lanes) {
   const int lane = threadIdx.x & 63;
   const int j0 = lane & (lanes - 1);
-  const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / lanes) + lane / lanes;
-  const bool ok = row < p.rows;
-  const int64_t r = ok ? row : 0;
-  const T* x = p.x + r * p.x_rs;
-  const T* t = DENSE ? p.target + r * p.t_rs : nullptr;
-  T m, s, dot;
-  row_max_sumexp<T, DENSE, VEC>(p, x, t, j0, lanes, m, s, dot);
-  if (!ok || j0 != 0) return;
-  const T lse = dev_log<T>(s) + m;
-  if constexpr (DENSE) {
-    p.row_loss[row] = lse - dot;
-  } else {
-    const int64_t label = p.labels[row * p.l_s];
-    // a label outside the row cannot be read: the loss says so
-    p.row_loss[row] = (label >= 0 && label < p.cols) ? lse - x[label * p.x_cs] : std::numeric_limits<T>::quiet_NaN();
+  const int rows_per_wave = 64 / lanes;
+  const int64_t groups = (p.rows + rows_per_wave - 1) / rows_per_wave;
+  // a wavefront walks over groups of 64 / lanes rows: with short rows and very many of them (a loss per pixel) a
+  // wavefront per group would live for a kilobyte of input
+  for (int64_t grp = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); grp < groups; grp += (int64_t)gridDim.x * 4) {
+    const int64_t row = grp * rows_per_wave + lane / lanes;
+    const bool ok = row < p.rows;
+    const int64_t r = ok ? row : 0;
+    const T* x = p.x + r * p.x_rs;
+    const T* t = DENSE ? p.target + r * p.t_rs : nullptr;
+    T m, s, dot;
+    row_max_sumexp<T, DENSE, VEC, SHORT>(p, x, t, j0, lanes, m, s, dot);
+    if (!ok || j0 != 0) continue;
+    const T lse = dev_log<T>(s) + m;
+    if constexpr (DENSE) {
+      p.row_loss[row] = lse - dot;
+    } else {
+      const int64_t label = p.labels[row * p.l_s];
+      // a label outside the row cannot be read: the loss says so
+      p.row_loss[row] = (label >= 0 && label < p.cols) ? lse - x[label * p.x_cs] : std::numeric_limits<T>::quiet_NaN();
+    }
   }
 }
 
@@ -151,21 +162,24 @@ __global__ __launch_bounds__(256) void sum_slices(const T* __restrict__ v, int64
   if (threadIdx.x == 0) out[blockIdx.x] = part[0] * scale;
 }
 
-template <typename T, bool DENSE, bool VEC>
+template <typename T, bool DENSE, bool VEC, bool SHORT>
 __global__ __launch_bounds__(256) void sce_backward(Args<T> p, int lanes) {
   constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
-  constexpr int U = VEC ? 2 : 4;
+  constexpr int U = SHORT ? 1 : (VEC ? 2 : 4);
   typedef T vec_t __attribute__((ext_vector_type(V)));
   const int lane = threadIdx.x & 63;
   const int j0 = lane & (lanes - 1);
-  const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / lanes) + lane / lanes;
+  const int rows_per_wave = 64 / lanes;
+  const int64_t groups = (p.rows + rows_per_wave - 1) / rows_per_wave;
+  for (int64_t grp = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); grp < groups; grp += (int64_t)gridDim.x * 4) {
+  const int64_t row = grp * rows_per_wave + lane / lanes;
   const bool ok = row < p.rows;
   const int64_t r = ok ? row : 0;
   const T* x = p.x + r * p.x_rs;
   const T* t = DENSE ? p.target + r * p.t_rs : nullptr;
   T m, s, dot;
-  row_max_sumexp<T, false, VEC>(p, x, t, j0, lanes, m, s, dot);
-  if (!ok) return;
+  row_max_sumexp<T, false, VEC, SHORT>(p, x, t, j0, lanes, m, s, dot);
+  if (!ok) continue;
   int64_t label = -1;
   if constexpr (!DENSE) label = p.labels[row * p.l_s];
   T* out = p.out + row * p.o_rs;
@@ -200,6 +214,7 @@ __global__ __launch_bounds__(256) void sce_backward(Args<T> p, int lanes) {
       if constexpr (VEC) __builtin_nontemporal_store(y, (vec_t*)(out + u * V));
       else out[u * p.o_cs] = y[0];
     }
+  }
   }
 }
 
@@ -292,9 +307,14 @@ static int forward(const char* fn, int64_t rows, int64_t cols, const T* x, int64
   const bool vec = vec_ok<T>(p, DENSE, false);
   const int lanes = lanes_for(vec ? cols / (16 / (int64_t)sizeof(T)) : cols);
   const int64_t rows_per_wg = 4 * (64 / lanes);
-  const dim3 grid((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
-  if (vec) hipLaunchKernelGGL((sce_forward<T, DENSE, true>), grid, dim3(256), 0, stream(), p, lanes);
-  else hipLaunchKernelGGL((sce_forward<T, DENSE, false>), grid, dim3(256), 0, stream(), p, lanes);
+  int64_t wgs = (rows + rows_per_wg - 1) / rows_per_wg;
+  if (wgs > (int64_t)num_cus() * 16) wgs = (int64_t)num_cus() * 16;
+  const dim3 grid((unsigned)wgs);
+  const bool short_rows = (vec ? cols / (16 / (int64_t)sizeof(T)) : cols) <= lanes;   // one unit per lane at most
+  if (vec && short_rows) hipLaunchKernelGGL((sce_forward<T, DENSE, true, true>), grid, dim3(256), 0, stream(), p, lanes);
+  else if (vec) hipLaunchKernelGGL((sce_forward<T, DENSE, true, false>), grid, dim3(256), 0, stream(), p, lanes);
+  else if (short_rows) hipLaunchKernelGGL((sce_forward<T, DENSE, false, true>), grid, dim3(256), 0, stream(), p, lanes);
+  else hipLaunchKernelGGL((sce_forward<T, DENSE, false, false>), grid, dim3(256), 0, stream(), p, lanes);
   AM_TRY(check_launch("sce_forward"));
   // the rows' losses -> their mean at ws[0]: slices of 8192 (and of 8192 slices) while there are many
   const T* v = p.row_loss;
@@ -325,9 +345,14 @@ static int backward(const char* fn, int64_t rows, int64_t cols, T gradient, cons
   const bool vec = vec_ok<T>(p, DENSE, true);
   const int lanes = lanes_for(vec ? cols / (16 / (int64_t)sizeof(T)) : cols);
   const int64_t rows_per_wg = 4 * (64 / lanes);
-  const dim3 grid((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
-  if (vec) hipLaunchKernelGGL((sce_backward<T, DENSE, true>), grid, dim3(256), 0, stream(), p, lanes);
-  else hipLaunchKernelGGL((sce_backward<T, DENSE, false>), grid, dim3(256), 0, stream(), p, lanes);
+  int64_t wgs = (rows + rows_per_wg - 1) / rows_per_wg;
+  if (wgs > (int64_t)num_cus() * 16) wgs = (int64_t)num_cus() * 16;
+  const dim3 grid((unsigned)wgs);
+  const bool short_rows = (vec ? cols / (16 / (int64_t)sizeof(T)) : cols) <= lanes;
+  if (vec && short_rows) hipLaunchKernelGGL((sce_backward<T, DENSE, true, true>), grid, dim3(256), 0, stream(), p, lanes);
+  else if (vec) hipLaunchKernelGGL((sce_backward<T, DENSE, true, false>), grid, dim3(256), 0, stream(), p, lanes);
+  else if (short_rows) hipLaunchKernelGGL((sce_backward<T, DENSE, false, true>), grid, dim3(256), 0, stream(), p, lanes);
+  else hipLaunchKernelGGL((sce_backward<T, DENSE, false, false>), grid, dim3(256), 0, stream(), p, lanes);
   return check_launch("sce_backward");
 }
 
