@@ -775,6 +775,60 @@ HipTensor<T> sparse_softmax_cross_entropy_backward(T gradient, const HipTensor<T
   return r;
 }
 
+// Sigmoid + binary cross-entropy averaged over the batch, and its gradient (nnp_sigmoid_cross_entropy.nim:23-62).
+namespace detail {
+inline int sigmoid_ce_(int64_t r, int64_t c, const float* x, int64_t xr, int64_t xc, const float* t, int64_t tr, int64_t tc, float* l) {
+  return am_hip_sigmoid_cross_entropy_f32(r, c, x, xr, xc, t, tr, tc, l);
+}
+inline int sigmoid_ce_(int64_t r, int64_t c, const double* x, int64_t xr, int64_t xc, const double* t, int64_t tr, int64_t tc, double* l) {
+  return am_hip_sigmoid_cross_entropy_f64(r, c, x, xr, xc, t, tr, tc, l);
+}
+inline int sigmoid_ce_bwd_(int64_t r, int64_t c, float g, const float* x, int64_t xr, int64_t xc, const float* t, int64_t tr, int64_t tc,
+                           float* o, int64_t orr, int64_t oc) {
+  return am_hip_sigmoid_cross_entropy_backward_f32(r, c, g, x, xr, xc, t, tr, tc, o, orr, oc);
+}
+inline int sigmoid_ce_bwd_(int64_t r, int64_t c, double g, const double* x, int64_t xr, int64_t xc, const double* t, int64_t tr, int64_t tc,
+                           double* o, int64_t orr, int64_t oc) {
+  return am_hip_sigmoid_cross_entropy_backward_f64(r, c, g, x, xr, xc, t, tr, tc, o, orr, oc);
+}
+inline int sgd_(int n, float* const* v, const float* const* g, const int64_t* s, float lr) { return am_hip_sgd_update_f32(n, v, g, s, lr); }
+inline int sgd_(int n, double* const* v, const double* const* g, const int64_t* s, double lr) { return am_hip_sgd_update_f64(n, v, g, s, lr); }
+}  // namespace detail
+template <typename T>
+T sigmoid_cross_entropy(const HipTensor<T>& input, const HipTensor<T>& target) {
+  if (input.rank() != 2 || input.shape != target.shape || input.shape[0] == 0)
+    throw std::invalid_argument("sigmoid_cross_entropy: input and target must be non-empty matrices of the same shape");
+  T loss = T(0);
+  check(detail::sigmoid_ce_(input.shape[0], input.shape[1], input.ptr(), input.strides[0], input.strides[1], target.ptr(),
+                            target.strides[0], target.strides[1], &loss));
+  return loss;
+}
+template <typename T>
+HipTensor<T> sigmoid_cross_entropy_backward(T gradient, const HipTensor<T>& cached_tensor, const HipTensor<T>& target) {
+  if (cached_tensor.rank() != 2 || cached_tensor.shape != target.shape)
+    throw std::invalid_argument("sigmoid_cross_entropy_backward: input and target must be matrices of the same shape");
+  HipTensor<T> r(cached_tensor.shape);
+  check(detail::sigmoid_ce_bwd_(cached_tensor.shape[0], cached_tensor.shape[1], gradient, cached_tensor.ptr(), cached_tensor.strides[0],
+                                cached_tensor.strides[1], target.ptr(), target.strides[0], target.strides[1], r.ptr(), r.strides[0], r.strides[1]));
+  return r;
+}
+
+// value -= learning_rate * gradient for every pair in ONE launch: the SGD optimizer's update
+// (nn/optimizers/optimizers.nim:35-51 runs one apply2_inline per parameter). C-contiguous tensors.
+template <typename T>
+void sgd_update(const std::vector<HipTensor<T>*>& values, const std::vector<const HipTensor<T>*>& gradients, T learning_rate) {
+  if (values.size() != gradients.size()) throw std::invalid_argument("sgd_update: one gradient per value");
+  std::vector<T*> v;
+  std::vector<const T*> g;
+  std::vector<int64_t> n;
+  for (size_t i = 0; i < values.size(); ++i) {
+    if (values[i]->shape != gradients[i]->shape || !values[i]->is_C_contiguous() || !gradients[i]->is_C_contiguous())
+      throw std::invalid_argument("sgd_update: each gradient must have its value's shape, both C-contiguous");
+    v.push_back(values[i]->ptr()); g.push_back(gradients[i]->ptr()); n.push_back(values[i]->size());
+  }
+  if (!v.empty()) check(detail::sgd_((int)v.size(), v.data(), g.data(), n.data(), learning_rate));
+}
+
 // conv2d = im2colgemm_conv2d (nn_primitives/fallback/conv.nim:81-106), bias [C_out] or [C_out, 1, 1], optionally
 // followed by relu. Float tensors with `fused`: one launch, the GEMM's B loader gathers the column matrix from the
 // images. Otherwise (integer tensors, or asked for): device im2col of the batch, then one strided-batched GEMM

@@ -698,6 +698,38 @@ proc sparse_softmax_cross_entropy_backward*[T: float32 | float64](gradient: T, c
   when T is float32: call am_hip_sparse_softmax_cross_entropy_backward_f32
   else: call am_hip_sparse_softmax_cross_entropy_backward_f64
 
+proc sigmoid_cross_entropy*[T: float32 | float64](input, target: HipTensor[T]): T =
+  ## nn_primitives/nnp_sigmoid_cross_entropy.nim:23-45: the map2 body and its sum in one pass, averaged over the batch.
+  assert input.rank == 2 and input.shape == target.shape
+  template call(f: untyped) =
+    check f(int64 input.shape[0], int64 input.shape[1], input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1],
+            target.get_offset_ptr, int64 target.strides[0], int64 target.strides[1], result.addr)
+  when T is float32: call am_hip_sigmoid_cross_entropy_f32
+  else: call am_hip_sigmoid_cross_entropy_f64
+
+proc sigmoid_cross_entropy_backward*[T: float32 | float64](gradient: T, cached_tensor, target: HipTensor[T]): HipTensor[T] =
+  ## nnp_sigmoid_cross_entropy.nim:47-62: gradient * (sigmoid(cached_tensor) - target) / batch_size.
+  assert cached_tensor.rank == 2 and cached_tensor.shape == target.shape
+  result = newHipTensor[T](cached_tensor.shape)
+  template call(f: untyped) =
+    check f(int64 cached_tensor.shape[0], int64 cached_tensor.shape[1], gradient, cached_tensor.get_offset_ptr,
+            int64 cached_tensor.strides[0], int64 cached_tensor.strides[1], target.get_offset_ptr, int64 target.strides[0],
+            int64 target.strides[1], result.get_offset_ptr, int64 result.strides[0], int64 result.strides[1])
+  when T is float32: call am_hip_sigmoid_cross_entropy_backward_f32
+  else: call am_hip_sigmoid_cross_entropy_backward_f64
+
+proc sgd_update*[T: float32 | float64](values: var openArray[HipTensor[T]], gradients: openArray[HipTensor[T]], learning_rate: T) =
+  ## nn/optimizers/optimizers.nim:35-51 (one apply2_inline per parameter: x - lr * y) for every parameter in ONE launch.
+  assert values.len == gradients.len
+  var v, g = newSeq[ptr T](values.len)
+  var n = newSeq[int64](values.len)
+  for i in 0 ..< values.len:
+    assert values[i].shape == gradients[i].shape and values[i].is_C_contiguous and gradients[i].is_C_contiguous
+    v[i] = values[i].get_offset_ptr; g[i] = gradients[i].get_offset_ptr; n[i] = int64 values[i].size
+  if values.len > 0:
+    when T is float32: check am_hip_sgd_update_f32(cint values.len, v[0].addr, g[0].addr, n[0].addr, learning_rate)
+    else: check am_hip_sgd_update_f64(cint values.len, v[0].addr, g[0].addr, n[0].addr, learning_rate)
+
 proc conv2d*[T: SomeFloat](input, kernel, bias: HipTensor[T], padding = (0, 0), stride = (1, 1), relu = false): HipTensor[T] =
   ## im2colgemm_conv2d (nn_primitives/fallback/conv.nim:81-106), optionally followed by relu, in one launch: the GEMM's
   ## B loader gathers the column matrix from the images. input [N, C, H, W], kernel [C_out, C, kH, kW] (C-contiguous),

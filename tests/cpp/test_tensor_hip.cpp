@@ -268,6 +268,21 @@ static void gru_cell_literals() {
   for (size_t i = 0; i < 6; ++i) CHECK(std::fabs((1 - z[i]) * n[i] + z[i] * -1.0 - hn[i]) < 1e-15);
 }
 
+static void sigmoid_loss_and_sgd() {
+  // sigmoid cross-entropy at x = 0 is ln 2 per element whatever the target; its gradient there is (0.5 - y) / batch
+  auto x = toHip<double>({0, 0, 0, 0, 0, 0}, {2, 3});
+  auto y = toHip<double>({1, 0, 0.5, 0, 1, 0.25}, {2, 3});
+  CHECK(std::fabs(am::sigmoid_cross_entropy(x, y) - 3 * std::log(2.0)) < 1e-14);
+  CHECK(eq(am::sigmoid_cross_entropy_backward(2.0, x, y), {-0.5, 0.5, 0.0, 0.5, -0.5, 0.25}));
+  // every parameter updated by one launch: value - lr * gradient
+  auto w = toHip<float>({1, 2, 3, 4}, {2, 2});
+  auto b = toHip<float>({10, 20, 30}, {3});
+  const auto gw = toHip<float>({1, 1, 2, 2}, {2, 2});
+  const auto gb = toHip<float>({4, 8, 12}, {3});
+  am::sgd_update<float>({&w, &b}, {&gw, &gb}, 0.5f);
+  CHECK(eq(w, {0.5f, 1.5f, 2.0f, 3.0f}) && eq(b, {8, 16, 24}));
+}
+
 static void graph_with_temporaries() {
   // A sequence with temporaries recorded as it is: out <- relu(a * w + a) through three operator results that are
   // dropped inside the recorded function; replays follow new values written into `a`.
@@ -495,6 +510,7 @@ int main(int argc, char** argv) {
   conv_literals<int64_t>();
   loss_literals();
   graph_with_temporaries();
+  sigmoid_loss_and_sgd();
   gru_cell_literals();
   conv_backward_known_answer<float>();
   conv_backward_known_answer<double>();
