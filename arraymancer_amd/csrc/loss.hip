@@ -137,10 +137,10 @@ __global__ __launch_bounds__(256) void sce_forward(Args<T> p, int lanes) {
 
 // Sum of v[0 .. n) in a fixed order, in up to three levels. sum_slices: workgroup b adds the slice
 // [b * per, (b + 1) * per) (each lane every 256th value, eight loads in flight, then the lanes pairwise through LDS)
-// into out[b], times `scale`; the host runs it over the rows' losses, then over the slices' sums if there are many,
-// and last with one workgroup and scale = 1 / rows.
+// into out[b], divided by `divisor`; the host runs it over the rows' losses, then over the slices' sums if there are
+// many (divisor 1), and last with one workgroup and the batch size as divisor, as the reference divides its sum.
 template <typename T>
-__global__ __launch_bounds__(256) void sum_slices(const T* __restrict__ v, int64_t n, int64_t per, T scale, T* __restrict__ out) {
+__global__ __launch_bounds__(256) void sum_slices(const T* __restrict__ v, int64_t n, int64_t per, T divisor, T* __restrict__ out) {
   __shared__ T part[256];
   const int64_t lo = (int64_t)blockIdx.x * per, hi = (lo + per < n) ? lo + per : n;
   T acc = (T)0;
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void sum_slices(const T* __restrict__ v, int64
     if ((int)threadIdx.x < d) part[threadIdx.x] += part[threadIdx.x + d];
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = part[0] * scale;
+  if (threadIdx.x == 0) out[blockIdx.x] = part[0] / divisor;
 }
 
 template <typename T, bool DENSE, bool VEC, bool SHORT>
@@ -326,7 +326,7 @@ static int forward(const char* fn, int64_t rows, int64_t cols, const T* x, int64
     AM_TRY(check_launch("sum_slices"));
     v = spare; n = slices; spare += slices;
   }
-  hipLaunchKernelGGL((sum_slices<T>), dim3(1), dim3(256), 0, stream(), v, n, n, (T)1 / (T)rows, (T*)ws);
+  hipLaunchKernelGGL((sum_slices<T>), dim3(1), dim3(256), 0, stream(), v, n, n, (T)rows, (T*)ws);
   AM_TRY(check_launch("sum_slices"));
   return fetch_result(loss, ws, sizeof(T));
 }
@@ -384,7 +384,7 @@ static int sigmoid_forward(const char* fn, int64_t rows, int64_t cols, const T* 
     AM_TRY(check_launch("sum_slices"));
     v = spare; n = slices; spare += slices;
   }
-  hipLaunchKernelGGL((sum_slices<T>), dim3(1), dim3(256), 0, stream(), v, n, n, (T)1 / (T)rows, (T*)ws);
+  hipLaunchKernelGGL((sum_slices<T>), dim3(1), dim3(256), 0, stream(), v, n, n, (T)rows, (T*)ws);
   AM_TRY(check_launch("sum_slices"));
   return fetch_result(loss, ws, sizeof(T));
 }
