@@ -15,7 +15,8 @@ enum LoadKind : int {
   kKContig = 0,   // ld_k == 1: 16-byte vectors along k
   kMNContig = 1,  // ld_mn == 1: 16-byte vectors along m (A) or n (B)
   kGeneric = 2,   // any strides (zero, negative, non-unit): scalar gathers
-  kGather = 3     // B only: the column matrix of a convolution, read straight from the image (ConvGeom)
+  kGather = 3,    // B only: the column matrix of a convolution, read straight from the image (ConvGeom)
+  kGatherVec = 4  // kGather in 16-byte pieces: unit stride along the image's and the window's width, whole vectors per output row
 };
 
 // Geometry of a convolution whose column matrix col(k, j) = image[c, oh * sh - ph + kh, ow * sw - pw + kw]

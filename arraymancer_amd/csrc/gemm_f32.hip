@@ -117,10 +117,11 @@ extern "C" int am_hip_conv2d_f32(int64_t N, int C, int H, int W, int Cout, int k
   if (rc > 0) return AM_OK;
   if (rc < 0) return rc;
   AM_TRY(ensure_init());
-  // (a 128 x 128 tile, eight gathered elements per lane and slab, measured half as fast as 64 x 64 with four)
-  static const TileChoice cand[] = {{64, 64, 0.88}, {32, 32, 0.60}};
-  switch (choose_tile(cand, 2, g.M, g.N, "AM_HIP_CONV_TILE_F32", g.batch)) {
+  // (128 x 128 and 64 x 128 tiles measured slower than these on every shape tried; 128 x 64 pays from 128 output channels on)
+  static const TileChoice cand[] = {{64, 64, 0.88}, {32, 32, 0.60}, {128, 64, 0.92}};
+  switch (choose_tile(cand, 3, g.M, g.N, "AM_HIP_CONV_TILE_F32", g.batch)) {
     case 0: return launch_conv<float, 64, 64, 16, 2, 2, 2>(g);
+    case 2: return launch_conv<float, 128, 64, 16, 2, 2, 2>(g);
     default: return launch_conv<float, 32, 32, 32, 2, 2, 2, true, true, MfmaF32x16>(g);
   }
 }

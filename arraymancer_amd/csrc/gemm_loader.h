@@ -327,5 +327,86 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
   }
 };
 
+// The same column matrix where VK neighbouring output pixels of one row read VK neighbouring image elements: unit
+// stride along the image's width and along the window's step, output rows that are whole vectors (the host checks).
+// A lane owns VK columns (their common window origin is decoded once) and NV k values per slab: one 16-byte load and
+// one 16-byte LDS write where the scalar loader issues VK of each, and one decode of k (now per lane: the lanes of a
+// wavefront no longer share it). A vector that hangs over the left or right edge of the image row is loaded from
+// where it fits inside the row instead and moved into place at the commit, zeros in the padding; a vector whose row
+// lies in the padding, or past the end of the k range, is loaded from the image's lowest address and committed as
+// zeros. Every load is unconditional. k-row LDS layout.
+template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kGatherVec, BMN, BK, NT, KG, PF> {
+  typedef typename VecTraits<T>::vec_t vec_t;
+  typedef typename VecTraits<T>::gvec_t gvec_t;
+  static constexpr int VK = VecTraits<T>::VK;
+  static constexpr int CG = BMN / VK;              // column groups of a slab
+  static constexpr int KSTRIDE = NT / CG;          // distance in k between a lane's vectors
+  static constexpr int NV = BK / KSTRIDE;          // vectors per thread
+  static constexpr int kZero = 127;                // `how`: every element is padding (0: every element is real; else the shift)
+  static_assert(BMN % VK == 0 && NT % CG == 0 && BK % KSTRIDE == 0 && NV >= 1, "a lane must own one column group of the slab");
+  const char* low;       // the image's lowest address
+  uint32_t noff;         // byte offset of the window origin from `low` (modulo 2^32: it may lie in the padding)
+  int ih0, iw0, kbase;
+  int64_t K;
+  ConvGeom g;
+  vec_t reg[PF][NV];
+  int how[PF][NV];
+  __device__ __forceinline__ Loader(const T* X, int64_t, int64_t, int64_t mn0, int64_t MN, int64_t K_, int, const ConvGeom* geom)
+      : K(K_), g(*geom) {
+    low = (const char*)X - g.origin;
+    const int64_t j = mn0 + (int)(threadIdx.x % CG) * VK;
+    const int jj = (int)(j < MN ? j : MN - VK);     // column groups past the edge repeat the last one (masked at the store)
+    const int oh = jj / g.Wo, ow = jj - oh * g.Wo;
+    ih0 = oh * g.sh - g.ph;
+    iw0 = ow - g.pw;
+    noff = g.origin + (uint32_t)(ih0 * g.in_h) + (uint32_t)(iw0 * g.in_w);
+    kbase = (int)(threadIdx.x / CG);
+  }
+  __device__ __forceinline__ bool tail_guard() const { return false; }
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
+    if (MASK && k0 >= K) return;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const uint32_t k = (uint32_t)k0 + (uint32_t)(kbase + i * KSTRIDE);
+      const uint32_t c = g.magic_khw ? __umulhi(k, g.magic_khw) : k;        // (multiplier 0: the divisor is 1)
+      const uint32_t r = k - c * (uint32_t)(g.kH * g.kW);
+      const uint32_t kh = g.magic_kw ? __umulhi(r, g.magic_kw) : r;
+      const uint32_t kw = r - kh * (uint32_t)g.kW;
+      const uint32_t koff = c * (uint32_t)g.in_c + kh * (uint32_t)g.in_h + kw * (uint32_t)g.in_w;   // modulo 2^32, like noff
+      const int iws = iw0 + (int)kw;               // image column of the vector's first element
+      const bool row_ok = (!MASK || (int64_t)k < K) && (uint32_t)(ih0 + (int)kh) < (uint32_t)g.H;
+      const bool some = row_ok && iws > -VK && iws < g.W;
+      const int fit = iws < 0 ? 0 : (iws > g.W - VK ? g.W - VK : iws);   // where a vector that hangs over an edge is read from
+      const int shift = iws - fit;
+      how[S][i] = some ? shift : kZero;
+      reg[S][i] = *(const gvec_t*)(low + (some ? noff + koff - (uint32_t)(shift * (int)sizeof(T)) : 0u));
+    }
+  }
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
+    constexpr int LD = Slab<T, kGatherVec, BMN, BK>::LDMN;
+    const bool none = MASK && k0 >= K;     // nothing was fetched
+    const int cgp = (int)(threadIdx.x % CG);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      vec_t v = {};
+      if (!none && how[S][i] != kZero) {
+        v = reg[S][i];
+        const int d = how[S][i];
+        if (d != 0) {        // element e is image column fit + e + d: real while 0 <= e + d < VK
+          const vec_t w = v;
+#pragma unroll
+          for (int e = 0; e < VK; ++e) {
+            T x = (T)0;
+#pragma unroll
+            for (int f = 0; f < VK; ++f) x = (e + d == f) ? w[f] : x;
+            v[e] = x;
+          }
+        }
+      }
+      *(vec_t*)(lds + (kbase + i * KSTRIDE) * LD + cgp * VK) = v;
+    }
+  }
+};
+
 }  // namespace gemm
 }  // namespace am

@@ -480,7 +480,14 @@ static int launch_conv(Args<T>& g) {
   if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "conv2d: too many tiles");
   plan_splitk(g, BK, WAVES_M * WAVES_N);
   const dim3 grid((unsigned)(nb * g.splits), (unsigned)g.batch), block(WAVES_M * WAVES_N * 64);
-  hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, kKContig, kGather>), grid, block, 0, stream(), g);
+  // 16-byte gathers where VK neighbouring output pixels of a row read VK neighbouring image elements
+  constexpr int VK = VecTraits<T>::VK;
+  const ConvGeom& cg = g.conv;
+  static const bool vec_on = [] { const char* e = getenv("AM_HIP_CONV_GATHER"); return !(e && strcmp(e, "scalar") == 0); }();   // tests
+  if (vec_on && cg.in_w == (int)sizeof(T) && cg.sw == 1 && cg.Wo % VK == 0 && cg.W >= VK)
+    hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, kKContig, kGatherVec>), grid, block, 0, stream(), g);
+  else
+    hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, kKContig, kGather>), grid, block, 0, stream(), g);
   AM_TRY(check_launch("gemm_mfma (convolution)"));
   if (g.splits > 1) return launch_splitk_reduce<T, T>(g);
   return AM_OK;

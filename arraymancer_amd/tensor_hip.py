@@ -560,8 +560,8 @@ def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None,
         grad_weight = g * col^T                          (one product with k = N*P; the per-image products summed)
         grad_input  = col2im(kernel_col^T * g)           (one product, one gather)
 
-    Float tensors with unit stride and up to 96 input channels take grad_input as ONE launch instead: the convolution
-    of grad_output with the turned kernel. grad_bias is None when `bias` is; grad_input is None (and not computed) when
+    Float tensors with unit stride and up to 96 input channels (float32: any number on images of 512 pixels or more)
+    take grad_input as ONE launch instead: the convolution of grad_output with the turned kernel. grad_bias is None when `bias` is; grad_input is None (and not computed) when
     `need_input_grad` is False: the first layer of a network has no use for the gradient of the images."""
     _same_dtype(input, weight, grad_output)
     N, C, H, W = input.shape
@@ -579,7 +579,8 @@ def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None,
     grad_weight = matmul(g, col.transpose()).reshape(co, ci, kh, kw)
     if not need_input_grad:
         return None, grad_weight, grad_bias
-    if (input.dtype.kind == "f" and tuple(stride) == (1, 1) and padding[0] < kh and padding[1] < kw and C <= 96 and N <= 65535
+    if (input.dtype.kind == "f" and tuple(stride) == (1, 1) and padding[0] < kh and padding[1] < kw and N <= 65535
+            and (C <= 96 or (input.dtype == np.float32 and H * W >= 512))
             and co * kh * kw * input.dtype.itemsize >= 16):
         # With unit stride the gradient is itself a convolution, of grad_output with the kernel turned by 180 degrees and
         # its two channel axes swapped, padded by k - 1 - p: one launch of the gathered form instead of a product that
@@ -628,8 +629,10 @@ def conv2d(x: HipTensor, kernel: HipTensor, bias: HipTensor | None = None, paddi
     is_float = x.dtype.kind == "f"
     if fused is None:
         # up to about a hundred output channels the gathered form wins (no column matrix is written and read back);
-        # beyond, the two-launch form's vector loads and larger tiles catch up (32 x 128 x 28 x 28 -> 128, 3 x 3: 122 against 116 us)
-        fused = is_float and ci * kh * kw * x.dtype.itemsize >= 16 and N <= 65535 and co <= 96
+        # beyond, the two-launch form's larger tiles catch up on small images (float32 32 x 256 x 14 x 14 -> 256, 3 x 3:
+        # 130 against 95 us) but not on large ones (64 x 64 x 56 x 56 -> 128: 324 against 427 us; 28 x 28 is even)
+        fused = (is_float and ci * kh * kw * x.dtype.itemsize >= 16 and N <= 65535
+                 and (co <= 96 or (x.dtype == np.float32 and ho * wo >= 512)))
     if fused:
         k = kernel if kernel.reshape(co, ci * kh * kw).strides[1] == 1 else kernel.clone()
         return conv2d_into(empty((N, co, ho, wo), x.dtype), x, k, bias, padding, stride, relu)

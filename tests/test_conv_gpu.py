@@ -48,6 +48,10 @@ GEOMS = [  # N, C, H, W, C_out, kH, kW, pad, stride
     (2, 5, 11, 13, 70, 1, 1, (0, 0), (1, 1)),       # 1 x 1 kernel (k is the channel alone), more output channels than a small tile
     (3, 8, 20, 20, 130, 3, 5, (2, 3), (1, 2)),      # padding wider than the kernel's reach on one side, 130 output channels
     (2, 16, 40, 40, 32, 3, 3, (1, 1), (1, 1)),      # 1600 outputs per image: the larger tiles
+    (2, 4, 6, 4, 5, 3, 3, (1, 1), (1, 1)),          # image rows of one 16-byte float vector: every gathered vector but the middle one hangs over an edge
+    (2, 3, 7, 12, 6, 2, 5, (0, 4), (1, 1)),         # padding as wide as a float vector: vectors wholly in the padding beside partial ones (16 outputs per row)
+    (1, 2, 5, 6, 3, 1, 3, (0, 2), (2, 1)),          # unit stride along the width only, rows 6 wide: a hanging vector is shifted by up to 2 either way
+    (3, 24, 28, 28, 40, 3, 3, (1, 1), (1, 1)),      # 784 outputs: whole tiles and an edge tile of 16 columns
 ]
 
 
@@ -75,10 +79,35 @@ def test_im2col_and_conv_vs_oracle(hip, oracle, sfx, geom):
         check(oracle, sfx, got, np.where(0 >= want, np.zeros_like(want), want), f"conv + bias + relu, fused={fused}")
         got = hip.conv2d(dx, hip.toHip(k), None, pad, stride, fused=fused).toCpu()
         check(oracle, sfx, got, oracle.conv2d(x, k, None, pad, stride), f"conv, fused={fused}")
+        if fused:
+            # every other column of an image twice as wide: the one-element gathers, where the contiguous image may take
+            # 16-byte ones; the products are added in the same order, so the results agree to the bit
+            wide = np.zeros((N, C, H, 2 * W), dt)
+            wide[..., ::2] = x
+            spaced = hip.conv2d(hip.toHip(wide)[:, :, :, ::2], hip.toHip(k), None, pad, stride, fused=True).toCpu()
+            assert np.array_equal(spaced, got), "one-element and 16-byte gathers differ"
         # a channel-sliced (strided) input goes through the same kernel
         if C > 1:
             got = hip.conv2d(dx[:, ::-1], hip.toHip(np.ascontiguousarray(k[:, ::-1])), None, pad, stride, fused=fused).toCpu()
             check(oracle, sfx, got, oracle.conv2d(x, k, None, pad, stride), f"reversed channels, fused={fused}")
+
+
+@pytest.mark.parametrize("geom", [(3, 8, 24, 24, 130, 3, 3, (1, 1), (1, 1)), (2, 6, 9, 11, 200, 3, 2, (1, 1), (2, 1))])
+def test_fused_conv_tiles(hip, oracle, geom, monkeypatch):
+    """Every workgroup tile of the one-launch float32 convolution, forced in turn on 130 and 200 output channels (edge
+    tiles in both directions), with 16-byte gathers (first geometry) and one-element gathers (second): the oracle's
+    result from each, and the same bits from the tiles that use the same matrix instruction."""
+    N, C, H, W, co, kh, kw, pad, stride = geom
+    rng = np.random.default_rng(seed_of("conv tiles", geom))
+    x, k, b = fill(rng, (N, C, H, W), np.float32), fill(rng, (co, C, kh, kw), np.float32), fill(rng, (co,), np.float32)
+    want = oracle.conv2d(x, k, b, pad, stride)
+    got = {}
+    for tile in (0, 1, 2):
+        say("conv tile", tile, geom)
+        monkeypatch.setenv("AM_HIP_CONV_TILE_F32", str(tile))
+        got[tile] = hip.conv2d(hip.toHip(x), hip.toHip(k), hip.toHip(b), pad, stride, fused=True).toCpu()
+        check(oracle, "f32", got[tile], want, f"tile {tile}")
+    assert np.array_equal(got[0], got[2])
 
 
 @pytest.mark.parametrize("sfx", ALL)
@@ -119,7 +148,8 @@ BWD_GEOMS = [  # N, C, H, W, C_out, kH, kW, pad, stride
     (1, 2, 9, 10, 3, 3, 4, (1, 2), (1, 1)),         # kernel widths 4, 7 and 9 at unit stride
     (1, 1, 10, 12, 2, 2, 7, (0, 3), (1, 1)),
     (1, 1, 6, 14, 2, 2, 9, (0, 4), (1, 1)),
-    (2, 100, 8, 8, 6, 3, 3, (1, 1), (1, 1)),        # more input channels than the one-launch form of grad_input takes
+    (2, 100, 8, 8, 6, 3, 3, (1, 1), (1, 1)),        # more input channels than the one-launch form of grad_input takes on small images
+    (1, 100, 24, 24, 6, 3, 3, (1, 1), (1, 1)),      # the same channels on 576 pixels: float32 takes the one-launch form, float64 the product + gather
 ]
 
 
