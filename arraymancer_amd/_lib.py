@@ -105,6 +105,7 @@ def _signatures():
         sig[f"am_hip_maxpool2d_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp])
         if sfx in ("f32", "f64"):
             sig[f"am_hip_conv2d_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, i64, i64, i64, i64, vp, i64, ci, vp, i64, vp])
+            sig[f"am_hip_conv2d_grad_weight_{sfx}"] = (ci, [i64, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp, i64, i64, i64, i64, vp, i64, vp])
             sig[f"am_hip_softmax_rows_{sfx}"] = (ci, [i64, i64, vp, i64, i64, vp, i64, i64])
             sig[f"am_hip_sgd_update_{sfx}"] = (ci, [ci, vp, vp, vp, ct])
             sig[f"am_hip_gru_gates_{sfx}"] = (ci, [i64, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, i64])

@@ -6,6 +6,7 @@
 #include <string.h>
 #include <type_traits>
 #include "common.h"
+#include "fastdiv.h"
 
 namespace am {
 namespace gemm {
@@ -16,8 +17,12 @@ enum LoadKind : int {
   kMNContig = 1,  // ld_mn == 1: 16-byte vectors along m (A) or n (B)
   kGeneric = 2,   // any strides (zero, negative, non-unit): scalar gathers
   kGather = 3,    // B only: the column matrix of a convolution, read straight from the image (ConvGeom)
-  kGatherVec = 4  // kGather in 16-byte pieces: unit stride along the image's and the window's width, whole vectors per output row
+  kGatherVec = 4, // kGather in 16-byte pieces: unit stride along the image's and the window's width, whole vectors per output row
+  kGatherVecT = 5 // B only: the TRANSPOSED column matrices of a batch side by side, B(n, k) with n = (c, kh, kw) and
+                  // k = image * P + output pixel, in 16-byte pieces along k (the weight gradient's operand); k-group LDS layout
 };
+// Kinds whose slab sits in LDS as k-groups (16-byte slots of VK consecutive k per row / column).
+constexpr bool k_grouped(int kind) { return kind == kKContig || kind == kGatherVecT; }
 
 // Geometry of a convolution whose column matrix col(k, j) = image[c, oh * sh - ph + kh, ow * sw - pw + kw]
 // (k = (c * kH + kh) * kW + kw, j = oh * Wo + ow; zero where the window leaves the image) is the B operand of
@@ -33,6 +38,10 @@ struct ConvGeom {
   // vector offset takes. The image pointer is the GEMM's B.
   int in_c, in_h, in_w;
   uint32_t origin;
+  // kGatherVecT only: output pixels per image, the distance between images in bytes, dividers by P and by Wo
+  int P;
+  int64_t in_n;
+  FastDiv by_p, by_wo;
 };
 
 template <typename T> struct Args {
@@ -221,6 +230,54 @@ static int prepare_conv(const char* fn, int64_t N, int C, int H, int W, int Cout
   }
   auto magic = [](int d) { return d == 1 ? 0u : (uint32_t)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d); };
   cg.magic_khw = magic(kH * kW); cg.magic_kw = magic(kW);
+  return AM_OK;
+}
+
+// Fills the GEMM view of a convolution's weight gradient (fallback/conv.nim:135-143 adds grad_output_col * input_col^T image
+// by image): M = C_out, N = C * kH * kW, K = images * P with the images' column matrices side by side, gathered by the
+// kGatherVecT loader. gout is grad_output as [C_out][images * P] with unit stride along its rows. Returns 1 when there is
+// nothing to do (no images or no outputs: the result is left as it is), a negative code on bad arguments, AM_E_SHAPE for geometries the gathered form does not take.
+template <typename T>
+static int prepare_conv_grad_weight(const char* fn, int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW,
+                                    int strideH, int strideW, const T* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                                    const T* gout, int64_t gout_rs, T* out, Args<T>* g_out) {
+  constexpr int VK = 16 / (int)sizeof(T);
+  if (N < 0 || C < 0 || H < 0 || W < 0 || Cout < 0 || kH <= 0 || kW <= 0 || padH < 0 || padW < 0 || strideH <= 0 || strideW <= 0)
+    return fail(AM_E_ARG, "%s: bad geometry", fn);
+  const int64_t Ho = ((int64_t)H + 2 * padH - kH) / strideH + 1, Wo = ((int64_t)W + 2 * padW - kW) / strideW + 1;
+  if ((int64_t)H + 2 * padH < kH || (int64_t)W + 2 * padW < kW) return fail(AM_E_SHAPE, "%s: kernel larger than the padded image", fn);
+  if (C == 0 || Cout == 0) return 1;
+  const int64_t CKK = (int64_t)C * kH * kW, P = Ho * Wo, K = N * P;
+  if (strideW != 1 || in_w != 1 || Wo % VK != 0 || W < VK)
+    return fail(AM_E_SHAPE, "%s: needs unit stride along the width (image and window) and output rows of whole 16-byte vectors "
+                "(use im2col_strided + gemm)", fn);
+  if (CKK * kH * kW >= ((int64_t)1 << 32) || K >= ((int64_t)1 << 31))
+    return fail(AM_E_SHAPE, "%s: C * kH * kW = %lld or images * outputs = %lld outside what the fused kernel takes (use im2col_strided + gemm)",
+                fn, (long long)CKK, (long long)K);
+  if (N == 0 || P <= 0) return 1;     // no column at all: the sum over none is the caller's zero
+  if (!out || !in || !gout) return fail(AM_E_ARG, "%s: null tensor pointer", fn);
+  const int rc = prepare<T>(fn, Cout, CKK, K, (T)1, gout, gout_rs, 1, in, 0, 1, (T)0, out, CKK, 1, 0, (const T*)nullptr, 0, 0, g_out);
+  if (rc != AM_OK) return rc;
+  Args<T>& g = *g_out;
+  ConvGeom& cg = g.conv;
+  cg.H = H; cg.W = W; cg.kH = kH; cg.kW = kW; cg.Wo = (int)Wo; cg.ph = padH; cg.pw = padW; cg.sh = strideH; cg.sw = strideW;
+  {
+    const int64_t sz = (int64_t)sizeof(T);
+    const int64_t ext[3] = {C, H, W}, str[3] = {in_c, in_h, in_w};
+    int64_t lowest = 0, highest = 0;
+    for (int d = 0; d < 3; ++d) {
+      if (str[d] < 0) lowest += str[d] * (ext[d] - 1); else highest += str[d] * (ext[d] - 1);
+    }
+    if ((highest - lowest + 1) * sz >= ((int64_t)1 << 32))
+      return fail(AM_E_SHAPE, "%s: one image spans 4 GiB or more (use im2col_strided + gemm)", fn);
+    cg.in_c = (int)(in_c * sz); cg.in_h = (int)(in_h * sz); cg.in_w = (int)(in_w * sz);
+    cg.origin = (uint32_t)(-lowest * sz);
+    cg.in_n = in_n * sz;
+  }
+  auto magic = [](int d) { return d == 1 ? 0u : (uint32_t)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d); };
+  cg.magic_khw = magic(kH * kW); cg.magic_kw = magic(kW);
+  cg.P = (int)P;
+  cg.by_p = FastDiv((uint32_t)P); cg.by_wo = FastDiv((uint32_t)Wo);
   return AM_OK;
 }
 

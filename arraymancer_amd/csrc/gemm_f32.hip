@@ -125,3 +125,24 @@ extern "C" int am_hip_conv2d_f32(int64_t N, int C, int H, int W, int Cout, int k
     default: return launch_conv<float, 32, 32, 32, 2, 2, 2, true, true, MfmaF32x16>(g);
   }
 }
+
+// The weight gradient of im2colgemm_conv2d_gradient (src/arraymancer/nn_primitives/fallback/conv.nim:135-143) over the whole
+// batch as ONE product with k = images * outputs: the column matrices are never written, the GEMM's B loader gathers
+// their transposes from the images in 16-byte pieces.
+extern "C" int am_hip_conv2d_grad_weight_f32(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH,
+                                             int strideW, const float* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                                             const float* gout, int64_t gout_rs, float* out) {
+  Args<float> g;
+  const int rc = prepare_conv_grad_weight<float>("am_hip_conv2d_grad_weight_f32", N, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW,
+                                                in, in_n, in_c, in_h, in_w, gout, gout_rs, out, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  // the candidates of the plain product that a gathered B takes (few output channels: 64 rows; 128 from 128 on)
+  static const TileChoice cand[] = {{64, 64, 0.88, 16, 4}, {32, 32, 0.74, 32, 4}, {128, 64, 0.92, 16, 4}};
+  switch (choose_tile_and_split(g, cand, 3, "AM_HIP_CONV_GW_TILE_F32", 157.3e6 / 256)) {
+    case 0: return launch_conv_grad_weight<float, 64, 64, 16, 2, 2, 2>(g);
+    case 2: return launch_conv_grad_weight<float, 128, 64, 16, 2, 2, 2>(g);
+    default: return launch_conv_grad_weight<float, 32, 32, 32, 2, 2, 2, true, true, MfmaF32x16>(g);
+  }
+}

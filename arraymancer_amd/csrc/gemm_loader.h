@@ -33,7 +33,7 @@ template <typename T, int KIND, int BMN, int BK, bool KG = true> struct Slab {
   static constexpr int LDKG = BMN + (QN_ >= 8 ? 1 : 8 / QN_);   // 16-byte slots per k-group plane
   static constexpr int LDMN = BMN + 4;   // k-row layout: elements per k row (4 * LDMN mod 32 banks = 16: the
                                          // four k-rows a transposing write touches fall on two bank halves, not one)
-  static constexpr int ELEMS = (KIND == kKContig && KG) ? (BK / VK) * LDKG * VK : BK * LDMN;
+  static constexpr int ELEMS = (k_grouped(KIND) && KG) ? (BK / VK) * LDKG * VK : BK * LDMN;
 };
 
 // Moves one operand slab global -> registers (fetch) -> LDS (commit). PF register stages let PF
@@ -404,6 +404,91 @@ template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T,
         }
       }
       *(vec_t*)(lds + (kbase + i * KSTRIDE) * LD + cgp * VK) = v;
+    }
+  }
+};
+
+// The transposed column matrices of a whole batch side by side, as the B operand of the weight gradient
+// grad_weight[C_out][C * kH * kW] = g[C_out][N * P] . col^T: B(n, k) with n = (c, kh, kw), k = image * P + pixel. Along k
+// neighbouring output pixels of one row read neighbouring image elements (same conditions as kGatherVec, checked by
+// the host: unit strides along the width, output rows that are whole vectors - so P and every image's first k are
+// multiples of VK too), so the operand moves like a k-contiguous one: a lane owns one n (decoded once) and one 16-byte
+// k-group per slab, whose k is decoded into (image, oh, ow) by two launch-constant divisions. Edges as in kGatherVec.
+// k-group LDS layout, the one the k-contiguous loader writes.
+template <typename T, int BMN, int BK, int NT, bool KG, int PF> struct Loader<T, kGatherVecT, BMN, BK, NT, KG, PF> {
+  typedef typename VecTraits<T>::vec_t vec_t;
+  typedef typename VecTraits<T>::gvec_t gvec_t;
+  static constexpr int VK = VecTraits<T>::VK;
+  static constexpr int QN = BK / VK;               // k-groups per row
+  static constexpr int NV = BMN * QN / NT;         // vectors per thread
+  static constexpr int kZero = 127;
+  static_assert(KG && BMN * QN % NT == 0 && NV >= 1, "slab must divide evenly over the workgroup");
+  const char* low;       // image 0's lowest address
+  uint32_t coff[NV];     // byte offset from `low` of the element that n reads for output pixel (0, 0) (modulo 2^32)
+  int dh[NV], dw[NV];    // kh - padH, kw - padW
+  int64_t K;
+  ConvGeom g;
+  vec_t reg[PF][NV];
+  int how[PF][NV];
+  __device__ __forceinline__ Loader(const T* X, int64_t, int64_t, int64_t mn0, int64_t MN, int64_t K_, int, const ConvGeom* geom)
+      : K(K_), g(*geom) {
+    low = (const char*)X - g.origin;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int64_t mn = mn0 + (int)((threadIdx.x + i * NT) / QN);
+      const uint32_t n = (uint32_t)(mn < MN ? mn : MN - 1);    // rows past the edge repeat the last one (masked at the store)
+      const uint32_t c = g.magic_khw ? __umulhi(n, g.magic_khw) : n;
+      const uint32_t r = n - c * (uint32_t)(g.kH * g.kW);
+      const uint32_t kh = g.magic_kw ? __umulhi(r, g.magic_kw) : r;
+      const uint32_t kw = r - kh * (uint32_t)g.kW;
+      dh[i] = (int)kh - g.ph;
+      dw[i] = (int)kw - g.pw;
+      coff[i] = g.origin + c * (uint32_t)g.in_c + (uint32_t)(dh[i] * g.in_h) + (uint32_t)(dw[i] * g.in_w);
+    }
+  }
+  __device__ __forceinline__ bool tail_guard() const { return false; }
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void fetch(int64_t k0) {
+    if (MASK && k0 >= K) return;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const uint32_t k = (uint32_t)k0 + (uint32_t)(((threadIdx.x + i * NT) % QN) * VK);
+      uint32_t pix, ow;
+      const uint32_t img = g.by_p.divmod(k, pix);
+      const uint32_t oh = g.by_wo.divmod(pix, ow);
+      const int ih = (int)oh * g.sh + dh[i];
+      const int iws = (int)ow + dw[i];             // image column of the vector's first element
+      const bool row_ok = (!MASK || (int64_t)k < K) && (uint32_t)ih < (uint32_t)g.H;
+      const bool some = row_ok && iws > -VK && iws < g.W;
+      const int fit = iws < 0 ? 0 : (iws > g.W - VK ? g.W - VK : iws);
+      const int shift = iws - fit;
+      how[S][i] = some ? shift : kZero;
+      const uint32_t off = coff[i] + oh * (uint32_t)(g.sh * g.in_h) + (ow - (uint32_t)shift) * (uint32_t)g.in_w;
+      reg[S][i] = *(const gvec_t*)(low + (some ? (int64_t)img * g.in_n + (int64_t)off : (int64_t)0));
+    }
+  }
+  template <int S = 0, bool MASK = true> __device__ __forceinline__ void commit(T* lds, int64_t k0) {
+    constexpr int LD = Slab<T, kGatherVecT, BMN, BK, true>::LDKG;
+    const bool none = MASK && k0 >= K;     // nothing was fetched
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v_ = threadIdx.x + i * NT;
+      const int q = v_ % QN, mn = v_ / QN;
+      vec_t v = {};
+      if (!none && how[S][i] != kZero) {
+        v = reg[S][i];
+        const int d = how[S][i];
+        if (d != 0) {
+          const vec_t w = v;
+#pragma unroll
+          for (int e = 0; e < VK; ++e) {
+            T x = (T)0;
+#pragma unroll
+            for (int f = 0; f < VK; ++f) x = (e + d == f) ? w[f] : x;
+            v[e] = x;
+          }
+        }
+      }
+      *(vec_t*)(lds + (q * LD + mn) * VK) = v;
     }
   }
 };

@@ -85,7 +85,7 @@ template <typename T, typename MF, int KIND, int BMN, int BK>
 __device__ __forceinline__ void read_frag(const T* lds, int mn, int ks, int kl, T (&out)[MF::VK]) {
   typedef typename MF::vec_t vec_t;
   constexpr int VK = MF::VK, KL = MF::KL;
-  if constexpr (KIND == kKContig) {
+  if constexpr (k_grouped(KIND)) {
     constexpr int LD = Slab<T, KIND, BMN, BK>::LDKG;
     const vec_t v = *(const vec_t*)(lds + ((ks * KL + kl) * LD + mn) * VK);
 #pragma unroll
@@ -284,7 +284,7 @@ void gemm_mfma(Args<T> p) {
           for (int s = 0; s < VK; ++s)
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = MF::mma(af[0][i][s], bf[0][j][s], acc[i][j]);
-        constexpr int RA = AK == kKContig ? 1 : VK, RB = BKIND == kKContig ? 1 : VK;   // LDS reads per fragment
+        constexpr int RA = k_grouped(AK) ? 1 : VK, RB = k_grouped(BKIND) ? 1 : VK;   // LDS reads per fragment
         __builtin_amdgcn_sched_group_barrier(0x100, TN * RB + RA, 0);   // the B fragments and A fragment 0
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -489,6 +489,22 @@ static int launch_conv(Args<T>& g) {
   else
     hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, kKContig, kGather>), grid, block, 0, stream(), g);
   AM_TRY(check_launch("gemm_mfma (convolution)"));
+  if (g.splits > 1) return launch_splitk_reduce<T, T>(g);
+  return AM_OK;
+}
+
+// The weight gradient of a convolution as one long-k GEMM whose B operand is gathered from the images (kGatherVecT):
+// A = grad_output as [C_out, N * P] with unit stride along k.
+template <typename T, int BM, int BN, int BK, int WAVES_M, int WAVES_N, int PF = 1, bool FPF = true, bool RU = true, typename MF = Mfma<T>>
+static int launch_conv_grad_weight(Args<T>& g) {
+  g.tiles_m = (int)((g.M + BM - 1) / BM);
+  g.tiles_n = (int)((g.N + BN - 1) / BN);
+  const int64_t nb = (int64_t)g.tiles_m * g.tiles_n;
+  if (nb >= ((int64_t)1 << 31)) return fail(AM_E_SHAPE, "conv2d_grad_weight: too many tiles");
+  plan_splitk(g, BK, WAVES_M * WAVES_N);
+  const dim3 grid((unsigned)(nb * g.splits), 1u), block(WAVES_M * WAVES_N * 64);
+  hipLaunchKernelGGL((gemm_mfma<T, MF, BM, BN, BK, WAVES_M, WAVES_N, PF, FPF, RU, kKContig, kGatherVecT>), grid, block, 0, stream(), g);
+  AM_TRY(check_launch("gemm_mfma (weight gradient of a convolution)"));
   if (g.splits > 1) return launch_splitk_reduce<T, T>(g);
   return AM_OK;
 }

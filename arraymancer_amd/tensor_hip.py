@@ -550,7 +550,7 @@ def col2im(col: HipTensor, channels: int, height: int, width: int, kernel_size, 
 
 
 def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None, padding, stride, grad_output: HipTensor,
-                    need_input_grad: bool = True):
+                    need_input_grad: bool = True, fused_weight_gradient: bool = True):
     """(grad_input, grad_weight, grad_bias) of conv2d_backward (src/arraymancer/nn_primitives/nnp_convolution.nim:65-107)
     over im2colgemm_conv2d_gradient (fallback/conv.nim:107-145). The reference loops over the images (two GEMMs, an
     im2col and a col2im each); here the batch is folded into the columns, g[C_out, N*P] = grad_output with its first
@@ -561,8 +561,12 @@ def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None,
         grad_input  = col2im(kernel_col^T * g)           (one product, one gather)
 
     Float tensors with unit stride and up to 96 input channels (float32: any number on images of 512 pixels or more)
-    take grad_input as ONE launch instead: the convolution of grad_output with the turned kernel. grad_bias is None when `bias` is; grad_input is None (and not computed) when
-    `need_input_grad` is False: the first layer of a network has no use for the gradient of the images."""
+    take grad_input as ONE launch instead: the convolution of grad_output with the turned kernel. Float tensors whose
+    window steps by one pixel along the width, with output rows of whole 16-byte vectors, take grad_weight as ONE launch
+    too: col^T is gathered from the images by the product's loader and never written (`fused_weight_gradient=False`:
+    im2col + product as above; the same bits wherever both pick the same tile and split of k). grad_bias is None when `bias` is;
+    grad_input is None (and not computed) when `need_input_grad` is False: the first layer of a network has no use for
+    the gradient of the images."""
     _same_dtype(input, weight, grad_output)
     N, C, H, W = input.shape
     co, ci, kh, kw = weight.shape
@@ -574,9 +578,21 @@ def conv2d_backward(input: HipTensor, weight: HipTensor, bias: HipTensor | None,
     P = ho * wo
     g = grad_output.reshape(N, co, P).permute(1, 0, 2).clone().reshape(co, N * P)
     grad_bias = tsum(g, axis=1).reshape(*bias.shape) if bias is not None else None
-    col = im2col_folded(input, (kh, kw), padding, stride)
     kcol = weight.reshape(co, ci * kh * kw)
-    grad_weight = matmul(g, col.transpose()).reshape(co, ci, kh, kw)
+    vk = 16 // input.dtype.itemsize
+    if (fused_weight_gradient and input.dtype.kind == "f" and stride[1] == 1 and input.strides[3] == 1 and wo % vk == 0 and W >= vk
+            and N >= 1 and P >= 1 and N * P < 2 ** 31 and ci * kh * kw * kh * kw < 2 ** 32 and co * ci * kh * kw < 1_000_000):
+        # one launch: the product's second operand is gathered from the images, the column matrix (k^2 times the batch)
+        # is neither written nor read back (float32 64 x 64 x 56 x 56, 3 x 3: 350 -> 257 us with the swap of grad_output).
+        # A gradient of a million elements or more stays with the plain product and its larger tiles
+        # (16 x 512 x 8 x 8 -> 512: 63 against 89 us).
+        grad_weight = empty((co, ci, kh, kw), input.dtype)
+        check(getattr(_lib.load(), f"am_hip_conv2d_grad_weight_{input.sfx}")(
+            N, C, H, W, co, kh, kw, padding[0], padding[1], stride[0], stride[1], ctypes.c_void_p(input.data_ptr()), *input.strides,
+            ctypes.c_void_p(g.data_ptr()), g.strides[0], ctypes.c_void_p(grad_weight.data_ptr())))
+    else:
+        col = im2col_folded(input, (kh, kw), padding, stride)
+        grad_weight = matmul(g, col.transpose()).reshape(co, ci, kh, kw)
     if not need_input_grad:
         return None, grad_weight, grad_bias
     if (input.dtype.kind == "f" and tuple(stride) == (1, 1) and padding[0] < kh and padding[1] < kw and N <= 65535

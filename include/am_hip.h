@@ -277,6 +277,25 @@ int am_hip_conv2d_f64(int64_t N, int C, int H, int W, int Cout, int kH, int kW, 
                       const double* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
                       const double* kernel, int64_t kernel_rs, int epilogue, const double* bias, int64_t bias_s, double* out);
 
+/* grad_weight[co][c*kH*kW + kh*kW + kw] <- sum over the images n and their output pixels (oh, ow) of
+ * grad_output[co][n*P + oh*W_out + ow] * (padded input patch element of image n), P = H_out * W_out: the weight
+ * gradient of the whole batch as ONE product with k = N * P whose second operand, the transposed column matrices of
+ * the images side by side, is never written: the GEMM's B loader gathers it from the images in 16-byte pieces.
+ * `in` is addressed through its four NCHW strides (elements); `grad_output` is the [C_out][N * P] matrix (grad_output
+ * with its first two axes swapped), rows `gout_rs` apart, unit stride within a row; `out` is a contiguous
+ * [C_out, C, kH, kW] tensor, overwritten (left as it is when N = 0). Float types. Takes: unit stride of the window
+ * and of the image along the width, W_out a multiple of the elements in 16 bytes, W at least that many, N * P < 2^31
+ * (AM_E_SHAPE otherwise: run am_hip_im2col_strided_* + am_hip_gemm_* then). The sum over k is split over workgroups
+ * and folded in a fixed order: results do not change from run to run.
+ * Replaces the weight-gradient half of im2colgemm_conv2d_gradient
+ * (src/arraymancer/nn_primitives/fallback/conv.nim:135-143: per image im2col, then gemm_nt accumulated into grad_weight). */
+int am_hip_conv2d_grad_weight_f32(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH,
+                                  int strideW, const float* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                                  const float* grad_output, int64_t gout_rs, float* out);
+int am_hip_conv2d_grad_weight_f64(int64_t N, int C, int H, int W, int Cout, int kH, int kW, int padH, int padW, int strideH,
+                                  int strideW, const double* in, int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w,
+                                  const double* grad_output, int64_t gout_rs, double* out);
+
 /* ---------------------------------------------------------------- GEMV and dot
  * y[M] <- alpha * A[M x N] * x[N] + beta * y, any strides (elements).
  * Replaces gemv (src/arraymancer/tensor/operators_blas_l2l3.nim:24-56; integer fallback

@@ -158,6 +158,14 @@ inline int gemm_ex_(int64_t M, int64_t N, int64_t K, double al, const double* A,
   return am_hip_gemm_ex_f64(M, N, K, al, A, ra, ca, B, rb, cb, be, C, rc, cc, epi, bias, brs, bcs);
 }
 
+inline int conv2d_grad_weight_(int64_t N, int C, int H, int W, int Co, int kH, int kW, int pH, int pW, int sH, int sW, const float* in,
+                               int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, const float* g, int64_t g_rs, float* out) {
+  return am_hip_conv2d_grad_weight_f32(N, C, H, W, Co, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, g, g_rs, out);
+}
+inline int conv2d_grad_weight_(int64_t N, int C, int H, int W, int Co, int kH, int kW, int pH, int pW, int sH, int sW, const double* in,
+                               int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, const double* g, int64_t g_rs, double* out) {
+  return am_hip_conv2d_grad_weight_f64(N, C, H, W, Co, kH, kW, pH, pW, sH, sW, in, in_n, in_c, in_h, in_w, g, g_rs, out);
+}
 inline int conv2d_(int64_t N, int C, int H, int W, int Co, int kH, int kW, int pH, int pW, int sH, int sW, const float* in,
                    int64_t in_n, int64_t in_c, int64_t in_h, int64_t in_w, const float* k, int64_t k_rs, int epi,
                    const float* bias, int64_t bias_s, float* out) {
@@ -919,15 +927,29 @@ Conv2dGrads<T> conv2d_backward(const HipTensor<T>& x, const HipTensor<T>& weight
     r.bias.shape = Shape{co, 1, 1};
     r.bias.strides = Shape{1, 1, 1};
   }
-  HipTensor<T> col(Shape{K, N * P});
-  check(detail::im2col_strided_(N, (int)C, (int)H, (int)W, (int)kH, (int)kW, padH, padW, strideH, strideW, x.ptr(), x.strides[0],
-                                x.strides[1], x.strides[2], x.strides[3], col.ptr(), P, N * P));
   HipTensor<T> kcol = weight.is_C_contiguous() ? weight : weight.clone();
   kcol.shape = Shape{co, K};
   kcol.strides = Shape{K, 1};
-  r.weight = g * col.transpose();
-  r.weight.shape = Shape{co, C, kH, kW};
-  r.weight.strides = Shape{K, kH * kW, kW, 1};
+  bool gathered = false;
+  if constexpr (std::is_floating_point<T>::value) {
+    // one launch where the library's loader can gather col^T from the images in 16-byte pieces: col is never written
+    constexpr int64_t VK = 16 / (int64_t)sizeof(T);
+    if (strideW == 1 && x.strides[3] == 1 && ow % VK == 0 && W >= VK && N >= 1 && P >= 1 && N * P < ((int64_t)1 << 31) &&
+        K * kH * kW < ((int64_t)1 << 32) && co * K < 1000000) {   // (larger gradients: the plain product's larger tiles win)
+      r.weight = HipTensor<T>(Shape{co, C, kH, kW});
+      check(detail::conv2d_grad_weight_(N, (int)C, (int)H, (int)W, (int)co, (int)kH, (int)kW, padH, padW, strideH, strideW, x.ptr(),
+                                        x.strides[0], x.strides[1], x.strides[2], x.strides[3], g.ptr(), g.strides[0], r.weight.ptr()));
+      gathered = true;
+    }
+  }
+  if (!gathered) {
+    HipTensor<T> col(Shape{K, N * P});
+    check(detail::im2col_strided_(N, (int)C, (int)H, (int)W, (int)kH, (int)kW, padH, padW, strideH, strideW, x.ptr(), x.strides[0],
+                                  x.strides[1], x.strides[2], x.strides[3], col.ptr(), P, N * P));
+    r.weight = g * col.transpose();
+    r.weight.shape = Shape{co, C, kH, kW};
+    r.weight.strides = Shape{K, kH * kW, kW, 1};
+  }
   const HipTensor<T> gcol = kcol.transpose() * g;
   r.input = HipTensor<T>(Shape{N, C, H, W});
   check(detail::col2im_(N, (int)C, (int)H, (int)W, (int)kH, (int)kW, padH, padW, strideH, strideW, gcol.ptr(), P, N * P, r.input.ptr(),

@@ -96,6 +96,12 @@ proc am_hip_conv2d_f32*(N: int64, C, H, W, Cout, kH, kW, padH, padW, strideH, st
 proc am_hip_conv2d_f64*(N: int64, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cdouble,
                         in_n, in_c, in_h, in_w: int64, kernel: ptr cdouble, kernel_rs: int64, epilogue: cint,
                         bias: ptr cdouble, bias_s: int64, output: ptr cdouble): cint {.importc.}
+proc am_hip_conv2d_grad_weight_f32*(N: int64, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cfloat,
+                                    in_n, in_c, in_h, in_w: int64, grad_output: ptr cfloat, gout_rs: int64,
+                                    output: ptr cfloat): cint {.importc.}
+proc am_hip_conv2d_grad_weight_f64*(N: int64, C, H, W, Cout, kH, kW, padH, padW, strideH, strideW: cint, inp: ptr cdouble,
+                                    in_n, in_c, in_h, in_w: int64, grad_output: ptr cdouble, gout_rs: int64,
+                                    output: ptr cdouble): cint {.importc.}
 proc am_hip_gemm_batched_i32*(batch, M, N, K: int64, alpha: int32, A: ptr int32, rsA, csA, bsA: int64,
                               B: ptr int32, rsB, csB, bsB: int64, beta: int32, C: ptr int32, rsC, csC, bsC: int64,
                               epilogue: cint, bias: ptr int32, bias_rs, bias_cs: int64): cint {.importc.}

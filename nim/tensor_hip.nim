@@ -773,20 +773,35 @@ proc conv2d_backward*[T: HipScalar](input, weight, bias: HipTensor[T], padding, 
   if bias.rank > 0:
     grad_bias = sum(g, axis = 1)
     grad_bias.shape.copyFrom([co, 1, 1]); grad_bias.strides.copyFrom([1, 1, 1])
-  var col = newHipTensor[T]([C * kH * kW, N * P])
-  template unroll(f: untyped) =
-    check f(int64 N, cint C, cint H, cint W, cint kH, cint kW, cint padding.height, cint padding.width, cint stride.height, cint stride.width,
-            input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1], int64 input.strides[2], int64 input.strides[3],
-            col.get_offset_ptr, int64 P, int64(N * P))
-  when T is float32: unroll am_hip_im2col_strided_f32
-  elif T is float64: unroll am_hip_im2col_strided_f64
-  elif T is int32: unroll am_hip_im2col_strided_i32
-  else: unroll am_hip_im2col_strided_i64
   let wc = if weight.is_C_contiguous: weight else: weight.clone()
   var kcol = wc
   kcol.shape.copyFrom([co, C * kH * kW]); kcol.strides.copyFrom([C * kH * kW, 1])
-  grad_weight = g * col.transpose
-  grad_weight.shape.copyFrom([co, C, kH, kW]); grad_weight.strides.copyFrom([C * kH * kW, kH * kW, kW, 1])
+  # one launch where the library's loader can gather col^T from the images in 16-byte pieces: col is never written
+  var gathered = false
+  when T is float32 or T is float64:
+    const vk = 16 div sizeof(T)
+    if stride.width == 1 and input.strides[3] == 1 and outW mod vk == 0 and W >= vk and N >= 1 and P >= 1 and
+       N * P < (1 shl 31) and C * kH * kW * kH * kW < (1 shl 32) and co * C * kH * kW < 1_000_000:   # (larger gradients: the plain product's larger tiles win)
+      grad_weight = newHipTensor[T]([co, C, kH, kW])
+      template gather(f: untyped) =
+        check f(int64 N, cint C, cint H, cint W, cint co, cint kH, cint kW, cint padding.height, cint padding.width,
+                cint stride.height, cint stride.width, input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1],
+                int64 input.strides[2], int64 input.strides[3], g.get_offset_ptr, int64 g.strides[0], grad_weight.get_offset_ptr)
+      when T is float32: gather am_hip_conv2d_grad_weight_f32
+      else: gather am_hip_conv2d_grad_weight_f64
+      gathered = true
+  if not gathered:
+    var col = newHipTensor[T]([C * kH * kW, N * P])
+    template unroll(f: untyped) =
+      check f(int64 N, cint C, cint H, cint W, cint kH, cint kW, cint padding.height, cint padding.width, cint stride.height, cint stride.width,
+              input.get_offset_ptr, int64 input.strides[0], int64 input.strides[1], int64 input.strides[2], int64 input.strides[3],
+              col.get_offset_ptr, int64 P, int64(N * P))
+    when T is float32: unroll am_hip_im2col_strided_f32
+    elif T is float64: unroll am_hip_im2col_strided_f64
+    elif T is int32: unroll am_hip_im2col_strided_i32
+    else: unroll am_hip_im2col_strided_i64
+    grad_weight = g * col.transpose
+    grad_weight.shape.copyFrom([co, C, kH, kW]); grad_weight.strides.copyFrom([C * kH * kW, kH * kW, kW, 1])
   let gcol = kcol.transpose * g
   grad_input = newHipTensor[T]([N, C, H, W])
   template fold(f: untyped) =

@@ -235,6 +235,10 @@ template <typename T> static void conv_backward_known_answer() {
   CHECK(r.bias.shape == (Shape{1, 1, 1}) && eq(r.bias, {8}));
   auto nb = am::conv2d_backward(x, k, false, 0, 0, 1, 1, g);
   CHECK(nb.bias.rank() == 0 && eq(nb.weight, {24, 32, 48, 56}));
+  // an output row of four pixels (one 16-byte float vector: the weight gradient gathered from the image): the 2 x 5 image
+  // 1..10 under a 2 x 2 kernel, grad_output all ones; each entry sums four neighbours of its row
+  auto wide = am::conv2d_backward(toHip<T>({1, 2, 3, 4, 5, 6, 7, 8, 9, 10}, {1, 1, 2, 5}), k, false, 0, 0, 1, 1, toHip<T>({1, 1, 1, 1}, {1, 1, 1, 4}));
+  CHECK(eq(wide.weight, {10, 14, 30, 34}) && eq(wide.input, {1, 3, 3, 3, 2, 3, 7, 7, 7, 4}));
   // col2im on its own: the column matrix of ones of that geometry counts the patches over each pixel
   auto ones = toHip<T>(std::vector<T>(16, T(1)), {1, 4, 4});
   CHECK(eq(am::col2im(ones, 1, 3, 3, 2, 2), {1, 2, 1, 2, 4, 2, 1, 2, 1}));

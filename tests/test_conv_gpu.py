@@ -150,6 +150,10 @@ BWD_GEOMS = [  # N, C, H, W, C_out, kH, kW, pad, stride
     (1, 1, 6, 14, 2, 2, 9, (0, 4), (1, 1)),
     (2, 100, 8, 8, 6, 3, 3, (1, 1), (1, 1)),        # more input channels than the one-launch form of grad_input takes on small images
     (1, 100, 24, 24, 6, 3, 3, (1, 1), (1, 1)),      # the same channels on 576 pixels: float32 takes the one-launch form, float64 the product + gather
+    (3, 4, 6, 4, 5, 3, 3, (1, 1), (1, 1)),          # image rows of one float vector: the gathered weight gradient's vectors hang over both edges
+    (2, 3, 7, 12, 6, 2, 5, (0, 4), (1, 1)),         # padding as wide as a float vector
+    (5, 2, 9, 8, 140, 3, 3, (1, 1), (2, 1)),        # window stepping by 2 rows and 1 column; 140 output channels (edge tile of rows), k = 5 * 32 not a slab multiple in float64's tile
+    (70, 3, 10, 10, 8, 3, 3, (0, 0), (1, 1)),       # k = 70 * 64 = 4480: split over workgroups
 ]
 
 
@@ -185,6 +189,14 @@ def test_col2im_and_conv_backward_vs_oracle(hip, oracle, sfx, geom):
     check(oracle, sfx, gb.toCpu(), wb, "grad_bias")
     gi2, gw2, gb2 = hip.conv2d_backward(hip.toHip(x), hip.toHip(k), None, pad, stride, hip.toHip(g))
     assert gb2 is None and np.array_equal(gi2.toCpu(), gi.toCpu()) and np.array_equal(gw2.toCpu(), gw.toCpu())
+    # grad_weight from the written column matrix (where the call above gathered it), and from an input with other strides
+    _, gw3, _ = hip.conv2d_backward(hip.toHip(x), hip.toHip(k), None, pad, stride, hip.toHip(g), need_input_grad=False,
+                                    fused_weight_gradient=False)
+    check(oracle, sfx, gw3.toCpu(), ww, "grad_weight, im2col + product")
+    if C > 1:
+        _, gw4, _ = hip.conv2d_backward(hip.toHip(np.ascontiguousarray(x[:, ::-1]))[:, ::-1], hip.toHip(k), None, pad, stride,
+                                        hip.toHip(g), need_input_grad=False)
+        check(oracle, sfx, gw4.toCpu(), ww, "grad_weight, reversed channel stride")
 
 
 def test_conv_backward_reference_check(hip, oracle):
