@@ -237,3 +237,43 @@ def test_conv_backward_errors(hip):
         hip.conv2d_backward(x, hip.zeros((4, 2, 3, 3), np.float32), None, (0, 0), (1, 1), hip.zeros((2, 4, 3, 3), np.float32))
     with pytest.raises(ValueError):
         hip.col2im(hip.zeros((27, 8), np.float32), 3, 5, 5, (3, 3))                               # 9 columns expected
+
+
+def test_gathered_weight_gradient_entry_point(hip):
+    """am_hip_conv2d_grad_weight_* through the C ABI on its own: the geometries it refuses (AM_E_SHAPE, nothing
+    launched, the result untouched), bad arguments, and a batch of no images, which leaves the result as it is."""
+    import ctypes
+    from arraymancer_amd import _lib
+    L = _lib.load()
+    fn = L.am_hip_conv2d_grad_weight_f32
+    x = hip.toHip(np.ones((2, 3, 6, 8), np.float32))
+    out = hip.toHip(np.full((4, 3, 3, 3), 7, np.float32))
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def call(N, W, pad_w, stride_w, xs=None, g=None, o=out, in_ptr=None):
+        wo = (W + 2 * pad_w - 3) // stride_w + 1
+        g = g if g is not None else hip.toHip(np.ones((4, max(N, 1) * 4 * wo), np.float32))
+        return fn(N, 3, 6, W, 4, 3, 3, 0, pad_w, 1, stride_w, in_ptr if in_ptr is not None else ptr(x), *(xs or x.strides), ptr(g), g.strides[0],
+                  ptr(o) if o is not None else None)
+
+    say("window stepping by two columns")
+    assert call(2, 8, 1, 2) == _lib.AM_E_SHAPE
+    say("output rows of 6 pixels")
+    assert call(2, 8, 0, 1) == _lib.AM_E_SHAPE
+    say("image with stride 2 along the width")
+    assert call(2, 8, 1, 1, xs=(144, 48, 8, 2)) == _lib.AM_E_SHAPE
+    say("null pointers, bad geometry")
+    assert call(2, 8, 1, 1, o=None) == _lib.AM_E_ARG
+    assert call(2, 8, 1, 1, in_ptr=ctypes.c_void_p(0)) == _lib.AM_E_ARG
+    assert fn(2, 3, 6, 8, 4, 0, 3, 0, 1, 1, 1, ptr(x), *x.strides, ptr(x), 8, ptr(out)) == _lib.AM_E_ARG
+    assert "am_hip_conv2d_grad_weight_f32" in _lib.last_error()
+    assert np.array_equal(out.toCpu(), np.full((4, 3, 3, 3), 7, np.float32))
+    say("no images")
+    assert call(0, 8, 1, 1) == _lib.AM_OK and np.array_equal(out.toCpu(), np.full((4, 3, 3, 3), 7, np.float32))
+    say("two images of ones: every entry counts the pixels its window position covers")
+    assert call(2, 8, 1, 1) == _lib.AM_OK
+    got = out.toCpu()
+    want = np.empty((4, 3, 3, 3), np.float32)
+    want[:, :, :, 0] = want[:, :, :, 2] = 2 * 4 * 7      # 4 output rows x 8 output columns, one of them in the padding
+    want[:, :, :, 1] = 2 * 4 * 8
+    assert np.array_equal(got, want)
