@@ -10,7 +10,7 @@ from .metadata import Layout, Step
 from .io_npy import read_npy, write_npy
 from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3, map3, bc_add, bc_div, bc_mod, bc_mul,
                          bc_sub, bias_relu, conv2d, conv2d_into, conv2d_backward, col2im, im2col_folded, dot, empty, gemm, gemm_batched, gemv, im2col, linear, map2, matmul, relu, scalar_op,
-                         sigmoid, sync, toHip, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
+                         sigmoid, sync, toHip, broadcast, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, softmax_cross_entropy, sparse_softmax_cross_entropy,
                          softmax_cross_entropy_backward, sparse_softmax_cross_entropy_backward, sigmoid_cross_entropy,
                          sigmoid_cross_entropy_backward, maxpool2d, tanh, relu_backward, sigmoid_backward,
@@ -22,7 +22,7 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
 
 __all__ = [
     "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
-    "toHip", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "im2col_folded", "col2im", "conv2d", "conv2d_into", "conv2d_backward", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
+    "toHip", "broadcast", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "im2col_folded", "col2im", "conv2d", "conv2d_into", "conv2d_backward", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
     "unary", "relu", "sigmoid", "bias_relu", "bc_add", "bc_sub", "bc_mul", "bc_div", "bc_mod",
     "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward", "gru_cell_inference", "gru_cell_forward", "gru_cell_backward", "gru_inference", "gru_forward", "gru_backward",
     "variance", "std", "sqrt", "square", "argmax_max", "argmax", "argmin_min", "argmin", "maxpool2d_backward",

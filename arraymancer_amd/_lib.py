@@ -60,6 +60,7 @@ def _signatures():
         "am_hip_stream": (vp, []),
         "am_hip_empty_cache": (ci, []),
         "am_hip_memory_stats": (ci, [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
+        "am_hip_device_free_bytes": (ci, [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
         "am_hip_event_create": (ci, [pp]),
         "am_hip_event_record": (ci, [vp]),
         "am_hip_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(ctypes.c_float)]),
@@ -72,6 +73,7 @@ def _signatures():
         "am_hip_diag_peak": (ci, [ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "am_hip_diag_clock_begin": (ci, []),
         "am_hip_diag_clock_end": (ci, [ctypes.POINTER(ctypes.c_double)]),
+        "am_hip_diag_phases": (ci, [ctypes.POINTER(ctypes.c_double)]),
         "am_hip_diag_hbm": (ci, [ci, sz, ci, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
     }
     for sfx, ct in CTYPE.items():

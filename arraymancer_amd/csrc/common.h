@@ -43,6 +43,37 @@ struct ClockProbe {
   }
 };
 
+// Where a short kernel's time goes, read inside it. While a clock window is open (same buffer as ClockProbe, slots 2..8),
+// the first lane of every workgroup reads the constant-rate counter when the kernel body starts and at four marks
+// and adds the four intervals to out[3..6]; out[2] counts the workgroups, out[7] keeps the earliest start (as
+// 2^62 - t, so that a maximum finds it from a zeroed buffer) and out[8] the latest last mark: their difference is the
+// time from the first wavefront's first instruction to the last workgroup's last mark, which the duration the
+// profiler reports for the launch exceeds by the dispatch and end-of-kernel work. settle() drains the wave's memory
+// operations before a mark, only while armed, so that a mark means "arrived", not "issued". Does nothing when `out`
+// is null.
+struct PhaseProbe {
+  long long* out;
+  long long t[5];
+  __device__ __forceinline__ explicit PhaseProbe(long long* o) : out(o) {
+    if (out) t[0] = wall_clock64();
+  }
+  __device__ __forceinline__ void settle() const {
+    if (out) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  }
+  __device__ __forceinline__ void mark(int i) {
+    if (out) t[i] = wall_clock64();
+  }
+  __device__ __forceinline__ void finish() const {
+    if (out && threadIdx.x == 0) {
+      atomicAdd((unsigned long long*)&out[2], 1ull);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) atomicAdd((unsigned long long*)&out[3 + i], (unsigned long long)(t[i + 1] - t[i]));
+      atomicMax(&out[7], (1LL << 62) - t[0]);
+      atomicMax(&out[8], t[4]);
+    }
+  }
+};
+
 #define AM_HIP_TRY(expr)                                                                    \
   do {                                                                                      \
     hipError_t _e = (expr);                                                                 \

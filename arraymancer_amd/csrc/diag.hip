@@ -119,6 +119,30 @@ __global__ __launch_bounds__(256) void peak_valu_mac(int iters, U* out, U seed) 
   if (s == (U)0x1234567) out[0] = s;
 }
 
+// The instruction of the int32 GEMM's inner loop alone: v_mad_u64_u32 (the low half of its 64-bit result is the wrapped
+// 32-bit multiply-accumulate), 32 independent accumulator pairs per lane, operands that never change, written in
+// assembly so that nothing else is in the loop (in C the compiler replaces a loop of constant multiply-adds by its
+// closed form). With the clock window open this gives cycles per instruction on the device, not an estimate.
+__global__ __launch_bounds__(256) void peak_mad_u64_u32(int iters, unsigned long long* out, unsigned seed, long long* clk) {
+  const ClockProbe probe(clk);
+  unsigned long long acc[32];
+  unsigned a[4], b[8];
+  for (int i = 0; i < 4; ++i) a[i] = seed + threadIdx.x * 3u + i;
+  for (int j = 0; j < 8; ++j) b[j] = seed * 7u + threadIdx.x + j * 5u;
+  for (int i = 0; i < 32; ++i) acc[i] = i;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        asm volatile("v_mad_u64_u32 %0, vcc, %1, %2, %0" : "+v"(acc[i * 8 + j]) : "v"(a[i]), "v"(b[j]) : "vcc");
+  }
+  unsigned long long s = 0;
+  for (int i = 0; i < 32; ++i) s += acc[i];
+  if (s == 0x123456789abcull) out[0] = s;
+  probe.finish();
+}
+
 // ---- HBM streams: what the memory system delivers to a kernel that does nothing else --------------
 // One workgroup walks tiles of 256 lanes x UNROLL x 16 bytes (every load instruction of a wavefront
 // covers 1 KiB of consecutive addresses, UNROLL of them in flight per lane), grid-stride over the
@@ -191,7 +215,8 @@ static void launch_hbm_u(int unroll, bool ntl, bool nts, bool chunked, unsigned 
 
 }  // namespace
 
-// HBM stream ceilings. kind: 0 read, 1 write, 2 copy. Each launch moves `bytes` (a multiple of 32 KiB) of
+// HBM stream ceilings. kind: 0 read, 1 write, 2 copy, 3 copy made by the runtime (hipMemcpyAsync device to device over the
+// same windows: not a kernel of this library; blocks_per_cu, unroll and flags do not apply). Each launch moves `bytes` (a multiple of 32 KiB) of
 // a window that rotates through `windows` disjoint buffers (windows * bytes should exceed the 256 MB
 // memory-side cache several times over, so that no launch finds its input there); blocks_per_cu x CUs
 // workgroups; `unroll` (1, 2, 4, 8) 16-byte accesses in flight per lane; flags: bit 0 non-temporal loads,
@@ -199,7 +224,7 @@ static void launch_hbm_u(int unroll, bool ntl, bool nts, bool chunked, unsigned 
 // (read + written) averaged over `launches` launches after `windows` untimed ones.
 extern "C" int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_per_cu, int unroll, int flags, int launches,
                                double* bytes_per_second) {
-  if (!bytes_per_second || kind < 0 || kind > 2 || bytes == 0 || bytes % 32768 != 0 || windows < 1 || windows > 64 ||
+  if (!bytes_per_second || kind < 0 || kind > 3 || bytes == 0 || bytes % 32768 != 0 || windows < 1 || windows > 64 ||
       blocks_per_cu < 1 || blocks_per_cu > 64 || (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8) || launches < 1)
     return fail(AM_E_ARG, "am_hip_diag_hbm: bad argument");
   AM_TRY(ensure_init());
@@ -224,6 +249,7 @@ extern "C" int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_p
     const v4u* s = (const v4u*)(src ? src + off : nullptr);
     v4u* d = (v4u*)(dst ? dst + off : nullptr);
     const bool ntl = flags & 1, nts = flags & 2, chunked = flags & 4;
+    if (kind == 3) { (void)hipMemcpyAsync(d, s, bytes, hipMemcpyDeviceToDevice, stream()); return; }
     if (kind == 0) launch_hbm_u<0>(unroll, ntl, nts, chunked, blocks, s, d, bytes, sink);
     else if (kind == 1) launch_hbm_u<1>(unroll, ntl, nts, chunked, blocks, s, d, bytes, sink);
     else launch_hbm_u<2>(unroll, ntl, nts, chunked, blocks, s, d, bytes, sink);
@@ -239,7 +265,7 @@ extern "C" int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_p
   AM_HIP_TRY(hipEventDestroy(e1));
   (void)hipFree(src); (void)hipFree(dst); (void)hipFree(sink);
   AM_TRY(check_launch("hbm_stream"));
-  *bytes_per_second = (double)bytes * (kind == 2 ? 2.0 : 1.0) * launches / (ms * 1e-3);
+  *bytes_per_second = (double)bytes * (kind >= 2 ? 2.0 : 1.0) * launches / (ms * 1e-3);
   return AM_OK;
 }
 
@@ -278,9 +304,30 @@ extern "C" int am_hip_diag_clock_end(double* shader_mhz) {
   return AM_OK;
 }
 
+// The phase marks of the small-product kernels (PhaseProbe, common.h) collected since am_hip_diag_clock_begin, in
+// microseconds: out[0] workgroups that reported, out[1..4] the mean of each of the four intervals (start -> first loads
+// issued -> arrived -> last matrix instruction and fold -> stores done), out[5] first start to last end over all of
+// them. Meaningful for ONE launch per window. Blocking; the window stays open.
+extern "C" int am_hip_diag_phases(double* out6) {
+  if (!out6) return fail(AM_E_ARG, "am_hip_diag_phases: null pointer");
+  if (!g_clock_armed) return fail(AM_E_ARG, "am_hip_diag_phases: am_hip_diag_clock_begin was not called");
+  long long h[9] = {0};
+  AM_TRY(fetch_result(h, g_clock_buf, sizeof(h)));
+  int khz = 100000;
+  (void)hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, 0);
+  const double us_per_tick = 1e3 / (double)khz;
+  const double n = h[2] > 0 ? (double)h[2] : 1.0;
+  out6[0] = (double)h[2];
+  for (int i = 0; i < 4; ++i) out6[1 + i] = (double)h[3 + i] / n * us_per_tick;
+  out6[5] = h[2] > 0 ? (double)(h[8] - ((1LL << 62) - h[7])) * us_per_tick : 0.0;
+  return AM_OK;
+}
+
 // kind: 0 = MFMA f32 32x32x2 (FLOP/s), 1 = MFMA f64 16x16x4 (FLOP/s),
 //       2 = VALU int32 multiply-add (integer op/s, 2 per MAC), 3 = VALU int64 multiply-add,
-//       4 = MFMA i32 32x32x32 int8 (integer op/s), 5 = LDS reads of 16 bytes per lane (bytes/s).
+//       4 = MFMA i32 32x32x32 int8 (integer op/s), 5 = LDS reads of 16 bytes per lane (bytes/s),
+//       6 = v_mad_u64_u32 alone, in assembly (integer op/s, 2 per instruction and lane; reads the shader clock when a
+//           clock window is open).
 // Launches `waves_per_simd` wavefronts on every SIMD of the device, `iters` loop trips each.
 extern "C" int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second) {
   if (!ops_per_second || iters <= 0 || waves_per_simd < 1 || waves_per_simd > 8)
@@ -319,6 +366,11 @@ extern "C" int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double*
       case 5:
         hipLaunchKernelGGL(peak_lds_read, dim3(blocks), dim3(256), 0, stream(), iters, (int*)scratch);
         ops_per_launch = (double)blocks * 256 * iters * 8 * 16.0;   // bytes
+        break;
+      case 6:
+        hipLaunchKernelGGL(peak_mad_u64_u32, dim3(blocks), dim3(256), 0, stream(), iters, (unsigned long long*)scratch, 12345u,
+                           clock_probe_buffer());
+        ops_per_launch = (double)blocks * 256 * iters * 32 * 2.0;
         break;
       default:
         (void)hipFree(scratch);

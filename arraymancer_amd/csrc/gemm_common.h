@@ -390,7 +390,11 @@ static inline int choose_tile_and_split(Args<T>& g, const TileChoice* cand, int 
   g.want_splits = 0;
   const int by_rounds = choose_tile(cand, ncand, g.M, g.N, env, g.batch);
   const char* forced = getenv(env);
-  if ((forced && *forced) || g.batch > 1 || g.static_ws) return by_rounds;
+  if ((forced && *forced) || g.batch > 1) return by_rounds;
+  // what the partial tiles of a plan may take: the workspace's share, or the whole static array of the allocation-free
+  // entry point (which therefore runs the same plan as the allocating one wherever that plan fits its array)
+  double partials_limit = 48.0 * 1024 * 1024;
+  if (g.static_ws) { size_t cap = 0; (void)static_scratch(&cap); partials_limit = (double)cap; }
   static const bool joint = [] { const char* e = getenv("AM_HIP_GEMM_JOINT"); return !(e && *e == '0'); }();
   if (!joint) return by_rounds;
   const int64_t cus = num_cus();
@@ -404,7 +408,7 @@ static inline int choose_tile_and_split(Args<T>& g, const TileChoice* cand, int 
     const int64_t chunk = (slabs + sp_in - 1) / sp_in;
     const int64_t sp = (slabs + chunk - 1) / chunk;
     *sp_out = sp;
-    if (sp > 1 && (double)sp * g.M * g.N * sizeof(T) > 48.0 * 1024 * 1024) return -1.0;
+    if (sp > 1 && (double)sp * g.M * g.N * sizeof(T) > partials_limit) return -1.0;
     // a slab's time: the matrix instructions; a workgroup alone on its CU cannot go below what its chain of LDS and
     // barrier waits allows (measured on the 32 x 32 tile: 0.23 us per slab of 32 k)
     double slab_us = 2.0 * c.bm * c.bn * bk / (flops_per_cu_us * c.eff);

@@ -41,6 +41,7 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
   __shared__ __attribute__((aligned(16))) T sB[2][BK * LDB];
 
   if (p.gate_flags != nullptr && live_digit_pairs<(int)sizeof(T)>(p.gate_flags, p.gate_gen) <= p.gate_max_pairs) return;
+  const ClockProbe probe(p.clock_out);
   int tile_m, tile_n, bid = (int)blockIdx.x, split = 0;
   if (p.splits > 1) {
     const int nt = p.tiles_m * p.tiles_n;
@@ -124,6 +125,7 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
         if (col < p.N) ws[row * p.N + col] = (T)(U)acc[i][j];
       }
     }
+    probe.finish();
     return;
   }
   const U alpha = (U)p.alpha, beta = (U)p.beta;
@@ -151,6 +153,7 @@ __global__ __launch_bounds__(256, 2) void gemm_valu(Args<T> p) {
       }
     }
   }
+  probe.finish();
 }
 
 template <typename T, int TM, int TN, int BK>

@@ -66,6 +66,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   typedef typename M16<T>::acc_t acc_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][256] partial tiles, W > 1 only
   T (*red)[256] = reinterpret_cast<T (*)[256]>(red_raw);
+  PhaseProbe probe(p.clock_out);   // marks: 1 first loads issued, 2 they have arrived, 3 last matrix instruction and fold, 4 stores done
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int i = lane & 15, g = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * 16;
@@ -117,6 +118,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   int64_t blk = blk0;
   if (nchunks > 0) {
     load_chunk(0, blk0);
+    probe.mark(1);
+    probe.settle();
+    probe.mark(2);
     int64_t c = 0;
     for (; c + 2 <= nchunks; c += 2) {
       load_chunk(1, blk0 + (c + 1) * CHUNK);
@@ -150,6 +154,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
     for (int s = 0; s < 4; ++s) acc = M16<T>::mma(tail_a[s], tail_b[s], acc);
   }
 
+  if (nchunks <= 0) { probe.mark(1); probe.settle(); probe.mark(2); }
   if (nw > 1) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][r * 64 + lane] = acc[r];
@@ -162,6 +167,8 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
       acc[r] = sum;
     }
   }
+  if (probe.out) { acc_t pin = acc; asm volatile("s_nop 0" : "+v"(pin)); acc = pin; }   // the accumulators are final before the mark is read
+  probe.mark(3);
 
   // Epilogue (gemm_ukernel_generic.nim:53-125): beta == 0 never reads C; C *= beta, then
   // C += alpha * AB, each rounded on its own; then the optional fused bias / ReLU.
@@ -193,6 +200,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
       p.C[row * p.c_m + col * p.c_n] = v;
     }
   }
+  probe.settle();
+  probe.mark(4);
+  probe.finish();
 }
 
 // The same product when B has unit stride along n (a row-major [k x n] operand, e.g. x * W with W stored
@@ -210,6 +220,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   typedef T vec_t __attribute__((ext_vector_type(VN)));
   extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][VN][256] partial tiles, W > 1 only
   T (*red)[VN * 256] = reinterpret_cast<T (*)[VN * 256]>(red_raw);
+  PhaseProbe probe(p.clock_out);   // marks as in gemm_rows16
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int i = lane & 15, g = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * (16 * VN);
@@ -269,6 +280,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   int64_t blk = blk0;
   if (nchunks > 0) {
     load_blocks(0, blk0, CHUNK);
+    probe.mark(1);
+    probe.settle();
+    probe.mark(2);
     int64_t c = 0;
     for (; c + 2 <= nchunks; c += 2) {
       load_blocks(1, blk0 + (c + 1) * CHUNK, CHUNK);
@@ -295,6 +309,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
       for (int j = 0; j < VN; ++j) acc[j] = M16<T>::mma(tail_a[s], tail_b[s][j], acc[j]);
   }
 
+  if (nchunks <= 0) { probe.mark(1); probe.settle(); probe.mark(2); }
   if (nw > 1) {
 #pragma unroll
     for (int j = 0; j < VN; ++j)
@@ -316,11 +331,12 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   const T alpha = p.alpha, beta = p.beta;
   const bool has_bias = (p.epilogue & AM_EPI_BIAS) != 0, relu = (p.epilogue & AM_EPI_RELU) != 0;
   const bool cvec = p.c_n == 1;
-  if (col0 >= p.N) return;
+  if (probe.out) { acc_t pin = acc[0]; asm volatile("s_nop 0" : "+v"(pin)); acc[0] = pin; }
+  probe.mark(3);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int64_t row = m0 + M16<T>::acc_row(r, lane);
-    if (row >= p.M) continue;
+    if (row >= p.M || col0 >= p.N) continue;
     T* c = p.C + row * p.c_m + col0 * p.c_n;
     vec_t old = vec_t{};
     if (beta != (T)0) {
@@ -351,6 +367,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
       for (int j = 0; j < VN; ++j) c[j * p.c_n] = out[j];
     }
   }
+  probe.settle();
+  probe.mark(4);
+  probe.finish();
 }
 
 // Whether this product belongs here: few rows or few columns, little work, not a batch member.

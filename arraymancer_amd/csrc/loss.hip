@@ -182,6 +182,9 @@ __global__ __launch_bounds__(256) void sce_backward(Args<T> p, int lanes) {
   if (!ok) continue;
   int64_t label = -1;
   if constexpr (!DENSE) label = p.labels[row * p.l_s];
+  // A label outside the row cannot raise on the device: its gradient row becomes NaN, as the forward pass makes the
+  // loss NaN, so that a bad label shows instead of training on silently.
+  const bool bad_label = !DENSE && (label < 0 || label >= p.cols);
   T* out = p.out + row * p.o_rs;
   const int64_t units = p.cols / V;
   for (int64_t u0 = j0; u0 < units; u0 += (int64_t)lanes * U) {
@@ -209,7 +212,7 @@ __global__ __launch_bounds__(256) void sce_backward(Args<T> p, int lanes) {
         const T sm = dev_exp<T>(xv[k][e] - m) / s;
         // dense: softmax - target; sparse: softmax + (-1 at the label, 0 elsewhere)
         const T inner = DENSE ? sm - tv[k][e] : sm + ((u * V + e == label) ? (T)-1 : (T)0);
-        y[e] = p.grad * inner / p.batch;
+        y[e] = bad_label ? (T)NAN : p.grad * inner / p.batch;
       }
       if constexpr (VEC) __builtin_nontemporal_store(y, (vec_t*)(out + u * V));
       else out[u * p.o_cs] = y[0];

@@ -4,6 +4,7 @@
 #include <stdarg.h>
 #include <stdlib.h>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 #include <string.h>
 #include "common.h"
@@ -125,6 +126,10 @@ static std::vector<void*> g_capture_freed;
 static bool g_hold = false;
 static std::vector<void*> g_held;
 static std::unordered_map<void*, std::vector<void*>> g_graph_blocks;   // executable graph -> blocks it keeps alive
+// Every executable graph am_hip_graph_end has handed out and am_hip_graph_destroy has not yet taken back: launch and
+// destroy refuse any other pointer (a stale, foreign or twice-destroyed handle would otherwise crash inside the runtime,
+// and a second destroy would hand the graph's blocks to the cache twice).
+static std::unordered_set<void*> g_graphs;
 
 // Hands a live block back: to the cache, or to the driver when the cache is full. g_alloc_mu held.
 static int free_block_locked(void* dptr) {
@@ -279,6 +284,15 @@ int am_hip_memory_stats(size_t* live_bytes, size_t* cached_bytes) {
   return AM_OK;
 }
 
+int am_hip_device_free_bytes(size_t* free_bytes, size_t* total_bytes) {
+  AM_TRY(ensure_init());
+  size_t f = 0, t = 0;
+  AM_HIP_TRY(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return AM_OK;
+}
+
 int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return AM_OK;
   if (!dst || !src) return fail(AM_E_ARG, "am_hip_memcpy_h2d: null pointer");
@@ -370,12 +384,18 @@ int am_hip_graph_end(void** graph_exec) {
   }
   if (!g_capture_freed.empty()) g_graph_blocks[(void*)exec] = std::move(g_capture_freed);
   g_capture_freed.clear();
+  g_graphs.insert((void*)exec);
   *graph_exec = (void*)exec;
   return AM_OK;
 }
 
 int am_hip_graph_launch(void* graph_exec) {
   if (!graph_exec) return fail(AM_E_ARG, "am_hip_graph_launch: null graph");
+  {   // (before anything touches the device: an unknown handle is refused on a machine without one too)
+    std::lock_guard<std::mutex> lk(g_alloc_mu);
+    if (!g_graphs.count(graph_exec))
+      return fail(AM_E_ARG, "am_hip_graph_launch: %p is not a graph of am_hip_graph_end (or was destroyed)", graph_exec);
+  }
   AM_TRY(ensure_init());
   if (g_capturing) return fail(AM_E_ARG, "am_hip_graph_launch: not allowed while a graph is being captured");
   AM_HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, g_stream));
@@ -384,6 +404,11 @@ int am_hip_graph_launch(void* graph_exec) {
 
 int am_hip_graph_destroy(void* graph_exec) {
   if (!graph_exec) return AM_OK;
+  {
+    std::lock_guard<std::mutex> lk(g_alloc_mu);
+    if (!g_graphs.erase(graph_exec))
+      return fail(AM_E_ARG, "am_hip_graph_destroy: %p is not a graph of am_hip_graph_end (or was destroyed already)", graph_exec);
+  }
   AM_HIP_TRY(hipStreamSynchronize(g_stream));
   AM_HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
   std::lock_guard<std::mutex> lk(g_alloc_mu);

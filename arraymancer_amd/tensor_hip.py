@@ -58,11 +58,32 @@ class HipStorage:
                 warnings.warn(f"am_hip_free failed ({rc}): {_lib.last_error()}", ResourceWarning)
 
 
+# Unsigned element types ride the kernels of their signed twins, like the reference's GEMM overload for
+# uint32 | uint64 | uint | int (laser/primitives/matrix_multiplication/gemm.nim:275-307: the pointers are cast onto the
+# int32 / int64 kernels). In the rings Z/2^32 and Z/2^64 the bits of + - * (hence of GEMM, gemv, dot, sums and
+# products, x*y+z) do not depend on how the operands are read; division, remainder, comparisons, min / max and
+# everything float-valued do, and are refused for these types.
+_UNSIGNED_TWIN = {np.dtype(np.uint32): "i32", np.dtype(np.uint64): "i64"}
+_RING_OPS = frozenset(("add", "sub", "mul"))
+_RING_UOPS = frozenset(("copy", "neg"))
+_RING_OP3 = frozenset(("muladd", "addmul"))
+_RING_RED = frozenset(("sum", "product"))
+
+
 def _dtype_sfx(dtype) -> str:
     try:
         return SFX[np.dtype(dtype)]
     except KeyError:
-        raise TypeError(f"HipTensor supports float32, float64, int32 and int64, not {dtype}")
+        if np.dtype(dtype) in _UNSIGNED_TWIN:
+            return _UNSIGNED_TWIN[np.dtype(dtype)]
+        raise TypeError(f"HipTensor supports float32, float64, int32, int64 (and uint32 / uint64 for + - * and "
+                        f"products), not {dtype}")
+
+
+def _ring_scalar(sfx: str, dtype, value):
+    """The scalar argument of a ring operation as the kernel's C type: an unsigned value above the signed twin's
+    range is passed as the same bits (ctypes integer types wrap instead of raising)."""
+    return CTYPE[sfx](int(value) if np.dtype(dtype).kind in "iu" else value)
 
 
 # Element types a HipTensor can hold as the RESULT of a map whose body changes the type (Tensor[bool] of the
@@ -104,7 +125,16 @@ class HipTensor:
         try:
             return SFX[self.dtype]
         except KeyError:
+            if self.dtype in _UNSIGNED_TWIN:
+                raise TypeError(f"this operation reads the sign of its operands and is not defined on a HipTensor of "
+                                f"{self.dtype}: unsigned tensors support + - *, matrix products, sums and products")
             raise TypeError(f"no arithmetic is defined on a HipTensor of {self.dtype}")
+
+    @property
+    def ring_sfx(self) -> str:
+        """Kernel suffix for an operation of the ring Z/2^n (+ - * and what is built from them): an unsigned tensor
+        takes the kernels of its signed twin (gemm.nim:275-307)."""
+        return _UNSIGNED_TWIN.get(self.dtype) or self.sfx
 
     def data_ptr(self) -> int:
         """Device address of element [0, 0, ...] (get_offset_ptr, data_structure.nim:206-211)."""
@@ -305,6 +335,26 @@ def toHip(arr) -> HipTensor:
     return t
 
 
+def broadcast(val, shape: Sequence[int], dtype=None) -> HipTensor:
+    """`broadcast(val, shape)` (src/arraymancer/tensor/shapeshifting.nim:136-176): a tensor of `shape` whose every
+    element is `val` - ONE element of storage, every stride 0. Like the reference's, it must not be written through
+    (all positions share the element); `clone` / `asContiguous` materialise it. A HipTensor as first argument is the
+    tensor form (explicit broadcast of its size-1 dimensions)."""
+    if isinstance(val, HipTensor):
+        return val.broadcast(shape)
+    if dtype is None:
+        dtype = np.asarray(val).dtype
+        if dtype == np.dtype(np.int_) and dtype not in SFX:
+            dtype = np.dtype(np.int64)
+    dtype = np.dtype(dtype)
+    _dtype_sfx(dtype)
+    one = toHip(np.full((1,), val, dtype=dtype))
+    shape = tuple(int(d) for d in shape)
+    if any(d < 0 for d in shape) or len(shape) > _lib.AM_MAXRANK:
+        raise ValueError(f"broadcast: invalid shape {list(shape)}")
+    return HipTensor(Layout(shape, (0,) * len(shape), 0), one.storage, dtype)
+
+
 def sync() -> None:
     check(_lib.load().am_hip_sync())
 
@@ -399,10 +449,9 @@ def gemm(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none",
     if C.shape != (M, N):
         raise IndexError(f"gemm: C has shape {list(C.shape)}, expected {[M, N]}")
     L = _lib.load()
-    sfx = C.sfx
-    ct = CTYPE[sfx]
-    args = [M, N, K, ct(alpha), ctypes.c_void_p(A.data_ptr()), A.strides[0], A.strides[1],
-            ctypes.c_void_p(B.data_ptr()), B.strides[0], B.strides[1], ct(beta),
+    sfx = C.ring_sfx
+    args = [M, N, K, _ring_scalar(sfx, dtype, alpha), ctypes.c_void_p(A.data_ptr()), A.strides[0], A.strides[1],
+            ctypes.c_void_p(B.data_ptr()), B.strides[0], B.strides[1], _ring_scalar(sfx, dtype, beta),
             ctypes.c_void_p(C.data_ptr()), C.strides[0], C.strides[1]]
     epi = EPI[epilogue] if isinstance(epilogue, str) else int(epilogue)
     if epi != 0:
@@ -451,10 +500,10 @@ def gemv(alpha, A: HipTensor, x: HipTensor, beta, y: HipTensor) -> HipTensor:
                          f"of rows in the vector: {x.shape[0]}")
     if y.shape[0] != A.shape[0]:
         raise IndexError(f"gemv: y has {y.shape[0]} elements, expected {A.shape[0]}")
-    ct = CTYPE[y.sfx]
-    check(getattr(_lib.load(), f"am_hip_gemv_{y.sfx}")(
-        A.shape[0], A.shape[1], ct(alpha), ctypes.c_void_p(A.data_ptr()), A.strides[0], A.strides[1],
-        ctypes.c_void_p(x.data_ptr()), x.strides[0], ct(beta), ctypes.c_void_p(y.data_ptr()), y.strides[0]))
+    sfx = y.ring_sfx
+    check(getattr(_lib.load(), f"am_hip_gemv_{sfx}")(
+        A.shape[0], A.shape[1], _ring_scalar(sfx, y.dtype, alpha), ctypes.c_void_p(A.data_ptr()), A.strides[0], A.strides[1],
+        ctypes.c_void_p(x.data_ptr()), x.strides[0], _ring_scalar(sfx, y.dtype, beta), ctypes.c_void_p(y.data_ptr()), y.strides[0]))
     return y
 
 
@@ -464,12 +513,20 @@ def dot(a: HipTensor, b: HipTensor):
     _same_dtype(a, b)
     if a.rank != 1 or b.rank != 1 or a.shape != b.shape:
         raise ValueError(f"dot: both operands must be vectors of the same length, got {list(a.shape)} and {list(b.shape)}")
-    ct = CTYPE[a.sfx]
-    out = ct()
-    check(getattr(_lib.load(), f"am_hip_dot_{a.sfx}")(
+    sfx = a.ring_sfx
+    out = CTYPE[sfx]()
+    check(getattr(_lib.load(), f"am_hip_dot_{sfx}")(
         a.shape[0], ctypes.c_void_p(a.data_ptr()), a.strides[0], ctypes.c_void_p(b.data_ptr()), b.strides[0],
         ctypes.byref(out)))
-    return a.dtype.type(out.value)
+    return _host_scalar(a.dtype, out.value)
+
+
+def _host_scalar(dtype, value):
+    """A kernel's scalar result as the tensor's element type (an unsigned tensor's result arrives in its signed twin)."""
+    dtype = np.dtype(dtype)
+    if dtype in _UNSIGNED_TWIN:
+        return dtype.type(int(value) % (1 << (8 * dtype.itemsize)))
+    return dtype.type(value)
 
 
 def gemm_batched(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none", bias: HipTensor | None = None):
@@ -897,7 +954,7 @@ def gru_backward(dOutput: HipTensor, dHiddenN: HipTensor, cache, W3s0: HipTensor
 
 # ---------------------------------------------------------------------- element-wise
 def _binary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor):
-    sfx = dst.sfx
+    sfx = dst.ring_sfx if op in _RING_OPS else dst.sfx
     code = OP[op] if isinstance(op, str) else int(op)
     check(getattr(_lib.load(), f"am_hip_ew_binary_{sfx}")(
         code, dst.rank, i64_array(dst.shape),
@@ -907,16 +964,17 @@ def _binary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor):
 
 
 def _scalar_into(op, dst: HipTensor, a: HipTensor, scalar, left: bool):
-    sfx = dst.sfx
+    sfx = dst.ring_sfx if op in _RING_OPS else dst.sfx
     code = OP[op] if isinstance(op, str) else int(op)
     check(getattr(_lib.load(), f"am_hip_ew_scalar_{sfx}")(
         code, int(bool(left)), dst.rank, i64_array(dst.shape),
         ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
-        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides), CTYPE[sfx](scalar)))
+        ctypes.c_void_p(a.data_ptr()), i64_array(a.strides),
+        _ring_scalar(sfx, dst.dtype, scalar) if dst.dtype in _UNSIGNED_TWIN else CTYPE[sfx](scalar)))
 
 
 def _unary_into(op, dst: HipTensor, a: HipTensor):
-    sfx = dst.sfx
+    sfx = dst.ring_sfx if op in _RING_UOPS else dst.sfx
     code = UOP[op] if isinstance(op, str) else int(op)
     check(getattr(_lib.load(), f"am_hip_ew_unary_{sfx}")(
         code, dst.rank, i64_array(dst.shape),
@@ -929,6 +987,7 @@ def map2(op, a: HipTensor, b: HipTensor) -> HipTensor:
     already have equal shapes (src/arraymancer/tensor/higher_order_applymap.nim:92-120)."""
     _same_dtype(a, b)
     _check_elementwise(a, b)
+    _ = a.ring_sfx if op in _RING_OPS else a.sfx      # (refuses before anything is allocated)
     if op in CMP:   # a body with a bool result: the output type follows the body, like the reference's template
         out = empty(a.shape, np.bool_)
         if out.size:
@@ -955,7 +1014,7 @@ def _compare_into(cmp, dst: HipTensor, a: HipTensor, b: HipTensor):
 
 def _ternary_into(op, dst: HipTensor, a: HipTensor, b: HipTensor, c: HipTensor):
     code = OP3[op] if isinstance(op, str) else int(op)
-    check(getattr(_lib.load(), f"am_hip_ew_ternary_{dst.sfx}")(
+    check(getattr(_lib.load(), f"am_hip_ew_ternary_{dst.ring_sfx if op in _RING_OP3 else dst.sfx}")(
         code, dst.rank, i64_array(dst.shape), ctypes.c_void_p(dst.data_ptr()), i64_array(dst.strides),
         ctypes.c_void_p(a.data_ptr()), i64_array(a.strides), ctypes.c_void_p(b.data_ptr()), i64_array(b.strides),
         ctypes.c_void_p(c.data_ptr()), i64_array(c.strides)))
@@ -967,6 +1026,7 @@ def map3(op, a: HipTensor, b: HipTensor, c: HipTensor) -> HipTensor:
     _same_dtype(a, b, c)
     _check_elementwise(a, b)
     _check_elementwise(a, c)
+    _ = a.ring_sfx if op in _RING_OP3 else a.sfx
     out = empty(a.shape, a.dtype)
     if out.size:
         _ternary_into(op, out, a, b, c)
@@ -1034,6 +1094,7 @@ def _bc_compare(cmp, a, b) -> HipTensor:
     if not (ta or tb):
         raise TypeError("at least one operand must be a HipTensor")
     t, value, cmp = (a, b, cmp) if ta else (b, a, _MIRROR[cmp])
+    _ = t.sfx
     out = empty(t.shape, np.bool_)      # returnEmptyIfEmpty: an empty tensor comes back empty
     if out.size:
         check(getattr(_lib.load(), f"am_hip_ew_compare_scalar_{t.sfx}")(
@@ -1083,6 +1144,7 @@ def classify(t: HipTensor) -> HipTensor:
 def sgn(t: HipTensor) -> HipTensor:
     """int64 tensor (the reference's Tensor[int]) of -1 / 0 / 1; zeros and NaN give 0
     (src/arraymancer/tensor/math_functions.nim:110-117)."""
+    _ = t.sfx
     out = empty(t.shape, np.int64)
     if out.size:
         check(getattr(_lib.load(), f"am_hip_ew_sgn_{t.sfx}")(
@@ -1133,6 +1195,7 @@ def _bc_inplace(op, a: HipTensor, b):
 
 
 def scalar_op(op, t: HipTensor, scalar, scalar_on_left: bool = False) -> HipTensor:
+    _ = t.ring_sfx if op in _RING_OPS else t.sfx
     out = empty(t.shape, t.dtype)
     if t.size:
         _scalar_into(op, out, t, scalar, scalar_on_left)
@@ -1140,6 +1203,7 @@ def scalar_op(op, t: HipTensor, scalar, scalar_on_left: bool = False) -> HipTens
 
 
 def unary(op, t: HipTensor) -> HipTensor:
+    _ = t.ring_sfx if op in _RING_UOPS else t.sfx
     out = empty(t.shape, t.dtype)
     if t.size:
         _unary_into(op, out, t)
@@ -1248,6 +1312,7 @@ def _clamp_into(dst: HipTensor, t: HipTensor, lo, hi):
 def clamp(t: HipTensor, min, max) -> HipTensor:
     """map_inline(clamp(x, min, max)): min where x < min, max where x > max, else x
     (src/arraymancer/tensor/math_functions.nim:146-148). One pass."""
+    _ = t.sfx
     out = empty(t.shape, t.dtype)
     if out.size:
         _clamp_into(out, t, min, max)
@@ -1277,6 +1342,7 @@ def reduce_axis(op, t: HipTensor, axis: int) -> HipTensor:
     (returnEmptyIfEmpty, aggregate.nim:40); an axis outside the rank raises IndexError."""
     if not 0 <= axis < t.rank:
         raise IndexError(f"Input tensor rank ({t.rank}) must be greater than reduction axis ({axis})")
+    _ = t.ring_sfx if op in _RING_RED else t.sfx
     if t.size == 0:
         return empty(t.shape, t.dtype)
     shape = list(t.shape)
@@ -1290,7 +1356,7 @@ def reduce_axis_into(op, out: HipTensor, t: HipTensor, axis: int) -> HipTensor:
     _same_dtype(out, t)
     if out.rank != t.rank or any(o != (1 if d == axis else n) for d, (o, n) in enumerate(zip(out.shape, t.shape))):
         raise ValueError(f"reduce_axis_into: result {out.shape} does not fit {t.shape} folded along axis {axis}")
-    check(getattr(_lib.load(), f"am_hip_reduce_axis_{t.sfx}")(
+    check(getattr(_lib.load(), f"am_hip_reduce_axis_{t.ring_sfx if op in _RING_RED else t.sfx}")(
         RED[op], t.rank, i64_array(t.shape), axis, ctypes.c_void_p(out.data_ptr()), i64_array(out.strides),
         ctypes.c_void_p(t.data_ptr()), i64_array(t.strides)))
     return out
@@ -1333,10 +1399,11 @@ def argmin(t: HipTensor, axis: int) -> HipTensor:
 
 def reduce_all(op, t: HipTensor):
     """reduce_inline (higher_order_foldreduce.nim:22-31): fold of every element, returned to the host."""
-    out = CTYPE[t.sfx]()
-    check(getattr(_lib.load(), f"am_hip_reduce_all_{t.sfx}")(
+    sfx = t.ring_sfx if op in _RING_RED else t.sfx
+    out = CTYPE[sfx]()
+    check(getattr(_lib.load(), f"am_hip_reduce_all_{sfx}")(
         RED[op], t.rank, i64_array(t.shape), ctypes.c_void_p(t.data_ptr()), i64_array(t.strides), ctypes.byref(out)))
-    return t.dtype.type(out.value)
+    return _host_scalar(t.dtype, out.value)
 
 
 def _aggregate(op):
@@ -1357,6 +1424,8 @@ tmax = _aggregate("max")
 
 def mean(t: HipTensor, axis: int | None = None):
     """aggregate.nim:58-86: the sum divided by the element count; integer tensors use `div`."""
+    if t.dtype in _UNSIGNED_TWIN:
+        raise TypeError("mean divides, which reads the sign of its operands: not defined on unsigned HipTensors")
     if axis is None:
         s = reduce_all("sum", t)
         if t.dtype.kind == "f":

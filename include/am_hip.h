@@ -67,6 +67,9 @@ int am_hip_free(void* dptr);                   /* NULL is a no-op. While a graph
  * Cache size limit: environment variable AM_HIP_CACHE_LIMIT_MB (default 32768; 0 = no caching). */
 int am_hip_empty_cache(void);
 int am_hip_memory_stats(size_t* live_bytes, size_t* cached_bytes);
+/* Free and total device memory as the driver reports them (hipMemGetInfo): unlike am_hip_memory_stats this sees
+ * every allocation of the process, the library's own workspaces included. No counterpart in the reference. */
+int am_hip_device_free_bytes(size_t* free_bytes, size_t* total_bytes);
 int am_hip_memcpy_h2d(void* dst, const void* src, size_t bytes);  /* host buffer reusable on return */
 int am_hip_memcpy_d2h(void* dst, const void* src, size_t bytes);  /* blocking, ordered after prior work */
 int am_hip_memcpy_d2d(void* dst, const void* src, size_t bytes);  /* stream ordered */
@@ -100,6 +103,9 @@ int am_hip_graph_begin(void);
  * reference. */
 int am_hip_alloc_hold(int on);
 int am_hip_graph_end(void** graph_exec);
+/* Both accept only a graph that am_hip_graph_end returned and am_hip_graph_destroy has not taken back yet: any other
+ * pointer (stale, destroyed twice, foreign) is refused with AM_E_ARG instead of reaching the runtime. NULL: launch
+ * refuses it, destroy ignores it. */
 int am_hip_graph_launch(void* graph_exec);
 int am_hip_graph_destroy(void* graph_exec);
 
@@ -146,8 +152,13 @@ int am_hip_gemm_i64(int64_t M, int64_t N, int64_t K, int64_t alpha,
 
 /* am_hip_gemm_f32 for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
- * arguments, kernels and result bits as am_hip_gemm_f32; the difference is where the split-K partial
- * tiles go (products with few output tiles and a long K are cut along K over several workgroups):
+ * arguments and kernels as am_hip_gemm_f32, and the same tile and split of K - hence the same result
+ * bits - wherever am_hip_gemm_f32's own plan keeps its partial tiles within 16 MiB and cuts no strips
+ * off (it runs extents of 512 or more that lie 1..16 above a multiple of 64 as an aligned block plus
+ * strips; this entry point runs them whole). Outside those cases this entry point takes the best plan
+ * that fits its array: both results meet the float32 bar, the last bits may differ. The difference is
+ * where the split-K partial tiles go (products with few output tiles and a long K are cut along K
+ * over several workgroups):
  * am_hip_gemm_f32 takes a workspace from hipMalloc on first use, this entry point uses a 16 MiB
  * array that is part of the library's device code and calls no hipMalloc / hipFree nor any routine
  * that allocates. Each device the library runs on holds that array until the process ends.
@@ -657,7 +668,7 @@ int am_hip_softmax_cross_entropy_backward_f64(int64_t rows, int64_t cols, double
                                               int64_t in_cs, const double* target, int64_t t_rs, int64_t t_cs,
                                               double* result, int64_t r_rs, int64_t r_cs);
 /* result[i, j] <- gradient * (softmax(input[i, :])[j] - (j == labels[i] ? 1 : 0)) / rows. A label outside [0, cols)
- * leaves its row the plain softmax term. Replaces sparse_softmax_cross_entropy_backward
+ * makes its row of the result NaN (the forward pass makes the loss NaN for the same input). Replaces sparse_softmax_cross_entropy_backward
  * (nnp_softmax_cross_entropy.nim:217-256). */
 int am_hip_sparse_softmax_cross_entropy_backward_f32(int64_t rows, int64_t cols, float gradient, const float* input,
                                                      int64_t in_rs, int64_t in_cs, const int64_t* labels, int64_t labels_s,
@@ -722,10 +733,14 @@ int am_hip_maxpool2d_backward_i64(int64_t N, int C, int H, int W, int kH, int kW
  *   kind 3: VALU int64 multiply-add
  *   kind 4: MFMA int8 32x32x32 (integer op/s), the instruction of the digit-sliced integer GEMM
  *   kind 5: LDS reads of 16 bytes per lane, no bank conflicts (bytes/s over the whole device)
+ *   kind 6: v_mad_u64_u32 alone (the int32 GEMM's multiply-accumulate instruction; integer op/s, 2 per lane and
+ *           instruction), written in assembly with constant operands; between am_hip_diag_clock_begin and _end it
+ *           also reads the shader clock, which turns the rate into cycles per instruction
  * waves_per_simd wavefronts are resident on every SIMD (1..8); iters loop trips each. */
 int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_second);
 /* What HBM delivers to a kernel that only streams: kind 0 reads, 1 writes, 2 copies `bytes` (a multiple of
- * 32 KiB) per launch with 16-byte accesses, `unroll` (1, 2, 4, 8) of them in flight per lane, from
+ * 32 KiB) per launch (kind 3: the same copy made by the runtime's own hipMemcpyAsync, device to device, as a
+ * figure that no kernel of this library is part of; blocks_per_cu, unroll and flags are ignored) with 16-byte accesses, `unroll` (1, 2, 4, 8) of them in flight per lane, from
  * blocks_per_cu x CUs workgroups of 256 lanes. Launches rotate through `windows` disjoint buffers of `bytes`
  * each (allocated and freed inside the call), so that with windows * bytes several times the 256 MB
  * memory-side cache every byte comes from HBM. flags: bit 0 non-temporal loads, bit 1 non-temporal stores,
@@ -735,12 +750,20 @@ int am_hip_diag_peak(int kind, int iters, int waves_per_simd, double* ops_per_se
 int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_per_cu, int unroll, int flags, int launches,
                     double* bytes_per_second);
 /* The shader clock the device sustains under the matrix-core GEMM kernels: between _begin and _end the first
- * lane of workgroup 0 of every gemm_mfma / gemm_i8_digits launch compares the shader-cycle counter with the
+ * lane of workgroup 0 of every gemm_mfma / gemm_i8_digits / gemm_valu launch (and of the kind-6 chain above) compares the shader-cycle counter with the
  * constant-rate counter over the kernel's own lifetime; _end (blocking) returns cycles / ticks as MHz, averaged
  * over those launches (0 if none ran). The matrix peaks are quoted at 2.4 GHz; a power-limited kernel settles
  * lower, and its fraction of peak is read against that. */
 int am_hip_diag_clock_begin(void);
 int am_hip_diag_clock_end(double* shader_mhz);
+/* Where the time of a small-product launch (min(M, N) <= 64: the kernels without LDS staging) goes, read inside the
+ * kernel between am_hip_diag_clock_begin and _end by the first lane of every workgroup, in microseconds: out6[0]
+ * workgroups that reported; out6[1..4] the mean time from the first instruction to the first loads issued, from there
+ * until they have arrived, from there to the last matrix instruction and the fold of the wavefronts' partial tiles,
+ * and from there until the stores are done; out6[5] from the earliest first instruction to the latest store over the
+ * whole launch (what the launch's duration on a profiler's timeline exceeds by the dispatch and end-of-kernel work).
+ * One launch per window. No counterpart in the reference. */
+int am_hip_diag_phases(double* out6);
 
 #ifdef __cplusplus
 }

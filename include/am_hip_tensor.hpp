@@ -147,6 +147,54 @@ AM_HPP_BIND(double, f64)
 AM_HPP_BIND(int32_t, i32)
 AM_HPP_BIND(int64_t, i64)
 #undef AM_HPP_BIND
+// Unsigned element types ride the kernels of their signed twins, like the reference's GEMM overload for
+// uint32 | uint64 | uint | int (laser/primitives/matrix_multiplication/gemm.nim:275-307: the pointers are cast onto the
+// int32 / int64 kernels). In the rings Z/2^32 and Z/2^64 the bits of + - * (hence of matrix products, dot, sums and
+// products of elements) do not depend on how the operands are read. Whatever reads the sign (division, remainder,
+// comparisons, min / max, clamp, sgn) has no overload for these types and does not compile; the run-time codes of
+// the generic entry points are checked here.
+inline void ring_only_(bool ok, const char* what) {
+  if (!ok) throw std::invalid_argument(std::string(what) + " reads the sign of its operands: not defined on unsigned tensors");
+}
+#define AM_HPP_UNSIGNED(U, S)                                                                            \
+  inline int gemm_(int64_t M, int64_t N, int64_t K, U al, const U* A, int64_t ra, int64_t ca, const U* B, \
+                   int64_t rb, int64_t cb, U be, U* C, int64_t rc, int64_t cc) {                         \
+    return gemm_(M, N, K, (S)al, (const S*)A, ra, ca, (const S*)B, rb, cb, (S)be, (S*)C, rc, cc);         \
+  }                                                                                                      \
+  inline int gemv_(int64_t M, int64_t N, U al, const U* A, int64_t ra, int64_t ca, const U* x, int64_t ix, \
+                   U be, U* y, int64_t iy) {                                                              \
+    return gemv_(M, N, (S)al, (const S*)A, ra, ca, (const S*)x, ix, (S)be, (S*)y, iy);                    \
+  }                                                                                                      \
+  inline int dot_(int64_t n, const U* x, int64_t ix, const U* y, int64_t iy, U* r) {                     \
+    return dot_(n, (const S*)x, ix, (const S*)y, iy, (S*)r);                                              \
+  }                                                                                                      \
+  inline int binary_(int op, int rank, const int64_t* sh, U* d, const int64_t* sd, const U* a,           \
+                     const int64_t* sa, const U* b, const int64_t* sb) {                                 \
+    ring_only_(op == AM_OP_ADD || op == AM_OP_SUB || op == AM_OP_MUL, "this map2 body");                  \
+    return binary_(op, rank, sh, (S*)d, sd, (const S*)a, sa, (const S*)b, sb);                            \
+  }                                                                                                      \
+  inline int scalar_(int op, int left, int rank, const int64_t* sh, U* d, const int64_t* sd, const U* a, \
+                     const int64_t* sa, U s) {                                                           \
+    ring_only_(op == AM_OP_ADD || op == AM_OP_SUB || op == AM_OP_MUL, "this scalar operation");           \
+    return scalar_(op, left, rank, sh, (S*)d, sd, (const S*)a, sa, (S)s);                                 \
+  }                                                                                                      \
+  inline int unary_(int op, int rank, const int64_t* sh, U* d, const int64_t* sd, const U* a,            \
+                    const int64_t* sa) {                                                                 \
+    ring_only_(op == AM_UOP_COPY || op == AM_UOP_NEG, "this map body");                                   \
+    return unary_(op, rank, sh, (S*)d, sd, (const S*)a, sa);                                              \
+  }                                                                                                      \
+  inline int reduce_axis_(int op, int rank, const int64_t* sh, int axis, U* d, const int64_t* sd, const U* a, \
+                          const int64_t* sa) {                                                            \
+    ring_only_(op == AM_RED_SUM || op == AM_RED_PROD, "min / max");                                       \
+    return reduce_axis_(op, rank, sh, axis, (S*)d, sd, (const S*)a, sa);                                  \
+  }                                                                                                      \
+  inline int reduce_all_(int op, int rank, const int64_t* sh, const U* a, const int64_t* sa, U* r) {      \
+    ring_only_(op == AM_RED_SUM || op == AM_RED_PROD, "min / max");                                       \
+    return reduce_all_(op, rank, sh, (const S*)a, sa, (S*)r);                                             \
+  }
+AM_HPP_UNSIGNED(uint32_t, int32_t)
+AM_HPP_UNSIGNED(uint64_t, int64_t)
+#undef AM_HPP_UNSIGNED
 inline int gemm_ex_(int64_t M, int64_t N, int64_t K, float al, const float* A, int64_t ra, int64_t ca,
                     const float* B, int64_t rb, int64_t cb, float be, float* C, int64_t rc, int64_t cc, int epi,
                     const float* bias, int64_t brs, int64_t bcs) {
@@ -221,8 +269,10 @@ class HipTensor {
   // byte per element, 0 / 1) and classify's FloatClass ordinals. Such a tensor can be viewed and copied to
   // the host; no arithmetic is defined on it.
   static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value ||
-                    std::is_same<T, int32_t>::value || std::is_same<T, int64_t>::value || std::is_same<T, uint8_t>::value,
-                "HipTensor supports float, double, int32_t and int64_t (and uint8_t as a result type)");
+                    std::is_same<T, int32_t>::value || std::is_same<T, int64_t>::value || std::is_same<T, uint8_t>::value ||
+                    std::is_same<T, uint32_t>::value || std::is_same<T, uint64_t>::value,
+                "HipTensor supports float, double, int32_t and int64_t (uint32_t and uint64_t for + - * and products, "
+                "uint8_t as a result type)");
 
  public:
   Shape shape, strides;     // elements
@@ -370,6 +420,19 @@ HipTensor<T> toHip(const std::vector<T>& host, const Shape& shape) {
   for (auto s : shape) n *= s;
   if ((int64_t)host.size() != n) throw std::invalid_argument("toHip: " + std::to_string(host.size()) + " values for shape " + detail::str(shape));
   return toHip(host.data(), shape);
+}
+
+// broadcast(val, shape) (shapeshifting.nim:136-176): a tensor of `shape` whose every element is `val` - ONE element of
+// storage, every stride 0. Not to be written through (all positions share the element); clone() materialises it.
+template <typename T>
+HipTensor<T> broadcast(T val, const Shape& shape) {
+  if (shape.size() > AM_MAXRANK) throw std::invalid_argument("rank exceeds " + std::to_string(AM_MAXRANK));
+  const HipTensor<T> one = toHip(&val, Shape{1});
+  HipTensor<T> r;
+  r.shape = shape;
+  r.strides.assign(shape.size(), 0);
+  r.storage = one.storage;
+  return r;
 }
 
 // ---- map2 / operators ---------------------------------------------------------------------------

@@ -32,6 +32,7 @@ proc am_hip_device_info*(name: cstring, name_cap: csize_t, compute_units, clock_
 proc am_hip_malloc*(bytes: csize_t, dptr: ptr pointer): cint {.importc.}
 proc am_hip_empty_cache*(): cint {.importc.}   # freed blocks are cached for reuse; this returns them to the driver
 proc am_hip_memory_stats*(live_bytes, cached_bytes: ptr csize_t): cint {.importc.}
+proc am_hip_device_free_bytes*(free_bytes, total_bytes: ptr csize_t): cint {.importc.}
 proc am_hip_free*(dptr: pointer): cint {.importc.}
 proc am_hip_memcpy_h2d*(dst, src: pointer, bytes: csize_t): cint {.importc.}
 proc am_hip_memcpy_d2h*(dst, src: pointer, bytes: csize_t): cint {.importc.}
@@ -52,6 +53,7 @@ proc am_hip_graph_destroy*(graph_exec: pointer): cint {.importc.}
 proc am_hip_diag_peak*(kind, iters, waves_per_simd: cint, ops_per_second: ptr cdouble): cint {.importc.}
 proc am_hip_diag_clock_begin*(): cint {.importc.}
 proc am_hip_diag_clock_end*(shader_mhz: ptr cdouble): cint {.importc.}
+proc am_hip_diag_phases*(out6: ptr cdouble): cint {.importc.}
 proc am_hip_diag_hbm*(kind: cint, bytes: csize_t, windows, blocks_per_cu, unroll, flags, launches: cint,
                       bytes_per_second: ptr cdouble): cint {.importc.}
 

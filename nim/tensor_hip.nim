@@ -25,9 +25,12 @@ import std/math                                     # scalar sqrt for `std`
 
 type
   HipScalar* = float32 | float64 | int32 | int64
-  HipElem* = HipScalar | bool | uint8
-    ## what a HipTensor can hold: the four arithmetic types, plus bool (one byte, the result of the
-    ## comparison family) and uint8 (FloatClass ordinals of `classify`) as result-only element types
+  HipUnsigned* = uint32 | uint64
+    ## ride the kernels of their signed twins for + - * and products (see the last section of this file)
+  HipElem* = HipScalar | HipUnsigned | bool | uint8
+    ## what a HipTensor can hold: the four arithmetic types, the two unsigned ones for ring operations, plus bool
+    ## (one byte, the result of the comparison family) and uint8 (FloatClass ordinals of `classify`) as
+    ## result-only element types
 
   HipRefTrackerObj*[T: HipElem] = object
     value*: ptr UncheckedArray[T]
@@ -84,14 +87,14 @@ template i64s(m: Metadata): array[LASER_MAXRANK, int64] =
   r
 
 # ---------------------------------------------------------------- transfers
-proc toHip*[T: HipScalar](t: Tensor[T]): HipTensor[T] =
+proc toHip*[T: HipScalar | HipUnsigned](t: Tensor[T]): HipTensor[T] =
   ## Host -> device (the `cuda` proc, init_cuda.nim:23-41). Row-major on the device.
   let contig = t.asContiguous(rowMajor, force = true)
   result = newHipTensor[T](t.shape)
   if result.size > 0:
     check am_hip_memcpy_h2d(result.storage.Fdata, contig.get_offset_ptr, csize_t(result.size * sizeof(T)))
 
-proc toCpu*[T: HipScalar](t: HipTensor[T]): Tensor[T] =
+proc toCpu*[T: HipScalar | HipUnsigned](t: HipTensor[T]): Tensor[T] =
   ## Device -> host, blocking (the `cpu` proc, init_cuda.nim:43-59): the whole storage is copied
   ## and shape / strides / offset are kept.
   result = newTensorUninit[T](t.storage.Flen)
@@ -127,6 +130,19 @@ proc broadcast*[T](t: HipTensor[T], shape: varargs[int]): HipTensor[T] =
         result.strides[i] = 0
     elif t.shape[i] != shape[i]:
       raise newException(ValueError, "The broadcasted size of the tensor must match existing size for non-singleton dimension")
+
+proc broadcast*[T: HipScalar | HipUnsigned](val: T, shape: varargs[int]): HipTensor[T] =
+  ## Broadcast a number (shapeshifting.nim:136-176): one element of storage, every stride 0. Like the reference's,
+  ## the result must not be written through (all positions share the element).
+  result.shape.copyFrom(shape)
+  result.strides = default(Metadata)
+  result.strides.len = shape.len
+  result.offset = 0
+  result.storage = newHipStorage[T](1)
+  var v = val
+  check am_hip_memcpy_h2d(result.storage.Fdata, v.addr, csize_t(sizeof(T)))
+
+template bc*[T: HipScalar | HipUnsigned](val: T, shape: varargs[int]): untyped = broadcast(val, shape)
 
 proc broadcast2*[T](a, b: HipTensor[T]): tuple[a, b: HipTensor[T]] =
   ## broadcast2Impl, private/p_shapeshifting.nim:96-134
@@ -195,6 +211,10 @@ proc map2*[T](a: HipTensor[T], op: AmBinaryOp, b: HipTensor[T]): HipTensor[T] =
   check_elementwise(a, b)
   result = newHipTensor[T](a.shape)
   if result.size > 0: ewBinary(T, op, result, a, b)
+
+proc apply2Into[T](dst: var HipTensor[T], a: HipTensor[T], op: AmBinaryOp, b: HipTensor[T]) =
+  ## dst[i] = op(a[i], b[i]) into an existing tensor of the operands' shape
+  if dst.size > 0: ewBinary(T, op, dst, a, b)
 
 proc apply2*[T](dest: var HipTensor[T], op: AmBinaryOp, src: HipTensor[T]) =
   check_elementwise(dest, src)
@@ -876,6 +896,78 @@ template recordGraph*(body: untyped): HipGraph =
     g
 
 proc launch*(g: HipGraph) = check am_hip_graph_launch(g.exec)
+
+# ---------------------------------------------------------------- unsigned element types
+# The reference's GEMM takes uint32 | uint64 | uint | int by casting the pointers onto its int32 / int64 kernels
+# (laser/primitives/matrix_multiplication/gemm.nim:275-307). In the rings Z/2^32 and Z/2^64 the bits of + - * (hence of
+# matrix products, dot, sums and products of elements) do not depend on how the operands are read, so those run on
+# the signed kernels here too. Whatever reads the sign (div, mod, comparisons, min / max, clamp, sgn) has no overload
+# for these types and does not compile.
+template signedTwin(T: typedesc): typedesc =
+  when sizeof(T) == 4: int32 else: int64
+
+proc signedView[T: HipUnsigned](t: HipTensor[T]): HipTensor[signedTwin(T)] =
+  ## The same device memory read as the signed twin. Non-owning (no ref tracker): valid while `t` is alive, i.e.
+  ## inside the proc that made it.
+  result.shape = t.shape
+  result.strides = t.strides
+  result.offset = t.offset
+  result.storage.Flen = t.storage.Flen
+  result.storage.Fdata = cast[ptr UncheckedArray[signedTwin(T)]](t.storage.Fdata)
+
+proc gemm*[T: HipUnsigned](alpha: T, A, B: HipTensor[T], beta: T, C: var HipTensor[T]) =
+  var c = C.signedView
+  gemm(cast[signedTwin(T)](alpha), A.signedView, B.signedView, cast[signedTwin(T)](beta), c)
+
+proc gemv*[T: HipUnsigned](alpha: T, A, x: HipTensor[T], beta: T, y: var HipTensor[T]) =
+  var v = y.signedView
+  gemv(cast[signedTwin(T)](alpha), A.signedView, x.signedView, cast[signedTwin(T)](beta), v)
+
+proc dot*[T: HipUnsigned](a, b: HipTensor[T]): T = cast[T](dot(a.signedView, b.signedView))
+
+proc `*`*[T: HipUnsigned](a, b: HipTensor[T]): HipTensor[T] =
+  if a.rank == 2 and b.rank == 2:
+    result = newHipTensor[T]([a.shape[0], b.shape[1]])
+    gemm(T(1), a, b, T(0), result)
+  elif a.rank == 2 and b.rank == 1:
+    result = newHipTensor[T]([a.shape[0]])
+    gemv(T(1), a, b, T(0), result)
+  else:
+    raise newException(ValueError, "Matrix-Matrix or Matrix-Vector multiplication valid only if first Tensor is a Matrix and second is a Matrix or Vector")
+
+proc ringMap2[T: HipUnsigned](a: HipTensor[T], op: AmBinaryOp, b: HipTensor[T]): HipTensor[T] =
+  check_elementwise(a, b)
+  result = newHipTensor[T](a.shape)
+  if result.size > 0:
+    var r = result.signedView
+    apply2Into(r, a.signedView, op, b.signedView)
+
+proc `+`*[T: HipUnsigned](a, b: HipTensor[T]): HipTensor[T] = ringMap2(a, opAdd, b)
+proc `-`*[T: HipUnsigned](a, b: HipTensor[T]): HipTensor[T] = ringMap2(a, opSub, b)
+proc `+.`*[T: HipUnsigned](a, b: HipTensor[T]): HipTensor[T] =
+  let (x, y) = broadcast2(a, b)
+  ringMap2(x, opAdd, y)
+proc `-.`*[T: HipUnsigned](a, b: HipTensor[T]): HipTensor[T] =
+  let (x, y) = broadcast2(a, b)
+  ringMap2(x, opSub, y)
+proc `*.`*[T: HipUnsigned](a, b: HipTensor[T]): HipTensor[T] =
+  let (x, y) = broadcast2(a, b)
+  ringMap2(x, opMul, y)
+proc `*`*[T: HipUnsigned](s: T, t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0:
+    var r = result.signedView
+    let tv = t.signedView
+    ewScalar(signedTwin(T), opMul, true, r, tv, cast[signedTwin(T)](s))
+proc `*`*[T: HipUnsigned](t: HipTensor[T], s: T): HipTensor[T] = s * t
+proc sum*[T: HipUnsigned](t: HipTensor[T]): T = cast[T](sum(t.signedView))
+proc product*[T: HipUnsigned](t: HipTensor[T]): T = cast[T](product(t.signedView))
+proc clone*[T: HipUnsigned](t: HipTensor[T]): HipTensor[T] =
+  result = newHipTensor[T](t.shape)
+  if result.size > 0:
+    var r = result.signedView
+    let tv = t.signedView
+    ewUnary(signedTwin(T), uopCopy, r, tv)
 
 # ---------------------------------------------------------------- .npy files and display
 # The file parsing and the pretty printer are the reference's own host code (io/io_npy.nim:64-183,

@@ -112,6 +112,38 @@ static void add_sub_scalars() {
   CHECK(eq(2.0f * f, {2, 6, -10}) && eq(f * 2.0f, {2, 6, -10}));
 }
 
+template <typename U>
+static void unsigned_ring_ops() {
+  // gemm.nim:275-307: unsigned element types ride the signed kernels. The small GEMM literals (gemm.nim:373-396) with
+  // non-negative entries, then values whose sum and product leave the signed range: the ring's answer modulo 2^n.
+  auto a = toHip<U>({1, 2, 3, 4, 5, 6}, {2, 3});
+  auto b = toHip<U>({7, 8, 9, 10, 11, 12}, {3, 2});
+  CHECK(eq(a * b, {58, 64, 139, 154}));
+  const U top = U(1) << (8 * sizeof(U) - 1);             // 2^(n-1): the sign bit of the twin
+  auto x = toHip<U>({top, U(top + 5), 3, U(~U(0))}, {2, 2});
+  auto y = toHip<U>({2, 1, 1, 3}, {2, 2});
+  // [[2*top + (top+5), top + 3*(top+5)], [6 + (2^n - 1), 3 + 3*(2^n - 1)]] modulo 2^n
+  CHECK(eq(x * y, {U(top + 5), U(15), U(5), U(0)}));
+  CHECK(eq(x + x, {U(0), U(10), U(6), U(~U(0) - 1)}));
+  CHECK(eq(x - y, {U(top - 2), U(top + 4), U(2), U(~U(0) - 3)}));
+  CHECK(eq(U(3) * x, {top, U(top + 15), U(9), U(~U(0) - 2)}));
+  CHECK(am::sum(x) == U(U(2) * top + 5 + 3 + ~U(0)));
+  CHECK(eq(am::broadcast(U(~U(0)), {2, 2}) + y, {U(1), U(0), U(0), U(2)}));   // scalar broadcast: strides 0, one element
+  EXPECT_THROW(am::scalar_op(AM_OP_DIV, x, U(2)), std::invalid_argument);
+  EXPECT_THROW(am::map2(AM_OP_MOD, x, y), std::invalid_argument);
+  EXPECT_THROW(am::reduce_all(AM_RED_MAX, x), std::invalid_argument);
+}
+
+static void scalar_broadcast() {
+  // broadcast(val, shape), shapeshifting.nim:136-176: one element of storage, every stride 0
+  auto t = am::broadcast(2.5f, {3, 4});
+  CHECK(t.storage->len == 1 && t.strides == Shape({0, 0}) && t.shape == Shape({3, 4}));
+  CHECK(eq(t, std::vector<float>(12, 2.5f)));
+  auto m = toHip<float>({1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12}, {3, 4});
+  CHECK(eq(m + t, {3.5f, 4.5f, 5.5f, 6.5f, 7.5f, 8.5f, 9.5f, 10.5f, 11.5f, 12.5f, 13.5f, 14.5f}));
+  CHECK(eq(am::broadcast(int64_t(-7), {2, 0, 3}), {}));
+}
+
 template <typename T>
 static void broadcasting() {
   // test_broadcasting_cuda.nim:18-189 / test_broadcasting.nim:58-240
@@ -500,6 +532,9 @@ int main(int argc, char** argv) {
     gemm_literals<int64_t>();
     integer_slices();
     add_sub_scalars();
+    unsigned_ring_ops<uint32_t>();
+    unsigned_ring_ops<uint64_t>();
+    scalar_broadcast();
     broadcasting<float>();
     broadcasting<double>();
     broadcasting<int32_t>();

@@ -176,3 +176,31 @@ def test_views_are_metadata_only():
     assert t.broadcast((6, 4)).strides == (4, 1)
     assert _fake((1, 4)).broadcast((6, 4)).strides == (0, 1)
     assert v.data_ptr() == 0x1000 + 4
+
+
+def test_graph_handles_that_the_library_did_not_hand_out_are_refused():
+    """am_hip_graph_launch / _destroy accept only a live graph of am_hip_graph_end: a stale, foreign or twice-destroyed
+    pointer is answered with AM_E_ARG before anything reaches the runtime (no device needed to refuse it)."""
+    L = am.load_library()
+    bogus = ctypes.c_void_p(0x1234560)
+    assert L.am_hip_graph_launch(bogus) == _lib.AM_E_ARG and "not a graph" in _lib.last_error()
+    assert L.am_hip_graph_destroy(bogus) == _lib.AM_E_ARG and "not a graph" in _lib.last_error()
+    assert L.am_hip_graph_destroy(None) == _lib.AM_OK          # NULL: nothing to destroy
+    assert L.am_hip_graph_launch(None) == _lib.AM_E_ARG
+
+
+def test_unsigned_tensors_take_the_signed_kernels_for_ring_operations_only():
+    """uint32 / uint64 ride the int32 / int64 kernels for + - * and products (gemm.nim:275-307); what reads the sign
+    is a TypeError before any device call."""
+    for dt, twin in ((np.uint32, "i32"), (np.uint64, "i64")):
+        t = _fake((2, 2), dt)
+        assert t.ring_sfx == twin
+        with pytest.raises(TypeError, match="sign"):
+            t.sfx
+        for refused in (lambda: am.bc_div(t, t), lambda: am.bc_mod(t, t), lambda: t / 2, lambda: am.bc_lt(t, t),
+                        lambda: am.min(t), lambda: am.max(t, 0), lambda: am.mean(t), lambda: am.relu(t), lambda: am.sgn(t)):
+            with pytest.raises(TypeError):
+                refused()
+    assert _fake((2, 2), np.int32).ring_sfx == "i32" and _fake((2, 2)).ring_sfx == "f32"
+    with pytest.raises(TypeError):
+        am.empty((2, 2), np.uint16)

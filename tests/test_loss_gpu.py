@@ -148,11 +148,14 @@ def test_edge_cases_and_errors(hip):
     x = hip.toHip(np.array([[1000.0, -1000.0, 999.0], [-1000.0, -1001.0, -999.0]], dtype=f32))
     v = hip.sparse_softmax_cross_entropy(x, hip.toHip(np.array([0, 2], dtype=np.int64)))
     assert np.isfinite(v) and abs(v - 0.36043) < 2e-4                                                 # no overflow at +-1000
-    # a label outside the row is not read: the loss is NaN, the gradient row is the plain softmax term
+    # a label outside the row is not read: the loss is NaN, and so is that row of the gradient (the other rows are not touched by it)
     bad = hip.toHip(np.array([0, 7], dtype=np.int64))
     assert np.isnan(hip.sparse_softmax_cross_entropy(x, bad))
     g = hip.sparse_softmax_cross_entropy_backward(1.0, x, bad).toCpu()
-    assert np.all(np.isfinite(g)) and np.all(g[1] >= 0)
+    good = hip.sparse_softmax_cross_entropy_backward(1.0, x, hip.toHip(np.array([0, 2], dtype=np.int64))).toCpu()
+    assert np.all(np.isnan(g[1])) and np.array_equal(g[0], good[0])
+    g = hip.sparse_softmax_cross_entropy_backward(1.0, x, hip.toHip(np.array([-1, 2], dtype=np.int64))).toCpu()
+    assert np.all(np.isnan(g[0])) and np.array_equal(g[1], good[1])
     with pytest.raises(ValueError):
         hip.softmax_cross_entropy(hip.zeros((2, 3), f32), hip.zeros((2, 4), f32))
     with pytest.raises(ValueError):

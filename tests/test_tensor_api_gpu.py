@@ -214,3 +214,65 @@ def test_free_during_graph_capture_is_deferred_to_the_graph(hip):
     gc.collect()
     assert L.am_hip_empty_cache() == 0
     assert stats() == (live0, 0)                # the deferred block came back when the graph went away
+
+
+@pytest.mark.parametrize("dt", [np.uint32, np.uint64])
+def test_unsigned_ring_operations_against_the_modular_closed_form(hip, dt):
+    """uint32 / uint64 on the signed kernels (laser gemm.nim:275-307 casts the pointers the same way). Pinned on what the
+    ring fixes: every result equals exact integer arithmetic reduced modulo 2^n (Python big integers), whatever the
+    sign reading of the operands - entries over the whole unsigned range, so most have the twin's sign bit set."""
+    bits = 8 * np.dtype(dt).itemsize
+    mod = 1 << bits
+    rng = np.random.default_rng(99001 + bits)
+    A = rng.integers(0, mod - 1, (37, 53), dtype=dt, endpoint=True)
+    B = rng.integers(0, mod - 1, (53, 29), dtype=dt, endpoint=True)
+    C0 = rng.integers(0, mod - 1, (37, 29), dtype=dt, endpoint=True)
+    big = lambda X: X.astype(object)
+    exact = lambda X: np.array(X % mod, dtype=dt)
+    dA, dB = hip.toHip(A), hip.toHip(B)
+    assert dA.dtype == np.dtype(dt) and (dA * dB).dtype == np.dtype(dt)
+    assert np.array_equal((dA * dB).toCpu(), exact(big(A) @ big(B)))
+    alpha, beta = mod - 3, (mod >> 1) + 7                       # scalars above the twin's positive range
+    dC = hip.toHip(C0)
+    hip.gemm(alpha, dA, dB.transpose().clone().transpose(), beta, dC)   # B through a column-major view
+    assert np.array_equal(dC.toCpu(), exact(alpha * (big(A) @ big(B)) + beta * big(C0)))
+    # the reference's own small literal (gemm.nim:373-396), unsigned
+    a = hip.toHip(np.array([[1, 2, 3], [4, 5, 6]], dtype=dt))
+    b = hip.toHip(np.array([[7, 8], [9, 10], [11, 12]], dtype=dt))
+    assert np.array_equal((a * b).toCpu(), [[58, 64], [139, 154]])
+    v = rng.integers(0, mod - 1, 53, dtype=dt, endpoint=True)
+    assert np.array_equal((dA * hip.toHip(v)).toCpu(), exact(big(A) @ big(v)))
+    assert int(hip.dot(hip.toHip(v), hip.toHip(A[0]))) == int(sum(int(x) * int(y) for x, y in zip(v, A[0])) % mod)
+    X, Y = A, rng.integers(0, mod - 1, A.shape, dtype=dt, endpoint=True)
+    dX, dY = hip.toHip(X), hip.toHip(Y)
+    assert np.array_equal((dX + dY).toCpu(), exact(big(X) + big(Y)))
+    assert np.array_equal((dX - dY).toCpu(), exact(big(X) - big(Y)))
+    assert np.array_equal(hip.bc_mul(dX, hip.toHip(Y[:1])).toCpu(), exact(big(X) * big(Y[:1])))
+    assert np.array_equal((dX * (mod - 2)).toCpu(), exact(big(X) * (mod - 2)))
+    assert np.array_equal(hip.bc_add(dX, mod - 1).toCpu(), exact(big(X) + (mod - 1)))
+    assert np.array_equal((-dX).toCpu(), exact(-big(X)))
+    assert int(hip.sum(dX)) == int(big(X).sum() % mod)
+    assert np.array_equal(hip.sum(dX, 0).toCpu(), exact(big(X).sum(axis=0, keepdims=True)))
+    assert int(hip.product(hip.toHip(X[0, :5]))) == int(np.prod(big(X[0, :5])) % mod)
+    for refused in (lambda: hip.bc_div(dX, dY), lambda: dX / 3, lambda: hip.bc_le(dX, dY), lambda: hip.max(dX)):
+        with pytest.raises(TypeError):
+            refused()
+
+
+def test_scalar_broadcast_is_one_element_with_zero_strides(hip):
+    """broadcast(val, shape), shapeshifting.nim:136-176: storage of ONE element, every stride 0, usable as an operand."""
+    t = hip.broadcast(2.5, (3, 4), np.float32)
+    assert t.shape == (3, 4) and t.strides == (0, 0) and t.offset == 0 and t.storage.nelems == 1 and t.dtype == np.float32
+    assert np.array_equal(t.toCpu(), np.full((3, 4), 2.5, np.float32))
+    m = np.arange(12, dtype=np.float32).reshape(3, 4)
+    assert np.array_equal((hip.toHip(m) + t).toCpu(), m + np.float32(2.5))
+    assert np.array_equal(hip.bc_mul(hip.toHip(m), t).toCpu(), m * np.float32(2.5))
+    c = t.clone()
+    assert c.is_C_contiguous() and c.storage.nelems == 12 and np.array_equal(c.toCpu(), np.full((3, 4), 2.5, np.float32))
+    i = hip.broadcast(-7, (2, 5))                      # a Python int: int64, like Nim's `int`
+    assert i.dtype == np.int64 and np.array_equal(i.toCpu(), np.full((2, 5), -7))
+    a = np.arange(10, dtype=np.int64).reshape(2, 5)
+    assert np.array_equal((hip.toHip(a) * hip.broadcast(3, (5, 2), np.int64)).toCpu(), a @ np.full((5, 2), 3))   # as a GEMM operand
+    assert hip.broadcast(1.0, (0, 3)).toCpu().shape == (0, 3)
+    # the tensor form under the same name
+    assert hip.broadcast(hip.toHip(np.ones((1, 4))), (3, 4)).strides == (0, 1)
