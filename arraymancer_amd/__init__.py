@@ -8,7 +8,7 @@ does, and raises if it is missing (there is no CPU fallback).
 from ._lib import HipAllocError, HipError, load as load_library
 from .metadata import Layout, Step
 from .io_npy import read_npy, write_npy
-from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3, map3, bc_add, bc_div, bc_mod, bc_mul,
+from .tensor_hip import (OPERATORS, Graph, DigitPlanes, digits_prepare, HipStorage, HipTensor, apply2, apply3, map3, bc_add, bc_div, bc_mod, bc_mul,
                          bc_sub, bias_relu, conv2d, conv2d_into, conv2d_backward, col2im, im2col_folded, dot, empty, gemm, gemm_batched, gemv, im2col, linear, map2, matmul, relu, scalar_op,
                          sigmoid, sync, toHip, broadcast, unary, zeros, reduce_axis, reduce_all, tsum as sum, tproduct as product,
                          tmin as min, tmax as max, mean, softmax, softmax_cross_entropy, sparse_softmax_cross_entropy,
@@ -21,7 +21,7 @@ from .tensor_hip import (OPERATORS, Graph, HipStorage, HipTensor, apply2, apply3
                          bc_ge, isNaN, isNotNaN, classify, FLOAT_CLASS, sgn, floorMod, copySign, mcopySign, degToRad, radToDeg, fac, sgd_update)
 
 __all__ = [
-    "HipTensor", "HipStorage", "Graph", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
+    "HipTensor", "HipStorage", "Graph", "DigitPlanes", "digits_prepare", "HipError", "HipAllocError", "Layout", "Step", "OPERATORS",
     "toHip", "broadcast", "empty", "zeros", "sync", "gemm", "gemm_batched", "gemv", "dot", "im2col", "im2col_folded", "col2im", "conv2d", "conv2d_into", "conv2d_backward", "matmul", "linear", "map2", "apply2", "map3", "apply3", "scalar_op",
     "unary", "relu", "sigmoid", "bias_relu", "bc_add", "bc_sub", "bc_mul", "bc_div", "bc_mod",
     "tanh", "relu_backward", "sigmoid_backward", "tanh_backward", "linear_backward", "gru_cell_inference", "gru_cell_forward", "gru_cell_backward", "gru_inference", "gru_forward", "gru_backward",

@@ -70,9 +70,11 @@ def _signatures():
         "am_hip_graph_end": (ci, [pp]),
         "am_hip_graph_launch": (ci, [vp]),
         "am_hip_graph_destroy": (ci, [vp]),
+        "am_hip_digits_release": (ci, [vp]),
         "am_hip_diag_peak": (ci, [ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "am_hip_diag_clock_begin": (ci, []),
         "am_hip_diag_clock_end": (ci, [ctypes.POINTER(ctypes.c_double)]),
+        "am_hip_diag_phases_begin": (ci, []),
         "am_hip_diag_phases": (ci, [ctypes.POINTER(ctypes.c_double)]),
         "am_hip_diag_hbm": (ci, [ci, sz, ci, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_double)]),
     }
@@ -81,6 +83,9 @@ def _signatures():
         sig[f"am_hip_gemm_{sfx}"] = (ci, gemm)
         if sfx == "f32":
             sig["am_hip_gemm_noalloc_f32"] = (ci, gemm)
+        if sfx in ("i32", "i64"):
+            sig[f"am_hip_digits_prepare_{sfx}"] = (ci, [ci, i64, i64, vp, i64, i64, pp])
+            sig[f"am_hip_gemm_prepared_{sfx}"] = (ci, [i64, i64, i64, ct, vp, i64, i64, vp, vp, i64, i64, vp, ct, vp, i64, i64])
         if sfx in ("f32", "f64"):
             sig[f"am_hip_gemm_ex_{sfx}"] = (ci, gemm + [ci, vp, i64, i64])
         sig[f"am_hip_gemm_batched_{sfx}"] = (ci, [i64, i64, i64, i64, ct, vp, i64, i64, i64, vp, i64, i64, i64, ct,

@@ -43,19 +43,22 @@ struct ClockProbe {
   }
 };
 
-// Where a short kernel's time goes, read inside it. While a clock window is open (same buffer as ClockProbe, slots 2..8),
-// the first lane of every workgroup reads the constant-rate counter when the kernel body starts and at four marks
-// and adds the four intervals to out[3..6]; out[2] counts the workgroups, out[7] keeps the earliest start (as
-// 2^62 - t, so that a maximum finds it from a zeroed buffer) and out[8] the latest last mark: their difference is the
-// time from the first wavefront's first instruction to the last workgroup's last mark, which the duration the
-// profiler reports for the launch exceeds by the dispatch and end-of-kernel work. settle() drains the wave's memory
-// operations before a mark, only while armed, so that a mark means "arrived", not "issued". Does nothing when `out`
-// is null.
+// Where a short kernel's time goes, read inside it. While a phase window is open (am_hip_diag_phases_begin), the first
+// lane of every workgroup reads the constant-rate counter when the kernel body starts and at four marks and writes the
+// five readings to its own slot of the window's buffer (plain stores: nothing is shared between workgroups; workgroups
+// beyond the buffer's capacity record nothing). The host turns them into mean intervals and into the time from the
+// earliest start to the latest last mark, which the duration a profiler reports for the launch exceeds by the
+// dispatch and end-of-kernel work. settle() drains the wave's memory operations before a mark, only while armed, so
+// that a mark means "arrived", not "issued". Does nothing when `out` is null.
 struct PhaseProbe {
   long long* out;
   long long t[5];
-  __device__ __forceinline__ explicit PhaseProbe(long long* o) : out(o) {
-    if (out) t[0] = wall_clock64();
+  // `row_pitch` = workgroups per row of the grid (passed in: reading gridDim costs the prologue another memory round trip)
+  __device__ __forceinline__ PhaseProbe(long long* base, int capacity, unsigned row_pitch) : out(nullptr) {
+    if (base) {
+      const unsigned slot = blockIdx.y * row_pitch + blockIdx.x;
+      if (slot < (unsigned)capacity) { out = base + (size_t)slot * 5; t[0] = wall_clock64(); }
+    }
   }
   __device__ __forceinline__ void settle() const {
     if (out) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -65,14 +68,13 @@ struct PhaseProbe {
   }
   __device__ __forceinline__ void finish() const {
     if (out && threadIdx.x == 0) {
-      atomicAdd((unsigned long long*)&out[2], 1ull);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) atomicAdd((unsigned long long*)&out[3 + i], (unsigned long long)(t[i + 1] - t[i]));
-      atomicMax(&out[7], (1LL << 62) - t[0]);
-      atomicMax(&out[8], t[4]);
+      for (int i = 0; i < 5; ++i) out[i] = t[i];
     }
   }
 };
+// The open phase window's buffer and its capacity in workgroups; nullptr when none is open.
+long long* phase_probe_buffer(int* capacity);
 
 #define AM_HIP_TRY(expr)                                                                    \
   do {                                                                                      \

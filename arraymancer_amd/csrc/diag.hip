@@ -304,22 +304,56 @@ extern "C" int am_hip_diag_clock_end(double* shader_mhz) {
   return AM_OK;
 }
 
-// The phase marks of the small-product kernels (PhaseProbe, common.h) collected since am_hip_diag_clock_begin, in
-// microseconds: out[0] workgroups that reported, out[1..4] the mean of each of the four intervals (start -> first loads
-// issued -> arrived -> last matrix instruction and fold -> stores done), out[5] first start to last end over all of
-// them. Meaningful for ONE launch per window. Blocking; the window stays open.
+// ---- phase marks of the small-product kernels (PhaseProbe, common.h) --------------------------------
+namespace {
+constexpr int kPhaseSlots = 8192;          // workgroups that can record
+long long* g_phase_buf = nullptr;          // device: [kPhaseSlots][5] readings of the constant-rate counter
+bool g_phase_armed = false;
+}  // namespace
+namespace am {
+long long* phase_probe_buffer(int* capacity) {
+  if (capacity) *capacity = kPhaseSlots;
+  return g_phase_armed ? g_phase_buf : nullptr;
+}
+}
+
+extern "C" int am_hip_diag_phases_begin(void) {
+  AM_TRY(ensure_init());
+  if (capturing()) return fail(AM_E_ARG, "am_hip_diag_phases_begin: not allowed while a graph is being captured");
+  if (!g_phase_buf) AM_HIP_TRY(hipMalloc((void**)&g_phase_buf, (size_t)kPhaseSlots * 5 * sizeof(long long)));
+  AM_HIP_TRY(hipMemsetAsync(g_phase_buf, 0, (size_t)kPhaseSlots * 5 * sizeof(long long), stream()));
+  g_phase_armed = true;
+  return AM_OK;
+}
+
+// Closes the window (blocking) and summarises it, in microseconds: out[0] workgroups that reported, out[1..4] the mean
+// of each of the four intervals (start -> first loads issued -> arrived -> last matrix instruction and fold -> stores
+// done), out[5] earliest start to latest end over all of them. Meaningful for ONE launch per window.
 extern "C" int am_hip_diag_phases(double* out6) {
   if (!out6) return fail(AM_E_ARG, "am_hip_diag_phases: null pointer");
-  if (!g_clock_armed) return fail(AM_E_ARG, "am_hip_diag_phases: am_hip_diag_clock_begin was not called");
-  long long h[9] = {0};
-  AM_TRY(fetch_result(h, g_clock_buf, sizeof(h)));
+  if (!g_phase_armed) return fail(AM_E_ARG, "am_hip_diag_phases: am_hip_diag_phases_begin was not called");
+  g_phase_armed = false;
+  static long long* host = nullptr;
+  const size_t bytes = (size_t)kPhaseSlots * 5 * sizeof(long long);
+  if (!host) AM_HIP_TRY(hipHostMalloc((void**)&host, bytes, hipHostMallocDefault));
+  AM_HIP_TRY(hipMemcpyAsync(host, g_phase_buf, bytes, hipMemcpyDeviceToHost, stream()));
+  AM_HIP_TRY(hipStreamSynchronize(stream()));
   int khz = 100000;
   (void)hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, 0);
   const double us_per_tick = 1e3 / (double)khz;
-  const double n = h[2] > 0 ? (double)h[2] : 1.0;
-  out6[0] = (double)h[2];
-  for (int i = 0; i < 4; ++i) out6[1 + i] = (double)h[3 + i] / n * us_per_tick;
-  out6[5] = h[2] > 0 ? (double)(h[8] - ((1LL << 62) - h[7])) * us_per_tick : 0.0;
+  double sum[4] = {0, 0, 0, 0};
+  long long first = 0, last = 0, n = 0;
+  for (int s = 0; s < kPhaseSlots; ++s) {
+    const long long* t = host + (size_t)s * 5;
+    if (t[0] == 0) continue;
+    for (int i = 0; i < 4; ++i) sum[i] += (double)(t[i + 1] - t[i]);
+    if (n == 0 || t[0] < first) first = t[0];
+    if (n == 0 || t[4] > last) last = t[4];
+    ++n;
+  }
+  out6[0] = (double)n;
+  for (int i = 0; i < 4; ++i) out6[1 + i] = n ? sum[i] / (double)n * us_per_tick : 0.0;
+  out6[5] = n ? (double)(last - first) * us_per_tick : 0.0;
   return AM_OK;
 }
 

@@ -79,6 +79,8 @@ template <typename T> struct Args {
   bool static_ws;
   size_t static_ws_short;
   long long* clock_out;            // where the matrix-core kernels add their cycle counts while a clock window is open
+  long long* phase_out;            // the small-product kernels' phase marks while a phase window is open (PhaseProbe)
+  int phase_cap;
   ConvGeom conv;                   // read by the kGather loader only
 };
 
@@ -154,6 +156,7 @@ static int prepare(const char* fn, int64_t M, int64_t N, int64_t K, T alpha, con
   g.static_ws = false; g.static_ws_short = 0;
   g.want_splits = 0;
   g.clock_out = clock_probe_buffer();
+  g.phase_out = phase_probe_buffer(&g.phase_cap);
   g.swapped = swap;
   g.a_kfast = iabs64(g.a_k) <= iabs64(g.a_mn);
   g.b_kfast = iabs64(g.b_k) < iabs64(g.b_mn);

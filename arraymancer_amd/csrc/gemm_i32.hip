@@ -1,10 +1,72 @@
 // int32 GEMM entry points (wraparound arithmetic): large products run on the int8 matrix cores by
 // digit slicing, the others on the vector ALU.
+#include <mutex>
+#include <unordered_set>
 #include "gemm_int_impl.h"
 #include "gemm_i8_digits.h"
 
 using namespace am;
 using namespace am::gemm;
+
+namespace am {
+namespace gemm {
+namespace i8 {
+static std::mutex g_prepared_mu;
+static std::unordered_set<const Prepared*> g_prepared;
+void remember_prepared(const Prepared* p) {
+  std::lock_guard<std::mutex> lk(g_prepared_mu);
+  g_prepared.insert(p);
+}
+const Prepared* lookup_prepared(const void* handle) {
+  std::lock_guard<std::mutex> lk(g_prepared_mu);
+  const Prepared* p = (const Prepared*)handle;
+  return g_prepared.count(p) ? p : nullptr;
+}
+}  // namespace i8
+}  // namespace gemm
+}  // namespace am
+
+extern "C" int am_hip_digits_release(void* handle) {
+  if (!handle) return AM_OK;
+  i8::Prepared* p = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(i8::g_prepared_mu);
+    auto it = i8::g_prepared.find((const i8::Prepared*)handle);
+    if (it == i8::g_prepared.end())
+      return fail(AM_E_ARG, "am_hip_digits_release: %p is not a handle of am_hip_digits_prepare_* (or was released already)", handle);
+    p = const_cast<i8::Prepared*>(*it);
+    i8::g_prepared.erase(it);
+  }
+  // (stream ordered: a product that still reads the planes is ahead of whoever receives the block next)
+  const int rc = am_hip_free(p->planes);
+  p->magic = 0;
+  delete p;
+  return rc;
+}
+
+// side 0: X is the left operand of later products, [rows x cols] = [M x K]; side 1: the right one, [K x N].
+template <typename T>
+static int digits_prepare(const char* who, int side, int64_t rows, int64_t cols, const T* X, int64_t rs, int64_t cs, void** handle) {
+  if (!handle) return fail(AM_E_ARG, "%s: null handle pointer", who);
+  *handle = nullptr;
+  if (side != 0 && side != 1) return fail(AM_E_ARG, "%s: side must be 0 (left operand) or 1 (right operand)", who);
+  if (rows <= 0 || cols <= 0 || !X) return fail(AM_E_SHAPE, "%s: empty operand", who);
+  AM_TRY(ensure_init());
+  if (capturing()) return fail(AM_E_ARG, "%s: not allowed while a graph is being captured", who);
+  i8::Prepared* p = new i8::Prepared();
+  const int rc = side == 0 ? i8::prepare_planes<T>(X, rows, cols, rs, cs, p) : i8::prepare_planes<T>(X, cols, rows, cs, rs, p);
+  if (rc != AM_OK) { delete p; return rc; }
+  i8::remember_prepared(p);
+  *handle = p;
+  return AM_OK;
+}
+
+extern "C" int am_hip_digits_prepare_i32(int side, int64_t rows, int64_t cols, const int32_t* X, int64_t rs, int64_t cs, void** handle) {
+  return digits_prepare<int32_t>("am_hip_digits_prepare_i32", side, rows, cols, X, rs, cs, handle);
+}
+extern "C" int am_hip_digits_prepare_i64(int side, int64_t rows, int64_t cols, const int64_t* X, int64_t rs, int64_t cs, void** handle) {
+  return digits_prepare<int64_t>("am_hip_digits_prepare_i64", side, rows, cols, X, rs, cs, handle);
+}
 
 static int run_i32(Args<int32_t>& g) {
 
@@ -33,6 +95,26 @@ extern "C" int am_hip_gemm_i32(int64_t M, int64_t N, int64_t K, int32_t alpha, c
   if (rc > 0) return AM_OK;
   if (rc < 0) return rc;
   AM_TRY(ensure_init());
+  return run_i32(g);
+}
+
+extern "C" int am_hip_gemm_prepared_i32(int64_t M, int64_t N, int64_t K, int32_t alpha, const int32_t* A, int64_t rsA,
+                                        int64_t csA, const void* A_digits, const int32_t* B, int64_t rsB, int64_t csB,
+                                        const void* B_digits, int32_t beta, int32_t* C, int64_t rsC, int64_t csC) {
+  const i8::Prepared* ha = A_digits ? i8::lookup_prepared(A_digits) : nullptr;
+  const i8::Prepared* hb = B_digits ? i8::lookup_prepared(B_digits) : nullptr;
+  if ((A_digits && !ha) || (B_digits && !hb))
+    return fail(AM_E_ARG, "am_hip_gemm_prepared_i32: not a live handle of am_hip_digits_prepare_i32");
+  Args<int32_t> g;
+  const int rc = prepare<int32_t>("am_hip_gemm_prepared_i32", M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC,
+                                  AM_EPI_NONE, nullptr, 0, 0, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  if (ha || hb) {
+    int r = AM_OK;
+    if (!i8::run_prepared(g, ha, hb, &r)) return r;
+  }
   return run_i32(g);
 }
 

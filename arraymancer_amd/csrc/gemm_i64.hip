@@ -35,6 +35,26 @@ extern "C" int am_hip_gemm_i64(int64_t M, int64_t N, int64_t K, int64_t alpha, c
   return run_i64(g);
 }
 
+extern "C" int am_hip_gemm_prepared_i64(int64_t M, int64_t N, int64_t K, int64_t alpha, const int64_t* A, int64_t rsA,
+                                        int64_t csA, const void* A_digits, const int64_t* B, int64_t rsB, int64_t csB,
+                                        const void* B_digits, int64_t beta, int64_t* C, int64_t rsC, int64_t csC) {
+  const i8::Prepared* ha = A_digits ? i8::lookup_prepared(A_digits) : nullptr;
+  const i8::Prepared* hb = B_digits ? i8::lookup_prepared(B_digits) : nullptr;
+  if ((A_digits && !ha) || (B_digits && !hb))
+    return fail(AM_E_ARG, "am_hip_gemm_prepared_i64: not a live handle of am_hip_digits_prepare_i64");
+  Args<int64_t> g;
+  const int rc = prepare<int64_t>("am_hip_gemm_prepared_i64", M, N, K, alpha, A, rsA, csA, B, rsB, csB, beta, C, rsC, csC,
+                                  AM_EPI_NONE, nullptr, 0, 0, &g);
+  if (rc > 0) return AM_OK;
+  if (rc < 0) return rc;
+  AM_TRY(ensure_init());
+  if (ha || hb) {
+    int r = AM_OK;
+    if (!i8::run_prepared(g, ha, hb, &r)) return r;
+  }
+  return run_i64(g);
+}
+
 // Integer batched product: no fused epilogue (pass AM_EPI_NONE; add a bias with the element-wise ops).
 extern "C" int am_hip_gemm_batched_i64(int64_t batch, int64_t M, int64_t N, int64_t K, int64_t alpha, const int64_t* A,
                                        int64_t rsA, int64_t csA, int64_t bsA, const int64_t* B, int64_t rsB, int64_t csB,

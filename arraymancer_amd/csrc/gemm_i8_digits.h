@@ -275,6 +275,8 @@ struct DigitArgs {
   T alpha, beta;
   int tiles_m, tiles_n;
   long long* clock_out;                 // see ClockProbe (common.h)
+  int preset_a, preset_b;               // >= 0: bit d set = plane d of that operand is live (planes split ahead of time,
+                                        // Prepared below); < 0: read the flag words
 };
 
 // WAVES_M x WAVES_N wavefronts, each with TM x TN accumulator tiles of 32 x 32; BK k (bytes) per slab.
@@ -330,7 +332,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, 1) void gemm_i8_digits(Digit
     int n = 0, prev_s = -1;
     for (int s = ND - 1; s >= 0; --s)
       for (int i = 0; i <= s; ++i)
-        if (p.flags[i] == p.gen && p.flags[ND + s - i] == p.gen) {
+        if ((p.preset_a >= 0 ? ((p.preset_a >> i) & 1) != 0 : p.flags[i] == p.gen) &&
+            (p.preset_b >= 0 ? ((p.preset_b >> (s - i)) & 1) != 0 : p.flags[ND + s - i] == p.gen)) {
           tab_a[n] = i; tab_b[n] = s - i;
           tab_shift[n] = prev_s < 0 ? 0 : 8 * (prev_s - s);
           prev_s = s;
@@ -637,39 +640,61 @@ static inline int applicable(const Args<T>& g) {
   return (g.M >= 64 && g.N >= 64 && g.K >= 256) ? 1 : 0;
 }
 
+// The digit planes of one operand split ahead of time (am_hip_digits_prepare_*): a weight matrix that enters many
+// products is read and split once instead of in every call. Rows are padded to 256, a multiple of every tile edge, so
+// the planes serve whatever tile a product chooses and either side of it (the layout does not depend on the side:
+// X(mn, k), mn = a row of a left operand or a column of a right one).
+struct Prepared {
+  uint32_t magic;        // kPreparedMagic while the handle is alive
+  int elem_size;         // 4 or 8
+  int64_t MN, K, MNp, Kp;
+  int8_t* planes;        // elem_size planes of MNp x Kp bytes, from am_hip_malloc
+  int mask;              // bit d set: plane d holds a non-zero digit somewhere
+};
+constexpr uint32_t kPreparedMagic = 0x44504c4eu;
+// The handles am_hip_digits_prepare_* has handed out and am_hip_digits_release has not taken back (gemm_i32.hip):
+// anything else passed as a handle is refused instead of being dereferenced.
+void remember_prepared(const Prepared* p);
+const Prepared* lookup_prepared(const void* handle);
+
 // max_pairs < all pairs: the product is left alone when the operands turn out to have more live digit
 // pairs; *gate_flags / *gate_gen then tell the caller what to hand to the kernels it launches next.
+// pa / pb: planes of the kernel's A / B operand split ahead of time (nullptr: split here, into scratch memory).
 template <typename T>
 static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const uint32_t** gate_flags = nullptr,
-               uint32_t* gate_gen = nullptr) {
+               uint32_t* gate_gen = nullptr, const Prepared* pa = nullptr, const Prepared* pb = nullptr) {
   constexpr int ND = (int)sizeof(T);
-  const int64_t Mp = pl.Mp, Np = pl.Np, Kp = pl.Kp;
+  const int64_t Mp = pa ? pa->MNp : pl.Mp, Np = pb ? pb->MNp : pl.Np, Kp = pl.Kp;
   if (Mp / 32 >= ((int64_t)1 << 31) || Np / 32 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return 1;
-  const int64_t tiles_m = Mp / kTileRows[pl.tile], tiles_n = Np / kTileCols[pl.tile];
+  const int64_t tiles_m = (g.M + kTileRows[pl.tile] - 1) / kTileRows[pl.tile], tiles_n = (g.N + kTileCols[pl.tile] - 1) / kTileCols[pl.tile];
   if (tiles_m * tiles_n >= ((int64_t)1 << 31)) return 1;
   // Flag words live as long as the process: every product uses a new generation number, so they are
   // cleared only once (and again should the 32-bit counter ever wrap).
   static uint32_t* flags = nullptr;
   static uint32_t gen = 0;
-  if (!flags) {
-    void* f = nullptr;
-    if (am_hip_malloc(256, &f) != AM_OK) return 1;
-    flags = (uint32_t*)f;
-    gen = 0;
+  if (!(pa && pb)) {   // (with both operands split ahead of time nothing reads the flag words: nothing to set up, so
+                       // such a product can be recorded into a graph even as the first of the process)
+    if (!flags) {
+      void* f = nullptr;
+      if (am_hip_malloc(256, &f) != AM_OK) return 1;
+      flags = (uint32_t*)f;
+      gen = 0;
+    }
+    if (gen == 0 || gen == 0xFFFFFFFFu) {
+      if (hipMemsetAsync(flags, 0, 256, stream()) != hipSuccess) { (void)hipGetLastError(); return 1; }
+      gen = 0;
+    }
+    ++gen;
   }
-  if (gen == 0 || gen == 0xFFFFFFFFu) {
-    if (hipMemsetAsync(flags, 0, 256, stream()) != hipSuccess) { (void)hipGetLastError(); return 1; }
-    gen = 0;
-  }
-  ++gen;
   void* ws = nullptr;
-  const size_t plane_bytes = (size_t)ND * (size_t)(Mp + Np) * (size_t)Kp;
-  if (am_hip_malloc(plane_bytes, &ws) != AM_OK) return 1;
-  int8_t* PA = (int8_t*)ws;
-  int8_t* PB = PA + (int64_t)ND * Mp * Kp;
+  const size_t plane_bytes = (size_t)ND * (size_t)((pa ? 0 : Mp) + (pb ? 0 : Np)) * (size_t)Kp;
+  if (plane_bytes > 0 && am_hip_malloc(plane_bytes, &ws) != AM_OK) return 1;
+  int8_t* PA = pa ? pa->planes : (int8_t*)ws;
+  int8_t* PB = pb ? pb->planes : (int8_t*)ws + (pa ? 0 : (int64_t)ND * Mp * Kp);
   SplitArgs<T> sp;
-  sp.X[0] = g.A; sp.ld_mn[0] = g.a_mn; sp.ld_k[0] = g.a_k; sp.MN[0] = g.M; sp.MNp[0] = Mp; sp.kfast[0] = g.a_kfast; sp.P[0] = PA;
-  sp.X[1] = g.B; sp.ld_mn[1] = g.b_mn; sp.ld_k[1] = g.b_k; sp.MN[1] = g.N; sp.MNp[1] = Np; sp.kfast[1] = g.b_kfast; sp.P[1] = PB;
+  // (an operand split ahead of time has no tiles for the passes to visit: MNp = 0)
+  sp.X[0] = g.A; sp.ld_mn[0] = g.a_mn; sp.ld_k[0] = g.a_k; sp.MN[0] = g.M; sp.MNp[0] = pa ? 0 : Mp; sp.kfast[0] = g.a_kfast; sp.P[0] = PA;
+  sp.X[1] = g.B; sp.ld_mn[1] = g.b_mn; sp.ld_k[1] = g.b_k; sp.MN[1] = g.N; sp.MNp[1] = pb ? 0 : Np; sp.kfast[1] = g.b_kfast; sp.P[1] = PB;
   sp.K = g.K; sp.Kp = Kp; sp.flags = flags; sp.gen = gen; sp.max_pairs = max_pairs;
   if (gate_flags) *gate_flags = flags;
   if (gate_gen) *gate_gen = gen;
@@ -680,16 +705,19 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
                   : (aligned && sp.ld_mn[op] == 1 && sp.ld_k[op] % VEC == 0) ? 2
                                                                              : 0;
   }
-  const int64_t stiles = (Mp + Np) / 32 * (Kp / 128), smax = (int64_t)num_cus() * 16;
-  const dim3 sgrid((unsigned)(stiles < smax ? stiles : smax));
-  // Operands beyond what the memory-side cache may still hold from their producer are read with non-temporal
-  // loads (int64 4096^3, 256 MiB of operands: first pass 65 -> 46 us); smaller ones are faster with ordinary loads.
-  const bool stream_loads = (double)(g.M + g.N) * (double)g.K * sizeof(T) > 192.0 * 1024 * 1024;
-  if (stream_loads) hipLaunchKernelGGL((split_digits<T, true, true>), sgrid, dim3(256), 0, stream(), sp);
-  else hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
-  // with at most one live pair allowed there is nothing above plane 0 that could be needed
-  if (max_pairs >= 2) hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
+  const int64_t stiles = (sp.MNp[0] + sp.MNp[1]) / 32 * (Kp / 128), smax = (int64_t)num_cus() * 16;
+  if (stiles > 0) {
+    const dim3 sgrid((unsigned)(stiles < smax ? stiles : smax));
+    // Operands beyond what the memory-side cache may still hold from their producer are read with non-temporal
+    // loads (int64 4096^3, 256 MiB of operands: first pass 65 -> 46 us); smaller ones are faster with ordinary loads.
+    const bool stream_loads = (double)((pa ? 0 : g.M) + (pb ? 0 : g.N)) * (double)g.K * sizeof(T) > 192.0 * 1024 * 1024;
+    if (stream_loads) hipLaunchKernelGGL((split_digits<T, true, true>), sgrid, dim3(256), 0, stream(), sp);
+    else hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
+    // with at most one live pair allowed there is nothing above plane 0 that could be needed
+    if (max_pairs >= 2) hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
+  }
   DigitArgs<T> d;
+  d.preset_a = pa ? pa->mask : -1; d.preset_b = pb ? pb->mask : -1;
   d.PA = PA; d.PB = PB; d.flags = flags; d.gen = gen; d.max_pairs = max_pairs; d.Mp = Mp; d.Np = Np; d.Kp = Kp;
   d.C = g.C; d.c_m = g.c_m; d.c_n = g.c_n; d.M = g.M; d.N = g.N; d.clock_out = g.clock_out;
   d.alpha = g.alpha; d.beta = g.beta;
@@ -706,8 +734,72 @@ static int run(const Args<T>& g, const Plan& pl, int max_pairs = 1 << 30, const 
   const int rc = check_launch("gemm_i8_digits");
   // The planes go back to the allocator's cache at once: whoever gets the block next reaches it
   // through the same stream, after this product.
-  (void)am_hip_free(ws);
+  if (ws) (void)am_hip_free(ws);
   return rc;
+}
+
+// Splits X(mn, k) = X[mn * ld_mn + k * ld_k] (MN x K) into planes of its own (both passes, then a blocking look at
+// which planes came out non-empty). Returns AM_OK and the planes in *out, or an error code.
+template <typename T>
+static int prepare_planes(const T* X, int64_t MN, int64_t K, int64_t ld_mn, int64_t ld_k, Prepared* out) {
+  constexpr int ND = (int)sizeof(T);
+  constexpr int64_t VEC = 16 / (int64_t)sizeof(T);
+  const int64_t MNp = (MN + 255) / 256 * 256, Kp = (K + kKPad - 1) / kKPad * kKPad;
+  if (MNp / 32 >= ((int64_t)1 << 31) || Kp / 128 > 65535) return fail(AM_E_SHAPE, "am_hip_digits_prepare: operand too large");
+  void* planes = nullptr;
+  void* fl = nullptr;
+  AM_TRY(am_hip_malloc((size_t)ND * (size_t)MNp * (size_t)Kp, &planes));
+  if (am_hip_malloc(256, &fl) != AM_OK) { (void)am_hip_free(planes); return AM_E_ALLOC; }
+  hipError_t e = hipMemsetAsync(fl, 0, 256, stream());
+  SplitArgs<T> sp;
+  sp.X[0] = X; sp.ld_mn[0] = ld_mn; sp.ld_k[0] = ld_k; sp.MN[0] = MN; sp.MNp[0] = MNp; sp.kfast[0] = iabs64(ld_k) <= iabs64(ld_mn); sp.P[0] = (int8_t*)planes;
+  sp.X[1] = X; sp.ld_mn[1] = ld_mn; sp.ld_k[1] = ld_k; sp.MN[1] = 0; sp.MNp[1] = 0; sp.kfast[1] = sp.kfast[0]; sp.P[1] = (int8_t*)planes;
+  sp.K = K; sp.Kp = Kp; sp.flags = (uint32_t*)fl; sp.gen = 1; sp.max_pairs = 1 << 30;
+  const bool aligned = ((uintptr_t)X & 15) == 0;
+  sp.mode[0] = sp.mode[1] = (aligned && ld_k == 1 && ld_mn % VEC == 0) ? 1 : (aligned && ld_mn == 1 && ld_k % VEC == 0) ? 2 : 0;
+  const int64_t stiles = MNp / 32 * (Kp / 128), smax = (int64_t)num_cus() * 16;
+  const dim3 sgrid((unsigned)(stiles < smax ? stiles : smax));
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL((split_digits<T, true>), sgrid, dim3(256), 0, stream(), sp);
+    hipLaunchKernelGGL((split_digits<T, false>), sgrid, dim3(256), 0, stream(), sp);
+    e = hipGetLastError();
+  }
+  uint32_t host_flags[ND];
+  int rc = e == hipSuccess ? fetch_result(host_flags, fl, sizeof(host_flags)) : fail(AM_E_HIP, "am_hip_digits_prepare: %s", hipGetErrorString(e));
+  (void)am_hip_free(fl);
+  if (rc != AM_OK) { (void)am_hip_free(planes); return rc; }
+  out->magic = kPreparedMagic; out->elem_size = ND; out->MN = MN; out->K = K; out->MNp = MNp; out->Kp = Kp;
+  out->planes = (int8_t*)planes;
+  out->mask = 0;
+  for (int d = 0; d < ND; ++d) out->mask |= (host_flags[d] == 1u) ? (1 << d) : 0;
+  return AM_OK;
+}
+
+// A product whose A and / or B operand (as the caller named them) was split ahead of time. The digit path is taken
+// outright (no estimate: the planes exist). Returns 1 when the product cannot run here (a batch member, a long int64
+// k, no scratch memory for the other operand): the caller then runs it from the original operands.
+template <typename T>
+static int run_prepared(const Args<T>& g, const Prepared* user_a, const Prepared* user_b, int* rc) {
+  *rc = AM_OK;
+  const Prepared* pa = g.swapped ? user_b : user_a;
+  const Prepared* pb = g.swapped ? user_a : user_b;
+  for (int side = 0; side < 2; ++side) {
+    const Prepared* h = side ? pb : pa;
+    if (!h) continue;
+    if (h->magic != kPreparedMagic || h->elem_size != (int)sizeof(T)) { *rc = fail(AM_E_ARG, "gemm with prepared digits: not a live handle of this element type"); return 0; }
+    if (h->MN != (side ? g.N : g.M) || h->K != g.K) {
+      *rc = fail(AM_E_SHAPE, "gemm with prepared digits: the handle holds a %lld x %lld operand, the product needs %lld x %lld on that side",
+                 (long long)h->MN, (long long)h->K, (long long)(side ? g.N : g.M), (long long)g.K);
+      return 0;
+    }
+  }
+  if (g.batch > 1 || (sizeof(T) == 8 && g.K > 131071)) return 1;
+  if (capturing() && !(pa && pb)) return 1;      // the other operand's planes would need scratch memory
+  const Plan pl = plan(g);
+  if (trace_choices()) fprintf(stderr, "am_hip gemm: int8 digit path with planes split ahead of time (%s%s), %s tiles\n", pa ? "A" : "", pb ? "B" : "", tile_name(pl.tile));
+  const int r = run(g, pl, 1 << 30, nullptr, nullptr, pa, pb);
+  if (r <= 0) { *rc = r; return 0; }
+  return 1;
 }
 
 // The integer product on the matrix cores, decided in three steps. (1) Estimated faster than the

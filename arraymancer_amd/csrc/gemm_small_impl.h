@@ -66,7 +66,8 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   typedef typename M16<T>::acc_t acc_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][256] partial tiles, W > 1 only
   T (*red)[256] = reinterpret_cast<T (*)[256]>(red_raw);
-  PhaseProbe probe(p.clock_out);   // marks: 1 first loads issued, 2 they have arrived, 3 last matrix instruction and fold, 4 stores done
+  // marks: 1 first loads issued, 2 they have arrived, 3 last matrix instruction and fold, 4 stores done
+  PhaseProbe probe(p.phase_out, p.phase_cap, (unsigned)((p.N + 15) >> 4));
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int i = lane & 15, g = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * 16;
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   typedef T vec_t __attribute__((ext_vector_type(VN)));
   extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][VN][256] partial tiles, W > 1 only
   T (*red)[VN * 256] = reinterpret_cast<T (*)[VN * 256]>(red_raw);
-  PhaseProbe probe(p.clock_out);   // marks as in gemm_rows16
+  PhaseProbe probe(p.phase_out, p.phase_cap, (unsigned)((p.N + 16 * VN - 1) / (16 * VN)));   // marks as in gemm_rows16
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int i = lane & 15, g = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * (16 * VN);

@@ -434,10 +434,48 @@ def _check_elementwise(a: HipTensor, b: HipTensor):
 
 
 # ---------------------------------------------------------------------- GEMM
-def gemm(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none", bias: HipTensor | None = None):
+class DigitPlanes:
+    """The base-256 digit planes of an integer matrix, split once on the device for products that reuse the matrix (a
+    weight matrix): `digits_prepare(W, side)` makes them, `gemm(..., a_digits=..., b_digits=...)` uses them in place
+    of splitting that operand in every call. A snapshot: prepare again after the matrix changes. Released with the
+    object (or `release()`)."""
+
+    def __init__(self, handle: int, side: int, shape, dtype):
+        self.handle, self.side, self.shape, self.dtype = handle, side, tuple(shape), np.dtype(dtype)
+
+    def release(self):
+        h, self.handle = getattr(self, "handle", 0), 0
+        if h:
+            check(_lib.load().am_hip_digits_release(ctypes.c_void_p(h)))
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
+def digits_prepare(t: HipTensor, side: str | int = "right") -> DigitPlanes:
+    """Splits the int32 / int64 (or unsigned twin) matrix `t` into its digit planes for later products in which it is
+    the "left" ([M x K]) or "right" ([K x N]) operand. Any strides; blocking."""
+    if t.rank != 2:
+        raise ValueError("digits_prepare: the operand must be a matrix")
+    sfx = t.ring_sfx
+    if sfx not in ("i32", "i64"):
+        raise TypeError("digits_prepare is defined for integer tensors")
+    s = {"left": 0, "right": 1}.get(side, side)
+    out = ctypes.c_void_p()
+    check(getattr(_lib.load(), f"am_hip_digits_prepare_{sfx}")(
+        int(s), t.shape[0], t.shape[1], ctypes.c_void_p(t.data_ptr()), t.strides[0], t.strides[1], ctypes.byref(out)))
+    return DigitPlanes(out.value, int(s), t.shape, t.dtype)
+
+
+def gemm(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none", bias: HipTensor | None = None,
+         a_digits: DigitPlanes | None = None, b_digits: DigitPlanes | None = None):
     """C <- alpha * A * B + beta * C in place (C may be any non-overlapping strided view).
     src/arraymancer/tensor/operators_blas_l2l3.nim:58-81. Optional fused epilogue
-    ("bias", "relu", "bias_relu") with `bias` broadcastable to C's shape (float types)."""
+    ("bias", "relu", "bias_relu") with `bias` broadcastable to C's shape (float types). a_digits / b_digits: the digit
+    planes of an integer A / B split ahead of time (`digits_prepare`)."""
     dtype = _same_dtype(A, B, C)
     if A.rank != 2 or B.rank != 2 or C.rank != 2:
         raise ValueError("gemm: A, B and C must be matrices")
@@ -454,6 +492,16 @@ def gemm(alpha, A: HipTensor, B: HipTensor, beta, C: HipTensor, epilogue="none",
             ctypes.c_void_p(B.data_ptr()), B.strides[0], B.strides[1], _ring_scalar(sfx, dtype, beta),
             ctypes.c_void_p(C.data_ptr()), C.strides[0], C.strides[1]]
     epi = EPI[epilogue] if isinstance(epilogue, str) else int(epilogue)
+    if a_digits is not None or b_digits is not None:
+        if sfx not in ("i32", "i64") or epi != 0:
+            raise TypeError("prepared digit planes belong to integer products without an epilogue")
+        for d, side in ((a_digits, 0), (b_digits, 1)):
+            if d is not None and (d.side != side or d.dtype != dtype):
+                raise ValueError("gemm: digit planes prepared for the other side of a product, or for another element type")
+        ha = ctypes.c_void_p(a_digits.handle) if a_digits is not None else None
+        hb = ctypes.c_void_p(b_digits.handle) if b_digits is not None else None
+        check(getattr(L, f"am_hip_gemm_prepared_{sfx}")(*args[:7], ha, *args[7:10], hb, *args[10:]))
+        return C
     if epi != 0:
         if sfx not in ("f32", "f64"):
             raise TypeError("fused epilogues are defined for float tensors")

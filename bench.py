@@ -192,16 +192,20 @@ def at_clock(roof, peak, sclk_mhz, nominal_mhz=2400.0):
     matrix peaks are CUs x ops per clock x 2.4 GHz)."""
     if sclk_mhz:
         roof["sclk_mhz"] = sclk_mhz
-        roof["frac_of_peak_at_sclk"] = round(roof["achieved"] / (peak * sclk_mhz / nominal_mhz), 4)
+        roof["frac_at_sclk"] = round(roof["achieved"] / (peak * sclk_mhz / nominal_mhz), 4)
     return roof
 
 
-def mfma_roof(tflops, peak, sclk, unit="TFLOP/s"):
-    return at_clock(dict(bound="mfma", achieved=round(tflops, 3), peak=peak, unit=unit, frac=round(tflops / peak, 4)), peak, sclk)
+def mfma_roof(tflops, peak, sclk, unit=None):
+    """(the unit is the entry's own unless given)"""
+    r = dict(bound="mfma", achieved=round(tflops, 3), peak=peak, frac=round(tflops / peak, 4))
+    if unit:
+        r["unit"] = unit
+    return at_clock(r, peak, sclk)
 
 
 def hbm_roof(gbs, **extra):
-    return dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4), **extra)
+    return dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, frac=round(gbs / HBM_PEAK_GBS, 4), **extra)
 
 
 class Ctx:
@@ -239,7 +243,7 @@ def bench_gemm_f32(ctx, steps, warmup, n=4096, host=None, spin=(SPIN_F32, 0.08))
 def gemm_f32_entry(ctx, n, config, steps):
     r = bench_gemm_f32(ctx, steps, ctx.warmup, n=n)
     t = r["flops"] / (r["ev"] / steps) / 1e12
-    return dict(workload=f"f32 GEMM {n}^3", config=config, dtype="f32", unit="TFLOP/s", value=round(r["flops"] * steps / r["wall"] / 1e12, 3),
+    return dict(workload=f"f32 GEMM {n}^3", config=config, unit="TFLOP/s", value=round(r["flops"] * steps / r["wall"] / 1e12, 3),
                 ms_per_step=round(r["ev"] / steps * 1e3, 5), roofline=mfma_roof(t, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"]))
 
 
@@ -275,7 +279,7 @@ def cpu_baseline_gemm_f32(A, B, budget_s=12.0):
     best = min(times)
     return dict(value=round(2.0 * n ** 3 / best / 1e12, 4), unit="TFLOP/s", cores=am_oracle.num_threads(),
                 kind="port",
-                sample=f"full workload f32 GEMM {n}^3, best of {len(times)} runs, oracle/laser_gemm.c (laser blocking, OpenMP)")
+                sample=f"full f32 GEMM {n}^3, best of {len(times)}, oracle/laser_gemm.c (OpenMP)")
 
 
 def cpu_blas_standin_gemm_f32(A, B, budget_s=6.0):
@@ -301,8 +305,7 @@ def cpu_blas_standin_gemm_f32(A, B, budget_s=6.0):
         times.append(time.perf_counter() - t0)
     best = min(times)
     return dict(value=round(2.0 * n ** 3 / best / 1e12, 4), unit="TFLOP/s", cores=threads or os.cpu_count(), kind="stand-in",
-                sample=f"full workload f32 GEMM {n}^3, best of {len(times)} runs, NumPy A @ B" + (f" ({lib})" if pools else "")
-                       + ": stand-in for the CBLAS behind the reference's float `*`")
+                sample=f"full f32 GEMM {n}^3, best of {len(times)}, NumPy A @ B" + (f" ({lib})" if pools else "") + " for the CBLAS behind `*`")
 
 
 # ------------------------------------------------------------------------------------------ C2: integer GEMM
@@ -334,8 +337,8 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
     kd = max(20, ctx.steps)
     wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), kd, ctx.warmup, (SPIN_I8, 0.08))
     tops = 2.0 * n ** 3 / (ev / kd) / 1e12
-    entry = dict(workload=f"{sfx} GEMM {n}^3, {label}", config=config, dtype=sfx, unit="Top/s", value=round(2.0 * n ** 3 * kd / wall / 1e12, 3),
-                 ms_per_step=round(ev / kd * 1e3, 5), path=f"int8 MFMA digits, {pairs}/{npairs} pairs, splitting passes included",
+    entry = dict(workload=f"{sfx} GEMM {n}^3, {label}", config=config, unit="Top/s", value=round(2.0 * n ** 3 * kd / wall / 1e12, 3),
+                 ms_per_step=round(ev / kd * 1e3, 5), digit_pairs=f"{pairs}/{npairs}",
                  roofline=mfma_roof(pairs * tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s executed"))
     out = [entry]
     if valu:
@@ -356,8 +359,8 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
             roof["sclk_mhz"] = timer.sclk_mhz
             if dt == np.int32:
                 roof["frac_of_full_rate_at_sclk"] = round(vt / (VALU_FULL_RATE_TOPS * timer.sclk_mhz / 2400.0), 4)
-        out.append(dict(workload=f"{sfx} GEMM {n}^3, {label}, VALU kernel", config=config, dtype=sfx, unit="Top/s", value=round(vt, 3),
-                        ms_per_step=round(ev_valu / k * 1e3, 5), path="VALU (forced)", roofline=roof))
+        out.append(dict(workload=f"{sfx} GEMM {n}^3, {label}, VALU kernel", config=config, unit="Top/s", value=round(vt, 3),
+                        ms_per_step=round(ev_valu / k * 1e3, 5), roofline=roof))
     return out
 
 
@@ -369,6 +372,26 @@ def wl_gemm_i32_1500(ctx):
 @workload("gemm_i32")
 def wl_gemm_i32(ctx):
     return int_gemm_entries(ctx, np.int32, 4096, -100, 100, "C2", "in [-100,100]")
+
+
+@workload("gemm_i32_prepared")
+def wl_gemm_i32_prepared(ctx):
+    """int32 4096^3 with the digit planes of B, then of both operands, split once ahead of the timed calls
+    (am_hip_digits_prepare_i32): what a weight matrix that enters many products costs per product."""
+    am, timer, n = ctx.am, ctx.timer, 4096
+    A = np.random.default_rng(2001).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
+    B = np.random.default_rng(2002).integers(-100, 100, (n, n), endpoint=True).astype(np.int32)
+    dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.int32)
+    pa, pb = am.digits_prepare(dA, "left"), am.digits_prepare(dB, "right")
+    kd = max(20, ctx.steps)
+    out = []
+    for label, kw in (("B's digit planes prepared", dict(b_digits=pb)), ("both operands' digit planes prepared", dict(a_digits=pa, b_digits=pb))):
+        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC, **kw), kd, ctx.warmup, (SPIN_I8, 0.08))
+        tops = 2.0 * n ** 3 / (ev / kd) / 1e12
+        out.append(dict(workload=f"i32 GEMM 4096^3, in [-100,100], {label}", config="C2", unit="Top/s",
+                        value=round(2.0 * n ** 3 * kd / wall / 1e12, 3), ms_per_step=round(ev / kd * 1e3, 5),
+                        roofline=mfma_roof(tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s executed")))
+    return out
 
 
 @workload("gemm_i32_whole_range")
@@ -391,7 +414,7 @@ def wl_gemm_i32_valu(ctx):
     k = max(3, ctx.steps // 4)
     _, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, (SPIN_VALU32, 0.08))
     vt = 2.0 * n ** 3 / (ev / k) / 1e12
-    return dict(workload="i32 GEMM 4096^3, entries in [-100, 100], VALU kernel", config="C2", dtype="i32", unit="Top/s", value=round(vt, 3),
+    return dict(workload="i32 GEMM 4096^3, entries in [-100, 100], VALU kernel", config="C2", unit="Top/s", value=round(vt, 3),
                 ms_per_step=round(ev / k * 1e3, 5), roofline={"bound": "valu", "achieved": round(vt, 3), "peak": VALU_FULL_RATE_TOPS,
                                                                "unit": "Top/s (full-rate bound)", "frac": round(vt / VALU_FULL_RATE_TOPS, 4),
                                                                "sclk_mhz": timer.sclk_mhz})
@@ -411,11 +434,11 @@ def wl_i64_1500(ctx):
     wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k5, ctx.warmup, (SPIN_I8, 0.08))
     want = A[n5 // 2] @ B          # one row of the product (the benchmark prints one element of it)
     tops = 2.0 * n5 ** 3 / (ev / k5) / 1e12
-    return dict(workload="i64 matmul 1500^2, entries in [0, 99]", config="published", dtype="i64",
+    return dict(workload="i64 matmul 1500^2, entries in [0, 99]", config="published",
                 unit="Top/s", value=round(2.0 * n5 ** 3 * k5 / wall / 1e12, 3), ms_per_step=round(ev / k5 * 1e3, 5),
                 row_750_matches_numpy=bool(np.array_equal(dC.toCpu()[n5 // 2], want)),
                 roofline=mfma_roof(tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s executed"),
-                published=dict(seconds=0.14, hardware="i9-9980XE 18 cores, whole process", source="benchmarks/integer_matmul.nim:8-33"))
+                published_s=0.14, published_on="i9-9980XE, benchmarks/integer_matmul.nim:8-33")
 
 
 # ------------------------------------------------------------------------------------------ C3: float64 views
@@ -431,7 +454,7 @@ def wl_gemm_f64_views(ctx):
     steps = max(ctx.steps, 50)
     wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, ctx.warmup, (SPIN_F64, 0.1), min_warm_s=0.3)
     fl = 2.0 * 2048 * 3072 * 1024
-    return dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", config="C3", dtype="f64", unit="TFLOP/s",
+    return dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", config="C3", unit="TFLOP/s",
                 value=round(fl * steps / wall / 1e12, 3), ms_per_step=round(ev / steps * 1e3, 5),
                 roofline=mfma_roof(fl / (ev / steps) / 1e12, MFMA_F64_PEAK_TFLOPS, timer.sclk_mhz))
 
@@ -466,13 +489,13 @@ def c4_entry(ctx, name, launch_of, nbytes, same_buffers=None):
         copy_ceiling = ctx.ceilings.get("hbm_copy_tbs")
         d2d = ctx.ceilings.get("runtime_d2d_copy_tbs")
         if copy_ceiling:
-            roof["frac_of_measured_copy_ceiling"] = round(gbs / (copy_ceiling * 1e3), 4)
+            roof["vs_copy_ceiling"] = round(gbs / (copy_ceiling * 1e3), 4)
         if d2d:
-            roof["frac_of_runtime_d2d_copy"] = round(gbs / (d2d * 1e3), 4)
-    e = dict(workload=f"f32 8192x8192 {name}", config="C4", dtype="f32", unit="GB/s", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 5), roofline=roof)
+            roof["vs_runtime_d2d"] = round(gbs / (d2d * 1e3), 4)
+    e = dict(workload=f"f32 8192x8192 {name}", config="C4", unit="GB/s", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 5), roofline=roof)
     if same_buffers is not None:
         _, ev = timer.run(same_buffers, ctx.steps, ctx.warmup, None)
-        e["same_buffers_every_step_ms"] = round(ev / ctx.steps * 1e3, 5)
+        e["same_buffers_ms"] = round(ev / ctx.steps * 1e3, 5)
     timer.launches = launches
     return e
 
@@ -520,7 +543,7 @@ def wl_transposed_add(ctx):
     cold = run_rotating(ctx.timer, [(lambda i=i: th._binary_into("add", dYs[i], dXs[i], dXs[(i + 1) % 3].transpose())) for i in range(3)],
                         max(ctx.steps // 3, 4))
     gbs = 3 * 8192 * 8192 * 4 / cold / 1e9
-    return dict(workload="f32 8192x8192 X + Z^T (Z a transposed view)", config="a18", dtype="f32", unit="GB/s", value=round(gbs, 1),
+    return dict(workload="f32 8192x8192 X + Z^T (Z a transposed view)", config="a18", unit="GB/s", value=round(gbs, 1),
                 ms_per_step=round(cold * 1e3, 5), roofline=hbm_roof(gbs))
 
 
@@ -579,8 +602,8 @@ def wl_chain(ctx):
     steps = max(ctx.steps, 50)
     r, best = eager_and_graph(ctx, issue, capture, steps)
     return dict(workload="f32 chain [20x25].[25x36864], [50x500].[500x4096], [64x800].[800x500]+bias+ReLU, [64x500].[500x10]",
-                config="C5", dtype="f32", unit="us per chain", higher_is_better=False, **r, gflops=round(flops / best / 1e9, 1),
-                roofline=hbm_roof(nbytes / best / 1e9))
+                config="C5", unit="us per chain", higher_is_better=False, **r, gflops=round(flops / best / 1e9, 1),
+                roofline=dict(hbm_roof(nbytes / best / 1e9), unit="GB/s"))
 
 
 @workload("chain_phases", default=False)
@@ -603,13 +626,12 @@ def wl_chain_phases(ctx):
         for _ in range(ctx.steps):
             for _ in range(3):
                 issue()                      # the launch that is measured follows others, as in the chain
-            L.am_hip_diag_clock_begin()
+            L.am_hip_diag_phases_begin()
             L.am_hip_event_record(timer.e0)
             f()
             L.am_hip_event_record(timer.e1)
             L.am_hip_diag_phases(buf)
             L.am_hip_event_elapsed_ms(timer.e0, timer.e1, ctypes.byref(ms))
-            L.am_hip_diag_clock_end(ctypes.byref(mhz))
             acc += np.array(list(buf))
             ev_us += ms.value * 1e3
         acc /= ctx.steps
@@ -633,7 +655,7 @@ def wl_ex02(ctx, batch=64):
     r, best = eager_and_graph(ctx, lambda: net.forward(dx), lambda: net.capture(dx), steps)
     flops = 2.0 * batch * (20 * 25 * 576 + 50 * 500 * 64 + 800 * 500 + 500 * 10)
     return dict(workload=f"f32 example-2 forward pass, batch {batch}, 6 launches",
-                config="f2", dtype="f32", unit="us per pass", higher_is_better=False, **r, images_per_s=round(batch / best, 0),
+                config="f2", unit="us per pass", higher_is_better=False, **r, images_per_s=round(batch / best, 0),
                 gflops=round(flops / best / 1e9, 1))
 
 
@@ -651,7 +673,7 @@ def tall_buffers(ctx):
 def hbm_entry(ctx, workload_name, config, launches, nbytes):
     cold = run_rotating(ctx.timer, launches, max(ctx.steps // len(launches), 4))
     gbs = nbytes / cold / 1e9
-    return dict(workload=workload_name, config=config, dtype="f32", unit="GB/s", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 5),
+    return dict(workload=workload_name, config=config, unit="GB/s", value=round(gbs, 1), ms_per_step=round(cold * 1e3, 5),
                 roofline=hbm_roof(gbs))
 
 
@@ -692,7 +714,7 @@ def wl_gemm_long_k(ctx):
     k = max(ctx.steps, 20)
     wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, ctx.warmup)
     fl = 2.0 * 500 * 800 * 65536
-    return dict(workload="f32 GEMM [500x65536].[65536x800]", config="a19", dtype="f32",
+    return dict(workload="f32 GEMM [500x65536].[65536x800]", config="a19",
                 unit="TFLOP/s", value=round(fl * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 5),
                 roofline=mfma_roof(fl / (ev / k) / 1e12, MFMA_F32_PEAK_TFLOPS, timer.sclk_mhz))
 
@@ -792,7 +814,7 @@ def wl_conv_backward(ctx):
     _, ev_f = timer.run(lambda: am.conv2d(x, w, b, (pad, pad), (1, 1)), steps, ctx.warmup)
     _, ev_b = timer.run(lambda: am.conv2d_backward(x, w, b, (pad, pad), (1, 1), g), steps, ctx.warmup)
     fl = 2.0 * N * co * ho * ho * C * k * k
-    return dict(workload="f32 conv2d_backward [64,64,56,56], 64 kernels 3x3, pad 1", unit="TFLOP/s", dtype="f32",
+    return dict(workload="f32 conv2d_backward [64,64,56,56], 64 kernels 3x3, pad 1", unit="TFLOP/s",
                 value=round(2 * fl / (ev_b / steps) / 1e12, 2), ms_per_step=round(ev_b / steps * 1e3, 5), forward_ms=round(ev_f / steps * 1e3, 5),
                 roofline=mfma_roof(2 * fl / (ev_b / steps) / 1e12, MFMA_F32_PEAK_TFLOPS, None))
 
@@ -809,7 +831,7 @@ def wl_ex02_train(ctx, batch=64):
     dl = am.toHip(rng.integers(0, 10, batch).astype(np.int64))
     steps = max(ctx.steps, 20)
     r, best = eager_and_graph(ctx, lambda: net.train_step(dx, dl, 0.01), lambda: net.capture_train_step(dx, dl, 0.01), steps)
-    return dict(workload=f"f32 example-2 training step, batch {batch}", unit="us per step", dtype="f32", higher_is_better=False, **r,
+    return dict(workload=f"f32 example-2 training step, batch {batch}", unit="us per step", higher_is_better=False, **r,
                 images_per_s=round(batch / best, 0))
 
 
@@ -850,7 +872,7 @@ def config_report(am, timer, L):
         want = am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy())
         cpu_s = cpu_time(lambda: am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy() if beta != 0 else C_host))
         ops = 2.0 * M * N * K
-        row = dict(config=config, dtype=sfx, shape=[M, N, K], gpu_ms=round(gpu_s * 1e3, 4),
+        row = dict(config=config, shape=[M, N, K], gpu_ms=round(gpu_s * 1e3, 4),
                    gpu_rate=round(ops / gpu_s / 1e12, 3), rate_unit=unit,
                    pct_peak=round(100 * ops / gpu_s / 1e12 / peak, 1) if peak else None, peak_used=peak_used,
                    cpu_impl="oracle/laser_gemm.c (port of laser gemm_strided, OpenMP)", cpu_threads=threads,
@@ -932,7 +954,7 @@ def config_report(am, timer, L):
         hb = am_oracle.broadcast(hv, X.shape)
         out = np.empty_like(X)
         cpu_s = cpu_time(lambda: am_oracle.map2(op, X, hb, out=out))
-        emit(config=f"f32 8192x8192 {name}", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
+        emit(config=f"f32 8192x8192 {name}", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
              gpu_rate=round(nbytes / gpu_s / 1e9, 1), rate_unit="GB/s", pct_peak=round(100 * nbytes / gpu_s / 1e9 / HBM_PEAK_GBS, 1),
              peak_used="HBM 8000 GB/s", cpu_impl="oracle/strided_map.c (port of map2_inline + strided iteration, OpenMP blocks)",
              cpu_threads=threads, cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1),
@@ -942,7 +964,7 @@ def config_report(am, timer, L):
     _, ev = timer.run(lambda: th._ternary_into("addmul", dY, dX, bb, sb), 50, 5)
     gpu_s = run_rotating(timer, [(lambda i=i: th._ternary_into("addmul", dYs[i], dXs[i], bb, sb)) for i in range(ROTATE)], 10)
     two_pass = ((X + b) * sc)
-    emit(config="f32 8192x8192 (X +. b) *. s fused (one pass)", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
+    emit(config="f32 8192x8192 (X +. b) *. s fused (one pass)", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
          gpu_rate=round((nbytes + 8192 * 4) / gpu_s / 1e9, 1), rate_unit="GB/s",
          pct_peak=round(100 * (nbytes + 8192 * 4) / gpu_s / 1e9 / HBM_PEAK_GBS, 1), peak_used="HBM 8000 GB/s",
          bit_exact=bool(np.array_equal(dYs[ROTATE - 1].toCpu(), two_pass)),
@@ -956,7 +978,7 @@ def config_report(am, timer, L):
              X + Xt, lambda: am_oracle.map2("add", X, X.T, out=out))):
         gpu_s = run_rotating(timer, [(lambda i=i: launch(i)) for i in range(ROTATE)], 10)
         cpu_s = cpu_time(cpu_fn, budget=2.0)
-        emit(config=f"f32 8192x8192 {name}", dtype="f32", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
+        emit(config=f"f32 8192x8192 {name}", shape=[8192, 8192], gpu_ms=round(gpu_s * 1e3, 4),
              gpu_rate=round(nb / gpu_s / 1e9, 1), rate_unit="GB/s", pct_peak=round(100 * nb / gpu_s / 1e9 / HBM_PEAK_GBS, 1),
              peak_used="HBM 8000 GB/s", cpu_impl="NumPy strided copy" if "clone" in name else "oracle/strided_map.c (strided iteration, OpenMP blocks)",
              cpu_threads=1 if "clone" in name else threads, cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1),
@@ -971,7 +993,7 @@ def config_report(am, timer, L):
         _, ev = timer.run(lambda: fn_gpu(inputs[0]), 50, 5)
         gpu_s = run_rotating(timer, [(lambda x=x: fn_gpu(x)) for x in inputs], 10)
         cpu_s = cpu_time(fn_cpu, budget=2.0)
-        emit(config=config, dtype="f32", gpu_ms=round(gpu_s * 1e3, 4), gpu_rate=round(nbytes / gpu_s / 1e9, 1), rate_unit="GB/s",
+        emit(config=config, gpu_ms=round(gpu_s * 1e3, 4), gpu_rate=round(nbytes / gpu_s / 1e9, 1), rate_unit="GB/s",
              pct_peak=round(100 * nbytes / gpu_s / 1e9 / HBM_PEAK_GBS, 1), peak_used="HBM 8000 GB/s",
              cpu_impl="oracle/reduce_pool.c (serial port of the reference's fold / softmax / maxpool2d)", cpu_threads=1,
              cpu_ms=round(cpu_s * 1e3, 2), speedup_vs_cpu=round(cpu_s / gpu_s, 1), note=warm_note(ev / 50, nbytes), **check(got, want))
@@ -991,19 +1013,19 @@ def config_report(am, timer, L):
              lambda g, w: dict(bit_exact=bool(np.array_equal(g[1].toCpu(), w[1]) and np.array_equal(g[0].toCpu(), w[0]))), dPs)
     del dPs
     r = wl_chain(ctx)
-    emit(config="f32 inference chain (4 GEMMs, fused bias+ReLU)", dtype="f32", hipgraph_us=r.get("hipgraph_us"), eager_us=r["eager_us"])
+    emit(config="f32 inference chain (4 GEMMs, fused bias+ReLU)", hipgraph_us=r.get("hipgraph_us"), eager_us=r["eager_us"])
     r = wl_ex02(ctx)
-    emit(config="f32 example-2 forward pass, batch 64 (6 kernels)", dtype="f32", hipgraph_us=r.get("hipgraph_us"), eager_us=r["eager_us"])
+    emit(config="f32 example-2 forward pass, batch 64 (6 kernels)", hipgraph_us=r.get("hipgraph_us"), eager_us=r["eager_us"])
 
 
 # Order of the default line: the float32 / float64 matrix workloads first (the int8 chains of the ceilings and the
 # digit-sliced products leave the chip at a lowered clock for a while), then the integer ones, then the rest.
 DEFAULT_ORDER = ["gemm_f32_1024", "gemm_f32_2048", "gemm_f64", "gemm_f32_long_k",
-                 "gemm_i32_1500", "gemm_i32", "gemm_i32_whole_range", "gemm_i64", "matmul_i64_1500_published",
+                 "gemm_i32_1500", "gemm_i32", "gemm_i32_prepared", "gemm_i32_whole_range", "gemm_i64", "matmul_i64_1500_published",
                  "bcast_add_rotating", "bcast_mul_rotating", "bias_relu_rotating", "bcast_addmul_fused_rotating", "transposed_add",
                  "bias_short_rows", "sum_cols_narrow", "sum_rows_512", "chain", "ex02"]
 # ... and the order they are printed in: by configuration
-PRINT_ORDER = ["gemm_f32_1024", "gemm_f32_2048", "gemm_i32_1500", "gemm_i32", "gemm_i32_whole_range", "gemm_i64", "matmul_i64_1500_published",
+PRINT_ORDER = ["gemm_f32_1024", "gemm_f32_2048", "gemm_i32_1500", "gemm_i32", "gemm_i32_prepared", "gemm_i32_whole_range", "gemm_i64", "matmul_i64_1500_published",
                "gemm_f64", "bcast_add_rotating", "bcast_mul_rotating", "bias_relu_rotating", "bcast_addmul_fused_rotating", "chain",
                "ex02", "transposed_add", "bias_short_rows", "sum_cols_narrow", "sum_rows_512", "gemm_f32_long_k"]
 
@@ -1051,10 +1073,9 @@ def main():
     tflops = r["flops"] * args.steps / r["wall"] / 1e12
     kern_tflops = r["flops"] / (r["ev"] / args.steps) / 1e12
     traffic, traffic_src = load_traffic("gemm_f32_4096")
-    roof = mfma_roof(kern_tflops, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"])
+    roof = mfma_roof(kern_tflops, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"], unit="TFLOP/s")
     roof.update(traffic=traffic, traffic_source=traffic_src)
-    protocol = ("every entry: register-only chain of its arithmetic type, >= 30 ms of its own launches, then K timed between HIP events; "
-                "HBM-bound entries rotate 3-5 buffer sets so every byte comes from HBM")
+    protocol = "per entry: register-only spin, >= 30 ms of its own launches, K timed between HIP events; HBM-bound ones rotate 3-5 buffer sets"
     line = {
         "metric": "GEMM TFLOP/s (%MFMA peak) fp32/int32 4096^3; broadcast op HBM GB/s (%peak)",
         "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -1064,7 +1085,7 @@ def main():
         "roofline": roof,
         "from_idle": {"value": round(idle["flops"] * args.steps / idle["wall"] / 1e12, 3), "unit": "TFLOP/s",
                       "ms_per_step": round(idle["wall"] / args.steps * 1e3, 4), "sclk_mhz": idle["sclk_mhz"],
-                      "what": "same W + K steps from an idle device; `value` follows 80 ms of register-only MFMA work (not the workload)"},
+                      "what": "same steps from an idle device; `value` follows 80 ms of register-only MFMA work"},
         "device": info, "protocol": protocol,
     }
     if not args.no_others:

@@ -150,6 +150,31 @@ int am_hip_gemm_i64(int64_t M, int64_t N, int64_t K, int64_t alpha,
                     const int64_t* B, int64_t rsB, int64_t csB,
                     int64_t beta, int64_t* C, int64_t rsC, int64_t csC);
 
+/* Integer products whose operand is reused (a weight matrix that enters many products): large int32 / int64 products
+ * run on the int8 matrix cores after both operands have been split into base-256 digit planes, two passes over every
+ * operand in every call. am_hip_digits_prepare_* makes those planes once for one operand and returns a handle;
+ * am_hip_gemm_prepared_* is am_hip_gemm_i32 / _i64 with such a handle beside either operand (NULL = split that operand
+ * in the call, as always). Same result bits as am_hip_gemm_* (ring arithmetic). No counterpart in the reference, whose
+ * gemm_strided packs both operands in every call (gemm_packing.nim:24-99).
+ *   side 0: X is the left operand [rows x cols] = [M x K]; side 1: the right operand [K x N]; element [r, c] at
+ *   X[r * rs + c * cs], any strides. Blocking (it reports which planes came out empty). The planes take
+ *   sizeof(T) x roundup(M or N, 256) x roundup(K, 256) bytes from am_hip_malloc until am_hip_digits_release.
+ * The planes are a snapshot: after the operand's elements change, release the handle and prepare again. The original
+ * operand is still passed to am_hip_gemm_prepared_*: products that cannot take the matrix-core path (a long int64 k,
+ * one operand unprepared while a graph is being captured) are computed from it. A handle whose extents do not match
+ * the product is refused with AM_E_SHAPE, a pointer that is no live handle with AM_E_ARG. */
+int am_hip_digits_prepare_i32(int side, int64_t rows, int64_t cols, const int32_t* X, int64_t rs, int64_t cs, void** handle);
+int am_hip_digits_prepare_i64(int side, int64_t rows, int64_t cols, const int64_t* X, int64_t rs, int64_t cs, void** handle);
+int am_hip_digits_release(void* handle);   /* NULL is a no-op; a released or foreign pointer is AM_E_ARG */
+int am_hip_gemm_prepared_i32(int64_t M, int64_t N, int64_t K, int32_t alpha,
+                             const int32_t* A, int64_t rsA, int64_t csA, const void* A_digits,
+                             const int32_t* B, int64_t rsB, int64_t csB, const void* B_digits,
+                             int32_t beta, int32_t* C, int64_t rsC, int64_t csC);
+int am_hip_gemm_prepared_i64(int64_t M, int64_t N, int64_t K, int64_t alpha,
+                             const int64_t* A, int64_t rsA, int64_t csA, const void* A_digits,
+                             const int64_t* B, int64_t rsB, int64_t csB, const void* B_digits,
+                             int64_t beta, int64_t* C, int64_t rsC, int64_t csC);
+
 /* am_hip_gemm_f32 for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
  * arguments and kernels as am_hip_gemm_f32, and the same tile and split of K - hence the same result
@@ -757,12 +782,14 @@ int am_hip_diag_hbm(int kind, size_t bytes, int windows, int blocks_per_cu, int 
 int am_hip_diag_clock_begin(void);
 int am_hip_diag_clock_end(double* shader_mhz);
 /* Where the time of a small-product launch (min(M, N) <= 64: the kernels without LDS staging) goes, read inside the
- * kernel between am_hip_diag_clock_begin and _end by the first lane of every workgroup, in microseconds: out6[0]
+ * kernel between am_hip_diag_phases_begin and am_hip_diag_phases (which closes the window; blocking) by the first lane
+ * of every workgroup (up to 8192 of them), in microseconds: out6[0]
  * workgroups that reported; out6[1..4] the mean time from the first instruction to the first loads issued, from there
  * until they have arrived, from there to the last matrix instruction and the fold of the wavefronts' partial tiles,
  * and from there until the stores are done; out6[5] from the earliest first instruction to the latest store over the
  * whole launch (what the launch's duration on a profiler's timeline exceeds by the dispatch and end-of-kernel work).
  * One launch per window. No counterpart in the reference. */
+int am_hip_diag_phases_begin(void);
 int am_hip_diag_phases(double* out6);
 
 #ifdef __cplusplus

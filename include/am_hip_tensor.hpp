@@ -604,6 +604,52 @@ void gemm(T alpha, const HipTensor<T>& A, const HipTensor<T>& B, T beta, HipTens
 }
 
 // y <- alpha A x + beta y (operators_blas_l2l3.nim:24-56)
+// Digit planes of an integer matrix split once for products that reuse it (a weight matrix). No counterpart in the
+// reference, whose gemm_strided packs both operands in every call (gemm_packing.nim:24-99). A snapshot of the matrix.
+class DigitPlanes {
+ public:
+  DigitPlanes() = default;
+  template <typename T>
+  DigitPlanes(const HipTensor<T>& t, bool right_operand) {
+    static_assert(std::is_same<T, int32_t>::value || std::is_same<T, int64_t>::value, "digit planes belong to int32_t / int64_t matrices");
+    if (t.rank() != 2) throw std::invalid_argument("DigitPlanes: the operand must be a matrix");
+    if constexpr (std::is_same<T, int32_t>::value)
+      check(am_hip_digits_prepare_i32(right_operand ? 1 : 0, t.shape[0], t.shape[1], t.ptr(), t.strides[0], t.strides[1], &handle_));
+    else
+      check(am_hip_digits_prepare_i64(right_operand ? 1 : 0, t.shape[0], t.shape[1], t.ptr(), t.strides[0], t.strides[1], &handle_));
+  }
+  ~DigitPlanes() { (void)am_hip_digits_release(handle_); }
+  DigitPlanes(const DigitPlanes&) = delete;
+  DigitPlanes& operator=(const DigitPlanes&) = delete;
+  DigitPlanes(DigitPlanes&& o) noexcept : handle_(o.handle_) { o.handle_ = nullptr; }
+  DigitPlanes& operator=(DigitPlanes&& o) noexcept {
+    if (this != &o) { (void)am_hip_digits_release(handle_); handle_ = o.handle_; o.handle_ = nullptr; }
+    return *this;
+  }
+  void* handle() const { return handle_; }
+
+ private:
+  void* handle_ = nullptr;
+};
+
+// gemm with the digit planes of A and / or B split ahead of time (nullptr: split that operand in the call).
+inline void gemm(int32_t alpha, const HipTensor<int32_t>& A, const HipTensor<int32_t>& B, int32_t beta, HipTensor<int32_t>& C,
+                 const DigitPlanes* a_digits, const DigitPlanes* b_digits) {
+  if (A.rank() != 2 || B.rank() != 2 || C.rank() != 2) throw std::invalid_argument("gemm: A, B and C must be matrices");
+  if (A.shape[1] != B.shape[0] || C.shape[0] != A.shape[0] || C.shape[1] != B.shape[1]) throw std::out_of_range("gemm: shapes do not agree");
+  check(am_hip_gemm_prepared_i32(A.shape[0], B.shape[1], A.shape[1], alpha, A.ptr(), A.strides[0], A.strides[1],
+                                 a_digits ? a_digits->handle() : nullptr, B.ptr(), B.strides[0], B.strides[1],
+                                 b_digits ? b_digits->handle() : nullptr, beta, C.ptr(), C.strides[0], C.strides[1]));
+}
+inline void gemm(int64_t alpha, const HipTensor<int64_t>& A, const HipTensor<int64_t>& B, int64_t beta, HipTensor<int64_t>& C,
+                 const DigitPlanes* a_digits, const DigitPlanes* b_digits) {
+  if (A.rank() != 2 || B.rank() != 2 || C.rank() != 2) throw std::invalid_argument("gemm: A, B and C must be matrices");
+  if (A.shape[1] != B.shape[0] || C.shape[0] != A.shape[0] || C.shape[1] != B.shape[1]) throw std::out_of_range("gemm: shapes do not agree");
+  check(am_hip_gemm_prepared_i64(A.shape[0], B.shape[1], A.shape[1], alpha, A.ptr(), A.strides[0], A.strides[1],
+                                 a_digits ? a_digits->handle() : nullptr, B.ptr(), B.strides[0], B.strides[1],
+                                 b_digits ? b_digits->handle() : nullptr, beta, C.ptr(), C.strides[0], C.strides[1]));
+}
+
 template <typename T>
 void gemv(T alpha, const HipTensor<T>& A, const HipTensor<T>& x, T beta, HipTensor<T>& y) {
   if (A.rank() != 2 || x.rank() != 1 || y.rank() != 1) throw std::invalid_argument("gemv: A must be a matrix, x and y vectors");

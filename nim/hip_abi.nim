@@ -53,6 +53,7 @@ proc am_hip_graph_destroy*(graph_exec: pointer): cint {.importc.}
 proc am_hip_diag_peak*(kind, iters, waves_per_simd: cint, ops_per_second: ptr cdouble): cint {.importc.}
 proc am_hip_diag_clock_begin*(): cint {.importc.}
 proc am_hip_diag_clock_end*(shader_mhz: ptr cdouble): cint {.importc.}
+proc am_hip_diag_phases_begin*(): cint {.importc.}
 proc am_hip_diag_phases*(out6: ptr cdouble): cint {.importc.}
 proc am_hip_diag_hbm*(kind: cint, bytes: csize_t, windows, blocks_per_cu, unroll, flags, launches: cint,
                       bytes_per_second: ptr cdouble): cint {.importc.}
@@ -73,6 +74,16 @@ proc am_hip_gemm_i32*(M, N, K: int64, alpha: int32, A: ptr int32, rsA, csA: int6
 proc am_hip_gemm_i64*(M, N, K: int64, alpha: int64, A: ptr int64, rsA, csA: int64,
                       B: ptr int64, rsB, csB: int64, beta: int64,
                       C: ptr int64, rsC, csC: int64): cint {.importc.}
+
+proc am_hip_digits_prepare_i32*(side: cint, rows, cols: int64, X: ptr int32, rs, cs: int64, handle: ptr pointer): cint {.importc.}
+proc am_hip_digits_prepare_i64*(side: cint, rows, cols: int64, X: ptr int64, rs, cs: int64, handle: ptr pointer): cint {.importc.}
+proc am_hip_digits_release*(handle: pointer): cint {.importc.}
+proc am_hip_gemm_prepared_i32*(M, N, K: int64, alpha: int32, A: ptr int32, rsA, csA: int64, A_digits: pointer,
+                               B: ptr int32, rsB, csB: int64, B_digits: pointer, beta: int32,
+                               C: ptr int32, rsC, csC: int64): cint {.importc.}
+proc am_hip_gemm_prepared_i64*(M, N, K: int64, alpha: int64, A: ptr int64, rsA, csA: int64, A_digits: pointer,
+                               B: ptr int64, rsB, csB: int64, B_digits: pointer, beta: int64,
+                               C: ptr int64, rsC, csC: int64): cint {.importc.}
 
 proc am_hip_gemm_batched_f32*(batch, M, N, K: int64, alpha: cfloat, A: ptr cfloat, rsA, csA, bsA: int64,
                               B: ptr cfloat, rsB, csB, bsB: int64, beta: cfloat, C: ptr cfloat, rsC, csC, bsC: int64,

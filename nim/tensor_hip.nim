@@ -490,6 +490,41 @@ proc gemm*[T: HipScalar](alpha: T, A, B: HipTensor[T], beta: T, C: var HipTensor
   elif T is int32: call am_hip_gemm_i32
   else: call am_hip_gemm_i64
 
+# Digit planes of an integer matrix split once for products that reuse it (a weight matrix): no counterpart in the
+# reference, whose gemm_strided packs both operands in every call (gemm_packing.nim:24-99).
+type
+  HipDigitPlanesObj* = object
+    handle*: pointer
+  HipDigitPlanes* = ref HipDigitPlanesObj
+
+proc `=destroy`*(p: HipDigitPlanesObj) =
+  if not p.handle.isNil: discard am_hip_digits_release(p.handle)
+
+proc digitsPrepare*[T: int32 | int64](t: HipTensor[T], rightOperand = true): HipDigitPlanes =
+  ## Planes of `t` as the right ([K x N]) or left ([M x K]) operand of later products. A snapshot: prepare again
+  ## after `t` changes. Blocking.
+  new result
+  when T is int32:
+    check am_hip_digits_prepare_i32(cint(ord(rightOperand)), int64 t.shape[0], int64 t.shape[1], t.get_offset_ptr,
+                                    int64 t.strides[0], int64 t.strides[1], result.handle.addr)
+  else:
+    check am_hip_digits_prepare_i64(cint(ord(rightOperand)), int64 t.shape[0], int64 t.shape[1], t.get_offset_ptr,
+                                    int64 t.strides[0], int64 t.strides[1], result.handle.addr)
+
+proc gemm*[T: int32 | int64](alpha: T, A, B: HipTensor[T], beta: T, C: var HipTensor[T], aDigits, bDigits: HipDigitPlanes) =
+  ## `gemm` with the digit planes of A and / or B split ahead of time (nil: split that operand in the call).
+  if A.rank != 2 or B.rank != 2 or C.rank != 2:
+    raise newException(ValueError, "gemm: A, B and C must be matrices")
+  let (M, N, K) = (int64 A.shape[0], int64 B.shape[1], int64 A.shape[1])
+  let ha = if aDigits.isNil: nil else: aDigits.handle
+  let hb = if bDigits.isNil: nil else: bDigits.handle
+  template call(f: untyped) =
+    check f(M, N, K, alpha, A.get_offset_ptr, int64 A.strides[0], int64 A.strides[1], ha,
+            B.get_offset_ptr, int64 B.strides[0], int64 B.strides[1], hb, beta,
+            C.get_offset_ptr, int64 C.strides[0], int64 C.strides[1])
+  when T is int32: call am_hip_gemm_prepared_i32
+  else: call am_hip_gemm_prepared_i64
+
 proc gemv*[T: HipScalar](alpha: T, A, x: HipTensor[T], beta: T, y: var HipTensor[T]) =
   ## y <- alpha A x + beta y (operators_blas_l2l3.nim:24-56)
   template call(f: untyped) =

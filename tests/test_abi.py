@@ -204,3 +204,13 @@ def test_unsigned_tensors_take_the_signed_kernels_for_ring_operations_only():
     assert _fake((2, 2), np.int32).ring_sfx == "i32" and _fake((2, 2)).ring_sfx == "f32"
     with pytest.raises(TypeError):
         am.empty((2, 2), np.uint16)
+
+
+def test_digit_plane_handles_that_the_library_did_not_hand_out_are_refused():
+    L = am.load_library()
+    bogus = ctypes.c_void_p(0x1234560)
+    assert L.am_hip_digits_release(bogus) == _lib.AM_E_ARG and "not a handle" in _lib.last_error()
+    assert L.am_hip_digits_release(None) == _lib.AM_OK
+    z = ctypes.c_void_p(0x1000)
+    rc = L.am_hip_gemm_prepared_i32(4, 4, 4, 1, z, 4, 1, bogus, z, 4, 1, None, 0, z, 4, 1)
+    assert rc == _lib.AM_E_ARG and "not a live handle" in _lib.last_error()

@@ -636,6 +636,82 @@ def test_int32_digit_sliced_matrix_core_path(hip, oracle, tile, monkeypatch):
         assert np.array_equal(dW.toCpu(), want), f"{shape} stepped destination"
 
 
+@pytest.mark.parametrize("sfx", ["i32", "i64"])
+@pytest.mark.parametrize("tile", ["", "0", "2", "3"])
+def test_prepared_digit_planes(hip, oracle, sfx, tile, monkeypatch):
+    """Products whose A and / or B operand was split into digit planes ahead of time (digits_prepare): the bits of
+    the plain product and of the oracle, for one-plane entries and whole-range ones, contiguous / transposed / stepped
+    operands on either side, ragged extents (the planes are padded to 256 rows whatever tile the product takes),
+    row- and column-major destinations (the latter exchanges the operands' roles inside the library), every alpha /
+    beta case; the same planes serve several products."""
+    if tile:
+        monkeypatch.setenv("AM_HIP_GEMM_TILE_I8", tile)
+    dt = DTYPES[sfx]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(seed_of("prepared", sfx, tile))
+    for (M, N, K), (lo, hi) in [((70, 90, 300), (-100, 100)), ((257, 129, 700), (info.min, info.max)), ((300, 513, 260), (-40000, 40000)),
+                                ((64, 64, 256), (info.min, info.max)), ((1, 5, 3), (-5, 5))]:
+        say("prepared digits", sfx, tile, (M, N, K), (lo, hi))
+        A, B, C = fill(rng, (M, K), dt, lo, hi), fill(rng, (K, N), dt, lo, hi), fill(rng, (M, N), dt, info.min, info.max)
+        # B as a transposed view of an [N x K] buffer, A as every other row of a taller one
+        A2 = np.zeros((2 * M, K), dtype=dt); A2[::2] = A
+        dA, dB = hip.toHip(A2)[::2], hip.toHip(np.ascontiguousarray(B.T)).transpose()
+        pa, pb = hip.digits_prepare(dA, "left"), hip.digits_prepare(dB, "right")
+        for alpha, beta in [(1, 0), (-3, 7), (info.min, info.max)]:
+            want = oracle.gemm_strided(alpha, A, B, beta, C.copy())
+            for a_d, b_d in [(pa, None), (None, pb), (pa, pb)]:
+                dC = hip.toHip(C)
+                hip.gemm(alpha, dA, dB, beta, dC, a_digits=a_d, b_digits=b_d)
+                assert np.array_equal(dC.toCpu(), want), f"{(M, N, K)} a={alpha} b={beta} prepared={(a_d is not None, b_d is not None)}"
+        dCt = hip.toHip(np.zeros((N, M), dtype=dt)).transpose()          # column-major C: roles exchanged inside
+        hip.gemm(1, dA, dB, 0, dCt, a_digits=pa, b_digits=pb)
+        assert np.array_equal(dCt.toCpu(), oracle.matmul(A, B))
+        dCt = hip.toHip(np.zeros((N, M), dtype=dt)).transpose()
+        hip.gemm(1, dA, dB, 0, dCt, b_digits=pb)
+        assert np.array_equal(dCt.toCpu(), oracle.matmul(A, B))
+        # the planes of B with another left operand
+        A3 = fill(rng, (33, K), dt, lo, hi)
+        out = hip.empty((33, N), dt)
+        hip.gemm(1, hip.toHip(A3), dB, 0, out, b_digits=pb)
+        assert np.array_equal(out.toCpu(), oracle.matmul(A3, B))
+        # a handle of the wrong extents or side is refused, a released one too
+        with pytest.raises(ValueError):
+            hip.gemm(1, hip.toHip(A3), dB, 0, out, a_digits=pa, b_digits=pb)
+        with pytest.raises(ValueError):
+            hip.gemm(1, dA, dB, 0, hip.empty((M, N), dt), a_digits=pb)
+        stale = hip.DigitPlanes(pa.handle, 0, pa.shape, pa.dtype)
+        pa.release()
+        with pytest.raises(ValueError):
+            hip.gemm(1, dA, dB, 0, hip.empty((M, N), dt), a_digits=stale)
+        with pytest.raises(ValueError):
+            stale.release()
+        stale.handle = 0
+
+
+def test_prepared_digit_planes_at_size_and_in_a_graph(hip, oracle):
+    """2048 x 1500 x 1700 int32 with entries in [-100, 100] and over the whole range, B prepared; and both operands
+    prepared inside a captured graph (nothing left to allocate), replayed twice."""
+    rng = np.random.default_rng(seed_of("prepared at size"))
+    for lo, hi in [(-100, 100), (-2**31, 2**31 - 1)]:
+        A, B = fill(rng, (2048, 1700), np.int32, lo, hi), fill(rng, (1700, 1500), np.int32, lo, hi)
+        dA, dB = hip.toHip(A), hip.toHip(B)
+        pb = hip.digits_prepare(dB, "right")
+        out = hip.empty((2048, 1500), np.int32)
+        hip.gemm(1, dA, dB, 0, out, b_digits=pb)
+        assert np.array_equal(out.toCpu(), oracle.matmul(A, B))
+    A, B = fill(rng, (300, 400), np.int64, -1000, 1000), fill(rng, (400, 200), np.int64, -1000, 1000)
+    dA, dB, out = hip.toHip(A), hip.toHip(B), hip.zeros((300, 200), np.int64)
+    pa, pb = hip.digits_prepare(dA, "left"), hip.digits_prepare(dB, "right")
+    hip.gemm(1, dA, dB, 0, out, a_digits=pa, b_digits=pb)
+    with hip.Graph() as g:
+        hip.gemm(1, dA, dB, 1, out, a_digits=pa, b_digits=pb)
+    want = oracle.matmul(A, B)
+    for rep in range(2):
+        g.launch()
+        hip.sync()
+        assert np.array_equal(out.toCpu(), (rep + 2) * want)
+
+
 def test_int32_paths_agree_at_size(hip, oracle, monkeypatch):
     """2048^3 and a ragged 1500 x 1300 x 1700 product: the automatic choice, the matrix-core path
     and the VALU path give the same bits (and those of the CPU oracle)."""
