@@ -48,6 +48,7 @@ VALU_FULL_RATE_TOPS = 78.6     # 256 CU x 64 lanes x 2 ops x 2.4 GHz: one 32-bit
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 SPIN_F32, SPIN_F64, SPIN_VALU32, SPIN_VALU64, SPIN_I8 = 0, 1, 2, 3, 4   # kinds of am_hip_diag_peak
+MATRIX_WARM_S = 1.0   # seconds of its own launches before a matrix-bound entry is timed (see Timer.run)
 ROTATE = 5   # buffer sets of the rotating protocol: together far beyond the 256 MB memory-side cache
 
 
@@ -81,17 +82,20 @@ class Timer:
         L.am_hip_event_create(ctypes.byref(self.e1))
         self.sclk_mhz = None
         self.launches = 0
+        self.history = []
 
-    def run(self, fn, steps, warmup, spin=(SPIN_F32, 0.08), min_warm_s=0.03):
+    def run(self, fn, steps, warmup, spin=(SPIN_F32, 0.08), min_warm_s=0.05):
         """`spin` = (kind, seconds) of register-only work first (None: start from whatever state the device is in, and
         no time-based warm-up either), then `warmup` untimed calls of fn - continued until they have kept the device
-        busy for min_warm_s: the clock governor reacts within milliseconds, so what a short kernel is timed at is the
-        clock its own launches sustain, and the spin only spares them the long climb from idle - then `steps` timed
-        ones. While the timed steps run, the GEMM kernels count shader cycles against the constant-rate counter
+        busy for min_warm_s: what a kernel is timed at is the clock its own launches sustain, and the governor settles
+        slowly after the kind of work changes (f32 1024^3 launches: 2.03 GHz after 30 ms of them, 2.20 after 0.3 s,
+        2.32 after 1 s; the matrix-bound entries therefore warm up for MATRIX_WARM_S) - then `steps` timed ones. While the timed steps run, the GEMM kernels count shader cycles against the constant-rate counter
         (am_hip_diag_clock_*): self.sclk_mhz is the shader clock they sustained (None when no such kernel ran).
         Returns (wall seconds, event seconds) for all timed steps."""
         if spin:
             spin_up(self.L, spin[1], spin[0])
+        if "BENCH_WARM_S" in os.environ:      # experiments
+            min_warm_s = float(os.environ["BENCH_WARM_S"])
         extra = 0
         self.L.am_hip_event_record(self.e0)
         for _ in range(warmup):
@@ -123,6 +127,7 @@ class Timer:
             if self.L.am_hip_diag_clock_end(ctypes.byref(mhz)) == 0 and mhz.value > 0:
                 self.sclk_mhz = round(mhz.value, 0)
         self.launches = steps + warmup + extra
+        self.history.append(steps)            # timed steps of every run, in order (what a trace of --only is cut by)
         return wall, ms.value / 1e3
 
 
@@ -231,17 +236,17 @@ def workload(name, default=True):
 
 
 # ------------------------------------------------------------------------------------------ headline and C1
-def bench_gemm_f32(ctx, steps, warmup, n=4096, host=None, spin=(SPIN_F32, 0.08)):
+def bench_gemm_f32(ctx, steps, warmup, n=4096, host=None, spin=(SPIN_F32, 0.08), min_warm_s=0.0):
     am, timer = ctx.am, ctx.timer
     A, B = host or (np.random.default_rng(1001).uniform(-1, 1, (n, n)).astype(np.float32),
                     np.random.default_rng(1002).uniform(-1, 1, (n, n)).astype(np.float32))
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), np.float32)
-    wall, ev = timer.run(lambda: am.gemm(1.0, dA, dB, 0.0, dC), steps, warmup, spin)
+    wall, ev = timer.run(lambda: am.gemm(1.0, dA, dB, 0.0, dC), steps, warmup, spin, min_warm_s)
     return dict(wall=wall, ev=ev, flops=2.0 * n ** 3, host=(A, B), sclk_mhz=timer.sclk_mhz)
 
 
-def gemm_f32_entry(ctx, n, config, steps):
-    r = bench_gemm_f32(ctx, steps, ctx.warmup, n=n)
+def gemm_f32_entry(ctx, n, config, steps, min_warm_s=MATRIX_WARM_S):
+    r = bench_gemm_f32(ctx, steps, ctx.warmup, n=n, min_warm_s=min_warm_s)
     t = r["flops"] / (r["ev"] / steps) / 1e12
     return dict(workload=f"f32 GEMM {n}^3", config=config, unit="TFLOP/s", value=round(r["flops"] * steps / r["wall"] / 1e12, 3),
                 ms_per_step=round(r["ev"] / steps * 1e3, 5), roofline=mfma_roof(t, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"]))
@@ -249,7 +254,7 @@ def gemm_f32_entry(ctx, n, config, steps):
 
 @workload("gemm_f32", default=False)     # the headline itself, for traces (the default line times it as `value`)
 def wl_gemm_f32(ctx):
-    return gemm_f32_entry(ctx, 4096, "headline", ctx.steps)
+    return gemm_f32_entry(ctx, 4096, "headline", ctx.steps, min_warm_s=0.0)   # the headline's own protocol: spin, W steps, K timed
 
 
 @workload("gemm_f32_1024")
@@ -335,7 +340,7 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
     pairs, npairs = digit_pairs(A, B), (10 if dt == np.int32 else 36)
     dA, dB, dC = am.toHip(A), am.toHip(B), am.empty((n, n), dt)
     kd = max(20, ctx.steps)
-    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), kd, ctx.warmup, (SPIN_I8, 0.08))
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), kd, ctx.warmup, (SPIN_I8, 0.08), min_warm_s=0.3)
     tops = 2.0 * n ** 3 / (ev / kd) / 1e12
     entry = dict(workload=f"{sfx} GEMM {n}^3, {label}", config=config, unit="Top/s", value=round(2.0 * n ** 3 * kd / wall / 1e12, 3),
                  ms_per_step=round(ev / kd * 1e3, 5), digit_pairs=f"{pairs}/{npairs}",
@@ -346,7 +351,7 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
         k = max(3, ctx.steps // 4) if n >= 4096 else max(20, ctx.steps)
         os.environ[env] = "valu"
         try:
-            _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, (SPIN_VALU32 if dt == np.int32 else SPIN_VALU64, 0.08))
+            _, ev_valu = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, 2, (SPIN_VALU32 if dt == np.int32 else SPIN_VALU64, 0.08), min_warm_s=0.3)
         finally:
             del os.environ[env]
         vt = 2.0 * n ** 3 / (ev_valu / k) / 1e12
@@ -386,7 +391,7 @@ def wl_gemm_i32_prepared(ctx):
     kd = max(20, ctx.steps)
     out = []
     for label, kw in (("B's digit planes prepared", dict(b_digits=pb)), ("both operands' digit planes prepared", dict(a_digits=pa, b_digits=pb))):
-        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC, **kw), kd, ctx.warmup, (SPIN_I8, 0.08))
+        wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC, **kw), kd, ctx.warmup, (SPIN_I8, 0.08), min_warm_s=0.3)
         tops = 2.0 * n ** 3 / (ev / kd) / 1e12
         out.append(dict(workload=f"i32 GEMM 4096^3, in [-100,100], {label}", config="C2", unit="Top/s",
                         value=round(2.0 * n ** 3 * kd / wall / 1e12, 3), ms_per_step=round(ev / kd * 1e3, 5),
@@ -452,7 +457,7 @@ def wl_gemm_f64_views(ctx):
     C = np.random.default_rng(3003).standard_normal((2048, 3072))
     dA, dB, dC = am.toHip(pa).transpose(), am.toHip(pb)[:, ::2], am.toHip(C)
     steps = max(ctx.steps, 50)
-    wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, ctx.warmup, (SPIN_F64, 0.1), min_warm_s=0.3)
+    wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, ctx.warmup, (SPIN_F64, 0.1), min_warm_s=MATRIX_WARM_S)
     fl = 2.0 * 2048 * 3072 * 1024
     return dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", config="C3", unit="TFLOP/s",
                 value=round(fl * steps / wall / 1e12, 3), ms_per_step=round(ev / steps * 1e3, 5),
@@ -712,7 +717,7 @@ def wl_gemm_long_k(ctx):
     dB = am.toHip(np.random.default_rng(1004).standard_normal((65536, 800)).astype(np.float32))
     dC = am.empty((500, 800), np.float32)
     k = max(ctx.steps, 20)
-    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, ctx.warmup)
+    wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC), k, ctx.warmup, min_warm_s=MATRIX_WARM_S)
     fl = 2.0 * 500 * 800 * 65536
     return dict(workload="f32 GEMM [500x65536].[65536x800]", config="a19",
                 unit="TFLOP/s", value=round(fl * k / wall / 1e12, 3), ms_per_step=round(ev / k * 1e3, 5),
@@ -1059,7 +1064,8 @@ def main():
         if args.only in ("gemm_i32_1500", "gemm_i32", "gemm_i64"):     # their VALU leg is priced against a measured ceiling
             ctx._ceilings = {}
         r = WORKLOADS[args.only][0](ctx)
-        print(json.dumps(dict(only=args.only, launches=timer.launches, entries=r if isinstance(r, list) else [r])))
+        print(json.dumps(dict(only=args.only, steps=args.steps, warmup=args.warmup, timed_steps_of_each_run=timer.history,
+                              entries=r if isinstance(r, list) else [r])))
         return
     if args.report:
         config_report(am, timer, L)
