@@ -114,6 +114,11 @@ template <typename T, typename MF, int BM, int BN, int BK, int WAVES_M, int WAVE
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 : 1))
 void gemm_mfma(Args<T> p) {
   typedef typename MF::acc_t acc_t;
+  // Every argument the prologue reads is wanted in a scalar register here, so that the argument block's cache lines
+  // are requested together and waited for once: left alone, the compiler requests each line where a field of it is
+  // first used, behind the branches in between (five dependent round trips to memory in front of the first operand load).
+  asm volatile("" ::"s"(p.M), "s"(p.N), "s"(p.K), "s"(p.A), "s"(p.a_mn), "s"(p.a_k), "s"(p.B), "s"(p.b_mn), "s"(p.b_k), "s"(p.C),
+               "s"(p.c_m), "s"(p.c_n), "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.splits), "s"(p.k_chunk), "s"(p.batch), "s"(p.clock_out));
   const ClockProbe probe(p.clock_out);
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int TILE = MF::TILE, VK = MF::VK, KL = MF::KL, KSTEP = VK * KL;

@@ -40,6 +40,40 @@ template <> struct M16<double> {
 
 constexpr int kMaxWaves = 4;
 
+// What the kernels of this file take: only the fields they read, packed into 160 bytes. A short kernel's first
+// instructions wait for its arguments to arrive from memory; the general argument block spreads the fields these
+// kernels need over six cache lines, which the compiler fetched in five dependent round trips (0.7 - 1.4 us before
+// the first operand load was issued, a fifth of the kernel).
+template <typename T> struct SmallArgs {
+  const T* A; const T* B; T* C; const T* bias;
+  int64_t a_mn, a_k, b_mn, b_k, c_m, c_n, bias_m, bias_n;
+  int64_t M, N, K;
+  long long* phase_out;            // PhaseProbe (common.h); null outside a phase window
+  T alpha, beta;
+  int epilogue, nw, phase_cap;     // nw: wavefronts per workgroup (reading blockDim costs another round trip)
+  int per;                         // blocks of 16 k per wavefront = ceil(ceil(K / 16) / nw), from the host: a 64-bit division
+                                   // by a run-time number is some 130 instructions in front of the kernel's first load
+};
+// Called first in a kernel: every field that the kernel reads early is wanted in a scalar register HERE, so that the
+// compiler requests the three cache lines of the argument block together and waits once (left alone it requests each
+// line where a field of it is first used, behind the branches in between: four dependent round trips).
+template <typename T>
+__device__ __forceinline__ void request_args(const SmallArgs<T>& p) {
+  asm volatile("" ::"s"(p.A), "s"(p.B), "s"(p.C), "s"(p.a_mn), "s"(p.a_k), "s"(p.b_mn), "s"(p.b_k), "s"(p.c_m), "s"(p.c_n),
+               "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.phase_out), "s"(p.epilogue), "s"(p.nw), "s"(p.per));
+}
+
+template <typename T>
+static inline SmallArgs<T> small_args(const Args<T>& g, int nw) {
+  SmallArgs<T> s;
+  s.A = g.A; s.B = g.B; s.C = g.C; s.bias = g.bias;
+  s.a_mn = g.a_mn; s.a_k = g.a_k; s.b_mn = g.b_mn; s.b_k = g.b_k; s.c_m = g.c_m; s.c_n = g.c_n; s.bias_m = g.bias_m; s.bias_n = g.bias_n;
+  s.M = g.M; s.N = g.N; s.K = g.K;
+  s.phase_out = g.phase_out; s.alpha = g.alpha; s.beta = g.beta; s.epilogue = g.epilogue; s.nw = nw; s.phase_cap = g.phase_cap;
+  s.per = (int)((((g.K + 15) >> 4) + nw - 1) / nw);
+  return s;
+}
+
 // The four values lane group g feeds to the four steps of the 16-k block at kb: X[x + (kb + 4 g + s) * ld_k].
 template <typename T, bool VEC>
 __device__ __forceinline__ void load4(const T* x, int64_t ld_k, int64_t k, T (&out)[4]) {
@@ -62,13 +96,14 @@ __device__ __forceinline__ void load4(const T* x, int64_t ld_k, int64_t k, T (&o
 // CHUNK: blocks of 16 k whose loads are issued together. The chunks of a wavefront's share are double
 // buffered: the loads of chunk c + 1 are in flight while chunk c is multiplied.
 template <typename T, bool AVEC, bool BVEC, int MAXW, int CHUNK>
-__global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
+__global__ __launch_bounds__(MAXW * 64) void gemm_rows16(SmallArgs<T> p) {
   typedef typename M16<T>::acc_t acc_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][256] partial tiles, W > 1 only
   T (*red)[256] = reinterpret_cast<T (*)[256]>(red_raw);
+  request_args(p);
   // marks: 1 first loads issued, 2 they have arrived, 3 last matrix instruction and fold, 4 stores done
   PhaseProbe probe(p.phase_out, p.phase_cap, (unsigned)((p.N + 15) >> 4));
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = p.nw;
   const int i = lane & 15, g = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * 16;
   // rows / columns past the edge read the last valid one; their results are not stored
@@ -78,7 +113,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
 
   // blocks of 16 k: nfull whole ones and possibly a partial one; wavefront w takes a contiguous share
   const int64_t nfull = p.K >> 4, nblk = (p.K + 15) >> 4;
-  const int64_t per = (nblk + nw - 1) / nw;
+  const int64_t per = p.per;
   const int64_t blk0 = (int64_t)wave * per;
   int64_t blk1 = blk0 + per;
   if (blk1 > nblk) blk1 = nblk;
@@ -88,16 +123,16 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   // The partial last block of the k range (elements past K count as zero), if this wavefront owns it:
   // requested first, multiplied last, so that its round trip to memory runs beside the whole blocks'.
   const bool has_tail = blk0 <= nfull && nfull < blk1;   // nfull is the number of the partial block, if there is one
+  // (the values are kept as loaded and zeroed where they are multiplied: a select here would make the wavefront wait
+  // for these loads before it has issued those of the whole blocks)
   T tail_a[4] = {0, 0, 0, 0}, tail_b[4] = {0, 0, 0, 0};
+  const int64_t tail_k = (nfull << 4) + 4 * g;
   if (has_tail) {
-    const int64_t k = (nfull << 4) + 4 * g;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const bool ok = k + s < p.K;
-      const int64_t kk = ok ? k + s : p.K - 1;
-      const T x = a[kk * p.a_k], y = b[kk * p.b_k];
-      tail_a[s] = ok ? x : (T)0;
-      tail_b[s] = ok ? y : (T)0;
+      const int64_t kk = tail_k + s < p.K ? tail_k + s : p.K - 1;
+      tail_a[s] = a[kk * p.a_k];
+      tail_b[s] = b[kk * p.b_k];
     }
   }
   T av[2][CHUNK][4], bv[2][CHUNK][4];
@@ -152,7 +187,10 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
   }
   if (has_tail) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) acc = M16<T>::mma(tail_a[s], tail_b[s], acc);
+    for (int s = 0; s < 4; ++s) {
+      const bool ok = tail_k + s < p.K;
+      acc = M16<T>::mma(ok ? tail_a[s] : (T)0, ok ? tail_b[s] : (T)0, acc);
+    }
   }
 
   if (nchunks <= 0) { probe.mark(1); probe.settle(); probe.mark(2); }
@@ -215,14 +253,15 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16(Args<T> p) {
 // 16-byte instead of 64-byte runs on both B and C, and VN independent accumulator chains per wavefront.
 // Requires N % VN == 0 (no vector crosses the end of a row of B).
 template <typename T, bool AVEC, int MAXW, int CHUNK>
-__global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
+__global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(SmallArgs<T> p) {
   typedef typename M16<T>::acc_t acc_t;
   constexpr int VN = 16 / (int)sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(VN)));
   extern __shared__ __attribute__((aligned(16))) unsigned char red_raw[];   // [W][VN][256] partial tiles, W > 1 only
   T (*red)[VN * 256] = reinterpret_cast<T (*)[VN * 256]>(red_raw);
+  request_args(p);
   PhaseProbe probe(p.phase_out, p.phase_cap, (unsigned)((p.N + 16 * VN - 1) / (16 * VN)));   // marks as in gemm_rows16
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = p.nw;
   const int i = lane & 15, g = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.y * 16, n0 = (int64_t)blockIdx.x * (16 * VN);
   // rows / column vectors past the edge read the last valid one; their results are not stored
@@ -232,7 +271,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   const T* b = p.B + bcol;
 
   const int64_t nfull = p.K >> 4, nblk = (p.K + 15) >> 4;
-  const int64_t per = (nblk + nw - 1) / nw;
+  const int64_t per = p.per;
   const int64_t blk0 = (int64_t)wave * per;
   int64_t blk1 = blk0 + per;
   if (blk1 > nblk) blk1 = nblk;
@@ -246,16 +285,13 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   vec_t tail_b[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) tail_b[s] = vec_t{};
-  if (has_tail) {
-    const int64_t k = (nfull << 4) + 4 * g;
+  const int64_t tail_k = (nfull << 4) + 4 * g;
+  if (has_tail) {   // kept as loaded, zeroed where they are multiplied (see gemm_rows16)
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const bool ok = k + s < p.K;
-      const int64_t kk = ok ? k + s : p.K - 1;
-      const T x = a[kk * p.a_k];
-      const vec_t y = *(const vec_t*)(b + kk * p.b_k);
-      tail_a[s] = ok ? x : (T)0;
-      tail_b[s] = ok ? y : vec_t{};
+      const int64_t kk = tail_k + s < p.K ? tail_k + s : p.K - 1;
+      tail_a[s] = a[kk * p.a_k];
+      tail_b[s] = *(const vec_t*)(b + kk * p.b_k);
     }
   }
   T av[2][CHUNK][4];
@@ -305,9 +341,12 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_rows16n(Args<T> p) {
   }
   if (has_tail) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
+    for (int s = 0; s < 4; ++s) {
+      const bool ok = tail_k + s < p.K;
+      const T x = ok ? tail_a[s] : (T)0;
 #pragma unroll
-      for (int j = 0; j < VN; ++j) acc[j] = M16<T>::mma(tail_a[s], tail_b[s][j], acc[j]);
+      for (int j = 0; j < VN; ++j) acc[j] = M16<T>::mma(x, ok ? tail_b[s][j] : (T)0, acc[j]);
+    }
   }
 
   if (nchunks <= 0) { probe.mark(1); probe.settle(); probe.mark(2); }
@@ -384,7 +423,13 @@ static inline bool applicable(const Args<T>& g) {
   if (mn > 64) return false;
   if (forced == 1) return true;
   const double macs = (double)g.M * (double)g.N * (double)g.K;
-  return macs <= 268435456.0 && g.K <= 8192;
+  if (!(macs <= 268435456.0 && g.K <= 8192)) return false;
+  // Where 32 x 32 tiles of the LDS-staged kernel already give every CU a workgroup without any split of k, that kernel
+  // is ahead: its operands cross the vector L1 once per 32 x 32 tile instead of once per 16 x 16 tile, and the number of
+  // L1 accesses is what bounds such a product here ([50 x 500] * [500 x 4096]: 7.3 against 8.0 us). A short k is not worth
+  // the staging ([20 x 25] * [25 x 36864]: 6.2 against 6.0).
+  const int64_t tiles32 = ((g.M + 31) / 32) * ((g.N + 31) / 32);
+  return !(tiles32 >= (int64_t)num_cus() && g.K >= 128);
 }
 
 template <typename T>
@@ -423,6 +468,7 @@ static int run(const Args<T>& g_in) {
   const bool avec = g.a_k == 1 && aligned16(g.A) && (g.a_mn % VK == 0 || g.M == 1);
   const bool bvec = g.b_k == 1 && aligned16(g.B) && (g.b_mn % VK == 0 || g.N == 1);
   const dim3 grid((unsigned)tiles_n, (unsigned)tiles_m), block((unsigned)nw * 64);
+  const SmallArgs<T> sa = small_args(g, nw);
   if (trace_choices()) fprintf(stderr, "am_hip gemm: small path, %lld x %lld tiles of 16 x 16, %d wavefronts per tile\n", (long long)tiles_m, (long long)tiles_n, nw);
   // Chunks of four (float) or two (double) blocks of 16 k where a wavefront has that many; one block at a
   // time where its share of k is one or two blocks: that instantiation needs a third of the registers,
@@ -433,18 +479,18 @@ static int run(const Args<T>& g_in) {
     if (trace_choices()) fprintf(stderr, "am_hip gemm: small path, B in 16-byte vectors along n\n");
     constexpr int CHN = 2;
     if (short_k) {
-      if (avec) hipLaunchKernelGGL((gemm_rows16n<T, true, kMaxWaves, 1>), grid, block, lds, stream(), g);
-      else hipLaunchKernelGGL((gemm_rows16n<T, false, kMaxWaves, 1>), grid, block, lds, stream(), g);
+      if (avec) hipLaunchKernelGGL((gemm_rows16n<T, true, kMaxWaves, 1>), grid, block, lds, stream(), sa);
+      else hipLaunchKernelGGL((gemm_rows16n<T, false, kMaxWaves, 1>), grid, block, lds, stream(), sa);
     } else {
-      if (avec) hipLaunchKernelGGL((gemm_rows16n<T, true, kMaxWaves, CHN>), grid, block, lds, stream(), g);
-      else hipLaunchKernelGGL((gemm_rows16n<T, false, kMaxWaves, CHN>), grid, block, lds, stream(), g);
+      if (avec) hipLaunchKernelGGL((gemm_rows16n<T, true, kMaxWaves, CHN>), grid, block, lds, stream(), sa);
+      else hipLaunchKernelGGL((gemm_rows16n<T, false, kMaxWaves, CHN>), grid, block, lds, stream(), sa);
     }
     return check_launch("gemm_rows16n");
   }
 #define AM_SMALL_LAUNCH(AV, BV)                                                                              \
   do {                                                                                                       \
-    if (short_k) hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, 1>), grid, block, lds, stream(), g);   \
-    else hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, CH>), grid, block, lds, stream(), g);          \
+    if (short_k) hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, 1>), grid, block, lds, stream(), sa);   \
+    else hipLaunchKernelGGL((gemm_rows16<T, AV, BV, kMaxWaves, CH>), grid, block, lds, stream(), sa);          \
   } while (0)
   if (avec && bvec) AM_SMALL_LAUNCH(true, true);
   else if (avec) AM_SMALL_LAUNCH(true, false);

@@ -356,7 +356,7 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
             del os.environ[env]
         vt = 2.0 * n ** 3 / (ev_valu / k) / 1e12
         peak = ctx.ceilings.get("valu_int32_mac" if dt == np.int32 else "valu_int64_mac")
-        roof = dict(bound="valu", achieved=round(vt, 3), peak=peak, unit="Top/s (measured VALU ceiling)",
+        roof = dict(bound="valu", achieved=round(vt, 3), peak=peak, unit="Top/s, measured ceiling",
                     frac=round(vt / peak, 4) if peak else None)
         if dt == np.int32:
             roof["frac_of_full_rate_78.6"] = round(vt / VALU_FULL_RATE_TOPS, 4)
@@ -364,7 +364,7 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
             roof["sclk_mhz"] = timer.sclk_mhz
             if dt == np.int32:
                 roof["frac_of_full_rate_at_sclk"] = round(vt / (VALU_FULL_RATE_TOPS * timer.sclk_mhz / 2400.0), 4)
-        out.append(dict(workload=f"{sfx} GEMM {n}^3, {label}, VALU kernel", config=config, unit="Top/s", value=round(vt, 3),
+        out.append(dict(workload=f"{sfx} GEMM {n}^3, {label}, VALU", config=config, unit="Top/s", value=round(vt, 3),
                         ms_per_step=round(ev_valu / k * 1e3, 5), roofline=roof))
     return out
 
@@ -390,7 +390,7 @@ def wl_gemm_i32_prepared(ctx):
     pa, pb = am.digits_prepare(dA, "left"), am.digits_prepare(dB, "right")
     kd = max(20, ctx.steps)
     out = []
-    for label, kw in (("B's digit planes prepared", dict(b_digits=pb)), ("both operands' digit planes prepared", dict(a_digits=pa, b_digits=pb))):
+    for label, kw in (("B's digits prepared", dict(b_digits=pb)), ("A's and B's digits prepared", dict(a_digits=pa, b_digits=pb))):
         wall, ev = timer.run(lambda: am.gemm(1, dA, dB, 0, dC, **kw), kd, ctx.warmup, (SPIN_I8, 0.08), min_warm_s=0.3)
         tops = 2.0 * n ** 3 / (ev / kd) / 1e12
         out.append(dict(workload=f"i32 GEMM 4096^3, in [-100,100], {label}", config="C2", unit="Top/s",
@@ -459,7 +459,7 @@ def wl_gemm_f64_views(ctx):
     steps = max(ctx.steps, 50)
     wall, ev = timer.run(lambda: am.gemm(1.5, dA, dB, 0.5, dC), steps, ctx.warmup, (SPIN_F64, 0.1), min_warm_s=MATRIX_WARM_S)
     fl = 2.0 * 2048 * 3072 * 1024
-    return dict(workload="f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C) 2048x3072x1024", config="C3", unit="TFLOP/s",
+    return dict(workload="f64 gemm(1.5, A^T, B[:, ::2], 0.5, C) 2048x3072x1024", config="C3", unit="TFLOP/s",
                 value=round(fl * steps / wall / 1e12, 3), ms_per_step=round(ev / steps * 1e3, 5),
                 roofline=mfma_roof(fl / (ev / steps) / 1e12, MFMA_F64_PEAK_TFLOPS, timer.sclk_mhz))
 
@@ -606,7 +606,7 @@ def wl_chain(ctx):
         return graph
     steps = max(ctx.steps, 50)
     r, best = eager_and_graph(ctx, issue, capture, steps)
-    return dict(workload="f32 chain [20x25].[25x36864], [50x500].[500x4096], [64x800].[800x500]+bias+ReLU, [64x500].[500x10]",
+    return dict(workload="f32 chain of 4 GEMMs [20x25x36864], [50x500x4096], [64x800x500]+bias+ReLU, [64x500x10]",
                 config="C5", unit="us per chain", higher_is_better=False, **r, gflops=round(flops / best / 1e9, 1),
                 roofline=dict(hbm_roof(nbytes / best / 1e9), unit="GB/s"))
 
@@ -1081,7 +1081,7 @@ def main():
     traffic, traffic_src = load_traffic("gemm_f32_4096")
     roof = mfma_roof(kern_tflops, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"], unit="TFLOP/s")
     roof.update(traffic=traffic, traffic_source=traffic_src)
-    protocol = "per entry: register-only spin, >= 30 ms of its own launches, K timed between HIP events; HBM-bound ones rotate 3-5 buffer sets"
+    protocol = "per entry: register-only spin, its own launches (1 s if matrix-bound), K timed by HIP events; HBM-bound: 3-5 rotating buffer sets"
     line = {
         "metric": "GEMM TFLOP/s (%MFMA peak) fp32/int32 4096^3; broadcast op HBM GB/s (%peak)",
         "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -1091,7 +1091,7 @@ def main():
         "roofline": roof,
         "from_idle": {"value": round(idle["flops"] * args.steps / idle["wall"] / 1e12, 3), "unit": "TFLOP/s",
                       "ms_per_step": round(idle["wall"] / args.steps * 1e3, 4), "sclk_mhz": idle["sclk_mhz"],
-                      "what": "same steps from an idle device; `value` follows 80 ms of register-only MFMA work"},
+                      "what": "no spin first; `value` follows 80 ms of register-only MFMA work"},
         "device": info, "protocol": protocol,
     }
     if not args.no_others:
