@@ -33,7 +33,15 @@ static int run_whole_f32(Args<float>& g) {
   const TileChoice* cand = candidates_f32(&nc);
   switch (choose_tile_and_split(g, cand, nc, "AM_HIP_GEMM_TILE_F32", 157.3e6 / 256)) {
     case 0: return launch_kinds<float, 256, 256, 16, 2, 4, 1, true, false>(g, ak, bk);   // its loop is long enough: unrolling it over the ring costs 4 %
-    case 1: return launch_kinds<float, 128, 128, 16, 2, 2, 2>(g, ak, bk);
+    case 1: {
+      // Eight wavefronts of 32 x 64 (two per SIMD, which cover each other's waits) where no split of k is planned and the
+      // four-wavefront form would not split either: 2048^3 127.2 -> 125.6 us, 2560^3 317 -> 302, 3072 x 3072 x 1024 193 ->
+      // 187, 2048 x 2048 x 256 23.4 -> 21.9. Eight of 64 x 32 lose (133.5 us at 2048^3). Products that are cut along k keep
+      // four wavefronts of 64 x 64: two workgroups, on different ranges of k, then share a CU.
+      const int64_t tiles = ((g.M + 127) / 128) * ((g.N + 127) / 128) * (g.batch > 1 ? g.batch : 1);
+      if (g.want_splits <= 1 && tiles * 8 > (int64_t)num_cus() * 4) return launch_kinds<float, 128, 128, 16, 4, 2, 2>(g, ak, bk);
+      return launch_kinds<float, 128, 128, 16, 2, 2, 2>(g, ak, bk);
+    }
     case 2: return launch_kinds<float, 64, 64, 16, 2, 2, 2>(g, ak, bk);
     case 3: return launch_kinds<float, 256, 128, 16, 4, 2>(g, ak, bk);
     case 4: return launch_kinds<float, 128, 64, 16, 2, 2, 2>(g, ak, bk);

@@ -344,7 +344,7 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
     tops = 2.0 * n ** 3 / (ev / kd) / 1e12
     entry = dict(workload=f"{sfx} GEMM {n}^3, {label}", config=config, unit="Top/s", value=round(2.0 * n ** 3 * kd / wall / 1e12, 3),
                  ms_per_step=round(ev / kd * 1e3, 5), digit_pairs=f"{pairs}/{npairs}",
-                 roofline=mfma_roof(pairs * tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s executed"))
+                 roofline=mfma_roof(pairs * tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s"))
     out = [entry]
     if valu:
         env = f"AM_HIP_GEMM_{sfx.upper()}_PATH"
@@ -356,14 +356,14 @@ def int_gemm_entries(ctx, dt, n, lo, hi, config, label, valu=True, seeds=(2001, 
             del os.environ[env]
         vt = 2.0 * n ** 3 / (ev_valu / k) / 1e12
         peak = ctx.ceilings.get("valu_int32_mac" if dt == np.int32 else "valu_int64_mac")
-        roof = dict(bound="valu", achieved=round(vt, 3), peak=peak, unit="Top/s, measured ceiling",
+        roof = dict(bound="valu", achieved=round(vt, 3), peak=peak, unit="Top/s, measured",
                     frac=round(vt / peak, 4) if peak else None)
         if dt == np.int32:
-            roof["frac_of_full_rate_78.6"] = round(vt / VALU_FULL_RATE_TOPS, 4)
+            roof["frac_of_78.6"] = round(vt / VALU_FULL_RATE_TOPS, 4)
         if timer.sclk_mhz:
             roof["sclk_mhz"] = timer.sclk_mhz
             if dt == np.int32:
-                roof["frac_of_full_rate_at_sclk"] = round(vt / (VALU_FULL_RATE_TOPS * timer.sclk_mhz / 2400.0), 4)
+                roof["frac_of_78.6_at_sclk"] = round(vt / (VALU_FULL_RATE_TOPS * timer.sclk_mhz / 2400.0), 4)
         out.append(dict(workload=f"{sfx} GEMM {n}^3, {label}, VALU", config=config, unit="Top/s", value=round(vt, 3),
                         ms_per_step=round(ev_valu / k * 1e3, 5), roofline=roof))
     return out
@@ -395,7 +395,7 @@ def wl_gemm_i32_prepared(ctx):
         tops = 2.0 * n ** 3 / (ev / kd) / 1e12
         out.append(dict(workload=f"i32 GEMM 4096^3, in [-100,100], {label}", config="C2", unit="Top/s",
                         value=round(2.0 * n ** 3 * kd / wall / 1e12, 3), ms_per_step=round(ev / kd * 1e3, 5),
-                        roofline=mfma_roof(tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s executed")))
+                        roofline=mfma_roof(tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s")))
     return out
 
 
@@ -442,8 +442,8 @@ def wl_i64_1500(ctx):
     return dict(workload="i64 matmul 1500^2, entries in [0, 99]", config="published",
                 unit="Top/s", value=round(2.0 * n5 ** 3 * k5 / wall / 1e12, 3), ms_per_step=round(ev / k5 * 1e3, 5),
                 row_750_matches_numpy=bool(np.array_equal(dC.toCpu()[n5 // 2], want)),
-                roofline=mfma_roof(tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s executed"),
-                published_s=0.14, published_on="i9-9980XE, benchmarks/integer_matmul.nim:8-33")
+                roofline=mfma_roof(tops, MFMA_I8_PEAK_TOPS, timer.sclk_mhz, unit="int8 TOP/s"),
+                published_s=0.14, published_on="i9-9980XE, integer_matmul.nim:8-33")
 
 
 # ------------------------------------------------------------------------------------------ C3: float64 views
@@ -581,7 +581,9 @@ def eager_and_graph(ctx, issue, capture, steps):
     """issue() from the host `steps` times, then (unless --no-graphs) the same sequence replayed from one HIP graph."""
     timer = ctx.timer
     wall_e, ev_e = timer.run(issue, steps, ctx.warmup, (SPIN_F32, 0.05))
-    out = dict(eager_us=round(ev_e / steps * 1e6, 2), eager_wall_us=round(wall_e / steps * 1e6, 2))
+    out = dict(eager_us=round(ev_e / steps * 1e6, 2))
+    if getattr(ctx, "solo", False):
+        out["eager_wall_us"] = round(wall_e / steps * 1e6, 2)
     best = ev_e
     if ctx.graphs:
         graph = capture()
@@ -1081,7 +1083,7 @@ def main():
     traffic, traffic_src = load_traffic("gemm_f32_4096")
     roof = mfma_roof(kern_tflops, MFMA_F32_PEAK_TFLOPS, r["sclk_mhz"], unit="TFLOP/s")
     roof.update(traffic=traffic, traffic_source=traffic_src)
-    protocol = "per entry: register-only spin, its own launches (1 s if matrix-bound), K timed by HIP events; HBM-bound: 3-5 rotating buffer sets"
+    protocol = "per entry: MFMA spin, own launches (1 s if matrix-bound), K timed by HIP events; HBM-bound: rotating buffers"
     line = {
         "metric": "GEMM TFLOP/s (%MFMA peak) fp32/int32 4096^3; broadcast op HBM GB/s (%peak)",
         "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -1091,14 +1093,14 @@ def main():
         "roofline": roof,
         "from_idle": {"value": round(idle["flops"] * args.steps / idle["wall"] / 1e12, 3), "unit": "TFLOP/s",
                       "ms_per_step": round(idle["wall"] / args.steps * 1e3, 4), "sclk_mhz": idle["sclk_mhz"],
-                      "what": "no spin first; `value` follows 80 ms of register-only MFMA work"},
+                      "what": "no spin or warm-up second first"},
         "device": info, "protocol": protocol,
     }
     if not args.no_others:
         results = {}
         for name in DEFAULT_ORDER:
             if name == "gemm_i32_1500":      # the first entry that needs them; after the float matrix workloads
-                line["measured_ceilings"] = dict(ctx.ceilings, unit="T(FL)OP/s (hbm_*, runtime_d2d_copy: TB/s)")
+                line["measured_ceilings"] = dict(ctx.ceilings, unit="T(FL)OP/s; *_tbs TB/s")
             results[name] = WORKLOADS[name][0](ctx)
             _C4.clear() if name == "transposed_add" else None
             _TALL.clear() if name == "sum_rows_512" else None

@@ -117,6 +117,25 @@ def test_every_tile_shape(hip, oracle, sfx, tile, monkeypatch):
     assert_parity(oracle, sfx, dC.toCpu(), want, f"tile {tile}")
 
 
+@pytest.mark.parametrize("layout", ["CC", "FC", "CF", "FF"])
+def test_f32_128_tile_with_eight_wavefronts(hip, oracle, layout, monkeypatch):
+    """More than 128 tiles of 128 x 128 and no split of k: the workgroup of eight wavefronts (32 x 64 each) that the
+    library uses there, on ragged extents, every operand layout, alpha/beta and a strided destination."""
+    monkeypatch.setenv("AM_HIP_GEMM_TILE_F32", "1")
+    rng = np.random.default_rng(seed_of("tile128x8", layout))
+    for (M, N, K) in [(1500, 1400, 77), (1409, 1537, 16), (1665, 1281, 131)]:
+        A, B = fill(rng, (M, K), np.float32), fill(rng, (K, N), np.float32)
+        C = fill(rng, (M, 2 * N), np.float32)
+        dA = hip.toHip(np.ascontiguousarray(A.T)).transpose() if layout[0] == "F" else hip.toHip(A)
+        dB = hip.toHip(np.ascontiguousarray(B.T)).transpose() if layout[1] == "F" else hip.toHip(B)
+        say("tile128x8", layout, (M, N, K))
+        want = C.copy()
+        oracle.gemm_strided(-0.5, A, B, 2, want[:, ::2])
+        dC = hip.toHip(C)
+        hip.gemm(-0.5, dA, dB, 2, dC[:, ::2])
+        assert_parity(oracle, "f32", dC.toCpu(), want, f"{(M, N, K)} {layout}")
+
+
 @pytest.mark.parametrize("sfx", ALL)
 @pytest.mark.parametrize("layout", ["CC", "FC", "CF", "FF"])
 def test_unit_stride_operands_of_any_pitch_and_alignment(hip, oracle, sfx, layout):
