@@ -375,7 +375,9 @@ void gemm_mfma(Args<T> p) {
   // each load wait for the store before it (one memory counter orders both), i.e. one round trip
   // to HBM per element. (A whole row of tiles at once needs more registers than the largest tile
   // shapes have left next to their accumulators.) INTERIOR: the workgroup's tile lies wholly inside C,
-  // nothing is tested per element. PLAIN: C <- AB (alpha = 1, beta = 0, no fused epilogue), stores only.
+  // nothing is tested per element. PLAIN: C <- AB (alpha = 1, beta = 0, no fused epilogue), stores only, and those
+  // non-temporal: every workgroup of a round writes its tile at the same moment and nothing of C is read again by this
+  // kernel (f32 2048^3: 125.4 -> 123.3 - 124.0 us; no change where C is read first, so those stores stay ordinary).
   auto write_out = [&](auto interior_tag, auto plain_tag) {
     constexpr bool INTERIOR = decltype(interior_tag)::value;
     constexpr bool PLAIN = decltype(plain_tag)::value;
@@ -389,7 +391,7 @@ void gemm_mfma(Args<T> p) {
 #pragma unroll
           for (int r = 0; r < MF::NACC; ++r) {
             const int dr = i * TILE + MF::acc_row(r, 0);
-            if (INTERIOR || (col_ok && row0 + dr < p.M)) c0[dr * p.c_m + j * TILE * p.c_n] = acc[i][j][r];
+            if (INTERIOR || (col_ok && row0 + dr < p.M)) __builtin_nontemporal_store(acc[i][j][r], &c0[dr * p.c_m + j * TILE * p.c_n]);
           }
           continue;
         }
