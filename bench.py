@@ -572,7 +572,29 @@ def chain_setup(am):
         for f in stages:
             f()
 
+    # the same four calls with their arguments converted to C types once: what a compiled host pays per launch (the
+    # Python wrapper's shape checks and conversions take about as long as the smallest of these kernels runs)
+    L, vp, f32 = am.load_library(), ctypes.c_void_p, ctypes.c_float
+
+    def bound(A, B, C, epi=0, bias=None):
+        (M, K), N = A.shape, B.shape[1]
+        a = (M, N, K, f32(1.0), vp(A.data_ptr()), A.strides[0], A.strides[1], vp(B.data_ptr()), B.strides[0], B.strides[1],
+             f32(0.0), vp(C.data_ptr()), C.strides[0], C.strides[1])
+        if not epi:
+            return L.am_hip_gemm_f32, a
+        bb = bias.broadcast((M, N))
+        return L.am_hip_gemm_ex_f32, a + (epi, vp(bb.data_ptr()), bb.strides[0], bb.strides[1])
+    calls = [bound(k1, x1, o1), bound(k2, x2, o2), bound(x3, w3t, h, 3, b3), bound(h, w4t, o4)]
+
+    def issue_bound():
+        rc = 0
+        for fn, a in calls:
+            rc |= fn(*a)
+        if rc:
+            raise RuntimeError("a product of the chain failed")
+
     issue.stages = stages
+    issue.bound = issue_bound
     flops = 2.0 * (20 * 25 * 36864 + 50 * 500 * 4096 + 64 * 800 * 500 + 64 * 500 * 10)
     return issue, flops, 17834080, (k1, x1, o1, k2, x2, o2, x3, w3, b3, h, w4, o4)
 
@@ -585,14 +607,18 @@ def eager_and_graph(ctx, issue, capture, steps):
     if getattr(ctx, "solo", False):
         out["eager_wall_us"] = round(wall_e / steps * 1e6, 2)
     best = ev_e
+    out["value_is"] = "eager"
+    if getattr(issue, "bound", None):
+        _, ev_b = timer.run(issue.bound, steps, ctx.warmup, (SPIN_F32, 0.05))
+        out["eager_c_abi_us"] = round(ev_b / steps * 1e6, 2)
+        if ev_b < best:
+            best, out["value_is"] = ev_b, "eager_c_abi"
     if ctx.graphs:
         graph = capture()
         _, ev_g = timer.run(graph.launch, steps, ctx.warmup, (SPIN_F32, 0.05))
         out["hipgraph_us"] = round(ev_g / steps * 1e6, 2)
-        best = min(best, ev_g)
-        out["value_is"] = "eager" if ev_e <= ev_g else "hipgraph"
-    else:
-        out["value_is"] = "eager"
+        if ev_g < best:
+            best, out["value_is"] = ev_g, "hipgraph"
     out["value"] = round(best / steps * 1e6, 2)
     return out, best / steps
 
