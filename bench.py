@@ -893,14 +893,14 @@ def config_report(am, timer, L):
         print(json.dumps(kw), flush=True)
 
     def gemm_case(config, sfx, M, N, K, A, B, dA, dB, alpha=1, beta=0, C0=None, peak=None, peak_used="", unit="TFLOP/s", steps=20,
-                  spin=(SPIN_F32, 0.08)):
+                  spin=(SPIN_F32, 0.08), warm=0.05):
         dt = A.dtype
         C_host = C0.copy() if C0 is not None else np.zeros((M, N), dt)
         dC = am.toHip(C_host)
         am.gemm(alpha, dA, dB, beta, dC)
         got = dC.toCpu().copy()
         # (with beta != 0 the timed calls go on accumulating into C: only their time is used)
-        _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3, spin)
+        _, ev = timer.run(lambda: am.gemm(alpha, dA, dB, beta, dC), steps, 3, spin, min_warm_s=warm)
         gpu_s = ev / steps
         want = am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy())
         cpu_s = cpu_time(lambda: am_oracle.gemm_strided(alpha, A, B, beta, C_host.copy() if beta != 0 else C_host))
@@ -925,7 +925,7 @@ def config_report(am, timer, L):
     for n in (1024, 2048, 4096):
         A = rng(1001).uniform(-1, 1, (n, n)).astype(np.float32); B = rng(1002).uniform(-1, 1, (n, n)).astype(np.float32)
         gemm_case(f"f32 GEMM {n}^3", "f32", n, n, n, A, B, am.toHip(A), am.toHip(B), peak=MFMA_F32_PEAK_TFLOPS,
-                  peak_used="MFMA fp32 157.3 TFLOP/s", steps=200 if n <= 2048 else 20)
+                  peak_used="MFMA fp32 157.3 TFLOP/s", steps=200 if n <= 2048 else 20, warm=MATRIX_WARM_S if n <= 2048 else 0.05)
     # extents that are not a multiple of the 16-byte vector, beside their aligned neighbour (4096): unit-stride
     # operands are moved in 16-byte pieces whatever their pitch; 4097 runs as the 4096^3 block plus two skinny strips
     for n in (4095, 4097):
@@ -965,7 +965,7 @@ def config_report(am, timer, L):
     C0 = rng(3003).standard_normal((2048, 3072))
     gemm_case("f64 gemm(1.5, A^T view, B[:, ::2] view, 0.5, C)", "f64", 2048, 3072, 1024, pa.T, pb[:, ::2],
               am.toHip(pa).transpose(), am.toHip(pb)[:, ::2], alpha=1.5, beta=0.5, C0=C0, peak=MFMA_F64_PEAK_TFLOPS,
-              peak_used="MFMA fp64 78.6 TFLOP/s", steps=1, spin=(SPIN_F64, 0.3))
+              peak_used="MFMA fp64 78.6 TFLOP/s", steps=20, spin=(SPIN_F64, 0.1), warm=MATRIX_WARM_S)   # the entry's protocol (wl_gemm_f64_views)
     # broadcast ops
     X = rng(4001).uniform(-1, 1, (8192, 8192)).astype(np.float32)
     b = rng(4002).uniform(-1, 1, (1, 8192)).astype(np.float32); sc = rng(4003).uniform(-1, 1, (8192, 1)).astype(np.float32)
