@@ -633,6 +633,16 @@ def wl_chain(ctx):
             issue()
         return graph
     steps = max(ctx.steps, 50)
+    # the pre-converted calls do the same work as the wrapper's: all four results, bit for bit
+    outs = [keep[2], keep[5], keep[9], keep[11]]
+    issue()
+    want = [o.toCpu().copy() for o in outs]
+    from arraymancer_amd import tensor_hip as th
+    for o in outs:
+        th._scalar_into("mul", o, o, 0.0, False)      # (the second run must write them again)
+    issue.bound()
+    if not all(np.array_equal(o.toCpu(), w) for o, w in zip(outs, want)):
+        raise RuntimeError("chain: the pre-converted C-ABI calls and the wrapper calls disagree")
     r, best = eager_and_graph(ctx, issue, capture, steps)
     return dict(workload="f32 chain of 4 GEMMs [20x25x36864], [50x500x4096], [64x800x500]+bias+ReLU, [64x500x10]",
                 config="C5", unit="us per chain", higher_is_better=False, **r, gflops=round(flops / best / 1e9, 1),
